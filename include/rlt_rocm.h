@@ -1,0 +1,399 @@
+/*
+ * rlt_rocm.h -- C ABI of the MI355X (gfx950) backend for the dense-network
+ * training hot path of rl-tools.
+ *
+ * The reference library dispatches every operation by C++ overload on a device
+ * tag (rl_tools/devices/cuda.h:52-122 is the tag this backend sits next to).
+ * Each entry point below is what one such overload for a `devices::ROCM` tag
+ * binds to; the comment above it names the reference function it stands in for.
+ *
+ * Conventions
+ *  - every function returns 0 on success, a positive hipError_t value when the
+ *    HIP runtime failed, or a negative RLT_E_* code for a rejected argument;
+ *  - all data pointers are DEVICE pointers unless the name ends in `_host`;
+ *  - matrices are row-major, fp32, with an explicit leading dimension (`ld*`,
+ *    in elements) wherever a view of a wider matrix can be passed;
+ *  - work is enqueued on the device handle's stream and returns without
+ *    synchronising, except for the host<->device copies, which synchronise the
+ *    stream like the reference's do (containers/matrix/operations_cuda.h:149-195);
+ *  - boolean tensors of the reference (terminated, masks) are uint8_t here.
+ */
+#ifndef RLT_ROCM_H
+#define RLT_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RLT_E_INVALID_ARGUMENT (-1) /* null pointer, non-positive dimension, ld too small */
+#define RLT_E_UNSUPPORTED      (-2) /* shape outside what the kernels are built for      */
+#define RLT_E_NOT_INITIALISED  (-3)
+
+/* nn/activation_functions.h:11-18 -- same numbering as the reference enum */
+enum rlt_activation {
+    RLT_ACT_IDENTITY  = 0,
+    RLT_ACT_RELU      = 1,
+    RLT_ACT_GELU      = 2,
+    RLT_ACT_TANH      = 3,
+    RLT_ACT_FAST_TANH = 4,
+    RLT_ACT_SIGMOID   = 5
+};
+
+/* Opaque device object: one HIP device + one stream (devices/cuda.h:52-77 holds
+ * the same for CUDA plus a BLAS handle, which this backend has no use for). */
+typedef struct rlt_rocm_device rlt_rocm_device;
+
+/* ---------------------------------------------------------------- device -- */
+
+/* init(device)            devices/cuda.h:130-154 */
+int rlt_rocm_init(int hip_device_index, rlt_rocm_device** out_device);
+/* (no counterpart: the reference never destroys its handle) */
+int rlt_rocm_destroy(rlt_rocm_device* device);
+/* check_status(device)    devices/cuda.h:156-174 -- synchronises, returns the sticky error */
+int rlt_rocm_check_status(rlt_rocm_device* device);
+/* Adopt a caller-owned hipStream_t (NULL selects the handle's own stream again). */
+int rlt_rocm_set_stream(rlt_rocm_device* device, void* hip_stream);
+void* rlt_rocm_get_stream(rlt_rocm_device* device);
+/* Human-readable text for any code returned by this library. */
+const char* rlt_rocm_error_string(int code);
+/* Number of compute units and LDS bytes per workgroup the kernels were sized against. */
+int rlt_rocm_device_info(rlt_rocm_device* device, int* compute_units, int* lds_bytes, char* name, int name_len);
+
+/* ------------------------------------------------------------ containers -- */
+
+/* malloc / free           containers/matrix/operations_cuda.h:16-45, tensor/operations_cuda.h:15-39 */
+int rlt_rocm_malloc(rlt_rocm_device* device, void** out_ptr, size_t bytes);
+int rlt_rocm_free(rlt_rocm_device* device, void* ptr);
+/* copy (dense)            containers/matrix/operations_cuda.h:105-195 */
+int rlt_rocm_memcpy_h2d(rlt_rocm_device* device, void* dst, const void* src_host, size_t bytes);
+int rlt_rocm_memcpy_d2h(rlt_rocm_device* device, void* dst_host, const void* src, size_t bytes);
+int rlt_rocm_memcpy_d2d(rlt_rocm_device* device, void* dst, const void* src, size_t bytes);
+/* copy (strided views)    containers/matrix/operations_cuda.h:48-60,98-103 ; tensor copy2d :94-168
+ * kind: 0 = device->device, 1 = host->device, 2 = device->host; widths/pitches in bytes. */
+int rlt_rocm_memcpy2d(rlt_rocm_device* device, void* dst, size_t dst_pitch, const void* src, size_t src_pitch,
+                      size_t width_bytes, size_t rows, int kind);
+/* set_all                 containers/matrix/operations_cuda.h:62-74,201-207 */
+int rlt_rocm_fill_f32(rlt_rocm_device* device, float* dst, int rows, int cols, int ld, float value);
+int rlt_rocm_fill_u8(rlt_rocm_device* device, uint8_t* dst, size_t count, uint8_t value);
+/* randn / rand            containers/tensor/operations_cuda.h:548-624 (counter-based: the stream of
+ * values is a pure function of (seed, offset, element index), no state array is needed) */
+int rlt_rocm_randn_f32(rlt_rocm_device* device, float* dst, size_t count, uint64_t seed, uint64_t offset);
+int rlt_rocm_rand_f32(rlt_rocm_device* device, float* dst, size_t count, float low, float high, uint64_t seed, uint64_t offset);
+/* scale(t, s, reciprocal) containers/tensor/operations_generic.h:433-445,713 : x <- reciprocal ? s/x : s*x */
+int rlt_rocm_scale_f32(rlt_rocm_device* device, float* x, size_t count, float s, int reciprocal);
+/* cast_reduce_sum<T>(bool tensor) containers/tensor/operations_generic.h:928-985 (CUDA: <<<1,1>>>, operations_cuda.h:287-307) */
+int rlt_rocm_cast_reduce_sum_u8(rlt_rocm_device* device, const uint8_t* mask, size_t count, float* out_sum);
+/* sum / squared-sum of a float tensor (gradient_norm, nn/parameters/operations_generic.h) */
+int rlt_rocm_reduce_sum_f32(rlt_rocm_device* device, const float* x, size_t count, int squared, float* out_sum);
+
+/* ------------------------------------------------------------ dense / MLP -- */
+
+/* One dense layer as the reference stores it (nn/layers/dense/layer.h:82-135 plus the Adam
+ * parameter instances, nn/optimizers/adam/adam.h:76-96). Unused members may be NULL. */
+typedef struct rlt_dense_layer {
+    float* weights;          /* [out_dim x in_dim], row-major, packed          */
+    float* biases;           /* [out_dim]                                      */
+    float* d_weights;        /* gradient accumulators (LayerGradient)          */
+    float* d_biases;
+    float* pre_activations;  /* [batch x out_dim] packed (LayerBackward)       */
+    float* output;           /* [batch x out_dim] packed (LayerGradient)       */
+    int32_t in_dim;
+    int32_t out_dim;
+    int32_t activation;      /* enum rlt_activation                            */
+    int32_t reserved;
+} rlt_dense_layer;
+
+/* evaluate(dense)         nn/layers/dense/operations_cpu_blas.h:36-72, operations_cuda.h:237-276
+ * y = act(x W^T + b); nothing is stored in the layer. */
+int rlt_rocm_dense_evaluate(rlt_rocm_device* device, const rlt_dense_layer* layer,
+                            const float* x, int ldx, float* y, int ldy, int batch);
+/* forward(dense)          nn/layers/dense/operations_cpu_blas.h:74-116, operations_cuda.h:278-316
+ * also stores layer->pre_activations and (if non-NULL) layer->output; y may be NULL. */
+int rlt_rocm_dense_forward(rlt_rocm_device* device, const rlt_dense_layer* layer,
+                           const float* x, int ldx, float* y, int ldy, int batch);
+/* backward_input(dense)   operations_cpu_blas.h:219-223: d_output <- d_pre = act'(pre) * d_output, d_input = d_pre W */
+int rlt_rocm_dense_backward_input(rlt_rocm_device* device, const rlt_dense_layer* layer,
+                                  float* d_output, int ldd, float* d_input, int ldi, int batch);
+/* backward(dense)         operations_cpu_blas.h:143-186: d_output <- d_pre, d_biases += sum_batch d_pre, d_weights += d_pre^T x */
+int rlt_rocm_dense_backward(rlt_rocm_device* device, const rlt_dense_layer* layer,
+                            const float* x, int ldx, float* d_output, int ldd, int batch);
+/* backward_full(dense)    operations_cpu_blas.h:224-228 = backward + d_input */
+int rlt_rocm_dense_backward_full(rlt_rocm_device* device, const rlt_dense_layer* layer,
+                                 const float* x, int ldx, float* d_output, int ldd,
+                                 float* d_input, int ldi, int batch);
+
+/* Workspace an MLP call needs (the reference's tick/tock buffers, nn_models/mlp/network.h:127-140):
+ * bytes for `batch` rows through `layers`. */
+size_t rlt_rocm_mlp_workspace_bytes(const rlt_dense_layer* layers, int n_layers, int batch);
+/* evaluate(mlp)           nn_models/mlp/operations_generic.h:77-102 */
+int rlt_rocm_mlp_evaluate(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers,
+                          const float* x, int ldx, float* y, int ldy, int batch,
+                          void* workspace, size_t workspace_bytes);
+/* forward(mlp)            nn_models/mlp/operations_generic.h:103-114 (stores pre_activations/output of every layer) */
+int rlt_rocm_mlp_forward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers,
+                         const float* x, int ldx, int batch);
+/* backward / backward_full / backward_input (mlp)   nn_models/mlp/operations_generic.h:126-204
+ *   want_weight_gradients = 0 -> backward_input, 1 -> backward (d_input == NULL) or backward_full.
+ * d_output is overwritten with the last layer's d_pre, as in the reference. */
+int rlt_rocm_mlp_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers,
+                          const float* x, int ldx, float* d_output, int ldd,
+                          float* d_input, int ldi, int batch, int want_weight_gradients,
+                          void* workspace, size_t workspace_bytes);
+/* zero_gradient(mlp)      nn_models/mlp/operations_generic.h:117-124 */
+int rlt_rocm_mlp_zero_gradient(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers);
+
+/* Fused forward + backward of a whole MLP for a caller that already holds the upstream gradient
+ * (the standalone microbenchmark shape, and PPO's critic where d_output = mse gradient is fused via
+ * `target`): one pass over the batch, activations never leave the chip.
+ *   y           [batch x out] network output (may be NULL)
+ *   d_output    [batch x out] upstream gradient, used when target == NULL (not modified)
+ *   target      if non-NULL, d_output is formed as (y - target) * mse_scale instead
+ * Weight/bias gradients are ACCUMULATED into the layers' d_weights/d_biases (beta = 1, as the
+ * reference's backward does). No pre_activations/output are stored. */
+int rlt_rocm_mlp_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers,
+                                  const float* x, int ldx, float* y, int ldy,
+                                  const float* d_output, int ldd,
+                                  const float* target, int ldt, float mse_scale,
+                                  int batch, void* workspace, size_t workspace_bytes);
+
+/* -------------------------------------------------------- optimiser/polyak -- */
+
+/* nn/optimizers/adam/adam.h:13-48 (Parameters<T>); the *_TENSORFLOW defaults are
+ * alpha 1e-3, beta (0.9, 0.999), epsilon = epsilon_sqrt = 1e-7; *_PYTORCH uses 1e-8. */
+typedef struct rlt_adam_parameters {
+    float alpha, beta_1, beta_2, epsilon, epsilon_sqrt;
+    float weight_decay;      /* applied to entries flagged is_weight when enable_weight_decay */
+    float bias_lr_factor;    /* applied to entries flagged is_bias when enable_bias_lr_factor */
+    int32_t enable_weight_decay;
+    int32_t enable_bias_lr_factor;
+    int32_t enable_gradient_clipping;
+    float gradient_clip_value;
+} rlt_adam_parameters;
+
+/* One parameter tensor with its Adam state (nn/optimizers/adam/adam.h:76-96). */
+typedef struct rlt_adam_tensor {
+    float* parameters;
+    float* gradient;
+    float* first_moment;
+    float* second_moment;
+    float* polyak_target;   /* optional: target <- polyak*target + (1-polyak)*new_parameter, fused */
+    uint32_t count;
+    uint32_t flags;         /* bit0: is_weight, bit1: is_bias */
+} rlt_adam_tensor;
+
+/* step(optimizer, model)  nn/optimizers/adam/operations_generic.h:49-66 + instance/operations_generic.h:26-72
+ * `age` is a device-resident uint32 (starts at 1, operations_generic.h:43-47); the bias corrections
+ * 1/(1-beta^age) are computed on the device from it and it is incremented by the same launch, so no
+ * host round trip is needed (the reference spends a <<<1,1>>> kernel on this, adam/operations_cuda.h:18-68).
+ * `tensors_host` is a host array; it is copied into the launch. polyak is ignored where polyak_target == NULL.
+ * If out_gradient_squared_norm is non-NULL it receives sum(g^2) over all tensors. */
+int rlt_rocm_adam_step(rlt_rocm_device* device, const rlt_adam_tensor* tensors_host, int n_tensors,
+                       const rlt_adam_parameters* parameters_host, uint32_t* age,
+                       float polyak, float* out_gradient_squared_norm);
+/* reset_optimizer_state   adam/operations_generic.h:43-47: age <- 1, moments <- 0 */
+int rlt_rocm_adam_reset(rlt_rocm_device* device, const rlt_adam_tensor* tensors_host, int n_tensors, uint32_t* age);
+/* utils::polyak::update / update_squared   utils/polyak/operations_generic.h:11-43, operations_cuda.h:13-48 */
+int rlt_rocm_polyak_update(rlt_rocm_device* device, const float* source, float* target, size_t count,
+                           float polyak, int squared);
+
+/* ------------------------------------------------------------------- loss -- */
+
+/* mse::gradient           nn/loss_functions/mse/operations_generic.h:41-97, operations_cuda.h:13-57
+ * d_a = (a - b) * 2/(rows*cols) * w ; w = *loss_weight_device if non-NULL else loss_weight. */
+int rlt_rocm_mse_gradient(rlt_rocm_device* device, const float* a, int lda, const float* b, int ldb,
+                          float* d_a, int ldda, int rows, int cols,
+                          float loss_weight, const float* loss_weight_device);
+/* mse::evaluate           mse/operations_generic.h:9-21 : out = sum((a-b)^2) * w / (rows*cols) */
+int rlt_rocm_mse_evaluate(rlt_rocm_device* device, const float* a, int lda, const float* b, int ldb,
+                          int rows, int cols, float loss_weight, float* out_loss);
+
+/* ----------------------------------------------------- sample_and_squash -- */
+
+/* nn/layers/sample_and_squash/layer.h:29-39 */
+typedef struct rlt_sas_parameters {
+    float log_std_lower_bound;   /* -20 */
+    float log_std_upper_bound;   /*   2 */
+    float log_probability_epsilon; /* 1e-6 */
+    float target_entropy;        /* -action_dim */
+} rlt_sas_parameters;
+
+/* evaluate / forward      sample_and_squash/operations_generic.h:148-280, operations_cuda.h:17-56
+ *   input  [batch x 2*dim] = [mean | log_std]; noise [batch x dim] (NULL = zeros, i.e. Evaluation mode
+ *   without the sample path: action = tanh(mean)); actions [batch x dim];
+ *   log_probabilities [batch]; pre_squashing [batch x dim] may be NULL (evaluate does not keep it). */
+int rlt_rocm_sas_forward(rlt_rocm_device* device, const rlt_sas_parameters* p,
+                         const float* input, int ldin, const float* noise, int ldn,
+                         float* actions, int lda, float* pre_squashing, int ldp,
+                         float* log_probabilities, int batch, int dim);
+/* backward_full           sample_and_squash/operations_generic.h:289-398, operations_cuda.h:58-115
+ *   d_input [batch x 2*dim]; d_log_alpha (device scalar) is INCREMENTED by
+ *   mean_batch( alpha * (-log_prob - target_entropy) ), alpha = exp(*log_alpha). */
+int rlt_rocm_sas_backward(rlt_rocm_device* device, const rlt_sas_parameters* p,
+                          const float* input, int ldin, const float* noise, int ldn,
+                          const float* actions, int lda, const float* pre_squashing, int ldp,
+                          const float* d_output, int lddo, float* d_input, int lddi,
+                          const float* log_alpha, float* d_log_alpha, int batch, int dim);
+
+/* ------------------------------------------------------------------ SAC --- */
+
+/* target_action_values    rl/algorithms/sac/operations_generic.h:133-179, operations_cuda.h:12-44
+ *   y = r + gamma * (!terminated) * (min(q1, q2) - exp(log_alpha) * log_prob) */
+int rlt_rocm_sac_target_action_values(rlt_rocm_device* device, const float* q1_next, const float* q2_next,
+                                      const float* rewards, const uint8_t* terminated,
+                                      const float* next_log_probabilities, const float* log_alpha,
+                                      float gamma, int ignore_termination, float* target, int batch);
+/* min_value_d_output      sac/operations_generic.h:358-393, operations_cuda.h:88-128 */
+int rlt_rocm_sac_min_value_d_output(rlt_rocm_device* device, const float* q1, const float* q2,
+                                    const float* d_critic_1_input, const float* d_critic_2_input, int ld_critic_input,
+                                    int critic_input_dim, int action_dim, float* d_actor_output, int ldo, int batch);
+/* mask_actions            sac/operations_generic.h:181-209, operations_cuda.h:47-66 : rows where (mask != invert) are copied */
+int rlt_rocm_mask_copy(rlt_rocm_device* device, const float* source, int lds, float* target, int ldt,
+                       const uint8_t* mask, int invert, int rows, int cols);
+/* mask_gradient           sac/operations_generic.h:210-234, operations_cuda.h:68-86 : rows where (mask != invert) are zeroed */
+int rlt_rocm_mask_zero(rlt_rocm_device* device, float* gradient, int ld, const uint8_t* mask, int invert, int rows, int cols);
+
+/* Everything one SAC agent owns on the device (rl/algorithms/sac/sac.h:62-145 ActorCritic and the
+ * Critic/ActorTrainingBuffers, plus the batch of rl/components/off_policy_runner/off_policy_runner.h:89-156
+ * for SEQUENCE_LENGTH = 1). All networks are MLPs described by rlt_dense_layer arrays (host arrays of
+ * descriptors whose pointers are device pointers). */
+typedef struct rlt_sac_agent {
+    int32_t batch, observation_dim, action_dim, n_actor_layers, n_critic_layers;
+    float gamma, polyak, reserved0;
+    rlt_sas_parameters sas;
+    rlt_adam_parameters actor_adam, critic_adam, alpha_adam;
+    const rlt_dense_layer* actor;            /* out_dim of last layer = 2*action_dim */
+    const rlt_dense_layer* critics[2];
+    const rlt_dense_layer* critics_target[2];
+    const rlt_adam_tensor* actor_adam_tensors;      int32_t n_actor_adam_tensors;   int32_t pad0;
+    const rlt_adam_tensor* critic_adam_tensors[2];  int32_t n_critic_adam_tensors;  int32_t pad1;
+    /* log_alpha as an Adam parameter instance (count = 1) */
+    rlt_adam_tensor log_alpha;
+    uint32_t* actor_age; uint32_t* critic_age[2]; uint32_t* alpha_age;
+    /* batch (SequentialBatch, SEQUENCE_LENGTH = 1): [2 x batch x (obs+act)] */
+    float* observations_actions_base;
+    float* rewards;            /* [batch] */
+    uint8_t* terminated;       /* [batch] */
+    /* masks of the batch; NULL means all true, which is what gather_batch yields for SEQUENCE_LENGTH = 1 */
+    const uint8_t* final_step_mask;        /* [batch] */
+    const uint8_t* next_final_step_mask;   /* [batch] */
+    const uint8_t* reset;                  /* [batch] */
+    /* training buffers */
+    float* next_state_action_value_input;   /* [batch x (obs+act)] */
+    float* next_q[2];                        /* [batch] each */
+    float* next_log_probabilities;           /* [batch] */
+    float* target_action_value;              /* [batch] */
+    float* d_output_critic[2];               /* [batch] */
+    float* state_action_value_input;         /* [batch x (obs+act)] (actor training) */
+    float* d_output_actor_critics;           /* [batch] */
+    float* d_critic_input[2];                /* [batch x (obs+act)] */
+    float* d_actor_output_squashing;         /* [batch x act] */
+    float* d_actor_output;                   /* [batch x 2*act] */
+    float* actor_pre_squashing;              /* [batch x act] */
+    float* actor_log_probabilities;          /* [batch] */
+    float* actor_actions;                    /* [batch x act] (sample_and_squash layer output) */
+    void* workspace; size_t workspace_bytes;
+} rlt_sac_agent;
+
+/* train_critic            rl/algorithms/sac/operations_generic.h:243-337 for critic `critic_index`;
+ *   action_noise [batch x action_dim] is the externally drawn N(0,1) noise. */
+int rlt_rocm_sac_train_critic(rlt_rocm_device* device, const rlt_sac_agent* agent, int critic_index,
+                              const float* action_noise);
+/* update_critic_targets   sac/operations_generic.h:488-527 */
+int rlt_rocm_sac_update_critic_targets(rlt_rocm_device* device, const rlt_sac_agent* agent);
+/* train_actor             sac/operations_generic.h:395-468 */
+int rlt_rocm_sac_train_actor(rlt_rocm_device* device, const rlt_sac_agent* agent, const float* action_noise);
+
+/* ------------------------------------------------- replay buffer / runner -- */
+
+/* Replay storage of one off-policy runner (rl/components/replay_buffer/replay_buffer.h:32-62):
+ * the reference keeps one ring per environment; here the rings of all environments live in one
+ * allocation, ring e at rows [e*capacity, (e+1)*capacity). Row layout (floats):
+ * [obs | action | reward | next_obs | terminated | truncated], row_dim = 2*obs + act + 3. */
+typedef struct rlt_replay_buffer {
+    float* data;              /* [n_envs*capacity x row_dim]                 */
+    uint32_t* episode_start;  /* [n_envs*capacity]                           */
+    uint32_t* position;       /* [n_envs] device-resident ring cursors       */
+    uint32_t* current_episode_start; /* [n_envs]                             */
+    uint8_t* full;            /* [n_envs]                                    */
+    int32_t n_envs, capacity, observation_dim, action_dim;
+} rlt_replay_buffer;
+
+/* add                     replay_buffer/operations_generic.h:54-78, one transition per environment:
+ *   observations/next_observations [n_envs x obs], actions [n_envs x act], rewards [n_envs],
+ *   terminated/truncated [n_envs]. Advances every ring cursor on the device. */
+int rlt_rocm_replay_add(rlt_rocm_device* device, const rlt_replay_buffer* rb,
+                        const float* observations, const float* actions, const float* rewards,
+                        const float* next_observations, const uint8_t* terminated, const uint8_t* truncated);
+
+/* gather_batch (SEQUENCE_LENGTH = 1)   off_policy_runner/operations_generic.h:240-430, operations_cuda.h:37-55,170-181
+ *   env_indices[i], sample_offsets[i]: the two draws the reference makes per sample (host-drawn and copied
+ *   for parity, or produced by rlt_rocm_gather_draw). deterministic != 0 uses offset = i, env = 0
+ *   (the reference's DETERMINISTIC template flag). max_episode_length enters the ring-wrap index
+ *   (position + max_episode_length + offset) % capacity once a ring is full.
+ *   Outputs: observations_actions_base [2 x batch x (obs+act)], rewards [batch], terminated [batch],
+ *   and the masks (reset, next_reset_base[2 x batch], final_step_mask, next_final_step_mask_base[2 x batch];
+ *   any may be NULL). */
+int rlt_rocm_gather_batch(rlt_rocm_device* device, const rlt_replay_buffer* rb,
+                          const uint32_t* env_indices, const uint32_t* sample_offsets, int deterministic,
+                          int max_episode_length, int batch,
+                          float* observations_actions_base, float* rewards, uint8_t* terminated,
+                          uint8_t* reset, uint8_t* next_reset_base, uint8_t* final_step_mask, uint8_t* next_final_step_mask_base);
+/* Device-side draw of (env, offset) pairs, uniform over the eligible rows of each ring
+ * (off_policy_runner/operations_generic.h:257,304,426). */
+int rlt_rocm_gather_draw(rlt_rocm_device* device, const rlt_replay_buffer* rb, int batch,
+                         uint64_t seed, uint64_t offset, uint32_t* env_indices, uint32_t* sample_offsets);
+
+/* rl/environments/pendulum/pendulum.h:12-25 */
+typedef struct rlt_pendulum_parameters {
+    float g, max_speed, max_torque, dt, m, l;
+} rlt_pendulum_parameters;
+
+/* step + reward + observe  rl/environments/pendulum/operations_generic.h:79-101,131-160
+ *   states [n_envs x 2] = (theta, theta_dot) updated in place; actions [n_envs] (un-clamped);
+ *   observations (pre-step) and next_observations [n_envs x 3]; rewards [n_envs]. */
+int rlt_rocm_pendulum_step(rlt_rocm_device* device, const rlt_pendulum_parameters* p, float* states,
+                           const float* actions, float* observations, float* next_observations,
+                           float* rewards, int n_envs);
+
+/* Per-environment runner state (rl/components/off_policy_runner/off_policy_runner.h:184-221). */
+typedef struct rlt_pendulum_runner {
+    float* states;            /* [n_envs x 2]  */
+    uint32_t* episode_step;   /* [n_envs]      */
+    float* episode_return;    /* [n_envs]      */
+    uint8_t* truncated;       /* [n_envs] initialised to 1 */
+    int32_t n_envs, episode_step_limit;
+    rlt_pendulum_parameters env;
+} rlt_pendulum_runner;
+
+/* One off-policy runner step for all environments in a single launch
+ * (prologue/interlude/epilogue, off_policy_runner/operations_generic.h:183-238, _per_env.h:8-108,
+ * operations_cuda.h:60-203): reset-if-truncated from `initial_states` [n_envs x 2] (consumed only where a
+ * reset happens; may be NULL to re-draw on the device from (seed, offset)), observe, deterministic
+ * tanh/identity actor MLP or tanh-Gaussian actor with `action_noise` [n_envs x act], env step, reward,
+ * next observation, truncation, and the replay `add`.
+ *   policy_kind: 0 = actions given in `actions_in` (e.g. uniform warm-up policy drawn by the host)
+ *                1 = MLP whose output IS the action (e.g. 3->64->64->1 tanh)
+ *                2 = MLP [mean | log_std] followed by sample_and_squash with action_noise */
+int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_runner* runner,
+                                  const rlt_replay_buffer* rb, int policy_kind,
+                                  const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas,
+                                  const float* actions_in, const float* action_noise,
+                                  const float* initial_states, uint64_t seed, uint64_t offset);
+
+/* --------------------------------------------------------------------- PPO -- */
+
+/* estimate_generalized_advantages   rl/algorithms/ppo/operations_generic.h:60-95
+ *   rows are step-major: row = step*n_envs + env (on_policy_runner.h:38-72); every column is passed
+ *   with the dataset's row stride `ld` (floats), flags are floats as in the reference dataset.
+ *   all_values has (steps+1)*n_envs rows (the last n_envs rows bootstrap). */
+int rlt_rocm_ppo_gae(rlt_rocm_device* device, const float* rewards, const float* terminated, const float* truncated,
+                     const float* all_values, float* advantages, float* target_values, int ld,
+                     int n_envs, int steps, float gamma, float lambda, int ignore_termination);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RLT_ROCM_H */

@@ -1,0 +1,760 @@
+// CPU restatement of the reference algorithms (test infrastructure only, see rlt_oracle.h).
+// Reference paths are relative to /root/reference/include/rl_tools/.
+#include "rlt_oracle.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <dlfcn.h>
+#include <vector>
+
+namespace {
+
+bool g_f64_accumulate = false;
+
+// ---- optional CBLAS provider (the reference's CPU_BLAS device calls cblas_sgemm, devices/cpu_openblas.h:9-27)
+enum { ORC_ROW_MAJOR = 101, ORC_NO_TRANS = 111, ORC_TRANS = 112 };
+typedef void (*sgemm_fn)(int, int, int, int, int, int, float, const float*, int, const float*, int, float, float*, int);
+sgemm_fn g_sgemm = nullptr;
+char g_cblas_name[512] = "loops";
+
+inline float dotf(const float* a, int sa, const float* b, int sb, int n, float init) {
+    if (g_f64_accumulate) {
+        double acc = init;
+        for (int i = 0; i < n; i++) acc += (double)a[(size_t)i * sa] * (double)b[(size_t)i * sb];
+        return (float)acc;
+    }
+    float acc = init;
+    for (int i = 0; i < n; i++) acc += a[(size_t)i * sa] * b[(size_t)i * sb];
+    return acc;
+}
+
+// math/operations_generic.h:247-251
+inline float fast_tanh(float x) {
+    x = x < -3.0f ? -3.0f : (x > 3.0f ? 3.0f : x);
+    float x2 = x * x;
+    return x * (27 + x2) / (27 + 9 * x2);
+}
+
+// random/operations_generic.h:72-105
+inline float normal_log_prob(float mean, float log_std, float value) {
+    // the reference writes the literals -0.5 and 0.5 as doubles, so the last term and the final subtraction are
+    // evaluated in double and rounded once on return
+    float neg_log_sqrt_pi = (float)(-0.5 * std::log(2 * (float)M_PI));
+    float diff = value - mean;
+    float sd = std::exp(log_std);
+    float pre_square = diff / sd;
+    return (float)((neg_log_sqrt_pi - log_std) - 0.5 * pre_square * pre_square);
+}
+inline float normal_d_log_prob_d_mean(float mean, float log_std, float value) {
+    float diff = value - mean;
+    float sd = std::exp(log_std);
+    float pre_square = diff / sd;
+    return pre_square / sd;
+}
+inline float normal_d_log_prob_d_log_std(float mean, float log_std, float value) {
+    float diff = value - mean;
+    float sd = std::exp(log_std);
+    float pre_square = diff / sd;
+    return -1 + pre_square * pre_square;
+}
+inline float normal_d_log_prob_d_sample(float mean, float log_std, float value) {
+    float diff = value - mean;
+    float sd = std::exp(log_std);
+    float pre_square = diff / sd;
+    return -pre_square / sd;
+}
+inline float clampf(float x, float lo, float hi) { return x < lo ? lo : (x > hi ? hi : x); }
+
+}  // namespace
+
+extern "C" {
+
+void rlt_oracle_set_f64_accumulate(int enabled) { g_f64_accumulate = enabled != 0; }
+
+int rlt_oracle_use_cblas(const char* library_path) {
+    if (!library_path) { g_sgemm = nullptr; std::snprintf(g_cblas_name, sizeof g_cblas_name, "loops"); return 0; }
+    void* h = dlopen(library_path, RTLD_NOW | RTLD_LOCAL);
+    if (!h) return 1;
+    void* f = dlsym(h, "cblas_sgemm");
+    if (!f) f = dlsym(h, "scipy_cblas_sgemm");
+    if (!f) return 2;
+    // single thread, as the reference's OpenBLAS device demands (devices/cpu_openblas.h:31-47)
+    typedef void (*set_threads_fn)(int);
+    const char* setters[] = {"openblas_set_num_threads", "scipy_openblas_set_num_threads", "MKL_Set_Num_Threads"};
+    for (const char* s : setters) { if (void* st = dlsym(h, s)) { ((set_threads_fn)st)(1); break; } }
+    g_sgemm = (sgemm_fn)f;
+    std::snprintf(g_cblas_name, sizeof g_cblas_name, "%s", library_path);
+    return 0;
+}
+const char* rlt_oracle_cblas_name(void) { return g_cblas_name; }
+
+// nn/activation_functions.h:25-55
+float rlt_oracle_activation(float x, int f) {
+    switch (f) {
+        case RLT_ACT_IDENTITY: return x;
+        case RLT_ACT_RELU: return x > 0 ? x : 0;
+        case RLT_ACT_GELU: { const float a = (float)(M_2_SQRTPI * M_SQRT1_2 * 0.5); return 0.5f * (x + x * std::tanh(a * (0.044715f * x * x * x + x))); }
+        case RLT_ACT_TANH: return std::tanh(x);
+        case RLT_ACT_FAST_TANH: return fast_tanh(x);
+        case RLT_ACT_SIGMOID: return 1.0f / (1.0f + std::exp(-x));
+    }
+    return 0;
+}
+// nn/activation_functions.h:57-90
+float rlt_oracle_d_activation(float x, int f) {
+    switch (f) {
+        case RLT_ACT_IDENTITY: return 1;
+        case RLT_ACT_RELU: return x > 0 ? 1 : 0;
+        case RLT_ACT_GELU: {
+            const float a = (float)(M_2_SQRTPI * M_SQRT1_2 * 0.5); const float b = 0.044715f;
+            float t = std::tanh(a * (b * x * x * x + x));
+            return 0.5f * (1 + t) + 0.5f * x * (1 - t * t) * a * (3 * b * x * x + 1);
+        }
+        case RLT_ACT_TANH: { float a = std::tanh(x); return 1 - a * a; }
+        case RLT_ACT_FAST_TANH: { float a = fast_tanh(x); return 1 - a * a; }
+        case RLT_ACT_SIGMOID: { float s = rlt_oracle_activation(x, RLT_ACT_SIGMOID); return s * (1 - s); }
+    }
+    return 0;
+}
+
+// nn/layers/dense/operations_generic.h:95-138 (loops) / operations_cpu_blas.h:36-116 (bias broadcast, sgemm beta=1,
+// copy to pre_activations, activation loop)
+static int dense_forward_impl(const rlt_dense_layer* L, const float* x, int ldx, float* y, int ldy, int batch, bool store) {
+    if (!L || !x || batch <= 0 || L->in_dim <= 0 || L->out_dim <= 0 || ldx < L->in_dim) return RLT_E_INVALID_ARGUMENT;
+    if (y && ldy < L->out_dim) return RLT_E_INVALID_ARGUMENT;
+    const int I = L->in_dim, O = L->out_dim;
+    std::vector<float> tmp;
+    float* acc = nullptr; int lda = O;
+    if (g_sgemm) {
+        tmp.resize((size_t)batch * O);
+        acc = tmp.data();
+        for (int b = 0; b < batch; b++) for (int o = 0; o < O; o++) acc[(size_t)b * O + o] = L->biases[o];
+        g_sgemm(ORC_ROW_MAJOR, ORC_NO_TRANS, ORC_TRANS, batch, O, I, 1.0f, x, ldx, L->weights, I, 1.0f, acc, lda);
+    }
+    for (int b = 0; b < batch; b++) {
+        for (int o = 0; o < O; o++) {
+            float pre = acc ? acc[(size_t)b * O + o] : dotf(L->weights + (size_t)o * I, 1, x + (size_t)b * ldx, 1, I, L->biases[o]);
+            float out = rlt_oracle_activation(pre, L->activation);
+            if (store && L->pre_activations) L->pre_activations[(size_t)b * O + o] = pre;
+            if (store && L->output) L->output[(size_t)b * O + o] = out;
+            if (y) y[(size_t)b * ldy + o] = out;
+        }
+    }
+    return 0;
+}
+int rlt_oracle_dense_evaluate(const rlt_dense_layer* L, const float* x, int ldx, float* y, int ldy, int batch) {
+    if (!y) return RLT_E_INVALID_ARGUMENT;
+    return dense_forward_impl(L, x, ldx, y, ldy, batch, false);
+}
+int rlt_oracle_dense_forward(const rlt_dense_layer* L, const float* x, int ldx, float* y, int ldy, int batch) {
+    if (!L || !L->pre_activations) return RLT_E_INVALID_ARGUMENT;
+    return dense_forward_impl(L, x, ldx, y, ldy, batch, true);
+}
+
+// operations_cpu_blas.h:119-141 backward_pre_activations (in place) ; with_bias: the fused loop of :165-171
+static void d_pre_inplace(const rlt_dense_layer* L, float* d_output, int ldd, int batch, bool with_bias) {
+    const int O = L->out_dim;
+    for (int b = 0; b < batch; b++) {
+        for (int o = 0; o < O; o++) {
+            float d_pre = rlt_oracle_d_activation(L->pre_activations[(size_t)b * O + o], L->activation) * d_output[(size_t)b * ldd + o];
+            if (with_bias) L->d_biases[o] += d_pre;
+            d_output[(size_t)b * ldd + o] = d_pre;
+        }
+    }
+}
+// operations_cpu_blas.h:188-218 : d_input = d_pre W (beta = 0)
+static void d_input_from_d_pre(const rlt_dense_layer* L, const float* d_pre, int ldd, float* d_input, int ldi, int batch) {
+    const int I = L->in_dim, O = L->out_dim;
+    if (g_sgemm) { g_sgemm(ORC_ROW_MAJOR, ORC_NO_TRANS, ORC_NO_TRANS, batch, I, O, 1.0f, d_pre, ldd, L->weights, I, 0.0f, d_input, ldi); return; }
+    for (int b = 0; b < batch; b++)
+        for (int i = 0; i < I; i++)
+            d_input[(size_t)b * ldi + i] = dotf(d_pre + (size_t)b * ldd, 1, L->weights + i, I, O, 0.0f);
+}
+// operations_cpu_blas.h:173-185 : d_weights += d_pre^T x (beta = 1)
+static void d_weights_accumulate(const rlt_dense_layer* L, const float* x, int ldx, const float* d_pre, int ldd, int batch) {
+    const int I = L->in_dim, O = L->out_dim;
+    if (g_sgemm) { g_sgemm(ORC_ROW_MAJOR, ORC_TRANS, ORC_NO_TRANS, O, I, batch, 1.0f, d_pre, ldd, x, ldx, 1.0f, L->d_weights, I); return; }
+    for (int o = 0; o < O; o++)
+        for (int i = 0; i < I; i++)
+            L->d_weights[(size_t)o * I + i] = dotf(d_pre + o, ldd, x + i, ldx, batch, L->d_weights[(size_t)o * I + i]);
+}
+int rlt_oracle_dense_backward_input(const rlt_dense_layer* L, float* d_output, int ldd, float* d_input, int ldi, int batch) {
+    if (!L || !L->pre_activations || !d_output || !d_input || batch <= 0 || ldd < L->out_dim || ldi < L->in_dim) return RLT_E_INVALID_ARGUMENT;
+    d_pre_inplace(L, d_output, ldd, batch, false);
+    d_input_from_d_pre(L, d_output, ldd, d_input, ldi, batch);
+    return 0;
+}
+int rlt_oracle_dense_backward(const rlt_dense_layer* L, const float* x, int ldx, float* d_output, int ldd, int batch) {
+    if (!L || !L->pre_activations || !L->d_weights || !L->d_biases || !x || !d_output || batch <= 0 || ldd < L->out_dim || ldx < L->in_dim) return RLT_E_INVALID_ARGUMENT;
+    d_pre_inplace(L, d_output, ldd, batch, true);
+    d_weights_accumulate(L, x, ldx, d_output, ldd, batch);
+    return 0;
+}
+int rlt_oracle_dense_backward_full(const rlt_dense_layer* L, const float* x, int ldx, float* d_output, int ldd, float* d_input, int ldi, int batch) {
+    int rc = rlt_oracle_dense_backward(L, x, ldx, d_output, ldd, batch);
+    if (rc) return rc;
+    if (!d_input || ldi < L->in_dim) return RLT_E_INVALID_ARGUMENT;
+    d_input_from_d_pre(L, d_output, ldd, d_input, ldi, batch);
+    return 0;
+}
+
+static int max_hidden(const rlt_dense_layer* layers, int n) { int m = 1; for (int i = 0; i + 1 < n; i++) if (layers[i].out_dim > m) m = layers[i].out_dim; return m; }
+
+// nn_models/mlp/operations_generic.h:77-102
+int rlt_oracle_mlp_evaluate(const rlt_dense_layer* layers, int n, const float* x, int ldx, float* y, int ldy, int batch) {
+    if (!layers || n < 1 || !x || !y || batch <= 0) return RLT_E_INVALID_ARGUMENT;
+    int H = max_hidden(layers, n);
+    std::vector<float> tick((size_t)batch * H), tock((size_t)batch * H);
+    const float* in = x; int ldin = ldx;
+    for (int l = 0; l < n; l++) {
+        float* out = (l == n - 1) ? y : ((l % 2 == 0) ? tick.data() : tock.data());
+        int ldo = (l == n - 1) ? ldy : layers[l].out_dim;
+        int rc = rlt_oracle_dense_evaluate(&layers[l], in, ldin, out, ldo, batch);
+        if (rc) return rc;
+        in = out; ldin = ldo;
+    }
+    return 0;
+}
+// nn_models/mlp/operations_generic.h:103-114
+int rlt_oracle_mlp_forward(const rlt_dense_layer* layers, int n, const float* x, int ldx, int batch) {
+    if (!layers || n < 1 || !x || batch <= 0) return RLT_E_INVALID_ARGUMENT;
+    const float* in = x; int ldin = ldx;
+    for (int l = 0; l < n; l++) {
+        if (!layers[l].output) return RLT_E_INVALID_ARGUMENT;
+        int rc = rlt_oracle_dense_forward(&layers[l], in, ldin, nullptr, 0, batch);
+        if (rc) return rc;
+        in = layers[l].output; ldin = layers[l].out_dim;
+    }
+    return 0;
+}
+// nn_models/mlp/operations_generic.h:126-204: output and hidden layers backward_full (or backward_input), the input layer
+// only produces d_input when asked for (backward_full / backward_input)
+int rlt_oracle_mlp_backward(const rlt_dense_layer* layers, int n, const float* x, int ldx, float* d_output, int ldd,
+                            float* d_input, int ldi, int batch, int want_w) {
+    if (!layers || n < 1 || !d_output || batch <= 0) return RLT_E_INVALID_ARGUMENT;
+    if (want_w && !x) return RLT_E_INVALID_ARGUMENT;
+    int H = max_hidden(layers, n);
+    std::vector<float> tick((size_t)batch * H), tock((size_t)batch * H);
+    float* d_out = d_output; int ld_out = ldd;
+    for (int l = n - 1; l >= 0; l--) {
+        const float* in = (l == 0) ? x : layers[l - 1].output; int ldin = (l == 0) ? ldx : layers[l - 1].out_dim;
+        float* d_in; int ld_in;
+        if (l == 0) { d_in = d_input; ld_in = ldi; }
+        else { d_in = ((n - 1 - l) % 2 == 0) ? tick.data() : tock.data(); ld_in = layers[l].in_dim; }
+        int rc;
+        if (want_w) {
+            if (l > 0 && !in) return RLT_E_INVALID_ARGUMENT;
+            rc = d_in ? rlt_oracle_dense_backward_full(&layers[l], in, ldin, d_out, ld_out, d_in, ld_in, batch)
+                      : rlt_oracle_dense_backward(&layers[l], in, ldin, d_out, ld_out, batch);
+        } else {
+            if (!d_in) return RLT_E_INVALID_ARGUMENT;
+            rc = rlt_oracle_dense_backward_input(&layers[l], d_out, ld_out, d_in, ld_in, batch);
+        }
+        if (rc) return rc;
+        d_out = d_in; ld_out = ld_in;
+    }
+    return 0;
+}
+// nn_models/mlp/operations_generic.h:117-124
+int rlt_oracle_mlp_zero_gradient(const rlt_dense_layer* layers, int n) {
+    for (int l = 0; l < n; l++) {
+        if (!layers[l].d_weights || !layers[l].d_biases) return RLT_E_INVALID_ARGUMENT;
+        std::memset(layers[l].d_weights, 0, sizeof(float) * (size_t)layers[l].in_dim * layers[l].out_dim);
+        std::memset(layers[l].d_biases, 0, sizeof(float) * (size_t)layers[l].out_dim);
+    }
+    return 0;
+}
+// forward (mlp :103-114) + optional mse::gradient (mse/operations_generic.h:41-56) + backward (mlp :180-204),
+// with private activation storage so the caller's layers are left untouched.
+int rlt_oracle_mlp_forward_backward(const rlt_dense_layer* layers, int n, const float* x, int ldx, float* y, int ldy,
+                                    const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch) {
+    if (!layers || n < 1 || !x || batch <= 0 || (!d_output && !target)) return RLT_E_INVALID_ARGUMENT;
+    std::vector<rlt_dense_layer> priv(layers, layers + n);
+    std::vector<std::vector<float>> pre(n), out(n);
+    for (int l = 0; l < n; l++) {
+        pre[l].resize((size_t)batch * layers[l].out_dim); out[l].resize((size_t)batch * layers[l].out_dim);
+        priv[l].pre_activations = pre[l].data(); priv[l].output = out[l].data();
+    }
+    int rc = rlt_oracle_mlp_forward(priv.data(), n, x, ldx, batch);
+    if (rc) return rc;
+    const int O = layers[n - 1].out_dim;
+    std::vector<float> d((size_t)batch * O);
+    for (int b = 0; b < batch; b++)
+        for (int o = 0; o < O; o++) {
+            float yv = out[n - 1][(size_t)b * O + o];
+            if (y) y[(size_t)b * ldy + o] = yv;
+            d[(size_t)b * O + o] = target ? (yv - target[(size_t)b * ldt + o]) * mse_scale : d_output[(size_t)b * ldd + o];
+        }
+    return rlt_oracle_mlp_backward(priv.data(), n, x, ldx, d.data(), O, nullptr, 0, batch, 1);
+}
+
+// nn/optimizers/adam/operations_generic.h:49-66 (_step: bias corrections from age, then age++) and
+// instance/operations_generic.h:26-72 (moments via utils/polyak, then gradient_descent)
+int rlt_oracle_adam_step(const rlt_adam_tensor* tensors, int n_tensors, const rlt_adam_parameters* p, uint32_t* age,
+                         float polyak, float* out_sq_norm) {
+    if (!tensors || n_tensors < 0 || !p || !age) return RLT_E_INVALID_ARGUMENT;
+    float bc1 = 1 / (1 - std::pow(p->beta_1, (float)*age));
+    float bc2 = 1 / (1 - std::pow(p->beta_2, (float)*age));
+    *age += 1;
+    double sq = 0;
+    for (int t = 0; t < n_tensors; t++) {
+        const rlt_adam_tensor& T = tensors[t];
+        if (!T.parameters || !T.gradient || !T.first_moment || !T.second_moment) return RLT_E_INVALID_ARGUMENT;
+        for (uint32_t i = 0; i < T.count; i++) {
+            float g = T.gradient[i];
+            sq += (double)g * g;
+            if (p->enable_gradient_clipping) g = clampf(g, -p->gradient_clip_value, p->gradient_clip_value);
+            float m = p->beta_1 * T.first_moment[i] + (1 - p->beta_1) * g;          // utils/polyak/operations_generic.h:11-24
+            float v = p->beta_2 * T.second_moment[i] + (1 - p->beta_2) * g * g;     // :27-41
+            T.first_moment[i] = m; T.second_moment[i] = v;
+            float pre_sqrt = v * bc2;
+            pre_sqrt = pre_sqrt > p->epsilon_sqrt ? pre_sqrt : p->epsilon_sqrt;
+            float update = p->alpha * bc1 * m / (std::sqrt(pre_sqrt) + p->epsilon);
+            if ((T.flags & 2u) && p->enable_bias_lr_factor) update *= p->bias_lr_factor;
+            if ((T.flags & 1u) && p->enable_weight_decay) update += T.parameters[i] * p->weight_decay / 2;
+            float value = T.parameters[i] - update;
+            T.parameters[i] = value;
+            if (T.polyak_target) T.polyak_target[i] = polyak * T.polyak_target[i] + (1 - polyak) * value;
+        }
+    }
+    if (out_sq_norm) *out_sq_norm = (float)sq;
+    return 0;
+}
+// adam/operations_generic.h:43-47 + instance/operations_generic.h:65-69
+int rlt_oracle_adam_reset(const rlt_adam_tensor* tensors, int n_tensors, uint32_t* age) {
+    if (!tensors || !age) return RLT_E_INVALID_ARGUMENT;
+    *age = 1;
+    for (int t = 0; t < n_tensors; t++) {
+        std::memset(tensors[t].first_moment, 0, sizeof(float) * tensors[t].count);
+        std::memset(tensors[t].second_moment, 0, sizeof(float) * tensors[t].count);
+    }
+    return 0;
+}
+// utils/polyak/operations_generic.h:11-43
+int rlt_oracle_polyak_update(const float* source, float* target, size_t count, float polyak, int squared) {
+    if (!source || !target) return RLT_E_INVALID_ARGUMENT;
+    for (size_t i = 0; i < count; i++) {
+        float s = source[i];
+        target[i] = squared ? polyak * target[i] + (1 - polyak) * s * s : polyak * target[i] + (1 - polyak) * s;
+    }
+    return 0;
+}
+
+// nn/loss_functions/mse/operations_generic.h:41-56,73-87
+int rlt_oracle_mse_gradient(const float* a, int lda, const float* b, int ldb, float* d_a, int ldda, int rows, int cols,
+                            float loss_weight, const float* loss_weight_ptr) {
+    if (!a || !b || !d_a || rows <= 0 || cols <= 0) return RLT_E_INVALID_ARGUMENT;
+    float w = loss_weight_ptr ? *loss_weight_ptr : loss_weight;
+    float constant = (float)2 / ((float)rows * cols) * w;
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) {
+            float diff = a[(size_t)r * lda + c] - b[(size_t)r * ldb + c];
+            d_a[(size_t)r * ldda + c] = diff * constant;
+        }
+    return 0;
+}
+// mse/operations_generic.h:9-21
+int rlt_oracle_mse_evaluate(const float* a, int lda, const float* b, int ldb, int rows, int cols, float loss_weight, float* out_loss) {
+    if (!a || !b || !out_loss || rows <= 0 || cols <= 0) return RLT_E_INVALID_ARGUMENT;
+    float acc = 0;
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) {
+            float diff = a[(size_t)r * lda + c] - b[(size_t)r * ldb + c];
+            acc += diff * diff;
+        }
+    *out_loss = acc * loss_weight / (rows * cols);
+    return 0;
+}
+
+// nn/layers/sample_and_squash/operations_generic.h:148-261
+int rlt_oracle_sas_forward(const rlt_sas_parameters* p, const float* input, int ldin, const float* noise, int ldn,
+                           float* actions, int lda, float* pre_squashing, int ldp, float* log_probabilities, int batch, int dim) {
+    if (!p || !input || !actions || !log_probabilities || batch <= 0 || dim <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int r = 0; r < batch; r++) {
+        float log_prob = 0;
+        for (int c = 0; c < dim; c++) {
+            float mean = input[(size_t)r * ldin + c];
+            float log_std = input[(size_t)r * ldin + dim + c];
+            float log_std_clipped = clampf(log_std, p->log_std_lower_bound, p->log_std_upper_bound);
+            float sd = std::exp(log_std_clipped);
+            float eps = noise ? noise[(size_t)r * ldn + c] : 0.0f;
+            float sample = noise ? mean + eps * sd : mean;
+            if (pre_squashing) pre_squashing[(size_t)r * ldp + c] = sample;
+            float squashed = std::tanh(sample);
+            actions[(size_t)r * lda + c] = squashed;
+            float one_minus_square_plus_eps = (1 - squashed * squashed + p->log_probability_epsilon);
+            log_prob += normal_log_prob(mean, log_std_clipped, sample) - std::log(one_minus_square_plus_eps);
+        }
+        log_probabilities[r] = log_prob;
+    }
+    return 0;
+}
+// nn/layers/sample_and_squash/operations_generic.h:289-398
+int rlt_oracle_sas_backward(const rlt_sas_parameters* p, const float* input, int ldin, const float* noise, int ldn,
+                            const float* actions, int lda, const float* pre_squashing, int ldp,
+                            const float* d_output, int lddo, float* d_input, int lddi,
+                            const float* log_alpha, float* d_log_alpha, int batch, int dim) {
+    if (!p || !input || !noise || !actions || !pre_squashing || !d_output || !d_input || !log_alpha || batch <= 0 || dim <= 0) return RLT_E_INVALID_ARGUMENT;
+    float alpha = std::exp(*log_alpha);
+    float d_log_alpha_sum = 0;
+    for (int b = 0; b < batch; b++) {
+        float entropy = 0;
+        for (int a = 0; a < dim; a++) {
+            float action = actions[(size_t)b * lda + a];
+            float d_output_value = d_output[(size_t)b * lddo + a];
+            float d_tanh_pre_activation = d_output_value * (1 - action * action);
+            float d_mu = d_tanh_pre_activation;
+            float eps = noise[(size_t)b * ldn + a];
+            float d_std = d_tanh_pre_activation * eps;
+            float log_std_pre_clamp = input[(size_t)b * ldin + dim + a];
+            float log_std_clamped = clampf(log_std_pre_clamp, p->log_std_lower_bound, p->log_std_upper_bound);
+            float sd = std::exp(log_std_clamped);
+            float d_log_std_clamped = sd * d_std;
+            float mu = input[(size_t)b * ldin + a];
+            float action_sample = pre_squashing[(size_t)b * ldp + a];
+            float dlp_dmean = normal_d_log_prob_d_mean(mu, log_std_clamped, action_sample);
+            float dlp_dsample = normal_d_log_prob_d_sample(mu, log_std_clamped, action_sample);
+            d_mu += alpha / batch * (dlp_dmean + dlp_dsample + 2 * action);
+            float dlp_dlogstd = normal_d_log_prob_d_log_std(mu, log_std_clamped, action_sample);
+            d_log_std_clamped += alpha / batch * (dlp_dlogstd + dlp_dsample * eps * sd + 2 * action * eps * sd);
+            float d_log_std = (log_std_pre_clamp < p->log_std_lower_bound || log_std_pre_clamp > p->log_std_upper_bound) ? 0 : d_log_std_clamped;
+            d_input[(size_t)b * lddi + a] = d_mu;
+            d_input[(size_t)b * lddi + dim + a] = d_log_std;
+            float one_minus_action_square_plus_eps = (1 - action * action + p->log_probability_epsilon);
+            float action_log_prob = normal_log_prob(mu, log_std_clamped, action_sample) - std::log(one_minus_action_square_plus_eps);
+            entropy += -action_log_prob;
+        }
+        float d_alpha = entropy - p->target_entropy;
+        d_log_alpha_sum += alpha * d_alpha;
+    }
+    if (d_log_alpha) *d_log_alpha += d_log_alpha_sum / batch;
+    return 0;
+}
+
+// rl/algorithms/sac/operations_generic.h:133-179
+int rlt_oracle_sac_target_action_values(const float* q1, const float* q2, const float* rewards, const uint8_t* terminated,
+                                        const float* next_log_probs, const float* log_alpha, float gamma, int ignore_termination,
+                                        float* target, int batch) {
+    if (!q1 || !q2 || !rewards || !terminated || !next_log_probs || !log_alpha || !target || batch <= 0) return RLT_E_INVALID_ARGUMENT;
+    float alpha = std::exp(*log_alpha);
+    for (int i = 0; i < batch; i++) {
+        float min_q = q1[i] < q2[i] ? q1[i] : q2[i];
+        float entropy_bonus = -alpha * next_log_probs[i];
+        min_q += entropy_bonus;
+        float future_value = (ignore_termination || !terminated[i]) ? gamma * min_q : 0;
+        target[i] = rewards[i] + future_value;
+    }
+    return 0;
+}
+// rl/algorithms/sac/operations_generic.h:358-393
+int rlt_oracle_sac_min_value_d_output(const float* q1, const float* q2, const float* d1, const float* d2, int ld, int critic_input_dim,
+                                      int action_dim, float* d_actor_output, int ldo, int batch) {
+    if (!q1 || !q2 || !d1 || !d2 || !d_actor_output || batch <= 0 || action_dim <= 0 || critic_input_dim < action_dim) return RLT_E_INVALID_ARGUMENT;
+    for (int b = 0; b < batch; b++) {
+        bool first = q1[b] < q2[b];
+        for (int a = 0; a < action_dim; a++) {
+            size_t src = (size_t)b * ld + critic_input_dim - action_dim + a;
+            d_actor_output[(size_t)b * ldo + a] = first ? d1[src] : d2[src];
+        }
+    }
+    return 0;
+}
+// rl/algorithms/sac/operations_generic.h:181-209
+int rlt_oracle_mask_copy(const float* source, int lds, float* target, int ldt, const uint8_t* mask, int invert, int rows, int cols) {
+    if (!source || !target || !mask) return RLT_E_INVALID_ARGUMENT;
+    for (int r = 0; r < rows; r++) {
+        bool m = mask[r] != 0; if (invert) m = !m;
+        if (m) for (int c = 0; c < cols; c++) target[(size_t)r * ldt + c] = source[(size_t)r * lds + c];
+    }
+    return 0;
+}
+// rl/algorithms/sac/operations_generic.h:210-234
+int rlt_oracle_mask_zero(float* gradient, int ld, const uint8_t* mask, int invert, int rows, int cols) {
+    if (!gradient || !mask) return RLT_E_INVALID_ARGUMENT;
+    for (int r = 0; r < rows; r++) {
+        bool m = mask[r] != 0; if (invert) m = !m;
+        if (m) for (int c = 0; c < cols; c++) gradient[(size_t)r * ld + c] = 0;
+    }
+    return 0;
+}
+// containers/tensor/operations_generic.h:433-445
+int rlt_oracle_scale_f32(float* x, size_t count, float s, int reciprocal) {
+    if (!x) return RLT_E_INVALID_ARGUMENT;
+    for (size_t i = 0; i < count; i++) x[i] = reciprocal ? s / x[i] : s * x[i];
+    return 0;
+}
+// containers/tensor/operations_generic.h:928-985 (CastSum)
+int rlt_oracle_cast_reduce_sum_u8(const uint8_t* mask, size_t count, float* out_sum) {
+    if (!mask || !out_sum) return RLT_E_INVALID_ARGUMENT;
+    float acc = 0;
+    for (size_t i = 0; i < count; i++) acc += (float)(mask[i] != 0);
+    *out_sum = acc;
+    return 0;
+}
+
+// --------------------------------------------------------------------------------------------- SAC update steps
+static int adam_over(const rlt_adam_tensor* t, int n, const rlt_adam_parameters* p, uint32_t* age) {
+    return rlt_oracle_adam_step(t, n, p, age, 0.0f, nullptr);
+}
+
+// rl/algorithms/sac/operations_generic.h:243-337 with SEQUENCE_LENGTH = 1
+int rlt_oracle_sac_train_critic(const rlt_sac_agent* A, int ci, const float* action_noise) {
+    if (!A || ci < 0 || ci > 1 || !action_noise) return RLT_E_INVALID_ARGUMENT;
+    const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    const rlt_dense_layer* critic = A->critics[ci];
+    int rc;
+    if ((rc = rlt_oracle_mlp_zero_gradient(critic, A->n_critic_layers))) return rc;                           // :263
+    const float* obs_next = A->observations_actions_base + (size_t)B * D;                                   // padded step 1
+    // actor evaluate on next observations with external noise (:266-273): MLP then sample_and_squash
+    std::vector<float> actor_out((size_t)B * 2 * ACT);
+    if ((rc = rlt_oracle_mlp_evaluate(A->actor, A->n_actor_layers, obs_next, D, actor_out.data(), 2 * ACT, B))) return rc;
+    float* next_actions = A->next_state_action_value_input + OBS;
+    if ((rc = rlt_oracle_sas_forward(&A->sas, actor_out.data(), 2 * ACT, action_noise, ACT, next_actions, D, nullptr, 0, A->next_log_probabilities, B, ACT))) return rc;
+    if (A->next_final_step_mask)                                                                            // :274-277
+        if ((rc = rlt_oracle_mask_copy(obs_next + OBS, D, next_actions, D, A->next_final_step_mask, 1, B, ACT))) return rc;
+    for (int b = 0; b < B; b++) std::memcpy(A->next_state_action_value_input + (size_t)b * D, obs_next + (size_t)b * D, sizeof(float) * OBS); // :278
+    for (int k = 0; k < 2; k++)                                                                             // :283-284
+        if ((rc = rlt_oracle_mlp_evaluate(A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, A->next_q[k], 1, B))) return rc;
+    if ((rc = rlt_oracle_sac_target_action_values(A->next_q[0], A->next_q[1], A->rewards, A->terminated, A->next_log_probabilities,
+                                                 A->log_alpha.parameters, A->gamma, 0, A->target_action_value, B))) return rc;      // :289
+    if ((rc = rlt_oracle_mlp_forward(critic, A->n_critic_layers, A->observations_actions_base, D, B))) return rc;                  // :294
+    const float* q = critic[A->n_critic_layers - 1].output;
+    // :298-306 loss_weight = (SEQ*B*0.5) / num_final_steps
+    float loss_weight = 0;
+    if (A->final_step_mask) rlt_oracle_cast_reduce_sum_u8(A->final_step_mask, B, &loss_weight); else loss_weight = (float)B;
+    rlt_oracle_scale_f32(&loss_weight, 1, 1 * B * 0.5f, 1);
+    float* d_out = A->d_output_critic[ci];
+    if ((rc = rlt_oracle_mse_gradient(q, 1, A->target_action_value, 1, d_out, 1, B, 1, 0, &loss_weight))) return rc;                 // :312
+    if (A->final_step_mask) rlt_oracle_mask_zero(d_out, 1, A->final_step_mask, 1, B, 1);                                          // :314-316
+    std::vector<float> scratch;
+    if ((rc = rlt_oracle_mlp_backward(critic, A->n_critic_layers, A->observations_actions_base, D, d_out, 1, nullptr, 0, B, 1))) return rc; // :329
+    return adam_over(A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci]);                  // :336
+}
+
+// rl/algorithms/sac/operations_generic.h:488-527
+int rlt_oracle_sac_update_critic_targets(const rlt_sac_agent* A) {
+    if (!A) return RLT_E_INVALID_ARGUMENT;
+    for (int k = 0; k < 2; k++)
+        for (int l = 0; l < A->n_critic_layers; l++) {
+            const rlt_dense_layer& s = A->critics[k][l]; const rlt_dense_layer& t = A->critics_target[k][l];
+            rlt_oracle_polyak_update(s.weights, t.weights, (size_t)s.in_dim * s.out_dim, A->polyak, 0);
+            rlt_oracle_polyak_update(s.biases, t.biases, (size_t)s.out_dim, A->polyak, 0);
+        }
+    return 0;
+}
+
+// rl/algorithms/sac/operations_generic.h:395-468 with SEQUENCE_LENGTH = 1
+int rlt_oracle_sac_train_actor(const rlt_sac_agent* A, const float* action_noise) {
+    if (!A || !action_noise) return RLT_E_INVALID_ARGUMENT;
+    const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    int rc;
+    if ((rc = rlt_oracle_mlp_zero_gradient(A->actor, A->n_actor_layers))) return rc;                          // :414
+    A->log_alpha.gradient[0] = 0;   // zero_gradient(actor) also clears the sample_and_squash layer's log_alpha gradient
+    const float* obs = A->observations_actions_base;
+    if ((rc = rlt_oracle_mlp_forward(A->actor, A->n_actor_layers, obs, D, B))) return rc;                     // :427 (MLP part)
+    const float* actor_out = A->actor[A->n_actor_layers - 1].output;
+    if ((rc = rlt_oracle_sas_forward(&A->sas, actor_out, 2 * ACT, action_noise, ACT, A->actor_actions, ACT, A->actor_pre_squashing, ACT,
+                                     A->actor_log_probabilities, B, ACT))) return rc;
+    float* sav_actions = A->state_action_value_input + OBS;
+    for (int b = 0; b < B; b++) std::memcpy(sav_actions + (size_t)b * D, A->actor_actions + (size_t)b * ACT, sizeof(float) * ACT);
+    if (A->final_step_mask)                                                                                 // :428-430
+        if ((rc = rlt_oracle_mask_copy(obs + OBS, D, sav_actions, D, A->final_step_mask, 1, B, ACT))) return rc;
+    for (int b = 0; b < B; b++) std::memcpy(A->state_action_value_input + (size_t)b * D, obs + (size_t)b * D, sizeof(float) * OBS); // :431
+    for (int k = 0; k < 2; k++)                                                                             // :432-433
+        if ((rc = rlt_oracle_mlp_forward(A->critics[k], A->n_critic_layers, A->state_action_value_input, D, B))) return rc;
+    // :437-453 d_output = -1/num_final_steps on final steps
+    float loss_weight = 0;
+    if (A->final_step_mask) rlt_oracle_cast_reduce_sum_u8(A->final_step_mask, B, &loss_weight); else loss_weight = (float)B;
+    rlt_oracle_scale_f32(&loss_weight, 1, -1.0f, 1);
+    std::vector<float> d_out((size_t)B);
+    for (int k = 0; k < 2; k++) {                                                                           // :458-459
+        for (int b = 0; b < B; b++) d_out[b] = loss_weight;
+        if (A->final_step_mask) rlt_oracle_mask_zero(d_out.data(), 1, A->final_step_mask, 1, B, 1);
+        // NOTE the reference reuses ONE d_output tensor for both critics and the first backward_input overwrites it with
+        // d_pre of critic 0's output layer; that layer's activation is IDENTITY, so d_pre == d_output and the second call
+        // sees the same values.
+        if ((rc = rlt_oracle_mlp_backward(A->critics[k], A->n_critic_layers, nullptr, 0, d_out.data(), 1, A->d_critic_input[k], D, B, 0))) return rc;
+    }
+    std::memcpy(A->d_output_actor_critics, d_out.data(), sizeof(float) * B);
+    const float* q1 = A->critics[0][A->n_critic_layers - 1].output; const float* q2 = A->critics[1][A->n_critic_layers - 1].output;
+    if ((rc = rlt_oracle_sac_min_value_d_output(q1, q2, A->d_critic_input[0], A->d_critic_input[1], D, D, ACT, A->d_actor_output_squashing, ACT, B))) return rc; // :460
+    if (A->final_step_mask) rlt_oracle_mask_zero(A->d_actor_output_squashing, ACT, A->final_step_mask, 1, B, ACT);           // :461-463
+    // sequential backward: sample_and_squash backward_full (divides d_log_alpha by num_resets = sum(reset)), then MLP backward (:464)
+    float d_log_alpha_mean = 0;
+    if ((rc = rlt_oracle_sas_backward(&A->sas, actor_out, 2 * ACT, action_noise, ACT, A->actor_actions, ACT, A->actor_pre_squashing, ACT,
+                                      A->d_actor_output_squashing, ACT, A->d_actor_output, 2 * ACT, A->log_alpha.parameters, &d_log_alpha_mean, B, ACT))) return rc;
+    if (A->reset) { float n = 0; rlt_oracle_cast_reduce_sum_u8(A->reset, B, &n); d_log_alpha_mean = d_log_alpha_mean * B / n; }
+    A->log_alpha.gradient[0] += d_log_alpha_mean;
+    if ((rc = rlt_oracle_mlp_backward(A->actor, A->n_actor_layers, obs, D, A->d_actor_output, 2 * ACT, nullptr, 0, B, 1))) return rc;
+    if ((rc = adam_over(A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age))) return rc;                // :465
+    return adam_over(&A->log_alpha, 1, &A->alpha_adam, A->alpha_age);                                                           // :466
+}
+
+// ------------------------------------------------------------------------------ replay buffer, gather, Pendulum
+static inline int rb_row_dim(const rlt_replay_buffer* rb) { return 2 * rb->observation_dim + rb->action_dim + 3; }
+
+// rl/components/replay_buffer/operations_generic.h:54-78, one transition per environment
+int rlt_oracle_replay_add(const rlt_replay_buffer* rb, const float* obs, const float* actions, const float* rewards,
+                          const float* next_obs, const uint8_t* terminated, const uint8_t* truncated) {
+    if (!rb || !rb->data || !obs || !actions || !rewards || !next_obs || !terminated || !truncated) return RLT_E_INVALID_ARGUMENT;
+    const int OBS = rb->observation_dim, ACT = rb->action_dim, R = rb_row_dim(rb);
+    for (int e = 0; e < rb->n_envs; e++) {
+        uint32_t pos = rb->position[e];
+        float* row = rb->data + ((size_t)e * rb->capacity + pos) * R;
+        for (int i = 0; i < OBS; i++) { row[i] = obs[(size_t)e * OBS + i]; row[OBS + ACT + 1 + i] = next_obs[(size_t)e * OBS + i]; }
+        for (int i = 0; i < ACT; i++) row[OBS + i] = actions[(size_t)e * ACT + i];
+        row[OBS + ACT] = rewards[e];
+        row[2 * OBS + ACT + 1] = terminated[e] ? 1.0f : 0.0f;
+        row[2 * OBS + ACT + 2] = truncated[e] ? 1.0f : 0.0f;
+        rb->episode_start[(size_t)e * rb->capacity + pos] = rb->current_episode_start[e];
+        pos = (pos + 1) % (uint32_t)rb->capacity;
+        rb->position[e] = pos;
+        if (truncated[e]) rb->current_episode_start[e] = pos;
+        if (pos == 0 && !rb->full[e]) rb->full[e] = 1;
+    }
+    return 0;
+}
+
+// rl/components/off_policy_runner/operations_generic.h:240-430 with SEQUENCE_LENGTH = 1 (PADDED = 2), no
+// ALWAYS_SAMPLE_FROM_INITIAL_STATE, no RANDOM_SEQ_LENGTH (off_policy_runner.h:79-87 for SEQUENCE_LENGTH == 1)
+int rlt_oracle_gather_batch(const rlt_replay_buffer* rb, const uint32_t* env_indices, const uint32_t* sample_offsets, int deterministic,
+                            int max_episode_length, int batch, float* oab, float* rewards, uint8_t* terminated,
+                            uint8_t* reset, uint8_t* next_reset_base, uint8_t* final_step_mask, uint8_t* next_final_step_mask_base) {
+    if (!rb || !rb->data || batch <= 0 || !oab || !rewards || !terminated) return RLT_E_INVALID_ARGUMENT;
+    if (!deterministic && (!env_indices || !sample_offsets)) return RLT_E_INVALID_ARGUMENT;
+    const int OBS = rb->observation_dim, ACT = rb->action_dim, R = rb_row_dim(rb), D = OBS + ACT;
+    for (int i = 0; i < batch; i++) {
+        uint32_t e = deterministic ? 0u : env_indices[i];
+        if (e >= (uint32_t)rb->n_envs) return RLT_E_INVALID_ARGUMENT;
+        uint32_t offset = deterministic ? (uint32_t)i : sample_offsets[i];
+        uint32_t index = rb->full[e] ? (rb->position[e] + (uint32_t)max_episode_length + offset) % (uint32_t)rb->capacity : offset;   // :305-311
+        if (index >= (uint32_t)rb->capacity) return RLT_E_INVALID_ARGUMENT;
+        const float* row = rb->data + ((size_t)e * rb->capacity + index) * R;
+        float* step0 = oab + (size_t)i * D; float* step1 = oab + ((size_t)batch + i) * D;
+        for (int k = 0; k < OBS; k++) step0[k] = row[k];                       // :322-327
+        for (int k = 0; k < ACT; k++) step0[OBS + k] = row[OBS + k];           // :338-343
+        rewards[i] = row[OBS + ACT];                                           // :346
+        terminated[i] = row[2 * OBS + ACT + 1] != 0.0f;                        // :347
+        // seq_step 0 == PADDED-2 forces truncated (:357-359): next observation into padded step 1, next action zeroed (:392-412)
+        for (int k = 0; k < OBS; k++) step1[k] = row[OBS + ACT + 1 + k];
+        for (int k = 0; k < ACT; k++) step1[OBS + k] = 0;
+        if (reset) reset[i] = 1;                                               // :283,298
+        if (next_reset_base) { next_reset_base[i] = 1; next_reset_base[batch + i] = 1; }   // :284,300 (step 0) and :285 via the offset-1 view (step 1)
+        if (final_step_mask) final_step_mask[i] = 1;                           // :389-391
+        if (next_final_step_mask_base) { next_final_step_mask_base[i] = 0; next_final_step_mask_base[batch + i] = 1; } // :279-280,291
+    }
+    return 0;
+}
+
+// rl/environments/pendulum/operations_generic.h: angle_normalize, step :79-101, reward :131-139, observe :142-160.
+// The literals 3.0, 0.1, 0.001 in the reference are doubles, so those sub-expressions evaluate in double (kept here).
+static inline float angle_normalize(float x) { // pendulum/operations_generic.h f_mod_python + angle_normalize
+    const float PI = (float)M_PI;
+    float a = x + PI, b = 2 * PI;
+    float m = a - b * std::floor(a / b);
+    return m - PI;
+}
+static inline void pendulum_observe(float theta, float theta_dot, float* o) { o[0] = std::cos(theta); o[1] = std::sin(theta); o[2] = theta_dot; }
+static inline void pendulum_dynamics(const rlt_pendulum_parameters* p, float theta, float theta_dot, float action, float* n_theta, float* n_theta_dot, float* reward) {
+    float u_normalised = clampf(action, -1.0f, 1.0f);
+    float u = p->max_torque * u_normalised;
+    u = clampf(u, -p->max_torque, p->max_torque);
+    float newthdot = (float)(theta_dot + (3 * p->g / (2 * p->l) * std::sin(theta) + 3.0 / (p->m * p->l * p->l) * u) * p->dt);
+    newthdot = clampf(newthdot, -p->max_speed, p->max_speed);
+    *n_theta = theta + newthdot * p->dt;
+    *n_theta_dot = newthdot;
+    float angle_norm = angle_normalize(theta);
+    float ur = p->max_torque * action;    // reward uses the un-clamped action
+    float costs = (float)(angle_norm * angle_norm + 0.1 * theta_dot * theta_dot + 0.001 * (ur * ur));
+    *reward = -costs;
+}
+int rlt_oracle_pendulum_step(const rlt_pendulum_parameters* p, float* states, const float* actions, float* observations,
+                             float* next_observations, float* rewards, int n_envs) {
+    if (!p || !states || !actions || n_envs <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int e = 0; e < n_envs; e++) {
+        float th = states[2 * e], thd = states[2 * e + 1], nth, nthd, r;
+        if (observations) pendulum_observe(th, thd, observations + 3 * (size_t)e);
+        pendulum_dynamics(p, th, thd, actions[e], &nth, &nthd, &r);
+        if (next_observations) pendulum_observe(nth, nthd, next_observations + 3 * (size_t)e);
+        if (rewards) rewards[e] = r;
+        states[2 * e] = nth; states[2 * e + 1] = nthd;
+    }
+    return 0;
+}
+
+// off_policy_runner/operations_generic.h:183-238 + operations_generic_per_env.h:8-108 for Pendulum
+int rlt_oracle_pendulum_runner_step(const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, int policy_kind,
+                                    const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas,
+                                    const float* actions_in, const float* action_noise, const float* initial_states) {
+    if (!rn || !rb || rn->n_envs != rb->n_envs || rb->observation_dim != 3 || rb->action_dim != 1) return RLT_E_INVALID_ARGUMENT;
+    const int N = rn->n_envs, R = rb_row_dim(rb);
+    std::vector<float> obs((size_t)N * 3), next_obs((size_t)N * 3), actions(N), rewards(N);
+    std::vector<uint8_t> term(N, 0), trunc(N, 0);
+    // prologue (:8-66): reset where truncated, mark previous replay row truncated, observe
+    for (int e = 0; e < N; e++) {
+        if (rn->truncated[e]) {
+            if (!initial_states) return RLT_E_INVALID_ARGUMENT;
+            rn->states[2 * e] = initial_states[2 * e]; rn->states[2 * e + 1] = initial_states[2 * e + 1];
+            rn->episode_step[e] = 0; rn->episode_return[e] = 0;
+            if (rb->full[e] || rb->position[e] > 0) {
+                uint32_t prev = rb->position[e] == 0 ? (uint32_t)rb->capacity - 1 : rb->position[e] - 1;
+                rb->data[((size_t)e * rb->capacity + prev) * R + (R - 1)] = 1.0f;
+                rb->current_episode_start[e] = rb->position[e];
+            }
+        }
+        pendulum_observe(rn->states[2 * e], rn->states[2 * e + 1], &obs[3 * (size_t)e]);
+    }
+    // interlude (:190-206): policy evaluate_step in Rollout mode
+    int rc = 0;
+    if (policy_kind == 0) { if (!actions_in) return RLT_E_INVALID_ARGUMENT; for (int e = 0; e < N; e++) actions[e] = actions_in[e]; }
+    else if (policy_kind == 1) { rc = rlt_oracle_mlp_evaluate(actor, n_actor_layers, obs.data(), 3, actions.data(), 1, N); }
+    else if (policy_kind == 2) {
+        std::vector<float> out((size_t)N * 2), lp(N);
+        rc = rlt_oracle_mlp_evaluate(actor, n_actor_layers, obs.data(), 3, out.data(), 2, N);
+        if (!rc) rc = rlt_oracle_sas_forward(sas, out.data(), 2, action_noise, 1, actions.data(), 1, nullptr, 0, lp.data(), N, 1);
+    } else return RLT_E_INVALID_ARGUMENT;
+    if (rc) return rc;
+    // epilogue (:67-108)
+    for (int e = 0; e < N; e++) {
+        float nth, nthd, r;
+        pendulum_dynamics(&rn->env, rn->states[2 * e], rn->states[2 * e + 1], actions[e], &nth, &nthd, &r);
+        pendulum_observe(nth, nthd, &next_obs[3 * (size_t)e]);
+        rewards[e] = r;
+        rn->episode_step[e] += 1; rn->episode_return[e] += r;
+        trunc[e] = rn->episode_step[e] == (uint32_t)rn->episode_step_limit;
+        rn->truncated[e] = trunc[e];
+        rn->states[2 * e] = nth; rn->states[2 * e + 1] = nthd;
+    }
+    return rlt_oracle_replay_add(rb, obs.data(), actions.data(), rewards.data(), next_obs.data(), term.data(), trunc.data());
+}
+
+// rl/algorithms/ppo/operations_generic.h:60-95
+int rlt_oracle_ppo_gae(const float* rewards, const float* terminated, const float* truncated, const float* all_values,
+                       float* advantages, float* target_values, int ld, int n_envs, int steps, float gamma, float lambda,
+                       int ignore_termination) {
+    if (!rewards || !terminated || !truncated || !all_values || !advantages || !target_values || ld < 1 || n_envs <= 0 || steps <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int env = 0; env < n_envs; env++) {
+        float previous_value = all_values[((size_t)steps * n_envs + env) * ld];
+        float previous_advantage = 0;
+        for (int sf = 0; sf < steps; sf++) {
+            int sb = steps - 1 - sf;
+            size_t pos = ((size_t)sb * n_envs + env) * ld;
+            bool term = terminated[pos] != 0.0f, trunc = truncated[pos] != 0.0f;
+            float current_step_value = all_values[pos];
+            bool terminated_actual = term && !ignore_termination;
+            float next_step_value = terminated_actual ? 0 : previous_value;
+            float td_error = rewards[pos] + gamma * next_step_value - current_step_value;
+            if (trunc) { if (!term) td_error = 0; previous_advantage = 0; }
+            float advantage = lambda * gamma * previous_advantage + td_error;
+            advantages[pos] = advantage;
+            target_values[pos] = advantage + current_step_value;
+            previous_advantage = advantage;
+            previous_value = current_step_value;
+        }
+    }
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,99 @@
+/*
+ * rlt_oracle.h -- CPU restatement of the reference algorithms of the dense-network training hot path.
+ *
+ * TEST INFRASTRUCTURE ONLY. Nothing shipped may call into this library: it exists so that tests,
+ * the smoke check and the benchmark's cpu_baseline leg can check / time the HIP path against a plain
+ * CPU statement of what the reference computes. Every function cites the reference file:line it follows.
+ *
+ * The entry points mirror include/rlt_rocm.h one to one (same structs, same argument meaning) with
+ * host pointers instead of device pointers and no device handle.
+ *
+ * Pinning status of each function (what, other than this file, fixes its answers):
+ *   dense/mlp forward+backward, adam, polyak, mse, sample_and_squash, sac target/min-q/train_*,
+ *   replay add, gather_batch, pendulum, gae: checked against the reference itself compiled from
+ *   /root/reference (oracle/_ref) and against golden vectors written by it (tests/golden), plus the
+ *   closed-form / finite-difference checks in tests/test_oracle_*.py.
+ */
+#ifndef RLT_ORACLE_H
+#define RLT_ORACLE_H
+#include "../include/rlt_rocm.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* 0: accumulate dot products in fp32 in the reference's loop order (default, the faithful restatement);
+ * 1: accumulate in fp64 and round once (used as ground truth when judging fp32 summation error). */
+void rlt_oracle_set_f64_accumulate(int enabled);
+/* 1: route the three GEMMs of a dense layer through cblas_sgemm of the given shared library
+ * (the reference's CPU_BLAS device does this); 0: plain loops. Returns 0 on success. */
+int rlt_oracle_use_cblas(const char* library_path);
+const char* rlt_oracle_cblas_name(void);
+
+float rlt_oracle_activation(float x, int activation);
+float rlt_oracle_d_activation(float x, int activation);
+
+int rlt_oracle_dense_evaluate(const rlt_dense_layer* layer, const float* x, int ldx, float* y, int ldy, int batch);
+int rlt_oracle_dense_forward(const rlt_dense_layer* layer, const float* x, int ldx, float* y, int ldy, int batch);
+int rlt_oracle_dense_backward_input(const rlt_dense_layer* layer, float* d_output, int ldd, float* d_input, int ldi, int batch);
+int rlt_oracle_dense_backward(const rlt_dense_layer* layer, const float* x, int ldx, float* d_output, int ldd, int batch);
+int rlt_oracle_dense_backward_full(const rlt_dense_layer* layer, const float* x, int ldx, float* d_output, int ldd, float* d_input, int ldi, int batch);
+
+int rlt_oracle_mlp_evaluate(const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy, int batch);
+int rlt_oracle_mlp_forward(const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, int batch);
+int rlt_oracle_mlp_backward(const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* d_output, int ldd,
+                            float* d_input, int ldi, int batch, int want_weight_gradients);
+int rlt_oracle_mlp_zero_gradient(const rlt_dense_layer* layers, int n_layers);
+int rlt_oracle_mlp_forward_backward(const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy,
+                                    const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch);
+
+int rlt_oracle_adam_step(const rlt_adam_tensor* tensors, int n_tensors, const rlt_adam_parameters* parameters, uint32_t* age,
+                         float polyak, float* out_gradient_squared_norm);
+int rlt_oracle_adam_reset(const rlt_adam_tensor* tensors, int n_tensors, uint32_t* age);
+int rlt_oracle_polyak_update(const float* source, float* target, size_t count, float polyak, int squared);
+
+int rlt_oracle_mse_gradient(const float* a, int lda, const float* b, int ldb, float* d_a, int ldda, int rows, int cols,
+                            float loss_weight, const float* loss_weight_ptr);
+int rlt_oracle_mse_evaluate(const float* a, int lda, const float* b, int ldb, int rows, int cols, float loss_weight, float* out_loss);
+
+int rlt_oracle_sas_forward(const rlt_sas_parameters* p, const float* input, int ldin, const float* noise, int ldn,
+                           float* actions, int lda, float* pre_squashing, int ldp, float* log_probabilities, int batch, int dim);
+int rlt_oracle_sas_backward(const rlt_sas_parameters* p, const float* input, int ldin, const float* noise, int ldn,
+                            const float* actions, int lda, const float* pre_squashing, int ldp,
+                            const float* d_output, int lddo, float* d_input, int lddi,
+                            const float* log_alpha, float* d_log_alpha, int batch, int dim);
+
+int rlt_oracle_sac_target_action_values(const float* q1_next, const float* q2_next, const float* rewards, const uint8_t* terminated,
+                                        const float* next_log_probabilities, const float* log_alpha, float gamma, int ignore_termination,
+                                        float* target, int batch);
+int rlt_oracle_sac_min_value_d_output(const float* q1, const float* q2, const float* d_critic_1_input, const float* d_critic_2_input,
+                                      int ld_critic_input, int critic_input_dim, int action_dim, float* d_actor_output, int ldo, int batch);
+int rlt_oracle_mask_copy(const float* source, int lds, float* target, int ldt, const uint8_t* mask, int invert, int rows, int cols);
+int rlt_oracle_mask_zero(float* gradient, int ld, const uint8_t* mask, int invert, int rows, int cols);
+int rlt_oracle_scale_f32(float* x, size_t count, float s, int reciprocal);
+int rlt_oracle_cast_reduce_sum_u8(const uint8_t* mask, size_t count, float* out_sum);
+
+int rlt_oracle_sac_train_critic(const rlt_sac_agent* agent, int critic_index, const float* action_noise);
+int rlt_oracle_sac_update_critic_targets(const rlt_sac_agent* agent);
+int rlt_oracle_sac_train_actor(const rlt_sac_agent* agent, const float* action_noise);
+
+int rlt_oracle_replay_add(const rlt_replay_buffer* rb, const float* observations, const float* actions, const float* rewards,
+                          const float* next_observations, const uint8_t* terminated, const uint8_t* truncated);
+int rlt_oracle_gather_batch(const rlt_replay_buffer* rb, const uint32_t* env_indices, const uint32_t* sample_offsets, int deterministic,
+                            int max_episode_length, int batch, float* observations_actions_base, float* rewards, uint8_t* terminated,
+                            uint8_t* reset, uint8_t* next_reset_base, uint8_t* final_step_mask, uint8_t* next_final_step_mask_base);
+
+int rlt_oracle_pendulum_step(const rlt_pendulum_parameters* p, float* states, const float* actions, float* observations,
+                             float* next_observations, float* rewards, int n_envs);
+int rlt_oracle_pendulum_runner_step(const rlt_pendulum_runner* runner, const rlt_replay_buffer* rb, int policy_kind,
+                                    const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas,
+                                    const float* actions_in, const float* action_noise, const float* initial_states);
+
+int rlt_oracle_ppo_gae(const float* rewards, const float* terminated, const float* truncated, const float* all_values,
+                       float* advantages, float* target_values, int ld, int n_envs, int steps, float gamma, float lambda,
+                       int ignore_termination);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
