@@ -1,0 +1,232 @@
+"""ctypes binding of include/rlt_rocm.h: structure mirrors, prototypes and a thin device-array helper.
+
+This is plumbing for tests, the smoke check and the benchmark; the product is the shared library itself.
+The HIP library must exist (built by build.py): loading fails loudly otherwise, there is no CPU fallback.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "librlt_rocm.so")
+
+c_float_p = C.POINTER(C.c_float)
+c_u8_p = C.POINTER(C.c_uint8)
+c_u32_p = C.POINTER(C.c_uint32)
+
+ACT = {"identity": 0, "relu": 1, "gelu": 2, "tanh": 3, "fast_tanh": 4, "sigmoid": 5}
+
+
+class DenseLayer(C.Structure):
+    _fields_ = [("weights", C.c_void_p), ("biases", C.c_void_p), ("d_weights", C.c_void_p), ("d_biases", C.c_void_p),
+                ("pre_activations", C.c_void_p), ("output", C.c_void_p),
+                ("in_dim", C.c_int32), ("out_dim", C.c_int32), ("activation", C.c_int32), ("reserved", C.c_int32)]
+
+
+class AdamParameters(C.Structure):
+    _fields_ = [("alpha", C.c_float), ("beta_1", C.c_float), ("beta_2", C.c_float), ("epsilon", C.c_float), ("epsilon_sqrt", C.c_float),
+                ("weight_decay", C.c_float), ("bias_lr_factor", C.c_float), ("enable_weight_decay", C.c_int32),
+                ("enable_bias_lr_factor", C.c_int32), ("enable_gradient_clipping", C.c_int32), ("gradient_clip_value", C.c_float)]
+
+
+def adam_parameters(alpha=1e-3, beta_1=0.9, beta_2=0.999, epsilon=1e-7, epsilon_sqrt=None):
+    return AdamParameters(alpha, beta_1, beta_2, epsilon, epsilon if epsilon_sqrt is None else epsilon_sqrt, 0.0, 1.0, 0, 0, 0, 1.0)
+
+
+class AdamTensor(C.Structure):
+    _fields_ = [("parameters", C.c_void_p), ("gradient", C.c_void_p), ("first_moment", C.c_void_p), ("second_moment", C.c_void_p),
+                ("polyak_target", C.c_void_p), ("count", C.c_uint32), ("flags", C.c_uint32)]
+
+
+class SasParameters(C.Structure):
+    _fields_ = [("log_std_lower_bound", C.c_float), ("log_std_upper_bound", C.c_float), ("log_probability_epsilon", C.c_float),
+                ("target_entropy", C.c_float)]
+
+
+class SacAgent(C.Structure):
+    _fields_ = [("batch", C.c_int32), ("observation_dim", C.c_int32), ("action_dim", C.c_int32), ("n_actor_layers", C.c_int32),
+                ("n_critic_layers", C.c_int32), ("gamma", C.c_float), ("polyak", C.c_float), ("reserved0", C.c_float),
+                ("sas", SasParameters), ("actor_adam", AdamParameters), ("critic_adam", AdamParameters), ("alpha_adam", AdamParameters),
+                ("actor", C.POINTER(DenseLayer)), ("critics", C.POINTER(DenseLayer) * 2), ("critics_target", C.POINTER(DenseLayer) * 2),
+                ("actor_adam_tensors", C.POINTER(AdamTensor)), ("n_actor_adam_tensors", C.c_int32), ("pad0", C.c_int32),
+                ("critic_adam_tensors", C.POINTER(AdamTensor) * 2), ("n_critic_adam_tensors", C.c_int32), ("pad1", C.c_int32),
+                ("log_alpha", AdamTensor),
+                ("actor_age", C.c_void_p), ("critic_age", C.c_void_p * 2), ("alpha_age", C.c_void_p),
+                ("observations_actions_base", C.c_void_p), ("rewards", C.c_void_p), ("terminated", C.c_void_p),
+                ("final_step_mask", C.c_void_p), ("next_final_step_mask", C.c_void_p), ("reset", C.c_void_p),
+                ("next_state_action_value_input", C.c_void_p), ("next_q", C.c_void_p * 2), ("next_log_probabilities", C.c_void_p),
+                ("target_action_value", C.c_void_p), ("d_output_critic", C.c_void_p * 2), ("state_action_value_input", C.c_void_p),
+                ("d_output_actor_critics", C.c_void_p), ("d_critic_input", C.c_void_p * 2), ("d_actor_output_squashing", C.c_void_p),
+                ("d_actor_output", C.c_void_p), ("actor_pre_squashing", C.c_void_p), ("actor_log_probabilities", C.c_void_p),
+                ("actor_actions", C.c_void_p), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+
+
+class ReplayBuffer(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("episode_start", C.c_void_p), ("position", C.c_void_p), ("current_episode_start", C.c_void_p),
+                ("full", C.c_void_p), ("n_envs", C.c_int32), ("capacity", C.c_int32), ("observation_dim", C.c_int32), ("action_dim", C.c_int32)]
+
+
+class PendulumParameters(C.Structure):
+    _fields_ = [("g", C.c_float), ("max_speed", C.c_float), ("max_torque", C.c_float), ("dt", C.c_float), ("m", C.c_float), ("l", C.c_float)]
+
+
+def pendulum_parameters():
+    return PendulumParameters(10.0, 8.0, 2.0, 0.05, 1.0, 1.0)
+
+
+class PendulumRunner(C.Structure):
+    _fields_ = [("states", C.c_void_p), ("episode_step", C.c_void_p), ("episode_return", C.c_void_p), ("truncated", C.c_void_p),
+                ("n_envs", C.c_int32), ("episode_step_limit", C.c_int32), ("env", PendulumParameters)]
+
+
+I, F, P, S, U64 = C.c_int, C.c_float, C.c_void_p, C.c_size_t, C.c_uint64
+LP = C.POINTER(DenseLayer)
+
+# name -> argument types after the leading device handle (shared by the HIP library and, minus the handle, the CPU checker)
+PROTOTYPES = {
+    "dense_evaluate": [LP, P, I, P, I, I],
+    "dense_forward": [LP, P, I, P, I, I],
+    "dense_backward_input": [LP, P, I, P, I, I],
+    "dense_backward": [LP, P, I, P, I, I],
+    "dense_backward_full": [LP, P, I, P, I, P, I, I],
+    "mlp_evaluate": [LP, I, P, I, P, I, I, P, S],
+    "mlp_forward": [LP, I, P, I, I],
+    "mlp_backward": [LP, I, P, I, P, I, P, I, I, I, P, S],
+    "mlp_zero_gradient": [LP, I],
+    "mlp_forward_backward": [LP, I, P, I, P, I, P, I, P, I, F, I, P, S],
+    "adam_step": [C.POINTER(AdamTensor), I, C.POINTER(AdamParameters), P, F, P],
+    "adam_reset": [C.POINTER(AdamTensor), I, P],
+    "polyak_update": [P, P, S, F, I],
+    "mse_gradient": [P, I, P, I, P, I, I, I, F, P],
+    "mse_evaluate": [P, I, P, I, I, I, F, P],
+    "sas_forward": [C.POINTER(SasParameters), P, I, P, I, P, I, P, I, P, I, I],
+    "sas_backward": [C.POINTER(SasParameters), P, I, P, I, P, I, P, I, P, I, P, I, P, P, I, I],
+    "sac_target_action_values": [P, P, P, P, P, P, F, I, P, I],
+    "sac_min_value_d_output": [P, P, P, P, I, I, I, P, I, I],
+    "mask_copy": [P, I, P, I, P, I, I, I],
+    "mask_zero": [P, I, P, I, I, I],
+    "scale_f32": [P, S, F, I],
+    "cast_reduce_sum_u8": [P, S, P],
+    "sac_train_critic": [C.POINTER(SacAgent), I, P],
+    "sac_update_critic_targets": [C.POINTER(SacAgent)],
+    "sac_train_actor": [C.POINTER(SacAgent), P],
+    "replay_add": [C.POINTER(ReplayBuffer), P, P, P, P, P, P],
+    "gather_batch": [C.POINTER(ReplayBuffer), P, P, I, I, I, P, P, P, P, P, P, P],
+    "pendulum_step": [C.POINTER(PendulumParameters), P, P, P, P, P, I],
+    "ppo_gae": [P, P, P, P, P, P, I, I, I, F, F, I],
+}
+# workspace arguments exist only in the device ABI (the CPU checker allocates its own)
+ROCM_ONLY = {
+    "init": ([I, C.POINTER(P)], I), "destroy": ([P], I), "check_status": ([P], I), "set_stream": ([P, P], I), "get_stream": ([P], P),
+    "error_string": ([I], C.c_char_p), "device_info": ([P, C.POINTER(I), C.POINTER(I), C.c_char_p, I], I),
+    "malloc": ([P, C.POINTER(P), S], I), "free": ([P, P], I),
+    "memcpy_h2d": ([P, P, P, S], I), "memcpy_d2h": ([P, P, P, S], I), "memcpy_d2d": ([P, P, P, S], I),
+    "memcpy2d": ([P, P, S, P, S, S, S, I], I),
+    "fill_f32": ([P, P, I, I, I, F], I), "fill_u8": ([P, P, S, C.c_uint8], I),
+    "randn_f32": ([P, P, S, U64, U64], I), "rand_f32": ([P, P, S, F, F, U64, U64], I),
+    "reduce_sum_f32": ([P, P, S, I, P], I),
+    "mlp_workspace_bytes": ([LP, I, I], S),
+    "gather_draw": ([P, C.POINTER(ReplayBuffer), I, U64, U64, P, P], I),
+    "pendulum_runner_step": ([P, C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, LP, I, C.POINTER(SasParameters), P, P, P, U64, U64], I),
+}
+
+
+def load_library(path=LIB_PATH):
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with `python rl-tools_amd/build.py` (there is no CPU fallback)")
+    lib = C.CDLL(path)
+    for name, args in PROTOTYPES.items():
+        fn = getattr(lib, "rlt_rocm_" + name)
+        fn.argtypes = [P] + args
+        fn.restype = I
+    for name, (args, res) in ROCM_ONLY.items():
+        fn = getattr(lib, "rlt_rocm_" + name)
+        fn.argtypes = args
+        fn.restype = res
+    return lib
+
+
+class RltError(RuntimeError):
+    pass
+
+
+class DeviceArray:
+    """A device allocation with a numpy-like shape/dtype; `ptr` is what the C ABI takes."""
+
+    def __init__(self, device, shape, dtype):
+        self.device, self.shape, self.dtype = device, tuple(shape), np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+        p = C.c_void_p()
+        device.check(device.lib.rlt_rocm_malloc(device.handle, C.byref(p), max(self.nbytes, 4)))
+        self.ptr = p.value
+
+    def upload(self, array):
+        a = np.ascontiguousarray(array, dtype=self.dtype)
+        assert a.nbytes == self.nbytes, (a.shape, self.shape)
+        if self.nbytes:
+            self.device.check(self.device.lib.rlt_rocm_memcpy_h2d(self.device.handle, self.ptr, a.ctypes.data, self.nbytes))
+        return self
+
+    def numpy(self):
+        out = np.empty(self.shape, self.dtype)
+        if self.nbytes:
+            self.device.check(self.device.lib.rlt_rocm_memcpy_d2h(self.device.handle, out.ctypes.data, self.ptr, self.nbytes))
+        return out
+
+    def offset(self, elements):
+        return self.ptr + int(elements) * self.dtype.itemsize
+
+    def free(self):
+        if self.ptr:
+            self.device.lib.rlt_rocm_free(self.device.handle, self.ptr)
+            self.ptr = None
+
+
+class Device:
+    """rlt_rocm_device handle plus convenience allocation/call helpers."""
+
+    def __init__(self, index=0, lib=None):
+        self.lib = lib or load_library()
+        h = C.c_void_p()
+        rc = self.lib.rlt_rocm_init(index, C.byref(h))
+        if rc != 0:
+            raise RltError(f"rlt_rocm_init failed: {self.lib.rlt_rocm_error_string(rc).decode()}")
+        self.handle = h
+        self._arrays = []
+
+    def check(self, rc):
+        if rc != 0:
+            raise RltError(f"rlt_rocm call failed ({rc}): {self.lib.rlt_rocm_error_string(rc).decode()}")
+
+    def call(self, name, *args):
+        self.check(getattr(self.lib, "rlt_rocm_" + name)(self.handle, *args))
+
+    def sync(self):
+        self.check(self.lib.rlt_rocm_check_status(self.handle))
+
+    def empty(self, shape, dtype=np.float32):
+        a = DeviceArray(self, shape, dtype)
+        self._arrays.append(a)
+        return a
+
+    def zeros(self, shape, dtype=np.float32):
+        return self.empty(shape, dtype).upload(np.zeros(shape, dtype))
+
+    def array(self, host):
+        host = np.asarray(host)
+        return self.empty(host.shape, host.dtype).upload(host)
+
+    def info(self):
+        cu, lds = C.c_int(), C.c_int()
+        name = C.create_string_buffer(128)
+        self.check(self.lib.rlt_rocm_device_info(self.handle, C.byref(cu), C.byref(lds), name, 128))
+        return {"compute_units": cu.value, "lds_bytes": lds.value, "name": name.value.decode()}
+
+    def close(self):
+        for a in self._arrays:
+            a.free()
+        self._arrays = []
+        if self.handle:
+            self.lib.rlt_rocm_destroy(self.handle)
+            self.handle = None

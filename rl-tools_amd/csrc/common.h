@@ -1,0 +1,74 @@
+// Shared declarations of the gfx950 backend: device handle, error plumbing, launch helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include "../../include/rlt_rocm.h"
+
+struct rlt_rocm_device {
+    int hip_device;
+    hipStream_t own_stream;
+    hipStream_t stream;          // the stream work is enqueued on (own_stream unless the caller set one)
+    int compute_units;
+    int lds_bytes;
+    char name[128];
+    void* scratch;               // grow-only device workspace for split reductions and partial sums
+    size_t scratch_bytes;
+    void* counters;              // 8 KiB, zero between launches: [0,256) ticket counters, [256,..) per-workgroup partial sums
+    int sticky_error;
+};
+
+#define RLT_HIP(expr)                                                        \
+    do {                                                                     \
+        hipError_t _e = (expr);                                              \
+        if (_e != hipSuccess) { if (device) device->sticky_error = (int)_e; return (int)_e; } \
+    } while (0)
+
+#define RLT_REQUIRE(cond) do { if (!(cond)) return RLT_E_INVALID_ARGUMENT; } while (0)
+
+// Grow-only scratch owned by the device handle.
+int rlt_scratch(rlt_rocm_device* device, size_t bytes, void** out);
+// 8 KiB of zero-initialised device memory for last-workgroup-done tickets and per-workgroup partials.
+int rlt_counters(rlt_rocm_device* device, void** out);
+// Returns hipGetLastError() folded into the return convention; called after every launch.
+int rlt_launch_status(rlt_rocm_device* device);
+
+static inline int rlt_div_up(int a, int b) { return (a + b - 1) / b; }
+
+// ---- activation functions on the device (nn/activation_functions.h:25-90 of the reference)
+__device__ __forceinline__ float rlt_fast_tanh(float x) {
+    x = fminf(fmaxf(x, -3.0f), 3.0f);
+    float x2 = x * x;
+    return x * (27.0f + x2) / (27.0f + 9.0f * x2);
+}
+__device__ __forceinline__ float rlt_act(float x, int f) {
+    switch (f) {
+        case RLT_ACT_RELU: return x > 0.0f ? x : 0.0f;
+        case RLT_ACT_GELU: { const float a = 0.7978845608028654f; return 0.5f * (x + x * tanhf(a * (0.044715f * x * x * x + x))); }
+        case RLT_ACT_TANH: return tanhf(x);
+        case RLT_ACT_FAST_TANH: return rlt_fast_tanh(x);
+        case RLT_ACT_SIGMOID: return 1.0f / (1.0f + expf(-x));
+        default: return x;
+    }
+}
+__device__ __forceinline__ float rlt_dact(float x, int f) {
+    switch (f) {
+        case RLT_ACT_RELU: return x > 0.0f ? 1.0f : 0.0f;
+        case RLT_ACT_GELU: {
+            const float a = 0.7978845608028654f, b = 0.044715f;
+            float t = tanhf(a * (b * x * x * x + x));
+            return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * a * (3.0f * b * x * x + 1.0f);
+        }
+        case RLT_ACT_TANH: { float t = tanhf(x); return 1.0f - t * t; }
+        case RLT_ACT_FAST_TANH: { float t = rlt_fast_tanh(x); return 1.0f - t * t; }
+        case RLT_ACT_SIGMOID: { float s = 1.0f / (1.0f + expf(-x)); return s * (1.0f - s); }
+        default: return 1.0f;
+    }
+}
+
+// 64-lane wavefront sum (butterfly over DPP/ds_swizzle via __shfl_xor)
+__device__ __forceinline__ float rlt_wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}

@@ -1,0 +1,257 @@
+// Device handle, memory and the small container operations of the C ABI
+// (reference: devices/cuda.h:130-174, containers/matrix/operations_cuda.h:16-218, containers/tensor/operations_cuda.h:15-624).
+#include "common.h"
+#include <cstdio>
+#include <cstring>
+
+int rlt_launch_status(rlt_rocm_device* device) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { device->sticky_error = (int)e; return (int)e; }
+    return 0;
+}
+
+int rlt_scratch(rlt_rocm_device* device, size_t bytes, void** out) {
+    if (bytes > device->scratch_bytes) {
+        if (device->scratch) RLT_HIP(hipFree(device->scratch));   // hipFree waits for the work that still uses it
+        device->scratch = nullptr; device->scratch_bytes = 0;
+        size_t want = bytes < (size_t)(1u << 20) ? (size_t)(1u << 20) : bytes + bytes / 4;
+        RLT_HIP(hipMalloc(&device->scratch, want));
+        device->scratch_bytes = want;
+    }
+    *out = device->scratch;
+    return 0;
+}
+
+int rlt_counters(rlt_rocm_device* device, void** out) {
+    *out = device->counters;
+    return device->counters ? 0 : RLT_E_NOT_INITIALISED;
+}
+
+namespace {
+
+__global__ __launch_bounds__(256) void fill_f32_kernel(float* __restrict__ dst, int rows, int cols, int ld, float value) {
+    const size_t total = (size_t)rows * cols;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        size_t r = i / cols, c = i % cols;
+        dst[r * ld + c] = value;
+    }
+}
+__global__ __launch_bounds__(256) void fill_u8_kernel(uint8_t* __restrict__ dst, size_t count, uint8_t value) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) dst[i] = value;
+}
+__global__ __launch_bounds__(256) void scale_kernel(float* __restrict__ x, size_t count, float s, int reciprocal) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        x[i] = reciprocal ? s / x[i] : s * x[i];
+}
+
+// Philox4x32-10 (Salmon et al. 2011): a pure function of (key = seed, counter = offset + element/4)
+__device__ __forceinline__ void philox_round(uint32_t& c0, uint32_t& c1, uint32_t& c2, uint32_t& c3, uint32_t k0, uint32_t k1) {
+    const uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u;
+    uint32_t hi0 = __umulhi(M0, c0), lo0 = M0 * c0;
+    uint32_t hi1 = __umulhi(M1, c2), lo1 = M1 * c2;
+    uint32_t n0 = hi1 ^ c1 ^ k0, n1 = lo1, n2 = hi0 ^ c3 ^ k1, n3 = lo0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+}
+__device__ __forceinline__ uint4 philox4x32(uint64_t seed, uint64_t counter) {
+    uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+    uint32_t c0 = (uint32_t)counter, c1 = (uint32_t)(counter >> 32), c2 = 0x9E3779B9u, c3 = 0xBB67AE85u;
+#pragma unroll
+    for (int r = 0; r < 10; r++) { philox_round(c0, c1, c2, c3, k0, k1); k0 += 0x9E3779B9u; k1 += 0xBB67AE85u; }
+    return make_uint4(c0, c1, c2, c3);
+}
+__device__ __forceinline__ float u01(uint32_t x) { return ((x >> 8) + 0.5f) * (1.0f / 16777216.0f); }   // (0,1)
+__global__ __launch_bounds__(256) void rand_kernel(float* __restrict__ dst, size_t count, float low, float high, uint64_t seed, uint64_t offset, int normal) {
+    const size_t quads = (count + 3) / 4;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (size_t)gridDim.x * blockDim.x) {
+        uint4 r = philox4x32(seed, offset + q);
+        float v[4];
+        if (normal) {   // Box-Muller, two normals per pair of uniforms
+            float r0 = sqrtf(-2.0f * logf(u01(r.x))), r1 = sqrtf(-2.0f * logf(u01(r.z)));
+            float s0, c0, s1, c1;
+            sincosf(6.283185307179586f * u01(r.y), &s0, &c0);
+            sincosf(6.283185307179586f * u01(r.w), &s1, &c1);
+            v[0] = r0 * c0; v[1] = r0 * s0; v[2] = r1 * c1; v[3] = r1 * s1;
+        } else {
+            v[0] = low + (high - low) * u01(r.x); v[1] = low + (high - low) * u01(r.y);
+            v[2] = low + (high - low) * u01(r.z); v[3] = low + (high - low) * u01(r.w);
+        }
+        for (int j = 0; j < 4; j++) if (q * 4 + j < count) dst[q * 4 + j] = v[j];
+    }
+}
+
+// single-workgroup reductions: 1024 lanes, wavefront butterflies then one pass over the 16 partials
+template <int KIND>   // 0: uint8 != 0 count, 1: sum, 2: sum of squares
+__global__ __launch_bounds__(1024) void reduce_kernel(const void* __restrict__ src, size_t count, float* __restrict__ out) {
+    __shared__ float partial[16];
+    float acc = 0.0f;
+    for (size_t i = threadIdx.x; i < count; i += blockDim.x) {
+        if (KIND == 0) acc += (float)(((const uint8_t*)src)[i] != 0);
+        else { float v = ((const float*)src)[i]; acc += KIND == 1 ? v : v * v; }
+    }
+    acc = rlt_wave_sum(acc);
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) { float s = 0.0f; for (int i = 0; i < 16; i++) s += partial[i]; *out = s; }
+}
+
+int grid_for(size_t n) { size_t b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : (b < 1 ? 1 : b)); }
+
+}  // namespace
+
+extern "C" {
+
+int rlt_rocm_init(int hip_device_index, rlt_rocm_device** out_device) {
+    if (!out_device) return RLT_E_INVALID_ARGUMENT;
+    rlt_rocm_device* device = nullptr;
+    hipError_t e = hipSetDevice(hip_device_index);
+    if (e != hipSuccess) return (int)e;
+    device = new rlt_rocm_device();
+    std::memset(device, 0, sizeof *device);
+    device->hip_device = hip_device_index;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, hip_device_index);
+    if (e != hipSuccess) { delete device; return (int)e; }
+    device->compute_units = prop.multiProcessorCount;
+    device->lds_bytes = (int)prop.sharedMemPerBlock;
+    std::snprintf(device->name, sizeof device->name, "%s (%s)", prop.name, prop.gcnArchName);
+    e = hipStreamCreate(&device->own_stream);   // default priority
+    if (e != hipSuccess) { delete device; return (int)e; }
+    device->stream = device->own_stream;
+    e = hipMalloc(&device->counters, 8192);
+    if (e == hipSuccess) e = hipMemset(device->counters, 0, 8192);
+    if (e != hipSuccess) { hipStreamDestroy(device->own_stream); delete device; return (int)e; }
+    *out_device = device;
+    return 0;
+}
+int rlt_rocm_destroy(rlt_rocm_device* device) {
+    if (!device) return RLT_E_INVALID_ARGUMENT;
+    hipStreamSynchronize(device->own_stream);
+    if (device->scratch) hipFree(device->scratch);
+    if (device->counters) hipFree(device->counters);
+    hipStreamDestroy(device->own_stream);
+    delete device;
+    return 0;
+}
+int rlt_rocm_check_status(rlt_rocm_device* device) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    hipError_t e = hipStreamSynchronize(device->stream);
+    if (e != hipSuccess) device->sticky_error = (int)e;
+    int s = device->sticky_error;
+    return s;
+}
+int rlt_rocm_set_stream(rlt_rocm_device* device, void* hip_stream) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    device->stream = hip_stream ? (hipStream_t)hip_stream : device->own_stream;
+    return 0;
+}
+void* rlt_rocm_get_stream(rlt_rocm_device* device) { return device ? (void*)device->stream : nullptr; }
+const char* rlt_rocm_error_string(int code) {
+    if (code == 0) return "success";
+    if (code == RLT_E_INVALID_ARGUMENT) return "rlt_rocm: invalid argument (null pointer, non-positive dimension or too small leading dimension)";
+    if (code == RLT_E_UNSUPPORTED) return "rlt_rocm: shape outside what the kernels support";
+    if (code == RLT_E_NOT_INITIALISED) return "rlt_rocm: device handle not initialised";
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "rlt_rocm: unknown error";
+}
+int rlt_rocm_device_info(rlt_rocm_device* device, int* compute_units, int* lds_bytes, char* name, int name_len) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    if (compute_units) *compute_units = device->compute_units;
+    if (lds_bytes) *lds_bytes = device->lds_bytes;
+    if (name && name_len > 0) std::snprintf(name, (size_t)name_len, "%s", device->name);
+    return 0;
+}
+
+int rlt_rocm_malloc(rlt_rocm_device* device, void** out_ptr, size_t bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(out_ptr && bytes > 0);
+    RLT_HIP(hipMalloc(out_ptr, bytes));
+    return 0;
+}
+int rlt_rocm_free(rlt_rocm_device* device, void* ptr) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    if (!ptr) return 0;
+    RLT_HIP(hipFree(ptr));
+    return 0;
+}
+int rlt_rocm_memcpy_h2d(rlt_rocm_device* device, void* dst, const void* src_host, size_t bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(dst && src_host);
+    if (bytes == 0) return 0;
+    RLT_HIP(hipMemcpyAsync(dst, src_host, bytes, hipMemcpyHostToDevice, device->stream));
+    RLT_HIP(hipStreamSynchronize(device->stream));
+    return 0;
+}
+int rlt_rocm_memcpy_d2h(rlt_rocm_device* device, void* dst_host, const void* src, size_t bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(dst_host && src);
+    if (bytes == 0) return 0;
+    RLT_HIP(hipMemcpyAsync(dst_host, src, bytes, hipMemcpyDeviceToHost, device->stream));
+    RLT_HIP(hipStreamSynchronize(device->stream));
+    return 0;
+}
+int rlt_rocm_memcpy_d2d(rlt_rocm_device* device, void* dst, const void* src, size_t bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(dst && src);
+    if (bytes == 0) return 0;
+    RLT_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, device->stream));
+    return 0;
+}
+int rlt_rocm_memcpy2d(rlt_rocm_device* device, void* dst, size_t dst_pitch, const void* src, size_t src_pitch,
+                      size_t width_bytes, size_t rows, int kind) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(dst && src && dst_pitch >= width_bytes && src_pitch >= width_bytes && kind >= 0 && kind <= 2);
+    if (width_bytes == 0 || rows == 0) return 0;
+    hipMemcpyKind k = kind == 0 ? hipMemcpyDeviceToDevice : (kind == 1 ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost);
+    RLT_HIP(hipMemcpy2DAsync(dst, dst_pitch, src, src_pitch, width_bytes, rows, k, device->stream));
+    if (kind != 0) RLT_HIP(hipStreamSynchronize(device->stream));
+    return 0;
+}
+int rlt_rocm_fill_f32(rlt_rocm_device* device, float* dst, int rows, int cols, int ld, float value) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(dst && rows > 0 && cols > 0 && ld >= cols);
+    hipLaunchKernelGGL(fill_f32_kernel, dim3(grid_for((size_t)rows * cols)), dim3(256), 0, device->stream, dst, rows, cols, ld, value);
+    return rlt_launch_status(device);
+}
+int rlt_rocm_fill_u8(rlt_rocm_device* device, uint8_t* dst, size_t count, uint8_t value) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(dst);
+    if (count == 0) return 0;
+    hipLaunchKernelGGL(fill_u8_kernel, dim3(grid_for(count)), dim3(256), 0, device->stream, dst, count, value);
+    return rlt_launch_status(device);
+}
+int rlt_rocm_randn_f32(rlt_rocm_device* device, float* dst, size_t count, uint64_t seed, uint64_t offset) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(dst);
+    if (count == 0) return 0;
+    hipLaunchKernelGGL(rand_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, 0.0f, 1.0f, seed, offset, 1);
+    return rlt_launch_status(device);
+}
+int rlt_rocm_rand_f32(rlt_rocm_device* device, float* dst, size_t count, float low, float high, uint64_t seed, uint64_t offset) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(dst);
+    if (count == 0) return 0;
+    hipLaunchKernelGGL(rand_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, low, high, seed, offset, 0);
+    return rlt_launch_status(device);
+}
+int rlt_rocm_scale_f32(rlt_rocm_device* device, float* x, size_t count, float s, int reciprocal) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(x);
+    if (count == 0) return 0;
+    hipLaunchKernelGGL(scale_kernel, dim3(grid_for(count)), dim3(256), 0, device->stream, x, count, s, reciprocal);
+    return rlt_launch_status(device);
+}
+int rlt_rocm_cast_reduce_sum_u8(rlt_rocm_device* device, const uint8_t* mask, size_t count, float* out_sum) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(mask && out_sum);
+    hipLaunchKernelGGL(reduce_kernel<0>, dim3(1), dim3(1024), 0, device->stream, (const void*)mask, count, out_sum);
+    return rlt_launch_status(device);
+}
+int rlt_rocm_reduce_sum_f32(rlt_rocm_device* device, const float* x, size_t count, int squared, float* out_sum) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(x && out_sum);
+    if (squared) hipLaunchKernelGGL(reduce_kernel<2>, dim3(1), dim3(1024), 0, device->stream, (const void*)x, count, out_sum);
+    else hipLaunchKernelGGL(reduce_kernel<1>, dim3(1), dim3(1024), 0, device->stream, (const void*)x, count, out_sum);
+    return rlt_launch_status(device);
+}
+
+}  // extern "C"

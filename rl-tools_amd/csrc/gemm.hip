@@ -1,0 +1,333 @@
+// fp32 MFMA tile kernels for the three contractions of a dense layer
+// (reference: nn/layers/dense/operations_cpu_blas.h:36-218 -- one sgemm each for forward, d_input and d_weights,
+//  with the bias broadcast, activation, activation derivative and bias-gradient loops around them; here those loops
+//  are the kernels' epilogues / side sums).
+//
+//   mode 0  forward        C[b][o] = act( sum_i x[b][i] W[o][i] + bias[o] )           A, B both K-contiguous
+//   mode 1  d_input        C[b][i] = sum_o d_pre[b][o] W[o][i]   (* act'(pre_prev))   A K-contiguous, B N-contiguous
+//   mode 2  d_weights      C[o][i] += sum_b d_pre[b][o] x[b][i], d_bias[o] += sum_b   A M-contiguous, B N-contiguous,
+//                                                                                      batch split over blockIdx.z
+//
+// A workgroup is 4 wavefronts (256 lanes) arranged WAVES_M x WAVES_N; each wavefront owns TM x TN tiles of 32x32 and
+// issues v_mfma_f32_32x32x2_f32. Operand tiles are staged through LDS k-major ([BK][rows+PAD]) so that the 32 lanes of
+// a half-wavefront read 32 consecutive words (no bank conflicts) and the two halves read consecutive k.
+#include "common.h"
+#include "gemm.h"
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int BK = 16;
+constexpr int PAD = 4;
+constexpr int THREADS = 256;
+
+struct GemmParams {
+    const float* A; int lda;
+    const float* B; int ldb;
+    int M, N, K;
+    int k_per_split;
+    int vecA, vecB;
+    // mode 0
+    const float* bias; int act; float* pre; float* out; float* y; int ldy;
+    // mode 1
+    float* C; int ldc; const float* dact_pre; int dact_kind;
+    // mode 2
+    float* dW; float* dbias; float* ws; int splits;
+};
+
+template <int R>
+struct TileRegs { float4 v[(R * 4 + THREADS - 1) / THREADS]; };
+
+// source rows are contiguous along k: tile element (row r, k) = src[(row0+r)*ld + k0+k]
+template <int R>
+__device__ __forceinline__ void gload_kcontig(TileRegs<R>& t, const float* __restrict__ src, int ld, int row0, int nrows,
+                                              int k0, int kend, bool vec, int tid) {
+    constexpr int NQ = (R * 4 + THREADS - 1) / THREADS;
+#pragma unroll
+    for (int i = 0; i < NQ; i++) {
+        int q = tid + i * THREADS;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (q < R * 4) {
+            int row = q >> 2, kq = (q & 3) * 4;
+            int gr = row0 + row, gk = k0 + kq;
+            if (gr < nrows && gk < kend) {
+                const float* p = src + (size_t)gr * ld + gk;
+                if (vec && gk + 3 < kend) v = *reinterpret_cast<const float4*>(p);
+                else {
+                    v.x = p[0];
+                    if (gk + 1 < kend) v.y = p[1];
+                    if (gk + 2 < kend) v.z = p[2];
+                    if (gk + 3 < kend) v.w = p[3];
+                }
+            }
+        }
+        t.v[i] = v;
+    }
+}
+template <int R>
+__device__ __forceinline__ void sstore_kcontig(const TileRegs<R>& t, float* s, int tid) {
+    constexpr int NQ = (R * 4 + THREADS - 1) / THREADS;
+#pragma unroll
+    for (int i = 0; i < NQ; i++) {
+        int q = tid + i * THREADS;
+        if (q < R * 4) {
+            int row = q >> 2, kq = (q & 3) * 4;
+            s[(kq + 0) * (R + PAD) + row] = t.v[i].x;
+            s[(kq + 1) * (R + PAD) + row] = t.v[i].y;
+            s[(kq + 2) * (R + PAD) + row] = t.v[i].z;
+            s[(kq + 3) * (R + PAD) + row] = t.v[i].w;
+        }
+    }
+}
+// source rows are k, contiguous along the tile's m/n: tile element (k, c) = src[(k0+k)*ld + col0+c]
+template <int R>
+__device__ __forceinline__ void gload_mncontig(TileRegs<R>& t, const float* __restrict__ src, int ld, int col0, int ncols,
+                                               int k0, int kend, bool vec, int tid) {
+    constexpr int NQ = (R * 4 + THREADS - 1) / THREADS;
+    constexpr int QPR = R / 4;  // quads per k-row
+#pragma unroll
+    for (int i = 0; i < NQ; i++) {
+        int q = tid + i * THREADS;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (q < R * 4) {
+            int k = q / QPR, c4 = (q % QPR) * 4;
+            int gk = k0 + k, gc = col0 + c4;
+            if (gk < kend && gc < ncols) {
+                const float* p = src + (size_t)gk * ld + gc;
+                if (vec && gc + 3 < ncols) v = *reinterpret_cast<const float4*>(p);
+                else {
+                    v.x = p[0];
+                    if (gc + 1 < ncols) v.y = p[1];
+                    if (gc + 2 < ncols) v.z = p[2];
+                    if (gc + 3 < ncols) v.w = p[3];
+                }
+            }
+        }
+        t.v[i] = v;
+    }
+}
+template <int R>
+__device__ __forceinline__ void sstore_mncontig(const TileRegs<R>& t, float* s, int tid) {
+    constexpr int NQ = (R * 4 + THREADS - 1) / THREADS;
+    constexpr int QPR = R / 4;
+#pragma unroll
+    for (int i = 0; i < NQ; i++) {
+        int q = tid + i * THREADS;
+        if (q < R * 4) {
+            int k = q / QPR, c4 = (q % QPR) * 4;
+            *reinterpret_cast<float4*>(&s[k * (R + PAD) + c4]) = t.v[i];
+        }
+    }
+}
+
+template <int MODE, int WAVES_M, int WAVES_N, int TM, int TN>
+__global__ __launch_bounds__(THREADS) void gemm_kernel(GemmParams p) {
+    static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per workgroup");
+    constexpr int BM = WAVES_M * TM * 32;
+    constexpr int BN = WAVES_N * TN * 32;
+    __shared__ __attribute__((aligned(16))) float sA[2][BK * (BM + PAD)];
+    __shared__ __attribute__((aligned(16))) float sB[2][BK * (BN + PAD)];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+    int ks = 0, ke = p.K;
+    if (MODE == 2) { ks = blockIdx.z * p.k_per_split; ke = min(p.K, ks + p.k_per_split); }
+    const int nk = (ke - ks + BK - 1) / BK;
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    TileRegs<BM> ra;
+    TileRegs<BN> rb;
+    auto gload = [&](int k0) {
+        if (MODE == 2) gload_mncontig<BM>(ra, p.A, p.lda, m0, p.M, k0, ke, p.vecA, tid);
+        else gload_kcontig<BM>(ra, p.A, p.lda, m0, p.M, k0, ke, p.vecA, tid);
+        if (MODE == 0) gload_kcontig<BN>(rb, p.B, p.ldb, n0, p.N, k0, ke, p.vecB, tid);
+        else gload_mncontig<BN>(rb, p.B, p.ldb, n0, p.N, k0, ke, p.vecB, tid);
+    };
+    auto sstore = [&](int buf) {
+        if (MODE == 2) sstore_mncontig<BM>(ra, sA[buf], tid); else sstore_kcontig<BM>(ra, sA[buf], tid);
+        if (MODE == 0) sstore_kcontig<BN>(rb, sB[buf], tid); else sstore_mncontig<BN>(rb, sB[buf], tid);
+    };
+
+    const bool bias_block = (MODE == 2) && (blockIdx.x == 0) && (p.dbias != nullptr);
+    float bsum = 0.0f;
+
+    if (nk > 0) { gload(ks); sstore(0); }
+    __syncthreads();
+    for (int t = 0; t < nk; t++) {
+        const int cur = t & 1;
+        if (t + 1 < nk) gload(ks + (t + 1) * BK);
+        const float* a_base = sA[cur] + (lane >> 5) * (BM + PAD) + wm * (TM * 32) + (lane & 31);
+        const float* b_base = sB[cur] + (lane >> 5) * (BN + PAD) + wn * (TN * 32) + (lane & 31);
+#pragma unroll
+        for (int kk = 0; kk < BK / 2; kk++) {
+            float a[TM], b[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) a[i] = a_base[kk * 2 * (BM + PAD) + i * 32];
+#pragma unroll
+            for (int j = 0; j < TN; j++) b[j] = b_base[kk * 2 * (BN + PAD) + j * 32];
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (bias_block && tid < BM) {
+#pragma unroll
+            for (int k = 0; k < BK; k++) bsum += sA[cur][k * (BM + PAD) + tid];
+        }
+        if (t + 1 < nk) sstore(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue. Accumulator element v of lane l in a 32x32 tile: row = 8*(v/4) + 4*(l/32) + v%4, col = l%32
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = m0 + wm * (TM * 32) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (row < p.M && col < p.N) {
+                    float val = acc[i][j][v];
+                    if (MODE == 0) {
+                        if (p.bias) val += p.bias[col];
+                        if (p.pre) p.pre[(size_t)row * p.N + col] = val;
+                        float o = rlt_act(val, p.act);
+                        if (p.out) p.out[(size_t)row * p.N + col] = o;
+                        if (p.y) p.y[(size_t)row * p.ldy + col] = o;
+                    } else if (MODE == 1) {
+                        if (p.dact_pre) val *= rlt_dact(p.dact_pre[(size_t)row * p.N + col], p.dact_kind);
+                        p.C[(size_t)row * p.ldc + col] = val;
+                    } else {
+                        if (p.splits == 1) p.dW[(size_t)row * p.N + col] += val;
+                        else p.ws[(size_t)blockIdx.z * ((size_t)p.M * p.N + p.M) + (size_t)row * p.N + col] = val;
+                    }
+                }
+            }
+        }
+    }
+    if (bias_block && tid < BM && m0 + tid < p.M) {
+        if (p.splits == 1) p.dbias[m0 + tid] += bsum;
+        else p.ws[(size_t)blockIdx.z * ((size_t)p.M * p.N + p.M) + (size_t)p.M * p.N + m0 + tid] = bsum;
+    }
+}
+
+// dW += sum_s ws[s][0:MN], dbias += sum_s ws[s][MN:MN+M]  (fixed summation order: deterministic)
+__global__ __launch_bounds__(256) void wgrad_reduce_kernel(float* __restrict__ dW, float* __restrict__ dbias, const float* __restrict__ ws,
+                                                           int mn, int m, int splits) {
+    const int total = mn + (dbias ? m : 0);
+    const size_t stride = (size_t)mn + m;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        float s = 0.0f;
+        for (int k = 0; k < splits; k++) s += ws[(size_t)k * stride + i];
+        if (i < mn) dW[i] += s; else dbias[i - mn] += s;
+    }
+}
+
+// d_pre = act'(pre) * d_output (nn/layers/dense/operations_cpu_blas.h:119-141); dst may alias src
+__global__ __launch_bounds__(256) void dpre_kernel(const float* src, int lds, float* dst, int ldd, const float* __restrict__ pre, int rows, int cols, int act) {
+    const size_t total = (size_t)rows * cols;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        int r = (int)(i / cols), c = (int)(i % cols);
+        dst[(size_t)r * ldd + c] = rlt_dact(pre[i], act) * src[(size_t)r * lds + c];
+    }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <int MODE>
+int launch(rlt_rocm_device* device, const GemmParams& p, int splits) {
+    dim3 block(THREADS);
+    // tile shape by problem shape: 128x128 for the wide contractions, 128x32 / 32x128 when one side is narrow,
+    // 64x64 when both are small
+    if (p.N <= 32) {
+        dim3 grid(rlt_div_up(p.N, 32), rlt_div_up(p.M, 128), splits);
+        hipLaunchKernelGGL((gemm_kernel<MODE, 4, 1, 1, 1>), grid, block, 0, device->stream, p);
+    } else if (p.M <= 32) {
+        dim3 grid(rlt_div_up(p.N, 128), rlt_div_up(p.M, 32), splits);
+        hipLaunchKernelGGL((gemm_kernel<MODE, 1, 4, 1, 1>), grid, block, 0, device->stream, p);
+    } else if ((long long)p.M * p.N <= 64ll * 1024 || p.M <= 64 || p.N <= 64) {
+        dim3 grid(rlt_div_up(p.N, 64), rlt_div_up(p.M, 64), splits);
+        hipLaunchKernelGGL((gemm_kernel<MODE, 2, 2, 1, 1>), grid, block, 0, device->stream, p);
+    } else {
+        dim3 grid(rlt_div_up(p.N, 128), rlt_div_up(p.M, 128), splits);
+        hipLaunchKernelGGL((gemm_kernel<MODE, 2, 2, 2, 2>), grid, block, 0, device->stream, p);
+    }
+    return rlt_launch_status(device);
+}
+
+}  // namespace
+
+int rlt_gemm_forward(rlt_rocm_device* device, const float* x, int ldx, const float* W, const float* bias, int act,
+                     float* pre, float* out, float* y, int ldy, int batch, int in_dim, int out_dim) {
+    if (rlt_div_up(batch, 32) > 65535) return RLT_E_UNSUPPORTED;
+    GemmParams p = {};
+    p.A = x; p.lda = ldx; p.B = W; p.ldb = in_dim; p.M = batch; p.N = out_dim; p.K = in_dim; p.k_per_split = in_dim;
+    p.vecA = aligned16(x) && (ldx % 4 == 0); p.vecB = aligned16(W) && (in_dim % 4 == 0);
+    p.bias = bias; p.act = act; p.pre = pre; p.out = out; p.y = y; p.ldy = ldy; p.splits = 1;
+    return launch<0>(device, p, 1);
+}
+
+int rlt_gemm_backward_input(rlt_rocm_device* device, const float* d_pre, int ldd, const float* W, float* d_in, int ldi,
+                            const float* dact_pre, int dact_kind, int batch, int in_dim, int out_dim) {
+    if (rlt_div_up(batch, 32) > 65535) return RLT_E_UNSUPPORTED;
+    GemmParams p = {};
+    p.A = d_pre; p.lda = ldd; p.B = W; p.ldb = in_dim; p.M = batch; p.N = in_dim; p.K = out_dim; p.k_per_split = out_dim;
+    p.vecA = aligned16(d_pre) && (ldd % 4 == 0); p.vecB = aligned16(W) && (in_dim % 4 == 0);
+    p.C = d_in; p.ldc = ldi; p.dact_pre = dact_pre; p.dact_kind = dact_kind; p.splits = 1;
+    return launch<1>(device, p, 1);
+}
+
+int rlt_gemm_wgrad(rlt_rocm_device* device, const float* d_pre, int ldd, const float* x, int ldx, float* dW, float* dbias,
+                   int batch, int in_dim, int out_dim) {
+    GemmParams p = {};
+    p.A = d_pre; p.lda = ldd; p.B = x; p.ldb = ldx; p.M = out_dim; p.N = in_dim; p.K = batch;
+    p.vecA = aligned16(d_pre) && (ldd % 4 == 0); p.vecB = aligned16(x) && (ldx % 4 == 0);
+    p.dW = dW; p.dbias = dbias;
+    // split the batch so that the grid fills the chip: about 2 workgroups per compute unit, at least 256 rows per split
+    int bm = out_dim <= 32 ? 32 : (((long long)out_dim * in_dim <= 64ll * 1024 || out_dim <= 64 || in_dim <= 64) ? 64 : 128);
+    int bn = in_dim <= 32 ? 32 : (out_dim <= 32 ? 128 : (bm == 64 ? 64 : 128));
+    int tiles = rlt_div_up(out_dim, bm) * rlt_div_up(in_dim, bn);
+    int splits = (2 * device->compute_units + tiles - 1) / tiles;
+    int max_splits = rlt_div_up(batch, 256);
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    int kps = rlt_div_up(rlt_div_up(batch, splits), BK) * BK;
+    splits = rlt_div_up(batch, kps);
+    p.k_per_split = kps; p.splits = splits;
+    if (splits > 1) {
+        void* ws = nullptr;
+        int rc = rlt_scratch(device, (size_t)splits * ((size_t)out_dim * in_dim + out_dim) * sizeof(float), &ws);
+        if (rc) return rc;
+        p.ws = (float*)ws;
+    }
+    int rc = launch<2>(device, p, splits);
+    if (rc) return rc;
+    if (splits > 1) {
+        int mn = out_dim * in_dim;
+        int blocks = rlt_div_up(mn + out_dim, 256);
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(blocks), dim3(256), 0, device->stream, dW, dbias, p.ws, mn, out_dim, splits);
+        return rlt_launch_status(device);
+    }
+    return 0;
+}
+
+int rlt_dpre(rlt_rocm_device* device, const float* src, int lds, float* dst, int ldd, const float* pre, int rows, int cols, int act) {
+    if (act == RLT_ACT_IDENTITY && src == dst) return 0;
+    size_t total = (size_t)rows * cols;
+    int blocks = (int)((total + 255) / 256); if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(dpre_kernel, dim3(blocks), dim3(256), 0, device->stream, src, lds, dst, ldd, pre, rows, cols, act);
+    return rlt_launch_status(device);
+}

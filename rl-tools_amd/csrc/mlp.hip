@@ -1,0 +1,214 @@
+// dense layer and MLP entry points of the C ABI, built on the contraction kernels of gemm.hip
+// (reference: nn/layers/dense/operations_cpu_blas.h:36-228, nn_models/mlp/operations_generic.h:77-204).
+#include "common.h"
+#include "gemm.h"
+
+namespace {
+
+bool layer_ok(const rlt_dense_layer* L) {
+    return L && L->weights && L->biases && L->in_dim > 0 && L->out_dim > 0 && L->activation >= 0 && L->activation <= RLT_ACT_SIGMOID;
+}
+int max_dim(const rlt_dense_layer* layers, int n) {
+    int m = 1;
+    for (int i = 0; i < n; i++) { if (layers[i].out_dim > m) m = layers[i].out_dim; if (layers[i].in_dim > m) m = layers[i].in_dim; }
+    return m;
+}
+size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
+bool chain_ok(const rlt_dense_layer* layers, int n) {
+    if (!layers || n < 1) return false;
+    for (int i = 0; i < n; i++) { if (!layer_ok(&layers[i])) return false; if (i > 0 && layers[i].in_dim != layers[i - 1].out_dim) return false; }
+    return true;
+}
+
+__global__ __launch_bounds__(256) void zero_kernel(float* __restrict__ a, size_t na, float* __restrict__ b, size_t nb) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < na + nb; i += (size_t)gridDim.x * blockDim.x) {
+        if (i < na) a[i] = 0.0f; else b[i - na] = 0.0f;
+    }
+}
+// d = (y - target) * scale  (nn/loss_functions/mse/operations_generic.h:41-56 with scale = 2/(rows*cols)*w)
+__global__ __launch_bounds__(256) void mse_d_kernel(const float* __restrict__ y, int ldy, const float* __restrict__ t, int ldt, float* __restrict__ d, int ldd,
+                                                    int rows, int cols, float scale) {
+    const size_t total = (size_t)rows * cols;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        size_t r = i / cols, c = i % cols;
+        d[r * ldd + c] = (y[r * ldy + c] - t[r * ldt + c]) * scale;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int rlt_rocm_dense_evaluate(rlt_rocm_device* device, const rlt_dense_layer* L, const float* x, int ldx, float* y, int ldy, int batch) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(layer_ok(L) && x && y && batch > 0 && ldx >= L->in_dim && ldy >= L->out_dim);
+    return rlt_gemm_forward(device, x, ldx, L->weights, L->biases, L->activation, nullptr, nullptr, y, ldy, batch, L->in_dim, L->out_dim);
+}
+int rlt_rocm_dense_forward(rlt_rocm_device* device, const rlt_dense_layer* L, const float* x, int ldx, float* y, int ldy, int batch) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(layer_ok(L) && L->pre_activations && x && batch > 0 && ldx >= L->in_dim && (!y || ldy >= L->out_dim));
+    return rlt_gemm_forward(device, x, ldx, L->weights, L->biases, L->activation, L->pre_activations, L->output, y, ldy, batch, L->in_dim, L->out_dim);
+}
+int rlt_rocm_dense_backward_input(rlt_rocm_device* device, const rlt_dense_layer* L, float* d_output, int ldd, float* d_input, int ldi, int batch) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(layer_ok(L) && L->pre_activations && d_output && d_input && batch > 0 && ldd >= L->out_dim && ldi >= L->in_dim);
+    int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, L->pre_activations, batch, L->out_dim, L->activation);
+    if (rc) return rc;
+    return rlt_gemm_backward_input(device, d_output, ldd, L->weights, d_input, ldi, nullptr, 0, batch, L->in_dim, L->out_dim);
+}
+int rlt_rocm_dense_backward(rlt_rocm_device* device, const rlt_dense_layer* L, const float* x, int ldx, float* d_output, int ldd, int batch) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(layer_ok(L) && L->pre_activations && L->d_weights && L->d_biases && x && d_output && batch > 0 && ldd >= L->out_dim && ldx >= L->in_dim);
+    int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, L->pre_activations, batch, L->out_dim, L->activation);
+    if (rc) return rc;
+    return rlt_gemm_wgrad(device, d_output, ldd, x, ldx, L->d_weights, L->d_biases, batch, L->in_dim, L->out_dim);
+}
+int rlt_rocm_dense_backward_full(rlt_rocm_device* device, const rlt_dense_layer* L, const float* x, int ldx, float* d_output, int ldd,
+                                 float* d_input, int ldi, int batch) {
+    int rc = rlt_rocm_dense_backward(device, L, x, ldx, d_output, ldd, batch);
+    if (rc) return rc;
+    RLT_REQUIRE(d_input && ldi >= L->in_dim);
+    return rlt_gemm_backward_input(device, d_output, ldd, L->weights, d_input, ldi, nullptr, 0, batch, L->in_dim, L->out_dim);
+}
+
+size_t rlt_rocm_mlp_workspace_bytes(const rlt_dense_layer* layers, int n_layers, int batch) {
+    if (!layers || n_layers < 1 || batch < 1) return 0;
+    size_t per_row = 0;
+    for (int i = 0; i < n_layers; i++) per_row += 2 * (size_t)layers[i].out_dim;   // private pre/out of forward_backward
+    per_row += 3 * (size_t)max_dim(layers, n_layers);                                // tick, tock, upstream gradient copy
+    return align_up(per_row * (size_t)batch * sizeof(float)) + 4 * 256;
+}
+
+int rlt_rocm_mlp_evaluate(rlt_rocm_device* device, const rlt_dense_layer* layers, int n, const float* x, int ldx, float* y, int ldy, int batch,
+                          void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(chain_ok(layers, n) && x && y && batch > 0 && ldx >= layers[0].in_dim && ldy >= layers[n - 1].out_dim);
+    const size_t buf = align_up((size_t)batch * max_dim(layers, n) * sizeof(float));
+    RLT_REQUIRE(n == 1 || (workspace && workspace_bytes >= 2 * buf));
+    float* tick = (float*)workspace; float* tock = (float*)((char*)workspace + buf);
+    const float* in = x; int ldin = ldx;
+    for (int l = 0; l < n; l++) {
+        float* out = (l == n - 1) ? y : ((l % 2 == 0) ? tick : tock);
+        int ldo = (l == n - 1) ? ldy : layers[l].out_dim;
+        int rc = rlt_gemm_forward(device, in, ldin, layers[l].weights, layers[l].biases, layers[l].activation, nullptr, nullptr, out, ldo, batch, layers[l].in_dim, layers[l].out_dim);
+        if (rc) return rc;
+        in = out; ldin = ldo;
+    }
+    return 0;
+}
+
+int rlt_rocm_mlp_forward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n, const float* x, int ldx, int batch) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(chain_ok(layers, n) && x && batch > 0 && ldx >= layers[0].in_dim);
+    for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].pre_activations && layers[l].output);
+    const float* in = x; int ldin = ldx;
+    for (int l = 0; l < n; l++) {
+        int rc = rlt_gemm_forward(device, in, ldin, layers[l].weights, layers[l].biases, layers[l].activation, layers[l].pre_activations, layers[l].output,
+                                  nullptr, 0, batch, layers[l].in_dim, layers[l].out_dim);
+        if (rc) return rc;
+        in = layers[l].output; ldin = layers[l].out_dim;
+    }
+    return 0;
+}
+
+// Shared by mlp_backward and mlp_forward_backward. d_pre_last: [batch x out] holding the LAST layer's d_pre already.
+static int mlp_backward_from_dpre(rlt_rocm_device* device, const rlt_dense_layer* layers, int n, const float* x, int ldx,
+                                  float* d_pre_last, int ldd, float* d_input, int ldi, int batch, int want_w, float* tick, float* tock) {
+    float* d_pre = d_pre_last; int ld_pre = ldd;
+    for (int l = n - 1; l >= 0; l--) {
+        const rlt_dense_layer& L = layers[l];
+        const float* in = (l == 0) ? x : layers[l - 1].output; int ldin = (l == 0) ? ldx : layers[l - 1].out_dim;
+        if (want_w) {
+            int rc = rlt_gemm_wgrad(device, d_pre, ld_pre, in, ldin, L.d_weights, L.d_biases, batch, L.in_dim, L.out_dim);
+            if (rc) return rc;
+        }
+        if (l > 0) {
+            // d_input of this layer becomes d_pre of the layer below: the activation derivative is applied in the epilogue
+            float* d_in = ((n - 1 - l) % 2 == 0) ? tick : tock;
+            int rc = rlt_gemm_backward_input(device, d_pre, ld_pre, L.weights, d_in, L.in_dim, layers[l - 1].pre_activations, layers[l - 1].activation,
+                                             batch, L.in_dim, L.out_dim);
+            if (rc) return rc;
+            d_pre = d_in; ld_pre = L.in_dim;
+        } else if (d_input) {
+            int rc = rlt_gemm_backward_input(device, d_pre, ld_pre, L.weights, d_input, ldi, nullptr, 0, batch, L.in_dim, L.out_dim);
+            if (rc) return rc;
+        }
+    }
+    return 0;
+}
+
+int rlt_rocm_mlp_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n, const float* x, int ldx, float* d_output, int ldd,
+                          float* d_input, int ldi, int batch, int want_w, void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(chain_ok(layers, n) && d_output && batch > 0 && ldd >= layers[n - 1].out_dim);
+    RLT_REQUIRE(!want_w || (x && ldx >= layers[0].in_dim));
+    RLT_REQUIRE(want_w || d_input);
+    RLT_REQUIRE(!d_input || ldi >= layers[0].in_dim);
+    for (int l = 0; l < n; l++) {
+        RLT_REQUIRE(layers[l].pre_activations);
+        if (want_w) RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases && (l == n - 1 || layers[l].output));
+    }
+    const size_t buf = align_up((size_t)batch * max_dim(layers, n) * sizeof(float));
+    RLT_REQUIRE(n == 1 || (workspace && workspace_bytes >= 2 * buf));
+    float* tick = (float*)workspace; float* tock = (float*)((char*)workspace + buf);
+    const rlt_dense_layer& last = layers[n - 1];
+    int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, last.pre_activations, batch, last.out_dim, last.activation);
+    if (rc) return rc;
+    return mlp_backward_from_dpre(device, layers, n, x, ldx, d_output, ldd, d_input, ldi, batch, want_w, tick, tock);
+}
+
+int rlt_rocm_mlp_zero_gradient(rlt_rocm_device* device, const rlt_dense_layer* layers, int n) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(layers && n >= 1);
+    for (int l = 0; l < n; l++) {
+        RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases && layers[l].in_dim > 0 && layers[l].out_dim > 0);
+        size_t nw = (size_t)layers[l].in_dim * layers[l].out_dim, nb = layers[l].out_dim;
+        int blocks = (int)((nw + nb + 255) / 256); if (blocks > 1024) blocks = 1024;
+        hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, device->stream, layers[l].d_weights, nw, layers[l].d_biases, nb);
+        int rc = rlt_launch_status(device);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+int rlt_rocm_mlp_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n, const float* x, int ldx, float* y, int ldy,
+                                  const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch,
+                                  void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(chain_ok(layers, n) && x && batch > 0 && ldx >= layers[0].in_dim && (d_output || target));
+    const int O = layers[n - 1].out_dim;
+    RLT_REQUIRE((!y || ldy >= O) && (!d_output || ldd >= O) && (!target || ldt >= O));
+    for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases);
+    RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_mlp_workspace_bytes(layers, n, batch));
+    // carve private activation storage out of the workspace
+    rlt_dense_layer priv[16];
+    RLT_REQUIRE(n <= 16);
+    char* w = (char*)workspace;
+    const size_t buf = align_up((size_t)batch * max_dim(layers, n) * sizeof(float));
+    float* tick = (float*)w; w += buf; float* tock = (float*)w; w += buf; float* dlast = (float*)w; w += buf;
+    for (int l = 0; l < n; l++) {
+        priv[l] = layers[l];
+        priv[l].pre_activations = (float*)w; w += (size_t)batch * layers[l].out_dim * sizeof(float);
+        priv[l].output = (float*)w; w += (size_t)batch * layers[l].out_dim * sizeof(float);
+    }
+    const float* in = x; int ldin = ldx;
+    for (int l = 0; l < n; l++) {
+        int rc = rlt_gemm_forward(device, in, ldin, priv[l].weights, priv[l].biases, priv[l].activation, priv[l].pre_activations, priv[l].output,
+                                  (l == n - 1) ? y : nullptr, ldy, batch, priv[l].in_dim, priv[l].out_dim);
+        if (rc) return rc;
+        in = priv[l].output; ldin = priv[l].out_dim;
+    }
+    const rlt_dense_layer& last = priv[n - 1];
+    int rc;
+    if (target) {
+        size_t total = (size_t)batch * O; int blocks = (int)((total + 255) / 256); if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(mse_d_kernel, dim3(blocks), dim3(256), 0, device->stream, last.output, O, target, ldt, dlast, O, batch, O, mse_scale);
+        if ((rc = rlt_launch_status(device))) return rc;
+        if ((rc = rlt_dpre(device, dlast, O, dlast, O, last.pre_activations, batch, O, last.activation))) return rc;
+    } else {
+        if ((rc = rlt_dpre(device, d_output, ldd, dlast, O, last.pre_activations, batch, O, last.activation))) return rc;
+    }
+    return mlp_backward_from_dpre(device, priv, n, x, ldx, dlast, O, nullptr, 0, batch, 1, tick, tock);
+}
+
+}  // extern "C"

@@ -1,0 +1,150 @@
+// Adam step (moments, bias correction, parameter update, optional polyak target and gradient norm) for a list of
+// parameter tensors in one launch, and the polyak soft update.
+// reference: nn/optimizers/adam/operations_generic.h:43-66, instance/operations_generic.h:26-72,
+//            utils/polyak/operations_generic.h:11-43; CUDA counterparts adam/operations_cuda.h:18-68 (scalar kernel for the
+//            bias corrections), nn/layers/dense/operations_cuda.h:195-233 (one launch per layer).
+#include "common.h"
+
+namespace {
+
+constexpr int MAX_T = 12;
+struct AdamLaunch {
+    rlt_adam_tensor t[MAX_T];
+    uint32_t prefix[MAX_T + 1];
+    int n;
+    rlt_adam_parameters p;
+    float polyak;
+    uint32_t* age;
+    uint32_t* done_counter;      // zero between launches
+    float* block_partials;       // [gridDim.x] sums of squared gradients
+    float* out_sq_norm;          // optional
+    int increment_age;
+    int accumulate_norm;         // add to *out_sq_norm instead of overwriting (later chunks of one step)
+};
+
+__global__ __launch_bounds__(256) void adam_kernel(AdamLaunch a) {
+    const uint32_t age = *a.age;
+    // bias corrections from the un-incremented age (adam/operations_generic.h:49-58)
+    const float bc1 = 1.0f / (1.0f - powf(a.p.beta_1, (float)age));
+    const float bc2 = 1.0f / (1.0f - powf(a.p.beta_2, (float)age));
+    const uint32_t total = a.prefix[a.n];
+    float sq = 0.0f;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        int ti = 0;
+#pragma unroll
+        for (int k = 1; k < MAX_T; k++) ti += (k < a.n && i >= a.prefix[k]) ? 1 : 0;
+        const rlt_adam_tensor& T = a.t[ti];
+        const uint32_t j = i - a.prefix[ti];
+        float g = T.gradient[j];
+        sq += g * g;
+        if (a.p.enable_gradient_clipping) g = fminf(fmaxf(g, -a.p.gradient_clip_value), a.p.gradient_clip_value);
+        float m = a.p.beta_1 * T.first_moment[j] + (1.0f - a.p.beta_1) * g;
+        float v = a.p.beta_2 * T.second_moment[j] + (1.0f - a.p.beta_2) * g * g;
+        T.first_moment[j] = m; T.second_moment[j] = v;
+        float pre_sqrt = fmaxf(v * bc2, a.p.epsilon_sqrt);
+        float update = a.p.alpha * bc1 * m / (sqrtf(pre_sqrt) + a.p.epsilon);
+        float param = T.parameters[j];
+        if ((T.flags & 2u) && a.p.enable_bias_lr_factor) update *= a.p.bias_lr_factor;
+        if ((T.flags & 1u) && a.p.enable_weight_decay) update += param * a.p.weight_decay / 2.0f;
+        param -= update;
+        T.parameters[j] = param;
+        if (T.polyak_target) T.polyak_target[j] = a.polyak * T.polyak_target[j] + (1.0f - a.polyak) * param;
+    }
+    // gradient norm + age increment: the last workgroup to finish has seen every other one read `age`
+    __shared__ float partial[4];
+    __shared__ bool last;
+    sq = rlt_wave_sum(sq);
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = sq;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        a.block_partials[blockIdx.x] = partial[0] + partial[1] + partial[2] + partial[3];
+        __threadfence();
+        uint32_t ticket = atomicAdd(a.done_counter, 1u);
+        last = (ticket == gridDim.x - 1);
+    }
+    __syncthreads();
+    if (last && threadIdx.x == 0) {
+        __threadfence();
+        if (a.out_sq_norm) {
+            float s = a.accumulate_norm ? *a.out_sq_norm : 0.0f;
+            for (uint32_t b = 0; b < gridDim.x; b++) s += ((volatile float*)a.block_partials)[b];
+            *a.out_sq_norm = s;
+        }
+        if (a.increment_age) *a.age = age + 1;
+        *a.done_counter = 0;
+    }
+}
+
+__global__ __launch_bounds__(256) void adam_reset_kernel(AdamLaunch a) {
+    const uint32_t total = a.prefix[a.n];
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        int ti = 0;
+#pragma unroll
+        for (int k = 1; k < MAX_T; k++) ti += (k < a.n && i >= a.prefix[k]) ? 1 : 0;
+        const uint32_t j = i - a.prefix[ti];
+        a.t[ti].first_moment[j] = 0.0f; a.t[ti].second_moment[j] = 0.0f;
+    }
+    if (a.increment_age && blockIdx.x == 0 && threadIdx.x == 0) *a.age = 1;
+}
+
+__global__ __launch_bounds__(256) void polyak_kernel(const float* __restrict__ source, float* __restrict__ target, size_t count, float polyak, int squared) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) {
+        float s = source[i];
+        target[i] = squared ? polyak * target[i] + (1.0f - polyak) * s * s : polyak * target[i] + (1.0f - polyak) * s;
+    }
+}
+
+}  // namespace
+
+// Layout of the device handle's scratch for this file: [0,256) the done counter, [256, ...) block partials.
+static int adam_launch(rlt_rocm_device* device, const rlt_adam_tensor* tensors, int n_tensors, const rlt_adam_parameters* p, uint32_t* age,
+                       float polyak, float* out_sq_norm, bool reset) {
+    void* counters = nullptr;
+    int rc = rlt_counters(device, &counters);
+    if (rc) return rc;
+    for (int base = 0; base < n_tensors; base += MAX_T) {
+        AdamLaunch a = {};
+        a.n = n_tensors - base < MAX_T ? n_tensors - base : MAX_T;
+        uint32_t total = 0;
+        for (int i = 0; i < a.n; i++) {
+            const rlt_adam_tensor& T = tensors[base + i];
+            if (!T.first_moment || !T.second_moment || (!reset && (!T.parameters || !T.gradient)) || T.count == 0) return RLT_E_INVALID_ARGUMENT;
+            a.t[i] = T; a.prefix[i] = total; total += T.count;
+        }
+        for (int i = a.n; i <= MAX_T; i++) a.prefix[i] = total;
+        if (p) a.p = *p;
+        a.polyak = polyak; a.age = age;
+        a.done_counter = (uint32_t*)counters; a.block_partials = (float*)((char*)counters + 256);
+        a.out_sq_norm = out_sq_norm; a.accumulate_norm = base > 0;
+        a.increment_age = (base + MAX_T >= n_tensors);
+        int blocks = (int)((total + 255) / 256); if (blocks > 960) blocks = 960; if (blocks < 1) blocks = 1;
+        if (reset) hipLaunchKernelGGL(adam_reset_kernel, dim3(blocks), dim3(256), 0, device->stream, a);
+        else hipLaunchKernelGGL(adam_kernel, dim3(blocks), dim3(256), 0, device->stream, a);
+        if ((rc = rlt_launch_status(device))) return rc;
+    }
+    return 0;
+}
+
+extern "C" {
+
+int rlt_rocm_adam_step(rlt_rocm_device* device, const rlt_adam_tensor* tensors_host, int n_tensors, const rlt_adam_parameters* parameters_host,
+                       uint32_t* age, float polyak, float* out_gradient_squared_norm) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(tensors_host && n_tensors > 0 && parameters_host && age);
+    return adam_launch(device, tensors_host, n_tensors, parameters_host, age, polyak, out_gradient_squared_norm, false);
+}
+int rlt_rocm_adam_reset(rlt_rocm_device* device, const rlt_adam_tensor* tensors_host, int n_tensors, uint32_t* age) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(tensors_host && n_tensors > 0 && age);
+    return adam_launch(device, tensors_host, n_tensors, nullptr, age, 0.0f, nullptr, true);
+}
+int rlt_rocm_polyak_update(rlt_rocm_device* device, const float* source, float* target, size_t count, float polyak, int squared) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(source && target);
+    if (count == 0) return 0;
+    size_t b = (count + 255) / 256; if (b > 960) b = 960;
+    hipLaunchKernelGGL(polyak_kernel, dim3((int)b), dim3(256), 0, device->stream, source, target, count, polyak, squared);
+    return rlt_launch_status(device);
+}
+
+}  // extern "C"

@@ -1,0 +1,300 @@
+"""Shared test plumbing: loads the package and the CPU checker, and builds the same network / agent descriptors on
+either of them so that one test body drives both."""
+import ctypes as C
+import importlib.util
+import os
+import subprocess
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_LIB = os.path.join(ORACLE_DIR, "librlt_oracle.so")
+REF_GENERIC = os.path.join(ORACLE_DIR, "_ref", "librlt_ref_generic.so")
+REF_BLAS = os.path.join(ORACLE_DIR, "_ref", "librlt_ref_blas.so")
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def package():
+    """The package directory is called `rl-tools_amd`; import it under an importable name."""
+    if "rl_tools_amd" in sys.modules:
+        return sys.modules["rl_tools_amd"]
+    path = os.path.join(ROOT, "rl-tools_amd")
+    spec = importlib.util.spec_from_file_location("rl_tools_amd", os.path.join(path, "__init__.py"), submodule_search_locations=[path])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules["rl_tools_amd"] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+capi = package().capi
+
+
+def build_oracle():
+    if not os.path.exists(ORACLE_LIB) or os.path.getmtime(ORACLE_LIB) < max(
+            os.path.getmtime(os.path.join(ORACLE_DIR, f)) for f in ("rlt_oracle.cpp", "rlt_oracle_sac_loop.cpp", "rlt_oracle.h")):
+        subprocess.run(["make", "-C", ORACLE_DIR, ORACLE_LIB], check=True, capture_output=True)
+    return ORACLE_LIB
+
+
+class LoopConfig(C.Structure):
+    _fields_ = [("seed", C.c_uint32), ("batch", C.c_int32), ("hidden_dim", C.c_int32), ("replay_capacity", C.c_int32),
+                ("n_warmup_steps", C.c_int32), ("episode_step_limit", C.c_int32), ("adam_epsilon", C.c_float)]
+
+
+def load_oracle():
+    lib = C.CDLL(build_oracle())
+    P, S, I = C.c_void_p, C.c_size_t, C.c_int
+    for name, args in capi.PROTOTYPES.items():
+        a = list(args)
+        if name in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward"):
+            a = a[:-2]      # the CPU checker allocates its own workspace
+        fn = getattr(lib, "rlt_oracle_" + name)
+        fn.argtypes = a
+        fn.restype = I
+    lib.rlt_oracle_set_f64_accumulate.argtypes = [I]
+    lib.rlt_oracle_use_cblas.argtypes = [C.c_char_p]
+    lib.rlt_oracle_cblas_name.restype = C.c_char_p
+    lib.rlt_oracle_activation.argtypes = [C.c_float, I]; lib.rlt_oracle_activation.restype = C.c_float
+    lib.rlt_oracle_d_activation.argtypes = [C.c_float, I]; lib.rlt_oracle_d_activation.restype = C.c_float
+    lib.rlt_oracle_pendulum_runner_step.argtypes = [C.POINTER(capi.PendulumRunner), C.POINTER(capi.ReplayBuffer), I, C.POINTER(capi.DenseLayer), I,
+                                                    C.POINTER(capi.SasParameters), P, P, P]
+    lib.rlt_oracle_sac_loop_create.argtypes = [C.POINTER(LoopConfig)]; lib.rlt_oracle_sac_loop_create.restype = P
+    for f in ("destroy", "step"):
+        getattr(lib, "rlt_oracle_sac_loop_" + f).argtypes = [P]
+    lib.rlt_oracle_sac_loop_agent.argtypes = [P]; lib.rlt_oracle_sac_loop_agent.restype = C.POINTER(capi.SacAgent)
+    lib.rlt_oracle_sac_loop_replay.argtypes = [P]; lib.rlt_oracle_sac_loop_replay.restype = C.POINTER(capi.ReplayBuffer)
+    lib.rlt_oracle_sac_loop_runner.argtypes = [P]; lib.rlt_oracle_sac_loop_runner.restype = C.POINTER(capi.PendulumRunner)
+    for f in ("noise_critic", "noise_actor"):
+        getattr(lib, "rlt_oracle_sac_loop_" + f).argtypes = [P]; getattr(lib, "rlt_oracle_sac_loop_" + f).restype = C.POINTER(C.c_float)
+    for f in ("env_indices", "sample_offsets"):
+        getattr(lib, "rlt_oracle_sac_loop_" + f).argtypes = [P]; getattr(lib, "rlt_oracle_sac_loop_" + f).restype = C.POINTER(C.c_uint32)
+    lib.rlt_oracle_sac_loop_step_count.argtypes = [P]; lib.rlt_oracle_sac_loop_step_count.restype = C.c_uint32
+    lib.rlt_oracle_sac_loop_critic_loss.argtypes = [P, I]; lib.rlt_oracle_sac_loop_critic_loss.restype = C.c_float
+    lib.rlt_oracle_sac_loop_last_env_step.argtypes = [P, P]
+    lib.rlt_oracle_sac_loop_parameter_count.argtypes = [P]; lib.rlt_oracle_sac_loop_parameter_count.restype = S
+    lib.rlt_oracle_sac_loop_get_parameters.argtypes = [P, P]
+    return lib
+
+
+class HostArray:
+    def __init__(self, a):
+        self.a = np.ascontiguousarray(a).copy()
+        self.shape, self.dtype = self.a.shape, self.a.dtype
+        self.ptr = self.a.ctypes.data
+
+    def numpy(self):
+        return self.a.copy()
+
+    def upload(self, x):
+        self.a[...] = np.asarray(x, dtype=self.dtype).reshape(self.a.shape)
+        return self
+
+    def offset(self, elements):
+        return self.ptr + int(elements) * self.dtype.itemsize
+
+
+class HostBackend:
+    """The CPU checker (oracle/): host pointers, no device handle, no workspaces."""
+    name = "oracle"
+
+    def __init__(self):
+        self.lib = load_oracle()
+
+    def array(self, a):
+        return HostArray(a)
+
+    def zeros(self, shape, dtype=np.float32):
+        return HostArray(np.zeros(shape, dtype))
+
+    def call(self, fn, *args):
+        if fn in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward"):
+            args = args[:-2]
+        rc = getattr(self.lib, "rlt_oracle_" + fn)(*args)
+        if rc != 0:
+            raise RuntimeError(f"rlt_oracle_{fn} returned {rc}")
+
+    def workspace(self, nbytes):
+        return None, 0
+
+    def sync(self):
+        pass
+
+
+class RocmBackend:
+    """The HIP library through its C ABI."""
+    name = "rocm"
+
+    def __init__(self):
+        self.device = package().Device(0)
+        self._ws = None
+
+    def array(self, a):
+        return self.device.array(np.ascontiguousarray(a))
+
+    def zeros(self, shape, dtype=np.float32):
+        return self.device.zeros(shape, dtype)
+
+    def call(self, fn, *args):
+        self.device.call(fn, *args)
+
+    def workspace(self, nbytes):
+        nbytes = int(nbytes)
+        if self._ws is None or self._ws.nbytes < nbytes:
+            self._ws = self.device.empty((nbytes,), np.uint8)
+        return self._ws.ptr, self._ws.nbytes
+
+    def sync(self):
+        self.device.sync()
+
+    def close(self):
+        self.device.close()
+
+
+def mlp_param_count(dims):
+    return sum(dims[i] * dims[i + 1] + dims[i + 1] for i in range(len(dims) - 1))
+
+
+def xavier_params(rng, dims):
+    """Xavier-uniform weights, zero biases, flattened per layer as [weights, biases]."""
+    parts = []
+    for i in range(len(dims) - 1):
+        bound = np.sqrt(6.0 / (dims[i] + dims[i + 1]))
+        parts.append(rng.uniform(-bound, bound, size=dims[i + 1] * dims[i]).astype(np.float32))
+        parts.append(np.zeros(dims[i + 1], np.float32))
+    return np.concatenate(parts)
+
+
+def random_params(rng, dims, bias_scale=0.1):
+    parts = []
+    for i in range(len(dims) - 1):
+        bound = 1.0 / np.sqrt(dims[i])
+        parts.append(rng.uniform(-bound, bound, size=dims[i + 1] * dims[i]).astype(np.float32))
+        parts.append(rng.uniform(-bias_scale, bias_scale, size=dims[i + 1]).astype(np.float32))
+    return np.concatenate(parts)
+
+
+class Mlp:
+    """A dense network laid out as flat arenas (parameters, gradients, Adam moments) on a backend, described to the C ABI
+    by an array of rlt_dense_layer."""
+
+    def __init__(self, backend, dims, params, batch, hidden_act="relu", out_act="identity", trainable=True):
+        self.backend, self.dims, self.batch, self.trainable = backend, list(dims), batch, trainable
+        self.n = len(dims) - 1
+        total = mlp_param_count(dims)
+        assert params.size == total
+        self.params = backend.array(params.astype(np.float32))
+        if trainable:
+            self.grads = backend.zeros((total,)); self.m = backend.zeros((total,)); self.v = backend.zeros((total,))
+            self.pre = [backend.zeros((batch, dims[i + 1])) for i in range(self.n)]
+            self.out = [backend.zeros((batch, dims[i + 1])) for i in range(self.n)]
+            self.age = backend.array(np.array([1], np.uint32))
+        self.layers = (capi.DenseLayer * self.n)()
+        adam = []
+        off = 0
+        self.offsets = []
+        for i in range(self.n):
+            nw, nb = dims[i] * dims[i + 1], dims[i + 1]
+            L = self.layers[i]
+            L.in_dim, L.out_dim = dims[i], dims[i + 1]
+            L.activation = capi.ACT[out_act if i == self.n - 1 else hidden_act]
+            L.weights, L.biases = self.params.offset(off), self.params.offset(off + nw)
+            if trainable:
+                L.d_weights, L.d_biases = self.grads.offset(off), self.grads.offset(off + nw)
+                L.pre_activations, L.output = self.pre[i].ptr, self.out[i].ptr
+                adam.append(capi.AdamTensor(L.weights, L.d_weights, self.m.offset(off), self.v.offset(off), None, nw, 1))
+                adam.append(capi.AdamTensor(L.biases, L.d_biases, self.m.offset(off + nw), self.v.offset(off + nw), None, nb, 2))
+            self.offsets.append((off, nw, nb))
+            off += nw + nb
+        self.adam = (capi.AdamTensor * len(adam))(*adam)
+        self.n_adam = len(adam)
+
+    def workspace(self):
+        if self.backend.name == "oracle":
+            return None, 0
+        nbytes = self.backend.device.lib.rlt_rocm_mlp_workspace_bytes(self.layers, self.n, self.batch)
+        return self.backend.workspace(nbytes)
+
+
+class ReplayOnBackend:
+    def __init__(self, backend, n_envs, capacity, obs_dim=3, act_dim=1):
+        self.backend = backend
+        self.row = 2 * obs_dim + act_dim + 3
+        self.data = backend.zeros((n_envs * capacity, self.row))
+        self.episode_start = backend.zeros((n_envs * capacity,), np.uint32)
+        self.position = backend.zeros((n_envs,), np.uint32)
+        self.current_episode_start = backend.zeros((n_envs,), np.uint32)
+        self.full = backend.zeros((n_envs,), np.uint8)
+        self.c = capi.ReplayBuffer(self.data.ptr, self.episode_start.ptr, self.position.ptr, self.current_episode_start.ptr, self.full.ptr,
+                                   n_envs, capacity, obs_dim, act_dim)
+
+
+class SacOnBackend:
+    """All SAC state for the Pendulum shapes (observation 3, action 1) on one backend."""
+
+    def __init__(self, backend, batch, hidden, params, adam_eps=1e-7, masks=True):
+        OBS, ACT, D = 3, 1, 4
+        self.backend, self.batch = backend, batch
+        n_actor = mlp_param_count([OBS, hidden, hidden, 2 * ACT]); n_critic = mlp_param_count([D, hidden, hidden, 1])
+        o = 0
+        self.actor = Mlp(backend, [OBS, hidden, hidden, 2 * ACT], params[o:o + n_actor], batch); o += n_actor
+        self.critics = []
+        for _ in range(2):
+            self.critics.append(Mlp(backend, [D, hidden, hidden, 1], params[o:o + n_critic], batch)); o += n_critic
+        self.targets = []
+        for _ in range(2):
+            self.targets.append(Mlp(backend, [D, hidden, hidden, 1], params[o:o + n_critic], batch, trainable=False)); o += n_critic
+        self.log_alpha = backend.array(np.array([params[o], 0, 0, 0], np.float32))
+        self.alpha_age = backend.array(np.array([1], np.uint32))
+        z = backend.zeros
+        self.oab = z((2, batch, D)); self.rewards = z((batch,)); self.terminated = z((batch,), np.uint8)
+        self.m_final = backend.array(np.ones(batch, np.uint8)); self.m_next_final = backend.array(np.ones(batch, np.uint8))
+        self.m_reset = backend.array(np.ones(batch, np.uint8))
+        self.nsavi = z((batch, D)); self.next_q = [z((batch,)), z((batch,))]; self.next_lp = z((batch,)); self.target_q = z((batch,))
+        self.d_out_c = [z((batch,)), z((batch,))]; self.savi = z((batch, D)); self.d_out_a = z((batch,))
+        self.d_ci = [z((batch, D)), z((batch, D))]; self.d_aos = z((batch, ACT)); self.d_ao = z((batch, 2 * ACT))
+        self.a_pre = z((batch, ACT)); self.a_lp = z((batch,)); self.a_act = z((batch, ACT))
+        A = capi.SacAgent()
+        A.batch, A.observation_dim, A.action_dim, A.n_actor_layers, A.n_critic_layers = batch, OBS, ACT, 3, 3
+        A.gamma, A.polyak = 0.99, float(np.float32(1.0 - 0.005))
+        A.sas = capi.SasParameters(-20.0, 2.0, 1e-6, -float(ACT))
+        A.actor_adam = A.critic_adam = A.alpha_adam = capi.adam_parameters(epsilon=adam_eps)
+        A.actor = self.actor.layers
+        A.actor_adam_tensors, A.n_actor_adam_tensors = self.actor.adam, self.actor.n_adam
+        for k in range(2):
+            A.critics[k] = self.critics[k].layers; A.critics_target[k] = self.targets[k].layers
+            A.critic_adam_tensors[k] = self.critics[k].adam; A.critic_age[k] = self.critics[k].age.ptr
+            A.next_q[k] = self.next_q[k].ptr; A.d_output_critic[k] = self.d_out_c[k].ptr; A.d_critic_input[k] = self.d_ci[k].ptr
+        A.n_critic_adam_tensors = self.critics[0].n_adam
+        la = self.log_alpha
+        A.log_alpha = capi.AdamTensor(la.offset(0), la.offset(1), la.offset(2), la.offset(3), None, 1, 0)
+        A.actor_age, A.alpha_age = self.actor.age.ptr, self.alpha_age.ptr
+        A.observations_actions_base, A.rewards, A.terminated = self.oab.ptr, self.rewards.ptr, self.terminated.ptr
+        if masks:
+            A.final_step_mask, A.next_final_step_mask, A.reset = self.m_final.ptr, self.m_next_final.ptr, self.m_reset.ptr
+        A.next_state_action_value_input, A.next_log_probabilities, A.target_action_value = self.nsavi.ptr, self.next_lp.ptr, self.target_q.ptr
+        A.state_action_value_input, A.d_output_actor_critics = self.savi.ptr, self.d_out_a.ptr
+        A.d_actor_output_squashing, A.d_actor_output = self.d_aos.ptr, self.d_ao.ptr
+        A.actor_pre_squashing, A.actor_log_probabilities, A.actor_actions = self.a_pre.ptr, self.a_lp.ptr, self.a_act.ptr
+        if backend.name == "rocm":
+            lib = backend.device.lib
+            nbytes = max(lib.rlt_rocm_mlp_workspace_bytes(self.actor.layers, 3, batch), lib.rlt_rocm_mlp_workspace_bytes(self.critics[0].layers, 3, batch))
+            nbytes += batch * 2 * ACT * 4 + 1024
+            self.ws = backend.device.empty((nbytes,), np.uint8)
+            A.workspace, A.workspace_bytes = self.ws.ptr, self.ws.nbytes
+        self.c = A
+
+    def parameters(self):
+        parts = [self.actor.params.numpy()] + [c.params.numpy() for c in self.critics] + [t.params.numpy() for t in self.targets]
+        return np.concatenate(parts + [self.log_alpha.numpy()[:1]])
+
+    def set_batch(self, oab, rewards, terminated):
+        self.oab.upload(oab); self.rewards.upload(rewards); self.terminated.upload(terminated)
+
+
+def rel_err(a, ref):
+    """max |a - ref| relative to the largest magnitude of the reference tensor (per-tensor scale)."""
+    a = np.asarray(a, np.float64); ref = np.asarray(ref, np.float64)
+    scale = max(np.abs(ref).max(), 1e-30)
+    return np.abs(a - ref).max() / scale
