@@ -104,7 +104,8 @@ def test_replay_add_and_gather_bit_exact(oracle, rocm, n_envs, capacity, steps):
         for deterministic in ((1, 0) if n_envs == 1 else (0,)):
             oab, rew, term = b.array(np.full((2, B, 4), 7.0, np.float32)), b.zeros((B,)), b.zeros((B,), np.uint8)
             masks = [b.array(np.full(n, 9, np.uint8)) for n in (B, 2 * B, B, 2 * B)]
-            b.call("gather_batch", C.byref(rb.c), b.array(envs).ptr, b.array(offs).ptr, deterministic, 5, B, oab.ptr, rew.ptr, term.ptr, *[m.ptr for m in masks])
+            ed, od = b.array(envs), b.array(offs)
+            b.call("gather_batch", C.byref(rb.c), ed.ptr, od.ptr, deterministic, 5, B, oab.ptr, rew.ptr, term.ptr, *[m.ptr for m in masks])
             b.sync()
             got.append([oab.numpy(), rew.numpy(), term.numpy()] + [m.numpy() for m in masks])
         out.append((state, got))
