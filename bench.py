@@ -1,0 +1,232 @@
+#!/usr/bin/env python3
+"""Benchmark of the dense-network training hot path on one MI355X.
+
+Prints ONE JSON line. `value` is SAC loop steps per second at batch 256 on the Pendulum-shaped configuration (one loop step =
+1 environment step + replay add + gather of 256 transitions + 2 critic updates + target update + 1 actor update, i.e. 3 network
+updates), everything resident on the device, synthetic data. The same line carries the fused MLP forward+backward TFLOP/s at
+batch 65,536 (17->256->256->6) with its roofline fraction, and the reference CPU path timed on this host.
+"""
+import argparse
+import ctypes as C
+import importlib.util
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+FP32_PEAK_TFLOPS = 157.3
+MLP_FLOP_PER_SAMPLE_FWD = 2 * (17 * 256 + 256 * 256 + 256 * 6)                       # 142,848
+MLP_FLOP_PER_SAMPLE_BWD = 2 * (17 * 256 + 256 * 256 + 256 * 6) + 2 * (256 * 256 + 256 * 6)   # weight grads + d_input of layers 2,3: 276,992
+
+
+def package():
+    path = os.path.join(ROOT, "rl-tools_amd")
+    spec = importlib.util.spec_from_file_location("rl_tools_amd", os.path.join(path, "__init__.py"), submodule_search_locations=[path])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules["rl_tools_amd"] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+class HipEvents:
+    """hipEvent timing on the library's own stream (the kernels are not launched on any framework's current stream)."""
+
+    def __init__(self, stream):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.stream = C.c_void_p(stream)
+
+    def record(self):
+        e = C.c_void_p()
+        assert self.hip.hipEventCreate(C.byref(e)) == 0
+        assert self.hip.hipEventRecord(e, self.stream) == 0
+        return e
+
+    def elapsed_ms(self, a, b):
+        assert self.hip.hipEventSynchronize(b) == 0
+        ms = C.c_float()
+        assert self.hip.hipEventElapsedTime(C.byref(ms), a, b) == 0
+        return ms.value
+
+
+def bench_mlp(helpers, rocm, batch, iters, warmup):
+    capi = helpers.capi
+    dims = [17, 256, 256, 6]
+    rng = np.random.default_rng(0)
+    net = helpers.Mlp(rocm, dims, helpers.xavier_params(rng, dims), batch)
+    x = rocm.array(rng.standard_normal((batch, 17)).astype(np.float32))
+    dy = rocm.array(rng.standard_normal((batch, 6)).astype(np.float32))
+    y = rocm.zeros((batch, 6))
+    ws, wsn = net.workspace()
+    adam = capi.adam_parameters(epsilon=1e-8)
+    ev = HipEvents(rocm.device.lib.rlt_rocm_get_stream(rocm.device.handle))
+
+    def fwd_bwd():
+        rocm.call("mlp_forward_backward", net.layers, net.n, x.ptr, 17, y.ptr, 6, dy.ptr, 6, None, 0, 0.0, batch, ws, wsn)
+
+    def fwd():
+        rocm.call("mlp_forward", net.layers, net.n, x.ptr, 17, batch)
+
+    def step():
+        rocm.call("adam_step", net.adam, net.n_adam, C.byref(adam), net.age.ptr, 0.0, None)
+
+    out = {}
+    for name, fn in (("forward_backward", fwd_bwd), ("forward", fwd), ("adam", step)):
+        rocm.call("mlp_zero_gradient", net.layers, net.n)
+        for _ in range(warmup):
+            fn()
+        rocm.sync()
+        a = ev.record()
+        for _ in range(iters):
+            fn()
+        b = ev.record()
+        out[name + "_ms"] = ev.elapsed_ms(a, b) / iters
+    flop = (MLP_FLOP_PER_SAMPLE_FWD + MLP_FLOP_PER_SAMPLE_BWD) * batch
+    out["tflops"] = flop / (out["forward_backward_ms"] * 1e-3) / 1e12
+    out["batch"] = batch
+    return out
+
+
+def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000):
+    """SAC loop steps entirely on the device: runner step with the actor, device-side gather draws and noise, training."""
+    capi = helpers.capi
+    lib, h = rocm.device.lib, rocm.device.handle
+    rng = np.random.default_rng(1)
+    na, nc = helpers.mlp_param_count([3, 64, 64, 2]), helpers.mlp_param_count([4, 64, 64, 1])
+    critics = [helpers.random_params(rng, [4, 64, 64, 1]) for _ in range(2)]
+    params = np.concatenate([helpers.random_params(rng, [3, 64, 64, 2])] + critics + critics + [np.array([np.log(0.5)], np.float32)])
+    agent = helpers.SacOnBackend(rocm, batch, 64, params, masks=False)
+    rb = helpers.ReplayOnBackend(rocm, 1, capacity)
+    states, ep_step, ep_ret, trunc = rocm.zeros((1, 2)), rocm.zeros((1,), np.uint32), rocm.zeros((1,)), rocm.array(np.ones(1, np.uint8))
+    runner = capi.PendulumRunner(states.ptr, ep_step.ptr, ep_ret.ptr, trunc.ptr, 1, 200, capi.pendulum_parameters())
+    rollout_noise, warm_action = rocm.zeros((1, 1)), rocm.zeros((1, 1))
+    noise_c, noise_a = rocm.zeros((batch, 1)), rocm.zeros((batch, 1))
+    env_idx, offs = rocm.zeros((batch,), np.uint32), rocm.zeros((batch,), np.uint32)
+    seed = 1234
+    counter = [0]
+
+    def env_step(policy):
+        counter[0] += 1
+        c = counter[0]
+        if policy == 0:
+            rocm.check(lib.rlt_rocm_rand_f32(h, warm_action.ptr, 1, -1.0, 1.0, seed, 8 * c))
+        else:
+            rocm.check(lib.rlt_rocm_randn_f32(h, rollout_noise.ptr, 1, seed, 8 * c))
+        rocm.check(lib.rlt_rocm_pendulum_runner_step(h, C.byref(runner), C.byref(rb.c), 2 if policy else 0, agent.actor.layers, 3, C.byref(agent.c.sas),
+                                                     warm_action.ptr, rollout_noise.ptr, None, seed, 8 * c + 1))
+
+    rocm.check = rocm.device.check
+
+    def loop_step():
+        env_step(1)
+        c = counter[0]
+        rocm.check(lib.rlt_rocm_gather_draw(h, C.byref(rb.c), batch, seed, 8 * c + 2, env_idx.ptr, offs.ptr))
+        rocm.call("gather_batch", C.byref(rb.c), env_idx.ptr, offs.ptr, 0, 200, batch, agent.oab.ptr, agent.rewards.ptr, agent.terminated.ptr, None, None, None, None)
+        rocm.check(lib.rlt_rocm_randn_f32(h, noise_c.ptr, batch, seed, 8 * c + 3))
+        for k in range(2):
+            rocm.call("sac_train_critic", C.byref(agent.c), k, noise_c.ptr)
+        rocm.call("sac_update_critic_targets", C.byref(agent.c))
+        rocm.check(lib.rlt_rocm_randn_f32(h, noise_a.ptr, batch, seed, 8 * c + 4))
+        rocm.call("sac_train_actor", C.byref(agent.c), noise_a.ptr)
+
+    for _ in range(batch):        # fill the replay buffer with the warm-up policy
+        env_step(0)
+    for _ in range(warmup):
+        loop_step()
+    rocm.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loop_step()
+    rocm.sync()
+    dt = time.perf_counter() - t0
+    p = agent.parameters()
+    assert np.all(np.isfinite(p)), "SAC parameters went non-finite"
+    return {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3}
+
+
+def cpu_baseline(batch=256, seconds=12.0):
+    """The reference's own SAC loop (compiled from the reference, CBLAS backend, one thread) on this host; falls back to the
+    CPU restatement when that build is not present."""
+    ref = os.path.join(ROOT, "oracle", "_ref", "librlt_ref_blas.so")
+    cores = 1
+    if os.path.exists(ref):
+        lib = C.CDLL(ref)
+        lib.rlt_ref_sac_create.restype = C.c_void_p
+        lib.rlt_ref_sac_time_steps.restype = C.c_double
+        lib.rlt_ref_sac_time_steps.argtypes = [C.c_void_p, C.c_int]
+        lib.rlt_ref_cblas_name.restype = C.c_char_p
+        lib.rlt_ref_sac_destroy.argtypes = [C.c_void_p]
+        n, total, seed = 0, 0.0, 0
+        while total < seconds:                                  # the reference's loop stops at its STEP_LIMIT of 10,000 steps
+            hdl = C.c_void_p(lib.rlt_ref_sac_create(seed, batch)); seed += 1
+            lib.rlt_ref_sac_time_steps(hdl, batch + 50)         # warm-up policy phase + first training steps (untimed)
+            for _ in range(9):
+                total += lib.rlt_ref_sac_time_steps(hdl, 1000); n += 1000
+                if total >= seconds:
+                    break
+            lib.rlt_ref_sac_destroy(hdl)
+        return {"value": n / total, "unit": "loop steps/s", "cores": cores, "kind": "reference",
+                "sample": f"{n} post-warm-up loop steps of the reference's Pendulum SAC loop at batch {batch}, CBLAS = {os.path.basename(lib.rlt_ref_cblas_name().decode())}, 1 thread"}
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import helpers
+    o = helpers.HostBackend()
+    cfg = helpers.LoopConfig(0, batch, 64, 10000, batch, 200, 1e-7)
+    loop = C.c_void_p(o.lib.rlt_oracle_sac_loop_create(C.byref(cfg)))
+    for _ in range(batch + 10):
+        o.lib.rlt_oracle_sac_loop_step(loop)
+    n, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(50):
+            o.lib.rlt_oracle_sac_loop_step(loop)
+        n += 50
+    dt = time.perf_counter() - t0
+    return {"value": n / dt, "unit": "loop steps/s", "cores": cores, "kind": "port", "sample": f"{n} loop steps of the CPU restatement (plain loops) at batch {batch}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--mlp-batch", type=int, default=65536)
+    ap.add_argument("--mlp-iters", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["all", "mlp", "sac"], default="all")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the hot path has no cross-GPU part); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    package()
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import helpers
+    rocm = helpers.RocmBackend()
+    info = rocm.device.info()
+    mlp = bench_mlp(helpers, rocm, args.mlp_batch, args.mlp_iters, 3) if args.only in ("all", "mlp") else None
+    sac = bench_sac(helpers, rocm, args.steps, args.warmup) if args.only in ("all", "sac") else {"steps_per_s": 0.0, "ms_per_step": 0.0}
+    cpu = None if (args.no_cpu_baseline or args.only == "mlp") else cpu_baseline()
+    line = {
+        "metric": "SAC updates/sec (critic+actor) at batch 256; fused MLP fwd+bwd TFLOP/s",
+        "value": sac["steps_per_s"], "unit": "SAC loop steps/s (each = 2 critic + 1 actor update)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sac["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "SAC Pendulum loop step, batch 256, actor 3-64-64-2, critics 4-64-64-1, replay 10000; plus MLP 17-256-256-6 fwd+bwd at batch %d" % args.mlp_batch,
+                   "device": info["name"], "compute_units": info["compute_units"]},
+        "network_updates_per_s": 3 * sac["steps_per_s"],
+    }
+    if mlp:
+        line["mlp_fwd_bwd_tflops"] = mlp["tflops"]
+        line["mlp"] = mlp
+        flop = (MLP_FLOP_PER_SAMPLE_FWD + MLP_FLOP_PER_SAMPLE_BWD) * mlp["batch"]
+        line["roofline"] = {"bound": "mfma", "achieved": mlp["tflops"], "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": mlp["tflops"] / FP32_PEAK_TFLOPS,
+                            "traffic": None, "kernel": "mlp_forward_backward (all launches of one call)", "flop_per_launch": flop}
+    if cpu:
+        line["cpu_baseline"] = cpu
+        line["speedup_vs_cpu_baseline"] = sac["steps_per_s"] / cpu["value"] if cpu["value"] else None
+    print(json.dumps(line), flush=True)
+    rocm.close()
+
+
+if __name__ == "__main__":
+    main()

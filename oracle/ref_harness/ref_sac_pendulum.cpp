@@ -34,7 +34,7 @@ using TI = typename DEVICE::index_t;
 using PENDULUM_SPEC = rlt::rl::environments::pendulum::Specification<float, TI, rlt::rl::environments::pendulum::DefaultParameters<float>>;
 using ENVIRONMENT = rlt::rl::environments::Pendulum<PENDULUM_SPEC>;
 
-template <TI BATCH>
+template <TI BATCH, TI CAPACITY>
 struct LoopParameters : rlt::rl::algorithms::sac::loop::core::DefaultParameters<TYPE_POLICY, TI, ENVIRONMENT> {
     struct SAC_PARAMETERS : rlt::rl::algorithms::sac::DefaultParameters<TYPE_POLICY, TI, ENVIRONMENT::ACTION_DIM> {
         static constexpr TI ACTOR_BATCH_SIZE = BATCH;
@@ -44,15 +44,16 @@ struct LoopParameters : rlt::rl::algorithms::sac::loop::core::DefaultParameters<
     static constexpr TI N_WARMUP_STEPS_CRITIC = N_WARMUP_STEPS;
     static constexpr TI N_WARMUP_STEPS_ACTOR = N_WARMUP_STEPS;
     static constexpr TI STEP_LIMIT = 10000;
+    static constexpr TI REPLAY_BUFFER_CAP = CAPACITY;
     static constexpr TI ACTOR_NUM_LAYERS = 3;
     static constexpr TI ACTOR_HIDDEN_DIM = 64;
     static constexpr TI CRITIC_NUM_LAYERS = 3;
     static constexpr TI CRITIC_HIDDEN_DIM = 64;
 };
 
-template <TI BATCH>
+template <TI BATCH, TI CAPACITY = 10000>
 struct Loop {
-    using CONFIG = rlt::rl::algorithms::sac::loop::core::Config<TYPE_POLICY, TI, RNG, ENVIRONMENT, LoopParameters<BATCH>>;
+    using CONFIG = rlt::rl::algorithms::sac::loop::core::Config<TYPE_POLICY, TI, RNG, ENVIRONMENT, LoopParameters<BATCH, CAPACITY>>;
     using STATE = typename CONFIG::template State<CONFIG>;
     DEVICE device;
     STATE ts;
@@ -89,10 +90,11 @@ struct Any {
     int batch;
     Loop<100>* l100 = nullptr;
     Loop<256>* l256 = nullptr;
+    Loop<32, 250>* l32 = nullptr;    // small ring: wraps every 250 steps (episodes are 200 steps long)
 };
 }  // namespace
 
-#define DISPATCH(h, expr) ((h)->batch == 100 ? [&](auto& L) { return expr; }(*(h)->l100) : [&](auto& L) { return expr; }(*(h)->l256))
+#define DISPATCH(h, expr) ((h)->batch == 100 ? [&](auto& L) { return expr; }(*(h)->l100) : ((h)->batch == 256 ? [&](auto& L) { return expr; }(*(h)->l256) : [&](auto& L) { return expr; }(*(h)->l32)))
 
 extern "C" {
 
@@ -108,11 +110,12 @@ void* rlt_ref_sac_create(uint32_t seed, int batch) {
     Any* a = new Any{batch};
     if (batch == 100) a->l100 = new Loop<100>(seed);
     else if (batch == 256) a->l256 = new Loop<256>(seed);
+    else if (batch == 32) a->l32 = new Loop<32, 250>(seed);
     else { delete a; return nullptr; }
     return a;
 }
-void rlt_ref_sac_destroy(void* h) { Any* a = (Any*)h; delete a->l100; delete a->l256; delete a; }
-int rlt_ref_sac_warmup_steps(void* h) { return ((Any*)h)->batch == 100 ? 100 : 256; }
+void rlt_ref_sac_destroy(void* h) { Any* a = (Any*)h; delete a->l100; delete a->l256; delete a->l32; delete a; }
+int rlt_ref_sac_warmup_steps(void* h) { return ((Any*)h)->batch == 256 ? 256 : 100; }
 int rlt_ref_sac_step(void* h) { Any* a = (Any*)h; return DISPATCH(a, (int)rlt::step(L.device, L.ts)); }
 uint32_t rlt_ref_sac_step_count(void* h) { Any* a = (Any*)h; return DISPATCH(a, (uint32_t)L.ts.step); }
 
@@ -170,7 +173,7 @@ void rlt_ref_sac_get_replay(void* h, float* data, uint32_t* position, uint8_t* f
     DISPATCH(a, ([&] {
         auto& rb = rlt::get(L.ts.off_policy_runner.replay_buffers, 0, 0);
         using RB = rlt::utils::typing::remove_reference_t<decltype(rb)>;
-        if (data) std::memcpy(data, rb.data._data, sizeof(float) * RB::CAPACITY * RB::DATA_COLS);
+        if (data) std::memcpy(data, rb.data._data, sizeof(float) * RB::CAPACITY * RB::DATA_COLS);   // caller sizes `data` for the ring's capacity
         *position = (uint32_t)rb.position; *full = rb.full;
         if (episode_start) for (TI i = 0; i < RB::CAPACITY; i++) episode_start[i] = (uint32_t)rlt::get(L.device, rb.episode_start, i);
         return 0;

@@ -44,7 +44,8 @@ __device__ __forceinline__ float rlt_fast_tanh(float x) {
 __device__ __forceinline__ float rlt_act(float x, int f) {
     switch (f) {
         case RLT_ACT_RELU: return x > 0.0f ? x : 0.0f;
-        case RLT_ACT_GELU: { const float a = 0.7978845608028654f; return 0.5f * (x + x * tanhf(a * (0.044715f * x * x * x + x))); }
+        // the reference's GELU constant is FRAC_2_SQRTPI * SQRT1_2 * 0.5, half of the textbook sqrt(2/pi) (nn/activation_functions.h:33-36)
+        case RLT_ACT_GELU: { const float a = 0.3989422804014327f; return 0.5f * (x + x * tanhf(a * (0.044715f * x * x * x + x))); }
         case RLT_ACT_TANH: return tanhf(x);
         case RLT_ACT_FAST_TANH: return rlt_fast_tanh(x);
         case RLT_ACT_SIGMOID: return 1.0f / (1.0f + expf(-x));
@@ -55,13 +56,24 @@ __device__ __forceinline__ float rlt_dact(float x, int f) {
     switch (f) {
         case RLT_ACT_RELU: return x > 0.0f ? 1.0f : 0.0f;
         case RLT_ACT_GELU: {
-            const float a = 0.7978845608028654f, b = 0.044715f;
+            const float a = 0.3989422804014327f, b = 0.044715f;
             float t = tanhf(a * (b * x * x * x + x));
             return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * a * (3.0f * b * x * x + 1.0f);
         }
         case RLT_ACT_TANH: { float t = tanhf(x); return 1.0f - t * t; }
         case RLT_ACT_FAST_TANH: { float t = rlt_fast_tanh(x); return 1.0f - t * t; }
         case RLT_ACT_SIGMOID: { float s = 1.0f / (1.0f + expf(-x)); return s * (1.0f - s); }
+        default: return 1.0f;
+    }
+}
+
+// the same derivative written in terms of the layer OUTPUT o = act(x), where that is possible (everything but GELU):
+// relu: o > 0 <=> x > 0; tanh / fast_tanh: 1 - o^2; sigmoid: o (1 - o)
+__device__ __forceinline__ float rlt_dact_from_output(float o, int f) {
+    switch (f) {
+        case RLT_ACT_RELU: return o > 0.0f ? 1.0f : 0.0f;
+        case RLT_ACT_TANH: case RLT_ACT_FAST_TANH: return 1.0f - o * o;
+        case RLT_ACT_SIGMOID: return o * (1.0f - o);
         default: return 1.0f;
     }
 }

@@ -119,16 +119,16 @@ int rlt_rocm_init(int hip_device_index, rlt_rocm_device** out_device) {
     device->stream = device->own_stream;
     e = hipMalloc(&device->counters, 8192);
     if (e == hipSuccess) e = hipMemset(device->counters, 0, 8192);
-    if (e != hipSuccess) { hipStreamDestroy(device->own_stream); delete device; return (int)e; }
+    if (e != hipSuccess) { (void)hipStreamDestroy(device->own_stream); delete device; return (int)e; }
     *out_device = device;
     return 0;
 }
 int rlt_rocm_destroy(rlt_rocm_device* device) {
     if (!device) return RLT_E_INVALID_ARGUMENT;
-    hipStreamSynchronize(device->own_stream);
-    if (device->scratch) hipFree(device->scratch);
-    if (device->counters) hipFree(device->counters);
-    hipStreamDestroy(device->own_stream);
+    (void)hipStreamSynchronize(device->own_stream);
+    if (device->scratch) (void)hipFree(device->scratch);
+    if (device->counters) (void)hipFree(device->counters);
+    (void)hipStreamDestroy(device->own_stream);
     delete device;
     return 0;
 }

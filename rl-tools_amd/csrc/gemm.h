@@ -5,11 +5,12 @@
 // y/out/pre (each optional) = act(x W^T + bias); pre/out are packed [batch x out_dim], y has leading dimension ldy
 int rlt_gemm_forward(rlt_rocm_device* device, const float* x, int ldx, const float* W, const float* bias, int act,
                      float* pre, float* out, float* y, int ldy, int batch, int in_dim, int out_dim);
-// d_in = d_pre W, optionally multiplied elementwise by act'(dact_pre) (dact_pre packed [batch x in_dim])
+// d_in = d_pre W, optionally multiplied elementwise by act'(.) of the layer below: dact_pre (packed [batch x in_dim]) holds that
+// layer's pre-activations, or its outputs when dact_from_output is set
 int rlt_gemm_backward_input(rlt_rocm_device* device, const float* d_pre, int ldd, const float* W, float* d_in, int ldi,
-                            const float* dact_pre, int dact_kind, int batch, int in_dim, int out_dim);
+                            const float* dact_pre, int dact_kind, int dact_from_output, int batch, int in_dim, int out_dim);
 // dW += d_pre^T x ; dbias += column sums of d_pre (dbias may be NULL)
 int rlt_gemm_wgrad(rlt_rocm_device* device, const float* d_pre, int ldd, const float* x, int ldx, float* dW, float* dbias,
                    int batch, int in_dim, int out_dim);
 // dst <- act'(pre) * src (dst may alias src; then a no-op for the identity)
-int rlt_dpre(rlt_rocm_device* device, const float* src, int lds, float* dst, int ldd, const float* pre, int rows, int cols, int act);
+int rlt_dpre(rlt_rocm_device* device, const float* src, int lds, float* dst, int ldd, const float* pre, int rows, int cols, int act, int from_output);

@@ -31,7 +31,7 @@ struct GemmParams {
     // mode 0
     const float* bias; int act; float* pre; float* out; float* y; int ldy;
     // mode 1
-    float* C; int ldc; const float* dact_pre; int dact_kind;
+    float* C; int ldc; const float* dact_pre; int dact_kind; int dact_from_output;
     // mode 2
     float* dW; float* dbias; float* ws; int splits;
 };
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(GemmParams p) {
                         if (p.out) p.out[(size_t)row * p.N + col] = o;
                         if (p.y) p.y[(size_t)row * p.ldy + col] = o;
                     } else if (MODE == 1) {
-                        if (p.dact_pre) val *= rlt_dact(p.dact_pre[(size_t)row * p.N + col], p.dact_kind);
+                        if (p.dact_pre) { float a = p.dact_pre[(size_t)row * p.N + col]; val *= p.dact_from_output ? rlt_dact_from_output(a, p.dact_kind) : rlt_dact(a, p.dact_kind); }
                         p.C[(size_t)row * p.ldc + col] = val;
                     } else {
                         if (p.splits == 1) p.dW[(size_t)row * p.N + col] += val;
@@ -224,41 +224,55 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(GemmParams p) {
     }
 }
 
-// dW += sum_s ws[s][0:MN], dbias += sum_s ws[s][MN:MN+M]  (fixed summation order: deterministic)
+// dW += sum_s ws[s][0:MN], dbias += sum_s ws[s][MN:MN+M]. A workgroup owns 64 consecutive outputs; its four wavefronts each sum
+// a quarter of the splits (every read is a 256-byte row segment) and the four partials are combined in a fixed order.
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(float* __restrict__ dW, float* __restrict__ dbias, const float* __restrict__ ws,
                                                            int mn, int m, int splits) {
+    __shared__ float partial[4][64];
     const int total = mn + (dbias ? m : 0);
     const size_t stride = (size_t)mn + m;
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
-        float s = 0.0f;
-        for (int k = 0; k < splits; k++) s += ws[(size_t)k * stride + i];
-        if (i < mn) dW[i] += s; else dbias[i - mn] += s;
+    const int e = blockIdx.x * 64 + (threadIdx.x & 63), g = threadIdx.x >> 6;
+    float s = 0.0f;
+    if (e < total) for (int k = g; k < splits; k += 4) s += ws[(size_t)k * stride + e];
+    partial[g][threadIdx.x & 63] = s;
+    __syncthreads();
+    if (g == 0 && e < total) {
+        float r = (partial[0][threadIdx.x] + partial[1][threadIdx.x]) + (partial[2][threadIdx.x] + partial[3][threadIdx.x]);
+        if (e < mn) dW[e] += r; else dbias[e - mn] += r;
     }
 }
 
 // d_pre = act'(pre) * d_output (nn/layers/dense/operations_cpu_blas.h:119-141); dst may alias src
-__global__ __launch_bounds__(256) void dpre_kernel(const float* src, int lds, float* dst, int ldd, const float* __restrict__ pre, int rows, int cols, int act) {
+__global__ __launch_bounds__(256) void dpre_kernel(const float* src, int lds, float* dst, int ldd, const float* __restrict__ pre, int rows, int cols, int act, int from_output) {
     const size_t total = (size_t)rows * cols;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         int r = (int)(i / cols), c = (int)(i % cols);
-        dst[(size_t)r * ldd + c] = rlt_dact(pre[i], act) * src[(size_t)r * lds + c];
+        dst[(size_t)r * ldd + c] = (from_output ? rlt_dact_from_output(pre[i], act) : rlt_dact(pre[i], act)) * src[(size_t)r * lds + c];
     }
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// tile shape by problem shape: 128x128 for the wide contractions, 128x32 / 32x128 when one side is narrow, 64x64 when both are small
+enum TileShape { TILE_128x32, TILE_32x128, TILE_64x64, TILE_128x128 };
+TileShape pick_tile(int M, int N) {
+    if (N <= 32) return TILE_128x32;
+    if (M <= 32) return TILE_32x128;
+    if (M <= 64 || N <= 64 || (long long)M * N < 128ll * 128) return TILE_64x64;
+    return TILE_128x128;
+}
+
 template <int MODE>
 int launch(rlt_rocm_device* device, const GemmParams& p, int splits) {
     dim3 block(THREADS);
-    // tile shape by problem shape: 128x128 for the wide contractions, 128x32 / 32x128 when one side is narrow,
-    // 64x64 when both are small
-    if (p.N <= 32) {
+    const TileShape shape = pick_tile(p.M, p.N);
+    if (shape == TILE_128x32) {
         dim3 grid(rlt_div_up(p.N, 32), rlt_div_up(p.M, 128), splits);
         hipLaunchKernelGGL((gemm_kernel<MODE, 4, 1, 1, 1>), grid, block, 0, device->stream, p);
-    } else if (p.M <= 32) {
+    } else if (shape == TILE_32x128) {
         dim3 grid(rlt_div_up(p.N, 128), rlt_div_up(p.M, 32), splits);
         hipLaunchKernelGGL((gemm_kernel<MODE, 1, 4, 1, 1>), grid, block, 0, device->stream, p);
-    } else if ((long long)p.M * p.N <= 64ll * 1024 || p.M <= 64 || p.N <= 64) {
+    } else if (shape == TILE_64x64) {
         dim3 grid(rlt_div_up(p.N, 64), rlt_div_up(p.M, 64), splits);
         hipLaunchKernelGGL((gemm_kernel<MODE, 2, 2, 1, 1>), grid, block, 0, device->stream, p);
     } else {
@@ -281,12 +295,12 @@ int rlt_gemm_forward(rlt_rocm_device* device, const float* x, int ldx, const flo
 }
 
 int rlt_gemm_backward_input(rlt_rocm_device* device, const float* d_pre, int ldd, const float* W, float* d_in, int ldi,
-                            const float* dact_pre, int dact_kind, int batch, int in_dim, int out_dim) {
+                            const float* dact_pre, int dact_kind, int dact_from_output, int batch, int in_dim, int out_dim) {
     if (rlt_div_up(batch, 32) > 65535) return RLT_E_UNSUPPORTED;
     GemmParams p = {};
     p.A = d_pre; p.lda = ldd; p.B = W; p.ldb = in_dim; p.M = batch; p.N = in_dim; p.K = out_dim; p.k_per_split = out_dim;
     p.vecA = aligned16(d_pre) && (ldd % 4 == 0); p.vecB = aligned16(W) && (in_dim % 4 == 0);
-    p.C = d_in; p.ldc = ldi; p.dact_pre = dact_pre; p.dact_kind = dact_kind; p.splits = 1;
+    p.C = d_in; p.ldc = ldi; p.dact_pre = dact_pre; p.dact_kind = dact_kind; p.dact_from_output = dact_from_output; p.splits = 1;
     return launch<1>(device, p, 1);
 }
 
@@ -297,8 +311,9 @@ int rlt_gemm_wgrad(rlt_rocm_device* device, const float* d_pre, int ldd, const f
     p.vecA = aligned16(d_pre) && (ldd % 4 == 0); p.vecB = aligned16(x) && (ldx % 4 == 0);
     p.dW = dW; p.dbias = dbias;
     // split the batch so that the grid fills the chip: about 2 workgroups per compute unit, at least 256 rows per split
-    int bm = out_dim <= 32 ? 32 : (((long long)out_dim * in_dim <= 64ll * 1024 || out_dim <= 64 || in_dim <= 64) ? 64 : 128);
-    int bn = in_dim <= 32 ? 32 : (out_dim <= 32 ? 128 : (bm == 64 ? 64 : 128));
+    const TileShape shape = pick_tile(out_dim, in_dim);
+    int bm = shape == TILE_128x32 ? 128 : (shape == TILE_32x128 ? 32 : (shape == TILE_64x64 ? 64 : 128));
+    int bn = shape == TILE_128x32 ? 32 : (shape == TILE_32x128 ? 128 : (shape == TILE_64x64 ? 64 : 128));
     int tiles = rlt_div_up(out_dim, bm) * rlt_div_up(in_dim, bn);
     int splits = (2 * device->compute_units + tiles - 1) / tiles;
     int max_splits = rlt_div_up(batch, 256);
@@ -317,17 +332,17 @@ int rlt_gemm_wgrad(rlt_rocm_device* device, const float* d_pre, int ldd, const f
     if (rc) return rc;
     if (splits > 1) {
         int mn = out_dim * in_dim;
-        int blocks = rlt_div_up(mn + out_dim, 256);
+        int blocks = rlt_div_up(mn + out_dim, 64);
         hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(blocks), dim3(256), 0, device->stream, dW, dbias, p.ws, mn, out_dim, splits);
         return rlt_launch_status(device);
     }
     return 0;
 }
 
-int rlt_dpre(rlt_rocm_device* device, const float* src, int lds, float* dst, int ldd, const float* pre, int rows, int cols, int act) {
+int rlt_dpre(rlt_rocm_device* device, const float* src, int lds, float* dst, int ldd, const float* pre, int rows, int cols, int act, int from_output) {
     if (act == RLT_ACT_IDENTITY && src == dst) return 0;
     size_t total = (size_t)rows * cols;
     int blocks = (int)((total + 255) / 256); if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(dpre_kernel, dim3(blocks), dim3(256), 0, device->stream, src, lds, dst, ldd, pre, rows, cols, act);
+    hipLaunchKernelGGL(dpre_kernel, dim3(blocks), dim3(256), 0, device->stream, src, lds, dst, ldd, pre, rows, cols, act, from_output);
     return rlt_launch_status(device);
 }

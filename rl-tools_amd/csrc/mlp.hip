@@ -52,14 +52,14 @@ int rlt_rocm_dense_forward(rlt_rocm_device* device, const rlt_dense_layer* L, co
 int rlt_rocm_dense_backward_input(rlt_rocm_device* device, const rlt_dense_layer* L, float* d_output, int ldd, float* d_input, int ldi, int batch) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(layer_ok(L) && L->pre_activations && d_output && d_input && batch > 0 && ldd >= L->out_dim && ldi >= L->in_dim);
-    int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, L->pre_activations, batch, L->out_dim, L->activation);
+    int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, L->pre_activations, batch, L->out_dim, L->activation, 0);
     if (rc) return rc;
-    return rlt_gemm_backward_input(device, d_output, ldd, L->weights, d_input, ldi, nullptr, 0, batch, L->in_dim, L->out_dim);
+    return rlt_gemm_backward_input(device, d_output, ldd, L->weights, d_input, ldi, nullptr, 0, 0, batch, L->in_dim, L->out_dim);
 }
 int rlt_rocm_dense_backward(rlt_rocm_device* device, const rlt_dense_layer* L, const float* x, int ldx, float* d_output, int ldd, int batch) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(layer_ok(L) && L->pre_activations && L->d_weights && L->d_biases && x && d_output && batch > 0 && ldd >= L->out_dim && ldx >= L->in_dim);
-    int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, L->pre_activations, batch, L->out_dim, L->activation);
+    int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, L->pre_activations, batch, L->out_dim, L->activation, 0);
     if (rc) return rc;
     return rlt_gemm_wgrad(device, d_output, ldd, x, ldx, L->d_weights, L->d_biases, batch, L->in_dim, L->out_dim);
 }
@@ -68,7 +68,7 @@ int rlt_rocm_dense_backward_full(rlt_rocm_device* device, const rlt_dense_layer*
     int rc = rlt_rocm_dense_backward(device, L, x, ldx, d_output, ldd, batch);
     if (rc) return rc;
     RLT_REQUIRE(d_input && ldi >= L->in_dim);
-    return rlt_gemm_backward_input(device, d_output, ldd, L->weights, d_input, ldi, nullptr, 0, batch, L->in_dim, L->out_dim);
+    return rlt_gemm_backward_input(device, d_output, ldd, L->weights, d_input, ldi, nullptr, 0, 0, batch, L->in_dim, L->out_dim);
 }
 
 size_t rlt_rocm_mlp_workspace_bytes(const rlt_dense_layer* layers, int n_layers, int batch) {
@@ -112,8 +112,10 @@ int rlt_rocm_mlp_forward(rlt_rocm_device* device, const rlt_dense_layer* layers,
 }
 
 // Shared by mlp_backward and mlp_forward_backward. d_pre_last: [batch x out] holding the LAST layer's d_pre already.
+// With from_output set, a layer's `pre_activations` may be NULL and the activation derivative is taken from its `output`.
 static int mlp_backward_from_dpre(rlt_rocm_device* device, const rlt_dense_layer* layers, int n, const float* x, int ldx,
-                                  float* d_pre_last, int ldd, float* d_input, int ldi, int batch, int want_w, float* tick, float* tock) {
+                                  float* d_pre_last, int ldd, float* d_input, int ldi, int batch, int want_w, float* tick, float* tock,
+                                  bool from_output = false) {
     float* d_pre = d_pre_last; int ld_pre = ldd;
     for (int l = n - 1; l >= 0; l--) {
         const rlt_dense_layer& L = layers[l];
@@ -125,12 +127,13 @@ static int mlp_backward_from_dpre(rlt_rocm_device* device, const rlt_dense_layer
         if (l > 0) {
             // d_input of this layer becomes d_pre of the layer below: the activation derivative is applied in the epilogue
             float* d_in = ((n - 1 - l) % 2 == 0) ? tick : tock;
-            int rc = rlt_gemm_backward_input(device, d_pre, ld_pre, L.weights, d_in, L.in_dim, layers[l - 1].pre_activations, layers[l - 1].activation,
-                                             batch, L.in_dim, L.out_dim);
+            const bool fo = from_output && layers[l - 1].pre_activations == nullptr;
+            int rc = rlt_gemm_backward_input(device, d_pre, ld_pre, L.weights, d_in, L.in_dim, fo ? layers[l - 1].output : layers[l - 1].pre_activations,
+                                             layers[l - 1].activation, fo ? 1 : 0, batch, L.in_dim, L.out_dim);
             if (rc) return rc;
             d_pre = d_in; ld_pre = L.in_dim;
         } else if (d_input) {
-            int rc = rlt_gemm_backward_input(device, d_pre, ld_pre, L.weights, d_input, ldi, nullptr, 0, batch, L.in_dim, L.out_dim);
+            int rc = rlt_gemm_backward_input(device, d_pre, ld_pre, L.weights, d_input, ldi, nullptr, 0, 0, batch, L.in_dim, L.out_dim);
             if (rc) return rc;
         }
     }
@@ -152,7 +155,7 @@ int rlt_rocm_mlp_backward(rlt_rocm_device* device, const rlt_dense_layer* layers
     RLT_REQUIRE(n == 1 || (workspace && workspace_bytes >= 2 * buf));
     float* tick = (float*)workspace; float* tock = (float*)((char*)workspace + buf);
     const rlt_dense_layer& last = layers[n - 1];
-    int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, last.pre_activations, batch, last.out_dim, last.activation);
+    int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, last.pre_activations, batch, last.out_dim, last.activation, 0);
     if (rc) return rc;
     return mlp_backward_from_dpre(device, layers, n, x, ldx, d_output, ldd, d_input, ldi, batch, want_w, tick, tock);
 }
@@ -188,7 +191,9 @@ int rlt_rocm_mlp_forward_backward(rlt_rocm_device* device, const rlt_dense_layer
     float* tick = (float*)w; w += buf; float* tock = (float*)w; w += buf; float* dlast = (float*)w; w += buf;
     for (int l = 0; l < n; l++) {
         priv[l] = layers[l];
-        priv[l].pre_activations = (float*)w; w += (size_t)batch * layers[l].out_dim * sizeof(float);
+        // the activation derivative is recovered from the output wherever the activation allows it, so only GELU layers keep both
+        priv[l].pre_activations = nullptr;
+        if (layers[l].activation == RLT_ACT_GELU) { priv[l].pre_activations = (float*)w; w += (size_t)batch * layers[l].out_dim * sizeof(float); }
         priv[l].output = (float*)w; w += (size_t)batch * layers[l].out_dim * sizeof(float);
     }
     const float* in = x; int ldin = ldx;
@@ -204,11 +209,13 @@ int rlt_rocm_mlp_forward_backward(rlt_rocm_device* device, const rlt_dense_layer
         size_t total = (size_t)batch * O; int blocks = (int)((total + 255) / 256); if (blocks > 4096) blocks = 4096;
         hipLaunchKernelGGL(mse_d_kernel, dim3(blocks), dim3(256), 0, device->stream, last.output, O, target, ldt, dlast, O, batch, O, mse_scale);
         if ((rc = rlt_launch_status(device))) return rc;
-        if ((rc = rlt_dpre(device, dlast, O, dlast, O, last.pre_activations, batch, O, last.activation))) return rc;
+        const bool fo = last.pre_activations == nullptr;
+        if ((rc = rlt_dpre(device, dlast, O, dlast, O, fo ? last.output : last.pre_activations, batch, O, last.activation, fo))) return rc;
     } else {
-        if ((rc = rlt_dpre(device, d_output, ldd, dlast, O, last.pre_activations, batch, O, last.activation))) return rc;
+        const bool fo = last.pre_activations == nullptr;
+        if ((rc = rlt_dpre(device, d_output, ldd, dlast, O, fo ? last.output : last.pre_activations, batch, O, last.activation, fo))) return rc;
     }
-    return mlp_backward_from_dpre(device, priv, n, x, ldx, dlast, O, nullptr, 0, batch, 1, tick, tock);
+    return mlp_backward_from_dpre(device, priv, n, x, ldx, dlast, O, nullptr, 0, batch, 1, tick, tock, true);
 }
 
 }  // extern "C"

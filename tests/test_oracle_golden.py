@@ -1,0 +1,53 @@
+"""The CPU checker against golden vectors written by the real reference (tests/golden/make_sac_golden.py): the seeded
+SAC-on-Pendulum loop must reproduce the reference's parameters, replay rows, gathered batches, masks and noise BIT-EXACTLY.
+Runs without /root/reference (the fixture is data)."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+import helpers
+
+GOLD = np.load(os.path.join(helpers.GOLDEN, "sac_pendulum_seed0.npz"))
+
+
+def np_from(ptr, shape, dtype=np.float32):
+    n = int(np.prod(shape))
+    return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(np.ctypeslib.as_ctypes_type(dtype))), (n,)).reshape(shape).copy()
+
+
+@pytest.mark.parametrize("batch,checkpoints", [(100, [0, 100, 101, 150, 300]), (256, [256, 257, 300, 500])])
+def test_seeded_loop_reproduces_reference_vectors(oracle, batch, checkpoints):
+    lib = oracle.lib
+    cfg = helpers.LoopConfig(0, batch, 64, 10000, max(batch, 100), 200, 1e-7)
+    loop = C.c_void_p(lib.rlt_oracle_sac_loop_create(C.byref(cfg)))
+    n = lib.rlt_oracle_sac_loop_parameter_count(loop)
+    p = np.zeros(n, np.float32)
+    A = lib.rlt_oracle_sac_loop_agent(loop).contents
+    rb = lib.rlt_oracle_sac_loop_replay(loop).contents
+    done = 0
+    for cp in checkpoints:
+        while done < cp:
+            assert lib.rlt_oracle_sac_loop_step(loop) == 0
+            done += 1
+        key = f"b{batch}_s{cp}"
+        lib.rlt_oracle_sac_loop_get_parameters(loop, p.ctypes.data)
+        assert np.array_equal(p[::16], GOLD[key + "_params16"]), key
+        assert p.astype(np.float64).sum() == GOLD[key + "_sum"][0] and (p.astype(np.float64) ** 2).sum() == GOLD[key + "_sum"][1]
+        pos, full = int(np_from(rb.position, (1,), np.uint32)[0]), int(np_from(rb.full, (1,), np.uint8)[0])
+        assert [pos, full] == list(GOLD[key + "_replay_pos"])
+        data = np_from(rb.data, (10000, 10))
+        assert np.array_equal(data[max(0, pos - 8):pos], GOLD[key + "_replay_tail"])
+        if cp > max(batch, 100):
+            assert np.array_equal(np_from(A.observations_actions_base, (2, batch, 4)), GOLD[key + "_oab"])
+            assert np.array_equal(np_from(A.rewards, (batch,)), GOLD[key + "_rewards"])
+            assert np.array_equal(np_from(A.terminated, (batch,), np.uint8), GOLD[key + "_terminated"])
+            assert np.array_equal(np_from(lib.rlt_oracle_sac_loop_noise_critic(loop), (batch,)), GOLD[key + "_noise_critic"])
+            assert np.array_equal(np_from(lib.rlt_oracle_sac_loop_noise_actor(loop), (batch,)), GOLD[key + "_noise_actor"])
+            # masks: final_step_mask / reset are the agent's views; next_final_step_mask is padded step 1 of its base tensor
+            assert np.array_equal(np_from(A.final_step_mask, (batch,), np.uint8), GOLD[key + "_final_step_mask"])
+            assert np.array_equal(np_from(A.reset, (batch,), np.uint8), GOLD[key + "_reset"])
+            assert np.array_equal(np_from(A.next_final_step_mask, (batch,), np.uint8), GOLD[key + "_next_final_step_mask_base"][batch:])
+            assert np.all(GOLD[key + "_next_final_step_mask_base"][:batch] == 0) and np.all(GOLD[key + "_next_reset_base"] == 1)
+    lib.rlt_oracle_sac_loop_destroy(loop)

@@ -1,0 +1,112 @@
+"""The CPU checker against the REAL reference compiled from /root/reference (oracle/_ref, built by oracle/Makefile): the whole
+seeded SAC-on-Pendulum loop, bit for bit. Skipped where the reference build is absent (the GPU box still carries the built
+library; a machine without it relies on tests/test_oracle_golden.py)."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+import helpers
+
+pytestmark = pytest.mark.skipif(not os.path.exists(helpers.REF_GENERIC), reason="oracle/_ref not built (needs /root/reference)")
+
+
+def load_ref(path):
+    ref = C.CDLL(path)
+    ref.rlt_ref_sac_create.restype = C.c_void_p
+    ref.rlt_ref_sac_parameter_count.restype = C.c_size_t
+    ref.rlt_ref_sac_parameter_count.argtypes = [C.c_void_p]
+    P = C.c_void_p
+    for name, args in dict(step=[P], destroy=[P], get_parameters=[P, P], get_batch=[P, P, P, P], get_noise=[P, P, P], get_replay=[P, P, P, P, P],
+                           get_critic_buffers=[P, C.c_int, P, P, P, P, P], get_actor_buffers=[P, P, P, P, P]).items():
+        getattr(ref, "rlt_ref_sac_" + name).argtypes = args
+    return ref
+
+
+def np_from(ptr, shape, dtype=np.float32):
+    n = int(np.prod(shape))
+    return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(np.ctypeslib.as_ctypes_type(dtype))), (n,)).reshape(shape).copy()
+
+
+@pytest.mark.parametrize("batch,steps", [(100, 400), (256, 420)])
+def test_loop_bit_exact_with_reference_generic_build(oracle, batch, steps):
+    """Parameters after every step, the replay ring, the gathered batch, the noise and the training buffers
+    (pattern: tests/src/rl/cuda/rl.cu:230-376 TRAIN_CRITIC_STEP_BY_STEP) are identical bit for bit."""
+    ref, lib = load_ref(helpers.REF_GENERIC), oracle.lib
+    cfg = helpers.LoopConfig(0, batch, 64, 10000, max(batch, 100), 200, 1e-7)
+    loop = C.c_void_p(lib.rlt_oracle_sac_loop_create(C.byref(cfg)))
+    h = C.c_void_p(ref.rlt_ref_sac_create(0, batch))
+    n = lib.rlt_oracle_sac_loop_parameter_count(loop)
+    assert n == ref.rlt_ref_sac_parameter_count(h)
+    po, pr = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    A = lib.rlt_oracle_sac_loop_agent(loop).contents
+    rb = lib.rlt_oracle_sac_loop_replay(loop).contents
+    for step in range(steps):
+        assert lib.rlt_oracle_sac_loop_step(loop) == 0
+        ref.rlt_ref_sac_step(h)
+        lib.rlt_oracle_sac_loop_get_parameters(loop, po.ctypes.data); ref.rlt_ref_sac_get_parameters(h, pr.ctypes.data)
+        assert np.array_equal(po, pr), f"parameters differ after step {step}"
+        if step > max(batch, 100) and step % 40 == 0:
+            oab = np.zeros((2, batch, 4), np.float32); rew = np.zeros(batch, np.float32); term = np.zeros(batch, np.uint8)
+            ref.rlt_ref_sac_get_batch(h, oab.ctypes.data, rew.ctypes.data, term.ctypes.data)
+            assert np.array_equal(oab, np_from(A.observations_actions_base, (2, batch, 4)))
+            assert np.array_equal(rew, np_from(A.rewards, (batch,))) and np.array_equal(term, np_from(A.terminated, (batch,), np.uint8))
+            y, q1, q2, nin, dout = (np.zeros(s, np.float32) for s in (batch, batch, batch, (batch, 4), batch))
+            ref.rlt_ref_sac_get_critic_buffers(h, 1, y.ctypes.data, q1.ctypes.data, q2.ctypes.data, nin.ctypes.data, dout.ctypes.data)
+            assert np.array_equal(y, np_from(A.target_action_value, (batch,)))
+            assert np.array_equal(q1, np_from(A.next_q[0], (batch,))) and np.array_equal(q2, np_from(A.next_q[1], (batch,)))
+            assert np.array_equal(nin, np_from(A.next_state_action_value_input, (batch, 4)))
+            sav, d1, d2, daos = (np.zeros(s, np.float32) for s in ((batch, 4), (batch, 4), (batch, 4), batch))
+            ref.rlt_ref_sac_get_actor_buffers(h, sav.ctypes.data, d1.ctypes.data, d2.ctypes.data, daos.ctypes.data)
+            assert np.array_equal(sav, np_from(A.state_action_value_input, (batch, 4)))
+            assert np.array_equal(d1, np_from(A.d_critic_input[0], (batch, 4))) and np.array_equal(d2, np_from(A.d_critic_input[1], (batch, 4)))
+            assert np.array_equal(daos, np_from(A.d_actor_output_squashing, (batch,)))
+    data = np.zeros((10000, 10), np.float32); pos = C.c_uint32(); full = C.c_uint8(); es = np.zeros(10000, np.uint32)
+    ref.rlt_ref_sac_get_replay(h, data.ctypes.data, C.byref(pos), C.byref(full), es.ctypes.data)
+    assert pos.value == np_from(rb.position, (1,), np.uint32)[0] and not full.value
+    assert np.array_equal(data[:pos.value], np_from(rb.data, (10000, 10))[:pos.value])      # rows beyond the cursor are uninitialised in the reference
+    assert np.array_equal(es[:pos.value], np_from(rb.episode_start, (10000,), np.uint32)[:pos.value])
+    lib.rlt_oracle_sac_loop_destroy(loop); ref.rlt_ref_sac_destroy(h)
+
+
+def test_small_ring_wraps_bit_exact_with_reference(oracle):
+    """Replay capacity 250 (< 900 steps): the ring wraps three times, so `add` past the end, the prologue's wrap of the
+    previous row, `full`, and gather's (position + MAX_EPISODE_LENGTH + offset) % CAPACITY index all run, and every
+    parameter still matches the reference bit for bit after each step."""
+    ref, lib = load_ref(helpers.REF_GENERIC), oracle.lib
+    batch, cap = 32, 250
+    cfg = helpers.LoopConfig(0, batch, 64, cap, 100, 200, 1e-7)
+    loop = C.c_void_p(lib.rlt_oracle_sac_loop_create(C.byref(cfg)))
+    h = C.c_void_p(ref.rlt_ref_sac_create(0, batch))
+    n = lib.rlt_oracle_sac_loop_parameter_count(loop)
+    po, pr = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    rb = lib.rlt_oracle_sac_loop_replay(loop).contents
+    for step in range(900):
+        assert lib.rlt_oracle_sac_loop_step(loop) == 0
+        ref.rlt_ref_sac_step(h)
+        lib.rlt_oracle_sac_loop_get_parameters(loop, po.ctypes.data); ref.rlt_ref_sac_get_parameters(h, pr.ctypes.data)
+        assert np.array_equal(po, pr), f"parameters differ after step {step}"
+    data = np.zeros((cap, 10), np.float32); pos = C.c_uint32(); full = C.c_uint8(); es = np.zeros(cap, np.uint32)
+    ref.rlt_ref_sac_get_replay(h, data.ctypes.data, C.byref(pos), C.byref(full), es.ctypes.data)
+    assert full.value == 1 == np_from(rb.full, (1,), np.uint8)[0] and pos.value == 900 % cap == np_from(rb.position, (1,), np.uint32)[0]
+    assert np.array_equal(data, np_from(rb.data, (cap, 10)))
+    assert np.array_equal(es, np_from(rb.episode_start, (cap,), np.uint32))
+    lib.rlt_oracle_sac_loop_destroy(loop); ref.rlt_ref_sac_destroy(h)
+
+
+@pytest.mark.skipif(not os.path.exists(helpers.REF_BLAS), reason="BLAS flavour of oracle/_ref not built")
+def test_blas_flavour_of_reference_agrees_for_one_update(oracle):
+    """The reference's CBLAS backend (its own -ffast-math build) after the first training step: same algorithm, different
+    summation order, so 1e-5 relative rather than bit-exact."""
+    ref, lib = load_ref(helpers.REF_BLAS), oracle.lib
+    batch = 100
+    cfg = helpers.LoopConfig(0, batch, 64, 10000, 100, 200, 1e-7)
+    loop = C.c_void_p(lib.rlt_oracle_sac_loop_create(C.byref(cfg)))
+    h = C.c_void_p(ref.rlt_ref_sac_create(0, batch))
+    n = lib.rlt_oracle_sac_loop_parameter_count(loop)
+    po, pr = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for step in range(103):
+        lib.rlt_oracle_sac_loop_step(loop); ref.rlt_ref_sac_step(h)
+    lib.rlt_oracle_sac_loop_get_parameters(loop, po.ctypes.data); ref.rlt_ref_sac_get_parameters(h, pr.ctypes.data)
+    assert helpers.rel_err(po, pr) <= 1e-5
