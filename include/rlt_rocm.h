@@ -383,6 +383,33 @@ int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_ru
                                   const float* actions_in, const float* action_noise,
                                   const float* initial_states, uint64_t seed, uint64_t offset);
 
+/* Host-drawn randomness for rlt_rocm_sac_pendulum_loop (parity runs feed the draws the reference's CPU RNG made); any member
+ * may be NULL, in which case the kernel draws from its counter-based generator keyed by (seed, step). */
+typedef struct rlt_sac_loop_inputs {
+    const float* rollout_noise;       /* [n_steps x action_dim] exploration noise of the runner's actor                 */
+    const float* initial_states;      /* [n_steps x 2] (theta, theta_dot), read at the steps where an episode resets    */
+    const uint32_t* sample_offsets;   /* [n_steps x batch] gather offsets (the env index is always 0: one environment)  */
+    const float* noise_critic;        /* [n_steps x batch x action_dim]                                                 */
+    const float* noise_actor;         /* [n_steps x batch x action_dim]                                                 */
+} rlt_sac_loop_inputs;
+typedef struct rlt_sac_loop_outputs {  /* all optional */
+    float* critic_loss;                /* [n_steps x 2] 0.5 * mean squared TD error of each critic at its update          */
+    float* observations_actions_base;  /* [2 x batch x (obs+act)] the last step's batch                                   */
+    float* rewards;                    /* [batch]                                                                         */
+    uint8_t* terminated;               /* [batch]                                                                         */
+    float* target_action_value;        /* [batch] the last step's TD targets                                              */
+} rlt_sac_loop_outputs;
+
+/* n_steps iterations of sac::loop::core::step (rl/algorithms/sac/loop/core/operations_generic.h:110-155, past the warm-up:
+ * actor-driven environment step + replay add, gather_batch, train_critic x2, update_critic_targets, train_actor) in ONE
+ * persistent launch of batch/16 workgroups that synchronise through device memory. Built for the Pendulum shapes of the
+ * reference's example (observation 3, action 1, 3-layer ReLU networks of width 64, batch a multiple of 16 up to 1024, one
+ * environment, networks laid out as contiguous [W1|b1|W2|b2|W3|b3] arenas, masks NULL); returns RLT_E_UNSUPPORTED otherwise and
+ * the caller takes the per-operation entry points above. Gradient arenas hold the last step's summed gradients on return. */
+int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_pendulum_runner* runner,
+                               const rlt_replay_buffer* rb, int n_steps, uint64_t seed, uint64_t step_offset,
+                               const rlt_sac_loop_inputs* inputs, const rlt_sac_loop_outputs* outputs);
+
 /* --------------------------------------------------------------------- PPO -- */
 
 /* estimate_generalized_advantages   rl/algorithms/ppo/operations_generic.h:60-95

@@ -80,6 +80,16 @@ class PendulumRunner(C.Structure):
                 ("n_envs", C.c_int32), ("episode_step_limit", C.c_int32), ("env", PendulumParameters)]
 
 
+class SacLoopInputs(C.Structure):
+    _fields_ = [("rollout_noise", C.c_void_p), ("initial_states", C.c_void_p), ("sample_offsets", C.c_void_p), ("noise_critic", C.c_void_p),
+                ("noise_actor", C.c_void_p)]
+
+
+class SacLoopOutputs(C.Structure):
+    _fields_ = [("critic_loss", C.c_void_p), ("observations_actions_base", C.c_void_p), ("rewards", C.c_void_p), ("terminated", C.c_void_p),
+                ("target_action_value", C.c_void_p)]
+
+
 I, F, P, S, U64 = C.c_int, C.c_float, C.c_void_p, C.c_size_t, C.c_uint64
 LP = C.POINTER(DenseLayer)
 
@@ -128,6 +138,8 @@ ROCM_ONLY = {
     "reduce_sum_f32": ([P, P, S, I, P], I),
     "mlp_workspace_bytes": ([LP, I, I], S),
     "gather_draw": ([P, C.POINTER(ReplayBuffer), I, U64, U64, P, P], I),
+    "sac_pendulum_loop": ([P, C.POINTER(SacAgent), C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, U64, U64, C.POINTER(SacLoopInputs),
+                           C.POINTER(SacLoopOutputs)], I),
     "pendulum_runner_step": ([P, C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, LP, I, C.POINTER(SasParameters), P, P, P, U64, U64], I),
 }
 

@@ -298,3 +298,81 @@ def rel_err(a, ref):
     a = np.asarray(a, np.float64); ref = np.asarray(ref, np.float64)
     scale = max(np.abs(ref).max(), 1e-30)
     return np.abs(a - ref).max() / scale
+
+
+# ---------------------------------------------------------------- the checker's seeded SAC loop as a source of states and draws
+def np_from(ptr, shape, dtype=np.float32):
+    n = int(np.prod(shape))
+    return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(np.ctypeslib.as_ctypes_type(dtype))), (n,)).reshape(shape).copy()
+
+
+def make_loop(oracle, batch, seed=0, capacity=10000):
+    cfg = LoopConfig(seed, batch, 64, capacity, max(batch, 100), 200, 1e-7)
+    return C.c_void_p(oracle.lib.rlt_oracle_sac_loop_create(C.byref(cfg))), cfg
+
+
+def loop_parameters(oracle, loop):
+    n = oracle.lib.rlt_oracle_sac_loop_parameter_count(loop)
+    out = np.zeros(n, np.float32)
+    oracle.lib.rlt_oracle_sac_loop_get_parameters(loop, out.ctypes.data)
+    return out
+
+
+def loop_state(oracle, loop, batch, hidden=64):
+    """Parameters, gradients, Adam moments and ages of the checker's loop (its arenas are contiguous per network)."""
+    A = oracle.lib.rlt_oracle_sac_loop_agent(loop).contents
+    na, nc = mlp_param_count([3, hidden, hidden, 2]), mlp_param_count([4, hidden, hidden, 1])
+    st = {}
+    for name, layers, tensors, age, n in (("actor", A.actor, A.actor_adam_tensors, A.actor_age, na),
+                                          ("critic0", A.critics[0], A.critic_adam_tensors[0], A.critic_age[0], nc),
+                                          ("critic1", A.critics[1], A.critic_adam_tensors[1], A.critic_age[1], nc)):
+        st[name] = dict(params=np_from(layers[0].weights, (n,)), m=np_from(tensors[0].first_moment, (n,)), v=np_from(tensors[0].second_moment, (n,)),
+                        grads=np_from(tensors[0].gradient, (n,)), age=np_from(age, (1,), np.uint32))
+    for k in range(2):
+        st[f"target{k}"] = dict(params=np_from(A.critics_target[k][0].weights, (nc,)))
+    st["log_alpha"] = np_from(A.log_alpha.parameters, (4,)); st["alpha_age"] = np_from(A.alpha_age, (1,), np.uint32)
+    return st
+
+
+def push_state(agent, st):
+    for name, net in (("actor", agent.actor), ("critic0", agent.critics[0]), ("critic1", agent.critics[1])):
+        net.params.upload(st[name]["params"]); net.m.upload(st[name]["m"]); net.v.upload(st[name]["v"]); net.age.upload(st[name]["age"])
+    for k in range(2):
+        agent.targets[k].params.upload(st[f"target{k}"]["params"])
+    agent.log_alpha.upload(st["log_alpha"]); agent.alpha_age.upload(st["alpha_age"])
+
+
+class RunnerOnBackend:
+    """Single-environment Pendulum runner state + its replay ring on a backend, optionally copied from the checker's loop."""
+
+    def __init__(self, backend, capacity, oracle=None, loop=None):
+        self.rb = ReplayOnBackend(backend, 1, capacity)
+        self.states = backend.zeros((1, 2)); self.ep_step = backend.zeros((1,), np.uint32); self.ep_ret = backend.zeros((1,))
+        self.trunc = backend.array(np.ones(1, np.uint8))
+        if loop is not None:
+            rn = oracle.lib.rlt_oracle_sac_loop_runner(loop).contents
+            rb = oracle.lib.rlt_oracle_sac_loop_replay(loop).contents
+            self.states.upload(np_from(rn.states, (1, 2))); self.ep_step.upload(np_from(rn.episode_step, (1,), np.uint32))
+            self.ep_ret.upload(np_from(rn.episode_return, (1,))); self.trunc.upload(np_from(rn.truncated, (1,), np.uint8))
+            self.rb.data.upload(np_from(rb.data, (capacity, 10))); self.rb.episode_start.upload(np_from(rb.episode_start, (capacity,), np.uint32))
+            self.rb.position.upload(np_from(rb.position, (1,), np.uint32)); self.rb.current_episode_start.upload(np_from(rb.current_episode_start, (1,), np.uint32))
+            self.rb.full.upload(np_from(rb.full, (1,), np.uint8))
+        self.c = capi.PendulumRunner(self.states.ptr, self.ep_step.ptr, self.ep_ret.ptr, self.trunc.ptr, 1, 200, capi.pendulum_parameters())
+
+
+def collect_loop_draws(oracle, loop, batch, n_steps):
+    """Steps the checker's loop n_steps times and records the random draws of every step plus its critic losses."""
+    lib = oracle.lib
+    d = dict(rollout_noise=np.zeros((n_steps, 1), np.float32), initial_states=np.zeros((n_steps, 2), np.float32),
+             sample_offsets=np.zeros((n_steps, batch), np.uint32), noise_critic=np.zeros((n_steps, batch, 1), np.float32),
+             noise_actor=np.zeros((n_steps, batch, 1), np.float32), critic_loss=np.zeros((n_steps, 2), np.float32))
+    env = np.zeros(6, np.float32)
+    for t in range(n_steps):
+        assert lib.rlt_oracle_sac_loop_step(loop) == 0
+        lib.rlt_oracle_sac_loop_last_env_step(loop, env.ctypes.data)
+        d["initial_states"][t] = env[1:3]; d["rollout_noise"][t, 0] = env[3]
+        d["sample_offsets"][t] = np_from(lib.rlt_oracle_sac_loop_sample_offsets(loop), (batch,), np.uint32)
+        d["noise_critic"][t, :, 0] = np_from(lib.rlt_oracle_sac_loop_noise_critic(loop), (batch,))
+        d["noise_actor"][t, :, 0] = np_from(lib.rlt_oracle_sac_loop_noise_actor(loop), (batch,))
+        d["critic_loss"][t] = [lib.rlt_oracle_sac_loop_critic_loss(loop, 0), lib.rlt_oracle_sac_loop_critic_loss(loop, 1)]
+    return d

@@ -13,45 +13,7 @@ from helpers import capi, rel_err
 pytestmark = pytest.mark.gpu
 
 
-def make_loop(oracle, batch, seed=0):
-    cfg = helpers.LoopConfig(seed, batch, 64, 10000, max(batch, 100), 200, 1e-7)
-    return C.c_void_p(oracle.lib.rlt_oracle_sac_loop_create(C.byref(cfg))), cfg
-
-
-def loop_parameters(oracle, loop):
-    n = oracle.lib.rlt_oracle_sac_loop_parameter_count(loop)
-    out = np.zeros(n, np.float32)
-    oracle.lib.rlt_oracle_sac_loop_get_parameters(loop, out.ctypes.data)
-    return out
-
-
-def np_from(ptr, shape, dtype=np.float32):
-    n = int(np.prod(shape))
-    return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(np.ctypeslib.as_ctypes_type(dtype))), (n,)).reshape(shape).copy()
-
-
-def loop_state(oracle, loop, batch, hidden=64):
-    """Parameters, Adam moments and ages of the checker's loop (its arenas are contiguous per network)."""
-    A = oracle.lib.rlt_oracle_sac_loop_agent(loop).contents
-    na, nc = helpers.mlp_param_count([3, hidden, hidden, 2]), helpers.mlp_param_count([4, hidden, hidden, 1])
-    st = {}
-    for name, layers, tensors, age, n in (("actor", A.actor, A.actor_adam_tensors, A.actor_age, na),
-                                          ("critic0", A.critics[0], A.critic_adam_tensors[0], A.critic_age[0], nc),
-                                          ("critic1", A.critics[1], A.critic_adam_tensors[1], A.critic_age[1], nc)):
-        st[name] = dict(params=np_from(layers[0].weights, (n,)), m=np_from(tensors[0].first_moment, (n,)), v=np_from(tensors[0].second_moment, (n,)),
-                        grads=np_from(tensors[0].gradient, (n,)), age=np_from(age, (1,), np.uint32))
-    for k in range(2):
-        st[f"target{k}"] = dict(params=np_from(A.critics_target[k][0].weights, (nc,)))
-    st["log_alpha"] = np_from(A.log_alpha.parameters, (4,)); st["alpha_age"] = np_from(A.alpha_age, (1,), np.uint32)
-    return st
-
-
-def push_state(agent, st):
-    for name, net in (("actor", agent.actor), ("critic0", agent.critics[0]), ("critic1", agent.critics[1])):
-        net.params.upload(st[name]["params"]); net.m.upload(st[name]["m"]); net.v.upload(st[name]["v"]); net.age.upload(st[name]["age"])
-    for k in range(2):
-        agent.targets[k].params.upload(st[f"target{k}"]["params"])
-    agent.log_alpha.upload(st["log_alpha"]); agent.alpha_age.upload(st["alpha_age"])
+make_loop, loop_parameters, np_from, loop_state, push_state = helpers.make_loop, helpers.loop_parameters, helpers.np_from, helpers.loop_state, helpers.push_state
 
 
 def run_update(rocm, agent, A, lib, loop, batch, loss_ptr=None):
