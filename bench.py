@@ -89,7 +89,7 @@ def bench_mlp(helpers, rocm, batch, iters, warmup):
     return out
 
 
-def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000):
+def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_operation=False, phase_profile=False):
     """SAC loop steps entirely on the device: runner step with the actor, device-side gather draws and noise, training."""
     capi = helpers.capi
     lib, h = rocm.device.lib, rocm.device.handle
@@ -133,17 +133,35 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000):
 
     for _ in range(batch):        # fill the replay buffer with the warm-up policy
         env_step(0)
-    for _ in range(warmup):
-        loop_step()
-    rocm.sync()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        loop_step()
-    rocm.sync()
-    dt = time.perf_counter() - t0
+    if per_operation:             # one launch per reference operation (the API-compatible path)
+        for _ in range(warmup):
+            loop_step()
+        rocm.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loop_step()
+        rocm.sync()
+        dt = time.perf_counter() - t0
+    else:                         # the persistent kernel: all `steps` loop steps in one launch
+        ticks = rocm.zeros((16,), np.uint64)
+        outputs = capi.SacLoopOutputs(None, None, None, None, None, ticks.ptr if phase_profile else None)
+
+        def run(n, offset):
+            rocm.check(lib.rlt_rocm_sac_pendulum_loop(h, C.byref(agent.c), C.byref(runner), C.byref(rb.c), n, seed, offset, None, C.byref(outputs)))
+        run(max(warmup, 1), 0)
+        rocm.sync()
+        t0 = time.perf_counter()
+        ticks.upload(np.zeros(16, np.uint64))
+        run(steps, warmup)
+        rocm.sync()
+        dt = time.perf_counter() - t0
+        if phase_profile:
+            names = ["env step", "critic phase", "barrier", "critic Adam", "barrier", "critic weight refresh", "actor phase", "barrier", "actor Adam", "barrier", "actor weight refresh"]
+            tk = ticks.numpy()[:11].astype(np.float64) / 100.0 / steps      # 100 MHz constant clock -> microseconds per step
+            print("phase profile (us per loop step, workgroup 0):", {f"{i}:{n}": round(float(v), 2) for i, (n, v) in enumerate(zip(names, tk))}, "sum", round(float(tk.sum()), 2), file=sys.stderr, flush=True)
     p = agent.parameters()
     assert np.all(np.isfinite(p)), "SAC parameters went non-finite"
-    return {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3}
+    return {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3, "launches_per_step": (1.0 / steps) if not per_operation else None}
 
 
 def cpu_baseline(batch=256, seconds=12.0):
@@ -188,12 +206,14 @@ def cpu_baseline(batch=256, seconds=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=20000)
+    ap.add_argument("--warmup", type=int, default=1000)
     ap.add_argument("--mlp-batch", type=int, default=65536)
     ap.add_argument("--mlp-iters", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", choices=["all", "mlp", "sac"], default="all")
+    ap.add_argument("--sac-phase-profile", action="store_true", help="print the persistent kernel's per-phase time (stderr)")
+    ap.add_argument("--sac-per-operation", action="store_true", help="time the one-launch-per-operation SAC path instead of the persistent kernel")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the hot path has no cross-GPU part); use --gpus 1", file=sys.stderr)
@@ -204,7 +224,7 @@ def main():
     rocm = helpers.RocmBackend()
     info = rocm.device.info()
     mlp = bench_mlp(helpers, rocm, args.mlp_batch, args.mlp_iters, 3) if args.only in ("all", "mlp") else None
-    sac = bench_sac(helpers, rocm, args.steps, args.warmup) if args.only in ("all", "sac") else {"steps_per_s": 0.0, "ms_per_step": 0.0}
+    sac = bench_sac(helpers, rocm, args.steps, args.warmup, per_operation=args.sac_per_operation, phase_profile=args.sac_phase_profile) if args.only in ("all", "sac") else {"steps_per_s": 0.0, "ms_per_step": 0.0}
     cpu = None if (args.no_cpu_baseline or args.only == "mlp") else cpu_baseline()
     line = {
         "metric": "SAC updates/sec (critic+actor) at batch 256; fused MLP fwd+bwd TFLOP/s",
@@ -213,7 +233,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "SAC Pendulum loop step, batch 256, actor 3-64-64-2, critics 4-64-64-1, replay 10000; plus MLP 17-256-256-6 fwd+bwd at batch %d" % args.mlp_batch,
                    "device": info["name"], "compute_units": info["compute_units"]},
-        "network_updates_per_s": 3 * sac["steps_per_s"],
+        "network_updates_per_s": 3 * sac["steps_per_s"], "sac_path": "per-operation launches" if args.sac_per_operation else "persistent kernel, one launch for all steps",
     }
     if mlp:
         line["mlp_fwd_bwd_tflops"] = mlp["tflops"]

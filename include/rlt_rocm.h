@@ -398,6 +398,9 @@ typedef struct rlt_sac_loop_outputs {  /* all optional */
     float* rewards;                    /* [batch]                                                                         */
     uint8_t* terminated;               /* [batch]                                                                         */
     float* target_action_value;        /* [batch] the last step's TD targets                                              */
+    uint64_t* phase_ticks;             /* [16] profiling aid: constant-rate (100 MHz) clock ticks workgroup 0 spent per phase,
+                                          ADDED to what is there: 0 env step, 1 critic phase, 2/4/7/9 grid barriers, 3 critic Adam,
+                                          5 critic weight refresh, 6 actor phase, 8 actor Adam, 10 actor weight refresh            */
 } rlt_sac_loop_outputs;
 
 /* n_steps iterations of sac::loop::core::step (rl/algorithms/sac/loop/core/operations_generic.h:110-155, past the warm-up:

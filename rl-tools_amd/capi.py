@@ -87,7 +87,7 @@ class SacLoopInputs(C.Structure):
 
 class SacLoopOutputs(C.Structure):
     _fields_ = [("critic_loss", C.c_void_p), ("observations_actions_base", C.c_void_p), ("rewards", C.c_void_p), ("terminated", C.c_void_p),
-                ("target_action_value", C.c_void_p)]
+                ("target_action_value", C.c_void_p), ("phase_ticks", C.c_void_p)]
 
 
 I, F, P, S, U64 = C.c_int, C.c_float, C.c_void_p, C.c_size_t, C.c_uint64

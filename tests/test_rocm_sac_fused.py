@@ -18,7 +18,7 @@ def run_fused(rocm, agent, runner, draws, n_steps, with_outputs=True):
     inputs = capi.SacLoopInputs(dev["rollout_noise"].ptr, dev["initial_states"].ptr, dev["sample_offsets"].ptr, dev["noise_critic"].ptr, dev["noise_actor"].ptr)
     B = agent.batch
     loss = rocm.zeros((n_steps, 2)); oab = rocm.zeros((2, B, 4)); rew = rocm.zeros((B,)); term = rocm.zeros((B,), np.uint8); y = rocm.zeros((B,))
-    outputs = capi.SacLoopOutputs(loss.ptr, oab.ptr, rew.ptr, term.ptr, y.ptr)
+    outputs = capi.SacLoopOutputs(loss.ptr, oab.ptr, rew.ptr, term.ptr, y.ptr, None)
     lib, h = rocm.device.lib, rocm.device.handle
     rc = lib.rlt_rocm_sac_pendulum_loop(h, C.byref(agent.c), C.byref(runner.c), C.byref(runner.rb.c), n_steps, 0, 0, C.byref(inputs), C.byref(outputs) if with_outputs else None)
     assert rc == 0, lib.rlt_rocm_error_string(rc)
@@ -91,7 +91,7 @@ def test_fused_loop_device_rng_trains_and_rejects_unsupported_shapes(oracle, roc
     pos0 = int(runner.rb.position.numpy()[0])
     n = 1500
     loss = rocm.zeros((n, 2))
-    outputs = capi.SacLoopOutputs(loss.ptr, None, None, None, None)
+    outputs = capi.SacLoopOutputs(loss.ptr, None, None, None, None, None)
     rlib, h = rocm.device.lib, rocm.device.handle
     assert rlib.rlt_rocm_sac_pendulum_loop(h, C.byref(agent.c), C.byref(runner.c), C.byref(runner.rb.c), n, 7, 0, None, C.byref(outputs)) == 0
     rocm.sync()
