@@ -82,7 +82,7 @@ struct FusedArgs {
     int batch, n_steps, lds_floats;
     rlt_pendulum_runner runner;
     rlt_replay_buffer rb;
-    float* partial;            // [G][N_PARTIAL]
+    float* partial;            // [G + 1][N_PARTIAL], row G stays zero
     unsigned* barrier_counter;
     // optional host-drawn randomness (parity runs); NULL -> counter-based device RNG
     const float* rollout_noise; const float* initial_states; const uint32_t* sample_offsets;
@@ -261,7 +261,7 @@ __device__ __forceinline__ void cache_nets(lptr const (&dst)[COUNT], const float
 #pragma unroll
     for (int k = 0; k < COUNT; k++)
 #pragma unroll
-        for (int u = 0; u < N::per_thread; u++) { const int idx = tid + u * THREADS; v[k][u] = idx < N::total ? __builtin_nontemporal_load(src[k] + idx) : 0.f; }
+        for (int u = 0; u < N::per_thread; u++) { const int idx = tid + u * THREADS; v[k][u] = src[k][idx < N::total ? idx : N::total - 1]; /* unconditional: a clamped duplicate load instead of a branch */ }
 #pragma unroll
     for (int u = 0; u < N::per_thread; u++) {
         const int idx = tid + u * THREADS;
@@ -280,6 +280,26 @@ __device__ __forceinline__ float adam_element(const rlt_adam_parameters& p, floa
     v = p.beta_2 * v + (1.0f - p.beta_2) * g * g;
     const float pre_sqrt = fmaxf(v * bc2, p.epsilon_sqrt);
     return param - p.alpha * bc1 * m / (sqrtf(pre_sqrt) + p.epsilon);
+}
+
+// sum over the workgroups' partial values of one or two gradient elements, in workgroup order; the loads of 16 workgroups are in
+// flight together
+template <int E>
+__device__ __forceinline__ void sum_partials(const float* __restrict__ partial, const int (&idx)[E], int G, float (&sum)[E]) {
+#pragma unroll
+    for (int e = 0; e < E; e++) sum[e] = 0.f;
+    for (int w0 = 0; w0 < G; w0 += 16) {
+        float pv[E][16];
+#pragma unroll
+        for (int e = 0; e < E; e++)
+#pragma unroll
+            for (int u = 0; u < 16; u++) pv[e][u] = partial[(size_t)min(w0 + u, G) * N_PARTIAL + idx[e]];   // row G is all zeros: no select, no branch
+        __builtin_amdgcn_sched_barrier(0);    // all loads are issued before the first add waits for one
+#pragma unroll
+        for (int e = 0; e < E; e++)
+#pragma unroll
+            for (int u = 0; u < 16; u++) sum[e] += pv[e][u];
+    }
 }
 
 // LDS working set of one wave group
@@ -519,13 +539,8 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
                     kq[e] = idc[e] >= NC::total ? 1 : 0; o[e] = idc[e] - kq[e] * NC::total;
                     m[e] = (kq[e] ? A.critic_m[1] : A.critic_m[0])[o[e]]; v[e] = (kq[e] ? A.critic_v[1] : A.critic_v[0])[o[e]];
                     p[e] = (kq[e] ? A.critic_p[1] : A.critic_p[0])[o[e]]; t[e] = (kq[e] ? A.target_p[1] : A.target_p[0])[o[e]];
-                    gsum[e] = 0.f;
                 }
-#pragma unroll 8
-                for (int ww = 0; ww < G; ww++) {
-#pragma unroll
-                    for (int e = 0; e < 2; e++) gsum[e] += A.partial[(size_t)ww * N_PARTIAL + idc[e]];
-                }
+                sum_partials<2>(A.partial, idc, G, gsum);
 #pragma unroll
                 for (int e = 0; e < 2; e++) {
                     if (ok[e]) {
@@ -613,18 +628,19 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         {
             const int chunk = (NA::total + G - 1) / G;
             const int begin = g * chunk, end = min(NA::total, begin + chunk);
-            for (int o = begin + tid; o < end; o += THREADS) {
+            for (int base = begin; base < end; base += THREADS) {
+                const bool ok = base + tid < end;
+                const int o = ok ? base + tid : begin;      // idle lanes redo the first element and drop the result: no branch around the loads
                 float m = A.actor_m[o], v = A.actor_v[o]; const float p = A.actor_p[o];
-                float gsum = 0.f;
-#pragma unroll 8
-                for (int ww = 0; ww < G; ww++) gsum += A.partial[(size_t)ww * N_PARTIAL + 2 * NC::total + o];
-                const float pnew = adam_element(A.adam_actor, S->bc[0], S->bc[1], gsum, m, v, p);
-                A.actor_g[o] = gsum; A.actor_m[o] = m; A.actor_v[o] = v; A.actor_p[o] = pnew;
+                const int idx[1] = {2 * NC::total + o}; float gs[1];
+                sum_partials<1>(A.partial, idx, G, gs);
+                const float pnew = adam_element(A.adam_actor, S->bc[0], S->bc[1], gs[0], m, v, p);
+                if (ok) { A.actor_g[o] = gs[0]; A.actor_m[o] = m; A.actor_v[o] = v; A.actor_p[o] = pnew; }
             }
             if (g == G - 1 && tid == THREADS - 1) {   // log_alpha: gradient = mean over the batch of alpha * (entropy - target entropy)
-                float gsum = 0.f;
-                for (int ww = 0; ww < G; ww++) gsum += A.partial[(size_t)ww * N_PARTIAL + 2 * NC::total + NA::total];
-                gsum /= (float)B;
+                const int idx[1] = {2 * NC::total + NA::total}; float gs[1];
+                sum_partials<1>(A.partial, idx, G, gs);
+                const float gsum = gs[0] / (float)B;
                 float m = A.log_alpha[2], v = A.log_alpha[3];
                 const float pnew = adam_element(A.adam_alpha, S->bc[6], S->bc[7], gsum, m, v, A.log_alpha[0]);
                 A.log_alpha[1] = gsum; A.log_alpha[2] = m; A.log_alpha[3] = v; A.log_alpha[0] = pnew;
@@ -700,7 +716,7 @@ extern "C" int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac
     const int G = B / ROWS;
     const size_t n_partial = (size_t)N_PARTIAL;
     void* scratch = nullptr;
-    int rc = rlt_scratch(device, (size_t)G * n_partial * sizeof(float) + 256, &scratch);
+    int rc = rlt_scratch(device, (size_t)(G + 1) * n_partial * sizeof(float) + 256, &scratch);
     if (rc) return rc;
     FusedArgs a = {};
     a.actor_p = agent->actor[0].weights; a.actor_g = agent->actor[0].d_weights;
@@ -728,6 +744,7 @@ extern "C" int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac
     if (lds_bytes > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
     RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sac_pendulum_loop_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     RLT_HIP(hipMemsetAsync(scratch, 0, 256, device->stream));
+    RLT_HIP(hipMemsetAsync((char*)scratch + 256 + (size_t)G * n_partial * sizeof(float), 0, n_partial * sizeof(float), device->stream));
     hipLaunchKernelGGL(sac_pendulum_loop_kernel, dim3(G), dim3(THREADS), lds_bytes, device->stream, a);
     return rlt_launch_status(device);
 }
