@@ -156,9 +156,12 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_opera
         rocm.sync()
         dt = time.perf_counter() - t0
         if phase_profile:
-            names = ["env step", "critic phase", "barrier", "critic Adam", "barrier", "critic weight refresh", "actor phase", "barrier", "actor Adam", "barrier", "actor weight refresh"]
-            tk = ticks.numpy()[:11].astype(np.float64) / 100.0 / steps      # 100 MHz constant clock -> microseconds per step
-            print("phase profile (us per loop step, workgroup 0):", {f"{i}:{n}": round(float(v), 2) for i, (n, v) in enumerate(zip(names, tk))}, "sum", round(float(tk.sum()), 2), file=sys.stderr, flush=True)
+            names = ["env step", "critic phase: TD error + both backward passes", "barrier", "critic Adam", "barrier", "critic weight refresh", "actor phase", "barrier", "actor Adam", "barrier", "actor weight refresh"]
+            names += ["critic phase: batch rows into LDS", "critic phase: actor on next obs | critic 1 forward", "critic phase: target critics", "critic phase: critic 0 forward", "unused"]
+            tk = ticks.numpy()[:16].astype(np.float64) / 100.0 / steps      # 100 MHz constant clock -> microseconds per step
+            shader_cycles = tk[15] * 100.0; tk = tk[:15]; names = names[:15]
+            print("phase profile (us per loop step, workgroup 0):", {f"{i}:{n}": round(float(v), 2) for i, (n, v) in enumerate(zip(names, tk))}, "sum", round(float(tk.sum()), 2),
+                  "shader clock MHz", round(shader_cycles / tk.sum(), 1), file=sys.stderr, flush=True)
     p = agent.parameters()
     assert np.all(np.isfinite(p)), "SAC parameters went non-finite"
     return {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3, "launches_per_step": (1.0 / steps) if not per_operation else None}

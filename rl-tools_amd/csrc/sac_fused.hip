@@ -110,7 +110,9 @@ __device__ __forceinline__ void grid_barrier(unsigned* counter, unsigned target)
     __syncthreads();
     if (threadIdx.x == 0) {
         __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        while (__hip_atomic_load(counter, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) __builtin_amdgcn_s_sleep(1);
+        // poll without ordering, then acquire once: an acquiring load invalidates the caches on every iteration
+        while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) __builtin_amdgcn_s_sleep(1);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     }
     __syncthreads();
 }
@@ -134,37 +136,74 @@ __device__ __forceinline__ float clampf(float x, float lo, float hi) { return fm
 // 64-long reduction (any fixed assignment is valid as long as both operands agree). Result element v of lane l belongs to row
 // 4 kk + v and column r of the tile. The stage functions contain no barrier; the caller separates them with __syncthreads().
 
-// layer 1: h1 = relu(x W1^T + b1)
+// The weights a stage needs are loaded from the LDS copy into registers by a load_* function that the caller places BEFORE the
+// barrier the stage waits behind (weights do not depend on the previous stage), so that after the barrier only activations are read.
+struct Fwd1W { float w, b; };
+struct Fwd2W { float b[16], bias, w3[2]; };
+struct Bwd1W { float w3[2]; };
+struct Bwd2W { float b[16], wa; };
 template <class N>
-__device__ __forceinline__ void forward_stage1(lptr x, lptr h1, lptr P, int w, int lane) {
+__device__ __forceinline__ Fwd1W load_fwd1(lptr P, int w, int lane) {
+    const int r = lane & 15, kk = lane >> 4, n = 16 * w + r;
+    Fwd1W f; f.w = P[N::lw1 + n * N::LD1 + kk]; f.b = P[N::lb1 + n];
+    return f;
+}
+template <class N>
+__device__ __forceinline__ Fwd2W load_fwd2(lptr P, int w, int lane) {
+    const int r = lane & 15, kk = lane >> 4, n = 16 * w + r;
+    Fwd2W f;
+#pragma unroll
+    for (int s = 0; s < 16; s++) f.b[s] = P[N::lw2 + n * N::LD2 + kk * 16 + s];
+    f.bias = P[N::lb2 + n];
+#pragma unroll
+    for (int c = 0; c < 2; c++) f.w3[c] = c < N::OUT ? P[N::lw3 + c * N::LD2 + n] : 0.f;
+    return f;
+}
+template <class N>
+__device__ __forceinline__ Bwd1W load_bwd1(lptr P, int w, int lane) {
+    const int n = 16 * w + (lane & 15);
+    Bwd1W f;
+#pragma unroll
+    for (int c = 0; c < 2; c++) f.w3[c] = c < N::OUT ? P[N::lw3 + c * N::LD2 + n] : 0.f;
+    return f;
+}
+template <class N>
+__device__ __forceinline__ Bwd2W load_bwd2(lptr P, int w, int lane) {
+    const int r = lane & 15, kk = lane >> 4, n = 16 * w + r;
+    Bwd2W f;
+#pragma unroll
+    for (int s = 0; s < 16; s++) f.b[s] = P[N::lw2 + (kk * 16 + s) * N::LD2 + n];
+    f.wa = P[N::lw1 + n * N::LD1 + OBS];
+    return f;
+}
+
+// layer 1: h1 = relu(x W1^T + b1)
+__device__ __forceinline__ void forward_stage1(lptr x, lptr h1, const Fwd1W& f, int w, int lane) {
     const int r = lane & 15, kk = lane >> 4, n = 16 * w + r;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-    const floatx4 acc = mfma16(x[r * XS + kk], P[N::lw1 + n * N::LD1 + kk], zero);
-    const float b = P[N::lb1 + n];
+    const floatx4 acc = mfma16(x[r * XS + kk], f.w, zero);
 #pragma unroll
-    for (int v = 0; v < 4; v++) h1[(4 * kk + v) * AS + n] = fmaxf(acc[v] + b, 0.f);
+    for (int v = 0; v < 4; v++) h1[(4 * kk + v) * AS + n] = fmaxf(acc[v] + f.b, 0.f);
 }
 // layer 2: h2 = relu(h1 W2^T + b2); layer 3 as per-wavefront partial dot products: part[(c*4 + w)*ROWS + row] = sum over the
 // wavefront's 16 hidden units of h2[row][n] W3[c][n]
-template <class N>
-__device__ __forceinline__ void forward_stage2(lptr h1, lptr h2, lptr part, lptr P, int w, int lane) {
+template <int OUT>
+__device__ __forceinline__ void forward_stage2(lptr h1, lptr h2, lptr part, const Fwd2W& f, int w, int lane) {
     const int r = lane & 15, kk = lane >> 4, n = 16 * w + r;
-    float a[16], b[16];
+    float a[16];
 #pragma unroll
-    for (int s = 0; s < 16; s++) { a[s] = h1[r * AS + kk * 16 + s]; b[s] = P[N::lw2 + n * N::LD2 + kk * 16 + s]; }
+    for (int s = 0; s < 16; s++) a[s] = h1[r * AS + kk * 16 + s];
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int s = 0; s < 16; s++) acc = mfma16(a[s], b[s], acc);
-    const float bias = P[N::lb2 + n];
+    for (int s = 0; s < 16; s++) acc = mfma16(a[s], f.b[s], acc);
     float hv[4];
 #pragma unroll
-    for (int v = 0; v < 4; v++) { hv[v] = fmaxf(acc[v] + bias, 0.f); h2[(4 * kk + v) * AS + n] = hv[v]; }
+    for (int v = 0; v < 4; v++) { hv[v] = fmaxf(acc[v] + f.bias, 0.f); h2[(4 * kk + v) * AS + n] = hv[v]; }
 #pragma unroll
-    for (int c = 0; c < N::OUT; c++) {
-        const float w3 = P[N::lw3 + c * N::LD2 + n];
+    for (int c = 0; c < OUT; c++) {
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            const float t = row16_sum(hv[v] * w3);
+            const float t = row16_sum(hv[v] * f.w3[c]);
             if (r == 0) part[(c * 4 + w) * ROWS + 4 * kk + v] = t;
         }
     }
@@ -178,11 +217,11 @@ __device__ __forceinline__ float net_output(lptr part, lptr P, int row, int c) {
 // backward, layer 3 and the gate of layer 2: dp2 = (dout W3) * relu'(h2); with WANT_W also dW3, db3, db2 of the 16 rows into the
 // gradient arena Gd. dout is [ROWS][2] (gradient at the identity output).
 template <class N, bool WANT_W>
-__device__ __forceinline__ void backward_stage1(lptr h2, lptr dp2, lptr dout, lptr P, float* __restrict__ Gd, int w, int lane) {
+__device__ __forceinline__ void backward_stage1(lptr h2, lptr dp2, lptr dout, const Bwd1W& f, float* __restrict__ Gd, int w, int lane) {
     const int r = lane & 15, kk = lane >> 4, n = 16 * w + r;
-    float w3[N::OUT], wsum[N::OUT];
+    float wsum[N::OUT];
 #pragma unroll
-    for (int c = 0; c < N::OUT; c++) { w3[c] = P[N::lw3 + c * N::LD2 + n]; wsum[c] = 0.f; }
+    for (int c = 0; c < N::OUT; c++) wsum[c] = 0.f;
     float dsum = 0.f;
 #pragma unroll
     for (int v = 0; v < 4; v++) {
@@ -190,7 +229,7 @@ __device__ __forceinline__ void backward_stage1(lptr h2, lptr dp2, lptr dout, lp
         const float hv = h2[row * AS + n];
         float g = 0.f;
 #pragma unroll
-        for (int c = 0; c < N::OUT; c++) { const float dc = dout[row * 2 + c]; g += dc * w3[c]; wsum[c] += dc * hv; }
+        for (int c = 0; c < N::OUT; c++) { const float dc = dout[row * 2 + c]; g += dc * f.w3[c]; wsum[c] += dc * hv; }
         const float d = hv > 0.f ? g : 0.f;
         dp2[row * AS + n] = d;
         dsum += d;
@@ -203,31 +242,33 @@ __device__ __forceinline__ void backward_stage1(lptr h2, lptr dp2, lptr dout, lp
         if (w == 0 && lane < N::OUT) { float t = 0.f; for (int i = 0; i < ROWS; i++) t += dout[i * 2 + lane]; Gd[N::b3 + lane] = t; }
     }
 }
-// backward, layer 2 and layer 1: with WANT_W dW2 = dp2^T h1 (wavefront w owns rows [16w, 16w+16) of it), then d_h1 = dp2 W2 gated
-// by relu'(h1) stays in registers and yields db1, dW1 (vector ALU, IN <= 4 columns) and, with WANT_DACT, the per-wavefront partial
-// of the gradient wrt the action input column: part[w*ROWS + row].
-template <class N, bool WANT_W, bool WANT_DACT>
-__device__ __forceinline__ void backward_stage2(lptr x, lptr h1, lptr dp2, lptr part, lptr P, float* __restrict__ Gd, int w, int lane) {
+// backward, layer 2 weight gradient: dW2 = dp2^T h1, wavefront w owns rows [16w, 16w+16) of it
+template <class N>
+__device__ __forceinline__ void backward_w2(lptr h1, lptr dp2, float* __restrict__ Gd, int w, int lane) {
     const int r = lane & 15, kk = lane >> 4, n = 16 * w + r;
-    if (WANT_W) {
-        float a[4];
+    float a[4];
 #pragma unroll
-        for (int s = 0; s < 4; s++) a[s] = dp2[(4 * kk + s) * AS + n];
+    for (int s = 0; s < 4; s++) a[s] = dp2[(4 * kk + s) * AS + n];
 #pragma unroll
-        for (int it = 0; it < 4; it++) {
-            floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < 4; it++) {
+        floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s = 0; s < 4; s++) acc = mfma16(a[s], h1[(4 * kk + s) * AS + 16 * it + r], acc);
+        for (int s = 0; s < 4; s++) acc = mfma16(a[s], h1[(4 * kk + s) * AS + 16 * it + r], acc);
 #pragma unroll
-            for (int v = 0; v < 4; v++) Gd[N::w2 + (16 * w + 4 * kk + v) * H + 16 * it + r] = acc[v];
-        }
+        for (int v = 0; v < 4; v++) Gd[N::w2 + (16 * w + 4 * kk + v) * H + 16 * it + r] = acc[v];
     }
-    float a[16], b[16];
+}
+// backward, layer 1: d_h1 = dp2 W2 gated by relu'(h1) stays in registers and yields, with WANT_W, db1 and dW1 (vector ALU, IN <= 4
+// columns) and, with WANT_DACT, the per-wavefront partial of the gradient wrt the action input column: part[w*ROWS + row]
+template <class N, bool WANT_W, bool WANT_DACT>
+__device__ __forceinline__ void backward_l1(lptr x, lptr h1, lptr dp2, lptr part, const Bwd2W& f, float* __restrict__ Gd, int w, int lane) {
+    const int r = lane & 15, kk = lane >> 4, n = 16 * w + r;
+    float a[16];
 #pragma unroll
-    for (int s = 0; s < 16; s++) { const int o = kk * 16 + s; a[s] = dp2[r * AS + o]; b[s] = P[N::lw2 + o * N::LD2 + n]; }
+    for (int s = 0; s < 16; s++) a[s] = dp2[r * AS + kk * 16 + s];
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int s = 0; s < 16; s++) acc = mfma16(a[s], b[s], acc);
+    for (int s = 0; s < 16; s++) acc = mfma16(a[s], f.b[s], acc);
     float d[4];
 #pragma unroll
     for (int v = 0; v < 4; v++) d[v] = h1[(4 * kk + v) * AS + n] > 0.f ? acc[v] : 0.f;
@@ -244,24 +285,25 @@ __device__ __forceinline__ void backward_stage2(lptr x, lptr h1, lptr dp2, lptr 
         }
     }
     if (WANT_DACT) {
-        const float wa = P[N::lw1 + n * N::LD1 + OBS];
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            const float t = row16_sum(d[v] * wa);
+            const float t = row16_sum(d[v] * f.wa);
             if (r == 0) part[w * ROWS + 4 * kk + v] = t;
         }
     }
 }
 
-// copy of network parameters from the global arena into the padded LDS layout: all loads are issued before the first store,
-// so the whole copy costs about one memory round trip
+// copy of network parameters from the global arena into the padded LDS layout, in two halves: all loads are issued before the
+// first store, so the whole copy costs about one memory round trip, and work that does not need the new values can run between
 template <class N, int COUNT>
-__device__ __forceinline__ void cache_nets(lptr const (&dst)[COUNT], const float* const (&src)[COUNT], int tid) {
-    float v[COUNT][N::per_thread];
+__device__ __forceinline__ void load_nets(float (&v)[COUNT][N::per_thread], const float* const (&src)[COUNT], int tid) {
 #pragma unroll
     for (int k = 0; k < COUNT; k++)
 #pragma unroll
         for (int u = 0; u < N::per_thread; u++) { const int idx = tid + u * THREADS; v[k][u] = src[k][idx < N::total ? idx : N::total - 1]; /* unconditional: a clamped duplicate load instead of a branch */ }
+}
+template <class N, int COUNT>
+__device__ __forceinline__ void store_nets(lptr const (&dst)[COUNT], const float (&v)[COUNT][N::per_thread], int tid) {
 #pragma unroll
     for (int u = 0; u < N::per_thread; u++) {
         const int idx = tid + u * THREADS;
@@ -271,6 +313,12 @@ __device__ __forceinline__ void cache_nets(lptr const (&dst)[COUNT], const float
             for (int k = 0; k < COUNT; k++) dst[k][slot] = v[k][u];
         }
     }
+}
+template <class N, int COUNT>
+__device__ __forceinline__ void cache_nets(lptr const (&dst)[COUNT], const float* const (&src)[COUNT], int tid) {
+    float v[COUNT][N::per_thread];
+    load_nets<N, COUNT>(v, src, tid);
+    store_nets<N, COUNT>(dst, v, tid);
 }
 
 // Adam on one element (nn/optimizers/adam/instance/operations_generic.h:26-72)
@@ -312,10 +360,15 @@ struct GroupLds {
 };
 struct Shared {
     GroupLds grp[2];
+    float actor_h1[ROWS * AS], actor_h2[ROWS * AS];   // the actor's activations on the batch observations, kept for its backward pass
+    float actor_dout[ROWS * 2];
     float x[ROWS * XS];           // [obs | action] rows of the batch
     float nx[ROWS * XS];          // [next_obs | next_action] (S1), [obs | new action] (S3)
     float dout_actor_critic[ROWS * 2];   // -1/batch: the gradient the actor loss puts on both critics' outputs
     float new_row[16];            // the transition added this step
+    unsigned long long ticks[16]; // per-phase clock ticks of this workgroup (profiling aid), flushed at the end
+    float alpha;                  // exp(log_alpha) of this step
+    float rollout_eps[2];         // exploration noise of this step and the next (indexed by step parity)
     float bc[8];                  // Adam bias corrections of this step: actor, critic 0, critic 1, alpha
     float reward[ROWS], notdone[ROWS], next_logp[ROWS], y[ROWS], q[2][ROWS];
     float noise_c[ROWS], noise_a[ROWS], mean[ROWS], ls_raw[ROWS], act_pre[ROWS], act_a[ROWS];
@@ -338,7 +391,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
     const lptr La1 = &S->grp[grp].a1[0], La2 = &S->grp[grp].a2[0], Le1 = &S->grp[grp].e1[0], Le2 = &S->grp[grp].e2[0];
     const lptr Ldp2 = &S->grp[grp].dp2[0], Lpart = &S->grp[grp].part[0], Ldout = &S->grp[grp].dout[0];
     const lptr part0 = &S->grp[0].part[0], part1 = &S->grp[1].part[0];
-    const lptr Sx = &S->x[0], Snx = &S->nx[0];
+    const lptr Sx = &S->x[0], Snx = &S->nx[0], Ah1 = &S->actor_h1[0], Ah2 = &S->actor_h2[0];
 
     // padding columns and input buffers are read by matrix instructions against zero weights: they must hold finite values
     for (int i = tid; i < A.lds_floats; i += THREADS) ((lptr)rlt_sac_lds)[i] = 0.f;
@@ -360,9 +413,12 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
     const uint32_t age_actor0 = *A.actor_age, age_c00 = *A.critic_age[0], age_c10 = *A.critic_age[1], age_alpha0 = *A.alpha_age;
     __syncthreads();
 
+    if (tid == 0) S->rollout_eps[0] = A.rollout_noise ? A.rollout_noise[0] : randn_at(A.seed, 3, A.step_offset);
+    __syncthreads();
     unsigned long long t_prev = A.phase_ticks ? wall_clock64() : 0ull;
+    const unsigned long long shader_clock_begin = A.phase_ticks ? clock64() : 0ull;
     auto tick = [&](int phase) {
-        if (A.phase_ticks && g == 0 && tid == 0) { const unsigned long long t = wall_clock64(); A.phase_ticks[phase] += t - t_prev; t_prev = t; }
+        if (A.phase_ticks && g == 0 && threadIdx.x == 0) { const unsigned long long t = wall_clock64(); S->ticks[phase] += t - t_prev; t_prev = t; }
     };
     const int lane_invariant = lane, wave_base = wave << 6;
     for (int step = 0; step < A.n_steps; step++) {
@@ -408,7 +464,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
                     rb_ces = new_pos;
                 }
             }
-            const float eps = A.rollout_noise ? A.rollout_noise[step] : randn_at(A.seed, 3, gstep);
+            const float eps = S->rollout_eps[step & 1];
             float sn0, cs0; sincosf(th, &sn0, &cs0);
             // actor on the single observation: lane u owns hidden unit u; layer 2 reads layer 1 across lanes
             const float h1 = fmaxf(((w_actor[NA::lb1 + lane] + w_actor[NA::lw1 + lane * NA::LD1] * cs0) + w_actor[NA::lw1 + lane * NA::LD1 + 1] * sn0) + w_actor[NA::lw1 + lane * NA::LD1 + 2] * thd, 0.f);
@@ -449,6 +505,10 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             if (g == 0 && lane == 0) A.rb.episode_start[new_pos] = rb_ces;
             truncated = trunc; th = nth; thd = nthd;
             if (trunc) rb_ces = rb_pos;
+        } else if (wave == 2) {
+            // off the critical path: entropy coefficient of this step, exploration noise of the next one
+            if (lane == 0) S->alpha = expf(A.log_alpha[0]);
+            if (lane == 1 && step + 1 < A.n_steps) S->rollout_eps[(step + 1) & 1] = A.rollout_noise ? A.rollout_noise[step + 1] : randn_at(A.seed, 3, gstep + 1);
         } else if (wave == 1 && lane < 4) {
             // bias corrections 1/(1 - beta^age) of this step (adam/operations_generic.h:43-66)
             const rlt_adam_parameters& p = lane == 0 ? A.adam_actor : (lane == 3 ? A.adam_alpha : A.adam_critic);
@@ -473,10 +533,17 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         } else if (tid < ROWS * 16 + ROWS) S->noise_c[tid & 15] = noise_reg;
         else if (tid < ROWS * 16 + 2 * ROWS) S->noise_a[tid & 15] = noise_reg;
         __syncthreads();
+        tick(11);
         // A: group 0 evaluates the actor on the next observations; group 1 meanwhile runs critic 1's training forward
-        if (grp == 0) forward_stage1<NA>(Snx, Le1, w_actor, w, lane); else forward_stage1<NC>(Sx, La1, w_critic1, w, lane);
-        __syncthreads();
-        if (grp == 0) forward_stage2<NA>(Le1, Le2, Lpart, w_actor, w, lane); else forward_stage2<NC>(La1, La2, Lpart, w_critic1, w, lane);
+        {
+            Fwd1W f1; Fwd2W f2;
+            if (grp == 0) { f1 = load_fwd1<NA>(w_actor, w, lane); f2 = load_fwd2<NA>(w_actor, w, lane); }
+            else { f1 = load_fwd1<NC>(w_critic1, w, lane); f2 = load_fwd2<NC>(w_critic1, w, lane); }
+            forward_stage1(grp == 0 ? Snx : Sx, grp == 0 ? Le1 : La1, f1, w, lane);
+            __syncthreads();
+            if (grp == 0) forward_stage2<2>(Le1, Le2, Lpart, f2, w, lane); else forward_stage2<1>(La1, La2, Lpart, f2, w, lane);
+        }
+        const Fwd1W t1 = load_fwd1<NC>(w_target, w, lane); const Fwd2W t2 = load_fwd2<NC>(w_target, w, lane);
         __syncthreads();
         if (wave == 0 && lane < ROWS) {   // sample_and_squash evaluate with the external noise -> next action, its log-probability
             const float mean = net_output<NA>(part0, w_actor, lane, 0);
@@ -489,34 +556,53 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         }
         if (wave == 4 && lane < ROWS) S->q[1][lane] = net_output<NC>(part1, w_critic1, lane, 0);
         __syncthreads();
+        tick(12);
         // B: target critic k on [next_obs | next_action] by group k
-        forward_stage1<NC>(Snx, Le1, w_target, w, lane);
+        forward_stage1(Snx, Le1, t1, w, lane);
         __syncthreads();
-        forward_stage2<NC>(Le1, Le2, Lpart, w_target, w, lane);
+        forward_stage2<1>(Le1, Le2, Lpart, t2, w, lane);
+        // D (weights): group 0 runs critic 0's training forward (critic 1's is already there), group 1 the actor on the batch
+        // observations, whose result the actor phase needs (x rows are [obs | action]; the actor's weights for the action column are zero)
+        Fwd1W d1; Fwd2W d2;
+        if (grp == 0) { d1 = load_fwd1<NC>(w_critic0, w, lane); d2 = load_fwd2<NC>(w_critic0, w, lane); }
+        else { d1 = load_fwd1<NA>(w_actor, w, lane); d2 = load_fwd2<NA>(w_actor, w, lane); }
         __syncthreads();
+        tick(13);
         // C: TD target (sac/operations_generic.h:133-179)
         if (wave == 0 && lane < ROWS) {
-            const float alpha = expf(A.log_alpha[0]);
+            const float alpha = S->alpha;
             const float min_q = fminf(net_output<NC>(part0, w_target0, lane, 0), net_output<NC>(part1, w_target1, lane, 0)) - alpha * S->next_logp[lane];
             const float y = S->reward[lane] + S->notdone[lane] * A.gamma * min_q;
             S->y[lane] = y;
             if (A.out_target) A.out_target[g * ROWS + lane] = y;
         }
-        // D: critic 0's training forward by group 0 (critic 1's is already there), then both backward passes
-        if (grp == 0) forward_stage1<NC>(Sx, La1, w_critic0, w, lane);
+        // D
+        forward_stage1(Sx, grp == 0 ? La1 : Ah1, d1, w, lane);
         __syncthreads();
-        if (grp == 0) forward_stage2<NC>(La1, La2, Lpart, w_critic0, w, lane);
+        if (grp == 0) forward_stage2<1>(La1, La2, Lpart, d2, w, lane); else forward_stage2<2>(Ah1, Ah2, Lpart, d2, w, lane);
+        const Bwd1W cb1 = load_bwd1<NC>(w_critic, w, lane); const Bwd2W cb2 = load_bwd2<NC>(w_critic, w, lane);
         __syncthreads();
+        tick(14);
         if (w == 0 && lane < ROWS) {
             // d_output = (Q - y) * 2/B * loss_weight, loss_weight = B*0.5 / num_final_steps = 0.5 (sac/operations_generic.h:298-312)
             float q;
             if (grp == 0) { q = net_output<NC>(part0, w_critic0, lane, 0); S->q[0][lane] = q; } else q = S->q[1][lane];
             Ldout[lane * 2] = (q - S->y[lane]) * (2.0f / (float)B) * (((float)B * 0.5f) / (float)B);
         }
+        if (wave == 5 && lane < ROWS) {   // sample_and_squash forward of the actor phase: keeps the pre-squashing sample and the action
+            const float mean = net_output<NA>(part1, w_actor, lane, 0), ls_raw = net_output<NA>(part1, w_actor, lane, 1);
+            const float ls = clampf(ls_raw, A.sas.log_std_lower_bound, A.sas.log_std_upper_bound);
+            const float sample = mean + S->noise_a[lane] * expf(ls), act = tanhf(sample);
+            S->mean[lane] = mean; S->ls_raw[lane] = ls_raw; S->act_pre[lane] = sample; S->act_a[lane] = act;
+#pragma unroll
+            for (int j = 0; j < OBS; j++) Snx[lane * XS + j] = Sx[lane * XS + j];   // [obs | new action] rows for the critics of the actor phase
+            Snx[lane * XS + OBS] = act;
+        }
         __syncthreads();
-        backward_stage1<NC, true>(La2, Ldp2, Ldout, w_critic, my_partial + grp * NC::total, w, lane);
+        backward_stage1<NC, true>(La2, Ldp2, Ldout, cb1, my_partial + grp * NC::total, w, lane);
         __syncthreads();
-        backward_stage2<NC, true, false>(Sx, La1, Ldp2, Lpart, w_critic, my_partial + grp * NC::total, w, lane);
+        backward_w2<NC>(La1, Ldp2, my_partial + grp * NC::total, w, lane);
+        backward_l1<NC, true, false>(Sx, La1, Ldp2, Lpart, cb2, my_partial + grp * NC::total, w, lane);
         if (A.out_critic_loss && w == 0) {      // sum of squared TD errors of this workgroup's rows
             float d = lane < ROWS ? (S->q[grp][lane] - S->y[lane]) : 0.f;
             d = kk_sum(row16_sum(d * d));
@@ -560,44 +646,40 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         tick(3);
         grid_barrier(A.barrier_counter, (unsigned)G * (++barrier_index));
         tick(4);
+        // both critics are needed at once; the target critics only in the next step's critic phase: their values wait in registers
+        float fresh[4][NC::per_thread];
         {
-            const lptr dst_c[4] = {w_critic0, w_critic1, w_target0, w_target1}; const float* const src_c[4] = {A.critic_p[0], A.critic_p[1], A.target_p[0], A.target_p[1]};
-            cache_nets<NC, 4>(dst_c, src_c, tid);
+            const float* const src_c[4] = {A.critic_p[0], A.critic_p[1], A.target_p[0], A.target_p[1]};
+            load_nets<NC, 4>(fresh, src_c, tid);
+            const lptr dst_c[2] = {w_critic0, w_critic1}; const float (&crit)[2][NC::per_thread] = reinterpret_cast<const float (&)[2][NC::per_thread]>(fresh);
+            store_nets<NC, 2>(dst_c, crit, tid);
         }
         __syncthreads();
         tick(5);
         // ================= S3: actor phase =================
-        // actor forward on the current observations by group 0 (x rows are [obs | action]; the actor's weights for the action column are zero)
-        if (grp == 0) forward_stage1<NA>(Sx, La1, w_actor, w, lane);
-        __syncthreads();
-        if (grp == 0) forward_stage2<NA>(La1, La2, Lpart, w_actor, w, lane);
-        __syncthreads();
-        if (wave == 0 && lane < ROWS) {   // sample_and_squash forward: keeps the pre-squashing sample and the action
-            const float mean = net_output<NA>(part0, w_actor, lane, 0), ls_raw = net_output<NA>(part0, w_actor, lane, 1);
-            const float ls = clampf(ls_raw, A.sas.log_std_lower_bound, A.sas.log_std_upper_bound);
-            const float sample = mean + S->noise_a[lane] * expf(ls), act = tanhf(sample);
-            S->mean[lane] = mean; S->ls_raw[lane] = ls_raw; S->act_pre[lane] = sample; S->act_a[lane] = act;
-#pragma unroll
-            for (int j = 0; j < OBS; j++) Snx[lane * XS + j] = Sx[lane * XS + j];
-            Snx[lane * XS + OBS] = act;
+        // (the actor's forward on the batch observations and its sample_and_squash forward were done in the critic phase)
+        // critic k forward + backward_input on [obs | new action] by group k
+        {
+            const Fwd1W f1 = load_fwd1<NC>(w_critic, w, lane); const Fwd2W f2 = load_fwd2<NC>(w_critic, w, lane);
+            forward_stage1(Snx, Le1, f1, w, lane);
+            __syncthreads();
+            forward_stage2<1>(Le1, Le2, Lpart, f2, w, lane);
         }
-        __syncthreads();
-        // critic k forward + backward_input on [obs | new action] by group k; activations go to the e buffers so that group 0 keeps the
-        // actor's for the actor backward
-        forward_stage1<NC>(Snx, Le1, w_critic, w, lane);
-        __syncthreads();
-        forward_stage2<NC>(Le1, Le2, Lpart, w_critic, w, lane);
-        __syncthreads();
-        if (w == 0 && lane < ROWS) S->q[grp][lane] = net_output<NC>(Lpart, w_critic, lane, 0);
-        backward_stage1<NC, false>(Le2, Ldp2, &S->dout_actor_critic[0], w_critic, nullptr, w, lane);
-        __syncthreads();
-        backward_stage2<NC, false, true>(Snx, Le1, Ldp2, Lpart, w_critic, nullptr, w, lane);
+        {
+            const Bwd1W b1 = load_bwd1<NC>(w_critic, w, lane); const Bwd2W b2 = load_bwd2<NC>(w_critic, w, lane);
+            __syncthreads();
+            if (w == 0 && lane < ROWS) S->q[grp][lane] = net_output<NC>(Lpart, w_critic, lane, 0);
+            backward_stage1<NC, false>(Le2, Ldp2, &S->dout_actor_critic[0], b1, nullptr, w, lane);
+            __syncthreads();
+            backward_l1<NC, false, true>(Snx, Le1, Ldp2, Lpart, b2, nullptr, w, lane);
+        }
+        const Bwd1W ab1 = load_bwd1<NA>(w_actor, w, lane); const Bwd2W ab2 = load_bwd2<NA>(w_actor, w, lane);
         __syncthreads();
         // min-Q routing (sac/operations_generic.h:358-393), sample_and_squash backward (nn/layers/sample_and_squash/operations_generic.h:289-398)
         if (wave == 0) {
             float alpha_term = 0.f;
             if (lane < ROWS) {
-                const float alpha = expf(A.log_alpha[0]), alpha_b = alpha / (float)B;
+                const float alpha = S->alpha, alpha_b = alpha / (float)B;
                 const lptr pk = S->q[0][lane] < S->q[1][lane] ? part0 : part1;
                 const float d_out = (pk[0 * ROWS + lane] + pk[1 * ROWS + lane]) + (pk[2 * ROWS + lane] + pk[3 * ROWS + lane]);
                 const float action = S->act_a[lane];
@@ -610,7 +692,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
                 const float d_mu = gte + alpha_b * ((z / sd) + (-z / sd) + 2.0f * action);
                 float d_ls = sd * (gte * eps) + alpha_b * ((z * z - 1.0f) + (-z / sd) * eps * sd + 2.0f * action * eps * sd);
                 if (ls_raw < A.sas.log_std_lower_bound || ls_raw > A.sas.log_std_upper_bound) d_ls = 0.f;
-                S->grp[0].dout[lane * 2] = d_mu; S->grp[0].dout[lane * 2 + 1] = d_ls;
+                S->actor_dout[lane * 2] = d_mu; S->actor_dout[lane * 2 + 1] = d_ls;
                 const float lp = (-0.9189385332046727f - ls - 0.5f * z * z) - logf(1.0f - action * action + A.sas.log_probability_epsilon);
                 alpha_term = alpha * (-lp - A.sas.target_entropy);
             }
@@ -618,9 +700,16 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             if (lane == 0) my_partial[2 * NC::total + NA::total] = alpha_term;
         }
         __syncthreads();
-        if (grp == 0) backward_stage1<NA, true>(La2, Ldp2, Ldout, w_actor, my_partial + 2 * NC::total, w, lane);
+        // actor backward: layer 3 and the layer-2 gate by group 0, then the layer-2 weight gradient by group 0 and layer 1 by group 1
+        const lptr dp2a = &S->grp[0].dp2[0];
+        if (grp == 0) backward_stage1<NA, true>(Ah2, dp2a, &S->actor_dout[0], ab1, my_partial + 2 * NC::total, w, lane);
         __syncthreads();
-        if (grp == 0) backward_stage2<NA, true, false>(Sx, La1, Ldp2, Lpart, w_actor, my_partial + 2 * NC::total, w, lane);
+        if (grp == 0) backward_w2<NA>(Ah1, dp2a, my_partial + 2 * NC::total, w, lane);
+        else backward_l1<NA, true, false>(Sx, Ah1, dp2a, Lpart, ab2, my_partial + 2 * NC::total, w, lane);
+        {
+            const lptr dst_t[2] = {w_target0, w_target1}; const float (&targ)[2][NC::per_thread] = reinterpret_cast<const float (&)[2][NC::per_thread]>(fresh[2]);
+            store_nets<NC, 2>(dst_t, targ, tid);     // read next after several barriers
+        }
         tick(6);
         grid_barrier(A.barrier_counter, (unsigned)G * (++barrier_index));
         tick(7);
@@ -655,6 +744,10 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         }
         __syncthreads();
         tick(10);
+    }
+    if (A.phase_ticks && g == 0 && tid == 0) {
+        S->ticks[15] = clock64() - shader_clock_begin;     // shader clock cycles of the whole run: with the sum of the others it gives the clock rate
+        for (int i = 0; i < 16; i++) A.phase_ticks[i] += S->ticks[i];
     }
     if (g == 0 && tid == 0) {
         A.runner.states[0] = th; A.runner.states[1] = thd; A.runner.episode_return[0] = ep_return;
