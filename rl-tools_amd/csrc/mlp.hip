@@ -2,6 +2,7 @@
 // (reference: nn/layers/dense/operations_cpu_blas.h:36-228, nn_models/mlp/operations_generic.h:77-204).
 #include "common.h"
 #include "gemm.h"
+#include "mlp_fused.h"
 
 namespace {
 
@@ -76,7 +77,9 @@ size_t rlt_rocm_mlp_workspace_bytes(const rlt_dense_layer* layers, int n_layers,
     size_t per_row = 0;
     for (int i = 0; i < n_layers; i++) per_row += 2 * (size_t)layers[i].out_dim;   // private pre/out of forward_backward
     per_row += 3 * (size_t)max_dim(layers, n_layers);                                // tick, tock, upstream gradient copy
-    return align_up(per_row * (size_t)batch * sizeof(float)) + 4 * 256;
+    const size_t per_layer = align_up(per_row * (size_t)batch * sizeof(float)) + 4 * 256;
+    const size_t fused = rlt_mlp3_fused_workspace_bytes(layers, n_layers, batch);
+    return per_layer > fused ? per_layer : fused;
 }
 
 int rlt_rocm_mlp_evaluate(rlt_rocm_device* device, const rlt_dense_layer* layers, int n, const float* x, int ldx, float* y, int ldy, int batch,
@@ -183,6 +186,11 @@ int rlt_rocm_mlp_forward_backward(rlt_rocm_device* device, const rlt_dense_layer
     RLT_REQUIRE((!y || ldy >= O) && (!d_output || ldd >= O) && (!target || ldt >= O));
     for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases);
     RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_mlp_workspace_bytes(layers, n, batch));
+    {
+        // one pass over the batch with on-chip activations where the network has the shape that kernel is built for
+        const int rc = rlt_mlp3_fused_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, workspace, workspace_bytes);
+        if (rc != RLT_E_UNSUPPORTED) return rc;
+    }
     // carve private activation storage out of the workspace
     rlt_dense_layer priv[16];
     RLT_REQUIRE(n <= 16);
