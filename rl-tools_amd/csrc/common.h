@@ -78,6 +78,14 @@ __device__ __forceinline__ float rlt_dact_from_output(float o, int f) {
     }
 }
 
+// Workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every global load and store the wavefront has in
+// flight, which defeats prefetching across a barrier; kernels whose wavefronts exchange data through LDS alone use this one.
+__device__ __forceinline__ void rlt_lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // 64-lane wavefront sum (butterfly over DPP/ds_swizzle via __shfl_xor)
 __device__ __forceinline__ float rlt_wave_sum(float v) {
 #pragma unroll

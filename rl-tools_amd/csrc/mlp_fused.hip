@@ -37,17 +37,17 @@ constexpr int XSP = 33;      // LDS row stride of the input rows (in <= 32, zero
 constexpr int DS = 17;       // LDS row stride of the output-gradient rows (out <= 16, zero padded)
 constexpr int THREADS = 256;
 constexpr int MAX_WORKGROUPS = 256;
-constexpr int LDS_FLOATS = 2 * BM * HS + BM * XSP + BM * DS;
+constexpr int LDS_FLOATS = 2 * BM * HS + BM * XSP + BM * DS + 16 * HS;   // h1, h2, input rows, output-gradient rows, W3 (zero padded to 16 rows)
 
 // swizzled weight copies (floats), built once per call by mlp3_prepare_kernel
-constexpr size_t W2F_FLOATS = 65536, W2B_FLOATS = 65536, W1S_FLOATS = 8 * 16 * 64, W3B_FLOATS = 8 * 8 * 64, W3S_FLOATS = 16 * 256;
-constexpr size_t PREP_FLOATS = W2F_FLOATS + W2B_FLOATS + W1S_FLOATS + W3B_FLOATS + W3S_FLOATS;
+constexpr size_t W2F_FLOATS = 65536, W2B_FLOATS = 65536, W1S_FLOATS = 8 * 16 * 64;
+constexpr size_t PREP_FLOATS = W2F_FLOATS + W2B_FLOATS + W1S_FLOATS;
 
 struct Mlp3Args {
     const float* x; int ldx; float* y; int ldy; const float* d_output; int ldd; const float* target; int ldt; float mse_scale;
     int batch, in, out, act1, act2, act3, n_tiles;
     const float* b1; const float* b2; const float* b3;
-    const float* w2f; const float* w2b; const float* w1s; const float* w3b; const float* w3s;
+    const float* w2f; const float* w2b; const float* w1s; const float* W3;
     float* partial;      // [workgroups][count]
 };
 
@@ -56,17 +56,43 @@ __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return 
 // row of element v of a 32x32 result tile held by a lane with hi = lane >> 5
 __device__ __forceinline__ int row32(int v, int hi) { return 8 * (v >> 2) + 4 * hi + (v & 3); }
 
+// activation and its derivative from the output, with the kind as a compile-time constant: the epilogues dispatch once per phase
+// instead of once per element
+template <int ACT> __device__ __forceinline__ float act_c(float x) { return rlt_act(x, ACT); }
+template <int ACT> __device__ __forceinline__ float dact_c(float o) { return rlt_dact_from_output(o, ACT); }
+template <int ACT> struct ActKind { static constexpr int value = ACT; };
+template <class F>
+__device__ __forceinline__ void act_dispatch(int kind, F&& body) {
+    switch (kind) {
+        case RLT_ACT_RELU: body(ActKind<RLT_ACT_RELU>{}); break;
+        case RLT_ACT_TANH: body(ActKind<RLT_ACT_TANH>{}); break;
+        case RLT_ACT_FAST_TANH: body(ActKind<RLT_ACT_FAST_TANH>{}); break;
+        case RLT_ACT_SIGMOID: body(ActKind<RLT_ACT_SIGMOID>{}); break;
+        default: body(ActKind<RLT_ACT_IDENTITY>{}); break;
+    }
+}
+
+// k-step count as a compile-time constant (rounded up to a multiple of 4; the padding steps multiply zeros): straight-line code whose
+// LDS reads are all issued before the first matrix instruction waits
+template <int N> struct StepCount { static constexpr int value = N; };
+template <class F>
+__device__ __forceinline__ void steps_dispatch(int steps, F&& body) {
+    if (steps <= 4) body(StepCount<4>{});
+    else if (steps <= 8) body(StepCount<8>{});
+    else if (steps <= 12) body(StepCount<12>{});
+    else body(StepCount<16>{});
+}
+
 // Operand layouts of the matrix instructions (lane l):
 //   32x32x2: A[row l%32][k l/32], B[k l/32][col l%32], result v -> row 8(v/4) + 4(l/32) + v%4, col l%32
 //   16x16x4: A[row l%16][k l/16], B[k l/16][col l%16], result v -> row 4(l/16) + v, col l%16
 // w2f[nt][g][l][t] = W2[32nt + l%32][2(4g+t) + l/32]    B operand of h1 W2^T   for column tile nt, k-step 4g+t
 // w2b[it][g][l][t] = W2[2(4g+t) + l/32][32it + l%32]    B operand of d_pre2 W2 for column tile it
 // w1s[nt][j][l]    = W1[32nt + l%32][2j + l/32]         (0 beyond in)
-// w3b[nt][j][l]    = W3[2j + l/32][32nt + l%32]         (0 beyond out)
-// w3s[n][k]        = W3[n][k]                           (0 for n >= out)
-__global__ void mlp3_prepare_kernel(const float* __restrict__ W1, const float* __restrict__ W2, const float* __restrict__ W3, int in, int out, float* __restrict__ prep) {
+// W3 (out x 256) is small enough to sit in LDS for the whole launch (rows padded to 16 with zeros).
+__global__ void mlp3_prepare_kernel(const float* __restrict__ W1, const float* __restrict__ W2, int in, float* __restrict__ prep) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    float* w2f = prep; float* w2b = w2f + W2F_FLOATS; float* w1s = w2b + W2B_FLOATS; float* w3b = w1s + W1S_FLOATS; float* w3s = w3b + W3B_FLOATS;
+    float* w2f = prep; float* w2b = w2f + W2F_FLOATS; float* w1s = w2b + W2B_FLOATS;
     if (idx < 65536) {
         const int t = idx & 3, l = (idx >> 2) & 63, g = (idx >> 8) & 31, tile = idx >> 13;
         const int k = 2 * (4 * g + t) + (l >> 5), c = 32 * tile + (l & 31);
@@ -78,18 +104,10 @@ __global__ void mlp3_prepare_kernel(const float* __restrict__ W1, const float* _
         const int k = 2 * j + (l >> 5), n = 32 * nt + (l & 31);
         w1s[idx] = k < in ? W1[n * in + k] : 0.f;
     }
-    if (idx < (int)W3B_FLOATS) {
-        const int l = idx & 63, j = (idx >> 6) & 7, nt = idx >> 9;
-        const int o = 2 * j + (l >> 5), n = 32 * nt + (l & 31);
-        w3b[idx] = o < out ? W3[o * HID + n] : 0.f;
-    }
-    if (idx < (int)W3S_FLOATS) {
-        const int n = idx >> 8;
-        w3s[idx] = n < out ? W3[idx] : 0.f;
-    }
 }
 
-// 64 x 64 block of  A[64 x 256] (LDS, row stride HS) times a pre-swizzled 256 x 256 weight: wavefront w owns column tiles 2w, 2w+1
+// 64 x 64 block of  A[64 x 256] (LDS, row stride HS) times a pre-swizzled 256 x 256 weight: wavefront w owns column tiles 2w, 2w+1.
+// The LDS operands of k-step s+1 and the weight group two ahead are requested before the matrix instructions of step s are issued.
 __device__ __forceinline__ void contract_256(lptr a, const float* __restrict__ wsw, int w, int lane, floatx16 (&acc)[2][2]) {
     const int c32 = lane & 31, hi = lane >> 5;
     const floatx4* b0p = reinterpret_cast<const floatx4*>(wsw) + (size_t)(2 * w) * 32 * 64 + lane;
@@ -97,24 +115,28 @@ __device__ __forceinline__ void contract_256(lptr a, const float* __restrict__ w
     const lptr a0 = a + c32 * HS + hi, a1 = a0 + 32 * HS;
     floatx4 b0 = b0p[0], b1 = b1p[0];
     floatx4 n0 = b0p[64], n1 = b1p[64];
-#pragma unroll 2
+    float x0 = a0[0], x1 = a1[0];
+#pragma unroll       // fully unrolled: the rotation of the prefetch registers becomes renaming instead of copies that wait for the loads
     for (int g = 0; g < 32; g++) {
         const int gp = g + 2 < 32 ? g + 2 : 31;      // two groups ahead; the last iterations re-read the final group
         const floatx4 p0 = b0p[gp * 64], p1 = b1p[gp * 64];
+        __builtin_amdgcn_sched_barrier(0);      // the requests above are not to be moved down to their first use
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            const float x0 = a0[2 * (4 * g + t)], x1 = a1[2 * (4 * g + t)];
+            const int next = 4 * g + t + 1 < 128 ? 4 * g + t + 1 : 127;
+            const float y0 = a0[2 * next], y1 = a1[2 * next];
             acc[0][0] = mfma32(x0, b0[t], acc[0][0]);
             acc[0][1] = mfma32(x0, b1[t], acc[0][1]);
             acc[1][0] = mfma32(x1, b0[t], acc[1][0]);
             acc[1][1] = mfma32(x1, b1[t], acc[1][1]);
+            x0 = y0; x1 = y1;
         }
         b0 = n0; b1 = n1; n0 = p0; n1 = p1;
     }
 }
 
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlp3_fused_kernel(Mlp3Args A) {
-    const lptr h1 = (lptr)rlt_mlp3_lds, h2 = h1 + BM * HS, xs = h2 + BM * HS, dp3 = xs + BM * XSP;
+    const lptr h1 = (lptr)rlt_mlp3_lds, h2 = h1 + BM * HS, xs = h2 + BM * HS, dp3 = xs + BM * XSP, w3l = dp3 + BM * DS;
     const int lane_invariant = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nk1 = (A.in + 1) >> 1, nk3 = (A.out + 1) >> 1;
     const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -132,76 +154,96 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
     const float bias2[2] = {A.b2[32 * (2 * w) + (lane_invariant & 31)], A.b2[32 * (2 * w + 1) + (lane_invariant & 31)]};
     const float bias3 = (lane_invariant & 15) < A.out ? A.b3[lane_invariant & 15] : 0.f;
 
+#ifdef RLT_MLP3_PROFILE      // build-time profiling aid: shader clock cycles workgroup 0 spends in each phase, printed at the end
+    unsigned long long phase_cycles[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, t_prev = clock64();
+#define RLT_TICK(i) { const unsigned long long t_now = clock64(); phase_cycles[i] += t_now - t_prev; t_prev = t_now; }
+#else
+#define RLT_TICK(i)
+#endif
+    // W3 into LDS once (rows beyond out stay zero)
+    for (int idx = threadIdx.x; idx < 16 * HS; idx += THREADS) { const int n = idx / HS, k = idx - n * HS; w3l[idx] = (n < A.out && k < HID) ? A.W3[n * HID + k] : 0.f; }
+    // input rows and upstream gradient (or target) rows of a tile travel through registers: requested a whole tile ahead
+    // four threads per row: thread t covers columns (t & 3) + 4u of row t >> 2
+    constexpr int NX = 8, ND = 4;
+    float vx[NX], vd[ND];
+    const float* dsrc = A.target ? A.target : A.d_output; const int ldsrc = A.target ? A.ldt : A.ldd;
+    auto request_tile = [&](int tile, int tid) {
+        const int row = tid >> 2, c0 = tid & 3, grow = tile * BM + row;
+        const bool row_ok = grow < A.batch;
+        const float* xr = A.x + (size_t)(row_ok ? grow : 0) * A.ldx;
+        const float* dr = dsrc + (size_t)(row_ok ? grow : 0) * ldsrc;
+#pragma unroll
+        for (int u = 0; u < NX; u++) { const int c = c0 + 4 * u; const bool ok = row_ok && c < A.in; const float v = xr[ok ? c : 0]; vx[u] = ok ? v : 0.f; }
+#pragma unroll
+        for (int u = 0; u < ND; u++) { const int c = c0 + 4 * u; const bool ok = row_ok && c < A.out; const float v = dr[ok ? c : 0]; vd[u] = ok ? v : 0.f; }
+    };
+    request_tile(blockIdx.x, threadIdx.x);
     int lane = lane_invariant;
     for (int tile = blockIdx.x; tile < A.n_tiles; tile += gridDim.x) {
         // per-lane addresses derive from a lane index the optimiser cannot see through, or it hoists them all out of this loop and spills them
         asm volatile("" : "+v"(lane));
         const int tid = (w << 6) | lane, c32 = lane & 31, hi = lane >> 5, r16 = lane & 15, q = lane >> 4;
         const int r0 = tile * BM;
-        // ---- P0: input rows and upstream gradient (or target) rows into LDS, zero padded
-        {
-            constexpr int NX = (BM * XSP + THREADS - 1) / THREADS, ND = (BM * DS + THREADS - 1) / THREADS;
-            float vx[NX], vd[ND];
-            const float* dsrc = A.target ? A.target : A.d_output; const int ldsrc = A.target ? A.ldt : A.ldd;
+        // ---- P0: this tile's rows into LDS (zero padded), the next tile's requested; layer-1 weight fragments requested
 #pragma unroll
-            for (int u = 0; u < NX; u++) {
-                const int idx = tid + u * THREADS, row = idx / XSP, c = idx - row * XSP;
-                const bool ok = idx < BM * XSP && c < A.in && r0 + row < A.batch;
-                vx[u] = A.x[ok ? (size_t)(r0 + row) * A.ldx + c : 0];     // unconditional load of a valid address, selected below
-                vx[u] = ok ? vx[u] : 0.f;
-            }
+        for (int u = 0; u < NX; u++) xs[(tid >> 2) * XSP + (tid & 3) + 4 * u] = vx[u];
 #pragma unroll
-            for (int u = 0; u < ND; u++) {
-                const int idx = tid + u * THREADS, row = idx / DS, c = idx - row * DS;
-                const bool ok = idx < BM * DS && c < A.out && r0 + row < A.batch;
-                vd[u] = dsrc[ok ? (size_t)(r0 + row) * ldsrc + c : 0];
-                vd[u] = ok ? vd[u] : 0.f;
-            }
+        for (int u = 0; u < ND; u++) dp3[(tid >> 2) * DS + (tid & 3) + 4 * u] = vd[u];
+        float wf[2][16];
 #pragma unroll
-            for (int u = 0; u < NX; u++) { const int idx = tid + u * THREADS; if (idx < BM * XSP) xs[idx] = vx[u]; }
+        for (int a = 0; a < 2; a++)
 #pragma unroll
-            for (int u = 0; u < ND; u++) { const int idx = tid + u * THREADS; if (idx < BM * DS) dp3[idx] = vd[u]; }
-        }
-        __syncthreads();
+            for (int j = 0; j < 16; j++) wf[a][j] = A.w1s[((2 * w + a) * 16 + j) * 64 + lane];
+        if (tile + (int)gridDim.x < A.n_tiles) request_tile(tile + gridDim.x, tid);
+        rlt_lds_barrier();
+        RLT_TICK(0)
         // ---- P1: h1 = act(x W1^T + b1); wavefront w owns columns [64w, 64w+64)
 #pragma unroll
         for (int a = 0; a < 2; a++) {
             const int nt = 2 * w + a;
             floatx16 acc[2] = {zero16, zero16};
-            for (int j = 0; j < nk1; j++) {
-                const float b = A.w1s[(nt * 16 + j) * 64 + lane];
-                acc[0] = mfma32(xs[c32 * XSP + 2 * j + hi], b, acc[0]);
-                acc[1] = mfma32(xs[(32 + c32) * XSP + 2 * j + hi], b, acc[1]);
-            }
+            steps_dispatch(nk1, [&](auto steps) { constexpr int NK = decltype(steps)::value;
+                float xa[2][NK];
+#pragma unroll
+                for (int j = 0; j < NK; j++) { xa[0][j] = xs[c32 * XSP + 2 * j + hi]; xa[1][j] = xs[(32 + c32) * XSP + 2 * j + hi]; }
+#pragma unroll
+                for (int j = 0; j < NK; j++) { acc[0] = mfma32(xa[0][j], wf[a][j], acc[0]); acc[1] = mfma32(xa[1][j], wf[a][j], acc[1]); }
+            });
+            act_dispatch(A.act1, [&](auto kind) { constexpr int ACT = decltype(kind)::value;
 #pragma unroll
             for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) h1[(32 * mt + row32(v, hi)) * HS + 32 * nt + c32] = rlt_act(acc[mt][v] + bias1[a], A.act1);
+                for (int v = 0; v < 16; v++) h1[(32 * mt + row32(v, hi)) * HS + 32 * nt + c32] = act_c<ACT>(acc[mt][v] + bias1[a]);
+            });
         }
-        __syncthreads();
+        rlt_lds_barrier();
+        RLT_TICK(1)
         // ---- P2: h2 = act(h1 W2^T + b2)
         {
             floatx16 acc[2][2] = {{zero16, zero16}, {zero16, zero16}};
             contract_256(h1, A.w2f, w, lane, acc);
+            act_dispatch(A.act2, [&](auto kind) { constexpr int ACT = decltype(kind)::value;
 #pragma unroll
             for (int mt = 0; mt < 2; mt++)
 #pragma unroll
                 for (int a = 0; a < 2; a++)
 #pragma unroll
-                    for (int v = 0; v < 16; v++) h2[(32 * mt + row32(v, hi)) * HS + 32 * (2 * w + a) + c32] = rlt_act(acc[mt][a][v] + bias2[a], A.act2);
+                    for (int v = 0; v < 16; v++) h2[(32 * mt + row32(v, hi)) * HS + 32 * (2 * w + a) + c32] = act_c<ACT>(acc[mt][a][v] + bias2[a]);
+            });
         }
-        __syncthreads();
+        rlt_lds_barrier();
+        RLT_TICK(2)
         // ---- P3: y = act(h2 W3^T + b3) for rows [16w, 16w+16) (lane group q takes the reduction range [64q, 64q+64)), then d_pre3
         {
-            floatx4 acc = zero4;
-            const floatx4* wp = reinterpret_cast<const floatx4*>(A.w3s + r16 * HID + 64 * q);
+            floatx4 acc = zero4, acc2 = zero4;
+            const lptr wp = w3l + r16 * HS + 64 * q;
             const lptr ap = h2 + (16 * w + r16) * HS + 64 * q;
-#pragma unroll 4
-            for (int u = 0; u < 16; u++) {
-                const floatx4 wv = wp[u];
-#pragma unroll
-                for (int t = 0; t < 4; t++) acc = mfma16(ap[4 * u + t], wv[t], acc);
+#pragma unroll 16
+            for (int u = 0; u < 64; u += 2) {
+                acc = mfma16(ap[u], wp[u], acc);
+                acc2 = mfma16(ap[u + 1], wp[u + 1], acc2);
             }
+            acc += acc2;
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const int row = 16 * w + 4 * q + v, grow = r0 + row;
@@ -214,80 +256,141 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
                 dp3[row * DS + r16] = ok ? d : 0.f;
             }
         }
-        __syncthreads();
+        rlt_lds_barrier();
+        RLT_TICK(3)
         // ---- P4: dW3 += d_pre3^T h2 (rows = outputs, wavefront w owns columns [64w, 64w+64)); db3
-#pragma unroll 4
+#pragma unroll 8
         for (int j = 0; j < 16; j++) {
             const float a = dp3[(4 * j + q) * DS + r16];
 #pragma unroll
             for (int t = 0; t < 4; t++) aW3[t] = mfma16(a, h2[(4 * j + q) * HS + 64 * w + 16 * t + r16], aW3[t]);
         }
-        if (tid < 16) { float s = 0.f; for (int row = 0; row < BM; row++) s += dp3[row * DS + tid]; db3 += s; }
-        __syncthreads();
+        if (tid < 16) {
+            float s = 0.f;
+#pragma unroll 1
+            for (int rb = 0; rb < BM; rb += 8) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = dp3[(rb + u) * DS + tid];
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < 8; u++) s += v[u];
+            }
+            db3 += s;
+        }
+        rlt_lds_barrier();
+        RLT_TICK(4)
         // ---- P5: d_pre2 = (d_pre3 W3) * act'(h2), in place of h2
 #pragma unroll
         for (int a = 0; a < 2; a++) {
             const int nt = 2 * w + a;
             floatx16 acc[2] = {zero16, zero16};
-            for (int j = 0; j < nk3; j++) {
-                const float b = A.w3b[(nt * 8 + j) * 64 + lane];
-                acc[0] = mfma32(dp3[c32 * DS + 2 * j + hi], b, acc[0]);
-                acc[1] = mfma32(dp3[(32 + c32) * DS + 2 * j + hi], b, acc[1]);
-            }
+            steps_dispatch(nk3, [&](auto steps) { constexpr int NK = decltype(steps)::value < 8 ? decltype(steps)::value : 8;
+                float da[2][NK], wb[NK];
 #pragma unroll
-            for (int mt = 0; mt < 2; mt++)
+                for (int j = 0; j < NK; j++) { wb[j] = w3l[(2 * j + hi) * HS + 32 * nt + c32]; da[0][j] = dp3[c32 * DS + 2 * j + hi]; da[1][j] = dp3[(32 + c32) * DS + 2 * j + hi]; }
 #pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const int idx = (32 * mt + row32(v, hi)) * HS + 32 * nt + c32;
-                    h2[idx] = acc[mt][v] * rlt_dact_from_output(h2[idx], A.act2);
+                for (int j = 0; j < NK; j++) { acc[0] = mfma32(da[0][j], wb[j], acc[0]); acc[1] = mfma32(da[1][j], wb[j], acc[1]); }
+            });
+            act_dispatch(A.act2, [&](auto kind) { constexpr int ACT = decltype(kind)::value;
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++) {
+#pragma unroll
+                for (int vb = 0; vb < 16; vb += 8) {
+                    float hv[8];
+#pragma unroll
+                    for (int v = 0; v < 8; v++) hv[v] = h2[(32 * mt + row32(vb + v, hi)) * HS + 32 * nt + c32];
+#pragma unroll
+                    for (int v = 0; v < 8; v++) h2[(32 * mt + row32(vb + v, hi)) * HS + 32 * nt + c32] = acc[mt][vb + v] * dact_c<ACT>(hv[v]);
                 }
+            }
+            });
         }
-        __syncthreads();
+        rlt_lds_barrier();
+        RLT_TICK(5)
         // ---- P6: dW2 += d_pre2^T h1 (wavefront w owns row tiles 2w, 2w+1 of it); db2; d_h1 = d_pre2 W2
-#pragma unroll 2
-        for (int k = 0; k < BM / 2; k++) {
-            const lptr dr = h2 + (2 * k + hi) * HS + c32, hr = h1 + (2 * k + hi) * HS + c32;
-            const float a0 = dr[32 * (2 * w)], a1 = dr[32 * (2 * w + 1)];
+        {
+            const lptr dbase = h2 + hi * HS + c32 + 32 * (2 * w), hbase = h1 + hi * HS + c32;
+            float a0 = dbase[0], a1 = dbase[32], bv[8];
 #pragma unroll
-            for (int b = 0; b < 8; b++) {
-                const float bv = hr[32 * b];
-                aW2[0][b] = mfma32(a0, bv, aW2[0][b]);
-                aW2[1][b] = mfma32(a1, bv, aW2[1][b]);
+            for (int b = 0; b < 8; b++) bv[b] = hbase[32 * b];
+#pragma unroll 2
+            for (int k = 0; k < BM / 2; k++) {
+                const int kn = k + 1 < BM / 2 ? k + 1 : k;       // operands of the next row pair, requested before this pair's matrix instructions
+                const float na0 = dbase[2 * kn * HS], na1 = dbase[2 * kn * HS + 32];
+                float nb[8];
+#pragma unroll
+                for (int b = 0; b < 8; b++) nb[b] = hbase[2 * kn * HS + 32 * b];
+#pragma unroll
+                for (int b = 0; b < 8; b++) {
+                    aW2[0][b] = mfma32(a0, bv[b], aW2[0][b]);
+                    aW2[1][b] = mfma32(a1, bv[b], aW2[1][b]);
+                }
+                a0 = na0; a1 = na1;
+#pragma unroll
+                for (int b = 0; b < 8; b++) bv[b] = nb[b];
             }
         }
-        { float s = 0.f;
-#pragma unroll 8
-          for (int row = 0; row < BM; row++) s += h2[row * HS + tid];
-          db2 += s; }
+        {
+            float s = 0.f;
+#pragma unroll 1
+            for (int rb = 0; rb < BM; rb += 8) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = h2[(rb + u) * HS + tid];
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < 8; u++) s += v[u];
+            }
+            db2 += s;
+        }
         {
             floatx16 acc[2][2] = {{zero16, zero16}, {zero16, zero16}};
             contract_256(h2, A.w2b, w, lane, acc);
-            __syncthreads();      // every wavefront is done reading h1
+            rlt_lds_barrier();      // every wavefront is done reading h1
+            RLT_TICK(6)
             // ---- P7: d_pre1 = d_h1 * act'(h1), in place of h1
+            act_dispatch(A.act1, [&](auto kind) { constexpr int ACT = decltype(kind)::value;
 #pragma unroll
             for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-                for (int a = 0; a < 2; a++)
+                for (int a = 0; a < 2; a++) {
 #pragma unroll
-                    for (int v = 0; v < 16; v++) {
-                        const int idx = (32 * mt + row32(v, hi)) * HS + 32 * (2 * w + a) + c32;
-                        h1[idx] = acc[mt][a][v] * rlt_dact_from_output(h1[idx], A.act1);
+                    for (int vb = 0; vb < 16; vb += 8) {
+                        float hv[8];
+#pragma unroll
+                        for (int v = 0; v < 8; v++) hv[v] = h1[(32 * mt + row32(vb + v, hi)) * HS + 32 * (2 * w + a) + c32];
+#pragma unroll
+                        for (int v = 0; v < 8; v++) h1[(32 * mt + row32(vb + v, hi)) * HS + 32 * (2 * w + a) + c32] = acc[mt][a][vb + v] * dact_c<ACT>(hv[v]);
                     }
+                }
+            });
         }
-        __syncthreads();
+        rlt_lds_barrier();
+        RLT_TICK(7)
         // ---- P8: dW1 += d_pre1^T x ; db1
-#pragma unroll 2
+#pragma unroll 8
         for (int k = 0; k < BM / 2; k++) {
             const float bv = xs[(2 * k + hi) * XSP + c32];
             const lptr dr = h1 + (2 * k + hi) * HS + c32;
             aW1[0] = mfma32(dr[32 * (2 * w)], bv, aW1[0]);
             aW1[1] = mfma32(dr[32 * (2 * w + 1)], bv, aW1[1]);
         }
-        { float s = 0.f;
-#pragma unroll 8
-          for (int row = 0; row < BM; row++) s += h1[row * HS + tid];
-          db1 += s; }
-        __syncthreads();
+        {
+            float s = 0.f;
+#pragma unroll 1
+            for (int rb = 0; rb < BM; rb += 8) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = h1[(rb + u) * HS + tid];
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < 8; u++) s += v[u];
+            }
+            db1 += s;
+        }
+        rlt_lds_barrier();
+        RLT_TICK(8)
     }
     // ---- this workgroup's partial gradients: [dW1 | db1 | dW2 | db2 | dW3 | db3]
     const int tid = threadIdx.x, c32 = lane & 31, hi = lane >> 5, r16 = lane & 15, q = lane >> 4;
@@ -309,6 +412,13 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
         for (int v = 0; v < 4; v++) { const int o = 4 * q + v; if (o < A.out) pW3[o * HID + 64 * w + 16 * t + r16] = aW3[t][v]; }
     pb1[tid] = db1; pb2[tid] = db2;
     if (tid < A.out) pb3[tid] = db3;
+#ifdef RLT_MLP3_PROFILE
+    RLT_TICK(9)
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        printf("mlp3 phase cycles: load %llu | L1 %llu | L2 %llu | L3 %llu | dW3 %llu | dpre2 %llu | dW2+dh1 %llu | gate1 %llu | dW1 %llu | store %llu\n", phase_cycles[0], phase_cycles[1],
+               phase_cycles[2], phase_cycles[3], phase_cycles[4], phase_cycles[5], phase_cycles[6], phase_cycles[7], phase_cycles[8], phase_cycles[9]);
+    }
+#endif
 }
 
 // destination of gradient element e (same order as a workgroup's partial block)
@@ -363,7 +473,7 @@ int rlt_mlp3_fused_forward_backward(rlt_rocm_device* device, const rlt_dense_lay
     if (workspace_bytes < rlt_mlp3_fused_workspace_bytes(L, n, batch)) return RLT_E_UNSUPPORTED;
     if ((size_t)LDS_FLOATS * sizeof(float) > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
     float* prep = reinterpret_cast<float*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
-    hipLaunchKernelGGL(mlp3_prepare_kernel, dim3(65536 / 256), dim3(256), 0, device->stream, L[0].weights, L[1].weights, L[2].weights, L[0].in_dim, L[2].out_dim, prep);
+    hipLaunchKernelGGL(mlp3_prepare_kernel, dim3(65536 / 256), dim3(256), 0, device->stream, L[0].weights, L[1].weights, L[0].in_dim, prep);
     int rc = rlt_launch_status(device);
     if (rc) return rc;
     Mlp3Args a = {};
@@ -371,7 +481,7 @@ int rlt_mlp3_fused_forward_backward(rlt_rocm_device* device, const rlt_dense_lay
     a.batch = batch; a.in = L[0].in_dim; a.out = L[2].out_dim; a.act1 = L[0].activation; a.act2 = L[1].activation; a.act3 = L[2].activation;
     a.n_tiles = (batch + BM - 1) / BM;
     a.b1 = L[0].biases; a.b2 = L[1].biases; a.b3 = L[2].biases;
-    a.w2f = prep; a.w2b = a.w2f + W2F_FLOATS; a.w1s = a.w2b + W2B_FLOATS; a.w3b = a.w1s + W1S_FLOATS; a.w3s = a.w3b + W3B_FLOATS;
+    a.w2f = prep; a.w2b = a.w2f + W2F_FLOATS; a.w1s = a.w2b + W2B_FLOATS; a.W3 = L[2].weights;
     a.partial = prep + PREP_FLOATS;
     const int groups = workgroups_for(batch);
     const size_t lds_bytes = (size_t)LDS_FLOATS * sizeof(float);
