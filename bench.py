@@ -51,6 +51,11 @@ class HipEvents:
         return ms.value
 
 
+# HBM bytes of one mlp_forward_backward call at batch 65,536, from two counter runs (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch,
+# the factors being what the same counters read for a 256 MiB copy): fused kernel 15.4 + 77.7, reduce kernel 106.0 + 0.3, prepare 1.2 + 0.5 MiB
+MLP_CALL_HBM_BYTES = int((15422 + 77676 + 106016 + 281 + 1228 + 544) * 1024)
+
+
 def bench_mlp(helpers, rocm, batch, iters, warmup):
     capi = helpers.capi
     dims = [17, 256, 256, 6]
@@ -87,6 +92,22 @@ def bench_mlp(helpers, rocm, batch, iters, warmup):
     out["tflops"] = flop / (out["forward_backward_ms"] * 1e-3) / 1e12
     out["batch"] = batch
     return out
+
+
+def pmc_probe(helpers, rocm, batch):
+    n = 64 * 1024 * 1024      # floats: 256 MiB read + 256 MiB written per copy
+    src, dst = rocm.zeros((n,)), rocm.zeros((n,))
+    for _ in range(3):
+        rocm.call("memcpy_d2d", dst.ptr, src.ptr, n * 4)
+    rocm.sync()
+    dims = [17, 256, 256, 6]
+    rng = np.random.default_rng(0)
+    net = helpers.Mlp(rocm, dims, helpers.xavier_params(rng, dims), batch)
+    x = rocm.array(rng.standard_normal((batch, 17)).astype(np.float32)); dy = rocm.array(rng.standard_normal((batch, 6)).astype(np.float32)); y = rocm.zeros((batch, 6))
+    ws, wsn = net.workspace()
+    for _ in range(3):
+        rocm.call("mlp_forward_backward", net.layers, net.n, x.ptr, 17, y.ptr, 6, dy.ptr, 6, None, 0, 0.0, batch, ws, wsn)
+    rocm.sync()
 
 
 def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_operation=False, phase_profile=False):
@@ -216,6 +237,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", choices=["all", "mlp", "sac"], default="all")
     ap.add_argument("--sac-phase-profile", action="store_true", help="print the persistent kernel's per-phase time (stderr)")
+    ap.add_argument("--pmc-probe", action="store_true", help="for counter runs under rocprofv3 --pmc: three 256 MiB device copies (a kernel of known traffic, to scale the counters by) "
+                    "and three MLP forward+backward calls, nothing timed")
     ap.add_argument("--sac-per-operation", action="store_true", help="time the one-launch-per-operation SAC path instead of the persistent kernel")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -226,6 +249,10 @@ def main():
     import helpers
     rocm = helpers.RocmBackend()
     info = rocm.device.info()
+    if args.pmc_probe:
+        pmc_probe(helpers, rocm, args.mlp_batch)
+        rocm.close()
+        return
     mlp = bench_mlp(helpers, rocm, args.mlp_batch, args.mlp_iters, 3) if args.only in ("all", "mlp") else None
     sac = bench_sac(helpers, rocm, args.steps, args.warmup, per_operation=args.sac_per_operation, phase_profile=args.sac_phase_profile) if args.only in ("all", "sac") else {"steps_per_s": 0.0, "ms_per_step": 0.0}
     cpu = None if (args.no_cpu_baseline or args.only == "mlp") else cpu_baseline()
@@ -243,7 +270,8 @@ def main():
         line["mlp"] = mlp
         flop = (MLP_FLOP_PER_SAMPLE_FWD + MLP_FLOP_PER_SAMPLE_BWD) * mlp["batch"]
         line["roofline"] = {"bound": "mfma", "achieved": mlp["tflops"], "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": mlp["tflops"] / FP32_PEAK_TFLOPS,
-                            "traffic": None, "kernel": "mlp_forward_backward (all launches of one call)", "flop_per_launch": flop}
+                            "traffic": MLP_CALL_HBM_BYTES if mlp["batch"] == 65536 else None, "traffic_unit": "bytes per call, from rocprofv3 FETCH_SIZE / WRITE_SIZE",
+                            "kernel": "mlp_forward_backward call = mlp3_prepare_kernel + mlp3_fused_kernel + mlp3_reduce_kernel", "flop_per_launch": flop}
     if cpu:
         line["cpu_baseline"] = cpu
         line["speedup_vs_cpu_baseline"] = sac["steps_per_s"] / cpu["value"] if cpu["value"] else None
