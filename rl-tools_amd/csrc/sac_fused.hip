@@ -517,7 +517,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             S->bc[2 * lane] = 1.0f / (1.0f - powf(p.beta_1, age)); S->bc[2 * lane + 1] = 1.0f / (1.0f - powf(p.beta_2, age));
         }
         // the gathered values land in LDS (other wavefronts do this while wavefront 0 steps the environment, except for the new row)
-        __syncthreads();
+        rlt_lds_barrier();
         tick(0);
         // ================= S1: critic phase =================
         if (tid < ROWS * 16) {
@@ -532,7 +532,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             if (j == 0 && A.out_oab) A.out_oab[((size_t)B + sample) * D + OBS] = 0.f;
         } else if (tid < ROWS * 16 + ROWS) S->noise_c[tid & 15] = noise_reg;
         else if (tid < ROWS * 16 + 2 * ROWS) S->noise_a[tid & 15] = noise_reg;
-        __syncthreads();
+        rlt_lds_barrier();
         tick(11);
         // A: group 0 evaluates the actor on the next observations; group 1 meanwhile runs critic 1's training forward
         {
@@ -540,11 +540,11 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             if (grp == 0) { f1 = load_fwd1<NA>(w_actor, w, lane); f2 = load_fwd2<NA>(w_actor, w, lane); }
             else { f1 = load_fwd1<NC>(w_critic1, w, lane); f2 = load_fwd2<NC>(w_critic1, w, lane); }
             forward_stage1(grp == 0 ? Snx : Sx, grp == 0 ? Le1 : La1, f1, w, lane);
-            __syncthreads();
+            rlt_lds_barrier();
             if (grp == 0) forward_stage2<2>(Le1, Le2, Lpart, f2, w, lane); else forward_stage2<1>(La1, La2, Lpart, f2, w, lane);
         }
         const Fwd1W t1 = load_fwd1<NC>(w_target, w, lane); const Fwd2W t2 = load_fwd2<NC>(w_target, w, lane);
-        __syncthreads();
+        rlt_lds_barrier();
         if (wave == 0 && lane < ROWS) {   // sample_and_squash evaluate with the external noise -> next action, its log-probability
             const float mean = net_output<NA>(part0, w_actor, lane, 0);
             const float ls = clampf(net_output<NA>(part0, w_actor, lane, 1), A.sas.log_std_lower_bound, A.sas.log_std_upper_bound);
@@ -555,18 +555,18 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             Snx[lane * XS + OBS] = act;
         }
         if (wave == 4 && lane < ROWS) S->q[1][lane] = net_output<NC>(part1, w_critic1, lane, 0);
-        __syncthreads();
+        rlt_lds_barrier();
         tick(12);
         // B: target critic k on [next_obs | next_action] by group k
         forward_stage1(Snx, Le1, t1, w, lane);
-        __syncthreads();
+        rlt_lds_barrier();
         forward_stage2<1>(Le1, Le2, Lpart, t2, w, lane);
         // D (weights): group 0 runs critic 0's training forward (critic 1's is already there), group 1 the actor on the batch
         // observations, whose result the actor phase needs (x rows are [obs | action]; the actor's weights for the action column are zero)
         Fwd1W d1; Fwd2W d2;
         if (grp == 0) { d1 = load_fwd1<NC>(w_critic0, w, lane); d2 = load_fwd2<NC>(w_critic0, w, lane); }
         else { d1 = load_fwd1<NA>(w_actor, w, lane); d2 = load_fwd2<NA>(w_actor, w, lane); }
-        __syncthreads();
+        rlt_lds_barrier();
         tick(13);
         // C: TD target (sac/operations_generic.h:133-179)
         if (wave == 0 && lane < ROWS) {
@@ -578,10 +578,10 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         }
         // D
         forward_stage1(Sx, grp == 0 ? La1 : Ah1, d1, w, lane);
-        __syncthreads();
+        rlt_lds_barrier();
         if (grp == 0) forward_stage2<1>(La1, La2, Lpart, d2, w, lane); else forward_stage2<2>(Ah1, Ah2, Lpart, d2, w, lane);
         const Bwd1W cb1 = load_bwd1<NC>(w_critic, w, lane); const Bwd2W cb2 = load_bwd2<NC>(w_critic, w, lane);
-        __syncthreads();
+        rlt_lds_barrier();
         tick(14);
         if (w == 0 && lane < ROWS) {
             // d_output = (Q - y) * 2/B * loss_weight, loss_weight = B*0.5 / num_final_steps = 0.5 (sac/operations_generic.h:298-312)
@@ -598,9 +598,9 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             for (int j = 0; j < OBS; j++) Snx[lane * XS + j] = Sx[lane * XS + j];   // [obs | new action] rows for the critics of the actor phase
             Snx[lane * XS + OBS] = act;
         }
-        __syncthreads();
+        rlt_lds_barrier();
         backward_stage1<NC, true>(La2, Ldp2, Ldout, cb1, my_partial + grp * NC::total, w, lane);
-        __syncthreads();
+        rlt_lds_barrier();
         backward_w2<NC>(La1, Ldp2, my_partial + grp * NC::total, w, lane);
         backward_l1<NC, true, false>(Sx, La1, Ldp2, Lpart, cb2, my_partial + grp * NC::total, w, lane);
         if (A.out_critic_loss && w == 0) {      // sum of squared TD errors of this workgroup's rows
@@ -654,7 +654,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             const lptr dst_c[2] = {w_critic0, w_critic1}; const float (&crit)[2][NC::per_thread] = reinterpret_cast<const float (&)[2][NC::per_thread]>(fresh);
             store_nets<NC, 2>(dst_c, crit, tid);
         }
-        __syncthreads();
+        rlt_lds_barrier();
         tick(5);
         // ================= S3: actor phase =================
         // (the actor's forward on the batch observations and its sample_and_squash forward were done in the critic phase)
@@ -662,19 +662,19 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         {
             const Fwd1W f1 = load_fwd1<NC>(w_critic, w, lane); const Fwd2W f2 = load_fwd2<NC>(w_critic, w, lane);
             forward_stage1(Snx, Le1, f1, w, lane);
-            __syncthreads();
+            rlt_lds_barrier();
             forward_stage2<1>(Le1, Le2, Lpart, f2, w, lane);
         }
         {
             const Bwd1W b1 = load_bwd1<NC>(w_critic, w, lane); const Bwd2W b2 = load_bwd2<NC>(w_critic, w, lane);
-            __syncthreads();
+            rlt_lds_barrier();
             if (w == 0 && lane < ROWS) S->q[grp][lane] = net_output<NC>(Lpart, w_critic, lane, 0);
             backward_stage1<NC, false>(Le2, Ldp2, &S->dout_actor_critic[0], b1, nullptr, w, lane);
-            __syncthreads();
+            rlt_lds_barrier();
             backward_l1<NC, false, true>(Snx, Le1, Ldp2, Lpart, b2, nullptr, w, lane);
         }
         const Bwd1W ab1 = load_bwd1<NA>(w_actor, w, lane); const Bwd2W ab2 = load_bwd2<NA>(w_actor, w, lane);
-        __syncthreads();
+        rlt_lds_barrier();
         // min-Q routing (sac/operations_generic.h:358-393), sample_and_squash backward (nn/layers/sample_and_squash/operations_generic.h:289-398)
         if (wave == 0) {
             float alpha_term = 0.f;
@@ -699,11 +699,11 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             alpha_term = row16_sum(alpha_term);
             if (lane == 0) my_partial[2 * NC::total + NA::total] = alpha_term;
         }
-        __syncthreads();
+        rlt_lds_barrier();
         // actor backward: layer 3 and the layer-2 gate by group 0, then the layer-2 weight gradient by group 0 and layer 1 by group 1
         const lptr dp2a = &S->grp[0].dp2[0];
         if (grp == 0) backward_stage1<NA, true>(Ah2, dp2a, &S->actor_dout[0], ab1, my_partial + 2 * NC::total, w, lane);
-        __syncthreads();
+        rlt_lds_barrier();
         if (grp == 0) backward_w2<NA>(Ah1, dp2a, my_partial + 2 * NC::total, w, lane);
         else backward_l1<NA, true, false>(Sx, Ah1, dp2a, Lpart, ab2, my_partial + 2 * NC::total, w, lane);
         {
@@ -742,7 +742,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             const lptr dst_a[1] = {w_actor}; const float* const src_a[1] = {A.actor_p};
             cache_nets<NA, 1>(dst_a, src_a, tid);
         }
-        __syncthreads();
+        rlt_lds_barrier();
         tick(10);
     }
     if (A.phase_ticks && g == 0 && tid == 0) {
