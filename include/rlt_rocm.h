@@ -423,6 +423,56 @@ int rlt_rocm_ppo_gae(rlt_rocm_device* device, const float* rewards, const float*
                      const float* all_values, float* advantages, float* target_values, int ld,
                      int n_envs, int steps, float gamma, float lambda, int ignore_termination);
 
+/* The part of rl/algorithms/ppo/ppo.h:13-40 (DefaultParameters) that the update reads. */
+typedef struct rlt_ppo_parameters {
+    float epsilon_clip;                 /* EPSILON_CLIP */
+    float action_entropy_coefficient;   /* ACTION_ENTROPY_COEFFICIENT */
+    float advantage_epsilon;            /* ADVANTAGE_EPSILON */
+    int normalize_advantage;            /* NORMALIZE_ADVANTAGE: per-minibatch mean / std */
+    int learn_action_std;               /* LEARN_ACTION_STD */
+    int reserved[3];
+} rlt_ppo_parameters;
+
+/* Actor = MLP + state-independent action log_std (nn_models/mlp_unconditional_stddev/network.h), critic = MLP, their
+ * optimisers (rl/algorithms/ppo/ppo.h:62-101). The layers' pre_activations/output buffers hold `batch` rows (the
+ * minibatch size); actor_adam_tensors includes the log_std tensor. The workspace needs
+ * rlt_rocm_ppo_workspace_bytes(agent) bytes. */
+typedef struct rlt_ppo_agent {
+    const rlt_dense_layer* actor;  int n_actor_layers;
+    const rlt_dense_layer* critic; int n_critic_layers;
+    float* log_std;                     /* [action_dim] */
+    float* d_log_std;                   /* [action_dim] gradient */
+    const rlt_adam_tensor* actor_adam_tensors;  int n_actor_adam_tensors;
+    const rlt_adam_tensor* critic_adam_tensors; int n_critic_adam_tensors;
+    rlt_adam_parameters actor_adam, critic_adam;
+    uint32_t* actor_age; uint32_t* critic_age;
+    int observation_dim, observation_privileged_dim, action_dim, batch;
+    void* workspace; size_t workspace_bytes;
+} rlt_ppo_agent;
+
+size_t rlt_rocm_ppo_workspace_bytes(const rlt_ppo_agent* agent);
+
+/* The per-sample part of the update between the actor's forward and backward pass,
+ * rl/algorithms/ppo/operations_generic.h:170-269 (ADAPTIVE_LEARNING_RATE off): advantage normalisation over the
+ * minibatch, log-probability of the rollout action under the current policy (random/operations_generic.h:73-97),
+ * ratio, clipping, d loss / d mean into d_action_means, and the entropy + surrogate terms ADDED to d_log_std.
+ * Columns are passed with their row strides (floats). */
+int rlt_rocm_ppo_surrogate_gradient(rlt_rocm_device* device, const float* action_means, int ld_means, const float* log_std,
+                                    const float* actions, int ld_actions, const float* action_log_probs, int ld_log_probs,
+                                    const float* advantages, int ld_advantages, const rlt_ppo_parameters* parameters,
+                                    float* d_action_means, int ld_d, float* d_log_std, int batch, int action_dim);
+
+/* One minibatch of train(), the body of the batch loop rl/algorithms/ppo/operations_generic.h:156-318: zero_gradient,
+ * actor forward, surrogate gradient, actor backward, critic forward + MSE gradient (loss weight 0.5) + backward, Adam
+ * step of both. The dataset columns are passed with the dataset's row stride `ld`; `row_indices` (device, `batch`
+ * entries) selects the minibatch's rows -- the reference shuffles the dataset in place per epoch (:126-155), a caller
+ * here passes that permutation instead -- NULL means rows [0, batch). out_critic_loss (device scalar, optional)
+ * receives mse::evaluate of the critic on the minibatch before its update (:313). */
+int rlt_rocm_ppo_train_minibatch(rlt_rocm_device* device, const rlt_ppo_agent* agent, const rlt_ppo_parameters* parameters,
+                                 const float* observations, const float* observations_privileged, const float* actions,
+                                 const float* action_log_probs, const float* advantages, const float* target_values, int ld,
+                                 const uint32_t* row_indices, float* out_critic_loss);
+
 #ifdef __cplusplus
 }
 #endif

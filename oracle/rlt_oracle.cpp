@@ -3,6 +3,10 @@
 #include "rlt_oracle.h"
 
 #include <cmath>
+#include <algorithm>
+#include <string>
+#include <random>
+#include <sstream>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -754,6 +758,128 @@ int rlt_oracle_ppo_gae(const float* rewards, const float* terminated, const floa
             previous_value = current_step_value;
         }
     }
+    return 0;
+}
+
+// rl/algorithms/ppo/operations_generic.h:170-269 with ADAPTIVE_LEARNING_RATE off; operation order and float/double promotion as there
+int rlt_oracle_ppo_surrogate_gradient(const float* action_means, int ld_means, const float* log_std, const float* actions, int ld_actions,
+                                      const float* action_log_probs, int ld_log_probs, const float* advantages, int ld_advantages,
+                                      const rlt_ppo_parameters* P, float* d_action_means, int ld_d, float* d_log_std, int batch, int action_dim) {
+    if (!action_means || !log_std || !actions || !action_log_probs || !advantages || !P || !d_action_means || batch <= 0 || action_dim <= 0) return RLT_E_INVALID_ARGUMENT;
+    if (P->learn_action_std && !d_log_std) return RLT_E_INVALID_ARGUMENT;
+    const size_t BATCH_SIZE = (size_t)batch;
+    float advantage_mean = 0, advantage_std = 0;
+    if (P->normalize_advantage) {                                                                       // :170-180
+        for (int b = 0; b < batch; b++) {
+            float advantage = advantages[(size_t)b * ld_advantages];
+            advantage_mean += advantage;
+            advantage_std += advantage * advantage;
+        }
+        advantage_mean /= BATCH_SIZE;
+        advantage_std /= BATCH_SIZE;
+        advantage_std = std::sqrt(std::max((float)0, advantage_std - advantage_mean * advantage_mean));
+    }
+    std::vector<float> d_lp_d_ls((size_t)action_dim);
+    for (int b = 0; b < batch; b++) {                                                                   // :205-269
+        float action_log_prob = 0;
+        for (int a = 0; a < action_dim; a++) {
+            float current_action = action_means[(size_t)b * ld_means + a];
+            float rollout_action = actions[(size_t)b * ld_actions + a];
+            float current_action_log_std = log_std[a];
+            action_log_prob += normal_log_prob(current_action, current_action_log_std, rollout_action);
+            d_action_means[(size_t)b * ld_d + a] = normal_d_log_prob_d_mean(current_action, current_action_log_std, rollout_action);
+            if (P->learn_action_std) {
+                float d_entropy_loss_d_current_action_log_std = -(float)1 / BATCH_SIZE * P->action_entropy_coefficient;
+                d_log_std[a] += d_entropy_loss_d_current_action_log_std;
+                float diff = rollout_action - current_action;                                           // random/operations_generic.h:90-97
+                float sd = std::exp(current_action_log_std);
+                float pre_square = diff / sd;
+                d_lp_d_ls[a] = -1 + pre_square * pre_square;
+            }
+        }
+        float rollout_action_log_prob = action_log_probs[(size_t)b * ld_log_probs];
+        float advantage = advantages[(size_t)b * ld_advantages];
+        if (P->normalize_advantage) advantage = (advantage - advantage_mean) / (advantage_std + P->advantage_epsilon);
+        float log_ratio = action_log_prob - rollout_action_log_prob;
+        float ratio = std::exp(log_ratio);
+        float clipped_ratio = std::clamp(ratio, 1 - P->epsilon_clip, 1 + P->epsilon_clip);
+        bool clipped = ratio != clipped_ratio;
+        float normal_advantage = ratio * advantage;
+        float clipped_advantage = clipped_ratio * advantage;
+        float slippage = 0.0;
+        bool ratio_min_switch = normal_advantage - clipped_advantage <= slippage;
+        float d_loss_d_pessimistic_surrogate = -(float)1 / BATCH_SIZE;
+        float d_pessimistic_surrogate_d_normal_advantage = ratio_min_switch ? 1 : 0;
+        float d_pessimistic_surrogate_d_clipped_advantage = ratio_min_switch ? 0 : 1;
+        float d_normal_advantage_d_ratio = advantage;
+        float d_clipped_advantage_d_clipped_ratio = advantage;
+        float d_clipped_ratio_d_ratio = clipped ? 0 : 1;
+        float d_pessimistic_surrogate_d_ratio = d_pessimistic_surrogate_d_normal_advantage * d_normal_advantage_d_ratio +
+                                                d_pessimistic_surrogate_d_clipped_advantage * d_clipped_advantage_d_clipped_ratio * d_clipped_ratio_d_ratio;
+        float d_loss_d_ratio = d_loss_d_pessimistic_surrogate * d_pessimistic_surrogate_d_ratio;
+        float d_ratio_d_action_log_prob = ratio;
+        float d_loss_d_action_log_prob = d_loss_d_ratio * d_ratio_d_action_log_prob;
+        for (int a = 0; a < action_dim; a++) {
+            d_action_means[(size_t)b * ld_d + a] *= d_loss_d_action_log_prob;
+            if (P->learn_action_std) d_log_std[a] += d_loss_d_action_log_prob * d_lp_d_ls[a];
+        }
+    }
+    return 0;
+}
+
+// body of the batch loop, rl/algorithms/ppo/operations_generic.h:156-318
+int rlt_oracle_ppo_train_minibatch(const rlt_ppo_agent* A, const rlt_ppo_parameters* P, const float* observations, const float* observations_privileged,
+                                   const float* actions, const float* action_log_probs, const float* advantages, const float* target_values, int ld,
+                                   const uint32_t* row_indices, float* out_critic_loss) {
+    if (!A || !P || !observations || !observations_privileged || !actions || !action_log_probs || !advantages || !target_values || ld < 1) return RLT_E_INVALID_ARGUMENT;
+    const int B = A->batch, O = A->observation_dim, OP = A->observation_privileged_dim, AD = A->action_dim;
+    std::vector<float> obs((size_t)B * O), obsp((size_t)B * OP), act((size_t)B * AD), lp(B), adv(B), tgt(B), d_act((size_t)B * AD), d_crit(B);
+    for (int b = 0; b < B; b++) {
+        const size_t row = row_indices ? row_indices[b] : (size_t)b;
+        std::memcpy(&obs[(size_t)b * O], observations + row * ld, sizeof(float) * O);
+        std::memcpy(&obsp[(size_t)b * OP], observations_privileged + row * ld, sizeof(float) * OP);
+        std::memcpy(&act[(size_t)b * AD], actions + row * ld, sizeof(float) * AD);
+        lp[b] = action_log_probs[row * ld]; adv[b] = advantages[row * ld]; tgt[b] = target_values[row * ld];
+    }
+    int rc;
+    if ((rc = rlt_oracle_mlp_zero_gradient(A->critic, A->n_critic_layers))) return rc;                   // :158
+    if ((rc = rlt_oracle_mlp_zero_gradient(A->actor, A->n_actor_layers))) return rc;                     // :159 (clears the log_std gradient too)
+    if (A->d_log_std) for (int a = 0; a < AD; a++) A->d_log_std[a] = 0;
+    if ((rc = rlt_oracle_mlp_forward(A->actor, A->n_actor_layers, obs.data(), O, B))) return rc;          // :203
+    const float* means = A->actor[A->n_actor_layers - 1].output;
+    if ((rc = rlt_oracle_ppo_surrogate_gradient(means, AD, A->log_std, act.data(), AD, lp.data(), 1, adv.data(), 1, P, d_act.data(), AD, A->d_log_std, B, AD))) return rc;
+    if ((rc = rlt_oracle_mlp_backward(A->actor, A->n_actor_layers, obs.data(), O, d_act.data(), AD, nullptr, 0, B, 1))) return rc;   // :285
+    if ((rc = rlt_oracle_mlp_forward(A->critic, A->n_critic_layers, obsp.data(), OP, B))) return rc;     // :291
+    const float* values = A->critic[A->n_critic_layers - 1].output;
+    float loss_weight = 0.5f;
+    if ((rc = rlt_oracle_mse_gradient(values, 1, tgt.data(), 1, d_crit.data(), 1, B, 1, 0, &loss_weight))) return rc;                // :295
+    if (out_critic_loss) if ((rc = rlt_oracle_mse_evaluate(values, 1, tgt.data(), 1, B, 1, 1.0f, out_critic_loss))) return rc;       // :303
+    if ((rc = rlt_oracle_mlp_backward(A->critic, A->n_critic_layers, obsp.data(), OP, d_crit.data(), 1, nullptr, 0, B, 1))) return rc; // :298
+    if ((rc = adam_over(A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age))) return rc;                   // :305
+    return adam_over(A->critic_adam_tensors, A->n_critic_adam_tensors, &A->critic_adam, A->critic_age);                              // :306
+}
+
+// The in-place dataset shuffle of train() (rl/algorithms/ppo/operations_generic.h:126-155) restated on a row-index array: for
+// each epoch, for i in [0, n): j = uniform_int(i, n-1) (std::uniform_int_distribution on the loop's std::mt19937, as
+// random/operations_cpu.h:26-29 does), swap(rows i, j). rng_state is the engine's text form (operator<<) and is advanced in place;
+// permutations receives [epochs][n]: the original row index that sits at each position while that epoch's minibatches are taken.
+int rlt_oracle_ppo_shuffle(char* rng_state, int rng_state_capacity, int n, int epochs, uint32_t* permutations) {
+    if (!rng_state || n <= 0 || epochs <= 0 || !permutations) return RLT_E_INVALID_ARGUMENT;
+    std::mt19937 engine;
+    { std::istringstream in(rng_state); in >> engine; if (in.fail()) return RLT_E_INVALID_ARGUMENT; }
+    std::vector<uint32_t> perm((size_t)n);
+    for (int i = 0; i < n; i++) perm[i] = (uint32_t)i;
+    for (int e = 0; e < epochs; e++) {
+        for (size_t i = 0; i < (size_t)n; i++) {
+            size_t j = std::uniform_int_distribution<size_t>(i, (size_t)n - 1)(engine);
+            std::swap(perm[i], perm[j]);
+        }
+        std::memcpy(permutations + (size_t)e * n, perm.data(), sizeof(uint32_t) * n);
+    }
+    std::ostringstream out; out << engine;
+    const std::string s = out.str();
+    if ((int)s.size() + 1 > rng_state_capacity) return RLT_E_INVALID_ARGUMENT;
+    std::memcpy(rng_state, s.c_str(), s.size() + 1);
     return 0;
 }
 

@@ -93,6 +93,15 @@ int rlt_oracle_ppo_gae(const float* rewards, const float* terminated, const floa
                        float* advantages, float* target_values, int ld, int n_envs, int steps, float gamma, float lambda,
                        int ignore_termination);
 
+int rlt_oracle_ppo_surrogate_gradient(const float* action_means, int ld_means, const float* log_std, const float* actions, int ld_actions,
+                                      const float* action_log_probs, int ld_log_probs, const float* advantages, int ld_advantages,
+                                      const rlt_ppo_parameters* parameters, float* d_action_means, int ld_d, float* d_log_std, int batch, int action_dim);
+int rlt_oracle_ppo_train_minibatch(const rlt_ppo_agent* agent, const rlt_ppo_parameters* parameters, const float* observations,
+                                   const float* observations_privileged, const float* actions, const float* action_log_probs,
+                                   const float* advantages, const float* target_values, int ld, const uint32_t* row_indices, float* out_critic_loss);
+/* the reference's per-epoch in-place dataset shuffle as row permutations, driven by the text form of its std::mt19937 */
+int rlt_oracle_ppo_shuffle(char* rng_state, int rng_state_capacity, int n, int epochs, uint32_t* permutations);
+
 #ifdef __cplusplus
 }
 #endif

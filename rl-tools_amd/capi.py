@@ -90,6 +90,25 @@ class SacLoopOutputs(C.Structure):
                 ("target_action_value", C.c_void_p), ("phase_ticks", C.c_void_p)]
 
 
+class PpoParameters(C.Structure):
+    _fields_ = [("epsilon_clip", C.c_float), ("action_entropy_coefficient", C.c_float), ("advantage_epsilon", C.c_float),
+                ("normalize_advantage", C.c_int32), ("learn_action_std", C.c_int32), ("reserved", C.c_int32 * 3)]
+
+
+def ppo_parameters(epsilon_clip=0.2, action_entropy_coefficient=0.01, advantage_epsilon=1e-8, normalize_advantage=1, learn_action_std=1):
+    return PpoParameters(epsilon_clip, action_entropy_coefficient, advantage_epsilon, normalize_advantage, learn_action_std)
+
+
+class PpoAgent(C.Structure):
+    _fields_ = [("actor", C.POINTER(DenseLayer)), ("n_actor_layers", C.c_int32), ("critic", C.POINTER(DenseLayer)), ("n_critic_layers", C.c_int32),
+                ("log_std", C.c_void_p), ("d_log_std", C.c_void_p),
+                ("actor_adam_tensors", C.POINTER(AdamTensor)), ("n_actor_adam_tensors", C.c_int32),
+                ("critic_adam_tensors", C.POINTER(AdamTensor)), ("n_critic_adam_tensors", C.c_int32),
+                ("actor_adam", AdamParameters), ("critic_adam", AdamParameters), ("actor_age", C.c_void_p), ("critic_age", C.c_void_p),
+                ("observation_dim", C.c_int32), ("observation_privileged_dim", C.c_int32), ("action_dim", C.c_int32), ("batch", C.c_int32),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+
+
 I, F, P, S, U64 = C.c_int, C.c_float, C.c_void_p, C.c_size_t, C.c_uint64
 LP = C.POINTER(DenseLayer)
 
@@ -125,6 +144,8 @@ PROTOTYPES = {
     "gather_batch": [C.POINTER(ReplayBuffer), P, P, I, I, I, P, P, P, P, P, P, P],
     "pendulum_step": [C.POINTER(PendulumParameters), P, P, P, P, P, I],
     "ppo_gae": [P, P, P, P, P, P, I, I, I, F, F, I],
+    "ppo_surrogate_gradient": [P, I, P, P, I, P, I, P, I, C.POINTER(PpoParameters), P, I, P, I, I],
+    "ppo_train_minibatch": [C.POINTER(PpoAgent), C.POINTER(PpoParameters), P, P, P, P, P, P, I, P, P],
 }
 # workspace arguments exist only in the device ABI (the CPU checker allocates its own)
 ROCM_ONLY = {
@@ -137,6 +158,7 @@ ROCM_ONLY = {
     "randn_f32": ([P, P, S, U64, U64], I), "rand_f32": ([P, P, S, F, F, U64, U64], I),
     "reduce_sum_f32": ([P, P, S, I, P], I),
     "mlp_workspace_bytes": ([LP, I, I], S),
+    "ppo_workspace_bytes": ([C.POINTER(PpoAgent)], S),
     "gather_draw": ([P, C.POINTER(ReplayBuffer), I, U64, U64, P, P], I),
     "sac_pendulum_loop": ([P, C.POINTER(SacAgent), C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, U64, U64, C.POINTER(SacLoopInputs),
                            C.POINTER(SacLoopOutputs)], I),

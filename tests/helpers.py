@@ -60,6 +60,7 @@ def load_oracle():
     lib.rlt_oracle_d_activation.argtypes = [C.c_float, I]; lib.rlt_oracle_d_activation.restype = C.c_float
     lib.rlt_oracle_pendulum_runner_step.argtypes = [C.POINTER(capi.PendulumRunner), C.POINTER(capi.ReplayBuffer), I, C.POINTER(capi.DenseLayer), I,
                                                     C.POINTER(capi.SasParameters), P, P, P]
+    lib.rlt_oracle_ppo_shuffle.argtypes = [C.c_char_p, I, I, I, P]
     lib.rlt_oracle_sac_loop_create.argtypes = [C.POINTER(LoopConfig)]; lib.rlt_oracle_sac_loop_create.restype = P
     for f in ("destroy", "step"):
         getattr(lib, "rlt_oracle_sac_loop_" + f).argtypes = [P]
@@ -215,6 +216,36 @@ class Mlp:
             return None, 0
         nbytes = self.backend.device.lib.rlt_rocm_mlp_workspace_bytes(self.layers, self.n, self.batch)
         return self.backend.workspace(nbytes)
+
+
+class PpoOnBackend:
+    """PPO actor (MLP + action log_std), critic and their Adam state on one backend. Flat parameter order:
+    actor [W|b per layer], log_std, critic [W|b per layer] (what the reference harness exports)."""
+
+    def __init__(self, backend, obs_dim, action_dim, actor_hidden, critic_hidden, batch, params, actor_act="relu", critic_act="relu",
+                 adam=None, obs_privileged_dim=None):
+        self.backend, self.batch, self.action_dim = backend, batch, action_dim
+        opd = obs_dim if obs_privileged_dim is None else obs_privileged_dim
+        adims, cdims = [obs_dim, actor_hidden, actor_hidden, action_dim], [opd, critic_hidden, critic_hidden, 1]
+        na, nc = mlp_param_count(adims), mlp_param_count(cdims)
+        assert params.size == na + action_dim + nc
+        self.actor = Mlp(backend, adims, params[:na], batch, actor_act, "identity")
+        self.critic = Mlp(backend, cdims, params[na + action_dim:], batch, critic_act, "identity")
+        self.log_std = backend.array(params[na:na + action_dim].astype(np.float32))
+        self.d_log_std, self.m_log_std, self.v_log_std = (backend.zeros((action_dim,)) for _ in range(3))
+        tensors = list(self.actor.adam) + [capi.AdamTensor(self.log_std.ptr, self.d_log_std.ptr, self.m_log_std.ptr, self.v_log_std.ptr, None, action_dim, 1)]
+        self.actor_adam = (capi.AdamTensor * len(tensors))(*tensors)
+        adam = adam or capi.adam_parameters(epsilon=1e-8)
+        self.c = capi.PpoAgent(self.actor.layers, self.actor.n, self.critic.layers, self.critic.n, self.log_std.ptr, self.d_log_std.ptr,
+                               self.actor_adam, len(tensors), self.critic.adam, self.critic.n_adam, adam, adam, self.actor.age.ptr, self.critic.age.ptr,
+                               obs_dim, opd, action_dim, batch, None, 0)
+        if backend.name == "rocm":
+            n = backend.device.lib.rlt_rocm_ppo_workspace_bytes(C.byref(self.c))
+            self.ws = backend.device.empty((int(n),), np.uint8)
+            self.c.workspace, self.c.workspace_bytes = self.ws.ptr, n
+
+    def parameters(self):
+        return np.concatenate([self.actor.params.numpy(), self.log_std.numpy(), self.critic.params.numpy()])
 
 
 class ReplayOnBackend:
@@ -376,3 +407,67 @@ def collect_loop_draws(oracle, loop, batch, n_steps):
         d["noise_actor"][t, :, 0] = np_from(lib.rlt_oracle_sac_loop_noise_actor(loop), (batch,))
         d["critic_loss"][t] = [lib.rlt_oracle_sac_loop_critic_loss(loop, 0), lib.rlt_oracle_sac_loop_critic_loss(loop, 1)]
     return d
+
+
+REF_PPO_GENERIC = os.path.join(ROOT, "oracle", "_ref", "librlt_ref_ppo_generic.so")
+PPO_COLUMNS = ("all_observations_privileged", "observations", "actions_mean", "actions", "action_log_probs", "rewards", "terminated", "truncated",
+               "all_reset", "reset", "all_values", "values", "advantages", "target_values")
+
+
+class RefPpo:
+    """The reference's own PPO-on-Pendulum loop through oracle/ref_harness/ref_ppo_pendulum.cpp."""
+
+    def __init__(self, seed=0):
+        lib = C.CDLL(REF_PPO_GENERIC)
+        P = C.c_void_p
+        lib.rlt_ref_ppo_create.restype = P
+        lib.rlt_ref_ppo_parameter_count.restype = C.c_size_t
+        for f, args in dict(destroy=[P], collect_and_gae=[P], train=[P], parameter_count=[P], get_parameters=[P, P], get_dataset=[P, P], columns=[P, P],
+                            hyperparameters=[P, P], get_ages=[P, P], get_rng_state=[P, C.c_char_p, C.c_int]).items():
+            getattr(lib, "rlt_ref_ppo_" + f).argtypes = args
+        self.lib, self.h = lib, P(lib.rlt_ref_ppo_create(seed))
+        d = (C.c_int * 11)(); lib.rlt_ref_ppo_dims(d)
+        (self.n_envs, self.steps, self.data_dim, self.rows, self.obs_dim, self.action_dim, self.batch, self.epochs, self.actor_hidden, self.critic_hidden,
+         self.episode_step_limit) = list(d)
+        c = (C.c_int * 14)(); lib.rlt_ref_ppo_columns(self.h, c)
+        self.col = dict(zip(PPO_COLUMNS, list(c)))
+        hy = (C.c_float * 12)(); lib.rlt_ref_ppo_hyperparameters(self.h, hy)
+        self.hyper = dict(zip(("gamma", "lambda", "epsilon_clip", "action_entropy_coefficient", "advantage_epsilon", "normalize_advantage", "learn_action_std",
+                               "alpha", "beta_1", "beta_2", "epsilon", "epsilon_sqrt"), [float(x) for x in hy]))
+
+    def parameters(self):
+        p = np.zeros(self.lib.rlt_ref_ppo_parameter_count(self.h), np.float32)
+        self.lib.rlt_ref_ppo_get_parameters(self.h, p.ctypes.data)
+        return p
+
+    def dataset(self):
+        d = np.zeros((self.rows, self.data_dim), np.float32)
+        self.lib.rlt_ref_ppo_get_dataset(self.h, d.ctypes.data)
+        return d
+
+    def rng_state(self):
+        buf = C.create_string_buffer(16384)
+        assert self.lib.rlt_ref_ppo_get_rng_state(self.h, buf, 16384) <= 16384
+        return buf
+
+    def ages(self):
+        a = (C.c_uint32 * 2)(); self.lib.rlt_ref_ppo_get_ages(self.h, a)
+        return list(a)
+
+    def close(self):
+        self.lib.rlt_ref_ppo_destroy(self.h)
+
+
+def ppo_train_like_reference(backend, agent, params, dataset, ld, col, n_rows, permutations, batch):
+    """train() of the reference on one collected dataset: for every epoch and minibatch one ppo_train_minibatch call on the rows the
+    reference's in-place shuffle would have put there (rl/algorithms/ppo/operations_generic.h:123-318)."""
+    losses = []
+    loss = backend.zeros((1,))
+    for perm in permutations:
+        idx = backend.array(perm.astype(np.uint32))
+        for b in range(n_rows // batch):
+            backend.call("ppo_train_minibatch", C.byref(agent.c), C.byref(params), dataset.offset(col["observations"]), dataset.offset(col["all_observations_privileged"]),
+                         dataset.offset(col["actions"]), dataset.offset(col["action_log_probs"]), dataset.offset(col["advantages"]),
+                         dataset.offset(col["target_values"]), ld, idx.offset(b * batch), loss.ptr)
+            losses.append(float(loss.numpy()[0]))
+    return losses

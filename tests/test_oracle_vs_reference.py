@@ -110,3 +110,40 @@ def test_blas_flavour_of_reference_agrees_for_one_update(oracle):
         lib.rlt_oracle_sac_loop_step(loop); ref.rlt_ref_sac_step(h)
     lib.rlt_oracle_sac_loop_get_parameters(loop, po.ctypes.data); ref.rlt_ref_sac_get_parameters(h, pr.ctypes.data)
     assert helpers.rel_err(po, pr) <= 1e-5
+
+
+@pytest.mark.skipif(not os.path.exists(helpers.REF_PPO_GENERIC), reason="oracle/_ref PPO harness not built (needs /root/reference)")
+def test_ppo_gae_and_update_bit_exact_with_reference(oracle):
+    """Three loop steps of the reference's PPO-on-Pendulum loop (8 envs x 40 steps, episodes truncated after 25 steps, 3 epochs of
+    5 shuffled minibatches): the restated GAE reproduces the dataset's advantages and target values, and the restated update
+    (surrogate gradient, log_std gradient, critic MSE, Adam) driven by the restated shuffle reproduces every parameter, bit for bit."""
+    capi = helpers.capi
+    ref = helpers.RefPpo(0)
+    hy = ref.hyper
+    adam = capi.adam_parameters(hy["alpha"], hy["beta_1"], hy["beta_2"], hy["epsilon"], hy["epsilon_sqrt"])
+    pp = capi.ppo_parameters(hy["epsilon_clip"], hy["action_entropy_coefficient"], hy["advantage_epsilon"], int(hy["normalize_advantage"]), int(hy["learn_action_std"]))
+    agent = helpers.PpoOnBackend(oracle, ref.obs_dim, ref.action_dim, ref.actor_hidden, ref.critic_hidden, ref.batch, ref.parameters(), "tanh", "relu", adam)
+    n = ref.n_envs * ref.steps
+    for loop_step in range(3):
+        ref.lib.rlt_ref_ppo_collect_and_gae(ref.h)
+        d = ref.dataset()
+        c = ref.col
+        assert d[:n, c["truncated"]].sum() >= ref.n_envs       # the case GAE treats specially does occur
+        # GAE (rl/algorithms/ppo/operations_generic.h:60-95)
+        dd = oracle.array(d)
+        adv, tgt = oracle.zeros((ref.rows, ref.data_dim)), oracle.zeros((ref.rows, ref.data_dim))
+        oracle.call("ppo_gae", dd.offset(c["rewards"]), dd.offset(c["terminated"]), dd.offset(c["truncated"]), dd.offset(c["all_values"]), adv.ptr, tgt.ptr,
+                    ref.data_dim, ref.n_envs, ref.steps, hy["gamma"], hy["lambda"], 0)
+        assert np.array_equal(adv.numpy()[:n, 0], d[:n, c["advantages"]]) and np.array_equal(tgt.numpy()[:n, 0], d[:n, c["target_values"]])
+        # the update
+        assert np.array_equal(agent.parameters(), ref.parameters())
+        state = ref.rng_state()
+        perms = np.zeros((ref.epochs, n), np.uint32)
+        assert oracle.lib.rlt_oracle_ppo_shuffle(state, 16384, n, ref.epochs, perms.ctypes.data) == 0
+        ref.lib.rlt_ref_ppo_train(ref.h)
+        assert ref.rng_state().value == state.value             # the restated shuffle drew exactly what the reference drew
+        helpers.ppo_train_like_reference(oracle, agent, pp, dd, ref.data_dim, c, n, perms, ref.batch)
+        got, want = agent.parameters(), ref.parameters()
+        assert np.array_equal(got, want), (loop_step, np.abs(got - want).max())
+        assert ref.ages() == [int(agent.actor.age.numpy()[0]), int(agent.critic.age.numpy()[0])]
+    ref.close()
