@@ -1,6 +1,7 @@
-// PPO generalized advantage estimation.
-// reference: rl/algorithms/ppo/operations_generic.h:60-95 (serial double loop on the host; rows are step-major,
-// row = step * n_envs + env, rl/components/on_policy_runner/on_policy_runner.h:38-72).
+// PPO: generalized advantage estimation and the minibatch update.
+// reference: rl/algorithms/ppo/operations_generic.h:60-95 (GAE: serial double loop on the host; rows are step-major,
+// row = step * n_envs + env, rl/components/on_policy_runner/on_policy_runner.h:38-72) and :96-330 (train: per-sample loops on the
+// host around the networks' forward / backward passes).
 #include "common.h"
 
 namespace {
@@ -26,6 +27,100 @@ __global__ __launch_bounds__(256) void gae_kernel(const float* __restrict__ rewa
         }
     }
 }
+
+// ---- minibatch update (train(), rl/algorithms/ppo/operations_generic.h:156-318)
+
+// rows of the dataset selected by row_indices (or [0, batch)) into packed minibatch buffers; 16 lanes per row
+__global__ __launch_bounds__(256) void ppo_gather_kernel(const float* __restrict__ observations, const float* __restrict__ observations_privileged,
+                                                         const float* __restrict__ actions, const float* __restrict__ log_probs, const float* __restrict__ advantages,
+                                                         const float* __restrict__ targets, int ld, const uint32_t* __restrict__ row_indices, int batch, int O, int OP, int A,
+                                                         float* __restrict__ obs, float* __restrict__ obsp, float* __restrict__ act, float* __restrict__ lp,
+                                                         float* __restrict__ adv, float* __restrict__ tgt) {
+    const int sub = threadIdx.x & 15;
+    for (int b = (blockIdx.x * blockDim.x + threadIdx.x) >> 4; b < batch; b += (gridDim.x * blockDim.x) >> 4) {
+        const size_t row = row_indices ? row_indices[b] : (size_t)b;
+        for (int c = sub; c < O; c += 16) obs[(size_t)b * O + c] = observations[row * ld + c];
+        for (int c = sub; c < OP; c += 16) obsp[(size_t)b * OP + c] = observations_privileged[row * ld + c];
+        for (int c = sub; c < A; c += 16) act[(size_t)b * A + c] = actions[row * ld + c];
+        if (sub == 0) { lp[b] = log_probs[row * ld]; adv[b] = advantages[row * ld]; tgt[b] = targets[row * ld]; }
+    }
+}
+
+// advantage mean and standard deviation over the minibatch (:170-180), one workgroup, fixed summation order: stats = {mean, std}
+__global__ __launch_bounds__(1024) void ppo_advantage_stats_kernel(const float* __restrict__ advantages, int ld, int batch, int normalize, float* __restrict__ stats) {
+    __shared__ float s1[16], s2[16];
+    float a = 0.f, q = 0.f;
+    if (normalize) for (int b = threadIdx.x; b < batch; b += 1024) { const float v = advantages[(size_t)b * ld]; a += v; q += v * v; }
+    a = rlt_wave_sum(a); q = rlt_wave_sum(q);
+    if ((threadIdx.x & 63) == 0) { s1[threadIdx.x >> 6] = a; s2[threadIdx.x >> 6] = q; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float m = 0.f, v = 0.f;
+        for (int i = 0; i < 16; i++) { m += s1[i]; v += s2[i]; }
+        m /= (float)batch; v /= (float)batch;
+        stats[0] = normalize ? m : 0.f;
+        stats[1] = normalize ? sqrtf(fmaxf(0.f, v - m * m)) : 0.f;
+    }
+}
+
+// per sample (:205-269): log-probability of the rollout action under the current policy, ratio, clipping, d loss / d mean; the
+// surrogate part of the log_std gradient as per-workgroup partial sums partial[block][action]
+constexpr int PPO_MAX_ACTION_DIM = 64;
+__global__ __launch_bounds__(256) void ppo_surrogate_kernel(const float* __restrict__ means, int ld_means, const float* __restrict__ log_std,
+                                                            const float* __restrict__ actions, int ld_actions, const float* __restrict__ log_probs, int ld_lp,
+                                                            const float* __restrict__ advantages, int ld_adv, rlt_ppo_parameters P, const float* __restrict__ stats,
+                                                            float* __restrict__ d_means, int ld_d, float* __restrict__ partial, int batch, int A) {
+    __shared__ float red[4][PPO_MAX_ACTION_DIM];
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool ok = b < batch;
+    float d_loss_d_lp = 0.f;
+    if (ok) {
+        float lp = 0.f;
+        for (int a = 0; a < A; a++) {
+            const float mean = means[(size_t)b * ld_means + a], ls = log_std[a], value = actions[(size_t)b * ld_actions + a];
+            const float pre = (value - mean) / expf(ls);
+            lp += (-0.9189385332046727f - ls) - 0.5f * pre * pre;        // random/operations_generic.h:73-81
+        }
+        float advantage = advantages[(size_t)b * ld_adv];
+        if (P.normalize_advantage) advantage = (advantage - stats[0]) / (stats[1] + P.advantage_epsilon);
+        const float ratio = expf(lp - log_probs[(size_t)b * ld_lp]);
+        const float clipped_ratio = fminf(fmaxf(ratio, 1.0f - P.epsilon_clip), 1.0f + P.epsilon_clip);
+        const bool clipped = ratio != clipped_ratio;
+        const bool ratio_min_switch = ratio * advantage - clipped_ratio * advantage <= 0.0f;
+        const float d_surrogate_d_ratio = ratio_min_switch ? advantage : (clipped ? 0.0f : advantage);
+        d_loss_d_lp = (-1.0f / (float)batch) * d_surrogate_d_ratio * ratio;
+    }
+    for (int a = 0; a < A; a++) {
+        float g_ls = 0.f;
+        if (ok) {
+            const float mean = means[(size_t)b * ld_means + a], ls = log_std[a], value = actions[(size_t)b * ld_actions + a];
+            const float sd = expf(ls), pre = (value - mean) / sd;
+            d_means[(size_t)b * ld_d + a] = d_loss_d_lp * (pre / sd);     // d log_prob / d mean (:82-88)
+            g_ls = d_loss_d_lp * (pre * pre - 1.0f);                      // d log_prob / d log_std (:89-96)
+        }
+        g_ls = rlt_wave_sum(g_ls);
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6][a] = g_ls;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < A) partial[(size_t)blockIdx.x * A + threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+}
+// d_log_std[a] += sum of the partials (workgroup order) + the entropy term batch * (-1/batch * coefficient) (:229-233)
+__global__ void ppo_log_std_gradient_kernel(const float* __restrict__ partial, int blocks, int A, float entropy_coefficient, float* __restrict__ d_log_std) {
+    const int a = blockIdx.x * blockDim.x + threadIdx.x;
+    if (a >= A) return;
+    float s = 0.f;
+    for (int i = 0; i < blocks; i++) s += partial[(size_t)i * A + a];
+    d_log_std[a] += s - entropy_coefficient;
+}
+
+bool ppo_agent_ok(const rlt_ppo_agent* A) {
+    return A && A->actor && A->critic && A->n_actor_layers >= 1 && A->n_critic_layers >= 1 && A->log_std && A->actor_adam_tensors && A->critic_adam_tensors &&
+           A->actor_age && A->critic_age && A->observation_dim >= 1 && A->observation_privileged_dim >= 1 && A->action_dim >= 1 && A->action_dim <= PPO_MAX_ACTION_DIM &&
+           A->batch >= 1 && A->actor[0].in_dim == A->observation_dim && A->actor[A->n_actor_layers - 1].out_dim == A->action_dim &&
+           A->critic[0].in_dim == A->observation_privileged_dim && A->critic[A->n_critic_layers - 1].out_dim == 1 && A->actor[A->n_actor_layers - 1].output;
+}
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+size_t ppo_surrogate_scratch_floats(int batch, int A) { return 2 + (size_t)((batch + 255) / 256) * A; }
 }  // namespace
 
 extern "C" int rlt_rocm_ppo_gae(rlt_rocm_device* device, const float* rewards, const float* terminated, const float* truncated, const float* all_values,
@@ -36,4 +131,77 @@ extern "C" int rlt_rocm_ppo_gae(rlt_rocm_device* device, const float* rewards, c
     hipLaunchKernelGGL(gae_kernel, dim3(blocks), dim3(64), 0, device->stream, rewards, terminated, truncated, all_values, advantages, target_values, ld, n_envs, steps,
                        gamma, lambda, ignore_termination);
     return rlt_launch_status(device);
+}
+
+extern "C" size_t rlt_rocm_ppo_workspace_bytes(const rlt_ppo_agent* A) {
+    if (!ppo_agent_ok(A)) return 0;
+    const size_t B = (size_t)A->batch;
+    size_t floats = B * (A->observation_dim + A->observation_privileged_dim + 2 * A->action_dim + 4) + ppo_surrogate_scratch_floats(A->batch, A->action_dim) + 64;
+    const size_t mlp_a = rlt_rocm_mlp_workspace_bytes(A->actor, A->n_actor_layers, A->batch), mlp_c = rlt_rocm_mlp_workspace_bytes(A->critic, A->n_critic_layers, A->batch);
+    return align256(floats * sizeof(float)) + align256(mlp_a > mlp_c ? mlp_a : mlp_c) + 256;
+}
+
+static int ppo_surrogate_impl(rlt_rocm_device* device, const float* means, int ld_means, const float* log_std, const float* actions, int ld_actions, const float* log_probs,
+                              int ld_lp, const float* advantages, int ld_adv, const rlt_ppo_parameters* P, float* d_means, int ld_d, float* d_log_std, int batch, int A,
+                              float* scratch) {
+    float* stats = scratch; float* partial = scratch + 2;
+    const int blocks = (batch + 255) / 256;
+    hipLaunchKernelGGL(ppo_advantage_stats_kernel, dim3(1), dim3(1024), 0, device->stream, advantages, ld_adv, batch, P->normalize_advantage, stats);
+    int rc = rlt_launch_status(device);
+    if (rc) return rc;
+    hipLaunchKernelGGL(ppo_surrogate_kernel, dim3(blocks), dim3(256), 0, device->stream, means, ld_means, log_std, actions, ld_actions, log_probs, ld_lp, advantages, ld_adv, *P,
+                       stats, d_means, ld_d, partial, batch, A);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if (P->learn_action_std) {
+        hipLaunchKernelGGL(ppo_log_std_gradient_kernel, dim3(1), dim3(64), 0, device->stream, partial, blocks, A, P->action_entropy_coefficient, d_log_std);
+        rc = rlt_launch_status(device);
+    }
+    return rc;
+}
+
+extern "C" int rlt_rocm_ppo_surrogate_gradient(rlt_rocm_device* device, const float* action_means, int ld_means, const float* log_std, const float* actions, int ld_actions,
+                                               const float* action_log_probs, int ld_log_probs, const float* advantages, int ld_advantages, const rlt_ppo_parameters* P,
+                                               float* d_action_means, int ld_d, float* d_log_std, int batch, int action_dim) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(action_means && log_std && actions && action_log_probs && advantages && P && d_action_means && batch > 0 && action_dim > 0 && action_dim <= PPO_MAX_ACTION_DIM);
+    RLT_REQUIRE(ld_means >= action_dim && ld_actions >= action_dim && ld_d >= action_dim && ld_log_probs >= 1 && ld_advantages >= 1 && (!P->learn_action_std || d_log_std));
+    void* scratch = nullptr;
+    int rc = rlt_scratch(device, ppo_surrogate_scratch_floats(batch, action_dim) * sizeof(float), &scratch);
+    if (rc) return rc;
+    return ppo_surrogate_impl(device, action_means, ld_means, log_std, actions, ld_actions, action_log_probs, ld_log_probs, advantages, ld_advantages, P, d_action_means, ld_d,
+                              d_log_std, batch, action_dim, (float*)scratch);
+}
+
+extern "C" int rlt_rocm_ppo_train_minibatch(rlt_rocm_device* device, const rlt_ppo_agent* A, const rlt_ppo_parameters* P, const float* observations,
+                                            const float* observations_privileged, const float* actions, const float* action_log_probs, const float* advantages,
+                                            const float* target_values, int ld, const uint32_t* row_indices, float* out_critic_loss) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(ppo_agent_ok(A) && P && observations && observations_privileged && actions && action_log_probs && advantages && target_values && ld >= 1);
+    RLT_REQUIRE(!P->learn_action_std || A->d_log_std);
+    RLT_REQUIRE(A->workspace && A->workspace_bytes >= rlt_rocm_ppo_workspace_bytes(A));
+    const int B = A->batch, O = A->observation_dim, OP = A->observation_privileged_dim, AD = A->action_dim;
+    // carve the workspace: packed minibatch, gradient at the actor output, critic output, surrogate scratch, then the networks' own workspace
+    float* w = (float*)A->workspace;
+    float* obs = w; w += (size_t)B * O; float* obsp = w; w += (size_t)B * OP; float* act = w; w += (size_t)B * AD; float* d_act = w; w += (size_t)B * AD;
+    float* lp = w; w += B; float* adv = w; w += B; float* tgt = w; w += B; float* values = w; w += B;
+    float* scratch = w; w += ppo_surrogate_scratch_floats(B, AD);
+    char* mlp_ws = (char*)A->workspace + align256((size_t)((char*)w - (char*)A->workspace) + 64 * sizeof(float));
+    const size_t mlp_ws_bytes = A->workspace_bytes - (size_t)(mlp_ws - (char*)A->workspace);
+    int blocks = (B * 16 + 255) / 256; if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(ppo_gather_kernel, dim3(blocks), dim3(256), 0, device->stream, observations, observations_privileged, actions, action_log_probs, advantages, target_values,
+                       ld, row_indices, B, O, OP, AD, obs, obsp, act, lp, adv, tgt);
+    int rc = rlt_launch_status(device);
+    if (rc) return rc;
+    if ((rc = rlt_rocm_mlp_zero_gradient(device, A->critic, A->n_critic_layers))) return rc;                      // :158
+    if ((rc = rlt_rocm_mlp_zero_gradient(device, A->actor, A->n_actor_layers))) return rc;                        // :159 (clears the log_std gradient too)
+    if (A->d_log_std) if ((rc = rlt_rocm_fill_f32(device, A->d_log_std, 1, AD, AD, 0.0f))) return rc;
+    if ((rc = rlt_rocm_mlp_forward(device, A->actor, A->n_actor_layers, obs, O, B))) return rc;                    // :203
+    const float* means = A->actor[A->n_actor_layers - 1].output;
+    if ((rc = ppo_surrogate_impl(device, means, AD, A->log_std, act, AD, lp, 1, adv, 1, P, d_act, AD, A->d_log_std, B, AD, scratch))) return rc;
+    if ((rc = rlt_rocm_mlp_backward(device, A->actor, A->n_actor_layers, obs, O, d_act, AD, nullptr, 0, B, 1, mlp_ws, mlp_ws_bytes))) return rc;   // :285
+    // critic: forward, MSE gradient with loss weight 0.5 (= (v - target)/batch), backward in one pass (:289-300)
+    if ((rc = rlt_rocm_mlp_forward_backward(device, A->critic, A->n_critic_layers, obsp, OP, values, 1, nullptr, 0, tgt, 1, 1.0f / (float)B, B, mlp_ws, mlp_ws_bytes))) return rc;
+    if (out_critic_loss) if ((rc = rlt_rocm_mse_evaluate(device, values, 1, tgt, 1, B, 1, 1.0f, out_critic_loss))) return rc;                      // :303
+    if ((rc = rlt_rocm_adam_step(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, 0.0f, nullptr))) return rc;  // :305
+    return rlt_rocm_adam_step(device, A->critic_adam_tensors, A->n_critic_adam_tensors, &A->critic_adam, A->critic_age, 0.0f, nullptr);             // :306
 }

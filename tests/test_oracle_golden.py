@@ -51,3 +51,31 @@ def test_seeded_loop_reproduces_reference_vectors(oracle, batch, checkpoints):
             assert np.array_equal(np_from(A.next_final_step_mask, (batch,), np.uint8), GOLD[key + "_next_final_step_mask_base"][batch:])
             assert np.all(GOLD[key + "_next_final_step_mask_base"][:batch] == 0) and np.all(GOLD[key + "_next_reset_base"] == 1)
     lib.rlt_oracle_sac_loop_destroy(loop)
+
+
+def ppo_golden_setup(backend):
+    """Agent, parameters and per-loop-step records from tests/golden/ppo_pendulum_seed0.npz (written by the real reference)."""
+    capi = helpers.capi
+    g = np.load(os.path.join(helpers.GOLDEN, "ppo_pendulum_seed0.npz"))
+    n_envs, steps, data_dim, rows, obs_dim, action_dim, batch, epochs, actor_hidden, critic_hidden = [int(x) for x in g["dims"]]
+    hy = dict(zip([str(k) for k in g["hyper_names"]], [float(v) for v in g["hyper"]]))
+    col = dict(zip(helpers.PPO_COLUMNS, [int(c) for c in g["columns"]]))
+    adam = capi.adam_parameters(hy["alpha"], hy["beta_1"], hy["beta_2"], hy["epsilon"], hy["epsilon_sqrt"])
+    pp = capi.ppo_parameters(hy["epsilon_clip"], hy["action_entropy_coefficient"], hy["advantage_epsilon"], int(hy["normalize_advantage"]), int(hy["learn_action_std"]))
+    agent = helpers.PpoOnBackend(backend, obs_dim, action_dim, actor_hidden, critic_hidden, batch, g["s0_before"], "tanh", "relu", adam)
+    return g, agent, pp, hy, col, dict(n_envs=n_envs, steps=steps, data_dim=data_dim, rows=rows, batch=batch, n=n_envs * steps)
+
+
+def test_ppo_gae_and_update_reproduce_reference_vectors(oracle):
+    """GAE and two loop steps' worth of PPO updates (30 minibatch updates) against what the reference itself produced: bit-exact."""
+    g, agent, pp, hy, col, d = ppo_golden_setup(oracle)
+    for step in range(2):
+        data = g[f"s{step}_dataset"]
+        dd = oracle.array(data)
+        adv, tgt = oracle.zeros(data.shape), oracle.zeros(data.shape)
+        oracle.call("ppo_gae", dd.offset(col["rewards"]), dd.offset(col["terminated"]), dd.offset(col["truncated"]), dd.offset(col["all_values"]), adv.ptr, tgt.ptr,
+                    d["data_dim"], d["n_envs"], d["steps"], hy["gamma"], hy["lambda"], 0)
+        assert np.array_equal(adv.numpy()[:d["n"], 0], data[:d["n"], col["advantages"]]) and np.array_equal(tgt.numpy()[:d["n"], 0], data[:d["n"], col["target_values"]])
+        assert np.array_equal(agent.parameters(), g[f"s{step}_before"])
+        helpers.ppo_train_like_reference(oracle, agent, pp, dd, d["data_dim"], col, d["n"], g[f"s{step}_permutations"], d["batch"])
+        assert np.array_equal(agent.parameters(), g[f"s{step}_after"]), step
