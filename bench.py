@@ -94,6 +94,47 @@ def bench_mlp(helpers, rocm, batch, iters, warmup):
     return out
 
 
+def bench_env(helpers, rocm, n_envs=65536, capacity=16, steps=200, batch=4096):
+    """Environment-step pipeline: Pendulum step of every environment with a deterministic 3-64-64-1 actor + replay add, then a gather."""
+    capi = helpers.capi
+    rng = np.random.default_rng(1)
+    dims = [3, 64, 64, 1]
+    actor = helpers.Mlp(rocm, dims, helpers.xavier_params(rng, dims), n_envs, "relu", "tanh", trainable=False)
+    rb = helpers.ReplayOnBackend(rocm, n_envs, capacity)
+    states, ep_step, ep_ret = rocm.zeros((n_envs, 2)), rocm.zeros((n_envs,), np.uint32), rocm.zeros((n_envs,))
+    trunc = rocm.array(np.ones(n_envs, np.uint8))
+    ini = rocm.array(np.stack([rng.uniform(-np.pi, np.pi, n_envs), rng.uniform(-1, 1, n_envs)], 1).astype(np.float32))
+    runner = capi.PendulumRunner(states.ptr, ep_step.ptr, ep_ret.ptr, trunc.ptr, n_envs, 200, capi.pendulum_parameters())
+    ev = HipEvents(rocm.device.lib.rlt_rocm_get_stream(rocm.device.handle))
+
+    def step():
+        rocm.call("pendulum_runner_step", C.byref(runner), C.byref(rb.c), 1, actor.layers, actor.n, None, None, None, ini.ptr, 0, 0)
+    for _ in range(5):
+        step()
+    rocm.sync()
+    a = ev.record()
+    for _ in range(steps):
+        step()
+    e = ev.record()
+    ms = ev.elapsed_ms(a, e)
+    envs = rocm.array(rng.integers(0, n_envs, batch).astype(np.uint32)); offs = rocm.array(rng.integers(0, capacity, batch).astype(np.uint32))
+    oab, rew, term = rocm.zeros((2, batch, 4)), rocm.zeros((batch,)), rocm.zeros((batch,), np.uint8)
+
+    def gather():
+        rocm.call("gather_batch", C.byref(rb.c), envs.ptr, offs.ptr, 0, 200, batch, oab.ptr, rew.ptr, term.ptr, None, None, None, None)
+    for _ in range(5):
+        gather()
+    rocm.sync()
+    a = ev.record()
+    for _ in range(100):
+        gather()
+    e = ev.record()
+    gather_us = ev.elapsed_ms(a, e) * 10.0
+    env_steps = n_envs * steps
+    return {"n_envs": n_envs, "replay_rows": n_envs * capacity, "steps": steps, "us_per_step": ms * 1e3 / steps, "env_steps_per_s": env_steps / (ms * 1e-3),
+            "algorithmic_GBps": env_steps * 68 / (ms * 1e-3) / 1e9, "gather_batch": batch, "gather_us": gather_us, "gather_algorithmic_GBps": batch * 85 / (gather_us * 1e-6) / 1e9}
+
+
 def pmc_probe(helpers, rocm, batch):
     n = 64 * 1024 * 1024      # floats: 256 MiB read + 256 MiB written per copy
     src, dst = rocm.zeros((n,)), rocm.zeros((n,))
@@ -235,7 +276,7 @@ def main():
     ap.add_argument("--mlp-batch", type=int, default=65536)
     ap.add_argument("--mlp-iters", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "mlp", "sac"], default="all")
+    ap.add_argument("--only", choices=["all", "mlp", "sac", "env"], default="all")
     ap.add_argument("--sac-phase-profile", action="store_true", help="print the persistent kernel's per-phase time (stderr)")
     ap.add_argument("--pmc-probe", action="store_true", help="for counter runs under rocprofv3 --pmc: three 256 MiB device copies (a kernel of known traffic, to scale the counters by) "
                     "and three MLP forward+backward calls, nothing timed")
@@ -255,7 +296,8 @@ def main():
         return
     mlp = bench_mlp(helpers, rocm, args.mlp_batch, args.mlp_iters, 3) if args.only in ("all", "mlp") else None
     sac = bench_sac(helpers, rocm, args.steps, args.warmup, per_operation=args.sac_per_operation, phase_profile=args.sac_phase_profile) if args.only in ("all", "sac") else {"steps_per_s": 0.0, "ms_per_step": 0.0}
-    cpu = None if (args.no_cpu_baseline or args.only == "mlp") else cpu_baseline()
+    env = bench_env(helpers, rocm) if args.only in ("all", "env") else None
+    cpu = None if (args.no_cpu_baseline or args.only in ("mlp", "env")) else cpu_baseline()
     line = {
         "metric": "SAC updates/sec (critic+actor) at batch 256; fused MLP fwd+bwd TFLOP/s",
         "value": sac["steps_per_s"], "unit": "SAC loop steps/s (each = 2 critic + 1 actor update)",
@@ -272,6 +314,8 @@ def main():
         line["roofline"] = {"bound": "mfma", "achieved": mlp["tflops"], "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": mlp["tflops"] / FP32_PEAK_TFLOPS,
                             "traffic": MLP_CALL_HBM_BYTES if mlp["batch"] == 65536 else None, "traffic_unit": "bytes per call, from rocprofv3 FETCH_SIZE / WRITE_SIZE",
                             "kernel": "mlp_forward_backward call = mlp3_prepare_kernel + mlp3_fused_kernel + mlp3_reduce_kernel", "flop_per_launch": flop}
+    if env:
+        line["env_pipeline"] = env
     if cpu:
         line["cpu_baseline"] = cpu
         line["speedup_vs_cpu_baseline"] = sac["steps_per_s"] / cpu["value"] if cpu["value"] else None
