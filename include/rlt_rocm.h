@@ -473,6 +473,37 @@ int rlt_rocm_ppo_train_minibatch(rlt_rocm_device* device, const rlt_ppo_agent* a
                                  const float* action_log_probs, const float* advantages, const float* target_values, int ld,
                                  const uint32_t* row_indices, float* out_critic_loss);
 
+/* --------------------------------------------------------------------- GRU -- */
+
+/* nn/layers/gru/layer.h:96-217 (LayerForward / LayerBackward / LayerGradient): gate order r, z, n along the 3H rows
+ * (the layout of torch.nn.GRU); LEARN_INITIAL_HIDDEN_STATE = false and FAST_TANH = false as in the reference's
+ * configuration default (layer.h:14-24). Tensors are [sequence x batch x features], row-major. */
+typedef struct rlt_gru_layer {
+    float* weights_input;          /* [3H x I] */
+    float* biases_input;           /* [3H] */
+    float* weights_hidden;         /* [3H x H] */
+    float* biases_hidden;          /* [3H] */
+    float* initial_hidden_state;   /* [H] */
+    float* d_weights_input; float* d_biases_input; float* d_weights_hidden; float* d_biases_hidden;   /* gradients, accumulated */
+    float* post_activation;        /* [S x B x 3H] r and z after the sigmoid, n after tanh (kept by forward for backward) */
+    float* n_pre_pre_activation;   /* [S x B x H]  W_hn h + b_hn */
+    float* output;                 /* [S x B x H]  hidden state of every step */
+    int input_dim, hidden_dim;
+} rlt_gru_layer;
+
+size_t rlt_rocm_gru_workspace_bytes(const rlt_gru_layer* layer, int sequence_length, int batch);
+/* forward (keeps the intermediates)   nn/layers/gru/operations_generic.h:231-341,418-421
+ *   reset [S x B] (optional): a sample whose flag is set at step t starts that step from initial_hidden_state, as do all
+ *   samples at step 0 (ResetMode, layer.h:56-68). */
+int rlt_rocm_gru_forward(rlt_rocm_device* device, const rlt_gru_layer* layer, const float* input, const uint8_t* reset,
+                         int sequence_length, int batch, void* workspace, size_t workspace_bytes);
+/* backward / backward_full / backward_input through time   nn/layers/gru/operations_generic.h:594-795
+ *   d_output [S x B x H] is modified (the gradient flowing back through the hidden state is accumulated into it, as in
+ *   the reference); d_input [S x B x I] may be NULL; want_weight_gradients = 0 -> backward_input. */
+int rlt_rocm_gru_backward(rlt_rocm_device* device, const rlt_gru_layer* layer, const float* input, float* d_output,
+                          float* d_input, const uint8_t* reset, int sequence_length, int batch, int want_weight_gradients,
+                          void* workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -883,4 +883,130 @@ int rlt_oracle_ppo_shuffle(char* rng_state, int rng_state_capacity, int n, int e
     return 0;
 }
 
+// nn/layers/gru/operations_generic.h:231-341 (evaluate with multi-step intermediates = forward), loop order as there
+int rlt_oracle_gru_forward(const rlt_gru_layer* L, const float* input, const uint8_t* reset, int S, int B) {
+    if (!L || !input || S <= 0 || B <= 0 || !L->weights_input || !L->biases_input || !L->weights_hidden || !L->biases_hidden || !L->initial_hidden_state ||
+        !L->post_activation || !L->n_pre_pre_activation || !L->output) return RLT_E_INVALID_ARGUMENT;
+    const int I = L->input_dim, H = L->hidden_dim, H3 = 3 * H;
+    std::vector<float> hprev((size_t)B * H);
+    for (int t = 0; t < S; t++) {
+        float* post = L->post_activation + (size_t)t * B * H3;
+        float* npp = L->n_pre_pre_activation + (size_t)t * B * H;
+        float* out = L->output + (size_t)t * B * H;
+        const float* x = input + (size_t)t * B * I;
+        for (int b = 0; b < B; b++) {
+            const bool from_initial = t == 0 || (reset && reset[(size_t)t * B + b]);
+            const float* src = from_initial ? L->initial_hidden_state : L->output + ((size_t)(t - 1) * B + b) * H;
+            std::memcpy(&hprev[(size_t)b * H], src, sizeof(float) * H);
+        }
+        for (int b = 0; b < B; b++)                                       // W_h h + b_h (:262-288)
+            for (int j = 0; j < H3; j++) {
+                float acc = L->biases_hidden[j];
+                for (int k = 0; k < H; k++) acc += hprev[(size_t)b * H + k] * L->weights_hidden[(size_t)j * H + k];
+                post[(size_t)b * H3 + j] = acc;
+            }
+        for (int b = 0; b < B; b++)                                       // :290-291
+            for (int j = 0; j < H; j++) { npp[(size_t)b * H + j] = post[(size_t)b * H3 + 2 * H + j]; post[(size_t)b * H3 + 2 * H + j] = 0; }
+        for (int b = 0; b < B; b++)                                       // += W_i x + b_i (:293)
+            for (int j = 0; j < H3; j++) {
+                float acc = post[(size_t)b * H3 + j] + L->biases_input[j];
+                for (int k = 0; k < I; k++) acc += x[(size_t)b * I + k] * L->weights_input[(size_t)j * I + k];
+                post[(size_t)b * H3 + j] = acc;
+            }
+        for (int b = 0; b < B; b++) {
+            float* p = post + (size_t)b * H3;
+            for (int j = 0; j < 2 * H; j++) p[j] = 1 / (1 + std::exp(-p[j]));                         // sigmoid (:301)
+            for (int j = 0; j < H; j++) p[2 * H + j] += npp[(size_t)b * H + j] * p[j];                 // :303
+            for (int j = 0; j < H; j++) p[2 * H + j] = std::tanh(p[2 * H + j]);                        // :311
+            for (int j = 0; j < H; j++) {
+                float o = 1 - p[H + j];                                                                 // one_minus (:313)
+                o = o * p[2 * H + j];                                                                   // multiply (:314)
+                o += p[H + j] * hprev[(size_t)b * H + j];                                               // multiply_accumulate (:315-330)
+                out[(size_t)b * H + j] = o;
+            }
+        }
+    }
+    return 0;
+}
+
+// nn/layers/gru/operations_generic.h:594-760, step by step from the last to the first
+int rlt_oracle_gru_backward(const rlt_gru_layer* L, const float* input, float* d_output, float* d_input, const uint8_t* reset, int S, int B, int want_w) {
+    if (!L || !d_output || S <= 0 || B <= 0 || (!input && want_w)) return RLT_E_INVALID_ARGUMENT;
+    if (want_w && (!L->d_weights_input || !L->d_biases_input || !L->d_weights_hidden || !L->d_biases_hidden)) return RLT_E_INVALID_ARGUMENT;
+    const int I = L->input_dim, H = L->hidden_dim, H3 = 3 * H;
+    std::vector<float> hprev((size_t)B * H), buf((size_t)B * H3);
+    for (int t = S - 1; t >= 0; t--) {
+        const float* post = L->post_activation + (size_t)t * B * H3;
+        const float* npp = L->n_pre_pre_activation + (size_t)t * B * H;
+        float* dout = d_output + (size_t)t * B * H;
+        float* dprev = t > 0 ? d_output + (size_t)(t - 1) * B * H : nullptr;
+        for (int b = 0; b < B; b++) {
+            const bool from_initial = t == 0 || (reset && reset[(size_t)t * B + b]);
+            const float* src = from_initial ? L->initial_hidden_state : L->output + ((size_t)(t - 1) * B + b) * H;
+            std::memcpy(&hprev[(size_t)b * H], src, sizeof(float) * H);
+            const float* p = post + (size_t)b * H3;
+            float* bb = &buf[(size_t)b * H3];
+            for (int j = 0; j < H; j++) {
+                const float dh = dout[(size_t)b * H + j];
+                if (!from_initial) dprev[(size_t)b * H + j] += dh * p[H + j];                            // :643-659
+                bb[H + j] = dh * (hprev[(size_t)b * H + j] - p[2 * H + j]);                              // buffer_z (:624,660)
+                bb[2 * H + j] = dh * (1 - p[H + j]) * (1 - p[2 * H + j] * p[2 * H + j]);                  // buffer_n (:668)
+                bb[j] = bb[2 * H + j] * npp[(size_t)b * H + j];                                         // buffer_r (:669)
+            }
+            for (int j = 0; j < 2 * H; j++) bb[j] = bb[j] * p[j] * (1 - p[j]);                           // :670
+        }
+        if (want_w) {
+            const float* x = input + (size_t)t * B * I;
+            for (int j = 0; j < H3; j++)                                                                 // :677
+                for (int k = 0; k < I; k++) {
+                    float acc = L->d_weights_input[(size_t)j * I + k];
+                    for (int b = 0; b < B; b++) acc += buf[(size_t)b * H3 + j] * x[(size_t)b * I + k];
+                    L->d_weights_input[(size_t)j * I + k] = acc;
+                }
+            for (int j = 0; j < H3; j++) {                                                               // reduce_sum<true> (:678): sum first, then add
+                float acc = 0;
+                for (int b = 0; b < B; b++) acc += buf[(size_t)b * H3 + j];
+                L->d_biases_input[j] = acc + L->d_biases_input[j];
+            }
+            for (int j = 0; j < 2 * H; j++) L->d_biases_hidden[j] = L->d_biases_input[j];                 // :679-681
+        }
+        if (d_input) {                                                                                   // :688
+            float* dx = d_input + (size_t)t * B * I;
+            for (int b = 0; b < B; b++)
+                for (int k = 0; k < I; k++) {
+                    float acc = 0;
+                    for (int j = 0; j < H3; j++) acc += buf[(size_t)b * H3 + j] * L->weights_input[(size_t)j * I + k];
+                    dx[(size_t)b * I + k] = acc;
+                }
+        }
+        for (int b = 0; b < B; b++) for (int j = 0; j < H; j++) buf[(size_t)b * H3 + 2 * H + j] *= post[(size_t)b * H3 + j];   // :691
+        if (want_w) {                                                                                    // :693-742
+            for (int j = 0; j < H3; j++)
+                for (int k = 0; k < H; k++) {
+                    float acc = L->d_weights_hidden[(size_t)j * H + k];
+                    for (int b = 0; b < B; b++) acc += buf[(size_t)b * H3 + j] * hprev[(size_t)b * H + k];
+                    L->d_weights_hidden[(size_t)j * H + k] = acc;
+                }
+        }
+        if (t > 0)
+            for (int b = 0; b < B; b++) {
+                if (reset && reset[(size_t)t * B + b]) continue;                                         // rows of reset samples are zeroed (:716-722)
+                for (int k = 0; k < H; k++) {
+                    float acc = dprev[(size_t)b * H + k];
+                    for (int j = 0; j < H3; j++) acc += buf[(size_t)b * H3 + j] * L->weights_hidden[(size_t)j * H + k];
+                    dprev[(size_t)b * H + k] = acc;
+                }
+            }
+        if (want_w)                                                                                      // :745-749
+            for (int j = 0; j < H; j++) {
+                // the reference has zeroed the buffer rows of samples that were reset at this step (t > 0) by now (:716-722), so they do not
+                // contribute to the b_hn gradient (they do contribute to everything above)
+                float acc = 0;
+                for (int b = 0; b < B; b++) acc += (t > 0 && reset && reset[(size_t)t * B + b]) ? 0.0f : buf[(size_t)b * H3 + 2 * H + j];
+                L->d_biases_hidden[2 * H + j] = acc + L->d_biases_hidden[2 * H + j];
+            }
+    }
+    return 0;
+}
+
 }  // extern "C"

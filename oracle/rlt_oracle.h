@@ -99,6 +99,9 @@ int rlt_oracle_ppo_surrogate_gradient(const float* action_means, int ld_means, c
 int rlt_oracle_ppo_train_minibatch(const rlt_ppo_agent* agent, const rlt_ppo_parameters* parameters, const float* observations,
                                    const float* observations_privileged, const float* actions, const float* action_log_probs,
                                    const float* advantages, const float* target_values, int ld, const uint32_t* row_indices, float* out_critic_loss);
+int rlt_oracle_gru_forward(const rlt_gru_layer* layer, const float* input, const uint8_t* reset, int sequence_length, int batch);
+int rlt_oracle_gru_backward(const rlt_gru_layer* layer, const float* input, float* d_output, float* d_input, const uint8_t* reset,
+                            int sequence_length, int batch, int want_weight_gradients);
 /* the reference's per-epoch in-place dataset shuffle as row permutations, driven by the text form of its std::mt19937 */
 int rlt_oracle_ppo_shuffle(char* rng_state, int rng_state_capacity, int n, int epochs, uint32_t* permutations);
 

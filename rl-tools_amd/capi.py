@@ -109,6 +109,13 @@ class PpoAgent(C.Structure):
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
 
 
+class GruLayer(C.Structure):
+    _fields_ = [("weights_input", C.c_void_p), ("biases_input", C.c_void_p), ("weights_hidden", C.c_void_p), ("biases_hidden", C.c_void_p),
+                ("initial_hidden_state", C.c_void_p), ("d_weights_input", C.c_void_p), ("d_biases_input", C.c_void_p), ("d_weights_hidden", C.c_void_p),
+                ("d_biases_hidden", C.c_void_p), ("post_activation", C.c_void_p), ("n_pre_pre_activation", C.c_void_p), ("output", C.c_void_p),
+                ("input_dim", C.c_int32), ("hidden_dim", C.c_int32)]
+
+
 I, F, P, S, U64 = C.c_int, C.c_float, C.c_void_p, C.c_size_t, C.c_uint64
 LP = C.POINTER(DenseLayer)
 
@@ -144,6 +151,8 @@ PROTOTYPES = {
     "gather_batch": [C.POINTER(ReplayBuffer), P, P, I, I, I, P, P, P, P, P, P, P],
     "pendulum_step": [C.POINTER(PendulumParameters), P, P, P, P, P, I],
     "ppo_gae": [P, P, P, P, P, P, I, I, I, F, F, I],
+    "gru_forward": [C.POINTER(GruLayer), P, P, I, I, P, S],
+    "gru_backward": [C.POINTER(GruLayer), P, P, P, P, I, I, I, P, S],
     "ppo_surrogate_gradient": [P, I, P, P, I, P, I, P, I, C.POINTER(PpoParameters), P, I, P, I, I],
     "ppo_train_minibatch": [C.POINTER(PpoAgent), C.POINTER(PpoParameters), P, P, P, P, P, P, I, P, P],
 }
@@ -159,6 +168,7 @@ ROCM_ONLY = {
     "reduce_sum_f32": ([P, P, S, I, P], I),
     "mlp_workspace_bytes": ([LP, I, I], S),
     "ppo_workspace_bytes": ([C.POINTER(PpoAgent)], S),
+    "gru_workspace_bytes": ([C.POINTER(GruLayer), I, I], S),
     "gather_draw": ([P, C.POINTER(ReplayBuffer), I, U64, U64, P, P], I),
     "sac_pendulum_loop": ([P, C.POINTER(SacAgent), C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, U64, U64, C.POINTER(SacLoopInputs),
                            C.POINTER(SacLoopOutputs)], I),

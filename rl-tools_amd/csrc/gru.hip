@@ -1,0 +1,180 @@
+// GRU layer: forward with kept intermediates and backward through time.
+// reference: nn/layers/gru/operations_generic.h:231-341 (evaluate / forward), :594-795 (_backward per step, from the last step to the
+// first). The reference walks the sequence on the host and issues a handful of small tensor operations per step.
+//
+// Here the work is split by what depends on time:
+//   * W_i x + b_i for ALL steps is one contraction over sequence*batch rows (gemm.hip), written straight into post_activation;
+//   * the recurrence runs in ONE launch: batch rows are independent, so a workgroup owns a few rows for the whole sequence, keeps W_h
+//     (48 KB at H = 64) and its rows' hidden state in LDS and loops over the steps without any grid-wide synchronisation;
+//   * backward does the same in reverse and stores, per step, the gradient at the gate pre-activations (one copy as the input path sees
+//     it, one as the hidden path sees it, which differs in the n gate by the factor r) and the previous hidden state; the weight
+//     gradients and d_input are then three contractions over sequence*batch rows.
+#include "common.h"
+#include "gemm.h"
+
+namespace {
+
+constexpr int GRU_THREADS = 256;
+
+struct GruArgs {
+    rlt_gru_layer L;
+    const float* input; const uint8_t* reset;
+    float* d_output; float* buffer_input; float* buffer_hidden; float* h_previous; float* db_hn_partial;
+    int S, B, rows_per_group;
+};
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// post_activation holds W_i x + b_i on entry. Thread (row, j): hidden unit j of one batch row.
+__global__ __launch_bounds__(GRU_THREADS) void gru_forward_kernel(GruArgs A) {
+    extern __shared__ float lds[];
+    const int H = A.L.hidden_dim, H3 = 3 * H, R = A.rows_per_group;
+    float* wt = lds;                 // W_h transposed: wt[k * 3H + j]
+    float* hs = wt + (size_t)H3 * H; // hidden state of the workgroup's rows
+    for (int i = threadIdx.x; i < H3 * H; i += blockDim.x) { const int j = i / H, k = i - j * H; wt[k * H3 + j] = A.L.weights_hidden[i]; }
+    const int row = threadIdx.x / H, j = threadIdx.x - row * H, b = blockIdx.x * R + row;
+    const bool active = row < R && b < A.B;
+    const float bhr = active ? A.L.biases_hidden[j] : 0.f, bhz = active ? A.L.biases_hidden[H + j] : 0.f, bhn = active ? A.L.biases_hidden[2 * H + j] : 0.f;
+    const float h0 = active ? A.L.initial_hidden_state[j] : 0.f;
+    float h = h0;
+    for (int t = 0; t < A.S; t++) {
+        if (active) {
+            if (t == 0 || (A.reset && A.reset[(size_t)t * A.B + b])) h = h0;
+            hs[row * H + j] = h;
+        }
+        __syncthreads();
+        if (active) {
+            float ar = bhr, az = bhz, an = bhn;
+            const float* hr = hs + row * H;
+            for (int k = 0; k < H; k++) { const float hk = hr[k]; const float* w = wt + k * H3; ar += hk * w[j]; az += hk * w[H + j]; an += hk * w[2 * H + j]; }
+            float* post = A.L.post_activation + ((size_t)t * A.B + b) * H3;
+            const float r = sigmoidf_(post[j] + ar), z = sigmoidf_(post[H + j] + az);
+            const float n = tanhf(post[2 * H + j] + an * r);
+            post[j] = r; post[H + j] = z; post[2 * H + j] = n;
+            A.L.n_pre_pre_activation[((size_t)t * A.B + b) * H + j] = an;
+            h = (1.0f - z) * n + z * h;
+            A.L.output[((size_t)t * A.B + b) * H + j] = h;
+        }
+        __syncthreads();
+    }
+}
+
+// Reverse pass. Thread (row, j). d_output is accumulated into in place as in the reference.
+__global__ __launch_bounds__(GRU_THREADS) void gru_backward_kernel(GruArgs A) {
+    extern __shared__ float lds[];
+    const int H = A.L.hidden_dim, H3 = 3 * H, R = A.rows_per_group;
+    float* w = lds;                          // W_h row-major: w[j * H + k]
+    float* bs = w + (size_t)H3 * H;          // hidden-path gate gradients of the workgroup's rows: bs[row * 3H + j]
+    for (int i = threadIdx.x; i < H3 * H; i += blockDim.x) w[i] = A.L.weights_hidden[i];
+    const int row = threadIdx.x / H, j = threadIdx.x - row * H, b = blockIdx.x * R + row;
+    const bool active = row < R && b < A.B;
+    const float h0 = active ? A.L.initial_hidden_state[j] : 0.f;
+    float carry = 0.f;       // gradient arriving at this step's hidden state from the step after it
+    float db_hn = 0.f;
+    __syncthreads();
+    for (int t = A.S - 1; t >= 0; t--) {
+        bool from_initial = true;
+        if (active) {
+            const size_t at = (size_t)t * A.B + b;
+            from_initial = t == 0 || (A.reset && A.reset[at]);
+            const float* post = A.L.post_activation + at * H3;
+            const float r = post[j], z = post[H + j], n = post[2 * H + j];
+            const float hp = from_initial ? h0 : A.L.output[((size_t)(t - 1) * A.B + b) * H + j];
+            const float dh = A.d_output[at * H + j] + carry;
+            A.d_output[at * H + j] = dh;
+            const float gz = dh * (hp - n) * z * (1.0f - z);
+            const float gn = dh * (1.0f - z) * (1.0f - n * n);
+            const float gr = gn * A.L.n_pre_pre_activation[at * H + j] * r * (1.0f - r);
+            float* bi = A.buffer_input + at * H3; float* bh = A.buffer_hidden + at * H3;
+            bi[j] = gr; bi[H + j] = gz; bi[2 * H + j] = gn;
+            bh[j] = gr; bh[H + j] = gz; bh[2 * H + j] = gn * r;
+            A.h_previous[at * H + j] = hp;
+            bs[row * H3 + j] = gr; bs[row * H3 + H + j] = gz; bs[row * H3 + 2 * H + j] = gn * r;
+            // the reference drops reset samples (t > 0) from the b_hn gradient (their buffer rows are zeroed before that sum, :716-749)
+            if (!(t > 0 && from_initial)) db_hn += gn * r;
+            carry = from_initial ? 0.f : dh * z;
+        }
+        __syncthreads();
+        if (active && !from_initial) {
+            float acc = 0.f;
+            const float* br = bs + row * H3;
+            for (int jj = 0; jj < H3; jj++) acc += br[jj] * w[jj * H + j];       // d h_prev[j] += sum over gates of buffer * W_h[., j]
+            carry += acc;
+        }
+        __syncthreads();
+    }
+    if (active && A.db_hn_partial) A.db_hn_partial[(size_t)b * H + j] = db_hn;
+}
+
+// db_h[n part] += sum over batch rows of the per-row sums (row order), db_h[r, z parts] = db_i[r, z parts] (the reference copies, :679-681)
+__global__ void gru_bias_hidden_kernel(const float* __restrict__ partial, int B, int H, const float* __restrict__ db_i, float* __restrict__ db_h) {
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j < 2 * H) db_h[j] = db_i[j];
+    else if (j < 3 * H) { float s = 0.f; for (int b = 0; b < B; b++) s += partial[(size_t)b * H + (j - 2 * H)]; db_h[j] += s; }
+}
+
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+bool layer_ok(const rlt_gru_layer* L) {
+    return L && L->weights_input && L->biases_input && L->weights_hidden && L->biases_hidden && L->initial_hidden_state && L->post_activation &&
+           L->n_pre_pre_activation && L->output && L->input_dim >= 1 && L->hidden_dim >= 1 && L->hidden_dim <= GRU_THREADS;
+}
+int rows_per_group(int H) { return GRU_THREADS / H; }
+size_t lds_bytes(int H, bool backward) { return ((size_t)3 * H * H + (size_t)rows_per_group(H) * (backward ? 3 * H : H)) * sizeof(float); }
+
+}  // namespace
+
+extern "C" {
+
+size_t rlt_rocm_gru_workspace_bytes(const rlt_gru_layer* L, int S, int B) {
+    if (!L || S < 1 || B < 1 || L->hidden_dim < 1) return 0;
+    const size_t rows = (size_t)S * B, H = (size_t)L->hidden_dim;
+    return align256(rows * 3 * H * sizeof(float)) * 2 + align256(rows * H * sizeof(float)) + align256((size_t)B * H * sizeof(float)) + 256;
+}
+
+int rlt_rocm_gru_forward(rlt_rocm_device* device, const rlt_gru_layer* L, const float* input, const uint8_t* reset, int S, int B, void* workspace, size_t workspace_bytes) {
+    (void)workspace; (void)workspace_bytes;
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(layer_ok(L) && input && S > 0 && B > 0);
+    const int H = L->hidden_dim;
+    if (lds_bytes(H, false) > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
+    // W_i x + b_i for every step at once, into post_activation
+    int rc = rlt_gemm_forward(device, input, L->input_dim, L->weights_input, L->biases_input, RLT_ACT_IDENTITY, nullptr, nullptr, L->post_activation, 3 * H, S * B, L->input_dim, 3 * H);
+    if (rc) return rc;
+    GruArgs a = {}; a.L = *L; a.input = input; a.reset = reset; a.S = S; a.B = B; a.rows_per_group = rows_per_group(H);
+    const size_t lds = lds_bytes(H, false);
+    RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gru_forward_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(gru_forward_kernel, dim3(rlt_div_up(B, a.rows_per_group)), dim3(GRU_THREADS), lds, device->stream, a);
+    return rlt_launch_status(device);
+}
+
+int rlt_rocm_gru_backward(rlt_rocm_device* device, const rlt_gru_layer* L, const float* input, float* d_output, float* d_input, const uint8_t* reset, int S, int B,
+                          int want_weight_gradients, void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(layer_ok(L) && d_output && S > 0 && B > 0 && (input || !want_weight_gradients));
+    RLT_REQUIRE(!want_weight_gradients || (L->d_weights_input && L->d_biases_input && L->d_weights_hidden && L->d_biases_hidden));
+    RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_gru_workspace_bytes(L, S, B));
+    const int H = L->hidden_dim, I = L->input_dim, rows = S * B;
+    if (lds_bytes(H, true) > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
+    char* w = reinterpret_cast<char*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    float* buffer_input = (float*)w; w += align256((size_t)rows * 3 * H * sizeof(float));
+    float* buffer_hidden = (float*)w; w += align256((size_t)rows * 3 * H * sizeof(float));
+    float* h_previous = (float*)w; w += align256((size_t)rows * H * sizeof(float));
+    float* db_hn_partial = (float*)w;
+    GruArgs a = {}; a.L = *L; a.input = input; a.reset = reset; a.d_output = d_output; a.buffer_input = buffer_input; a.buffer_hidden = buffer_hidden;
+    a.h_previous = h_previous; a.db_hn_partial = want_weight_gradients ? db_hn_partial : nullptr; a.S = S; a.B = B; a.rows_per_group = rows_per_group(H);
+    const size_t lds = lds_bytes(H, true);
+    RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gru_backward_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(gru_backward_kernel, dim3(rlt_div_up(B, a.rows_per_group)), dim3(GRU_THREADS), lds, device->stream, a);
+    int rc = rlt_launch_status(device);
+    if (rc) return rc;
+    if (want_weight_gradients) {
+        if ((rc = rlt_gemm_wgrad(device, buffer_input, 3 * H, input, I, L->d_weights_input, L->d_biases_input, rows, I, 3 * H))) return rc;       // :677-678
+        if ((rc = rlt_gemm_wgrad(device, buffer_hidden, 3 * H, h_previous, H, L->d_weights_hidden, nullptr, rows, H, 3 * H))) return rc;         // :693-742
+        hipLaunchKernelGGL(gru_bias_hidden_kernel, dim3(rlt_div_up(3 * H, 128)), dim3(128), 0, device->stream, db_hn_partial, B, H, L->d_biases_input, L->d_biases_hidden);
+        if ((rc = rlt_launch_status(device))) return rc;
+    }
+    if (d_input) rc = rlt_gemm_backward_input(device, buffer_input, 3 * H, L->weights_input, d_input, I, nullptr, 0, 0, rows, I, 3 * H);           // :688
+    return rc;
+}
+
+}  // extern "C"

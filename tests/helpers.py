@@ -48,7 +48,7 @@ def load_oracle():
     P, S, I = C.c_void_p, C.c_size_t, C.c_int
     for name, args in capi.PROTOTYPES.items():
         a = list(args)
-        if name in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward"):
+        if name in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward"):
             a = a[:-2]      # the CPU checker allocates its own workspace
         fn = getattr(lib, "rlt_oracle_" + name)
         fn.argtypes = a
@@ -110,7 +110,7 @@ class HostBackend:
         return HostArray(np.zeros(shape, dtype))
 
     def call(self, fn, *args):
-        if fn in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward"):
+        if fn in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward"):
             args = args[:-2]
         rc = getattr(self.lib, "rlt_oracle_" + fn)(*args)
         if rc != 0:
@@ -216,6 +216,51 @@ class Mlp:
             return None, 0
         nbytes = self.backend.device.lib.rlt_rocm_mlp_workspace_bytes(self.layers, self.n, self.batch)
         return self.backend.workspace(nbytes)
+
+
+REF_GRU_GENERIC = os.path.join(ORACLE_DIR, "_ref", "librlt_ref_gru_generic.so")
+
+
+class GruOnBackend:
+    """One GRU layer (parameters, gradients, kept intermediates) on a backend. params: dict W_i [3H x I], b_i, W_h [3H x H], b_h, h0."""
+
+    def __init__(self, backend, S, B, I, H, params):
+        self.backend, self.S, self.B, self.I, self.H = backend, S, B, I, H
+        f = lambda k: backend.array(np.asarray(params[k], np.float32))
+        self.W_i, self.b_i, self.W_h, self.b_h, self.h0 = f("W_i"), f("b_i"), f("W_h"), f("b_h"), f("h0")
+        self.dW_i, self.db_i, self.dW_h, self.db_h = backend.zeros((3 * H, I)), backend.zeros((3 * H,)), backend.zeros((3 * H, H)), backend.zeros((3 * H,))
+        self.post, self.npp, self.out = backend.zeros((S, B, 3 * H)), backend.zeros((S, B, H)), backend.zeros((S, B, H))
+        self.c = capi.GruLayer(self.W_i.ptr, self.b_i.ptr, self.W_h.ptr, self.b_h.ptr, self.h0.ptr, self.dW_i.ptr, self.db_i.ptr, self.dW_h.ptr, self.db_h.ptr,
+                               self.post.ptr, self.npp.ptr, self.out.ptr, I, H)
+        self.ws, self.wsn = (None, 0)
+        if backend.name == "rocm":
+            n = backend.device.lib.rlt_rocm_gru_workspace_bytes(C.byref(self.c), S, B)
+            self._ws = backend.device.empty((max(int(n), 4),), np.uint8)
+            self.ws, self.wsn = self._ws.ptr, int(n)
+
+    def forward(self, x, reset=None):
+        self.x = self.backend.array(np.asarray(x, np.float32))
+        self.reset = self.backend.array(np.asarray(reset, np.uint8)) if reset is not None else None
+        self.backend.call("gru_forward", C.byref(self.c), self.x.ptr, self.reset.ptr if self.reset else None, self.S, self.B, self.ws, self.wsn)
+
+    def backward(self, d_output, want_d_input=True, want_w=1):
+        self.dy = self.backend.array(np.asarray(d_output, np.float32))
+        self.dx = self.backend.zeros((self.S, self.B, self.I))
+        self.backend.call("gru_backward", C.byref(self.c), self.x.ptr, self.dy.ptr, self.dx.ptr if want_d_input else None, self.reset.ptr if self.reset else None,
+                          self.S, self.B, want_w, self.ws, self.wsn)
+
+    def results(self):
+        return dict(output=self.out.numpy(), post=self.post.numpy(), npp=self.npp.numpy(), dx=self.dx.numpy(), dy=self.dy.numpy(), dW_i=self.dW_i.numpy(),
+                    db_i=self.db_i.numpy(), dW_h=self.dW_h.numpy(), db_h=self.db_h.numpy())
+
+
+def gru_random_case(rng, S, B, I, H, with_reset):
+    params = dict(W_i=rng.uniform(-0.4, 0.4, (3 * H, I)), b_i=rng.uniform(-0.4, 0.4, 3 * H), W_h=rng.uniform(-0.4, 0.4, (3 * H, H)), b_h=rng.uniform(-0.4, 0.4, 3 * H),
+                  h0=rng.uniform(-0.5, 0.5, H))
+    params = {k: v.astype(np.float32) for k, v in params.items()}
+    x = rng.standard_normal((S, B, I)).astype(np.float32); dy = rng.standard_normal((S, B, H)).astype(np.float32)
+    reset = (rng.random((S, B)) < 0.25).astype(np.uint8) if with_reset else None
+    return params, x, dy, reset
 
 
 class PpoOnBackend:

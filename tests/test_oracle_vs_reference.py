@@ -147,3 +147,31 @@ def test_ppo_gae_and_update_bit_exact_with_reference(oracle):
         assert np.array_equal(got, want), (loop_step, np.abs(got - want).max())
         assert ref.ages() == [int(agent.actor.age.numpy()[0]), int(agent.critic.age.numpy()[0])]
     ref.close()
+
+
+@pytest.mark.skipif(not os.path.exists(helpers.REF_GRU_GENERIC), reason="oracle/_ref GRU harness not built (needs /root/reference)")
+@pytest.mark.parametrize("with_reset", [False, True])
+def test_gru_forward_and_backward_through_time_bit_exact_with_reference(oracle, with_reset):
+    """The reference's own GRU layer (forward with kept intermediates, backward_full through 7 steps, optional per-sample resets) on random
+    weights and inputs: outputs, intermediates, d_input, the in-place accumulated d_output and all four gradients, bit for bit."""
+    ref = C.CDLL(helpers.REF_GRU_GENERIC)
+    dims = (C.c_int * 4)(); ref.rlt_ref_gru_dims(dims)
+    S, B, I, H = list(dims)
+    rng = np.random.default_rng(12 + with_reset)
+    params, x, dy, reset = helpers.gru_random_case(rng, S, B, I, H, with_reset)
+    want = dict(output=np.zeros((S, B, H), np.float32), post=np.zeros((S, B, 3 * H), np.float32), npp=np.zeros((S, B, H), np.float32), dx=np.zeros((S, B, I), np.float32),
+                dW_i=np.zeros((3 * H, I), np.float32), db_i=np.zeros(3 * H, np.float32), dW_h=np.zeros((3 * H, H), np.float32), db_h=np.zeros(3 * H, np.float32),
+                dy=np.zeros((S, B, H), np.float32))
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    ref.rlt_ref_gru_forward_backward.argtypes = [C.c_void_p] * 17
+    assert ref.rlt_ref_gru_forward_backward(p(params["W_i"]), p(params["b_i"]), p(params["W_h"]), p(params["b_h"]), p(params["h0"]), p(x), p(reset) if with_reset else None,
+                                            p(dy), p(want["output"]), p(want["post"]), p(want["npp"]), p(want["dx"]), p(want["dW_i"]), p(want["db_i"]), p(want["dW_h"]),
+                                            p(want["db_h"]), p(want["dy"])) == 0
+    g = helpers.GruOnBackend(oracle, S, B, I, H, params)
+    g.forward(x, reset)
+    g.backward(dy)
+    got = g.results()
+    if with_reset:
+        assert reset[1:].sum() > 3
+    for k in want:
+        assert np.array_equal(got[k], want[k]), (k, np.abs(got[k] - want[k]).max())
