@@ -504,6 +504,72 @@ int rlt_rocm_gru_backward(rlt_rocm_device* device, const rlt_gru_layer* layer, c
                           float* d_input, const uint8_t* reset, int sequence_length, int batch, int want_weight_gradients,
                           void* workspace, size_t workspace_bytes);
 
+/* --------------------------------------------------------------------- TD3 -- */
+
+/* td3_sampling layer      nn/layers/td3_sampling/operations_generic.h:75-128
+ *   sample = mean + noise * std (noise [batch x dim] are externally drawn N(0,1) values; NULL: sample = mean, the
+ *   Evaluation mode), output = clamp(sample, -1, 1); pre_clip (optional) receives sample, as forward() keeps it. */
+int rlt_rocm_td3_sampling_forward(rlt_rocm_device* device, const float* input, int ldin, const float* noise, int ldn, float std,
+                                  float* pre_clip, int ldp, float* output, int ldo, int batch, int dim);
+/* backward_full           td3_sampling/operations_generic.h:139-163 : d_input = (pre_clip < -1 || pre_clip > 1) ? 0 : d_output */
+int rlt_rocm_td3_sampling_backward(rlt_rocm_device* device, const float* pre_clip, int ldp, const float* d_output, int lddo,
+                                   float* d_input, int lddi, int batch, int dim);
+/* target_action_noise     rl/algorithms/td3/operations_generic.h:116-128, operations_cuda.h:8-44
+ *   from N(0,1) draws z: out = clamp(z * std + 0, -clip, clip) (the reference draws N(0, std) directly). */
+int rlt_rocm_td3_target_action_noise(rlt_rocm_device* device, const float* standard_normal, float std, float clip, float* out, size_t count);
+/* noisy_next_actions      td3/operations_generic.h:129-145, operations_cuda.h:46-75 : a = clamp(a + noise, -1, 1) in place */
+int rlt_rocm_td3_noisy_next_actions(rlt_rocm_device* device, float* next_actions, int lda, const float* noise, int ldn, int batch, int dim);
+/* target_action_values    td3/operations_generic.h:146-169, operations_cuda.h:77-110
+ *   y = r + (ignore_termination || !terminated ? gamma * min(q1', q2') : 0) */
+int rlt_rocm_td3_target_action_values(rlt_rocm_device* device, const float* q1_next, const float* q2_next, const float* rewards,
+                                      const uint8_t* terminated, float gamma, int ignore_termination, float* target, int batch);
+
+/* Everything one TD3 agent owns on the device (rl/algorithms/td3/td3.h ActorCritic, Critic/ActorTrainingBuffers, and the
+ * batch of rl/components/off_policy_runner/off_policy_runner.h:89-156 for SEQUENCE_LENGTH = 1). The actor is an MLP
+ * (output activation as configured, TANH in td3/loop/core/approximators_mlp.h:15-31) followed by the td3_sampling layer. */
+typedef struct rlt_td3_agent {
+    int32_t batch, observation_dim, action_dim, n_actor_layers, n_critic_layers, ignore_termination;
+    float gamma, actor_polyak, critic_polyak;
+    float sampling_std;                       /* std of the actor's td3_sampling layer (EXPLORATION_NOISE) */
+    rlt_adam_parameters actor_adam, critic_adam;
+    const rlt_dense_layer* actor;             /* out_dim of last layer = action_dim */
+    const rlt_dense_layer* actor_target;
+    const rlt_dense_layer* critics[2];
+    const rlt_dense_layer* critics_target[2];
+    const rlt_adam_tensor* actor_adam_tensors;      int32_t n_actor_adam_tensors;   int32_t pad0;
+    const rlt_adam_tensor* critic_adam_tensors[2];  int32_t n_critic_adam_tensors;  int32_t pad1;
+    uint32_t* actor_age; uint32_t* critic_age[2];
+    /* batch (SequentialBatch, SEQUENCE_LENGTH = 1): [2 x batch x (obs+act)] */
+    float* observations_actions_base;
+    float* rewards;            /* [batch] */
+    uint8_t* terminated;       /* [batch] */
+    const uint8_t* final_step_mask;        /* [batch]; NULL = all true */
+    const uint8_t* next_final_step_mask;   /* [batch]; NULL = all true */
+    /* critic training buffers */
+    float* target_next_action_noise;        /* [batch x act], already clamped (target_action_noise) */
+    float* next_state_action_value_input;   /* [batch x (obs+act)] */
+    float* next_q[2];                        /* [batch] each */
+    float* target_action_value;              /* [batch] */
+    float* d_output_critic;                  /* [batch] */
+    /* actor training buffers */
+    float* state_action_value_input;         /* [batch x (obs+act)] */
+    float* actor_pre_clip;                   /* [batch x act] */
+    float* d_output_actor;                   /* [batch] */
+    float* d_critic_input;                   /* [batch x (obs+act)] */
+    float* d_actor_output;                   /* [batch x act] */
+    void* workspace; size_t workspace_bytes;
+} rlt_td3_agent;
+
+/* train_critic            rl/algorithms/td3/operations_generic.h:170-235 for critic `critic_index`; sampling_noise [batch x act] are
+ *   the N(0,1) draws of the target actor's sampling layer (its evaluate runs in the default mode, which samples). */
+int rlt_rocm_td3_train_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
+/* train_actor             td3/operations_generic.h:236-281; sampling_noise as above, for the actor's forward pass */
+int rlt_rocm_td3_train_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise);
+/* update_critic_targets   td3/operations_generic.h:317-321 */
+int rlt_rocm_td3_update_critic_targets(rlt_rocm_device* device, const rlt_td3_agent* agent);
+/* update_actor_target     td3/operations_generic.h:322-325 */
+int rlt_rocm_td3_update_actor_target(rlt_rocm_device* device, const rlt_td3_agent* agent);
+
 #ifdef __cplusplus
 }
 #endif

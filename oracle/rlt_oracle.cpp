@@ -1009,4 +1009,142 @@ int rlt_oracle_gru_backward(const rlt_gru_layer* L, const float* input, float* d
     return 0;
 }
 
+// --------------------------------------------------------------------------------------------- TD3
+static inline float clamp_f(float x, float lo, float hi) { return x < lo ? lo : (x > hi ? hi : x); }   // math::clamp
+
+// nn/layers/td3_sampling/operations_generic.h:75-128
+int rlt_oracle_td3_sampling_forward(const float* input, int ldin, const float* noise, int ldn, float std, float* pre_clip, int ldp,
+                                    float* output, int ldo, int batch, int dim) {
+    if (!input || !output || batch <= 0 || dim <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int r = 0; r < batch; r++)
+        for (int c = 0; c < dim; c++) {
+            float mean = input[(size_t)r * ldin + c];
+            float sample = noise ? mean + noise[(size_t)r * ldn + c] * std : mean;
+            if (pre_clip) pre_clip[(size_t)r * ldp + c] = sample;
+            output[(size_t)r * ldo + c] = clamp_f(sample, -1.0f, 1.0f);
+        }
+    return 0;
+}
+// td3_sampling/operations_generic.h:139-163
+int rlt_oracle_td3_sampling_backward(const float* pre_clip, int ldp, const float* d_output, int lddo, float* d_input, int lddi, int batch, int dim) {
+    if (!pre_clip || !d_output || !d_input || batch <= 0 || dim <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int r = 0; r < batch; r++)
+        for (int c = 0; c < dim; c++) {
+            float pc = pre_clip[(size_t)r * ldp + c];
+            d_input[(size_t)r * lddi + c] = (pc < -1 || pc > 1) ? 0.0f : d_output[(size_t)r * lddo + c];
+        }
+    return 0;
+}
+// rl/algorithms/td3/operations_generic.h:116-128; std::normal_distribution(mean, std) returns z * std + mean
+int rlt_oracle_td3_target_action_noise(const float* z, float std, float clip, float* out, size_t count) {
+    if (!z || !out) return RLT_E_INVALID_ARGUMENT;
+    for (size_t i = 0; i < count; i++) out[i] = clamp_f(z[i] * std + 0.0f, -clip, clip);
+    return 0;
+}
+// td3/operations_generic.h:129-145
+int rlt_oracle_td3_noisy_next_actions(float* next_actions, int lda, const float* noise, int ldn, int batch, int dim) {
+    if (!next_actions || !noise || batch <= 0 || dim <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int r = 0; r < batch; r++)
+        for (int c = 0; c < dim; c++) {
+            float a = next_actions[(size_t)r * lda + c] + noise[(size_t)r * ldn + c];
+            next_actions[(size_t)r * lda + c] = clamp_f(a, -1.0f, 1.0f);
+        }
+    return 0;
+}
+// td3/operations_generic.h:146-169
+int rlt_oracle_td3_target_action_values(const float* q1, const float* q2, const float* rewards, const uint8_t* terminated,
+                                        float gamma, int ignore_termination, float* target, int batch) {
+    if (!q1 || !q2 || !rewards || !terminated || !target || batch <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int b = 0; b < batch; b++) {
+        float m = q1[b] < q2[b] ? q1[b] : q2[b];
+        float future = (ignore_termination || !terminated[b]) ? gamma * m : 0.0f;
+        target[b] = rewards[b] + future;
+    }
+    return 0;
+}
+
+// td3/operations_generic.h:170-235 with SEQUENCE_LENGTH = 1
+int rlt_oracle_td3_train_critic(const rlt_td3_agent* A, int ci, const float* sampling_noise) {
+    if (!A || ci < 0 || ci > 1 || !sampling_noise) return RLT_E_INVALID_ARGUMENT;
+    const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    const rlt_dense_layer* critic = A->critics[ci];
+    int rc;
+    if ((rc = rlt_oracle_mlp_zero_gradient(critic, A->n_critic_layers))) return rc;                                                  // :185
+    const float* obs_next = A->observations_actions_base + (size_t)B * D;
+    std::vector<float> mean((size_t)B * ACT);
+    if ((rc = rlt_oracle_mlp_evaluate(A->actor_target, A->n_actor_layers, obs_next, D, mean.data(), ACT, B))) return rc;             // :191 (MLP part)
+    float* next_actions = A->next_state_action_value_input + OBS;
+    if ((rc = rlt_oracle_td3_sampling_forward(mean.data(), ACT, sampling_noise, ACT, A->sampling_std, nullptr, 0, next_actions, D, B, ACT))) return rc;
+    if ((rc = rlt_oracle_td3_noisy_next_actions(next_actions, D, A->target_next_action_noise, ACT, B, ACT))) return rc;              // :192
+    if (A->next_final_step_mask)                                                                                                   // :193-195
+        if ((rc = rlt_oracle_mask_copy(obs_next + OBS, D, next_actions, D, A->next_final_step_mask, 1, B, ACT))) return rc;
+    for (int b = 0; b < B; b++) std::memcpy(A->next_state_action_value_input + (size_t)b * D, obs_next + (size_t)b * D, sizeof(float) * OBS);   // :196
+    for (int k = 0; k < 2; k++)                                                                                                    // :197-198
+        if ((rc = rlt_oracle_mlp_evaluate(A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, A->next_q[k], 1, B))) return rc;
+    if ((rc = rlt_oracle_td3_target_action_values(A->next_q[0], A->next_q[1], A->rewards, A->terminated, A->gamma, A->ignore_termination,
+                                                 A->target_action_value, B))) return rc;                                           // :200
+    if ((rc = rlt_oracle_mlp_forward(critic, A->n_critic_layers, A->observations_actions_base, D, B))) return rc;                   // :205
+    float* q = critic[A->n_critic_layers - 1].output;
+    // :207-212 loss_weight = 1 * (SEQ * B / num_final_steps)
+    float n_final = (float)B;
+    if (A->final_step_mask) rlt_oracle_cast_reduce_sum_u8(A->final_step_mask, B, &n_final);
+    float loss_weight = 1.0f; loss_weight *= (float)(1 * B) / n_final;
+    if ((rc = rlt_oracle_mse_gradient(q, 1, A->target_action_value, 1, A->d_output_critic, 1, B, 1, loss_weight, nullptr))) return rc;   // :217
+    if (A->final_step_mask) {                                                                                                      // :218-227
+        rlt_oracle_mask_zero(A->d_output_critic, 1, A->final_step_mask, 1, B, 1);
+        rlt_oracle_mask_zero(q, 1, A->final_step_mask, 1, B, 1);                      // the logging block zeroes these in place
+        rlt_oracle_mask_zero(A->target_action_value, 1, A->final_step_mask, 1, B, 1);
+    }
+    if ((rc = rlt_oracle_mlp_backward(critic, A->n_critic_layers, A->observations_actions_base, D, A->d_output_critic, 1, nullptr, 0, B, 1))) return rc;   // :233
+    return adam_over(A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci]);                   // :234
+}
+
+// td3/operations_generic.h:236-281 with SEQUENCE_LENGTH = 1
+int rlt_oracle_td3_train_actor(const rlt_td3_agent* A, const float* sampling_noise) {
+    if (!A || !sampling_noise) return RLT_E_INVALID_ARGUMENT;
+    const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    const float* obs = A->observations_actions_base;
+    int rc;
+    if ((rc = rlt_oracle_mlp_forward(A->actor, A->n_actor_layers, obs, D, B))) return rc;                                          // :255 (MLP part)
+    const float* mean = A->actor[A->n_actor_layers - 1].output;
+    float* actions = A->state_action_value_input + OBS;
+    if ((rc = rlt_oracle_td3_sampling_forward(mean, ACT, sampling_noise, ACT, A->sampling_std, A->actor_pre_clip, ACT, actions, D, B, ACT))) return rc;
+    if (A->final_step_mask)                                                                                                        // :256-258
+        if ((rc = rlt_oracle_mask_copy(obs + OBS, D, actions, D, A->final_step_mask, 1, B, ACT))) return rc;
+    for (int b = 0; b < B; b++) std::memcpy(A->state_action_value_input + (size_t)b * D, obs + (size_t)b * D, sizeof(float) * OBS);  // :259
+    const rlt_dense_layer* critic = A->critics[0];
+    if ((rc = rlt_oracle_mlp_forward(critic, A->n_critic_layers, A->state_action_value_input, D, B))) return rc;                    // :261
+    float n_final = (float)B;                                                                                                      // :262-267
+    if (A->final_step_mask) rlt_oracle_cast_reduce_sum_u8(A->final_step_mask, B, &n_final);
+    for (int b = 0; b < B; b++) A->d_output_actor[b] = (float)-1 / n_final;
+    if (A->final_step_mask) rlt_oracle_mask_zero(A->d_output_actor, 1, A->final_step_mask, 1, B, 1);
+    if ((rc = rlt_oracle_mlp_backward(critic, A->n_critic_layers, nullptr, 0, A->d_output_actor, 1, A->d_critic_input, D, B, 0))) return rc;   // :271
+    float* d_actions = A->d_critic_input + OBS;                                                                                    // :272
+    if (A->final_step_mask) rlt_oracle_mask_zero(d_actions, D, A->final_step_mask, 1, B, ACT);                                     // :273-275
+    if ((rc = rlt_oracle_mlp_zero_gradient(A->actor, A->n_actor_layers))) return rc;                                                // :277
+    // :278 sequential backward: the sampling layer's backward_full, then the MLP's backward
+    if ((rc = rlt_oracle_td3_sampling_backward(A->actor_pre_clip, ACT, d_actions, D, A->d_actor_output, ACT, B, ACT))) return rc;
+    if ((rc = rlt_oracle_mlp_backward(A->actor, A->n_actor_layers, obs, D, A->d_actor_output, ACT, nullptr, 0, B, 1))) return rc;
+    return adam_over(A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age);                               // :280
+}
+
+static void polyak_mlp(const rlt_dense_layer* source, const rlt_dense_layer* target, int n, float polyak) {
+    for (int l = 0; l < n; l++) {
+        rlt_oracle_polyak_update(source[l].weights, target[l].weights, (size_t)source[l].in_dim * source[l].out_dim, polyak, 0);
+        rlt_oracle_polyak_update(source[l].biases, target[l].biases, (size_t)source[l].out_dim, polyak, 0);
+    }
+}
+// td3/operations_generic.h:317-321
+int rlt_oracle_td3_update_critic_targets(const rlt_td3_agent* A) {
+    if (!A) return RLT_E_INVALID_ARGUMENT;
+    for (int k = 0; k < 2; k++) polyak_mlp(A->critics[k], A->critics_target[k], A->n_critic_layers, A->critic_polyak);
+    return 0;
+}
+// td3/operations_generic.h:322-325
+int rlt_oracle_td3_update_actor_target(const rlt_td3_agent* A) {
+    if (!A) return RLT_E_INVALID_ARGUMENT;
+    polyak_mlp(A->actor, A->actor_target, A->n_actor_layers, A->actor_polyak);
+    return 0;
+}
+
 }  // extern "C"

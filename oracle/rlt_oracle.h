@@ -13,6 +13,9 @@
  *   replay add, gather_batch, pendulum, gae: checked against the reference itself compiled from
  *   /root/reference (oracle/_ref) and against golden vectors written by it (tests/golden), plus the
  *   closed-form / finite-difference checks in tests/test_oracle_*.py.
+ *   ppo surrogate/train, gru forward/backward, td3 (sampling layer, noise, targets, train_*, target updates):
+ *   checked bit for bit against the reference's own PPO loop, GRU layer and TD3 loop compiled from
+ *   /root/reference (oracle/_ref), and against golden vectors written by them (tests/golden).
  */
 #ifndef RLT_ORACLE_H
 #define RLT_ORACLE_H
@@ -104,6 +107,18 @@ int rlt_oracle_gru_backward(const rlt_gru_layer* layer, const float* input, floa
                             int sequence_length, int batch, int want_weight_gradients);
 /* the reference's per-epoch in-place dataset shuffle as row permutations, driven by the text form of its std::mt19937 */
 int rlt_oracle_ppo_shuffle(char* rng_state, int rng_state_capacity, int n, int epochs, uint32_t* permutations);
+
+int rlt_oracle_td3_sampling_forward(const float* input, int ldin, const float* noise, int ldn, float std, float* pre_clip, int ldp,
+                                    float* output, int ldo, int batch, int dim);
+int rlt_oracle_td3_sampling_backward(const float* pre_clip, int ldp, const float* d_output, int lddo, float* d_input, int lddi, int batch, int dim);
+int rlt_oracle_td3_target_action_noise(const float* standard_normal, float std, float clip, float* out, size_t count);
+int rlt_oracle_td3_noisy_next_actions(float* next_actions, int lda, const float* noise, int ldn, int batch, int dim);
+int rlt_oracle_td3_target_action_values(const float* q1_next, const float* q2_next, const float* rewards, const uint8_t* terminated,
+                                        float gamma, int ignore_termination, float* target, int batch);
+int rlt_oracle_td3_train_critic(const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
+int rlt_oracle_td3_train_actor(const rlt_td3_agent* agent, const float* sampling_noise);
+int rlt_oracle_td3_update_critic_targets(const rlt_td3_agent* agent);
+int rlt_oracle_td3_update_actor_target(const rlt_td3_agent* agent);
 
 #ifdef __cplusplus
 }

@@ -116,6 +116,25 @@ class GruLayer(C.Structure):
                 ("input_dim", C.c_int32), ("hidden_dim", C.c_int32)]
 
 
+class Td3Agent(C.Structure):
+    _fields_ = [("batch", C.c_int32), ("observation_dim", C.c_int32), ("action_dim", C.c_int32), ("n_actor_layers", C.c_int32),
+                ("n_critic_layers", C.c_int32), ("ignore_termination", C.c_int32),
+                ("gamma", C.c_float), ("actor_polyak", C.c_float), ("critic_polyak", C.c_float), ("sampling_std", C.c_float),
+                ("actor_adam", AdamParameters), ("critic_adam", AdamParameters),
+                ("actor", C.POINTER(DenseLayer)), ("actor_target", C.POINTER(DenseLayer)),
+                ("critics", C.POINTER(DenseLayer) * 2), ("critics_target", C.POINTER(DenseLayer) * 2),
+                ("actor_adam_tensors", C.POINTER(AdamTensor)), ("n_actor_adam_tensors", C.c_int32), ("pad0", C.c_int32),
+                ("critic_adam_tensors", C.POINTER(AdamTensor) * 2), ("n_critic_adam_tensors", C.c_int32), ("pad1", C.c_int32),
+                ("actor_age", C.c_void_p), ("critic_age", C.c_void_p * 2),
+                ("observations_actions_base", C.c_void_p), ("rewards", C.c_void_p), ("terminated", C.c_void_p),
+                ("final_step_mask", C.c_void_p), ("next_final_step_mask", C.c_void_p),
+                ("target_next_action_noise", C.c_void_p), ("next_state_action_value_input", C.c_void_p), ("next_q", C.c_void_p * 2),
+                ("target_action_value", C.c_void_p), ("d_output_critic", C.c_void_p),
+                ("state_action_value_input", C.c_void_p), ("actor_pre_clip", C.c_void_p), ("d_output_actor", C.c_void_p),
+                ("d_critic_input", C.c_void_p), ("d_actor_output", C.c_void_p),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+
+
 I, F, P, S, U64 = C.c_int, C.c_float, C.c_void_p, C.c_size_t, C.c_uint64
 LP = C.POINTER(DenseLayer)
 
@@ -155,6 +174,15 @@ PROTOTYPES = {
     "gru_backward": [C.POINTER(GruLayer), P, P, P, P, I, I, I, P, S],
     "ppo_surrogate_gradient": [P, I, P, P, I, P, I, P, I, C.POINTER(PpoParameters), P, I, P, I, I],
     "ppo_train_minibatch": [C.POINTER(PpoAgent), C.POINTER(PpoParameters), P, P, P, P, P, P, I, P, P],
+    "td3_sampling_forward": [P, I, P, I, F, P, I, P, I, I, I],
+    "td3_sampling_backward": [P, I, P, I, P, I, I, I],
+    "td3_target_action_noise": [P, F, F, P, S],
+    "td3_noisy_next_actions": [P, I, P, I, I, I],
+    "td3_target_action_values": [P, P, P, P, F, I, P, I],
+    "td3_train_critic": [C.POINTER(Td3Agent), I, P],
+    "td3_train_actor": [C.POINTER(Td3Agent), P],
+    "td3_update_critic_targets": [C.POINTER(Td3Agent)],
+    "td3_update_actor_target": [C.POINTER(Td3Agent)],
 }
 # workspace arguments exist only in the device ABI (the CPU checker allocates its own)
 ROCM_ONLY = {

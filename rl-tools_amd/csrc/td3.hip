@@ -1,0 +1,278 @@
+// TD3: the actor's clipped-Gaussian sampling layer, target-policy smoothing noise, TD target, and train_critic / train_actor /
+// target updates assembled from them and the shared network kernels.
+// reference: nn/layers/td3_sampling/operations_generic.h:75-163,
+//            rl/algorithms/td3/operations_generic.h:116-325 (CUDA: operations_cuda.h:8-110).
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float clampf(float x, float lo, float hi) { return x < lo ? lo : (x > hi ? hi : x); }
+// a * b + c rounded twice, as the reference's CPU build computes it (keeps the compiler from contracting into one fused operation)
+__device__ __forceinline__ float mul_add(float a, float b, float c) {
+#pragma clang fp contract(off)
+    float product = a * b;
+    return product + c;
+}
+
+__global__ __launch_bounds__(256) void td3_sampling_forward_kernel(const float* __restrict__ input, int ldin, const float* __restrict__ noise, int ldn, float std,
+                                                                   float* __restrict__ pre_clip, int ldp, float* __restrict__ output, int ldo, int batch, int dim) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < batch * dim; i += gridDim.x * blockDim.x) {
+        int r = i / dim, c = i % dim;
+        float mean = input[(size_t)r * ldin + c];
+        float sample = noise ? mul_add(noise[(size_t)r * ldn + c], std, mean) : mean;
+        if (pre_clip) pre_clip[(size_t)r * ldp + c] = sample;
+        output[(size_t)r * ldo + c] = clampf(sample, -1.0f, 1.0f);
+    }
+}
+
+__global__ __launch_bounds__(256) void td3_sampling_backward_kernel(const float* __restrict__ pre_clip, int ldp, const float* __restrict__ d_output, int lddo,
+                                                                    float* __restrict__ d_input, int lddi, int batch, int dim) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < batch * dim; i += gridDim.x * blockDim.x) {
+        int r = i / dim, c = i % dim;
+        float pc = pre_clip[(size_t)r * ldp + c];
+        d_input[(size_t)r * lddi + c] = (pc < -1.0f || pc > 1.0f) ? 0.0f : d_output[(size_t)r * lddo + c];
+    }
+}
+
+__global__ __launch_bounds__(256) void td3_target_action_noise_kernel(const float* __restrict__ z, float std, float clip, float* __restrict__ out, size_t count) {
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        out[i] = clampf(mul_add(z[i], std, 0.0f), -clip, clip);
+}
+
+__global__ __launch_bounds__(256) void td3_noisy_next_actions_kernel(float* __restrict__ a, int lda, const float* __restrict__ noise, int ldn, int batch, int dim) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < batch * dim; i += gridDim.x * blockDim.x) {
+        int r = i / dim, c = i % dim;
+        a[(size_t)r * lda + c] = clampf(a[(size_t)r * lda + c] + noise[(size_t)r * ldn + c], -1.0f, 1.0f);
+    }
+}
+
+__global__ __launch_bounds__(256) void td3_target_q_kernel(const float* __restrict__ q1, const float* __restrict__ q2, const float* __restrict__ rewards,
+                                                           const uint8_t* __restrict__ terminated, float gamma, int ignore_termination,
+                                                           float* __restrict__ target, int batch) {
+    for (int b = blockIdx.x * blockDim.x + threadIdx.x; b < batch; b += gridDim.x * blockDim.x) {
+        float m = fminf(q1[b], q2[b]);
+        float future = (ignore_termination || !terminated[b]) ? gamma * m : 0.0f;
+        target[b] = mul_add(1.0f, rewards[b], future);
+    }
+}
+
+// The input of the target critics in one pass over the rows (td3/operations_generic.h:191-196): the target actor's mean through the
+// sampling layer, the smoothing noise, the mask that keeps the stored next action on non-final steps, and the observation copy.
+__global__ __launch_bounds__(256) void td3_next_input_kernel(const float* __restrict__ mean, const float* __restrict__ sampling_noise, float std,
+                                                             const float* __restrict__ target_noise, const uint8_t* __restrict__ next_final_step_mask,
+                                                             const float* __restrict__ obs_next, float* __restrict__ next_input, int batch, int obs, int act) {
+    const int D = obs + act;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < batch * D; i += gridDim.x * blockDim.x) {
+        int r = i / D, c = i % D;
+        float v = obs_next[i];
+        if (c >= obs && (!next_final_step_mask || next_final_step_mask[r])) {
+            int a = c - obs;
+            float sample = mul_add(sampling_noise[(size_t)r * act + a], std, mean[(size_t)r * act + a]);
+            v = clampf(clampf(sample, -1.0f, 1.0f) + target_noise[(size_t)r * act + a], -1.0f, 1.0f);
+        }
+        next_input[i] = v;
+    }
+}
+
+// The input of critic 0 in train_actor (:255-259): sampled action (or the stored one on non-final steps) beside the observation.
+__global__ __launch_bounds__(256) void td3_actor_input_kernel(const float* __restrict__ mean, const float* __restrict__ sampling_noise, float std,
+                                                              const uint8_t* __restrict__ final_step_mask, const float* __restrict__ obs_act,
+                                                              float* __restrict__ pre_clip, float* __restrict__ input, int batch, int obs, int act) {
+    const int D = obs + act;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < batch * D; i += gridDim.x * blockDim.x) {
+        int r = i / D, c = i % D;
+        float v = obs_act[i];
+        if (c >= obs) {
+            int a = c - obs;
+            float sample = mul_add(sampling_noise[(size_t)r * act + a], std, mean[(size_t)r * act + a]);
+            pre_clip[(size_t)r * act + a] = sample;
+            if (!final_step_mask || final_step_mask[r]) v = clampf(sample, -1.0f, 1.0f);
+        }
+        input[i] = v;
+    }
+}
+
+// One workgroup: n = count(final_step_mask) (or rows), then
+//   critic (:200-227): y = r + gamma * min(q1', q2') unless terminated; d = (q - y) * 2/rows * (rows/n); where the mask is clear d, q and y
+//                      are zeroed (the reference zeroes the latter two in its logging block);
+//   actor  (:262-267): d = -1/n, zeroed where the mask is clear.
+__global__ __launch_bounds__(1024) void td3_d_output_kernel(float* __restrict__ q, const float* __restrict__ q1n, const float* __restrict__ q2n,
+                                                            const float* __restrict__ rewards, const uint8_t* __restrict__ terminated, float gamma,
+                                                            int ignore_termination, float* __restrict__ y, const uint8_t* __restrict__ mask,
+                                                            float* __restrict__ d, int rows, int actor) {
+    __shared__ float partial[16];
+    __shared__ float n_final;
+    float cnt = 0.0f;
+    for (int i = threadIdx.x; i < rows; i += blockDim.x) cnt += mask ? (float)(mask[i] != 0) : 1.0f;
+    cnt = rlt_wave_sum(cnt);
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = cnt;
+    __syncthreads();
+    if (threadIdx.x == 0) { float s = 0.0f; for (int i = 0; i < 16; i++) s += partial[i]; n_final = s; }
+    __syncthreads();
+    if (actor) {
+        const float v = -1.0f / n_final;
+        for (int i = threadIdx.x; i < rows; i += blockDim.x) d[i] = (!mask || mask[i]) ? v : 0.0f;
+        return;
+    }
+    float loss_weight = 1.0f; loss_weight *= (float)rows / n_final;
+    const float constant = 2.0f / (float)rows * loss_weight;
+    for (int i = threadIdx.x; i < rows; i += blockDim.x) {
+        float m = fminf(q1n[i], q2n[i]);
+        float future = (ignore_termination || !terminated[i]) ? gamma * m : 0.0f;
+        float target = mul_add(1.0f, rewards[i], future);
+        float diff = q[i] - target;
+        if (!mask || mask[i]) { y[i] = target; d[i] = diff * constant; }
+        else { y[i] = 0.0f; d[i] = 0.0f; q[i] = 0.0f; }
+    }
+}
+
+// d_actions (columns obs.. of d_critic_input) through the mask and the sampling layer's backward (:272-278)
+__global__ __launch_bounds__(256) void td3_actor_d_output_kernel(float* __restrict__ d_critic_input, const float* __restrict__ pre_clip,
+                                                                 const uint8_t* __restrict__ final_step_mask, float* __restrict__ d_actor_output,
+                                                                 int batch, int obs, int act) {
+    const int D = obs + act;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < batch * act; i += gridDim.x * blockDim.x) {
+        int r = i / act, a = i % act;
+        float g = d_critic_input[(size_t)r * D + obs + a];
+        float pc = pre_clip[i];
+        if (final_step_mask && !final_step_mask[r]) { g = 0.0f; d_critic_input[(size_t)r * D + obs + a] = 0.0f; }   // mask_gradient works in place
+        d_actor_output[i] = (pc < -1.0f || pc > 1.0f) ? 0.0f : g;
+    }
+}
+
+int grid1(long n) { long b = (n + 255) / 256; return (int)(b > 1024 ? 1024 : (b < 1 ? 1 : b)); }
+
+bool agent_ok(const rlt_td3_agent* A) {
+    return A && A->batch > 0 && A->observation_dim > 0 && A->action_dim > 0 && A->n_actor_layers >= 1 && A->n_critic_layers >= 1 && A->actor && A->actor_target &&
+           A->critics[0] && A->critics[1] && A->critics_target[0] && A->critics_target[1] && A->observations_actions_base && A->rewards && A->terminated &&
+           A->workspace && A->actor[A->n_actor_layers - 1].out_dim == A->action_dim && A->critics[0][0].in_dim == A->observation_dim + A->action_dim;
+}
+
+int polyak_mlp(rlt_rocm_device* device, const rlt_dense_layer* source, const rlt_dense_layer* target, int n, float polyak) {
+    for (int l = 0; l < n; l++) {
+        int rc;
+        if ((rc = rlt_rocm_polyak_update(device, source[l].weights, target[l].weights, (size_t)source[l].in_dim * source[l].out_dim, polyak, 0))) return rc;
+        if ((rc = rlt_rocm_polyak_update(device, source[l].biases, target[l].biases, (size_t)source[l].out_dim, polyak, 0))) return rc;
+    }
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rlt_rocm_td3_sampling_forward(rlt_rocm_device* device, const float* input, int ldin, const float* noise, int ldn, float std, float* pre_clip, int ldp,
+                                  float* output, int ldo, int batch, int dim) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(input && output && batch > 0 && dim > 0 && ldin >= dim && ldo >= dim && (!noise || ldn >= dim) && (!pre_clip || ldp >= dim));
+    hipLaunchKernelGGL(td3_sampling_forward_kernel, dim3(grid1((long)batch * dim)), dim3(256), 0, device->stream, input, ldin, noise, ldn, std, pre_clip, ldp, output, ldo, batch, dim);
+    return rlt_launch_status(device);
+}
+
+int rlt_rocm_td3_sampling_backward(rlt_rocm_device* device, const float* pre_clip, int ldp, const float* d_output, int lddo, float* d_input, int lddi, int batch, int dim) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(pre_clip && d_output && d_input && batch > 0 && dim > 0 && ldp >= dim && lddo >= dim && lddi >= dim);
+    hipLaunchKernelGGL(td3_sampling_backward_kernel, dim3(grid1((long)batch * dim)), dim3(256), 0, device->stream, pre_clip, ldp, d_output, lddo, d_input, lddi, batch, dim);
+    return rlt_launch_status(device);
+}
+
+int rlt_rocm_td3_target_action_noise(rlt_rocm_device* device, const float* standard_normal, float std, float clip, float* out, size_t count) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(standard_normal && out && count > 0 && clip >= 0.0f);
+    hipLaunchKernelGGL(td3_target_action_noise_kernel, dim3(grid1((long)count)), dim3(256), 0, device->stream, standard_normal, std, clip, out, count);
+    return rlt_launch_status(device);
+}
+
+int rlt_rocm_td3_noisy_next_actions(rlt_rocm_device* device, float* next_actions, int lda, const float* noise, int ldn, int batch, int dim) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(next_actions && noise && batch > 0 && dim > 0 && lda >= dim && ldn >= dim);
+    hipLaunchKernelGGL(td3_noisy_next_actions_kernel, dim3(grid1((long)batch * dim)), dim3(256), 0, device->stream, next_actions, lda, noise, ldn, batch, dim);
+    return rlt_launch_status(device);
+}
+
+int rlt_rocm_td3_target_action_values(rlt_rocm_device* device, const float* q1_next, const float* q2_next, const float* rewards, const uint8_t* terminated,
+                                      float gamma, int ignore_termination, float* target, int batch) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(q1_next && q2_next && rewards && terminated && target && batch > 0);
+    hipLaunchKernelGGL(td3_target_q_kernel, dim3(grid1(batch)), dim3(256), 0, device->stream, q1_next, q2_next, rewards, terminated, gamma, ignore_termination, target, batch);
+    return rlt_launch_status(device);
+}
+
+// rl/algorithms/td3/operations_generic.h:170-235. The elementwise steps between the network passes are folded into two launches.
+int rlt_rocm_td3_train_critic(rlt_rocm_device* device, const rlt_td3_agent* A, int ci, const float* sampling_noise) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(agent_ok(A) && (ci == 0 || ci == 1) && sampling_noise);
+    RLT_REQUIRE(A->target_next_action_noise && A->next_state_action_value_input && A->next_q[0] && A->next_q[1] && A->target_action_value && A->d_output_critic);
+    RLT_REQUIRE(A->critic_adam_tensors[ci] && A->critic_age[ci]);
+    const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    const rlt_dense_layer* critic = A->critics[ci];
+    const size_t mean_bytes = ((size_t)B * ACT * sizeof(float) + 255) & ~(size_t)255;
+    RLT_REQUIRE(A->workspace_bytes >= rlt_rocm_mlp_workspace_bytes(critic, A->n_critic_layers, B) + mean_bytes);
+    RLT_REQUIRE(A->workspace_bytes >= rlt_rocm_mlp_workspace_bytes(A->actor_target, A->n_actor_layers, B) + mean_bytes);
+    float* mean = (float*)A->workspace;
+    void* ws = (char*)A->workspace + mean_bytes;
+    const size_t ws_bytes = A->workspace_bytes - mean_bytes;
+    int rc;
+    if ((rc = rlt_rocm_mlp_zero_gradient(device, critic, A->n_critic_layers))) return rc;
+    const float* obs_next = A->observations_actions_base + (size_t)B * D;
+    if ((rc = rlt_rocm_mlp_evaluate(device, A->actor_target, A->n_actor_layers, obs_next, D, mean, ACT, B, ws, ws_bytes))) return rc;
+    hipLaunchKernelGGL(td3_next_input_kernel, dim3(grid1((long)B * D)), dim3(256), 0, device->stream, (const float*)mean, sampling_noise, A->sampling_std,
+                       (const float*)A->target_next_action_noise, A->next_final_step_mask, obs_next, A->next_state_action_value_input, B, OBS, ACT);
+    if ((rc = rlt_launch_status(device))) return rc;
+    for (int k = 0; k < 2; k++)
+        if ((rc = rlt_rocm_mlp_evaluate(device, A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, A->next_q[k], 1, B, ws, ws_bytes))) return rc;
+    if ((rc = rlt_rocm_mlp_forward(device, critic, A->n_critic_layers, A->observations_actions_base, D, B))) return rc;
+    float* q = critic[A->n_critic_layers - 1].output;
+    hipLaunchKernelGGL(td3_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, q, (const float*)A->next_q[0], (const float*)A->next_q[1], (const float*)A->rewards,
+                       (const uint8_t*)A->terminated, A->gamma, A->ignore_termination, A->target_action_value, A->final_step_mask, A->d_output_critic, B, 0);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if ((rc = rlt_rocm_mlp_backward(device, critic, A->n_critic_layers, A->observations_actions_base, D, A->d_output_critic, 1, nullptr, 0, B, 1, ws, ws_bytes))) return rc;
+    return rlt_rocm_adam_step(device, A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], 0.0f, nullptr);
+}
+
+// rl/algorithms/td3/operations_generic.h:236-281
+int rlt_rocm_td3_train_actor(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(agent_ok(A) && sampling_noise);
+    RLT_REQUIRE(A->state_action_value_input && A->actor_pre_clip && A->d_output_actor && A->d_critic_input && A->d_actor_output && A->actor_adam_tensors && A->actor_age);
+    const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    RLT_REQUIRE(A->workspace_bytes >= rlt_rocm_mlp_workspace_bytes(A->critics[0], A->n_critic_layers, B));
+    RLT_REQUIRE(A->workspace_bytes >= rlt_rocm_mlp_workspace_bytes(A->actor, A->n_actor_layers, B));
+    void* ws = A->workspace; const size_t ws_bytes = A->workspace_bytes;
+    const float* obs = A->observations_actions_base;
+    const rlt_dense_layer* critic = A->critics[0];
+    int rc;
+    if ((rc = rlt_rocm_mlp_forward(device, A->actor, A->n_actor_layers, obs, D, B))) return rc;
+    const float* mean = A->actor[A->n_actor_layers - 1].output;
+    hipLaunchKernelGGL(td3_actor_input_kernel, dim3(grid1((long)B * D)), dim3(256), 0, device->stream, mean, sampling_noise, A->sampling_std, A->final_step_mask, obs,
+                       A->actor_pre_clip, A->state_action_value_input, B, OBS, ACT);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if ((rc = rlt_rocm_mlp_forward(device, critic, A->n_critic_layers, A->state_action_value_input, D, B))) return rc;
+    hipLaunchKernelGGL(td3_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, (float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+                       (const uint8_t*)nullptr, 0.0f, 0, (float*)nullptr, A->final_step_mask, A->d_output_actor, B, 1);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if ((rc = rlt_rocm_mlp_backward(device, critic, A->n_critic_layers, nullptr, 0, A->d_output_actor, 1, A->d_critic_input, D, B, 0, ws, ws_bytes))) return rc;
+    hipLaunchKernelGGL(td3_actor_d_output_kernel, dim3(grid1((long)B * ACT)), dim3(256), 0, device->stream, A->d_critic_input, (const float*)A->actor_pre_clip,
+                       A->final_step_mask, A->d_actor_output, B, OBS, ACT);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if ((rc = rlt_rocm_mlp_zero_gradient(device, A->actor, A->n_actor_layers))) return rc;
+    if ((rc = rlt_rocm_mlp_backward(device, A->actor, A->n_actor_layers, obs, D, A->d_actor_output, ACT, nullptr, 0, B, 1, ws, ws_bytes))) return rc;
+    return rlt_rocm_adam_step(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, 0.0f, nullptr);
+}
+
+// rl/algorithms/td3/operations_generic.h:317-321
+int rlt_rocm_td3_update_critic_targets(rlt_rocm_device* device, const rlt_td3_agent* A) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(agent_ok(A));
+    for (int k = 0; k < 2; k++) { int rc = polyak_mlp(device, A->critics[k], A->critics_target[k], A->n_critic_layers, A->critic_polyak); if (rc) return rc; }
+    return 0;
+}
+
+// rl/algorithms/td3/operations_generic.h:322-325
+int rlt_rocm_td3_update_actor_target(rlt_rocm_device* device, const rlt_td3_agent* A) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(agent_ok(A));
+    return polyak_mlp(device, A->actor, A->actor_target, A->n_actor_layers, A->actor_polyak);
+}
+
+}  // extern "C"

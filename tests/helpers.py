@@ -516,3 +516,186 @@ def ppo_train_like_reference(backend, agent, params, dataset, ld, col, n_rows, p
                          dataset.offset(col["target_values"]), ld, idx.offset(b * batch), loss.ptr)
             losses.append(float(loss.numpy()[0]))
     return losses
+
+
+# ------------------------------------------------------------------------------------------------------------------ TD3
+REF_TD3_GENERIC = os.path.join(ROOT, "oracle", "_ref", "librlt_ref_td3_generic.so")
+
+
+class Td3OnBackend:
+    """All TD3 state for the Pendulum shapes (observation 3, action 1) on one backend. `params` is the flat vector
+    [actor, actor_target, critic 0, critic 1, critic target 0, critic target 1], each [W|b] per layer."""
+
+    def __init__(self, backend, batch, hidden, params, hyper=None, masks=False, obs=3, act=1):
+        OBS, ACT, D = obs, act, obs + act
+        self.backend, self.batch, self.OBS, self.ACT = backend, batch, OBS, ACT
+        adims, cdims = [OBS, hidden, hidden, ACT], [D, hidden, hidden, 1]
+        na, nc = mlp_param_count(adims), mlp_param_count(cdims)
+        assert params.size == 2 * na + 4 * nc
+        o = 0
+        self.actor = Mlp(backend, adims, params[o:o + na], batch, out_act="tanh"); o += na
+        self.actor_target = Mlp(backend, adims, params[o:o + na], batch, out_act="tanh", trainable=False); o += na
+        self.critics = []
+        for _ in range(2):
+            self.critics.append(Mlp(backend, cdims, params[o:o + nc], batch)); o += nc
+        self.targets = []
+        for _ in range(2):
+            self.targets.append(Mlp(backend, cdims, params[o:o + nc], batch, trainable=False)); o += nc
+        z = backend.zeros
+        self.oab = z((2, batch, D)); self.rewards = z((batch,)); self.terminated = z((batch,), np.uint8)
+        self.m_final = backend.array(np.ones(batch, np.uint8)); self.m_next_final = backend.array(np.ones(batch, np.uint8))
+        self.target_noise = z((batch, ACT)); self.nsavi = z((batch, D)); self.next_q = [z((batch,)), z((batch,))]; self.target_q = z((batch,))
+        self.d_out_c = z((batch,)); self.savi = z((batch, D)); self.pre_clip = z((batch, ACT)); self.d_out_a = z((batch,))
+        self.d_ci = z((batch, D)); self.d_ao = z((batch, ACT))
+        h = hyper if hyper is not None else dict(gamma=0.99, actor_polyak=float(np.float32(1.0 - 0.005)), critic_polyak=float(np.float32(1.0 - 0.005)),
+                                                 sampling_std=0.1, adam=capi.adam_parameters(epsilon=1e-7))
+        A = capi.Td3Agent()
+        A.batch, A.observation_dim, A.action_dim, A.n_actor_layers, A.n_critic_layers, A.ignore_termination = batch, OBS, ACT, 3, 3, 0
+        A.gamma, A.actor_polyak, A.critic_polyak, A.sampling_std = h["gamma"], h["actor_polyak"], h["critic_polyak"], h["sampling_std"]
+        A.actor_adam = A.critic_adam = h["adam"]
+        A.actor, A.actor_target = self.actor.layers, self.actor_target.layers
+        A.actor_adam_tensors, A.n_actor_adam_tensors, A.actor_age = self.actor.adam, self.actor.n_adam, self.actor.age.ptr
+        for k in range(2):
+            A.critics[k] = self.critics[k].layers; A.critics_target[k] = self.targets[k].layers
+            A.critic_adam_tensors[k] = self.critics[k].adam; A.critic_age[k] = self.critics[k].age.ptr
+            A.next_q[k] = self.next_q[k].ptr
+        A.n_critic_adam_tensors = self.critics[0].n_adam
+        A.observations_actions_base, A.rewards, A.terminated = self.oab.ptr, self.rewards.ptr, self.terminated.ptr
+        if masks:
+            A.final_step_mask, A.next_final_step_mask = self.m_final.ptr, self.m_next_final.ptr
+        A.target_next_action_noise, A.next_state_action_value_input, A.target_action_value = self.target_noise.ptr, self.nsavi.ptr, self.target_q.ptr
+        A.d_output_critic, A.state_action_value_input, A.actor_pre_clip = self.d_out_c.ptr, self.savi.ptr, self.pre_clip.ptr
+        A.d_output_actor, A.d_critic_input, A.d_actor_output = self.d_out_a.ptr, self.d_ci.ptr, self.d_ao.ptr
+        if backend.name == "rocm":
+            lib = backend.device.lib
+            nbytes = max(lib.rlt_rocm_mlp_workspace_bytes(self.actor.layers, 3, batch), lib.rlt_rocm_mlp_workspace_bytes(self.critics[0].layers, 3, batch))
+            nbytes += batch * ACT * 4 + 1024
+            self.ws = backend.device.empty((nbytes,), np.uint8)
+            A.workspace, A.workspace_bytes = self.ws.ptr, self.ws.nbytes
+        else:
+            self.ws = backend.zeros((64,), np.uint8)
+            A.workspace, A.workspace_bytes = self.ws.ptr, 64
+        self.c = A
+
+    def parameters(self):
+        nets = [self.actor, self.actor_target] + self.critics + self.targets
+        return np.concatenate([n.params.numpy() for n in nets])
+
+    def ages(self):
+        return np.array([self.actor.age.numpy()[0], self.critics[0].age.numpy()[0], self.critics[1].age.numpy()[0]], np.uint32)
+
+    def state(self):
+        """Everything an update reads and writes: parameters of all six networks, Adam moments and ages of the three trained ones."""
+        nets = [self.actor] + self.critics
+        return dict(params=[n.params.numpy() for n in [self.actor, self.actor_target] + self.critics + self.targets],
+                    m=[n.m.numpy() for n in nets], v=[n.v.numpy() for n in nets], age=[n.age.numpy() for n in nets])
+
+    def push(self, st):
+        nets = [self.actor] + self.critics
+        for n, p in zip([self.actor, self.actor_target] + self.critics + self.targets, st["params"]):
+            n.params.upload(p)
+        for n, m, v, a in zip(nets, st["m"], st["v"], st["age"]):
+            n.m.upload(m); n.v.upload(v); n.age.upload(a)
+
+    def gradients(self):
+        return np.concatenate([n.grads.numpy() for n in [self.actor] + self.critics])
+
+    def set_batch(self, oab, rewards, terminated, target_noise):
+        self.oab.upload(oab); self.rewards.upload(rewards); self.terminated.upload(terminated); self.target_noise.upload(target_noise)
+
+    def loop_step(self, flags, noise_c0, noise_c1, noise_a):
+        """The training half of td3::loop::core::step (rl/algorithms/td3/loop/core/operations_generic.h:98-133) on the batch set before."""
+        b = self.backend
+        if flags[0]:
+            for k, nz in enumerate((noise_c0, noise_c1)):
+                n = b.array(nz.astype(np.float32))
+                b.call("td3_train_critic", C.byref(self.c), k, n.ptr)
+                b.sync()
+        if flags[1]:
+            b.call("td3_update_critic_targets", C.byref(self.c))
+        if flags[2]:
+            n = b.array(noise_a.astype(np.float32))
+            b.call("td3_train_actor", C.byref(self.c), n.ptr)
+            b.sync()
+        if flags[3]:
+            b.call("td3_update_actor_target", C.byref(self.c))
+        b.sync()
+
+
+class RefTd3:
+    """The reference's own TD3-on-Pendulum loop (oracle/_ref, compiled from /root/reference)."""
+    BATCH = 100
+
+    def __init__(self, seed):
+        self.lib = lib = C.CDLL(REF_TD3_GENERIC)
+        P = C.c_void_p
+        lib.rlt_ref_td3_create.restype = P; lib.rlt_ref_td3_create.argtypes = [C.c_uint32]
+        lib.rlt_ref_td3_parameter_count.restype = C.c_size_t; lib.rlt_ref_td3_parameter_count.argtypes = [P]
+        lib.rlt_ref_td3_step_count.restype = C.c_uint32; lib.rlt_ref_td3_step_count.argtypes = [P]
+        for f, n in (("destroy", 1), ("step", 1), ("get_parameters", 2), ("get_ages", 2), ("hyperparameters", 2), ("get_noise", 2), ("get_batch", 6), ("manual_step", 6)):
+            getattr(lib, "rlt_ref_td3_" + f).argtypes = [P] * n
+        lib.rlt_ref_td3_dims.argtypes = [P]
+        self.h = lib.rlt_ref_td3_create(seed)
+        d = np.zeros(6, np.int32); lib.rlt_ref_td3_dims(d.ctypes.data)
+        self.batch, self.n_warmup, self.actor_interval, self.critic_target_interval, self.actor_target_interval, self.hidden = [int(x) for x in d]
+        hp = np.zeros(11, np.float32); lib.rlt_ref_td3_hyperparameters(self.h, hp.ctypes.data)
+        self.hp = hp
+
+    def hyper(self):
+        hp = self.hp
+        return dict(gamma=float(hp[0]), actor_polyak=float(hp[1]), critic_polyak=float(hp[2]), sampling_std=float(hp[10]),
+                    adam=capi.adam_parameters(alpha=float(hp[5]), beta_1=float(hp[6]), beta_2=float(hp[7]), epsilon=float(hp[8]), epsilon_sqrt=float(hp[9])))
+
+    def step(self):
+        self.lib.rlt_ref_td3_step(self.h)
+
+    def manual_step(self):
+        B = self.batch
+        z, c0, c1, a = (np.zeros((B, 1), np.float32) for _ in range(4))
+        flags = np.zeros(4, np.int32)
+        self.lib.rlt_ref_td3_manual_step(self.h, z.ctypes.data, c0.ctypes.data, c1.ctypes.data, a.ctypes.data, flags.ctypes.data)
+        return z, c0, c1, a, [int(f) for f in flags]
+
+    def parameters(self):
+        p = np.zeros(self.lib.rlt_ref_td3_parameter_count(self.h), np.float32)
+        self.lib.rlt_ref_td3_get_parameters(self.h, p.ctypes.data)
+        return p
+
+    def ages(self):
+        a = np.zeros(3, np.uint32); self.lib.rlt_ref_td3_get_ages(self.h, a.ctypes.data); return a
+
+    def batch_data(self):
+        B = self.batch
+        oab = np.zeros((2, B, 4), np.float32); r = np.zeros(B, np.float32); t = np.zeros(B, np.uint8); fm = np.zeros(B, np.uint8); nfm = np.zeros(2 * B, np.uint8)
+        self.lib.rlt_ref_td3_get_batch(self.h, oab.ctypes.data, r.ctypes.data, t.ctypes.data, fm.ctypes.data, nfm.ctypes.data)
+        return oab, r, t, fm, nfm
+
+    def target_noise(self):
+        n = np.zeros((self.batch, 1), np.float32); self.lib.rlt_ref_td3_get_noise(self.h, n.ctypes.data); return n
+
+    def close(self):
+        self.lib.rlt_ref_td3_destroy(self.h)
+
+
+def td3_digest(params, hidden, obs=3, act=1):
+    """float64 (sum, sum of squares) of each of the six networks in the flat TD3 parameter vector."""
+    na, nc = mlp_param_count([obs, hidden, hidden, act]), mlp_param_count([obs + act, hidden, hidden, 1])
+    out, o = [], 0
+    for n in (na, na, nc, nc, nc, nc):
+        v = params[o:o + n].astype(np.float64); o += n
+        out.append((v.sum(), (v * v).sum()))
+    return np.array(out)
+
+
+def td3_golden():
+    """The committed TD3 vectors (tests/golden/make_td3_golden.py) as (dims, hyperparameters for Td3OnBackend, the npz)."""
+    g = np.load(os.path.join(GOLDEN, "td3_pendulum_seed7.npz"))
+    hp = g["hyperparameters"]
+    hyper = dict(gamma=float(hp[0]), actor_polyak=float(hp[1]), critic_polyak=float(hp[2]), sampling_std=float(hp[10]),
+                 adam=capi.adam_parameters(alpha=float(hp[5]), beta_1=float(hp[6]), beta_2=float(hp[7]), epsilon=float(hp[8]), epsilon_sqrt=float(hp[9])))
+    return [int(v) for v in g["dims"]], hyper, g
+
+
+def td3_golden_step(agent, g, i):
+    agent.set_batch(g[f"s{i}_oab"], g[f"s{i}_rewards"], g[f"s{i}_terminated"], g[f"s{i}_target_noise"])
+    agent.loop_step([int(f) for f in g[f"s{i}_flags"]], g[f"s{i}_noise_critic_0"], g[f"s{i}_noise_critic_1"], g[f"s{i}_noise_actor"])

@@ -100,3 +100,82 @@ def test_gru_reproduces_reference_vectors(oracle, case):
     got = g.results()
     for k in want:
         assert np.array_equal(got[k], want[k]), k
+
+
+def test_td3_reproduces_reference_vectors(oracle):
+    """36 loop steps of the reference's TD3-on-Pendulum run (both critic updates every step; critic targets, the delayed actor update and
+    the actor target every second step), from the reference's parameters, batches and noise draws: bit-exact digests of all six
+    networks after every step, all parameters after steps 1 and 35, the Adam ages at the end; the smoothing noise from its N(0,1) draws."""
+    (batch, hidden, steps), hyper, g = helpers.td3_golden()
+    agent = helpers.Td3OnBackend(oracle, batch, hidden, g["parameters_before"], hyper=hyper)
+    blocked = 0
+    for i in range(steps):
+        z, out = oracle.array(g[f"s{i}_target_noise_z"]), oracle.zeros((batch, 1))
+        oracle.call("td3_target_action_noise", z.ptr, float(g["hyperparameters"][3]), float(g["hyperparameters"][4]), out.ptr, batch)
+        assert np.array_equal(out.numpy(), g[f"s{i}_target_noise"])
+        helpers.td3_golden_step(agent, g, i)
+        assert np.array_equal(helpers.td3_digest(agent.parameters(), hidden), g[f"s{i}_digest"]), i
+        if f"s{i}_after" in g:
+            assert np.array_equal(agent.parameters(), g[f"s{i}_after"]), i
+        if g[f"s{i}_flags"][2]:
+            blocked += int((np.abs(agent.pre_clip.numpy()) > 1).sum())
+    assert np.array_equal(agent.ages(), g["ages_after"])
+    assert blocked >= 1           # the sampling layer's backward pass blocked at least one gradient on the way
+
+
+def test_td3_operations_closed_forms(oracle):
+    """Each elementwise TD3 operation against its definition written independently in numpy (float32 arithmetic)."""
+    rng = np.random.default_rng(3)
+    B, A = 37, 3
+    f32 = np.float32
+    mean = rng.uniform(-1.2, 1.2, (B, A)).astype(f32); noise = rng.standard_normal((B, A)).astype(f32); std = f32(0.3)
+    m, n, pc, out = oracle.array(mean), oracle.array(noise), oracle.zeros((B, A)), oracle.zeros((B, A))
+    oracle.call("td3_sampling_forward", m.ptr, A, n.ptr, A, float(std), pc.ptr, A, out.ptr, A, B, A)
+    sample = mean + noise * std
+    assert np.array_equal(pc.numpy(), sample) and np.array_equal(out.numpy(), np.clip(sample, -1, 1))
+    assert (np.abs(sample) > 1).sum() > 5
+    oracle.call("td3_sampling_forward", m.ptr, A, None, 0, float(std), None, 0, out.ptr, A, B, A)     # evaluation mode: no noise
+    assert np.array_equal(out.numpy(), np.clip(mean, -1, 1))
+    # backward: derivative of clip(x, -1, 1), by central differences of the forward pass on samples away from the kinks
+    dy = rng.standard_normal((B, A)).astype(f32)
+    d, dx = oracle.array(dy), oracle.zeros((B, A))
+    oracle.call("td3_sampling_backward", pc.ptr, A, d.ptr, A, dx.ptr, A, B, A)
+    h = 1e-3
+    numeric = (np.clip(sample.astype(np.float64) + h, -1, 1) - np.clip(sample.astype(np.float64) - h, -1, 1)) / (2 * h) * dy
+    away = np.abs(np.abs(sample) - 1) > 2 * h
+    assert np.allclose(dx.numpy()[away], numeric[away], atol=1e-6) and away.sum() > B * A - 6
+    # noisy next actions, target values
+    a = rng.uniform(-1, 1, (B, A)).astype(f32); tn = np.clip(rng.standard_normal((B, A)) * 0.2, -0.5, 0.5).astype(f32)
+    aa, tt = oracle.array(a), oracle.array(tn)
+    oracle.call("td3_noisy_next_actions", aa.ptr, A, tt.ptr, A, B, A)
+    assert np.array_equal(aa.numpy(), np.clip(a + tn, -1, 1))
+    q1, q2, r = (rng.standard_normal(B).astype(f32) for _ in range(3)); term = (rng.random(B) < 0.4).astype(np.uint8)
+    gamma = f32(0.97)
+    for ignore in (0, 1):
+        a1, a2, ar, at, y = oracle.array(q1), oracle.array(q2), oracle.array(r), oracle.array(term), oracle.zeros((B,))
+        oracle.call("td3_target_action_values", a1.ptr, a2.ptr, ar.ptr, at.ptr, float(gamma), ignore, y.ptr, B)
+        keep = np.ones(B, bool) if ignore else term == 0
+        assert np.array_equal(y.numpy(), r + np.where(keep, gamma * np.minimum(q1, q2), f32(0)))
+
+
+def test_td3_masks_equal_training_on_the_unmasked_rows(oracle):
+    """With a final-step mask, the critic and actor updates must equal (to rounding) the same updates on a batch that holds only the
+    unmasked rows: the loss weight batch/n turns the mean over the batch into the mean over the n final steps."""
+    (batch, hidden, _), hyper, g = helpers.td3_golden()
+    rng = np.random.default_rng(5)
+    keep = rng.random(batch) < 0.6; keep[:2] = [True, False]
+    idx = np.nonzero(keep)[0]; n = idx.size
+    noises = [rng.standard_normal((batch, 1)).astype(np.float32) for _ in range(3)]
+    full = helpers.Td3OnBackend(oracle, batch, hidden, g["parameters_before"], hyper=hyper, masks=True)
+    full.m_final.upload(keep.astype(np.uint8))
+    full.set_batch(g["s0_oab"], g["s0_rewards"], g["s0_terminated"], g["s0_target_noise"])
+    full.loop_step([1, 1, 1, 1], *noises)
+    sub = helpers.Td3OnBackend(oracle, n, hidden, g["parameters_before"], hyper=hyper)
+    sub.set_batch(g["s0_oab"][:, idx], g["s0_rewards"][idx], g["s0_terminated"][idx], g["s0_target_noise"][idx])
+    sub.loop_step([1, 1, 1, 1], *[z[idx] for z in noises])
+    assert helpers.rel_err(full.parameters(), sub.parameters()) < 2e-6
+    # a clear next-step mask keeps the stored next action in the target critics' input
+    full.m_next_final.upload(np.zeros(batch, np.uint8))
+    noise = oracle.array(noises[0])
+    oracle.call("td3_train_critic", C.byref(full.c), 0, noise.ptr)
+    assert np.array_equal(full.nsavi.numpy(), g["s0_oab"][1])

@@ -175,3 +175,39 @@ def test_gru_forward_and_backward_through_time_bit_exact_with_reference(oracle, 
         assert reset[1:].sum() > 3
     for k in want:
         assert np.array_equal(got[k], want[k]), (k, np.abs(got[k] - want[k]).max())
+
+
+@pytest.mark.skipif(not os.path.exists(helpers.REF_TD3_GENERIC), reason="oracle/_ref TD3 harness not built (needs /root/reference)")
+def test_td3_updates_bit_exact_with_reference(oracle):
+    """The reference's own TD3-on-Pendulum loop. Two copies with one seed: one advanced by the reference's step(), one by the same
+    operations called one by one (so that the sampling-layer draws can be written out) -- they must agree, which ties what follows to
+    step() itself. From the first training step on, the restatement gets the reference's batch, smoothing noise and sampling draws
+    and must reproduce every parameter (actor, target actor, critics, target critics) and Adam age, bit for bit, over 100 loop steps
+    (50 delayed actor updates, some with samples outside [-1, 1], where the sampling layer's backward pass blocks the gradient). The smoothing noise itself is restated from the N(0,1) draws behind it."""
+    a, b = helpers.RefTd3(7), helpers.RefTd3(7)
+    assert (b.batch, b.actor_interval, b.critic_target_interval, b.actor_target_interval) == (100, 2, 2, 2)
+    for _ in range(b.n_warmup):
+        a.step(); b.step()
+    agent = helpers.Td3OnBackend(oracle, b.batch, b.hidden, b.parameters(), hyper=b.hyper())
+    actor_updates = clipped = blocked = 0
+    for i in range(100):
+        a.step()
+        z, c0, c1, na, flags = b.manual_step()
+        assert np.array_equal(a.parameters(), b.parameters())
+        assert flags[0] == 1 and flags[2] == flags[1] == flags[3] == (1 if i % 2 == 0 else 0)
+        oab, r, t, fm, nfm = b.batch_data()
+        assert fm.all() and nfm[b.batch:].all()          # SEQUENCE_LENGTH = 1: every step is a final step
+        noise = b.target_noise()
+        zd, out = oracle.array(z), oracle.zeros((b.batch, 1))
+        oracle.call("td3_target_action_noise", zd.ptr, float(b.hp[3]), float(b.hp[4]), out.ptr, b.batch)
+        assert np.array_equal(out.numpy(), noise)
+        clipped += int((np.abs(noise) == np.float32(0.5)).sum())
+        agent.set_batch(oab, r, t, noise)
+        agent.loop_step(flags, c0, c1, na)
+        actor_updates += flags[2]
+        blocked += int((np.abs(agent.pre_clip.numpy()) > 1).sum()) if flags[2] else 0
+        got, want = agent.parameters(), b.parameters()
+        assert np.array_equal(got, want), (i, np.abs(got - want).max())
+        assert np.array_equal(agent.ages(), b.ages())
+    assert actor_updates == 50 and clipped >= 3 and blocked >= 3          # the clip at 2.5 standard deviations was exercised
+    a.close(); b.close()

@@ -1,0 +1,132 @@
+"""TD3 on the HIP path through the C ABI against the CPU checker: the elementwise operations bit for bit, the critic / delayed actor /
+target updates in lock step with the checker on the batches and noise draws of the reference's own run (tests/golden), and one update
+at a wider shape with masks. fp32 tolerance of the updates: 1e-5 relative to the largest parameter (the contraction order differs)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import helpers
+from helpers import rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+@pytest.mark.parametrize("B,A", [(1, 1), (100, 1), (4099, 6), (65537, 3)])
+def test_elementwise_operations_bit_exact(oracle, rocm, B, A):
+    print("case", B, A, flush=True)
+    rng = np.random.default_rng(B + A)
+    f32 = np.float32
+    mean = rng.uniform(-1.2, 1.2, (B, A)).astype(f32); noise = rng.standard_normal((B, A)).astype(f32); dy = rng.standard_normal((B, A)).astype(f32)
+    z = rng.standard_normal((B, A)).astype(f32); act = rng.uniform(-1, 1, (B, A)).astype(f32)
+    q1, q2, r = (rng.standard_normal(B).astype(f32) for _ in range(3)); term = (rng.random(B) < 0.4).astype(np.uint8)
+    res = {}
+    for b in (oracle, rocm):
+        m, n, d = b.array(mean), b.array(noise), b.array(dy)
+        pc, out, out_eval, dx = b.zeros((B, A)), b.zeros((B, A)), b.zeros((B, A)), b.zeros((B, A))
+        b.call("td3_sampling_forward", m.ptr, A, n.ptr, A, 0.3, pc.ptr, A, out.ptr, A, B, A)
+        b.call("td3_sampling_forward", m.ptr, A, None, 0, 0.3, None, 0, out_eval.ptr, A, B, A)
+        b.call("td3_sampling_backward", pc.ptr, A, d.ptr, A, dx.ptr, A, B, A)
+        zz, tn = b.array(z), b.zeros((B, A))
+        b.call("td3_target_action_noise", zz.ptr, 0.2, 0.5, tn.ptr, B * A)
+        aa = b.array(act)
+        b.call("td3_noisy_next_actions", aa.ptr, A, tn.ptr, A, B, A)
+        a1, a2, ar, at, y, y_ignore = b.array(q1), b.array(q2), b.array(r), b.array(term), b.zeros((B,)), b.zeros((B,))
+        b.call("td3_target_action_values", a1.ptr, a2.ptr, ar.ptr, at.ptr, 0.99, 0, y.ptr, B)
+        b.call("td3_target_action_values", a1.ptr, a2.ptr, ar.ptr, at.ptr, 0.99, 1, y_ignore.ptr, B)
+        b.sync()
+        res[b.name] = dict(pre_clip=pc.numpy(), out=out.numpy(), out_eval=out_eval.numpy(), dx=dx.numpy(), target_noise=tn.numpy(), noisy=aa.numpy(),
+                           y=y.numpy(), y_ignore=y_ignore.numpy())
+    for k, want in res["oracle"].items():
+        assert np.array_equal(res["rocm"][k], want), k
+
+
+def test_lock_step_with_the_checker_on_the_references_run(oracle, rocm):
+    """The 36 loop steps of the committed reference run (72 critic updates, 18 delayed actor updates, 18 target updates of each kind).
+    Before every step the HIP side gets the checker's exact state; both run the step on the reference's batch and draws; updated
+    parameters of all six networks agree to 1e-5 of the largest parameter, gradients to 1e-5 of the largest gradient component times
+    kappa = max|y| / max|Q - y| (rounding of Q is amplified by that factor in the TD error for any fp32 implementation)."""
+    (batch, hidden, steps), hyper, g = helpers.td3_golden()
+    ref = helpers.Td3OnBackend(oracle, batch, hidden, g["parameters_before"], hyper=hyper)
+    dev = helpers.Td3OnBackend(rocm, batch, hidden, g["parameters_before"], hyper=hyper)
+    worst_p = worst_g = 0.0
+    for i in range(steps):
+        dev.push(ref.state())
+        helpers.td3_golden_step(ref, g, i)
+        helpers.td3_golden_step(dev, g, i)
+        pe = rel_err(dev.parameters(), ref.parameters())
+        y, td = ref.target_q.numpy(), ref.d_out_c.numpy() * batch / 2
+        kappa = max(1.0, np.abs(y).max() / max(np.abs(td).max(), 1e-30))
+        ge = rel_err(dev.gradients(), ref.gradients()) / kappa
+        assert np.array_equal(dev.ages(), ref.ages())
+        assert rel_err(dev.target_q.numpy(), y) <= TOL and rel_err(dev.nsavi.numpy(), ref.nsavi.numpy()) <= TOL
+        worst_p, worst_g = max(worst_p, pe), max(worst_g, ge)
+        if i % 6 == 0:
+            print(f"step {i}: parameters {pe:.2e} gradients/kappa {ge:.2e} kappa {kappa:.1f}", flush=True)
+        assert pe <= TOL and ge <= TOL, (i, pe, ge)
+    # the checker itself reproduced the reference's parameters bit for bit on the way (the CPU suite asserts the same)
+    assert np.array_equal(ref.parameters(), g[f"s{steps - 1}_after"])
+    print("worst: parameters %.2e gradients %.2e" % (worst_p, worst_g))
+
+
+def test_free_running_first_updates_match_the_reference_vectors(rocm):
+    """No checker in the loop: the HIP side alone, from the reference's initial parameters, over the first two loop steps (4 critic
+    updates, 1 actor update, both target updates) against the parameters the reference itself had after them."""
+    (batch, hidden, _), hyper, g = helpers.td3_golden()
+    dev = helpers.Td3OnBackend(rocm, batch, hidden, g["parameters_before"], hyper=hyper)
+    for i in range(2):
+        helpers.td3_golden_step(dev, g, i)
+    assert rel_err(dev.parameters(), g["s1_after"]) <= TOL
+    assert np.array_equal(helpers.td3_digest(dev.parameters(), hidden) != 0, np.ones((6, 2), bool))
+
+
+@pytest.mark.parametrize("batch,hidden,obs,act,masks", [(256, 64, 3, 1, True), (1000, 256, 17, 6, True), (4096, 256, 17, 6, False)])
+def test_one_update_at_other_shapes_with_masks(oracle, rocm, batch, hidden, obs, act, masks):
+    """A full loop step (both critics, targets, actor, actor target) on random data at shapes beyond the Pendulum example, with final-step
+    and next-final-step masks that clear a third of the rows, terminated flags, and samples outside [-1, 1]."""
+    print("case", batch, hidden, obs, act, masks, flush=True)
+    rng = np.random.default_rng(batch + act)
+    D = obs + act
+    adims, cdims = [obs, hidden, hidden, act], [D, hidden, hidden, 1]
+    nets = [helpers.random_params(rng, adims)] * 2 + [helpers.random_params(rng, cdims) for _ in range(2)]
+    params = np.concatenate(nets + [nets[2] * 0.9, nets[3] * 1.1]).astype(np.float32)
+    oab = rng.standard_normal((2, batch, D)).astype(np.float32); oab[:, :, obs:] = np.clip(oab[:, :, obs:], -1, 1)
+    rewards = rng.standard_normal(batch).astype(np.float32); term = (rng.random(batch) < 0.2).astype(np.uint8)
+    tn = np.clip(rng.standard_normal((batch, act)) * 0.2, -0.5, 0.5).astype(np.float32)
+    noises = [rng.standard_normal((batch, act)).astype(np.float32) for _ in range(3)]
+    hyper = dict(gamma=0.99, actor_polyak=0.995, critic_polyak=0.99, sampling_std=0.5, adam=helpers.capi.adam_parameters(epsilon=1e-7))
+    out = {}
+    for b in (oracle, rocm):
+        ag = helpers.Td3OnBackend(b, batch, hidden, params, hyper=hyper, masks=masks, obs=obs, act=act)
+        if masks:
+            ag.m_final.upload((rng.random(batch) < 0.67).astype(np.uint8) if b is oracle else out["oracle"]["m_final"])
+            ag.m_next_final.upload((rng.random(batch) < 0.67).astype(np.uint8) if b is oracle else out["oracle"]["m_next"])
+        ag.set_batch(oab, rewards, term, tn)
+        ag.loop_step([1, 1, 1, 1], *noises)
+        out[b.name] = dict(params=ag.parameters(), grads=ag.gradients(), nsavi=ag.nsavi.numpy(), savi=ag.savi.numpy(), y=ag.target_q.numpy(), d_c=ag.d_out_c.numpy(),
+                           d_a=ag.d_out_a.numpy(), d_ci=ag.d_ci.numpy(), d_ao=ag.d_ao.numpy(), pre_clip=ag.pre_clip.numpy(), m_final=ag.m_final.numpy(), m_next=ag.m_next_final.numpy(),
+                           critic_pre=np.concatenate([ag.critics[0].pre[0].numpy(), ag.critics[0].pre[1].numpy()], axis=1))
+    want, got = out["oracle"], out["rocm"]
+    assert (np.abs(want["pre_clip"]) > 1).sum() > batch * act // 20
+    for k in ("nsavi", "savi", "y", "d_c", "d_a", "pre_clip"):
+        e = rel_err(got[k], want[k])
+        print(k, "%.2e" % e, flush=True)
+        assert e <= TOL, (k, e)
+    # The gradient that reaches the actor passes through critic 0's ReLUs. A pre-activation within rounding of zero may switch on one
+    # side only, which changes that row's input gradient by O(1): such rows are allowed if the checker's pre-activation shows the
+    # near-zero unit, and the quantities summed over the batch are then compared with that many rows' worth of slack.
+    scale = np.abs(want["d_ci"]).max()
+    row_err = np.abs(got["d_ci"] - want["d_ci"]).max(axis=1) / scale
+    bad = np.nonzero(row_err > TOL)[0]
+    print("rows of d_critic_input beyond tolerance:", bad.size, flush=True)
+    assert bad.size <= 3
+    for r in bad:
+        assert np.abs(want["critic_pre"][r]).min() <= 1e-5 * np.abs(want["critic_pre"]).max(), (r, row_err[r])
+    ok = np.ones(batch, bool); ok[bad] = False
+    assert rel_err(got["d_ci"][ok], want["d_ci"][ok]) <= TOL and rel_err(got["d_ao"][ok], want["d_ao"][ok]) <= TOL
+    slack = TOL + 2.0 * bad.size / batch
+    for k in ("grads", "params"):
+        e = rel_err(got[k], want[k])
+        print(k, "%.2e" % e, flush=True)
+        assert e <= slack, (k, e)
