@@ -135,6 +135,97 @@ def bench_env(helpers, rocm, n_envs=65536, capacity=16, steps=200, batch=4096):
             "algorithmic_GBps": env_steps * 68 / (ms * 1e-3) / 1e9, "gather_batch": batch, "gather_us": gather_us, "gather_algorithmic_GBps": batch * 85 / (gather_us * 1e-6) / 1e9}
 
 
+def bench_ppo(helpers, rocm, n_envs=4096, steps=128, epochs=4, minibatch=8192):
+    """Synthetic PPO iteration: GAE over a (steps+1) x n_envs dataset, then epochs x (rows / minibatch) minibatch updates of an actor
+    105-64-64-8 (tanh, learned log_std) and a critic 105-64-64-1 (tanh) on host-drawn row permutations."""
+    capi = helpers.capi
+    O, A, H = 105, 8, 64
+    rows = n_envs * steps
+    rng = np.random.default_rng(3)
+    col = dict(observations=0, actions=O, action_log_probs=O + A, rewards=O + A + 1, terminated=O + A + 2, truncated=O + A + 3, all_values=O + A + 4,
+               advantages=O + A + 5, target_values=O + A + 6)
+    ld = O + A + 7
+    data = rng.standard_normal((rows + n_envs, ld)).astype(np.float32)
+    done = (rng.random(rows + n_envs) < 0.01).astype(np.float32)
+    data[:, col["terminated"]] = done; data[:, col["truncated"]] = done
+    data[:, col["action_log_probs"]] = (-0.9189385 - np.log(0.5) - 0.5 * (data[:, O:O + A] / 0.5) ** 2).sum(1)
+    params = np.concatenate([helpers.random_params(rng, [O, H, H, A]) * 0.1, np.log(np.full(A, 0.5, np.float32)), helpers.random_params(rng, [O, H, H, 1])]).astype(np.float32)
+    agent = helpers.PpoOnBackend(rocm, O, A, H, H, minibatch, params, "tanh", "tanh", capi.adam_parameters(3e-4, epsilon=1e-8))
+    pp = capi.ppo_parameters()
+    dd = rocm.array(data)
+    perms = [rocm.array(rng.permutation(rows).astype(np.uint32)) for _ in range(epochs)]
+    ev = HipEvents(rocm.device.lib.rlt_rocm_get_stream(rocm.device.handle))
+
+    def gae():
+        rocm.call("ppo_gae", dd.offset(col["rewards"]), dd.offset(col["terminated"]), dd.offset(col["truncated"]), dd.offset(col["all_values"]),
+                  dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld, n_envs, steps, 0.99, 0.95, 0)
+
+    def iteration():
+        for perm in perms:
+            for b in range(rows // minibatch):
+                rocm.call("ppo_train_minibatch", C.byref(agent.c), C.byref(pp), dd.offset(col["observations"]), dd.offset(col["observations"]), dd.offset(col["actions"]),
+                          dd.offset(col["action_log_probs"]), dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld, perm.offset(b * minibatch), None)
+    for _ in range(3):
+        gae()
+    rocm.sync()
+    a = ev.record()
+    for _ in range(20):
+        gae()
+    e = ev.record()
+    gae_us = ev.elapsed_ms(a, e) * 1e3 / 20
+    iteration(); rocm.sync()
+    a = ev.record(); iteration(); e = ev.record()
+    ms = ev.elapsed_ms(a, e)
+    n_updates = epochs * (rows // minibatch)
+    flop = 106368.0 * rows * epochs
+    return {"rows": rows, "minibatch": minibatch, "epochs": epochs, "gae_us": gae_us, "gae_algorithmic_GBps": rows * 24 / (gae_us * 1e-6) / 1e9,
+            "iteration_ms": ms, "us_per_minibatch_update": ms * 1e3 / n_updates, "samples_per_s": rows * epochs / (ms * 1e-3), "tflops": flop / (ms * 1e-3) / 1e12}
+
+
+def bench_gru(helpers, rocm, batch, S=64, I=146, H=64, iters=10):
+    """Sequence model step: GRU 146->64 over 64 steps, head 64->64 (tanh) ->4, MSE loss, backward through time, Adam on everything."""
+    capi = helpers.capi
+    rng = np.random.default_rng(4)
+    params, x, _, _ = helpers.gru_random_case(rng, S, batch, I, H, False)
+    params["h0"] = np.zeros(H, np.float32)
+    gru = helpers.GruOnBackend(rocm, S, batch, I, H, params)
+    rows = S * batch
+    head = helpers.Mlp(rocm, [H, 64, 4], helpers.xavier_params(rng, [H, 64, 4]), rows, "tanh", "identity")
+    target = rocm.array(rng.standard_normal((rows, 4)).astype(np.float32))
+    d_out, d_h = rocm.zeros((rows, 4)), rocm.zeros((S, batch, H))
+    xd = rocm.array(x)
+    moments = [rocm.zeros(a.shape) for a in (gru.W_i, gru.b_i, gru.W_h, gru.b_h) for _ in range(2)]
+    tensors = []
+    for k, (p, g, flag) in enumerate(((gru.W_i, gru.dW_i, 1), (gru.b_i, gru.db_i, 2), (gru.W_h, gru.dW_h, 1), (gru.b_h, gru.db_h, 2))):
+        tensors.append(capi.AdamTensor(p.ptr, g.ptr, moments[2 * k].ptr, moments[2 * k + 1].ptr, None, int(np.prod(p.shape)), flag))
+    gru_adam = (capi.AdamTensor * 4)(*tensors)
+    age = rocm.array(np.array([1], np.uint32))
+    adam = capi.adam_parameters(epsilon=1e-8)
+    ws, wsn = head.workspace()
+    ev = HipEvents(rocm.device.lib.rlt_rocm_get_stream(rocm.device.handle))
+
+    def step():
+        for g in (gru.dW_i, gru.db_i, gru.dW_h, gru.db_h):
+            rocm.call("fill_f32", g.ptr, 1, int(np.prod(g.shape)), int(np.prod(g.shape)), 0.0)
+        rocm.call("mlp_zero_gradient", head.layers, head.n)
+        rocm.call("gru_forward", C.byref(gru.c), xd.ptr, None, S, batch, gru.ws, gru.wsn)
+        rocm.call("mlp_forward", head.layers, head.n, gru.out.ptr, H, rows)
+        rocm.call("mse_gradient", head.out[-1].ptr, 4, target.ptr, 4, d_out.ptr, 4, rows, 4, 1.0, None)
+        rocm.call("mlp_backward", head.layers, head.n, gru.out.ptr, H, d_out.ptr, 4, d_h.ptr, H, rows, 1, ws, wsn)
+        rocm.call("gru_backward", C.byref(gru.c), xd.ptr, d_h.ptr, None, None, S, batch, 1, gru.ws, gru.wsn)
+        rocm.call("adam_step", gru_adam, 4, C.byref(adam), age.ptr, 0.0, None)
+        rocm.call("adam_step", head.adam, head.n_adam, C.byref(adam), head.age.ptr, 0.0, None)
+    for _ in range(3):
+        step()
+    rocm.sync()
+    a = ev.record()
+    for _ in range(iters):
+        step()
+    e = ev.record()
+    ms = ev.elapsed_ms(a, e) / iters
+    return {"batch": batch, "sequence_length": S, "ms_per_step": ms, "sequences_per_s": batch / (ms * 1e-3), "tflops": 211968.0 * rows / (ms * 1e-3) / 1e12}
+
+
 def pmc_probe(helpers, rocm, batch):
     n = 64 * 1024 * 1024      # floats: 256 MiB read + 256 MiB written per copy
     src, dst = rocm.zeros((n,)), rocm.zeros((n,))
@@ -218,7 +309,8 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_opera
         rocm.sync()
         dt = time.perf_counter() - t0
         if phase_profile:
-            names = ["env step", "critic phase: TD error + both backward passes", "barrier", "critic Adam", "barrier", "critic weight refresh", "actor phase", "barrier", "actor Adam", "barrier", "actor weight refresh"]
+            names = ["env step", "critic phase: TD error + both backward passes", "announce critic gradients", "wait + critic Adam", "announce + wait for critic parameters", "critic weight refresh",
+                     "actor phase", "announce + wait for actor gradients", "actor Adam", "announce + wait for actor parameters", "actor weight refresh"]
             names += ["critic phase: batch rows into LDS", "critic phase: actor on next obs | critic 1 forward", "critic phase: target critics", "critic phase: critic 0 forward", "unused"]
             tk = ticks.numpy()[:16].astype(np.float64) / 100.0 / steps      # 100 MHz constant clock -> microseconds per step
             shader_cycles = tk[15] * 100.0; tk = tk[:15]; names = names[:15]
@@ -276,7 +368,7 @@ def main():
     ap.add_argument("--mlp-batch", type=int, default=65536)
     ap.add_argument("--mlp-iters", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "mlp", "sac", "env"], default="all")
+    ap.add_argument("--only", choices=["all", "mlp", "sac", "env", "ppo", "gru"], default="all")
     ap.add_argument("--sac-phase-profile", action="store_true", help="print the persistent kernel's per-phase time (stderr)")
     ap.add_argument("--pmc-probe", action="store_true", help="for counter runs under rocprofv3 --pmc: three 256 MiB device copies (a kernel of known traffic, to scale the counters by) "
                     "and three MLP forward+backward calls, nothing timed")
@@ -297,7 +389,9 @@ def main():
     mlp = bench_mlp(helpers, rocm, args.mlp_batch, args.mlp_iters, 3) if args.only in ("all", "mlp") else None
     sac = bench_sac(helpers, rocm, args.steps, args.warmup, per_operation=args.sac_per_operation, phase_profile=args.sac_phase_profile) if args.only in ("all", "sac") else {"steps_per_s": 0.0, "ms_per_step": 0.0}
     env = bench_env(helpers, rocm) if args.only in ("all", "env") else None
-    cpu = None if (args.no_cpu_baseline or args.only in ("mlp", "env")) else cpu_baseline()
+    ppo = bench_ppo(helpers, rocm) if args.only in ("all", "ppo") else None
+    gru = [bench_gru(helpers, rocm, b) for b in (64, 1024)] if args.only in ("all", "gru") else None
+    cpu = None if (args.no_cpu_baseline or args.only in ("mlp", "env", "ppo", "gru")) else cpu_baseline()
     line = {
         "metric": "SAC updates/sec (critic+actor) at batch 256; fused MLP fwd+bwd TFLOP/s",
         "value": sac["steps_per_s"], "unit": "SAC loop steps/s (each = 2 critic + 1 actor update)",
@@ -316,6 +410,10 @@ def main():
                             "kernel": "mlp_forward_backward call = mlp3_prepare_kernel + mlp3_fused_kernel + mlp3_reduce_kernel", "flop_per_launch": flop}
     if env:
         line["env_pipeline"] = env
+    if ppo:
+        line["ppo_iteration"] = ppo
+    if gru:
+        line["gru_training_step"] = gru
     if cpu:
         line["cpu_baseline"] = cpu
         line["speedup_vs_cpu_baseline"] = sac["steps_per_s"] / cpu["value"] if cpu["value"] else None

@@ -31,6 +31,7 @@ extern "C" {
 #define RLT_E_INVALID_ARGUMENT (-1) /* null pointer, non-positive dimension, ld too small */
 #define RLT_E_UNSUPPORTED      (-2) /* shape outside what the kernels are built for      */
 #define RLT_E_NOT_INITIALISED  (-3)
+#define RLT_E_DEVICE_TIMEOUT   (-4) /* a persistent kernel gave up waiting for another workgroup (reported by check_status) */
 
 /* nn/activation_functions.h:11-18 -- same numbering as the reference enum */
 enum rlt_activation {

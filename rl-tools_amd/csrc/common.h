@@ -15,6 +15,9 @@ struct rlt_rocm_device {
     void* scratch;               // grow-only device workspace for split reductions and partial sums
     size_t scratch_bytes;
     void* counters;              // 8 KiB, zero between launches: [0,256) ticket counters, [256,..) per-workgroup partial sums
+    unsigned* fault;             // [0]: set by a persistent kernel that gave up waiting for another workgroup; read back by check_status
+    int fault_armed;             // a kernel that can set it was launched since the last check
+    int xcd_stride;              // workgroups b and b + xcd_stride run on the same XCD (0: not established; consecutive workgroups go round the XCDs)
     int sticky_error;
 };
 

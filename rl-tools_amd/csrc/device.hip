@@ -94,6 +94,11 @@ __global__ __launch_bounds__(1024) void reduce_kernel(const void* __restrict__ s
     if (threadIdx.x == 0) { float s = 0.0f; for (int i = 0; i < 16; i++) s += partial[i]; *out = s; }
 }
 
+// which XCD every workgroup of a launch lands on (bits 3:0 of the XCC_ID hardware register)
+__global__ __launch_bounds__(64) void xcd_probe_kernel(unsigned* __restrict__ out) {
+    if (threadIdx.x == 0) out[blockIdx.x] = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 0xf;
+}
+
 int grid_for(size_t n) { size_t b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : (b < 1 ? 1 : b)); }
 
 }  // namespace
@@ -120,6 +125,25 @@ int rlt_rocm_init(int hip_device_index, rlt_rocm_device** out_device) {
     e = hipMalloc(&device->counters, 8192);
     if (e == hipSuccess) e = hipMemset(device->counters, 0, 8192);
     if (e != hipSuccess) { (void)hipStreamDestroy(device->own_stream); delete device; return (int)e; }
+    device->fault = (unsigned*)((char*)device->counters + 8192 - 64);   // the last 64 bytes of the block are never used as counters
+    // Dispatch order over the XCDs: probe twice with 64 workgroups; if workgroup b always shares its XCD with b + 8 (and with no
+    // workgroup in between), persistent kernels may place a small grid on one XCD by using every 8th workgroup of a larger one.
+    {
+        unsigned* probe = (unsigned*)((char*)device->counters + 4096);
+        unsigned host[64];
+        bool ok = true;
+        for (int rep = 0; rep < 2 && ok; rep++) {
+            hipLaunchKernelGGL(xcd_probe_kernel, dim3(64), dim3(64), 0, device->stream, probe);
+            ok = hipMemcpyAsync(host, probe, sizeof host, hipMemcpyDeviceToHost, device->stream) == hipSuccess && hipStreamSynchronize(device->stream) == hipSuccess;
+            for (int b = 0; b < 64 && ok; b++) {
+                if (b >= 8 && host[b] != host[b - 8]) ok = false;
+                for (int k = 1; k < 8 && b >= k && ok; k++) if (host[b] == host[b - k]) ok = false;
+            }
+        }
+        (void)hipMemsetAsync(probe, 0, sizeof host, device->stream);
+        (void)hipStreamSynchronize(device->stream);
+        device->xcd_stride = ok ? 8 : 0;
+    }
     *out_device = device;
     return 0;
 }
@@ -136,6 +160,14 @@ int rlt_rocm_check_status(rlt_rocm_device* device) {
     if (!device) return RLT_E_NOT_INITIALISED;
     hipError_t e = hipStreamSynchronize(device->stream);
     if (e != hipSuccess) device->sticky_error = (int)e;
+    if (device->fault_armed && e == hipSuccess) {
+        unsigned fault = 0;
+        device->fault_armed = 0;
+        if (hipMemcpy(&fault, device->fault, sizeof fault, hipMemcpyDeviceToHost) == hipSuccess && fault) {
+            (void)hipMemset(device->fault, 0, sizeof fault);
+            if (!device->sticky_error) device->sticky_error = RLT_E_DEVICE_TIMEOUT;
+        }
+    }
     int s = device->sticky_error;
     return s;
 }
@@ -149,6 +181,7 @@ const char* rlt_rocm_error_string(int code) {
     if (code == 0) return "success";
     if (code == RLT_E_INVALID_ARGUMENT) return "rlt_rocm: invalid argument (null pointer, non-positive dimension or too small leading dimension)";
     if (code == RLT_E_UNSUPPORTED) return "rlt_rocm: shape outside what the kernels support";
+    if (code == RLT_E_DEVICE_TIMEOUT) return "rlt_rocm: a persistent kernel gave up waiting for another workgroup; its results are invalid";
     if (code == RLT_E_NOT_INITIALISED) return "rlt_rocm: device handle not initialised";
     if (code > 0) return hipGetErrorString((hipError_t)code);
     return "rlt_rocm: unknown error";

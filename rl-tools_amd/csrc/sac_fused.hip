@@ -16,16 +16,30 @@
 //       ring. The replay rows of this step's batch were requested from memory before S0 and arrive while it runs.
 //   S1  next actions + log-probabilities from the actor; both target critics; TD target; both critics forward + backward
 //       -> per-workgroup partial gradients
-//   --- grid barrier ---
-//   S2  each workgroup sums a slice of the partial gradients (fixed order), applies Adam and the polyak target update
-//   --- grid barrier ---   (then every workgroup reloads the critics and targets into LDS)
+//   S2  each workgroup sums a slice of the partial gradients (fixed order), applies Adam and the polyak target update;
+//       then every workgroup reloads the critics and targets into LDS
 //   S3  actor forward, both critics forward / backward_input, min-Q routing, sample_and_squash backward, actor backward
 //       -> partial gradients
-//   --- grid barrier ---
-//   S4  Adam on the actor slice and on log_alpha
-//   --- grid barrier ---   (then every workgroup reloads the actor)
+//   S4  Adam on the actor slice and on log_alpha; then every workgroup reloads the actor
 // Two wave groups of four wavefronts each work on independent networks (critic 0 / critic 1) at the same time.
+//
+// The workgroups exchange partial gradients (S1 -> S2, S3 -> S4) and updated parameters (S2 -> S3, S4 -> next step) through
+// memory with one word per workgroup and exchange instead of grid barriers with agent-scope release / acquire (which write back
+// and invalidate the whole L2 of the XCD and cost 3.2 us one way for 8 KB between two CUs, against 1.6 us for this): a
+// workgroup waits until its own stores have completed (s_waitcnt), sets its word, and the consumers, once all words are set,
+// load the data past their CU's vector cache. Up to 32 workgroups are placed on ONE XCD (every 8th workgroup of an 8x larger
+// grid; the others exit at once): there plain stores land in the L2 that all of them share, and non-temporal loads, which
+// never allocate in the vector cache, read it. Larger grids spread over the XCDs, store through to memory and load with agent
+// scope. Any address that another workgroup may have rewritten is read in one of these two ways everywhere in the kernel.
+// No slot is overwritten before its consumer has read it: a workgroup rewrites its partial gradients of a phase only after
+// every consumer has announced the parameters it made from them, and a consumer rewrites parameters only after every workgroup
+// has announced its next partial gradients, which they write after having read the old parameters.
+// The target critics are not exchanged at all: every workgroup applies the polyak update to its own LDS copy, with the same
+// arithmetic on the same bits as the owner of the element applies to the arena in memory.
 #include "common.h"
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) float* lptr;      // LDS address (32 bit): keeps every access a ds_* instruction
@@ -42,6 +56,8 @@ constexpr int XS = 17;          // LDS row stride of network inputs
 constexpr int THREADS = 512;
 constexpr int MAX_G = 64;
 constexpr int R = 2 * OBS + ACT + 3;    // floats per replay row
+constexpr int MAX_PACKED_G = 32;        // workgroups that fit on one XCD (32 CUs) with one workgroup per CU
+constexpr unsigned MAX_POLL = 1u << 20; // bounded wait for another workgroup's data (about a second), then the run is abandoned
 
 // A 3-layer network IN -> H -> H -> OUT: offsets in its flat arena [W1|b1|W2|b2|W3|b3] and in the workgroup's LDS copy. The
 // LDS rows are padded to odd strides so that the 16 rows a tile reads side by side fall into different banks; W1 rows are
@@ -83,7 +99,9 @@ struct FusedArgs {
     rlt_pendulum_runner runner;
     rlt_replay_buffer rb;
     float* partial;            // [G + 1][N_PARTIAL], row G stays zero
-    unsigned* barrier_counter;
+    unsigned* fault;           // set when a workgroup gave up waiting
+    unsigned* xcd_mask;        // bit x set: some workgroup of this launch ran on XCD x
+    unsigned* ready;           // [4][64] per exchange kind and workgroup: the sequence number of the last completed exchange
     // optional host-drawn randomness (parity runs); NULL -> counter-based device RNG
     const float* rollout_noise; const float* initial_states; const uint32_t* sample_offsets;
     const float* noise_critic; const float* noise_actor;
@@ -106,15 +124,54 @@ __device__ __forceinline__ float row16_sum(float x) {
 // sum over the four rows of a wavefront (lanes l, l^16, l^32, l^48), result in all
 __device__ __forceinline__ float kk_sum(float x) { x += __shfl_xor(x, 16, 64); x += __shfl_xor(x, 32, 64); return x; }
 
-__device__ __forceinline__ void grid_barrier(unsigned* counter, unsigned target) {
-    __syncthreads();
+// ---- exchange between workgroups
+// loads of data that another workgroup may have rewritten: never from this CU's vector cache
+template <bool PACKED>
+__device__ __forceinline__ float get_shared(const float* p) {
+    if (PACKED) return __builtin_nontemporal_load(p);                                   // never allocates in the vector cache; reads the XCD's L2
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);            // past the vector cache, coherent across XCDs
+}
+template <bool PACKED>
+__device__ __forceinline__ void put_shared(float* p, float v) {
+    if (PACKED) *p = v;                                                                 // lands in the XCD's L2, which every consumer reads
+    else __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);          // written through to memory
+}
+// the target update, in one place so that the owner of an element and every workgroup's LDS copy compute the same bits
+__device__ __forceinline__ float polyak_step(float polyak, float target, float source) { return __builtin_fmaf(polyak, target, (1.0f - polyak) * source); }
+// after a failed wait: tell every workgroup (they look at this word while they wait) and this workgroup (it leaves the step loop)
+__device__ __forceinline__ void give_up(unsigned* fault, __attribute__((address_space(3))) int* abort_flag) {
+    __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *abort_flag = 1;
+}
+// true while waiting may go on: not too long yet, and no workgroup has given up
+__device__ __forceinline__ bool keep_waiting(unsigned& tries, const unsigned* fault) {
+    __builtin_amdgcn_s_sleep(1);      // a waiting wavefront should not keep the memory system busy
+    ++tries;
+    if (tries >= MAX_POLL) return false;
+    if ((tries & 63u) == 0u && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) return false;
+    return true;
+}
+// One word per workgroup and exchange kind holds the sequence number of the last exchange the workgroup has completed its stores
+// for. announce: wait for this wavefront's stores (and loads) to complete, meet the other wavefronts, set the word.
+constexpr int READY_STRIDE = 64;     // words per exchange kind (MAX_G)
+enum { READY_CRITIC_GRADIENTS = 0, READY_CRITIC_PARAMETERS = 1, READY_ACTOR_GRADIENTS = 2, READY_ACTOR_PARAMETERS = 3 };
+template <bool PACKED>
+__device__ __forceinline__ void announce(unsigned* ready, int kind, int g, unsigned tag) {
+    __builtin_amdgcn_s_waitcnt(0);
+    rlt_lds_barrier();
     if (threadIdx.x == 0) {
-        __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        // poll without ordering, then acquire once: an acquiring load invalidates the caches on every iteration
-        while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) __builtin_amdgcn_s_sleep(1);
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        if (PACKED) ready[kind * READY_STRIDE + g] = tag;
+        else __hip_atomic_store(ready + kind * READY_STRIDE + g, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    __syncthreads();
+}
+// wavefront 0 waits for all G words, the others wait for it at the workgroup barrier
+__device__ __forceinline__ void await(const unsigned* ready, int kind, int G, unsigned tag, const unsigned* fault, __attribute__((address_space(3))) int* abort_flag) {
+    if (threadIdx.x < 64) {
+        const unsigned* p = ready + kind * READY_STRIDE + min((int)threadIdx.x, G - 1);
+        unsigned tries = 0;
+        while (__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < tag) if (!keep_waiting(tries, fault)) { give_up(const_cast<unsigned*>(fault), abort_flag); break; }
+    }
+    rlt_lds_barrier();
 }
 
 __device__ __forceinline__ uint32_t mix32(uint64_t x) {
@@ -216,7 +273,7 @@ __device__ __forceinline__ float net_output(lptr part, lptr P, int row, int c) {
 
 // backward, layer 3 and the gate of layer 2: dp2 = (dout W3) * relu'(h2); with WANT_W also dW3, db3, db2 of the 16 rows into the
 // gradient arena Gd. dout is [ROWS][2] (gradient at the identity output).
-template <class N, bool WANT_W>
+template <class N, bool WANT_W, bool PK>
 __device__ __forceinline__ void backward_stage1(lptr h2, lptr dp2, lptr dout, const Bwd1W& f, float* __restrict__ Gd, int w, int lane) {
     const int r = lane & 15, kk = lane >> 4, n = 16 * w + r;
     float wsum[N::OUT];
@@ -236,14 +293,14 @@ __device__ __forceinline__ void backward_stage1(lptr h2, lptr dp2, lptr dout, co
     }
     if (WANT_W) {
 #pragma unroll
-        for (int c = 0; c < N::OUT; c++) { const float s = kk_sum(wsum[c]); if (kk == 0) Gd[N::w3 + c * H + n] = s; }
+        for (int c = 0; c < N::OUT; c++) { const float s = kk_sum(wsum[c]); if (kk == 0) put_shared<PK>(Gd + N::w3 + c * H + n, s); }
         const float s = kk_sum(dsum);
-        if (kk == 0) Gd[N::b2 + n] = s;
-        if (w == 0 && lane < N::OUT) { float t = 0.f; for (int i = 0; i < ROWS; i++) t += dout[i * 2 + lane]; Gd[N::b3 + lane] = t; }
+        if (kk == 0) put_shared<PK>(Gd + N::b2 + n, s);
+        if (w == 0 && lane < N::OUT) { float t = 0.f; for (int i = 0; i < ROWS; i++) t += dout[i * 2 + lane]; put_shared<PK>(Gd + N::b3 + lane, t); }
     }
 }
 // backward, layer 2 weight gradient: dW2 = dp2^T h1, wavefront w owns rows [16w, 16w+16) of it
-template <class N>
+template <class N, bool PK>
 __device__ __forceinline__ void backward_w2(lptr h1, lptr dp2, float* __restrict__ Gd, int w, int lane) {
     const int r = lane & 15, kk = lane >> 4, n = 16 * w + r;
     float a[4];
@@ -255,12 +312,12 @@ __device__ __forceinline__ void backward_w2(lptr h1, lptr dp2, float* __restrict
 #pragma unroll
         for (int s = 0; s < 4; s++) acc = mfma16(a[s], h1[(4 * kk + s) * AS + 16 * it + r], acc);
 #pragma unroll
-        for (int v = 0; v < 4; v++) Gd[N::w2 + (16 * w + 4 * kk + v) * H + 16 * it + r] = acc[v];
+        for (int v = 0; v < 4; v++) put_shared<PK>(Gd + N::w2 + (16 * w + 4 * kk + v) * H + 16 * it + r, acc[v]);
     }
 }
 // backward, layer 1: d_h1 = dp2 W2 gated by relu'(h1) stays in registers and yields, with WANT_W, db1 and dW1 (vector ALU, IN <= 4
 // columns) and, with WANT_DACT, the per-wavefront partial of the gradient wrt the action input column: part[w*ROWS + row]
-template <class N, bool WANT_W, bool WANT_DACT>
+template <class N, bool WANT_W, bool WANT_DACT, bool PK>
 __device__ __forceinline__ void backward_l1(lptr x, lptr h1, lptr dp2, lptr part, const Bwd2W& f, float* __restrict__ Gd, int w, int lane) {
     const int r = lane & 15, kk = lane >> 4, n = 16 * w + r;
     float a[16];
@@ -274,14 +331,14 @@ __device__ __forceinline__ void backward_l1(lptr x, lptr h1, lptr dp2, lptr part
     for (int v = 0; v < 4; v++) d[v] = h1[(4 * kk + v) * AS + n] > 0.f ? acc[v] : 0.f;
     if (WANT_W) {
         const float s = kk_sum((d[0] + d[1]) + (d[2] + d[3]));
-        if (kk == 0) Gd[N::b1 + n] = s;
+        if (kk == 0) put_shared<PK>(Gd + N::b1 + n, s);
 #pragma unroll
         for (int i = 0; i < N::IN; i++) {
             float t = 0.f;
 #pragma unroll
             for (int v = 0; v < 4; v++) t += d[v] * x[(4 * kk + v) * XS + i];
             t = kk_sum(t);
-            if (kk == 0) Gd[N::w1 + n * N::IN + i] = t;
+            if (kk == 0) put_shared<PK>(Gd + N::w1 + n * N::IN + i, t);
         }
     }
     if (WANT_DACT) {
@@ -295,12 +352,12 @@ __device__ __forceinline__ void backward_l1(lptr x, lptr h1, lptr dp2, lptr part
 
 // copy of network parameters from the global arena into the padded LDS layout, in two halves: all loads are issued before the
 // first store, so the whole copy costs about one memory round trip, and work that does not need the new values can run between
-template <class N, int COUNT>
+template <class N, int COUNT, bool PK>
 __device__ __forceinline__ void load_nets(float (&v)[COUNT][N::per_thread], const float* const (&src)[COUNT], int tid) {
 #pragma unroll
     for (int k = 0; k < COUNT; k++)
 #pragma unroll
-        for (int u = 0; u < N::per_thread; u++) { const int idx = tid + u * THREADS; v[k][u] = src[k][idx < N::total ? idx : N::total - 1]; /* unconditional: a clamped duplicate load instead of a branch */ }
+        for (int u = 0; u < N::per_thread; u++) { const int idx = tid + u * THREADS; v[k][u] = get_shared<PK>(src[k] + (idx < N::total ? idx : N::total - 1)); /* unconditional: a clamped duplicate load instead of a branch */ }
 }
 template <class N, int COUNT>
 __device__ __forceinline__ void store_nets(lptr const (&dst)[COUNT], const float (&v)[COUNT][N::per_thread], int tid) {
@@ -314,10 +371,23 @@ __device__ __forceinline__ void store_nets(lptr const (&dst)[COUNT], const float
         }
     }
 }
+// target networks in LDS: target = polyak * target + (1 - polyak) * source, source being freshly loaded parameters
 template <class N, int COUNT>
+__device__ __forceinline__ void polyak_nets(lptr const (&dst)[COUNT], const float (&v)[COUNT][N::per_thread], float polyak, int tid) {
+#pragma unroll
+    for (int u = 0; u < N::per_thread; u++) {
+        const int idx = tid + u * THREADS;
+        if (idx < N::total) {
+            const int slot = N::slot(idx);
+#pragma unroll
+            for (int k = 0; k < COUNT; k++) dst[k][slot] = polyak_step(polyak, dst[k][slot], v[k][u]);
+        }
+    }
+}
+template <class N, int COUNT, bool PK>
 __device__ __forceinline__ void cache_nets(lptr const (&dst)[COUNT], const float* const (&src)[COUNT], int tid) {
     float v[COUNT][N::per_thread];
-    load_nets<N, COUNT>(v, src, tid);
+    load_nets<N, COUNT, PK>(v, src, tid);
     store_nets<N, COUNT>(dst, v, tid);
 }
 
@@ -332,7 +402,7 @@ __device__ __forceinline__ float adam_element(const rlt_adam_parameters& p, floa
 
 // sum over the workgroups' partial values of one or two gradient elements, in workgroup order; the loads of 16 workgroups are in
 // flight together
-template <int E>
+template <int E, bool PK>
 __device__ __forceinline__ void sum_partials(const float* __restrict__ partial, const int (&idx)[E], int G, float (&sum)[E]) {
 #pragma unroll
     for (int e = 0; e < E; e++) sum[e] = 0.f;
@@ -341,7 +411,7 @@ __device__ __forceinline__ void sum_partials(const float* __restrict__ partial, 
 #pragma unroll
         for (int e = 0; e < E; e++)
 #pragma unroll
-            for (int u = 0; u < 16; u++) pv[e][u] = partial[(size_t)min(w0 + u, G) * N_PARTIAL + idx[e]];   // row G is all zeros: no select, no branch
+            for (int u = 0; u < 16; u++) pv[e][u] = get_shared<PK>(partial + (size_t)min(w0 + u, G) * N_PARTIAL + idx[e]);   // row G is all zeros: no select, no branch
         __builtin_amdgcn_sched_barrier(0);    // all loads are issued before the first add waits for one
 #pragma unroll
         for (int e = 0; e < E; e++)
@@ -367,6 +437,7 @@ struct Shared {
     float dout_actor_critic[ROWS * 2];   // -1/batch: the gradient the actor loss puts on both critics' outputs
     float new_row[16];            // the transition added this step
     unsigned long long ticks[16]; // per-phase clock ticks of this workgroup (profiling aid), flushed at the end
+    int abort;                    // a wait for another workgroup failed: leave the step loop
     float alpha;                  // exp(log_alpha) of this step
     float rollout_eps[2];         // exploration noise of this step and the next (indexed by step parity)
     float bc[8];                  // Adam bias corrections of this step: actor, critic 0, critic 1, alpha
@@ -375,14 +446,16 @@ struct Shared {
 };
 typedef __attribute__((address_space(3))) Shared* sptr;
 
+template <bool PACKED>
 __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A) {
+    if (PACKED && (blockIdx.x & 7)) return;      // only every 8th workgroup works: they share one XCD
     const sptr S = (sptr)rlt_sac_lds;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), grp = wave >> 2, w = wave & 3;
-    const int g = blockIdx.x, G = gridDim.x;
+    const int g = PACKED ? blockIdx.x >> 3 : blockIdx.x, G = PACKED ? gridDim.x >> 3 : gridDim.x;
     const int B = A.batch;
     float* const my_partial = A.partial + (size_t)g * N_PARTIAL;
-    unsigned barrier_index = 0;
+    if (threadIdx.x == 0) atomicOr(A.xcd_mask, 1u << (__builtin_amdgcn_s_getreg((3 << 11) | 20) & 0xf));
     // LDS copies of all five networks, refreshed after the grid barrier that follows each optimiser phase
     const lptr w_actor = (lptr)rlt_sac_lds + ((sizeof(Shared) / 4 + 3) & ~3);
     const lptr w_critic0 = w_actor + NA::ltotal, w_critic1 = w_critic0 + NC::ltotal, w_target0 = w_critic1 + NC::ltotal, w_target1 = w_target0 + NC::ltotal;
@@ -398,9 +471,9 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
     __syncthreads();
     {
         const lptr dst_a[1] = {w_actor}; const float* const src_a[1] = {A.actor_p};
-        cache_nets<NA, 1>(dst_a, src_a, tid);
+        cache_nets<NA, 1, PACKED>(dst_a, src_a, tid);
         const lptr dst_c[4] = {w_critic0, w_critic1, w_target0, w_target1}; const float* const src_c[4] = {A.critic_p[0], A.critic_p[1], A.target_p[0], A.target_p[1]};
-        cache_nets<NC, 4>(dst_c, src_c, tid);
+        cache_nets<NC, 4, PACKED>(dst_c, src_c, tid);
     }
     if (tid < ROWS) { S->dout_actor_critic[2 * tid] = -1.0f / (float)B; S->dout_actor_critic[2 * tid + 1] = 0.f; }   // d_output = -1/num_final_steps (sac/operations_generic.h:437-453)
 
@@ -428,6 +501,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         asm volatile("" : "+v"(lane));
         const int tid = wave_base | lane;
         const uint64_t gstep = A.step_offset + (uint64_t)step;
+        const unsigned seq = (unsigned)step + 1u;    // sequence number of this step's exchanges
         // ---- replay cursor after this step's add (replay_buffer add: position advances, full latches when it wraps)
         const unsigned new_pos = rb_pos; const int full_before = rb_full;
         rb_pos = rb_pos + 1 == cap ? 0u : rb_pos + 1;
@@ -443,7 +517,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             if (rb_full) { index = rb_pos + (unsigned)A.runner.episode_step_limit + off; index = index % cap; }
             if (index >= cap) index = 0;     // cannot happen for valid offsets; keeps the access in bounds
             is_new = index == new_pos;       // the row added in S0 may not have reached memory from workgroup 0: every workgroup holds its own copy
-            if (j < R) gathered = A.rb.data[(size_t)index * R + j];
+            if (j < R) gathered = get_shared<PACKED>(A.rb.data + (size_t)index * R + j);   // written by workgroup 0 in an earlier step
         } else if (tid < ROWS * 16 + 2 * ROWS) {
             const int s = tid & 15, sample = g * ROWS + s; const bool actor_phase = tid >= ROWS * 16 + ROWS;
             const float* src = actor_phase ? A.noise_actor : A.noise_critic;
@@ -460,7 +534,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
                 ep_step = 0; ep_return = 0.f;
                 if (full_before || new_pos > 0) {
                     const unsigned prev = new_pos == 0 ? cap - 1 : new_pos - 1;
-                    if (g == 0 && lane == 0) A.rb.data[(size_t)prev * R + (R - 1)] = 1.0f;
+                    if (g == 0 && lane == 0) put_shared<PACKED>(A.rb.data + (size_t)prev * R + (R - 1), 1.0f);
                     rb_ces = new_pos;
                 }
             }
@@ -500,14 +574,16 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             rowv = lane == 9 ? (trunc ? 1.f : 0.f) : rowv;
             if (lane < R) {
                 S->new_row[lane] = rowv;
-                if (g == 0) A.rb.data[(size_t)new_pos * R + lane] = rowv;
+                if (g == 0) put_shared<PACKED>(A.rb.data + (size_t)new_pos * R + lane, rowv);
             }
             if (g == 0 && lane == 0) A.rb.episode_start[new_pos] = rb_ces;
             truncated = trunc; th = nth; thd = nthd;
             if (trunc) rb_ces = rb_pos;
         } else if (wave == 2) {
             // off the critical path: entropy coefficient of this step, exploration noise of the next one
-            if (lane == 0) S->alpha = expf(A.log_alpha[0]);
+            if (lane == 0) {
+                S->alpha = expf(get_shared<PACKED>(A.log_alpha));      // rewritten by the last workgroup in the previous step's S4
+            }
             if (lane == 1 && step + 1 < A.n_steps) S->rollout_eps[(step + 1) & 1] = A.rollout_noise ? A.rollout_noise[step + 1] : randn_at(A.seed, 3, gstep + 1);
         } else if (wave == 1 && lane < 4) {
             // bias corrections 1/(1 - beta^age) of this step (adam/operations_generic.h:43-66)
@@ -519,6 +595,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         // the gathered values land in LDS (other wavefronts do this while wavefront 0 steps the environment, except for the new row)
         rlt_lds_barrier();
         tick(0);
+        if (S->abort) break;      // uniform: every write to it is separated from this read by a workgroup barrier on both sides
         // ================= S1: critic phase =================
         if (tid < ROWS * 16) {
             const int s = tid >> 4, j = tid & 15, sample = g * ROWS + s;
@@ -599,19 +676,20 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             Snx[lane * XS + OBS] = act;
         }
         rlt_lds_barrier();
-        backward_stage1<NC, true>(La2, Ldp2, Ldout, cb1, my_partial + grp * NC::total, w, lane);
+        backward_stage1<NC, true, PACKED>(La2, Ldp2, Ldout, cb1, my_partial + grp * NC::total, w, lane);
         rlt_lds_barrier();
-        backward_w2<NC>(La1, Ldp2, my_partial + grp * NC::total, w, lane);
-        backward_l1<NC, true, false>(Sx, La1, Ldp2, Lpart, cb2, my_partial + grp * NC::total, w, lane);
+        backward_w2<NC, PACKED>(La1, Ldp2, my_partial + grp * NC::total, w, lane);
+        backward_l1<NC, true, false, PACKED>(Sx, La1, Ldp2, Lpart, cb2, my_partial + grp * NC::total, w, lane);
         if (A.out_critic_loss && w == 0) {      // sum of squared TD errors of this workgroup's rows
             float d = lane < ROWS ? (S->q[grp][lane] - S->y[lane]) : 0.f;
             d = kk_sum(row16_sum(d * d));
-            if (lane == 0) my_partial[2 * NC::total + NA::total + 1 + grp] = d;
+            if (lane == 0) put_shared<PACKED>(my_partial + 2 * NC::total + NA::total + 1 + grp, d);
         }
         tick(1);
-        grid_barrier(A.barrier_counter, (unsigned)G * (++barrier_index));
+        announce<PACKED>(A.ready, READY_CRITIC_GRADIENTS, g, seq);
         tick(2);
         // ================= S2: reduce + Adam + polyak for both critics =================
+        await(A.ready, READY_CRITIC_GRADIENTS, G, seq, A.fault, &S->abort);
         {
             constexpr int total = 2 * NC::total;
             const int chunk = (total + G - 1) / G;
@@ -624,35 +702,37 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
                     ok[e] = idx < end; idc[e] = ok[e] ? idx : begin;
                     kq[e] = idc[e] >= NC::total ? 1 : 0; o[e] = idc[e] - kq[e] * NC::total;
                     m[e] = (kq[e] ? A.critic_m[1] : A.critic_m[0])[o[e]]; v[e] = (kq[e] ? A.critic_v[1] : A.critic_v[0])[o[e]];
-                    p[e] = (kq[e] ? A.critic_p[1] : A.critic_p[0])[o[e]]; t[e] = (kq[e] ? A.target_p[1] : A.target_p[0])[o[e]];
+                    p[e] = get_shared<PACKED>((kq[e] ? A.critic_p[1] : A.critic_p[0]) + o[e]); t[e] = (kq[e] ? A.target_p[1] : A.target_p[0])[o[e]];
                 }
-                sum_partials<2>(A.partial, idc, G, gsum);
+                sum_partials<2, PACKED>(A.partial, idc, G, gsum);
 #pragma unroll
                 for (int e = 0; e < 2; e++) {
                     if (ok[e]) {
                         const float pnew = adam_element(A.adam_critic, S->bc[2 + 2 * kq[e]], S->bc[3 + 2 * kq[e]], gsum[e], m[e], v[e], p[e]);
+                        put_shared<PACKED>((kq[e] ? A.critic_p[1] : A.critic_p[0]) + o[e], pnew);      // what the other workgroups wait for first
                         (kq[e] ? A.critic_g[1] : A.critic_g[0])[o[e]] = gsum[e]; (kq[e] ? A.critic_m[1] : A.critic_m[0])[o[e]] = m[e];
-                        (kq[e] ? A.critic_v[1] : A.critic_v[0])[o[e]] = v[e]; (kq[e] ? A.critic_p[1] : A.critic_p[0])[o[e]] = pnew;
-                        (kq[e] ? A.target_p[1] : A.target_p[0])[o[e]] = A.polyak * t[e] + (1.0f - A.polyak) * pnew;
+                        (kq[e] ? A.critic_v[1] : A.critic_v[0])[o[e]] = v[e];
+                        (kq[e] ? A.target_p[1] : A.target_p[0])[o[e]] = polyak_step(A.polyak, t[e], pnew);
                     }
                 }
             }
             if (g == 0 && A.out_critic_loss && tid < 2) {
-                float s = 0.f;
-                for (int ww = 0; ww < G; ww++) s += A.partial[(size_t)ww * N_PARTIAL + 2 * NC::total + NA::total + 1 + tid];
-                A.out_critic_loss[(size_t)step * 2 + tid] = s * 0.5f / (float)B;
+                const int idx[1] = {2 * NC::total + NA::total + 1 + tid}; float s[1];
+                sum_partials<1, PACKED>(A.partial, idx, G, s);
+                A.out_critic_loss[(size_t)step * 2 + tid] = s[0] * 0.5f / (float)B;
             }
         }
         tick(3);
-        grid_barrier(A.barrier_counter, (unsigned)G * (++barrier_index));
+        announce<PACKED>(A.ready, READY_CRITIC_PARAMETERS, g, seq);
+        await(A.ready, READY_CRITIC_PARAMETERS, G, seq, A.fault, &S->abort);
         tick(4);
-        // both critics are needed at once; the target critics only in the next step's critic phase: their values wait in registers
-        float fresh[4][NC::per_thread];
+        // both critics are needed now; the target critics, read next in the following step's critic phase, follow from them later in this step
+        float fresh[2][NC::per_thread];
         {
-            const float* const src_c[4] = {A.critic_p[0], A.critic_p[1], A.target_p[0], A.target_p[1]};
-            load_nets<NC, 4>(fresh, src_c, tid);
-            const lptr dst_c[2] = {w_critic0, w_critic1}; const float (&crit)[2][NC::per_thread] = reinterpret_cast<const float (&)[2][NC::per_thread]>(fresh);
-            store_nets<NC, 2>(dst_c, crit, tid);
+            const float* const src_c[2] = {A.critic_p[0], A.critic_p[1]};
+            load_nets<NC, 2, PACKED>(fresh, src_c, tid);
+            const lptr dst_c[2] = {w_critic0, w_critic1};
+            store_nets<NC, 2>(dst_c, fresh, tid);
         }
         rlt_lds_barrier();
         tick(5);
@@ -669,9 +749,9 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             const Bwd1W b1 = load_bwd1<NC>(w_critic, w, lane); const Bwd2W b2 = load_bwd2<NC>(w_critic, w, lane);
             rlt_lds_barrier();
             if (w == 0 && lane < ROWS) S->q[grp][lane] = net_output<NC>(Lpart, w_critic, lane, 0);
-            backward_stage1<NC, false>(Le2, Ldp2, &S->dout_actor_critic[0], b1, nullptr, w, lane);
+            backward_stage1<NC, false, PACKED>(Le2, Ldp2, &S->dout_actor_critic[0], b1, nullptr, w, lane);
             rlt_lds_barrier();
-            backward_l1<NC, false, true>(Snx, Le1, Ldp2, Lpart, b2, nullptr, w, lane);
+            backward_l1<NC, false, true, PACKED>(Snx, Le1, Ldp2, Lpart, b2, nullptr, w, lane);
         }
         const Bwd1W ab1 = load_bwd1<NA>(w_actor, w, lane); const Bwd2W ab2 = load_bwd2<NA>(w_actor, w, lane);
         rlt_lds_barrier();
@@ -697,21 +777,22 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
                 alpha_term = alpha * (-lp - A.sas.target_entropy);
             }
             alpha_term = row16_sum(alpha_term);
-            if (lane == 0) my_partial[2 * NC::total + NA::total] = alpha_term;
+            if (lane == 0) put_shared<PACKED>(my_partial + 2 * NC::total + NA::total, alpha_term);
         }
         rlt_lds_barrier();
         // actor backward: layer 3 and the layer-2 gate by group 0, then the layer-2 weight gradient by group 0 and layer 1 by group 1
         const lptr dp2a = &S->grp[0].dp2[0];
-        if (grp == 0) backward_stage1<NA, true>(Ah2, dp2a, &S->actor_dout[0], ab1, my_partial + 2 * NC::total, w, lane);
+        if (grp == 0) backward_stage1<NA, true, PACKED>(Ah2, dp2a, &S->actor_dout[0], ab1, my_partial + 2 * NC::total, w, lane);
         rlt_lds_barrier();
-        if (grp == 0) backward_w2<NA>(Ah1, dp2a, my_partial + 2 * NC::total, w, lane);
-        else backward_l1<NA, true, false>(Sx, Ah1, dp2a, Lpart, ab2, my_partial + 2 * NC::total, w, lane);
+        if (grp == 0) backward_w2<NA, PACKED>(Ah1, dp2a, my_partial + 2 * NC::total, w, lane);
+        else backward_l1<NA, true, false, PACKED>(Sx, Ah1, dp2a, Lpart, ab2, my_partial + 2 * NC::total, w, lane);
         {
-            const lptr dst_t[2] = {w_target0, w_target1}; const float (&targ)[2][NC::per_thread] = reinterpret_cast<const float (&)[2][NC::per_thread]>(fresh[2]);
-            store_nets<NC, 2>(dst_t, targ, tid);     // read next after several barriers
+            const lptr dst_t[2] = {w_target0, w_target1};
+            polyak_nets<NC, 2>(dst_t, fresh, A.polyak, tid);     // read next after several barriers
         }
         tick(6);
-        grid_barrier(A.barrier_counter, (unsigned)G * (++barrier_index));
+        announce<PACKED>(A.ready, READY_ACTOR_GRADIENTS, g, seq);
+        await(A.ready, READY_ACTOR_GRADIENTS, G, seq, A.fault, &S->abort);
         tick(7);
         // ================= S4: reduce + Adam for the actor and log_alpha =================
         {
@@ -720,27 +801,29 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             for (int base = begin; base < end; base += THREADS) {
                 const bool ok = base + tid < end;
                 const int o = ok ? base + tid : begin;      // idle lanes redo the first element and drop the result: no branch around the loads
-                float m = A.actor_m[o], v = A.actor_v[o]; const float p = A.actor_p[o];
+                float m = A.actor_m[o], v = A.actor_v[o]; const float p = get_shared<PACKED>(A.actor_p + o);
                 const int idx[1] = {2 * NC::total + o}; float gs[1];
-                sum_partials<1>(A.partial, idx, G, gs);
+                sum_partials<1, PACKED>(A.partial, idx, G, gs);
                 const float pnew = adam_element(A.adam_actor, S->bc[0], S->bc[1], gs[0], m, v, p);
-                if (ok) { A.actor_g[o] = gs[0]; A.actor_m[o] = m; A.actor_v[o] = v; A.actor_p[o] = pnew; }
+                if (ok) { put_shared<PACKED>(A.actor_p + o, pnew); A.actor_g[o] = gs[0]; A.actor_m[o] = m; A.actor_v[o] = v; }
             }
             if (g == G - 1 && tid == THREADS - 1) {   // log_alpha: gradient = mean over the batch of alpha * (entropy - target entropy)
                 const int idx[1] = {2 * NC::total + NA::total}; float gs[1];
-                sum_partials<1>(A.partial, idx, G, gs);
+                sum_partials<1, PACKED>(A.partial, idx, G, gs);
                 const float gsum = gs[0] / (float)B;
-                float m = A.log_alpha[2], v = A.log_alpha[3];
-                const float pnew = adam_element(A.adam_alpha, S->bc[6], S->bc[7], gsum, m, v, A.log_alpha[0]);
-                A.log_alpha[1] = gsum; A.log_alpha[2] = m; A.log_alpha[3] = v; A.log_alpha[0] = pnew;
+                // gradient and moments share the parameter's cache line, which every workgroup reads: all four go the shared way
+                float m = get_shared<PACKED>(A.log_alpha + 2), v = get_shared<PACKED>(A.log_alpha + 3);
+                const float pnew = adam_element(A.adam_alpha, S->bc[6], S->bc[7], gsum, m, v, get_shared<PACKED>(A.log_alpha));
+                put_shared<PACKED>(A.log_alpha + 1, gsum); put_shared<PACKED>(A.log_alpha + 2, m); put_shared<PACKED>(A.log_alpha + 3, v); put_shared<PACKED>(A.log_alpha, pnew);
             }
         }
         tick(8);
-        grid_barrier(A.barrier_counter, (unsigned)G * (++barrier_index));
+        announce<PACKED>(A.ready, READY_ACTOR_PARAMETERS, g, seq);
+        await(A.ready, READY_ACTOR_PARAMETERS, G, seq, A.fault, &S->abort);
         tick(9);
         {
             const lptr dst_a[1] = {w_actor}; const float* const src_a[1] = {A.actor_p};
-            cache_nets<NA, 1>(dst_a, src_a, tid);
+            cache_nets<NA, 1, PACKED>(dst_a, src_a, tid);
         }
         rlt_lds_barrier();
         tick(10);
@@ -748,6 +831,11 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
     if (A.phase_ticks && g == 0 && tid == 0) {
         S->ticks[15] = clock64() - shader_clock_begin;     // shader clock cycles of the whole run: with the sum of the others it gives the clock rate
         for (int i = 0; i < 16; i++) A.phase_ticks[i] += S->ticks[i];
+    }
+    // the placement on one XCD is what makes plain stores visible to the other workgroups: a run that was placed otherwise is void
+    if (PACKED && g == 0 && tid == 0) {
+        const unsigned mask = __hip_atomic_load(A.xcd_mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (mask & (mask - 1)) __hip_atomic_store(A.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (g == 0 && tid == 0) {
         A.runner.states[0] = th; A.runner.states[1] = thd; A.runner.episode_return[0] = ep_return;
@@ -809,7 +897,8 @@ extern "C" int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac
     const int G = B / ROWS;
     const size_t n_partial = (size_t)N_PARTIAL;
     void* scratch = nullptr;
-    int rc = rlt_scratch(device, (size_t)(G + 1) * n_partial * sizeof(float) + 256, &scratch);
+    const size_t scratch_bytes = 2048 + (size_t)(G + 1) * n_partial * sizeof(float);
+    int rc = rlt_scratch(device, scratch_bytes, &scratch);
     if (rc) return rc;
     FusedArgs a = {};
     a.actor_p = agent->actor[0].weights; a.actor_g = agent->actor[0].d_weights;
@@ -825,7 +914,8 @@ extern "C" int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac
     a.sas = agent->sas; a.gamma = agent->gamma; a.polyak = agent->polyak;
     a.batch = B; a.n_steps = n_steps;
     a.runner = *runner; a.rb = *rb;
-    a.barrier_counter = (unsigned*)scratch; a.partial = (float*)((char*)scratch + 256);
+    a.xcd_mask = (unsigned*)scratch; a.ready = (unsigned*)((char*)scratch + 256); a.partial = (float*)((char*)scratch + 2048);
+    a.fault = device->fault;
     if (inputs) { a.rollout_noise = inputs->rollout_noise; a.initial_states = inputs->initial_states; a.sample_offsets = inputs->sample_offsets;
                   a.noise_critic = inputs->noise_critic; a.noise_actor = inputs->noise_actor; }
     a.seed = seed; a.step_offset = step_offset;
@@ -835,9 +925,22 @@ extern "C" int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac
     const size_t lds_bytes = lds_floats * sizeof(float);
     a.lds_floats = (int)lds_floats;
     if (lds_bytes > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
-    RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sac_pendulum_loop_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-    RLT_HIP(hipMemsetAsync(scratch, 0, 256, device->stream));
-    RLT_HIP(hipMemsetAsync((char*)scratch + 256 + (size_t)G * n_partial * sizeof(float), 0, n_partial * sizeof(float), device->stream));
-    hipLaunchKernelGGL(sac_pendulum_loop_kernel, dim3(G), dim3(THREADS), lds_bytes, device->stream, a);
+    // sequence numbers restart with every launch; the zero row of the partial sums
+    RLT_HIP(hipMemsetAsync(scratch, 0, 2048, device->stream));
+    RLT_HIP(hipMemsetAsync((char*)scratch + 2048 + (size_t)G * n_partial * sizeof(float), 0, n_partial * sizeof(float), device->stream));
+    device->fault_armed = 1;
+    // one XCD holds 32 CUs: up to that many workgroups are placed on one XCD if the device hands out workgroups round robin
+    // RLT_SAC_LOOP_PLACEMENT=spread keeps the workgroups spread over the XCDs (the path larger batches take), for tests and comparisons
+    const char* placement = std::getenv("RLT_SAC_LOOP_PLACEMENT");
+    const bool spread = placement && std::strcmp(placement, "spread") == 0;
+    if (std::getenv("RLT_ROCM_VERBOSE")) std::fprintf(stderr, "rlt_rocm_sac_pendulum_loop: %d workgroups, xcd stride %d, %s\n", G, device->xcd_stride,
+                                                      (G <= MAX_PACKED_G && device->xcd_stride == 8 && !spread) ? "on one XCD" : "spread");
+    if (G <= MAX_PACKED_G && device->xcd_stride == 8 && !spread) {
+        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sac_pendulum_loop_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        hipLaunchKernelGGL(sac_pendulum_loop_kernel<true>, dim3(8 * G), dim3(THREADS), lds_bytes, device->stream, a);
+    } else {
+        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sac_pendulum_loop_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        hipLaunchKernelGGL(sac_pendulum_loop_kernel<false>, dim3(G), dim3(THREADS), lds_bytes, device->stream, a);
+    }
     return rlt_launch_status(device);
 }

@@ -26,9 +26,13 @@ def run_fused(rocm, agent, runner, draws, n_steps, with_outputs=True):
     return dict(loss=loss.numpy(), oab=oab.numpy(), rewards=rew.numpy(), terminated=term.numpy(), target=y.numpy())
 
 
-@pytest.mark.parametrize("batch,n_steps", [(256, 1), (256, 100), (64, 250)])
-def test_fused_loop_replays_the_checkers_steps(oracle, rocm, batch, n_steps):
-    print("case", batch, n_steps, flush=True)
+@pytest.mark.parametrize("batch,n_steps,placement", [(256, 1, None), (256, 100, None), (64, 250, None), (256, 100, "spread"), (640, 30, None)])
+def test_fused_loop_replays_the_checkers_steps(oracle, rocm, batch, n_steps, placement, monkeypatch):
+    """placement: up to 32 workgroups (batch 512) run on one XCD and exchange through its L2; "spread" forces the layout that larger
+    batches (here 640 = 40 workgroups) take, spread over the XCDs with stores written through to memory."""
+    print("case", batch, n_steps, placement, flush=True)
+    if placement:
+        monkeypatch.setenv("RLT_SAC_LOOP_PLACEMENT", placement)
     lib = oracle.lib
     loop, cfg = helpers.make_loop(oracle, batch)
     for _ in range(cfg.n_warmup_steps + 3):        # a few trained steps so that Adam moments and ages are non-trivial
