@@ -4,8 +4,9 @@
 //
 // Here the work is split by what depends on time:
 //   * W_i x + b_i for ALL steps is one contraction over sequence*batch rows (gemm.hip), written straight into post_activation;
-//   * the recurrence runs in ONE launch: batch rows are independent, so a workgroup owns a few rows for the whole sequence, keeps W_h
-//     (48 KB at H = 64) and its rows' hidden state in LDS and loops over the steps without any grid-wide synchronisation;
+//   * the recurrence runs in ONE launch: batch rows are independent, so no grid-wide synchronisation is needed. At hidden width 64 a
+//     wavefront owns one row for the whole sequence with W_h in its registers; at other widths a workgroup owns a few rows and keeps W_h
+//     and its rows' hidden state in LDS;
 //   * backward does the same in reverse and stores, per step, the gradient at the gate pre-activations (one copy as the input path sees
 //     it, one as the hidden path sees it, which differs in the n gate by the factor r) and the previous hidden state; the weight
 //     gradients and d_input are then three contractions over sequence*batch rows.
@@ -106,11 +107,124 @@ __global__ __launch_bounds__(GRU_THREADS) void gru_backward_kernel(GruArgs A) {
     if (active && A.db_hn_partial) A.db_hn_partial[(size_t)b * H + j] = db_hn;
 }
 
-// db_h[n part] += sum over batch rows of the per-row sums (row order), db_h[r, z parts] = db_i[r, z parts] (the reference copies, :679-681)
-__global__ void gru_bias_hidden_kernel(const float* __restrict__ partial, int B, int H, const float* __restrict__ db_i, float* __restrict__ db_h) {
-    const int j = blockIdx.x * blockDim.x + threadIdx.x;
-    if (j < 2 * H) db_h[j] = db_i[j];
-    else if (j < 3 * H) { float s = 0.f; for (int b = 0; b < B; b++) s += partial[(size_t)b * H + (j - 2 * H)]; db_h[j] += s; }
+// ---- hidden width 64: one wavefront per batch row, W_h in registers ------------------------------------------------------------
+// Lane j owns hidden unit j of its row and keeps rows j, 64 + j, 128 + j of W_h (192 values) in registers for the whole sequence; the
+// previous hidden state reaches all lanes through 64 lane reads per step, so a step needs neither LDS nor a barrier, and the
+// wavefronts of a workgroup are independent (they only share the launch). The step's inputs W_i x + b_i are requested one step ahead.
+constexpr int HW = 64;
+
+__device__ __forceinline__ float lane_read(float x, int k) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), k)); }
+
+__global__ __launch_bounds__(GRU_THREADS) void gru_forward64_kernel(GruArgs A) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int b = blockIdx.x * (GRU_THREADS / 64) + wave;
+    if (b >= A.B) return;                                   // whole wavefronts leave; no barrier follows
+    float wr[HW], wz[HW], wn[HW];
+    {
+        const float4* r4 = reinterpret_cast<const float4*>(A.L.weights_hidden + (size_t)lane * HW);
+        const float4* z4 = reinterpret_cast<const float4*>(A.L.weights_hidden + (size_t)(HW + lane) * HW);
+        const float4* n4 = reinterpret_cast<const float4*>(A.L.weights_hidden + (size_t)(2 * HW + lane) * HW);
+#pragma unroll
+        for (int q = 0; q < HW / 4; q++) {
+            const float4 a = r4[q], c = z4[q], d = n4[q];
+            wr[4 * q] = a.x; wr[4 * q + 1] = a.y; wr[4 * q + 2] = a.z; wr[4 * q + 3] = a.w;
+            wz[4 * q] = c.x; wz[4 * q + 1] = c.y; wz[4 * q + 2] = c.z; wz[4 * q + 3] = c.w;
+            wn[4 * q] = d.x; wn[4 * q + 1] = d.y; wn[4 * q + 2] = d.z; wn[4 * q + 3] = d.w;
+        }
+    }
+    const float bhr = A.L.biases_hidden[lane], bhz = A.L.biases_hidden[HW + lane], bhn = A.L.biases_hidden[2 * HW + lane];
+    const float h0 = A.L.initial_hidden_state[lane];
+    float h = h0;
+    const size_t stride = (size_t)A.B * 3 * HW;
+    float* post = A.L.post_activation + (size_t)b * 3 * HW;
+    float xr = post[lane], xz = post[HW + lane], xn = post[2 * HW + lane];
+    int rs = A.reset ? A.reset[b] : 0;
+    for (int t = 0; t < A.S; t++) {
+        // next step's inputs (the last step requests its own again: no branch around the loads)
+        const int tn = t + 1 < A.S ? t + 1 : t;
+        const float* pn = A.L.post_activation + (size_t)tn * stride + (size_t)b * 3 * HW;
+        const float nxr = pn[lane], nxz = pn[HW + lane], nxn = pn[2 * HW + lane];
+        const int nrs = A.reset ? A.reset[(size_t)tn * A.B + b] : 0;
+        if (t == 0 || rs) h = h0;
+        float ar = bhr, az = bhz, an = bhn;
+#pragma unroll
+        for (int k = 0; k < HW; k++) { const float hk = lane_read(h, k); ar += hk * wr[k]; az += hk * wz[k]; an += hk * wn[k]; }
+        const float r = sigmoidf_(xr + ar), z = sigmoidf_(xz + az);
+        const float n = tanhf(xn + an * r);
+        float* po = A.L.post_activation + (size_t)t * stride + (size_t)b * 3 * HW;
+        po[lane] = r; po[HW + lane] = z; po[2 * HW + lane] = n;
+        const size_t at = ((size_t)t * A.B + b) * HW + lane;
+        A.L.n_pre_pre_activation[at] = an;
+        h = (1.0f - z) * n + z * h;
+        A.L.output[at] = h;
+        xr = nxr; xz = nxz; xn = nxn; rs = nrs;
+    }
+}
+
+// Reverse pass at hidden width 64: lane k keeps column k of W_h (the 192 weights that multiply the gate gradients on the way to
+// d h_prev[k]); the gate gradients of the 64 units reach all lanes through lane reads.
+__global__ __launch_bounds__(GRU_THREADS) void gru_backward64_kernel(GruArgs A) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int b = blockIdx.x * (GRU_THREADS / 64) + wave;
+    if (b >= A.B) return;
+    float cr[HW], cz[HW], cn[HW];
+#pragma unroll
+    for (int j = 0; j < HW; j++) {
+        cr[j] = A.L.weights_hidden[(size_t)j * HW + lane]; cz[j] = A.L.weights_hidden[(size_t)(HW + j) * HW + lane]; cn[j] = A.L.weights_hidden[(size_t)(2 * HW + j) * HW + lane];
+    }
+    const float h0 = A.L.initial_hidden_state[lane];
+    float carry = 0.f, db_hn = 0.f;
+    // this step's saved values are requested one step ahead
+    size_t at = (size_t)(A.S - 1) * A.B + b;
+    float r = A.L.post_activation[at * 3 * HW + lane], z = A.L.post_activation[at * 3 * HW + HW + lane], n = A.L.post_activation[at * 3 * HW + 2 * HW + lane];
+    float npp = A.L.n_pre_pre_activation[at * HW + lane], dy = A.d_output[at * HW + lane];
+    float hp_raw = A.S > 1 ? A.L.output[((size_t)(A.S - 2) * A.B + b) * HW + lane] : 0.f;
+    int rs = A.reset ? A.reset[at] : 0;
+    for (int t = A.S - 1; t >= 0; t--) {
+        at = (size_t)t * A.B + b;
+        const int tp = t > 0 ? t - 1 : 0;
+        const size_t ap = (size_t)tp * A.B + b;
+        const float pr = A.L.post_activation[ap * 3 * HW + lane], pz = A.L.post_activation[ap * 3 * HW + HW + lane], pnn = A.L.post_activation[ap * 3 * HW + 2 * HW + lane];
+        const float pnpp = A.L.n_pre_pre_activation[ap * HW + lane], pdy = A.d_output[ap * HW + lane];
+        const float php = A.L.output[((size_t)(tp > 0 ? tp - 1 : 0) * A.B + b) * HW + lane];
+        const int prs = A.reset ? A.reset[ap] : 0;
+        const bool from_initial = t == 0 || rs;
+        const float hp = from_initial ? h0 : hp_raw;
+        const float dh = dy + carry;
+        A.d_output[at * HW + lane] = dh;
+        const float gz = dh * (hp - n) * z * (1.0f - z);
+        const float gn = dh * (1.0f - z) * (1.0f - n * n);
+        const float gr = gn * npp * r * (1.0f - r);
+        const float gnr = gn * r;
+        float* bi = A.buffer_input + at * 3 * HW; float* bh = A.buffer_hidden + at * 3 * HW;
+        bi[lane] = gr; bi[HW + lane] = gz; bi[2 * HW + lane] = gn;
+        bh[lane] = gr; bh[HW + lane] = gz; bh[2 * HW + lane] = gnr;
+        A.h_previous[at * HW + lane] = hp;
+        // the reference drops reset samples (t > 0) from the b_hn gradient (their buffer rows are zeroed before that sum, :716-749)
+        if (!(t > 0 && from_initial)) db_hn += gnr;
+        carry = 0.f;
+        if (!from_initial) {        // uniform over the wavefront: one row
+            float a0 = dh * z, a1 = 0.f, a2 = 0.f;
+#pragma unroll
+            for (int j = 0; j < HW; j++) { a0 += lane_read(gr, j) * cr[j]; a1 += lane_read(gz, j) * cz[j]; a2 += lane_read(gnr, j) * cn[j]; }
+            carry = a0 + (a1 + a2);
+        }
+        r = pr; z = pz; n = pnn; npp = pnpp; dy = pdy; hp_raw = php; rs = prs;
+    }
+    if (A.db_hn_partial) A.db_hn_partial[(size_t)b * HW + lane] = db_hn;
+}
+
+// db_h[n part] += sum over batch rows of the per-row sums, db_h[r, z parts] = db_i[r, z parts] (the reference copies, :679-681).
+// One workgroup per hidden unit.
+__global__ __launch_bounds__(256) void gru_bias_hidden_kernel(const float* __restrict__ partial, int B, int H, const float* __restrict__ db_i, float* __restrict__ db_h) {
+    __shared__ float part[4];
+    const int j = blockIdx.x;
+    float s = 0.f;
+    for (int b = threadIdx.x; b < B; b += blockDim.x) s += partial[(size_t)b * H + j];
+    s = rlt_wave_sum(s);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) { db_h[2 * H + j] += (part[0] + part[1]) + (part[2] + part[3]); db_h[j] = db_i[j]; db_h[H + j] = db_i[H + j]; }
 }
 
 size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
@@ -141,6 +255,10 @@ int rlt_rocm_gru_forward(rlt_rocm_device* device, const rlt_gru_layer* L, const 
     int rc = rlt_gemm_forward(device, input, L->input_dim, L->weights_input, L->biases_input, RLT_ACT_IDENTITY, nullptr, nullptr, L->post_activation, 3 * H, S * B, L->input_dim, 3 * H);
     if (rc) return rc;
     GruArgs a = {}; a.L = *L; a.input = input; a.reset = reset; a.S = S; a.B = B; a.rows_per_group = rows_per_group(H);
+    if (H == HW) {
+        hipLaunchKernelGGL(gru_forward64_kernel, dim3(rlt_div_up(B, GRU_THREADS / 64)), dim3(GRU_THREADS), 0, device->stream, a);
+        return rlt_launch_status(device);
+    }
     const size_t lds = lds_bytes(H, false);
     RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gru_forward_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(gru_forward_kernel, dim3(rlt_div_up(B, a.rows_per_group)), dim3(GRU_THREADS), lds, device->stream, a);
@@ -162,15 +280,18 @@ int rlt_rocm_gru_backward(rlt_rocm_device* device, const rlt_gru_layer* L, const
     float* db_hn_partial = (float*)w;
     GruArgs a = {}; a.L = *L; a.input = input; a.reset = reset; a.d_output = d_output; a.buffer_input = buffer_input; a.buffer_hidden = buffer_hidden;
     a.h_previous = h_previous; a.db_hn_partial = want_weight_gradients ? db_hn_partial : nullptr; a.S = S; a.B = B; a.rows_per_group = rows_per_group(H);
-    const size_t lds = lds_bytes(H, true);
-    RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gru_backward_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(gru_backward_kernel, dim3(rlt_div_up(B, a.rows_per_group)), dim3(GRU_THREADS), lds, device->stream, a);
+    if (H == HW) hipLaunchKernelGGL(gru_backward64_kernel, dim3(rlt_div_up(B, GRU_THREADS / 64)), dim3(GRU_THREADS), 0, device->stream, a);
+    else {
+        const size_t lds = lds_bytes(H, true);
+        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gru_backward_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(gru_backward_kernel, dim3(rlt_div_up(B, a.rows_per_group)), dim3(GRU_THREADS), lds, device->stream, a);
+    }
     int rc = rlt_launch_status(device);
     if (rc) return rc;
     if (want_weight_gradients) {
         if ((rc = rlt_gemm_wgrad(device, buffer_input, 3 * H, input, I, L->d_weights_input, L->d_biases_input, rows, I, 3 * H))) return rc;       // :677-678
         if ((rc = rlt_gemm_wgrad(device, buffer_hidden, 3 * H, h_previous, H, L->d_weights_hidden, nullptr, rows, H, 3 * H))) return rc;         // :693-742
-        hipLaunchKernelGGL(gru_bias_hidden_kernel, dim3(rlt_div_up(3 * H, 128)), dim3(128), 0, device->stream, db_hn_partial, B, H, L->d_biases_input, L->d_biases_hidden);
+        hipLaunchKernelGGL(gru_bias_hidden_kernel, dim3(H), dim3(256), 0, device->stream, (const float*)db_hn_partial, B, H, (const float*)L->d_biases_input, L->d_biases_hidden);
         if ((rc = rlt_launch_status(device))) return rc;
     }
     if (d_input) rc = rlt_gemm_backward_input(device, buffer_input, 3 * H, L->weights_input, d_input, I, nullptr, 0, 0, rows, I, 3 * H);           // :688
