@@ -159,7 +159,166 @@ __global__ __launch_bounds__(256) void runner_epilogue_kernel(rlt_pendulum_runne
     }
 }
 
+// ---- the whole runner step in one launch for 3 -> 64 -> 64 -> {1, 2} actors ---------------------------------------------------
+// A wavefront owns tiles of 32 environments, one per lane of its lower half, and keeps the actor in registers (W2 as 64
+// matrix-instruction operands; one workgroup per CU stages it through LDS once). Per tile the owning lanes run the prologue for
+// their environments and write the observations into the wavefront's corner of LDS; the network then runs on
+// v_mfma_f32_16x16x4_f32 as two independent groups of 16 rows: layer 1, the hidden activations through that same corner (no
+// workgroup barrier: nothing is shared between wavefronts), layer 2, layer 3 as a 16-lane reduction whose results go back through
+// LDS to the lanes that own the rows; these finish with the policy head, the dynamics, the reward and the replay add. Two
+// wavefronts share a SIMD so that one's per-environment arithmetic overlaps the other's matrix instructions, which bound the
+// kernel: 8,704 flop per environment on the fp32 matrix pipe. Traffic is what the step must move: state in, state and one replay
+// row out, all but the replay rows coalesced.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) float* lptr;
+constexpr int FH = 64, FTILE = 32, FAS = FH + 1, FXS = 5;
+constexpr int FUSED_LDS_PER_WAVE = 2 * 16 * FAS + FTILE * FXS + FTILE * 2;  // hidden activations of 2 x 16 rows, observations, outputs
+constexpr int FWAVES = 8;        // wavefronts per workgroup: two per SIMD, one's scalar work (prologue, dynamics) overlaps the other's matrix instructions
+
+__device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+template <int CTRL>
+__device__ __forceinline__ float dpp(float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true)); }
+__device__ __forceinline__ float row16_sum(float x) { x += dpp<0xB1>(x); x += dpp<0x4E>(x); x += dpp<0x141>(x); x += dpp<0x140>(x); return x; }
+
+struct FusedRunnerArgs {
+    rlt_pendulum_runner rn; rlt_replay_buffer rb;
+    const float* w1; const float* b1; const float* w2; const float* b2; const float* w3; const float* b3;
+    int act_hidden, act_out, out_dim, policy_kind;
+    rlt_sas_parameters sas;
+    const float* action_noise; const float* initial_states;
+    uint64_t seed, offset;
+};
+
+template <int ACT_H>      // hidden activation, a compile-time constant: it sits inside the unrolled matrix-instruction loops
+__global__ __launch_bounds__(64 * FWAVES) void runner_fused_kernel(FusedRunnerArgs A) {
+    __shared__ float lds[FWAVES * FUSED_LDS_PER_WAVE + FH * FAS];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, kk = lane >> 4;
+    const lptr hs = (lptr)lds + wave * FUSED_LDS_PER_WAVE, xs = hs + 2 * 16 * FAS, ys = xs + FTILE * FXS, w2s = (lptr)lds + FWAVES * FUSED_LDS_PER_WAVE;
+    // W2 goes through LDS (coalesced rows in, padded rows out), the small tensors straight from memory
+    for (int i = threadIdx.x; i < FH * FH; i += 64 * FWAVES) w2s[(i >> 6) * FAS + (i & 63)] = A.w2[i];
+    __syncthreads();
+    // the actor, as the operands this lane feeds to the matrix instructions (any fixed assignment of the reduction index to the
+    // four lane groups is valid as long as both operands agree: group kk takes [16 kk, 16 kk + 16) of a 64-long reduction)
+    float w1r[4], b1r[4], w2r[4][16], b2r[4], w3r[2][4];
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+        const int n = 16 * nt + r;
+        w1r[nt] = kk < 3 ? A.w1[n * 3 + kk] : 0.f; b1r[nt] = A.b1[n]; b2r[nt] = A.b2[n];
+#pragma unroll
+        for (int q = 0; q < 16; q++) w2r[nt][q] = w2s[n * FAS + kk * 16 + q];
+#pragma unroll
+        for (int c = 0; c < 2; c++) w3r[c][nt] = c < A.out_dim ? A.w3[c * FH + n] : 0.f;
+    }
+    const float b3r0 = A.b3[0], b3r1 = A.out_dim > 1 ? A.b3[1] : 0.f;
+    const int n_tiles = (A.rn.n_envs + FTILE - 1) / FTILE;
+    const int R = 10;
+    for (int tile = blockIdx.x * FWAVES + wave; tile < n_tiles; tile += gridDim.x * FWAVES) {
+        const int e = tile * FTILE + lane;
+        const bool live = lane < FTILE && e < A.rn.n_envs;
+        float th = 0.f, thd = 0.f, ep_ret = 0.f, noise = 0.f; uint32_t ep_step = 0, pos = 0, ces = 0; int full = 0;
+        if (live) {
+            const float2 st = reinterpret_cast<const float2*>(A.rn.states)[e];
+            th = st.x; thd = st.y; ep_step = A.rn.episode_step[e]; ep_ret = A.rn.episode_return[e];
+            pos = A.rb.position[e]; ces = A.rb.current_episode_start[e]; full = A.rb.full[e];
+            if (A.policy_kind == 2) noise = A.action_noise[e];
+            if (A.rn.truncated[e]) {    // prologue (operations_generic_per_env.h:8-66): reset, flag the previous replay row
+                if (A.initial_states) { const float2 ini = reinterpret_cast<const float2*>(A.initial_states)[e]; th = ini.x; thd = ini.y; }
+                else {
+                    const float PI = 3.14159265358979323846f;
+                    const float u0 = ((mix32(A.seed ^ ((A.offset + (uint64_t)e) * 2u)) >> 8) + 0.5f) * (1.0f / 16777216.0f);
+                    const float u1 = ((mix32(A.seed ^ ((A.offset + (uint64_t)e) * 2u + 1u)) >> 8) + 0.5f) * (1.0f / 16777216.0f);
+                    th = -PI + 2.0f * PI * u0; thd = -1.0f + 2.0f * u1;
+                }
+                ep_step = 0; ep_ret = 0.f;
+                if (full || pos > 0) {
+                    const uint32_t prev = pos == 0 ? (uint32_t)A.rb.capacity - 1 : pos - 1;
+                    A.rb.data[((size_t)e * A.rb.capacity + prev) * R + (R - 1)] = 1.0f;
+                    ces = pos;
+                }
+            }
+        }
+        if (lane < FTILE) {
+            float sn, cs; sincosf(th, &sn, &cs);
+            xs[lane * FXS] = cs; xs[lane * FXS + 1] = sn; xs[lane * FXS + 2] = thd; xs[lane * FXS + 3] = 0.f;
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll 1
+        for (int m = 0; m < FTILE / 16; m += 2) {       // 2 x 16 environments at a time: two independent chains of matrix instructions in flight
+            // layer 1
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const float xa = xs[(16 * (m + h) + r) * FXS + kk];
+#pragma unroll
+                for (int nt = 0; nt < 4; nt++) {
+                    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                    const floatx4 acc = mfma16(xa, w1r[nt], zero);
+#pragma unroll
+                    for (int v = 0; v < 4; v++) hs[h * 16 * FAS + (4 * kk + v) * FAS + 16 * nt + r] = rlt_act(acc[v] + b1r[nt], ACT_H);
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+            // layer 2, and layer 3 as partial dot products over this lane's hidden units
+            float a[2][16];
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int q = 0; q < 16; q++) a[h][q] = hs[h * 16 * FAS + r * FAS + kk * 16 + q];
+            float p0[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, p1[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) {
+                floatx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int q = 0; q < 16; q++) { acc0 = mfma16(a[0][q], w2r[nt][q], acc0); acc1 = mfma16(a[1][q], w2r[nt][q], acc1); }
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const float g0 = rlt_act(acc0[v] + b2r[nt], ACT_H), g1 = rlt_act(acc1[v] + b2r[nt], ACT_H);
+                    p0[0][v] += g0 * w3r[0][nt]; p1[0][v] += g0 * w3r[1][nt]; p0[1][v] += g1 * w3r[0][nt]; p1[1][v] += g1 * w3r[1][nt];
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const float s0 = row16_sum(p0[h][v]), s1 = row16_sum(p1[h][v]);
+                    if (r == v) { ys[(16 * (m + h) + 4 * kk + v) * 2] = s0; ys[(16 * (m + h) + 4 * kk + v) * 2 + 1] = s1; }
+                }
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (live) {
+            const float y0 = ys[lane * 2] + b3r0, y1 = ys[lane * 2 + 1] + b3r1;
+            float action;
+            if (A.policy_kind == 1) action = rlt_act(y0, A.act_out);
+            else {      // sample_and_squash in rollout mode (nn/layers/sample_and_squash/operations_generic.h:149-195)
+                const float ls = clampf(rlt_act(y1, A.act_out), A.sas.log_std_lower_bound, A.sas.log_std_upper_bound);
+                action = tanhf(rlt_act(y0, A.act_out) + noise * expf(ls));
+            }
+            Transition t;
+            pendulum_transition(A.rn.env, th, thd, action, t);     // epilogue (operations_generic_per_env.h:67-108)
+            ep_step += 1;
+            const bool truncated = ep_step == (uint32_t)A.rn.episode_step_limit;
+            A.rn.episode_step[e] = ep_step; A.rn.episode_return[e] = ep_ret + t.reward; A.rn.truncated[e] = truncated;
+            reinterpret_cast<float2*>(A.rn.states)[e] = make_float2(t.theta, t.theta_dot);
+            float2* row = reinterpret_cast<float2*>(A.rb.data + ((size_t)e * A.rb.capacity + pos) * R);       // rows are 40 bytes: 8-byte aligned
+            row[0] = make_float2(t.obs[0], t.obs[1]); row[1] = make_float2(t.obs[2], t.action); row[2] = make_float2(t.reward, t.next_obs[0]);
+            row[3] = make_float2(t.next_obs[1], t.next_obs[2]); row[4] = make_float2(0.0f, truncated ? 1.0f : 0.0f);
+            A.rb.episode_start[(size_t)e * A.rb.capacity + pos] = ces;
+            pos = (pos + 1) % (uint32_t)A.rb.capacity;
+            A.rb.position[e] = pos;
+            if (truncated) ces = pos;
+            A.rb.current_episode_start[e] = ces;
+            if (pos == 0 && !full) A.rb.full[e] = 1;
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 int grid1(int n) { int b = (n + 255) / 256; return b > 2048 ? 2048 : (b < 1 ? 1 : b); }
+// the shapes the one-launch step is built for
+bool fused_runner_ok(const rlt_dense_layer* L, int n, int policy_kind, const rlt_replay_buffer* rb, const rlt_pendulum_runner* rn, const float* initial_states) {
+    if (policy_kind == 0 || n != 3 || L[0].in_dim != 3 || L[0].out_dim != FH || L[1].in_dim != FH || L[1].out_dim != FH || L[2].in_dim != FH) return false;
+    if (L[0].activation != L[1].activation) return false;
+    return (((uintptr_t)rb->data | (uintptr_t)rn->states | (uintptr_t)initial_states) & 7) == 0;      // replay rows and states move as 8-byte pairs
+}
 bool rb_ok(const rlt_replay_buffer* rb) {
     return rb && rb->data && rb->episode_start && rb->position && rb->current_episode_start && rb->full && rb->n_envs > 0 && rb->capacity > 0 &&
            rb->observation_dim > 0 && rb->action_dim > 0;
@@ -215,6 +374,25 @@ int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_ru
     RLT_REQUIRE(policy_kind == 0 || (actor && n_actor_layers >= 1 && actor[0].in_dim == 3 && actor[n_actor_layers - 1].out_dim == (policy_kind == 2 ? 2 : 1)));
     RLT_REQUIRE(policy_kind != 2 || (sas && action_noise));
     const int N = rn->n_envs;
+    if (fused_runner_ok(actor, n_actor_layers, policy_kind, rb, rn, initial_states)) {
+        FusedRunnerArgs a = {};
+        a.rn = *rn; a.rb = *rb;
+        a.w1 = actor[0].weights; a.b1 = actor[0].biases; a.w2 = actor[1].weights; a.b2 = actor[1].biases; a.w3 = actor[2].weights; a.b3 = actor[2].biases;
+        a.act_hidden = actor[0].activation; a.act_out = actor[2].activation; a.out_dim = actor[2].out_dim; a.policy_kind = policy_kind;
+        if (sas) a.sas = *sas;
+        a.action_noise = action_noise; a.initial_states = initial_states; a.seed = seed; a.offset = offset;
+        const int tiles = rlt_div_up(N, FTILE);
+        int blocks = rlt_div_up(tiles, FWAVES); if (blocks > device->compute_units) blocks = device->compute_units;
+        switch (a.act_hidden) {
+            case RLT_ACT_RELU: hipLaunchKernelGGL(runner_fused_kernel<RLT_ACT_RELU>, dim3(blocks), dim3(64 * FWAVES), 0, device->stream, a); break;
+            case RLT_ACT_TANH: hipLaunchKernelGGL(runner_fused_kernel<RLT_ACT_TANH>, dim3(blocks), dim3(64 * FWAVES), 0, device->stream, a); break;
+            case RLT_ACT_FAST_TANH: hipLaunchKernelGGL(runner_fused_kernel<RLT_ACT_FAST_TANH>, dim3(blocks), dim3(64 * FWAVES), 0, device->stream, a); break;
+            case RLT_ACT_GELU: hipLaunchKernelGGL(runner_fused_kernel<RLT_ACT_GELU>, dim3(blocks), dim3(64 * FWAVES), 0, device->stream, a); break;
+            case RLT_ACT_SIGMOID: hipLaunchKernelGGL(runner_fused_kernel<RLT_ACT_SIGMOID>, dim3(blocks), dim3(64 * FWAVES), 0, device->stream, a); break;
+            default: hipLaunchKernelGGL(runner_fused_kernel<RLT_ACT_IDENTITY>, dim3(blocks), dim3(64 * FWAVES), 0, device->stream, a); break;
+        }
+        return rlt_launch_status(device);
+    }
     // scratch: observations [N x 3], actor output [N x 2], actions [N], log-probs [N], then the MLP workspace
     size_t mlp_ws = policy_kind ? rlt_rocm_mlp_workspace_bytes(actor, n_actor_layers, N) : 0;
     size_t head = (((size_t)N * 7 * sizeof(float)) + 255) & ~(size_t)255;

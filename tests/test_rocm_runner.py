@@ -23,9 +23,13 @@ class Runner:
         self.trunc = b.array(np.ones(n_envs, np.uint8))
         self.c = capi.PendulumRunner(self.states.ptr, self.ep_step.ptr, self.ep_ret.ptr, self.trunc.ptr, n_envs, limit, capi.pendulum_parameters())
 
-    def step(self, actor, initial_states):
+    def step(self, actor, initial_states, kind=1, actions=None, noise=None):
+        """kind 0: given actions; 1: the actor's output is the action; 2: actor [mean | log_std] + tanh-Gaussian head with the given noise"""
         ini = self.b.array(initial_states)
-        args = (C.byref(self.c), C.byref(self.rb.c), 1, actor.layers, actor.n, None, None, None, ini.ptr)
+        self._keep = [self.b.array(x) for x in (actions, noise) if x is not None]
+        sas = helpers.capi.SasParameters(-20.0, 2.0, 1e-6, -1.0)
+        args = (C.byref(self.c), C.byref(self.rb.c), kind, actor.layers if actor else None, actor.n if actor else 0, C.byref(sas) if kind == 2 else None,
+                self._keep[0].ptr if kind == 0 else None, self._keep[0].ptr if kind == 2 else None, ini.ptr)
         if self.b.name == "oracle":
             assert self.b.lib.rlt_oracle_pendulum_runner_step(*args) == 0
         else:
@@ -101,3 +105,26 @@ def test_runner_and_gather_at_benchmark_size(oracle, rocm):
     got = oab.numpy()
     assert np.array_equal(got[0], rows[:, 0:4]) and np.array_equal(got[1, :, :3], rows[:, 5:8]) and np.array_equal(rew.numpy(), rows[:, 4])
     assert np.array_equal(term.numpy(), (rows[:, 8] != 0).astype(np.uint8))
+
+
+@pytest.mark.parametrize("kind,hidden,hidden_act,n", [(2, 64, "relu", 1000), (2, 64, "tanh", 70), (1, 64, "tanh", 33), (1, 32, "relu", 100), (2, 48, "relu", 100), (0, 0, "", 100)])
+def test_runner_policy_kinds_and_shapes(oracle, rocm, kind, hidden, hidden_act, n):
+    """The three policy kinds; hidden width 64 takes the one-launch kernel (ragged last tile, every hidden activation class), other widths
+    and given actions the per-operation path. Ten steps with short episodes, GPU state re-seeded from the checker's each step."""
+    print("case", kind, hidden, hidden_act, n, flush=True)
+    cap, limit = 8, 4
+    rng = np.random.default_rng(kind * 100 + hidden + n)
+    actors = (None, None)
+    if kind:
+        dims = [3, hidden, hidden, kind]
+        params = helpers.random_params(rng, dims)
+        actors = [helpers.Mlp(b, dims, params, n, hidden_act, "tanh" if kind == 1 else "identity", trainable=False) for b in (oracle, rocm)]
+    r_o, r_r = Runner(oracle, n, cap, limit), Runner(rocm, n, cap, limit)
+    for t in range(10):
+        ini = np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n)], 1).astype(np.float32)
+        actions = rng.uniform(-1.5, 1.5, (n, 1)).astype(np.float32) if kind == 0 else None
+        noise = rng.standard_normal((n, 1)).astype(np.float32) if kind == 2 else None
+        r_r.load(r_o.snapshot())
+        r_o.step(actors[0], ini, kind, actions, noise); r_r.step(actors[1], ini, kind, actions, noise)
+        rocm.sync()
+        compare(r_r.snapshot(), r_o.snapshot())
