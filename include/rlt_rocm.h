@@ -571,6 +571,52 @@ int rlt_rocm_td3_update_critic_targets(rlt_rocm_device* device, const rlt_td3_ag
 /* update_actor_target     td3/operations_generic.h:322-325 */
 int rlt_rocm_td3_update_actor_target(rlt_rocm_device* device, const rlt_td3_agent* agent);
 
+/* ------------------------------------------- on-policy collection, normalisation -- */
+
+/* standardize layer       nn/layers/standardize/operations_generic.h:54-67 (set_statistics), :68-86 (evaluate / forward),
+ *                         :101-120 (backward_input; backward is a no-op: the layer has no trainable parameters)
+ *   set_statistics: layer_mean = mean, layer_precision = std == 0 ? 0 : 1 / std
+ *   forward:        out = (in - layer_mean), times layer_precision where that is not 0
+ *   backward_input: d_in = d_out * layer_precision */
+int rlt_rocm_standardize_set_statistics(rlt_rocm_device* device, const float* mean, const float* std, float* layer_mean, float* layer_precision, int dim);
+int rlt_rocm_standardize_forward(rlt_rocm_device* device, const float* layer_mean, const float* layer_precision, const float* input, int ldin,
+                                 float* output, int ldo, int batch, int dim);
+int rlt_rocm_standardize_backward_input(rlt_rocm_device* device, const float* layer_precision, const float* d_output, int ldd, float* d_input, int ldi,
+                                        int batch, int dim);
+/* running normaliser      rl/components/running_normalizer/operations_generic.h:18-45 (init: mean 0, std 1, age 0; update)
+ *   update: age += 1; per column: m = mean(column), s = sqrt(sum (x - m)^2 / (rows - 1)) (0 if that sum < 1e-6,
+ *   containers/matrix/operations_generic.h:640-691); mean += (m - mean) / age; std += (s - std) / age. age is a device counter. */
+int rlt_rocm_running_normalizer_update(rlt_rocm_device* device, const float* data, int ld, int rows, int dim, float* mean, float* std, uint32_t* age);
+
+/* The columns of the on-policy dataset that collect() writes (rl/components/on_policy_runner/on_policy_runner.h:38-72), each passed
+ * with the dataset's row stride `ld`; rows are step-major (row = step * n_envs + env). observations and all_reset have
+ * (steps_per_env + 1) * n_envs rows: the observation after the last step and the delayed reset flags go there. */
+typedef struct rlt_on_policy_dataset {
+    float* observations;       /* [(steps + 1) * n_envs x observation_dim] */
+    float* actions_mean;       /* [steps * n_envs x action_dim] */
+    float* actions;            /* [steps * n_envs x action_dim] */
+    float* action_log_probs;   /* [steps * n_envs] */
+    float* rewards;            /* [steps * n_envs] */
+    float* terminated;         /* [steps * n_envs], flags as floats */
+    float* truncated;          /* [steps * n_envs] */
+    float* all_reset;          /* [(steps + 1) * n_envs] */
+    int32_t ld, steps_per_env;
+} rlt_on_policy_dataset;
+
+size_t rlt_rocm_on_policy_collect_workspace_bytes(const rlt_pendulum_runner* runner, const rlt_dense_layer* actor, int n_actor_layers);
+/* collect                 rl/components/on_policy_runner/operations_generic.h:105-146, operations_generic_per_env.h:8-74
+ *   for the Pendulum environments of `runner` (episode_step_limit 0 = none): per step the prologue (reset where truncated from
+ *   initial_states [steps x n_envs x 2], consumed only where a reset happens; observe), the actor (optional standardize layer,
+ *   then the MLP giving the action means) and the epilogue (action = mean + exp(log_std) * action_noise [steps x n_envs x
+ *   action_dim], its log-probability, environment step, reward, episode counters, truncation, delayed reset flag); at the end
+ *   the final observation. The reference draws the noise and the initial states from its RNG while it goes; a caller here
+ *   draws them beforehand (rlt_rocm_randn_f32 / rlt_rocm_rand_f32). */
+int rlt_rocm_on_policy_collect(rlt_rocm_device* device, const rlt_pendulum_runner* runner, const rlt_on_policy_dataset* dataset,
+                               const rlt_dense_layer* actor, int n_actor_layers, const float* log_std,
+                               const float* standardize_mean, const float* standardize_precision,
+                               const float* action_noise, const float* initial_states, int truncate_on_each_iteration,
+                               void* workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

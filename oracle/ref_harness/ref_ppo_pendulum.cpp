@@ -35,6 +35,10 @@ struct LoopParameters : rlt::rl::algorithms::ppo::loop::core::DefaultParameters<
     static constexpr TI N_ENVIRONMENTS = 8;
     static constexpr TI STEP_LIMIT = 1000;
     static constexpr TI EPISODE_STEP_LIMIT = 25;       // several truncations inside one dataset
+#ifdef RLT_REF_PPO_NORMALIZE                           // second flavour of this harness: running observation normalisation switched on
+    static constexpr bool NORMALIZE_OBSERVATIONS = true;
+    static constexpr bool NORMALIZE_OBSERVATIONS_CONTINUOUSLY = true;
+#endif
     static constexpr auto ACTOR_ACTIVATION_FUNCTION = rlt::nn::activation_functions::ActivationFunction::TANH;
     using ACTOR_OPTIMIZER_PARAMETERS = rlt::nn::optimizers::adam::DEFAULT_PARAMETERS_PYTORCH<TYPE_POLICY>;
     using CRITIC_OPTIMIZER_PARAMETERS = ACTOR_OPTIMIZER_PARAMETERS;
@@ -84,11 +88,65 @@ extern "C" {
 void* rlt_ref_ppo_create(uint32_t seed) { return new Loop(seed); }
 void rlt_ref_ppo_destroy(void* h) { delete static_cast<Loop*>(h); }
 
-// first half of rl/algorithms/ppo/loop/core/operations_generic.h:89-154 (observation normalisation is off in this configuration)
-void rlt_ref_ppo_collect_and_gae(void* h) {
+// The loop step (rl/algorithms/ppo/loop/core/operations_generic.h:89-154) in the pieces it is made of, so that tests can look at the
+// state between them; rlt_ref_ppo_step runs the reference's own step() for comparison.
+void rlt_ref_ppo_step(void* h) { auto& L = *static_cast<Loop*>(h); rlt::step(L.device, L.ts); }
+void rlt_ref_ppo_collect(void* h) {
+    auto& L = *static_cast<Loop*>(h);
+    rlt::collect(L.device, L.ts.on_policy_runner_dataset, L.ts.on_policy_runner, L.ts.ppo.actor, L.ts.actor_eval_buffers, L.ts.rng);
+}
+// :106-109 / :115-119: both running normalisers take the dataset just collected, and their statistics go into the standardize layers
+void rlt_ref_ppo_update_normalizers(void* h) {
     auto& L = *static_cast<Loop*>(h);
     auto& ts = L.ts; auto& device = L.device;
-    rlt::collect(device, ts.on_policy_runner_dataset, ts.on_policy_runner, ts.ppo.actor, ts.actor_eval_buffers, ts.rng);
+    rlt::copy(device, device, ts.on_policy_runner_dataset.observations, ts.observations_dense);
+    rlt::update(device, ts.observation_normalizer, ts.observations_dense);
+    rlt::update(device, ts.observation_privileged_normalizer, ts.on_policy_runner_dataset.all_observations_privileged);
+    rlt::set_statistics(device, rlt::get_first_layer(ts.ppo.actor), ts.observation_normalizer.mean, ts.observation_normalizer.std);
+    rlt::set_statistics(device, ts.ppo.critic.content, ts.observation_privileged_normalizer.mean, ts.observation_privileged_normalizer.std);
+}
+// :111 re-initialisation of the runner after the warm-up collect
+void rlt_ref_ppo_reinit_runner(void* h) {
+    auto& L = *static_cast<Loop*>(h);
+    rlt::init(L.device, L.ts.on_policy_runner, L.ts.envs, L.ts.env_parameters, L.ts.ppo.actor, L.ts.rng);
+}
+// [normalize_observations, normalize_observations_continuously, truncate_on_each_iteration]
+void rlt_ref_ppo_flags(int* out) {
+    out[0] = LoopParameters::NORMALIZE_OBSERVATIONS; out[1] = LoopParameters::NORMALIZE_OBSERVATIONS_CONTINUOUSLY; out[2] = CONFIG::ON_POLICY_RUNNER_SPEC::TRUNCATE_ON_EACH_ITERATION;
+}
+// runner state: states [n x 2] (theta, theta_dot), episode_step [n], episode_return [n], truncated [n]
+void rlt_ref_ppo_get_runner(void* h, float* states, uint32_t* episode_step, float* episode_return, uint8_t* truncated) {
+    auto& L = *static_cast<Loop*>(h); auto& r = L.ts.on_policy_runner;
+    for (TI e = 0; e < LoopParameters::N_ENVIRONMENTS; e++) {
+        auto& st = rlt::get(r.states, 0, e);
+        states[2 * e] = st.theta; states[2 * e + 1] = st.theta_dot;
+        episode_step[e] = (uint32_t)rlt::get(r.episode_step, 0, e); episode_return[e] = rlt::get(r.episode_return, 0, e); truncated[e] = rlt::get(r.truncated, 0, e);
+    }
+}
+// running normalisers (observation, privileged observation): mean [obs], std [obs] each, ages [2]
+void rlt_ref_ppo_get_normalizers(void* h, float* mean, float* std, float* mean_privileged, float* std_privileged, uint32_t* ages) {
+    auto& ts = static_cast<Loop*>(h)->ts;
+    constexpr TI D = ENVIRONMENT::Observation::DIM;
+    std::memcpy(mean, ts.observation_normalizer.mean._data, sizeof(float) * D); std::memcpy(std, ts.observation_normalizer.std._data, sizeof(float) * D);
+    std::memcpy(mean_privileged, ts.observation_privileged_normalizer.mean._data, sizeof(float) * D); std::memcpy(std_privileged, ts.observation_privileged_normalizer.std._data, sizeof(float) * D);
+    ages[0] = (uint32_t)ts.observation_normalizer.age; ages[1] = (uint32_t)ts.observation_privileged_normalizer.age;
+}
+// the standardize layers in front of actor and critic: mean [obs], precision [obs] each
+void rlt_ref_ppo_get_standardize(void* h, float* actor_mean, float* actor_precision, float* critic_mean, float* critic_precision) {
+    auto& L = *static_cast<Loop*>(h); auto& ts = L.ts;
+    constexpr TI D = ENVIRONMENT::Observation::DIM;
+    auto& a = rlt::get_first_layer(ts.ppo.actor); auto& c = ts.ppo.critic.content;
+    for (TI i = 0; i < D; i++) {
+        actor_mean[i] = rlt::get(L.device, a.mean.parameters, i); actor_precision[i] = rlt::get(L.device, a.precision.parameters, i);
+        critic_mean[i] = rlt::get(L.device, c.mean.parameters, i); critic_precision[i] = rlt::get(L.device, c.precision.parameters, i);
+    }
+}
+void rlt_ref_ppo_values_and_gae(void* h);
+void rlt_ref_ppo_collect_and_gae(void* h) { rlt_ref_ppo_collect(h); rlt_ref_ppo_values_and_gae(h); }
+// :122-136 critic on all observations, then the advantage estimate
+void rlt_ref_ppo_values_and_gae(void* h) {
+    auto& L = *static_cast<Loop*>(h);
+    auto& ts = L.ts; auto& device = L.device;
     constexpr TI STEPS = 1, FORWARD_BATCH_SIZE = CONFIG::ON_POLICY_RUNNER_DATASET_SPEC::STEPS_TOTAL_ALL;
     auto obs = rlt::to_tensor(device, ts.on_policy_runner_dataset.all_observations_privileged);
     auto obs_r = rlt::reshape_row_major(device, obs, rlt::tensor::Shape<TI, STEPS, FORWARD_BATCH_SIZE, decltype(obs)::SHAPE::LAST>{});

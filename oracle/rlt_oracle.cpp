@@ -1147,4 +1147,135 @@ int rlt_oracle_td3_update_actor_target(const rlt_td3_agent* A) {
     return 0;
 }
 
+// --------------------------------------------------------------------------------------------- on-policy collection, normalisation
+// nn/layers/standardize/operations_generic.h:54-67
+int rlt_oracle_standardize_set_statistics(const float* mean, const float* std, float* layer_mean, float* layer_precision, int dim) {
+    if (!mean || !std || !layer_mean || !layer_precision || dim <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int i = 0; i < dim; i++) { layer_mean[i] = mean[i]; layer_precision[i] = std[i] == 0 ? 0.0f : 1 / std[i]; }
+    return 0;
+}
+// standardize/operations_generic.h:68-86
+int rlt_oracle_standardize_forward(const float* layer_mean, const float* layer_precision, const float* input, int ldin, float* output, int ldo, int batch, int dim) {
+    if (!layer_mean || !layer_precision || !input || !output || batch <= 0 || dim <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int b = 0; b < batch; b++)
+        for (int i = 0; i < dim; i++) {
+            float v = input[(size_t)b * ldin + i] - layer_mean[i];
+            if (layer_precision[i] != 0) v *= layer_precision[i];
+            output[(size_t)b * ldo + i] = v;
+        }
+    return 0;
+}
+// standardize/operations_generic.h:101-120
+int rlt_oracle_standardize_backward_input(const float* layer_precision, const float* d_output, int ldd, float* d_input, int ldi, int batch, int dim) {
+    if (!layer_precision || !d_output || !d_input || batch <= 0 || dim <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int b = 0; b < batch; b++)
+        for (int i = 0; i < dim; i++) d_input[(size_t)b * ldi + i] = d_output[(size_t)b * ldd + i] * layer_precision[i];
+    return 0;
+}
+// rl/components/running_normalizer/operations_generic.h:24-45 with mean / std of containers/matrix/operations_generic.h:640-691
+int rlt_oracle_running_normalizer_update(const float* data, int ld, int rows, int dim, float* mean, float* std, uint32_t* age) {
+    if (!data || !mean || !std || !age || rows < 2 || dim <= 0) return RLT_E_INVALID_ARGUMENT;
+    *age += 1;
+    for (int c = 0; c < dim; c++) {
+        float acc = 0;
+        for (int r = 0; r < rows; r++) acc += data[(size_t)r * ld + c];
+        const float data_mean = acc / (rows * 1);
+        float sq = 0;
+        for (int r = 0; r < rows; r++) { const float diff = data[(size_t)r * ld + c] - data_mean; sq += diff * diff; }
+        const float data_std = sq < 1e-6 ? 0.0f : std::sqrt(sq / (rows * 1 - 1));
+        mean[c] = mean[c] + (data_mean - mean[c]) / (*age);
+        std[c] = std[c] + (data_std - std[c]) / (*age);
+    }
+    return 0;
+}
+
+// rl/components/on_policy_runner/operations_generic.h:105-146 and operations_generic_per_env.h:8-74 for Pendulum environments.
+// engine != nullptr: the draws come from it in the reference's order and are written to action_noise / initial_states; otherwise they are read.
+static int on_policy_collect_impl(const rlt_pendulum_runner* rn, const rlt_on_policy_dataset* D, const rlt_dense_layer* actor, int n_layers, const float* log_std,
+                                  const float* st_mean, const float* st_precision, float* action_noise, float* initial_states, int truncate_on_each_iteration,
+                                  std::mt19937* engine) {
+    if (!rn || !D || !actor || n_layers < 1 || !log_std || !action_noise || !rn->states || !rn->episode_step || !rn->episode_return || !rn->truncated) return RLT_E_INVALID_ARGUMENT;
+    if (!D->observations || !D->actions_mean || !D->actions || !D->action_log_probs || !D->rewards || !D->terminated || !D->truncated || !D->all_reset) return RLT_E_INVALID_ARGUMENT;
+    const int N = rn->n_envs, S = D->steps_per_env, ld = D->ld, OBS = 3, ACT = actor[n_layers - 1].out_dim;
+    if (N <= 0 || S <= 0 || actor[0].in_dim != OBS || ACT != 1) return RLT_E_INVALID_ARGUMENT;     // the Pendulum takes one torque
+    if (truncate_on_each_iteration) for (int e = 0; e < N; e++) rn->truncated[e] = 1;                                           // :112-114
+    for (int e = 0; e < N; e++) D->all_reset[(size_t)e * ld] = rn->truncated[e];                                                  // :115-117 (reset aliases all_reset)
+    std::vector<float> standardized((size_t)N * OBS);
+    for (int step = 0; step < S; step++) {
+        float* obs = D->observations + (size_t)step * N * ld;
+        float* means = D->actions_mean + (size_t)step * N * ld;
+        float* actions = D->actions + (size_t)step * N * ld;
+        for (int e = 0; e < N; e++) {                                                                                          // prologue, per_env :8-35
+            if (rn->truncated[e]) {
+                rn->truncated[e] = 0; rn->episode_step[e] = 0; rn->episode_return[e] = 0;
+                float* ini = initial_states ? initial_states + ((size_t)step * N + e) * 2 : nullptr;
+                if (engine) {       // sample_initial_state, pendulum/operations_generic.h:66-77
+                    const float th = std::uniform_real_distribution<float>(-(float)M_PI, (float)M_PI)(*engine);
+                    const float thd = std::uniform_real_distribution<float>(-1.0f, 1.0f)(*engine);
+                    if (ini) { ini[0] = th; ini[1] = thd; }
+                    rn->states[2 * e] = th; rn->states[2 * e + 1] = thd;
+                } else {
+                    if (!ini) return RLT_E_INVALID_ARGUMENT;
+                    rn->states[2 * e] = ini[0]; rn->states[2 * e + 1] = ini[1];
+                }
+            }
+            pendulum_observe(rn->states[2 * e], rn->states[2 * e + 1], obs + (size_t)e * ld);
+        }
+        int rc;                                                                                                                 // :131 evaluate_step of the actor in Rollout mode
+        if (st_mean) {
+            if ((rc = rlt_oracle_standardize_forward(st_mean, st_precision, obs, ld, standardized.data(), OBS, N, OBS))) return rc;
+            if ((rc = rlt_oracle_mlp_evaluate(actor, n_layers, standardized.data(), OBS, means, ld, N))) return rc;
+        } else if ((rc = rlt_oracle_mlp_evaluate(actor, n_layers, obs, ld, means, ld, N))) return rc;
+        for (int e = 0; e < N; e++) {                                                                                          // epilogue, per_env :37-74
+            const size_t pos = (size_t)step * N + e;
+            float log_prob = 0;
+            for (int a = 0; a < ACT; a++) {
+                const float mean = means[(size_t)e * ld + a];
+                const float action_std = std::exp(log_std[a]);
+                float* z = action_noise + pos * ACT + a;
+                if (engine) { std::mt19937 copy = *engine; *z = std::normal_distribution<float>(0.0f, 1.0f)(copy); }
+                // std::normal_distribution(mean, std) returns z * std + mean for the standard normal value z it generates
+                const float noisy = engine ? std::normal_distribution<float>(mean, action_std)(*engine) : *z * action_std + mean;
+                log_prob += normal_log_prob(mean, log_std[a], noisy);
+                actions[(size_t)e * ld + a] = noisy;
+            }
+            D->action_log_probs[pos * ld] = log_prob;
+            float nth, nthd, reward;
+            pendulum_dynamics(&rn->env, rn->states[2 * e], rn->states[2 * e + 1], actions[(size_t)e * ld], &nth, &nthd, &reward);
+            D->terminated[pos * ld] = 0.0f;                                                 // the Pendulum never terminates
+            rn->episode_return[e] += reward;
+            D->rewards[pos * ld] = reward;
+            rn->episode_step[e] += 1;
+            const bool truncated = rn->episode_step_limit > 0 && rn->episode_step[e] >= (uint32_t)rn->episode_step_limit;
+            D->truncated[pos * ld] = truncated;
+            D->all_reset[(pos + N) * ld] = truncated;
+            rn->truncated[e] = truncated;
+            rn->states[2 * e] = nth; rn->states[2 * e + 1] = nthd;
+        }
+    }
+    for (int e = 0; e < N; e++) pendulum_observe(rn->states[2 * e], rn->states[2 * e + 1], D->observations + ((size_t)S * N + e) * ld);   // :137-144
+    return 0;
+}
+int rlt_oracle_on_policy_collect(const rlt_pendulum_runner* runner, const rlt_on_policy_dataset* dataset, const rlt_dense_layer* actor, int n_actor_layers,
+                                 const float* log_std, const float* standardize_mean, const float* standardize_precision, const float* action_noise,
+                                 const float* initial_states, int truncate_on_each_iteration) {
+    return on_policy_collect_impl(runner, dataset, actor, n_actor_layers, log_std, standardize_mean, standardize_precision, const_cast<float*>(action_noise),
+                                  const_cast<float*>(initial_states), truncate_on_each_iteration, nullptr);
+}
+int rlt_oracle_on_policy_collect_with_rng(const rlt_pendulum_runner* runner, const rlt_on_policy_dataset* dataset, const rlt_dense_layer* actor, int n_actor_layers,
+                                          const float* log_std, const float* standardize_mean, const float* standardize_precision, float* action_noise,
+                                          float* initial_states, int truncate_on_each_iteration, char* rng_state, int rng_state_capacity) {
+    if (!rng_state) return RLT_E_INVALID_ARGUMENT;
+    std::mt19937 engine;
+    { std::istringstream in(rng_state); in >> engine; if (in.fail()) return RLT_E_INVALID_ARGUMENT; }
+    int rc = on_policy_collect_impl(runner, dataset, actor, n_actor_layers, log_std, standardize_mean, standardize_precision, action_noise, initial_states,
+                                    truncate_on_each_iteration, &engine);
+    if (rc) return rc;
+    std::ostringstream out; out << engine;
+    const std::string s = out.str();
+    if ((int)s.size() + 1 > rng_state_capacity) return RLT_E_INVALID_ARGUMENT;
+    std::memcpy(rng_state, s.c_str(), s.size() + 1);
+    return 0;
+}
+
 }  // extern "C"

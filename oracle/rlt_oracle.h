@@ -16,6 +16,8 @@
  *   ppo surrogate/train, gru forward/backward, td3 (sampling layer, noise, targets, train_*, target updates):
  *   checked bit for bit against the reference's own PPO loop, GRU layer and TD3 loop compiled from
  *   /root/reference (oracle/_ref), and against golden vectors written by them (tests/golden).
+ *   on-policy collect (with the reference's RNG order), running normaliser, standardize statistics: bit for bit against the
+ *   reference's PPO loop with observation normalisation on (oracle/_ref), golden vectors, and closed forms in numpy.
  */
 #ifndef RLT_ORACLE_H
 #define RLT_ORACLE_H
@@ -119,6 +121,22 @@ int rlt_oracle_td3_train_critic(const rlt_td3_agent* agent, int critic_index, co
 int rlt_oracle_td3_train_actor(const rlt_td3_agent* agent, const float* sampling_noise);
 int rlt_oracle_td3_update_critic_targets(const rlt_td3_agent* agent);
 int rlt_oracle_td3_update_actor_target(const rlt_td3_agent* agent);
+
+int rlt_oracle_standardize_set_statistics(const float* mean, const float* std, float* layer_mean, float* layer_precision, int dim);
+int rlt_oracle_standardize_forward(const float* layer_mean, const float* layer_precision, const float* input, int ldin, float* output, int ldo, int batch, int dim);
+int rlt_oracle_standardize_backward_input(const float* layer_precision, const float* d_output, int ldd, float* d_input, int ldi, int batch, int dim);
+int rlt_oracle_running_normalizer_update(const float* data, int ld, int rows, int dim, float* mean, float* std, uint32_t* age);
+int rlt_oracle_on_policy_collect(const rlt_pendulum_runner* runner, const rlt_on_policy_dataset* dataset, const rlt_dense_layer* actor, int n_actor_layers,
+                                 const float* log_std, const float* standardize_mean, const float* standardize_precision, const float* action_noise,
+                                 const float* initial_states, int truncate_on_each_iteration);
+/* The draws collect() takes from the reference's std::mt19937, in its order, without running the networks' arithmetic twice: the engine (text
+ * form, advanced in place) is consumed exactly as the reference's collect consumes it -- per step, per environment that resets two uniform
+ * draws (initial theta, theta_dot), then per environment and action dimension one normal draw -- which needs the truncation pattern, so this
+ * runs the collection itself with the drawn values and also returns them: action_noise receives the N(0,1) value behind every N(mean, std)
+ * draw, initial_states the drawn states (rows of environments that do not reset are left untouched). */
+int rlt_oracle_on_policy_collect_with_rng(const rlt_pendulum_runner* runner, const rlt_on_policy_dataset* dataset, const rlt_dense_layer* actor, int n_actor_layers,
+                                          const float* log_std, const float* standardize_mean, const float* standardize_precision, float* action_noise,
+                                          float* initial_states, int truncate_on_each_iteration, char* rng_state, int rng_state_capacity);
 
 #ifdef __cplusplus
 }

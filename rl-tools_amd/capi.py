@@ -135,6 +135,11 @@ class Td3Agent(C.Structure):
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
 
 
+class OnPolicyDataset(C.Structure):
+    _fields_ = [("observations", C.c_void_p), ("actions_mean", C.c_void_p), ("actions", C.c_void_p), ("action_log_probs", C.c_void_p), ("rewards", C.c_void_p),
+                ("terminated", C.c_void_p), ("truncated", C.c_void_p), ("all_reset", C.c_void_p), ("ld", C.c_int32), ("steps_per_env", C.c_int32)]
+
+
 I, F, P, S, U64 = C.c_int, C.c_float, C.c_void_p, C.c_size_t, C.c_uint64
 LP = C.POINTER(DenseLayer)
 
@@ -174,6 +179,11 @@ PROTOTYPES = {
     "gru_backward": [C.POINTER(GruLayer), P, P, P, P, I, I, I, P, S],
     "ppo_surrogate_gradient": [P, I, P, P, I, P, I, P, I, C.POINTER(PpoParameters), P, I, P, I, I],
     "ppo_train_minibatch": [C.POINTER(PpoAgent), C.POINTER(PpoParameters), P, P, P, P, P, P, I, P, P],
+    "standardize_set_statistics": [P, P, P, P, I],
+    "standardize_forward": [P, P, P, I, P, I, I, I],
+    "standardize_backward_input": [P, P, I, P, I, I, I],
+    "running_normalizer_update": [P, I, I, I, P, P, P],
+    "on_policy_collect": [C.POINTER(PendulumRunner), C.POINTER(OnPolicyDataset), LP, I, P, P, P, P, P, I, P, S],
     "td3_sampling_forward": [P, I, P, I, F, P, I, P, I, I, I],
     "td3_sampling_backward": [P, I, P, I, P, I, I, I],
     "td3_target_action_noise": [P, F, F, P, S],
@@ -197,6 +207,7 @@ ROCM_ONLY = {
     "mlp_workspace_bytes": ([LP, I, I], S),
     "ppo_workspace_bytes": ([C.POINTER(PpoAgent)], S),
     "gru_workspace_bytes": ([C.POINTER(GruLayer), I, I], S),
+    "on_policy_collect_workspace_bytes": ([C.POINTER(PendulumRunner), LP, I], S),
     "gather_draw": ([P, C.POINTER(ReplayBuffer), I, U64, U64, P, P], I),
     "sac_pendulum_loop": ([P, C.POINTER(SacAgent), C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, U64, U64, C.POINTER(SacLoopInputs),
                            C.POINTER(SacLoopOutputs)], I),

@@ -312,6 +312,58 @@ __global__ __launch_bounds__(64 * FWAVES) void runner_fused_kernel(FusedRunnerAr
     }
 }
 
+// ---- on-policy collection (rl/components/on_policy_runner/operations_generic_per_env.h:8-74), one lane per environment ----------
+__device__ __forceinline__ float mul_add_rn(float a, float b, float c) {
+#pragma clang fp contract(off)
+    const float product = a * b;
+    return product + c;
+}
+// prologue of step `step`: reset where truncated (the flag is cleared), observe into the dataset row of this step; with final = 1 only the
+// observation after the last step is written
+__global__ __launch_bounds__(256) void on_policy_prologue_kernel(rlt_pendulum_runner rn, rlt_on_policy_dataset D, const float* __restrict__ initial_states, int step, int final,
+                                                                 int force_truncated) {
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) {
+        const size_t row = (size_t)step * rn.n_envs + e;
+        if (!final) {
+            bool truncated = rn.truncated[e] != 0 || force_truncated;
+            if (step == 0) D.all_reset[(size_t)e * D.ld] = truncated ? 1.0f : 0.0f;      // reset aliases the first rows of all_reset
+            if (truncated) {
+                rn.truncated[e] = 0; rn.episode_step[e] = 0; rn.episode_return[e] = 0.0f;
+                rn.states[2 * e] = initial_states[2 * row]; rn.states[2 * e + 1] = initial_states[2 * row + 1];
+            }
+        }
+        float s, c;
+        sincosf(rn.states[2 * e], &s, &c);
+        float* o = D.observations + row * D.ld;
+        o[0] = c; o[1] = s; o[2] = rn.states[2 * e + 1];
+    }
+}
+// epilogue: sample the action around the actor's mean, its log-probability (random/operations_generic.h:73-81), step, reward, flags
+__global__ __launch_bounds__(256) void on_policy_epilogue_kernel(rlt_pendulum_runner rn, rlt_on_policy_dataset D, const float* __restrict__ log_std,
+                                                                 const float* __restrict__ action_noise, int step) {
+    const float ls = log_std[0], sd = expf(ls);
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) {
+        const size_t row = (size_t)step * rn.n_envs + e;
+        const float mean = D.actions_mean[row * D.ld];
+        const float action = mul_add_rn(action_noise[row], sd, mean);      // z * std + mean, rounded twice as the reference's CPU build does
+        const float pre = (action - mean) / sd;
+        D.actions[row * D.ld] = action;
+        D.action_log_probs[row * D.ld] = (-0.9189385332046727f - ls) - 0.5f * pre * pre;
+        Transition t;
+        pendulum_transition(rn.env, rn.states[2 * e], rn.states[2 * e + 1], action, t);
+        D.terminated[row * D.ld] = 0.0f;
+        D.rewards[row * D.ld] = t.reward;
+        rn.episode_return[e] += t.reward;
+        const uint32_t n = rn.episode_step[e] + 1;
+        rn.episode_step[e] = n;
+        const bool truncated = rn.episode_step_limit > 0 && n >= (uint32_t)rn.episode_step_limit;
+        D.truncated[row * D.ld] = truncated ? 1.0f : 0.0f;
+        D.all_reset[(row + rn.n_envs) * D.ld] = truncated ? 1.0f : 0.0f;
+        rn.truncated[e] = truncated;
+        rn.states[2 * e] = t.theta; rn.states[2 * e + 1] = t.theta_dot;
+    }
+}
+
 int grid1(int n) { int b = (n + 255) / 256; return b > 2048 ? 2048 : (b < 1 ? 1 : b); }
 // the shapes the one-launch step is built for
 bool fused_runner_ok(const rlt_dense_layer* L, int n, int policy_kind, const rlt_replay_buffer* rb, const rlt_pendulum_runner* rn, const float* initial_states) {
@@ -409,6 +461,43 @@ int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_ru
         if ((rc = rlt_rocm_sas_forward(device, sas, actor_out, 2, action_noise, 1, actions, 1, nullptr, 0, lp, N, 1))) return rc;
     }
     hipLaunchKernelGGL(runner_epilogue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *rb, act_ptr);
+    return rlt_launch_status(device);
+}
+
+size_t rlt_rocm_on_policy_collect_workspace_bytes(const rlt_pendulum_runner* rn, const rlt_dense_layer* actor, int n_actor_layers) {
+    if (!rn || !actor || n_actor_layers < 1 || rn->n_envs < 1) return 0;
+    return (((size_t)rn->n_envs * 3 * sizeof(float) + 255) & ~(size_t)255) + rlt_rocm_mlp_workspace_bytes(actor, n_actor_layers, rn->n_envs) + 256;
+}
+
+// rl/components/on_policy_runner/operations_generic.h:105-146: per step prologue, actor, epilogue; then the final observation
+int rlt_rocm_on_policy_collect(rlt_rocm_device* device, const rlt_pendulum_runner* rn, const rlt_on_policy_dataset* D, const rlt_dense_layer* actor, int n_actor_layers,
+                               const float* log_std, const float* standardize_mean, const float* standardize_precision, const float* action_noise,
+                               const float* initial_states, int truncate_on_each_iteration, void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(rn && rn->states && rn->episode_step && rn->episode_return && rn->truncated && rn->n_envs > 0 && D && D->steps_per_env > 0 && D->ld >= 3);
+    RLT_REQUIRE(D->observations && D->actions_mean && D->actions && D->action_log_probs && D->rewards && D->terminated && D->truncated && D->all_reset);
+    RLT_REQUIRE(actor && n_actor_layers >= 1 && actor[0].in_dim == 3 && actor[n_actor_layers - 1].out_dim == 1 && log_std && action_noise && initial_states);
+    RLT_REQUIRE((standardize_mean == nullptr) == (standardize_precision == nullptr));
+    RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_on_policy_collect_workspace_bytes(rn, actor, n_actor_layers));
+    const int N = rn->n_envs;
+    float* standardized = reinterpret_cast<float*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    const size_t head = ((size_t)N * 3 * sizeof(float) + 255) & ~(size_t)255;
+    void* ws = (char*)standardized + head;
+    const size_t ws_bytes = workspace_bytes - (size_t)((char*)ws - (char*)workspace);
+    int rc;
+    for (int step = 0; step < D->steps_per_env; step++) {
+        hipLaunchKernelGGL(on_policy_prologue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *D, initial_states, step, 0, step == 0 && truncate_on_each_iteration);
+        if ((rc = rlt_launch_status(device))) return rc;
+        const float* obs = D->observations + (size_t)step * N * D->ld; int ldo = D->ld;
+        if (standardize_mean) {
+            if ((rc = rlt_rocm_standardize_forward(device, standardize_mean, standardize_precision, obs, D->ld, standardized, 3, N, 3))) return rc;
+            obs = standardized; ldo = 3;
+        }
+        if ((rc = rlt_rocm_mlp_evaluate(device, actor, n_actor_layers, obs, ldo, D->actions_mean + (size_t)step * N * D->ld, D->ld, N, ws, ws_bytes))) return rc;
+        hipLaunchKernelGGL(on_policy_epilogue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *D, log_std, action_noise, step);
+        if ((rc = rlt_launch_status(device))) return rc;
+    }
+    hipLaunchKernelGGL(on_policy_prologue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *D, initial_states, D->steps_per_env, 1, 0);
     return rlt_launch_status(device);
 }
 

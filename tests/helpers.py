@@ -48,7 +48,7 @@ def load_oracle():
     P, S, I = C.c_void_p, C.c_size_t, C.c_int
     for name, args in capi.PROTOTYPES.items():
         a = list(args)
-        if name in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward"):
+        if name in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward", "on_policy_collect"):
             a = a[:-2]      # the CPU checker allocates its own workspace
         fn = getattr(lib, "rlt_oracle_" + name)
         fn.argtypes = a
@@ -61,6 +61,8 @@ def load_oracle():
     lib.rlt_oracle_pendulum_runner_step.argtypes = [C.POINTER(capi.PendulumRunner), C.POINTER(capi.ReplayBuffer), I, C.POINTER(capi.DenseLayer), I,
                                                     C.POINTER(capi.SasParameters), P, P, P]
     lib.rlt_oracle_ppo_shuffle.argtypes = [C.c_char_p, I, I, I, P]
+    lib.rlt_oracle_on_policy_collect_with_rng.argtypes = [C.POINTER(capi.PendulumRunner), C.POINTER(capi.OnPolicyDataset), C.POINTER(capi.DenseLayer), I, P, P, P, P, P, I,
+                                                          C.c_char_p, I]
     lib.rlt_oracle_sac_loop_create.argtypes = [C.POINTER(LoopConfig)]; lib.rlt_oracle_sac_loop_create.restype = P
     for f in ("destroy", "step"):
         getattr(lib, "rlt_oracle_sac_loop_" + f).argtypes = [P]
@@ -110,7 +112,7 @@ class HostBackend:
         return HostArray(np.zeros(shape, dtype))
 
     def call(self, fn, *args):
-        if fn in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward"):
+        if fn in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward", "on_policy_collect"):
             args = args[:-2]
         rc = getattr(self.lib, "rlt_oracle_" + fn)(*args)
         if rc != 0:
@@ -459,16 +461,21 @@ PPO_COLUMNS = ("all_observations_privileged", "observations", "actions_mean", "a
                "all_reset", "reset", "all_values", "values", "advantages", "target_values")
 
 
-class RefPpo:
-    """The reference's own PPO-on-Pendulum loop through oracle/ref_harness/ref_ppo_pendulum.cpp."""
+REF_PPO_NORMALIZE_GENERIC = os.path.join(ROOT, "oracle", "_ref", "librlt_ref_ppo_normalize_generic.so")
 
-    def __init__(self, seed=0):
-        lib = C.CDLL(REF_PPO_GENERIC)
+
+class RefPpo:
+    """The reference's own PPO-on-Pendulum loop through oracle/ref_harness/ref_ppo_pendulum.cpp (normalize: the flavour built with running
+    observation normalisation switched on)."""
+
+    def __init__(self, seed=0, normalize=False):
+        lib = C.CDLL(REF_PPO_NORMALIZE_GENERIC if normalize else REF_PPO_GENERIC)
         P = C.c_void_p
         lib.rlt_ref_ppo_create.restype = P
         lib.rlt_ref_ppo_parameter_count.restype = C.c_size_t
         for f, args in dict(destroy=[P], collect_and_gae=[P], train=[P], parameter_count=[P], get_parameters=[P, P], get_dataset=[P, P], columns=[P, P],
-                            hyperparameters=[P, P], get_ages=[P, P], get_rng_state=[P, C.c_char_p, C.c_int]).items():
+                            hyperparameters=[P, P], get_ages=[P, P], get_rng_state=[P, C.c_char_p, C.c_int], step=[P], collect=[P], update_normalizers=[P],
+                            reinit_runner=[P], values_and_gae=[P], get_runner=[P] * 5, get_normalizers=[P] * 6, get_standardize=[P] * 5).items():
             getattr(lib, "rlt_ref_ppo_" + f).argtypes = args
         self.lib, self.h = lib, P(lib.rlt_ref_ppo_create(seed))
         d = (C.c_int * 11)(); lib.rlt_ref_ppo_dims(d)
@@ -498,6 +505,28 @@ class RefPpo:
     def ages(self):
         a = (C.c_uint32 * 2)(); self.lib.rlt_ref_ppo_get_ages(self.h, a)
         return list(a)
+
+    def flags(self):
+        f = (C.c_int * 3)(); self.lib.rlt_ref_ppo_flags(f)
+        return dict(normalize=bool(f[0]), continuously=bool(f[1]), truncate_on_each_iteration=bool(f[2]))
+
+    def runner(self):
+        n = self.n_envs
+        st, es, er, tr = np.zeros((n, 2), np.float32), np.zeros(n, np.uint32), np.zeros(n, np.float32), np.zeros(n, np.uint8)
+        self.lib.rlt_ref_ppo_get_runner(self.h, st.ctypes.data, es.ctypes.data, er.ctypes.data, tr.ctypes.data)
+        return dict(states=st, episode_step=es, episode_return=er, truncated=tr)
+
+    def normalizers(self):
+        d = self.obs_dim
+        m, s, mp, sp = (np.zeros(d, np.float32) for _ in range(4)); ages = np.zeros(2, np.uint32)
+        self.lib.rlt_ref_ppo_get_normalizers(self.h, m.ctypes.data, s.ctypes.data, mp.ctypes.data, sp.ctypes.data, ages.ctypes.data)
+        return dict(mean=m, std=s, mean_privileged=mp, std_privileged=sp, ages=ages)
+
+    def standardize(self):
+        d = self.obs_dim
+        am, ap, cm, cp = (np.zeros(d, np.float32) for _ in range(4))
+        self.lib.rlt_ref_ppo_get_standardize(self.h, am.ctypes.data, ap.ctypes.data, cm.ctypes.data, cp.ctypes.data)
+        return dict(actor_mean=am, actor_precision=ap, critic_mean=cm, critic_precision=cp)
 
     def close(self):
         self.lib.rlt_ref_ppo_destroy(self.h)
@@ -699,3 +728,54 @@ def td3_golden():
 def td3_golden_step(agent, g, i):
     agent.set_batch(g[f"s{i}_oab"], g[f"s{i}_rewards"], g[f"s{i}_terminated"], g[f"s{i}_target_noise"])
     agent.loop_step([int(f) for f in g[f"s{i}_flags"]], g[f"s{i}_noise_critic_0"], g[f"s{i}_noise_critic_1"], g[f"s{i}_noise_actor"])
+
+
+class OnPolicyOnBackend:
+    """Pendulum on-policy runner state and one dataset (all columns in one [rows + n_envs, ld] array, the reference's layout) on a backend."""
+
+    def __init__(self, backend, n_envs, steps, ld, col, limit, runner_state=None):
+        self.backend, self.n, self.steps, self.ld, self.col = backend, n_envs, steps, ld, col
+        rs = runner_state or dict(states=np.zeros((n_envs, 2), np.float32), episode_step=np.zeros(n_envs, np.uint32), episode_return=np.zeros(n_envs, np.float32),
+                                  truncated=np.ones(n_envs, np.uint8))
+        self.states, self.ep_step, self.ep_ret, self.trunc = (backend.array(rs[k]) for k in ("states", "episode_step", "episode_return", "truncated"))
+        self.c = capi.PendulumRunner(self.states.ptr, self.ep_step.ptr, self.ep_ret.ptr, self.trunc.ptr, n_envs, limit, capi.pendulum_parameters())
+        self.data = backend.zeros(((steps + 1) * n_envs, ld))
+        o = self.data.offset
+        self.d = capi.OnPolicyDataset(o(col["observations"]), o(col["actions_mean"]), o(col["actions"]), o(col["action_log_probs"]), o(col["rewards"]), o(col["terminated"]),
+                                      o(col["truncated"]), o(col["all_reset"]), ld, steps)
+
+    def runner_state(self):
+        return dict(states=self.states.numpy(), episode_step=self.ep_step.numpy(), episode_return=self.ep_ret.numpy(), truncated=self.trunc.numpy())
+
+    def load_runner(self, rs):
+        self.states.upload(rs["states"]); self.ep_step.upload(rs["episode_step"]); self.ep_ret.upload(rs["episode_return"]); self.trunc.upload(rs["truncated"])
+
+    def collect(self, actor, log_std, noise, initial_states, standardize=None, truncate_on_each_iteration=0):
+        b = self.backend
+        ls, nz, ini = b.array(log_std), b.array(noise), b.array(initial_states)
+        sm = b.array(standardize[0]) if standardize else None; sp = b.array(standardize[1]) if standardize else None
+        ws, wsn = (None, 0)
+        if b.name == "rocm":
+            wsn = b.device.lib.rlt_rocm_on_policy_collect_workspace_bytes(C.byref(self.c), actor.layers, actor.n)
+            ws, wsn = b.workspace(wsn)
+        b.call("on_policy_collect", C.byref(self.c), C.byref(self.d), actor.layers, actor.n, ls.ptr, sm.ptr if sm else None, sp.ptr if sp else None, nz.ptr, ini.ptr,
+               truncate_on_each_iteration, ws, wsn)
+        b.sync()
+
+
+def on_policy_golden():
+    """The committed on-policy vectors (tests/golden/make_on_policy_golden.py): dims, column map, npz."""
+    g = np.load(os.path.join(GOLDEN, "on_policy_pendulum_seed3.npz"))
+    n, S, ld, hidden, limit = [int(v) for v in g["dims"]]
+    col = dict(zip(PPO_COLUMNS, [int(v) for v in g["columns"]]))
+    return (n, S, ld, hidden, limit), col, g
+
+
+def on_policy_golden_collect(backend, g, k, dims, col):
+    """Runs collect number k of the fixture on a backend; returns the helper object (dataset, runner state)."""
+    n, S, ld, hidden, limit = dims
+    before = {name: g[f"c{k}_before_{name}"] for name in ("states", "episode_step", "episode_return", "truncated")}
+    o = OnPolicyOnBackend(backend, n, S, ld, col, limit, before)
+    actor = Mlp(backend, [3, hidden, hidden, 1], g[f"c{k}_actor"], n, "tanh", "identity", trainable=False)
+    o.collect(actor, g[f"c{k}_log_std"], g[f"c{k}_noise"], g[f"c{k}_initial_states"], standardize=(g[f"c{k}_standardize_mean"], g[f"c{k}_standardize_precision"]))
+    return o

@@ -179,3 +179,69 @@ def test_td3_masks_equal_training_on_the_unmasked_rows(oracle):
     noise = oracle.array(noises[0])
     oracle.call("td3_train_critic", C.byref(full.c), 0, noise.ptr)
     assert np.array_equal(full.nsavi.numpy(), g["s0_oab"][1])
+
+
+def test_on_policy_collect_and_normalisers_reproduce_reference_vectors(oracle):
+    """Three collect() calls of the reference's PPO loop with observation normalisation (the warm-up one, one after the runner was
+    re-initialised, one that continues running episodes): the restated collection, from the reference's runner state, actor, standardize
+    statistics and draws, reproduces every column and the runner state afterwards bit for bit; the running normalisers and the standardize
+    statistics after each update likewise."""
+    dims, col, g = helpers.on_policy_golden()
+    n, S, ld, hidden, limit = dims
+    rows = n * S
+    mean, std, age = oracle.zeros((3,)), oracle.array(np.ones(3, np.float32)), oracle.array(np.zeros(1, np.uint32))
+    mean_p, std_p, age_p = oracle.zeros((3,)), oracle.array(np.ones(3, np.float32)), oracle.array(np.zeros(1, np.uint32))
+    lm, lp = oracle.zeros((3,)), oracle.zeros((3,))
+    for k in range(3):
+        o = helpers.on_policy_golden_collect(oracle, g, k, dims, col)
+        got, want = o.data.numpy()[:, :col["all_values"]], g[f"c{k}_dataset"]
+        assert np.array_equal(got, want), k
+        for name, v in o.runner_state().items():
+            assert np.array_equal(v, g[f"c{k}_after_{name}"]), (k, name)
+        if k > 0:
+            assert g[f"c{k}_standardize_precision"].max() > 1.2        # the statistics in use are not the trivial ones
+        dd = oracle.array(np.concatenate([want, np.zeros((want.shape[0], ld - want.shape[1]), np.float32)], 1))
+        oracle.call("running_normalizer_update", dd.offset(col["observations"]), ld, rows, 3, mean.ptr, std.ptr, age.ptr)
+        oracle.call("running_normalizer_update", dd.offset(col["observations"]), ld, rows + n, 3, mean_p.ptr, std_p.ptr, age_p.ptr)
+        assert np.array_equal(mean.numpy(), g[f"u{k}_mean"]) and np.array_equal(std.numpy(), g[f"u{k}_std"])
+        assert np.array_equal(mean_p.numpy(), g[f"u{k}_mean_privileged"]) and np.array_equal(std_p.numpy(), g[f"u{k}_std_privileged"])
+        assert [int(age.numpy()[0]), int(age_p.numpy()[0])] == list(g[f"u{k}_ages"])
+        oracle.call("standardize_set_statistics", mean.ptr, std.ptr, lm.ptr, lp.ptr, 3)
+        assert np.array_equal(lm.numpy(), g[f"u{k}_actor_mean"]) and np.array_equal(lp.numpy(), g[f"u{k}_actor_precision"])
+    assert g["c2_before_episode_step"].max() > 0 and g["c2_dataset"][n:rows, col["all_reset"]].sum() >= n    # episodes carried over, truncations inside
+
+
+def test_standardize_and_running_normaliser_closed_forms(oracle):
+    """The standardize layer and the running normaliser against their definitions written independently in numpy."""
+    rng = np.random.default_rng(8)
+    f32 = np.float32
+    B, D, ld = 57, 5, 9
+    x = rng.standard_normal((B, ld)).astype(f32) * 3 + 1
+    x[:, 2] = 0.25                                  # a constant column: its deviation is reported as exactly 0
+    mean = rng.standard_normal(D).astype(f32); std = np.abs(rng.standard_normal(D)).astype(f32) + 0.1; std[3] = 0
+    lm, lp = oracle.zeros((D,)), oracle.zeros((D,))
+    m, s = oracle.array(mean), oracle.array(std)
+    oracle.call("standardize_set_statistics", m.ptr, s.ptr, lm.ptr, lp.ptr, D)
+    precision = np.where(std == 0, f32(0), f32(1) / np.where(std == 0, f32(1), std)).astype(f32)
+    assert np.array_equal(lm.numpy(), mean) and np.array_equal(lp.numpy(), precision) and precision[3] == 0
+    xd, y = oracle.array(x), oracle.zeros((B, D))
+    oracle.call("standardize_forward", lm.ptr, lp.ptr, xd.ptr, ld, y.ptr, D, B, D)
+    want = (x[:, :D] - mean) * np.where(precision == 0, f32(1), precision)       # a zero precision leaves the centred value unscaled
+    assert np.array_equal(y.numpy(), want)
+    dy = rng.standard_normal((B, D)).astype(f32)
+    d, dx = oracle.array(dy), oracle.zeros((B, D))
+    oracle.call("standardize_backward_input", lp.ptr, d.ptr, D, dx.ptr, D, B, D)
+    assert np.array_equal(dx.numpy(), dy * precision)
+    # running normaliser: after k updates the mean is the average of the k batch means, likewise for the deviations (sample deviation, n - 1)
+    rm, rs, age = oracle.zeros((D,)), oracle.array(np.ones(D, f32)), oracle.array(np.zeros(1, np.uint32))
+    means, stds = [], []
+    for k in range(4):
+        batch = (rng.standard_normal((B, ld)) * (k + 1) + k).astype(f32); batch[:, 2] = 0.25
+        bd = oracle.array(batch)
+        oracle.call("running_normalizer_update", bd.ptr, ld, B, D, rm.ptr, rs.ptr, age.ptr)
+        means.append(batch[:, :D].astype(np.float64).mean(0)); stds.append(batch[:, :D].astype(np.float64).std(0, ddof=1))
+        assert int(age.numpy()[0]) == k + 1
+        assert np.allclose(rm.numpy(), np.mean(means, 0), rtol=2e-6, atol=2e-6)
+        want_std = np.mean(stds, 0); want_std[2] = 0 if k == 0 else want_std[2]
+        assert np.allclose(np.delete(rs.numpy(), 2), np.delete(np.mean(stds, 0), 2), rtol=1e-5)
+    assert rs.numpy()[2] == 0                      # first update: 1 + (0 - 1) / 1, then 0 + (0 - 0) / k

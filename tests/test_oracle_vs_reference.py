@@ -211,3 +211,80 @@ def test_td3_updates_bit_exact_with_reference(oracle):
         assert np.array_equal(agent.ages(), b.ages())
     assert actor_updates == 50 and clipped >= 3 and blocked >= 3          # the clip at 2.5 standard deviations was exercised
     a.close(); b.close()
+
+
+@pytest.mark.skipif(not os.path.exists(helpers.REF_PPO_NORMALIZE_GENERIC), reason="oracle/_ref PPO harness (normalising flavour) not built (needs /root/reference)")
+def test_on_policy_collect_and_observation_normalisation_bit_exact_with_reference(oracle):
+    """The reference's PPO loop with running observation normalisation on. One copy is advanced by the reference's step(), a second by
+    the pieces step() is made of (collect, normaliser update, runner re-initialisation, critic values + GAE, train); they must stay
+    identical, which ties the pieces to step(). Around every collect() of the second copy the restatement is given the runner state, the
+    actor with its standardize statistics and the text form of the RNG, and must reproduce: every dataset column collect writes
+    (observations incl. the final ones, action means, sampled actions, their log-probabilities, rewards, flags, delayed resets), the
+    runner state and the RNG state afterwards, bit for bit; the same again from the returned draws instead of the RNG; and after
+    update(): both running normalisers and the statistics set into the two standardize layers."""
+    a, b = helpers.RefPpo(3, normalize=True), helpers.RefPpo(3, normalize=True)
+    assert b.flags() == dict(normalize=True, continuously=True, truncate_on_each_iteration=False)
+    n, S, ld, c = b.n_envs, b.steps, b.data_dim, b.col
+    rows = n * S
+    norm = dict(mean=oracle.zeros((3,)), std=oracle.array(np.ones(3, np.float32)), age=oracle.array(np.zeros(1, np.uint32)),
+                mean_p=oracle.zeros((3,)), std_p=oracle.array(np.ones(3, np.float32)), age_p=oracle.array(np.zeros(1, np.uint32)))
+    layer = {k: oracle.zeros((3,)) for k in ("actor_mean", "actor_precision", "critic_mean", "critic_precision")}
+    n_collects = resets_inside = 0
+
+    def collect_and_check():
+        nonlocal n_collects, resets_inside
+        p = b.parameters()
+        na = helpers.mlp_param_count([3, b.actor_hidden, b.actor_hidden, 1])
+        actor = helpers.Mlp(oracle, [3, b.actor_hidden, b.actor_hidden, 1], p[:na], n, "tanh", "identity", trainable=False)
+        log_std = p[na:na + 1]
+        st = b.standardize()
+        before, rng = b.runner(), b.rng_state()
+        b.lib.rlt_ref_ppo_collect(b.h)
+        want = b.dataset()
+        o = helpers.OnPolicyOnBackend(oracle, n, S, ld, c, b.episode_step_limit, before)
+        noise, ini = np.zeros((S, n, 1), np.float32), np.full((S, n, 2), np.nan, np.float32)
+        ls, sm, sp = oracle.array(log_std), oracle.array(st["actor_mean"]), oracle.array(st["actor_precision"])
+        assert oracle.lib.rlt_oracle_on_policy_collect_with_rng(C.byref(o.c), C.byref(o.d), actor.layers, actor.n, ls.ptr, sm.ptr, sp.ptr, noise.ctypes.data, ini.ctypes.data,
+                                                                0, rng, 16384) == 0
+        got = o.data.numpy()
+        for name, nrows in (("observations", rows + n), ("actions_mean", rows), ("actions", rows), ("action_log_probs", rows), ("rewards", rows), ("terminated", rows),
+                            ("truncated", rows), ("all_reset", rows + n)):
+            w = 3 if name == "observations" else 1
+            assert np.array_equal(got[:nrows, c[name]:c[name] + w], want[:nrows, c[name]:c[name] + w]), (n_collects, name)
+        assert rng.value == b.rng_state().value              # the restatement drew exactly what the reference drew
+        after = b.runner()
+        for k, v in o.runner_state().items():
+            assert np.array_equal(v, after[k]), k
+        # the same collection from the returned draws
+        o2 = helpers.OnPolicyOnBackend(oracle, n, S, ld, c, b.episode_step_limit, before)
+        o2.collect(actor, log_std, noise, np.nan_to_num(ini), standardize=(st["actor_mean"], st["actor_precision"]))
+        assert np.array_equal(o2.data.numpy()[:, :c["all_values"]], got[:, :c["all_values"]])
+        n_collects += 1
+        resets_inside += int(want[n:rows, c["all_reset"]].sum())
+        return want
+
+    def update_and_check(d):
+        b.lib.rlt_ref_ppo_update_normalizers(b.h)
+        dd = oracle.array(d)
+        oracle.call("running_normalizer_update", dd.offset(c["observations"]), ld, rows, 3, norm["mean"].ptr, norm["std"].ptr, norm["age"].ptr)
+        oracle.call("running_normalizer_update", dd.offset(c["all_observations_privileged"]), ld, rows + n, 3, norm["mean_p"].ptr, norm["std_p"].ptr, norm["age_p"].ptr)
+        oracle.call("standardize_set_statistics", norm["mean"].ptr, norm["std"].ptr, layer["actor_mean"].ptr, layer["actor_precision"].ptr, 3)
+        oracle.call("standardize_set_statistics", norm["mean_p"].ptr, norm["std_p"].ptr, layer["critic_mean"].ptr, layer["critic_precision"].ptr, 3)
+        wn, ws = b.normalizers(), b.standardize()
+        assert np.array_equal(norm["mean"].numpy(), wn["mean"]) and np.array_equal(norm["std"].numpy(), wn["std"])
+        assert np.array_equal(norm["mean_p"].numpy(), wn["mean_privileged"]) and np.array_equal(norm["std_p"].numpy(), wn["std_privileged"])
+        assert [int(norm["age"].numpy()[0]), int(norm["age_p"].numpy()[0])] == list(wn["ages"])
+        for k in layer:
+            assert np.array_equal(layer[k].numpy(), ws[k]), k
+
+    for loop_step in range(3):
+        a.lib.rlt_ref_ppo_step(a.h)
+        if loop_step == 0:            # warm-up of the normalisers (rl/algorithms/ppo/loop/core/operations_generic.h:104-114)
+            update_and_check(collect_and_check())
+            b.lib.rlt_ref_ppo_reinit_runner(b.h)
+        update_and_check(collect_and_check())
+        b.lib.rlt_ref_ppo_values_and_gae(b.h)
+        b.lib.rlt_ref_ppo_train(b.h)
+        assert np.array_equal(a.parameters(), b.parameters()) and a.rng_state().value == b.rng_state().value
+    assert n_collects == 4 and resets_inside >= n           # truncations in the middle of a dataset did occur
+    a.close(); b.close()
