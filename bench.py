@@ -74,11 +74,14 @@ def bench_mlp(helpers, rocm, batch, iters, warmup):
     def fwd():
         rocm.call("mlp_forward", net.layers, net.n, x.ptr, 17, batch)
 
+    def bwd():      # after a forward(): the reference's call pattern (the gradient buffer becomes d_pre of the last layer in place, the identity here)
+        rocm.call("mlp_backward", net.layers, net.n, x.ptr, 17, dy.ptr, 6, None, 0, batch, 1, ws, wsn)
+
     def step():
         rocm.call("adam_step", net.adam, net.n_adam, C.byref(adam), net.age.ptr, 0.0, None)
 
     out = {}
-    for name, fn in (("forward_backward", fwd_bwd), ("forward", fwd), ("adam", step)):
+    for name, fn in (("forward_backward", fwd_bwd), ("forward", fwd), ("backward", bwd), ("adam", step)):
         rocm.call("mlp_zero_gradient", net.layers, net.n)
         for _ in range(warmup):
             fn()

@@ -1,6 +1,7 @@
 // dense layer and MLP entry points of the C ABI, built on the contraction kernels of gemm.hip
 // (reference: nn/layers/dense/operations_cpu_blas.h:36-228, nn_models/mlp/operations_generic.h:77-204).
 #include "common.h"
+#include <cstdlib>
 #include "gemm.h"
 #include "mlp_fused.h"
 
@@ -15,6 +16,10 @@ int max_dim(const rlt_dense_layer* layers, int n) {
     return m;
 }
 size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
+// below this batch the single-pass kernels (one 64-row tile per workgroup, plus the weight swizzle) do not pay against the per-layer kernels
+constexpr int FUSED_MIN_BATCH = 1024;
+// RLT_MLP_SINGLE_PASS=0 keeps forward() / backward() on the per-layer kernels (tests compare the two paths with each other)
+bool single_pass_enabled() { const char* v = std::getenv("RLT_MLP_SINGLE_PASS"); return !(v && v[0] == '0'); }
 bool chain_ok(const rlt_dense_layer* layers, int n) {
     if (!layers || n < 1) return false;
     for (int i = 0; i < n; i++) { if (!layer_ok(&layers[i])) return false; if (i > 0 && layers[i].in_dim != layers[i - 1].out_dim) return false; }
@@ -104,6 +109,10 @@ int rlt_rocm_mlp_forward(rlt_rocm_device* device, const rlt_dense_layer* layers,
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(chain_ok(layers, n) && x && batch > 0 && ldx >= layers[0].in_dim);
     for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].pre_activations && layers[l].output);
+    if (batch >= FUSED_MIN_BATCH && single_pass_enabled()) {       // in -> 256 -> 256 -> out: one pass that keeps the hidden activations on chip on their way to the next layer
+        const int rc = rlt_mlp3_fused_forward(device, layers, n, x, ldx, batch);
+        if (rc != RLT_E_UNSUPPORTED) return rc;
+    }
     const float* in = x; int ldin = ldx;
     for (int l = 0; l < n; l++) {
         int rc = rlt_gemm_forward(device, in, ldin, layers[l].weights, layers[l].biases, layers[l].activation, layers[l].pre_activations, layers[l].output,
@@ -160,6 +169,10 @@ int rlt_rocm_mlp_backward(rlt_rocm_device* device, const rlt_dense_layer* layers
     const rlt_dense_layer& last = layers[n - 1];
     int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, last.pre_activations, batch, last.out_dim, last.activation, 0);
     if (rc) return rc;
+    if (want_w && !d_input && batch >= FUSED_MIN_BATCH && single_pass_enabled()) {
+        rc = rlt_mlp3_fused_backward(device, layers, n, x, ldx, d_output, ldd, batch, workspace, workspace_bytes);
+        if (rc != RLT_E_UNSUPPORTED) return rc;
+    }
     return mlp_backward_from_dpre(device, layers, n, x, ldx, d_output, ldd, d_input, ldi, batch, want_w, tick, tock);
 }
 

@@ -9,3 +9,9 @@ size_t rlt_mlp3_fused_workspace_bytes(const rlt_dense_layer* layers, int n_layer
 int rlt_mlp3_fused_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy,
                                     const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch,
                                     void* workspace, size_t workspace_bytes);
+// forward(mlp) writing every layer's pre-activations and outputs; RLT_E_UNSUPPORTED if the shape does not fit
+int rlt_mlp3_fused_forward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, int batch);
+// backward(mlp) with weight gradients and no input gradient, from the outputs a forward() left in the layers; d_pre_last [batch x out] is the
+// gradient at the last layer's pre-activations. RLT_E_UNSUPPORTED if the shape or the workspace does not fit
+int rlt_mlp3_fused_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, const float* d_pre_last, int ldd,
+                            int batch, void* workspace, size_t workspace_bytes);

@@ -19,6 +19,10 @@
 // The weight-gradient accumulators (256 + 32 + 16 registers per lane) live in registers for the whole launch; at the end every
 // workgroup writes its partial gradients and a second kernel sums them in a fixed order into the layers' gradients (beta = 1).
 // act' is taken from the layer output, which relu / tanh / fast_tanh / sigmoid / identity allow.
+//
+// The reference's own call pattern is forward(), then (after the caller has formed the loss gradient) backward(). The same kernel
+// serves it in two more modes: FORWARD runs P1-P3 and writes every layer's pre-activations and outputs, as forward() must;
+// BACKWARD reads the outputs of layers 1 and 2 back into LDS and runs P4-P8 on the gradient it is given.
 #include "common.h"
 #include "mlp_fused.h"
 
@@ -43,8 +47,11 @@ constexpr int LDS_FLOATS = 2 * BM * HS + BM * XSP + BM * DS + 16 * HS;   // h1, 
 constexpr size_t W2F_FLOATS = 65536, W2B_FLOATS = 65536, W1S_FLOATS = 8 * 16 * 64;
 constexpr size_t PREP_FLOATS = W2F_FLOATS + W2B_FLOATS + W1S_FLOATS;
 
+enum { MODE_FUSED = 0, MODE_FORWARD = 1, MODE_BACKWARD = 2 };
+
 struct Mlp3Args {
     const float* x; int ldx; float* y; int ldy; const float* d_output; int ldd; const float* target; int ldt; float mse_scale;
+    float* act_pre[3]; float* act_out[3];      // FORWARD: written (each may be NULL); BACKWARD: act_out[0], act_out[1] are read
     int batch, in, out, act1, act2, act3, n_tiles;
     const float* b1; const float* b2; const float* b3;
     const float* w2f; const float* w2b; const float* w1s; const float* W3;
@@ -135,6 +142,7 @@ __device__ __forceinline__ void contract_256(lptr a, const float* __restrict__ w
     }
 }
 
+template <int MODE>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlp3_fused_kernel(Mlp3Args A) {
     const lptr h1 = (lptr)rlt_mlp3_lds, h2 = h1 + BM * HS, xs = h2 + BM * HS, dp3 = xs + BM * XSP, w3l = dp3 + BM * DS;
     const int lane_invariant = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -166,7 +174,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
     // four threads per row: thread t covers columns (t & 3) + 4u of row t >> 2
     constexpr int NX = 8, ND = 4;
     float vx[NX], vd[ND];
-    const float* dsrc = A.target ? A.target : A.d_output; const int ldsrc = A.target ? A.ldt : A.ldd;
+    const float* dsrc = MODE == MODE_FORWARD ? A.x : (A.target ? A.target : A.d_output); const int ldsrc = A.target ? A.ldt : A.ldd;
     auto request_tile = [&](int tile, int tid) {
         const int row = tid >> 2, c0 = tid & 3, grow = tile * BM + row;
         const bool row_ok = grow < A.batch;
@@ -174,8 +182,10 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
         const float* dr = dsrc + (size_t)(row_ok ? grow : 0) * ldsrc;
 #pragma unroll
         for (int u = 0; u < NX; u++) { const int c = c0 + 4 * u; const bool ok = row_ok && c < A.in; const float v = xr[ok ? c : 0]; vx[u] = ok ? v : 0.f; }
+        if (MODE != MODE_FORWARD) {
 #pragma unroll
-        for (int u = 0; u < ND; u++) { const int c = c0 + 4 * u; const bool ok = row_ok && c < A.out; const float v = dr[ok ? c : 0]; vd[u] = ok ? v : 0.f; }
+            for (int u = 0; u < ND; u++) { const int c = c0 + 4 * u; const bool ok = row_ok && c < A.out; const float v = dr[ok ? c : 0]; vd[u] = ok ? v : 0.f; }
+        }
     };
     request_tile(blockIdx.x, threadIdx.x);
     int lane = lane_invariant;
@@ -187,17 +197,45 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
         // ---- P0: this tile's rows into LDS (zero padded), the next tile's requested; layer-1 weight fragments requested
 #pragma unroll
         for (int u = 0; u < NX; u++) xs[(tid >> 2) * XSP + (tid & 3) + 4 * u] = vx[u];
+        if (MODE != MODE_FORWARD) {
 #pragma unroll
-        for (int u = 0; u < ND; u++) dp3[(tid >> 2) * DS + (tid & 3) + 4 * u] = vd[u];
+            for (int u = 0; u < ND; u++) dp3[(tid >> 2) * DS + (tid & 3) + 4 * u] = vd[u];
+        }
         float wf[2][16];
+        if (MODE != MODE_BACKWARD) {
 #pragma unroll
-        for (int a = 0; a < 2; a++)
+            for (int a = 0; a < 2; a++)
 #pragma unroll
-            for (int j = 0; j < 16; j++) wf[a][j] = A.w1s[((2 * w + a) * 16 + j) * 64 + lane];
+                for (int j = 0; j < 16; j++) wf[a][j] = A.w1s[((2 * w + a) * 16 + j) * 64 + lane];
+        }
+        if (MODE == MODE_BACKWARD) {
+            // the outputs of layers 1 and 2 of this tile, as forward() left them in memory, into LDS (rows beyond the batch as zeros)
+#pragma unroll 1
+            for (int half = 0; half < 2; half++) {
+                const float* src = A.act_out[half]; const lptr dst = half ? h2 : h1;
+#pragma unroll
+                for (int i0 = 0; i0 < 16; i0 += 8) {
+                    floatx4 v[8];
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const int idx = tid + THREADS * (i0 + i), row = idx >> 6, grow = r0 + row;
+                        v[i] = reinterpret_cast<const floatx4*>(src + (size_t)(grow < A.batch ? grow : 0) * HID)[idx & 63];
+                    }
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const int idx = tid + THREADS * (i0 + i), row = idx >> 6, c4 = (idx & 63) * 4;
+                        const bool ok = r0 + row < A.batch;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) dst[row * HS + c4 + e] = ok ? v[i][e] : 0.f;
+                    }
+                }
+            }
+        }
         if (tile + (int)gridDim.x < A.n_tiles) request_tile(tile + gridDim.x, tid);
         rlt_lds_barrier();
         RLT_TICK(0)
         // ---- P1: h1 = act(x W1^T + b1); wavefront w owns columns [64w, 64w+64)
+        if (MODE != MODE_BACKWARD) {
 #pragma unroll
         for (int a = 0; a < 2; a++) {
             const int nt = 2 * w + a;
@@ -213,13 +251,21 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
 #pragma unroll
             for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) h1[(32 * mt + row32(v, hi)) * HS + 32 * nt + c32] = act_c<ACT>(acc[mt][v] + bias1[a]);
+                for (int v = 0; v < 16; v++) {
+                    const float pre = acc[mt][v] + bias1[a], o = act_c<ACT>(pre);
+                    h1[(32 * mt + row32(v, hi)) * HS + 32 * nt + c32] = o;
+                    if (MODE == MODE_FORWARD) {
+                        const int grow = r0 + 32 * mt + row32(v, hi);
+                        if (grow < A.batch) { if (A.act_pre[0]) A.act_pre[0][(size_t)grow * HID + 32 * nt + c32] = pre; if (A.act_out[0]) A.act_out[0][(size_t)grow * HID + 32 * nt + c32] = o; }
+                    }
+                }
             });
         }
         rlt_lds_barrier();
+        }
         RLT_TICK(1)
         // ---- P2: h2 = act(h1 W2^T + b2)
-        {
+        if (MODE != MODE_BACKWARD) {
             floatx16 acc[2][2] = {{zero16, zero16}, {zero16, zero16}};
             contract_256(h1, A.w2f, w, lane, acc);
             act_dispatch(A.act2, [&](auto kind) { constexpr int ACT = decltype(kind)::value;
@@ -228,13 +274,21 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
 #pragma unroll
                 for (int a = 0; a < 2; a++)
 #pragma unroll
-                    for (int v = 0; v < 16; v++) h2[(32 * mt + row32(v, hi)) * HS + 32 * (2 * w + a) + c32] = act_c<ACT>(acc[mt][a][v] + bias2[a]);
+                    for (int v = 0; v < 16; v++) {
+                        const float pre = acc[mt][a][v] + bias2[a], o = act_c<ACT>(pre);
+                        h2[(32 * mt + row32(v, hi)) * HS + 32 * (2 * w + a) + c32] = o;
+                        if (MODE == MODE_FORWARD) {
+                            const int grow = r0 + 32 * mt + row32(v, hi);
+                            if (grow < A.batch) { if (A.act_pre[1]) A.act_pre[1][(size_t)grow * HID + 32 * (2 * w + a) + c32] = pre; if (A.act_out[1]) A.act_out[1][(size_t)grow * HID + 32 * (2 * w + a) + c32] = o; }
+                        }
+                    }
             });
+            rlt_lds_barrier();
         }
-        rlt_lds_barrier();
         RLT_TICK(2)
         // ---- P3: y = act(h2 W3^T + b3) for rows [16w, 16w+16) (lane group q takes the reduction range [64q, 64q+64)), then d_pre3
-        {
+        // (BACKWARD is handed d_pre3 itself: the caller has applied the output activation's derivative, as dense backward does in place)
+        if (MODE != MODE_BACKWARD) {
             floatx4 acc = zero4, acc2 = zero4;
             const lptr wp = w3l + r16 * HS + 64 * q;
             const lptr ap = h2 + (16 * w + r16) * HS + 64 * q;
@@ -248,16 +302,21 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
             for (int v = 0; v < 4; v++) {
                 const int row = 16 * w + 4 * q + v, grow = r0 + row;
                 const bool ok = r16 < A.out && grow < A.batch;
-                const float yv = rlt_act(acc[v] + bias3, A.act3);
+                const float pre = acc[v] + bias3, yv = rlt_act(pre, A.act3);
                 if (ok && A.y) A.y[(size_t)grow * A.ldy + r16] = yv;
-                const float raw = dp3[row * DS + r16];
-                float d = A.target ? (yv - raw) * A.mse_scale : raw;
-                d *= rlt_dact_from_output(yv, A.act3);
-                dp3[row * DS + r16] = ok ? d : 0.f;
+                if (MODE == MODE_FORWARD) {
+                    if (ok && A.act_pre[2]) A.act_pre[2][(size_t)grow * A.out + r16] = pre;
+                } else {
+                    const float raw = dp3[row * DS + r16];
+                    float d = A.target ? (yv - raw) * A.mse_scale : raw;
+                    d *= rlt_dact_from_output(yv, A.act3);
+                    dp3[row * DS + r16] = ok ? d : 0.f;
+                }
             }
+            rlt_lds_barrier();
         }
-        rlt_lds_barrier();
         RLT_TICK(3)
+        if (MODE == MODE_FORWARD) continue;
         // ---- P4: dW3 += d_pre3^T h2 (rows = outputs, wavefront w owns columns [64w, 64w+64)); db3
 #pragma unroll 8
         for (int j = 0; j < 16; j++) {
@@ -392,6 +451,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
         rlt_lds_barrier();
         RLT_TICK(8)
     }
+    if (MODE == MODE_FORWARD) return;
     // ---- this workgroup's partial gradients: [dW1 | db1 | dW2 | db2 | dW3 | db3]
     const int tid = threadIdx.x, c32 = lane & 31, hi = lane >> 5, r16 = lane & 15, q = lane >> 4;
     const int count = HID * A.in + HID + HID * HID + HID + A.out * HID + A.out;
@@ -466,6 +526,34 @@ size_t rlt_mlp3_fused_workspace_bytes(const rlt_dense_layer* layers, int n_layer
     return (PREP_FLOATS + (size_t)workgroups_for(batch) * gradient_count(layers)) * sizeof(float) + 256;
 }
 
+namespace {
+
+Mlp3Args base_args(const rlt_dense_layer* L, const float* x, int ldx, int batch, float* prep) {
+    Mlp3Args a = {};
+    a.x = x; a.ldx = ldx; a.batch = batch; a.in = L[0].in_dim; a.out = L[2].out_dim;
+    a.act1 = L[0].activation; a.act2 = L[1].activation; a.act3 = L[2].activation;
+    a.n_tiles = (batch + BM - 1) / BM;
+    a.b1 = L[0].biases; a.b2 = L[1].biases; a.b3 = L[2].biases;
+    a.w2f = prep; a.w2b = a.w2f + W2F_FLOATS; a.w1s = a.w2b + W2B_FLOATS; a.W3 = L[2].weights;
+    a.partial = prep + PREP_FLOATS;
+    return a;
+}
+template <int MODE>
+int launch_mode(rlt_rocm_device* device, const Mlp3Args& a, int groups) {
+    const size_t lds_bytes = (size_t)LDS_FLOATS * sizeof(float);
+    RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp3_fused_kernel<MODE>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    hipLaunchKernelGGL(mlp3_fused_kernel<MODE>, dim3(groups), dim3(THREADS), lds_bytes, device->stream, a);
+    return rlt_launch_status(device);
+}
+int reduce_partials(rlt_rocm_device* device, const rlt_dense_layer* L, const Mlp3Args& a, int groups) {
+    const int count = (int)gradient_count(L);
+    GradTargets T = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases, L[0].in_dim, L[2].out_dim};
+    hipLaunchKernelGGL(mlp3_reduce_kernel, dim3((count + 63) / 64), dim3(256), 0, device->stream, a.partial, groups, count, T);
+    return rlt_launch_status(device);
+}
+
+}  // namespace
+
 int rlt_mlp3_fused_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n, const float* x, int ldx, float* y, int ldy,
                                     const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch,
                                     void* workspace, size_t workspace_bytes) {
@@ -476,20 +564,45 @@ int rlt_mlp3_fused_forward_backward(rlt_rocm_device* device, const rlt_dense_lay
     hipLaunchKernelGGL(mlp3_prepare_kernel, dim3(65536 / 256), dim3(256), 0, device->stream, L[0].weights, L[1].weights, L[0].in_dim, prep);
     int rc = rlt_launch_status(device);
     if (rc) return rc;
-    Mlp3Args a = {};
-    a.x = x; a.ldx = ldx; a.y = y; a.ldy = ldy; a.d_output = d_output; a.ldd = ldd; a.target = target; a.ldt = ldt; a.mse_scale = mse_scale;
-    a.batch = batch; a.in = L[0].in_dim; a.out = L[2].out_dim; a.act1 = L[0].activation; a.act2 = L[1].activation; a.act3 = L[2].activation;
-    a.n_tiles = (batch + BM - 1) / BM;
-    a.b1 = L[0].biases; a.b2 = L[1].biases; a.b3 = L[2].biases;
-    a.w2f = prep; a.w2b = a.w2f + W2F_FLOATS; a.w1s = a.w2b + W2B_FLOATS; a.W3 = L[2].weights;
-    a.partial = prep + PREP_FLOATS;
+    Mlp3Args a = base_args(L, x, ldx, batch, prep);
+    a.y = y; a.ldy = ldy; a.d_output = d_output; a.ldd = ldd; a.target = target; a.ldt = ldt; a.mse_scale = mse_scale;
     const int groups = workgroups_for(batch);
-    const size_t lds_bytes = (size_t)LDS_FLOATS * sizeof(float);
-    RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp3_fused_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-    hipLaunchKernelGGL(mlp3_fused_kernel, dim3(groups), dim3(THREADS), lds_bytes, device->stream, a);
+    if ((rc = launch_mode<MODE_FUSED>(device, a, groups))) return rc;
+    return reduce_partials(device, L, a, groups);
+}
+
+// forward(mlp): every layer's pre-activations and outputs are written; the swizzled weight copies live in the device handle's scratch
+int rlt_mlp3_fused_forward(rlt_rocm_device* device, const rlt_dense_layer* L, int n, const float* x, int ldx, int batch) {
+    if (!shape_ok(L, n)) return RLT_E_UNSUPPORTED;
+    if ((size_t)LDS_FLOATS * sizeof(float) > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
+    if ((((uintptr_t)L[0].output | (uintptr_t)L[1].output) & 15) != 0) return RLT_E_UNSUPPORTED;
+    void* scratch = nullptr;
+    int rc = rlt_scratch(device, PREP_FLOATS * sizeof(float) + 256, &scratch);
+    if (rc) return rc;
+    float* prep = reinterpret_cast<float*>(((uintptr_t)scratch + 255) & ~(uintptr_t)255);
+    hipLaunchKernelGGL(mlp3_prepare_kernel, dim3(65536 / 256), dim3(256), 0, device->stream, L[0].weights, L[1].weights, L[0].in_dim, prep);
     if ((rc = rlt_launch_status(device))) return rc;
-    const int count = (int)gradient_count(L);
-    GradTargets T = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases, L[0].in_dim, L[2].out_dim};
-    hipLaunchKernelGGL(mlp3_reduce_kernel, dim3((count + 63) / 64), dim3(256), 0, device->stream, a.partial, groups, count, T);
-    return rlt_launch_status(device);
+    Mlp3Args a = base_args(L, x, ldx, batch, prep);
+    for (int l = 0; l < 3; l++) { a.act_pre[l] = L[l].pre_activations; a.act_out[l] = L[l].output; }
+    a.y = L[2].output; a.ldy = L[2].out_dim;
+    return launch_mode<MODE_FORWARD>(device, a, workgroups_for(batch));
+}
+
+// backward(mlp) with weight gradients and no input gradient; d_pre_last is the gradient at the last layer's pre-activations
+int rlt_mlp3_fused_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n, const float* x, int ldx, const float* d_pre_last, int ldd, int batch,
+                            void* workspace, size_t workspace_bytes) {
+    if (!shape_ok(L, n) || !L[0].output || !L[1].output) return RLT_E_UNSUPPORTED;
+    if (workspace_bytes < rlt_mlp3_fused_workspace_bytes(L, n, batch)) return RLT_E_UNSUPPORTED;
+    if ((size_t)LDS_FLOATS * sizeof(float) > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
+    if ((((uintptr_t)L[0].output | (uintptr_t)L[1].output) & 15) != 0) return RLT_E_UNSUPPORTED;      // the activations are read back 16 bytes at a time
+    float* prep = reinterpret_cast<float*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    hipLaunchKernelGGL(mlp3_prepare_kernel, dim3(65536 / 256), dim3(256), 0, device->stream, L[0].weights, L[1].weights, L[0].in_dim, prep);
+    int rc = rlt_launch_status(device);
+    if (rc) return rc;
+    Mlp3Args a = base_args(L, x, ldx, batch, prep);
+    a.d_output = d_pre_last; a.ldd = ldd;
+    a.act_out[0] = L[0].output; a.act_out[1] = L[1].output;
+    const int groups = workgroups_for(batch);
+    if ((rc = launch_mode<MODE_BACKWARD>(device, a, groups))) return rc;
+    return reduce_partials(device, L, a, groups);
 }

@@ -67,7 +67,54 @@ def test_fused_accumulates_and_tolerates_null_output(oracle, rocm):
     assert np.all(twice[0] == 0.0)                            # y == NULL: nothing written
 
 
-def test_fused_full_size_against_per_layer_path_and_linearity(rocm):
+def forward_then_backward(backend, dims, params, x, dy, ha, oa):
+    """The reference's call pattern: forward() (keeps every layer's pre-activations and outputs), then backward() of a given gradient."""
+    B = x.shape[0]
+    net = Mlp(backend, dims, params, B, ha, oa)
+    xd, dyd = backend.array(x), backend.array(dy)
+    ws, wsn = net.workspace()
+    backend.call("mlp_zero_gradient", net.layers, net.n)
+    backend.call("mlp_forward", net.layers, net.n, xd.ptr, dims[0], B)
+    backend.call("mlp_backward", net.layers, net.n, xd.ptr, dims[0], dyd.ptr, dims[-1], None, 0, B, 1, ws, wsn)
+    backend.sync()
+    return dict(pre=[p.numpy() for p in net.pre], out=[o.numpy() for o in net.out], grads=net.grads.numpy(), d_output=dyd.numpy(), offsets=net.offsets)
+
+
+@pytest.mark.parametrize("case", [(1024, 17, 6, "relu", "identity"), (4099, 17, 6, "tanh", "tanh"), (1100, 32, 16, "sigmoid", "sigmoid"), (2048, 1, 1, "fast_tanh", "identity")])
+def test_forward_then_backward_single_pass_modes_match_checker(oracle, rocm, case):
+    """forward() and backward() as separate calls at batch >= 1,024 run the single-pass kernel in its forward-only and backward-only modes:
+    every layer's pre-activations and outputs, the in-place d_pre of the last layer, and all gradients against the checker."""
+    print("case", case, flush=True)
+    B, I, O, ha, oa = case
+    dims = [I, 256, 256, O]
+    rng = np.random.default_rng(B + I)
+    params = helpers.random_params(rng, dims)
+    x = rng.standard_normal((B, I)).astype(np.float32); dy = rng.standard_normal((B, O)).astype(np.float32)
+    want, got = forward_then_backward(oracle, dims, params, x, dy, ha, oa), forward_then_backward(rocm, dims, params, x, dy, ha, oa)
+    for l in range(3):
+        assert rel_err(got["pre"][l], want["pre"][l]) <= TOL and rel_err(got["out"][l], want["out"][l]) <= TOL, l
+    assert rel_err(got["d_output"], want["d_output"]) <= TOL          # backward leaves the gradient at the last pre-activations there
+    for (off, nw, nb) in want["offsets"]:
+        ew = rel_err(got["grads"][off:off + nw], want["grads"][off:off + nw]); eb = rel_err(got["grads"][off + nw:off + nw + nb], want["grads"][off + nw:off + nw + nb])
+        assert ew <= TOL and eb <= TOL, (off, ew, eb)
+
+
+def test_single_pass_modes_full_size_against_per_layer_kernels(rocm, monkeypatch):
+    """Batch 65,536: forward() + backward() through the single-pass modes against the same calls kept on the per-layer kernels."""
+    B, dims = 65536, [17, 256, 256, 6]
+    rng = np.random.default_rng(12)
+    params = helpers.random_params(rng, dims)
+    x = rng.standard_normal((B, 17)).astype(np.float32); dy = (rng.standard_normal((B, 6)) / B).astype(np.float32)
+    got = forward_then_backward(rocm, dims, params, x, dy, "relu", "identity")
+    monkeypatch.setenv("RLT_MLP_SINGLE_PASS", "0")
+    want = forward_then_backward(rocm, dims, params, x, dy, "relu", "identity")
+    for l in range(3):
+        assert rel_err(got["pre"][l], want["pre"][l]) <= TOL and rel_err(got["out"][l], want["out"][l]) <= TOL, l
+    for (off, nw, nb) in want["offsets"]:
+        assert rel_err(got["grads"][off:off + nw], want["grads"][off:off + nw]) <= TOL and rel_err(got["grads"][off + nw:off + nw + nb], want["grads"][off + nw:off + nw + nb]) <= TOL
+
+
+def test_fused_full_size_against_per_layer_path_and_linearity(rocm, monkeypatch):
     """Batch 65,536 (the benchmark shape): the checker would take minutes, so compare with the per-layer kernels of the same
     library (themselves checked against the checker at small sizes) and use linearity of the gradients in d_output."""
     B, dims = 65536, [17, 256, 256, 6]
@@ -76,6 +123,7 @@ def test_fused_full_size_against_per_layer_path_and_linearity(rocm):
     x = rng.standard_normal((B, 17)).astype(np.float32); dy = (rng.standard_normal((B, 6)) / B).astype(np.float32)
     y, g, offsets = run(rocm, dims, params, x, dy, "relu", "identity", False, 0.0)
     # per-layer path: forward (stores activations), backward
+    monkeypatch.setenv("RLT_MLP_SINGLE_PASS", "0")
     net = Mlp(rocm, dims, params, B)
     xd, dyd = rocm.array(x), rocm.array(dy)
     ws, wsn = net.workspace()
