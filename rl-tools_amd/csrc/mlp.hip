@@ -4,6 +4,7 @@
 #include <cstdlib>
 #include "gemm.h"
 #include "mlp_fused.h"
+#include "mlp_small.h"
 
 namespace {
 
@@ -202,6 +203,10 @@ int rlt_rocm_mlp_forward_backward(rlt_rocm_device* device, const rlt_dense_layer
     {
         // one pass over the batch with on-chip activations where the network has the shape that kernel is built for
         const int rc = rlt_mlp3_fused_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, workspace, workspace_bytes);
+        if (rc != RLT_E_UNSUPPORTED) return rc;
+    }
+    if (single_pass_enabled()) {
+        const int rc = rlt_mlp3s_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch);
         if (rc != RLT_E_UNSUPPORTED) return rc;
     }
     // carve private activation storage out of the workspace

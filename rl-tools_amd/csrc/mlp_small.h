@@ -1,0 +1,27 @@
+// Single-pass forward + backward of a 3-layer MLP in -> 64 -> 64 -> out (mlp_small.hip).
+#pragma once
+#include "common.h"
+
+// true if the network has the shape the kernel is built for: 3 layers, in <= 128, both hidden widths 64 with the same activation
+// (relu, tanh or fast_tanh), out <= 16 with an activation whose derivative follows from the output
+bool rlt_mlp3s_supported(const rlt_dense_layer* layers, int n_layers);
+
+// same contract as rlt_rocm_mlp_forward_backward (partial sums live in the device handle's scratch); RLT_E_UNSUPPORTED if the shape does not fit
+int rlt_mlp3s_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy,
+                               const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch);
+
+// PPO actor pass (rl/algorithms/ppo/operations_generic.h:203-285): forward, the clipped-surrogate gradient per sample, backward. `stats` =
+// {advantage mean, advantage std} on the device. Means go to `means` [batch x action_dim]; weight gradients are accumulated into the layers,
+// the surrogate part of the log_std gradient plus `log_std_gradient_offset` into d_log_std (if non-NULL).
+int rlt_mlp3s_ppo_actor(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* means, int ld_means,
+                        const float* log_std, const float* actions, int ld_actions, const float* log_probs, int ld_lp, const float* advantages, int ld_adv,
+                        const float* stats, const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset, int batch);
+
+// The same actor pass and the critic's forward + MSE gradient + backward (:289-300) in ONE launch, each network on half of the compute units. The
+// gradients are OVERWRITTEN (what zero_gradient followed by backward leaves), so the caller skips zeroing them. RLT_E_UNSUPPORTED unless both networks
+// have the supported shape, the same hidden activation and input widths on the same side of 32.
+int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* actor, int n_actor, const float* x, int ldx, float* means, int ld_means,
+                               const float* log_std, const float* actions, int ld_actions, const float* log_probs, int ld_lp, const float* advantages, int ld_adv,
+                               const float* stats, const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset,
+                               const rlt_dense_layer* critic, int n_critic, const float* x_critic, int ldx_critic, float* values, int ld_values,
+                               const float* target_values, int ld_targets, float mse_scale, int batch);

@@ -1,0 +1,542 @@
+// Single-pass forward + backward of a 3-layer MLP in -> 64 -> 64 -> out for the narrow networks of PPO, TD3 and SAC
+// (nn_models/mlp/operations_generic.h:128-181 forward, :183-260 backward; nn/layers/dense/operations_generic.h:98-260).
+//
+// A workgroup of four wavefronts takes 64 batch rows per round. The work is split two ways:
+//   by rows      each wavefront runs its own 16 rows through the three layers, the loss and the input-gradient products
+//                  h1 = f(x W1^T + b1), h2 = f(h1 W2^T + b2), y = g(h2 W3^T + b3), d_pre3 from the caller's d_output / an MSE target / PPO's
+//                  clipped surrogate, d_pre2 = (d_pre3 W3) f'(h2), d_pre1 = (d_pre2 W2) f'(h1)
+//   by columns   for the weight gradients dW3 += d_pre3^T h2, dW2 += d_pre2^T h1, dW1 += d_pre1^T x the reduction runs over all 64 rows of the
+//                  round, and wavefront w owns the 16 output rows 16 w .. 16 w + 15 of dW1 and dW2 and 16 columns of dW3
+// so every accumulator tile of a weight gradient lives in exactly one wavefront's registers for the whole kernel (8 + 4 + 1 tiles), no sums
+// are exchanged between wavefronts, and a workgroup writes one block of partial sums at the end, which a second kernel adds to the layers'
+// gradients in workgroup order: the result does not depend on scheduling. Activations and gradients of the round sit in LDS in the layouts
+// v_mfma_f32_16x16x4_f32 wants (lane l = r + 16 kk feeds A[r][kk] and B[kk][r] and receives D[4 kk + v][r], v = 0..3); the weights are staged
+// once per workgroup in LDS (padded rows, read as both W and W^T). Four workgroup barriers per round order the two kinds of phase.
+// Bound: the fp32 matrix pipe, 2 (in + 64 + out) 64 flop per row forward and twice that backward less the input gradient of layer 1.
+#include "mlp_small.h"
+
+namespace {
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) float* lptr;
+constexpr int H = 64, HS = H + 1, WAVES = 4, ROWS = 16 * WAVES, THREADS = 64 * WAVES, MAX_IN = 128, MAX_OUT = 16, MAX_NT1 = MAX_IN / 16, D3S = MAX_OUT + 1,
+              N_EXTRA = 16, N_SUMS = 2 * H + MAX_OUT + N_EXTRA;
+enum { LOSS_GIVEN = 0, LOSS_MSE = 1, LOSS_PPO = 2 };
+
+struct SmallArgs {
+    const float* x; int ldx, batch, in, out, act3;
+    const float *W1, *b1, *W2, *b2, *W3, *b3;
+    float* y; int ldy;
+    int loss;
+    const float* d_output; int ldd;
+    const float* target; int ldt; float mse_scale;
+    const float* log_std; const float* actions; int ld_actions; const float* log_probs; int ld_lp; const float* advantages; int ld_adv; const float* stats;
+    float epsilon_clip, advantage_epsilon; int normalize_advantage;
+    float* partial; int count;      // per workgroup: dW1 [64 x in], db1 [64], dW2 [64 x 64], db2 [64], dW3 [out x 64], db3 [out], extra [16]
+};
+
+__device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+template <int CTRL>
+__device__ __forceinline__ float dpp(float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true)); }
+__device__ __forceinline__ float row16_sum(float x) { x += dpp<0xB1>(x); x += dpp<0x4E>(x); x += dpp<0x141>(x); x += dpp<0x140>(x); return x; }
+// lanes of one wavefront exchange data through LDS: the hardware executes a wavefront's LDS instructions in order, the fences keep
+// the compiler from moving them across
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+// sum over the four lane groups (lanes r, r + 16, r + 32, r + 48), in a fixed order
+__device__ __forceinline__ float groups_sum(float v) { v += __shfl_xor(v, 16, 64); v += __shfl_xor(v, 32, 64); return v; }
+
+// LDS: W1 [64][SX], W2 [64][HS], W3 [16][HS], then per round x [64][SX], h1 [64][HS], h2 [64][HS], g2 [64][HS], d3 [64][D3S]; SX = 16 nt1c + 1
+constexpr size_t lds_floats(int nt1c) {
+    const int sx = 16 * nt1c + 1;
+    return (size_t)H * sx + H * HS + MAX_OUT * HS + (size_t)ROWS * (sx + 3 * HS + D3S);
+}
+
+#ifdef MLP3S_TIMING
+__device__ unsigned long long mlp3s_stamps[32];
+#define STAMP(i) do { if (blockIdx.x == 0 && threadIdx.x == 0) mlp3s_stamps[i] = clock64(); } while (0)
+#else
+#define STAMP(i)
+#endif
+
+// global loads of one tile of 16 rows, issued together: the inputs (lane = column, up to two columns per lane) and what the loss needs of the
+// rows this lane will hold after the forward pass (rows 4 kk + v, column r); rows and columns beyond the extent are clamped here and masked later
+struct TileRegs { float xa[16], xb[16], in0[4], in1[4], in2[4]; };
+__device__ __forceinline__ void request_tile(const SmallArgs& A, int tile, int lane, TileRegs& T) {
+    const int row0 = tile * 16, r = lane & 15, kk = lane >> 4;
+    const int c0 = min(lane, A.in - 1), c1 = min(64 + lane, A.in - 1), c = min(r, A.out - 1);
+#pragma unroll
+    for (int row = 0; row < 16; row++) {
+        const float* src = A.x + (size_t)min(row0 + row, A.batch - 1) * A.ldx;
+        T.xa[row] = src[c0];
+        T.xb[row] = A.in > 64 ? src[c1] : 0.f;
+    }
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const size_t row = (size_t)min(row0 + 4 * kk + v, A.batch - 1);
+        T.in0[v] = T.in1[v] = T.in2[v] = 0.f;
+        if (A.loss == LOSS_GIVEN) T.in0[v] = A.d_output[row * A.ldd + c];
+        else if (A.loss == LOSS_MSE) T.in0[v] = A.target[row * A.ldt + c];
+        else { T.in0[v] = A.actions[row * A.ld_actions + c]; T.in1[v] = A.advantages[row * A.ld_adv]; T.in2[v] = A.log_probs[row * A.ld_lp]; }
+    }
+}
+
+// ACT_H: hidden activation; NT1C: number of 16-column tiles of dW1 the code is unrolled for (>= the NT1 the input width needs; the surplus
+// tiles multiply zero columns and are never stored). Both are compile-time constants: a matrix instruction under a run-time
+// condition makes the compiler carry both versions of its accumulator.
+// One launch can carry two networks (PPO's actor and critic on the same minibatch): workgroups [0, groups0) work on A0, the rest on A1.
+template <int ACT_H, int NT1C>
+__global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs A1, int groups0) {
+    extern __shared__ float lds_raw[];
+    const bool second = (int)blockIdx.x >= groups0;
+    const SmallArgs& A = second ? A1 : A0;
+    const int block = second ? blockIdx.x - groups0 : blockIdx.x, n_blocks = second ? gridDim.x - groups0 : groups0;
+    const int lane = threadIdx.x & 63, r = lane & 15, kk = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);      // wavefront-uniform: addresses derived from it are computed on the scalar unit
+    const int IN = A.in, OUT = A.out, NT1 = (IN + 15) >> 4;
+    constexpr int SX = 16 * NT1C + 1;        // row stride of the input tile and of W1 in LDS: a constant, so that LDS offsets fold into the instructions
+    const lptr w1s = (lptr)lds_raw, w2s = w1s + H * SX, w3s = w2s + H * HS;
+    const lptr xs_all = w3s + MAX_OUT * HS, h1s_all = xs_all + ROWS * SX, h2s_all = h1s_all + ROWS * HS, g2s_all = h2s_all + ROWS * HS, d3s_all = g2s_all + ROWS * HS;
+    const lptr xs = xs_all + 16 * wave * SX, h1s = h1s_all + 16 * wave * HS, h2s = h2s_all + 16 * wave * HS, g2s = g2s_all + 16 * wave * HS, d3s = d3s_all + 16 * wave * D3S;
+    const int n_tiles = (A.batch + 15) >> 4, n_rounds = (n_tiles + WAVES - 1) / WAVES;
+
+    STAMP(0);
+    // the first tile's loads go out ahead of the weights'; a wavefront whose tile lies beyond the batch computes on clamped rows and masks them
+    TileRegs T;
+    request_tile(A, min(block * WAVES + wave, n_tiles - 1), lane, T);
+    float b1r[4], b2r[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) { b1r[nt] = A.b1[16 * nt + r]; b2r[nt] = A.b2[16 * nt + r]; }
+    const float b3r = A.b3[min(r, OUT - 1)];
+    float ls = 0.f, adv_mean = 0.f, adv_std = 0.f;
+    if (A.loss == LOSS_PPO) {
+        ls = A.log_std[min(r, OUT - 1)];
+        if (A.normalize_advantage) { adv_mean = A.stats[0]; adv_std = A.stats[1]; }
+    }
+    // weights into LDS, rows padded to SX (zero beyond the input width, so the padded reduction steps add nothing); every load is in flight
+    // before the first is stored
+    {
+        float v1[H / WAVES][2], v2[H * H / THREADS], v3[MAX_OUT * H / THREADS];
+#pragma unroll
+        for (int j = 0; j < H / WAVES; j++) {
+            const float* src = A.W1 + (size_t)(wave * (H / WAVES) + j) * IN;
+            v1[j][0] = src[min(lane, IN - 1)];
+            v1[j][1] = IN > 64 ? src[min(64 + lane, IN - 1)] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < H * H / THREADS; u++) v2[u] = A.W2[u * THREADS + threadIdx.x];
+#pragma unroll
+        for (int u = 0; u < MAX_OUT * H / THREADS; u++) v3[u] = A.W3[min(u * THREADS + (int)threadIdx.x, OUT * H - 1)];
+#pragma unroll
+        for (int j = 0; j < H / WAVES; j++) {
+            const lptr dst = w1s + (wave * (H / WAVES) + j) * SX;
+            if (lane < SX) dst[lane] = lane < IN ? v1[j][0] : 0.f;
+            if (64 + lane < SX) dst[64 + lane] = 64 + lane < IN ? v1[j][1] : 0.f;
+            if (lane == 0 && SX > 128) dst[128] = 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < H * H / THREADS; u++) { const int i = u * THREADS + threadIdx.x; w2s[(i >> 6) * HS + (i & 63)] = v2[u]; }
+#pragma unroll
+        for (int u = 0; u < MAX_OUT * H / THREADS; u++) { const int i = u * THREADS + threadIdx.x; w3s[(i >> 6) * HS + (i & 63)] = (i >> 6) < OUT ? v3[u] : 0.f; }
+    }
+    const float sd = expf(ls);
+    rlt_lds_barrier();
+    STAMP(1);
+
+    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    // this wavefront's share of the weight gradients: rows 16 wave + 4 kk + v of dW1 (columns 16 nt + r) and of dW2, columns 16 wave + r of dW3 (rows 4 kk + v)
+    floatx4 aW1[NT1C], aW2[4], aW3a = zero4, aW3b = zero4;
+#pragma unroll
+    for (int nt = 0; nt < NT1C; nt++) aW1[nt] = zero4;
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) aW2[nt] = zero4;
+    float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f}, s3 = 0.f, gls = 0.f;      // bias gradients and the log_std gradient over this wavefront's rows
+
+    for (int round = block; round < n_rounds; round += n_blocks) {
+        const int tile = round * WAVES + wave, row0 = tile * 16;
+        // inputs of the tile into LDS, zero beyond the batch and beyond the input width
+#pragma unroll
+        for (int row = 0; row < 16; row++) {
+            const bool rok = row0 + row < A.batch;
+            if (lane < 16 * NT1C) xs[row * SX + lane] = (rok && lane < IN) ? T.xa[row] : 0.f;
+            if (64 + lane < 16 * NT1C) xs[row * SX + 64 + lane] = (rok && 64 + lane < IN) ? T.xb[row] : 0.f;
+        }
+        float in0[4], in1[4], in2[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) { in0[v] = T.in0[v]; in1[v] = T.in1[v]; in2[v] = T.in2[v]; }
+        wave_sync();
+        // the next round's loads travel while this one is computed (the last round asks for its own rows again)
+        request_tile(A, min((round + n_blocks) * WAVES + wave, n_tiles - 1), lane, T);
+        STAMP(2);
+
+        // layer 1: groups of four reduction steps, the operands of the next group requested before this group's matrix instructions
+        floatx4 acc[4] = {zero4, zero4, zero4, zero4};
+        {
+            float a_c[4], b_c[4][4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                a_c[q] = xs[r * SX + 4 * q + kk];
+#pragma unroll
+                for (int nt = 0; nt < 4; nt++) b_c[q][nt] = w1s[(16 * nt + r) * SX + 4 * q + kk];
+            }
+            for (int g = 0; g < NT1; g++) {
+                const int gn = min(g + 1, NT1 - 1);
+                float a_n[4], b_n[4][4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    a_n[q] = xs[r * SX + 16 * gn + 4 * q + kk];
+#pragma unroll
+                    for (int nt = 0; nt < 4; nt++) b_n[q][nt] = w1s[(16 * nt + r) * SX + 16 * gn + 4 * q + kk];
+                }
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+#pragma unroll
+                    for (int nt = 0; nt < 4; nt++) acc[nt] = mfma16(a_c[q], b_c[q][nt], acc[nt]);
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    a_c[q] = a_n[q];
+#pragma unroll
+                    for (int nt = 0; nt < 4; nt++) b_c[q][nt] = b_n[q][nt];
+                }
+            }
+        }
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) h1s[(4 * kk + v) * HS + 16 * nt + r] = rlt_act(acc[nt][v] + b1r[nt], ACT_H);
+        wave_sync();
+        STAMP(3);
+
+        // layer 2
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) acc[nt] = zero4;
+#pragma unroll
+        for (int s = 0; s < 16; s++) {
+            const float a = h1s[r * HS + 16 * kk + s];
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) acc[nt] = mfma16(a, w2s[(16 * nt + r) * HS + 16 * kk + s], acc[nt]);
+        }
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) h2s[(4 * kk + v) * HS + 16 * nt + r] = rlt_act(acc[nt][v] + b2r[nt], ACT_H);
+        wave_sync();
+        STAMP(4);
+
+        // layer 3 (two chains of matrix instructions) and the gradient at its pre-activations
+        floatx4 y0 = zero4, y1 = zero4;
+#pragma unroll
+        for (int s = 0; s < 16; s += 2) {
+            y0 = mfma16(h2s[r * HS + 16 * kk + s], w3s[r * HS + 16 * kk + s], y0);
+            y1 = mfma16(h2s[r * HS + 16 * kk + s + 1], w3s[r * HS + 16 * kk + s + 1], y1);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int row = row0 + 4 * kk + v;
+            const bool ok = row < A.batch && r < OUT;
+            const float yv = rlt_act((y0[v] + y1[v]) + b3r, A.act3);
+            if (A.y && ok) A.y[(size_t)row * A.ldy + r] = yv;
+            float d = 0.f;
+            if (A.loss == LOSS_GIVEN) d = in0[v];
+            else if (A.loss == LOSS_MSE) d = (yv - in0[v]) * A.mse_scale;
+            else {
+                // per sample (rl/algorithms/ppo/operations_generic.h:205-269): log-probability of the rollout action under the current
+                // policy (random/operations_generic.h:73-96), ratio, clipping, d loss / d mean and the surrogate part of d loss / d log_std
+                const float value = in0[v];
+                const float pre = (value - yv) / sd;
+                const float lp = row16_sum(ok ? (-0.9189385332046727f - ls) - 0.5f * pre * pre : 0.f);
+                float advantage = in1[v];
+                if (A.normalize_advantage) advantage = (advantage - adv_mean) / (adv_std + A.advantage_epsilon);
+                const float ratio = expf(lp - in2[v]);
+                const float clipped_ratio = fminf(fmaxf(ratio, 1.0f - A.epsilon_clip), 1.0f + A.epsilon_clip);
+                const bool clipped = ratio != clipped_ratio;
+                const bool ratio_min_switch = ratio * advantage - clipped_ratio * advantage <= 0.0f;
+                const float d_surrogate_d_ratio = ratio_min_switch ? advantage : (clipped ? 0.0f : advantage);
+                const float d_loss_d_lp = (-1.0f / (float)A.batch) * d_surrogate_d_ratio * ratio;
+                if (ok) { d = d_loss_d_lp * (pre / sd); gls += d_loss_d_lp * (pre * pre - 1.0f); }
+            }
+            const float dp = ok ? d * rlt_dact_from_output(yv, A.act3) : 0.f;
+            s3 += dp;
+            d3s[(4 * kk + v) * D3S + r] = dp;
+        }
+        rlt_lds_barrier();      // every wavefront's h2 and d_pre3 are in place
+        STAMP(5);
+
+        // dW3 (columns 16 wave + r) += d_pre3^T h2 over the 64 rows, two chains
+        {
+            float a_c = d3s_all[kk * D3S + r], b_c = h2s_all[kk * HS + 16 * wave + r];
+#pragma unroll
+            for (int ks = 0; ks < ROWS / 4; ks++) {
+                const int kn = min(ks + 1, ROWS / 4 - 1);
+                const float a_n = d3s_all[(4 * kn + kk) * D3S + r], b_n = h2s_all[(4 * kn + kk) * HS + 16 * wave + r];
+                if (ks & 1) aW3b = mfma16(a_c, b_c, aW3b); else aW3a = mfma16(a_c, b_c, aW3a);
+                a_c = a_n; b_c = b_n;
+            }
+        }
+        // d_pre2 = (d_pre3 W3) f'(h2) for the wavefront's own rows, into g2
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) acc[nt] = zero4;
+#pragma unroll
+        for (int ks = 0; ks < MAX_OUT / 4; ks++) {      // columns of d_pre3 and rows of W3 beyond `out` are zero
+            const float a = d3s[r * D3S + 4 * ks + kk];
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) acc[nt] = mfma16(a, w3s[(4 * ks + kk) * HS + 16 * nt + r], acc[nt]);
+        }
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int idx = (4 * kk + v) * HS + 16 * nt + r;
+                const float dp = acc[nt][v] * rlt_dact_from_output(h2s[idx], ACT_H);
+                g2s[idx] = dp; s2[nt] += dp;
+            }
+        rlt_lds_barrier();      // every wavefront's d_pre2 is in place, and nobody reads h2 any more
+        STAMP(6);
+
+        // dW2 (rows 16 wave + ..) += d_pre2^T h1 over the 64 rows
+        {
+            float a_c = g2s_all[kk * HS + 16 * wave + r], b_c[4];
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) b_c[nt] = h1s_all[kk * HS + 16 * nt + r];
+#pragma unroll
+            for (int ks = 0; ks < ROWS / 4; ks++) {
+                const int kn = min(ks + 1, ROWS / 4 - 1);
+                float a_n = g2s_all[(4 * kn + kk) * HS + 16 * wave + r], b_n[4];
+#pragma unroll
+                for (int nt = 0; nt < 4; nt++) b_n[nt] = h1s_all[(4 * kn + kk) * HS + 16 * nt + r];
+#pragma unroll
+                for (int nt = 0; nt < 4; nt++) aW2[nt] = mfma16(a_c, b_c[nt], aW2[nt]);
+                a_c = a_n;
+#pragma unroll
+                for (int nt = 0; nt < 4; nt++) b_c[nt] = b_n[nt];
+            }
+        }
+        // d_pre1 = (d_pre2 W2) f'(h1) for the wavefront's own rows, into the place of h2
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) acc[nt] = zero4;
+#pragma unroll
+        for (int s = 0; s < 16; s++) {
+            const float a = g2s[r * HS + 16 * kk + s];
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) acc[nt] = mfma16(a, w2s[(16 * kk + s) * HS + 16 * nt + r], acc[nt]);
+        }
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int idx = (4 * kk + v) * HS + 16 * nt + r;
+                const float dp = acc[nt][v] * rlt_dact_from_output(h1s[idx], ACT_H);
+                h2s[idx] = dp; s1[nt] += dp;
+            }
+        rlt_lds_barrier();      // every wavefront's d_pre1 is in place
+        STAMP(7);
+
+        // dW1 (rows 16 wave + ..) += d_pre1^T x over the 64 rows
+        {
+            float a_c = h2s_all[kk * HS + 16 * wave + r], b_c[NT1C];
+#pragma unroll
+            for (int nt = 0; nt < NT1C; nt++) b_c[nt] = xs_all[kk * SX + 16 * nt + r];
+#pragma unroll 4
+            for (int ks = 0; ks < ROWS / 4; ks++) {
+                const int kn = min(ks + 1, ROWS / 4 - 1);
+                float a_n = h2s_all[(4 * kn + kk) * HS + 16 * wave + r], b_n[NT1C];
+#pragma unroll
+                for (int nt = 0; nt < NT1C; nt++) b_n[nt] = xs_all[(4 * kn + kk) * SX + 16 * nt + r];
+#pragma unroll
+                for (int nt = 0; nt < NT1C; nt++) aW1[nt] = mfma16(a_c, b_c[nt], aW1[nt]);
+                a_c = a_n;
+#pragma unroll
+                for (int nt = 0; nt < NT1C; nt++) b_c[nt] = b_n[nt];
+            }
+        }
+        rlt_lds_barrier();      // the round's tiles may be overwritten
+    }
+    STAMP(8);
+
+    // the workgroup's block of partial sums: weight gradients straight from the registers that own them, ...
+    float* dst = A.partial + (size_t)block * A.count;
+    const int o_b1 = H * IN, o_w2 = o_b1 + H, o_b2 = o_w2 + H * H, o_w3 = o_b2 + H, o_b3 = o_w3 + OUT * H, o_ex = o_b3 + OUT;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int m = 16 * wave + 4 * kk + v;
+#pragma unroll
+        for (int nt = 0; nt < NT1C; nt++)
+            if (nt < NT1 && 16 * nt + r < IN) dst[m * IN + 16 * nt + r] = aW1[nt][v];
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) dst[o_w2 + m * H + 16 * nt + r] = aW2[nt][v];
+        if (4 * kk + v < OUT) dst[o_w3 + (4 * kk + v) * H + 16 * wave + r] = aW3a[v] + aW3b[v];
+    }
+    // ... the bias and log_std gradients, which every wavefront holds for its own rows, summed in wavefront order through LDS
+    const lptr sums = (lptr)lds_raw;        // [WAVES][N_SUMS]; the weights are no longer needed
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) { s1[nt] = groups_sum(s1[nt]); s2[nt] = groups_sum(s2[nt]); }
+    s3 = groups_sum(s3); gls = groups_sum(gls);
+    if (kk == 0) {
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) { sums[wave * N_SUMS + 16 * nt + r] = s1[nt]; sums[wave * N_SUMS + H + 16 * nt + r] = s2[nt]; }
+        sums[wave * N_SUMS + 2 * H + r] = s3; sums[wave * N_SUMS + 2 * H + MAX_OUT + r] = gls;
+    }
+    rlt_lds_barrier();
+    if (threadIdx.x < N_SUMS) {
+        const int i = threadIdx.x;
+        const float total = (sums[i] + sums[N_SUMS + i]) + (sums[2 * N_SUMS + i] + sums[3 * N_SUMS + i]);
+        if (i < H) dst[o_b1 + i] = total;
+        else if (i < 2 * H) dst[o_b2 + i - H] = total;
+        else if (i < 2 * H + MAX_OUT) { if (i - 2 * H < OUT) dst[o_b3 + i - 2 * H] = total; }
+        else dst[o_ex + i - 2 * H - MAX_OUT] = total;
+    }
+    STAMP(9);
+}
+
+// where the elements of a block of partial sums go; overwrite: gradient = sum instead of gradient += sum (for a caller that would zero the gradient first)
+struct SmallTargets { float* dW1; float* db1; float* dW2; float* db2; float* dW3; float* db3; float* extra; int in, out, n_extra; float extra_offset; int overwrite;
+                      const float* partial; int groups, count, blocks; };
+// gradient[e] (+)= sum over the workgroups' partial values, in workgroup order: a block of 256 threads handles 64 elements, four threads
+// per element each sum a quarter of the workgroups and are combined in a fixed order. Blocks [0, T0.blocks) serve T0, the rest T1.
+__global__ __launch_bounds__(256) void mlp3s_reduce_kernel(SmallTargets T0, SmallTargets T1) {
+    __shared__ float part[4][64];
+    const bool second = (int)blockIdx.x >= T0.blocks;
+    const SmallTargets& T = second ? T1 : T0;
+    const int el = threadIdx.x & 63, qtr = threadIdx.x >> 6, e = (second ? blockIdx.x - T0.blocks : blockIdx.x) * 64 + el, count = T.count, groups = T.groups;
+    const int ec = e < count ? e : count - 1;
+    const int per = (groups + 3) / 4, g0 = qtr * per, g1 = min(groups, g0 + per);
+    const float* __restrict__ partial = T.partial;
+    float s = 0.f;
+    for (int gb = g0; gb < g1; gb += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = partial[(size_t)min(gb + u, g1 - 1) * count + ec];
+#pragma unroll
+        for (int u = 0; u < 8; u++) s += (gb + u < g1) ? v[u] : 0.f;
+    }
+    part[qtr][el] = s;
+    __syncthreads();
+    if (qtr != 0 || e >= count) return;
+    float total = (part[0][el] + part[1][el]) + (part[2][el] + part[3][el]);
+    float* slot = nullptr;
+    int i = e, n = H * T.in;
+    if (i < n) slot = T.dW1 + i;
+    else if ((i -= n) < H) slot = T.db1 + i;
+    else if ((i -= H) < H * H) slot = T.dW2 + i;
+    else if ((i -= H * H) < H) slot = T.db2 + i;
+    else if ((i -= H) < T.out * H) slot = T.dW3 + i;
+    else if ((i -= T.out * H) < T.out) slot = T.db3 + i;
+    else if ((i -= T.out) < T.n_extra && T.extra) { slot = T.extra + i; total += T.extra_offset; }
+    if (slot) *slot = T.overwrite ? total : *slot + total;
+}
+
+bool hidden_act_ok(int a) { return a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH; }
+bool out_act_ok(int a) { return a == RLT_ACT_IDENTITY || a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH || a == RLT_ACT_SIGMOID; }
+
+struct SmallJob { const rlt_dense_layer* L; SmallArgs a; float* extra; int n_extra; float extra_offset; int overwrite; };
+
+bool shape_ok(const rlt_dense_layer* L, int n) {
+    return L && n == 3 && L[0].in_dim >= 1 && L[0].in_dim <= MAX_IN && L[0].out_dim == H && L[1].in_dim == H && L[1].out_dim == H && L[2].in_dim == H &&
+           L[2].out_dim >= 1 && L[2].out_dim <= MAX_OUT && L[0].activation == L[1].activation && hidden_act_ok(L[0].activation) && out_act_ok(L[2].activation);
+}
+int tile_bucket(int in) { return in <= 32 ? 2 : MAX_NT1; }
+
+// one or two networks in one launch; two only if they share the hidden activation and the input-width bucket
+int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
+    int groups[2] = {0, 0};
+    size_t offset[2] = {0, 0}, total = 0;
+    for (int j = 0; j < n_jobs; j++) {
+        const rlt_dense_layer* L = jobs[j].L; SmallArgs& a = jobs[j].a;
+        for (int l = 0; l < 3; l++) RLT_REQUIRE(L[l].weights && L[l].biases && L[l].d_weights && L[l].d_biases);
+        a.in = L[0].in_dim; a.out = L[2].out_dim; a.act3 = L[2].activation;
+        a.W1 = L[0].weights; a.b1 = L[0].biases; a.W2 = L[1].weights; a.b2 = L[1].biases; a.W3 = L[2].weights; a.b3 = L[2].biases;
+        a.count = H * a.in + H + H * H + H + a.out * H + a.out + N_EXTRA;
+        const int rounds = (a.batch + ROWS - 1) / ROWS, share = device->compute_units / n_jobs;
+        groups[j] = rounds < share ? rounds : share;
+        offset[j] = total; total += ((size_t)groups[j] * a.count + 63) & ~(size_t)63;
+    }
+    const int bucket = tile_bucket(jobs[0].a.in), act = jobs[0].L[0].activation;
+    if (n_jobs == 2 && (tile_bucket(jobs[1].a.in) != bucket || jobs[1].L[0].activation != act)) return RLT_E_UNSUPPORTED;
+    const size_t lds_bytes = lds_floats(bucket) * sizeof(float);
+    if (lds_bytes > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
+    void* scratch = nullptr;
+    int rc = rlt_scratch(device, total * sizeof(float), &scratch);
+    if (rc) return rc;
+    for (int j = 0; j < n_jobs; j++) jobs[j].a.partial = (float*)scratch + offset[j];
+    const SmallArgs& a0 = jobs[0].a; const SmallArgs& a1 = jobs[n_jobs - 1].a;
+    const int grid = groups[0] + (n_jobs == 2 ? groups[1] : 0);
+#define RLT_LAUNCH_SMALL(ACT, NT)                                                                                                                         \
+    do {                                                                                                                                                  \
+        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp3s_kernel<ACT, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
+        hipLaunchKernelGGL((mlp3s_kernel<ACT, NT>), dim3(grid), dim3(THREADS), lds_bytes, device->stream, a0, a1, groups[0]);                           \
+    } while (0)
+    switch (act) {
+        case RLT_ACT_RELU: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_RELU, 2); else RLT_LAUNCH_SMALL(RLT_ACT_RELU, MAX_NT1); break;
+        case RLT_ACT_TANH: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_TANH, 2); else RLT_LAUNCH_SMALL(RLT_ACT_TANH, MAX_NT1); break;
+        default: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_FAST_TANH, 2); else RLT_LAUNCH_SMALL(RLT_ACT_FAST_TANH, MAX_NT1); break;
+    }
+#undef RLT_LAUNCH_SMALL
+    if ((rc = rlt_launch_status(device))) return rc;
+    SmallTargets T[2] = {};
+    int blocks = 0;
+    for (int j = 0; j < n_jobs; j++) {
+        const rlt_dense_layer* L = jobs[j].L; const SmallArgs& a = jobs[j].a;
+        const int count = jobs[j].extra ? a.count : a.count - N_EXTRA;      // the extra slots sit at the end of a block
+        T[j] = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases, jobs[j].extra, a.in, a.out, jobs[j].n_extra,
+                jobs[j].extra_offset, jobs[j].overwrite, a.partial, groups[j], a.count, (count + 63) / 64};
+        blocks += T[j].blocks;
+    }
+    if (n_jobs == 1) T[1] = T[0];
+    hipLaunchKernelGGL(mlp3s_reduce_kernel, dim3(blocks), dim3(256), 0, device->stream, T[0], T[1]);
+    return rlt_launch_status(device);
+}
+
+SmallJob plain_job(const rlt_dense_layer* L, const float* x, int ldx, float* y, int ldy, const float* d_output, int ldd, const float* target, int ldt, float mse_scale,
+                   int batch, int overwrite) {
+    SmallJob job = {};
+    job.L = L; job.overwrite = overwrite;
+    SmallArgs& a = job.a;
+    a.x = x; a.ldx = ldx; a.batch = batch; a.y = y; a.ldy = ldy;
+    a.loss = target ? LOSS_MSE : LOSS_GIVEN; a.d_output = d_output; a.ldd = ldd; a.target = target; a.ldt = ldt; a.mse_scale = mse_scale;
+    return job;
+}
+SmallJob ppo_actor_job(const rlt_dense_layer* L, const float* x, int ldx, float* means, int ld_means, const float* log_std, const float* actions, int ld_actions,
+                       const float* log_probs, int ld_lp, const float* advantages, int ld_adv, const float* stats, const rlt_ppo_parameters* P, float* d_log_std,
+                       float log_std_gradient_offset, int batch, int overwrite) {
+    SmallJob job = {};
+    job.L = L; job.overwrite = overwrite; job.extra = d_log_std; job.n_extra = L[2].out_dim; job.extra_offset = log_std_gradient_offset;
+    SmallArgs& a = job.a;
+    a.x = x; a.ldx = ldx; a.batch = batch; a.y = means; a.ldy = ld_means;
+    a.loss = LOSS_PPO; a.log_std = log_std; a.actions = actions; a.ld_actions = ld_actions; a.log_probs = log_probs; a.ld_lp = ld_lp;
+    a.advantages = advantages; a.ld_adv = ld_adv; a.stats = stats;
+    a.epsilon_clip = P->epsilon_clip; a.advantage_epsilon = P->advantage_epsilon; a.normalize_advantage = P->normalize_advantage;
+    return job;
+}
+}  // namespace
+
+bool rlt_mlp3s_supported(const rlt_dense_layer* L, int n) { return shape_ok(L, n); }
+
+int rlt_mlp3s_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n, const float* x, int ldx, float* y, int ldy, const float* d_output, int ldd,
+                               const float* target, int ldt, float mse_scale, int batch) {
+    if (!shape_ok(L, n)) return RLT_E_UNSUPPORTED;
+    SmallJob job = plain_job(L, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, 0);
+    return launch(device, &job, 1);
+}
+
+int rlt_mlp3s_ppo_actor(rlt_rocm_device* device, const rlt_dense_layer* L, int n, const float* x, int ldx, float* means, int ld_means, const float* log_std,
+                        const float* actions, int ld_actions, const float* log_probs, int ld_lp, const float* advantages, int ld_adv, const float* stats,
+                        const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset, int batch) {
+    if (!shape_ok(L, n)) return RLT_E_UNSUPPORTED;
+    SmallJob job = ppo_actor_job(L, x, ldx, means, ld_means, log_std, actions, ld_actions, log_probs, ld_lp, advantages, ld_adv, stats, P, d_log_std,
+                                 log_std_gradient_offset, batch, 0);
+    return launch(device, &job, 1);
+}
+
+int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* actor, int n_actor, const float* x, int ldx, float* means, int ld_means,
+                               const float* log_std, const float* actions, int ld_actions, const float* log_probs, int ld_lp, const float* advantages, int ld_adv,
+                               const float* stats, const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset,
+                               const rlt_dense_layer* critic, int n_critic, const float* x_critic, int ldx_critic, float* values, int ld_values,
+                               const float* target_values, int ld_targets, float mse_scale, int batch) {
+    if (!shape_ok(actor, n_actor) || !shape_ok(critic, n_critic)) return RLT_E_UNSUPPORTED;
+    SmallJob jobs[2] = {ppo_actor_job(actor, x, ldx, means, ld_means, log_std, actions, ld_actions, log_probs, ld_lp, advantages, ld_adv, stats, P, d_log_std,
+                                      log_std_gradient_offset, batch, 1),
+                        plain_job(critic, x_critic, ldx_critic, values, ld_values, nullptr, 0, target_values, ld_targets, mse_scale, batch, 1)};
+    return launch(device, jobs, 2);
+}

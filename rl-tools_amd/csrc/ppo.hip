@@ -3,6 +3,8 @@
 // row = step * n_envs + env, rl/components/on_policy_runner/on_policy_runner.h:38-72) and :96-330 (train: per-sample loops on the
 // host around the networks' forward / backward passes).
 #include "common.h"
+#include <cstdlib>
+#include "mlp_small.h"
 
 namespace {
 // one lane per environment, reverse scan over the steps; at a fixed step adjacent lanes touch adjacent dataset rows
@@ -113,6 +115,8 @@ __global__ void ppo_log_std_gradient_kernel(const float* __restrict__ partial, i
     d_log_std[a] += s - entropy_coefficient;
 }
 
+// RLT_MLP_SINGLE_PASS=0 keeps the actor on the per-layer kernels (tests compare the two paths with each other)
+bool narrow_pass_enabled() { const char* v = std::getenv("RLT_MLP_SINGLE_PASS"); return !(v && v[0] == '0'); }
 bool ppo_agent_ok(const rlt_ppo_agent* A) {
     return A && A->actor && A->critic && A->n_actor_layers >= 1 && A->n_critic_layers >= 1 && A->log_std && A->actor_adam_tensors && A->critic_adam_tensors &&
            A->actor_age && A->critic_age && A->observation_dim >= 1 && A->observation_privileged_dim >= 1 && A->action_dim >= 1 && A->action_dim <= PPO_MAX_ACTION_DIM &&
@@ -192,15 +196,42 @@ extern "C" int rlt_rocm_ppo_train_minibatch(rlt_rocm_device* device, const rlt_p
                        ld, row_indices, B, O, OP, AD, obs, obsp, act, lp, adv, tgt);
     int rc = rlt_launch_status(device);
     if (rc) return rc;
-    if ((rc = rlt_rocm_mlp_zero_gradient(device, A->critic, A->n_critic_layers))) return rc;                      // :158
-    if ((rc = rlt_rocm_mlp_zero_gradient(device, A->actor, A->n_actor_layers))) return rc;                        // :159 (clears the log_std gradient too)
-    if (A->d_log_std) if ((rc = rlt_rocm_fill_f32(device, A->d_log_std, 1, AD, AD, 0.0f))) return rc;
-    if ((rc = rlt_rocm_mlp_forward(device, A->actor, A->n_actor_layers, obs, O, B))) return rc;                    // :203
-    const float* means = A->actor[A->n_actor_layers - 1].output;
-    if ((rc = ppo_surrogate_impl(device, means, AD, A->log_std, act, AD, lp, 1, adv, 1, P, d_act, AD, A->d_log_std, B, AD, scratch))) return rc;
-    if ((rc = rlt_rocm_mlp_backward(device, A->actor, A->n_actor_layers, obs, O, d_act, AD, nullptr, 0, B, 1, mlp_ws, mlp_ws_bytes))) return rc;   // :285
-    // critic: forward, MSE gradient with loss weight 0.5 (= (v - target)/batch), backward in one pass (:289-300)
-    if ((rc = rlt_rocm_mlp_forward_backward(device, A->critic, A->n_critic_layers, obsp, OP, values, 1, nullptr, 0, tgt, 1, 1.0f / (float)B, B, mlp_ws, mlp_ws_bytes))) return rc;
+    const bool narrow = narrow_pass_enabled() && rlt_mlp3s_supported(A->actor, A->n_actor_layers);
+    rc = RLT_E_UNSUPPORTED;
+    if (narrow && rlt_mlp3s_supported(A->critic, A->n_critic_layers)) {
+        // both networks in -> 64 -> 64 -> out: one launch runs the actor (forward, surrogate gradient, backward, :203-285) on half of the compute units
+        // and the critic (forward, MSE gradient with loss weight 0.5 = (v - target) / batch, backward, :289-300) on the other half, and its gradients
+        // replace the old ones, which is what zero_gradient (:158-159) followed by backward leaves. The means still land in the actor's last output
+        // buffer; the hidden layers' buffers are not written.
+        hipLaunchKernelGGL(ppo_advantage_stats_kernel, dim3(1), dim3(1024), 0, device->stream, adv, 1, B, P->normalize_advantage, scratch);
+        if ((rc = rlt_launch_status(device))) return rc;
+        rc = rlt_mlp3s_ppo_actor_critic(device, A->actor, A->n_actor_layers, obs, O, A->actor[A->n_actor_layers - 1].output, AD, A->log_std, act, AD, lp, 1, adv, 1,
+                                        scratch, P, P->learn_action_std ? A->d_log_std : nullptr, -P->action_entropy_coefficient,
+                                        A->critic, A->n_critic_layers, obsp, OP, values, 1, tgt, 1, 1.0f / (float)B, B);
+        if (rc && rc != RLT_E_UNSUPPORTED) return rc;
+        if (rc == 0 && A->d_log_std && !P->learn_action_std) if ((rc = rlt_rocm_fill_f32(device, A->d_log_std, 1, AD, AD, 0.0f))) return rc;
+    }
+    if (rc == RLT_E_UNSUPPORTED) {
+        if ((rc = rlt_rocm_mlp_zero_gradient(device, A->critic, A->n_critic_layers))) return rc;                      // :158
+        if ((rc = rlt_rocm_mlp_zero_gradient(device, A->actor, A->n_actor_layers))) return rc;                        // :159 (clears the log_std gradient too)
+        if (A->d_log_std) if ((rc = rlt_rocm_fill_f32(device, A->d_log_std, 1, AD, AD, 0.0f))) return rc;
+        rc = RLT_E_UNSUPPORTED;
+        if (narrow) {       // the actor alone in one kernel
+            hipLaunchKernelGGL(ppo_advantage_stats_kernel, dim3(1), dim3(1024), 0, device->stream, adv, 1, B, P->normalize_advantage, scratch);
+            if ((rc = rlt_launch_status(device))) return rc;
+            rc = rlt_mlp3s_ppo_actor(device, A->actor, A->n_actor_layers, obs, O, A->actor[A->n_actor_layers - 1].output, AD, A->log_std, act, AD, lp, 1, adv, 1, scratch, P,
+                                     P->learn_action_std ? A->d_log_std : nullptr, -P->action_entropy_coefficient, B);
+            if (rc && rc != RLT_E_UNSUPPORTED) return rc;
+        }
+        if (rc == RLT_E_UNSUPPORTED) {
+            if ((rc = rlt_rocm_mlp_forward(device, A->actor, A->n_actor_layers, obs, O, B))) return rc;                    // :203
+            const float* means = A->actor[A->n_actor_layers - 1].output;
+            if ((rc = ppo_surrogate_impl(device, means, AD, A->log_std, act, AD, lp, 1, adv, 1, P, d_act, AD, A->d_log_std, B, AD, scratch))) return rc;
+            if ((rc = rlt_rocm_mlp_backward(device, A->actor, A->n_actor_layers, obs, O, d_act, AD, nullptr, 0, B, 1, mlp_ws, mlp_ws_bytes))) return rc;   // :285
+        }
+        // critic: forward, MSE gradient with loss weight 0.5 (= (v - target)/batch), backward in one pass (:289-300)
+        if ((rc = rlt_rocm_mlp_forward_backward(device, A->critic, A->n_critic_layers, obsp, OP, values, 1, nullptr, 0, tgt, 1, 1.0f / (float)B, B, mlp_ws, mlp_ws_bytes))) return rc;
+    }
     if (out_critic_loss) if ((rc = rlt_rocm_mse_evaluate(device, values, 1, tgt, 1, B, 1, 1.0f, out_critic_loss))) return rc;                      // :303
     if ((rc = rlt_rocm_adam_step(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, 0.0f, nullptr))) return rc;  // :305
     return rlt_rocm_adam_step(device, A->critic_adam_tensors, A->n_critic_adam_tensors, &A->critic_adam, A->critic_age, 0.0f, nullptr);             // :306
