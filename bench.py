@@ -164,10 +164,9 @@ def bench_ppo(helpers, rocm, n_envs=4096, steps=128, epochs=4, minibatch=8192):
                   dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld, n_envs, steps, 0.99, 0.95, 0)
 
     def iteration():
-        for perm in perms:
-            for b in range(rows // minibatch):
-                rocm.call("ppo_train_minibatch", C.byref(agent.c), C.byref(pp), dd.offset(col["observations"]), dd.offset(col["observations"]), dd.offset(col["actions"]),
-                          dd.offset(col["action_log_probs"]), dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld, perm.offset(b * minibatch), None)
+        for perm in perms:      # one call per epoch: the reference's batch loop over the epoch's shuffled rows
+            rocm.call("ppo_train_epoch", C.byref(agent.c), C.byref(pp), dd.offset(col["observations"]), dd.offset(col["observations"]), dd.offset(col["actions"]),
+                      dd.offset(col["action_log_probs"]), dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld, perm.ptr, rows // minibatch, None)
     for _ in range(3):
         gae()
     rocm.sync()

@@ -474,6 +474,16 @@ int rlt_rocm_ppo_train_minibatch(rlt_rocm_device* device, const rlt_ppo_agent* a
                                  const float* action_log_probs, const float* advantages, const float* target_values, int ld,
                                  const uint32_t* row_indices, float* out_critic_loss);
 
+/* One epoch of train(): the batch loop rl/algorithms/ppo/operations_generic.h:156-318 over the rows that the epoch's shuffle
+ * (:126-155) put in place, given here as the permutation `row_indices` (device, n_minibatches x batch entries; minibatch i
+ * takes entries [i * batch, (i + 1) * batch)). Same result as n_minibatches calls of rlt_rocm_ppo_train_minibatch; the
+ * per-minibatch advantage statistics (:170-180) of the whole epoch are formed up front by one pair of launches.
+ * out_critic_losses (device, optional) receives n_minibatches values. */
+int rlt_rocm_ppo_train_epoch(rlt_rocm_device* device, const rlt_ppo_agent* agent, const rlt_ppo_parameters* parameters,
+                             const float* observations, const float* observations_privileged, const float* actions,
+                             const float* action_log_probs, const float* advantages, const float* target_values, int ld,
+                             const uint32_t* row_indices, int n_minibatches, float* out_critic_losses);
+
 /* --------------------------------------------------------------------- GRU -- */
 
 /* nn/layers/gru/layer.h:96-217 (LayerForward / LayerBackward / LayerGradient): gate order r, z, n along the 3H rows

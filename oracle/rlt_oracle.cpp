@@ -859,6 +859,20 @@ int rlt_oracle_ppo_train_minibatch(const rlt_ppo_agent* A, const rlt_ppo_paramet
     return adam_over(A->critic_adam_tensors, A->n_critic_adam_tensors, &A->critic_adam, A->critic_age);                              // :306
 }
 
+// One epoch of train(): the batch loop rl/algorithms/ppo/operations_generic.h:156-318 over the rows the epoch's shuffle (:126-155) put in place,
+// given here as a permutation; minibatch i takes entries [i * batch, (i + 1) * batch).
+int rlt_oracle_ppo_train_epoch(const rlt_ppo_agent* A, const rlt_ppo_parameters* P, const float* observations, const float* observations_privileged,
+                               const float* actions, const float* action_log_probs, const float* advantages, const float* target_values, int ld,
+                               const uint32_t* row_indices, int n_minibatches, float* out_critic_losses) {
+    if (!A || !row_indices || n_minibatches < 1) return RLT_E_INVALID_ARGUMENT;
+    for (int i = 0; i < n_minibatches; i++) {
+        const int rc = rlt_oracle_ppo_train_minibatch(A, P, observations, observations_privileged, actions, action_log_probs, advantages, target_values, ld,
+                                                      row_indices + (size_t)i * A->batch, out_critic_losses ? out_critic_losses + i : nullptr);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
 // The in-place dataset shuffle of train() (rl/algorithms/ppo/operations_generic.h:126-155) restated on a row-index array: for
 // each epoch, for i in [0, n): j = uniform_int(i, n-1) (std::uniform_int_distribution on the loop's std::mt19937, as
 // random/operations_cpu.h:26-29 does), swap(rows i, j). rng_state is the engine's text form (operator<<) and is advanced in place;

@@ -104,6 +104,11 @@ int rlt_oracle_ppo_surrogate_gradient(const float* action_means, int ld_means, c
 int rlt_oracle_ppo_train_minibatch(const rlt_ppo_agent* agent, const rlt_ppo_parameters* parameters, const float* observations,
                                    const float* observations_privileged, const float* actions, const float* action_log_probs,
                                    const float* advantages, const float* target_values, int ld, const uint32_t* row_indices, float* out_critic_loss);
+/* the batch loop of train() (rl/algorithms/ppo/operations_generic.h:156-318) over one epoch's permutation */
+int rlt_oracle_ppo_train_epoch(const rlt_ppo_agent* agent, const rlt_ppo_parameters* parameters, const float* observations,
+                               const float* observations_privileged, const float* actions, const float* action_log_probs,
+                               const float* advantages, const float* target_values, int ld, const uint32_t* row_indices, int n_minibatches,
+                               float* out_critic_losses);
 int rlt_oracle_gru_forward(const rlt_gru_layer* layer, const float* input, const uint8_t* reset, int sequence_length, int batch);
 int rlt_oracle_gru_backward(const rlt_gru_layer* layer, const float* input, float* d_output, float* d_input, const uint8_t* reset,
                             int sequence_length, int batch, int want_weight_gradients);

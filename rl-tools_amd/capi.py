@@ -179,6 +179,7 @@ PROTOTYPES = {
     "gru_backward": [C.POINTER(GruLayer), P, P, P, P, I, I, I, P, S],
     "ppo_surrogate_gradient": [P, I, P, P, I, P, I, P, I, C.POINTER(PpoParameters), P, I, P, I, I],
     "ppo_train_minibatch": [C.POINTER(PpoAgent), C.POINTER(PpoParameters), P, P, P, P, P, P, I, P, P],
+    "ppo_train_epoch": [C.POINTER(PpoAgent), C.POINTER(PpoParameters), P, P, P, P, P, P, I, P, I, P],
     "standardize_set_statistics": [P, P, P, P, I],
     "standardize_forward": [P, P, P, I, P, I, I, I],
     "standardize_backward_input": [P, P, I, P, I, I, I],

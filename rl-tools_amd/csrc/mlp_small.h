@@ -17,11 +17,16 @@ int rlt_mlp3s_ppo_actor(rlt_rocm_device* device, const rlt_dense_layer* layers, 
                         const float* log_std, const float* actions, int ld_actions, const float* log_probs, int ld_lp, const float* advantages, int ld_adv,
                         const float* stats, const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset, int batch);
 
-// The same actor pass and the critic's forward + MSE gradient + backward (:289-300) in ONE launch, each network on half of the compute units. The
-// gradients are OVERWRITTEN (what zero_gradient followed by backward leaves), so the caller skips zeroing them. RLT_E_UNSUPPORTED unless both networks
-// have the supported shape, the same hidden activation and input widths on the same side of 32.
-int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* actor, int n_actor, const float* x, int ldx, float* means, int ld_means,
-                               const float* log_std, const float* actions, int ld_actions, const float* log_probs, int ld_lp, const float* advantages, int ld_adv,
+// true if the two networks can share a launch: both of the supported shape, the same hidden activation, input widths on the same side of 32
+bool rlt_mlp3s_pair_supported(const rlt_dense_layer* a, int n_a, const rlt_dense_layer* b, int n_b);
+
+// The same actor pass and the critic's forward + MSE gradient + backward (:289-300) in ONE launch, each network on half of the compute units,
+// straight from the dataset: every input column has the dataset's row stride `ld`, and minibatch row b is dataset row rows[b] (rows == NULL: b).
+// Means [batch x action_dim] and values [batch] are written packed; out_critic_loss (optional, critic output width 1) receives
+// mse::evaluate(values, targets) = sum((v - t)^2) / batch. The gradients are OVERWRITTEN (what zero_gradient followed by backward
+// leaves), so the caller skips zeroing them. RLT_E_UNSUPPORTED unless rlt_mlp3s_pair_supported.
+int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* actor, int n_actor, const float* x, float* means, int ld_means,
+                               const float* log_std, const float* actions, const float* log_probs, const float* advantages,
                                const float* stats, const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset,
-                               const rlt_dense_layer* critic, int n_critic, const float* x_critic, int ldx_critic, float* values, int ld_values,
-                               const float* target_values, int ld_targets, float mse_scale, int batch);
+                               const rlt_dense_layer* critic, int n_critic, const float* x_critic, float* values, int ld_values,
+                               const float* target_values, float mse_scale, float* out_critic_loss, int ld, const uint32_t* rows, int batch);

@@ -24,6 +24,7 @@ enum { LOSS_GIVEN = 0, LOSS_MSE = 1, LOSS_PPO = 2 };
 
 struct SmallArgs {
     const float* x; int ldx, batch, in, out, act3;
+    const uint32_t* rows;           // optional: batch row b reads row rows[b] of x, d_output / target / actions / log_probs / advantages (y is written at row b)
     const float *W1, *b1, *W2, *b2, *W3, *b3;
     float* y; int ldy;
     int loss;
@@ -61,21 +62,27 @@ __device__ unsigned long long mlp3s_stamps[32];
 #define STAMP(i)
 #endif
 
+// lane l: the row of the input arrays that row (l & 15) of a tile reads; rows beyond the batch are clamped here and masked later
+__device__ __forceinline__ int tile_rows(const SmallArgs& A, int tile, int lane) {
+    const int b = min(tile * 16 + (lane & 15), A.batch - 1);
+    return A.rows ? (int)A.rows[b] : b;
+}
 // global loads of one tile of 16 rows, issued together: the inputs (lane = column, up to two columns per lane) and what the loss needs of the
-// rows this lane will hold after the forward pass (rows 4 kk + v, column r); rows and columns beyond the extent are clamped here and masked later
+// rows this lane will hold after the forward pass (rows 4 kk + v, column r); columns beyond the extent are clamped here and masked later.
+// `vrows` comes from tile_rows(), requested a round earlier so that nothing waits for it here.
 struct TileRegs { float xa[16], xb[16], in0[4], in1[4], in2[4]; };
-__device__ __forceinline__ void request_tile(const SmallArgs& A, int tile, int lane, TileRegs& T) {
-    const int row0 = tile * 16, r = lane & 15, kk = lane >> 4;
+__device__ __forceinline__ void request_tile(const SmallArgs& A, int vrows, int lane, TileRegs& T) {
+    const int r = lane & 15, kk = lane >> 4;
     const int c0 = min(lane, A.in - 1), c1 = min(64 + lane, A.in - 1), c = min(r, A.out - 1);
 #pragma unroll
     for (int row = 0; row < 16; row++) {
-        const float* src = A.x + (size_t)min(row0 + row, A.batch - 1) * A.ldx;
+        const float* src = A.x + (size_t)__builtin_amdgcn_readlane(vrows, row) * A.ldx;      // wavefront-uniform: scalar address arithmetic
         T.xa[row] = src[c0];
         T.xb[row] = A.in > 64 ? src[c1] : 0.f;
     }
 #pragma unroll
     for (int v = 0; v < 4; v++) {
-        const size_t row = (size_t)min(row0 + 4 * kk + v, A.batch - 1);
+        const size_t row = (size_t)__shfl(vrows, 4 * kk + v, 64);
         T.in0[v] = T.in1[v] = T.in2[v] = 0.f;
         if (A.loss == LOSS_GIVEN) T.in0[v] = A.d_output[row * A.ldd + c];
         else if (A.loss == LOSS_MSE) T.in0[v] = A.target[row * A.ldt + c];
@@ -103,9 +110,11 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
     const int n_tiles = (A.batch + 15) >> 4, n_rounds = (n_tiles + WAVES - 1) / WAVES;
 
     STAMP(0);
-    // the first tile's loads go out ahead of the weights'; a wavefront whose tile lies beyond the batch computes on clamped rows and masks them
+    // row indices of this wavefront's first two tiles, then the first tile's loads, ahead of the weights'; a wavefront whose tile lies beyond the
+    // batch computes on clamped rows and masks them
+    int rows_next = tile_rows(A, min(block * WAVES + wave, n_tiles - 1), lane), rows_after = tile_rows(A, min((block + n_blocks) * WAVES + wave, n_tiles - 1), lane);
     TileRegs T;
-    request_tile(A, min(block * WAVES + wave, n_tiles - 1), lane, T);
+    request_tile(A, rows_next, lane, T);
     float b1r[4], b2r[4];
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) { b1r[nt] = A.b1[16 * nt + r]; b2r[nt] = A.b2[16 * nt + r]; }
@@ -152,7 +161,7 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
     for (int nt = 0; nt < NT1C; nt++) aW1[nt] = zero4;
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) aW2[nt] = zero4;
-    float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f}, s3 = 0.f, gls = 0.f;      // bias gradients and the log_std gradient over this wavefront's rows
+    float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f}, s3 = 0.f, gls = 0.f;      // bias gradients and the extra sums (PPO: log_std gradient; MSE: squared error) over this wavefront's rows
 
     for (int round = block; round < n_rounds; round += n_blocks) {
         const int tile = round * WAVES + wave, row0 = tile * 16;
@@ -167,8 +176,10 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
 #pragma unroll
         for (int v = 0; v < 4; v++) { in0[v] = T.in0[v]; in1[v] = T.in1[v]; in2[v] = T.in2[v]; }
         wave_sync();
-        // the next round's loads travel while this one is computed (the last round asks for its own rows again)
-        request_tile(A, min((round + n_blocks) * WAVES + wave, n_tiles - 1), lane, T);
+        // the next round's loads travel while this one is computed, with row indices requested a round earlier (the last rounds ask for the last tile again)
+        rows_next = rows_after;
+        rows_after = tile_rows(A, min((round + 2 * n_blocks) * WAVES + wave, n_tiles - 1), lane);
+        request_tile(A, rows_next, lane, T);
         STAMP(2);
 
         // layer 1: groups of four reduction steps, the operands of the next group requested before this group's matrix instructions
@@ -240,7 +251,7 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
             if (A.y && ok) A.y[(size_t)row * A.ldy + r] = yv;
             float d = 0.f;
             if (A.loss == LOSS_GIVEN) d = in0[v];
-            else if (A.loss == LOSS_MSE) d = (yv - in0[v]) * A.mse_scale;
+            else if (A.loss == LOSS_MSE) { const float diff = yv - in0[v]; d = diff * A.mse_scale; if (ok) gls += diff * diff; }    // gls: the column's summed squared error
             else {
                 // per sample (rl/algorithms/ppo/operations_generic.h:205-269): log-probability of the rollout action under the current
                 // policy (random/operations_generic.h:73-96), ratio, clipping, d loss / d mean and the surrogate part of d loss / d log_std
@@ -391,7 +402,7 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
 }
 
 // where the elements of a block of partial sums go; overwrite: gradient = sum instead of gradient += sum (for a caller that would zero the gradient first)
-struct SmallTargets { float* dW1; float* db1; float* dW2; float* db2; float* dW3; float* db3; float* extra; int in, out, n_extra; float extra_offset; int overwrite;
+struct SmallTargets { float* dW1; float* db1; float* dW2; float* db2; float* dW3; float* db3; float* extra; int in, out, n_extra; float extra_scale, extra_offset; int overwrite;
                       const float* partial; int groups, count, blocks; };
 // gradient[e] (+)= sum over the workgroups' partial values, in workgroup order: a block of 256 threads handles 64 elements, four threads
 // per element each sum a quarter of the workgroups and are combined in a fixed order. Blocks [0, T0.blocks) serve T0, the rest T1.
@@ -423,14 +434,14 @@ __global__ __launch_bounds__(256) void mlp3s_reduce_kernel(SmallTargets T0, Smal
     else if ((i -= H * H) < H) slot = T.db2 + i;
     else if ((i -= H) < T.out * H) slot = T.dW3 + i;
     else if ((i -= T.out * H) < T.out) slot = T.db3 + i;
-    else if ((i -= T.out) < T.n_extra && T.extra) { slot = T.extra + i; total += T.extra_offset; }
+    else if ((i -= T.out) < T.n_extra && T.extra) { slot = T.extra + i; total = total * T.extra_scale + T.extra_offset; }
     if (slot) *slot = T.overwrite ? total : *slot + total;
 }
 
 bool hidden_act_ok(int a) { return a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH; }
 bool out_act_ok(int a) { return a == RLT_ACT_IDENTITY || a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH || a == RLT_ACT_SIGMOID; }
 
-struct SmallJob { const rlt_dense_layer* L; SmallArgs a; float* extra; int n_extra; float extra_offset; int overwrite; };
+struct SmallJob { const rlt_dense_layer* L; SmallArgs a; float* extra; int n_extra; float extra_scale, extra_offset; int overwrite; };
 
 bool shape_ok(const rlt_dense_layer* L, int n) {
     return L && n == 3 && L[0].in_dim >= 1 && L[0].in_dim <= MAX_IN && L[0].out_dim == H && L[1].in_dim == H && L[1].out_dim == H && L[2].in_dim == H &&
@@ -480,7 +491,7 @@ int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
         const rlt_dense_layer* L = jobs[j].L; const SmallArgs& a = jobs[j].a;
         const int count = jobs[j].extra ? a.count : a.count - N_EXTRA;      // the extra slots sit at the end of a block
         T[j] = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases, jobs[j].extra, a.in, a.out, jobs[j].n_extra,
-                jobs[j].extra_offset, jobs[j].overwrite, a.partial, groups[j], a.count, (count + 63) / 64};
+                jobs[j].extra_scale, jobs[j].extra_offset, jobs[j].overwrite, a.partial, groups[j], a.count, (count + 63) / 64};
         blocks += T[j].blocks;
     }
     if (n_jobs == 1) T[1] = T[0];
@@ -489,21 +500,21 @@ int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
 }
 
 SmallJob plain_job(const rlt_dense_layer* L, const float* x, int ldx, float* y, int ldy, const float* d_output, int ldd, const float* target, int ldt, float mse_scale,
-                   int batch, int overwrite) {
+                   int batch, int overwrite, const uint32_t* rows) {
     SmallJob job = {};
     job.L = L; job.overwrite = overwrite;
     SmallArgs& a = job.a;
-    a.x = x; a.ldx = ldx; a.batch = batch; a.y = y; a.ldy = ldy;
+    a.rows = rows; a.x = x; a.ldx = ldx; a.batch = batch; a.y = y; a.ldy = ldy;
     a.loss = target ? LOSS_MSE : LOSS_GIVEN; a.d_output = d_output; a.ldd = ldd; a.target = target; a.ldt = ldt; a.mse_scale = mse_scale;
     return job;
 }
 SmallJob ppo_actor_job(const rlt_dense_layer* L, const float* x, int ldx, float* means, int ld_means, const float* log_std, const float* actions, int ld_actions,
                        const float* log_probs, int ld_lp, const float* advantages, int ld_adv, const float* stats, const rlt_ppo_parameters* P, float* d_log_std,
-                       float log_std_gradient_offset, int batch, int overwrite) {
+                       float log_std_gradient_offset, int batch, int overwrite, const uint32_t* rows) {
     SmallJob job = {};
-    job.L = L; job.overwrite = overwrite; job.extra = d_log_std; job.n_extra = L[2].out_dim; job.extra_offset = log_std_gradient_offset;
+    job.L = L; job.overwrite = overwrite; job.extra = d_log_std; job.n_extra = L[2].out_dim; job.extra_scale = 1.0f; job.extra_offset = log_std_gradient_offset;
     SmallArgs& a = job.a;
-    a.x = x; a.ldx = ldx; a.batch = batch; a.y = means; a.ldy = ld_means;
+    a.rows = rows; a.x = x; a.ldx = ldx; a.batch = batch; a.y = means; a.ldy = ld_means;
     a.loss = LOSS_PPO; a.log_std = log_std; a.actions = actions; a.ld_actions = ld_actions; a.log_probs = log_probs; a.ld_lp = ld_lp;
     a.advantages = advantages; a.ld_adv = ld_adv; a.stats = stats;
     a.epsilon_clip = P->epsilon_clip; a.advantage_epsilon = P->advantage_epsilon; a.normalize_advantage = P->normalize_advantage;
@@ -516,7 +527,7 @@ bool rlt_mlp3s_supported(const rlt_dense_layer* L, int n) { return shape_ok(L, n
 int rlt_mlp3s_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n, const float* x, int ldx, float* y, int ldy, const float* d_output, int ldd,
                                const float* target, int ldt, float mse_scale, int batch) {
     if (!shape_ok(L, n)) return RLT_E_UNSUPPORTED;
-    SmallJob job = plain_job(L, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, 0);
+    SmallJob job = plain_job(L, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, 0, nullptr);
     return launch(device, &job, 1);
 }
 
@@ -525,18 +536,23 @@ int rlt_mlp3s_ppo_actor(rlt_rocm_device* device, const rlt_dense_layer* L, int n
                         const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset, int batch) {
     if (!shape_ok(L, n)) return RLT_E_UNSUPPORTED;
     SmallJob job = ppo_actor_job(L, x, ldx, means, ld_means, log_std, actions, ld_actions, log_probs, ld_lp, advantages, ld_adv, stats, P, d_log_std,
-                                 log_std_gradient_offset, batch, 0);
+                                 log_std_gradient_offset, batch, 0, nullptr);
     return launch(device, &job, 1);
 }
 
-int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* actor, int n_actor, const float* x, int ldx, float* means, int ld_means,
-                               const float* log_std, const float* actions, int ld_actions, const float* log_probs, int ld_lp, const float* advantages, int ld_adv,
+bool rlt_mlp3s_pair_supported(const rlt_dense_layer* a, int n_a, const rlt_dense_layer* b, int n_b) {
+    return shape_ok(a, n_a) && shape_ok(b, n_b) && a[0].activation == b[0].activation && tile_bucket(a[0].in_dim) == tile_bucket(b[0].in_dim);
+}
+
+int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* actor, int n_actor, const float* x, float* means, int ld_means,
+                               const float* log_std, const float* actions, const float* log_probs, const float* advantages,
                                const float* stats, const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset,
-                               const rlt_dense_layer* critic, int n_critic, const float* x_critic, int ldx_critic, float* values, int ld_values,
-                               const float* target_values, int ld_targets, float mse_scale, int batch) {
-    if (!shape_ok(actor, n_actor) || !shape_ok(critic, n_critic)) return RLT_E_UNSUPPORTED;
-    SmallJob jobs[2] = {ppo_actor_job(actor, x, ldx, means, ld_means, log_std, actions, ld_actions, log_probs, ld_lp, advantages, ld_adv, stats, P, d_log_std,
-                                      log_std_gradient_offset, batch, 1),
-                        plain_job(critic, x_critic, ldx_critic, values, ld_values, nullptr, 0, target_values, ld_targets, mse_scale, batch, 1)};
+                               const rlt_dense_layer* critic, int n_critic, const float* x_critic, float* values, int ld_values,
+                               const float* target_values, float mse_scale, float* out_critic_loss, int ld, const uint32_t* rows, int batch) {
+    if (!rlt_mlp3s_pair_supported(actor, n_actor, critic, n_critic) || (out_critic_loss && critic[2].out_dim != 1)) return RLT_E_UNSUPPORTED;
+    SmallJob jobs[2] = {ppo_actor_job(actor, x, ld, means, ld_means, log_std, actions, ld, log_probs, ld, advantages, ld, stats, P, d_log_std,
+                                      log_std_gradient_offset, batch, 1, rows),
+                        plain_job(critic, x_critic, ld, values, ld_values, nullptr, 0, target_values, ld, mse_scale, batch, 1, rows)};
+    if (out_critic_loss) { jobs[1].extra = out_critic_loss; jobs[1].n_extra = 1; jobs[1].extra_scale = 1.0f / (float)batch; jobs[1].extra_offset = 0.0f; }
     return launch(device, jobs, 2);
 }

@@ -4,6 +4,7 @@
 //            utils/polyak/operations_generic.h:11-43; CUDA counterparts adam/operations_cuda.h:18-68 (scalar kernel for the
 //            bias corrections), nn/layers/dense/operations_cuda.h:195-233 (one launch per layer).
 #include "common.h"
+#include "optim.h"
 
 namespace {
 
@@ -22,14 +23,15 @@ struct AdamLaunch {
     int accumulate_norm;         // add to *out_sq_norm instead of overwriting (later chunks of one step)
 };
 
-__global__ __launch_bounds__(256) void adam_kernel(AdamLaunch a) {
+// the step for one optimiser by workgroups [0, n_blocks) numbered `block`
+__device__ __forceinline__ void adam_body(const AdamLaunch& a, uint32_t block, uint32_t n_blocks) {
     const uint32_t age = *a.age;
     // bias corrections from the un-incremented age (adam/operations_generic.h:49-58)
     const float bc1 = 1.0f / (1.0f - powf(a.p.beta_1, (float)age));
     const float bc2 = 1.0f / (1.0f - powf(a.p.beta_2, (float)age));
     const uint32_t total = a.prefix[a.n];
     float sq = 0.0f;
-    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+    for (uint32_t i = block * blockDim.x + threadIdx.x; i < total; i += n_blocks * blockDim.x) {
         int ti = 0;
 #pragma unroll
         for (int k = 1; k < MAX_T; k++) ti += (k < a.n && i >= a.prefix[k]) ? 1 : 0;
@@ -57,22 +59,29 @@ __global__ __launch_bounds__(256) void adam_kernel(AdamLaunch a) {
     if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = sq;
     __syncthreads();
     if (threadIdx.x == 0) {
-        a.block_partials[blockIdx.x] = partial[0] + partial[1] + partial[2] + partial[3];
+        a.block_partials[block] = partial[0] + partial[1] + partial[2] + partial[3];
         __threadfence();
         uint32_t ticket = atomicAdd(a.done_counter, 1u);
-        last = (ticket == gridDim.x - 1);
+        last = (ticket == n_blocks - 1);
     }
     __syncthreads();
     if (last && threadIdx.x == 0) {
         __threadfence();
         if (a.out_sq_norm) {
             float s = a.accumulate_norm ? *a.out_sq_norm : 0.0f;
-            for (uint32_t b = 0; b < gridDim.x; b++) s += ((volatile float*)a.block_partials)[b];
+            for (uint32_t b = 0; b < n_blocks; b++) s += ((volatile float*)a.block_partials)[b];
             *a.out_sq_norm = s;
         }
         if (a.increment_age) *a.age = age + 1;
         *a.done_counter = 0;
     }
+}
+
+__global__ __launch_bounds__(256) void adam_kernel(AdamLaunch a) { adam_body(a, blockIdx.x, gridDim.x); }
+// two optimisers in one launch: workgroups [0, blocks_a) take the first
+__global__ __launch_bounds__(256) void adam_pair_kernel(AdamLaunch a, AdamLaunch b, uint32_t blocks_a) {
+    if (blockIdx.x < blocks_a) adam_body(a, blockIdx.x, blocks_a);
+    else adam_body(b, blockIdx.x - blocks_a, gridDim.x - blocks_a);
 }
 
 __global__ __launch_bounds__(256) void adam_reset_kernel(AdamLaunch a) {
@@ -123,6 +132,40 @@ static int adam_launch(rlt_rocm_device* device, const rlt_adam_tensor* tensors, 
         if ((rc = rlt_launch_status(device))) return rc;
     }
     return 0;
+}
+
+int rlt_adam_step_pair(rlt_rocm_device* device, const rlt_adam_tensor* tensors_a, int n_a, const rlt_adam_parameters* parameters_a, uint32_t* age_a,
+                       const rlt_adam_tensor* tensors_b, int n_b, const rlt_adam_parameters* parameters_b, uint32_t* age_b) {
+    RLT_REQUIRE(tensors_a && tensors_b && n_a > 0 && n_b > 0 && parameters_a && parameters_b && age_a && age_b);
+    if (n_a > MAX_T || n_b > MAX_T) {
+        const int rc = adam_launch(device, tensors_a, n_a, parameters_a, age_a, 0.0f, nullptr, false);
+        return rc ? rc : adam_launch(device, tensors_b, n_b, parameters_b, age_b, 0.0f, nullptr, false);
+    }
+    void* counters = nullptr;
+    int rc = rlt_counters(device, &counters);
+    if (rc) return rc;
+    AdamLaunch L[2] = {};
+    uint32_t blocks[2];
+    for (int k = 0; k < 2; k++) {
+        AdamLaunch& a = L[k];
+        const rlt_adam_tensor* tensors = k ? tensors_b : tensors_a;
+        a.n = k ? n_b : n_a;
+        uint32_t total = 0;
+        for (int i = 0; i < a.n; i++) {
+            const rlt_adam_tensor& T = tensors[i];
+            if (!T.first_moment || !T.second_moment || !T.parameters || !T.gradient || T.count == 0) return RLT_E_INVALID_ARGUMENT;
+            a.t[i] = T; a.prefix[i] = total; total += T.count;
+        }
+        for (int i = a.n; i <= MAX_T; i++) a.prefix[i] = total;
+        a.p = k ? *parameters_b : *parameters_a;
+        a.age = k ? age_b : age_a;
+        // the second optimiser's ticket counter and partial sums sit in their own part of the counters block
+        a.done_counter = (uint32_t*)((char*)counters + (k ? 64 : 0)); a.block_partials = (float*)((char*)counters + 256) + (k ? 480 : 0);
+        a.increment_age = 1;
+        blocks[k] = (total + 255) / 256; if (blocks[k] > 480) blocks[k] = 480; if (blocks[k] < 1) blocks[k] = 1;
+    }
+    hipLaunchKernelGGL(adam_pair_kernel, dim3(blocks[0] + blocks[1]), dim3(256), 0, device->stream, L[0], L[1], blocks[0]);
+    return rlt_launch_status(device);
 }
 
 extern "C" {

@@ -5,6 +5,7 @@
 #include "common.h"
 #include <cstdlib>
 #include "mlp_small.h"
+#include "optim.h"
 
 namespace {
 // one lane per environment, reverse scan over the steps; at a fixed step adjacent lanes touch adjacent dataset rows
@@ -48,21 +49,77 @@ __global__ __launch_bounds__(256) void ppo_gather_kernel(const float* __restrict
     }
 }
 
-// advantage mean and standard deviation over the minibatch (:170-180), one workgroup, fixed summation order: stats = {mean, std}
-__global__ __launch_bounds__(1024) void ppo_advantage_stats_kernel(const float* __restrict__ advantages, int ld, int batch, int normalize, float* __restrict__ stats) {
-    __shared__ float s1[16], s2[16];
+// advantage mean and standard deviation over the minibatch (:170-180): stats = {mean, std}. Minibatch row b is dataset row rows[b] (rows == NULL: b).
+// Shuffled rows of a large dataset sit on as many pages as there are rows, so the rows are spread over up to STAT_GROUPS workgroups; each leaves
+// {sum, sum of squares} of its rows in `partial`, and they are added up in workgroup order: the result does not depend on scheduling.
+constexpr int STAT_GROUPS = 64, EPOCH_CHUNK = 32;
+// thread 0 of workgroup `block` of `n_blocks` returns the sums over the workgroup's share of the rows
+__device__ __forceinline__ void advantage_block_sums(const float* __restrict__ advantages, int ld, int batch, const uint32_t* __restrict__ rows, int block, int n_blocks,
+                                                     float& sum, float& sum_sq) {
+    __shared__ float s1[4], s2[4];
     float a = 0.f, q = 0.f;
-    if (normalize) for (int b = threadIdx.x; b < batch; b += 1024) { const float v = advantages[(size_t)b * ld]; a += v; q += v * v; }
+    // four rows per lane at a time: their indices are requested together, then their values
+    const int stride = n_blocks * 256;
+    for (int base = block * 256; base < batch; base += 4 * stride) {
+        size_t row[4]; float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) { const int b = min(base + u * stride + (int)threadIdx.x, batch - 1); row[u] = rows ? rows[b] : (size_t)b; }
+#pragma unroll
+        for (int u = 0; u < 4; u++) v[u] = advantages[row[u] * ld];
+#pragma unroll
+        for (int u = 0; u < 4; u++) if (base + u * stride + (int)threadIdx.x < batch) { a += v[u]; q += v[u] * v[u]; }
+    }
     a = rlt_wave_sum(a); q = rlt_wave_sum(q);
     if ((threadIdx.x & 63) == 0) { s1[threadIdx.x >> 6] = a; s2[threadIdx.x >> 6] = q; }
     __syncthreads();
+    sum = (s1[0] + s1[1]) + (s1[2] + s1[3]); sum_sq = (s2[0] + s2[1]) + (s2[2] + s2[3]);
+}
+__device__ __forceinline__ void advantage_stats_from_partials(const float* partial, int groups, int batch, int normalize, float* __restrict__ stats) {
+    float m = 0.f, v = 0.f;
+    for (int g = 0; g < groups; g++) { m += ((const volatile float*)partial)[2 * g]; v += ((const volatile float*)partial)[2 * g + 1]; }
+    m /= (float)batch; v /= (float)batch;
+    stats[0] = normalize ? m : 0.f;
+    stats[1] = normalize ? sqrtf(fmaxf(0.f, v - m * m)) : 0.f;
+}
+// one minibatch: the last workgroup to finish (ticket counter, zero between launches) adds the partial sums up
+__global__ __launch_bounds__(256) void ppo_advantage_stats_kernel(const float* __restrict__ advantages, int ld, int batch, int normalize, float* __restrict__ stats,
+                                                                  const uint32_t* __restrict__ rows, float* __restrict__ partial, uint32_t* __restrict__ ticket) {
+    __shared__ bool last;
+    float a = 0.f, q = 0.f;
+    if (normalize) advantage_block_sums(advantages, ld, batch, rows, blockIdx.x, gridDim.x, a, q);
     if (threadIdx.x == 0) {
-        float m = 0.f, v = 0.f;
-        for (int i = 0; i < 16; i++) { m += s1[i]; v += s2[i]; }
-        m /= (float)batch; v /= (float)batch;
-        stats[0] = normalize ? m : 0.f;
-        stats[1] = normalize ? sqrtf(fmaxf(0.f, v - m * m)) : 0.f;
+        partial[2 * blockIdx.x] = a; partial[2 * blockIdx.x + 1] = q;
+        __threadfence();
+        last = atomicAdd(ticket, 1u) == gridDim.x - 1;
     }
+    __syncthreads();
+    if (last && threadIdx.x == 0) {
+        __threadfence();
+        advantage_stats_from_partials(partial, gridDim.x, batch, normalize, stats);
+        *ticket = 0;
+    }
+}
+// the minibatches of an epoch at once: blockIdx.y = minibatch, rows = its `batch` entries of the epoch's permutation; then one lane per minibatch
+__global__ __launch_bounds__(256) void ppo_epoch_stats_partial_kernel(const float* __restrict__ advantages, int ld, int batch, const uint32_t* __restrict__ rows,
+                                                                      float* __restrict__ partial) {
+    float a, q;
+    advantage_block_sums(advantages, ld, batch, rows + (size_t)blockIdx.y * batch, blockIdx.x, gridDim.x, a, q);
+    if (threadIdx.x == 0) { float* p = partial + ((size_t)blockIdx.y * STAT_GROUPS + blockIdx.x) * 2; p[0] = a; p[1] = q; }
+}
+__global__ void ppo_epoch_stats_final_kernel(const float* __restrict__ partial, int groups, int batch, int normalize, int n_minibatches, float* __restrict__ stats) {
+    const int mb = blockIdx.x * blockDim.x + threadIdx.x;
+    if (mb < n_minibatches) advantage_stats_from_partials(partial + (size_t)mb * STAT_GROUPS * 2, normalize ? groups : 0, batch, normalize, stats + 2 * mb);
+}
+int stat_groups(int batch) { const int g = (batch + 255) / 256; return g > STAT_GROUPS ? STAT_GROUPS : g; }
+// stats = scratch[0..1]; the workgroups' partial sums sit behind the surrogate kernel's own partials
+int ppo_advantage_stats(rlt_rocm_device* device, const float* advantages, int ld, int batch, int normalize, float* scratch, int action_dim, const uint32_t* rows) {
+    void* counters = nullptr;
+    int rc = rlt_counters(device, &counters);
+    if (rc) return rc;
+    float* partial = scratch + 2 + (size_t)((batch + 255) / 256) * action_dim;
+    hipLaunchKernelGGL(ppo_advantage_stats_kernel, dim3(stat_groups(batch)), dim3(256), 0, device->stream, advantages, ld, batch, normalize, scratch, rows, partial,
+                       (uint32_t*)((char*)counters + 192));
+    return rlt_launch_status(device);
 }
 
 // per sample (:205-269): log-probability of the rollout action under the current policy, ratio, clipping, d loss / d mean; the
@@ -124,7 +181,8 @@ bool ppo_agent_ok(const rlt_ppo_agent* A) {
            A->critic[0].in_dim == A->observation_privileged_dim && A->critic[A->n_critic_layers - 1].out_dim == 1 && A->actor[A->n_actor_layers - 1].output;
 }
 size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
-size_t ppo_surrogate_scratch_floats(int batch, int A) { return 2 + (size_t)((batch + 255) / 256) * A; }
+// stats, surrogate partials, stats partials, then for an epoch's minibatches in chunks: their stats and stats partials
+size_t ppo_surrogate_scratch_floats(int batch, int A) { return 2 + (size_t)((batch + 255) / 256) * A + 2 * STAT_GROUPS + (size_t)EPOCH_CHUNK * (2 + 2 * STAT_GROUPS); }
 }  // namespace
 
 extern "C" int rlt_rocm_ppo_gae(rlt_rocm_device* device, const float* rewards, const float* terminated, const float* truncated, const float* all_values,
@@ -150,8 +208,7 @@ static int ppo_surrogate_impl(rlt_rocm_device* device, const float* means, int l
                               float* scratch) {
     float* stats = scratch; float* partial = scratch + 2;
     const int blocks = (batch + 255) / 256;
-    hipLaunchKernelGGL(ppo_advantage_stats_kernel, dim3(1), dim3(1024), 0, device->stream, advantages, ld_adv, batch, P->normalize_advantage, stats);
-    int rc = rlt_launch_status(device);
+    int rc = ppo_advantage_stats(device, advantages, ld_adv, batch, P->normalize_advantage, scratch, A, nullptr);
     if (rc) return rc;
     hipLaunchKernelGGL(ppo_surrogate_kernel, dim3(blocks), dim3(256), 0, device->stream, means, ld_means, log_std, actions, ld_actions, log_probs, ld_lp, advantages, ld_adv, *P,
                        stats, d_means, ld_d, partial, batch, A);
@@ -176,6 +233,21 @@ extern "C" int rlt_rocm_ppo_surrogate_gradient(rlt_rocm_device* device, const fl
                               d_log_std, batch, action_dim, (float*)scratch);
 }
 
+// actor and critic of the supported narrow shape in one launch (stats = {advantage mean, std} of the minibatch on the device), then both Adam steps in one
+static int ppo_pair_update(rlt_rocm_device* device, const rlt_ppo_agent* A, const rlt_ppo_parameters* P, const float* observations, const float* observations_privileged,
+                           const float* actions, const float* action_log_probs, const float* advantages, const float* target_values, int ld, const uint32_t* row_indices,
+                           const float* stats, float* values, float* out_critic_loss) {
+    const int B = A->batch, AD = A->action_dim;
+    int rc = rlt_mlp3s_ppo_actor_critic(device, A->actor, A->n_actor_layers, observations, A->actor[A->n_actor_layers - 1].output, AD, A->log_std, actions,
+                                        action_log_probs, advantages, stats, P, P->learn_action_std ? A->d_log_std : nullptr, -P->action_entropy_coefficient,
+                                        A->critic, A->n_critic_layers, observations_privileged, values, 1, target_values, 1.0f / (float)B, out_critic_loss,   // :303
+                                        ld, row_indices, B);
+    if (rc) return rc;
+    if (A->d_log_std && !P->learn_action_std) if ((rc = rlt_rocm_fill_f32(device, A->d_log_std, 1, AD, AD, 0.0f))) return rc;
+    return rlt_adam_step_pair(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age,                                            // :305-306
+                              A->critic_adam_tensors, A->n_critic_adam_tensors, &A->critic_adam, A->critic_age);
+}
+
 extern "C" int rlt_rocm_ppo_train_minibatch(rlt_rocm_device* device, const rlt_ppo_agent* A, const rlt_ppo_parameters* P, const float* observations,
                                             const float* observations_privileged, const float* actions, const float* action_log_probs, const float* advantages,
                                             const float* target_values, int ld, const uint32_t* row_indices, float* out_critic_loss) {
@@ -191,48 +263,77 @@ extern "C" int rlt_rocm_ppo_train_minibatch(rlt_rocm_device* device, const rlt_p
     float* scratch = w; w += ppo_surrogate_scratch_floats(B, AD);
     char* mlp_ws = (char*)A->workspace + align256((size_t)((char*)w - (char*)A->workspace) + 64 * sizeof(float));
     const size_t mlp_ws_bytes = A->workspace_bytes - (size_t)(mlp_ws - (char*)A->workspace);
+    int rc;
+    if (narrow_pass_enabled() && rlt_mlp3s_pair_supported(A->actor, A->n_actor_layers, A->critic, A->n_critic_layers)) {
+        // both networks in -> 64 -> 64 -> out: one launch runs the actor (forward, surrogate gradient, backward, :203-285) on half of the compute units
+        // and the critic (forward, MSE gradient with loss weight 0.5 = (v - target) / batch, backward, :289-300) on the other half, reading the
+        // minibatch's rows straight out of the dataset; its gradients replace the old ones, which is what zero_gradient (:158-159) followed by
+        // backward leaves. The means still land in the actor's last output buffer; the hidden layers' buffers are not written.
+        if ((rc = ppo_advantage_stats(device, advantages, ld, B, P->normalize_advantage, scratch, AD, row_indices))) return rc;
+        return ppo_pair_update(device, A, P, observations, observations_privileged, actions, action_log_probs, advantages, target_values, ld, row_indices, scratch,
+                               values, out_critic_loss);
+    }
     int blocks = (B * 16 + 255) / 256; if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(ppo_gather_kernel, dim3(blocks), dim3(256), 0, device->stream, observations, observations_privileged, actions, action_log_probs, advantages, target_values,
                        ld, row_indices, B, O, OP, AD, obs, obsp, act, lp, adv, tgt);
-    int rc = rlt_launch_status(device);
-    if (rc) return rc;
-    const bool narrow = narrow_pass_enabled() && rlt_mlp3s_supported(A->actor, A->n_actor_layers);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if ((rc = rlt_rocm_mlp_zero_gradient(device, A->critic, A->n_critic_layers))) return rc;                      // :158
+    if ((rc = rlt_rocm_mlp_zero_gradient(device, A->actor, A->n_actor_layers))) return rc;                        // :159 (clears the log_std gradient too)
+    if (A->d_log_std) if ((rc = rlt_rocm_fill_f32(device, A->d_log_std, 1, AD, AD, 0.0f))) return rc;
     rc = RLT_E_UNSUPPORTED;
-    if (narrow && rlt_mlp3s_supported(A->critic, A->n_critic_layers)) {
-        // both networks in -> 64 -> 64 -> out: one launch runs the actor (forward, surrogate gradient, backward, :203-285) on half of the compute units
-        // and the critic (forward, MSE gradient with loss weight 0.5 = (v - target) / batch, backward, :289-300) on the other half, and its gradients
-        // replace the old ones, which is what zero_gradient (:158-159) followed by backward leaves. The means still land in the actor's last output
-        // buffer; the hidden layers' buffers are not written.
-        hipLaunchKernelGGL(ppo_advantage_stats_kernel, dim3(1), dim3(1024), 0, device->stream, adv, 1, B, P->normalize_advantage, scratch);
-        if ((rc = rlt_launch_status(device))) return rc;
-        rc = rlt_mlp3s_ppo_actor_critic(device, A->actor, A->n_actor_layers, obs, O, A->actor[A->n_actor_layers - 1].output, AD, A->log_std, act, AD, lp, 1, adv, 1,
-                                        scratch, P, P->learn_action_std ? A->d_log_std : nullptr, -P->action_entropy_coefficient,
-                                        A->critic, A->n_critic_layers, obsp, OP, values, 1, tgt, 1, 1.0f / (float)B, B);
+    if (narrow_pass_enabled() && rlt_mlp3s_supported(A->actor, A->n_actor_layers)) {       // the actor alone in one kernel
+        if ((rc = ppo_advantage_stats(device, adv, 1, B, P->normalize_advantage, scratch, AD, nullptr))) return rc;
+        rc = rlt_mlp3s_ppo_actor(device, A->actor, A->n_actor_layers, obs, O, A->actor[A->n_actor_layers - 1].output, AD, A->log_std, act, AD, lp, 1, adv, 1, scratch, P,
+                                 P->learn_action_std ? A->d_log_std : nullptr, -P->action_entropy_coefficient, B);
         if (rc && rc != RLT_E_UNSUPPORTED) return rc;
-        if (rc == 0 && A->d_log_std && !P->learn_action_std) if ((rc = rlt_rocm_fill_f32(device, A->d_log_std, 1, AD, AD, 0.0f))) return rc;
     }
     if (rc == RLT_E_UNSUPPORTED) {
-        if ((rc = rlt_rocm_mlp_zero_gradient(device, A->critic, A->n_critic_layers))) return rc;                      // :158
-        if ((rc = rlt_rocm_mlp_zero_gradient(device, A->actor, A->n_actor_layers))) return rc;                        // :159 (clears the log_std gradient too)
-        if (A->d_log_std) if ((rc = rlt_rocm_fill_f32(device, A->d_log_std, 1, AD, AD, 0.0f))) return rc;
-        rc = RLT_E_UNSUPPORTED;
-        if (narrow) {       // the actor alone in one kernel
-            hipLaunchKernelGGL(ppo_advantage_stats_kernel, dim3(1), dim3(1024), 0, device->stream, adv, 1, B, P->normalize_advantage, scratch);
-            if ((rc = rlt_launch_status(device))) return rc;
-            rc = rlt_mlp3s_ppo_actor(device, A->actor, A->n_actor_layers, obs, O, A->actor[A->n_actor_layers - 1].output, AD, A->log_std, act, AD, lp, 1, adv, 1, scratch, P,
-                                     P->learn_action_std ? A->d_log_std : nullptr, -P->action_entropy_coefficient, B);
-            if (rc && rc != RLT_E_UNSUPPORTED) return rc;
-        }
-        if (rc == RLT_E_UNSUPPORTED) {
-            if ((rc = rlt_rocm_mlp_forward(device, A->actor, A->n_actor_layers, obs, O, B))) return rc;                    // :203
-            const float* means = A->actor[A->n_actor_layers - 1].output;
-            if ((rc = ppo_surrogate_impl(device, means, AD, A->log_std, act, AD, lp, 1, adv, 1, P, d_act, AD, A->d_log_std, B, AD, scratch))) return rc;
-            if ((rc = rlt_rocm_mlp_backward(device, A->actor, A->n_actor_layers, obs, O, d_act, AD, nullptr, 0, B, 1, mlp_ws, mlp_ws_bytes))) return rc;   // :285
-        }
-        // critic: forward, MSE gradient with loss weight 0.5 (= (v - target)/batch), backward in one pass (:289-300)
-        if ((rc = rlt_rocm_mlp_forward_backward(device, A->critic, A->n_critic_layers, obsp, OP, values, 1, nullptr, 0, tgt, 1, 1.0f / (float)B, B, mlp_ws, mlp_ws_bytes))) return rc;
+        if ((rc = rlt_rocm_mlp_forward(device, A->actor, A->n_actor_layers, obs, O, B))) return rc;                    // :203
+        const float* means = A->actor[A->n_actor_layers - 1].output;
+        if ((rc = ppo_surrogate_impl(device, means, AD, A->log_std, act, AD, lp, 1, adv, 1, P, d_act, AD, A->d_log_std, B, AD, scratch))) return rc;
+        if ((rc = rlt_rocm_mlp_backward(device, A->actor, A->n_actor_layers, obs, O, d_act, AD, nullptr, 0, B, 1, mlp_ws, mlp_ws_bytes))) return rc;   // :285
     }
+    // critic: forward, MSE gradient with loss weight 0.5 (= (v - target)/batch), backward in one pass (:289-300)
+    if ((rc = rlt_rocm_mlp_forward_backward(device, A->critic, A->n_critic_layers, obsp, OP, values, 1, nullptr, 0, tgt, 1, 1.0f / (float)B, B, mlp_ws, mlp_ws_bytes))) return rc;
     if (out_critic_loss) if ((rc = rlt_rocm_mse_evaluate(device, values, 1, tgt, 1, B, 1, 1.0f, out_critic_loss))) return rc;                      // :303
     if ((rc = rlt_rocm_adam_step(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, 0.0f, nullptr))) return rc;  // :305
     return rlt_rocm_adam_step(device, A->critic_adam_tensors, A->n_critic_adam_tensors, &A->critic_adam, A->critic_age, 0.0f, nullptr);             // :306
+}
+
+extern "C" int rlt_rocm_ppo_train_epoch(rlt_rocm_device* device, const rlt_ppo_agent* A, const rlt_ppo_parameters* P, const float* observations,
+                                        const float* observations_privileged, const float* actions, const float* action_log_probs, const float* advantages,
+                                        const float* target_values, int ld, const uint32_t* row_indices, int n_minibatches, float* out_critic_losses) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(ppo_agent_ok(A) && P && observations && observations_privileged && actions && action_log_probs && advantages && target_values && ld >= 1);
+    RLT_REQUIRE(row_indices && n_minibatches >= 1 && (!P->learn_action_std || A->d_log_std));
+    RLT_REQUIRE(A->workspace && A->workspace_bytes >= rlt_rocm_ppo_workspace_bytes(A));
+    const int B = A->batch, O = A->observation_dim, OP = A->observation_privileged_dim, AD = A->action_dim;
+    if (!(narrow_pass_enabled() && rlt_mlp3s_pair_supported(A->actor, A->n_actor_layers, A->critic, A->n_critic_layers))) {
+        for (int mb = 0; mb < n_minibatches; mb++) {
+            const int rc = rlt_rocm_ppo_train_minibatch(device, A, P, observations, observations_privileged, actions, action_log_probs, advantages, target_values, ld,
+                                                        row_indices + (size_t)mb * B, out_critic_losses ? out_critic_losses + mb : nullptr);
+            if (rc) return rc;
+        }
+        return 0;
+    }
+    // same carving of the workspace as the minibatch call; the advantage statistics of up to EPOCH_CHUNK minibatches are formed by one pair of launches
+    float* w = (float*)A->workspace;
+    w += (size_t)B * O; w += (size_t)B * OP; w += (size_t)B * AD; w += (size_t)B * AD; w += 3 * (size_t)B;
+    float* values = w; w += B;
+    float* stats_all = w + 2 + (size_t)((B + 255) / 256) * AD + 2 * STAT_GROUPS; float* partial_all = stats_all + 2 * EPOCH_CHUNK;
+    const int groups = stat_groups(B);
+    for (int first = 0; first < n_minibatches; first += EPOCH_CHUNK) {
+        const int n = n_minibatches - first < EPOCH_CHUNK ? n_minibatches - first : EPOCH_CHUNK;
+        int rc;
+        if (P->normalize_advantage) {
+            hipLaunchKernelGGL(ppo_epoch_stats_partial_kernel, dim3(groups, n), dim3(256), 0, device->stream, advantages, ld, B, row_indices + (size_t)first * B, partial_all);
+            if ((rc = rlt_launch_status(device))) return rc;
+        }
+        hipLaunchKernelGGL(ppo_epoch_stats_final_kernel, dim3(1), dim3(EPOCH_CHUNK), 0, device->stream, partial_all, groups, B, P->normalize_advantage, n, stats_all);
+        if ((rc = rlt_launch_status(device))) return rc;
+        for (int mb = first; mb < first + n; mb++)
+            if ((rc = ppo_pair_update(device, A, P, observations, observations_privileged, actions, action_log_probs, advantages, target_values, ld,
+                                      row_indices + (size_t)mb * B, stats_all + 2 * (mb - first), values, out_critic_losses ? out_critic_losses + mb : nullptr))) return rc;
+    }
+    return 0;
 }

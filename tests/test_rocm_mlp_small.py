@@ -98,11 +98,14 @@ def test_narrow_full_size_against_per_layer_kernels_and_linearity(rocm, monkeypa
         assert ew <= slack and eb <= slack, (off, ew, eb)
 
 
-def test_ppo_update_narrow_actor_against_per_layer_kernels(rocm, monkeypatch):
-    """The PPO minibatch update at the benchmark's minibatch size (8,192 rows, observation 105, 8 actions) with the actor's forward, surrogate
-    gradient and backward in one kernel, against the same update on the per-layer kernels; at 512 rows the checker covers the same path."""
+@pytest.mark.parametrize("sizes", [(8192, 16384), (1000, 3000)])
+def test_ppo_update_narrow_networks_against_per_layer_kernels(rocm, monkeypatch, sizes):
+    """The PPO minibatch update at the benchmark's minibatch size (8,192 rows, observation 105, 8 actions) and at a ragged one, with actor and critic
+    in one launch reading shuffled rows straight out of the dataset, against the same update on the per-layer kernels (which gather the rows
+    first); at 512 rows the checker covers the same path."""
     capi = helpers.capi
-    O, A, H, B, N = 105, 8, 64, 8192, 16384
+    O, A, H = 105, 8, 64
+    B, N = sizes
     rng = np.random.default_rng(21)
     na = helpers.mlp_param_count([O, H, H, A])
     params = np.concatenate([helpers.random_params(rng, [O, H, H, A]), np.log(np.full(A, 0.5, np.float32)), helpers.random_params(rng, [O, H, H, 1])])

@@ -91,6 +91,45 @@ def test_train_minibatch_matches_checker_on_synthetic_dataset(oracle, rocm):
     assert rel_err(p1, p0) <= 2e-4 and rel_err(l1, l0) <= 1e-4
 
 
+@pytest.mark.parametrize("normalize", [1, 0])
+def test_train_epoch_matches_checker_and_minibatch_calls(oracle, rocm, normalize):
+    """One epoch call (advantage statistics of all minibatches formed up front, 40 minibatches = two chunks of that) against the checker's batch
+    loop and against the same minibatches issued one call at a time; ragged minibatch size, losses per minibatch."""
+    capi = helpers.capi
+    O, A, H, B, NMB = 105, 8, 64, 200, 40
+    N = B * NMB
+    rng = np.random.default_rng(9)
+    na = helpers.mlp_param_count([O, H, H, A])
+    params = np.concatenate([helpers.random_params(rng, [O, H, H, A]), np.log(np.full(A, 0.5, np.float32)), helpers.random_params(rng, [O, H, H, 1])])
+    ld = O + 2 * A + 8
+    data = rng.standard_normal((N, ld)).astype(np.float32)
+    col = dict(observations=0, actions=O + A, action_log_probs=O + 2 * A, advantages=O + 2 * A + 6, target_values=O + 2 * A + 7)
+    net = helpers.Mlp(oracle, [O, H, H, A], params[:na], N, "tanh", trainable=False)
+    out, data0 = oracle.zeros((N, A)), oracle.array(data)
+    oracle.call("mlp_evaluate", net.layers, net.n, data0.offset(0), ld, out.ptr, A, N, None, 0)
+    z = (data[:, col["actions"]:col["actions"] + A] - out.numpy()) / 0.5
+    data[:, col["action_log_probs"]] = (-0.9189385332046727 - np.log(0.5) - 0.5 * z * z).sum(1) + 0.2 * rng.standard_normal(N).astype(np.float32)
+    perm = rng.permutation(N).astype(np.uint32)
+    pp = capi.ppo_parameters()
+    pp.normalize_advantage = normalize
+    results = []
+    for b, epoch_call in ((oracle, True), (rocm, True), (rocm, False)):
+        agent = helpers.PpoOnBackend(b, O, A, H, H, B, params, "tanh", "tanh", capi.adam_parameters(3e-4, epsilon=1e-8))
+        dd, idx, losses = b.array(data), b.array(perm), b.zeros((NMB,))
+        args = (dd.offset(col["observations"]), dd.offset(col["observations"]), dd.offset(col["actions"]), dd.offset(col["action_log_probs"]),
+                dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld)
+        if epoch_call:
+            b.call("ppo_train_epoch", C.byref(agent.c), C.byref(pp), *args, idx.ptr, NMB, losses.ptr)
+        else:
+            for k in range(NMB):
+                b.call("ppo_train_minibatch", C.byref(agent.c), C.byref(pp), *args, idx.offset(k * B), losses.offset(k))
+        b.sync()
+        results.append((agent.parameters(), losses.numpy(), agent.d_log_std.numpy()))
+    want, got, single = results
+    assert np.array_equal(got[0], single[0]) and np.array_equal(got[1], single[1])        # the same kernels on the same statistics: bitwise
+    assert rel_err(got[0], want[0]) <= 2e-4 and rel_err(got[1], want[1]) <= 1e-4 and rel_err(got[2], want[2]) <= 1e-3
+
+
 def test_ppo_against_reference_vectors(rocm):
     """GAE bit-exact structure aside (fp32, same operation order per environment), the 30 minibatch updates of two loop steps reproduce the
     reference's parameters; the dataset, permutations and parameters come from the reference's own run (tests/golden/ppo_pendulum_seed0.npz)."""
