@@ -55,13 +55,6 @@ constexpr size_t lds_floats(int nt1c) {
     return (size_t)H * sx + H * HS + MAX_OUT * HS + (size_t)ROWS * (sx + 3 * HS + D3S);
 }
 
-#ifdef MLP3S_TIMING
-__device__ unsigned long long mlp3s_stamps[32];
-#define STAMP(i) do { if (blockIdx.x == 0 && threadIdx.x == 0) mlp3s_stamps[i] = clock64(); } while (0)
-#else
-#define STAMP(i)
-#endif
-
 // lane l: the row of the input arrays that row (l & 15) of a tile reads; rows beyond the batch are clamped here and masked later
 __device__ __forceinline__ int tile_rows(const SmallArgs& A, int tile, int lane) {
     const int b = min(tile * 16 + (lane & 15), A.batch - 1);
@@ -108,8 +101,6 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
     const lptr xs_all = w3s + MAX_OUT * HS, h1s_all = xs_all + ROWS * SX, h2s_all = h1s_all + ROWS * HS, g2s_all = h2s_all + ROWS * HS, d3s_all = g2s_all + ROWS * HS;
     const lptr xs = xs_all + 16 * wave * SX, h1s = h1s_all + 16 * wave * HS, h2s = h2s_all + 16 * wave * HS, g2s = g2s_all + 16 * wave * HS, d3s = d3s_all + 16 * wave * D3S;
     const int n_tiles = (A.batch + 15) >> 4, n_rounds = (n_tiles + WAVES - 1) / WAVES;
-
-    STAMP(0);
     // row indices of this wavefront's first two tiles, then the first tile's loads, ahead of the weights'; a wavefront whose tile lies beyond the
     // batch computes on clamped rows and masks them
     int rows_next = tile_rows(A, min(block * WAVES + wave, n_tiles - 1), lane), rows_after = tile_rows(A, min((block + n_blocks) * WAVES + wave, n_tiles - 1), lane);
@@ -152,7 +143,6 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
     }
     const float sd = expf(ls);
     rlt_lds_barrier();
-    STAMP(1);
 
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
     // this wavefront's share of the weight gradients: rows 16 wave + 4 kk + v of dW1 (columns 16 nt + r) and of dW2, columns 16 wave + r of dW3 (rows 4 kk + v)
@@ -180,7 +170,6 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
         rows_next = rows_after;
         rows_after = tile_rows(A, min((round + 2 * n_blocks) * WAVES + wave, n_tiles - 1), lane);
         request_tile(A, rows_next, lane, T);
-        STAMP(2);
 
         // layer 1: groups of four reduction steps, the operands of the next group requested before this group's matrix instructions
         floatx4 acc[4] = {zero4, zero4, zero4, zero4};
@@ -218,7 +207,6 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
 #pragma unroll
             for (int v = 0; v < 4; v++) h1s[(4 * kk + v) * HS + 16 * nt + r] = rlt_act(acc[nt][v] + b1r[nt], ACT_H);
         wave_sync();
-        STAMP(3);
 
         // layer 2
 #pragma unroll
@@ -234,7 +222,6 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
 #pragma unroll
             for (int v = 0; v < 4; v++) h2s[(4 * kk + v) * HS + 16 * nt + r] = rlt_act(acc[nt][v] + b2r[nt], ACT_H);
         wave_sync();
-        STAMP(4);
 
         // layer 3 (two chains of matrix instructions) and the gradient at its pre-activations
         floatx4 y0 = zero4, y1 = zero4;
@@ -273,7 +260,6 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
             d3s[(4 * kk + v) * D3S + r] = dp;
         }
         rlt_lds_barrier();      // every wavefront's h2 and d_pre3 are in place
-        STAMP(5);
 
         // dW3 (columns 16 wave + r) += d_pre3^T h2 over the 64 rows, two chains
         {
@@ -304,7 +290,6 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
                 g2s[idx] = dp; s2[nt] += dp;
             }
         rlt_lds_barrier();      // every wavefront's d_pre2 is in place, and nobody reads h2 any more
-        STAMP(6);
 
         // dW2 (rows 16 wave + ..) += d_pre2^T h1 over the 64 rows
         {
@@ -342,7 +327,6 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
                 h2s[idx] = dp; s1[nt] += dp;
             }
         rlt_lds_barrier();      // every wavefront's d_pre1 is in place
-        STAMP(7);
 
         // dW1 (rows 16 wave + ..) += d_pre1^T x over the 64 rows
         {
@@ -364,7 +348,6 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
         }
         rlt_lds_barrier();      // the round's tiles may be overwritten
     }
-    STAMP(8);
 
     // the workgroup's block of partial sums: weight gradients straight from the registers that own them, ...
     float* dst = A.partial + (size_t)block * A.count;
@@ -398,7 +381,6 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
         else if (i < 2 * H + MAX_OUT) { if (i - 2 * H < OUT) dst[o_b3 + i - 2 * H] = total; }
         else dst[o_ex + i - 2 * H - MAX_OUT] = total;
     }
-    STAMP(9);
 }
 
 // where the elements of a block of partial sums go; overwrite: gradient = sum instead of gradient += sum (for a caller that would zero the gradient first)
