@@ -134,8 +134,23 @@ def bench_env(helpers, rocm, n_envs=65536, capacity=16, steps=200, batch=4096):
     e = ev.record()
     gather_us = ev.elapsed_ms(a, e) * 10.0
     env_steps = n_envs * steps
+    # evaluation step of the training loop: 10 episodes x 200 steps with the deterministic actor, one launch
+    env_p = capi.pendulum_parameters()
+    e_ini, e_ret, e_len, e_sum = rocm.array(ini.numpy()[:10].copy()), rocm.zeros((10,)), rocm.zeros((10,), np.uint32), rocm.zeros((6,))
+
+    def evaluate():
+        rocm.call("pendulum_evaluate", C.byref(env_p), 1, actor.layers, actor.n, e_ini.ptr, 10, 200, e_ret.ptr, e_len.ptr, e_sum.ptr)
+    for _ in range(3):
+        evaluate()
+    rocm.sync()
+    a = ev.record()
+    for _ in range(20):
+        evaluate()
+    e = ev.record()
+    evaluate_us = ev.elapsed_ms(a, e) * 1e3 / 20
     return {"n_envs": n_envs, "replay_rows": n_envs * capacity, "steps": steps, "us_per_step": ms * 1e3 / steps, "env_steps_per_s": env_steps / (ms * 1e-3),
-            "algorithmic_GBps": env_steps * 68 / (ms * 1e-3) / 1e9, "gather_batch": batch, "gather_us": gather_us, "gather_algorithmic_GBps": batch * 85 / (gather_us * 1e-6) / 1e9}
+            "algorithmic_GBps": env_steps * 68 / (ms * 1e-3) / 1e9, "gather_batch": batch, "gather_us": gather_us, "gather_algorithmic_GBps": batch * 85 / (gather_us * 1e-6) / 1e9,
+            "evaluation_10_episodes_x_200_steps_us": evaluate_us}
 
 
 def bench_ppo(helpers, rocm, n_envs=4096, steps=128, epochs=4, minibatch=8192):

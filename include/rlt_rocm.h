@@ -384,6 +384,19 @@ int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_ru
                                   const float* actions_in, const float* action_noise,
                                   const float* initial_states, uint64_t seed, uint64_t offset);
 
+/* rl::utils::evaluation::evaluate  rl/utils/evaluation/operations_generic.h:106-233 (called by the evaluation loop step,
+ * rl/loop/steps/evaluation/operations_generic.h:56-92) for the Pendulum environment: n_episodes episodes of step_limit steps
+ * from `initial_states` [n_episodes x 2] (what sample_initial_state draws, or the deterministic initial state), the actor in
+ * Evaluation mode:
+ *   policy_kind 1 = the actor's output is the action; 2 = the actor's output is [mean | log_std] and the action is tanh(mean)
+ *   (sample_and_squash with zero noise, nn/layers/sample_and_squash/operations_generic.h:149-195).
+ * Device outputs: returns [n_episodes], episode_length [n_episodes], summary [6] = {returns_mean, returns_std,
+ * episode_length_mean, episode_length_std, num_terminated, share_terminated} (Result, evaluation.h:54-68). Actors
+ * 3 -> H -> H -> out with H <= 64 run all steps in one launch, a wavefront per episode. */
+int rlt_rocm_pendulum_evaluate(rlt_rocm_device* device, const rlt_pendulum_parameters* env, int policy_kind,
+                               const rlt_dense_layer* actor, int n_actor_layers, const float* initial_states,
+                               int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary);
+
 /* Host-drawn randomness for rlt_rocm_sac_pendulum_loop (parity runs feed the draws the reference's CPU RNG made); any member
  * may be NULL, in which case the kernel draws from its counter-based generator keyed by (seed, step). */
 typedef struct rlt_sac_loop_inputs {

@@ -19,6 +19,7 @@
 #include <rl_tools/nn/optimizers/adam/operations_generic.h>
 #include <rl_tools/rl/algorithms/sac/loop/core/config.h>
 #include <rl_tools/rl/algorithms/sac/loop/core/operations_generic.h>
+#include <rl_tools/rl/utils/evaluation/operations_generic.h>
 
 #include <chrono>
 #include <cstdint>
@@ -212,6 +213,43 @@ double rlt_ref_sac_time_steps(void* h, int steps) {
     for (int i = 0; i < steps; i++) DISPATCH(a, (int)rlt::step(L.device, L.ts));
     auto t1 = std::chrono::steady_clock::now();
     return std::chrono::duration<double>(t1 - t0).count();
+}
+
+// rl::utils::evaluation::evaluate (rl/utils/evaluation/operations_generic.h:106-233) of the loop's current actor in Evaluation mode: 10 episodes of
+// 200 steps from sampled initial states, the configuration of the evaluation loop step (rl/loop/steps/evaluation/config.h:12-24). The initial
+// states the call will draw are exported by drawing them first from a copy of the engine.
+// summary = {returns_mean, returns_std, episode_length_mean, episode_length_std, num_terminated, share_terminated}
+void rlt_ref_sac_evaluate(void* h, uint32_t seed, float* initial_states, float* returns, uint32_t* episode_length, float* summary) {
+    Any* a = (Any*)h;
+    DISPATCH(a, ([&] {
+        constexpr TI N_EPISODES = 10, STEP_LIMIT = 200;
+        using SPEC = rlt::rl::utils::evaluation::Specification<TYPE_POLICY, TI, ENVIRONMENT, N_EPISODES, STEP_LIMIT>;
+        RNG rng;
+        rlt::malloc(L.device, rng);
+        rlt::init(L.device, rng, seed);
+        ENVIRONMENT env;
+        ENVIRONMENT::Parameters parameters;
+        rlt::init(L.device, env);
+        rlt::initial_parameters(L.device, env, parameters);
+        {
+            RNG copy = rng;
+            for (TI e = 0; e < N_EPISODES; e++) {
+                ENVIRONMENT::State state;
+                rlt::sample_initial_parameters(L.device, env, parameters, copy);
+                rlt::sample_initial_state(L.device, env, parameters, state, copy);
+                initial_states[2 * e] = state.theta; initial_states[2 * e + 1] = state.theta_dot;
+            }
+        }
+        rlt::rl::utils::evaluation::Result<SPEC> result;
+        rlt::rl::environments::DummyUI ui;
+        rlt::Mode<rlt::mode::Evaluation<>> mode;
+        rlt::evaluate(L.device, env, ui, L.ts.actor_critic.actor, result, rng, mode);
+        for (TI e = 0; e < N_EPISODES; e++) { returns[e] = result.returns[e]; episode_length[e] = (uint32_t)result.episode_length[e]; }
+        summary[0] = result.returns_mean; summary[1] = result.returns_std; summary[2] = result.episode_length_mean; summary[3] = result.episode_length_std;
+        summary[4] = (float)result.num_terminated; summary[5] = result.share_terminated;
+        rlt::free(L.device, rng);
+        return 0;
+    }()));
 }
 
 }  // extern "C"

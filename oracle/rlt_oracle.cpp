@@ -734,6 +734,47 @@ int rlt_oracle_pendulum_runner_step(const rlt_pendulum_runner* rn, const rlt_rep
     return rlt_oracle_replay_add(rb, obs.data(), actions.data(), rewards.data(), next_obs.data(), term.data(), trunc.data());
 }
 
+// rl::utils::evaluation::evaluate (rl/utils/evaluation/operations_generic.h:106-233) with the Pendulum environment: n_episodes environments from the
+// given initial states (what sample_initial_state drew, :139-142), step_limit steps of observe -> policy in Evaluation mode -> step -> reward;
+// an episode stops counting once it has terminated (:188-197; Pendulum never terminates, pendulum/operations_generic.h:161-164). The statistics
+// are accumulated in float in episode order (:213-227).
+//   policy_kind 1: the actor's output is the action;  2: the actor's output is [mean | log_std] and the action is tanh(mean), which is what
+//   sample_and_squash yields in Evaluation mode (noise = 0, nn/layers/sample_and_squash/operations_generic.h:149-195)
+//   summary = {returns_mean, returns_std, episode_length_mean, episode_length_std, num_terminated, share_terminated}
+int rlt_oracle_pendulum_evaluate(const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers, const float* initial_states,
+                                 int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary) {
+    if (!env || !actor || n_actor_layers < 1 || !initial_states || n_episodes < 1 || step_limit < 1 || !returns || !episode_length || !summary) return RLT_E_INVALID_ARGUMENT;
+    if (policy_kind != 1 && policy_kind != 2) return RLT_E_INVALID_ARGUMENT;
+    const int N = n_episodes, out_dim = actor[n_actor_layers - 1].out_dim;
+    if (actor[0].in_dim != 3 || out_dim != policy_kind) return RLT_E_INVALID_ARGUMENT;
+    std::vector<float> states(initial_states, initial_states + 2 * (size_t)N), obs((size_t)N * 3), out((size_t)N * out_dim);
+    std::vector<uint8_t> terminated(N, 0);
+    uint32_t num_terminated = 0;
+    for (int e = 0; e < N; e++) { returns[e] = 0; episode_length[e] = 0; }
+    for (int step = 0; step < step_limit; step++) {
+        for (int e = 0; e < N; e++) pendulum_observe(states[2 * e], states[2 * e + 1], &obs[3 * (size_t)e]);
+        const int rc = rlt_oracle_mlp_evaluate(actor, n_actor_layers, obs.data(), 3, out.data(), out_dim, N);
+        if (rc) return rc;
+        for (int e = 0; e < N; e++) {
+            if (step > 0 && terminated[e]) continue;
+            const float action = policy_kind == 1 ? out[e] : std::tanh(out[2 * (size_t)e]);
+            float nth, nthd, r;
+            pendulum_dynamics(env, states[2 * e], states[2 * e + 1], action, &nth, &nthd, &r);
+            const bool terminated_flag = false;      // the Pendulum has no terminal states
+            if (!terminated[e]) { returns[e] += r; episode_length[e] += 1; num_terminated += terminated_flag ? 1 : 0; }
+            terminated[e] = terminated_flag || terminated[e];
+            states[2 * e] = nth; states[2 * e + 1] = nthd;
+        }
+    }
+    float rm = 0, rs = 0, lm = 0, ls = 0;
+    for (int e = 0; e < N; e++) { rm += returns[e]; rs += returns[e] * returns[e]; lm += (float)episode_length[e]; ls += (float)(episode_length[e] * episode_length[e]); }
+    rm /= N; lm /= N;
+    summary[0] = rm; summary[1] = std::sqrt(std::max(0.0f, rs / N - rm * rm));
+    summary[2] = lm; summary[3] = std::sqrt(std::max(0.0f, ls / N - lm * lm));
+    summary[4] = (float)num_terminated; summary[5] = num_terminated / (float)N;
+    return 0;
+}
+
 // rl/algorithms/ppo/operations_generic.h:60-95
 int rlt_oracle_ppo_gae(const float* rewards, const float* terminated, const float* truncated, const float* all_values,
                        float* advantages, float* target_values, int ld, int n_envs, int steps, float gamma, float lambda,

@@ -98,6 +98,9 @@ int rlt_oracle_ppo_gae(const float* rewards, const float* terminated, const floa
                        float* advantages, float* target_values, int ld, int n_envs, int steps, float gamma, float lambda,
                        int ignore_termination);
 
+/* rl::utils::evaluation::evaluate with the Pendulum environment (rl/utils/evaluation/operations_generic.h:106-233) */
+int rlt_oracle_pendulum_evaluate(const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers, const float* initial_states,
+                                 int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary);
 int rlt_oracle_ppo_surrogate_gradient(const float* action_means, int ld_means, const float* log_std, const float* actions, int ld_actions,
                                       const float* action_log_probs, int ld_log_probs, const float* advantages, int ld_advantages,
                                       const rlt_ppo_parameters* parameters, float* d_action_means, int ld_d, float* d_log_std, int batch, int action_dim);

@@ -174,6 +174,7 @@ PROTOTYPES = {
     "replay_add": [C.POINTER(ReplayBuffer), P, P, P, P, P, P],
     "gather_batch": [C.POINTER(ReplayBuffer), P, P, I, I, I, P, P, P, P, P, P, P],
     "pendulum_step": [C.POINTER(PendulumParameters), P, P, P, P, P, I],
+    "pendulum_evaluate": [C.POINTER(PendulumParameters), I, LP, I, P, I, I, P, P, P],
     "ppo_gae": [P, P, P, P, P, P, I, I, I, F, F, I],
     "gru_forward": [C.POINTER(GruLayer), P, P, I, I, P, S],
     "gru_backward": [C.POINTER(GruLayer), P, P, P, P, I, I, I, P, S],

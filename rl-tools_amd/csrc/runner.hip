@@ -376,6 +376,71 @@ bool rb_ok(const rlt_replay_buffer* rb) {
            rb->observation_dim > 0 && rb->action_dim > 0;
 }
 
+
+// ---- evaluation episodes (rl/utils/evaluation/operations_generic.h:106-233) ----------------------------------------------------
+// One launch runs every step of every episode for actors 3 -> H -> H -> out with H <= 64: a wavefront per episode, lane j holds hidden unit j of both
+// hidden layers (its row of W1, its bias, its column of W3 in registers, W2 in LDS), the first layer's activations pass between lanes with
+// v_readlane, the output is a wavefront sum; every lane carries the environment state, so nothing else is exchanged. The chain of step_limit
+// dependent steps bounds the kernel.
+struct EvaluateArgs {
+    rlt_pendulum_parameters env;
+    const float *w1, *b1, *w2, *b2, *w3, *b3;
+    int H, act1, act2, act_out, policy_kind, step_limit;
+    const float* initial_states; float* returns; uint32_t* episode_length;
+};
+__global__ __launch_bounds__(64) void pendulum_evaluate_kernel(EvaluateArgs A) {
+    __shared__ float w2s[64 * 65];
+    const int j = threadIdx.x, e = blockIdx.x, H = A.H;
+    for (int n = 0; n < H; n++) if (j < H) w2s[n * 65 + j] = A.w2[n * H + j];
+    __syncthreads();
+    const bool live = j < H;
+    const int jc = live ? j : 0;
+    const float w10 = A.w1[jc * 3], w11 = A.w1[jc * 3 + 1], w12 = A.w1[jc * 3 + 2], b1 = A.b1[jc], b2 = A.b2[jc], w3 = live ? A.w3[jc] : 0.f, b3 = A.b3[0];
+    float theta = A.initial_states[2 * e], theta_dot = A.initial_states[2 * e + 1], episode_return = 0.f;
+    float sn, cs;
+    sincosf(theta, &sn, &cs);
+    for (int step = 0; step < A.step_limit; step++) {
+        const float h1 = live ? rlt_act(b1 + w10 * cs + w11 * sn + w12 * theta_dot, A.act1) : 0.f;
+        float acc = b2;
+        for (int k = 0; k < H; k++) acc += w2s[j * 65 + k] * __int_as_float(__builtin_amdgcn_readlane(__float_as_int(h1), k));
+        const float h2 = live ? rlt_act(acc, A.act2) : 0.f;
+        const float y = rlt_act(rlt_wave_sum(w3 * h2) + b3, A.act_out);
+        // Evaluation mode: the action is the output, or the squashed mean of a [mean | log_std] head (sample_and_squash with zero noise)
+        const float action = A.policy_kind == 2 ? tanhf(y) : y;
+        Transition t;
+        pendulum_transition(A.env, theta, theta_dot, action, t);
+        theta = t.theta; theta_dot = t.theta_dot; cs = t.next_obs[0]; sn = t.next_obs[1];
+        episode_return += t.reward;      // the Pendulum has no terminal states: every step counts (:188-197)
+    }
+    if (j == 0) { A.returns[e] = episode_return; A.episode_length[e] = (uint32_t)A.step_limit; }
+}
+// other actor shapes: one step of all episodes per launch around the per-layer network kernels
+__global__ __launch_bounds__(256) void evaluate_observe_kernel(const float* __restrict__ states, float* __restrict__ obs, int n) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    float sn, cs; sincosf(states[2 * e], &sn, &cs);
+    obs[3 * e] = cs; obs[3 * e + 1] = sn; obs[3 * e + 2] = states[2 * e + 1];
+}
+__global__ __launch_bounds__(256) void evaluate_step_kernel(rlt_pendulum_parameters env, float* __restrict__ states, const float* __restrict__ actor_out, int ld_out, int policy_kind,
+                                                            float* __restrict__ returns, uint32_t* __restrict__ episode_length, int n) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    const float y = actor_out[(size_t)e * ld_out], action = policy_kind == 2 ? tanhf(y) : y;
+    Transition t;
+    pendulum_transition(env, states[2 * e], states[2 * e + 1], action, t);
+    states[2 * e] = t.theta; states[2 * e + 1] = t.theta_dot;
+    returns[e] += t.reward; episode_length[e] += 1;
+}
+// mean and standard deviation of returns and episode lengths, accumulated in episode order as the reference does (:213-227)
+__global__ void evaluate_summary_kernel(const float* __restrict__ returns, const uint32_t* __restrict__ episode_length, int n, float* __restrict__ summary) {
+    if (blockIdx.x != 0 || threadIdx.x != 0) return;
+    float rm = 0.f, rs = 0.f, lm = 0.f, ls = 0.f;
+    for (int e = 0; e < n; e++) { rm += returns[e]; rs += returns[e] * returns[e]; lm += (float)episode_length[e]; ls += (float)(episode_length[e] * episode_length[e]); }
+    rm /= (float)n; lm /= (float)n;
+    summary[0] = rm; summary[1] = sqrtf(fmaxf(0.f, rs / (float)n - rm * rm));
+    summary[2] = lm; summary[3] = sqrtf(fmaxf(0.f, ls / (float)n - lm * lm));
+    summary[4] = 0.f; summary[5] = 0.f;       // num_terminated, share_terminated
+}
 }  // namespace
 
 extern "C" {
@@ -501,4 +566,46 @@ int rlt_rocm_on_policy_collect(rlt_rocm_device* device, const rlt_pendulum_runne
     return rlt_launch_status(device);
 }
 
+// rl::utils::evaluation::evaluate with the Pendulum environment (rl/utils/evaluation/operations_generic.h:106-233)
+int rlt_rocm_pendulum_evaluate(rlt_rocm_device* device, const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers,
+                               const float* initial_states, int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(env && actor && n_actor_layers >= 1 && initial_states && n_episodes >= 1 && step_limit >= 1 && returns && episode_length && summary);
+    RLT_REQUIRE((policy_kind == 1 || policy_kind == 2) && actor[0].in_dim == 3 && actor[n_actor_layers - 1].out_dim == policy_kind);
+    for (int l = 0; l < n_actor_layers; l++) RLT_REQUIRE(actor[l].weights && actor[l].biases && (l == 0 || actor[l].in_dim == actor[l - 1].out_dim));
+    const int N = n_episodes;
+    int rc;
+    if (n_actor_layers == 3 && actor[0].out_dim <= 64 && actor[1].out_dim == actor[0].out_dim) {
+        EvaluateArgs a = {};
+        a.env = *env;
+        a.w1 = actor[0].weights; a.b1 = actor[0].biases; a.w2 = actor[1].weights; a.b2 = actor[1].biases; a.w3 = actor[2].weights; a.b3 = actor[2].biases;
+        a.H = actor[0].out_dim; a.act1 = actor[0].activation; a.act2 = actor[1].activation; a.act_out = actor[2].activation; a.policy_kind = policy_kind; a.step_limit = step_limit;
+        a.initial_states = initial_states; a.returns = returns; a.episode_length = episode_length;
+        hipLaunchKernelGGL(pendulum_evaluate_kernel, dim3(N), dim3(64), 0, device->stream, a);
+        if ((rc = rlt_launch_status(device))) return rc;
+    } else {
+        // scratch: states [N x 2], observations [N x 3], actor output [N x out], then the network workspace
+        const int out_dim = policy_kind;
+        const size_t mlp_ws = rlt_rocm_mlp_workspace_bytes(actor, n_actor_layers, N);
+        const size_t head = (((size_t)N * (5 + out_dim) * sizeof(float)) + 255) & ~(size_t)255;
+        void* scratch;
+        if ((rc = rlt_scratch(device, head + mlp_ws, &scratch))) return rc;
+        float* states = (float*)scratch; float* obs = states + (size_t)N * 2; float* out = obs + (size_t)N * 3;
+        void* ws = (char*)scratch + head;
+        RLT_HIP(hipMemcpyAsync(states, initial_states, (size_t)N * 2 * sizeof(float), hipMemcpyDeviceToDevice, device->stream));
+        if ((rc = rlt_rocm_fill_f32(device, returns, 1, N, N, 0.0f))) return rc;
+        if ((rc = rlt_rocm_fill_f32(device, (float*)episode_length, 1, N, N, 0.0f))) return rc;      // the bit pattern of 0.0f is the integer 0
+        for (int step = 0; step < step_limit; step++) {
+            hipLaunchKernelGGL(evaluate_observe_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, states, obs, N);
+            if ((rc = rlt_launch_status(device))) return rc;
+            if ((rc = rlt_rocm_mlp_evaluate(device, actor, n_actor_layers, obs, 3, out, out_dim, N, ws, mlp_ws))) return rc;
+            hipLaunchKernelGGL(evaluate_step_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *env, states, out, out_dim, policy_kind, returns, episode_length, N);
+            if ((rc = rlt_launch_status(device))) return rc;
+        }
+    }
+    hipLaunchKernelGGL(evaluate_summary_kernel, dim3(1), dim3(64), 0, device->stream, returns, episode_length, N, summary);
+    return rlt_launch_status(device);
+}
+
 }  // extern "C"
+

@@ -779,3 +779,14 @@ def on_policy_golden_collect(backend, g, k, dims, col):
     actor = Mlp(backend, [3, hidden, hidden, 1], g[f"c{k}_actor"], n, "tanh", "identity", trainable=False)
     o.collect(actor, g[f"c{k}_log_std"], g[f"c{k}_noise"], g[f"c{k}_initial_states"], standardize=(g[f"c{k}_standardize_mean"], g[f"c{k}_standardize_precision"]))
     return o
+
+
+def evaluate_on_backend(backend, dims, params, hidden_act, out_act, policy_kind, initial_states, step_limit):
+    """rl::utils::evaluation::evaluate on a backend: returns (returns, episode_length, summary) as numpy arrays."""
+    n = initial_states.shape[0]
+    actor = Mlp(backend, dims, params, n, hidden_act, out_act, trainable=False)
+    ini, ret, length, summary = backend.array(initial_states.astype(np.float32)), backend.zeros((n,)), backend.zeros((n,), np.uint32), backend.zeros((6,))
+    env = capi.pendulum_parameters()
+    backend.call("pendulum_evaluate", C.byref(env), policy_kind, actor.layers, actor.n, ini.ptr, n, step_limit, ret.ptr, length.ptr, summary.ptr)
+    backend.sync()
+    return ret.numpy(), length.numpy(), summary.numpy()

@@ -245,3 +245,24 @@ def test_standardize_and_running_normaliser_closed_forms(oracle):
         want_std = np.mean(stds, 0); want_std[2] = 0 if k == 0 else want_std[2]
         assert np.allclose(np.delete(rs.numpy(), 2), np.delete(np.mean(stds, 0), 2), rtol=1e-5)
     assert rs.numpy()[2] == 0                      # first update: 1 + (0 - 1) / 1, then 0 + (0 - 0) / k
+
+
+def test_evaluation_reproduces_reference_vectors(oracle):
+    """rl::utils::evaluation::evaluate (10 episodes x 200 steps, Evaluation mode) of the SAC actor after 0, 150 and 400 loop steps: returns, episode
+    lengths and summary statistics equal the reference's bit for bit (tests/golden/make_evaluation_golden.py). A deterministic actor with a tanh
+    output layer whose single output row is the mean row of the same network must give the same episodes: that pins policy kind 1."""
+    g = np.load(os.path.join(helpers.GOLDEN, "evaluation_pendulum_seed0.npz"))
+    for k in range(3):
+        params, ini = g[f"e{k}_actor"], g[f"e{k}_initial_states"]
+        ret, length, summary = helpers.evaluate_on_backend(oracle, [3, 64, 64, 2], params, "relu", "identity", 2, ini, 200)
+        assert np.array_equal(ret, g[f"e{k}_returns"]) and np.array_equal(length, g[f"e{k}_episode_length"]) and np.array_equal(summary, g[f"e{k}_summary"])
+        # statistics as the definition has them (population standard deviation), in float64
+        assert abs(summary[0] - ret.astype(np.float64).mean()) <= 1e-3 and abs(summary[1] - ret.astype(np.float64).std()) <= 1e-2
+        assert summary[2] == 200 and summary[3] == 0 and summary[4] == 0 and summary[5] == 0
+        head = 3 * 64 + 64 + 64 * 64 + 64
+        mean_only = np.concatenate([params[:head], params[head:head + 64], params[head + 128:head + 129]])     # first row of W3, first bias
+        ret1, length1, summary1 = helpers.evaluate_on_backend(oracle, [3, 64, 64, 1], mean_only, "relu", "tanh", 1, ini, 200)
+        assert np.array_equal(ret1, ret) and np.array_equal(summary1, summary)
+    # shorter horizon: the return is a prefix sum of the same rewards, so it is larger (rewards are negative) and the lengths follow the limit
+    ret50, length50, _ = helpers.evaluate_on_backend(oracle, [3, 64, 64, 2], g["e2_actor"], "relu", "identity", 2, g["e2_initial_states"], 50)
+    assert np.all(length50 == 50) and np.all(ret50 > g["e2_returns"]) and np.all(ret50 < 0)

@@ -21,7 +21,15 @@ def load_ref(path):
     for name, args in dict(step=[P], destroy=[P], get_parameters=[P, P], get_batch=[P, P, P, P], get_noise=[P, P, P], get_replay=[P, P, P, P, P],
                            get_critic_buffers=[P, C.c_int, P, P, P, P, P], get_actor_buffers=[P, P, P, P, P]).items():
         getattr(ref, "rlt_ref_sac_" + name).argtypes = args
+    ref.rlt_ref_sac_evaluate.argtypes = [P, C.c_uint32, P, P, P, P]
     return ref
+
+
+def reference_evaluation(ref, h, seed):
+    """rl::utils::evaluation::evaluate of the loop's current actor by the reference: 10 episodes x 200 steps in Evaluation mode."""
+    ini, ret, length, summary = np.zeros((10, 2), np.float32), np.zeros(10, np.float32), np.zeros(10, np.uint32), np.zeros(6, np.float32)
+    ref.rlt_ref_sac_evaluate(h, seed, ini.ctypes.data, ret.ctypes.data, length.ctypes.data, summary.ctypes.data)
+    return ini, ret, length, summary
 
 
 def np_from(ptr, shape, dtype=np.float32):
@@ -67,6 +75,33 @@ def test_loop_bit_exact_with_reference_generic_build(oracle, batch, steps):
     assert pos.value == np_from(rb.position, (1,), np.uint32)[0] and not full.value
     assert np.array_equal(data[:pos.value], np_from(rb.data, (10000, 10))[:pos.value])      # rows beyond the cursor are uninitialised in the reference
     assert np.array_equal(es[:pos.value], np_from(rb.episode_start, (10000,), np.uint32)[:pos.value])
+    lib.rlt_oracle_sac_loop_destroy(loop); ref.rlt_ref_sac_destroy(h)
+
+
+def test_evaluation_bit_exact_with_reference(oracle):
+    """rl::utils::evaluation::evaluate (10 episodes x 200 steps, Evaluation mode, sampled initial states) of the actor after 0, 150 and 400 loop
+    steps: the reference's returns, episode lengths and statistics against the checker's, which is handed the same actor and the initial states
+    the reference drew. Bit for bit: dynamics, observation, network and tanh are the same float operations in the same order."""
+    ref, lib = load_ref(helpers.REF_GENERIC), oracle.lib
+    batch = 100
+    cfg = helpers.LoopConfig(0, batch, 64, 10000, 100, 200, 1e-7)
+    loop = C.c_void_p(lib.rlt_oracle_sac_loop_create(C.byref(cfg)))
+    h = C.c_void_p(ref.rlt_ref_sac_create(0, batch))
+    A = lib.rlt_oracle_sac_loop_agent(loop).contents
+    env = helpers.capi.pendulum_parameters()
+    seen = []
+    for stop, seed in ((0, 5), (150, 6), (400, 7)):
+        while ref.rlt_ref_sac_step_count(h) < stop:
+            assert lib.rlt_oracle_sac_loop_step(loop) == 0
+            ref.rlt_ref_sac_step(h)
+        ini, want_ret, want_len, want_sum = reference_evaluation(ref, h, seed)
+        assert np.all(np.abs(ini[:, 0]) <= np.pi) and np.all(np.abs(ini[:, 1]) <= 1.0) and len(np.unique(ini[:, 0])) == 10
+        ret, length, summary = np.zeros(10, np.float32), np.zeros(10, np.uint32), np.zeros(6, np.float32)
+        assert lib.rlt_oracle_pendulum_evaluate(C.byref(env), 2, A.actor, 3, ini.ctypes.data, 10, 200, ret.ctypes.data, length.ctypes.data, summary.ctypes.data) == 0
+        assert np.array_equal(ret, want_ret) and np.array_equal(length, want_len) and np.array_equal(summary, want_sum), (stop, ret, want_ret)
+        assert np.all(length == 200) and summary[4] == 0 and np.all(ret < 0)
+        seen.append(summary[0])
+    assert len(set(seen)) == 3          # the actor changed between the evaluations
     lib.rlt_oracle_sac_loop_destroy(loop); ref.rlt_ref_sac_destroy(h)
 
 

@@ -1,0 +1,61 @@
+"""Evaluation episodes on the device (rlt_rocm_pendulum_evaluate) against the CPU checker and the reference's own results, through the C ABI.
+
+Tolerance: fp32 rollouts of a closed loop amplify rounding differences step by step, so returns are compared at 1e-5 relative over short horizons
+(20 steps) and at 2e-3 over the reference's 200 steps; episode lengths and the terminated counts are integers and must be equal."""
+import os
+
+import numpy as np
+import pytest
+
+import helpers
+from helpers import rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def test_evaluation_against_reference_vectors(rocm):
+    """The SAC actor after 0, 150 and 400 loop steps, 10 episodes x 200 steps from the initial states the reference drew: the reference's returns and
+    statistics (tests/golden/evaluation_pendulum_seed0.npz)."""
+    g = np.load(os.path.join(helpers.GOLDEN, "evaluation_pendulum_seed0.npz"))
+    for k in range(3):
+        ret, length, summary = helpers.evaluate_on_backend(rocm, [3, 64, 64, 2], g[f"e{k}_actor"], "relu", "identity", 2, g[f"e{k}_initial_states"], 200)
+        assert np.array_equal(length, g[f"e{k}_episode_length"])
+        assert rel_err(ret, g[f"e{k}_returns"]) <= 2e-3, (k, ret, g[f"e{k}_returns"])
+        assert rel_err(summary[:2], g[f"e{k}_summary"][:2]) <= 2e-3 and np.array_equal(summary[2:], g[f"e{k}_summary"][2:])
+
+
+# (hidden width, layers, policy kind, hidden activation, output activation, episodes): one launch for three layers of width <= 64, else step by step
+CASES = [(64, 3, 2, "relu", "identity", 10), (64, 3, 1, "tanh", "tanh", 100), (32, 3, 1, "relu", "tanh", 7), (17, 3, 2, "fast_tanh", "identity", 64),
+         (256, 3, 2, "relu", "identity", 33), (64, 2, 1, "tanh", "tanh", 10), (48, 4, 2, "relu", "identity", 300)]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_evaluation_matches_checker(oracle, rocm, case):
+    print("case", case, flush=True)
+    H, layers, kind, ha, oa, n = case
+    dims = [3] + [H] * (layers - 1) + [kind]
+    rng = np.random.default_rng(H + n)
+    params = helpers.random_params(rng, dims)
+    ini = np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n)], 1).astype(np.float32)
+    for steps, tol in ((20, 1e-5), (200, 2e-3)):
+        want = helpers.evaluate_on_backend(oracle, dims, params, ha, oa, kind, ini, steps)
+        got = helpers.evaluate_on_backend(rocm, dims, params, ha, oa, kind, ini, steps)
+        assert np.array_equal(got[1], want[1]) and np.all(got[1] == steps)
+        assert rel_err(got[0], want[0]) <= tol, (steps, rel_err(got[0], want[0]))
+        assert rel_err(got[2][:2], want[2][:2]) <= tol and np.array_equal(got[2][2:], want[2][2:])
+
+
+def test_evaluation_rejects_bad_arguments(rocm):
+    capi = helpers.capi
+    import ctypes as C
+    dims = [3, 64, 64, 2]
+    actor = helpers.Mlp(rocm, dims, helpers.random_params(np.random.default_rng(0), dims), 4, trainable=False)
+    ini, ret, length, summary = rocm.zeros((4, 2)), rocm.zeros((4,)), rocm.zeros((4,), np.uint32), rocm.zeros((6,))
+    env = capi.pendulum_parameters()
+    lib, h = rocm.device.lib, rocm.device.handle
+    bad = capi.RLT_E_INVALID_ARGUMENT if hasattr(capi, "RLT_E_INVALID_ARGUMENT") else -1
+    assert lib.rlt_rocm_pendulum_evaluate(h, C.byref(env), 1, actor.layers, 3, ini.ptr, 4, 10, ret.ptr, length.ptr, summary.ptr) != 0      # kind 1 needs one output
+    assert lib.rlt_rocm_pendulum_evaluate(h, C.byref(env), 2, actor.layers, 3, ini.ptr, 0, 10, ret.ptr, length.ptr, summary.ptr) != 0
+    assert lib.rlt_rocm_pendulum_evaluate(h, C.byref(env), 2, actor.layers, 3, None, 4, 10, ret.ptr, length.ptr, summary.ptr) != 0
+    assert lib.rlt_rocm_pendulum_evaluate(h, C.byref(env), 2, actor.layers, 3, ini.ptr, 4, 10, ret.ptr, length.ptr, summary.ptr) == 0
+    rocm.sync()
