@@ -18,6 +18,10 @@
  *   /root/reference (oracle/_ref), and against golden vectors written by them (tests/golden).
  *   on-policy collect (with the reference's RNG order), running normaliser, standardize statistics: bit for bit against the
  *   reference's PPO loop with observation normalisation on (oracle/_ref), golden vectors, and closed forms in numpy.
+ *   pendulum evaluate (evaluation episodes): returns, episode lengths and summary statistics bit for bit against the reference's
+ *   rl::utils::evaluation::evaluate on the SAC loop's actor at three stages of training (oracle/_ref), golden vectors, and the
+ *   identity between the two policy kinds on a mean-only copy of the actor.
+ *   ppo train_epoch: the loop over ppo train_minibatch (pinned above) that the reference's train() runs per epoch.
  */
 #ifndef RLT_ORACLE_H
 #define RLT_ORACLE_H
