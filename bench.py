@@ -148,9 +148,26 @@ def bench_env(helpers, rocm, n_envs=65536, capacity=16, steps=200, batch=4096):
         evaluate()
     e = ev.record()
     evaluate_us = ev.elapsed_ms(a, e) * 1e3 / 20
+    # AcrobotSwingup: one Runge-Kutta step of a million environments with all outputs (state 16 B in and out, action 4, observations 2 x 24, reward 4, flag 1 = 89 B each)
+    n_acro = 1 << 20
+    acro_p = capi.acrobot_parameters()
+    a_states = rocm.array(rng.uniform(-1, 1, (n_acro, 4)).astype(np.float32)); a_actions = rocm.array(rng.uniform(-1, 1, n_acro).astype(np.float32))
+    a_obs, a_next, a_rew, a_term = rocm.zeros((n_acro, 6)), rocm.zeros((n_acro, 6)), rocm.zeros((n_acro,)), rocm.zeros((n_acro,), np.uint8)
+
+    def acrobot():
+        rocm.call("acrobot_step", C.byref(acro_p), 1, a_states.ptr, a_actions.ptr, a_obs.ptr, a_next.ptr, a_rew.ptr, a_term.ptr, n_acro)
+    for _ in range(3):
+        acrobot()
+    rocm.sync()
+    a = ev.record()
+    for _ in range(50):
+        acrobot()
+    e = ev.record()
+    acrobot_us = ev.elapsed_ms(a, e) * 1e3 / 50
     return {"n_envs": n_envs, "replay_rows": n_envs * capacity, "steps": steps, "us_per_step": ms * 1e3 / steps, "env_steps_per_s": env_steps / (ms * 1e-3),
             "algorithmic_GBps": env_steps * 68 / (ms * 1e-3) / 1e9, "gather_batch": batch, "gather_us": gather_us, "gather_algorithmic_GBps": batch * 85 / (gather_us * 1e-6) / 1e9,
-            "evaluation_10_episodes_x_200_steps_us": evaluate_us}
+            "evaluation_10_episodes_x_200_steps_us": evaluate_us,
+            "acrobot": {"n_envs": n_acro, "us_per_step": acrobot_us, "env_steps_per_s": n_acro / (acrobot_us * 1e-6), "algorithmic_GBps": n_acro * 89 / (acrobot_us * 1e-6) / 1e9}}
 
 
 def bench_ppo(helpers, rocm, n_envs=4096, steps=128, epochs=4, minibatch=8192):

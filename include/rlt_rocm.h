@@ -359,6 +359,20 @@ int rlt_rocm_pendulum_step(rlt_rocm_device* device, const rlt_pendulum_parameter
                            const float* actions, float* observations, float* next_observations,
                            float* rewards, int n_envs);
 
+/* rl/environments/acrobot/acrobot.h:14-37 (DefaultParameters; EasyParameters widen the torque range to +-10) */
+typedef struct rlt_acrobot_parameters {
+    float dt, link_length_1, link_length_2, link_mass_1, link_mass_2, link_com_pos_1, link_com_pos_2, link_moi;
+    float max_vel_1, max_vel_2, min_torque, max_torque;
+} rlt_acrobot_parameters;
+
+/* step + reward + terminated + observe of the Acrobot (swingup = 0) or the AcrobotSwingup (swingup = 1)
+ * rl/environments/acrobot/operations_generic.h:56-117 (dsdt, rk4), :118-144 (step), :145-171 (reward), :173-193 (observe, terminated)
+ *   states [n_envs x 4] = (theta_1, theta_2, theta_1_dot, theta_2_dot) updated in place; actions [n_envs] (un-clamped, in [-1, 1]
+ *   after clamping, scaled to [min_torque, max_torque]); observations (pre-step) and next_observations [n_envs x 6];
+ *   rewards [n_envs]; terminated [n_envs] of the NEXT state. Any output may be NULL. */
+int rlt_rocm_acrobot_step(rlt_rocm_device* device, const rlt_acrobot_parameters* p, int swingup, float* states, const float* actions,
+                          float* observations, float* next_observations, float* rewards, uint8_t* terminated, int n_envs);
+
 /* Per-environment runner state (rl/components/off_policy_runner/off_policy_runner.h:184-221). */
 typedef struct rlt_pendulum_runner {
     float* states;            /* [n_envs x 2]  */

@@ -1,0 +1,55 @@
+// Harness around the REAL reference's analytic environments other than the Pendulum (compiled from /root/reference/include where it lies; nothing
+// of it is copied here): batched step / reward / observe / terminated of the Acrobot and the AcrobotSwingup with their default parameters, and the
+// initial states their sample_initial_state draws. Built by oracle/Makefile into oracle/_ref/librlt_ref_envs_generic.so.
+#include <rl_tools/operations/cpu_mux.h>
+#include <rl_tools/rl/environments/acrobot/operations_cpu.h>
+
+#include <cstdint>
+
+namespace rlt = rl_tools;
+
+namespace {
+using DEVICE = rlt::devices::DEVICE_FACTORY<>;
+using RNG = DEVICE::SPEC::RANDOM::ENGINE<>;
+using TI = typename DEVICE::index_t;
+using SPEC = rlt::rl::environments::acrobot::Specification<float, TI, rlt::rl::environments::acrobot::DefaultParameters<float>>;
+using EASY_SPEC = rlt::rl::environments::acrobot::Specification<float, TI, rlt::rl::environments::acrobot::EasyParameters<float>>;
+
+template <typename ENVIRONMENT>
+void steps(const float* states, const float* actions, float* next_states, float* observations, float* next_observations, float* rewards, uint8_t* terminated, int n) {
+    DEVICE device;
+    RNG rng;
+    rlt::malloc(device, rng);
+    rlt::init(device, rng, 0);
+    ENVIRONMENT env;
+    typename ENVIRONMENT::Parameters parameters;
+    rlt::Matrix<rlt::matrix::Specification<float, TI, 1, 1, false>> action;
+    rlt::Matrix<rlt::matrix::Specification<float, TI, 1, 6, false>> observation;
+    for (int e = 0; e < n; e++) {
+        typename ENVIRONMENT::State state, next;
+        state.theta_1 = states[4 * e]; state.theta_2 = states[4 * e + 1]; state.theta_1_dot = states[4 * e + 2]; state.theta_2_dot = states[4 * e + 3];
+        rlt::set(action, 0, 0, actions[e]);
+        rlt::observe(device, env, parameters, state, typename ENVIRONMENT::Observation{}, observation, rng);
+        for (TI i = 0; i < 6; i++) observations[6 * e + i] = rlt::get(observation, 0, i);
+        rlt::step(device, env, parameters, state, action, next, rng);
+        rewards[e] = rlt::reward(device, env, parameters, state, action, next, rng);
+        terminated[e] = rlt::terminated(device, env, parameters, next, rng);
+        rlt::observe(device, env, parameters, next, typename ENVIRONMENT::Observation{}, observation, rng);
+        for (TI i = 0; i < 6; i++) next_observations[6 * e + i] = rlt::get(observation, 0, i);
+        next_states[4 * e] = next.theta_1; next_states[4 * e + 1] = next.theta_2; next_states[4 * e + 2] = next.theta_1_dot; next_states[4 * e + 3] = next.theta_2_dot;
+    }
+    rlt::free(device, rng);
+}
+}  // namespace
+
+extern "C" {
+// kind 0: Acrobot, 1: AcrobotSwingup, 2: AcrobotSwingup with EasyParameters (torque +-10)
+int rlt_ref_acrobot_steps(int kind, const float* states, const float* actions, float* next_states, float* observations, float* next_observations, float* rewards,
+                          uint8_t* terminated, int n) {
+    if (kind == 0) steps<rlt::rl::environments::Acrobot<SPEC>>(states, actions, next_states, observations, next_observations, rewards, terminated, n);
+    else if (kind == 1) steps<rlt::rl::environments::AcrobotSwingup<SPEC>>(states, actions, next_states, observations, next_observations, rewards, terminated, n);
+    else if (kind == 2) steps<rlt::rl::environments::AcrobotSwingup<EASY_SPEC>>(states, actions, next_states, observations, next_observations, rewards, terminated, n);
+    else return -1;
+    return 0;
+}
+}

@@ -674,6 +674,64 @@ static inline void pendulum_dynamics(const rlt_pendulum_parameters* p, float the
     float costs = (float)(angle_norm * angle_norm + 0.1 * theta_dot * theta_dot + 0.001 * (ur * ur));
     *reward = -costs;
 }
+// rl/environments/acrobot/operations_generic.h:56-117 (dsdt, rk4), :118-144 (step), :145-171 (reward), :173-193 (observe, terminated).
+// The reference writes these with T = float but with double literals (2.0, 6.0, 1.0, 0.02) and with unqualified cos / sin in dsdt and
+// terminated, which resolve to the double functions; the sub-expressions they touch are evaluated in double and rounded once on assignment.
+// The expressions below are typed so that the same promotions happen (bit-identical to the compiled reference on random states).
+static void acrobot_dsdt(const rlt_acrobot_parameters* P, const float state[4], float action, float d_state[4]) {
+    const float m1 = P->link_mass_1, m2 = P->link_mass_2, l1 = P->link_length_1, lc1 = P->link_com_pos_1, lc2 = P->link_com_pos_2, I1 = P->link_moi, I2 = P->link_moi;
+    const float g = 9.8;
+    const float PI = (float)M_PI;
+    const float theta1 = state[0], theta2 = state[1], dtheta1 = state[2], dtheta2 = state[3];
+    auto c = [](double x) { return std::cos(x); };
+    auto sn = [](double x) { return std::sin(x); };
+    const float d1 = m1 * lc1 * lc1 + m2 * (l1 * l1 + lc2 * lc2 + 2 * l1 * lc2 * c(theta2)) + I1 + I2;
+    const float d2 = m2 * (lc2 * lc2 + l1 * lc2 * c(theta2)) + I2;
+    const float phi2 = m2 * lc2 * g * c(theta1 + theta2 - PI / 2.0);
+    const float phi1 = -m2 * l1 * lc2 * dtheta2 * dtheta2 * sn(theta2) - 2 * m2 * l1 * lc2 * dtheta2 * dtheta1 * sn(theta2) + (m1 * lc1 + m2 * l1) * g * c(theta1 - PI / 2) + phi2;
+    const float ddtheta2 = (action + d2 / d1 * phi1 - m2 * l1 * lc2 * dtheta1 * dtheta1 * sn(theta2) - phi2) / (m2 * lc2 * lc2 + I2 - d2 * d2 / d1);
+    const float ddtheta1 = -(d2 * ddtheta2 + phi1) / d1;
+    d_state[0] = dtheta1; d_state[1] = dtheta2; d_state[2] = ddtheta1; d_state[3] = ddtheta2;
+}
+static void acrobot_rk4(const rlt_acrobot_parameters* P, const float state[4], float action, float next_state[4], float dt) {
+    float k1[4], k2[4], k3[4], k4[4], y1[4], y2[4], y3[4];
+    const float dt2 = dt / 2.0;
+    acrobot_dsdt(P, state, action, k1);
+    for (int i = 0; i < 4; i++) y1[i] = state[i] + dt2 * k1[i];
+    acrobot_dsdt(P, y1, action, k2);
+    for (int i = 0; i < 4; i++) y2[i] = state[i] + dt2 * k2[i];
+    acrobot_dsdt(P, y2, action, k3);
+    for (int i = 0; i < 4; i++) y3[i] = state[i] + dt * k3[i];
+    acrobot_dsdt(P, y3, action, k4);
+    for (int i = 0; i < 4; i++) next_state[i] = state[i] + dt / 6.0 * (k1[i] + 2 * k2[i] + 2 * k3[i] + k4[i]);
+}
+int rlt_oracle_acrobot_step(const rlt_acrobot_parameters* P, int swingup, float* states, const float* actions, float* observations, float* next_observations,
+                            float* rewards, uint8_t* terminated, int n_envs) {
+    if (!P || !states || !actions || n_envs <= 0) return RLT_E_INVALID_ARGUMENT;
+    const float PI = (float)M_PI;
+    for (int e = 0; e < n_envs; e++) {
+        float* s = states + 4 * (size_t)e;
+        float next[4];
+        if (observations) { float* o = observations + 6 * (size_t)e; o[0] = std::cos(s[0]); o[1] = std::sin(s[0]); o[2] = std::cos(s[1]); o[3] = std::sin(s[1]); o[4] = s[2]; o[5] = s[3]; }
+        const float action_clamped = clampf(actions[e], -1.0f, 1.0f);
+        const float action_scaled = (action_clamped + 1.0) / 2.0 * (P->max_torque - (P->min_torque)) + (P->min_torque);
+        acrobot_rk4(P, s, action_scaled, next, P->dt);
+        next[0] = angle_normalize(next[0]); next[1] = angle_normalize(next[1]);
+        next[2] = clampf(next[2], -P->max_vel_1, P->max_vel_1); next[3] = clampf(next[3], -P->max_vel_2, P->max_vel_2);
+        if (rewards) {
+            if (!swingup) rewards[e] = -1;
+            else {
+                const float a_angle_cost = std::fabs(angle_normalize(next[0] - PI)), b_angle_cost = std::fabs(angle_normalize(next[1]));
+                rewards[e] = (-a_angle_cost - b_angle_cost) / 100 * P->dt / 0.02;
+            }
+        }
+        if (terminated) terminated[e] = swingup ? 0 : ((-std::cos((double)next[0]) - std::cos((double)(next[1] + next[0]))) > 1.0);
+        if (next_observations) { float* o = next_observations + 6 * (size_t)e; o[0] = std::cos(next[0]); o[1] = std::sin(next[0]); o[2] = std::cos(next[1]); o[3] = std::sin(next[1]); o[4] = next[2]; o[5] = next[3]; }
+        for (int i = 0; i < 4; i++) s[i] = next[i];
+    }
+    return 0;
+}
+
 int rlt_oracle_pendulum_step(const rlt_pendulum_parameters* p, float* states, const float* actions, float* observations,
                              float* next_observations, float* rewards, int n_envs) {
     if (!p || !states || !actions || n_envs <= 0) return RLT_E_INVALID_ARGUMENT;

@@ -21,6 +21,9 @@
  *   pendulum evaluate (evaluation episodes): returns, episode lengths and summary statistics bit for bit against the reference's
  *   rl::utils::evaluation::evaluate on the SAC loop's actor at three stages of training (oracle/_ref), golden vectors, and the
  *   identity between the two policy kinds on a mean-only copy of the actor.
+ *   acrobot step (dsdt, Runge-Kutta, reward, terminated, observe): bit for bit against the reference's Acrobot, AcrobotSwingup and EasyParameters
+ *   environments (oracle/_ref/librlt_ref_envs_generic.so) on random states and closed chains, golden vectors, and energy conservation /
+ *   integration order / work-energy checks that do not involve the reference.
  *   ppo train_epoch: the loop over ppo train_minibatch (pinned above) that the reference's train() runs per epoch.
  */
 #ifndef RLT_ORACLE_H
@@ -102,6 +105,9 @@ int rlt_oracle_ppo_gae(const float* rewards, const float* terminated, const floa
                        float* advantages, float* target_values, int ld, int n_envs, int steps, float gamma, float lambda,
                        int ignore_termination);
 
+/* rl/environments/acrobot/operations_generic.h:56-193 */
+int rlt_oracle_acrobot_step(const rlt_acrobot_parameters* p, int swingup, float* states, const float* actions, float* observations, float* next_observations,
+                            float* rewards, uint8_t* terminated, int n_envs);
 /* rl::utils::evaluation::evaluate with the Pendulum environment (rl/utils/evaluation/operations_generic.h:106-233) */
 int rlt_oracle_pendulum_evaluate(const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers, const float* initial_states,
                                  int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary);

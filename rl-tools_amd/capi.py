@@ -75,6 +75,19 @@ def pendulum_parameters():
     return PendulumParameters(10.0, 8.0, 2.0, 0.05, 1.0, 1.0)
 
 
+class AcrobotParameters(C.Structure):
+    _fields_ = [(name, C.c_float) for name in ("dt", "link_length_1", "link_length_2", "link_mass_1", "link_mass_2", "link_com_pos_1", "link_com_pos_2", "link_moi",
+                                               "max_vel_1", "max_vel_2", "min_torque", "max_torque")]
+
+
+def acrobot_parameters(easy=False):
+    """rl/environments/acrobot/acrobot.h:14-37 DefaultParameters (EasyParameters: torque range +-10)"""
+    import math
+    t = 10.0 if easy else 5.0
+    pi = C.c_float(math.pi).value
+    return AcrobotParameters(0.2, 1.0, 1.0, 1.0, 1.0, 0.5, 0.5, 1.0, 4 * pi, 9 * pi, -t, t)
+
+
 class PendulumRunner(C.Structure):
     _fields_ = [("states", C.c_void_p), ("episode_step", C.c_void_p), ("episode_return", C.c_void_p), ("truncated", C.c_void_p),
                 ("n_envs", C.c_int32), ("episode_step_limit", C.c_int32), ("env", PendulumParameters)]
@@ -174,6 +187,7 @@ PROTOTYPES = {
     "replay_add": [C.POINTER(ReplayBuffer), P, P, P, P, P, P],
     "gather_batch": [C.POINTER(ReplayBuffer), P, P, I, I, I, P, P, P, P, P, P, P],
     "pendulum_step": [C.POINTER(PendulumParameters), P, P, P, P, P, I],
+    "acrobot_step": [C.POINTER(AcrobotParameters), I, P, P, P, P, P, P, I],
     "pendulum_evaluate": [C.POINTER(PendulumParameters), I, LP, I, P, I, I, P, P, P],
     "ppo_gae": [P, P, P, P, P, P, I, I, I, F, F, I],
     "gru_forward": [C.POINTER(GruLayer), P, P, I, I, P, S],

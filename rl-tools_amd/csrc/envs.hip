@@ -1,0 +1,72 @@
+// Analytic environments other than the Pendulum as batched kernels, one lane per environment.
+// Acrobot / AcrobotSwingup: rl/environments/acrobot/operations_generic.h:56-117 (dsdt, rk4), :118-144 (step), :145-171 (reward),
+// :173-193 (observe, terminated). The reference evaluates parts of dsdt in double (double literals and the double cos / sin); the kernel computes in
+// fp32 throughout, which stays within 1e-5 relative of it per step. 4 Runge-Kutta stages of ~60 flop: the kernel is bound by its 52 bytes per
+// environment (state in and out, observations, reward, flag) once there are enough environments to fill the device.
+#include "common.h"
+
+namespace {
+struct Acrobot4 { float v[4]; };
+__device__ __forceinline__ float clampf(float x, float lo, float hi) { return fminf(fmaxf(x, lo), hi); }
+__device__ __forceinline__ float angle_normalize(float x) {
+    const float PI = 3.14159265358979323846f;
+    const float a = x + PI, b = 2.0f * PI;
+    return (a - b * floorf(a / b)) - PI;
+}
+__device__ __forceinline__ Acrobot4 acrobot_dsdt(const rlt_acrobot_parameters& P, const Acrobot4& s, float action) {
+    const float m1 = P.link_mass_1, m2 = P.link_mass_2, l1 = P.link_length_1, lc1 = P.link_com_pos_1, lc2 = P.link_com_pos_2, I1 = P.link_moi, I2 = P.link_moi;
+    const float g = 9.8f, HALF_PI = 1.57079632679489661923f;
+    const float theta1 = s.v[0], theta2 = s.v[1], dtheta1 = s.v[2], dtheta2 = s.v[3];
+    float s2, c2;
+    sincosf(theta2, &s2, &c2);
+    const float d1 = m1 * lc1 * lc1 + m2 * (l1 * l1 + lc2 * lc2 + 2.0f * l1 * lc2 * c2) + I1 + I2;
+    const float d2 = m2 * (lc2 * lc2 + l1 * lc2 * c2) + I2;
+    const float phi2 = m2 * lc2 * g * cosf(theta1 + theta2 - HALF_PI);
+    const float phi1 = -m2 * l1 * lc2 * dtheta2 * dtheta2 * s2 - 2.0f * m2 * l1 * lc2 * dtheta2 * dtheta1 * s2 + (m1 * lc1 + m2 * l1) * g * cosf(theta1 - HALF_PI) + phi2;
+    const float ddtheta2 = (action + d2 / d1 * phi1 - m2 * l1 * lc2 * dtheta1 * dtheta1 * s2 - phi2) / (m2 * lc2 * lc2 + I2 - d2 * d2 / d1);
+    const float ddtheta1 = -(d2 * ddtheta2 + phi1) / d1;
+    return {{dtheta1, dtheta2, ddtheta1, ddtheta2}};
+}
+__device__ __forceinline__ Acrobot4 axpy(const Acrobot4& s, float a, const Acrobot4& k) { return {{s.v[0] + a * k.v[0], s.v[1] + a * k.v[1], s.v[2] + a * k.v[2], s.v[3] + a * k.v[3]}}; }
+__device__ __forceinline__ void acrobot_observe(const Acrobot4& s, float* __restrict__ o) {
+    float sn, cs;
+    sincosf(s.v[0], &sn, &cs); o[0] = cs; o[1] = sn;
+    sincosf(s.v[1], &sn, &cs); o[2] = cs; o[3] = sn;
+    o[4] = s.v[2]; o[5] = s.v[3];
+}
+
+__global__ __launch_bounds__(256) void acrobot_step_kernel(rlt_acrobot_parameters P, int swingup, float* __restrict__ states, const float* __restrict__ actions,
+                                                           float* __restrict__ observations, float* __restrict__ next_observations, float* __restrict__ rewards,
+                                                           uint8_t* __restrict__ terminated, int n) {
+    const float PI = 3.14159265358979323846f;
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
+        const float4 raw = reinterpret_cast<const float4*>(states)[e];
+        const Acrobot4 s = {{raw.x, raw.y, raw.z, raw.w}};
+        if (observations) acrobot_observe(s, observations + 6 * (size_t)e);
+        const float action = (clampf(actions[e], -1.0f, 1.0f) + 1.0f) / 2.0f * (P.max_torque - P.min_torque) + P.min_torque;
+        // classic Runge-Kutta over one time step (:98-117)
+        const Acrobot4 k1 = acrobot_dsdt(P, s, action);
+        const Acrobot4 k2 = acrobot_dsdt(P, axpy(s, P.dt / 2.0f, k1), action);
+        const Acrobot4 k3 = acrobot_dsdt(P, axpy(s, P.dt / 2.0f, k2), action);
+        const Acrobot4 k4 = acrobot_dsdt(P, axpy(s, P.dt, k3), action);
+        Acrobot4 next;
+#pragma unroll
+        for (int i = 0; i < 4; i++) next.v[i] = s.v[i] + P.dt / 6.0f * (k1.v[i] + 2.0f * k2.v[i] + 2.0f * k3.v[i] + k4.v[i]);
+        next.v[0] = angle_normalize(next.v[0]); next.v[1] = angle_normalize(next.v[1]);
+        next.v[2] = clampf(next.v[2], -P.max_vel_1, P.max_vel_1); next.v[3] = clampf(next.v[3], -P.max_vel_2, P.max_vel_2);
+        if (rewards) rewards[e] = swingup ? (-fabsf(angle_normalize(next.v[0] - PI)) - fabsf(angle_normalize(next.v[1]))) / 100.0f * P.dt / 0.02f : -1.0f;
+        if (terminated) terminated[e] = swingup ? 0 : ((-cosf(next.v[0]) - cosf(next.v[1] + next.v[0])) > 1.0f);
+        if (next_observations) acrobot_observe(next, next_observations + 6 * (size_t)e);
+        reinterpret_cast<float4*>(states)[e] = make_float4(next.v[0], next.v[1], next.v[2], next.v[3]);
+    }
+}
+}  // namespace
+
+extern "C" int rlt_rocm_acrobot_step(rlt_rocm_device* device, const rlt_acrobot_parameters* p, int swingup, float* states, const float* actions, float* observations,
+                                     float* next_observations, float* rewards, uint8_t* terminated, int n_envs) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(p && states && actions && n_envs > 0 && ((uintptr_t)states & 15) == 0);
+    int blocks = (n_envs + 255) / 256; if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(acrobot_step_kernel, dim3(blocks), dim3(256), 0, device->stream, *p, swingup, states, actions, observations, next_observations, rewards, terminated, n_envs);
+    return rlt_launch_status(device);
+}

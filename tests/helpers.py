@@ -790,3 +790,18 @@ def evaluate_on_backend(backend, dims, params, hidden_act, out_act, policy_kind,
     backend.call("pendulum_evaluate", C.byref(env), policy_kind, actor.layers, actor.n, ini.ptr, n, step_limit, ret.ptr, length.ptr, summary.ptr)
     backend.sync()
     return ret.numpy(), length.numpy(), summary.numpy()
+
+
+REF_ENVS_GENERIC = os.path.join(ORACLE_DIR, "_ref", "librlt_ref_envs_generic.so")
+
+
+def acrobot_on_backend(backend, kind, states, actions, params=None):
+    """One step of n Acrobot environments on a backend (kind 0: Acrobot, 1: AcrobotSwingup, 2: AcrobotSwingup with EasyParameters):
+    returns (next_states, observations, next_observations, rewards, terminated)."""
+    n = states.shape[0]
+    p = params if params is not None else capi.acrobot_parameters(easy=kind == 2)
+    s, a = backend.array(states.astype(np.float32)), backend.array(actions.astype(np.float32))
+    o, no, r, t = backend.zeros((n, 6)), backend.zeros((n, 6)), backend.zeros((n,)), backend.zeros((n,), np.uint8)
+    backend.call("acrobot_step", C.byref(p), int(kind > 0), s.ptr, a.ptr, o.ptr, no.ptr, r.ptr, t.ptr, n)
+    backend.sync()
+    return s.numpy(), o.numpy(), no.numpy(), r.numpy(), t.numpy()

@@ -266,3 +266,49 @@ def test_evaluation_reproduces_reference_vectors(oracle):
     # shorter horizon: the return is a prefix sum of the same rewards, so it is larger (rewards are negative) and the lengths follow the limit
     ret50, length50, _ = helpers.evaluate_on_backend(oracle, [3, 64, 64, 2], g["e2_actor"], "relu", "identity", 2, g["e2_initial_states"], 50)
     assert np.all(length50 == 50) and np.all(ret50 > g["e2_returns"]) and np.all(ret50 < 0)
+
+
+def test_acrobot_reproduces_reference_vectors_and_conserves_energy(oracle):
+    """Acrobot / AcrobotSwingup / EasyParameters steps against the reference's own outputs (tests/golden/make_acrobot_golden.py), bit for bit, random
+    states and 200-step trajectories. Then what the mechanics fix: without torque the equations of motion conserve
+    E = 1/2 dq^T M(q) dq - (m1 lc1 + m2 l1) g cos(q1) - m2 lc2 g cos(q1 + q2) with M = [[d1, d2], [d2, m2 lc2^2 + I2]], so E drifts only by the
+    integration error, and that error falls about 16-fold (32-fold per unit time) when the classic Runge-Kutta step is halved."""
+    g = np.load(os.path.join(helpers.GOLDEN, "acrobot_steps.npz"))
+    for kind in range(3):
+        got = helpers.acrobot_on_backend(oracle, kind, g["states"], g["actions"])
+        for name, v in zip(("next_states", "observations", "next_observations", "rewards", "terminated"), got):
+            assert np.array_equal(v, g[f"k{kind}_{name}"]), (kind, name)
+        s = g[f"k{kind}_trajectory"][:1].copy()
+        for k in range(200):
+            s, _, _, r, t = helpers.acrobot_on_backend(oracle, kind, s, g["trajectory_actions"][k:k + 1])
+            assert np.array_equal(s[0], g[f"k{kind}_trajectory"][k + 1]) and r[0] == g[f"k{kind}_trajectory_rewards"][k] and t[0] == g[f"k{kind}_trajectory_terminated"][k], (kind, k)
+
+    def energy(s):
+        q1, q2, w1, w2 = (s[:, i].astype(np.float64) for i in range(4))
+        m1 = m2 = l1 = 1.0; lc1 = lc2 = 0.5; I1 = I2 = 1.0; grav = float(np.float32(9.8))
+        d1 = m1 * lc1 ** 2 + m2 * (l1 ** 2 + lc2 ** 2 + 2 * l1 * lc2 * np.cos(q2)) + I1 + I2
+        d2 = m2 * (lc2 ** 2 + l1 * lc2 * np.cos(q2)) + I2
+        kinetic = 0.5 * (d1 * w1 ** 2 + 2 * d2 * w1 * w2 + (m2 * lc2 ** 2 + I2) * w2 ** 2)
+        return kinetic - (m1 * lc1 + m2 * l1) * grav * np.cos(q1) - m2 * lc2 * grav * np.cos(q1 + q2)
+    rng = np.random.default_rng(0)
+    start = np.stack([rng.uniform(-1.5, 1.5, 32), rng.uniform(-1.5, 1.5, 32), rng.uniform(-1, 1, 32), rng.uniform(-1, 1, 32)], 1).astype(np.float32)
+    zero = np.zeros(32, np.float32)         # action 0 is torque 0 for the symmetric torque range
+    drift = {}
+    for dt, steps in ((0.1, 10), (0.05, 20)):       # one second of motion either way
+        p = helpers.capi.acrobot_parameters(); p.dt = dt
+        s = start.copy()
+        for _ in range(steps):
+            s = helpers.acrobot_on_backend(oracle, 0, s, zero, params=p)[0]
+        drift[dt] = np.abs(energy(s) - energy(start)).max()
+    scale = np.abs(energy(start)).max()
+    assert drift[0.1] <= 2e-4 * scale and drift[0.05] <= 1.5e-5 * scale, drift
+    assert drift[0.1] / max(drift[0.05], 1e-9) >= 6.0, drift        # fourth-order method, float32 round-off included
+    # a torque does work on the second joint: E changes by about torque * angle swept there
+    p = helpers.capi.acrobot_parameters(); p.dt = 0.01
+    s = np.zeros((1, 4), np.float32)
+    swept = 0.0
+    for _ in range(20):
+        before = s[0, 1]
+        s = helpers.acrobot_on_backend(oracle, 0, s, np.array([0.4], np.float32), params=p)[0]
+        swept += float(s[0, 1] - before)
+    assert abs((energy(s) - energy(np.zeros((1, 4), np.float32)))[0] - 2.0 * swept) <= 0.02 * abs(2.0 * swept)      # action 0.4 -> torque 2

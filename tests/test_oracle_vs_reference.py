@@ -105,6 +105,40 @@ def test_evaluation_bit_exact_with_reference(oracle):
     lib.rlt_oracle_sac_loop_destroy(loop); ref.rlt_ref_sac_destroy(h)
 
 
+@pytest.mark.skipif(not os.path.exists(helpers.REF_ENVS_GENERIC), reason="environment flavour of oracle/_ref not built")
+@pytest.mark.parametrize("kind", [0, 1, 2])
+def test_acrobot_bit_exact_with_reference(oracle, kind):
+    """Acrobot (0), AcrobotSwingup (1) and AcrobotSwingup with EasyParameters (2): observe, step (Runge-Kutta over dsdt, angle wrap, velocity clamp),
+    reward and terminated of the reference on 20,000 random states, and a 500-step closed chain where each side feeds on its own next state."""
+    ref = C.CDLL(helpers.REF_ENVS_GENERIC)
+    P = C.c_void_p
+    ref.rlt_ref_acrobot_steps.argtypes = [C.c_int, P, P, P, P, P, P, P, C.c_int]
+
+    def reference(states, actions):
+        n = states.shape[0]
+        ns, o, no, r, t = np.zeros((n, 4), np.float32), np.zeros((n, 6), np.float32), np.zeros((n, 6), np.float32), np.zeros(n, np.float32), np.zeros(n, np.uint8)
+        assert ref.rlt_ref_acrobot_steps(kind, states.ctypes.data, actions.ctypes.data, ns.ctypes.data, o.ctypes.data, no.ctypes.data, r.ctypes.data, t.ctypes.data, n) == 0
+        return ns, o, no, r, t
+    rng = np.random.default_rng(kind)
+    n = 20000
+    states = np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-np.pi, np.pi, n), rng.uniform(-13, 13, n), rng.uniform(-29, 29, n)], 1).astype(np.float32)
+    states[:10] = 0
+    actions = rng.uniform(-1.3, 1.3, n).astype(np.float32)
+    want, got = reference(states, actions), helpers.acrobot_on_backend(oracle, kind, states, actions)
+    for w, g, name in zip(want, got, ("next_states", "observations", "next_observations", "rewards", "terminated")):
+        assert np.array_equal(w, g), name
+    if kind == 0:
+        assert 0 < want[4].sum() < n and np.all(want[3] == -1)
+    else:
+        assert want[4].sum() == 0 and np.all(want[3] <= 0) and len(np.unique(want[3])) > n // 2
+    assert (np.abs(want[0][:, 2]) == np.float32(4 * np.float32(np.pi))).sum() > 0        # the velocity clamp is reached
+    sr = so = np.array([[0.05, -0.03, 0.02, 0.01]] * 4, np.float32) * np.arange(1, 5, dtype=np.float32)[:, None]
+    for k in range(500):
+        a = rng.uniform(-1, 1, 4).astype(np.float32)
+        sr, so = reference(sr, a)[0], helpers.acrobot_on_backend(oracle, kind, so, a)[0]
+        assert np.array_equal(sr, so), k
+
+
 def test_small_ring_wraps_bit_exact_with_reference(oracle):
     """Replay capacity 250 (< 900 steps): the ring wraps three times, so `add` past the end, the prologue's wrap of the
     previous row, `full`, and gather's (position + MAX_EPISODE_LENGTH + offset) % CAPACITY index all run, and every
