@@ -373,6 +373,20 @@ typedef struct rlt_acrobot_parameters {
 int rlt_rocm_acrobot_step(rlt_rocm_device* device, const rlt_acrobot_parameters* p, int swingup, float* states, const float* actions,
                           float* observations, float* next_observations, float* rewards, uint8_t* terminated, int n_envs);
 
+/* rl/environments/car/car.h:13-33 (Parameters with the front / rear tire coefficients B, C, D) */
+typedef struct rlt_car_parameters {
+    float g, m, I, lf, lr, tf_B, tf_C, tf_D, tr_B, tr_C, tr_D, cm, cr0, cr2, vt, dt;
+} rlt_car_parameters;
+
+/* step + reward + terminated + observe of the Car (the variant without a track)
+ * rl/environments/car/operations_generic.h:80-84 (terminated), :99-127 (step: single-track model with Pacejka tire forces, explicit
+ * Euler), :128-135 (reward from the pre-step state), :143-155 (observe = the state)
+ *   states [n_envs x 6] = (x, y, mu, vx, vy, omega) updated in place; actions [n_envs x 2] = (throttle / brake, steering), clamped
+ *   to [-1, 1]; observations (pre-step) and next_observations [n_envs x 6]; rewards [n_envs]; terminated [n_envs] of the NEXT
+ *   state. Any output may be NULL. */
+int rlt_rocm_car_step(rlt_rocm_device* device, const rlt_car_parameters* p, float* states, const float* actions,
+                      float* observations, float* next_observations, float* rewards, uint8_t* terminated, int n_envs);
+
 /* Per-environment runner state (rl/components/off_policy_runner/off_policy_runner.h:184-221). */
 typedef struct rlt_pendulum_runner {
     float* states;            /* [n_envs x 2]  */

@@ -1,8 +1,9 @@
 // Harness around the REAL reference's analytic environments other than the Pendulum (compiled from /root/reference/include where it lies; nothing
-// of it is copied here): batched step / reward / observe / terminated of the Acrobot and the AcrobotSwingup with their default parameters, and the
-// initial states their sample_initial_state draws. Built by oracle/Makefile into oracle/_ref/librlt_ref_envs_generic.so.
+// of it is copied here): batched step / reward / observe / terminated of the Acrobot and the AcrobotSwingup with their default parameters, and of
+// the Car (the variant without a track). Built by oracle/Makefile into oracle/_ref/librlt_ref_envs_generic.so.
 #include <rl_tools/operations/cpu_mux.h>
 #include <rl_tools/rl/environments/acrobot/operations_cpu.h>
+#include <rl_tools/rl/environments/car/operations_cpu.h>
 
 #include <cstdint>
 
@@ -42,7 +43,41 @@ void steps(const float* states, const float* actions, float* next_states, float*
 }
 }  // namespace
 
+namespace {
+using CAR_SPEC = rlt::rl::environments::car::Specification<float, TI>;
+using CAR = rlt::rl::environments::Car<CAR_SPEC>;
+}  // namespace
+
 extern "C" {
+// states [n x 6] = (x, y, mu, vx, vy, omega), actions [n x 2] = (throttle / brake, steering)
+int rlt_ref_car_steps(const float* states, const float* actions, float* next_states, float* observations, float* next_observations, float* rewards, uint8_t* terminated, int n) {
+    DEVICE device;
+    RNG rng;
+    rlt::malloc(device, rng);
+    rlt::init(device, rng, 0);
+    CAR env;
+    CAR::Parameters parameters;
+    rlt::initial_parameters(device, env, parameters);
+    rlt::Matrix<rlt::matrix::Specification<float, TI, 1, 2, false>> action;
+    rlt::Matrix<rlt::matrix::Specification<float, TI, 1, 6, false>> observation;
+    for (int e = 0; e < n; e++) {
+        CAR::State state, next;
+        const float* s = states + 6 * e;
+        state.x = s[0]; state.y = s[1]; state.mu = s[2]; state.vx = s[3]; state.vy = s[4]; state.omega = s[5];
+        rlt::set(action, 0, 0, actions[2 * e]); rlt::set(action, 0, 1, actions[2 * e + 1]);
+        rlt::observe(device, env, parameters, state, CAR::Observation{}, observation, rng);
+        for (TI i = 0; i < 6; i++) observations[6 * e + i] = rlt::get(observation, 0, i);
+        rlt::step(device, env, parameters, state, action, next, rng);
+        rewards[e] = rlt::reward(device, env, parameters, state, action, next, rng);
+        terminated[e] = rlt::terminated(device, env, parameters, next, rng);
+        rlt::observe(device, env, parameters, next, CAR::Observation{}, observation, rng);
+        for (TI i = 0; i < 6; i++) next_observations[6 * e + i] = rlt::get(observation, 0, i);
+        float* o = next_states + 6 * e;
+        o[0] = next.x; o[1] = next.y; o[2] = next.mu; o[3] = next.vx; o[4] = next.vy; o[5] = next.omega;
+    }
+    rlt::free(device, rng);
+    return 0;
+}
 // kind 0: Acrobot, 1: AcrobotSwingup, 2: AcrobotSwingup with EasyParameters (torque +-10)
 int rlt_ref_acrobot_steps(int kind, const float* states, const float* actions, float* next_states, float* observations, float* next_observations, float* rewards,
                           uint8_t* terminated, int n) {

@@ -732,6 +732,43 @@ int rlt_oracle_acrobot_step(const rlt_acrobot_parameters* P, int swingup, float*
     return 0;
 }
 
+// rl/environments/car/operations_generic.h:80-84 (terminated), :99-127 (step), :128-135 (reward), :143-155 (observe). T = float; the tire
+// force goes through an unqualified atan (the double function) and the reward through the double literal 0.1, kept as the C++ expression has them.
+int rlt_oracle_car_step(const rlt_car_parameters* P, float* states, const float* actions, float* observations, float* next_observations, float* rewards,
+                        uint8_t* terminated, int n_envs) {
+    if (!P || !states || !actions || n_envs <= 0) return RLT_E_INVALID_ARGUMENT;
+    const rlt_car_parameters& p = *P;
+    for (int e = 0; e < n_envs; e++) {
+        float* s = states + 6 * (size_t)e;
+        const float x = s[0], y = s[1], mu = s[2], vx = s[3], vy = s[4], omega = s[5];
+        if (observations) for (int i = 0; i < 6; i++) observations[6 * (size_t)e + i] = s[i];
+        const float throttle_break = clampf(actions[2 * (size_t)e], -1.0f, 1.0f), delta = clampf(actions[2 * (size_t)e + 1], -1.0f, 1.0f);
+        const float alpha_f = std::atan2((vy + p.lf * omega), vx) - delta;
+        const float alpha_r = std::atan2((vy - p.lr * omega), vx);
+        const float FnF = p.lr / (p.lf + p.lr) * p.m * p.g;
+        const float FnR = p.lf / (p.lf + p.lr) * p.m * p.g;
+        const float FyF = vx > p.vt || vy > p.vt ? FnF * p.tf_D * std::sin(p.tf_C * std::atan((double)(p.tf_B * (-alpha_f)))) : 0;
+        const float FyR = vx > p.vt || vy > p.vt ? FnR * p.tr_D * std::sin(p.tr_C * std::atan((double)(p.tr_B * (-alpha_r)))) : 0;
+        const float Fx = p.cm * throttle_break - p.cr0 - p.cr2 * vx * vx;
+        float n[6] = {x, y, mu, vx, vy, omega};
+        n[0] += p.dt * (std::cos(mu) * vx - std::sin(mu) * vy);
+        n[1] += p.dt * (std::sin(mu) * vx + std::cos(mu) * vy);
+        n[2] += p.dt * (omega);
+        n[3] += p.dt * (1 / p.m * (Fx - FyF * std::sin(delta)) + omega * vy);
+        n[4] += p.dt * (1 / p.m * (FyF * std::cos(delta) + FyR) - omega * vx);
+        n[5] += p.dt * (1 / p.I * (FyF * p.lf * std::cos(delta) - FyR * p.lr));
+        if (rewards) {
+            const float angle_norm = angle_normalize(mu);
+            const float cost = 0.1 * angle_norm * angle_norm + x * x + y * y;
+            rewards[e] = std::exp(-5 * cost);
+        }
+        if (terminated) terminated[e] = n[0] > 1.0 || n[0] < -1.0 || n[1] > 1.0 || n[1] < -1.0;
+        if (next_observations) for (int i = 0; i < 6; i++) next_observations[6 * (size_t)e + i] = n[i];
+        for (int i = 0; i < 6; i++) s[i] = n[i];
+    }
+    return 0;
+}
+
 int rlt_oracle_pendulum_step(const rlt_pendulum_parameters* p, float* states, const float* actions, float* observations,
                              float* next_observations, float* rewards, int n_envs) {
     if (!p || !states || !actions || n_envs <= 0) return RLT_E_INVALID_ARGUMENT;

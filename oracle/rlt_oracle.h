@@ -24,6 +24,8 @@
  *   acrobot step (dsdt, Runge-Kutta, reward, terminated, observe): bit for bit against the reference's Acrobot, AcrobotSwingup and EasyParameters
  *   environments (oracle/_ref/librlt_ref_envs_generic.so) on random states and closed chains, golden vectors, and energy conservation /
  *   integration order / work-energy checks that do not involve the reference.
+ *   car step (single-track model, reward, terminated; no track): bit for bit against the reference's Car (oracle/_ref/librlt_ref_envs_generic.so),
+ *   golden vectors, and closed forms (straight rolling, pose equivariance, no tire force below the speed threshold).
  *   ppo train_epoch: the loop over ppo train_minibatch (pinned above) that the reference's train() runs per epoch.
  */
 #ifndef RLT_ORACLE_H
@@ -108,6 +110,9 @@ int rlt_oracle_ppo_gae(const float* rewards, const float* terminated, const floa
 /* rl/environments/acrobot/operations_generic.h:56-193 */
 int rlt_oracle_acrobot_step(const rlt_acrobot_parameters* p, int swingup, float* states, const float* actions, float* observations, float* next_observations,
                             float* rewards, uint8_t* terminated, int n_envs);
+/* rl/environments/car/operations_generic.h:80-155 (the Car without a track) */
+int rlt_oracle_car_step(const rlt_car_parameters* p, float* states, const float* actions, float* observations, float* next_observations, float* rewards,
+                        uint8_t* terminated, int n_envs);
 /* rl::utils::evaluation::evaluate with the Pendulum environment (rl/utils/evaluation/operations_generic.h:106-233) */
 int rlt_oracle_pendulum_evaluate(const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers, const float* initial_states,
                                  int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary);

@@ -88,6 +88,15 @@ def acrobot_parameters(easy=False):
     return AcrobotParameters(0.2, 1.0, 1.0, 1.0, 1.0, 0.5, 0.5, 1.0, 4 * pi, 9 * pi, -t, t)
 
 
+class CarParameters(C.Structure):
+    _fields_ = [(name, C.c_float) for name in ("g", "m", "I", "lf", "lr", "tf_B", "tf_C", "tf_D", "tr_B", "tr_C", "tr_D", "cm", "cr0", "cr2", "vt", "dt")]
+
+
+def car_parameters():
+    """rl/environments/car/car.h:19-33"""
+    return CarParameters(9.81, 0.041, 27.8e-6, 0.029, 0.033, 2.5790, 1.2000, 0.1920, 3.3852, 1.2691, 0.1737, 0.287, 0.0, 0.00035, 0.01, 0.01)
+
+
 class PendulumRunner(C.Structure):
     _fields_ = [("states", C.c_void_p), ("episode_step", C.c_void_p), ("episode_return", C.c_void_p), ("truncated", C.c_void_p),
                 ("n_envs", C.c_int32), ("episode_step_limit", C.c_int32), ("env", PendulumParameters)]
@@ -188,6 +197,7 @@ PROTOTYPES = {
     "gather_batch": [C.POINTER(ReplayBuffer), P, P, I, I, I, P, P, P, P, P, P, P],
     "pendulum_step": [C.POINTER(PendulumParameters), P, P, P, P, P, I],
     "acrobot_step": [C.POINTER(AcrobotParameters), I, P, P, P, P, P, P, I],
+    "car_step": [C.POINTER(CarParameters), P, P, P, P, P, P, I],
     "pendulum_evaluate": [C.POINTER(PendulumParameters), I, LP, I, P, I, I, P, P, P],
     "ppo_gae": [P, P, P, P, P, P, I, I, I, F, F, I],
     "gru_forward": [C.POINTER(GruLayer), P, P, I, I, P, S],

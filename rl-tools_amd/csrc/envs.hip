@@ -1,4 +1,4 @@
-// Analytic environments other than the Pendulum as batched kernels, one lane per environment.
+// Analytic environments other than the Pendulum as batched kernels, one lane per environment: the Acrobot and the Car.
 // Acrobot / AcrobotSwingup: rl/environments/acrobot/operations_generic.h:56-117 (dsdt, rk4), :118-144 (step), :145-171 (reward),
 // :173-193 (observe, terminated). The reference evaluates parts of dsdt in double (double literals and the double cos / sin); the kernel computes in
 // fp32 throughout, which stays within 1e-5 relative of it per step. 4 Runge-Kutta stages of ~60 flop: the kernel is bound by its 52 bytes per
@@ -60,7 +60,51 @@ __global__ __launch_bounds__(256) void acrobot_step_kernel(rlt_acrobot_parameter
         reinterpret_cast<float4*>(states)[e] = make_float4(next.v[0], next.v[1], next.v[2], next.v[3]);
     }
 }
+
+// Car without a track: single-track model with Pacejka tire forces, explicit Euler over dt (rl/environments/car/operations_generic.h:99-127); the
+// reward comes from the pre-step state (:128-135), terminated from the next one (:80-84), the observation is the state (:143-155).
+__global__ __launch_bounds__(256) void car_step_kernel(rlt_car_parameters p, float* __restrict__ states, const float* __restrict__ actions, float* __restrict__ observations,
+                                                       float* __restrict__ next_observations, float* __restrict__ rewards, uint8_t* __restrict__ terminated, int n) {
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
+        float2* sp = reinterpret_cast<float2*>(states) + 3 * (size_t)e;
+        const float2 s0 = sp[0], s1 = sp[1], s2 = sp[2];
+        const float x = s0.x, y = s0.y, mu = s1.x, vx = s1.y, vy = s2.x, omega = s2.y;
+        if (observations) { float2* o = reinterpret_cast<float2*>(observations) + 3 * (size_t)e; o[0] = s0; o[1] = s1; o[2] = s2; }
+        const float2 a = reinterpret_cast<const float2*>(actions)[e];
+        const float throttle_break = clampf(a.x, -1.0f, 1.0f), delta = clampf(a.y, -1.0f, 1.0f);
+        const float alpha_f = atan2f(vy + p.lf * omega, vx) - delta;
+        const float alpha_r = atan2f(vy - p.lr * omega, vx);
+        const float FnF = p.lr / (p.lf + p.lr) * p.m * p.g, FnR = p.lf / (p.lf + p.lr) * p.m * p.g;
+        const bool moving = vx > p.vt || vy > p.vt;
+        const float FyF = moving ? FnF * p.tf_D * sinf(p.tf_C * atanf(p.tf_B * (-alpha_f))) : 0.0f;
+        const float FyR = moving ? FnR * p.tr_D * sinf(p.tr_C * atanf(p.tr_B * (-alpha_r))) : 0.0f;
+        const float Fx = p.cm * throttle_break - p.cr0 - p.cr2 * vx * vx;
+        float sm, cm_, sd, cd;
+        sincosf(mu, &sm, &cm_);
+        sincosf(delta, &sd, &cd);
+        const float nx = x + p.dt * (cm_ * vx - sm * vy);
+        const float ny = y + p.dt * (sm * vx + cm_ * vy);
+        const float nmu = mu + p.dt * omega;
+        const float nvx = vx + p.dt * (1.0f / p.m * (Fx - FyF * sd) + omega * vy);
+        const float nvy = vy + p.dt * (1.0f / p.m * (FyF * cd + FyR) - omega * vx);
+        const float nomega = omega + p.dt * (1.0f / p.I * (FyF * p.lf * cd - FyR * p.lr));
+        if (rewards) { const float an = angle_normalize(mu); rewards[e] = expf(-5.0f * (0.1f * an * an + x * x + y * y)); }
+        if (terminated) terminated[e] = nx > 1.0f || nx < -1.0f || ny > 1.0f || ny < -1.0f;
+        if (next_observations) { float2* o = reinterpret_cast<float2*>(next_observations) + 3 * (size_t)e; o[0] = make_float2(nx, ny); o[1] = make_float2(nmu, nvx); o[2] = make_float2(nvy, nomega); }
+        sp[0] = make_float2(nx, ny); sp[1] = make_float2(nmu, nvx); sp[2] = make_float2(nvy, nomega);
+    }
+}
 }  // namespace
+
+extern "C" int rlt_rocm_car_step(rlt_rocm_device* device, const rlt_car_parameters* p, float* states, const float* actions, float* observations, float* next_observations,
+                                 float* rewards, uint8_t* terminated, int n_envs) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(p && states && actions && n_envs > 0);
+    RLT_REQUIRE((((uintptr_t)states | (uintptr_t)actions | (uintptr_t)observations | (uintptr_t)next_observations) & 7) == 0);      // rows move as 8-byte pairs
+    int blocks = (n_envs + 255) / 256; if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(car_step_kernel, dim3(blocks), dim3(256), 0, device->stream, *p, states, actions, observations, next_observations, rewards, terminated, n_envs);
+    return rlt_launch_status(device);
+}
 
 extern "C" int rlt_rocm_acrobot_step(rlt_rocm_device* device, const rlt_acrobot_parameters* p, int swingup, float* states, const float* actions, float* observations,
                                      float* next_observations, float* rewards, uint8_t* terminated, int n_envs) {

@@ -56,26 +56,26 @@ constexpr size_t lds_floats(int nt1c) {
 }
 
 // lane l: the row of the input arrays that row (l & 15) of a tile reads; rows beyond the batch are clamped here and masked later
-__device__ __forceinline__ int tile_rows(const SmallArgs& A, int tile, int lane) {
+__device__ __forceinline__ uint32_t tile_rows(const SmallArgs& A, int tile, int lane) {
     const int b = min(tile * 16 + (lane & 15), A.batch - 1);
-    return A.rows ? (int)A.rows[b] : b;
+    return A.rows ? A.rows[b] : (uint32_t)b;
 }
 // global loads of one tile of 16 rows, issued together: the inputs (lane = column, up to two columns per lane) and what the loss needs of the
 // rows this lane will hold after the forward pass (rows 4 kk + v, column r); columns beyond the extent are clamped here and masked later.
 // `vrows` comes from tile_rows(), requested a round earlier so that nothing waits for it here.
 struct TileRegs { float xa[16], xb[16], in0[4], in1[4], in2[4]; };
-__device__ __forceinline__ void request_tile(const SmallArgs& A, int vrows, int lane, TileRegs& T) {
+__device__ __forceinline__ void request_tile(const SmallArgs& A, uint32_t vrows, int lane, TileRegs& T) {
     const int r = lane & 15, kk = lane >> 4;
     const int c0 = min(lane, A.in - 1), c1 = min(64 + lane, A.in - 1), c = min(r, A.out - 1);
 #pragma unroll
     for (int row = 0; row < 16; row++) {
-        const float* src = A.x + (size_t)__builtin_amdgcn_readlane(vrows, row) * A.ldx;      // wavefront-uniform: scalar address arithmetic
+        const float* src = A.x + (size_t)(uint32_t)__builtin_amdgcn_readlane((int)vrows, row) * A.ldx;      // wavefront-uniform: scalar address arithmetic
         T.xa[row] = src[c0];
         T.xb[row] = A.in > 64 ? src[c1] : 0.f;
     }
 #pragma unroll
     for (int v = 0; v < 4; v++) {
-        const size_t row = (size_t)__shfl(vrows, 4 * kk + v, 64);
+        const size_t row = (size_t)(uint32_t)__shfl((int)vrows, 4 * kk + v, 64);
         T.in0[v] = T.in1[v] = T.in2[v] = 0.f;
         if (A.loss == LOSS_GIVEN) T.in0[v] = A.d_output[row * A.ldd + c];
         else if (A.loss == LOSS_MSE) T.in0[v] = A.target[row * A.ldt + c];
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
     const int n_tiles = (A.batch + 15) >> 4, n_rounds = (n_tiles + WAVES - 1) / WAVES;
     // row indices of this wavefront's first two tiles, then the first tile's loads, ahead of the weights'; a wavefront whose tile lies beyond the
     // batch computes on clamped rows and masks them
-    int rows_next = tile_rows(A, min(block * WAVES + wave, n_tiles - 1), lane), rows_after = tile_rows(A, min((block + n_blocks) * WAVES + wave, n_tiles - 1), lane);
+    uint32_t rows_next = tile_rows(A, min(block * WAVES + wave, n_tiles - 1), lane), rows_after = tile_rows(A, min((block + n_blocks) * WAVES + wave, n_tiles - 1), lane);
     TileRegs T;
     request_tile(A, rows_next, lane, T);
     float b1r[4], b2r[4];

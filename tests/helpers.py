@@ -805,3 +805,14 @@ def acrobot_on_backend(backend, kind, states, actions, params=None):
     backend.call("acrobot_step", C.byref(p), int(kind > 0), s.ptr, a.ptr, o.ptr, no.ptr, r.ptr, t.ptr, n)
     backend.sync()
     return s.numpy(), o.numpy(), no.numpy(), r.numpy(), t.numpy()
+
+
+def car_on_backend(backend, states, actions, params=None):
+    """One step of n Car environments on a backend: returns (next_states, observations, next_observations, rewards, terminated)."""
+    n = states.shape[0]
+    p = params if params is not None else capi.car_parameters()
+    s, a = backend.array(states.astype(np.float32)), backend.array(actions.astype(np.float32))
+    o, no, r, t = backend.zeros((n, 6)), backend.zeros((n, 6)), backend.zeros((n,)), backend.zeros((n,), np.uint8)
+    backend.call("car_step", C.byref(p), s.ptr, a.ptr, o.ptr, no.ptr, r.ptr, t.ptr, n)
+    backend.sync()
+    return s.numpy(), o.numpy(), no.numpy(), r.numpy(), t.numpy()

@@ -312,3 +312,48 @@ def test_acrobot_reproduces_reference_vectors_and_conserves_energy(oracle):
         s = helpers.acrobot_on_backend(oracle, 0, s, np.array([0.4], np.float32), params=p)[0]
         swept += float(s[0, 1] - before)
     assert abs((energy(s) - energy(np.zeros((1, 4), np.float32)))[0] - 2.0 * swept) <= 0.02 * abs(2.0 * swept)      # action 0.4 -> torque 2
+
+
+def test_car_reproduces_reference_vectors_and_kinematics(oracle):
+    """Car steps against the reference's own outputs (tests/golden/make_car_golden.py), bit for bit, random states and a 300-step trajectory. Then what
+    the model fixes by itself: (1) a car rolling straight (no lateral speed, no yaw rate, no steering) has no slip angles, hence no lateral forces: it
+    keeps its heading and obeys x' = x + dt cos(mu) vx, vx' = vx + dt (cm u - cr0 - cr2 vx^2) / m; (2) the dynamics do not depend on where the car is or
+    which way it points: shifting and rotating the pose shifts and rotates the next pose and leaves the body-frame velocities alone; (3) below the
+    speed threshold the tires transmit no lateral force, so yaw rate and lateral speed change only by the omega x v terms."""
+    g = np.load(os.path.join(helpers.GOLDEN, "car_steps.npz"))
+    got = helpers.car_on_backend(oracle, g["states"], g["actions"])
+    for name, v in zip(("next_states", "observations", "next_observations", "rewards", "terminated"), got):
+        assert np.array_equal(v, g[name]), name
+    s = g["trajectory"][:1].copy()
+    for k in range(300):
+        s, _, _, r, t = helpers.car_on_backend(oracle, s, g["trajectory_actions"][k:k + 1])
+        assert np.array_equal(s[0], g["trajectory"][k + 1]) and r[0] == g["trajectory_rewards"][k] and t[0] == g["trajectory_terminated"][k], k
+    p = helpers.capi.car_parameters()
+    rng = np.random.default_rng(0)
+    n = 64
+    # (1) straight rolling
+    mu, vx, u = rng.uniform(-3, 3, n), rng.uniform(0.1, 2.5, n), rng.uniform(-1, 1, n)
+    st = np.stack([rng.uniform(-0.5, 0.5, n), rng.uniform(-0.5, 0.5, n), mu, vx, np.zeros(n), np.zeros(n)], 1).astype(np.float32)
+    nx = helpers.car_on_backend(oracle, st, np.stack([u, np.zeros(n)], 1))[0].astype(np.float64)
+    s64 = st.astype(np.float64); u32 = u.astype(np.float32).astype(np.float64)
+    assert np.abs(nx[:, 0] - (s64[:, 0] + p.dt * np.cos(s64[:, 2]) * s64[:, 3])).max() <= 1e-6
+    assert np.abs(nx[:, 1] - (s64[:, 1] + p.dt * np.sin(s64[:, 2]) * s64[:, 3])).max() <= 1e-6
+    assert np.abs(nx[:, 3] - (s64[:, 3] + p.dt * (p.cm * u32 - p.cr0 - p.cr2 * s64[:, 3] ** 2) / p.m)).max() <= 1e-5
+    assert np.array_equal(nx[:, 2], s64[:, 2]) and np.all(nx[:, 4] == 0) and np.all(nx[:, 5] == 0)
+    # (2) pose equivariance
+    st = np.stack([rng.uniform(-0.3, 0.3, n), rng.uniform(-0.3, 0.3, n), rng.uniform(-1, 1, n), rng.uniform(0.2, 2, n), rng.uniform(-0.5, 0.5, n), rng.uniform(-4, 4, n)], 1).astype(np.float32)
+    act = rng.uniform(-1, 1, (n, 2)).astype(np.float32)
+    base = helpers.car_on_backend(oracle, st, act)[0].astype(np.float64)
+    phi, shift = 0.7, np.array([0.2, -0.1])
+    rot = np.array([[np.cos(phi), -np.sin(phi)], [np.sin(phi), np.cos(phi)]])
+    moved = st.astype(np.float64).copy()
+    moved[:, :2] = moved[:, :2] @ rot.T + shift; moved[:, 2] += phi
+    nm = helpers.car_on_backend(oracle, moved.astype(np.float32), act)[0].astype(np.float64)
+    assert np.abs(nm[:, :2] - (base[:, :2] @ rot.T + shift)).max() <= 2e-6 and np.abs(nm[:, 2] - (base[:, 2] + phi)).max() <= 1e-6
+    assert np.abs(nm[:, 3:] - base[:, 3:]).max() <= 1e-6 * np.abs(base[:, 3:]).max()
+    # (3) below the threshold: no tire forces
+    st = np.stack([np.zeros(n), np.zeros(n), rng.uniform(-1, 1, n), rng.uniform(-0.01, 0.009, n), rng.uniform(-0.01, 0.009, n), rng.uniform(-2, 2, n)], 1).astype(np.float32)
+    nx = helpers.car_on_backend(oracle, st, np.stack([np.zeros(n), rng.uniform(-1, 1, n)], 1))[0].astype(np.float64)
+    s64 = st.astype(np.float64)
+    assert np.array_equal(nx[:, 5], s64[:, 5])
+    assert np.abs(nx[:, 4] - (s64[:, 4] - p.dt * s64[:, 5] * s64[:, 3])).max() <= 1e-8

@@ -139,6 +139,37 @@ def test_acrobot_bit_exact_with_reference(oracle, kind):
         assert np.array_equal(sr, so), k
 
 
+@pytest.mark.skipif(not os.path.exists(helpers.REF_ENVS_GENERIC), reason="environment flavour of oracle/_ref not built")
+def test_car_bit_exact_with_reference(oracle):
+    """The Car without a track: observe, step (tire forces on and off around the speed threshold, steering and throttle clamps), reward and terminated of
+    the reference on 50,000 random states, and a 500-step closed chain."""
+    ref = C.CDLL(helpers.REF_ENVS_GENERIC)
+    P = C.c_void_p
+    ref.rlt_ref_car_steps.argtypes = [P, P, P, P, P, P, P, C.c_int]
+
+    def reference(states, actions):
+        n = states.shape[0]
+        ns, o, no, r, t = np.zeros((n, 6), np.float32), np.zeros((n, 6), np.float32), np.zeros((n, 6), np.float32), np.zeros(n, np.float32), np.zeros(n, np.uint8)
+        assert ref.rlt_ref_car_steps(states.ctypes.data, actions.ctypes.data, ns.ctypes.data, o.ctypes.data, no.ctypes.data, r.ctypes.data, t.ctypes.data, n) == 0
+        return ns, o, no, r, t
+    rng = np.random.default_rng(2)
+    n = 50000
+    states = np.stack([rng.uniform(-1.2, 1.2, n), rng.uniform(-1.2, 1.2, n), rng.uniform(-4, 4, n), rng.uniform(-0.5, 3, n), rng.uniform(-1, 1, n), rng.uniform(-8, 8, n)], 1).astype(np.float32)
+    states[:100, 3:] = 0
+    states[100:1000, 3] = rng.uniform(0.005, 0.015, 900); states[100:1000, 4] = rng.uniform(0.005, 0.015, 900)
+    actions = rng.uniform(-1.3, 1.3, (n, 2)).astype(np.float32)
+    want, got = reference(states, actions), helpers.car_on_backend(oracle, states, actions)
+    for w, g, name in zip(want, got, ("next_states", "observations", "next_observations", "rewards", "terminated")):
+        assert np.array_equal(w, g), name
+    assert 0 < want[4].sum() < n and np.all(want[3] > 0) and np.all(want[3] <= 1)
+    sr = so = np.zeros((4, 6), np.float32)
+    for k in range(500):
+        a = np.stack([rng.uniform(0, 1, 4), rng.uniform(-0.3, 0.3, 4)], 1).astype(np.float32)
+        sr, so = reference(sr, a)[0], helpers.car_on_backend(oracle, so, a)[0]
+        assert np.array_equal(sr, so), k
+    assert np.abs(sr[:, 3]).max() > 0.5          # the cars got going
+
+
 def test_small_ring_wraps_bit_exact_with_reference(oracle):
     """Replay capacity 250 (< 900 steps): the ring wraps three times, so `add` past the end, the prologue's wrap of the
     previous row, `full`, and gather's (position + MAX_EPISODE_LENGTH + offset) % CAPACITY index all run, and every
