@@ -342,6 +342,41 @@ int rlt_rocm_gather_batch(rlt_rocm_device* device, const rlt_replay_buffer* rb,
                           int max_episode_length, int batch,
                           float* observations_actions_base, float* rewards, uint8_t* terminated,
                           uint8_t* reset, uint8_t* next_reset_base, uint8_t* final_step_mask, uint8_t* next_final_step_mask_base);
+/* SequentialBatch for any SEQUENCE_LENGTH (off_policy_runner.h:102-156); padded = sequence_length + 1. */
+typedef struct rlt_sequence_batch {
+    float* observations_actions_base;    /* [padded x batch x (obs + act)] */
+    float* rewards;                      /* [sequence_length x batch] */
+    uint8_t* terminated;                 /* [sequence_length x batch] */
+    uint8_t* reset;                      /* [sequence_length x batch] */
+    uint8_t* next_reset_base;            /* [padded x batch] */
+    uint8_t* final_step_mask;            /* [sequence_length x batch] */
+    uint8_t* next_final_step_mask_base;  /* [padded x batch] */
+    int32_t batch, sequence_length;
+} rlt_sequence_batch;
+/* SequentialBatchParameters (off_policy_runner.h:79-87; the defaults switch the first two on for sequence_length > 1) */
+typedef struct rlt_sequence_sampling {
+    int32_t always_sample_from_initial_state, random_seq_length, enable_nominal_sequence_length_probability;
+    float nominal_sequence_length_probability;
+    int32_t include_first_step_in_targets;   /* 0: the `next` views start at padded step 1 (the default for sequence_length = 1), so the first
+                                                 next_reset flag lands in next_reset_base[1] (operations_generic.h:85-92,286) */
+} rlt_sequence_sampling;
+/* The random draws of gather_batch, per sample in the order the sample consumes each kind (k-th use by sample b = entry
+ * [b][k]); a sample restarts at most `padded` times and decides a sequence length at most padded + 1 times. */
+typedef struct rlt_sequence_draws {
+    const uint32_t* env_indices;      /* [batch]                  uniform_int(0, n_envs - 1), :426                       */
+    const uint32_t* sample_offsets;   /* [batch x padded]         uniform_int(0, eligible rows - 1) at every (re)start, :305 */
+    const uint8_t* nominal;           /* [batch x (padded + 1)]   1 where uniform_real(0, 1) < nominal probability, :267,362 */
+    const uint32_t* lengths;          /* [batch x (padded + 1)]   uniform_int(1, sequence_length - 1), used where nominal = 0, :272,367 */
+} rlt_sequence_draws;
+/* gather_batch / gather_batch_step for sequences, rl/components/off_policy_runner/operations_generic.h:239-430: every sample
+ * walks `padded` steps through one environment's ring from a drawn row (or from the first step of that row's episode),
+ * copies observation / action / reward / terminated, ends a sequence at an episode end, at the ring's cursor, after a drawn
+ * length or at the last step, writes the next observation and a zero action into the following step and restarts there
+ * from a new draw; reset / final-step masks mark the boundaries. Entries the reference leaves untouched are left untouched.
+ * Bit-exact (copies and index arithmetic). With sequence_length = 1 and both switches off it equals rlt_rocm_gather_batch. */
+int rlt_rocm_gather_sequence_batch(rlt_rocm_device* device, const rlt_replay_buffer* rb, const rlt_sequence_sampling* sampling,
+                                   const rlt_sequence_draws* draws, int max_episode_length, const rlt_sequence_batch* batch);
+
 /* Device-side draw of (env, offset) pairs, uniform over the eligible rows of each ring
  * (off_policy_runner/operations_generic.h:257,304,426). */
 int rlt_rocm_gather_draw(rlt_rocm_device* device, const rlt_replay_buffer* rb, int batch,

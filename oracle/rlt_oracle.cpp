@@ -652,6 +652,132 @@ int rlt_oracle_gather_batch(const rlt_replay_buffer* rb, const uint32_t* env_ind
     return 0;
 }
 
+// gather_batch_step for sequences (rl/components/off_policy_runner/operations_generic.h:239-418), one sample. DRAWS supplies the randomness:
+// offset(max) = uniform_int(0, max), nominal() = uniform_real(0, 1) < probability, length() = uniform_int(1, sequence_length - 1).
+extern "C++" {
+template <typename DRAWS>
+static int gather_sequence_sample(const rlt_replay_buffer* rb, uint32_t e, const rlt_sequence_sampling* P, int max_episode_length, const rlt_sequence_batch* B, int b, DRAWS& draws) {
+    const int OBS = rb->observation_dim, ACT = rb->action_dim, R = rb_row_dim(rb), D = OBS + ACT, N = B->batch, SEQ = B->sequence_length, PADDED = SEQ + 1;
+    const uint32_t CAP = (uint32_t)rb->capacity, position = rb->position[e];
+    const bool full = rb->full[e] != 0;
+    const uint32_t eligible = full ? (P->always_sample_from_initial_state ? CAP - (uint32_t)max_episode_length : CAP) : position;      // :259
+    if (eligible == 0) return RLT_E_INVALID_ARGUMENT;
+    const uint32_t sample_index_max = eligible - 1;
+    uint32_t sample_index = 0;
+    int current_seq_length = SEQ;
+    auto draw_length = [&]() {       // :266-275 and :362-371
+        if (P->enable_nominal_sequence_length_probability && draws.nominal()) return SEQ;
+        return SEQ > 1 ? (int)draws.length() : current_seq_length;
+    };
+    if (P->random_seq_length) current_seq_length = draw_length();
+    int current_seq_step = 0;
+    bool previous_step_truncated = false, previous_padding_step = true;
+    for (int s = 0; s < SEQ; s++) { B->final_step_mask[(size_t)s * N + b] = 0; B->reset[(size_t)s * N + b] = 0; }            // :279-287
+    for (int s = 0; s < PADDED; s++) { B->next_final_step_mask_base[(size_t)s * N + b] = 0; B->next_reset_base[(size_t)s * N + b] = 0; }
+    B->reset[b] = 1; B->next_reset_base[b] = 1;
+    B->next_reset_base[(size_t)(P->include_first_step_in_targets ? 0 : 1) * N + b] = 1;           // batch.next_reset is a view from step 0 or 1 (:85-92,286)
+    for (int s = 0; s < PADDED; s++) {
+        if (previous_step_truncated) {                                                                                       // :289-298
+            previous_step_truncated = false; previous_padding_step = true;
+            B->next_final_step_mask_base[(size_t)s * N + b] = 1;
+            if (s < PADDED - 1) B->reset[(size_t)s * N + b] = 1;
+            continue;
+        }
+        if (previous_padding_step) {                                                                                         // :299-318
+            if (s < PADDED - 1) B->reset[(size_t)s * N + b] = 1;
+            B->next_reset_base[(size_t)s * N + b] = 1;
+            const uint32_t sample_offset = draws.offset(sample_index_max);
+            sample_index = full ? (position + (uint32_t)max_episode_length + sample_offset) % CAP : sample_offset;
+            if (P->always_sample_from_initial_state) sample_index = rb->episode_start[(size_t)e * CAP + sample_index];
+        }
+        if (sample_index >= CAP) return RLT_E_INVALID_ARGUMENT;
+        const float* row = rb->data + ((size_t)e * CAP + sample_index) * R;
+        float* step = B->observations_actions_base + ((size_t)s * N + b) * D;
+        for (int k = 0; k < OBS; k++) step[k] = row[k];                                                                      // :321-326
+        for (int k = 0; k < ACT; k++) step[OBS + k] = row[OBS + k];                                                          // :336-341
+        if (s < PADDED - 1) { B->rewards[(size_t)s * N + b] = row[OBS + ACT]; B->terminated[(size_t)s * N + b] = row[2 * OBS + ACT + 1] != 0.0f; }   // :343-346
+        bool truncated = row[2 * OBS + ACT + 2] != 0.0f;                                                                     // :348
+        uint32_t next_sample_index = sample_index + 1;
+        if (full) next_sample_index %= CAP;
+        if (next_sample_index == position) truncated = true;                                                                 // :354-356
+        if (s == PADDED - 2) truncated = true;                                                                               // :357-359
+        if (P->random_seq_length) {                                                                                          // :360-383
+            if (current_seq_step == current_seq_length - 1) {
+                truncated = true;
+                current_seq_length = SEQ > 1 ? draw_length() : SEQ;
+            }
+            current_seq_step = truncated ? 0 : current_seq_step + 1;
+        }
+        if (truncated && s < PADDED - 1) {                                                                                   // :388-413
+            B->final_step_mask[(size_t)s * N + b] = 1;
+            float* next = B->observations_actions_base + ((size_t)(s + 1) * N + b) * D;
+            for (int k = 0; k < OBS; k++) next[k] = row[OBS + ACT + 1 + k];
+            for (int k = 0; k < ACT; k++) next[OBS + k] = 0;
+        }
+        sample_index = next_sample_index;
+        previous_padding_step = false;
+        previous_step_truncated = truncated;
+    }
+    return 0;
+}
+struct ArrayDraws {
+    const rlt_sequence_draws* d; int b, padded, n_offset = 0, n_length = 0;
+    uint32_t offset(uint32_t) { return d->sample_offsets[(size_t)b * padded + n_offset++]; }
+    bool nominal() { return d->nominal[(size_t)b * (padded + 1) + n_length] != 0; }        // the length decision's index advances once per decision:
+    uint32_t length() { return d->lengths[(size_t)b * (padded + 1) + n_length]; }
+};
+struct EngineDraws {
+    std::mt19937* engine; const rlt_sequence_sampling* P; int sequence_length, b, padded, n_offset = 0, n_length = 0;
+    uint32_t* offsets; uint8_t* nominals; uint32_t* lengths;
+    uint32_t offset(uint32_t max) { const uint32_t v = (uint32_t)std::uniform_int_distribution<size_t>(0, max)(*engine); offsets[(size_t)b * padded + n_offset++] = v; return v; }
+    bool nominal() { const bool v = std::uniform_real_distribution<double>(0.0, 1.0)(*engine) < P->nominal_sequence_length_probability; nominals[(size_t)b * (padded + 1) + n_length] = v; return v; }
+    uint32_t length() { const uint32_t v = (uint32_t)std::uniform_int_distribution<size_t>(1, (size_t)sequence_length - 1)(*engine); lengths[(size_t)b * (padded + 1) + n_length] = v; return v; }
+};
+}  // extern "C++"
+static bool sequence_arguments_ok(const rlt_replay_buffer* rb, const rlt_sequence_sampling* P, const rlt_sequence_batch* B) {
+    return rb && rb->data && rb->episode_start && P && B && B->batch > 0 && B->sequence_length >= 1 && B->observations_actions_base && B->rewards && B->terminated && B->reset &&
+           B->next_reset_base && B->final_step_mask && B->next_final_step_mask_base;
+}
+int rlt_oracle_gather_sequence_batch(const rlt_replay_buffer* rb, const rlt_sequence_sampling* P, const rlt_sequence_draws* draws, int max_episode_length,
+                                     const rlt_sequence_batch* B) {
+    if (!sequence_arguments_ok(rb, P, B) || !draws || !draws->env_indices || !draws->sample_offsets || (P->random_seq_length && (!draws->nominal || !draws->lengths))) return RLT_E_INVALID_ARGUMENT;
+    for (int b = 0; b < B->batch; b++) {
+        const uint32_t e = draws->env_indices[b];
+        if (e >= (uint32_t)rb->n_envs) return RLT_E_INVALID_ARGUMENT;
+        // a length decision consumes nominal[k] and, where that is 0, lengths[k]: one index for both
+        struct Fed : ArrayDraws { bool nominal() { const bool v = ArrayDraws::nominal(); if (v) n_length++; return v; } uint32_t length() { const uint32_t v = ArrayDraws::length(); n_length++; return v; } };
+        Fed fed; fed.d = draws; fed.b = b; fed.padded = B->sequence_length + 1;
+        const int rc = gather_sequence_sample(rb, e, P, max_episode_length, B, b, fed);
+        if (rc) return rc;
+    }
+    return 0;
+}
+// The same with the draws made here, in the reference's order, on the std::mt19937 given in its text form (updated on return); the draws are
+// written out in the layout rlt_sequence_draws has, so that feeding them back reproduces the batch. env_indices is drawn too (:426).
+int rlt_oracle_gather_sequence_batch_with_rng(const rlt_replay_buffer* rb, const rlt_sequence_sampling* P, int max_episode_length, const rlt_sequence_batch* B,
+                                              char* rng_state, int rng_capacity, uint32_t* env_indices, uint32_t* sample_offsets, uint8_t* nominal, uint32_t* lengths) {
+    if (!sequence_arguments_ok(rb, P, B) || !rng_state || !env_indices || !sample_offsets || !nominal || !lengths) return RLT_E_INVALID_ARGUMENT;
+    std::mt19937 engine;
+    { std::istringstream in(rng_state); in >> engine; if (in.fail()) return RLT_E_INVALID_ARGUMENT; }
+    const int padded = B->sequence_length + 1;
+    std::memset(sample_offsets, 0, sizeof(uint32_t) * (size_t)B->batch * padded);
+    std::memset(nominal, 0, (size_t)B->batch * (padded + 1)); std::memset(lengths, 0, sizeof(uint32_t) * (size_t)B->batch * (padded + 1));
+    for (int b = 0; b < B->batch; b++) {
+        const uint32_t e = (uint32_t)std::uniform_int_distribution<size_t>(0, (size_t)rb->n_envs - 1)(engine);
+        env_indices[b] = e;
+        struct Drawn : EngineDraws { bool nominal() { const bool v = EngineDraws::nominal(); if (v) n_length++; return v; } uint32_t length() { const uint32_t v = EngineDraws::length(); n_length++; return v; } };
+        Drawn drawn; drawn.engine = &engine; drawn.P = P; drawn.sequence_length = B->sequence_length; drawn.b = b; drawn.padded = padded;
+        drawn.offsets = sample_offsets; drawn.nominals = nominal; drawn.lengths = lengths;
+        const int rc = gather_sequence_sample(rb, e, P, max_episode_length, B, b, drawn);
+        if (rc) return rc;
+    }
+    std::ostringstream out; out << engine;
+    const std::string text = out.str();
+    if ((int)text.size() + 1 > rng_capacity) return RLT_E_INVALID_ARGUMENT;
+    std::memcpy(rng_state, text.c_str(), text.size() + 1);
+    return 0;
+}
+
 // rl/environments/pendulum/operations_generic.h: angle_normalize, step :79-101, reward :131-139, observe :142-160.
 // The literals 3.0, 0.1, 0.001 in the reference are doubles, so those sub-expressions evaluate in double (kept here).
 static inline float angle_normalize(float x) { // pendulum/operations_generic.h f_mod_python + angle_normalize

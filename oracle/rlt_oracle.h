@@ -26,6 +26,9 @@
  *   integration order / work-energy checks that do not involve the reference.
  *   car step (single-track model, reward, terminated; no track): bit for bit against the reference's Car (oracle/_ref/librlt_ref_envs_generic.so),
  *   golden vectors, and closed forms (straight rolling, pose equivariance, no tire force below the speed threshold).
+ *   gather for sequence batches: all seven tensors of the batch entry for entry against the reference's gather_batch on its own runner's rings
+ *   (oracle/_ref/librlt_ref_gather_seq_generic.so; sequence length 8 with and without the default sampling switches, and 1), draws made on the
+ *   reference's std::mt19937 in its order; golden vectors; structural invariants on synthetic rings.
  *   ppo train_epoch: the loop over ppo train_minibatch (pinned above) that the reference's train() runs per epoch.
  */
 #ifndef RLT_ORACLE_H
@@ -107,6 +110,12 @@ int rlt_oracle_ppo_gae(const float* rewards, const float* terminated, const floa
                        float* advantages, float* target_values, int ld, int n_envs, int steps, float gamma, float lambda,
                        int ignore_termination);
 
+/* gather_batch for sequence batches, rl/components/off_policy_runner/operations_generic.h:239-430; the second form makes the draws itself on the
+ * reference's std::mt19937 (text form in, text form out) and returns them in the layout of rlt_sequence_draws */
+int rlt_oracle_gather_sequence_batch(const rlt_replay_buffer* rb, const rlt_sequence_sampling* sampling, const rlt_sequence_draws* draws, int max_episode_length,
+                                     const rlt_sequence_batch* batch);
+int rlt_oracle_gather_sequence_batch_with_rng(const rlt_replay_buffer* rb, const rlt_sequence_sampling* sampling, int max_episode_length, const rlt_sequence_batch* batch,
+                                              char* rng_state, int rng_capacity, uint32_t* env_indices, uint32_t* sample_offsets, uint8_t* nominal, uint32_t* lengths);
 /* rl/environments/acrobot/operations_generic.h:56-193 */
 int rlt_oracle_acrobot_step(const rlt_acrobot_parameters* p, int swingup, float* states, const float* actions, float* observations, float* next_observations,
                             float* rewards, uint8_t* terminated, int n_envs);

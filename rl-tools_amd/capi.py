@@ -67,6 +67,20 @@ class ReplayBuffer(C.Structure):
                 ("full", C.c_void_p), ("n_envs", C.c_int32), ("capacity", C.c_int32), ("observation_dim", C.c_int32), ("action_dim", C.c_int32)]
 
 
+class SequenceBatch(C.Structure):
+    _fields_ = [("observations_actions_base", C.c_void_p), ("rewards", C.c_void_p), ("terminated", C.c_void_p), ("reset", C.c_void_p), ("next_reset_base", C.c_void_p),
+                ("final_step_mask", C.c_void_p), ("next_final_step_mask_base", C.c_void_p), ("batch", C.c_int32), ("sequence_length", C.c_int32)]
+
+
+class SequenceSampling(C.Structure):
+    _fields_ = [("always_sample_from_initial_state", C.c_int32), ("random_seq_length", C.c_int32), ("enable_nominal_sequence_length_probability", C.c_int32),
+                ("nominal_sequence_length_probability", C.c_float), ("include_first_step_in_targets", C.c_int32)]
+
+
+class SequenceDraws(C.Structure):
+    _fields_ = [("env_indices", C.c_void_p), ("sample_offsets", C.c_void_p), ("nominal", C.c_void_p), ("lengths", C.c_void_p)]
+
+
 class PendulumParameters(C.Structure):
     _fields_ = [("g", C.c_float), ("max_speed", C.c_float), ("max_torque", C.c_float), ("dt", C.c_float), ("m", C.c_float), ("l", C.c_float)]
 
@@ -164,6 +178,8 @@ class OnPolicyDataset(C.Structure):
 
 I, F, P, S, U64 = C.c_int, C.c_float, C.c_void_p, C.c_size_t, C.c_uint64
 LP = C.POINTER(DenseLayer)
+# return codes of the C ABI (include/rlt_rocm.h)
+RLT_E_INVALID_ARGUMENT, RLT_E_UNSUPPORTED, RLT_E_NOT_INITIALISED, RLT_E_DEVICE_TIMEOUT = -1, -2, -3, -4
 
 # name -> argument types after the leading device handle (shared by the HIP library and, minus the handle, the CPU checker)
 PROTOTYPES = {
@@ -196,6 +212,7 @@ PROTOTYPES = {
     "replay_add": [C.POINTER(ReplayBuffer), P, P, P, P, P, P],
     "gather_batch": [C.POINTER(ReplayBuffer), P, P, I, I, I, P, P, P, P, P, P, P],
     "pendulum_step": [C.POINTER(PendulumParameters), P, P, P, P, P, I],
+    "gather_sequence_batch": [C.POINTER(ReplayBuffer), C.POINTER(SequenceSampling), C.POINTER(SequenceDraws), I, C.POINTER(SequenceBatch)],
     "acrobot_step": [C.POINTER(AcrobotParameters), I, P, P, P, P, P, P, I],
     "car_step": [C.POINTER(CarParameters), P, P, P, P, P, P, I],
     "pendulum_evaluate": [C.POINTER(PendulumParameters), I, LP, I, P, I, I, P, P, P],

@@ -161,11 +161,12 @@ int rlt_rocm_check_status(rlt_rocm_device* device) {
     hipError_t e = hipStreamSynchronize(device->stream);
     if (e != hipSuccess) device->sticky_error = (int)e;
     if (device->fault_armed && e == hipSuccess) {
-        unsigned fault = 0;
+        // word 0: a persistent kernel gave up waiting; word 1: a kernel met an index on the device that points outside its arrays (and skipped that element)
+        unsigned fault[2] = {0, 0};
         device->fault_armed = 0;
-        if (hipMemcpy(&fault, device->fault, sizeof fault, hipMemcpyDeviceToHost) == hipSuccess && fault) {
+        if (hipMemcpy(fault, device->fault, sizeof fault, hipMemcpyDeviceToHost) == hipSuccess && (fault[0] || fault[1])) {
             (void)hipMemset(device->fault, 0, sizeof fault);
-            if (!device->sticky_error) device->sticky_error = RLT_E_DEVICE_TIMEOUT;
+            if (!device->sticky_error) device->sticky_error = fault[0] ? RLT_E_DEVICE_TIMEOUT : RLT_E_INVALID_ARGUMENT;
         }
     }
     int s = device->sticky_error;

@@ -94,6 +94,82 @@ __global__ __launch_bounds__(256) void gather_kernel(rlt_replay_buffer rb, const
     }
 }
 
+// gather_batch_step for sequences (rl/components/off_policy_runner/operations_generic.h:239-418): a lane per sample walks its padded steps through one
+// ring; the draws come from arrays, the k-th use of a kind by sample b being entry [b][k]. Copies and index arithmetic only.
+__global__ __launch_bounds__(256) void gather_sequence_kernel(rlt_replay_buffer rb, rlt_sequence_sampling P, rlt_sequence_draws draws, int max_episode_length, rlt_sequence_batch B,
+                                                              int* __restrict__ error_flag) {
+    const int OBS = rb.observation_dim, ACT = rb.action_dim, R = 2 * OBS + ACT + 3, D = OBS + ACT, N = B.batch, SEQ = B.sequence_length, PADDED = SEQ + 1;
+    const uint32_t CAP = (uint32_t)rb.capacity;
+    for (int b = blockIdx.x * blockDim.x + threadIdx.x; b < N; b += gridDim.x * blockDim.x) {
+        const uint32_t e = draws.env_indices[b];
+        if (e >= (uint32_t)rb.n_envs) { *error_flag = 1; continue; }
+        const uint32_t position = rb.position[e];
+        const bool full = rb.full[e] != 0;
+        const uint32_t* offsets = draws.sample_offsets + (size_t)b * PADDED;
+        const uint8_t* nominal = draws.nominal + (size_t)b * (PADDED + 1);
+        const uint32_t* lengths = draws.lengths + (size_t)b * (PADDED + 1);
+        int n_offset = 0, n_length = 0;
+        uint32_t sample_index = 0;
+        int current_seq_length = SEQ;
+        // a length decision (:266-275, :362-371): nominal[k] says whether the full length is taken, lengths[k] is used where it does not
+        auto draw_length = [&]() {
+            int length = current_seq_length;
+            if (P.enable_nominal_sequence_length_probability && nominal[n_length]) length = SEQ;
+            else if (SEQ > 1) length = (int)lengths[n_length];
+            n_length++;
+            return length;
+        };
+        if (P.random_seq_length) current_seq_length = draw_length();
+        int current_seq_step = 0;
+        bool previous_step_truncated = false, previous_padding_step = true;
+        for (int s = 0; s < SEQ; s++) { B.final_step_mask[(size_t)s * N + b] = 0; B.reset[(size_t)s * N + b] = 0; }
+        for (int s = 0; s < PADDED; s++) { B.next_final_step_mask_base[(size_t)s * N + b] = 0; B.next_reset_base[(size_t)s * N + b] = 0; }
+        B.reset[b] = 1; B.next_reset_base[b] = 1;
+        B.next_reset_base[(size_t)(P.include_first_step_in_targets ? 0 : 1) * N + b] = 1;
+        for (int s = 0; s < PADDED; s++) {
+            if (previous_step_truncated) {
+                previous_step_truncated = false; previous_padding_step = true;
+                B.next_final_step_mask_base[(size_t)s * N + b] = 1;
+                if (s < PADDED - 1) B.reset[(size_t)s * N + b] = 1;
+                continue;
+            }
+            if (previous_padding_step) {
+                if (s < PADDED - 1) B.reset[(size_t)s * N + b] = 1;
+                B.next_reset_base[(size_t)s * N + b] = 1;
+                const uint32_t sample_offset = offsets[n_offset++];
+                sample_index = full ? (position + (uint32_t)max_episode_length + sample_offset) % CAP : sample_offset;
+                if (P.always_sample_from_initial_state && sample_index < CAP) sample_index = rb.episode_start[(size_t)e * CAP + sample_index];
+            }
+            if (sample_index >= CAP) { *error_flag = 1; break; }
+            const float* row = rb.data + ((size_t)e * CAP + sample_index) * R;
+            float* step = B.observations_actions_base + ((size_t)s * N + b) * D;
+            for (int k = 0; k < D; k++) step[k] = row[k];
+            if (s < PADDED - 1) { B.rewards[(size_t)s * N + b] = row[D]; B.terminated[(size_t)s * N + b] = row[2 * OBS + ACT + 1] != 0.0f; }
+            bool truncated = row[2 * OBS + ACT + 2] != 0.0f;
+            uint32_t next_sample_index = sample_index + 1;
+            if (full) next_sample_index %= CAP;
+            if (next_sample_index == position) truncated = true;
+            if (s == PADDED - 2) truncated = true;
+            if (P.random_seq_length) {
+                if (current_seq_step == current_seq_length - 1) {
+                    truncated = true;
+                    current_seq_length = SEQ > 1 ? draw_length() : SEQ;
+                }
+                current_seq_step = truncated ? 0 : current_seq_step + 1;
+            }
+            if (truncated && s < PADDED - 1) {
+                B.final_step_mask[(size_t)s * N + b] = 1;
+                float* next = B.observations_actions_base + ((size_t)(s + 1) * N + b) * D;
+                for (int k = 0; k < OBS; k++) next[k] = row[D + 1 + k];
+                for (int k = 0; k < ACT; k++) next[OBS + k] = 0.0f;
+            }
+            sample_index = next_sample_index;
+            previous_padding_step = false;
+            previous_step_truncated = truncated;
+        }
+    }
+}
+
 __device__ __forceinline__ uint32_t mix32(uint64_t x) {   // splitmix64 finaliser
     x += 0x9E3779B97F4A7C15ull; x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull; x = (x ^ (x >> 27)) * 0x94D049BB133111EBull; x ^= x >> 31;
     return (uint32_t)(x >> 32);
@@ -459,10 +535,22 @@ int rlt_rocm_gather_batch(rlt_rocm_device* device, const rlt_replay_buffer* rb, 
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(rb_ok(rb) && batch > 0 && observations_actions_base && rewards && terminated && max_episode_length >= 0);
     RLT_REQUIRE(deterministic || (env_indices && sample_offsets));
-    void* counters; int rc = rlt_counters(device, &counters); if (rc) return rc;
-    int* error_flag = (int*)((char*)counters + 128);
+    int* error_flag = (int*)(device->fault + 1);        // read back by rlt_rocm_check_status
+    device->fault_armed = 1;
     hipLaunchKernelGGL(gather_kernel, dim3(grid1(batch * 16)), dim3(256), 0, device->stream, *rb, env_indices, sample_offsets, deterministic, max_episode_length, batch,
                        observations_actions_base, rewards, terminated, reset, next_reset_base, final_step_mask, next_final_step_mask_base, error_flag);
+    return rlt_launch_status(device);
+}
+
+int rlt_rocm_gather_sequence_batch(rlt_rocm_device* device, const rlt_replay_buffer* rb, const rlt_sequence_sampling* sampling, const rlt_sequence_draws* draws,
+                                   int max_episode_length, const rlt_sequence_batch* B) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(rb_ok(rb) && sampling && draws && B && max_episode_length >= 0 && B->batch > 0 && B->sequence_length >= 1);
+    RLT_REQUIRE(B->observations_actions_base && B->rewards && B->terminated && B->reset && B->next_reset_base && B->final_step_mask && B->next_final_step_mask_base);
+    RLT_REQUIRE(draws->env_indices && draws->sample_offsets && (!sampling->random_seq_length || (draws->nominal && draws->lengths)));
+    RLT_REQUIRE(!sampling->always_sample_from_initial_state || rb->capacity > max_episode_length);      // otherwise no row is eligible once a ring is full (:259)
+    device->fault_armed = 1;
+    hipLaunchKernelGGL(gather_sequence_kernel, dim3(grid1(B->batch)), dim3(256), 0, device->stream, *rb, *sampling, *draws, max_episode_length, *B, (int*)(device->fault + 1));
     return rlt_launch_status(device);
 }
 

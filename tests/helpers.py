@@ -63,6 +63,7 @@ def load_oracle():
     lib.rlt_oracle_ppo_shuffle.argtypes = [C.c_char_p, I, I, I, P]
     lib.rlt_oracle_on_policy_collect_with_rng.argtypes = [C.POINTER(capi.PendulumRunner), C.POINTER(capi.OnPolicyDataset), C.POINTER(capi.DenseLayer), I, P, P, P, P, P, I,
                                                           C.c_char_p, I]
+    lib.rlt_oracle_gather_sequence_batch_with_rng.argtypes = [C.POINTER(capi.ReplayBuffer), C.POINTER(capi.SequenceSampling), I, C.POINTER(capi.SequenceBatch), C.c_char_p, I, P, P, P, P]
     lib.rlt_oracle_sac_loop_create.argtypes = [C.POINTER(LoopConfig)]; lib.rlt_oracle_sac_loop_create.restype = P
     for f in ("destroy", "step"):
         getattr(lib, "rlt_oracle_sac_loop_" + f).argtypes = [P]
@@ -816,3 +817,93 @@ def car_on_backend(backend, states, actions, params=None):
     backend.call("car_step", C.byref(p), s.ptr, a.ptr, o.ptr, no.ptr, r.ptr, t.ptr, n)
     backend.sync()
     return s.numpy(), o.numpy(), no.numpy(), r.numpy(), t.numpy()
+
+
+REF_GATHER_SEQ_GENERIC = os.path.join(ORACLE_DIR, "_ref", "librlt_ref_gather_seq_generic.so")
+SEQUENCE_BATCH_FIELDS = ("observations_actions_base", "rewards", "terminated", "reset", "next_reset_base", "final_step_mask", "next_final_step_mask_base")
+
+
+class SequenceBatchOnBackend:
+    """A SequentialBatch on a backend, pre-filled the way the reference harness fills its own before gather_batch (what the gather does not write
+    stays: -777 in the float tensors, 0 in the flags)."""
+
+    def __init__(self, backend, batch, sequence_length, data_dim):
+        S, PS = sequence_length, sequence_length + 1
+        self.backend = backend
+        self.arrays = dict(observations_actions_base=backend.array(np.full((PS, batch, data_dim), -777.0, np.float32)), rewards=backend.array(np.full((S, batch), -777.0, np.float32)),
+                           terminated=backend.zeros((S, batch), np.uint8), reset=backend.zeros((S, batch), np.uint8), next_reset_base=backend.zeros((PS, batch), np.uint8),
+                           final_step_mask=backend.zeros((S, batch), np.uint8), next_final_step_mask_base=backend.zeros((PS, batch), np.uint8))
+        self.c = capi.SequenceBatch(*[self.arrays[k].ptr for k in SEQUENCE_BATCH_FIELDS], batch, sequence_length)
+
+    def numpy(self):
+        return {k: v.numpy() for k, v in self.arrays.items()}
+
+
+def replay_on_backend(backend, rings):
+    """rings: list of (data [capacity x row], position, full, episode_start [capacity]) per environment -> ReplayOnBackend filled with them."""
+    n, cap, row = len(rings), rings[0][0].shape[0], rings[0][0].shape[1]
+    rb = ReplayOnBackend(backend, n, cap, obs_dim=(row - 4) // 2, act_dim=1)
+    rb.data.upload(np.concatenate([r[0] for r in rings])); rb.episode_start.upload(np.concatenate([r[3] for r in rings]).astype(np.uint32))
+    rb.position.upload(np.array([r[1] for r in rings], np.uint32)); rb.full.upload(np.array([r[2] for r in rings], np.uint8))
+    return rb
+
+
+def gather_sequence_on_backend(backend, rings, sampling, draws, max_episode_length, batch, sequence_length):
+    """Array-fed sequence gather on a backend; draws = (env_indices, sample_offsets, nominal, lengths) as numpy arrays."""
+    rb = replay_on_backend(backend, rings)
+    out = SequenceBatchOnBackend(backend, batch, sequence_length, rings[0][0].shape[1] // 2 - 1)
+    d = [backend.array(np.ascontiguousarray(a)) for a in draws]
+    dc = capi.SequenceDraws(*[a.ptr for a in d])
+    backend.call("gather_sequence_batch", C.byref(rb.c), C.byref(sampling), C.byref(dc), max_episode_length, C.byref(out.c))
+    backend.sync()
+    return out.numpy()
+
+
+def sequence_gather_golden():
+    """The committed sequence-gather vectors (tests/golden/make_sequence_gather_golden.py) as a list of cases:
+    (rings, sampling, draws, max_episode_length, batch, sequence_length, expected tensors)."""
+    g = np.load(os.path.join(GOLDEN, "sequence_gather.npz"))
+    n_envs, capacity, max_len, batch, seq, row = [int(v) for v in g["dims"]]
+    cases = []
+    for si in range(len(g["stops"])):
+        rings = [(g[f"s{si}_data"][e], int(g[f"s{si}_position"][e]), int(g[f"s{si}_full"][e]), g[f"s{si}_episode_start"][e]) for e in range(n_envs)]
+        for variant in range(3):
+            v = g["sampling"][variant]
+            sampling = capi.SequenceSampling(int(v[0]), int(v[1]), int(v[2]), float(v[3]), int(v[4]))
+            draws = tuple(g[f"s{si}_v{variant}_{k}"] for k in ("env_indices", "sample_offsets", "nominal", "lengths"))
+            want = {k: g[f"s{si}_v{variant}_{k}"] for k in SEQUENCE_BATCH_FIELDS}
+            cases.append((rings, sampling, draws, max_len, batch, 1 if variant == 2 else seq, want))
+    return cases
+
+
+def synthetic_rings(rng, n_envs, capacity, obs_dim, steps, episode_limit):
+    """Replay rings as a runner would leave them after `steps` steps per environment with episodes of random length up to episode_limit."""
+    row = 2 * obs_dim + 4
+    rings = []
+    for e in range(n_envs):
+        data, es = np.zeros((capacity, row), np.float32), np.zeros(capacity, np.uint32)
+        position, full, start, left = 0, 0, 0, int(rng.integers(1, episode_limit + 1))
+        for t in range(steps):
+            data[position] = rng.standard_normal(row).astype(np.float32)
+            left -= 1
+            data[position, row - 2] = float(rng.random() < 0.02)          # terminated
+            data[position, row - 1] = float(left == 0)                    # truncated
+            es[position] = start
+            position = (position + 1) % capacity
+            if position == 0:
+                full = 1
+            if left == 0:
+                start, left = position, int(rng.integers(1, episode_limit + 1))
+        rings.append((data, position, full, es))
+    return rings
+
+
+def random_sequence_draws(rng, rings, sampling, max_episode_length, batch, sequence_length):
+    """Draws with the ranges gather_batch uses (every sample gets a full set; it consumes a prefix)."""
+    n_envs, cap = len(rings), rings[0][0].shape[0]
+    env = rng.integers(0, n_envs, batch).astype(np.uint32)
+    eligible = np.array([(cap - max_episode_length if sampling.always_sample_from_initial_state else cap) if r[2] else r[1] for r in rings])
+    off = (rng.random((batch, sequence_length + 1)) * eligible[env][:, None]).astype(np.uint32)
+    nom = (rng.random((batch, sequence_length + 2)) < sampling.nominal_sequence_length_probability).astype(np.uint8)
+    length = rng.integers(1, max(sequence_length, 2), (batch, sequence_length + 2)).astype(np.uint32)
+    return env, off, nom, length

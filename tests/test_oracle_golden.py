@@ -357,3 +357,46 @@ def test_car_reproduces_reference_vectors_and_kinematics(oracle):
     s64 = st.astype(np.float64)
     assert np.array_equal(nx[:, 5], s64[:, 5])
     assert np.abs(nx[:, 4] - (s64[:, 4] - p.dt * s64[:, 5] * s64[:, 3])).max() <= 1e-8
+
+
+def test_sequence_gather_reproduces_reference_vectors_and_invariants(oracle):
+    """gather_batch for sequence batches against the reference's own batches (tests/golden/make_sequence_gather_golden.py), every tensor entry for entry,
+    from the stored draws. Then on synthetic rings what the construction guarantees whatever the draws: observation/action rows of the batch are rows of
+    the chosen ring or the step after a sequence end (next observation + zero action); sequences never run across an episode end or the ring's cursor;
+    every sample's masks are consistent (the step after a final step carries the next observation and a zero action, and a new sequence starts
+    behind it; the last unpadded step ends a sequence or is such a padding step)."""
+    for rings, sampling, draws, max_len, batch, seq, want in helpers.sequence_gather_golden():
+        got = helpers.gather_sequence_on_backend(oracle, rings, sampling, draws, max_len, batch, seq)
+        for k in helpers.SEQUENCE_BATCH_FIELDS:
+            assert np.array_equal(got[k], want[k]), k
+    rng = np.random.default_rng(0)
+    for (always, random_len, steps) in ((1, 1, 700), (0, 0, 700), (1, 1, 100), (0, 1, 180)):
+        obs, cap, max_len, batch, seq = 5, 300, 40, 128, 12
+        rings = helpers.synthetic_rings(rng, 4, cap, obs, steps, max_len)
+        sampling = helpers.capi.SequenceSampling(always, random_len, 1, 0.5, 1)
+        env, off, nom, length = helpers.random_sequence_draws(rng, rings, sampling, max_len, batch, seq)
+        got = helpers.gather_sequence_on_backend(oracle, rings, sampling, (env, off, nom, length), max_len, batch, seq)
+        oab, final, reset, nfinal = got["observations_actions_base"], got["final_step_mask"], got["reset"], got["next_final_step_mask_base"]
+        assert np.all((final[-1] == 1) | (final[-2] == 1)) and np.all(reset[0] == 1) and np.all(nfinal[0] == 0)      # the last step ends a sequence or pads after one
+        for b in range(batch):
+            data, position, full, es = rings[env[b]]
+            valid = np.arange(cap) if full else np.arange(position)
+            s = 0
+            while s <= seq:
+                # a sequence starts at s: find the ring row it starts from
+                rows = np.nonzero((data[valid][:, :obs + 1] == oab[s, b]).all(1))[0]
+                assert len(rows) >= 1 and reset[min(s, seq - 1), b] == 1 or s == seq, (b, s)
+                if s == seq:
+                    break
+                r = valid[rows[0]]
+                if always:
+                    assert es[r] == r
+                while True:
+                    assert np.array_equal(oab[s, b], data[r, :obs + 1]) and got["rewards"][s, b] == data[r, obs + 1]
+                    if final[s, b]:
+                        assert np.array_equal(oab[s + 1, b, :obs], data[r, obs + 2:2 * obs + 2]) and oab[s + 1, b, obs] == 0 and nfinal[s + 1, b] == 1
+                        s += 2      # the step after a final step holds the next observation; a new sequence starts after it
+                        break
+                    assert data[r, -1] == 0 and (r + 1) % cap != position       # not the end of an episode, not the cursor
+                    r = (r + 1) % cap
+                    s += 1

@@ -170,6 +170,86 @@ def test_car_bit_exact_with_reference(oracle):
     assert np.abs(sr[:, 3]).max() > 0.5          # the cars got going
 
 
+class RefGatherSeq:
+    """The reference's SAC loop with three environments, episodes of 30 steps and rings of 260 rows (oracle/ref_harness/ref_gather_seq.cpp)."""
+
+    def __init__(self, seed):
+        self.lib = C.CDLL(helpers.REF_GATHER_SEQ_GENERIC)
+        P = C.c_void_p
+        self.lib.rlt_ref_gather_seq_create.restype = P
+        self.lib.rlt_ref_gather_seq_step.argtypes = [P]; self.lib.rlt_ref_gather_seq_destroy.argtypes = [P]
+        self.lib.rlt_ref_gather_seq_get_replay.argtypes = [P, C.c_int, P, P, P, P]
+        self.lib.rlt_ref_gather_seq_gather.argtypes = [P, C.c_int, C.c_uint32, C.c_char_p, C.c_int] + [P] * 7
+        dims = (C.c_int * 6)()
+        self.lib.rlt_ref_gather_seq_dims(dims)
+        self.n_envs, self.capacity, self.max_episode_length, self.batch, self.sequence_length, self.row = list(dims)
+        self.h = P(self.lib.rlt_ref_gather_seq_create(seed))
+
+    def rings(self):
+        out = []
+        for e in range(self.n_envs):
+            data, pos, full, es = np.zeros((self.capacity, self.row), np.float32), C.c_uint32(), C.c_uint8(), np.zeros(self.capacity, np.uint32)
+            self.lib.rlt_ref_gather_seq_get_replay(self.h, e, data.ctypes.data, C.byref(pos), C.byref(full), es.ctypes.data)
+            out.append((data, pos.value, full.value, es))
+        return out
+
+    def gather(self, variant, seed):
+        S = 1 if variant == 2 else self.sequence_length
+        PS, N, D = S + 1, self.batch, self.row // 2 - 1
+        rng = C.create_string_buffer(16384)
+        out = dict(observations_actions_base=np.zeros((PS, N, D), np.float32), rewards=np.zeros((S, N), np.float32), terminated=np.zeros((S, N), np.uint8),
+                   reset=np.zeros((S, N), np.uint8), next_reset_base=np.zeros((PS, N), np.uint8), final_step_mask=np.zeros((S, N), np.uint8),
+                   next_final_step_mask_base=np.zeros((PS, N), np.uint8))
+        assert self.lib.rlt_ref_gather_seq_gather(self.h, variant, seed, rng, 16384, *[out[k].ctypes.data for k in helpers.SEQUENCE_BATCH_FIELDS]) == 0
+        return S, rng, out
+
+
+SEQUENCE_SAMPLING = {0: (1, 1, 1, 0.5, 1), 1: (0, 0, 1, 0.5, 1), 2: (0, 0, 1, 0.5, 0)}     # the harness's variants as SequentialBatchParameters
+
+
+@pytest.mark.skipif(not os.path.exists(helpers.REF_GATHER_SEQ_GENERIC), reason="sequence-gather flavour of oracle/_ref not built")
+def test_sequence_gather_bit_exact_with_reference(oracle):
+    """gather_batch for SequentialBatch with SEQUENCE_LENGTH 8 (the reference's defaults: sequences start at their episode's first step and have random
+    lengths; and both switched off) and 1, on the replay rings of the reference's own runner with three environments and 30-step episodes, before the
+    rings are full (90 and 150 rows) and after they wrapped (600 loop steps into 260 rows, 60 of them eligible): every tensor of the batch equals the reference's, entry for
+    entry including the entries gather_batch leaves untouched, with the draws made in the reference's order on its std::mt19937; and the draws the
+    restatement hands back reproduce the same batch when fed in as arrays."""
+    ref = RefGatherSeq(0)
+    steps = 0
+    seen_restart = seen_short = False
+    for stop in (90, 150, 600):
+        while steps < stop:
+            ref.lib.rlt_ref_gather_seq_step(ref.h); steps += 1
+        rings = ref.rings()
+        assert all(r[1] == stop % ref.capacity for r in rings) and all(bool(r[2]) == (stop >= ref.capacity) for r in rings)
+        for variant in (0, 1, 2):
+            for seed in (1, 2, 3):
+                S, rng, want = ref.gather(variant, seed)
+                sampling = helpers.capi.SequenceSampling(*SEQUENCE_SAMPLING[variant])
+                rb = helpers.replay_on_backend(oracle, rings)
+                out = helpers.SequenceBatchOnBackend(oracle, ref.batch, S, ref.row // 2 - 1)
+                env, off, nom, length = np.zeros(ref.batch, np.uint32), np.zeros((ref.batch, S + 1), np.uint32), np.zeros((ref.batch, S + 2), np.uint8), np.zeros((ref.batch, S + 2), np.uint32)
+                assert oracle.lib.rlt_oracle_gather_sequence_batch_with_rng(C.byref(rb.c), C.byref(sampling), ref.max_episode_length, C.byref(out.c), rng, 16384,
+                                                                            env.ctypes.data, off.ctypes.data, nom.ctypes.data, length.ctypes.data) == 0
+                got = out.numpy()
+                for k in helpers.SEQUENCE_BATCH_FIELDS:
+                    assert np.array_equal(got[k], want[k]), (stop, variant, seed, k)
+                fed = helpers.gather_sequence_on_backend(oracle, rings, sampling, (env, off, nom, length), ref.max_episode_length, ref.batch, S)
+                for k in helpers.SEQUENCE_BATCH_FIELDS:
+                    assert np.array_equal(fed[k], want[k]), ("fed", stop, variant, seed, k)
+                assert len(np.unique(env)) == ref.n_envs
+                if variant == 0:
+                    seen_restart |= bool((want["reset"][1:].sum(0) > 0).any())            # a sequence ended early and another started inside the sample
+                    seen_short |= bool((want["final_step_mask"][:-1].sum(0) > 0).any())
+                if variant == 2:     # single steps: what rlt_*_gather_batch computes
+                    oab, rew, term = oracle.zeros((2, ref.batch, 4)), oracle.zeros((ref.batch,)), oracle.zeros((ref.batch,), np.uint8)
+                    e_, o_ = oracle.array(env), oracle.array(np.ascontiguousarray(off[:, 0]))
+                    oracle.call("gather_batch", C.byref(rb.c), e_.ptr, o_.ptr, 0, ref.max_episode_length, ref.batch, oab.ptr, rew.ptr, term.ptr, None, None, None, None)
+                    assert np.array_equal(oab.numpy(), want["observations_actions_base"]) and np.array_equal(rew.numpy(), want["rewards"][0])
+    assert seen_restart and seen_short
+    ref.lib.rlt_ref_gather_seq_destroy(ref.h)
+
+
 def test_small_ring_wraps_bit_exact_with_reference(oracle):
     """Replay capacity 250 (< 900 steps): the ring wraps three times, so `add` past the end, the prologue's wrap of the
     previous row, `full`, and gather's (position + MAX_EPISODE_LENGTH + offset) % CAPACITY index all run, and every
