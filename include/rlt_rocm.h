@@ -422,6 +422,18 @@ typedef struct rlt_car_parameters {
 int rlt_rocm_car_step(rlt_rocm_device* device, const rlt_car_parameters* p, float* states, const float* actions,
                       float* observations, float* next_observations, float* rewards, uint8_t* terminated, int n_envs);
 
+/* The Car on a track (CarTrack, rl/environments/car/car.h:34-41,101-108): `track` is a height x width bitmap (1 = drivable) of square cells
+ * `track_scale` metres wide, centred on the origin, row 0 at the top (largest y).
+ *   terminated (operations_generic.h:85-98): the next state's cell is not drivable or lies outside the bitmap
+ *   reward (:136-141): the pre-step forward speed vx;  step: as rlt_rocm_car_step
+ *   observe (:156-190): the state, then for the directions -20, 0, +20 degrees off the heading the distance to the first cell that is
+ *   not drivable along a ray of 50 steps of half a cell, as a fraction of the ray's length. A ray that leaves the bitmap ends there
+ *   (the reference reads past the array in that case).
+ *   states [n_envs x 6], actions [n_envs x 2], observations and next_observations [n_envs x 9]. Any output may be NULL. */
+int rlt_rocm_car_track_step(rlt_rocm_device* device, const rlt_car_parameters* p, const uint8_t* track, int height, int width, float track_scale,
+                            float* states, const float* actions, float* observations, float* next_observations, float* rewards,
+                            uint8_t* terminated, int n_envs);
+
 /* Per-environment runner state (rl/components/off_policy_runner/off_policy_runner.h:184-221). */
 typedef struct rlt_pendulum_runner {
     float* states;            /* [n_envs x 2]  */

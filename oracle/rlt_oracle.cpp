@@ -860,29 +860,33 @@ int rlt_oracle_acrobot_step(const rlt_acrobot_parameters* P, int swingup, float*
 
 // rl/environments/car/operations_generic.h:80-84 (terminated), :99-127 (step), :128-135 (reward), :143-155 (observe). T = float; the tire
 // force goes through an unqualified atan (the double function) and the reward through the double literal 0.1, kept as the C++ expression has them.
+static void car_dynamics(const rlt_car_parameters& p, const float* s, const float* action, float* n) {      // step, :99-127
+    const float mu = s[2], vx = s[3], vy = s[4], omega = s[5];
+    const float throttle_break = clampf(action[0], -1.0f, 1.0f), delta = clampf(action[1], -1.0f, 1.0f);
+    const float alpha_f = std::atan2((vy + p.lf * omega), vx) - delta;
+    const float alpha_r = std::atan2((vy - p.lr * omega), vx);
+    const float FnF = p.lr / (p.lf + p.lr) * p.m * p.g;
+    const float FnR = p.lf / (p.lf + p.lr) * p.m * p.g;
+    const float FyF = vx > p.vt || vy > p.vt ? FnF * p.tf_D * std::sin(p.tf_C * std::atan((double)(p.tf_B * (-alpha_f)))) : 0;
+    const float FyR = vx > p.vt || vy > p.vt ? FnR * p.tr_D * std::sin(p.tr_C * std::atan((double)(p.tr_B * (-alpha_r)))) : 0;
+    const float Fx = p.cm * throttle_break - p.cr0 - p.cr2 * vx * vx;
+    for (int i = 0; i < 6; i++) n[i] = s[i];
+    n[0] += p.dt * (std::cos(mu) * vx - std::sin(mu) * vy);
+    n[1] += p.dt * (std::sin(mu) * vx + std::cos(mu) * vy);
+    n[2] += p.dt * (omega);
+    n[3] += p.dt * (1 / p.m * (Fx - FyF * std::sin(delta)) + omega * vy);
+    n[4] += p.dt * (1 / p.m * (FyF * std::cos(delta) + FyR) - omega * vx);
+    n[5] += p.dt * (1 / p.I * (FyF * p.lf * std::cos(delta) - FyR * p.lr));
+}
 int rlt_oracle_car_step(const rlt_car_parameters* P, float* states, const float* actions, float* observations, float* next_observations, float* rewards,
                         uint8_t* terminated, int n_envs) {
     if (!P || !states || !actions || n_envs <= 0) return RLT_E_INVALID_ARGUMENT;
-    const rlt_car_parameters& p = *P;
     for (int e = 0; e < n_envs; e++) {
         float* s = states + 6 * (size_t)e;
-        const float x = s[0], y = s[1], mu = s[2], vx = s[3], vy = s[4], omega = s[5];
+        const float x = s[0], y = s[1], mu = s[2];
         if (observations) for (int i = 0; i < 6; i++) observations[6 * (size_t)e + i] = s[i];
-        const float throttle_break = clampf(actions[2 * (size_t)e], -1.0f, 1.0f), delta = clampf(actions[2 * (size_t)e + 1], -1.0f, 1.0f);
-        const float alpha_f = std::atan2((vy + p.lf * omega), vx) - delta;
-        const float alpha_r = std::atan2((vy - p.lr * omega), vx);
-        const float FnF = p.lr / (p.lf + p.lr) * p.m * p.g;
-        const float FnR = p.lf / (p.lf + p.lr) * p.m * p.g;
-        const float FyF = vx > p.vt || vy > p.vt ? FnF * p.tf_D * std::sin(p.tf_C * std::atan((double)(p.tf_B * (-alpha_f)))) : 0;
-        const float FyR = vx > p.vt || vy > p.vt ? FnR * p.tr_D * std::sin(p.tr_C * std::atan((double)(p.tr_B * (-alpha_r)))) : 0;
-        const float Fx = p.cm * throttle_break - p.cr0 - p.cr2 * vx * vx;
-        float n[6] = {x, y, mu, vx, vy, omega};
-        n[0] += p.dt * (std::cos(mu) * vx - std::sin(mu) * vy);
-        n[1] += p.dt * (std::sin(mu) * vx + std::cos(mu) * vy);
-        n[2] += p.dt * (omega);
-        n[3] += p.dt * (1 / p.m * (Fx - FyF * std::sin(delta)) + omega * vy);
-        n[4] += p.dt * (1 / p.m * (FyF * std::cos(delta) + FyR) - omega * vx);
-        n[5] += p.dt * (1 / p.I * (FyF * p.lf * std::cos(delta) - FyR * p.lr));
+        float n[6];
+        car_dynamics(*P, s, actions + 2 * (size_t)e, n);
         if (rewards) {
             const float angle_norm = angle_normalize(mu);
             const float cost = 0.1 * angle_norm * angle_norm + x * x + y * y;
@@ -890,6 +894,49 @@ int rlt_oracle_car_step(const rlt_car_parameters* P, float* states, const float*
         }
         if (terminated) terminated[e] = n[0] > 1.0 || n[0] < -1.0 || n[1] > 1.0 || n[1] < -1.0;
         if (next_observations) for (int i = 0; i < 6; i++) next_observations[6 * (size_t)e + i] = n[i];
+        for (int i = 0; i < 6; i++) s[i] = n[i];
+    }
+    return 0;
+}
+// CarTrack: terminated :85-98, reward :136-141, observe :156-190 (T = float, TI = size_t; the double literal 2.0 makes the cell coordinates go through
+// double). Cells outside the bitmap count as not drivable; the reference's observe would read past its array there.
+struct CarTrackMap { const uint8_t* track; int height, width; float scale; };
+static bool car_track_cell(const CarTrackMap& M, float x_coord, float y_coord) {
+    if (!(x_coord > 0 && x_coord < M.width && y_coord > 0 && y_coord < M.height)) return false;
+    return M.track[(size_t)y_coord * M.width + (size_t)x_coord] != 0;
+}
+static void car_track_observe(const CarTrackMap& M, const float* s, float* o) {
+    for (int i = 0; i < 6; i++) o[i] = s[i];
+    const float PI = (float)M_PI;
+    const int NUM_STEPS = 50;
+    const float step_size = M.scale / 2;
+    const float directions[3] = {(float)(-20 / 180.0 * PI), 0, (float)(20 / 180.0 * PI)};
+    for (int d = 0; d < 3; d++) {
+        const float direction_x = std::cos(s[2] + directions[d]) * step_size, direction_y = std::sin(s[2] + directions[d]) * step_size;
+        float distance = NUM_STEPS * step_size;
+        for (size_t step_i = 0; step_i < (size_t)NUM_STEPS; step_i++) {
+            const float x_coord = (+s[0] + direction_x * step_i + M.scale * (size_t)M.width / 2.0) / ((float)M.scale);
+            const float y_coord = (-s[1] - direction_y * step_i + M.scale * (size_t)M.height / 2.0) / ((float)M.scale);
+            if (!car_track_cell(M, x_coord, y_coord)) { distance = step_i * step_size; break; }
+        }
+        o[6 + d] = distance / (NUM_STEPS * step_size);
+    }
+}
+int rlt_oracle_car_track_step(const rlt_car_parameters* P, const uint8_t* track, int height, int width, float track_scale, float* states, const float* actions,
+                              float* observations, float* next_observations, float* rewards, uint8_t* terminated, int n_envs) {
+    if (!P || !track || height < 1 || width < 1 || !(track_scale > 0) || !states || !actions || n_envs <= 0) return RLT_E_INVALID_ARGUMENT;
+    const CarTrackMap M = {track, height, width, track_scale};
+    for (int e = 0; e < n_envs; e++) {
+        float* s = states + 6 * (size_t)e;
+        if (observations) car_track_observe(M, s, observations + 9 * (size_t)e);
+        float n[6];
+        car_dynamics(*P, s, actions + 2 * (size_t)e, n);
+        if (rewards) rewards[e] = s[3];
+        if (terminated) {
+            const float x_coord = (n[0] + M.scale * (size_t)width / 2.0) / ((float)M.scale), y_coord = (-n[1] + M.scale * (size_t)height / 2.0) / ((float)M.scale);
+            terminated[e] = !car_track_cell(M, x_coord, y_coord);
+        }
+        if (next_observations) car_track_observe(M, n, next_observations + 9 * (size_t)e);
         for (int i = 0; i < 6; i++) s[i] = n[i];
     }
     return 0;

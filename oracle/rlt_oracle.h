@@ -25,7 +25,9 @@
  *   environments (oracle/_ref/librlt_ref_envs_generic.so) on random states and closed chains, golden vectors, and energy conservation /
  *   integration order / work-energy checks that do not involve the reference.
  *   car step (single-track model, reward, terminated; no track): bit for bit against the reference's Car (oracle/_ref/librlt_ref_envs_generic.so),
- *   golden vectors, and closed forms (straight rolling, pose equivariance, no tire force below the speed threshold).
+ *   golden vectors, and closed forms (straight rolling, pose equivariance, no tire force below the speed threshold). On a track: bit for bit against
+ *   the reference's CarTrack on its default track where the reference is mounted (the bitmap is not kept as a fixture), closed-form ray lengths in a
+ *   straight corridor.
  *   gather for sequence batches: all seven tensors of the batch entry for entry against the reference's gather_batch on its own runner's rings
  *   (oracle/_ref/librlt_ref_gather_seq_generic.so; sequence length 8 with and without the default sampling switches, and 1), draws made on the
  *   reference's std::mt19937 in its order; golden vectors; structural invariants on synthetic rings.
@@ -122,6 +124,8 @@ int rlt_oracle_acrobot_step(const rlt_acrobot_parameters* p, int swingup, float*
 /* rl/environments/car/operations_generic.h:80-155 (the Car without a track) */
 int rlt_oracle_car_step(const rlt_car_parameters* p, float* states, const float* actions, float* observations, float* next_observations, float* rewards,
                         uint8_t* terminated, int n_envs);
+int rlt_oracle_car_track_step(const rlt_car_parameters* p, const uint8_t* track, int height, int width, float track_scale, float* states, const float* actions,
+                              float* observations, float* next_observations, float* rewards, uint8_t* terminated, int n_envs);
 /* rl::utils::evaluation::evaluate with the Pendulum environment (rl/utils/evaluation/operations_generic.h:106-233) */
 int rlt_oracle_pendulum_evaluate(const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers, const float* initial_states,
                                  int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary);

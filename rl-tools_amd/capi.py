@@ -215,6 +215,7 @@ PROTOTYPES = {
     "gather_sequence_batch": [C.POINTER(ReplayBuffer), C.POINTER(SequenceSampling), C.POINTER(SequenceDraws), I, C.POINTER(SequenceBatch)],
     "acrobot_step": [C.POINTER(AcrobotParameters), I, P, P, P, P, P, P, I],
     "car_step": [C.POINTER(CarParameters), P, P, P, P, P, P, I],
+    "car_track_step": [C.POINTER(CarParameters), P, I, I, F, P, P, P, P, P, P, I],
     "pendulum_evaluate": [C.POINTER(PendulumParameters), I, LP, I, P, I, I, P, P, P],
     "ppo_gae": [P, P, P, P, P, P, I, I, I, F, F, I],
     "gru_forward": [C.POINTER(GruLayer), P, P, I, I, P, S],

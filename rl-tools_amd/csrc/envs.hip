@@ -61,37 +61,92 @@ __global__ __launch_bounds__(256) void acrobot_step_kernel(rlt_acrobot_parameter
     }
 }
 
-// Car without a track: single-track model with Pacejka tire forces, explicit Euler over dt (rl/environments/car/operations_generic.h:99-127); the
-// reward comes from the pre-step state (:128-135), terminated from the next one (:80-84), the observation is the state (:143-155).
+// Car: single-track model with Pacejka tire forces, explicit Euler over dt (rl/environments/car/operations_generic.h:99-127)
+struct Car6 { float x, y, mu, vx, vy, omega; };
+__device__ __forceinline__ Car6 car_dynamics(const rlt_car_parameters& p, const Car6& s, float2 a) {
+    const float throttle_break = clampf(a.x, -1.0f, 1.0f), delta = clampf(a.y, -1.0f, 1.0f);
+    const float alpha_f = atan2f(s.vy + p.lf * s.omega, s.vx) - delta;
+    const float alpha_r = atan2f(s.vy - p.lr * s.omega, s.vx);
+    const float FnF = p.lr / (p.lf + p.lr) * p.m * p.g, FnR = p.lf / (p.lf + p.lr) * p.m * p.g;
+    const bool moving = s.vx > p.vt || s.vy > p.vt;
+    const float FyF = moving ? FnF * p.tf_D * sinf(p.tf_C * atanf(p.tf_B * (-alpha_f))) : 0.0f;
+    const float FyR = moving ? FnR * p.tr_D * sinf(p.tr_C * atanf(p.tr_B * (-alpha_r))) : 0.0f;
+    const float Fx = p.cm * throttle_break - p.cr0 - p.cr2 * s.vx * s.vx;
+    float sm, cm_, sd, cd;
+    sincosf(s.mu, &sm, &cm_);
+    sincosf(delta, &sd, &cd);
+    Car6 n;
+    n.x = s.x + p.dt * (cm_ * s.vx - sm * s.vy);
+    n.y = s.y + p.dt * (sm * s.vx + cm_ * s.vy);
+    n.mu = s.mu + p.dt * s.omega;
+    n.vx = s.vx + p.dt * (1.0f / p.m * (Fx - FyF * sd) + s.omega * s.vy);
+    n.vy = s.vy + p.dt * (1.0f / p.m * (FyF * cd + FyR) - s.omega * s.vx);
+    n.omega = s.omega + p.dt * (1.0f / p.I * (FyF * p.lf * cd - FyR * p.lr));
+    return n;
+}
+__device__ __forceinline__ Car6 car_load(const float* __restrict__ states, int e) {
+    const float2* sp = reinterpret_cast<const float2*>(states) + 3 * (size_t)e;
+    const float2 s0 = sp[0], s1 = sp[1], s2 = sp[2];
+    return {s0.x, s0.y, s1.x, s1.y, s2.x, s2.y};
+}
+__device__ __forceinline__ void car_store(float* __restrict__ rows, size_t row_floats, int e, const Car6& s) {       // the state as the first six values of row e (rows start 8-byte aligned)
+    float2* o = reinterpret_cast<float2*>(rows + row_floats * (size_t)e);
+    o[0] = make_float2(s.x, s.y); o[1] = make_float2(s.mu, s.vx); o[2] = make_float2(s.vy, s.omega);
+}
+
+// without a track: the reward comes from the pre-step state (:128-135), terminated from the next one (:80-84), the observation is the state (:143-155)
 __global__ __launch_bounds__(256) void car_step_kernel(rlt_car_parameters p, float* __restrict__ states, const float* __restrict__ actions, float* __restrict__ observations,
                                                        float* __restrict__ next_observations, float* __restrict__ rewards, uint8_t* __restrict__ terminated, int n) {
     for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
-        float2* sp = reinterpret_cast<float2*>(states) + 3 * (size_t)e;
-        const float2 s0 = sp[0], s1 = sp[1], s2 = sp[2];
-        const float x = s0.x, y = s0.y, mu = s1.x, vx = s1.y, vy = s2.x, omega = s2.y;
-        if (observations) { float2* o = reinterpret_cast<float2*>(observations) + 3 * (size_t)e; o[0] = s0; o[1] = s1; o[2] = s2; }
-        const float2 a = reinterpret_cast<const float2*>(actions)[e];
-        const float throttle_break = clampf(a.x, -1.0f, 1.0f), delta = clampf(a.y, -1.0f, 1.0f);
-        const float alpha_f = atan2f(vy + p.lf * omega, vx) - delta;
-        const float alpha_r = atan2f(vy - p.lr * omega, vx);
-        const float FnF = p.lr / (p.lf + p.lr) * p.m * p.g, FnR = p.lf / (p.lf + p.lr) * p.m * p.g;
-        const bool moving = vx > p.vt || vy > p.vt;
-        const float FyF = moving ? FnF * p.tf_D * sinf(p.tf_C * atanf(p.tf_B * (-alpha_f))) : 0.0f;
-        const float FyR = moving ? FnR * p.tr_D * sinf(p.tr_C * atanf(p.tr_B * (-alpha_r))) : 0.0f;
-        const float Fx = p.cm * throttle_break - p.cr0 - p.cr2 * vx * vx;
-        float sm, cm_, sd, cd;
-        sincosf(mu, &sm, &cm_);
-        sincosf(delta, &sd, &cd);
-        const float nx = x + p.dt * (cm_ * vx - sm * vy);
-        const float ny = y + p.dt * (sm * vx + cm_ * vy);
-        const float nmu = mu + p.dt * omega;
-        const float nvx = vx + p.dt * (1.0f / p.m * (Fx - FyF * sd) + omega * vy);
-        const float nvy = vy + p.dt * (1.0f / p.m * (FyF * cd + FyR) - omega * vx);
-        const float nomega = omega + p.dt * (1.0f / p.I * (FyF * p.lf * cd - FyR * p.lr));
-        if (rewards) { const float an = angle_normalize(mu); rewards[e] = expf(-5.0f * (0.1f * an * an + x * x + y * y)); }
-        if (terminated) terminated[e] = nx > 1.0f || nx < -1.0f || ny > 1.0f || ny < -1.0f;
-        if (next_observations) { float2* o = reinterpret_cast<float2*>(next_observations) + 3 * (size_t)e; o[0] = make_float2(nx, ny); o[1] = make_float2(nmu, nvx); o[2] = make_float2(nvy, nomega); }
-        sp[0] = make_float2(nx, ny); sp[1] = make_float2(nmu, nvx); sp[2] = make_float2(nvy, nomega);
+        const Car6 s = car_load(states, e);
+        if (observations) car_store(observations, 6, e, s);
+        const Car6 nx = car_dynamics(p, s, reinterpret_cast<const float2*>(actions)[e]);
+        if (rewards) { const float an = angle_normalize(s.mu); rewards[e] = expf(-5.0f * (0.1f * an * an + s.x * s.x + s.y * s.y)); }
+        if (terminated) terminated[e] = nx.x > 1.0f || nx.x < -1.0f || nx.y > 1.0f || nx.y < -1.0f;
+        if (next_observations) car_store(next_observations, 6, e, nx);
+        car_store(states, 6, e, nx);
+    }
+}
+
+// on a track (:85-98 terminated, :136-141 reward, :156-190 observe): cell coordinates in double, as the reference's double literal makes them
+struct TrackMap { const uint8_t* track; int height, width; float scale; };
+__device__ __forceinline__ bool track_cell(const TrackMap& M, float x_coord, float y_coord) {
+    if (!(x_coord > 0.0f && x_coord < (float)M.width && y_coord > 0.0f && y_coord < (float)M.height)) return false;       // beyond the bitmap: not drivable
+    return M.track[(size_t)y_coord * M.width + (size_t)x_coord] != 0;
+}
+__device__ __forceinline__ void track_observe(const TrackMap& M, const Car6& s, float* __restrict__ o) {
+    const float step_size = M.scale / 2.0f;
+    const float directions[3] = {(float)(-20 / 180.0 * 3.14159274101257324), 0.0f, (float)(20 / 180.0 * 3.14159274101257324)};      // 20 degrees of the float pi
+    const int NUM_STEPS = 50;
+#pragma unroll
+    for (int d = 0; d < 3; d++) {
+        float sn, cs;
+        sincosf(s.mu + directions[d], &sn, &cs);
+        const float direction_x = cs * step_size, direction_y = sn * step_size;
+        float distance = NUM_STEPS * step_size;
+        for (int step_i = 0; step_i < NUM_STEPS; step_i++) {
+            const float x_coord = (float)(((double)(s.x + direction_x * (float)step_i) + (double)(M.scale * (float)M.width) / 2.0) / (double)M.scale);
+            const float y_coord = (float)(((double)(-s.y - direction_y * (float)step_i) + (double)(M.scale * (float)M.height) / 2.0) / (double)M.scale);
+            if (!track_cell(M, x_coord, y_coord)) { distance = (float)step_i * step_size; break; }
+        }
+        o[6 + d] = distance / (NUM_STEPS * step_size);
+    }
+}
+__global__ __launch_bounds__(256) void car_track_step_kernel(rlt_car_parameters p, TrackMap M, float* __restrict__ states, const float* __restrict__ actions,
+                                                             float* __restrict__ observations, float* __restrict__ next_observations, float* __restrict__ rewards,
+                                                             uint8_t* __restrict__ terminated, int n) {
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
+        const Car6 s = car_load(states, e);
+        if (observations) { float* o = observations + 9 * (size_t)e; o[0] = s.x; o[1] = s.y; o[2] = s.mu; o[3] = s.vx; o[4] = s.vy; o[5] = s.omega; track_observe(M, s, o); }
+        const Car6 nx = car_dynamics(p, s, reinterpret_cast<const float2*>(actions)[e]);
+        if (rewards) rewards[e] = s.vx;
+        if (terminated) {
+            const float x_coord = (float)(((double)nx.x + (double)(M.scale * (float)M.width) / 2.0) / (double)M.scale);
+            const float y_coord = (float)(((double)(-nx.y) + (double)(M.scale * (float)M.height) / 2.0) / (double)M.scale);
+            terminated[e] = !track_cell(M, x_coord, y_coord);
+        }
+        if (next_observations) { float* o = next_observations + 9 * (size_t)e; o[0] = nx.x; o[1] = nx.y; o[2] = nx.mu; o[3] = nx.vx; o[4] = nx.vy; o[5] = nx.omega; track_observe(M, nx, o); }
+        car_store(states, 6, e, nx);
     }
 }
 }  // namespace
@@ -103,6 +158,17 @@ extern "C" int rlt_rocm_car_step(rlt_rocm_device* device, const rlt_car_paramete
     RLT_REQUIRE((((uintptr_t)states | (uintptr_t)actions | (uintptr_t)observations | (uintptr_t)next_observations) & 7) == 0);      // rows move as 8-byte pairs
     int blocks = (n_envs + 255) / 256; if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(car_step_kernel, dim3(blocks), dim3(256), 0, device->stream, *p, states, actions, observations, next_observations, rewards, terminated, n_envs);
+    return rlt_launch_status(device);
+}
+
+extern "C" int rlt_rocm_car_track_step(rlt_rocm_device* device, const rlt_car_parameters* p, const uint8_t* track, int height, int width, float track_scale, float* states,
+                                       const float* actions, float* observations, float* next_observations, float* rewards, uint8_t* terminated, int n_envs) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(p && track && height >= 1 && width >= 1 && track_scale > 0.0f && states && actions && n_envs > 0);
+    RLT_REQUIRE((((uintptr_t)states | (uintptr_t)actions) & 7) == 0);      // states and actions move as 8-byte pairs
+    int blocks = (n_envs + 255) / 256; if (blocks > 4096) blocks = 4096;
+    const TrackMap M = {track, height, width, track_scale};
+    hipLaunchKernelGGL(car_track_step_kernel, dim3(blocks), dim3(256), 0, device->stream, *p, M, states, actions, observations, next_observations, rewards, terminated, n_envs);
     return rlt_launch_status(device);
 }
 

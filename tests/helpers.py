@@ -907,3 +907,22 @@ def random_sequence_draws(rng, rings, sampling, max_episode_length, batch, seque
     nom = (rng.random((batch, sequence_length + 2)) < sampling.nominal_sequence_length_probability).astype(np.uint8)
     length = rng.integers(1, max(sequence_length, 2), (batch, sequence_length + 2)).astype(np.uint32)
     return env, off, nom, length
+
+
+def car_track_on_backend(backend, track, scale, states, actions, params=None):
+    """One step of n CarTrack environments on a backend: returns (next_states, observations [n x 9], next_observations [n x 9], rewards, terminated)."""
+    n = states.shape[0]
+    p = params if params is not None else capi.car_parameters()
+    t = backend.array(np.ascontiguousarray(track, np.uint8))
+    s, a = backend.array(states.astype(np.float32)), backend.array(actions.astype(np.float32))
+    o, no, r, term = backend.zeros((n, 9)), backend.zeros((n, 9)), backend.zeros((n,)), backend.zeros((n,), np.uint8)
+    backend.call("car_track_step", C.byref(p), t.ptr, track.shape[0], track.shape[1], float(np.float32(scale)), s.ptr, a.ptr, o.ptr, no.ptr, r.ptr, term.ptr, n)
+    backend.sync()
+    return s.numpy(), o.numpy(), no.numpy(), r.numpy(), term.numpy()
+
+
+def ring_track(height=80, width=120, inner=0.45, outer=0.85):
+    """A synthetic closed track: the cells between two ellipses around the centre of the bitmap are drivable."""
+    yy, xx = np.mgrid[0:height, 0:width]
+    rr = np.hypot((xx + 0.5 - width / 2) / (width / 2), (yy + 0.5 - height / 2) / (height / 2))
+    return ((rr > inner) & (rr < outer)).astype(np.uint8)

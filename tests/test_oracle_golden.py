@@ -400,3 +400,37 @@ def test_sequence_gather_reproduces_reference_vectors_and_invariants(oracle):
                     assert data[r, -1] == 0 and (r + 1) % cap != position       # not the end of an episode, not the cursor
                     r = (r + 1) % cap
                     s += 1
+
+
+def test_car_on_track_rays_and_flags_on_a_synthetic_track(oracle):
+    """CarTrack without the reference: on a straight corridor the three ray distances have closed forms (the ray leaves the corridor through a wall at
+    a known distance, in steps of half a cell), terminated says whether the next position is in a drivable cell, the reward is the forward speed, and
+    the step is the Car's. Cells beyond the bitmap count as not drivable."""
+    H, W, scale = 60, 200, 0.02
+    track = np.zeros((H, W), np.uint8)
+    track[20:40, :] = 1                                  # a corridor along x, 20 cells = 0.4 m wide, centred on y = 0
+    rng = np.random.default_rng(0)
+    n = 200
+    x = rng.uniform(-1.0, 1.0, n); y = rng.uniform(-0.15, 0.15, n)
+    states = np.stack([x, y, np.zeros(n), rng.uniform(0.1, 1, n), np.zeros(n), np.zeros(n)], 1).astype(np.float32)      # heading along +x
+    ns, o, no, r, t = helpers.car_track_on_backend(oracle, track, scale, states, np.zeros((n, 2), np.float32))
+    assert np.array_equal(r, states[:, 3]) and np.array_equal(o[:, :6], states)
+    assert np.array_equal(ns, helpers.car_on_backend(oracle, states, np.zeros((n, 2), np.float32))[0])
+    half = scale / 2
+    # straight ahead: the corridor runs to the end of the bitmap at x = +2.0, farther than the ray (50 half-cells = 0.5 m) unless the car is near it
+    free = np.minimum(np.floor((2.0 - states[:, 0].astype(np.float64)) / half - 1e-9) + 1, 50)
+    assert np.abs(o[:, 7] * 50 - free).max() <= 1
+    # 20 degrees to the left (+y): the wall at y = +0.2 is (0.2 - y) / sin(20 deg) away along the ray
+    ang = 20 / 180 * np.pi
+    left = np.minimum((0.2 - states[:, 1].astype(np.float64)) / np.sin(ang) / half, 50)
+    right = np.minimum((0.2 + states[:, 1].astype(np.float64)) / np.sin(ang) / half, 50)
+    assert np.abs(o[:, 8] * 50 - left).max() <= 1.5 and np.abs(o[:, 6] * 50 - right).max() <= 1.5
+    # terminated: the next position's cell
+    cx = np.floor((ns[:, 0].astype(np.float64) + scale * W / 2) / scale).astype(int); cy = np.floor((-ns[:, 1].astype(np.float64) + scale * H / 2) / scale).astype(int)
+    inside = (cx >= 0) & (cx < W) & (cy >= 0) & (cy < H)
+    want = np.ones(n, np.uint8); want[inside] = 1 - track[cy[inside], cx[inside]]
+    assert np.array_equal(t, want)
+    # off the bitmap: everything reads as not drivable
+    far = np.array([[5.0, 0.0, 0.0, 1.0, 0.0, 0.0], [0.0, -3.0, 1.0, 1.0, 0.0, 0.0]], np.float32)
+    _, o2, _, _, t2 = helpers.car_track_on_backend(oracle, track, scale, far, np.zeros((2, 2), np.float32))
+    assert np.all(o2[:, 6:] == 0) and np.all(t2 == 1)

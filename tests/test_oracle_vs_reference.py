@@ -250,6 +250,31 @@ def test_sequence_gather_bit_exact_with_reference(oracle):
     ref.lib.rlt_ref_gather_seq_destroy(ref.h)
 
 
+@pytest.mark.skipif(not os.path.exists(helpers.REF_ENVS_GENERIC), reason="environment flavour of oracle/_ref not built")
+def test_car_on_track_bit_exact_with_reference(oracle):
+    """CarTrack on the reference's default track (100 x 100 cells of 20 mm, read from the compiled reference at run time): the nine observations with the
+    three ray distances before and after the step, the step itself, reward = forward speed and terminated = off the track, on 50,000 random states
+    inside the bitmap, on and off the track."""
+    ref = C.CDLL(helpers.REF_ENVS_GENERIC)
+    P = C.c_void_p
+    ref.rlt_ref_car_track_steps.argtypes = [P, P, P, P, P, P, P, C.c_int]; ref.rlt_ref_car_track_bitmap.argtypes = [P]
+    track = np.zeros((100, 100), np.uint8)
+    ref.rlt_ref_car_track_bitmap(track.ctypes.data)
+    assert 1000 < track.sum() < 5000
+    rng = np.random.default_rng(3)
+    n = 50000
+    states = np.stack([rng.uniform(-0.95, 0.95, n), rng.uniform(-0.95, 0.95, n), rng.uniform(-4, 4, n), rng.uniform(-0.5, 3, n), rng.uniform(-1, 1, n), rng.uniform(-8, 8, n)], 1).astype(np.float32)
+    actions = rng.uniform(-1.3, 1.3, (n, 2)).astype(np.float32)
+    ns, o, no, r, t = np.zeros((n, 6), np.float32), np.zeros((n, 9), np.float32), np.zeros((n, 9), np.float32), np.zeros(n, np.float32), np.zeros(n, np.uint8)
+    assert ref.rlt_ref_car_track_steps(states.ctypes.data, actions.ctypes.data, ns.ctypes.data, o.ctypes.data, no.ctypes.data, r.ctypes.data, t.ctypes.data, n) == 0
+    got = helpers.car_track_on_backend(oracle, track, 20 / 1000.0, states, actions)
+    for w, g, name in zip((ns, o, no, r, t), got, ("next_states", "observations", "next_observations", "rewards", "terminated")):
+        assert np.array_equal(w, g), name
+    on_track = o[:, 7] > 0
+    assert 0.1 < on_track.mean() < 0.5 and 0 < t.sum() < n and np.array_equal(r, states[:, 3])
+    assert len(np.unique(o[on_track, 6:])) > 20 and o[:, 6:].max() <= 1.0          # many different ray lengths, as fractions of the full ray
+
+
 def test_small_ring_wraps_bit_exact_with_reference(oracle):
     """Replay capacity 250 (< 900 steps): the ring wraps three times, so `add` past the end, the prologue's wrap of the
     previous row, `full`, and gather's (position + MAX_EPISODE_LENGTH + offset) % CAPACITY index all run, and every
