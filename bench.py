@@ -212,8 +212,29 @@ def bench_ppo(helpers, rocm, n_envs=4096, steps=128, epochs=4, minibatch=8192):
     ms = ev.elapsed_ms(a, e)
     n_updates = epochs * (rows // minibatch)
     flop = 106368.0 * rows * epochs
+    # on-policy collection with the Pendulum: 4,096 environments x 128 steps (actor 3-64-64-1, standardized observations), one launch for all steps
+    pn, ps = 4096, 128
+    pcol = dict(observations=0, actions_mean=3, actions=4, action_log_probs=5, rewards=6, terminated=7, truncated=8, all_reset=9, all_values=10)
+    runner = helpers.OnPolicyOnBackend(rocm, pn, ps, 13, pcol, 200)
+    pdims = [3, 64, 64, 1]
+    pactor = helpers.Mlp(rocm, pdims, helpers.random_params(rng, pdims), pn, "relu", "tanh", trainable=False)
+    ls, nz = rocm.array(np.array([-0.5], np.float32)), rocm.array(rng.standard_normal((ps, pn, 1)).astype(np.float32))
+    ini = rocm.array(np.stack([rng.uniform(-np.pi, np.pi, (ps, pn)), rng.uniform(-1, 1, (ps, pn))], 2).astype(np.float32))
+    sm, sp = rocm.array(np.zeros(3, np.float32)), rocm.array(np.ones(3, np.float32))
+    wsn = rocm.device.lib.rlt_rocm_on_policy_collect_workspace_bytes(C.byref(runner.c), pactor.layers, pactor.n)
+    ws, wsn = rocm.workspace(wsn)
+
+    def collect():
+        rocm.call("on_policy_collect", C.byref(runner.c), C.byref(runner.d), pactor.layers, pactor.n, ls.ptr, sm.ptr, sp.ptr, nz.ptr, ini.ptr, 0, ws, wsn)
+    collect(); rocm.sync()
+    a = ev.record()
+    for _ in range(5):
+        collect()
+    e = ev.record()
+    collect_ms = ev.elapsed_ms(a, e) / 5
     return {"rows": rows, "minibatch": minibatch, "epochs": epochs, "gae_us": gae_us, "gae_algorithmic_GBps": rows * 24 / (gae_us * 1e-6) / 1e9,
-            "iteration_ms": ms, "us_per_minibatch_update": ms * 1e3 / n_updates, "samples_per_s": rows * epochs / (ms * 1e-3), "tflops": flop / (ms * 1e-3) / 1e12}
+            "iteration_ms": ms, "us_per_minibatch_update": ms * 1e3 / n_updates, "samples_per_s": rows * epochs / (ms * 1e-3), "tflops": flop / (ms * 1e-3) / 1e12,
+            "pendulum_collect": {"n_envs": pn, "steps": ps, "ms": collect_ms, "env_steps_per_s": pn * ps / (collect_ms * 1e-3)}}
 
 
 def bench_gru(helpers, rocm, batch, S=64, I=146, H=64, iters=10):
@@ -376,7 +397,7 @@ def cpu_baseline(batch=256, seconds=12.0):
                 if total >= seconds:
                     break
             lib.rlt_ref_sac_destroy(hdl)
-        return {"value": n / total, "unit": "loop steps/s", "cores": cores, "kind": "reference",
+        return {"value": n / total, "unit": "loop steps/s", "cores": cores, "kind": "reference", "cblas_path": lib.rlt_ref_cblas_name(),
                 "sample": f"{n} post-warm-up loop steps of the reference's Pendulum SAC loop at batch {batch}, CBLAS = {os.path.basename(lib.rlt_ref_cblas_name().decode())}, 1 thread"}
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import helpers
@@ -392,6 +413,65 @@ def cpu_baseline(batch=256, seconds=12.0):
         n += 50
     dt = time.perf_counter() - t0
     return {"value": n / dt, "unit": "loop steps/s", "cores": cores, "kind": "port", "sample": f"{n} loop steps of the CPU restatement (plain loops) at batch {batch}"}
+
+
+def cpu_other_configurations(helpers, cblas_path):
+    """The other configurations on this host's CPU, one thread, bounded samples (a few seconds in all): the CPU restatement with its three GEMMs per dense
+    layer routed through the same CBLAS the reference's CPU build uses (what its CPU_BLAS device does), or plain loops where no CBLAS was found."""
+    o = helpers.HostBackend()
+    capi = helpers.capi
+    blas = bool(cblas_path) and o.lib.rlt_oracle_use_cblas(cblas_path) == 0
+    out = {"kind": "port", "cores": 1, "gemm": os.path.basename(cblas_path.decode()) if blas else "plain loops"}
+    rng = np.random.default_rng(0)
+    try:
+        # configuration 1: MLP 17-256-256-6 forward + backward on a 4,096-row sample
+        B, dims = 4096, [17, 256, 256, 6]
+        net = helpers.Mlp(o, dims, helpers.xavier_params(rng, dims), B)
+        x, dy, y = o.array(rng.standard_normal((B, 17)).astype(np.float32)), o.array(rng.standard_normal((B, 6)).astype(np.float32)), o.zeros((B, 6))
+
+        def fwd_bwd():
+            o.call("mlp_forward_backward", net.layers, net.n, x.ptr, 17, y.ptr, 6, dy.ptr, 6, None, 0, 0.0, B, None, 0)
+        fwd_bwd()
+        t0 = time.perf_counter(); n = 0
+        while time.perf_counter() - t0 < 2.0:
+            fwd_bwd(); n += 1
+        dt = (time.perf_counter() - t0) / n
+        out["mlp_forward_backward"] = {"sample_rows": B, "ms": dt * 1e3, "tflops": (MLP_FLOP_PER_SAMPLE_FWD + MLP_FLOP_PER_SAMPLE_BWD) * B / dt / 1e12}
+        # configuration 3: one PPO minibatch update of 8,192 rows (observation 105, 8 actions, hidden 64, tanh)
+        O, A, H, B = 105, 8, 64, 8192
+        params = np.concatenate([helpers.random_params(rng, [O, H, H, A]) * 0.1, np.log(np.full(A, 0.5, np.float32)), helpers.random_params(rng, [O, H, H, 1])]).astype(np.float32)
+        agent = helpers.PpoOnBackend(o, O, A, H, H, B, params, "tanh", "tanh", capi.adam_parameters(3e-4, epsilon=1e-8))
+        ld = O + A + 7
+        data = rng.standard_normal((B, ld)).astype(np.float32)
+        data[:, O + A] = (-0.9189385 - np.log(0.5) - 0.5 * (data[:, O:O + A] / 0.5) ** 2).sum(1)
+        dd, pp = o.array(data), capi.ppo_parameters()
+
+        def update():
+            o.call("ppo_train_minibatch", C.byref(agent.c), C.byref(pp), dd.offset(0), dd.offset(0), dd.offset(O), dd.offset(O + A), dd.offset(O + A + 5), dd.offset(O + A + 6), ld, None, None)
+        update()
+        t0 = time.perf_counter(); n = 0
+        while time.perf_counter() - t0 < 2.0:
+            update(); n += 1
+        out["ppo_minibatch_update"] = {"rows": B, "us": (time.perf_counter() - t0) / n * 1e6}
+        # configuration 2: one runner step of 65,536 Pendulum environments (actor 3-64-64-1, replay add)
+        N = 65536
+        dims = [3, 64, 64, 1]
+        actor = helpers.Mlp(o, dims, helpers.xavier_params(rng, dims), N, "relu", "tanh", trainable=False)
+        rb = helpers.ReplayOnBackend(o, N, 16)
+        states, ep_step, ep_ret, trunc = o.zeros((N, 2)), o.zeros((N,), np.uint32), o.zeros((N,)), o.array(np.ones(N, np.uint8))
+        ini = o.array(np.stack([rng.uniform(-np.pi, np.pi, N), rng.uniform(-1, 1, N)], 1).astype(np.float32))
+        runner = capi.PendulumRunner(states.ptr, ep_step.ptr, ep_ret.ptr, trunc.ptr, N, 200, capi.pendulum_parameters())
+
+        def step():
+            assert o.lib.rlt_oracle_pendulum_runner_step(C.byref(runner), C.byref(rb.c), 1, actor.layers, actor.n, None, None, None, ini.ptr) == 0
+        step()
+        t0 = time.perf_counter(); n = 0
+        while time.perf_counter() - t0 < 2.0:
+            step(); n += 1
+        out["runner_step"] = {"n_envs": N, "us": (time.perf_counter() - t0) / n * 1e6}
+    finally:
+        o.lib.rlt_oracle_use_cblas(None)
+    return out
 
 
 def main():
@@ -451,6 +531,9 @@ def main():
     if cpu:
         line["cpu_baseline"] = cpu
         line["speedup_vs_cpu_baseline"] = sac["steps_per_s"] / cpu["value"] if cpu["value"] else None
+        line["cpu_other_configurations"] = cpu_other_configurations(helpers, cpu.get("cblas_path"))
+    if cpu:
+        cpu.pop("cblas_path", None)
     print(json.dumps(line), flush=True)
     rocm.close()
 

@@ -2,6 +2,7 @@
 // reference: rl/components/replay_buffer/operations_generic.h:54-78, rl/components/off_policy_runner/operations_generic.h:183-430
 //            (CUDA :14-230), operations_generic_per_env.h:8-108, rl/environments/pendulum/operations_generic.h:14-160.
 #include "common.h"
+#include <cstdlib>
 
 namespace {
 
@@ -440,6 +441,124 @@ __global__ __launch_bounds__(256) void on_policy_epilogue_kernel(rlt_pendulum_ru
     }
 }
 
+// The whole collection in one launch for 3 -> 64 -> 64 -> 1 actors: the environments do not interact, so a wavefront takes 16 of them through all the
+// steps (prologue, standardize, actor on v_mfma_f32_16x16x4_f32 with W2 in registers, epilogue; the same arithmetic as the per-step kernels above), with
+// the environment state in the registers of the 16 owning lanes between steps. Bound by the chain of steps_per_env dependent steps per wavefront.
+struct CollectArgs {
+    rlt_pendulum_runner rn; rlt_on_policy_dataset D;
+    const float *w1, *b1, *w2, *b2, *w3, *b3;
+    int act_out, force_truncated;
+    const float* log_std; const float* standardize_mean; const float* standardize_precision; const float* action_noise; const float* initial_states;
+};
+constexpr int CWAVES = 4, COLLECT_LDS_PER_WAVE = 16 * FAS + 16 * 4 + 16;
+template <int ACT_H>
+__global__ __launch_bounds__(64 * CWAVES) void on_policy_collect_kernel(CollectArgs A) {
+    __shared__ float lds[CWAVES * COLLECT_LDS_PER_WAVE + FH * FAS];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, kk = lane >> 4;
+    const lptr hs = (lptr)lds + wave * COLLECT_LDS_PER_WAVE, xs = hs + 16 * FAS, ys = xs + 16 * 4, w2s = (lptr)lds + CWAVES * COLLECT_LDS_PER_WAVE;
+    for (int i = threadIdx.x; i < FH * FH; i += 64 * CWAVES) w2s[(i >> 6) * FAS + (i & 63)] = A.w2[i];
+    __syncthreads();
+    float w1r[4], b1r[4], w2r[4][16], b2r[4], w3r[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+        const int n = 16 * nt + r;
+        w1r[nt] = kk < 3 ? A.w1[n * 3 + kk] : 0.f; b1r[nt] = A.b1[n]; b2r[nt] = A.b2[n]; w3r[nt] = A.w3[n];
+#pragma unroll
+        for (int q = 0; q < 16; q++) w2r[nt][q] = w2s[n * FAS + kk * 16 + q];
+    }
+    const float b3 = A.b3[0], ls = A.log_std[0], sd = expf(ls);
+    float sm[3] = {0.f, 0.f, 0.f}, sp[3] = {0.f, 0.f, 0.f};
+    if (A.standardize_mean) for (int c = 0; c < 3; c++) { sm[c] = A.standardize_mean[c]; sp[c] = A.standardize_precision[c]; }
+    const int N = A.rn.n_envs, S = A.D.steps_per_env, n_tiles = (N + 15) / 16;
+    const size_t ld = A.D.ld;
+    for (int tile = blockIdx.x * CWAVES + wave; tile < n_tiles; tile += gridDim.x * CWAVES) {
+        const int e = tile * 16 + lane;
+        const bool live = lane < 16 && e < N;
+        float th = 0.f, thd = 0.f, ep_ret = 0.f; uint32_t ep_step = 0; bool trunc = false;
+        if (live) { th = A.rn.states[2 * e]; thd = A.rn.states[2 * e + 1]; ep_ret = A.rn.episode_return[e]; ep_step = A.rn.episode_step[e]; trunc = A.rn.truncated[e] != 0; }
+        for (int step = 0; step < S; step++) {
+            const size_t row = (size_t)step * N + e;
+            if (live) {         // prologue (operations_generic_per_env.h:8-35): reset where truncated, observe into the dataset row of this step
+                const bool truncated = trunc || (step == 0 && A.force_truncated);
+                if (step == 0) A.D.all_reset[(size_t)e * ld] = truncated ? 1.0f : 0.0f;
+                if (truncated) { trunc = false; ep_step = 0; ep_ret = 0.0f; th = A.initial_states[2 * row]; thd = A.initial_states[2 * row + 1]; }
+                float sn, cs;
+                sincosf(th, &sn, &cs);
+                float* o = A.D.observations + row * ld;
+                o[0] = cs; o[1] = sn; o[2] = thd;
+                float x[3] = {cs, sn, thd};
+                if (A.standardize_mean) {
+#pragma unroll
+                    for (int c = 0; c < 3; c++) { x[c] -= sm[c]; if (sp[c] != 0.0f) x[c] *= sp[c]; }
+                }
+                xs[lane * 4] = x[0]; xs[lane * 4 + 1] = x[1]; xs[lane * 4 + 2] = x[2]; xs[lane * 4 + 3] = 0.f;
+            } else if (lane < 16) { xs[lane * 4] = 0.f; xs[lane * 4 + 1] = 0.f; xs[lane * 4 + 2] = 0.f; xs[lane * 4 + 3] = 0.f; }
+            __builtin_amdgcn_wave_barrier();
+            {   // layer 1
+                const float xa = xs[r * 4 + kk];
+#pragma unroll
+                for (int nt = 0; nt < 4; nt++) {
+                    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                    const floatx4 acc = mfma16(xa, w1r[nt], zero);
+#pragma unroll
+                    for (int v = 0; v < 4; v++) hs[(4 * kk + v) * FAS + 16 * nt + r] = rlt_act(acc[v] + b1r[nt], ACT_H);
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+            {   // layer 2, and layer 3 as partial dot products over this lane's hidden units
+                float a[16];
+#pragma unroll
+                for (int q = 0; q < 16; q++) a[q] = hs[r * FAS + kk * 16 + q];
+                float p[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int nt = 0; nt < 4; nt++) {
+                    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int q = 0; q < 16; q++) acc = mfma16(a[q], w2r[nt][q], acc);
+#pragma unroll
+                    for (int v = 0; v < 4; v++) p[v] += rlt_act(acc[v] + b2r[nt], ACT_H) * w3r[nt];
+                }
+#pragma unroll
+                for (int v = 0; v < 4; v++) { const float sum = row16_sum(p[v]); if (r == v) ys[4 * kk + v] = sum; }
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (live) {         // epilogue (:36-74): sample around the mean, log-probability (random/operations_generic.h:73-81), step, reward, flags
+                const float mean = rlt_act(ys[lane] + b3, A.act_out);
+                const float action = mul_add_rn(A.action_noise[row], sd, mean);
+                const float pre = (action - mean) / sd;
+                A.D.actions_mean[row * ld] = mean;
+                A.D.actions[row * ld] = action;
+                A.D.action_log_probs[row * ld] = (-0.9189385332046727f - ls) - 0.5f * pre * pre;
+                Transition t;
+                pendulum_transition(A.rn.env, th, thd, action, t);
+                A.D.terminated[row * ld] = 0.0f;
+                A.D.rewards[row * ld] = t.reward;
+                ep_ret += t.reward;
+                ep_step += 1;
+                const bool truncated = A.rn.episode_step_limit > 0 && ep_step >= (uint32_t)A.rn.episode_step_limit;
+                A.D.truncated[row * ld] = truncated ? 1.0f : 0.0f;
+                A.D.all_reset[(row + N) * ld] = truncated ? 1.0f : 0.0f;
+                trunc = truncated;
+                th = t.theta; thd = t.theta_dot;
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (live) {             // the observation after the last step, and the runner's state
+            float sn, cs;
+            sincosf(th, &sn, &cs);
+            float* o = A.D.observations + ((size_t)S * N + e) * ld;
+            o[0] = cs; o[1] = sn; o[2] = thd;
+            A.rn.states[2 * e] = th; A.rn.states[2 * e + 1] = thd; A.rn.episode_return[e] = ep_ret; A.rn.episode_step[e] = ep_step; A.rn.truncated[e] = trunc;
+        }
+    }
+}
+// RLT_COLLECT_ONE_LAUNCH=0 keeps the collection on the per-step kernels (tests compare the two paths with each other)
+bool collect_one_launch_enabled() { const char* v = std::getenv("RLT_COLLECT_ONE_LAUNCH"); return !(v && v[0] == '0'); }
+bool fused_collect_ok(const rlt_dense_layer* L, int n) {
+    return n == 3 && L[0].in_dim == 3 && L[0].out_dim == FH && L[1].in_dim == FH && L[1].out_dim == FH && L[2].in_dim == FH && L[2].out_dim == 1 &&
+           L[0].activation == L[1].activation;
+}
+
 int grid1(int n) { int b = (n + 255) / 256; return b > 2048 ? 2048 : (b < 1 ? 1 : b); }
 // the shapes the one-launch step is built for
 bool fused_runner_ok(const rlt_dense_layer* L, int n, int policy_kind, const rlt_replay_buffer* rb, const rlt_pendulum_runner* rn, const float* initial_states) {
@@ -633,6 +752,23 @@ int rlt_rocm_on_policy_collect(rlt_rocm_device* device, const rlt_pendulum_runne
     RLT_REQUIRE((standardize_mean == nullptr) == (standardize_precision == nullptr));
     RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_on_policy_collect_workspace_bytes(rn, actor, n_actor_layers));
     const int N = rn->n_envs;
+    if (fused_collect_ok(actor, n_actor_layers) && collect_one_launch_enabled()) {
+        CollectArgs a = {};
+        a.rn = *rn; a.D = *D;
+        a.w1 = actor[0].weights; a.b1 = actor[0].biases; a.w2 = actor[1].weights; a.b2 = actor[1].biases; a.w3 = actor[2].weights; a.b3 = actor[2].biases;
+        a.act_out = actor[2].activation; a.force_truncated = truncate_on_each_iteration;
+        a.log_std = log_std; a.standardize_mean = standardize_mean; a.standardize_precision = standardize_precision; a.action_noise = action_noise; a.initial_states = initial_states;
+        int blocks = rlt_div_up(rlt_div_up(N, 16), CWAVES); if (blocks > device->compute_units) blocks = device->compute_units;
+        switch (actor[0].activation) {
+            case RLT_ACT_RELU: hipLaunchKernelGGL(on_policy_collect_kernel<RLT_ACT_RELU>, dim3(blocks), dim3(64 * CWAVES), 0, device->stream, a); break;
+            case RLT_ACT_TANH: hipLaunchKernelGGL(on_policy_collect_kernel<RLT_ACT_TANH>, dim3(blocks), dim3(64 * CWAVES), 0, device->stream, a); break;
+            case RLT_ACT_FAST_TANH: hipLaunchKernelGGL(on_policy_collect_kernel<RLT_ACT_FAST_TANH>, dim3(blocks), dim3(64 * CWAVES), 0, device->stream, a); break;
+            case RLT_ACT_GELU: hipLaunchKernelGGL(on_policy_collect_kernel<RLT_ACT_GELU>, dim3(blocks), dim3(64 * CWAVES), 0, device->stream, a); break;
+            case RLT_ACT_SIGMOID: hipLaunchKernelGGL(on_policy_collect_kernel<RLT_ACT_SIGMOID>, dim3(blocks), dim3(64 * CWAVES), 0, device->stream, a); break;
+            default: hipLaunchKernelGGL(on_policy_collect_kernel<RLT_ACT_IDENTITY>, dim3(blocks), dim3(64 * CWAVES), 0, device->stream, a); break;
+        }
+        return rlt_launch_status(device);
+    }
     float* standardized = reinterpret_cast<float*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
     const size_t head = ((size_t)N * 3 * sizeof(float) + 255) & ~(size_t)255;
     void* ws = (char*)standardized + head;

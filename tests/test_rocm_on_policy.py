@@ -16,14 +16,14 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-5
 
 
-def compare_datasets(got, want, col, n, S):
+def compare_datasets(got, want, col, n, S, tol=TOL):
     rows = n * S
     for name in ("terminated", "truncated"):
         assert np.array_equal(got[:rows, col[name]], want[:rows, col[name]]), name
     assert np.array_equal(got[:rows + n, col["all_reset"]], want[:rows + n, col["all_reset"]])
     for name, nrows, w in (("observations", rows + n, 3), ("actions_mean", rows, 1), ("actions", rows, 1), ("action_log_probs", rows, 1), ("rewards", rows, 1)):
         e = rel_err(got[:nrows, col[name]:col[name] + w], want[:nrows, col[name]:col[name] + w])
-        assert e <= TOL, (name, e)
+        assert e <= tol, (name, e)
 
 
 def test_collect_matches_the_references_vectors(rocm):
@@ -40,7 +40,8 @@ def test_collect_matches_the_references_vectors(rocm):
         assert rel_err(rs["states"], g[f"c{k}_after_states"]) <= TOL and rel_err(rs["episode_return"], g[f"c{k}_after_episode_return"]) <= TOL
 
 
-@pytest.mark.parametrize("n,S,hidden,limit,standardize,force", [(4096, 16, 64, 7, True, 0), (1000, 5, 32, 0, False, 1), (3, 30, 16, 4, True, 0)])
+@pytest.mark.parametrize("n,S,hidden,limit,standardize,force", [(4096, 16, 64, 7, True, 0), (1000, 5, 32, 0, False, 1), (3, 30, 16, 4, True, 0), (1000, 40, 64, 0, False, 1),
+                                                                (17, 64, 64, 9, True, 0)])
 def test_collect_matches_checker_at_other_sizes(oracle, rocm, n, S, hidden, limit, standardize, force):
     """Wider cases against the checker: 4,096 environments, no step limit, truncate-on-each-iteration, tiny batches; environments start
     from a mixed state (some mid-episode, some flagged for reset)."""
@@ -64,9 +65,11 @@ def test_collect_matches_checker_at_other_sizes(oracle, rocm, n, S, hidden, limi
         o.collect(actor, log_std, noise, ini, standardize=st, truncate_on_each_iteration=force)
         out[b.name] = (o.data.numpy(), o.runner_state())
     (got, grs), (want, wrs) = out["rocm"], out["oracle"]
-    compare_datasets(got, want, col, n, S)
+    # episodes that run for 40 steps without a reset let rounding differences grow along the closed loop: 5e-5 there
+    tol = 5e-5 if (limit == 0 and S >= 40) else TOL
+    compare_datasets(got, want, col, n, S, tol)
     assert np.array_equal(grs["episode_step"], wrs["episode_step"]) and np.array_equal(grs["truncated"], wrs["truncated"])
-    assert rel_err(grs["states"], wrs["states"]) <= TOL and rel_err(grs["episode_return"], wrs["episode_return"]) <= TOL
+    assert rel_err(grs["states"], wrs["states"]) <= tol and rel_err(grs["episode_return"], wrs["episode_return"]) <= tol
     if force:
         assert want[:n, col["all_reset"]].all()
 
@@ -100,3 +103,31 @@ def test_running_normaliser_and_standardize_match_checker(oracle, rocm, rows, di
         tol = max(TOL, rows * 2.0 ** -24) if k in ("mean", "std", "lm", "lp", "y", "dx") else TOL
         e = rel_err(got[k], want[k])
         assert e <= tol, (k, e)
+
+
+def test_one_launch_collection_against_per_step_kernels(rocm, monkeypatch):
+    """3 -> 64 -> 64 -> 1 actors are collected in one launch for all steps; the same collection kept on the per-step kernels (the path of other actor
+    shapes, checked against the checker above) must give the same dataset: 4,096 environments x 128 steps, episodes of 25 steps."""
+    n, S, limit = 4096, 128, 25
+    rng = np.random.default_rng(5)
+    col = dict(observations=0, actions_mean=3, actions=4, action_log_probs=5, rewards=6, terminated=7, truncated=8, all_reset=9, all_values=10)
+    ld = 13
+    dims = [3, 64, 64, 1]
+    params = helpers.random_params(rng, dims)
+    log_std = np.array([-0.5], np.float32)
+    st = (rng.standard_normal(3).astype(np.float32) * 0.2, (1.0 / (0.5 + rng.random(3))).astype(np.float32))
+    before = dict(states=np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n)], 1).astype(np.float32), episode_step=rng.integers(0, limit, n).astype(np.uint32),
+                  episode_return=rng.standard_normal(n).astype(np.float32), truncated=(rng.random(n) < 0.3).astype(np.uint8))
+    noise = rng.standard_normal((S, n, 1)).astype(np.float32)
+    ini = np.stack([rng.uniform(-np.pi, np.pi, (S, n)), rng.uniform(-1, 1, (S, n))], 2).astype(np.float32)
+    out = []
+    for flag in ("1", "0"):
+        monkeypatch.setenv("RLT_COLLECT_ONE_LAUNCH", flag)
+        o = helpers.OnPolicyOnBackend(rocm, n, S, ld, col, limit, before)
+        actor = helpers.Mlp(rocm, dims, params, n, "relu", "tanh", trainable=False)
+        o.collect(actor, log_std, noise, ini, standardize=st)
+        out.append((o.data.numpy(), o.runner_state()))
+    (got, grs), (want, wrs) = out
+    compare_datasets(got, want, col, n, S)
+    assert np.array_equal(grs["episode_step"], wrs["episode_step"]) and np.array_equal(grs["truncated"], wrs["truncated"])
+    assert rel_err(grs["states"], wrs["states"]) <= TOL and rel_err(grs["episode_return"], wrs["episode_return"]) <= TOL
