@@ -83,7 +83,7 @@ int rlt_rocm_fill_u8(rlt_rocm_device* device, uint8_t* dst, size_t count, uint8_
  * values is a pure function of (seed, offset, element index), no state array is needed) */
 int rlt_rocm_randn_f32(rlt_rocm_device* device, float* dst, size_t count, uint64_t seed, uint64_t offset);
 int rlt_rocm_rand_f32(rlt_rocm_device* device, float* dst, size_t count, float low, float high, uint64_t seed, uint64_t offset);
-/* scale(t, s, reciprocal) containers/tensor/operations_generic.h:433-445,713 : x <- reciprocal ? s/x : s*x */
+/* scale(t, s, reciprocal) containers/tensor/operations_generic.h:433-445,713 : x <- reciprocal ? (1/x)*s : x*s (rounded in that order) */
 int rlt_rocm_scale_f32(rlt_rocm_device* device, float* x, size_t count, float s, int reciprocal);
 /* cast_reduce_sum<T>(bool tensor) containers/tensor/operations_generic.h:928-985 (CUDA: <<<1,1>>>, operations_cuda.h:287-307) */
 int rlt_rocm_cast_reduce_sum_u8(rlt_rocm_device* device, const uint8_t* mask, size_t count, float* out_sum);
@@ -575,8 +575,11 @@ int rlt_rocm_ppo_train_epoch(rlt_rocm_device* device, const rlt_ppo_agent* agent
 /* --------------------------------------------------------------------- GRU -- */
 
 /* nn/layers/gru/layer.h:96-217 (LayerForward / LayerBackward / LayerGradient): gate order r, z, n along the 3H rows
- * (the layout of torch.nn.GRU); LEARN_INITIAL_HIDDEN_STATE = false and FAST_TANH = false as in the reference's
- * configuration default (layer.h:14-24). Tensors are [sequence x batch x features], row-major. */
+ * (the layout of torch.nn.GRU); LEARN_INITIAL_HIDDEN_STATE = false as in the reference's configuration (layer.h:14-24).
+ * fast_tanh selects the reference's FAST_TANH switch (layer.h:12,18; operations_generic.h:302-320): the gates then use
+ * math::fast_sigmoid / math::fast_tanh (math/operations_generic.h:247-255) in the forward pass, while the backward pass
+ * keeps the derivative formulas of the exact functions on the stored outputs; the reference's SAC / TD3 GRU approximators
+ * set it (rl/algorithms/sac/loop/core/approximators_gru.h:18). Tensors are [sequence x batch x features], row-major. */
 typedef struct rlt_gru_layer {
     float* weights_input;          /* [3H x I] */
     float* biases_input;           /* [3H] */
@@ -588,6 +591,7 @@ typedef struct rlt_gru_layer {
     float* n_pre_pre_activation;   /* [S x B x H]  W_hn h + b_hn */
     float* output;                 /* [S x B x H]  hidden state of every step */
     int input_dim, hidden_dim;
+    int fast_tanh, reserved;
 } rlt_gru_layer;
 
 size_t rlt_rocm_gru_workspace_bytes(const rlt_gru_layer* layer, int sequence_length, int batch);
@@ -602,6 +606,85 @@ int rlt_rocm_gru_forward(rlt_rocm_device* device, const rlt_gru_layer* layer, co
 int rlt_rocm_gru_backward(rlt_rocm_device* device, const rlt_gru_layer* layer, const float* input, float* d_output,
                           float* d_input, const uint8_t* reset, int sequence_length, int batch, int want_weight_gradients,
                           void* workspace, size_t workspace_bytes);
+
+/* ------------------------------------- SAC on sequence batches (recurrent) -- */
+
+/* One layer of a sequential model (nn_models/sequential/model.h:196-215 holds `content` and `next_module`): a dense layer,
+ * applied to all steps x batch rows at once, or a GRU layer. The reference's recurrent approximators
+ * (rl/algorithms/sac/loop/core/approximators_gru.h:13-74) are dense -> GRU [-> GRU] [-> dense] -> dense, for the actor
+ * followed by the sample_and_squash layer, which lives in the agent below. The kept intermediates of every layer
+ * (dense: pre_activations / output; GRU: post_activation / n_pre_pre_activation / output) hold steps x batch rows, with
+ * steps = sequence_length + 1 where the network is also evaluated on the `next` views. */
+typedef struct rlt_seq_layer {
+    int32_t kind;                /* 0 dense, 1 GRU */
+    int32_t reserved;
+    rlt_dense_layer dense;
+    rlt_gru_layer gru;
+} rlt_seq_layer;
+
+/* forward / evaluate of a sequential model   nn_models/sequential/operations_generic.h:277-347
+ *   x [steps x batch x in] with leading dimension ldx (a GRU as first layer needs ldx = in); reset [steps x batch] or NULL
+ *   (the ResetMode of nn/layers/gru/layer.h:56-68, handed to every layer); every layer keeps its intermediates, the result
+ *   is the last layer's output. */
+int rlt_rocm_seq_forward(rlt_rocm_device* device, const rlt_seq_layer* layers, int n_layers, const float* x, int ldx,
+                         const uint8_t* reset, int steps, int batch, void* workspace, size_t workspace_bytes);
+/* backward / backward_full / backward_input of a sequential model   nn_models/sequential/operations_generic.h:369-428
+ *   d_output [steps x batch x out] packed, modified (every layer leaves its d_pre / accumulated hidden-state gradient in
+ *   the buffer it was handed, as in the reference); d_input [steps x batch x in] packed or NULL;
+ *   want_weight_gradients = 0 -> backward_input. The reference's backward_input hands the mode only to a model's first
+ *   layer when that layer is also its last (operations_generic.h:399-407 call the inner layers without it), so in a deeper
+ *   model the GRU layers run their backward_input as if no step had been a reset; reset_in_backward_input = 0 reproduces
+ *   that, 1 hands the resets to every layer. Ignored when want_weight_gradients != 0 (those paths pass the mode on). */
+int rlt_rocm_seq_backward(rlt_rocm_device* device, const rlt_seq_layer* layers, int n_layers, const float* x, int ldx,
+                          float* d_output, float* d_input, const uint8_t* reset, int steps, int batch,
+                          int want_weight_gradients, int reset_in_backward_input, void* workspace, size_t workspace_bytes);
+int rlt_rocm_seq_zero_gradient(rlt_rocm_device* device, const rlt_seq_layer* layers, int n_layers);
+size_t rlt_rocm_seq_workspace_bytes(const rlt_seq_layer* layers, int n_layers, int steps, int batch);
+
+/* Everything one SAC agent with sequential (recurrent) networks owns on the device: rl/algorithms/sac/sac.h:62-145 for
+ * SEQUENCE_LENGTH >= 1 and the batch of rl/components/off_policy_runner/off_policy_runner.h:102-156 as
+ * rlt_rocm_gather_sequence_batch fills it. S = batch.sequence_length, B = batch.batch, T = S + 1 if
+ * include_first_step_in_targets (then the `next` views start at padded step 0) else S (they start at step 1). */
+typedef struct rlt_sac_sequence_agent {
+    int32_t observation_dim, action_dim, n_actor_layers, n_critic_layers;
+    int32_t include_first_step_in_targets, reserved0;
+    float gamma, polyak;
+    rlt_sas_parameters sas;
+    rlt_adam_parameters actor_adam, critic_adam, alpha_adam;
+    const rlt_seq_layer* actor;              /* last layer: out_dim = 2 * action_dim, intermediates for T x B rows */
+    const rlt_seq_layer* critics[2];         /* intermediates for S x B rows */
+    const rlt_seq_layer* critics_target[2];  /* intermediates for T x B rows */
+    const rlt_adam_tensor* actor_adam_tensors;      int32_t n_actor_adam_tensors;   int32_t pad0;
+    const rlt_adam_tensor* critic_adam_tensors[2];  int32_t n_critic_adam_tensors;  int32_t pad1;
+    rlt_adam_tensor log_alpha;               /* count = 1 */
+    uint32_t* actor_age; uint32_t* critic_age[2]; uint32_t* alpha_age;
+    rlt_sequence_batch batch;
+    /* training buffers (sac.h:73-131) */
+    float* next_state_action_value_input;    /* [T x B x (obs + act)] */
+    float* next_q[2];                        /* [T x B] */
+    float* next_log_probabilities;           /* [T x B] */
+    float* target_action_value;              /* [S x B] */
+    float* d_output;                         /* [S x B] */
+    float* state_action_value_input;         /* [S x B x (obs + act)] */
+    float* d_critic_input[2];                /* [S x B x (obs + act)] */
+    float* d_actor_output_squashing;         /* [S x B x act] */
+    float* d_actor_output;                   /* [S x B x 2 act] */
+    float* actor_actions;                    /* [T x B x act] sample_and_squash output */
+    float* actor_pre_squashing;              /* [S x B x act] */
+    float* actor_log_probabilities;          /* [S x B] */
+    void* workspace; size_t workspace_bytes; /* >= rlt_rocm_sac_sequence_workspace_bytes */
+} rlt_sac_sequence_agent;
+
+size_t rlt_rocm_sac_sequence_workspace_bytes(const rlt_sac_sequence_agent* agent);
+/* train_critic on a sequence batch   rl/algorithms/sac/operations_generic.h:243-337
+ *   action_noise [T x B x action_dim]: the N(0,1) noise of the actor's sample_and_squash layer on the `next` views.
+ *   As in the reference, the target of step t takes the target critics' value of step t + 1 but the entropy bonus from the
+ *   log-probability at index t of the evaluated `next` steps (operations_generic.h:144-154). */
+int rlt_rocm_sac_sequence_train_critic(rlt_rocm_device* device, const rlt_sac_sequence_agent* agent, int critic_index, const float* action_noise);
+/* update_critic_targets   sac/operations_generic.h:486-527 (dense and GRU layers, incl. the initial hidden state) */
+int rlt_rocm_sac_sequence_update_critic_targets(rlt_rocm_device* device, const rlt_sac_sequence_agent* agent);
+/* train_actor on a sequence batch   sac/operations_generic.h:395-468; action_noise [S x B x action_dim] */
+int rlt_rocm_sac_sequence_train_actor(rlt_rocm_device* device, const rlt_sac_sequence_agent* agent, const float* action_noise);
 
 /* --------------------------------------------------------------------- TD3 -- */
 

@@ -18,7 +18,11 @@ using TI = typename DEVICE::index_t;
 constexpr TI S = 7, B = 5, I = 6, H = 8;
 using CAPABILITY = rlt::nn::capability::Gradient<rlt::nn::parameters::Adam>;
 using INPUT_SHAPE = rlt::tensor::Shape<TI, S, B, I>;
+#ifdef RLT_REF_GRU_FAST_TANH   // the switch the reference's SAC / TD3 GRU approximators set
+using GRU_CONFIG = rlt::nn::layers::gru::Configuration<TYPE_POLICY, TI, H, rlt::nn::parameters::groups::Normal, true>;
+#else
 using GRU_CONFIG = rlt::nn::layers::gru::Configuration<TYPE_POLICY, TI, H>;
+#endif
 using GRU = rlt::nn::layers::gru::Layer<GRU_CONFIG, CAPABILITY, INPUT_SHAPE>;
 using RESET = rlt::Tensor<rlt::tensor::Specification<bool, TI, rlt::tensor::Shape<TI, S, B, 1>>>;
 using RESET_MODE_SPEC = rlt::nn::layers::gru::ResetModeSpecification<TI, RESET>;

@@ -396,10 +396,10 @@ int rlt_oracle_sas_forward(const rlt_sas_parameters* p, const float* input, int 
     return 0;
 }
 // nn/layers/sample_and_squash/operations_generic.h:289-398
-int rlt_oracle_sas_backward(const rlt_sas_parameters* p, const float* input, int ldin, const float* noise, int ldn,
+static int sas_backward_impl(const rlt_sas_parameters* p, const float* input, int ldin, const float* noise, int ldn,
                             const float* actions, int lda, const float* pre_squashing, int ldp,
                             const float* d_output, int lddo, float* d_input, int lddi,
-                            const float* log_alpha, float* d_log_alpha, int batch, int dim) {
+                            const float* log_alpha, float* d_log_alpha, int batch, int dim, float divisor) {
     if (!p || !input || !noise || !actions || !pre_squashing || !d_output || !d_input || !log_alpha || batch <= 0 || dim <= 0) return RLT_E_INVALID_ARGUMENT;
     float alpha = std::exp(*log_alpha);
     float d_log_alpha_sum = 0;
@@ -433,8 +433,24 @@ int rlt_oracle_sas_backward(const rlt_sas_parameters* p, const float* input, int
         float d_alpha = entropy - p->target_entropy;
         d_log_alpha_sum += alpha * d_alpha;
     }
-    if (d_log_alpha) *d_log_alpha += d_log_alpha_sum / batch;
+    if (d_log_alpha) *d_log_alpha += d_log_alpha_sum / divisor;
     return 0;
+}
+int rlt_oracle_sas_backward(const rlt_sas_parameters* p, const float* input, int ldin, const float* noise, int ldn,
+                            const float* actions, int lda, const float* pre_squashing, int ldp,
+                            const float* d_output, int lddo, float* d_input, int lddi,
+                            const float* log_alpha, float* d_log_alpha, int batch, int dim) {
+    return sas_backward_impl(p, input, ldin, noise, ldn, actions, lda, pre_squashing, ldp, d_output, lddo, d_input, lddi, log_alpha, d_log_alpha, batch, dim, (float)batch);
+}
+// the same under a ResetMode (:390-394): the sum over the rows is divided by the number of set reset flags (an integer count) instead of the row count
+int rlt_oracle_sas_backward_reset(const rlt_sas_parameters* p, const float* input, int ldin, const float* noise, int ldn,
+                                  const float* actions, int lda, const float* pre_squashing, int ldp,
+                                  const float* d_output, int lddo, float* d_input, int lddi,
+                                  const float* log_alpha, float* d_log_alpha, const uint8_t* reset, int batch, int dim) {
+    if (!reset) return RLT_E_INVALID_ARGUMENT;
+    size_t n = 0;
+    for (int i = 0; i < batch; i++) n += reset[i] != 0;
+    return sas_backward_impl(p, input, ldin, noise, ldn, actions, lda, pre_squashing, ldp, d_output, lddo, d_input, lddi, log_alpha, d_log_alpha, batch, dim, (float)n);
 }
 
 // rl/algorithms/sac/operations_generic.h:133-179
@@ -486,7 +502,7 @@ int rlt_oracle_mask_zero(float* gradient, int ld, const uint8_t* mask, int inver
 // containers/tensor/operations_generic.h:433-445
 int rlt_oracle_scale_f32(float* x, size_t count, float s, int reciprocal) {
     if (!x) return RLT_E_INVALID_ARGUMENT;
-    for (size_t i = 0; i < count; i++) x[i] = reciprocal ? s / x[i] : s * x[i];
+    for (size_t i = 0; i < count; i++) x[i] = reciprocal ? (1.0f / x[i]) * s : x[i] * s;   // containers/tensor/operations_generic.h:437-443: the reciprocal first, then the scale
     return 0;
 }
 // containers/tensor/operations_generic.h:928-985 (CastSum)
@@ -586,11 +602,11 @@ int rlt_oracle_sac_train_actor(const rlt_sac_agent* A, const float* action_noise
     if ((rc = rlt_oracle_sac_min_value_d_output(q1, q2, A->d_critic_input[0], A->d_critic_input[1], D, D, ACT, A->d_actor_output_squashing, ACT, B))) return rc; // :460
     if (A->final_step_mask) rlt_oracle_mask_zero(A->d_actor_output_squashing, ACT, A->final_step_mask, 1, B, ACT);           // :461-463
     // sequential backward: sample_and_squash backward_full (divides d_log_alpha by num_resets = sum(reset)), then MLP backward (:464)
-    float d_log_alpha_mean = 0;
-    if ((rc = rlt_oracle_sas_backward(&A->sas, actor_out, 2 * ACT, action_noise, ACT, A->actor_actions, ACT, A->actor_pre_squashing, ACT,
-                                      A->d_actor_output_squashing, ACT, A->d_actor_output, 2 * ACT, A->log_alpha.parameters, &d_log_alpha_mean, B, ACT))) return rc;
-    if (A->reset) { float n = 0; rlt_oracle_cast_reduce_sum_u8(A->reset, B, &n); d_log_alpha_mean = d_log_alpha_mean * B / n; }
-    A->log_alpha.gradient[0] += d_log_alpha_mean;
+    if (A->reset) rc = rlt_oracle_sas_backward_reset(&A->sas, actor_out, 2 * ACT, action_noise, ACT, A->actor_actions, ACT, A->actor_pre_squashing, ACT,
+                                                     A->d_actor_output_squashing, ACT, A->d_actor_output, 2 * ACT, A->log_alpha.parameters, &A->log_alpha.gradient[0], A->reset, B, ACT);
+    else rc = rlt_oracle_sas_backward(&A->sas, actor_out, 2 * ACT, action_noise, ACT, A->actor_actions, ACT, A->actor_pre_squashing, ACT,
+                                      A->d_actor_output_squashing, ACT, A->d_actor_output, 2 * ACT, A->log_alpha.parameters, &A->log_alpha.gradient[0], B, ACT);
+    if (rc) return rc;
     if ((rc = rlt_oracle_mlp_backward(A->actor, A->n_actor_layers, obs, D, A->d_actor_output, 2 * ACT, nullptr, 0, B, 1))) return rc;
     if ((rc = adam_over(A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age))) return rc;                // :465
     return adam_over(&A->log_alpha, 1, &A->alpha_adam, A->alpha_age);                                                           // :466
@@ -1238,9 +1254,9 @@ int rlt_oracle_gru_forward(const rlt_gru_layer* L, const float* input, const uin
             }
         for (int b = 0; b < B; b++) {
             float* p = post + (size_t)b * H3;
-            for (int j = 0; j < 2 * H; j++) p[j] = 1 / (1 + std::exp(-p[j]));                         // sigmoid (:301)
+            for (int j = 0; j < 2 * H; j++) p[j] = L->fast_tanh ? 0.5f * fast_tanh(0.5f * p[j]) + 0.5f : 1 / (1 + std::exp(-p[j]));   // (fast_)sigmoid (:302-310)
             for (int j = 0; j < H; j++) p[2 * H + j] += npp[(size_t)b * H + j] * p[j];                 // :303
-            for (int j = 0; j < H; j++) p[2 * H + j] = std::tanh(p[2 * H + j]);                        // :311
+            for (int j = 0; j < H; j++) p[2 * H + j] = L->fast_tanh ? fast_tanh(p[2 * H + j]) : std::tanh(p[2 * H + j]);   // :312-320
             for (int j = 0; j < H; j++) {
                 float o = 1 - p[H + j];                                                                 // one_minus (:313)
                 o = o * p[2 * H + j];                                                                   // multiply (:314)

@@ -95,6 +95,18 @@ int rlt_oracle_cast_reduce_sum_u8(const uint8_t* mask, size_t count, float* out_
 int rlt_oracle_sac_train_critic(const rlt_sac_agent* agent, int critic_index, const float* action_noise);
 int rlt_oracle_sac_update_critic_targets(const rlt_sac_agent* agent);
 int rlt_oracle_sac_train_actor(const rlt_sac_agent* agent, const float* action_noise);
+int rlt_oracle_sas_backward_reset(const rlt_sas_parameters* p, const float* input, int ldin, const float* noise, int ldn,
+                                  const float* actions, int lda, const float* pre_squashing, int ldp,
+                                  const float* d_output, int lddo, float* d_input, int lddi,
+                                  const float* log_alpha, float* d_log_alpha, const uint8_t* reset, int batch, int dim);
+/* sequential (recurrent) models and SAC on sequence batches: oracle/rlt_oracle_seq.cpp */
+int rlt_oracle_seq_forward(const rlt_seq_layer* layers, int n_layers, const float* x, int ldx, const uint8_t* reset, int steps, int batch);
+int rlt_oracle_seq_backward(const rlt_seq_layer* layers, int n_layers, const float* x, int ldx, float* d_output, float* d_input, const uint8_t* reset,
+                            int steps, int batch, int want_weight_gradients, int reset_in_backward_input);
+int rlt_oracle_seq_zero_gradient(const rlt_seq_layer* layers, int n_layers);
+int rlt_oracle_sac_sequence_train_critic(const rlt_sac_sequence_agent* agent, int critic_index, const float* action_noise);
+int rlt_oracle_sac_sequence_update_critic_targets(const rlt_sac_sequence_agent* agent);
+int rlt_oracle_sac_sequence_train_actor(const rlt_sac_sequence_agent* agent, const float* action_noise);
 
 int rlt_oracle_replay_add(const rlt_replay_buffer* rb, const float* observations, const float* actions, const float* rewards,
                           const float* next_observations, const uint8_t* terminated, const uint8_t* truncated);

@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "librlt_rocm.so")
-SOURCES = ["device.hip", "gemm.hip", "mlp.hip", "mlp_fused.hip", "mlp_small.hip", "optim.hip", "sac.hip", "sac_fused.hip", "runner.hip", "ppo.hip", "gru.hip", "td3.hip", "normalize.hip", "envs.hip"]
+SOURCES = ["device.hip", "gemm.hip", "mlp.hip", "mlp_fused.hip", "mlp_small.hip", "optim.hip", "sac.hip", "sac_fused.hip", "runner.hip", "ppo.hip", "gru.hip", "td3.hip", "normalize.hip", "envs.hip", "seq.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc",
     # keep the compiler from forming packed-fp32 VALU instructions

@@ -149,7 +149,28 @@ class GruLayer(C.Structure):
     _fields_ = [("weights_input", C.c_void_p), ("biases_input", C.c_void_p), ("weights_hidden", C.c_void_p), ("biases_hidden", C.c_void_p),
                 ("initial_hidden_state", C.c_void_p), ("d_weights_input", C.c_void_p), ("d_biases_input", C.c_void_p), ("d_weights_hidden", C.c_void_p),
                 ("d_biases_hidden", C.c_void_p), ("post_activation", C.c_void_p), ("n_pre_pre_activation", C.c_void_p), ("output", C.c_void_p),
-                ("input_dim", C.c_int32), ("hidden_dim", C.c_int32)]
+                ("input_dim", C.c_int32), ("hidden_dim", C.c_int32), ("fast_tanh", C.c_int32), ("reserved", C.c_int32)]
+
+
+class SeqLayer(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("reserved", C.c_int32), ("dense", DenseLayer), ("gru", GruLayer)]
+
+
+class SacSequenceAgent(C.Structure):
+    _fields_ = [("observation_dim", C.c_int32), ("action_dim", C.c_int32), ("n_actor_layers", C.c_int32), ("n_critic_layers", C.c_int32),
+                ("include_first_step_in_targets", C.c_int32), ("reserved0", C.c_int32), ("gamma", C.c_float), ("polyak", C.c_float),
+                ("sas", SasParameters), ("actor_adam", AdamParameters), ("critic_adam", AdamParameters), ("alpha_adam", AdamParameters),
+                ("actor", C.POINTER(SeqLayer)), ("critics", C.POINTER(SeqLayer) * 2), ("critics_target", C.POINTER(SeqLayer) * 2),
+                ("actor_adam_tensors", C.POINTER(AdamTensor)), ("n_actor_adam_tensors", C.c_int32), ("pad0", C.c_int32),
+                ("critic_adam_tensors", C.POINTER(AdamTensor) * 2), ("n_critic_adam_tensors", C.c_int32), ("pad1", C.c_int32),
+                ("log_alpha", AdamTensor),
+                ("actor_age", C.c_void_p), ("critic_age", C.c_void_p * 2), ("alpha_age", C.c_void_p),
+                ("batch", SequenceBatch),
+                ("next_state_action_value_input", C.c_void_p), ("next_q", C.c_void_p * 2), ("next_log_probabilities", C.c_void_p),
+                ("target_action_value", C.c_void_p), ("d_output", C.c_void_p), ("state_action_value_input", C.c_void_p),
+                ("d_critic_input", C.c_void_p * 2), ("d_actor_output_squashing", C.c_void_p), ("d_actor_output", C.c_void_p),
+                ("actor_actions", C.c_void_p), ("actor_pre_squashing", C.c_void_p), ("actor_log_probabilities", C.c_void_p),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
 
 
 class Td3Agent(C.Structure):
@@ -228,6 +249,12 @@ PROTOTYPES = {
     "standardize_backward_input": [P, P, I, P, I, I, I],
     "running_normalizer_update": [P, I, I, I, P, P, P],
     "on_policy_collect": [C.POINTER(PendulumRunner), C.POINTER(OnPolicyDataset), LP, I, P, P, P, P, P, I, P, S],
+    "seq_forward": [C.POINTER(SeqLayer), I, P, I, P, I, I, P, S],
+    "seq_backward": [C.POINTER(SeqLayer), I, P, I, P, P, P, I, I, I, I, P, S],
+    "seq_zero_gradient": [C.POINTER(SeqLayer), I],
+    "sac_sequence_train_critic": [C.POINTER(SacSequenceAgent), I, P],
+    "sac_sequence_update_critic_targets": [C.POINTER(SacSequenceAgent)],
+    "sac_sequence_train_actor": [C.POINTER(SacSequenceAgent), P],
     "td3_sampling_forward": [P, I, P, I, F, P, I, P, I, I, I],
     "td3_sampling_backward": [P, I, P, I, P, I, I, I],
     "td3_target_action_noise": [P, F, F, P, S],
@@ -251,6 +278,8 @@ ROCM_ONLY = {
     "mlp_workspace_bytes": ([LP, I, I], S),
     "ppo_workspace_bytes": ([C.POINTER(PpoAgent)], S),
     "gru_workspace_bytes": ([C.POINTER(GruLayer), I, I], S),
+    "seq_workspace_bytes": ([C.POINTER(SeqLayer), I, I, I], S),
+    "sac_sequence_workspace_bytes": ([C.POINTER(SacSequenceAgent)], S),
     "on_policy_collect_workspace_bytes": ([C.POINTER(PendulumRunner), LP, I], S),
     "gather_draw": ([P, C.POINTER(ReplayBuffer), I, U64, U64, P, P], I),
     "sac_pendulum_loop": ([P, C.POINTER(SacAgent), C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, U64, U64, C.POINTER(SacLoopInputs),

@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void fill_u8_kernel(uint8_t* __restrict__ dst,
 }
 __global__ __launch_bounds__(256) void scale_kernel(float* __restrict__ x, size_t count, float s, int reciprocal) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
-        x[i] = reciprocal ? s / x[i] : s * x[i];
+        x[i] = reciprocal ? (1.0f / x[i]) * s : x[i] * s;   // the reciprocal first, then the scale, as the reference's Scale operation rounds
 }
 
 // Philox4x32-10 (Salmon et al. 2011): a pure function of (key = seed, counter = offset + element/4)

@@ -25,6 +25,9 @@ struct GruArgs {
 };
 
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+// the gate functions; fast = the rational approximations of math/operations_generic.h:247-255 (a wavefront-uniform switch)
+__device__ __forceinline__ float gate_sigmoid(float x, int fast) { return fast ? 0.5f * rlt_fast_tanh(0.5f * x) + 0.5f : sigmoidf_(x); }
+__device__ __forceinline__ float gate_tanh(float x, int fast) { return fast ? rlt_fast_tanh(x) : tanhf(x); }
 
 // post_activation holds W_i x + b_i on entry. Thread (row, j): hidden unit j of one batch row.
 __global__ __launch_bounds__(GRU_THREADS) void gru_forward_kernel(GruArgs A) {
@@ -49,8 +52,8 @@ __global__ __launch_bounds__(GRU_THREADS) void gru_forward_kernel(GruArgs A) {
             const float* hr = hs + row * H;
             for (int k = 0; k < H; k++) { const float hk = hr[k]; const float* w = wt + k * H3; ar += hk * w[j]; az += hk * w[H + j]; an += hk * w[2 * H + j]; }
             float* post = A.L.post_activation + ((size_t)t * A.B + b) * H3;
-            const float r = sigmoidf_(post[j] + ar), z = sigmoidf_(post[H + j] + az);
-            const float n = tanhf(post[2 * H + j] + an * r);
+            const float r = gate_sigmoid(post[j] + ar, A.L.fast_tanh), z = gate_sigmoid(post[H + j] + az, A.L.fast_tanh);
+            const float n = gate_tanh(post[2 * H + j] + an * r, A.L.fast_tanh);
             post[j] = r; post[H + j] = z; post[2 * H + j] = n;
             A.L.n_pre_pre_activation[((size_t)t * A.B + b) * H + j] = an;
             h = (1.0f - z) * n + z * h;
@@ -149,8 +152,8 @@ __global__ __launch_bounds__(GRU_THREADS) void gru_forward64_kernel(GruArgs A) {
         float ar = bhr, az = bhz, an = bhn;
 #pragma unroll
         for (int k = 0; k < HW; k++) { const float hk = lane_read(h, k); ar += hk * wr[k]; az += hk * wz[k]; an += hk * wn[k]; }
-        const float r = sigmoidf_(xr + ar), z = sigmoidf_(xz + az);
-        const float n = tanhf(xn + an * r);
+        const float r = gate_sigmoid(xr + ar, A.L.fast_tanh), z = gate_sigmoid(xz + az, A.L.fast_tanh);
+        const float n = gate_tanh(xn + an * r, A.L.fast_tanh);
         float* po = A.L.post_activation + (size_t)t * stride + (size_t)b * 3 * HW;
         po[lane] = r; po[HW + lane] = z; po[2 * HW + lane] = n;
         const size_t at = ((size_t)t * A.B + b) * HW + lane;

@@ -4,6 +4,7 @@
 //            rl/algorithms/sac/operations_generic.h:133-527 (CUDA :12-128), nn/loss_functions/mse/operations_generic.h:9-97,
 //            random/operations_generic.h:72-105.
 #include "common.h"
+#include <algorithm>
 
 namespace {
 
@@ -155,7 +156,8 @@ __global__ __launch_bounds__(1024) void sac_d_output_kernel(const float* __restr
     __syncthreads();
     if (threadIdx.x == 0) { float s = 0.0f; for (int i = 0; i < 16; i++) s += partial[i]; n_final = s; }
     __syncthreads();
-    const float loss_weight = actor ? (-1.0f / n_final) : ((float)rows * 0.5f) / n_final;
+    // scale(loss_weight, s, reciprocal) is (1 / n) * s in the reference (containers/tensor/operations_generic.h:437-443): two roundings when n is no power of two
+    const float loss_weight = (1.0f / n_final) * (actor ? -1.0f : (float)rows * 0.5f);
     const float constant = 2.0f / (float)rows * loss_weight;
     for (int i = threadIdx.x; i < rows; i += blockDim.x) {
         bool m = mask ? (mask[i] != 0) : true;
@@ -328,6 +330,128 @@ int rlt_rocm_sac_train_actor(rlt_rocm_device* device, const rlt_sac_agent* A, co
     if ((rc = rlt_rocm_mlp_backward(device, A->actor, A->n_actor_layers, obs, D, A->d_actor_output, 2 * ACT, nullptr, 0, B, 1, ws, ws_bytes))) return rc;
     if ((rc = rlt_rocm_adam_step(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, 0.0f, nullptr))) return rc;
     return rlt_rocm_adam_step(device, &A->log_alpha, 1, &A->alpha_adam, A->alpha_age, 0.0f, nullptr);
+}
+
+// ---------------------------------------------------------------------------------------- sequence batches, sequential (recurrent) networks
+static inline const float* seq_output(const rlt_seq_layer* layers, int n) { const rlt_seq_layer& L = layers[n - 1]; return L.kind ? L.gru.output : L.dense.output; }
+static inline int seq_out_dim(const rlt_seq_layer* layers, int n) { const rlt_seq_layer& L = layers[n - 1]; return L.kind ? L.gru.hidden_dim : L.dense.out_dim; }
+static bool sequence_agent_ok(const rlt_sac_sequence_agent* A) {
+    if (!A || A->observation_dim <= 0 || A->action_dim <= 0 || A->n_actor_layers < 1 || A->n_critic_layers < 1) return false;
+    if (!A->actor || !A->critics[0] || !A->critics[1] || !A->critics_target[0] || !A->critics_target[1] || !A->log_alpha.parameters) return false;
+    const rlt_sequence_batch& K = A->batch;
+    if (K.batch <= 0 || K.sequence_length <= 0 || !K.observations_actions_base || !K.rewards || !K.terminated || !K.reset || !K.next_reset_base || !K.final_step_mask ||
+        !K.next_final_step_mask_base) return false;
+    if (seq_out_dim(A->actor, A->n_actor_layers) != 2 * A->action_dim) return false;
+    for (int k = 0; k < 2; k++) if (seq_out_dim(A->critics[k], A->n_critic_layers) != 1 || seq_out_dim(A->critics_target[k], A->n_critic_layers) != 1) return false;
+    return A->workspace && A->workspace_bytes >= rlt_rocm_sac_sequence_workspace_bytes(A);
+}
+
+size_t rlt_rocm_sac_sequence_workspace_bytes(const rlt_sac_sequence_agent* A) {
+    if (!A || !A->actor || !A->critics[0] || !A->critics_target[0]) return 0;
+    const int T = A->batch.sequence_length + 1, B = A->batch.batch;
+    size_t n = rlt_rocm_seq_workspace_bytes(A->actor, A->n_actor_layers, T, B);
+    n = std::max(n, rlt_rocm_seq_workspace_bytes(A->critics[0], A->n_critic_layers, T, B));
+    return std::max(n, rlt_rocm_seq_workspace_bytes(A->critics_target[0], A->n_critic_layers, T, B));
+}
+
+// rl/algorithms/sac/operations_generic.h:243-337 on a sequence batch, one launch per reference operation
+int rlt_rocm_sac_sequence_train_critic(rlt_rocm_device* device, const rlt_sac_sequence_agent* A, int ci, const float* action_noise) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(sequence_agent_ok(A) && (ci == 0 || ci == 1) && action_noise);
+    RLT_REQUIRE(A->next_state_action_value_input && A->next_q[0] && A->next_q[1] && A->next_log_probabilities && A->target_action_value && A->d_output);
+    const rlt_sequence_batch& K = A->batch;
+    const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    const int first = A->include_first_step_in_targets ? 1 : 0, T = S + first, next_offset = first ? 0 : 1;   // off_policy_runner/operations_generic.h:85-92
+    const rlt_seq_layer* critic = A->critics[ci];
+    void* ws = A->workspace; const size_t ws_bytes = A->workspace_bytes;
+    int rc;
+    if ((rc = rlt_rocm_seq_zero_gradient(device, critic, A->n_critic_layers))) return rc;                                                  // :263
+    const float* base_next = K.observations_actions_base + (size_t)next_offset * B * D;
+    const uint8_t* next_reset = K.next_reset_base + (size_t)next_offset * B;
+    const uint8_t* next_final = K.next_final_step_mask_base + (size_t)next_offset * B;
+    if ((rc = rlt_rocm_seq_forward(device, A->actor, A->n_actor_layers, base_next, D, next_reset, T, B, ws, ws_bytes))) return rc;           // :266-273
+    float* next_actions = A->next_state_action_value_input + OBS;
+    if ((rc = rlt_rocm_sas_forward(device, &A->sas, seq_output(A->actor, A->n_actor_layers), 2 * ACT, action_noise, ACT, next_actions, D, nullptr, 0,
+                                   A->next_log_probabilities, T * B, ACT))) return rc;
+    if ((rc = rlt_rocm_mask_copy(device, base_next + OBS, D, next_actions, D, next_final, 1, T * B, ACT))) return rc;                      // :274-277
+    if ((rc = copy2d(device, base_next, D, A->next_state_action_value_input, D, T * B, OBS))) return rc;                                   // :278
+    for (int k = 0; k < 2; k++) {                                                                                                          // :283-284
+        if ((rc = rlt_rocm_seq_forward(device, A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, next_reset, T, B, ws, ws_bytes))) return rc;
+        if ((rc = rlt_rocm_memcpy_d2d(device, A->next_q[k], seq_output(A->critics_target[k], A->n_critic_layers), sizeof(float) * T * B))) return rc;
+    }
+    // the value of the step after (offset B where the first step is included), the log-probability at the same index (:144-154)
+    if ((rc = rlt_rocm_sac_target_action_values(device, A->next_q[0] + first * B, A->next_q[1] + first * B, K.rewards, K.terminated, A->next_log_probabilities,
+                                               A->log_alpha.parameters, A->gamma, 0, A->target_action_value, S * B))) return rc;             // :289
+    if ((rc = rlt_rocm_seq_forward(device, critic, A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, ws, ws_bytes))) return rc;   // :294
+    hipLaunchKernelGGL(sac_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, seq_output(critic, A->n_critic_layers), (const float*)A->target_action_value,
+                       (const uint8_t*)K.final_step_mask, A->d_output, S * B, 0);                                                          // :298-316
+    if ((rc = rlt_launch_status(device))) return rc;
+    if ((rc = rlt_rocm_seq_backward(device, critic, A->n_critic_layers, K.observations_actions_base, D, A->d_output, nullptr, K.reset, S, B, 1, 0, ws, ws_bytes))) return rc;   // :329
+    return rlt_rocm_adam_step(device, A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], 0.0f, nullptr);   // :336
+}
+
+// sac/operations_generic.h:486-527
+int rlt_rocm_sac_sequence_update_critic_targets(rlt_rocm_device* device, const rlt_sac_sequence_agent* A) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(sequence_agent_ok(A));
+    int rc;
+    for (int k = 0; k < 2; k++)
+        for (int l = 0; l < A->n_critic_layers; l++) {
+            const rlt_seq_layer& s = A->critics[k][l]; const rlt_seq_layer& t = A->critics_target[k][l];
+            RLT_REQUIRE(s.kind == t.kind);
+            if (s.kind == 0) {
+                if ((rc = rlt_rocm_polyak_update(device, s.dense.weights, t.dense.weights, (size_t)s.dense.in_dim * s.dense.out_dim, A->polyak, 0))) return rc;
+                if ((rc = rlt_rocm_polyak_update(device, s.dense.biases, t.dense.biases, (size_t)s.dense.out_dim, A->polyak, 0))) return rc;
+            } else {
+                const size_t H = s.gru.hidden_dim, I = s.gru.input_dim;
+                if ((rc = rlt_rocm_polyak_update(device, s.gru.weights_input, t.gru.weights_input, 3 * H * I, A->polyak, 0))) return rc;
+                if ((rc = rlt_rocm_polyak_update(device, s.gru.biases_input, t.gru.biases_input, 3 * H, A->polyak, 0))) return rc;
+                if ((rc = rlt_rocm_polyak_update(device, s.gru.weights_hidden, t.gru.weights_hidden, 3 * H * H, A->polyak, 0))) return rc;
+                if ((rc = rlt_rocm_polyak_update(device, s.gru.biases_hidden, t.gru.biases_hidden, 3 * H, A->polyak, 0))) return rc;
+                if ((rc = rlt_rocm_polyak_update(device, s.gru.initial_hidden_state, t.gru.initial_hidden_state, H, A->polyak, 0))) return rc;
+            }
+        }
+    return 0;
+}
+
+// sac/operations_generic.h:395-468 on a sequence batch
+int rlt_rocm_sac_sequence_train_actor(rlt_rocm_device* device, const rlt_sac_sequence_agent* A, const float* action_noise) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(sequence_agent_ok(A) && action_noise);
+    RLT_REQUIRE(A->state_action_value_input && A->d_output && A->d_critic_input[0] && A->d_critic_input[1] && A->d_actor_output_squashing && A->d_actor_output &&
+                A->actor_pre_squashing && A->actor_log_probabilities && A->actor_actions && A->log_alpha.gradient);
+    const rlt_sequence_batch& K = A->batch;
+    const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT, R = S * B;
+    void* ws = A->workspace; const size_t ws_bytes = A->workspace_bytes;
+    int rc;
+    if ((rc = rlt_rocm_seq_zero_gradient(device, A->actor, A->n_actor_layers))) return rc;                                                  // :414
+    if ((rc = rlt_rocm_fill_f32(device, A->log_alpha.gradient, 1, 1, 1, 0.0f))) return rc;
+    const float* obs = K.observations_actions_base;
+    if ((rc = rlt_rocm_seq_forward(device, A->actor, A->n_actor_layers, obs, D, K.reset, S, B, ws, ws_bytes))) return rc;                   // :427
+    const float* actor_out = seq_output(A->actor, A->n_actor_layers);
+    if ((rc = rlt_rocm_sas_forward(device, &A->sas, actor_out, 2 * ACT, action_noise, ACT, A->actor_actions, ACT, A->actor_pre_squashing, ACT,
+                                   A->actor_log_probabilities, R, ACT))) return rc;
+    float* sav_actions = A->state_action_value_input + OBS;
+    if ((rc = copy2d(device, A->actor_actions, ACT, sav_actions, D, R, ACT))) return rc;
+    if ((rc = rlt_rocm_mask_copy(device, obs + OBS, D, sav_actions, D, K.final_step_mask, 1, R, ACT))) return rc;                           // :428-430
+    if ((rc = copy2d(device, obs, D, A->state_action_value_input, D, R, OBS))) return rc;                                                   // :431
+    for (int k = 0; k < 2; k++)                                                                                                            // :432-433
+        if ((rc = rlt_rocm_seq_forward(device, A->critics[k], A->n_critic_layers, A->state_action_value_input, D, K.reset, S, B, ws, ws_bytes))) return rc;
+    hipLaunchKernelGGL(sac_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, (const float*)nullptr, (const float*)nullptr, (const uint8_t*)K.final_step_mask,
+                       A->d_output, R, 1);                                                                                                 // :437-453
+    if ((rc = rlt_launch_status(device))) return rc;
+    // :458-459: the inner layers of backward_input run without the reset mode (nn_models/sequential/operations_generic.h:399-407); the critics'
+    // output layer has no activation function, so d_output survives the first call unchanged
+    for (int k = 0; k < 2; k++)
+        if ((rc = rlt_rocm_seq_backward(device, A->critics[k], A->n_critic_layers, nullptr, 0, A->d_output, A->d_critic_input[k], K.reset, S, B, 0, 0, ws, ws_bytes))) return rc;
+    if ((rc = rlt_rocm_sac_min_value_d_output(device, seq_output(A->critics[0], A->n_critic_layers), seq_output(A->critics[1], A->n_critic_layers), A->d_critic_input[0],
+                                             A->d_critic_input[1], D, D, ACT, A->d_actor_output_squashing, ACT, R))) return rc;             // :460
+    if ((rc = rlt_rocm_mask_zero(device, A->d_actor_output_squashing, ACT, K.final_step_mask, 1, R, ACT))) return rc;                       // :461-463
+    if ((rc = sas_backward_impl(device, &A->sas, actor_out, 2 * ACT, action_noise, ACT, A->actor_actions, ACT, A->actor_pre_squashing, ACT, A->d_actor_output_squashing, ACT,
+                                A->d_actor_output, 2 * ACT, A->log_alpha.parameters, A->log_alpha.gradient, K.reset, R, ACT))) return rc;   // :464
+    if ((rc = rlt_rocm_seq_backward(device, A->actor, A->n_actor_layers, obs, D, A->d_actor_output, nullptr, K.reset, S, B, 1, 0, ws, ws_bytes))) return rc;
+    if ((rc = rlt_rocm_adam_step(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, 0.0f, nullptr))) return rc;   // :465
+    return rlt_rocm_adam_step(device, &A->log_alpha, 1, &A->alpha_adam, A->alpha_age, 0.0f, nullptr);                                      // :466
 }
 
 }  // extern "C"

@@ -43,12 +43,15 @@ class LoopConfig(C.Structure):
                 ("n_warmup_steps", C.c_int32), ("episode_step_limit", C.c_int32), ("adam_epsilon", C.c_float)]
 
 
+WITH_WORKSPACE = ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward", "on_policy_collect", "seq_forward", "seq_backward")
+
+
 def load_oracle():
     lib = C.CDLL(build_oracle())
     P, S, I = C.c_void_p, C.c_size_t, C.c_int
     for name, args in capi.PROTOTYPES.items():
         a = list(args)
-        if name in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward", "on_policy_collect"):
+        if name in WITH_WORKSPACE:
             a = a[:-2]      # the CPU checker allocates its own workspace
         fn = getattr(lib, "rlt_oracle_" + name)
         fn.argtypes = a
@@ -113,7 +116,7 @@ class HostBackend:
         return HostArray(np.zeros(shape, dtype))
 
     def call(self, fn, *args):
-        if fn in ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward", "on_policy_collect"):
+        if fn in WITH_WORKSPACE:
             args = args[:-2]
         rc = getattr(self.lib, "rlt_oracle_" + fn)(*args)
         if rc != 0:
@@ -222,19 +225,20 @@ class Mlp:
 
 
 REF_GRU_GENERIC = os.path.join(ORACLE_DIR, "_ref", "librlt_ref_gru_generic.so")
+REF_GRU_FAST_GENERIC = os.path.join(ORACLE_DIR, "_ref", "librlt_ref_gru_fast_generic.so")
 
 
 class GruOnBackend:
     """One GRU layer (parameters, gradients, kept intermediates) on a backend. params: dict W_i [3H x I], b_i, W_h [3H x H], b_h, h0."""
 
-    def __init__(self, backend, S, B, I, H, params):
+    def __init__(self, backend, S, B, I, H, params, fast_tanh=False):
         self.backend, self.S, self.B, self.I, self.H = backend, S, B, I, H
         f = lambda k: backend.array(np.asarray(params[k], np.float32))
         self.W_i, self.b_i, self.W_h, self.b_h, self.h0 = f("W_i"), f("b_i"), f("W_h"), f("b_h"), f("h0")
         self.dW_i, self.db_i, self.dW_h, self.db_h = backend.zeros((3 * H, I)), backend.zeros((3 * H,)), backend.zeros((3 * H, H)), backend.zeros((3 * H,))
         self.post, self.npp, self.out = backend.zeros((S, B, 3 * H)), backend.zeros((S, B, H)), backend.zeros((S, B, H))
         self.c = capi.GruLayer(self.W_i.ptr, self.b_i.ptr, self.W_h.ptr, self.b_h.ptr, self.h0.ptr, self.dW_i.ptr, self.db_i.ptr, self.dW_h.ptr, self.db_h.ptr,
-                               self.post.ptr, self.npp.ptr, self.out.ptr, I, H)
+                               self.post.ptr, self.npp.ptr, self.out.ptr, I, H, int(fast_tanh), 0)
         self.ws, self.wsn = (None, 0)
         if backend.name == "rocm":
             n = backend.device.lib.rlt_rocm_gru_workspace_bytes(C.byref(self.c), S, B)
@@ -926,3 +930,230 @@ def ring_track(height=80, width=120, inner=0.45, outer=0.85):
     yy, xx = np.mgrid[0:height, 0:width]
     rr = np.hypot((xx + 0.5 - width / 2) / (width / 2), (yy + 0.5 - height / 2) / (height / 2))
     return ((rr > inner) & (rr < outer)).astype(np.uint8)
+
+
+# ---------------------------------------------------------------------------------------------- SAC on sequence batches with recurrent networks
+ACT_NAMES = {v: k for k, v in capi.ACT.items()}     # the reference's enum values (nn/activation_functions.h:11-18) are the ABI's
+
+
+def ref_sac_gru_path(n_layers):
+    return os.path.join(ORACLE_DIR, "_ref", f"librlt_ref_sac_gru{n_layers}_generic.so")
+
+
+def seq_param_count(specs):
+    """specs: list of (kind, in, out, activation name); dense [W | b], GRU [W_i | b_i | W_h | b_h | h0]."""
+    return sum((i * o + o) if kind == 0 else (3 * o * i + 3 * o + 3 * o * o + 3 * o + o) for kind, i, o, _ in specs)
+
+
+def random_seq_params(rng, specs):
+    parts = []
+    for kind, i, o, _ in specs:
+        if kind == 0:
+            parts += [rng.uniform(-1, 1, o * i) / np.sqrt(i), rng.uniform(-0.1, 0.1, o)]
+        else:
+            parts += [rng.uniform(-1, 1, 3 * o * i) / np.sqrt(i), rng.uniform(-0.1, 0.1, 3 * o), rng.uniform(-1, 1, 3 * o * o) / np.sqrt(o), rng.uniform(-0.1, 0.1, 3 * o), np.zeros(o)]
+    return np.concatenate(parts).astype(np.float32)
+
+
+class SeqNet:
+    """A sequential model of dense and GRU layers on a backend: flat arenas (parameters, gradients, Adam moments), kept intermediates for `steps`
+    x `batch` rows, described to the C ABI by an array of rlt_seq_layer."""
+
+    def __init__(self, backend, specs, params, steps, batch, trainable=True, fast_tanh=True):
+        self.backend, self.specs, self.steps, self.batch, self.n = backend, list(specs), steps, batch, len(specs)
+        total = seq_param_count(specs)
+        assert params.size == total, (params.size, total)
+        self.params = backend.array(params.astype(np.float32))
+        self.grads, self.m, self.v = (backend.zeros((total,)) for _ in range(3)) if trainable else (None, None, None)
+        self.age = backend.array(np.array([1], np.uint32))
+        self.layers = (capi.SeqLayer * self.n)()
+        self.keep, adam, off = [], [], 0
+        z = backend.zeros
+        g = lambda o: self.grads.offset(o) if trainable else None
+        def tensor(o, n, flags):
+            if trainable:
+                adam.append(capi.AdamTensor(self.params.offset(o), self.grads.offset(o), self.m.offset(o), self.v.offset(o), None, n, flags))
+        for l, (kind, i, o, act) in enumerate(specs):
+            L = self.layers[l]
+            L.kind = kind
+            if kind == 0:
+                pre, out = z((steps * batch, o)), z((steps * batch, o))
+                self.keep.append((pre, out))
+                L.dense = capi.DenseLayer(self.params.offset(off), self.params.offset(off + i * o), g(off), g(off + i * o), pre.ptr, out.ptr, i, o, capi.ACT[act], 0)
+                tensor(off, i * o, 1); tensor(off + i * o, o, 2)
+                off += i * o + o
+            else:
+                post, npp, out = z((steps, batch, 3 * o)), z((steps, batch, o)), z((steps, batch, o))
+                self.keep.append((post, npp, out))
+                o_wi, o_bi, o_wh, o_bh, o_h0 = off, off + 3 * o * i, off + 3 * o * i + 3 * o, off + 3 * o * i + 3 * o + 3 * o * o, off + 3 * o * i + 3 * o + 3 * o * o + 3 * o
+                L.gru = capi.GruLayer(self.params.offset(o_wi), self.params.offset(o_bi), self.params.offset(o_wh), self.params.offset(o_bh), self.params.offset(o_h0),
+                                      g(o_wi), g(o_bi), g(o_wh), g(o_bh), post.ptr, npp.ptr, out.ptr, i, o, int(fast_tanh), 0)
+                for oo, n, fl in ((o_wi, 3 * o * i, 1), (o_bi, 3 * o, 2), (o_wh, 3 * o * o, 1), (o_bh, 3 * o, 2), (o_h0, o, 2)):
+                    tensor(oo, n, fl)
+                off = o_h0 + o
+        self.adam = (capi.AdamTensor * max(len(adam), 1))(*adam)
+        self.n_adam = len(adam)
+
+    def output(self):
+        return self.keep[-1][-1].numpy()
+
+    def workspace(self):
+        if self.backend.name == "oracle":
+            return None, 0
+        return self.backend.workspace(self.backend.device.lib.rlt_rocm_seq_workspace_bytes(self.layers, self.n, self.steps, self.batch))
+
+
+class SacSequenceOnBackend:
+    """All state of a SAC agent with sequential (recurrent) networks on one backend. params: flat [actor, critic 0, critic 1, target 0, target 1,
+    log_alpha] with every network laid out layer after layer (the order the reference harness exports)."""
+
+    def __init__(self, backend, actor_specs, critic_specs, params, S, B, obs_dim, act_dim, include_first=True, hyper=None):
+        self.backend, self.S, self.B = backend, S, B
+        T, D = S + (1 if include_first else 0), obs_dim + act_dim
+        self.T = T
+        na, nc = seq_param_count(actor_specs), seq_param_count(critic_specs)
+        o = 0
+        self.actor = SeqNet(backend, actor_specs, params[o:o + na], T, B); o += na
+        self.critics = [SeqNet(backend, critic_specs, params[o + k * nc:o + (k + 1) * nc], S, B) for k in range(2)]; o += 2 * nc
+        self.targets = [SeqNet(backend, critic_specs, params[o + k * nc:o + (k + 1) * nc], T, B, trainable=False) for k in range(2)]; o += 2 * nc
+        self.log_alpha = backend.array(np.array([params[o], 0, 0, 0], np.float32))
+        self.alpha_age = backend.array(np.array([1], np.uint32))
+        self.batch = SequenceBatchOnBackend(backend, B, S, D)
+        z = backend.zeros
+        self.buf = dict(nsavi=z((T, B, D)), next_q0=z((T, B)), next_q1=z((T, B)), next_lp=z((T, B)), target=z((S, B)), d_output=z((S, B)), savi=z((S, B, D)),
+                        d_ci0=z((S, B, D)), d_ci1=z((S, B, D)), d_aos=z((S, B, act_dim)), d_ao=z((S, B, 2 * act_dim)), a_act=z((T, B, act_dim)), a_pre=z((S, B, act_dim)), a_lp=z((S, B)))
+        A = capi.SacSequenceAgent()
+        A.observation_dim, A.action_dim, A.n_actor_layers, A.n_critic_layers, A.include_first_step_in_targets = obs_dim, act_dim, len(actor_specs), len(critic_specs), int(include_first)
+        hyper = hyper or {}
+        A.gamma, A.polyak = hyper.get("gamma", 0.99), hyper.get("polyak", float(np.float32(1.0 - 0.005)))
+        A.sas = hyper.get("sas", capi.SasParameters(-20.0, 2.0, 1e-6, -float(act_dim)))
+        A.actor_adam, A.critic_adam, A.alpha_adam = (hyper.get(k, capi.adam_parameters()) for k in ("actor_adam", "critic_adam", "alpha_adam"))
+        A.actor, A.actor_adam_tensors, A.n_actor_adam_tensors, A.actor_age = self.actor.layers, self.actor.adam, self.actor.n_adam, self.actor.age.ptr
+        b = self.buf
+        for k in range(2):
+            A.critics[k], A.critics_target[k] = self.critics[k].layers, self.targets[k].layers
+            A.critic_adam_tensors[k], A.critic_age[k] = self.critics[k].adam, self.critics[k].age.ptr
+            A.next_q[k], A.d_critic_input[k] = b[f"next_q{k}"].ptr, b[f"d_ci{k}"].ptr
+        A.n_critic_adam_tensors = self.critics[0].n_adam
+        la = self.log_alpha
+        A.log_alpha = capi.AdamTensor(la.offset(0), la.offset(1), la.offset(2), la.offset(3), None, 1, 0)
+        A.alpha_age = self.alpha_age.ptr
+        A.batch = self.batch.c
+        A.next_state_action_value_input, A.next_log_probabilities, A.target_action_value, A.d_output = b["nsavi"].ptr, b["next_lp"].ptr, b["target"].ptr, b["d_output"].ptr
+        A.state_action_value_input, A.d_actor_output_squashing, A.d_actor_output = b["savi"].ptr, b["d_aos"].ptr, b["d_ao"].ptr
+        A.actor_actions, A.actor_pre_squashing, A.actor_log_probabilities = b["a_act"].ptr, b["a_pre"].ptr, b["a_lp"].ptr
+        if backend.name == "rocm":
+            n = int(backend.device.lib.rlt_rocm_sac_sequence_workspace_bytes(C.byref(A)))
+            self.ws = backend.device.empty((max(n, 4),), np.uint8)
+            A.workspace, A.workspace_bytes = self.ws.ptr, n
+        self.c = A
+
+    def set_batch(self, data):
+        for k in SEQUENCE_BATCH_FIELDS:
+            self.batch.arrays[k].upload(data[k])
+
+    def train(self, noise_critic, noise_actor):
+        """The training part of one loop step with a shared batch (rl/algorithms/sac/loop/core/operations_generic.h:127-154)."""
+        be = self.backend
+        nc, na = be.array(np.ascontiguousarray(noise_critic, np.float32)), be.array(np.ascontiguousarray(noise_actor, np.float32))
+        for k in range(2):
+            be.call("sac_sequence_train_critic", C.byref(self.c), k, nc.ptr)
+        be.call("sac_sequence_update_critic_targets", C.byref(self.c))
+        be.call("sac_sequence_train_actor", C.byref(self.c), na.ptr)
+        be.sync()
+
+    def parameters(self):
+        parts = [self.actor.params.numpy()] + [c.params.numpy() for c in self.critics] + [t.params.numpy() for t in self.targets]
+        return np.concatenate(parts + [self.log_alpha.numpy()[:1]])
+
+    def ages(self):
+        return [int(x.numpy()[0]) for x in (self.actor.age, self.critics[0].age, self.critics[1].age, self.alpha_age)]
+
+
+class RefSacGru:
+    """The reference's own SAC loop with recurrent approximators on sequence batches (oracle/_ref, compiled from /root/reference)."""
+
+    def __init__(self, n_layers, seed):
+        self.lib = lib = C.CDLL(ref_sac_gru_path(n_layers))
+        P = C.c_void_p
+        lib.rlt_ref_sac_gru_create.restype = P; lib.rlt_ref_sac_gru_create.argtypes = [C.c_uint32]
+        lib.rlt_ref_sac_gru_parameter_count.restype = C.c_size_t; lib.rlt_ref_sac_gru_parameter_count.argtypes = [P]
+        lib.rlt_ref_sac_gru_step_count.restype = C.c_uint32; lib.rlt_ref_sac_gru_step_count.argtypes = [P]
+        lib.rlt_ref_sac_gru_layers.argtypes = [P, C.c_int, P]
+        for f, n in (("destroy", 1), ("step", 1), ("get_parameters", 2), ("get_ages", 2), ("hyperparameters", 2), ("get_noise", 3), ("get_batch", 8), ("dims", 1)):
+            getattr(lib, "rlt_ref_sac_gru_" + f).argtypes = [P] * n
+        self.h = lib.rlt_ref_sac_gru_create(seed)
+        d = np.zeros(6, np.int32); lib.rlt_ref_sac_gru_dims(d.ctypes.data)
+        self.batch, self.seq, self.n_warmup, self.obs_dim, self.act_dim, self.include_first = [int(x) for x in d]
+        buf = np.zeros(64, np.int32)
+        self.specs = []
+        for critic in (0, 1):
+            n = lib.rlt_ref_sac_gru_layers(self.h, critic, buf.ctypes.data)
+            self.specs.append([(int(k), int(i), int(o), ACT_NAMES[int(a)]) for k, i, o, a in buf[:n].reshape(-1, 4)])
+        self.actor_specs, self.critic_specs = self.specs
+        hp = np.zeros(21, np.float32); lib.rlt_ref_sac_gru_hyperparameters(self.h, hp.ctypes.data)
+        self.hp = hp
+
+    def hyper(self):
+        hp = self.hp
+        adam = lambda o: capi.adam_parameters(alpha=float(hp[o]), beta_1=float(hp[o + 1]), beta_2=float(hp[o + 2]), epsilon=float(hp[o + 3]), epsilon_sqrt=float(hp[o + 4]))
+        return dict(gamma=float(hp[0]), polyak=float(hp[1]), sas=capi.SasParameters(float(hp[3]), float(hp[4]), float(hp[5]), float(hp[2])),
+                    actor_adam=adam(6), critic_adam=adam(11), alpha_adam=adam(16))
+
+    def step(self):
+        self.lib.rlt_ref_sac_gru_step(self.h)
+
+    def parameters(self):
+        p = np.zeros(self.lib.rlt_ref_sac_gru_parameter_count(self.h), np.float32)
+        self.lib.rlt_ref_sac_gru_get_parameters(self.h, p.ctypes.data)
+        return p
+
+    def ages(self):
+        a = np.zeros(4, np.uint32); self.lib.rlt_ref_sac_gru_get_ages(self.h, a.ctypes.data); return [int(x) for x in a]
+
+    def batch_data(self):
+        S, B, D = self.seq, self.batch, self.obs_dim + self.act_dim
+        out = dict(observations_actions_base=np.zeros((S + 1, B, D), np.float32), rewards=np.zeros((S, B), np.float32), terminated=np.zeros((S, B), np.uint8),
+                   reset=np.zeros((S, B), np.uint8), next_reset_base=np.zeros((S + 1, B), np.uint8), final_step_mask=np.zeros((S, B), np.uint8),
+                   next_final_step_mask_base=np.zeros((S + 1, B), np.uint8))
+        self.lib.rlt_ref_sac_gru_get_batch(self.h, *[out[k].ctypes.data for k in SEQUENCE_BATCH_FIELDS])
+        return out
+
+    def noise(self):
+        S, B = self.seq, self.batch
+        nc, na = np.zeros((S + 1, B, self.act_dim), np.float32), np.zeros((S, B, self.act_dim), np.float32)
+        self.lib.rlt_ref_sac_gru_get_noise(self.h, nc.ctypes.data, na.ctypes.data)
+        return nc, na
+
+    def close(self):
+        self.lib.rlt_ref_sac_gru_destroy(self.h)
+
+
+def sac_sequence_digest(params, actor_specs, critic_specs):
+    """float64 (sum, sum of squares) of the actor, both critics, both target critics and log_alpha out of the flat parameter vector."""
+    na, nc = seq_param_count(actor_specs), seq_param_count(critic_specs)
+    bounds = np.cumsum([0, na, nc, nc, nc, nc, 1])
+    p = params.astype(np.float64)
+    return np.array([[p[a:b].sum(), (p[a:b] ** 2).sum()] for a, b in zip(bounds[:-1], bounds[1:])])
+
+
+def sac_sequence_golden():
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sac_sequence_pendulum.npz")
+    return dict(np.load(path)) if os.path.exists(path) else None
+
+
+def sac_sequence_golden_case(g, n_layers):
+    """(specs of actor and critic, dims, hyper dict) of one depth of the fixture."""
+    p = f"l{n_layers}_"
+    specs = [[(int(k), int(i), int(o), ACT_NAMES[int(a)]) for k, i, o, a in g[p + name + "_layers"]] for name in ("actor", "critic")]
+    hp = g[p + "hyperparameters"]
+    adam = lambda o: capi.adam_parameters(alpha=float(hp[o]), beta_1=float(hp[o + 1]), beta_2=float(hp[o + 2]), epsilon=float(hp[o + 3]), epsilon_sqrt=float(hp[o + 4]))
+    hyper = dict(gamma=float(hp[0]), polyak=float(hp[1]), sas=capi.SasParameters(float(hp[3]), float(hp[4]), float(hp[5]), float(hp[2])),
+                 actor_adam=adam(6), critic_adam=adam(11), alpha_adam=adam(16))
+    return specs[0], specs[1], [int(x) for x in g[p + "dims"]], hyper
+
+
+def sac_sequence_golden_step(agent, g, n_layers, i):
+    p = f"l{n_layers}_s{i}_"
+    agent.set_batch({k: g[p + k] for k in SEQUENCE_BATCH_FIELDS})
+    agent.train(g[p + "noise_critic"], g[p + "noise_actor"])

@@ -434,3 +434,99 @@ def test_car_on_track_rays_and_flags_on_a_synthetic_track(oracle):
     far = np.array([[5.0, 0.0, 0.0, 1.0, 0.0, 0.0], [0.0, -3.0, 1.0, 1.0, 0.0, 0.0]], np.float32)
     _, o2, _, _, t2 = helpers.car_track_on_backend(oracle, track, scale, far, np.zeros((2, 2), np.float32))
     assert np.all(o2[:, 6:] == 0) and np.all(t2 == 1)
+
+
+@pytest.mark.parametrize("n_layers", [3, 5])
+def test_sac_on_sequence_batches_reproduces_reference_vectors(oracle, n_layers):
+    """SAC with the reference's recurrent approximators on sequence batches: from the fixture's parameters, batches and noise the restatement
+    reproduces the parameter digests after every loop step and the full parameter snapshots, bit for bit."""
+    g = helpers.sac_sequence_golden()
+    actor_specs, critic_specs, (B, S, obs, act, first, steps), hyper = helpers.sac_sequence_golden_case(g, n_layers)
+    p = f"l{n_layers}_"
+    agent = helpers.SacSequenceOnBackend(oracle, actor_specs, critic_specs, g[p + "parameters_before"], S, B, obs, act, bool(first), hyper)
+    resets_inside = 0
+    for i in range(steps):
+        helpers.sac_sequence_golden_step(agent, g, n_layers, i)
+        resets_inside += int(g[f"{p}s{i}_reset"][1:].sum())
+        params = agent.parameters()
+        assert np.array_equal(helpers.sac_sequence_digest(params, actor_specs, critic_specs), g[f"{p}s{i}_digest"]), i
+        if i in g[p + "snapshots"]:
+            assert np.array_equal(params, g[f"{p}s{i}_after"]), i
+    assert agent.ages() == [int(a) for a in g[p + "ages_after"]]
+    assert resets_inside > 20       # sequences that restart inside the batch are what the reset modes are about
+
+
+def test_sac_sequence_of_length_one_equals_the_single_step_update(oracle):
+    """Independent of the sequence fixture: with sequence length 1, dense layers only, every step final and the `next` views starting at padded
+    step 1, the sequence update must give what the single-step SAC update (pinned against the reference's default loop) gives."""
+    rng = np.random.default_rng(3)
+    B, H, OBS, ACT = 64, 16, 3, 1
+    actor_specs = [(0, OBS, H, "relu"), (0, H, H, "relu"), (0, H, 2 * ACT, "identity")]
+    critic_specs = [(0, OBS + ACT, H, "relu"), (0, H, H, "relu"), (0, H, 1, "identity")]
+    na, nc = helpers.seq_param_count(actor_specs), helpers.seq_param_count(critic_specs)
+    critics = [helpers.random_seq_params(rng, critic_specs) for _ in range(2)]
+    params = np.concatenate([helpers.random_seq_params(rng, actor_specs)] + critics + [c.copy() for c in critics] + [np.array([np.log(0.5)], np.float32)])
+    assert params.size == na + 4 * nc + 1
+    oab = rng.standard_normal((2, B, OBS + ACT)).astype(np.float32)
+    rewards, terminated = rng.standard_normal((1, B)).astype(np.float32), (rng.uniform(size=(1, B)) < 0.2).astype(np.uint8)
+    ones = np.ones((1, B), np.uint8)
+    seq = helpers.SacSequenceOnBackend(oracle, actor_specs, critic_specs, params, 1, B, OBS, ACT, include_first=False)
+    seq.set_batch(dict(observations_actions_base=oab, rewards=rewards, terminated=terminated, reset=ones, next_reset_base=np.ones((2, B), np.uint8), final_step_mask=ones,
+                       next_final_step_mask_base=np.ones((2, B), np.uint8)))
+    one = helpers.SacOnBackend(oracle, B, H, params)
+    one.set_batch(oab, rewards[0], terminated[0])
+    for _ in range(3):
+        nc_, na_ = rng.standard_normal((1, B, ACT)).astype(np.float32), rng.standard_normal((1, B, ACT)).astype(np.float32)
+        seq.train(nc_, na_)
+        n1, n2 = oracle.array(nc_), oracle.array(na_)
+        for k in range(2):
+            oracle.call("sac_train_critic", C.byref(one.c), k, n1.ptr)
+        oracle.call("sac_update_critic_targets", C.byref(one.c))
+        oracle.call("sac_train_actor", C.byref(one.c), n2.ptr)
+        assert np.array_equal(seq.parameters(), one.parameters())
+
+
+@pytest.mark.parametrize("with_reset", [False, True])
+def test_sequential_model_gradients_against_finite_differences(oracle, with_reset):
+    """dense -> GRU -> GRU -> dense with exact gate functions: the gradients of sum(output * g) with respect to the input and to a sample of
+    every layer's parameters, by central differences in float64-accumulated outputs, with and without resets inside the sequence."""
+    rng = np.random.default_rng(17 + with_reset)
+    S, B, I, H, O = 5, 3, 4, 6, 2
+    specs = [(0, I, H, "tanh"), (1, H, H, "identity"), (1, H, H, "identity"), (0, H, O, "identity")]
+    params = helpers.random_seq_params(rng, specs)
+    x, g = rng.standard_normal((S, B, I)).astype(np.float32), rng.standard_normal((S, B, O)).astype(np.float32)
+    reset = np.zeros((S, B), np.uint8)
+    if with_reset:
+        reset[2, 0] = reset[3, 2] = reset[1, 1] = 1
+
+    def loss(p, xx):
+        net = helpers.SeqNet(oracle, specs, p, S, B, fast_tanh=False)
+        xd, rd = oracle.array(xx), oracle.array(reset)
+        oracle.call("seq_forward", net.layers, net.n, xd.ptr, I, rd.ptr if with_reset else None, S, B, None, 0)
+        return float((net.output().astype(np.float64).reshape(g.shape) * g).sum())
+    net = helpers.SeqNet(oracle, specs, params, S, B, fast_tanh=False)
+    xd, rd, gd, dx = oracle.array(x), oracle.array(reset), oracle.array(g), oracle.zeros((S, B, I))
+    oracle.call("seq_zero_gradient", net.layers, net.n)
+    oracle.call("seq_forward", net.layers, net.n, xd.ptr, I, rd.ptr if with_reset else None, S, B, None, 0)
+    oracle.call("seq_backward", net.layers, net.n, xd.ptr, I, gd.ptr, dx.ptr, rd.ptr if with_reset else None, S, B, 1, 0, None, 0)
+    grads, dxn = net.grads.numpy(), dx.numpy()
+    eps = 2e-3
+    checked = 0
+    for idx in rng.choice(params.size, 60, replace=False):
+        hi, lo = params.copy(), params.copy(); hi[idx] += eps; lo[idx] -= eps
+        fd = (loss(hi, x) - loss(lo, x)) / (2 * eps)
+        assert abs(fd - grads[idx]) <= 2e-2 * max(1.0, abs(fd)), (idx, fd, grads[idx])
+        checked += grads[idx] != 0
+    assert checked > 40       # the initial hidden state is not learned: its gradient stays zero
+    for idx in [(0, 0, 0), (2, 0, 1), (4, 2, 3), (1, 1, 2)]:
+        hi, lo = x.copy(), x.copy(); hi[idx] += eps; lo[idx] -= eps
+        fd = (loss(params, hi) - loss(params, lo)) / (2 * eps)
+        assert abs(fd - dxn[idx]) <= 2e-2 * max(1.0, abs(fd)), (idx, fd, dxn[idx])
+    # the switch of backward_input: without the resets the input gradient of a multi-layer model differs where a reset cut the sequence
+    if with_reset:
+        out = []
+        for flag in (0, 1):
+            gd2, dx2 = oracle.array(g), oracle.zeros((S, B, I))
+            oracle.call("seq_backward", net.layers, net.n, None, 0, gd2.ptr, dx2.ptr, rd.ptr, S, B, 0, flag, None, 0)
+            out.append(dx2.numpy())
+        assert np.allclose(out[1], dxn, rtol=1e-5, atol=1e-6) and not np.allclose(out[0], out[1], rtol=1e-3, atol=1e-5)

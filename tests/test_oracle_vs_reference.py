@@ -354,16 +354,21 @@ def test_ppo_gae_and_update_bit_exact_with_reference(oracle):
     ref.close()
 
 
-@pytest.mark.skipif(not os.path.exists(helpers.REF_GRU_GENERIC), reason="oracle/_ref GRU harness not built (needs /root/reference)")
+@pytest.mark.skipif(not (os.path.exists(helpers.REF_GRU_GENERIC) and os.path.exists(helpers.REF_GRU_FAST_GENERIC)), reason="oracle/_ref GRU harness not built (needs /root/reference)")
+@pytest.mark.parametrize("fast_tanh", [False, True])
 @pytest.mark.parametrize("with_reset", [False, True])
-def test_gru_forward_and_backward_through_time_bit_exact_with_reference(oracle, with_reset):
+def test_gru_forward_and_backward_through_time_bit_exact_with_reference(oracle, with_reset, fast_tanh):
     """The reference's own GRU layer (forward with kept intermediates, backward_full through 7 steps, optional per-sample resets) on random
-    weights and inputs: outputs, intermediates, d_input, the in-place accumulated d_output and all four gradients, bit for bit."""
-    ref = C.CDLL(helpers.REF_GRU_GENERIC)
+    weights and inputs: outputs, intermediates, d_input, the in-place accumulated d_output and all four gradients, bit for bit; with the
+    exact gate functions and with the FAST_TANH switch (a second build of the harness), whose inputs are scaled so that the clamp of the
+    rational approximation at |x| = 3 is reached."""
+    ref = C.CDLL(helpers.REF_GRU_FAST_GENERIC if fast_tanh else helpers.REF_GRU_GENERIC)
     dims = (C.c_int * 4)(); ref.rlt_ref_gru_dims(dims)
     S, B, I, H = list(dims)
     rng = np.random.default_rng(12 + with_reset)
     params, x, dy, reset = helpers.gru_random_case(rng, S, B, I, H, with_reset)
+    if fast_tanh:
+        x = (x * 6).astype(np.float32)
     want = dict(output=np.zeros((S, B, H), np.float32), post=np.zeros((S, B, 3 * H), np.float32), npp=np.zeros((S, B, H), np.float32), dx=np.zeros((S, B, I), np.float32),
                 dW_i=np.zeros((3 * H, I), np.float32), db_i=np.zeros(3 * H, np.float32), dW_h=np.zeros((3 * H, H), np.float32), db_h=np.zeros(3 * H, np.float32),
                 dy=np.zeros((S, B, H), np.float32))
@@ -372,12 +377,14 @@ def test_gru_forward_and_backward_through_time_bit_exact_with_reference(oracle, 
     assert ref.rlt_ref_gru_forward_backward(p(params["W_i"]), p(params["b_i"]), p(params["W_h"]), p(params["b_h"]), p(params["h0"]), p(x), p(reset) if with_reset else None,
                                             p(dy), p(want["output"]), p(want["post"]), p(want["npp"]), p(want["dx"]), p(want["dW_i"]), p(want["db_i"]), p(want["dW_h"]),
                                             p(want["db_h"]), p(want["dy"])) == 0
-    g = helpers.GruOnBackend(oracle, S, B, I, H, params)
+    g = helpers.GruOnBackend(oracle, S, B, I, H, params, fast_tanh=fast_tanh)
     g.forward(x, reset)
     g.backward(dy)
     got = g.results()
     if with_reset:
         assert reset[1:].sum() > 3
+    if fast_tanh:
+        assert (want["post"][..., :2 * H] == 1.0).any() or (want["post"][..., 2 * H:] == 1.0).any() or (np.abs(want["post"][..., 2 * H:]) == 1.0).any()   # the clamp was reached
     for k in want:
         assert np.array_equal(got[k], want[k]), (k, np.abs(got[k] - want[k]).max())
 
@@ -493,3 +500,54 @@ def test_on_policy_collect_and_observation_normalisation_bit_exact_with_referenc
         assert np.array_equal(a.parameters(), b.parameters()) and a.rng_state().value == b.rng_state().value
     assert n_collects == 4 and resets_inside >= n           # truncations in the middle of a dataset did occur
     a.close(); b.close()
+
+
+@pytest.mark.skipif(not (os.path.exists(helpers.ref_sac_gru_path(3)) and os.path.exists(helpers.ref_sac_gru_path(5))), reason="oracle/_ref recurrent SAC harness not built (needs /root/reference)")
+@pytest.mark.parametrize("n_layers", [3, 5])
+def test_sac_on_sequence_batches_bit_exact_with_reference(oracle, n_layers):
+    """The reference's own SAC loop with its recurrent approximators (dense -> GRU -> dense, and dense -> GRU -> GRU -> dense -> dense, FAST_TANH
+    gates) on sequence batches of 6 steps with the first step included in the targets. From the first training step on the restatement gets
+    the batch the reference trained on (all seven tensors as its gather_batch left them) and both noise tensors, and must reproduce every
+    parameter of the five networks, log_alpha and the four Adam ages bit for bit over 400 loop steps -- through the wrap of the 260-row rings,
+    with sequences that restart inside the batch, shortened sequences and final-step counts that are no powers of two. What that fixes
+    beyond the layers themselves: the `next` views starting at padded step 0, the target taking the value one step later but the
+    log-probability at the same index, the loss weight formed as (1 / n) * s, backward_input of the critics running without the resets
+    during the actor update, the log_alpha gradient divided by the number of set reset flags, polyak on the GRU tensors."""
+    ref = helpers.RefSacGru(n_layers, 4)
+    assert (ref.seq, ref.batch, ref.include_first) == (6, 16, 1)
+    assert [k for k, _, _, _ in ref.critic_specs] == ([0, 1, 0] if n_layers == 3 else [0, 1, 1, 0, 0])
+    for _ in range(ref.n_warmup):
+        ref.step()
+    agent = helpers.SacSequenceOnBackend(oracle, ref.actor_specs, ref.critic_specs, ref.parameters(), ref.seq, ref.batch, ref.obs_dim, ref.act_dim, True, ref.hyper())
+    restarts = odd_counts = 0
+    for i in range(400):
+        ref.step()
+        data = ref.batch_data()
+        agent.set_batch(data)
+        agent.train(*ref.noise())
+        got, want = agent.parameters(), ref.parameters()
+        assert np.array_equal(got, want), (i, np.abs(got - want).max())
+        restarts += int(data["reset"][1:].sum())
+        n = int(data["final_step_mask"].sum())
+        odd_counts += (n & (n - 1)) != 0
+    assert agent.ages() == ref.ages() == [401] * 4
+    assert restarts > 1000 and odd_counts > 300
+    ref.close()
+
+
+@pytest.mark.skipif(not (os.path.exists(helpers.ref_sac_gru_path(3)) and os.path.exists(helpers.ref_sac_gru_path(5))), reason="oracle/_ref recurrent SAC harness not built (needs /root/reference)")
+def test_sac_sequence_fixture_is_what_the_reference_gives():
+    g = helpers.sac_sequence_golden()
+    for n_layers in (3, 5):
+        p = f"l{n_layers}_"
+        ref = helpers.RefSacGru(n_layers, 4)
+        for _ in range(ref.n_warmup):
+            ref.step()
+        assert np.array_equal(ref.parameters(), g[p + "parameters_before"])
+        for i in range(int(g[p + "dims"][5])):
+            ref.step()
+            data = ref.batch_data()
+            assert all(np.array_equal(data[k], g[f"{p}s{i}_{k}"]) for k in helpers.SEQUENCE_BATCH_FIELDS)
+            if i in g[p + "snapshots"]:
+                assert np.array_equal(ref.parameters(), g[f"{p}s{i}_after"])
+        ref.close()
