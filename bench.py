@@ -281,6 +281,56 @@ def bench_gru(helpers, rocm, batch, S=64, I=146, H=64, iters=10):
     return {"batch": batch, "sequence_length": S, "ms_per_step": ms, "sequences_per_s": batch / (ms * 1e-3), "tflops": 211968.0 * rows / (ms * 1e-3) / 1e12}
 
 
+def bench_sac_sequence(helpers, rocm, S=100, B=100, iters=10, cpu_seconds=1.5):
+    """The training part of one SAC loop step on a sequence batch with the reference's recurrent approximators at the sizes of its Pendulum
+    configuration with memory (100 sequences of 100 steps; actor dense-GRU-GRU-dense at width 16, critics at width 32): 2 critic updates,
+    target update, actor update. The same calls on the CPU checker (one thread, plain loops) are timed next to it on a bounded sample."""
+    rng = np.random.default_rng(6)
+    OBS, ACT = 3, 1
+    actor_specs = [(0, OBS, 16, "relu"), (1, 16, 16, "identity"), (1, 16, 16, "identity"), (0, 16, 2 * ACT, "identity")]
+    critic_specs = [(0, OBS + ACT, 32, "relu"), (1, 32, 32, "identity"), (1, 32, 32, "identity"), (0, 32, 1, "identity")]
+    critics = [helpers.random_seq_params(rng, critic_specs) for _ in range(2)]
+    params = np.concatenate([helpers.random_seq_params(rng, actor_specs)] + critics + [c.copy() for c in critics] + [np.array([0.0], np.float32)])
+    final = (rng.uniform(size=(S, B)) < 0.05).astype(np.uint8); final[-1] = 1
+    reset = np.zeros((S, B), np.uint8); reset[0] = 1; reset[1:] = final[:-1]
+    next_reset = np.zeros((S + 1, B), np.uint8); next_reset[0] = 1; next_reset[1:] = final
+    next_final = np.zeros((S + 1, B), np.uint8); next_final[1:] = final
+    data = dict(observations_actions_base=rng.standard_normal((S + 1, B, OBS + ACT)).astype(np.float32), rewards=rng.standard_normal((S, B)).astype(np.float32),
+                terminated=np.zeros((S, B), np.uint8), reset=reset, next_reset_base=next_reset, final_step_mask=final, next_final_step_mask_base=next_final)
+    nc, na = rng.standard_normal((S + 1, B, ACT)).astype(np.float32), rng.standard_normal((S, B, ACT)).astype(np.float32)
+    out = {"sequence_length": S, "batch": B, "actor": "3-16-GRU16-GRU16-2", "critic": "4-32-GRU32-GRU32-1"}
+    for be in (rocm, helpers.HostBackend()):
+        agent = helpers.SacSequenceOnBackend(be, actor_specs, critic_specs, params, S, B, OBS, ACT, True)
+        agent.set_batch(data)
+        ncd, nad = be.array(nc), be.array(na)
+
+        def step():
+            for k in range(2):
+                be.call("sac_sequence_train_critic", C.byref(agent.c), k, ncd.ptr)
+            be.call("sac_sequence_update_critic_targets", C.byref(agent.c))
+            be.call("sac_sequence_train_actor", C.byref(agent.c), nad.ptr)
+        if be.name == "rocm":
+            ev = HipEvents(rocm.device.lib.rlt_rocm_get_stream(rocm.device.handle))
+            for _ in range(3):
+                step()
+            rocm.sync()
+            a = ev.record()
+            for _ in range(iters):
+                step()
+            e = ev.record()
+            ms = ev.elapsed_ms(a, e) / iters
+            out["ms_per_training_step"] = ms
+            out["sequences_per_s"] = 3 * B / (ms * 1e-3)
+        else:
+            step()
+            t0 = time.perf_counter(); n = 0
+            while time.perf_counter() - t0 < cpu_seconds:
+                step(); n += 1
+            out["cpu_checker_ms_per_training_step"] = (time.perf_counter() - t0) / n * 1e3
+            out["cpu_sample"] = f"{n} training steps of the CPU restatement, one thread"
+    return out
+
+
 def pmc_probe(helpers, rocm, batch):
     n = 64 * 1024 * 1024      # floats: 256 MiB read + 256 MiB written per copy
     src, dst = rocm.zeros((n,)), rocm.zeros((n,))
@@ -482,7 +532,7 @@ def main():
     ap.add_argument("--mlp-batch", type=int, default=65536)
     ap.add_argument("--mlp-iters", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "mlp", "sac", "env", "ppo", "gru"], default="all")
+    ap.add_argument("--only", choices=["all", "mlp", "sac", "env", "ppo", "gru", "seq"], default="all")
     ap.add_argument("--sac-phase-profile", action="store_true", help="print the persistent kernel's per-phase time (stderr)")
     ap.add_argument("--pmc-probe", action="store_true", help="for counter runs under rocprofv3 --pmc: three 256 MiB device copies (a kernel of known traffic, to scale the counters by) "
                     "and three MLP forward+backward calls, nothing timed")
@@ -505,7 +555,8 @@ def main():
     env = bench_env(helpers, rocm) if args.only in ("all", "env") else None
     ppo = bench_ppo(helpers, rocm) if args.only in ("all", "ppo") else None
     gru = [bench_gru(helpers, rocm, b) for b in (64, 1024)] if args.only in ("all", "gru") else None
-    cpu = None if (args.no_cpu_baseline or args.only in ("mlp", "env", "ppo", "gru")) else cpu_baseline()
+    seq = bench_sac_sequence(helpers, rocm) if args.only in ("all", "seq") else None
+    cpu = None if (args.no_cpu_baseline or args.only in ("mlp", "env", "ppo", "gru", "seq")) else cpu_baseline()
     line = {
         "metric": "SAC updates/sec (critic+actor) at batch 256; fused MLP fwd+bwd TFLOP/s",
         "value": sac["steps_per_s"], "unit": "SAC loop steps/s (each = 2 critic + 1 actor update)",
@@ -528,6 +579,8 @@ def main():
         line["ppo_iteration"] = ppo
     if gru:
         line["gru_training_step"] = gru
+    if seq:
+        line["sac_sequence_training_step"] = seq
     if cpu:
         line["cpu_baseline"] = cpu
         line["speedup_vs_cpu_baseline"] = sac["steps_per_s"] / cpu["value"] if cpu["value"] else None

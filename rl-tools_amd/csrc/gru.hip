@@ -110,111 +110,159 @@ __global__ __launch_bounds__(GRU_THREADS) void gru_backward_kernel(GruArgs A) {
     if (active && A.db_hn_partial) A.db_hn_partial[(size_t)b * H + j] = db_hn;
 }
 
-// ---- hidden width 64: one wavefront per batch row, W_h in registers ------------------------------------------------------------
-// Lane j owns hidden unit j of its row and keeps rows j, 64 + j, 128 + j of W_h (192 values) in registers for the whole sequence; the
-// previous hidden state reaches all lanes through 64 lane reads per step, so a step needs neither LDS nor a barrier, and the
-// wavefronts of a workgroup are independent (they only share the launch). The step's inputs W_i x + b_i are requested one step ahead.
-constexpr int HW = 64;
-
+// ---- hidden widths 64, 32 and 16: W_h in registers, no LDS, no barrier -------------------------------------------------------
+// A wavefront carries 64 / H batch rows; lane (row, j) owns hidden unit j of its row and keeps rows j, H + j, 2H + j of W_h (3H values) in
+// registers for the whole sequence. The previous hidden state reaches the lanes of its row through H lane reads per step at H = 64, where the
+// wavefront is one row, and through a 64-float slot of LDS private to the wavefront below that (one write, H / 4 broadcast reads of four
+// values); a step needs no workgroup barrier, and the wavefronts of a workgroup are independent (they only share the launch). The step's inputs W_i x + b_i
+// are requested one step ahead.
 __device__ __forceinline__ float lane_read(float x, int k) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), k)); }
+// lanes of one wavefront exchange data through LDS: the hardware executes a wavefront's LDS instructions in order, the fences keep the
+// compiler from moving them across
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 
-__global__ __launch_bounds__(GRU_THREADS) void gru_forward64_kernel(GruArgs A) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int b = blockIdx.x * (GRU_THREADS / 64) + wave;
-    if (b >= A.B) return;                                   // whole wavefronts leave; no barrier follows
-    float wr[HW], wz[HW], wn[HW];
+template <int H>
+__global__ __launch_bounds__(GRU_THREADS) void gru_forward_reg_kernel(GruArgs A) {
+    constexpr int G = 64 / H;                               // batch rows per wavefront
+    __shared__ __align__(16) float exchange[GRU_THREADS / 64][1][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, u = lane & (H - 1), row_base = lane & ~(H - 1);
+    const int b = (blockIdx.x * (GRU_THREADS / 64) + wave) * G + lane / H;
+    if (b >= A.B) return;                                   // the lanes of whole rows leave; lane reads stay within a row; no barrier follows
+    float wr[H], wz[H], wn[H];
     {
-        const float4* r4 = reinterpret_cast<const float4*>(A.L.weights_hidden + (size_t)lane * HW);
-        const float4* z4 = reinterpret_cast<const float4*>(A.L.weights_hidden + (size_t)(HW + lane) * HW);
-        const float4* n4 = reinterpret_cast<const float4*>(A.L.weights_hidden + (size_t)(2 * HW + lane) * HW);
+        const float4* r4 = reinterpret_cast<const float4*>(A.L.weights_hidden + (size_t)u * H);
+        const float4* z4 = reinterpret_cast<const float4*>(A.L.weights_hidden + (size_t)(H + u) * H);
+        const float4* n4 = reinterpret_cast<const float4*>(A.L.weights_hidden + (size_t)(2 * H + u) * H);
 #pragma unroll
-        for (int q = 0; q < HW / 4; q++) {
+        for (int q = 0; q < H / 4; q++) {
             const float4 a = r4[q], c = z4[q], d = n4[q];
             wr[4 * q] = a.x; wr[4 * q + 1] = a.y; wr[4 * q + 2] = a.z; wr[4 * q + 3] = a.w;
             wz[4 * q] = c.x; wz[4 * q + 1] = c.y; wz[4 * q + 2] = c.z; wz[4 * q + 3] = c.w;
             wn[4 * q] = d.x; wn[4 * q + 1] = d.y; wn[4 * q + 2] = d.z; wn[4 * q + 3] = d.w;
         }
     }
-    const float bhr = A.L.biases_hidden[lane], bhz = A.L.biases_hidden[HW + lane], bhn = A.L.biases_hidden[2 * HW + lane];
-    const float h0 = A.L.initial_hidden_state[lane];
+    const float bhr = A.L.biases_hidden[u], bhz = A.L.biases_hidden[H + u], bhn = A.L.biases_hidden[2 * H + u];
+    const float h0 = A.L.initial_hidden_state[u];
     float h = h0;
-    const size_t stride = (size_t)A.B * 3 * HW;
-    float* post = A.L.post_activation + (size_t)b * 3 * HW;
-    float xr = post[lane], xz = post[HW + lane], xn = post[2 * HW + lane];
+    const size_t stride = (size_t)A.B * 3 * H;
+    float* post = A.L.post_activation + (size_t)b * 3 * H;
+    float xr = post[u], xz = post[H + u], xn = post[2 * H + u];
     int rs = A.reset ? A.reset[b] : 0;
+    // the inputs of the step after are already on their way (two steps of distance: consecutive steps lie 12 H B bytes apart, on other pages)
+    const int t1 = A.S > 1 ? 1 : 0;
+    const float* p1 = A.L.post_activation + (size_t)t1 * stride + (size_t)b * 3 * H;
+    float nxr = p1[u], nxz = p1[H + u], nxn = p1[2 * H + u];
+    int nrs = A.reset ? A.reset[(size_t)t1 * A.B + b] : 0;
     for (int t = 0; t < A.S; t++) {
-        // next step's inputs (the last step requests its own again: no branch around the loads)
-        const int tn = t + 1 < A.S ? t + 1 : t;
-        const float* pn = A.L.post_activation + (size_t)tn * stride + (size_t)b * 3 * HW;
-        const float nxr = pn[lane], nxz = pn[HW + lane], nxn = pn[2 * HW + lane];
-        const int nrs = A.reset ? A.reset[(size_t)tn * A.B + b] : 0;
+        // the inputs two steps ahead (the last steps request the last one again: no branch around the loads)
+        const int tn = t + 2 < A.S ? t + 2 : A.S - 1;
+        const float* pn = A.L.post_activation + (size_t)tn * stride + (size_t)b * 3 * H;
+        const float nnxr = pn[u], nnxz = pn[H + u], nnxn = pn[2 * H + u];
+        const int nnrs = A.reset ? A.reset[(size_t)tn * A.B + b] : 0;
         if (t == 0 || rs) h = h0;
         float ar = bhr, az = bhz, an = bhn;
+        if (H == 64) {       // measured: 64 scalar lane reads beat the LDS slot here (60 against 67 us for 64 steps), in the reverse pass they lose (103 against 64 us)
 #pragma unroll
-        for (int k = 0; k < HW; k++) { const float hk = lane_read(h, k); ar += hk * wr[k]; az += hk * wz[k]; an += hk * wn[k]; }
+            for (int k = 0; k < H; k++) { const float hk = lane_read(h, k); ar += hk * wr[k]; az += hk * wz[k]; an += hk * wn[k]; }
+        } else {
+            float* xw = &exchange[wave][0][0];
+            xw[lane] = h;
+            wave_sync();
+#pragma unroll
+            for (int k = 0; k < H; k += 4) {
+                const float4 hv = *reinterpret_cast<const float4*>(xw + row_base + k);
+                ar += hv.x * wr[k]; az += hv.x * wz[k]; an += hv.x * wn[k];
+                ar += hv.y * wr[k + 1]; az += hv.y * wz[k + 1]; an += hv.y * wn[k + 1];
+                ar += hv.z * wr[k + 2]; az += hv.z * wz[k + 2]; an += hv.z * wn[k + 2];
+                ar += hv.w * wr[k + 3]; az += hv.w * wz[k + 3]; an += hv.w * wn[k + 3];
+            }
+            wave_sync();
+        }
         const float r = gate_sigmoid(xr + ar, A.L.fast_tanh), z = gate_sigmoid(xz + az, A.L.fast_tanh);
         const float n = gate_tanh(xn + an * r, A.L.fast_tanh);
-        float* po = A.L.post_activation + (size_t)t * stride + (size_t)b * 3 * HW;
-        po[lane] = r; po[HW + lane] = z; po[2 * HW + lane] = n;
-        const size_t at = ((size_t)t * A.B + b) * HW + lane;
+        float* po = A.L.post_activation + (size_t)t * stride + (size_t)b * 3 * H;
+        po[u] = r; po[H + u] = z; po[2 * H + u] = n;
+        const size_t at = ((size_t)t * A.B + b) * H + u;
         A.L.n_pre_pre_activation[at] = an;
         h = (1.0f - z) * n + z * h;
         A.L.output[at] = h;
         xr = nxr; xz = nxz; xn = nxn; rs = nrs;
+        nxr = nnxr; nxz = nnxz; nxn = nnxn; nrs = nnrs;
     }
 }
 
-// Reverse pass at hidden width 64: lane k keeps column k of W_h (the 192 weights that multiply the gate gradients on the way to
-// d h_prev[k]); the gate gradients of the 64 units reach all lanes through lane reads.
-__global__ __launch_bounds__(GRU_THREADS) void gru_backward64_kernel(GruArgs A) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int b = blockIdx.x * (GRU_THREADS / 64) + wave;
+// Reverse pass at these widths: lane (row, k) keeps column k of W_h (the 3H weights that multiply the gate gradients on the way to
+// d h_prev[k]); the gate gradients of the row's H units reach its lanes through three 64-float slots of LDS private to the wavefront.
+template <int H>
+__global__ __launch_bounds__(GRU_THREADS) void gru_backward_reg_kernel(GruArgs A) {
+    constexpr int G = 64 / H;
+    __shared__ __align__(16) float exchange[GRU_THREADS / 64][3][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, u = lane & (H - 1), row_base = lane & ~(H - 1);
+    const int b = (blockIdx.x * (GRU_THREADS / 64) + wave) * G + lane / H;
     if (b >= A.B) return;
-    float cr[HW], cz[HW], cn[HW];
+    float cr[H], cz[H], cn[H];
 #pragma unroll
-    for (int j = 0; j < HW; j++) {
-        cr[j] = A.L.weights_hidden[(size_t)j * HW + lane]; cz[j] = A.L.weights_hidden[(size_t)(HW + j) * HW + lane]; cn[j] = A.L.weights_hidden[(size_t)(2 * HW + j) * HW + lane];
+    for (int j = 0; j < H; j++) {
+        cr[j] = A.L.weights_hidden[(size_t)j * H + u]; cz[j] = A.L.weights_hidden[(size_t)(H + j) * H + u]; cn[j] = A.L.weights_hidden[(size_t)(2 * H + j) * H + u];
     }
-    const float h0 = A.L.initial_hidden_state[lane];
+    const float h0 = A.L.initial_hidden_state[u];
     float carry = 0.f, db_hn = 0.f;
-    // this step's saved values are requested one step ahead
-    size_t at = (size_t)(A.S - 1) * A.B + b;
-    float r = A.L.post_activation[at * 3 * HW + lane], z = A.L.post_activation[at * 3 * HW + HW + lane], n = A.L.post_activation[at * 3 * HW + 2 * HW + lane];
-    float npp = A.L.n_pre_pre_activation[at * HW + lane], dy = A.d_output[at * HW + lane];
-    float hp_raw = A.S > 1 ? A.L.output[((size_t)(A.S - 2) * A.B + b) * HW + lane] : 0.f;
-    int rs = A.reset ? A.reset[at] : 0;
+    // a step's saved values are requested two steps ahead (consecutive steps lie on different pages); steps before the first read the first again
+    struct Saved { float r, z, n, npp, dy, hp; int rs; };
+    auto request = [&](int t) {
+        const size_t a = (size_t)(t > 0 ? t : 0) * A.B + b;
+        Saved v;
+        v.r = A.L.post_activation[a * 3 * H + u]; v.z = A.L.post_activation[a * 3 * H + H + u]; v.n = A.L.post_activation[a * 3 * H + 2 * H + u];
+        v.npp = A.L.n_pre_pre_activation[a * H + u]; v.dy = A.d_output[a * H + u];
+        v.hp = A.L.output[((size_t)(t > 1 ? t - 1 : 0) * A.B + b) * H + u];
+        v.rs = A.reset ? A.reset[a] : 0;
+        return v;
+    };
+    Saved cur = request(A.S - 1), nxt = request(A.S - 2);
     for (int t = A.S - 1; t >= 0; t--) {
-        at = (size_t)t * A.B + b;
-        const int tp = t > 0 ? t - 1 : 0;
-        const size_t ap = (size_t)tp * A.B + b;
-        const float pr = A.L.post_activation[ap * 3 * HW + lane], pz = A.L.post_activation[ap * 3 * HW + HW + lane], pnn = A.L.post_activation[ap * 3 * HW + 2 * HW + lane];
-        const float pnpp = A.L.n_pre_pre_activation[ap * HW + lane], pdy = A.d_output[ap * HW + lane];
-        const float php = A.L.output[((size_t)(tp > 0 ? tp - 1 : 0) * A.B + b) * HW + lane];
-        const int prs = A.reset ? A.reset[ap] : 0;
+        const size_t at = (size_t)t * A.B + b;
+        const Saved far = request(t - 2);
+        const float r = cur.r, z = cur.z, n = cur.n, npp = cur.npp, dy = cur.dy, hp_raw = cur.hp;
+        const int rs = cur.rs;
         const bool from_initial = t == 0 || rs;
         const float hp = from_initial ? h0 : hp_raw;
         const float dh = dy + carry;
-        A.d_output[at * HW + lane] = dh;
+        A.d_output[at * H + u] = dh;
         const float gz = dh * (hp - n) * z * (1.0f - z);
         const float gn = dh * (1.0f - z) * (1.0f - n * n);
         const float gr = gn * npp * r * (1.0f - r);
         const float gnr = gn * r;
-        float* bi = A.buffer_input + at * 3 * HW; float* bh = A.buffer_hidden + at * 3 * HW;
-        bi[lane] = gr; bi[HW + lane] = gz; bi[2 * HW + lane] = gn;
-        bh[lane] = gr; bh[HW + lane] = gz; bh[2 * HW + lane] = gnr;
-        A.h_previous[at * HW + lane] = hp;
+        float* bi = A.buffer_input + at * 3 * H; float* bh = A.buffer_hidden + at * 3 * H;
+        bi[u] = gr; bi[H + u] = gz; bi[2 * H + u] = gn;
+        bh[u] = gr; bh[H + u] = gz; bh[2 * H + u] = gnr;
+        A.h_previous[at * H + u] = hp;
         // the reference drops reset samples (t > 0) from the b_hn gradient (their buffer rows are zeroed before that sum, :716-749)
         if (!(t > 0 && from_initial)) db_hn += gnr;
-        carry = 0.f;
-        if (!from_initial) {        // uniform over the wavefront: one row
-            float a0 = dh * z, a1 = 0.f, a2 = 0.f;
+        // the rows of one wavefront restart at different steps: every lane forms the sum, a restarting row drops it
+        float a0 = dh * z, a1 = 0.f, a2 = 0.f;
+        {
+            float* xw = &exchange[wave][0][0];
+            xw[lane] = gr; xw[64 + lane] = gz; xw[128 + lane] = gnr;
+            wave_sync();
 #pragma unroll
-            for (int j = 0; j < HW; j++) { a0 += lane_read(gr, j) * cr[j]; a1 += lane_read(gz, j) * cz[j]; a2 += lane_read(gnr, j) * cn[j]; }
-            carry = a0 + (a1 + a2);
+            for (int j = 0; j < H; j += 4) {
+                const float4 vr = *reinterpret_cast<const float4*>(xw + row_base + j), vz = *reinterpret_cast<const float4*>(xw + 64 + row_base + j),
+                             vn = *reinterpret_cast<const float4*>(xw + 128 + row_base + j);
+                a0 += vr.x * cr[j]; a1 += vz.x * cz[j]; a2 += vn.x * cn[j];
+                a0 += vr.y * cr[j + 1]; a1 += vz.y * cz[j + 1]; a2 += vn.y * cn[j + 1];
+                a0 += vr.z * cr[j + 2]; a1 += vz.z * cz[j + 2]; a2 += vn.z * cn[j + 2];
+                a0 += vr.w * cr[j + 3]; a1 += vz.w * cz[j + 3]; a2 += vn.w * cn[j + 3];
+            }
+            wave_sync();
         }
-        r = pr; z = pz; n = pnn; npp = pnpp; dy = pdy; hp_raw = php; rs = prs;
+        carry = from_initial ? 0.f : a0 + (a1 + a2);
+        cur = nxt; nxt = far;
     }
-    if (A.db_hn_partial) A.db_hn_partial[(size_t)b * HW + lane] = db_hn;
+    if (A.db_hn_partial) A.db_hn_partial[(size_t)b * H + u] = db_hn;
 }
 
 // db_h[n part] += sum over batch rows of the per-row sums, db_h[r, z parts] = db_i[r, z parts] (the reference copies, :679-681).
@@ -258,8 +306,11 @@ int rlt_rocm_gru_forward(rlt_rocm_device* device, const rlt_gru_layer* L, const 
     int rc = rlt_gemm_forward(device, input, L->input_dim, L->weights_input, L->biases_input, RLT_ACT_IDENTITY, nullptr, nullptr, L->post_activation, 3 * H, S * B, L->input_dim, 3 * H);
     if (rc) return rc;
     GruArgs a = {}; a.L = *L; a.input = input; a.reset = reset; a.S = S; a.B = B; a.rows_per_group = rows_per_group(H);
-    if (H == HW) {
-        hipLaunchKernelGGL(gru_forward64_kernel, dim3(rlt_div_up(B, GRU_THREADS / 64)), dim3(GRU_THREADS), 0, device->stream, a);
+    if (H == 64 || H == 32 || H == 16) {
+        const dim3 grid(rlt_div_up(B, GRU_THREADS / H)), block(GRU_THREADS);      // GRU_THREADS / 64 wavefronts of 64 / H rows
+        if (H == 64) hipLaunchKernelGGL(gru_forward_reg_kernel<64>, grid, block, 0, device->stream, a);
+        else if (H == 32) hipLaunchKernelGGL(gru_forward_reg_kernel<32>, grid, block, 0, device->stream, a);
+        else hipLaunchKernelGGL(gru_forward_reg_kernel<16>, grid, block, 0, device->stream, a);
         return rlt_launch_status(device);
     }
     const size_t lds = lds_bytes(H, false);
@@ -283,8 +334,12 @@ int rlt_rocm_gru_backward(rlt_rocm_device* device, const rlt_gru_layer* L, const
     float* db_hn_partial = (float*)w;
     GruArgs a = {}; a.L = *L; a.input = input; a.reset = reset; a.d_output = d_output; a.buffer_input = buffer_input; a.buffer_hidden = buffer_hidden;
     a.h_previous = h_previous; a.db_hn_partial = want_weight_gradients ? db_hn_partial : nullptr; a.S = S; a.B = B; a.rows_per_group = rows_per_group(H);
-    if (H == HW) hipLaunchKernelGGL(gru_backward64_kernel, dim3(rlt_div_up(B, GRU_THREADS / 64)), dim3(GRU_THREADS), 0, device->stream, a);
-    else {
+    if (H == 64 || H == 32 || H == 16) {
+        const dim3 grid(rlt_div_up(B, GRU_THREADS / H)), block(GRU_THREADS);
+        if (H == 64) hipLaunchKernelGGL(gru_backward_reg_kernel<64>, grid, block, 0, device->stream, a);
+        else if (H == 32) hipLaunchKernelGGL(gru_backward_reg_kernel<32>, grid, block, 0, device->stream, a);
+        else hipLaunchKernelGGL(gru_backward_reg_kernel<16>, grid, block, 0, device->stream, a);
+    } else {
         const size_t lds = lds_bytes(H, true);
         RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gru_backward_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         hipLaunchKernelGGL(gru_backward_kernel, dim3(rlt_div_up(B, a.rows_per_group)), dim3(GRU_THREADS), lds, device->stream, a);
