@@ -125,7 +125,7 @@ __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <int H>
+template <int H, bool FAST>
 __global__ __launch_bounds__(GRU_THREADS) void gru_forward_reg_kernel(GruArgs A) {
     constexpr int G = 64 / H;                               // batch rows per wavefront
     __shared__ __align__(16) float exchange[GRU_THREADS / 64][1][64];
@@ -152,17 +152,22 @@ __global__ __launch_bounds__(GRU_THREADS) void gru_forward_reg_kernel(GruArgs A)
     float* post = A.L.post_activation + (size_t)b * 3 * H;
     float xr = post[u], xz = post[H + u], xn = post[2 * H + u];
     int rs = A.reset ? A.reset[b] : 0;
-    // the inputs of the step after are already on their way (two steps of distance: consecutive steps lie 12 H B bytes apart, on other pages)
-    const int t1 = A.S > 1 ? 1 : 0;
-    const float* p1 = A.L.post_activation + (size_t)t1 * stride + (size_t)b * 3 * H;
-    float nxr = p1[u], nxz = p1[H + u], nxn = p1[2 * H + u];
-    int nrs = A.reset ? A.reset[(size_t)t1 * A.B + b] : 0;
+    // The inputs of later steps are requested D steps ahead and wait in a queue of D - 1 entries. Consecutive steps lie 12 H B bytes apart, on
+    // other pages; two steps of distance pay at widths 16 and 32 (85 -> 59 us for 101 steps at 32), at 64 one step measures faster (60 against 67 us).
+    constexpr int D = H == 64 ? 1 : 2, Q = D > 1 ? D - 1 : 1;
+    float qr[Q], qz[Q], qn[Q]; int qs[Q];
+#pragma unroll
+    for (int d = 0; d < D - 1; d++) {
+        const int tq = d + 1 < A.S ? d + 1 : A.S - 1;
+        const float* pq = A.L.post_activation + (size_t)tq * stride + (size_t)b * 3 * H;
+        qr[d] = pq[u]; qz[d] = pq[H + u]; qn[d] = pq[2 * H + u]; qs[d] = A.reset ? A.reset[(size_t)tq * A.B + b] : 0;
+    }
     for (int t = 0; t < A.S; t++) {
-        // the inputs two steps ahead (the last steps request the last one again: no branch around the loads)
-        const int tn = t + 2 < A.S ? t + 2 : A.S - 1;
+        // (the last steps request the last one again: no branch around the loads)
+        const int tn = t + D < A.S ? t + D : A.S - 1;
         const float* pn = A.L.post_activation + (size_t)tn * stride + (size_t)b * 3 * H;
-        const float nnxr = pn[u], nnxz = pn[H + u], nnxn = pn[2 * H + u];
-        const int nnrs = A.reset ? A.reset[(size_t)tn * A.B + b] : 0;
+        const float fr = pn[u], fz = pn[H + u], fn = pn[2 * H + u];
+        const int fs = A.reset ? A.reset[(size_t)tn * A.B + b] : 0;
         if (t == 0 || rs) h = h0;
         float ar = bhr, az = bhz, an = bhn;
         if (H == 64) {       // measured: 64 scalar lane reads beat the LDS slot here (60 against 67 us for 64 steps), in the reverse pass they lose (103 against 64 us)
@@ -182,16 +187,21 @@ __global__ __launch_bounds__(GRU_THREADS) void gru_forward_reg_kernel(GruArgs A)
             }
             wave_sync();
         }
-        const float r = gate_sigmoid(xr + ar, A.L.fast_tanh), z = gate_sigmoid(xz + az, A.L.fast_tanh);
-        const float n = gate_tanh(xn + an * r, A.L.fast_tanh);
+        const float r = gate_sigmoid(xr + ar, FAST), z = gate_sigmoid(xz + az, FAST);
+        const float n = gate_tanh(xn + an * r, FAST);
         float* po = A.L.post_activation + (size_t)t * stride + (size_t)b * 3 * H;
         po[u] = r; po[H + u] = z; po[2 * H + u] = n;
         const size_t at = ((size_t)t * A.B + b) * H + u;
         A.L.n_pre_pre_activation[at] = an;
         h = (1.0f - z) * n + z * h;
         A.L.output[at] = h;
-        xr = nxr; xz = nxz; xn = nxn; rs = nrs;
-        nxr = nnxr; nxz = nnxz; nxn = nnxn; nrs = nnrs;
+        if (D == 1) { xr = fr; xz = fz; xn = fn; rs = fs; }
+        else {
+            xr = qr[0]; xz = qz[0]; xn = qn[0]; rs = qs[0];
+#pragma unroll
+            for (int d = 0; d + 1 < D - 1; d++) { qr[d] = qr[d + 1]; qz[d] = qz[d + 1]; qn[d] = qn[d + 1]; qs[d] = qs[d + 1]; }
+            qr[Q - 1] = fr; qz[Q - 1] = fz; qn[Q - 1] = fn; qs[Q - 1] = fs;
+        }
     }
 }
 
@@ -308,9 +318,10 @@ int rlt_rocm_gru_forward(rlt_rocm_device* device, const rlt_gru_layer* L, const 
     GruArgs a = {}; a.L = *L; a.input = input; a.reset = reset; a.S = S; a.B = B; a.rows_per_group = rows_per_group(H);
     if (H == 64 || H == 32 || H == 16) {
         const dim3 grid(rlt_div_up(B, GRU_THREADS / H)), block(GRU_THREADS);      // GRU_THREADS / 64 wavefronts of 64 / H rows
-        if (H == 64) hipLaunchKernelGGL(gru_forward_reg_kernel<64>, grid, block, 0, device->stream, a);
-        else if (H == 32) hipLaunchKernelGGL(gru_forward_reg_kernel<32>, grid, block, 0, device->stream, a);
-        else hipLaunchKernelGGL(gru_forward_reg_kernel<16>, grid, block, 0, device->stream, a);
+        const bool fast = L->fast_tanh != 0;      // a template parameter: as a run-time switch inside the step it cost 10% at width 64
+        if (H == 64) { if (fast) hipLaunchKernelGGL((gru_forward_reg_kernel<64, true>), grid, block, 0, device->stream, a); else hipLaunchKernelGGL((gru_forward_reg_kernel<64, false>), grid, block, 0, device->stream, a); }
+        else if (H == 32) { if (fast) hipLaunchKernelGGL((gru_forward_reg_kernel<32, true>), grid, block, 0, device->stream, a); else hipLaunchKernelGGL((gru_forward_reg_kernel<32, false>), grid, block, 0, device->stream, a); }
+        else { if (fast) hipLaunchKernelGGL((gru_forward_reg_kernel<16, true>), grid, block, 0, device->stream, a); else hipLaunchKernelGGL((gru_forward_reg_kernel<16, false>), grid, block, 0, device->stream, a); }
         return rlt_launch_status(device);
     }
     const size_t lds = lds_bytes(H, false);
