@@ -32,6 +32,10 @@
  *   (oracle/_ref/librlt_ref_gather_seq_generic.so; sequence length 8 with and without the default sampling switches, and 1), draws made on the
  *   reference's std::mt19937 in its order; golden vectors; structural invariants on synthetic rings.
  *   ppo train_epoch: the loop over ppo train_minibatch (pinned above) that the reference's train() runs per epoch.
+ *   sequential models (dense / GRU layers, FAST_TANH gates) and sac train_critic / train_actor / target update on sequence batches
+ *   (rlt_oracle_seq.cpp): every parameter bit for bit against the reference's SAC loop with its recurrent approximators over 400 loop steps at two
+ *   depths (oracle/_ref/librlt_ref_sac_gru{3,5}_generic.so), the FAST_TANH gates also on the GRU layer alone (librlt_ref_gru_fast_generic.so);
+ *   golden vectors; equality with the single-step update at sequence length 1, finite differences of a dense-GRU-GRU-dense model.
  */
 #ifndef RLT_ORACLE_H
 #define RLT_ORACLE_H
