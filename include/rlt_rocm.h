@@ -458,6 +458,11 @@ int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_ru
                                   const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas,
                                   const float* actions_in, const float* action_noise,
                                   const float* initial_states, uint64_t seed, uint64_t offset);
+/* The same runner step with a sequential (recurrent) policy whose last layer yields [mean | log_std]
+ * (rl/components/off_policy_runner/operations_generic.h:189-206): the policy state of the environments that start a new
+ * episode is reset, then one evaluate_step in Rollout mode (sample_and_squash with action_noise [n_envs x 1]).
+ * Declared after rlt_seq_layer / rlt_seq_state. */
+
 
 /* rl::utils::evaluation::evaluate  rl/utils/evaluation/operations_generic.h:106-233 (called by the evaluation loop step,
  * rl/loop/steps/evaluation/operations_generic.h:56-92) for the Pendulum environment: n_episodes episodes of step_limit steps
@@ -640,6 +645,33 @@ int rlt_rocm_seq_backward(rlt_rocm_device* device, const rlt_seq_layer* layers, 
                           int want_weight_gradients, int reset_in_backward_input, void* workspace, size_t workspace_bytes);
 int rlt_rocm_seq_zero_gradient(rlt_rocm_device* device, const rlt_seq_layer* layers, int n_layers);
 size_t rlt_rocm_seq_workspace_bytes(const rlt_seq_layer* layers, int n_layers, int steps, int batch);
+
+/* What a sequential model carries from one rollout step to the next (nn/layers/gru/layer.h State: hidden state and the
+ * number of steps since its last reset, per batch row), indexed by layer; entries at dense layers are unused. */
+#define RLT_SEQ_MAX_LAYERS 8
+typedef struct rlt_seq_state {
+    float* hidden[RLT_SEQ_MAX_LAYERS];     /* [batch x H] */
+    uint32_t* step[RLT_SEQ_MAX_LAYERS];    /* [batch] */
+} rlt_seq_state;
+/* reset(model, state, mode)   nn_models/sequential/operations_generic.h:35-41, nn/layers/gru/operations_generic.h:87-120
+ *   rows whose mask byte is set (all rows if mask == NULL) start again: hidden <- initial_hidden_state, step <- 0. */
+int rlt_rocm_seq_reset_state(rlt_rocm_device* device, const rlt_seq_layer* layers, int n_layers, const rlt_seq_state* state,
+                             const uint8_t* mask, int batch);
+/* evaluate_step(model, input, state, output)   nn_models/sequential/operations_generic.h:303-327, nn/layers/gru/operations_generic.h:348-416
+ *   one step of every layer on x [batch x in] (leading dimension ldx); GRU layers read and advance their state and, like the
+ *   reference outside its NoAutoResetMode, start again from the initial hidden state once a row has run auto_reset_period
+ *   steps (the SEQUENCE_LENGTH of the model's input shape; 0 switches that off). y [batch x out] with leading dimension ldy.
+ *   The layers' kept intermediates are not touched. */
+int rlt_rocm_seq_evaluate_step(rlt_rocm_device* device, const rlt_seq_layer* layers, int n_layers, const float* x, int ldx,
+                               const rlt_seq_state* state, int auto_reset_period, float* y, int ldy, int batch,
+                               void* workspace, size_t workspace_bytes);
+size_t rlt_rocm_seq_evaluate_step_workspace_bytes(const rlt_seq_layer* layers, int n_layers, int batch);
+/* runner step with a recurrent policy (see rlt_rocm_pendulum_runner_step) and the workspace it needs */
+size_t rlt_rocm_pendulum_runner_step_recurrent_workspace_bytes(const rlt_seq_layer* policy, int n_policy_layers, int n_envs);
+int rlt_rocm_pendulum_runner_step_recurrent(rlt_rocm_device* device, const rlt_pendulum_runner* runner, const rlt_replay_buffer* rb,
+                                            const rlt_seq_layer* policy, int n_policy_layers, const rlt_seq_state* policy_state,
+                                            int auto_reset_period, const rlt_sas_parameters* sas, const float* action_noise,
+                                            const float* initial_states, void* workspace, size_t workspace_bytes);
 
 /* Everything one SAC agent with sequential (recurrent) networks owns on the device: rl/algorithms/sac/sac.h:62-145 for
  * SEQUENCE_LENGTH >= 1 and the batch of rl/components/off_policy_runner/off_policy_runner.h:102-156 as

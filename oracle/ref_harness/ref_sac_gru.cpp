@@ -121,6 +121,17 @@ template <typename M> void model_dims(M& m, std::vector<int>& out) {
     layer_dims(m.content, out, 0);
     if constexpr (!rlt::utils::typing::is_same_v<typename M::NEXT_MODULE, rlt::nn_models::sequential::OutputModule>) model_dims(m.next_module, out);
 }
+// the policy state of the runner's actor (policy index 1): per GRU layer the hidden state [N_ENVS x H] and the step counters [N_ENVS]
+template <typename S> auto layer_state(DEVICE& device, S& s, std::vector<float>& hidden, std::vector<uint32_t>& steps, int) -> decltype(s.step, void()) {
+    constexpr size_t H = rlt::get<1>(typename decltype(s.state)::SPEC::SHAPE{});
+    const float* p = rlt::data(s.state); hidden.insert(hidden.end(), p, p + N_ENVS * H);
+    for (TI i = 0; i < N_ENVS; i++) steps.push_back((uint32_t)rlt::get(device, s.step, i));
+}
+template <typename S> void layer_state(DEVICE&, S&, std::vector<float>&, std::vector<uint32_t>&, long) {}
+template <typename CS> void walk_state(DEVICE& device, CS& cs, std::vector<float>& hidden, std::vector<uint32_t>& steps) {
+    layer_state(device, cs.state, hidden, steps, 0);
+    if constexpr (!rlt::utils::typing::is_same_v<typename CS::NEXT_CONTENT_STATE, rlt::nn_models::sequential::OutputModule>) walk_state(device, cs.next_content_state, hidden, steps);
+}
 std::vector<float> all_parameters(Loop& L) {
     auto& ac = L.ts.actor_critic;
     std::vector<float> out;
@@ -195,6 +206,79 @@ void rlt_ref_sac_gru_get_critic_buffers(void* h, int k, float* target_action_val
     std::memcpy(d_output, rlt::data(tb.d_output), sizeof(float) * SEQ * BATCH);
     std::memcpy(next_q_1, rlt::data(tb.next_state_action_value_critic_1), sizeof(float) * (SEQ + 1) * BATCH);
     std::memcpy(next_q_2, rlt::data(tb.next_state_action_value_critic_2), sizeof(float) * (SEQ + 1) * BATCH);
+}
+// One loop step past the warm-up assembled from the reference's own operations in the order of sac::loop::core::step, so that what the runner step draws
+// can be written out: before it the engine is copied and the same draws are taken from the copy with the reference's own functions (per environment that
+// starts a new episode: parameters, initial state; then one N(0,1) value per environment for the sample_and_squash layer). Returns 1 if the copy then
+// equals the engine, i.e. exactly these draws were made. Tests compare everything after this with a second loop advanced with rlt_ref_sac_gru_step.
+int rlt_ref_sac_gru_manual_step(void* h, float* initial_states, float* action_noise, uint8_t* reset_flags) {
+    auto& L = *static_cast<Loop*>(h);
+    auto& device = L.device; auto& ts = L.ts; auto& runner = ts.off_policy_runner;
+    using CP = CONFIG::CORE_PARAMETERS; using P = CP::SAC_PARAMETERS;
+    if (ts.step < CP::N_WARMUP_STEPS) return -1;
+    rlt::set_step(device, device.logger, ts.step);
+    RNG copy = ts.rng;
+    const bool policy_switch = runner.previous_policy_set && runner.previous_policy != 1;      // the first step after the warm-up truncates every episode
+    for (TI e = 0; e < N_ENVS; e++) {
+        reset_flags[e] = policy_switch || rlt::get(runner.truncated, 0, e);
+        initial_states[2 * e] = initial_states[2 * e + 1] = 0;
+        if (reset_flags[e]) {
+            auto& env = rlt::get(runner.envs, 0, e);
+            auto parameters = rlt::get(runner.env_parameters, 0, e);
+            typename ENVIRONMENT::State state;
+            if (CONFIG::OFF_POLICY_RUNNER_PARAMETERS::SAMPLE_PARAMETERS) rlt::sample_initial_parameters(device, env, parameters, copy);
+            rlt::sample_initial_state(device, env, parameters, state, copy);
+            initial_states[2 * e] = state.theta; initial_states[2 * e + 1] = state.theta_dot;
+        }
+    }
+    for (TI e = 0; e < N_ENVS; e++) action_noise[e] = rlt::random::normal_distribution::sample(device.random, 0.0f, 1.0f, copy);
+    rlt::step<1>(device, runner, rlt::get_actor(ts), ts.actor_buffers_eval, ts.rng);
+    const int same = copy.engine == ts.rng.engine;
+    const bool train_critic_flag = ts.step >= CP::N_WARMUP_STEPS_CRITIC && ts.step % P::CRITIC_TRAINING_INTERVAL == 0;
+    const bool update_critic_targets_flag = ts.step >= CP::N_WARMUP_STEPS_CRITIC && ts.step % P::CRITIC_TARGET_UPDATE_INTERVAL == 0;
+    const bool train_actor_flag = ts.step >= CP::N_WARMUP_STEPS_ACTOR && ts.step % P::ACTOR_TRAINING_INTERVAL == 0;
+    static_assert(CP::SHARED_BATCH);
+    if (train_critic_flag || train_actor_flag) { rlt::gather_batch(device, runner, ts.critic_batch, ts.rng); rlt::randn(device, ts.action_noise_critic, ts.rng); }
+    if (train_critic_flag)
+        for (int i = 0; i < 2; i++)
+            rlt::train_critic(device, ts.actor_critic, ts.actor_critic.critics[i], ts.critic_batch, ts.actor_critic.critic_optimizers[i], ts.actor_target_buffers[i], ts.critic_buffers[i],
+                              ts.critic_target_buffers[i], ts.critic_training_buffers[i], ts.action_noise_critic, ts.rng);
+    if (update_critic_targets_flag) rlt::update_critic_targets(device, ts.actor_critic);
+    if (train_actor_flag) {
+        rlt::randn(device, ts.action_noise_actor, ts.rng);
+        rlt::train_actor(device, ts.actor_critic, ts.critic_batch, ts.actor_critic.actor_optimizer, ts.actor_buffers[0], ts.critic_buffers[0], ts.actor_training_buffers, ts.action_noise_actor, ts.rng);
+    }
+    ts.step++;
+    return same;
+}
+// [n_envs, replay capacity, episode step limit, the actor's auto-reset period (the SEQUENCE_LENGTH of its input shape), number of GRU layers in the actor]
+void rlt_ref_sac_gru_runner_dims(void* h, int* out) {
+    auto& L = *static_cast<Loop*>(h);
+    std::vector<float> hidden; std::vector<uint32_t> steps;
+    walk_state(L.device, rlt::get<1>(L.ts.off_policy_runner.policy_states).content_state, hidden, steps);
+    out[0] = N_ENVS; out[1] = CAPACITY; out[2] = EPISODE_LIMIT; out[3] = SEQ; out[4] = (int)(steps.size() / N_ENVS);
+}
+// the runner: states [n_envs x 2], episode_step, episode_return, truncated [n_envs]; the actor's policy state: hidden [GRU layers x n_envs x H] (layer after layer),
+// step counters [GRU layers x n_envs]
+void rlt_ref_sac_gru_get_runner(void* h, float* states, uint32_t* episode_step, float* episode_return, uint8_t* truncated, float* hidden, uint32_t* steps) {
+    auto& L = *static_cast<Loop*>(h); auto& runner = L.ts.off_policy_runner;
+    for (TI e = 0; e < N_ENVS; e++) {
+        auto& st = rlt::get(runner.states, 0, e);
+        states[2 * e] = st.theta; states[2 * e + 1] = st.theta_dot;
+        episode_step[e] = (uint32_t)rlt::get(runner.episode_step, 0, e); episode_return[e] = rlt::get(runner.episode_return, 0, e); truncated[e] = rlt::get(runner.truncated, 0, e);
+    }
+    std::vector<float> hv; std::vector<uint32_t> sv;
+    walk_state(L.device, rlt::get<1>(runner.policy_states).content_state, hv, sv);
+    std::memcpy(hidden, hv.data(), hv.size() * sizeof(float)); std::memcpy(steps, sv.data(), sv.size() * sizeof(uint32_t));
+}
+// replay ring of one environment: data [capacity x 10], cursor, full flag, start of the running episode, episode starts
+void rlt_ref_sac_gru_get_replay(void* h, int env, float* data, uint32_t* position, uint8_t* full, uint32_t* current_episode_start, uint32_t* episode_start) {
+    Loop& L = *static_cast<Loop*>(h);
+    auto& rb = rlt::get(L.ts.off_policy_runner.replay_buffers, 0, env);
+    using RB = rlt::utils::typing::remove_reference_t<decltype(rb)>;
+    std::memcpy(data, rb.data._data, sizeof(float) * RB::CAPACITY * RB::DATA_COLS);
+    *position = (uint32_t)rb.position; *full = rb.full; *current_episode_start = (uint32_t)rb.current_episode_start;
+    for (TI i = 0; i < RB::CAPACITY; i++) episode_start[i] = (uint32_t)rlt::get(L.device, rb.episode_start, i);
 }
 // the N(0,1) noise of the last training step: critic [(S+1) x B x 1], actor [S x B x 1]
 void rlt_ref_sac_gru_get_noise(void* h, float* noise_critic, float* noise_actor) {

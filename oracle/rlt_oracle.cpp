@@ -972,15 +972,10 @@ int rlt_oracle_pendulum_step(const rlt_pendulum_parameters* p, float* states, co
     return 0;
 }
 
-// off_policy_runner/operations_generic.h:183-238 + operations_generic_per_env.h:8-108 for Pendulum
-int rlt_oracle_pendulum_runner_step(const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, int policy_kind,
-                                    const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas,
-                                    const float* actions_in, const float* action_noise, const float* initial_states) {
-    if (!rn || !rb || rn->n_envs != rb->n_envs || rb->observation_dim != 3 || rb->action_dim != 1) return RLT_E_INVALID_ARGUMENT;
+// prologue of the off-policy runner step (operations_generic_per_env.h:8-66): reset where truncated, mark the previous replay row truncated, observe
+int rlt_oracle_pendulum_runner_prologue(const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, const float* initial_states, float* observations) {
+    if (!rn || !rb || !observations || rn->n_envs != rb->n_envs || rb->observation_dim != 3 || rb->action_dim != 1) return RLT_E_INVALID_ARGUMENT;
     const int N = rn->n_envs, R = rb_row_dim(rb);
-    std::vector<float> obs((size_t)N * 3), next_obs((size_t)N * 3), actions(N), rewards(N);
-    std::vector<uint8_t> term(N, 0), trunc(N, 0);
-    // prologue (:8-66): reset where truncated, mark previous replay row truncated, observe
     for (int e = 0; e < N; e++) {
         if (rn->truncated[e]) {
             if (!initial_states) return RLT_E_INVALID_ARGUMENT;
@@ -992,19 +987,16 @@ int rlt_oracle_pendulum_runner_step(const rlt_pendulum_runner* rn, const rlt_rep
                 rb->current_episode_start[e] = rb->position[e];
             }
         }
-        pendulum_observe(rn->states[2 * e], rn->states[2 * e + 1], &obs[3 * (size_t)e]);
+        pendulum_observe(rn->states[2 * e], rn->states[2 * e + 1], observations + 3 * (size_t)e);
     }
-    // interlude (:190-206): policy evaluate_step in Rollout mode
-    int rc = 0;
-    if (policy_kind == 0) { if (!actions_in) return RLT_E_INVALID_ARGUMENT; for (int e = 0; e < N; e++) actions[e] = actions_in[e]; }
-    else if (policy_kind == 1) { rc = rlt_oracle_mlp_evaluate(actor, n_actor_layers, obs.data(), 3, actions.data(), 1, N); }
-    else if (policy_kind == 2) {
-        std::vector<float> out((size_t)N * 2), lp(N);
-        rc = rlt_oracle_mlp_evaluate(actor, n_actor_layers, obs.data(), 3, out.data(), 2, N);
-        if (!rc) rc = rlt_oracle_sas_forward(sas, out.data(), 2, action_noise, 1, actions.data(), 1, nullptr, 0, lp.data(), N, 1);
-    } else return RLT_E_INVALID_ARGUMENT;
-    if (rc) return rc;
-    // epilogue (:67-108)
+    return 0;
+}
+// epilogue (operations_generic_per_env.h:67-108): step, reward, next observation, counters, truncation, replay add
+int rlt_oracle_pendulum_runner_epilogue(const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, const float* observations, const float* actions) {
+    if (!rn || !rb || !observations || !actions || rn->n_envs != rb->n_envs) return RLT_E_INVALID_ARGUMENT;
+    const int N = rn->n_envs;
+    std::vector<float> next_obs((size_t)N * 3), rewards(N);
+    std::vector<uint8_t> term(N, 0), trunc(N, 0);
     for (int e = 0; e < N; e++) {
         float nth, nthd, r;
         pendulum_dynamics(&rn->env, rn->states[2 * e], rn->states[2 * e + 1], actions[e], &nth, &nthd, &r);
@@ -1015,7 +1007,28 @@ int rlt_oracle_pendulum_runner_step(const rlt_pendulum_runner* rn, const rlt_rep
         rn->truncated[e] = trunc[e];
         rn->states[2 * e] = nth; rn->states[2 * e + 1] = nthd;
     }
-    return rlt_oracle_replay_add(rb, obs.data(), actions.data(), rewards.data(), next_obs.data(), term.data(), trunc.data());
+    return rlt_oracle_replay_add(rb, observations, actions, rewards.data(), next_obs.data(), term.data(), trunc.data());
+}
+
+// off_policy_runner/operations_generic.h:183-238 + operations_generic_per_env.h:8-108 for Pendulum
+int rlt_oracle_pendulum_runner_step(const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, int policy_kind,
+                                    const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas,
+                                    const float* actions_in, const float* action_noise, const float* initial_states) {
+    if (!rn || !rb || rn->n_envs != rb->n_envs || rb->observation_dim != 3 || rb->action_dim != 1) return RLT_E_INVALID_ARGUMENT;
+    const int N = rn->n_envs;
+    std::vector<float> obs((size_t)N * 3), actions(N);
+    int rc = rlt_oracle_pendulum_runner_prologue(rn, rb, initial_states, obs.data());
+    if (rc) return rc;
+    // interlude (:190-206): policy evaluate_step in Rollout mode
+    if (policy_kind == 0) { if (!actions_in) return RLT_E_INVALID_ARGUMENT; for (int e = 0; e < N; e++) actions[e] = actions_in[e]; }
+    else if (policy_kind == 1) { rc = rlt_oracle_mlp_evaluate(actor, n_actor_layers, obs.data(), 3, actions.data(), 1, N); }
+    else if (policy_kind == 2) {
+        std::vector<float> out((size_t)N * 2), lp(N);
+        rc = rlt_oracle_mlp_evaluate(actor, n_actor_layers, obs.data(), 3, out.data(), 2, N);
+        if (!rc) rc = rlt_oracle_sas_forward(sas, out.data(), 2, action_noise, 1, actions.data(), 1, nullptr, 0, lp.data(), N, 1);
+    } else return RLT_E_INVALID_ARGUMENT;
+    if (rc) return rc;
+    return rlt_oracle_pendulum_runner_epilogue(rn, rb, obs.data(), actions.data());
 }
 
 // rl::utils::evaluation::evaluate (rl/utils/evaluation/operations_generic.h:106-233) with the Pendulum environment: n_episodes environments from the

@@ -108,6 +108,14 @@ int rlt_oracle_seq_forward(const rlt_seq_layer* layers, int n_layers, const floa
 int rlt_oracle_seq_backward(const rlt_seq_layer* layers, int n_layers, const float* x, int ldx, float* d_output, float* d_input, const uint8_t* reset,
                             int steps, int batch, int want_weight_gradients, int reset_in_backward_input);
 int rlt_oracle_seq_zero_gradient(const rlt_seq_layer* layers, int n_layers);
+int rlt_oracle_seq_reset_state(const rlt_seq_layer* layers, int n_layers, const rlt_seq_state* state, const uint8_t* mask, int batch);
+int rlt_oracle_seq_evaluate_step(const rlt_seq_layer* layers, int n_layers, const float* x, int ldx, const rlt_seq_state* state, int auto_reset_period,
+                                 float* y, int ldy, int batch);
+int rlt_oracle_pendulum_runner_prologue(const rlt_pendulum_runner* runner, const rlt_replay_buffer* rb, const float* initial_states, float* observations);
+int rlt_oracle_pendulum_runner_epilogue(const rlt_pendulum_runner* runner, const rlt_replay_buffer* rb, const float* observations, const float* actions);
+int rlt_oracle_pendulum_runner_step_recurrent(const rlt_pendulum_runner* runner, const rlt_replay_buffer* rb, const rlt_seq_layer* policy, int n_policy_layers,
+                                              const rlt_seq_state* policy_state, int auto_reset_period, const rlt_sas_parameters* sas, const float* action_noise,
+                                              const float* initial_states);
 int rlt_oracle_sac_sequence_train_critic(const rlt_sac_sequence_agent* agent, int critic_index, const float* action_noise);
 int rlt_oracle_sac_sequence_update_critic_targets(const rlt_sac_sequence_agent* agent);
 int rlt_oracle_sac_sequence_train_actor(const rlt_sac_sequence_agent* agent, const float* action_noise);

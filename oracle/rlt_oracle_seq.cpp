@@ -6,10 +6,18 @@
 // compute the same values (evaluate keeps its intermediates in buffers instead of in the layer), so both are stated as forward here.
 #include "rlt_oracle.h"
 
+#include <cmath>
 #include <cstring>
 #include <vector>
 
 namespace {
+
+// math/operations_generic.h:247-251
+inline float fast_tanh_(float x) {
+    x = x < -3.0f ? -3.0f : (x > 3.0f ? 3.0f : x);
+    float x2 = x * x;
+    return x * (27 + x2) / (27 + 9 * x2);
+}
 
 int layer_in(const rlt_seq_layer& L) { return L.kind ? L.gru.input_dim : L.dense.in_dim; }
 int layer_out(const rlt_seq_layer& L) { return L.kind ? L.gru.hidden_dim : L.dense.out_dim; }
@@ -96,6 +104,91 @@ int rlt_oracle_seq_zero_gradient(const rlt_seq_layer* layers, int n) {
         }
     }
     return 0;
+}
+
+// reset(model, state, mode): nn_models/sequential/operations_generic.h:35-41 walks the layers; a GRU layer (nn/layers/gru/operations_generic.h:87-120) starts
+// the masked rows (all rows without a mask) again from the initial hidden state, step counter 0
+int rlt_oracle_seq_reset_state(const rlt_seq_layer* layers, int n, const rlt_seq_state* state, const uint8_t* mask, int batch) {
+    if (!layers || n <= 0 || n > RLT_SEQ_MAX_LAYERS || !state || batch <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int l = 0; l < n; l++) {
+        if (!layers[l].kind) continue;
+        const rlt_gru_layer& G = layers[l].gru;
+        if (!state->hidden[l] || !state->step[l]) return RLT_E_INVALID_ARGUMENT;
+        for (int b = 0; b < batch; b++)
+            if (!mask || mask[b]) { state->step[l][b] = 0; std::memcpy(state->hidden[l] + (size_t)b * G.hidden_dim, G.initial_hidden_state, sizeof(float) * G.hidden_dim); }
+    }
+    return 0;
+}
+
+// evaluate_step: nn_models/sequential/operations_generic.h:303-327 (tick / tock between the layers); dense layers evaluate; a GRU layer
+// (nn/layers/gru/operations_generic.h:348-416) runs the arithmetic of one forward step on its state, in the same order of operations
+int rlt_oracle_seq_evaluate_step(const rlt_seq_layer* layers, int n, const float* x, int ldx, const rlt_seq_state* state, int auto_reset_period, float* y, int ldy, int batch) {
+    if (!layers || n <= 0 || n > RLT_SEQ_MAX_LAYERS || !x || !state || !y || batch <= 0) return RLT_E_INVALID_ARGUMENT;
+    std::vector<float> buffers[2];
+    const float* in = x; int ld = ldx, which = 0, rc;
+    for (int l = 0; l < n; l++) {
+        const rlt_seq_layer& L = layers[l];
+        const int out_dim = layer_out(L);
+        float* out = y; int ldo = ldy;
+        if (l + 1 < n) { buffers[which].assign((size_t)batch * out_dim, 0.0f); out = buffers[which].data(); ldo = out_dim; which ^= 1; }
+        if (L.kind == 0) {
+            if ((rc = rlt_oracle_dense_evaluate(&L.dense, in, ld, out, ldo, batch))) return rc;
+        } else {
+            const rlt_gru_layer& G = L.gru;
+            const int H = G.hidden_dim, I = G.input_dim, H3 = 3 * H;
+            float* hidden = state->hidden[l]; uint32_t* step = state->step[l];
+            if (!hidden || !step) return RLT_E_INVALID_ARGUMENT;
+            for (int b = 0; b < batch; b++)                                  // reset_truncate (:76-86)
+                if (auto_reset_period > 0 && step[b] >= (uint32_t)auto_reset_period) { std::memcpy(hidden + (size_t)b * H, G.initial_hidden_state, sizeof(float) * H); step[b] = 0; }
+            std::vector<float> post((size_t)batch * H3), npp((size_t)batch * H);
+            for (int b = 0; b < batch; b++) {
+                const float* hp = hidden + (size_t)b * H; const float* xb = in + (size_t)b * ld;
+                float* p = &post[(size_t)b * H3];
+                for (int j = 0; j < H3; j++) {                              // W_h h + b_h (:373)
+                    float acc = G.biases_hidden[j];
+                    for (int k = 0; k < H; k++) acc += hp[k] * G.weights_hidden[(size_t)j * H + k];
+                    p[j] = acc;
+                }
+                for (int j = 0; j < H; j++) { npp[(size_t)b * H + j] = p[2 * H + j]; p[2 * H + j] = 0; }       // :375-376
+                for (int j = 0; j < H3; j++) {                              // += W_i x + b_i (:378)
+                    float acc = p[j] + G.biases_input[j];
+                    for (int k = 0; k < I; k++) acc += xb[k] * G.weights_input[(size_t)j * I + k];
+                    p[j] = acc;
+                }
+                for (int j = 0; j < 2 * H; j++) p[j] = G.fast_tanh ? 0.5f * fast_tanh_(0.5f * p[j]) + 0.5f : 1 / (1 + std::exp(-p[j]));      // :379-387
+                for (int j = 0; j < H; j++) p[2 * H + j] += npp[(size_t)b * H + j] * p[j];                                                   // :388
+                for (int j = 0; j < H; j++) p[2 * H + j] = G.fast_tanh ? fast_tanh_(p[2 * H + j]) : std::tanh(p[2 * H + j]);                // :389-397
+                for (int j = 0; j < H; j++) {
+                    float o = 1 - p[H + j];                                  // one_minus (:398)
+                    o = o * p[2 * H + j];                                    // multiply (:403)
+                    o += p[H + j] * hp[j];                                   // multiply_accumulate with the previous state (:404)
+                    out[(size_t)b * ldo + j] = o;
+                }
+            }
+            for (int b = 0; b < batch; b++) {                                // the new state; auto-reset (:405-415)
+                std::memcpy(hidden + (size_t)b * H, out + (size_t)b * ldo, sizeof(float) * H);
+                uint32_t new_step = step[b] + 1;
+                if (auto_reset_period > 0 && new_step >= (uint32_t)auto_reset_period) { new_step = 0; std::memcpy(hidden + (size_t)b * H, G.initial_hidden_state, sizeof(float) * H); }
+                step[b] = new_step;
+            }
+        }
+        in = out; ld = ldo;
+    }
+    return 0;
+}
+
+// rl/components/off_policy_runner/operations_generic.h:189-238 with a sequential policy that ends in [mean | log_std]
+int rlt_oracle_pendulum_runner_step_recurrent(const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, const rlt_seq_layer* policy, int n, const rlt_seq_state* state,
+                                              int auto_reset_period, const rlt_sas_parameters* sas, const float* action_noise, const float* initial_states) {
+    if (!rn || !rb || !policy || !state || !sas || !action_noise || n <= 0 || layer_out(policy[n - 1]) != 2) return RLT_E_INVALID_ARGUMENT;
+    const int N = rn->n_envs;
+    std::vector<float> obs((size_t)N * 3), out((size_t)N * 2), actions(N), lp(N);
+    int rc;
+    if ((rc = rlt_oracle_pendulum_runner_prologue(rn, rb, initial_states, obs.data()))) return rc;
+    if ((rc = rlt_oracle_seq_reset_state(policy, n, state, rn->truncated, N))) return rc;                      // :199-202: the flags the prologue acted on
+    if ((rc = rlt_oracle_seq_evaluate_step(policy, n, obs.data(), 3, state, auto_reset_period, out.data(), 2, N))) return rc;   // :203-204
+    if ((rc = rlt_oracle_sas_forward(sas, out.data(), 2, action_noise, 1, actions.data(), 1, nullptr, 0, lp.data(), N, 1))) return rc;
+    return rlt_oracle_pendulum_runner_epilogue(rn, rb, obs.data(), actions.data());
 }
 
 // rl/algorithms/sac/operations_generic.h:243-337

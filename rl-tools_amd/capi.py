@@ -156,6 +156,13 @@ class SeqLayer(C.Structure):
     _fields_ = [("kind", C.c_int32), ("reserved", C.c_int32), ("dense", DenseLayer), ("gru", GruLayer)]
 
 
+RLT_SEQ_MAX_LAYERS = 8
+
+
+class SeqState(C.Structure):
+    _fields_ = [("hidden", C.c_void_p * RLT_SEQ_MAX_LAYERS), ("step", C.c_void_p * RLT_SEQ_MAX_LAYERS)]
+
+
 class SacSequenceAgent(C.Structure):
     _fields_ = [("observation_dim", C.c_int32), ("action_dim", C.c_int32), ("n_actor_layers", C.c_int32), ("n_critic_layers", C.c_int32),
                 ("include_first_step_in_targets", C.c_int32), ("reserved0", C.c_int32), ("gamma", C.c_float), ("polyak", C.c_float),
@@ -252,6 +259,9 @@ PROTOTYPES = {
     "seq_forward": [C.POINTER(SeqLayer), I, P, I, P, I, I, P, S],
     "seq_backward": [C.POINTER(SeqLayer), I, P, I, P, P, P, I, I, I, I, P, S],
     "seq_zero_gradient": [C.POINTER(SeqLayer), I],
+    "seq_reset_state": [C.POINTER(SeqLayer), I, C.POINTER(SeqState), P, I],
+    "seq_evaluate_step": [C.POINTER(SeqLayer), I, P, I, C.POINTER(SeqState), I, P, I, I, P, S],
+    "pendulum_runner_step_recurrent": [C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), C.POINTER(SeqLayer), I, C.POINTER(SeqState), I, C.POINTER(SasParameters), P, P, P, S],
     "sac_sequence_train_critic": [C.POINTER(SacSequenceAgent), I, P],
     "sac_sequence_update_critic_targets": [C.POINTER(SacSequenceAgent)],
     "sac_sequence_train_actor": [C.POINTER(SacSequenceAgent), P],
@@ -279,6 +289,8 @@ ROCM_ONLY = {
     "ppo_workspace_bytes": ([C.POINTER(PpoAgent)], S),
     "gru_workspace_bytes": ([C.POINTER(GruLayer), I, I], S),
     "seq_workspace_bytes": ([C.POINTER(SeqLayer), I, I, I], S),
+    "seq_evaluate_step_workspace_bytes": ([C.POINTER(SeqLayer), I, I], S),
+    "pendulum_runner_step_recurrent_workspace_bytes": ([C.POINTER(SeqLayer), I, I], S),
     "sac_sequence_workspace_bytes": ([C.POINTER(SacSequenceAgent)], S),
     "on_policy_collect_workspace_bytes": ([C.POINTER(PendulumRunner), LP, I], S),
     "gather_draw": ([P, C.POINTER(ReplayBuffer), I, U64, U64, P, P], I),

@@ -736,6 +736,35 @@ int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_ru
     return rlt_launch_status(device);
 }
 
+size_t rlt_rocm_pendulum_runner_step_recurrent_workspace_bytes(const rlt_seq_layer* policy, int n_layers, int n_envs) {
+    if (!policy || n_layers < 1 || n_envs < 1) return 0;
+    return ((((size_t)n_envs * 7 * sizeof(float)) + 255) & ~(size_t)255) + rlt_rocm_seq_evaluate_step_workspace_bytes(policy, n_layers, n_envs) + 256;
+}
+
+// rl/components/off_policy_runner/operations_generic.h:189-238 with a sequential (recurrent) policy ending in [mean | log_std]: prologue, reset of the policy
+// state where a new episode starts (the flags the prologue acted on: it leaves `truncated` as it found it), one evaluate_step, sample_and_squash, epilogue
+int rlt_rocm_pendulum_runner_step_recurrent(rlt_rocm_device* device, const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, const rlt_seq_layer* policy, int n_layers,
+                                            const rlt_seq_state* state, int auto_reset_period, const rlt_sas_parameters* sas, const float* action_noise,
+                                            const float* initial_states, void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(rn && rn->states && rn->episode_step && rn->episode_return && rn->truncated && rn->n_envs > 0 && rb_ok(rb));
+    RLT_REQUIRE(rn->n_envs == rb->n_envs && rb->observation_dim == 3 && rb->action_dim == 1 && policy && n_layers >= 1 && state && sas && action_noise && initial_states);
+    const int N = rn->n_envs;
+    const size_t head = (((size_t)N * 7 * sizeof(float)) + 255) & ~(size_t)255;      // observations [N x 3], policy output [N x 2], actions [N], log-probabilities [N]
+    const size_t step_ws = rlt_rocm_seq_evaluate_step_workspace_bytes(policy, n_layers, N);
+    RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_pendulum_runner_step_recurrent_workspace_bytes(policy, n_layers, N));
+    char* w = reinterpret_cast<char*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    float* obs = (float*)w; float* policy_out = obs + (size_t)N * 3; float* actions = policy_out + (size_t)N * 2; float* lp = actions + N;
+    int rc;
+    hipLaunchKernelGGL(runner_prologue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *rb, initial_states, (uint64_t)0, (uint64_t)0, obs);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if ((rc = rlt_rocm_seq_reset_state(device, policy, n_layers, state, rn->truncated, N))) return rc;
+    if ((rc = rlt_rocm_seq_evaluate_step(device, policy, n_layers, obs, 3, state, auto_reset_period, policy_out, 2, N, w + head, step_ws))) return rc;
+    if ((rc = rlt_rocm_sas_forward(device, sas, policy_out, 2, action_noise, 1, actions, 1, nullptr, 0, lp, N, 1))) return rc;
+    hipLaunchKernelGGL(runner_epilogue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *rb, (const float*)actions);
+    return rlt_launch_status(device);
+}
+
 size_t rlt_rocm_on_policy_collect_workspace_bytes(const rlt_pendulum_runner* rn, const rlt_dense_layer* actor, int n_actor_layers) {
     if (!rn || !actor || n_actor_layers < 1 || rn->n_envs < 1) return 0;
     return (((size_t)rn->n_envs * 3 * sizeof(float) + 255) & ~(size_t)255) + rlt_rocm_mlp_workspace_bytes(actor, n_actor_layers, rn->n_envs) + 256;

@@ -2,6 +2,7 @@
 // forward / backward / zero_gradient assembled from the dense and GRU entry points of this library.
 // reference: nn_models/sequential/operations_generic.h:277-428.
 #include "common.h"
+#include "gemm.h"
 #include <algorithm>
 
 namespace {
@@ -40,6 +41,57 @@ bool carve(const rlt_seq_layer* layers, int n, int steps, int batch, void* works
     W->gru = w + 2 * one; W->gru_bytes = gru_bytes(layers, n, steps, batch);
     return true;
 }
+
+// ---- rollout state of the GRU layers (nn/layers/gru/layer.h State) ---------------------------------------------------------------
+__global__ __launch_bounds__(256) void seq_reset_state_kernel(float* __restrict__ hidden, uint32_t* __restrict__ step, const float* __restrict__ h0,
+                                                              const uint8_t* __restrict__ mask, int batch, int H) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < batch * H; i += gridDim.x * blockDim.x) {
+        const int b = i / H, j = i - b * H;
+        if (mask && !mask[b]) continue;
+        hidden[i] = h0[j];
+        if (j == 0) step[b] = 0;
+    }
+}
+__device__ __forceinline__ float fast_tanh_gate(float x) { return rlt_fast_tanh(x); }
+// One GRU step on the kept state: thread (row, unit). `post` holds W_i x + b_i of the step; the new hidden state goes to `out` (the state itself
+// is advanced by the commit kernel, after every thread has read the old one).
+__global__ __launch_bounds__(256) void gru_state_step_kernel(rlt_gru_layer L, const float* __restrict__ post, const float* __restrict__ hidden, const uint32_t* __restrict__ step,
+                                                             int period, float* __restrict__ out, int ldo, int batch) {
+    const int H = L.hidden_dim;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < batch * H; i += gridDim.x * blockDim.x) {
+        const int b = i / H, j = i - b * H;
+        const bool restart = period > 0 && step[b] >= (uint32_t)period;                 // reset_truncate (nn/layers/gru/operations_generic.h:76-86)
+        const float* hp = restart ? L.initial_hidden_state : hidden + (size_t)b * H;
+        float ar = L.biases_hidden[j], az = L.biases_hidden[H + j], an = L.biases_hidden[2 * H + j];
+        const float* wr = L.weights_hidden + (size_t)j * H; const float* wz = wr + (size_t)H * H; const float* wn = wz + (size_t)H * H;
+        for (int k = 0; k < H; k++) { const float hk = hp[k]; ar += hk * wr[k]; az += hk * wz[k]; an += hk * wn[k]; }
+        const float* p = post + (size_t)b * 3 * H;
+        const float xr = p[j] + ar, xz = p[H + j] + az;
+        const float r = L.fast_tanh ? 0.5f * fast_tanh_gate(0.5f * xr) + 0.5f : 1.0f / (1.0f + expf(-xr));
+        const float z = L.fast_tanh ? 0.5f * fast_tanh_gate(0.5f * xz) + 0.5f : 1.0f / (1.0f + expf(-xz));
+        const float xn = p[2 * H + j] + an * r;
+        const float n = L.fast_tanh ? fast_tanh_gate(xn) : tanhf(xn);
+        out[(size_t)b * ldo + j] = (1.0f - z) * n + z * hp[j];
+    }
+}
+// the new state; a row that has run `period` steps starts again from the initial hidden state (:405-415). The step counters are read here and
+// advanced by the launch after this one (gru_state_count_kernel), so that no thread reads a counter another one has already advanced.
+__device__ __forceinline__ uint32_t next_step(uint32_t old, int period) { return ((period > 0 && old >= (uint32_t)period) ? 0u : old) + 1u; }
+__global__ __launch_bounds__(256) void gru_state_commit_kernel(const float* __restrict__ out, int ldo, const float* __restrict__ h0, float* __restrict__ hidden,
+                                                               const uint32_t* __restrict__ step, int period, int batch, int H) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < batch * H; i += gridDim.x * blockDim.x) {
+        const int b = i / H, j = i - b * H;
+        const bool restart = period > 0 && next_step(step[b], period) >= (uint32_t)period;
+        hidden[i] = restart ? h0[j] : out[(size_t)b * ldo + j];
+    }
+}
+__global__ __launch_bounds__(256) void gru_state_count_kernel(uint32_t* __restrict__ step, int period, int batch) {
+    for (int b = blockIdx.x * blockDim.x + threadIdx.x; b < batch; b += gridDim.x * blockDim.x) {
+        const uint32_t next = next_step(step[b], period);
+        step[b] = (period > 0 && next >= (uint32_t)period) ? 0u : next;
+    }
+}
+inline int grid_for_elements(size_t n) { size_t b = (n + 255) / 256; return (int)(b > 2048 ? 2048 : (b < 1 ? 1 : b)); }
 
 }  // namespace
 
@@ -96,6 +148,70 @@ int rlt_rocm_seq_backward(rlt_rocm_device* device, const rlt_seq_layer* layers, 
         }
         if (rc) return rc;
         d_cur = d_in;
+    }
+    return 0;
+}
+
+int rlt_rocm_seq_reset_state(rlt_rocm_device* device, const rlt_seq_layer* layers, int n, const rlt_seq_state* state, const uint8_t* mask, int batch) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(layers && n > 0 && n <= RLT_SEQ_MAX_LAYERS && state && batch > 0);
+    for (int l = 0; l < n; l++) {
+        if (!layers[l].kind) continue;
+        const rlt_gru_layer& G = layers[l].gru;
+        RLT_REQUIRE(state->hidden[l] && state->step[l] && G.initial_hidden_state && G.hidden_dim > 0);
+        hipLaunchKernelGGL(seq_reset_state_kernel, dim3(grid_for_elements((size_t)batch * G.hidden_dim)), dim3(256), 0, device->stream, state->hidden[l], state->step[l],
+                           (const float*)G.initial_hidden_state, mask, batch, G.hidden_dim);
+        int rc = rlt_launch_status(device);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+// two buffers of batch x (widest layer output) between the layers, one of batch x 3H for the GRU input projections
+size_t rlt_rocm_seq_evaluate_step_workspace_bytes(const rlt_seq_layer* layers, int n, int batch) {
+    if (!layers || n <= 0 || batch <= 0) return 0;
+    size_t width = 1, h3 = 1;
+    for (int l = 0; l < n; l++) { width = std::max(width, (size_t)layer_out(layers[l])); if (layers[l].kind) h3 = std::max(h3, (size_t)3 * layers[l].gru.hidden_dim); }
+    return 2 * align256((size_t)batch * width * sizeof(float)) + align256((size_t)batch * h3 * sizeof(float)) + 256;
+}
+
+int rlt_rocm_seq_evaluate_step(rlt_rocm_device* device, const rlt_seq_layer* layers, int n, const float* x, int ldx, const rlt_seq_state* state, int period,
+                               float* y, int ldy, int batch, void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(layers && n > 0 && n <= RLT_SEQ_MAX_LAYERS && x && state && y && batch > 0 && period >= 0);
+    RLT_REQUIRE(ldx >= layer_in(layers[0]) && ldy >= layer_out(layers[n - 1]));
+    for (int l = 1; l < n; l++) RLT_REQUIRE(layer_in(layers[l]) == layer_out(layers[l - 1]));
+    RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_seq_evaluate_step_workspace_bytes(layers, n, batch));
+    size_t width = 1;
+    for (int l = 0; l < n; l++) width = std::max(width, (size_t)layer_out(layers[l]));
+    char* w = reinterpret_cast<char*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    const size_t one = align256((size_t)batch * width * sizeof(float));
+    float* buffers[2] = {(float*)w, (float*)(w + one)};
+    float* post = (float*)(w + 2 * one);
+    const float* in = x; int ld = ldx, which = 0, rc;
+    for (int l = 0; l < n; l++) {
+        const rlt_seq_layer& L = layers[l];
+        const int out_dim = layer_out(L);
+        float* out = y; int ldo = ldy;
+        if (l + 1 < n) { out = buffers[which]; ldo = out_dim; which ^= 1; }
+        if (L.kind == 0) {
+            if ((rc = rlt_rocm_dense_evaluate(device, &L.dense, in, ld, out, ldo, batch))) return rc;
+        } else {
+            const rlt_gru_layer& G = L.gru;
+            RLT_REQUIRE(state->hidden[l] && state->step[l] && G.weights_input && G.biases_input && G.weights_hidden && G.biases_hidden && G.initial_hidden_state);
+            const int H = G.hidden_dim;
+            if ((rc = rlt_gemm_forward(device, in, ld, G.weights_input, G.biases_input, RLT_ACT_IDENTITY, nullptr, nullptr, post, 3 * H, batch, G.input_dim, 3 * H))) return rc;
+            const dim3 grid(grid_for_elements((size_t)batch * H));
+            hipLaunchKernelGGL(gru_state_step_kernel, grid, dim3(256), 0, device->stream, G, (const float*)post, (const float*)state->hidden[l], (const uint32_t*)state->step[l],
+                               period, out, ldo, batch);
+            if ((rc = rlt_launch_status(device))) return rc;
+            hipLaunchKernelGGL(gru_state_commit_kernel, grid, dim3(256), 0, device->stream, (const float*)out, ldo, (const float*)G.initial_hidden_state, state->hidden[l],
+                               (const uint32_t*)state->step[l], period, batch, H);
+            if ((rc = rlt_launch_status(device))) return rc;
+            hipLaunchKernelGGL(gru_state_count_kernel, dim3(grid_for_elements(batch)), dim3(256), 0, device->stream, state->step[l], period, batch);
+            if ((rc = rlt_launch_status(device))) return rc;
+        }
+        in = out; ld = ldo;
     }
     return 0;
 }

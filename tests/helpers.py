@@ -43,7 +43,8 @@ class LoopConfig(C.Structure):
                 ("n_warmup_steps", C.c_int32), ("episode_step_limit", C.c_int32), ("adam_epsilon", C.c_float)]
 
 
-WITH_WORKSPACE = ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward", "on_policy_collect", "seq_forward", "seq_backward")
+WITH_WORKSPACE = ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward", "on_policy_collect", "seq_forward", "seq_backward", "seq_evaluate_step",
+                  "pendulum_runner_step_recurrent")
 
 
 def load_oracle():
@@ -1003,6 +1004,68 @@ class SeqNet:
         return self.backend.workspace(self.backend.device.lib.rlt_rocm_seq_workspace_bytes(self.layers, self.n, self.steps, self.batch))
 
 
+class SeqStateOnBackend:
+    """The rollout state of a sequential model's GRU layers (hidden state and step counter per batch row) on a backend."""
+
+    def __init__(self, backend, specs, batch):
+        self.backend, self.specs, self.batch = backend, list(specs), batch
+        self.hidden, self.step = {}, {}
+        self.c = capi.SeqState()
+        for l, (kind, _, o, _) in enumerate(specs):
+            if kind == 1:
+                self.hidden[l], self.step[l] = backend.zeros((batch, o)), backend.zeros((batch,), np.uint32)
+                self.c.hidden[l], self.c.step[l] = self.hidden[l].ptr, self.step[l].ptr
+
+    def set(self, hidden, steps):
+        """hidden: list of [batch x H] per GRU layer, steps: list of [batch], in layer order."""
+        for k, l in enumerate(sorted(self.hidden)):
+            self.hidden[l].upload(hidden[k]); self.step[l].upload(np.asarray(steps[k], np.uint32))
+
+    def numpy(self):
+        ls = sorted(self.hidden)
+        return [self.hidden[l].numpy() for l in ls], [self.step[l].numpy() for l in ls]
+
+
+class RecurrentRunnerOnBackend:
+    """Pendulum off-policy runner (n environments, one replay ring each) with a sequential policy and its rollout state on a backend."""
+
+    def __init__(self, backend, specs, params, n_envs, capacity, episode_limit, auto_reset_period):
+        self.backend, self.n, self.period = backend, n_envs, auto_reset_period
+        self.policy = SeqNet(backend, specs, params, 1, n_envs, trainable=False)
+        self.state = SeqStateOnBackend(backend, specs, n_envs)
+        self.rb = ReplayOnBackend(backend, n_envs, capacity)
+        self.states, self.ep_step, self.ep_ret = backend.zeros((n_envs, 2)), backend.zeros((n_envs,), np.uint32), backend.zeros((n_envs,))
+        self.trunc = backend.array(np.ones(n_envs, np.uint8))
+        self.c = capi.PendulumRunner(self.states.ptr, self.ep_step.ptr, self.ep_ret.ptr, self.trunc.ptr, n_envs, episode_limit, capi.pendulum_parameters())
+        self.sas = capi.SasParameters(-20.0, 2.0, 1e-6, -1.0)
+        self.ws, self.wsn = (None, 0)
+        if backend.name == "rocm":
+            n = int(backend.device.lib.rlt_rocm_pendulum_runner_step_recurrent_workspace_bytes(self.policy.layers, self.policy.n, n_envs))
+            self._ws = backend.device.empty((n,), np.uint8)
+            self.ws, self.wsn = self._ws.ptr, n
+
+    def load(self, runner, rings):
+        """runner: dict states / episode_step / episode_return / truncated / hidden / steps; rings: list of (data, position, full, current_episode_start, episode_start)."""
+        self.states.upload(runner["states"]); self.ep_step.upload(runner["episode_step"]); self.ep_ret.upload(runner["episode_return"]); self.trunc.upload(runner["truncated"])
+        self.state.set(runner["hidden"], runner["steps"])
+        self.rb.data.upload(np.concatenate([r[0] for r in rings])); self.rb.position.upload(np.array([r[1] for r in rings], np.uint32))
+        self.rb.full.upload(np.array([r[2] for r in rings], np.uint8)); self.rb.current_episode_start.upload(np.array([r[3] for r in rings], np.uint32))
+        self.rb.episode_start.upload(np.concatenate([r[4] for r in rings]).astype(np.uint32))
+
+    def step(self, action_noise, initial_states):
+        be = self.backend
+        nz, ini = be.array(np.ascontiguousarray(action_noise, np.float32)), be.array(np.ascontiguousarray(initial_states, np.float32))
+        be.call("pendulum_runner_step_recurrent", C.byref(self.c), C.byref(self.rb.c), self.policy.layers, self.policy.n, C.byref(self.state.c), self.period, C.byref(self.sas),
+                nz.ptr, ini.ptr, self.ws, self.wsn)
+        be.sync()
+
+    def numpy(self):
+        hidden, steps = self.state.numpy()
+        return dict(states=self.states.numpy(), episode_step=self.ep_step.numpy(), episode_return=self.ep_ret.numpy(), truncated=self.trunc.numpy(), hidden=hidden, steps=steps,
+                    data=self.rb.data.numpy(), position=self.rb.position.numpy(), full=self.rb.full.numpy(), current_episode_start=self.rb.current_episode_start.numpy(),
+                    episode_start=self.rb.episode_start.numpy())
+
+
 class SacSequenceOnBackend:
     """All state of a SAC agent with sequential (recurrent) networks on one backend. params: flat [actor, critic 0, critic 1, target 0, target 1,
     log_alpha] with every network laid out layer after layer (the order the reference harness exports)."""
@@ -1125,6 +1188,48 @@ class RefSacGru:
         self.lib.rlt_ref_sac_gru_get_noise(self.h, nc.ctypes.data, na.ctypes.data)
         return nc, na
 
+    def manual_step(self):
+        """One loop step past the warm-up with the runner step's draws written out: (initial states [n_envs x 2], noise [n_envs], reset flags [n_envs]);
+        asserts that exactly these draws were taken."""
+        lib = self.lib
+        lib.rlt_ref_sac_gru_manual_step.argtypes = [C.c_void_p] * 4
+        n = self.runner_dims()[0]
+        ini, nz, flags = np.zeros((n, 2), np.float32), np.zeros(n, np.float32), np.zeros(n, np.uint8)
+        assert lib.rlt_ref_sac_gru_manual_step(self.h, ini.ctypes.data, nz.ctypes.data, flags.ctypes.data) == 1
+        return ini, nz, flags
+
+    def runner_dims(self):
+        """[n_envs, replay capacity, episode step limit, auto-reset period of the actor, GRU layers in the actor]"""
+        self.lib.rlt_ref_sac_gru_runner_dims.argtypes = [C.c_void_p] * 2
+        d = np.zeros(5, np.int32); self.lib.rlt_ref_sac_gru_runner_dims(self.h, d.ctypes.data)
+        return [int(x) for x in d]
+
+    def runner(self):
+        n, _, _, _, n_gru = self.runner_dims()
+        H = [o for k, _, o, _ in self.actor_specs if k == 1]
+        self.lib.rlt_ref_sac_gru_get_runner.argtypes = [C.c_void_p] * 7
+        states, es, er, tr = np.zeros((n, 2), np.float32), np.zeros(n, np.uint32), np.zeros(n, np.float32), np.zeros(n, np.uint8)
+        hidden, steps = np.zeros(sum(n * h for h in H), np.float32), np.zeros(n_gru * n, np.uint32)
+        self.lib.rlt_ref_sac_gru_get_runner(self.h, states.ctypes.data, es.ctypes.data, er.ctypes.data, tr.ctypes.data, hidden.ctypes.data, steps.ctypes.data)
+        hs, o = [], 0
+        for h in H:
+            hs.append(hidden[o:o + n * h].reshape(n, h).copy()); o += n * h
+        return dict(states=states, episode_step=es, episode_return=er, truncated=tr, hidden=hs, steps=[steps[k * n:(k + 1) * n].copy() for k in range(n_gru)])
+
+    def rings(self):
+        n, cap = self.runner_dims()[:2]
+        self.lib.rlt_ref_sac_gru_get_replay.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5
+        out = []
+        for e in range(n):
+            data, es = np.zeros((cap, 10), np.float32), np.zeros(cap, np.uint32)
+            pos, full, ces = C.c_uint32(), C.c_uint8(), C.c_uint32()
+            self.lib.rlt_ref_sac_gru_get_replay(self.h, e, data.ctypes.data, C.byref(pos), C.byref(full), C.byref(ces), es.ctypes.data)
+            out.append((data, pos.value, full.value, ces.value, es))
+        return out
+
+    def actor_parameters(self):
+        return self.parameters()[:seq_param_count(self.actor_specs)]
+
     def close(self):
         self.lib.rlt_ref_sac_gru_destroy(self.h)
 
@@ -1157,3 +1262,37 @@ def sac_sequence_golden_step(agent, g, n_layers, i):
     p = f"l{n_layers}_s{i}_"
     agent.set_batch({k: g[p + k] for k in SEQUENCE_BATCH_FIELDS})
     agent.train(g[p + "noise_critic"], g[p + "noise_actor"])
+
+
+def recurrent_runner_golden():
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "recurrent_runner_pendulum.npz")
+    return dict(np.load(path)) if os.path.exists(path) else None
+
+
+def recurrent_runner_from_golden(backend, g):
+    n, cap, limit, period, n_gru, steps = [int(x) for x in g["dims"]]
+    specs = [(int(k), int(i), int(o), ACT_NAMES[int(a)]) for k, i, o, a in g["actor_layers"]]
+    run = RecurrentRunnerOnBackend(backend, specs, g["s0_actor"], n, cap, limit, period)
+    run.states.upload(g["before_states"]); run.ep_step.upload(g["before_episode_step"]); run.ep_ret.upload(g["before_episode_return"]); run.trunc.upload(g["before_truncated"])
+    run.state.set(list(g["before_hidden"]), list(g["before_steps"]))
+    run.rb.data.upload(g["before_data"]); run.rb.position.upload(g["before_position"]); run.rb.full.upload(g["before_full"])
+    run.rb.current_episode_start.upload(g["before_current_episode_start"]); run.rb.episode_start.upload(g["before_episode_start"])
+    return run, steps
+
+
+def recurrent_runner_golden_step(run, g, i):
+    """Runs fixture step i on `run`; returns what the step left behind in the fixture's terms."""
+    run.policy.params.upload(g[f"s{i}_actor"])
+    if i == 0:
+        run.trunc.upload(g["s0_reset"])          # the first step with the actor after the warm-up: the reference truncates every episode (policy switch)
+    else:
+        assert np.array_equal(run.trunc.numpy(), g[f"s{i}_reset"])
+    cap = run.rb.c.capacity
+    before = run.rb.position.numpy().astype(np.int64)
+    run.step(g[f"s{i}_noise"], g[f"s{i}_initial_states"])
+    out = run.numpy()
+    data = out["data"].reshape(run.n, cap, -1)
+    out["rows"] = np.stack([data[e, before[e]] for e in range(run.n)])
+    out["previous_truncated"] = np.array([data[e, (before[e] - 1) % cap, 9] for e in range(run.n)], np.float32)
+    out["hidden"], out["steps"] = np.stack(out["hidden"]), np.stack(out["steps"])
+    return out

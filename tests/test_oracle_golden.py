@@ -530,3 +530,59 @@ def test_sequential_model_gradients_against_finite_differences(oracle, with_rese
             oracle.call("seq_backward", net.layers, net.n, None, 0, gd2.ptr, dx2.ptr, rd.ptr, S, B, 0, flag, None, 0)
             out.append(dx2.numpy())
         assert np.allclose(out[1], dxn, rtol=1e-5, atol=1e-6) and not np.allclose(out[0], out[1], rtol=1e-3, atol=1e-5)
+
+
+def test_recurrent_runner_step_reproduces_reference_vectors(oracle):
+    """The off-policy runner step with the reference's recurrent actor (fixture written by its SAC loop): states, counters, truncation flags, the policy's
+    hidden state and step counters (with their automatic restart every 6 steps and the reset where an episode starts), ring cursors and the rows written,
+    bit for bit over 24 loop steps."""
+    g = helpers.recurrent_runner_golden()
+    run, steps = helpers.recurrent_runner_from_golden(oracle, g)
+    restarts = new_episodes = 0
+    for i in range(steps):
+        got = helpers.recurrent_runner_golden_step(run, g, i)
+        for k in ("states", "episode_step", "episode_return", "truncated", "hidden", "steps", "position", "current_episode_start", "rows", "previous_truncated"):
+            assert np.array_equal(got[k], g[f"s{i}_{k}"]), (i, k)
+        restarts += int((g[f"s{i}_steps"] == 0).sum()); new_episodes += int(g[f"s{i}_reset"].sum())
+    assert restarts >= 9 and new_episodes >= 3
+
+
+@pytest.mark.parametrize("fast_tanh", [False, True])
+def test_evaluate_step_chain_equals_the_sequence_forward_pass(oracle, fast_tanh):
+    """Independent of the reference: S single steps on the kept state give what one forward pass over the S-step sequence gives (same arithmetic, bit for
+    bit), a reset mask in the middle equals a reset flag of the sequence, and with an auto-reset period the state restarts after that many steps."""
+    rng = np.random.default_rng(31 + fast_tanh)
+    S, B, I, H, O = 7, 5, 3, 8, 2
+    specs = [(0, I, H, "relu"), (1, H, H, "identity"), (1, H, H, "identity"), (0, H, O, "identity")]
+    params = helpers.random_seq_params(rng, specs)
+    # a non-zero initial hidden state, so that a restart is visible
+    off = helpers.seq_param_count(specs[:1]) + 3 * H * H + 3 * H + 3 * H * H + 3 * H
+    params[off:off + H] = rng.uniform(-0.5, 0.5, H)
+    x = rng.standard_normal((S, B, I)).astype(np.float32)
+    reset = np.zeros((S, B), np.uint8); reset[3, 1] = reset[5, 4] = 1
+    net = helpers.SeqNet(oracle, specs, params, S, B, fast_tanh=fast_tanh)
+    xd, rd = oracle.array(x), oracle.array(reset)
+    oracle.call("seq_forward", net.layers, net.n, xd.ptr, I, rd.ptr, S, B, None, 0)
+    want = net.output().reshape(S, B, O)
+    state = helpers.SeqStateOnBackend(oracle, specs, B)
+    oracle.call("seq_reset_state", net.layers, net.n, C.byref(state.c), None, B)
+    y = oracle.zeros((B, O))
+    for t in range(S):
+        if reset[t].any():
+            m = oracle.array(reset[t])
+            oracle.call("seq_reset_state", net.layers, net.n, C.byref(state.c), m.ptr, B)
+        xt = oracle.array(x[t])
+        oracle.call("seq_evaluate_step", net.layers, net.n, xt.ptr, I, C.byref(state.c), 0, y.ptr, O, B, None, 0)
+        assert np.array_equal(y.numpy(), want[t]), t
+    assert all(list(s) == [S, S - 3, S, S, S - 5] for s in state.numpy()[1])      # steps since each row's last reset
+    # auto-reset every 3 steps == a sequence with reset flags at steps 3 and 6
+    reset3 = np.zeros((S, B), np.uint8); reset3[3] = reset3[6] = 1
+    rd3 = oracle.array(reset3)
+    oracle.call("seq_forward", net.layers, net.n, xd.ptr, I, rd3.ptr, S, B, None, 0)
+    want3 = net.output().reshape(S, B, O)
+    oracle.call("seq_reset_state", net.layers, net.n, C.byref(state.c), None, B)
+    for t in range(S):
+        xt = oracle.array(x[t])
+        oracle.call("seq_evaluate_step", net.layers, net.n, xt.ptr, I, C.byref(state.c), 3, y.ptr, O, B, None, 0)
+        assert np.array_equal(y.numpy(), want3[t]), t
+    assert not np.array_equal(want3[3:], want[3:])

@@ -551,3 +551,41 @@ def test_sac_sequence_fixture_is_what_the_reference_gives():
             if i in g[p + "snapshots"]:
                 assert np.array_equal(ref.parameters(), g[f"{p}s{i}_after"])
         ref.close()
+
+
+@pytest.mark.skipif(not (os.path.exists(helpers.ref_sac_gru_path(3)) and os.path.exists(helpers.ref_sac_gru_path(5))), reason="oracle/_ref recurrent SAC harness not built (needs /root/reference)")
+@pytest.mark.parametrize("n_layers", [3, 5])
+def test_recurrent_runner_step_bit_exact_with_reference(oracle, n_layers):
+    """The runner step of the reference's SAC loop with its recurrent actor. Two copies with one seed: one advanced by the reference's step(), one by the same
+    operations called one by one with the runner step's draws taken from a copy of the engine first (the harness checks that the engine then stands where the
+    copy stands) -- they must agree in every parameter, which ties what follows to step() itself. Each step the restatement starts from the reference's runner,
+    policy state and rings, gets the actor's parameters and the draws, and must reproduce environment states, counters, truncation flags, hidden states, step
+    counters and the replay rings bit for bit over 300 loop steps (30 new episodes, the hidden state restarting every 6 steps, ring wrap at 260 rows)."""
+    a, b = helpers.RefSacGru(n_layers, 4), helpers.RefSacGru(n_layers, 4)
+    for _ in range(a.n_warmup):
+        a.step(); b.step()
+    n, cap, limit, period, n_gru = b.runner_dims()
+    assert (n, cap, limit, period, n_gru) == (3, 260, 30, 6, 1 if n_layers == 3 else 2)
+    run = helpers.RecurrentRunnerOnBackend(oracle, b.actor_specs, b.actor_parameters(), n, cap, limit, period)
+    new_episodes = restarts = 0
+    for i in range(300):
+        run.load(b.runner(), b.rings())
+        run.policy.params.upload(b.actor_parameters())
+        a.step()
+        ini, noise, flags = b.manual_step()
+        assert np.array_equal(a.parameters(), b.parameters()), i
+        if i == 0:
+            assert flags.all()              # policy switch after the warm-up: every episode is truncated
+            run.trunc.upload(flags)
+        run.step(noise, ini)
+        got, want, rings = run.numpy(), b.runner(), b.rings()
+        for k in ("states", "episode_step", "episode_return", "truncated"):
+            assert np.array_equal(got[k], want[k]), (i, k)
+        for k in range(n_gru):
+            assert np.array_equal(got["hidden"][k], want["hidden"][k]) and np.array_equal(got["steps"][k], want["steps"][k]), (i, k)
+        assert np.array_equal(got["data"], np.concatenate([r[0] for r in rings])), i
+        assert np.array_equal(got["position"], [r[1] for r in rings]) and np.array_equal(got["full"], [r[2] for r in rings])
+        assert np.array_equal(got["current_episode_start"], [r[3] for r in rings]) and np.array_equal(got["episode_start"], np.concatenate([r[4] for r in rings]))
+        new_episodes += int(flags.sum()); restarts += int(sum((s == 0).sum() for s in want["steps"]))
+    assert new_episodes == 30 and restarts >= 150 and got["full"].all()
+    a.close(); b.close()
