@@ -328,6 +328,25 @@ def bench_sac_sequence(helpers, rocm, S=100, B=100, iters=10, cpu_seconds=1.5):
                 step(); n += 1
             out["cpu_checker_ms_per_training_step"] = (time.perf_counter() - t0) / n * 1e3
             out["cpu_sample"] = f"{n} training steps of the CPU restatement, one thread"
+    # the runner step with the recurrent actor over 4,096 environments (prologue, policy state reset, one evaluate_step, action draw, epilogue + replay add)
+    N = 4096
+    run = helpers.RecurrentRunnerOnBackend(rocm, actor_specs, params[:helpers.seq_param_count(actor_specs)], N, 16, 200, S)
+    noise = rocm.array(rng.standard_normal(N).astype(np.float32))
+    ini = rocm.array(np.stack([rng.uniform(-np.pi, np.pi, N), rng.uniform(-1, 1, N)], 1).astype(np.float32))
+
+    def runner_step():
+        rocm.call("pendulum_runner_step_recurrent", C.byref(run.c), C.byref(run.rb.c), run.policy.layers, run.policy.n, C.byref(run.state.c), run.period, C.byref(run.sas),
+                  noise.ptr, ini.ptr, run.ws, run.wsn)
+    for _ in range(3):
+        runner_step()
+    rocm.sync()
+    ev = HipEvents(rocm.device.lib.rlt_rocm_get_stream(rocm.device.handle))
+    a = ev.record()
+    for _ in range(50):
+        runner_step()
+    e = ev.record()
+    us = ev.elapsed_ms(a, e) / 50 * 1e3
+    out["recurrent_runner_step"] = {"n_envs": N, "us_per_step": us, "env_steps_per_s": N / (us * 1e-6)}
     return out
 
 

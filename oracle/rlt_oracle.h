@@ -36,6 +36,9 @@
  *   (rlt_oracle_seq.cpp): every parameter bit for bit against the reference's SAC loop with its recurrent approximators over 400 loop steps at two
  *   depths (oracle/_ref/librlt_ref_sac_gru{3,5}_generic.so), the FAST_TANH gates also on the GRU layer alone (librlt_ref_gru_fast_generic.so);
  *   golden vectors; equality with the single-step update at sequence length 1, finite differences of a dense-GRU-GRU-dense model.
+ *   seq reset_state / evaluate_step / pendulum runner step with a recurrent policy: runner, policy state and replay rings bit for bit against the
+ *   same loop over 300 steps at two depths, the step's draws taken from a copy of the reference's engine; golden vectors; a chain of single steps
+ *   equals the sequence forward pass.
  */
 #ifndef RLT_ORACLE_H
 #define RLT_ORACLE_H
