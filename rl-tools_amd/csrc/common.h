@@ -90,7 +90,10 @@ __device__ __forceinline__ void rlt_lds_barrier() {
 }
 
 // 64-lane wavefront sum (butterfly over DPP/ds_swizzle via __shfl_xor)
+// Every lane receives the same sum bit for bit (each exchange adds the same two numbers on both sides). The summand is pinned to a register first: otherwise the compiler may contract the multiplication that produced it into the first addition
+// (fma(a_i, b_i, partner's rounded product)), and the two lanes of an exchange then round differently -- the lanes no longer hold the same sum bit for bit.
 __device__ __forceinline__ float rlt_wave_sum(float v) {
+    asm volatile("" : "+v"(v));
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     return v;

@@ -38,7 +38,7 @@ struct SmallArgs {
 __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
 template <int CTRL>
 __device__ __forceinline__ float dpp(float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true)); }
-__device__ __forceinline__ float row16_sum(float x) { x += dpp<0xB1>(x); x += dpp<0x4E>(x); x += dpp<0x141>(x); x += dpp<0x140>(x); return x; }
+__device__ __forceinline__ float row16_sum(float x) { asm volatile("" : "+v"(x)); /* keeps a producing multiplication out of the first addition: all lanes then hold the same sum */ x += dpp<0xB1>(x); x += dpp<0x4E>(x); x += dpp<0x141>(x); x += dpp<0x140>(x); return x; }
 // lanes of one wavefront exchange data through LDS: the hardware executes a wavefront's LDS instructions in order, the fences keep
 // the compiler from moving them across
 __device__ __forceinline__ void wave_sync() {
@@ -47,7 +47,7 @@ __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 // sum over the four lane groups (lanes r, r + 16, r + 32, r + 48), in a fixed order
-__device__ __forceinline__ float groups_sum(float v) { v += __shfl_xor(v, 16, 64); v += __shfl_xor(v, 32, 64); return v; }
+__device__ __forceinline__ float groups_sum(float v) { asm volatile("" : "+v"(v)); v += __shfl_xor(v, 16, 64); v += __shfl_xor(v, 32, 64); return v; }
 
 // LDS: W1 [64][SX], W2 [64][HS], W3 [16][HS], then per round x [64][SX], h1 [64][HS], h2 [64][HS], g2 [64][HS], d3 [64][D3S]; SX = 16 nt1c + 1
 constexpr size_t lds_floats(int nt1c) {

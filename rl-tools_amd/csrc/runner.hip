@@ -255,7 +255,7 @@ constexpr int FWAVES = 8;        // wavefronts per workgroup: two per SIMD, one'
 __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
 template <int CTRL>
 __device__ __forceinline__ float dpp(float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true)); }
-__device__ __forceinline__ float row16_sum(float x) { x += dpp<0xB1>(x); x += dpp<0x4E>(x); x += dpp<0x141>(x); x += dpp<0x140>(x); return x; }
+__device__ __forceinline__ float row16_sum(float x) { asm volatile("" : "+v"(x)); /* keeps a producing multiplication out of the first addition: all lanes then hold the same sum */ x += dpp<0xB1>(x); x += dpp<0x4E>(x); x += dpp<0x141>(x); x += dpp<0x140>(x); return x; }
 
 struct FusedRunnerArgs {
     rlt_pendulum_runner rn; rlt_replay_buffer rb;
@@ -553,6 +553,7 @@ __global__ __launch_bounds__(64 * CWAVES) void on_policy_collect_kernel(CollectA
     }
 }
 // RLT_COLLECT_ONE_LAUNCH=0 keeps the collection on the per-step kernels (tests compare the two paths with each other)
+bool evaluate_one_launch_enabled() { const char* v = std::getenv("RLT_EVALUATE_ONE_LAUNCH"); return !(v && v[0] == '0'); }
 bool collect_one_launch_enabled() { const char* v = std::getenv("RLT_COLLECT_ONE_LAUNCH"); return !(v && v[0] == '0'); }
 bool fused_collect_ok(const rlt_dense_layer* L, int n) {
     return n == 3 && L[0].in_dim == 3 && L[0].out_dim == FH && L[1].in_dim == FH && L[1].out_dim == FH && L[2].in_dim == FH && L[2].out_dim == 1 &&
@@ -600,8 +601,12 @@ __global__ __launch_bounds__(64) void pendulum_evaluate_kernel(EvaluateArgs A) {
         for (int k = 0; k < H; k++) acc += w2s[j * 65 + k] * __int_as_float(__builtin_amdgcn_readlane(__float_as_int(h1), k));
         const float h2 = live ? rlt_act(acc, A.act2) : 0.f;
         const float y = rlt_act(rlt_wave_sum(w3 * h2) + b3, A.act_out);
-        // Evaluation mode: the action is the output, or the squashed mean of a [mean | log_std] head (sample_and_squash with zero noise)
-        const float action = A.policy_kind == 2 ? tanhf(y) : y;
+        // Evaluation mode: the action is the output, or the squashed mean of a [mean | log_std] head (sample_and_squash with zero noise).
+        // Every lane carries a copy of the episode's state, and lane j's hidden unit is computed from lane j's copy: the copies must stay identical bit
+        // for bit, or the network sees a state no single pendulum is in (a trained actor that balances the pendulum then loses it within 100 steps).
+        // Taking the action from one lane makes that hold whatever the compiler does with the reduction above.
+        const float action_own = A.policy_kind == 2 ? tanhf(y) : y;
+        const float action = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(action_own)));
         Transition t;
         pendulum_transition(A.env, theta, theta_dot, action, t);
         theta = t.theta; theta_dot = t.theta_dot; cs = t.next_obs[0]; sn = t.next_obs[1];
@@ -828,7 +833,7 @@ int rlt_rocm_pendulum_evaluate(rlt_rocm_device* device, const rlt_pendulum_param
     for (int l = 0; l < n_actor_layers; l++) RLT_REQUIRE(actor[l].weights && actor[l].biases && (l == 0 || actor[l].in_dim == actor[l - 1].out_dim));
     const int N = n_episodes;
     int rc;
-    if (n_actor_layers == 3 && actor[0].out_dim <= 64 && actor[1].out_dim == actor[0].out_dim) {
+    if (n_actor_layers == 3 && actor[0].out_dim <= 64 && actor[1].out_dim == actor[0].out_dim && evaluate_one_launch_enabled()) {
         EvaluateArgs a = {};
         a.env = *env;
         a.w1 = actor[0].weights; a.b1 = actor[0].biases; a.w2 = actor[1].weights; a.b2 = actor[1].biases; a.w3 = actor[2].weights; a.b3 = actor[2].biases;

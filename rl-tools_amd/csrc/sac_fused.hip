@@ -118,11 +118,12 @@ template <int CTRL>
 __device__ __forceinline__ float dpp(float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true)); }
 // sum over each row of 16 lanes, result in all 16 (quad swaps, then mirror within 8, then within 16)
 __device__ __forceinline__ float row16_sum(float x) {
+    asm volatile("" : "+v"(x));      // keeps a producing multiplication out of the first addition: all lanes of the row then hold the same sum bit for bit
     x += dpp<0xB1>(x); x += dpp<0x4E>(x); x += dpp<0x141>(x); x += dpp<0x140>(x);
     return x;
 }
 // sum over the four rows of a wavefront (lanes l, l^16, l^32, l^48), result in all
-__device__ __forceinline__ float kk_sum(float x) { x += __shfl_xor(x, 16, 64); x += __shfl_xor(x, 32, 64); return x; }
+__device__ __forceinline__ float kk_sum(float x) { asm volatile("" : "+v"(x)); x += __shfl_xor(x, 16, 64); x += __shfl_xor(x, 32, 64); return x; }
 
 // ---- exchange between workgroups
 // loads of data that another workgroup may have rewritten: never from this CU's vector cache
@@ -553,7 +554,9 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             const float ls_raw = kk_sum(row16_sum(w_actor[NA::lw3 + NA::LD2 + lane] * h2)) + w_actor[NA::lb3 + 1];
             // sample_and_squash in rollout mode (one action dimension), dynamics, reward, replay add
             const float ls = clampf(ls_raw, A.sas.log_std_lower_bound, A.sas.log_std_upper_bound);
-            const float action = tanhf(mean + eps * expf(ls));
+            // every lane of this wavefront carries the environment's state and feeds its own hidden unit from its own copy: the action comes from one lane, so
+            // that the copies stay identical bit for bit
+            const float action = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(tanhf(mean + eps * expf(ls)))));
             const rlt_pendulum_parameters& p = A.runner.env;
             float u = p.max_torque * clampf(action, -1.f, 1.f);
             u = clampf(u, -p.max_torque, p.max_torque);

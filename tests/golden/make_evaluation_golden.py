@@ -1,9 +1,10 @@
 """Writes tests/golden/evaluation_pendulum_seed0.npz from the REAL reference (oracle/_ref/librlt_ref_generic.so, built by oracle/Makefile from
 /root/reference). Runs only where the reference is mounted; the committed .npz is data, not source.
 
-The reference's SAC-on-Pendulum loop (seed 0, batch 100) is stopped after 0, 150 and 400 steps; at each stop the reference's
+The reference's SAC-on-Pendulum loop (seed 0, batch 100) is stopped after 0, 150, 400 and 6,000 steps (the last one a trained actor that swings
+the pendulum up and balances it: a closed loop in which a policy evaluated inconsistently loses the pendulum again); at each stop the reference's
 rl::utils::evaluation::evaluate runs 10 episodes of 200 steps with the current actor in Evaluation mode from initial states it samples
-(engine seeds 5, 6, 7). Kept per stop: the actor's parameters (flat, per layer [weights | biases]), the sampled initial states, and the
+(engine seeds 5, 6, 7, 8). Kept per stop: the actor's parameters (flat, per layer [weights | biases]), the sampled initial states, and the
 reference's result (returns, episode lengths, the six summary values)."""
 import ctypes as C
 import os
@@ -24,7 +25,7 @@ ref.rlt_ref_sac_evaluate.argtypes = [P, C.c_uint32, P, P, P, P]
 h = P(ref.rlt_ref_sac_create(0, 100))
 params = np.zeros(ref.rlt_ref_sac_parameter_count(h), np.float32)
 n_actor = helpers.mlp_param_count([3, 64, 64, 2])
-out = {"stops": np.array([0, 150, 400]), "seeds": np.array([5, 6, 7])}
+out = {"stops": np.array([0, 150, 400, 6000]), "seeds": np.array([5, 6, 7, 8])}
 for k, (stop, seed) in enumerate(zip(out["stops"], out["seeds"])):
     while ref.rlt_ref_sac_step_count(h) < stop:
         ref.rlt_ref_sac_step(h)

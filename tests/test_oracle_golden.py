@@ -252,7 +252,8 @@ def test_evaluation_reproduces_reference_vectors(oracle):
     lengths and summary statistics equal the reference's bit for bit (tests/golden/make_evaluation_golden.py). A deterministic actor with a tanh
     output layer whose single output row is the mean row of the same network must give the same episodes: that pins policy kind 1."""
     g = np.load(os.path.join(helpers.GOLDEN, "evaluation_pendulum_seed0.npz"))
-    for k in range(3):
+    assert list(g["stops"]) == [0, 150, 400, 6000] and g["e3_summary"][0] > -250 > g["e0_summary"][0]      # the last actor is a trained one
+    for k in range(len(g["stops"])):
         params, ini = g[f"e{k}_actor"], g[f"e{k}_initial_states"]
         ret, length, summary = helpers.evaluate_on_backend(oracle, [3, 64, 64, 2], params, "relu", "identity", 2, ini, 200)
         assert np.array_equal(ret, g[f"e{k}_returns"]) and np.array_equal(length, g[f"e{k}_episode_length"]) and np.array_equal(summary, g[f"e{k}_summary"])

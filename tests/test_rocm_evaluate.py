@@ -14,10 +14,10 @@ pytestmark = pytest.mark.gpu
 
 
 def test_evaluation_against_reference_vectors(rocm):
-    """The SAC actor after 0, 150 and 400 loop steps, 10 episodes x 200 steps from the initial states the reference drew: the reference's returns and
-    statistics (tests/golden/evaluation_pendulum_seed0.npz)."""
+    """The SAC actor after 0, 150, 400 and 6,000 loop steps, 10 episodes x 200 steps from the initial states the reference drew: the reference's returns
+    and statistics (tests/golden/evaluation_pendulum_seed0.npz)."""
     g = np.load(os.path.join(helpers.GOLDEN, "evaluation_pendulum_seed0.npz"))
-    for k in range(3):
+    for k in range(len(g["stops"])):
         ret, length, summary = helpers.evaluate_on_backend(rocm, [3, 64, 64, 2], g[f"e{k}_actor"], "relu", "identity", 2, g[f"e{k}_initial_states"], 200)
         assert np.array_equal(length, g[f"e{k}_episode_length"])
         assert rel_err(ret, g[f"e{k}_returns"]) <= 2e-3, (k, ret, g[f"e{k}_returns"])
@@ -59,3 +59,22 @@ def test_evaluation_rejects_bad_arguments(rocm):
     assert lib.rlt_rocm_pendulum_evaluate(h, C.byref(env), 2, actor.layers, 3, None, 4, 10, ret.ptr, length.ptr, summary.ptr) != 0
     assert lib.rlt_rocm_pendulum_evaluate(h, C.byref(env), 2, actor.layers, 3, ini.ptr, 4, 10, ret.ptr, length.ptr, summary.ptr) == 0
     rocm.sync()
+
+
+def test_evaluation_of_a_trained_actor_on_both_device_paths(oracle, rocm, monkeypatch):
+    """A trained actor holds the pendulum at its unstable equilibrium for most of the 200 steps: 100 episodes on the one-launch kernel, on the per-step
+    kernels of the same library and on the checker must agree episode by episode. (A wavefront of the one-launch kernel keeps a copy of the episode's
+    state in every lane; copies that differ in the last bit feed the network a state no pendulum is in, and the balanced pendulum is lost within 100
+    steps -- returns then differ by hundreds.)"""
+    g = np.load(os.path.join(helpers.GOLDEN, "evaluation_pendulum_seed0.npz"))
+    params = g["e3_actor"]
+    rng = np.random.default_rng(11)
+    ini = np.stack([rng.uniform(-np.pi, np.pi, 100), rng.uniform(-1, 1, 100)], 1).astype(np.float32)
+    want = helpers.evaluate_on_backend(oracle, [3, 64, 64, 2], params, "relu", "identity", 2, ini, 200)
+    one_launch = helpers.evaluate_on_backend(rocm, [3, 64, 64, 2], params, "relu", "identity", 2, ini, 200)
+    monkeypatch.setenv("RLT_EVALUATE_ONE_LAUNCH", "0")
+    per_step = helpers.evaluate_on_backend(rocm, [3, 64, 64, 2], params, "relu", "identity", 2, ini, 200)
+    assert want[2][0] > -250 and (want[0] > -20).sum() >= 5          # trained: several episodes are balanced from the start
+    for got in (one_launch, per_step):
+        assert np.abs(got[0] - want[0]).max() <= 0.05, np.abs(got[0] - want[0]).max()
+        assert abs(got[2][0] - want[2][0]) <= 0.01

@@ -111,3 +111,40 @@ def test_fused_loop_device_rng_trains_and_rejects_unsupported_shapes(oracle, roc
     odd = helpers.SacOnBackend(rocm, 40, 64, helpers.loop_parameters(oracle, loop), masks=False)
     assert rlib.rlt_rocm_sac_pendulum_loop(h, C.byref(odd.c), C.byref(runner.c), C.byref(runner.rb.c), 1, 7, 0, None, None) == -2
     lib.rlt_oracle_sac_loop_destroy(loop)
+
+
+def test_sac_learns_the_pendulum_to_the_reference_acceptance_bar(oracle, rocm):
+    """The reference's own acceptance test for this loop (tests/src/rl/algorithms/sac/cpu/test.cpp:9-43): 10,000 loop steps from a fresh agent, the mean return
+    of the evaluation episodes taken every 1,000 steps, and the 80th percentile of those ten means must exceed -200. Here: 100 warm-up steps on the checker,
+    9,900 loop steps in the persistent kernel with the device's own generator, 10 evaluation episodes of 200 steps on the device from sampled initial states
+    (an untrained actor scores below -1,000). For comparison, the CPU checker's loop (bit-identical to the reference) at this batch size gives the means
+    -1783, -1110, -707, -226, -176, -196, -156, -131, -316, -441 (80th percentile -156): late dips below the bar belong to the algorithm at batch 256."""
+    batch = 256
+    lib = oracle.lib
+    loop, cfg = helpers.make_loop(oracle, batch)
+    for _ in range(cfg.n_warmup_steps):
+        assert lib.rlt_oracle_sac_loop_step(loop) == 0
+    agent = helpers.SacOnBackend(rocm, batch, 64, helpers.loop_parameters(oracle, loop), masks=False)
+    runner = helpers.RunnerOnBackend(rocm, 10000, oracle, loop)
+    rlib, h = rocm.device.lib, rocm.device.handle
+    rng = np.random.default_rng(11)
+    env = capi.pendulum_parameters()
+    ret, length, summary = rocm.zeros((10,)), rocm.zeros((10,), np.uint32), rocm.zeros((6,))
+
+    def evaluate():
+        ini = rocm.array(np.stack([rng.uniform(-np.pi, np.pi, 10), rng.uniform(-1, 1, 10)], 1).astype(np.float32))
+        rocm.call("pendulum_evaluate", C.byref(env), 2, agent.actor.layers, agent.actor.n, ini.ptr, 10, 200, ret.ptr, length.ptr, summary.ptr)
+        rocm.sync()
+        return float(summary.numpy()[0])
+    untrained = evaluate()
+    returns = []
+    done = 0
+    for chunk in [900] + [1000] * 9:
+        assert rlib.rlt_rocm_sac_pendulum_loop(h, C.byref(agent.c), C.byref(runner.c), C.byref(runner.rb.c), chunk, 7, done, None, None) == 0
+        rocm.sync()
+        done += chunk
+        returns.append(evaluate())
+    print("mean evaluation returns", round(untrained), [round(r) for r in returns], flush=True)
+    assert untrained < -600 and len(returns) == 10
+    assert sorted(returns)[int(len(returns) * 0.8)] > -200, returns
+    lib.rlt_oracle_sac_loop_destroy(loop)
