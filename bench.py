@@ -442,7 +442,14 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_opera
                   "shader clock MHz", round(shader_cycles / tk.sum(), 1), file=sys.stderr, flush=True)
     p = agent.parameters()
     assert np.all(np.isfinite(p)), "SAC parameters went non-finite"
-    return {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3, "launches_per_step": (1.0 / steps) if not per_operation else None}
+    # what the run has learned (untimed): 100 evaluation episodes of 200 steps with the actor as it stands after warmup + steps loop steps from random weights
+    ini = rocm.array(np.stack([rng.uniform(-np.pi, np.pi, 100), rng.uniform(-1, 1, 100)], 1).astype(np.float32))
+    ret, length, summary = rocm.zeros((100,)), rocm.zeros((100,), np.uint32), rocm.zeros((6,))
+    env = capi.pendulum_parameters()
+    rocm.call("pendulum_evaluate", C.byref(env), 2, agent.actor.layers, agent.actor.n, ini.ptr, 100, 200, ret.ptr, length.ptr, summary.ptr)
+    rocm.sync()
+    return {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3, "launches_per_step": (1.0 / steps) if not per_operation else None,
+            "evaluation_return_after_run": float(summary.numpy()[0])}
 
 
 def cpu_baseline(batch=256, seconds=12.0):
@@ -583,7 +590,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "SAC Pendulum loop step, batch 256, actor 3-64-64-2, critics 4-64-64-1, replay 10000; plus MLP 17-256-256-6 fwd+bwd at batch %d" % args.mlp_batch,
                    "device": info["name"], "compute_units": info["compute_units"]},
-        "network_updates_per_s": 3 * sac["steps_per_s"], "sac_path": "per-operation launches" if args.sac_per_operation else "persistent kernel, one launch for all steps",
+        "network_updates_per_s": 3 * sac["steps_per_s"], "mean_return_of_100_evaluation_episodes_after_the_run": sac.get("evaluation_return_after_run"), "sac_path": "per-operation launches" if args.sac_per_operation else "persistent kernel, one launch for all steps",
     }
     if mlp:
         line["mlp_fwd_bwd_tflops"] = mlp["tflops"]
