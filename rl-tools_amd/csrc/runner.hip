@@ -576,8 +576,8 @@ bool rb_ok(const rlt_replay_buffer* rb) {
 // ---- evaluation episodes (rl/utils/evaluation/operations_generic.h:106-233) ----------------------------------------------------
 // One launch runs every step of every episode for actors 3 -> H -> H -> out with H <= 64: a wavefront per episode, lane j holds hidden unit j of both
 // hidden layers (its row of W1, its bias, its column of W3 in registers, W2 in LDS), the first layer's activations pass between lanes with
-// v_readlane, the output is a wavefront sum; every lane carries the environment state, so nothing else is exchanged. The chain of step_limit
-// dependent steps bounds the kernel.
+// v_readlane, the output is a wavefront sum; every lane carries a copy of the environment state, and the action that advances it is taken from one
+// lane, so that the copies stay identical bit for bit. The chain of step_limit dependent steps bounds the kernel.
 struct EvaluateArgs {
     rlt_pendulum_parameters env;
     const float *w1, *b1, *w2, *b2, *w3, *b3;
