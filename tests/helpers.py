@@ -1296,3 +1296,52 @@ def recurrent_runner_golden_step(run, g, i):
     out["previous_truncated"] = np.array([data[e, (before[e] - 1) % cap, 9] for e in range(run.n)], np.float32)
     out["hidden"], out["steps"] = np.stack(out["hidden"]), np.stack(out["steps"])
     return out
+
+
+def ppo_pendulum_loop(be, iterations, seed=0, n_envs=64, steps=128, minibatch=1024, H=64, eval_every=25, log=True):
+    """The whole PPO loop on one backend (rl/algorithms/ppo/loop/core/operations_generic.h:89-154): collect with the current actor, critic values of every
+    state, generalized advantages, one shuffled epoch of minibatch updates -- with the hyperparameters of the reference's Pendulum configuration
+    (src/rl/zoo/pendulum-v1/ppo.h: 64 environments x 128 steps, minibatches of 1,024, one epoch, gamma 0.9, initial action std 2, entropy coefficient 0.1,
+    Adam 1e-3, fast_tanh) except for the width (64 instead of 32) and observation normalisation (off). The random draws are made on the host from `seed`,
+    the same for every backend. Returns the mean return of 100 evaluation episodes after every `eval_every` iterations."""
+    rng = np.random.default_rng(seed)
+    col = dict(observations=0, actions_mean=3, actions=4, action_log_probs=5, rewards=6, terminated=7, truncated=8, all_reset=9, all_values=10, advantages=11, target_values=12)
+    ld = 13
+    rows = n_envs * steps
+    runner = OnPolicyOnBackend(be, n_envs, steps, ld, col, 200)
+    adims, cdims = [3, H, H, 1], [3, H, H, 1]
+    params = np.concatenate([random_params(rng, adims, bias_scale=0.0), np.log(np.full(1, 2.0, np.float32)), random_params(rng, cdims, bias_scale=0.0)]).astype(np.float32)
+    agent = PpoOnBackend(be, 3, 1, H, H, minibatch, params, "fast_tanh", "fast_tanh", capi.adam_parameters(1e-3, epsilon=1e-7))
+    pp = capi.ppo_parameters(0.2, 0.1, 1e-8, 1, 1)
+    # network descriptors for whole-dataset passes (the agent's own hold one minibatch)
+    critic_all = Mlp(be, cdims, agent.critic.params.numpy(), (steps + 1) * n_envs, "fast_tanh", "identity", trainable=False)
+    actor_run = Mlp(be, adims, agent.actor.params.numpy(), n_envs, "fast_tanh", "identity", trainable=False)
+    dd = runner.data
+    zeros3, ones3 = np.zeros(3, np.float32), np.ones(3, np.float32)
+    ws, wsn = critic_all.workspace()
+    env = capi.pendulum_parameters()
+    ret, length, summary = be.zeros((100,)), be.zeros((100,), np.uint32), be.zeros((6,))
+    erng = np.random.default_rng(11)
+    returns = []
+    for it in range(iterations):
+        actor_run.params.upload(agent.actor.params.numpy())
+        noise = rng.standard_normal((steps, n_envs, 1)).astype(np.float32)
+        ini = np.stack([rng.uniform(-np.pi, np.pi, (steps, n_envs)), rng.uniform(-1, 1, (steps, n_envs))], 2).astype(np.float32)
+        runner.collect(actor_run, agent.log_std.numpy(), noise, ini, standardize=(zeros3, ones3))
+        critic_all.params.upload(agent.critic.params.numpy())
+        be.call("mlp_evaluate", critic_all.layers, critic_all.n, dd.offset(col["observations"]), ld, dd.offset(col["all_values"]), ld, (steps + 1) * n_envs, ws, wsn)
+        be.call("ppo_gae", dd.offset(col["rewards"]), dd.offset(col["terminated"]), dd.offset(col["truncated"]), dd.offset(col["all_values"]),
+                dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld, n_envs, steps, 0.9, 0.95, 0)
+        perm = be.array(rng.permutation(rows).astype(np.uint32))
+        be.call("ppo_train_epoch", C.byref(agent.c), C.byref(pp), dd.offset(col["observations"]), dd.offset(col["observations"]), dd.offset(col["actions"]),
+                dd.offset(col["action_log_probs"]), dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld, perm.ptr, rows // minibatch, None)
+        be.sync()
+        if (it + 1) % eval_every == 0:
+            actor_eval = Mlp(be, adims, agent.actor.params.numpy(), 100, "fast_tanh", "identity", trainable=False)
+            ini_e = be.array(np.stack([erng.uniform(-np.pi, np.pi, 100), erng.uniform(-1, 1, 100)], 1).astype(np.float32))
+            be.call("pendulum_evaluate", C.byref(env), 1, actor_eval.layers, actor_eval.n, ini_e.ptr, 100, 200, ret.ptr, length.ptr, summary.ptr)
+            be.sync()
+            returns.append(float(summary.numpy()[0]))
+            if log:
+                print(be.name, it + 1, round(returns[-1]), 'log_std', float(agent.log_std.numpy()[0]), flush=True)
+    return returns
