@@ -347,6 +347,25 @@ def bench_sac_sequence(helpers, rocm, S=100, B=100, iters=10, cpu_seconds=1.5):
     e = ev.record()
     us = ev.elapsed_ms(a, e) / 50 * 1e3
     out["recurrent_runner_step"] = {"n_envs": N, "us_per_step": us, "env_steps_per_s": N / (us * 1e-6)}
+    # the evaluation step of the loop with the recurrent actor: 10 episodes of 200 steps (state reset, then observe, evaluate_step and environment step per step)
+    E, L = 10, 200
+    policy = helpers.SeqNet(rocm, actor_specs, params[:helpers.seq_param_count(actor_specs)], 1, E, trainable=False)
+    state = helpers.SeqStateOnBackend(rocm, actor_specs, E)
+    env = helpers.capi.pendulum_parameters()
+    ini_e = rocm.array(np.stack([rng.uniform(-np.pi, np.pi, E), rng.uniform(-1, 1, E)], 1).astype(np.float32))
+    ret, length, summary = rocm.zeros((E,)), rocm.zeros((E,), np.uint32), rocm.zeros((6,))
+    wsn = int(rocm.device.lib.rlt_rocm_pendulum_evaluate_recurrent_workspace_bytes(policy.layers, policy.n, E))
+    ws = rocm.device.empty((wsn,), np.uint8)
+
+    def evaluation():
+        rocm.call("pendulum_evaluate_recurrent", C.byref(env), 2, policy.layers, policy.n, C.byref(state.c), S, ini_e.ptr, E, L, ret.ptr, length.ptr, summary.ptr, ws.ptr, wsn)
+    evaluation()
+    rocm.sync()
+    a = ev.record()
+    for _ in range(3):
+        evaluation()
+    e = ev.record()
+    out["recurrent_evaluation"] = {"episodes": E, "steps": L, "ms": ev.elapsed_ms(a, e) / 3}
     return out
 
 

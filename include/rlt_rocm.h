@@ -672,6 +672,18 @@ int rlt_rocm_pendulum_runner_step_recurrent(rlt_rocm_device* device, const rlt_p
                                             const rlt_seq_layer* policy, int n_policy_layers, const rlt_seq_state* policy_state,
                                             int auto_reset_period, const rlt_sas_parameters* sas, const float* action_noise,
                                             const float* initial_states, void* workspace, size_t workspace_bytes);
+/* rl::utils::evaluation::evaluate  rl/utils/evaluation/operations_generic.h:106-233 with a sequential (recurrent) policy on the
+ * Pendulum (see rlt_rocm_pendulum_evaluate for the arguments and outputs): reset(policy, policy_state) before the first step
+ * (:135), then evaluate_step per step in Evaluation mode (:163) -- GRU layers restart their hidden state every
+ * auto_reset_period steps as in rlt_rocm_seq_evaluate_step. policy_state holds n_episodes rows and is left as the last
+ * step left it. policy_kind 2: the policy's last layer yields [mean | log_std] and sample_and_squash follows (action
+ * tanh(mean)); 1: its output is the action. */
+size_t rlt_rocm_pendulum_evaluate_recurrent_workspace_bytes(const rlt_seq_layer* policy, int n_policy_layers, int n_episodes);
+int rlt_rocm_pendulum_evaluate_recurrent(rlt_rocm_device* device, const rlt_pendulum_parameters* env, int policy_kind,
+                                         const rlt_seq_layer* policy, int n_policy_layers, const rlt_seq_state* policy_state,
+                                         int auto_reset_period, const float* initial_states, int n_episodes, int step_limit,
+                                         float* returns, uint32_t* episode_length, float* summary, void* workspace,
+                                         size_t workspace_bytes);
 
 /* Everything one SAC agent with sequential (recurrent) networks owns on the device: rl/algorithms/sac/sac.h:62-145 for
  * SEQUENCE_LENGTH >= 1 and the batch of rl/components/off_policy_runner/off_policy_runner.h:102-156 as

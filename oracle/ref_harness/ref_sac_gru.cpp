@@ -18,6 +18,7 @@
 #include <rl_tools/nn/optimizers/adam/operations_generic.h>
 #include <rl_tools/rl/algorithms/sac/loop/core/config.h>
 #include <rl_tools/rl/algorithms/sac/loop/core/operations_generic.h>
+#include <rl_tools/rl/utils/evaluation/operations_generic.h>
 
 #include <cstdint>
 #include <cstring>
@@ -285,6 +286,39 @@ void rlt_ref_sac_gru_get_noise(void* h, float* noise_critic, float* noise_actor)
     auto& ts = static_cast<Loop*>(h)->ts;
     std::memcpy(noise_critic, ts.action_noise_critic._data, sizeof(float) * (SEQ + 1) * BATCH);
     std::memcpy(noise_actor, ts.action_noise_actor._data, sizeof(float) * SEQ * BATCH);
+}
+
+// rl::utils::evaluation::evaluate (rl/utils/evaluation/operations_generic.h:106-233) of the loop's current recurrent actor in Evaluation mode: 5 episodes of 40
+// steps from sampled initial states (the actor restarts its hidden state every 6 steps by itself). The initial states the call will draw are exported by drawing
+// them first from a copy of the engine. summary = {returns_mean, returns_std, episode_length_mean, episode_length_std, num_terminated, share_terminated}
+void rlt_ref_sac_gru_evaluate(void* h, uint32_t seed, float* initial_states, float* returns, uint32_t* episode_length, float* summary) {
+    Loop& L = *static_cast<Loop*>(h);
+    constexpr TI N_EPISODES = 5, STEP_LIMIT = 40;
+    using SPEC = rlt::rl::utils::evaluation::Specification<TYPE_POLICY, TI, ENVIRONMENT, N_EPISODES, STEP_LIMIT>;
+    RNG rng;
+    rlt::malloc(L.device, rng);
+    rlt::init(L.device, rng, seed);
+    ENVIRONMENT env;
+    ENVIRONMENT::Parameters parameters;
+    rlt::init(L.device, env);
+    rlt::initial_parameters(L.device, env, parameters);
+    {
+        RNG copy = rng;
+        for (TI e = 0; e < N_EPISODES; e++) {
+            ENVIRONMENT::State state;
+            rlt::sample_initial_parameters(L.device, env, parameters, copy);
+            rlt::sample_initial_state(L.device, env, parameters, state, copy);
+            initial_states[2 * e] = state.theta; initial_states[2 * e + 1] = state.theta_dot;
+        }
+    }
+    rlt::rl::utils::evaluation::Result<SPEC> result;
+    rlt::rl::environments::DummyUI ui;
+    rlt::Mode<rlt::mode::Evaluation<>> mode;
+    rlt::evaluate(L.device, env, ui, L.ts.actor_critic.actor, result, rng, mode);
+    for (TI e = 0; e < N_EPISODES; e++) { returns[e] = result.returns[e]; episode_length[e] = (uint32_t)result.episode_length[e]; }
+    summary[0] = result.returns_mean; summary[1] = result.returns_std; summary[2] = result.episode_length_mean; summary[3] = result.episode_length_std;
+    summary[4] = (float)result.num_terminated; summary[5] = result.share_terminated;
+    rlt::free(L.device, rng);
 }
 
 }  // extern "C"

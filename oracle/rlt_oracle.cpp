@@ -1038,19 +1038,18 @@ int rlt_oracle_pendulum_runner_step(const rlt_pendulum_runner* rn, const rlt_rep
 //   policy_kind 1: the actor's output is the action;  2: the actor's output is [mean | log_std] and the action is tanh(mean), which is what
 //   sample_and_squash yields in Evaluation mode (noise = 0, nn/layers/sample_and_squash/operations_generic.h:149-195)
 //   summary = {returns_mean, returns_std, episode_length_mean, episode_length_std, num_terminated, share_terminated}
-int rlt_oracle_pendulum_evaluate(const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers, const float* initial_states,
-                                 int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary) {
-    if (!env || !actor || n_actor_layers < 1 || !initial_states || n_episodes < 1 || step_limit < 1 || !returns || !episode_length || !summary) return RLT_E_INVALID_ARGUMENT;
-    if (policy_kind != 1 && policy_kind != 2) return RLT_E_INVALID_ARGUMENT;
-    const int N = n_episodes, out_dim = actor[n_actor_layers - 1].out_dim;
-    if (actor[0].in_dim != 3 || out_dim != policy_kind) return RLT_E_INVALID_ARGUMENT;
+}  // extern "C"
+template <typename POLICY>
+static int pendulum_evaluate_impl(const rlt_pendulum_parameters* env, int policy_kind, POLICY&& policy, const float* initial_states,
+                                  int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary) {
+    const int N = n_episodes, out_dim = policy_kind;
     std::vector<float> states(initial_states, initial_states + 2 * (size_t)N), obs((size_t)N * 3), out((size_t)N * out_dim);
     std::vector<uint8_t> terminated(N, 0);
     uint32_t num_terminated = 0;
     for (int e = 0; e < N; e++) { returns[e] = 0; episode_length[e] = 0; }
     for (int step = 0; step < step_limit; step++) {
         for (int e = 0; e < N; e++) pendulum_observe(states[2 * e], states[2 * e + 1], &obs[3 * (size_t)e]);
-        const int rc = rlt_oracle_mlp_evaluate(actor, n_actor_layers, obs.data(), 3, out.data(), out_dim, N);
+        const int rc = policy(obs.data(), out.data());
         if (rc) return rc;
         for (int e = 0; e < N; e++) {
             if (step > 0 && terminated[e]) continue;
@@ -1070,6 +1069,31 @@ int rlt_oracle_pendulum_evaluate(const rlt_pendulum_parameters* env, int policy_
     summary[2] = lm; summary[3] = std::sqrt(std::max(0.0f, ls / N - lm * lm));
     summary[4] = (float)num_terminated; summary[5] = num_terminated / (float)N;
     return 0;
+}
+extern "C" {
+
+int rlt_oracle_pendulum_evaluate(const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers, const float* initial_states,
+                                 int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary) {
+    if (!env || !actor || n_actor_layers < 1 || !initial_states || n_episodes < 1 || step_limit < 1 || !returns || !episode_length || !summary) return RLT_E_INVALID_ARGUMENT;
+    if (policy_kind != 1 && policy_kind != 2) return RLT_E_INVALID_ARGUMENT;
+    if (actor[0].in_dim != 3 || actor[n_actor_layers - 1].out_dim != policy_kind) return RLT_E_INVALID_ARGUMENT;
+    return pendulum_evaluate_impl(env, policy_kind, [&](const float* obs, float* out) { return rlt_oracle_mlp_evaluate(actor, n_actor_layers, obs, 3, out, policy_kind, n_episodes); },
+                                  initial_states, n_episodes, step_limit, returns, episode_length, summary);
+}
+
+// The same evaluation with a sequential (recurrent) policy: its kept state is reset for every episode before the first step (:135) and every step goes through
+// evaluate_step (:163), whose GRU layers restart their hidden state by themselves every auto_reset_period steps (nn/layers/gru/operations_generic.h:406-413;
+// 0: never). Terminated episodes keep being fed to the policy (:155-163), only their environment stops (:166-170).
+int rlt_oracle_pendulum_evaluate_recurrent(const rlt_pendulum_parameters* env, int policy_kind, const rlt_seq_layer* policy, int n_layers, const rlt_seq_state* state,
+                                           int auto_reset_period, const float* initial_states, int n_episodes, int step_limit, float* returns, uint32_t* episode_length,
+                                           float* summary) {
+    if (!env || !policy || n_layers < 1 || !state || !initial_states || n_episodes < 1 || step_limit < 1 || !returns || !episode_length || !summary) return RLT_E_INVALID_ARGUMENT;
+    if (policy_kind != 1 && policy_kind != 2) return RLT_E_INVALID_ARGUMENT;
+    const int rc = rlt_oracle_seq_reset_state(policy, n_layers, state, nullptr, n_episodes);
+    if (rc) return rc;
+    return pendulum_evaluate_impl(env, policy_kind, [&](const float* obs, float* out) {
+        return rlt_oracle_seq_evaluate_step(policy, n_layers, obs, 3, state, auto_reset_period, out, policy_kind, n_episodes); },
+                                  initial_states, n_episodes, step_limit, returns, episode_length, summary);
 }
 
 // rl/algorithms/ppo/operations_generic.h:60-95

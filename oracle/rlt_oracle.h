@@ -39,6 +39,8 @@
  *   seq reset_state / evaluate_step / pendulum runner step with a recurrent policy: runner, policy state and replay rings bit for bit against the
  *   same loop over 300 steps at two depths, the step's draws taken from a copy of the reference's engine; golden vectors; a chain of single steps
  *   equals the sequence forward pass.
+ *   pendulum_evaluate_recurrent: returns, lengths and summary bit for bit against rl::utils::evaluation::evaluate on that loop's recurrent actor at two
+ *   depths, untrained and trained; golden vectors; equality with pendulum_evaluate for a policy of dense layers only.
  */
 #ifndef RLT_ORACLE_H
 #define RLT_ORACLE_H
@@ -156,6 +158,10 @@ int rlt_oracle_car_track_step(const rlt_car_parameters* p, const uint8_t* track,
 /* rl::utils::evaluation::evaluate with the Pendulum environment (rl/utils/evaluation/operations_generic.h:106-233) */
 int rlt_oracle_pendulum_evaluate(const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers, const float* initial_states,
                                  int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary);
+/* the same with a sequential (recurrent) policy: state reset before the first step, evaluate_step per step (:135,:163) */
+int rlt_oracle_pendulum_evaluate_recurrent(const rlt_pendulum_parameters* env, int policy_kind, const rlt_seq_layer* policy, int n_layers, const rlt_seq_state* state,
+                                           int auto_reset_period, const float* initial_states, int n_episodes, int step_limit, float* returns,
+                                           uint32_t* episode_length, float* summary);
 int rlt_oracle_ppo_surrogate_gradient(const float* action_means, int ld_means, const float* log_std, const float* actions, int ld_actions,
                                       const float* action_log_probs, int ld_log_probs, const float* advantages, int ld_advantages,
                                       const rlt_ppo_parameters* parameters, float* d_action_means, int ld_d, float* d_log_std, int batch, int action_dim);

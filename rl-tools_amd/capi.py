@@ -261,6 +261,7 @@ PROTOTYPES = {
     "seq_zero_gradient": [C.POINTER(SeqLayer), I],
     "seq_reset_state": [C.POINTER(SeqLayer), I, C.POINTER(SeqState), P, I],
     "seq_evaluate_step": [C.POINTER(SeqLayer), I, P, I, C.POINTER(SeqState), I, P, I, I, P, S],
+    "pendulum_evaluate_recurrent": [C.POINTER(PendulumParameters), I, C.POINTER(SeqLayer), I, C.POINTER(SeqState), I, P, I, I, P, P, P, P, S],
     "pendulum_runner_step_recurrent": [C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), C.POINTER(SeqLayer), I, C.POINTER(SeqState), I, C.POINTER(SasParameters), P, P, P, S],
     "sac_sequence_train_critic": [C.POINTER(SacSequenceAgent), I, P],
     "sac_sequence_update_critic_targets": [C.POINTER(SacSequenceAgent)],
@@ -291,6 +292,7 @@ ROCM_ONLY = {
     "seq_workspace_bytes": ([C.POINTER(SeqLayer), I, I, I], S),
     "seq_evaluate_step_workspace_bytes": ([C.POINTER(SeqLayer), I, I], S),
     "pendulum_runner_step_recurrent_workspace_bytes": ([C.POINTER(SeqLayer), I, I], S),
+    "pendulum_evaluate_recurrent_workspace_bytes": ([C.POINTER(SeqLayer), I, I], S),
     "sac_sequence_workspace_bytes": ([C.POINTER(SacSequenceAgent)], S),
     "on_policy_collect_workspace_bytes": ([C.POINTER(PendulumRunner), LP, I], S),
     "gather_draw": ([P, C.POINTER(ReplayBuffer), I, U64, U64, P, P], I),

@@ -865,5 +865,41 @@ int rlt_rocm_pendulum_evaluate(rlt_rocm_device* device, const rlt_pendulum_param
     return rlt_launch_status(device);
 }
 
-}  // extern "C"
+size_t rlt_rocm_pendulum_evaluate_recurrent_workspace_bytes(const rlt_seq_layer* policy, int n_layers, int n_episodes) {
+    if (!policy || n_layers < 1 || n_episodes < 1) return 0;
+    return ((((size_t)n_episodes * 7 * sizeof(float)) + 255) & ~(size_t)255) + rlt_rocm_seq_evaluate_step_workspace_bytes(policy, n_layers, n_episodes) + 256;
+}
 
+// rl::utils::evaluation::evaluate (rl/utils/evaluation/operations_generic.h:106-233) with a sequential (recurrent) policy: the kept state of every episode is reset
+// before the first step (:135), every step is one evaluate_step (:163); the policy keeps seeing terminated episodes, only their environment stops
+int rlt_rocm_pendulum_evaluate_recurrent(rlt_rocm_device* device, const rlt_pendulum_parameters* env, int policy_kind, const rlt_seq_layer* policy, int n_layers,
+                                         const rlt_seq_state* state, int auto_reset_period, const float* initial_states, int n_episodes, int step_limit,
+                                         float* returns, uint32_t* episode_length, float* summary, void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(env && policy && n_layers >= 1 && state && initial_states && n_episodes >= 1 && step_limit >= 1 && returns && episode_length && summary);
+    RLT_REQUIRE((policy_kind == 1 || policy_kind == 2) && auto_reset_period >= 0 && n_layers <= RLT_SEQ_MAX_LAYERS);
+    RLT_REQUIRE((policy[0].kind ? policy[0].gru.input_dim : policy[0].dense.in_dim) == 3);
+    RLT_REQUIRE((policy[n_layers - 1].kind ? policy[n_layers - 1].gru.hidden_dim : policy[n_layers - 1].dense.out_dim) == policy_kind);
+    RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_pendulum_evaluate_recurrent_workspace_bytes(policy, n_layers, n_episodes));
+    const int N = n_episodes;
+    const size_t head = (((size_t)N * 7 * sizeof(float)) + 255) & ~(size_t)255;      // states [N x 2], observations [N x 3], policy output [N x kind]
+    const size_t step_ws = rlt_rocm_seq_evaluate_step_workspace_bytes(policy, n_layers, N);
+    char* w = reinterpret_cast<char*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    float* states = (float*)w; float* obs = states + (size_t)N * 2; float* out = obs + (size_t)N * 3;
+    int rc;
+    RLT_HIP(hipMemcpyAsync(states, initial_states, (size_t)N * 2 * sizeof(float), hipMemcpyDeviceToDevice, device->stream));
+    if ((rc = rlt_rocm_fill_f32(device, returns, 1, N, N, 0.0f))) return rc;
+    if ((rc = rlt_rocm_fill_f32(device, (float*)episode_length, 1, N, N, 0.0f))) return rc;      // the bit pattern of 0.0f is the integer 0
+    if ((rc = rlt_rocm_seq_reset_state(device, policy, n_layers, state, nullptr, N))) return rc;
+    for (int step = 0; step < step_limit; step++) {
+        hipLaunchKernelGGL(evaluate_observe_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, states, obs, N);
+        if ((rc = rlt_launch_status(device))) return rc;
+        if ((rc = rlt_rocm_seq_evaluate_step(device, policy, n_layers, obs, 3, state, auto_reset_period, out, policy_kind, N, w + head, step_ws))) return rc;
+        hipLaunchKernelGGL(evaluate_step_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *env, states, out, policy_kind, policy_kind, returns, episode_length, N);
+        if ((rc = rlt_launch_status(device))) return rc;
+    }
+    hipLaunchKernelGGL(evaluate_summary_kernel, dim3(1), dim3(64), 0, device->stream, returns, episode_length, N, summary);
+    return rlt_launch_status(device);
+}
+
+}  // extern "C"

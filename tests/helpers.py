@@ -44,7 +44,7 @@ class LoopConfig(C.Structure):
 
 
 WITH_WORKSPACE = ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward", "on_policy_collect", "seq_forward", "seq_backward", "seq_evaluate_step",
-                  "pendulum_runner_step_recurrent")
+                  "pendulum_runner_step_recurrent", "pendulum_evaluate_recurrent")
 
 
 def load_oracle():
@@ -1066,6 +1066,28 @@ class RecurrentRunnerOnBackend:
                     episode_start=self.rb.episode_start.numpy())
 
 
+def evaluate_recurrent(backend, specs, params, period, initial_states, step_limit, policy_kind=2, fast_tanh=True):
+    """Evaluation episodes on the Pendulum with a sequential (recurrent) policy on a backend: dict of returns, episode lengths, summary, and the policy state
+    (hidden, steps) the run ends with."""
+    N = len(initial_states)
+    policy = SeqNet(backend, specs, params, 1, N, trainable=False, fast_tanh=fast_tanh)
+    state = SeqStateOnBackend(backend, specs, N)
+    for l in state.hidden:                                   # the call resets the state itself: start from values a missing reset would show
+        state.hidden[l].upload(np.full((N, specs[l][2]), 0.5, np.float32)); state.step[l].upload(np.full(N, 3, np.uint32))
+    ini = backend.array(np.ascontiguousarray(initial_states, np.float32))
+    ret, length, summary = backend.zeros((N,)), backend.zeros((N,), np.uint32), backend.zeros((6,))
+    ws, wsn = None, 0
+    if backend.name == "rocm":
+        wsn = int(backend.device.lib.rlt_rocm_pendulum_evaluate_recurrent_workspace_bytes(policy.layers, policy.n, N))
+        keep = backend.device.empty((wsn,), np.uint8); ws = keep.ptr
+    env = capi.pendulum_parameters()
+    backend.call("pendulum_evaluate_recurrent", C.byref(env), policy_kind, policy.layers, policy.n, C.byref(state.c), period, ini.ptr, N, step_limit, ret.ptr, length.ptr,
+                 summary.ptr, ws, wsn)
+    backend.sync()
+    hidden, steps = state.numpy()
+    return dict(returns=ret.numpy(), length=length.numpy(), summary=summary.numpy(), hidden=hidden, steps=steps)
+
+
 class SacSequenceOnBackend:
     """All state of a SAC agent with sequential (recurrent) networks on one backend. params: flat [actor, critic 0, critic 1, target 0, target 1,
     log_alpha] with every network laid out layer after layer (the order the reference harness exports)."""
@@ -1230,6 +1252,14 @@ class RefSacGru:
     def actor_parameters(self):
         return self.parameters()[:seq_param_count(self.actor_specs)]
 
+    def evaluate(self, seed):
+        """rl::utils::evaluation::evaluate of the loop's current actor by the reference: 5 episodes x 40 steps in Evaluation mode from initial states drawn with
+        `seed`; (initial states, returns, episode lengths, summary)."""
+        self.lib.rlt_ref_sac_gru_evaluate.argtypes = [C.c_void_p, C.c_uint32] + [C.c_void_p] * 4
+        ini, ret, length, summary = np.zeros((5, 2), np.float32), np.zeros(5, np.float32), np.zeros(5, np.uint32), np.zeros(6, np.float32)
+        self.lib.rlt_ref_sac_gru_evaluate(self.h, seed, ini.ctypes.data, ret.ctypes.data, length.ctypes.data, summary.ctypes.data)
+        return ini, ret, length, summary
+
     def close(self):
         self.lib.rlt_ref_sac_gru_destroy(self.h)
 
@@ -1267,6 +1297,21 @@ def sac_sequence_golden_step(agent, g, n_layers, i):
 def recurrent_runner_golden():
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "recurrent_runner_pendulum.npz")
     return dict(np.load(path)) if os.path.exists(path) else None
+
+
+def evaluation_recurrent_golden():
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "evaluation_recurrent_pendulum.npz")
+    return dict(np.load(path)) if os.path.exists(path) else None
+
+
+def evaluation_recurrent_golden_cases(g):
+    """(label, actor specs, parameters, auto-reset period, initial states, step limit, expected returns / length / summary) of every run in the fixture."""
+    for n_layers in (3, 5):
+        specs = [(int(k), int(i), int(o), ACT_NAMES[int(a)]) for k, i, o, a in g[f"l{n_layers}_actor_layers"]]
+        period, step_limit = int(g["dims"][0]), int(g["dims"][1])
+        for k in range(int(g["dims"][2])):
+            p = f"l{n_layers}_e{k}_"
+            yield p, specs, g[p + "actor"], period, g[p + "initial_states"], step_limit, g[p + "returns"], g[p + "length"], g[p + "summary"]
 
 
 def recurrent_runner_from_golden(backend, g):

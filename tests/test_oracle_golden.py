@@ -269,6 +269,41 @@ def test_evaluation_reproduces_reference_vectors(oracle):
     assert np.all(length50 == 50) and np.all(ret50 > g["e2_returns"]) and np.all(ret50 < 0)
 
 
+def test_evaluation_with_recurrent_policy_reproduces_reference_vectors(oracle):
+    """rl::utils::evaluation::evaluate with the reference's recurrent SAC actor (one and two GRU layers; 5 episodes x 40 steps, the hidden state restarting every
+    6 steps), untrained and after 40 and 150 training steps: returns, lengths and summary equal the reference's bit for bit
+    (tests/golden/make_evaluation_recurrent_golden.py). Independently of the reference: the call resets the policy state itself (the helper hands it a state
+    filled with other values), the state it leaves is that of 40 steps (40 mod 6 = 4 steps after the last restart), a horizon that ends on a restart leaves the
+    initial hidden state, and a sequential policy of dense layers only gives the episodes of the same network evaluated as an MLP."""
+    g = helpers.evaluation_recurrent_golden()
+    n = 0
+    for label, specs, params, period, ini, step_limit, ret, length, summary in helpers.evaluation_recurrent_golden_cases(g):
+        got = helpers.evaluate_recurrent(oracle, specs, params, period, ini, step_limit)
+        assert np.array_equal(got["returns"], ret) and np.array_equal(got["length"], length) and np.array_equal(got["summary"], summary), label
+        assert all(np.all(s == step_limit % period) for s in got["steps"])
+        ends_on_restart = helpers.evaluate_recurrent(oracle, specs, params, period, ini, 3 * period)
+        off = 0
+        for k, (kind, i, o, _) in enumerate(specs):
+            if kind == 1:
+                h0 = params[off + 3 * o * i + 3 * o + 3 * o * o + 3 * o:off + 3 * o * i + 3 * o + 3 * o * o + 3 * o + o]
+                layer = [l for l, sp in enumerate(specs) if sp[0] == 1].index(k)
+                assert np.array_equal(ends_on_restart["hidden"][layer], np.tile(h0, (len(ini), 1))) and np.all(ends_on_restart["steps"][layer] == 0)
+                off += 3 * o * i + 3 * o + 3 * o * o + 3 * o + o
+            else:
+                off += i * o + o
+        never = helpers.evaluate_recurrent(oracle, specs, params, 0, ini, step_limit)          # without the restarts the episodes differ
+        assert not np.array_equal(never["returns"], ret) and all(np.all(s == step_limit) for s in never["steps"])
+        n += 1
+    assert n == 6
+    rng = np.random.default_rng(5)
+    dims = [3, 24, 24, 2]
+    params = helpers.random_params(rng, dims)
+    ini = np.stack([rng.uniform(-np.pi, np.pi, 9), rng.uniform(-1, 1, 9)], 1).astype(np.float32)
+    want = helpers.evaluate_on_backend(oracle, dims, params, "tanh", "identity", 2, ini, 60)
+    got = helpers.evaluate_recurrent(oracle, [(0, 3, 24, "tanh"), (0, 24, 24, "tanh"), (0, 24, 2, "identity")], params, 7, ini, 60)
+    assert np.array_equal(got["returns"], want[0]) and np.array_equal(got["length"], want[1]) and np.array_equal(got["summary"], want[2])
+
+
 def test_acrobot_reproduces_reference_vectors_and_conserves_energy(oracle):
     """Acrobot / AcrobotSwingup / EasyParameters steps against the reference's own outputs (tests/golden/make_acrobot_golden.py), bit for bit, random
     states and 200-step trajectories. Then what the mechanics fix: without torque the equations of motion conserve

@@ -589,3 +589,27 @@ def test_recurrent_runner_step_bit_exact_with_reference(oracle, n_layers):
         new_episodes += int(flags.sum()); restarts += int(sum((s == 0).sum() for s in want["steps"]))
     assert new_episodes == 30 and restarts >= 150 and got["full"].all()
     a.close(); b.close()
+
+
+@pytest.mark.parametrize("n_layers", [3, 5])
+def test_evaluation_with_recurrent_policy_bit_exact_with_reference(oracle, n_layers):
+    """rl::utils::evaluation::evaluate on the reference's recurrent SAC actor (one or two GRU layers, hidden state restarting every 6 steps), untrained and after
+    40 and 150 training steps: the restatement reproduces every episode's return, the lengths and the summary bit for bit from the same initial states. The
+    committed fixture (tests/golden/evaluation_recurrent_pendulum.npz) holds exactly these runs."""
+    ref = helpers.RefSacGru(n_layers, 9)
+    g = helpers.evaluation_recurrent_golden()
+    period = ref.runner_dims()[3]
+    done = 0
+    for k, stop in enumerate([0, ref.n_warmup + 40, ref.n_warmup + 150]):
+        while done < stop:
+            ref.step(); done += 1
+        ini, ret, length, summary = ref.evaluate(100 + k)
+        got = helpers.evaluate_recurrent(oracle, ref.actor_specs, ref.actor_parameters(), period, ini, 40)
+        assert np.array_equal(got["returns"], ret) and np.array_equal(got["length"], length) and np.array_equal(got["summary"], summary), (k, got["returns"], ret)
+        assert np.all(length == 40) and np.all(ret < 0)
+        if g is not None:
+            p = f"l{n_layers}_e{k}_"
+            assert np.array_equal(g[p + "actor"], ref.actor_parameters()) and np.array_equal(g[p + "initial_states"], ini) and np.array_equal(g[p + "returns"], ret)
+            assert np.array_equal(g[p + "summary"], summary)
+    ref.close()
+

@@ -78,3 +78,62 @@ def test_evaluation_of_a_trained_actor_on_both_device_paths(oracle, rocm, monkey
     for got in (one_launch, per_step):
         assert np.abs(got[0] - want[0]).max() <= 0.05, np.abs(got[0] - want[0]).max()
         assert abs(got[2][0] - want[2][0]) <= 0.01
+
+
+def test_evaluation_with_recurrent_policy_against_reference_vectors(oracle, rocm):
+    """The reference's recurrent SAC actor (one and two GRU layers, hidden state restarting every 6 steps), 5 episodes x 40 steps from the initial states the
+    reference drew: the reference's returns and statistics (tests/golden/evaluation_recurrent_pendulum.npz), and the policy state the run leaves."""
+    n = 0
+    for label, specs, params, period, ini, step_limit, ret, length, summary in helpers.evaluation_recurrent_golden_cases(helpers.evaluation_recurrent_golden()):
+        print("case", label, flush=True)
+        got, want = (helpers.evaluate_recurrent(be, specs, params, period, ini, step_limit) for be in (rocm, oracle))
+        assert np.array_equal(got["length"], length) and rel_err(got["returns"], ret) <= 1e-4, (label, got["returns"], ret)
+        assert rel_err(got["summary"][:2], summary[:2]) <= 1e-4 and np.array_equal(got["summary"][2:], summary[2:])
+        for a, b in zip(got["steps"], want["steps"]):
+            assert np.array_equal(a, b)
+        for a, b in zip(got["hidden"], want["hidden"]):
+            assert rel_err(a, b) <= 1e-4
+        n += 1
+    assert n == 6
+
+
+@pytest.mark.parametrize("case", [(16, 1, True, 6, 2, 10), (64, 2, False, 50, 2, 300), (32, 1, True, 0, 1, 4096), (24, 2, True, 7, 2, 33)])
+def test_evaluation_with_recurrent_policy_matches_checker(oracle, rocm, case):
+    """Other widths (register-resident and generic GRU step kernels), depths, exact and fast gates, restart periods (0: never), both policy kinds, many episodes."""
+    print("case", case, flush=True)
+    H, n_gru, fast, period, kind, n = case
+    rng = np.random.default_rng(H + n)
+    specs = [(0, 3, H, "relu")] + [(1, H, H, "identity")] * n_gru + [(0, H, kind, "identity" if kind == 2 else "tanh")]
+    params = helpers.random_seq_params(rng, specs)
+    ini = np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n)], 1).astype(np.float32)
+    for steps, tol in ((20, 1e-5), (200, 2e-3)):
+        want, got = (helpers.evaluate_recurrent(be, specs, params, period, ini, steps, kind, fast) for be in (oracle, rocm))
+        assert np.array_equal(got["length"], want["length"]) and np.all(got["length"] == steps)
+        assert rel_err(got["returns"], want["returns"]) <= tol, (steps, rel_err(got["returns"], want["returns"]))
+        assert rel_err(got["summary"][:2], want["summary"][:2]) <= tol and np.array_equal(got["summary"][2:], want["summary"][2:])
+        for a, b in zip(got["steps"], want["steps"]):
+            assert np.array_equal(a, b)
+
+
+def test_evaluation_with_recurrent_policy_rejects_bad_arguments(rocm):
+    import ctypes as C
+    capi = helpers.capi
+    specs = [(0, 3, 16, "relu"), (1, 16, 16, "identity"), (0, 16, 2, "identity")]
+    N = 4
+    policy = helpers.SeqNet(rocm, specs, helpers.random_seq_params(np.random.default_rng(0), specs), 1, N, trainable=False)
+    state = helpers.SeqStateOnBackend(rocm, specs, N)
+    ini, ret, length, summary = rocm.zeros((N, 2)), rocm.zeros((N,)), rocm.zeros((N,), np.uint32), rocm.zeros((6,))
+    env = capi.pendulum_parameters()
+    lib, h = rocm.device.lib, rocm.device.handle
+    wsn = int(lib.rlt_rocm_pendulum_evaluate_recurrent_workspace_bytes(policy.layers, policy.n, N))
+    ws = rocm.device.empty((wsn,), np.uint8)
+    call = lambda kind, n, period, w, wn: lib.rlt_rocm_pendulum_evaluate_recurrent(h, C.byref(env), kind, policy.layers, policy.n, C.byref(state.c), period, ini.ptr, n, 10,
+                                                                                    ret.ptr, length.ptr, summary.ptr, w, wn)
+    assert call(1, N, 6, ws.ptr, wsn) != 0           # kind 1 needs one output
+    assert call(2, 0, 6, ws.ptr, wsn) != 0
+    assert call(2, N, -1, ws.ptr, wsn) != 0
+    assert call(2, N, 6, ws.ptr, wsn // 2) != 0      # workspace too small
+    assert call(2, N, 6, None, 0) != 0
+    assert call(2, N, 6, ws.ptr, wsn) == 0
+    rocm.sync()
+
