@@ -796,6 +796,45 @@ int rlt_rocm_td3_update_critic_targets(rlt_rocm_device* device, const rlt_td3_ag
 /* update_actor_target     td3/operations_generic.h:322-325 */
 int rlt_rocm_td3_update_actor_target(rlt_rocm_device* device, const rlt_td3_agent* agent);
 
+/* TD3 on sequence batches with sequential (recurrent) networks: rl/algorithms/td3/td3.h ActorCritic and training buffers for
+ * SEQUENCE_LENGTH >= 1 with the approximators of td3/loop/core/approximators_gru.h:9-75 (GRU [-> GRU] [-> dense] -> dense, no
+ * sampling layer, MASK_NON_TERMINAL). S, B, T as in rlt_sac_sequence_agent. */
+typedef struct rlt_td3_sequence_agent {
+    int32_t observation_dim, action_dim, n_actor_layers, n_critic_layers;
+    int32_t include_first_step_in_targets, ignore_termination;
+    float gamma, actor_polyak, critic_polyak, reserved0;
+    rlt_adam_parameters actor_adam, critic_adam;
+    const rlt_seq_layer* actor;              /* last layer: out_dim = action_dim, intermediates for S x B rows */
+    const rlt_seq_layer* actor_target;       /* intermediates for T x B rows */
+    const rlt_seq_layer* critics[2];         /* intermediates for S x B rows */
+    const rlt_seq_layer* critics_target[2];  /* intermediates for T x B rows */
+    const rlt_adam_tensor* actor_adam_tensors;      int32_t n_actor_adam_tensors;   int32_t pad0;
+    const rlt_adam_tensor* critic_adam_tensors[2];  int32_t n_critic_adam_tensors;  int32_t pad1;
+    uint32_t* actor_age; uint32_t* critic_age[2];
+    rlt_sequence_batch batch;
+    float* target_next_action_noise;         /* [T x B x act], already clamped (rlt_rocm_td3_target_action_noise) */
+    float* next_state_action_value_input;    /* [T x B x (obs + act)] */
+    float* next_q[2];                        /* [T x B] */
+    float* target_action_value;              /* [S x B] */
+    float* d_output;                         /* [S x B] */
+    float* state_action_value_input;         /* [S x B x (obs + act)] */
+    float* d_critic_input;                   /* [S x B x (obs + act)] */
+    float* d_actor_output;                   /* [S x B x act] */
+    float* actor_input;                      /* [T x B x obs]: the observation columns of the batch, contiguous, for an actor whose first layer is a GRU */
+    void* workspace; size_t workspace_bytes; /* >= rlt_rocm_td3_sequence_workspace_bytes */
+} rlt_td3_sequence_agent;
+
+size_t rlt_rocm_td3_sequence_workspace_bytes(const rlt_td3_sequence_agent* agent);
+/* train_critic on a sequence batch   rl/algorithms/td3/operations_generic.h:170-235: target actor and target critics over the
+ * `next` views with next_reset, noisy clamped next actions, actions of non-final steps taken from the batch, targets from the
+ * step after, loss reweighted by S*B / (number of final steps), gradient masked to the final steps */
+int rlt_rocm_td3_sequence_train_critic(rlt_rocm_device* device, const rlt_td3_sequence_agent* agent, int critic_index);
+/* train_actor on a sequence batch    td3/operations_generic.h:236-281 (through critic 0) */
+int rlt_rocm_td3_sequence_train_actor(rlt_rocm_device* device, const rlt_td3_sequence_agent* agent);
+/* update_critic_targets / update_actor_target   td3/operations_generic.h:283-325 (dense and GRU layers incl. the initial hidden state) */
+int rlt_rocm_td3_sequence_update_critic_targets(rlt_rocm_device* device, const rlt_td3_sequence_agent* agent);
+int rlt_rocm_td3_sequence_update_actor_target(rlt_rocm_device* device, const rlt_td3_sequence_agent* agent);
+
 /* ------------------------------------------- on-policy collection, normalisation -- */
 
 /* standardize layer       nn/layers/standardize/operations_generic.h:54-67 (set_statistics), :68-86 (evaluate / forward),

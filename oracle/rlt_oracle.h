@@ -39,6 +39,8 @@
  *   seq reset_state / evaluate_step / pendulum runner step with a recurrent policy: runner, policy state and replay rings bit for bit against the
  *   same loop over 300 steps at two depths, the step's draws taken from a copy of the reference's engine; golden vectors; a chain of single steps
  *   equals the sequence forward pass.
+ *   td3_sequence_*: every parameter and Adam age bit for bit against the reference's TD3 loop with its recurrent approximators over 300 loop steps at two
+ *   depths (oracle/_ref/librlt_ref_td3_gru{4,5}_generic.so), target values and d_output too.
  *   pendulum_evaluate_recurrent: returns, lengths and summary bit for bit against rl::utils::evaluation::evaluate on that loop's recurrent actor at two
  *   depths, untrained and trained; golden vectors; equality with pendulum_evaluate for a policy of dense layers only.
  */
@@ -190,6 +192,11 @@ int rlt_oracle_td3_train_critic(const rlt_td3_agent* agent, int critic_index, co
 int rlt_oracle_td3_train_actor(const rlt_td3_agent* agent, const float* sampling_noise);
 int rlt_oracle_td3_update_critic_targets(const rlt_td3_agent* agent);
 int rlt_oracle_td3_update_actor_target(const rlt_td3_agent* agent);
+/* TD3 on sequence batches with sequential (recurrent) networks: rl/algorithms/td3/operations_generic.h:170-325 */
+int rlt_oracle_td3_sequence_train_critic(const rlt_td3_sequence_agent* agent, int critic_index);
+int rlt_oracle_td3_sequence_train_actor(const rlt_td3_sequence_agent* agent);
+int rlt_oracle_td3_sequence_update_critic_targets(const rlt_td3_sequence_agent* agent);
+int rlt_oracle_td3_sequence_update_actor_target(const rlt_td3_sequence_agent* agent);
 
 int rlt_oracle_standardize_set_statistics(const float* mean, const float* std, float* layer_mean, float* layer_precision, int dim);
 int rlt_oracle_standardize_forward(const float* layer_mean, const float* layer_precision, const float* input, int ldin, float* output, int ldo, int batch, int dim);

@@ -231,24 +231,27 @@ int rlt_oracle_sac_sequence_train_critic(const rlt_sac_sequence_agent* A, int ci
     return adam_over(A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci]);   // :336
 }
 
+// polyak update of a sequential model, layer by layer (sac/operations_generic.h:486-527, td3/operations_generic.h:283-316)
+static void polyak_seq(const rlt_seq_layer* source, const rlt_seq_layer* target, int n, float polyak) {
+    for (int l = 0; l < n; l++) {
+        const rlt_seq_layer& s = source[l]; const rlt_seq_layer& t = target[l];
+        if (s.kind == 0) {
+            rlt_oracle_polyak_update(s.dense.weights, t.dense.weights, (size_t)s.dense.in_dim * s.dense.out_dim, polyak, 0);
+            rlt_oracle_polyak_update(s.dense.biases, t.dense.biases, (size_t)s.dense.out_dim, polyak, 0);
+        } else {
+            const size_t H = s.gru.hidden_dim, I = s.gru.input_dim;
+            rlt_oracle_polyak_update(s.gru.weights_input, t.gru.weights_input, 3 * H * I, polyak, 0);
+            rlt_oracle_polyak_update(s.gru.biases_input, t.gru.biases_input, 3 * H, polyak, 0);
+            rlt_oracle_polyak_update(s.gru.weights_hidden, t.gru.weights_hidden, 3 * H * H, polyak, 0);
+            rlt_oracle_polyak_update(s.gru.biases_hidden, t.gru.biases_hidden, 3 * H, polyak, 0);
+            rlt_oracle_polyak_update(s.gru.initial_hidden_state, t.gru.initial_hidden_state, H, polyak, 0);
+        }
+    }
+}
 // :486-527
 int rlt_oracle_sac_sequence_update_critic_targets(const rlt_sac_sequence_agent* A) {
     if (!A) return RLT_E_INVALID_ARGUMENT;
-    for (int k = 0; k < 2; k++)
-        for (int l = 0; l < A->n_critic_layers; l++) {
-            const rlt_seq_layer& s = A->critics[k][l]; const rlt_seq_layer& t = A->critics_target[k][l];
-            if (s.kind == 0) {
-                rlt_oracle_polyak_update(s.dense.weights, t.dense.weights, (size_t)s.dense.in_dim * s.dense.out_dim, A->polyak, 0);
-                rlt_oracle_polyak_update(s.dense.biases, t.dense.biases, (size_t)s.dense.out_dim, A->polyak, 0);
-            } else {
-                const size_t H = s.gru.hidden_dim, I = s.gru.input_dim;
-                rlt_oracle_polyak_update(s.gru.weights_input, t.gru.weights_input, 3 * H * I, A->polyak, 0);
-                rlt_oracle_polyak_update(s.gru.biases_input, t.gru.biases_input, 3 * H, A->polyak, 0);
-                rlt_oracle_polyak_update(s.gru.weights_hidden, t.gru.weights_hidden, 3 * H * H, A->polyak, 0);
-                rlt_oracle_polyak_update(s.gru.biases_hidden, t.gru.biases_hidden, 3 * H, A->polyak, 0);
-                rlt_oracle_polyak_update(s.gru.initial_hidden_state, t.gru.initial_hidden_state, H, A->polyak, 0);
-            }
-        }
+    for (int k = 0; k < 2; k++) polyak_seq(A->critics[k], A->critics_target[k], A->n_critic_layers, A->polyak);
     return 0;
 }
 
@@ -291,6 +294,91 @@ int rlt_oracle_sac_sequence_train_actor(const rlt_sac_sequence_agent* A, const f
     if ((rc = rlt_oracle_seq_backward(A->actor, A->n_actor_layers, obs, D, A->d_actor_output, nullptr, K.reset, S, B, 1, 0))) return rc;
     if ((rc = adam_over(A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age))) return rc;   // :465
     return adam_over(&A->log_alpha, 1, &A->alpha_adam, A->alpha_age);                                             // :466
+}
+
+// ------------------------------------------------------------------------------------------------ TD3 on sequence batches
+static inline const float* seq_out(const rlt_seq_layer* layers, int n) { const rlt_seq_layer& L = layers[n - 1]; return L.kind ? L.gru.output : L.dense.output; }
+
+// rl/algorithms/td3/operations_generic.h:170-235
+int rlt_oracle_td3_sequence_train_critic(const rlt_td3_sequence_agent* A, int ci) {
+    if (!A || ci < 0 || ci > 1 || !A->target_next_action_noise) return RLT_E_INVALID_ARGUMENT;
+    const rlt_sequence_batch& K = A->batch;
+    const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    const int first = A->include_first_step_in_targets ? 1 : 0, T = S + first, next_offset = first ? 0 : 1;     // off_policy_runner/operations_generic.h:85-92
+    const rlt_seq_layer* critic = A->critics[ci];
+    int rc;
+    if ((rc = rlt_oracle_seq_zero_gradient(critic, A->n_critic_layers))) return rc;                                // :185
+    const float* base_next = K.observations_actions_base + (size_t)next_offset * B * D;
+    const uint8_t* next_reset = K.next_reset_base + (size_t)next_offset * B;
+    const uint8_t* next_final = K.next_final_step_mask_base + (size_t)next_offset * B;
+    // batch.observations_next is a view of OBS columns out of D; the layers here take contiguous rows
+    if (!A->actor_input) return RLT_E_INVALID_ARGUMENT;
+    for (int i = 0; i < T * B; i++) std::memcpy(A->actor_input + (size_t)i * OBS, base_next + (size_t)i * D, sizeof(float) * OBS);
+    if ((rc = rlt_oracle_seq_forward(A->actor_target, A->n_actor_layers, A->actor_input, OBS, next_reset, T, B))) return rc;   // :191
+    const float* mean = seq_out(A->actor_target, A->n_actor_layers);
+    float* next_actions = A->next_state_action_value_input + OBS;
+    for (int i = 0; i < T * B; i++) std::memcpy(next_actions + (size_t)i * D, mean + (size_t)i * ACT, sizeof(float) * ACT);
+    if ((rc = rlt_oracle_td3_noisy_next_actions(next_actions, D, A->target_next_action_noise, ACT, T * B, ACT))) return rc;   // :192
+    if ((rc = rlt_oracle_mask_copy(base_next + OBS, D, next_actions, D, next_final, 1, T * B, ACT))) return rc;      // :193-195
+    for (int i = 0; i < T * B; i++) std::memcpy(A->next_state_action_value_input + (size_t)i * D, base_next + (size_t)i * D, sizeof(float) * OBS);   // :196
+    for (int k = 0; k < 2; k++) {                                                                                  // :197-198
+        if ((rc = rlt_oracle_seq_forward(A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, next_reset, T, B))) return rc;
+        std::memcpy(A->next_q[k], seq_out(A->critics_target[k], A->n_critic_layers), sizeof(float) * T * B);
+    }
+    if ((rc = rlt_oracle_td3_target_action_values(A->next_q[0] + first * B, A->next_q[1] + first * B, K.rewards, K.terminated, A->gamma, A->ignore_termination,
+                                                 A->target_action_value, S * B))) return rc;                      // :200 (:146-169: the value of the step after)
+    if ((rc = rlt_oracle_seq_forward(critic, A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B))) return rc;      // :205
+    float n_final = 0;                                                                                             // :207-212
+    rlt_oracle_cast_reduce_sum_u8(K.final_step_mask, (size_t)S * B, &n_final);
+    if (!(n_final > 0)) return RLT_E_INVALID_ARGUMENT;
+    float loss_weight = 1.0f; loss_weight *= (float)(S * B) / n_final;
+    if ((rc = rlt_oracle_mse_gradient(seq_out(critic, A->n_critic_layers), 1, A->target_action_value, 1, A->d_output, 1, S * B, 1, loss_weight, nullptr))) return rc;   // :217
+    rlt_oracle_mask_zero(A->d_output, 1, K.final_step_mask, 1, S * B, 1);                                          // :218-220
+    rlt_oracle_mask_zero(A->target_action_value, 1, K.final_step_mask, 1, S * B, 1);                               // :226 (the logging block, in place)
+    if ((rc = rlt_oracle_seq_backward(critic, A->n_critic_layers, K.observations_actions_base, D, A->d_output, nullptr, K.reset, S, B, 1, 0))) return rc;   // :233
+    return adam_over(A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci]);   // :234
+}
+
+// td3/operations_generic.h:236-281
+int rlt_oracle_td3_sequence_train_actor(const rlt_td3_sequence_agent* A) {
+    if (!A) return RLT_E_INVALID_ARGUMENT;
+    const rlt_sequence_batch& K = A->batch;
+    const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT, R = S * B;
+    const float* obs = K.observations_actions_base;
+    int rc;
+    if (!A->actor_input) return RLT_E_INVALID_ARGUMENT;
+    for (int i = 0; i < R; i++) std::memcpy(A->actor_input + (size_t)i * OBS, obs + (size_t)i * D, sizeof(float) * OBS);
+    if ((rc = rlt_oracle_seq_forward(A->actor, A->n_actor_layers, A->actor_input, OBS, K.reset, S, B))) return rc;   // :255
+    const float* actions = seq_out(A->actor, A->n_actor_layers);
+    float* sav_actions = A->state_action_value_input + OBS;
+    for (int i = 0; i < R; i++) std::memcpy(sav_actions + (size_t)i * D, actions + (size_t)i * ACT, sizeof(float) * ACT);
+    if ((rc = rlt_oracle_mask_copy(obs + OBS, D, sav_actions, D, K.final_step_mask, 1, R, ACT))) return rc;         // :256-258
+    for (int i = 0; i < R; i++) std::memcpy(A->state_action_value_input + (size_t)i * D, obs + (size_t)i * D, sizeof(float) * OBS);   // :259
+    const rlt_seq_layer* critic = A->critics[0];
+    if ((rc = rlt_oracle_seq_forward(critic, A->n_critic_layers, A->state_action_value_input, D, K.reset, S, B))) return rc;      // :261
+    float n_final = 0;                                                                                             // :262-267
+    rlt_oracle_cast_reduce_sum_u8(K.final_step_mask, (size_t)R, &n_final);
+    if (!(n_final > 0)) return RLT_E_INVALID_ARGUMENT;
+    for (int i = 0; i < R; i++) A->d_output[i] = (float)-1 / n_final;
+    rlt_oracle_mask_zero(A->d_output, 1, K.final_step_mask, 1, R, 1);
+    if ((rc = rlt_oracle_seq_backward(critic, A->n_critic_layers, nullptr, 0, A->d_output, A->d_critic_input, K.reset, S, B, 0, 0))) return rc;   // :271
+    for (int i = 0; i < R; i++) std::memcpy(A->d_actor_output + (size_t)i * ACT, A->d_critic_input + (size_t)i * D + OBS, sizeof(float) * ACT);   // :272
+    rlt_oracle_mask_zero(A->d_actor_output, ACT, K.final_step_mask, 1, R, ACT);                                    // :273-275
+    if ((rc = rlt_oracle_seq_zero_gradient(A->actor, A->n_actor_layers))) return rc;                               // :277
+    if ((rc = rlt_oracle_seq_backward(A->actor, A->n_actor_layers, A->actor_input, OBS, A->d_actor_output, nullptr, K.reset, S, B, 1, 0))) return rc;   // :278
+    return adam_over(A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age);               // :280
+}
+
+// td3/operations_generic.h:317-325
+int rlt_oracle_td3_sequence_update_critic_targets(const rlt_td3_sequence_agent* A) {
+    if (!A) return RLT_E_INVALID_ARGUMENT;
+    for (int k = 0; k < 2; k++) polyak_seq(A->critics[k], A->critics_target[k], A->n_critic_layers, A->critic_polyak);
+    return 0;
+}
+int rlt_oracle_td3_sequence_update_actor_target(const rlt_td3_sequence_agent* A) {
+    if (!A) return RLT_E_INVALID_ARGUMENT;
+    polyak_seq(A->actor, A->actor_target, A->n_actor_layers, A->actor_polyak);
+    return 0;
 }
 
 }  // extern "C"

@@ -180,6 +180,22 @@ class SacSequenceAgent(C.Structure):
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
 
 
+class Td3SequenceAgent(C.Structure):
+    _fields_ = [("observation_dim", C.c_int32), ("action_dim", C.c_int32), ("n_actor_layers", C.c_int32), ("n_critic_layers", C.c_int32),
+                ("include_first_step_in_targets", C.c_int32), ("ignore_termination", C.c_int32),
+                ("gamma", C.c_float), ("actor_polyak", C.c_float), ("critic_polyak", C.c_float), ("reserved0", C.c_float),
+                ("actor_adam", AdamParameters), ("critic_adam", AdamParameters),
+                ("actor", C.POINTER(SeqLayer)), ("actor_target", C.POINTER(SeqLayer)), ("critics", C.POINTER(SeqLayer) * 2), ("critics_target", C.POINTER(SeqLayer) * 2),
+                ("actor_adam_tensors", C.POINTER(AdamTensor)), ("n_actor_adam_tensors", C.c_int32), ("pad0", C.c_int32),
+                ("critic_adam_tensors", C.POINTER(AdamTensor) * 2), ("n_critic_adam_tensors", C.c_int32), ("pad1", C.c_int32),
+                ("actor_age", C.c_void_p), ("critic_age", C.c_void_p * 2),
+                ("batch", SequenceBatch),
+                ("target_next_action_noise", C.c_void_p), ("next_state_action_value_input", C.c_void_p), ("next_q", C.c_void_p * 2),
+                ("target_action_value", C.c_void_p), ("d_output", C.c_void_p), ("state_action_value_input", C.c_void_p),
+                ("d_critic_input", C.c_void_p), ("d_actor_output", C.c_void_p), ("actor_input", C.c_void_p),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+
+
 class Td3Agent(C.Structure):
     _fields_ = [("batch", C.c_int32), ("observation_dim", C.c_int32), ("action_dim", C.c_int32), ("n_actor_layers", C.c_int32),
                 ("n_critic_layers", C.c_int32), ("ignore_termination", C.c_int32),
@@ -263,6 +279,10 @@ PROTOTYPES = {
     "seq_evaluate_step": [C.POINTER(SeqLayer), I, P, I, C.POINTER(SeqState), I, P, I, I, P, S],
     "pendulum_evaluate_recurrent": [C.POINTER(PendulumParameters), I, C.POINTER(SeqLayer), I, C.POINTER(SeqState), I, P, I, I, P, P, P, P, S],
     "pendulum_runner_step_recurrent": [C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), C.POINTER(SeqLayer), I, C.POINTER(SeqState), I, C.POINTER(SasParameters), P, P, P, S],
+    "td3_sequence_train_critic": [C.POINTER(Td3SequenceAgent), I],
+    "td3_sequence_train_actor": [C.POINTER(Td3SequenceAgent)],
+    "td3_sequence_update_critic_targets": [C.POINTER(Td3SequenceAgent)],
+    "td3_sequence_update_actor_target": [C.POINTER(Td3SequenceAgent)],
     "sac_sequence_train_critic": [C.POINTER(SacSequenceAgent), I, P],
     "sac_sequence_update_critic_targets": [C.POINTER(SacSequenceAgent)],
     "sac_sequence_train_actor": [C.POINTER(SacSequenceAgent), P],
@@ -294,6 +314,7 @@ ROCM_ONLY = {
     "pendulum_runner_step_recurrent_workspace_bytes": ([C.POINTER(SeqLayer), I, I], S),
     "pendulum_evaluate_recurrent_workspace_bytes": ([C.POINTER(SeqLayer), I, I], S),
     "sac_sequence_workspace_bytes": ([C.POINTER(SacSequenceAgent)], S),
+    "td3_sequence_workspace_bytes": ([C.POINTER(Td3SequenceAgent)], S),
     "on_policy_collect_workspace_bytes": ([C.POINTER(PendulumRunner), LP, I], S),
     "gather_draw": ([P, C.POINTER(ReplayBuffer), I, U64, U64, P, P], I),
     "sac_pendulum_loop": ([P, C.POINTER(SacAgent), C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, U64, U64, C.POINTER(SacLoopInputs),

@@ -276,3 +276,142 @@ int rlt_rocm_td3_update_actor_target(rlt_rocm_device* device, const rlt_td3_agen
 }
 
 }  // extern "C"
+
+// ------------------------------------------------------------------------------------------------ TD3 on sequence batches
+namespace {
+__global__ __launch_bounds__(256) void td3_copy_columns_kernel(const float* __restrict__ src, int lds, float* __restrict__ dst, int ldd, int rows, int cols) {
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < (long)rows * cols; i += (long)gridDim.x * blockDim.x) {
+        const long r = i / cols; const int c = (int)(i - r * cols);
+        dst[r * ldd + c] = src[r * lds + c];
+    }
+}
+int copy_columns(rlt_rocm_device* device, const float* src, int lds, float* dst, int ldd, int rows, int cols) {
+    long blocks = ((long)rows * cols + 255) / 256; if (blocks > 4096) blocks = 4096; if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(td3_copy_columns_kernel, dim3((unsigned)blocks), dim3(256), 0, device->stream, src, lds, dst, ldd, rows, cols);
+    return rlt_launch_status(device);
+}
+inline const float* seq_last_output(const rlt_seq_layer* layers, int n) { const rlt_seq_layer& L = layers[n - 1]; return L.kind ? L.gru.output : L.dense.output; }
+inline int seq_last_dim(const rlt_seq_layer* layers, int n) { const rlt_seq_layer& L = layers[n - 1]; return L.kind ? L.gru.hidden_dim : L.dense.out_dim; }
+int polyak_seq(rlt_rocm_device* device, const rlt_seq_layer* source, const rlt_seq_layer* target, int n, float polyak) {
+    int rc;
+    for (int l = 0; l < n; l++) {
+        const rlt_seq_layer& s = source[l]; const rlt_seq_layer& t = target[l];
+        RLT_REQUIRE(s.kind == t.kind);
+        if (s.kind == 0) {
+            if ((rc = rlt_rocm_polyak_update(device, s.dense.weights, t.dense.weights, (size_t)s.dense.in_dim * s.dense.out_dim, polyak, 0))) return rc;
+            if ((rc = rlt_rocm_polyak_update(device, s.dense.biases, t.dense.biases, (size_t)s.dense.out_dim, polyak, 0))) return rc;
+        } else {
+            const size_t H = s.gru.hidden_dim, I = s.gru.input_dim;
+            if ((rc = rlt_rocm_polyak_update(device, s.gru.weights_input, t.gru.weights_input, 3 * H * I, polyak, 0))) return rc;
+            if ((rc = rlt_rocm_polyak_update(device, s.gru.biases_input, t.gru.biases_input, 3 * H, polyak, 0))) return rc;
+            if ((rc = rlt_rocm_polyak_update(device, s.gru.weights_hidden, t.gru.weights_hidden, 3 * H * H, polyak, 0))) return rc;
+            if ((rc = rlt_rocm_polyak_update(device, s.gru.biases_hidden, t.gru.biases_hidden, 3 * H, polyak, 0))) return rc;
+            if ((rc = rlt_rocm_polyak_update(device, s.gru.initial_hidden_state, t.gru.initial_hidden_state, H, polyak, 0))) return rc;
+        }
+    }
+    return 0;
+}
+bool td3_sequence_agent_ok(const rlt_td3_sequence_agent* A) {
+    if (!A || A->observation_dim <= 0 || A->action_dim <= 0 || A->n_actor_layers < 1 || A->n_critic_layers < 1) return false;
+    if (!A->actor || !A->actor_target || !A->critics[0] || !A->critics[1] || !A->critics_target[0] || !A->critics_target[1]) return false;
+    const rlt_sequence_batch& K = A->batch;
+    if (K.batch <= 0 || K.sequence_length <= 0 || !K.observations_actions_base || !K.rewards || !K.terminated || !K.reset || !K.next_reset_base || !K.final_step_mask ||
+        !K.next_final_step_mask_base) return false;
+    if (seq_last_dim(A->actor, A->n_actor_layers) != A->action_dim || seq_last_dim(A->actor_target, A->n_actor_layers) != A->action_dim) return false;
+    for (int k = 0; k < 2; k++) if (seq_last_dim(A->critics[k], A->n_critic_layers) != 1 || seq_last_dim(A->critics_target[k], A->n_critic_layers) != 1) return false;
+    if (!A->actor_input || !A->d_output || !A->target_action_value) return false;
+    return A->workspace && A->workspace_bytes >= rlt_rocm_td3_sequence_workspace_bytes(A);
+}
+}  // namespace
+
+extern "C" {
+
+size_t rlt_rocm_td3_sequence_workspace_bytes(const rlt_td3_sequence_agent* A) {
+    if (!A || !A->actor || !A->actor_target || !A->critics[0] || !A->critics_target[0]) return 0;
+    const int T = A->batch.sequence_length + 1, B = A->batch.batch;
+    size_t n = rlt_rocm_seq_workspace_bytes(A->actor, A->n_actor_layers, T, B);
+    n = std::max(n, rlt_rocm_seq_workspace_bytes(A->actor_target, A->n_actor_layers, T, B));
+    n = std::max(n, rlt_rocm_seq_workspace_bytes(A->critics[0], A->n_critic_layers, T, B));
+    return std::max(n, rlt_rocm_seq_workspace_bytes(A->critics_target[0], A->n_critic_layers, T, B));
+}
+
+// rl/algorithms/td3/operations_generic.h:170-235 on a sequence batch, one launch per reference operation
+int rlt_rocm_td3_sequence_train_critic(rlt_rocm_device* device, const rlt_td3_sequence_agent* A, int ci) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(td3_sequence_agent_ok(A) && (ci == 0 || ci == 1));
+    RLT_REQUIRE(A->target_next_action_noise && A->next_state_action_value_input && A->next_q[0] && A->next_q[1]);
+    const rlt_sequence_batch& K = A->batch;
+    const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    const int first = A->include_first_step_in_targets ? 1 : 0, T = S + first, next_offset = first ? 0 : 1;   // off_policy_runner/operations_generic.h:85-92
+    const rlt_seq_layer* critic = A->critics[ci];
+    void* ws = A->workspace; const size_t ws_bytes = A->workspace_bytes;
+    int rc;
+    if ((rc = rlt_rocm_seq_zero_gradient(device, critic, A->n_critic_layers))) return rc;                                                  // :185
+    const float* base_next = K.observations_actions_base + (size_t)next_offset * B * D;
+    const uint8_t* next_reset = K.next_reset_base + (size_t)next_offset * B;
+    const uint8_t* next_final = K.next_final_step_mask_base + (size_t)next_offset * B;
+    if ((rc = copy_columns(device, base_next, D, A->actor_input, OBS, T * B, OBS))) return rc;                                             // the observation columns, contiguous
+    if ((rc = rlt_rocm_seq_forward(device, A->actor_target, A->n_actor_layers, A->actor_input, OBS, next_reset, T, B, ws, ws_bytes))) return rc;   // :191
+    float* next_actions = A->next_state_action_value_input + OBS;
+    if ((rc = copy_columns(device, seq_last_output(A->actor_target, A->n_actor_layers), ACT, next_actions, D, T * B, ACT))) return rc;
+    if ((rc = rlt_rocm_td3_noisy_next_actions(device, next_actions, D, A->target_next_action_noise, ACT, T * B, ACT))) return rc;          // :192
+    if ((rc = rlt_rocm_mask_copy(device, base_next + OBS, D, next_actions, D, next_final, 1, T * B, ACT))) return rc;                      // :193-195
+    if ((rc = copy_columns(device, base_next, D, A->next_state_action_value_input, D, T * B, OBS))) return rc;                             // :196
+    for (int k = 0; k < 2; k++) {                                                                                                          // :197-198
+        if ((rc = rlt_rocm_seq_forward(device, A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, next_reset, T, B, ws, ws_bytes))) return rc;
+        if ((rc = rlt_rocm_memcpy_d2d(device, A->next_q[k], seq_last_output(A->critics_target[k], A->n_critic_layers), sizeof(float) * T * B))) return rc;
+    }
+    if ((rc = rlt_rocm_seq_forward(device, critic, A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, ws, ws_bytes))) return rc;   // :205
+    // :200-227: targets from the value of the step after (offset B where the first step is included), reweighted and masked gradient
+    hipLaunchKernelGGL(td3_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, const_cast<float*>(seq_last_output(critic, A->n_critic_layers)),
+                       (const float*)(A->next_q[0] + (size_t)first * B), (const float*)(A->next_q[1] + (size_t)first * B), (const float*)K.rewards, (const uint8_t*)K.terminated,
+                       A->gamma, A->ignore_termination, A->target_action_value, (const uint8_t*)K.final_step_mask, A->d_output, S * B, 0);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if ((rc = rlt_rocm_seq_backward(device, critic, A->n_critic_layers, K.observations_actions_base, D, A->d_output, nullptr, K.reset, S, B, 1, 0, ws, ws_bytes))) return rc;   // :233
+    return rlt_rocm_adam_step(device, A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], 0.0f, nullptr);   // :234
+}
+
+// td3/operations_generic.h:236-281 on a sequence batch
+int rlt_rocm_td3_sequence_train_actor(rlt_rocm_device* device, const rlt_td3_sequence_agent* A) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(td3_sequence_agent_ok(A) && A->state_action_value_input && A->d_critic_input && A->d_actor_output && A->actor_adam_tensors && A->actor_age);
+    const rlt_sequence_batch& K = A->batch;
+    const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT, R = S * B;
+    const float* obs = K.observations_actions_base;
+    void* ws = A->workspace; const size_t ws_bytes = A->workspace_bytes;
+    int rc;
+    if ((rc = copy_columns(device, obs, D, A->actor_input, OBS, R, OBS))) return rc;
+    if ((rc = rlt_rocm_seq_forward(device, A->actor, A->n_actor_layers, A->actor_input, OBS, K.reset, S, B, ws, ws_bytes))) return rc;      // :255
+    float* sav_actions = A->state_action_value_input + OBS;
+    if ((rc = copy_columns(device, seq_last_output(A->actor, A->n_actor_layers), ACT, sav_actions, D, R, ACT))) return rc;
+    if ((rc = rlt_rocm_mask_copy(device, obs + OBS, D, sav_actions, D, K.final_step_mask, 1, R, ACT))) return rc;                          // :256-258
+    if ((rc = copy_columns(device, obs, D, A->state_action_value_input, D, R, OBS))) return rc;                                            // :259
+    const rlt_seq_layer* critic = A->critics[0];
+    if ((rc = rlt_rocm_seq_forward(device, critic, A->n_critic_layers, A->state_action_value_input, D, K.reset, S, B, ws, ws_bytes))) return rc;   // :261
+    hipLaunchKernelGGL(td3_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, (float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+                       (const uint8_t*)nullptr, 0.0f, 0, (float*)nullptr, (const uint8_t*)K.final_step_mask, A->d_output, R, 1);           // :262-267
+    if ((rc = rlt_launch_status(device))) return rc;
+    if ((rc = rlt_rocm_seq_backward(device, critic, A->n_critic_layers, nullptr, 0, A->d_output, A->d_critic_input, K.reset, S, B, 0, 0, ws, ws_bytes))) return rc;   // :271
+    if ((rc = copy_columns(device, A->d_critic_input + OBS, D, A->d_actor_output, ACT, R, ACT))) return rc;                                // :272
+    if ((rc = rlt_rocm_mask_zero(device, A->d_actor_output, ACT, K.final_step_mask, 1, R, ACT))) return rc;                                // :273-275
+    if ((rc = rlt_rocm_seq_zero_gradient(device, A->actor, A->n_actor_layers))) return rc;                                                 // :277
+    if ((rc = rlt_rocm_seq_backward(device, A->actor, A->n_actor_layers, A->actor_input, OBS, A->d_actor_output, nullptr, K.reset, S, B, 1, 0, ws, ws_bytes))) return rc;   // :278
+    return rlt_rocm_adam_step(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, 0.0f, nullptr);        // :280
+}
+
+// td3/operations_generic.h:283-325
+int rlt_rocm_td3_sequence_update_critic_targets(rlt_rocm_device* device, const rlt_td3_sequence_agent* A) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(td3_sequence_agent_ok(A));
+    int rc;
+    for (int k = 0; k < 2; k++)
+        if ((rc = polyak_seq(device, A->critics[k], A->critics_target[k], A->n_critic_layers, A->critic_polyak))) return rc;
+    return 0;
+}
+int rlt_rocm_td3_sequence_update_actor_target(rlt_rocm_device* device, const rlt_td3_sequence_agent* A) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(td3_sequence_agent_ok(A));
+    return polyak_seq(device, A->actor, A->actor_target, A->n_actor_layers, A->actor_polyak);
+}
+
+}  // extern "C"

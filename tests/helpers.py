@@ -1155,6 +1155,145 @@ class SacSequenceOnBackend:
         return [int(x.numpy()[0]) for x in (self.actor.age, self.critics[0].age, self.critics[1].age, self.alpha_age)]
 
 
+class Td3SequenceOnBackend:
+    """All state of a TD3 agent with sequential (recurrent) networks on one backend. params: flat [actor, critic 0, critic 1, actor target, critic target 0,
+    critic target 1] with every network laid out layer after layer (the order the reference harness exports)."""
+
+    def __init__(self, backend, actor_specs, critic_specs, params, S, B, obs_dim, act_dim, include_first=True, hyper=None):
+        self.backend, self.S, self.B = backend, S, B
+        T, D = S + (1 if include_first else 0), obs_dim + act_dim
+        self.T = T
+        na, nc = seq_param_count(actor_specs), seq_param_count(critic_specs)
+        o = 0
+        self.actor = SeqNet(backend, actor_specs, params[o:o + na], S, B); o += na
+        self.critics = [SeqNet(backend, critic_specs, params[o + k * nc:o + (k + 1) * nc], S, B) for k in range(2)]; o += 2 * nc
+        self.actor_target = SeqNet(backend, actor_specs, params[o:o + na], T, B, trainable=False); o += na
+        self.targets = [SeqNet(backend, critic_specs, params[o + k * nc:o + (k + 1) * nc], T, B, trainable=False) for k in range(2)]; o += 2 * nc
+        self.batch = SequenceBatchOnBackend(backend, B, S, D)
+        z = backend.zeros
+        self.buf = dict(noise=z((T, B, act_dim)), nsavi=z((T, B, D)), next_q0=z((T, B)), next_q1=z((T, B)), target=z((S, B)), d_output=z((S, B)), savi=z((S, B, D)),
+                        d_ci=z((S, B, D)), d_ao=z((S, B, act_dim)), a_in=z((T, B, obs_dim)))
+        A = capi.Td3SequenceAgent()
+        A.observation_dim, A.action_dim, A.n_actor_layers, A.n_critic_layers, A.include_first_step_in_targets = obs_dim, act_dim, len(actor_specs), len(critic_specs), int(include_first)
+        hyper = hyper or {}
+        polyak = float(np.float32(1.0 - 0.005))
+        A.gamma, A.actor_polyak, A.critic_polyak = hyper.get("gamma", 0.99), hyper.get("actor_polyak", polyak), hyper.get("critic_polyak", polyak)
+        A.ignore_termination = int(hyper.get("ignore_termination", 0))
+        A.actor_adam, A.critic_adam = (hyper.get(k, capi.adam_parameters()) for k in ("actor_adam", "critic_adam"))
+        A.actor, A.actor_target, A.actor_adam_tensors, A.n_actor_adam_tensors, A.actor_age = self.actor.layers, self.actor_target.layers, self.actor.adam, self.actor.n_adam, self.actor.age.ptr
+        b = self.buf
+        for k in range(2):
+            A.critics[k], A.critics_target[k] = self.critics[k].layers, self.targets[k].layers
+            A.critic_adam_tensors[k], A.critic_age[k] = self.critics[k].adam, self.critics[k].age.ptr
+            A.next_q[k] = b[f"next_q{k}"].ptr
+        A.n_critic_adam_tensors = self.critics[0].n_adam
+        A.batch = self.batch.c
+        A.target_next_action_noise, A.next_state_action_value_input, A.target_action_value, A.d_output = b["noise"].ptr, b["nsavi"].ptr, b["target"].ptr, b["d_output"].ptr
+        A.state_action_value_input, A.d_critic_input, A.d_actor_output, A.actor_input = b["savi"].ptr, b["d_ci"].ptr, b["d_ao"].ptr, b["a_in"].ptr
+        if backend.name == "rocm":
+            n = int(backend.device.lib.rlt_rocm_td3_sequence_workspace_bytes(C.byref(A)))
+            self.ws = backend.device.empty((max(n, 4),), np.uint8)
+            A.workspace, A.workspace_bytes = self.ws.ptr, n
+        self.c = A
+
+    def set_batch(self, data):
+        for k in SEQUENCE_BATCH_FIELDS:
+            self.batch.arrays[k].upload(data[k])
+
+    def train(self, noise, flags=(1, 1, 1, 1)):
+        """The training part of one loop step with a shared batch (rl/algorithms/td3/loop/core/operations_generic.h:91-127); noise: the clamped target-action
+        noise [T x B x act]; flags: (train critics, update critic targets, train actor, update actor target)."""
+        be = self.backend
+        self.buf["noise"].upload(np.ascontiguousarray(noise, np.float32).reshape(self.buf["noise"].shape))
+        if flags[0]:
+            for k in range(2):
+                be.call("td3_sequence_train_critic", C.byref(self.c), k)
+        if flags[1]:
+            be.call("td3_sequence_update_critic_targets", C.byref(self.c))
+        if flags[2]:
+            be.call("td3_sequence_train_actor", C.byref(self.c))
+        if flags[3]:
+            be.call("td3_sequence_update_actor_target", C.byref(self.c))
+        be.sync()
+
+    def parameters(self):
+        return np.concatenate([self.actor.params.numpy()] + [c.params.numpy() for c in self.critics] + [self.actor_target.params.numpy()] + [t.params.numpy() for t in self.targets])
+
+    def ages(self):
+        return [int(x.numpy()[0]) for x in (self.actor.age, self.critics[0].age, self.critics[1].age)]
+
+
+class RefTd3Gru:
+    """The reference's own TD3 loop with recurrent approximators on sequence batches (oracle/_ref, compiled from /root/reference)."""
+
+    def __init__(self, n_layers, seed):
+        self.lib = lib = C.CDLL(os.path.join(ORACLE_DIR, "_ref", f"librlt_ref_td3_gru{n_layers}_generic.so"))
+        P = C.c_void_p
+        lib.rlt_ref_td3_gru_create.restype = P; lib.rlt_ref_td3_gru_create.argtypes = [C.c_uint32]
+        lib.rlt_ref_td3_gru_parameter_count.restype = C.c_size_t; lib.rlt_ref_td3_gru_parameter_count.argtypes = [P]
+        lib.rlt_ref_td3_gru_step_count.restype = C.c_uint32; lib.rlt_ref_td3_gru_step_count.argtypes = [P]
+        lib.rlt_ref_td3_gru_layers.argtypes = [P, C.c_int, P]
+        for f, n in (("destroy", 1), ("step", 1), ("get_parameters", 2), ("get_ages", 2), ("hyperparameters", 2), ("get_noise", 2), ("get_batch", 8), ("dims", 1),
+                     ("get_critic_buffers", 3)):
+            getattr(lib, "rlt_ref_td3_gru_" + f).argtypes = [P] * n
+        self.h = lib.rlt_ref_td3_gru_create(seed)
+        d = np.zeros(11, np.int32); lib.rlt_ref_td3_gru_dims(d.ctypes.data)
+        self.batch, self.seq, self.n_warmup, self.obs_dim, self.act_dim, self.include_first = [int(x) for x in d[:6]]
+        self.intervals, self.ignore_termination = [int(x) for x in d[6:10]], int(d[10])
+        buf = np.zeros(64, np.int32)
+        self.specs = []
+        for critic in (0, 1):
+            n = lib.rlt_ref_td3_gru_layers(self.h, critic, buf.ctypes.data)
+            self.specs.append([(int(k), int(i), int(o), ACT_NAMES[int(a)]) for k, i, o, a in buf[:n].reshape(-1, 4)])
+        self.actor_specs, self.critic_specs = self.specs
+        hp = np.zeros(15, np.float32); lib.rlt_ref_td3_gru_hyperparameters(self.h, hp.ctypes.data)
+        self.hp = hp
+
+    def hyper(self):
+        hp = self.hp
+        adam = lambda o: capi.adam_parameters(alpha=float(hp[o]), beta_1=float(hp[o + 1]), beta_2=float(hp[o + 2]), epsilon=float(hp[o + 3]), epsilon_sqrt=float(hp[o + 4]))
+        return dict(gamma=float(hp[0]), actor_polyak=float(hp[1]), critic_polyak=float(hp[2]), ignore_termination=self.ignore_termination, actor_adam=adam(5), critic_adam=adam(10))
+
+    def flags(self, step):
+        """(train critics, update critic targets, train actor, update actor target) of loop step number `step` (td3/loop/core/operations_generic.h:91-94)."""
+        return tuple(int(step >= self.n_warmup and step % iv == 0) for iv in self.intervals)
+
+    def step_count(self):
+        return int(self.lib.rlt_ref_td3_gru_step_count(self.h))
+
+    def step(self):
+        self.lib.rlt_ref_td3_gru_step(self.h)
+
+    def parameters(self):
+        p = np.zeros(self.lib.rlt_ref_td3_gru_parameter_count(self.h), np.float32)
+        self.lib.rlt_ref_td3_gru_get_parameters(self.h, p.ctypes.data)
+        return p
+
+    def ages(self):
+        a = np.zeros(3, np.uint32); self.lib.rlt_ref_td3_gru_get_ages(self.h, a.ctypes.data); return [int(x) for x in a]
+
+    def batch_data(self):
+        S, B, D = self.seq, self.batch, self.obs_dim + self.act_dim
+        out = dict(observations_actions_base=np.zeros((S + 1, B, D), np.float32), rewards=np.zeros((S, B), np.float32), terminated=np.zeros((S, B), np.uint8),
+                   reset=np.zeros((S, B), np.uint8), next_reset_base=np.zeros((S + 1, B), np.uint8), final_step_mask=np.zeros((S, B), np.uint8),
+                   next_final_step_mask_base=np.zeros((S + 1, B), np.uint8))
+        self.lib.rlt_ref_td3_gru_get_batch(self.h, *[out[k].ctypes.data for k in SEQUENCE_BATCH_FIELDS])
+        return out
+
+    def noise(self):
+        nz = np.zeros((self.seq + 1, self.batch, self.act_dim), np.float32)
+        self.lib.rlt_ref_td3_gru_get_noise(self.h, nz.ctypes.data)
+        return nz
+
+    def critic_buffers(self):
+        y, d = np.zeros((self.seq, self.batch), np.float32), np.zeros((self.seq, self.batch), np.float32)
+        self.lib.rlt_ref_td3_gru_get_critic_buffers(self.h, y.ctypes.data, d.ctypes.data)
+        return y, d
+
+    def close(self):
+        self.lib.rlt_ref_td3_gru_destroy(self.h)
+
+
 class RefSacGru:
     """The reference's own SAC loop with recurrent approximators on sequence batches (oracle/_ref, compiled from /root/reference)."""
 

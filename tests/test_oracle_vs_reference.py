@@ -613,3 +613,32 @@ def test_evaluation_with_recurrent_policy_bit_exact_with_reference(oracle, n_lay
             assert np.array_equal(g[p + "summary"], summary)
     ref.close()
 
+
+@pytest.mark.parametrize("n_layers", [4, 5])
+def test_td3_sequence_bit_exact_with_reference(oracle, n_layers):
+    """The reference's TD3 loop with its recurrent approximators (actor GRU 16, GRU 16[, dense 16], dense 1; critics alike) on sequence batches of 16 x 6 steps:
+    from the parameters after the warm-up, the restatement is given the batch and the clamped target-action noise of every loop step and must reproduce every
+    parameter of the six networks (incl. the polyak-averaged targets, every second step) and the Adam ages bit for bit over 300 loop steps, free-running (its own
+    parameters are never re-synchronised); the critic's target values and d_output of the last update are compared too."""
+    ref = helpers.RefTd3Gru(n_layers, 5)
+    for _ in range(ref.n_warmup):
+        ref.step()
+    assert ref.intervals == [1, 2, 2, 2] and ref.include_first == 1
+    assert [k for k, _, _, _ in ref.actor_specs] == ([1, 1, 0] if n_layers == 4 else [1, 1, 0, 0])
+    agent = helpers.Td3SequenceOnBackend(oracle, ref.actor_specs, ref.critic_specs, ref.parameters(), ref.seq, ref.batch, ref.obs_dim, ref.act_dim, True, ref.hyper())
+    trained_actor = 0
+    for i in range(300):
+        flags = ref.flags(ref.step_count())
+        ref.step()
+        agent.set_batch(ref.batch_data())
+        agent.train(ref.noise(), flags)
+        trained_actor += flags[2]
+        assert np.array_equal(agent.parameters(), ref.parameters()), (i, flags, float(np.abs(agent.parameters() - ref.parameters()).max()))
+        assert agent.ages() == ref.ages()
+        y, d = ref.critic_buffers()
+        assert np.array_equal(agent.buf["target"].numpy(), y), i
+        if not flags[2]:                        # the agent here has one d_output for critic and actor updates
+            assert np.array_equal(agent.buf["d_output"].numpy(), d), i
+    assert trained_actor == 150
+    ref.close()
+
