@@ -79,10 +79,17 @@ int rlt_rocm_memcpy2d(rlt_rocm_device* device, void* dst, size_t dst_pitch, cons
 /* set_all                 containers/matrix/operations_cuda.h:62-74,201-207 */
 int rlt_rocm_fill_f32(rlt_rocm_device* device, float* dst, int rows, int cols, int ld, float value);
 int rlt_rocm_fill_u8(rlt_rocm_device* device, uint8_t* dst, size_t count, uint8_t value);
-/* randn / rand            containers/tensor/operations_cuda.h:548-624 (counter-based: the stream of
- * values is a pure function of (seed, offset, element index), no state array is needed) */
-int rlt_rocm_randn_f32(rlt_rocm_device* device, float* dst, size_t count, uint64_t seed, uint64_t offset);
-int rlt_rocm_rand_f32(rlt_rocm_device* device, float* dst, size_t count, float low, float high, uint64_t seed, uint64_t offset);
+/* randn / rand            containers/tensor/operations_cuda.h:548-624
+ * Counter-based (Philox4x32-10): element i of a call is word i % 4 of group i / 4 of the sequence that (seed, stream) selects --
+ * key = seed, counter = (group index, stream). No state array exists. Calls with different `stream` values (or seeds) draw from
+ * disjoint sequences of 2^64 groups whatever their lengths, so a caller that passes a fresh stream number per call (a counter it
+ * increments, as the reference advances its generator state) never sees a value twice. rand is uniform on (low, high) from 24 bits
+ * per value, randn is Box-Muller on the two word pairs of a group. */
+int rlt_rocm_randn_f32(rlt_rocm_device* device, float* dst, size_t count, uint64_t seed, uint64_t stream);
+int rlt_rocm_rand_f32(rlt_rocm_device* device, float* dst, size_t count, float low, float high, uint64_t seed, uint64_t stream);
+/* The raw 32-bit words of the same sequence (no counterpart in the reference: lets a caller check the generator against the
+ * published Philox4x32-10 vectors or build other distributions). */
+int rlt_rocm_rand_bits_u32(rlt_rocm_device* device, uint32_t* dst, size_t count, uint64_t seed, uint64_t stream);
 /* scale(t, s, reciprocal) containers/tensor/operations_generic.h:433-445,713 : x <- reciprocal ? (1/x)*s : x*s (rounded in that order) */
 int rlt_rocm_scale_f32(rlt_rocm_device* device, float* x, size_t count, float s, int reciprocal);
 /* cast_reduce_sum<T>(bool tensor) containers/tensor/operations_generic.h:928-985 (CUDA: <<<1,1>>>, operations_cuda.h:287-307) */
@@ -378,9 +385,10 @@ int rlt_rocm_gather_sequence_batch(rlt_rocm_device* device, const rlt_replay_buf
                                    const rlt_sequence_draws* draws, int max_episode_length, const rlt_sequence_batch* batch);
 
 /* Device-side draw of (env, offset) pairs, uniform over the eligible rows of each ring
- * (off_policy_runner/operations_generic.h:257,304,426). */
+ * (off_policy_runner/operations_generic.h:257,304,426): sample i takes words 0 and 1 of Philox group i of the sequence that
+ * (seed, stream) selects (see rlt_rocm_randn_f32); pass a fresh stream number per call. */
 int rlt_rocm_gather_draw(rlt_rocm_device* device, const rlt_replay_buffer* rb, int batch,
-                         uint64_t seed, uint64_t offset, uint32_t* env_indices, uint32_t* sample_offsets);
+                         uint64_t seed, uint64_t stream, uint32_t* env_indices, uint32_t* sample_offsets);
 
 /* rl/environments/pendulum/pendulum.h:12-25 */
 typedef struct rlt_pendulum_parameters {
@@ -447,7 +455,8 @@ typedef struct rlt_pendulum_runner {
 /* One off-policy runner step for all environments in a single launch
  * (prologue/interlude/epilogue, off_policy_runner/operations_generic.h:183-238, _per_env.h:8-108,
  * operations_cuda.h:60-203): reset-if-truncated from `initial_states` [n_envs x 2] (consumed only where a
- * reset happens; may be NULL to re-draw on the device from (seed, offset)), observe, deterministic
+ * reset happens; may be NULL to re-draw on the device: environment e takes words 0 and 1 of Philox group e of the
+ * sequence that (seed, stream) selects, a fresh stream number per call), observe, deterministic
  * tanh/identity actor MLP or tanh-Gaussian actor with `action_noise` [n_envs x act], env step, reward,
  * next observation, truncation, and the replay `add`.
  *   policy_kind: 0 = actions given in `actions_in` (e.g. uniform warm-up policy drawn by the host)
@@ -457,7 +466,7 @@ int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_ru
                                   const rlt_replay_buffer* rb, int policy_kind,
                                   const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas,
                                   const float* actions_in, const float* action_noise,
-                                  const float* initial_states, uint64_t seed, uint64_t offset);
+                                  const float* initial_states, uint64_t seed, uint64_t stream);
 /* The same runner step with a sequential (recurrent) policy whose last layer yields [mean | log_std]
  * (rl/components/off_policy_runner/operations_generic.h:189-206): the policy state of the environments that start a new
  * episode is reset, then one evaluate_step in Rollout mode (sample_and_squash with action_noise [n_envs x 1]).
@@ -478,7 +487,10 @@ int rlt_rocm_pendulum_evaluate(rlt_rocm_device* device, const rlt_pendulum_param
                                int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary);
 
 /* Host-drawn randomness for rlt_rocm_sac_pendulum_loop (parity runs feed the draws the reference's CPU RNG made); any member
- * may be NULL, in which case the kernel draws from its counter-based generator keyed by (seed, step). */
+ * may be NULL, in which case the kernel draws it itself: Philox4x32-10 groups keyed by the launch's seed, one stream per kind of
+ * draw (1 initial state: words 0, 1 -> theta, theta_dot; 3 rollout noise; 4 gather offset: word 0 scaled to the eligible rows;
+ * 5 / 6 critic / actor noise; normals are Box-Muller on words 0, 1), group index = step_offset + step, times batch plus the
+ * sample where the draw is per sample. Launches that continue a run pass the same seed and the next step_offset. */
 typedef struct rlt_sac_loop_inputs {
     const float* rollout_noise;       /* [n_steps x action_dim] exploration noise of the runner's actor                 */
     const float* initial_states;      /* [n_steps x 2] (theta, theta_dot), read at the steps where an episode resets    */
@@ -495,6 +507,13 @@ typedef struct rlt_sac_loop_outputs {  /* all optional */
     uint64_t* phase_ticks;             /* [16] profiling aid: constant-rate (100 MHz) clock ticks workgroup 0 spent per phase,
                                           ADDED to what is there: 0 env step, 1 critic phase, 2/4/7/9 grid barriers, 3 critic Adam,
                                           5 critic weight refresh, 6 actor phase, 8 actor Adam, 10 actor weight refresh            */
+    /* the draws every step used -- the caller's arrays echoed, or what the kernel drew itself -- in the layout of rlt_sac_loop_inputs,
+     * so that a run on device-drawn randomness can be replayed step by step elsewhere */
+    float* drawn_rollout_noise;        /* [n_steps]                                                                       */
+    float* drawn_initial_states;       /* [n_steps x 2] written at the steps where an episode resets, untouched elsewhere */
+    uint32_t* drawn_sample_offsets;    /* [n_steps x batch]                                                               */
+    float* drawn_noise_critic;         /* [n_steps x batch]                                                               */
+    float* drawn_noise_actor;          /* [n_steps x batch]                                                               */
 } rlt_sac_loop_outputs;
 
 /* n_steps iterations of sac::loop::core::step (rl/algorithms/sac/loop/core/operations_generic.h:110-155, past the warm-up:

@@ -41,6 +41,10 @@
  *   equals the sequence forward pass.
  *   td3_sequence_*: every parameter and Adam age bit for bit against the reference's TD3 loop with its recurrent approximators over 300 loop steps at two
  *   depths (oracle/_ref/librlt_ref_td3_gru{4,5}_generic.so), target values and d_output too.
+ *   philox4x32_10, rand_bits / rand / randn / gather_draw / pendulum_initial_states (rlt_oracle_rng.cpp): the block function against the three
+ *   published known-answer vectors of Philox4x32-10; the conversions by range, moments and Kolmogorov-Smirnov distance; no reference counterpart
+ *   fixes the sequence itself (the reference's CUDA and CPU generators differ from each other).
+ *   reduce_sum_f32, adam_reset: against numpy closed forms (tests/test_oracle_rng.py, tests/test_oracle_closed_forms.py).
  *   pendulum_evaluate_recurrent: returns, lengths and summary bit for bit against rl::utils::evaluation::evaluate on that loop's recurrent actor at two
  *   depths, untrained and trained; golden vectors; equality with pendulum_evaluate for a policy of dense layers only.
  */
@@ -102,6 +106,17 @@ int rlt_oracle_mask_copy(const float* source, int lds, float* target, int ldt, c
 int rlt_oracle_mask_zero(float* gradient, int ld, const uint8_t* mask, int invert, int rows, int cols);
 int rlt_oracle_scale_f32(float* x, size_t count, float s, int reciprocal);
 int rlt_oracle_cast_reduce_sum_u8(const uint8_t* mask, size_t count, float* out_sum);
+/* squared_sum / sum of a tensor (containers/tensor/operations_generic.h:497-520,803; gradient_norm of a parameter,
+ * nn/parameters/operations_generic.h:85-87), accumulated in double and rounded once */
+int rlt_oracle_reduce_sum_f32(const float* x, size_t count, int squared, float* out_sum);
+
+/* ---- random draws (rlt_oracle_rng.cpp): Philox4x32-10 and the (seed, stream, element) mapping of include/rlt_rocm.h */
+int rlt_oracle_philox4x32_10(const uint32_t* counter, const uint32_t* key, uint32_t* out);   /* the block function on explicit words */
+int rlt_oracle_rand_bits_u32(uint32_t* dst, size_t count, uint64_t seed, uint64_t stream);
+int rlt_oracle_rand_f32(float* dst, size_t count, float low, float high, uint64_t seed, uint64_t stream);
+int rlt_oracle_randn_f32(float* dst, size_t count, uint64_t seed, uint64_t stream);
+int rlt_oracle_gather_draw(const rlt_replay_buffer* rb, int batch, uint64_t seed, uint64_t stream, uint32_t* env_indices, uint32_t* sample_offsets);
+int rlt_oracle_pendulum_initial_states(float* states, int n_envs, uint64_t seed, uint64_t stream);
 
 int rlt_oracle_sac_train_critic(const rlt_sac_agent* agent, int critic_index, const float* action_noise);
 int rlt_oracle_sac_update_critic_targets(const rlt_sac_agent* agent);

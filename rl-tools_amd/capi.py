@@ -123,7 +123,9 @@ class SacLoopInputs(C.Structure):
 
 class SacLoopOutputs(C.Structure):
     _fields_ = [("critic_loss", C.c_void_p), ("observations_actions_base", C.c_void_p), ("rewards", C.c_void_p), ("terminated", C.c_void_p),
-                ("target_action_value", C.c_void_p), ("phase_ticks", C.c_void_p)]
+                ("target_action_value", C.c_void_p), ("phase_ticks", C.c_void_p),
+                ("drawn_rollout_noise", C.c_void_p), ("drawn_initial_states", C.c_void_p), ("drawn_sample_offsets", C.c_void_p),
+                ("drawn_noise_critic", C.c_void_p), ("drawn_noise_actor", C.c_void_p)]
 
 
 class PpoParameters(C.Structure):
@@ -304,7 +306,7 @@ ROCM_ONLY = {
     "memcpy_h2d": ([P, P, P, S], I), "memcpy_d2h": ([P, P, P, S], I), "memcpy_d2d": ([P, P, P, S], I),
     "memcpy2d": ([P, P, S, P, S, S, S, I], I),
     "fill_f32": ([P, P, I, I, I, F], I), "fill_u8": ([P, P, S, C.c_uint8], I),
-    "randn_f32": ([P, P, S, U64, U64], I), "rand_f32": ([P, P, S, F, F, U64, U64], I),
+    "randn_f32": ([P, P, S, U64, U64], I), "rand_f32": ([P, P, S, F, F, U64, U64], I), "rand_bits_u32": ([P, P, S, U64, U64], I),
     "reduce_sum_f32": ([P, P, S, I, P], I),
     "mlp_workspace_bytes": ([LP, I, I], S),
     "ppo_workspace_bytes": ([C.POINTER(PpoAgent)], S),

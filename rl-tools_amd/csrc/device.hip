@@ -1,6 +1,7 @@
 // Device handle, memory and the small container operations of the C ABI
 // (reference: devices/cuda.h:130-174, containers/matrix/operations_cuda.h:16-218, containers/tensor/operations_cuda.h:15-624).
 #include "common.h"
+#include "rng.h"
 #include <cstdio>
 #include <cstring>
 
@@ -44,37 +45,32 @@ __global__ __launch_bounds__(256) void scale_kernel(float* __restrict__ x, size_
         x[i] = reciprocal ? (1.0f / x[i]) * s : x[i] * s;   // the reciprocal first, then the scale, as the reference's Scale operation rounds
 }
 
-// Philox4x32-10 (Salmon et al. 2011): a pure function of (key = seed, counter = offset + element/4)
-__device__ __forceinline__ void philox_round(uint32_t& c0, uint32_t& c1, uint32_t& c2, uint32_t& c3, uint32_t k0, uint32_t k1) {
-    const uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u;
-    uint32_t hi0 = __umulhi(M0, c0), lo0 = M0 * c0;
-    uint32_t hi1 = __umulhi(M1, c2), lo1 = M1 * c2;
-    uint32_t n0 = hi1 ^ c1 ^ k0, n1 = lo1, n2 = hi0 ^ c3 ^ k1, n3 = lo0;
-    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
-}
-__device__ __forceinline__ uint4 philox4x32(uint64_t seed, uint64_t counter) {
-    uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
-    uint32_t c0 = (uint32_t)counter, c1 = (uint32_t)(counter >> 32), c2 = 0x9E3779B9u, c3 = 0xBB67AE85u;
-#pragma unroll
-    for (int r = 0; r < 10; r++) { philox_round(c0, c1, c2, c3, k0, k1); k0 += 0x9E3779B9u; k1 += 0xBB67AE85u; }
-    return make_uint4(c0, c1, c2, c3);
-}
-__device__ __forceinline__ float u01(uint32_t x) { return ((x >> 8) + 0.5f) * (1.0f / 16777216.0f); }   // (0,1)
-__global__ __launch_bounds__(256) void rand_kernel(float* __restrict__ dst, size_t count, float low, float high, uint64_t seed, uint64_t offset, int normal) {
+// randn / rand: element i is word i % 4 of Philox group i / 4 of the call's stream (rng.h). Two calls with different `stream` values
+// (or different seeds) share no group, whatever their lengths.
+__global__ __launch_bounds__(256) void rand_kernel(float* __restrict__ dst, size_t count, float low, float high, uint64_t seed, uint64_t stream, int normal) {
     const size_t quads = (count + 3) / 4;
     for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (size_t)gridDim.x * blockDim.x) {
-        uint4 r = philox4x32(seed, offset + q);
+        const rlt_u32x4 r = rlt_philox(seed, stream, q);
         float v[4];
         if (normal) {   // Box-Muller, two normals per pair of uniforms
-            float r0 = sqrtf(-2.0f * logf(u01(r.x))), r1 = sqrtf(-2.0f * logf(u01(r.z)));
+            float r0 = sqrtf(-2.0f * logf(rlt_u01(r.x))), r1 = sqrtf(-2.0f * logf(rlt_u01(r.z)));
             float s0, c0, s1, c1;
-            sincosf(6.283185307179586f * u01(r.y), &s0, &c0);
-            sincosf(6.283185307179586f * u01(r.w), &s1, &c1);
+            sincosf(6.283185307179586f * rlt_u01(r.y), &s0, &c0);
+            sincosf(6.283185307179586f * rlt_u01(r.w), &s1, &c1);
             v[0] = r0 * c0; v[1] = r0 * s0; v[2] = r1 * c1; v[3] = r1 * s1;
         } else {
-            v[0] = low + (high - low) * u01(r.x); v[1] = low + (high - low) * u01(r.y);
-            v[2] = low + (high - low) * u01(r.z); v[3] = low + (high - low) * u01(r.w);
+            v[0] = low + (high - low) * rlt_u01(r.x); v[1] = low + (high - low) * rlt_u01(r.y);
+            v[2] = low + (high - low) * rlt_u01(r.z); v[3] = low + (high - low) * rlt_u01(r.w);
         }
+        for (int j = 0; j < 4; j++) if (q * 4 + j < count) dst[q * 4 + j] = v[j];
+    }
+}
+// the raw 32-bit words of a stream, for checking the generator against a host restatement
+__global__ __launch_bounds__(256) void rand_bits_kernel(uint32_t* __restrict__ dst, size_t count, uint64_t seed, uint64_t stream) {
+    const size_t quads = (count + 3) / 4;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (size_t)gridDim.x * blockDim.x) {
+        const rlt_u32x4 r = rlt_philox(seed, stream, q);
+        const uint32_t v[4] = {r.x, r.y, r.z, r.w};
         for (int j = 0; j < 4; j++) if (q * 4 + j < count) dst[q * 4 + j] = v[j];
     }
 }
@@ -253,18 +249,25 @@ int rlt_rocm_fill_u8(rlt_rocm_device* device, uint8_t* dst, size_t count, uint8_
     hipLaunchKernelGGL(fill_u8_kernel, dim3(grid_for(count)), dim3(256), 0, device->stream, dst, count, value);
     return rlt_launch_status(device);
 }
-int rlt_rocm_randn_f32(rlt_rocm_device* device, float* dst, size_t count, uint64_t seed, uint64_t offset) {
+int rlt_rocm_rand_bits_u32(rlt_rocm_device* device, uint32_t* dst, size_t count, uint64_t seed, uint64_t stream) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(dst);
     if (count == 0) return 0;
-    hipLaunchKernelGGL(rand_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, 0.0f, 1.0f, seed, offset, 1);
+    hipLaunchKernelGGL(rand_bits_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, seed, stream);
     return rlt_launch_status(device);
 }
-int rlt_rocm_rand_f32(rlt_rocm_device* device, float* dst, size_t count, float low, float high, uint64_t seed, uint64_t offset) {
+int rlt_rocm_randn_f32(rlt_rocm_device* device, float* dst, size_t count, uint64_t seed, uint64_t stream) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(dst);
     if (count == 0) return 0;
-    hipLaunchKernelGGL(rand_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, low, high, seed, offset, 0);
+    hipLaunchKernelGGL(rand_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, 0.0f, 1.0f, seed, stream, 1);
+    return rlt_launch_status(device);
+}
+int rlt_rocm_rand_f32(rlt_rocm_device* device, float* dst, size_t count, float low, float high, uint64_t seed, uint64_t stream) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(dst);
+    if (count == 0) return 0;
+    hipLaunchKernelGGL(rand_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, low, high, seed, stream, 0);
     return rlt_launch_status(device);
 }
 int rlt_rocm_scale_f32(rlt_rocm_device* device, float* x, size_t count, float s, int reciprocal) {

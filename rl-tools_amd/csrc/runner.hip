@@ -2,6 +2,7 @@
 // reference: rl/components/replay_buffer/operations_generic.h:54-78, rl/components/off_policy_runner/operations_generic.h:183-430
 //            (CUDA :14-230), operations_generic_per_env.h:8-108, rl/environments/pendulum/operations_generic.h:14-160.
 #include "common.h"
+#include "rng.h"
 #include <cstdlib>
 
 namespace {
@@ -171,14 +172,11 @@ __global__ __launch_bounds__(256) void gather_sequence_kernel(rlt_replay_buffer 
     }
 }
 
-__device__ __forceinline__ uint32_t mix32(uint64_t x) {   // splitmix64 finaliser
-    x += 0x9E3779B97F4A7C15ull; x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull; x = (x ^ (x >> 27)) * 0x94D049BB133111EBull; x ^= x >> 31;
-    return (uint32_t)(x >> 32);
-}
-__global__ __launch_bounds__(256) void gather_draw_kernel(rlt_replay_buffer rb, int batch, uint64_t seed, uint64_t offset, uint32_t* __restrict__ env_indices, uint32_t* __restrict__ sample_offsets) {
+__global__ __launch_bounds__(256) void gather_draw_kernel(rlt_replay_buffer rb, int batch, uint64_t seed, uint64_t stream, uint32_t* __restrict__ env_indices, uint32_t* __restrict__ sample_offsets) {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < batch; i += gridDim.x * blockDim.x) {
-        uint32_t r0 = mix32(seed ^ ((offset + (uint64_t)i) * 2u)), r1 = mix32(seed ^ ((offset + (uint64_t)i) * 2u + 1u));
-        uint32_t e = (uint32_t)(((uint64_t)r0 * (uint32_t)rb.n_envs) >> 32);
+        const rlt_u32x4 draw = rlt_philox(seed, stream, (uint64_t)i);   // sample i takes words 0 and 1 of group i of the call's stream
+        const uint32_t r1 = draw.y;
+        uint32_t e = rlt_uniform_below(draw.x, (uint32_t)rb.n_envs);
         uint32_t eligible = rb.full[e] ? (uint32_t)rb.capacity : rb.position[e];
         env_indices[i] = e;
         sample_offsets[i] = eligible ? (uint32_t)(((uint64_t)r1 * eligible) >> 32) : 0u;
@@ -186,7 +184,7 @@ __global__ __launch_bounds__(256) void gather_draw_kernel(rlt_replay_buffer rb, 
 }
 
 // prologue of the runner step (operations_generic_per_env.h:8-66): reset where truncated, flag the previous replay row, observe
-__global__ __launch_bounds__(256) void runner_prologue_kernel(rlt_pendulum_runner rn, rlt_replay_buffer rb, const float* __restrict__ initial_states, uint64_t seed, uint64_t offset,
+__global__ __launch_bounds__(256) void runner_prologue_kernel(rlt_pendulum_runner rn, rlt_replay_buffer rb, const float* __restrict__ initial_states, uint64_t seed, uint64_t stream,
                                                               float* __restrict__ observations) {
     const int R = 2 * rb.observation_dim + rb.action_dim + 3;
     for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) {
@@ -195,8 +193,8 @@ __global__ __launch_bounds__(256) void runner_prologue_kernel(rlt_pendulum_runne
             if (initial_states) { th = initial_states[2 * e]; thd = initial_states[2 * e + 1]; }
             else {
                 const float PI = 3.14159265358979323846f;
-                float u0 = ((mix32(seed ^ ((offset + (uint64_t)e) * 2u)) >> 8) + 0.5f) * (1.0f / 16777216.0f);
-                float u1 = ((mix32(seed ^ ((offset + (uint64_t)e) * 2u + 1u)) >> 8) + 0.5f) * (1.0f / 16777216.0f);
+                const rlt_u32x4 draw = rlt_philox(seed, stream, (uint64_t)e);   // environment e takes words 0 and 1 of group e of the call's stream
+                const float u0 = rlt_u01(draw.x), u1 = rlt_u01(draw.y);
                 th = -PI + 2.0f * PI * u0; thd = -1.0f + 2.0f * u1;
             }
             rn.states[2 * e] = th; rn.states[2 * e + 1] = thd;
@@ -263,7 +261,7 @@ struct FusedRunnerArgs {
     int act_hidden, act_out, out_dim, policy_kind;
     rlt_sas_parameters sas;
     const float* action_noise; const float* initial_states;
-    uint64_t seed, offset;
+    uint64_t seed, stream;
 };
 
 template <int ACT_H>      // hidden activation, a compile-time constant: it sits inside the unrolled matrix-instruction loops
@@ -302,8 +300,8 @@ __global__ __launch_bounds__(64 * FWAVES) void runner_fused_kernel(FusedRunnerAr
                 if (A.initial_states) { const float2 ini = reinterpret_cast<const float2*>(A.initial_states)[e]; th = ini.x; thd = ini.y; }
                 else {
                     const float PI = 3.14159265358979323846f;
-                    const float u0 = ((mix32(A.seed ^ ((A.offset + (uint64_t)e) * 2u)) >> 8) + 0.5f) * (1.0f / 16777216.0f);
-                    const float u1 = ((mix32(A.seed ^ ((A.offset + (uint64_t)e) * 2u + 1u)) >> 8) + 0.5f) * (1.0f / 16777216.0f);
+                    const rlt_u32x4 draw = rlt_philox(A.seed, A.stream, (uint64_t)e);
+                    const float u0 = rlt_u01(draw.x), u1 = rlt_u01(draw.y);
                     th = -PI + 2.0f * PI * u0; thd = -1.0f + 2.0f * u1;
                 }
                 ep_step = 0; ep_ret = 0.f;
@@ -678,10 +676,10 @@ int rlt_rocm_gather_sequence_batch(rlt_rocm_device* device, const rlt_replay_buf
     return rlt_launch_status(device);
 }
 
-int rlt_rocm_gather_draw(rlt_rocm_device* device, const rlt_replay_buffer* rb, int batch, uint64_t seed, uint64_t offset, uint32_t* env_indices, uint32_t* sample_offsets) {
+int rlt_rocm_gather_draw(rlt_rocm_device* device, const rlt_replay_buffer* rb, int batch, uint64_t seed, uint64_t stream, uint32_t* env_indices, uint32_t* sample_offsets) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(rb_ok(rb) && batch > 0 && env_indices && sample_offsets);
-    hipLaunchKernelGGL(gather_draw_kernel, dim3(grid1(batch)), dim3(256), 0, device->stream, *rb, batch, seed, offset, env_indices, sample_offsets);
+    hipLaunchKernelGGL(gather_draw_kernel, dim3(grid1(batch)), dim3(256), 0, device->stream, *rb, batch, seed, stream, env_indices, sample_offsets);
     return rlt_launch_status(device);
 }
 
@@ -695,7 +693,7 @@ int rlt_rocm_pendulum_step(rlt_rocm_device* device, const rlt_pendulum_parameter
 
 int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, int policy_kind,
                                   const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas, const float* actions_in, const float* action_noise,
-                                  const float* initial_states, uint64_t seed, uint64_t offset) {
+                                  const float* initial_states, uint64_t seed, uint64_t stream) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(rn && rn->states && rn->episode_step && rn->episode_return && rn->truncated && rn->n_envs > 0 && rb_ok(rb));
     RLT_REQUIRE(rn->n_envs == rb->n_envs && rb->observation_dim == 3 && rb->action_dim == 1 && policy_kind >= 0 && policy_kind <= 2);
@@ -709,7 +707,7 @@ int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_ru
         a.w1 = actor[0].weights; a.b1 = actor[0].biases; a.w2 = actor[1].weights; a.b2 = actor[1].biases; a.w3 = actor[2].weights; a.b3 = actor[2].biases;
         a.act_hidden = actor[0].activation; a.act_out = actor[2].activation; a.out_dim = actor[2].out_dim; a.policy_kind = policy_kind;
         if (sas) a.sas = *sas;
-        a.action_noise = action_noise; a.initial_states = initial_states; a.seed = seed; a.offset = offset;
+        a.action_noise = action_noise; a.initial_states = initial_states; a.seed = seed; a.stream = stream;
         const int tiles = rlt_div_up(N, FTILE);
         int blocks = rlt_div_up(tiles, FWAVES); if (blocks > device->compute_units) blocks = device->compute_units;
         switch (a.act_hidden) {
@@ -728,7 +726,7 @@ int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_ru
     void* scratch; int rc = rlt_scratch(device, head + mlp_ws, &scratch); if (rc) return rc;
     float* obs = (float*)scratch; float* actor_out = obs + (size_t)N * 3; float* actions = actor_out + (size_t)N * 2; float* lp = actions + N;
     void* ws = (char*)scratch + head;
-    hipLaunchKernelGGL(runner_prologue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *rb, initial_states, seed, offset, obs);
+    hipLaunchKernelGGL(runner_prologue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *rb, initial_states, seed, stream, obs);
     if ((rc = rlt_launch_status(device))) return rc;
     const float* act_ptr = actions;
     if (policy_kind == 0) act_ptr = actions_in;

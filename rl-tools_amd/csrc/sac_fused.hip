@@ -37,6 +37,7 @@
 // The target critics are not exchanged at all: every workgroup applies the polyak update to its own LDS copy, with the same
 // arithmetic on the same bits as the owner of the element applies to the arena in memory.
 #include "common.h"
+#include "rng.h"
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -110,6 +111,8 @@ struct FusedArgs {
     // batch views for inspection (optional): last gathered batch / targets
     float* out_oab; float* out_rewards; uint8_t* out_terminated; float* out_target;
     unsigned long long* phase_ticks;   // [16] optional: constant-rate clock ticks workgroup 0 spent in each phase, summed over the steps
+    // optional: the draws every step used (host-drawn or the kernel's own), so that a run can be replayed elsewhere
+    float* drawn_rollout; float* drawn_initial; uint32_t* drawn_offsets; float* drawn_noise_c; float* drawn_noise_a;
 };
 
 __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
@@ -175,16 +178,13 @@ __device__ __forceinline__ void await(const unsigned* ready, int kind, int G, un
     rlt_lds_barrier();
 }
 
-__device__ __forceinline__ uint32_t mix32(uint64_t x) {
-    x += 0x9E3779B97F4A7C15ull; x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull; x = (x ^ (x >> 27)) * 0x94D049BB133111EBull; x ^= x >> 31;
-    return (uint32_t)(x >> 32);
-}
-__device__ __forceinline__ float u01(uint32_t x) { return ((x >> 8) + 0.5f) * (1.0f / 16777216.0f); }
-// standard normal from a (seed, stream, index) triple: Box-Muller on two hashed uniforms
+// The kernel's own draws (taken when the caller passes no host-drawn array): Philox groups (rng.h) of these streams under the
+// launch's seed; the index is the global step (step_offset + step), times the batch size plus the sample where a draw is per sample.
+enum { STREAM_INITIAL_STATE = 1, STREAM_ROLLOUT_NOISE = 3, STREAM_GATHER = 4, STREAM_NOISE_CRITIC = 5, STREAM_NOISE_ACTOR = 6 };
+// standard normal from one group: Box-Muller on its first two words
 __device__ __forceinline__ float randn_at(uint64_t seed, uint64_t stream, uint64_t index) {
-    uint64_t key = seed ^ (stream * 0xD1B54A32D192ED03ull) ^ (index * 0x9E3779B97F4A7C15ull);
-    float u1 = u01(mix32(key)), u2 = u01(mix32(key ^ 0xA5A5A5A5A5A5A5A5ull));
-    return sqrtf(-2.0f * logf(u1)) * cosf(6.283185307179586f * u2);
+    const rlt_u32x4 r = rlt_philox(seed, stream, index);
+    return sqrtf(-2.0f * logf(rlt_u01(r.x))) * cosf(6.283185307179586f * rlt_u01(r.y));
 }
 __device__ __forceinline__ float clampf(float x, float lo, float hi) { return fminf(fmaxf(x, lo), hi); }
 
@@ -487,7 +487,11 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
     const uint32_t age_actor0 = *A.actor_age, age_c00 = *A.critic_age[0], age_c10 = *A.critic_age[1], age_alpha0 = *A.alpha_age;
     __syncthreads();
 
-    if (tid == 0) S->rollout_eps[0] = A.rollout_noise ? A.rollout_noise[0] : randn_at(A.seed, 3, A.step_offset);
+    if (tid == 0) {
+        const float eps0 = A.rollout_noise ? A.rollout_noise[0] : randn_at(A.seed, STREAM_ROLLOUT_NOISE, A.step_offset);
+        S->rollout_eps[0] = eps0;
+        if (g == 0 && A.drawn_rollout) A.drawn_rollout[0] = eps0;
+    }
     __syncthreads();
     unsigned long long t_prev = A.phase_ticks ? wall_clock64() : 0ull;
     const unsigned long long shader_clock_begin = A.phase_ticks ? clock64() : 0ull;
@@ -513,7 +517,8 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             const int s = tid >> 4, j = tid & 15, sample = g * ROWS + s;
             const unsigned eligible = rb_full ? cap : rb_pos;
             const unsigned off = A.sample_offsets ? A.sample_offsets[(size_t)step * B + sample]
-                                                  : (unsigned)(((uint64_t)mix32(A.seed ^ ((gstep * (uint64_t)B + sample) * 8 + 4)) * eligible) >> 32);
+                                                  : rlt_uniform_below(rlt_philox(A.seed, STREAM_GATHER, gstep * (uint64_t)B + sample).x, eligible);
+            if (j == 0 && A.drawn_offsets) A.drawn_offsets[(size_t)step * B + sample] = off;
             unsigned index = off;
             if (rb_full) { index = rb_pos + (unsigned)A.runner.episode_step_limit + off; index = index % cap; }
             if (index >= cap) index = 0;     // cannot happen for valid offsets; keeps the access in bounds
@@ -522,7 +527,9 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         } else if (tid < ROWS * 16 + 2 * ROWS) {
             const int s = tid & 15, sample = g * ROWS + s; const bool actor_phase = tid >= ROWS * 16 + ROWS;
             const float* src = actor_phase ? A.noise_actor : A.noise_critic;
-            noise_reg = src ? src[(size_t)step * B + sample] : randn_at(A.seed, actor_phase ? 6 : 5, gstep * (uint64_t)B + sample);
+            noise_reg = src ? src[(size_t)step * B + sample] : randn_at(A.seed, actor_phase ? STREAM_NOISE_ACTOR : STREAM_NOISE_CRITIC, gstep * (uint64_t)B + sample);
+            float* const drawn = actor_phase ? A.drawn_noise_a : A.drawn_noise_c;
+            if (drawn) drawn[(size_t)step * B + sample] = noise_reg;
         }
         // ================= S0: environment step (wavefront 0, identical in every workgroup) =================
         if (wave == 0) {
@@ -530,8 +537,10 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
                 if (A.initial_states) { th = A.initial_states[2 * step]; thd = A.initial_states[2 * step + 1]; }
                 else {
                     const float PI = 3.14159265358979323846f;
-                    th = -PI + 2.0f * PI * u01(mix32(A.seed ^ (gstep * 8 + 1))); thd = -1.0f + 2.0f * u01(mix32(A.seed ^ (gstep * 8 + 2)));
+                    const rlt_u32x4 draw = rlt_philox(A.seed, STREAM_INITIAL_STATE, gstep);
+                    th = -PI + 2.0f * PI * rlt_u01(draw.x); thd = -1.0f + 2.0f * rlt_u01(draw.y);
                 }
+                if (g == 0 && lane == 0 && A.drawn_initial) { A.drawn_initial[2 * step] = th; A.drawn_initial[2 * step + 1] = thd; }
                 ep_step = 0; ep_return = 0.f;
                 if (full_before || new_pos > 0) {
                     const unsigned prev = new_pos == 0 ? cap - 1 : new_pos - 1;
@@ -587,7 +596,11 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             if (lane == 0) {
                 S->alpha = expf(get_shared<PACKED>(A.log_alpha));      // rewritten by the last workgroup in the previous step's S4
             }
-            if (lane == 1 && step + 1 < A.n_steps) S->rollout_eps[(step + 1) & 1] = A.rollout_noise ? A.rollout_noise[step + 1] : randn_at(A.seed, 3, gstep + 1);
+            if (lane == 1 && step + 1 < A.n_steps) {
+                const float eps1 = A.rollout_noise ? A.rollout_noise[step + 1] : randn_at(A.seed, STREAM_ROLLOUT_NOISE, gstep + 1);
+                S->rollout_eps[(step + 1) & 1] = eps1;
+                if (g == 0 && A.drawn_rollout) A.drawn_rollout[step + 1] = eps1;
+            }
         } else if (wave == 1 && lane < 4) {
             // bias corrections 1/(1 - beta^age) of this step (adam/operations_generic.h:43-66)
             const rlt_adam_parameters& p = lane == 0 ? A.adam_actor : (lane == 3 ? A.adam_alpha : A.adam_critic);
@@ -923,7 +936,9 @@ extern "C" int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac
                   a.noise_critic = inputs->noise_critic; a.noise_actor = inputs->noise_actor; }
     a.seed = seed; a.step_offset = step_offset;
     if (outputs) { a.out_critic_loss = outputs->critic_loss; a.out_oab = outputs->observations_actions_base; a.out_rewards = outputs->rewards;
-                   a.out_terminated = outputs->terminated; a.out_target = outputs->target_action_value; a.phase_ticks = (unsigned long long*)outputs->phase_ticks; }
+                   a.out_terminated = outputs->terminated; a.out_target = outputs->target_action_value; a.phase_ticks = (unsigned long long*)outputs->phase_ticks;
+                   a.drawn_rollout = outputs->drawn_rollout_noise; a.drawn_initial = outputs->drawn_initial_states; a.drawn_offsets = outputs->drawn_sample_offsets;
+                   a.drawn_noise_c = outputs->drawn_noise_critic; a.drawn_noise_a = outputs->drawn_noise_actor; }
     const size_t lds_floats = ((sizeof(Shared) / 4 + 3) & ~(size_t)3) + (size_t)(NA::ltotal + 4 * NC::ltotal);
     const size_t lds_bytes = lds_floats * sizeof(float);
     a.lds_floats = (int)lds_floats;

@@ -32,8 +32,8 @@ capi = package().capi
 
 
 def build_oracle():
-    if not os.path.exists(ORACLE_LIB) or os.path.getmtime(ORACLE_LIB) < max(
-            os.path.getmtime(os.path.join(ORACLE_DIR, f)) for f in ("rlt_oracle.cpp", "rlt_oracle_sac_loop.cpp", "rlt_oracle.h")):
+    sources = [f for f in os.listdir(ORACLE_DIR) if f.endswith((".cpp", ".h"))]
+    if not os.path.exists(ORACLE_LIB) or os.path.getmtime(ORACLE_LIB) < max(os.path.getmtime(os.path.join(ORACLE_DIR, f)) for f in sources):
         subprocess.run(["make", "-C", ORACLE_DIR, ORACLE_LIB], check=True, capture_output=True)
     return ORACLE_LIB
 
@@ -58,6 +58,14 @@ def load_oracle():
         fn.argtypes = a
         fn.restype = I
     lib.rlt_oracle_set_f64_accumulate.argtypes = [I]
+    U64, F = C.c_uint64, C.c_float
+    lib.rlt_oracle_philox4x32_10.argtypes = [P, P, P]
+    lib.rlt_oracle_rand_bits_u32.argtypes = [P, S, U64, U64]
+    lib.rlt_oracle_rand_f32.argtypes = [P, S, F, F, U64, U64]
+    lib.rlt_oracle_randn_f32.argtypes = [P, S, U64, U64]
+    lib.rlt_oracle_gather_draw.argtypes = [C.POINTER(capi.ReplayBuffer), I, U64, U64, P, P]
+    lib.rlt_oracle_pendulum_initial_states.argtypes = [P, I, U64, U64]
+    lib.rlt_oracle_reduce_sum_f32.argtypes = [P, S, I, P]
     lib.rlt_oracle_use_cblas.argtypes = [C.c_char_p]
     lib.rlt_oracle_cblas_name.restype = C.c_char_p
     lib.rlt_oracle_activation.argtypes = [C.c_float, I]; lib.rlt_oracle_activation.restype = C.c_float

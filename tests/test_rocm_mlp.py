@@ -34,6 +34,18 @@ def build_pair(oracle, rocm, shape, seed, hidden_act="relu", out_act="identity")
 @pytest.mark.parametrize("shape", SHAPES)
 @pytest.mark.parametrize("acts", [("relu", "identity"), ("tanh", "tanh")])
 def test_mlp_forward_backward_matches_oracle(oracle, rocm, shape, acts):
+    check_forward_backward(oracle, rocm, shape, acts)
+
+
+# GELU (with the reference's constant, nn/activation_functions.h:33-36), FAST_TANH and SIGMOID as hidden and as output activation, on a
+# ragged shape (per-layer kernels), the 256-wide shapes below and above the single-pass threshold, and a 64-wide one
+@pytest.mark.parametrize("shape", [(77, 5, 33, 3), (300, 17, 256, 6), (4096, 17, 256, 6), (2048, 105, 64, 8)])
+@pytest.mark.parametrize("acts", [("gelu", "identity"), ("gelu", "gelu"), ("fast_tanh", "sigmoid"), ("sigmoid", "fast_tanh")])
+def test_every_activation_function(oracle, rocm, shape, acts):
+    check_forward_backward(oracle, rocm, shape, acts)
+
+
+def check_forward_backward(oracle, rocm, shape, acts):
     print("case", shape, acts, flush=True)
     nets, x, dy = build_pair(oracle, rocm, shape, seed=hash(shape) % 1000, hidden_act=acts[0], out_act=acts[1])
     B, I, H, O = shape
