@@ -32,6 +32,7 @@ extern "C" {
 #define RLT_E_UNSUPPORTED      (-2) /* shape outside what the kernels are built for      */
 #define RLT_E_NOT_INITIALISED  (-3)
 #define RLT_E_DEVICE_TIMEOUT   (-4) /* a persistent kernel gave up waiting for another workgroup (reported by check_status) */
+#define RLT_E_WORKSPACE_TOO_SMALL (-5) /* the call needs more scratch memory than the fixed array of RLT_STATIC_SCRATCH_BYTES holds */
 
 /* nn/activation_functions.h:11-18 -- same numbering as the reference enum */
 enum rlt_activation {
@@ -128,6 +129,18 @@ int rlt_rocm_dense_backward_input(rlt_rocm_device* device, const rlt_dense_layer
 /* backward(dense)         operations_cpu_blas.h:143-186: d_output <- d_pre, d_biases += sum_batch d_pre, d_weights += d_pre^T x */
 int rlt_rocm_dense_backward(rlt_rocm_device* device, const rlt_dense_layer* layer,
                             const float* x, int ldx, float* d_output, int ldd, int batch);
+/* backward(dense) WITHOUT ANY ALLOCATION. No counterpart in the reference. For callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. rlt_rocm_dense_backward splits the batch over
+ * workgroups and keeps their partial sums in a workspace the handle grows on demand; this variant keeps them in a fixed array of
+ * RLT_STATIC_SCRATCH_BYTES that is part of the library's device image (each GPU the library is initialised on holds one copy until
+ * the process ends) and calls neither hipMalloc nor hipFree nor any allocating routine. Same arguments, same launches and bit for
+ * bit the same results as rlt_rocm_dense_backward. It returns RLT_E_WORKSPACE_TOO_SMALL when
+ * splits * (out_dim * in_dim + out_dim) * 4 bytes exceed the array (splits = min(ceil(batch / 256), about two workgroups per compute
+ * unit divided by the number of output tiles); every 64-wide layer fits at any batch, a 256 x 256 layer up to batch 16,128).
+ * All calls on one GPU share the array, whatever handle or stream they use: calls that overlap on one GPU race; order them. */
+#define RLT_STATIC_SCRATCH_BYTES (16u << 20)
+int rlt_rocm_dense_backward_static(rlt_rocm_device* device, const rlt_dense_layer* layer,
+                                   const float* x, int ldx, float* d_output, int ldd, int batch);
 /* backward_full(dense)    operations_cpu_blas.h:224-228 = backward + d_input */
 int rlt_rocm_dense_backward_full(rlt_rocm_device* device, const rlt_dense_layer* layer,
                                  const float* x, int ldx, float* d_output, int ldd,

@@ -225,7 +225,8 @@ class OnPolicyDataset(C.Structure):
 I, F, P, S, U64 = C.c_int, C.c_float, C.c_void_p, C.c_size_t, C.c_uint64
 LP = C.POINTER(DenseLayer)
 # return codes of the C ABI (include/rlt_rocm.h)
-RLT_E_INVALID_ARGUMENT, RLT_E_UNSUPPORTED, RLT_E_NOT_INITIALISED, RLT_E_DEVICE_TIMEOUT = -1, -2, -3, -4
+RLT_E_INVALID_ARGUMENT, RLT_E_UNSUPPORTED, RLT_E_NOT_INITIALISED, RLT_E_DEVICE_TIMEOUT, RLT_E_WORKSPACE_TOO_SMALL = -1, -2, -3, -4, -5
+STATIC_SCRATCH_BYTES = 16 << 20
 
 # name -> argument types after the leading device handle (shared by the HIP library and, minus the handle, the CPU checker)
 PROTOTYPES = {
@@ -308,6 +309,7 @@ ROCM_ONLY = {
     "fill_f32": ([P, P, I, I, I, F], I), "fill_u8": ([P, P, S, C.c_uint8], I),
     "randn_f32": ([P, P, S, U64, U64], I), "rand_f32": ([P, P, S, F, F, U64, U64], I), "rand_bits_u32": ([P, P, S, U64, U64], I),
     "reduce_sum_f32": ([P, P, S, I, P], I),
+    "dense_backward_static": ([P, LP, P, I, P, I, I], I),
     "mlp_workspace_bytes": ([LP, I, I], S),
     "ppo_workspace_bytes": ([C.POINTER(PpoAgent)], S),
     "gru_workspace_bytes": ([C.POINTER(GruLayer), I, I], S),

@@ -2,6 +2,7 @@
 // (reference: devices/cuda.h:130-174, containers/matrix/operations_cuda.h:16-218, containers/tensor/operations_cuda.h:15-624).
 #include "common.h"
 #include "rng.h"
+#include "gemm.h"
 #include <cstdio>
 #include <cstring>
 
@@ -140,6 +141,10 @@ int rlt_rocm_init(int hip_device_index, rlt_rocm_device** out_device) {
         (void)hipStreamSynchronize(device->stream);
         device->xcd_stride = ok ? 8 : 0;
     }
+    {   // where this GPU keeps the library's fixed scratch array (looked up once per GPU)
+        const int rc = rlt_gemm_static_scratch_setup(device);
+        if (rc) { (void)hipFree(device->counters); (void)hipStreamDestroy(device->own_stream); delete device; return rc; }
+    }
     *out_device = device;
     return 0;
 }
@@ -180,6 +185,7 @@ const char* rlt_rocm_error_string(int code) {
     if (code == RLT_E_UNSUPPORTED) return "rlt_rocm: shape outside what the kernels support";
     if (code == RLT_E_DEVICE_TIMEOUT) return "rlt_rocm: a persistent kernel gave up waiting for another workgroup; its results are invalid";
     if (code == RLT_E_NOT_INITIALISED) return "rlt_rocm: device handle not initialised";
+    if (code == RLT_E_WORKSPACE_TOO_SMALL) return "rlt_rocm: the call needs more scratch memory than the library's fixed array (RLT_STATIC_SCRATCH_BYTES) holds; use the allocating entry point or a smaller batch";
     if (code > 0) return hipGetErrorString((hipError_t)code);
     return "rlt_rocm: unknown error";
 }

@@ -9,8 +9,11 @@ int rlt_gemm_forward(rlt_rocm_device* device, const float* x, int ldx, const flo
 // layer's pre-activations, or its outputs when dact_from_output is set
 int rlt_gemm_backward_input(rlt_rocm_device* device, const float* d_pre, int ldd, const float* W, float* d_in, int ldi,
                             const float* dact_pre, int dact_kind, int dact_from_output, int batch, int in_dim, int out_dim);
-// dW += d_pre^T x ; dbias += column sums of d_pre (dbias may be NULL)
+// dW += d_pre^T x ; dbias += column sums of d_pre (dbias may be NULL). The partial sums of a split batch go to the handle's grow-only
+// workspace, or, with static_scratch, to the library's fixed device array (RLT_E_WORKSPACE_TOO_SMALL beyond RLT_STATIC_SCRATCH_BYTES).
 int rlt_gemm_wgrad(rlt_rocm_device* device, const float* d_pre, int ldd, const float* x, int ldx, float* dW, float* dbias,
-                   int batch, int in_dim, int out_dim);
+                   int batch, int in_dim, int out_dim, bool static_scratch = false);
+// looks up, once per GPU, where that GPU keeps the fixed array (called by rlt_rocm_init with the handle's device)
+int rlt_gemm_static_scratch_setup(rlt_rocm_device* device);
 // dst <- act'(pre) * src (dst may alias src; then a no-op for the identity)
 int rlt_dpre(rlt_rocm_device* device, const float* src, int lds, float* dst, int ldd, const float* pre, int rows, int cols, int act, int from_output);

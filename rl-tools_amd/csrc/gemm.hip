@@ -13,6 +13,7 @@
 // a half-wavefront read 32 consecutive words (no bank conflicts) and the two halves read consecutive k.
 #include "common.h"
 #include "gemm.h"
+#include <mutex>
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
@@ -306,29 +307,70 @@ int rlt_gemm_backward_input(rlt_rocm_device* device, const float* d_pre, int ldd
     return launch<1>(device, p, 1);
 }
 
-int rlt_gemm_wgrad(rlt_rocm_device* device, const float* d_pre, int ldd, const float* x, int ldx, float* dW, float* dbias,
-                   int batch, int in_dim, int out_dim) {
-    GemmParams p = {};
-    p.A = d_pre; p.lda = ldd; p.B = x; p.ldb = ldx; p.M = out_dim; p.N = in_dim; p.K = batch;
-    p.vecA = aligned16(d_pre) && (ldd % 4 == 0); p.vecB = aligned16(x) && (ldx % 4 == 0);
-    p.dW = dW; p.dbias = dbias;
-    // split the batch so that the grid fills the chip: about 2 workgroups per compute unit, at least 256 rows per split
+// How the weight-gradient contraction splits the batch so that the grid fills the chip: about 2 workgroups per compute unit, at least
+// 256 rows per split. Each split writes one block of out_dim * in_dim + out_dim partial sums.
+static void wgrad_split(const rlt_rocm_device* device, int batch, int in_dim, int out_dim, int& splits, int& kps) {
     const TileShape shape = pick_tile(out_dim, in_dim);
     int bm = shape == TILE_128x32 ? 128 : (shape == TILE_32x128 ? 32 : (shape == TILE_64x64 ? 64 : 128));
     int bn = shape == TILE_128x32 ? 32 : (shape == TILE_32x128 ? 128 : (shape == TILE_64x64 ? 64 : 128));
     int tiles = rlt_div_up(out_dim, bm) * rlt_div_up(in_dim, bn);
-    int splits = (2 * device->compute_units + tiles - 1) / tiles;
+    splits = (2 * device->compute_units + tiles - 1) / tiles;
     int max_splits = rlt_div_up(batch, 256);
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
-    int kps = rlt_div_up(rlt_div_up(batch, splits), BK) * BK;
+    kps = rlt_div_up(rlt_div_up(batch, splits), BK) * BK;
     splits = rlt_div_up(batch, kps);
+}
+
+// ---- partial sums without an allocation ------------------------------------------------------------------------------------
+// Callers that must not allocate (code under HIP graph capture, tight serving loops) get their split-batch partial sums from this
+// array instead of the handle's grow-only workspace. It is part of the library's device image: every GPU the library runs on holds
+// its own copy, at its own address, from the first use of the library on that GPU to the end of the process. In host code the
+// array's NAME is only a handle for hipGetSymbolAddress; what kernels and copies receive is the address looked up below.
+static __device__ __align__(256) float scratch[RLT_STATIC_SCRATCH_BYTES / sizeof(float)];
+namespace {
+constexpr int MAX_HIP_DEVICES = 64;
+float* scratch_address[MAX_HIP_DEVICES];      // per HIP device: where that GPU keeps its copy of `scratch`
+std::mutex scratch_mutex;
+}
+int rlt_gemm_static_scratch_setup(rlt_rocm_device* device) {
+    const int index = device->hip_device;
+    if (index < 0 || index >= MAX_HIP_DEVICES) return RLT_E_UNSUPPORTED;
+    std::lock_guard<std::mutex> guard(scratch_mutex);
+    if (scratch_address[index]) return 0;
+    int current = -1;
+    RLT_HIP(hipGetDevice(&current));
+    if (current != index) RLT_HIP(hipSetDevice(index));
+    void* address = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+    if (current != index) (void)hipSetDevice(current);
+    if (e != hipSuccess || !address) { device->sticky_error = (int)(e != hipSuccess ? e : hipErrorInvalidSymbol); return device->sticky_error; }
+    scratch_address[index] = (float*)address;
+    return 0;
+}
+
+int rlt_gemm_wgrad(rlt_rocm_device* device, const float* d_pre, int ldd, const float* x, int ldx, float* dW, float* dbias,
+                   int batch, int in_dim, int out_dim, bool static_scratch) {
+    GemmParams p = {};
+    p.A = d_pre; p.lda = ldd; p.B = x; p.ldb = ldx; p.M = out_dim; p.N = in_dim; p.K = batch;
+    p.vecA = aligned16(d_pre) && (ldd % 4 == 0); p.vecB = aligned16(x) && (ldx % 4 == 0);
+    p.dW = dW; p.dbias = dbias;
+    int splits, kps;
+    wgrad_split(device, batch, in_dim, out_dim, splits, kps);
     p.k_per_split = kps; p.splits = splits;
     if (splits > 1) {
-        void* ws = nullptr;
-        int rc = rlt_scratch(device, (size_t)splits * ((size_t)out_dim * in_dim + out_dim) * sizeof(float), &ws);
-        if (rc) return rc;
-        p.ws = (float*)ws;
+        const size_t floats = (size_t)splits * ((size_t)out_dim * in_dim + out_dim);
+        if (static_scratch) {
+            if (floats * sizeof(float) > (size_t)RLT_STATIC_SCRATCH_BYTES) return RLT_E_WORKSPACE_TOO_SMALL;
+            const int index = device->hip_device;
+            if (index < 0 || index >= MAX_HIP_DEVICES || !scratch_address[index]) return RLT_E_NOT_INITIALISED;
+            p.ws = scratch_address[index];        // every partial the reduction reads is written by this call's contraction first: nothing to clear
+        } else {
+            void* ws = nullptr;
+            int rc = rlt_scratch(device, floats * sizeof(float), &ws);
+            if (rc) return rc;
+            p.ws = (float*)ws;
+        }
     }
     int rc = launch<2>(device, p, splits);
     if (rc) return rc;
@@ -347,4 +389,20 @@ int rlt_dpre(rlt_rocm_device* device, const float* src, int lds, float* dst, int
     int blocks = (int)((total + 255) / 256); if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(dpre_kernel, dim3(blocks), dim3(256), 0, device->stream, src, lds, dst, ldd, pre, rows, cols, act, from_output);
     return rlt_launch_status(device);
+}
+
+// backward(dense) for callers that cannot allocate: the same launches as rlt_rocm_dense_backward (act'(pre) * d_output in place, then the
+// split-batch contraction and its fixed-order reduction), with the partial sums in the library's fixed device array.
+extern "C" int rlt_rocm_dense_backward_static(rlt_rocm_device* device, const rlt_dense_layer* L, const float* x, int ldx, float* d_output, int ldd, int batch) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(L && L->weights && L->biases && L->in_dim > 0 && L->out_dim > 0 && L->activation >= RLT_ACT_IDENTITY && L->activation <= RLT_ACT_SIGMOID);
+    RLT_REQUIRE(L->pre_activations && L->d_weights && L->d_biases && x && d_output && batch > 0 && ldd >= L->out_dim && ldx >= L->in_dim);
+    {   // refuse before anything is launched
+        int splits, kps;
+        wgrad_split(device, batch, L->in_dim, L->out_dim, splits, kps);
+        if (splits > 1 && (size_t)splits * ((size_t)L->out_dim * L->in_dim + L->out_dim) * sizeof(float) > (size_t)RLT_STATIC_SCRATCH_BYTES) return RLT_E_WORKSPACE_TOO_SMALL;
+    }
+    int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, L->pre_activations, batch, L->out_dim, L->activation, 0);
+    if (rc) return rc;
+    return rlt_gemm_wgrad(device, d_output, ldd, x, ldx, L->d_weights, L->d_biases, batch, L->in_dim, L->out_dim, true);
 }
