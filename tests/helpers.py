@@ -441,15 +441,29 @@ class RunnerOnBackend:
         self.rb = ReplayOnBackend(backend, 1, capacity)
         self.states = backend.zeros((1, 2)); self.ep_step = backend.zeros((1,), np.uint32); self.ep_ret = backend.zeros((1,))
         self.trunc = backend.array(np.ones(1, np.uint8))
+        self.capacity = capacity
         if loop is not None:
-            rn = oracle.lib.rlt_oracle_sac_loop_runner(loop).contents
-            rb = oracle.lib.rlt_oracle_sac_loop_replay(loop).contents
-            self.states.upload(np_from(rn.states, (1, 2))); self.ep_step.upload(np_from(rn.episode_step, (1,), np.uint32))
-            self.ep_ret.upload(np_from(rn.episode_return, (1,))); self.trunc.upload(np_from(rn.truncated, (1,), np.uint8))
-            self.rb.data.upload(np_from(rb.data, (capacity, 10))); self.rb.episode_start.upload(np_from(rb.episode_start, (capacity,), np.uint32))
-            self.rb.position.upload(np_from(rb.position, (1,), np.uint32)); self.rb.current_episode_start.upload(np_from(rb.current_episode_start, (1,), np.uint32))
-            self.rb.full.upload(np_from(rb.full, (1,), np.uint8))
+            self.load_from(oracle, loop)
         self.c = capi.PendulumRunner(self.states.ptr, self.ep_step.ptr, self.ep_ret.ptr, self.trunc.ptr, 1, 200, capi.pendulum_parameters())
+
+    def load_from(self, oracle, loop):
+        """Copies the runner state and the whole replay ring of the checker's loop."""
+        capacity = self.capacity
+        rn = oracle.lib.rlt_oracle_sac_loop_runner(loop).contents
+        rb = oracle.lib.rlt_oracle_sac_loop_replay(loop).contents
+        self.states.upload(np_from(rn.states, (1, 2))); self.ep_step.upload(np_from(rn.episode_step, (1,), np.uint32))
+        self.ep_ret.upload(np_from(rn.episode_return, (1,))); self.trunc.upload(np_from(rn.truncated, (1,), np.uint8))
+        self.rb.data.upload(np_from(rb.data, (capacity, 10))); self.rb.episode_start.upload(np_from(rb.episode_start, (capacity,), np.uint32))
+        self.rb.position.upload(np_from(rb.position, (1,), np.uint32)); self.rb.current_episode_start.upload(np_from(rb.current_episode_start, (1,), np.uint32))
+        self.rb.full.upload(np_from(rb.full, (1,), np.uint8))
+
+
+def oracle_stream_words(oracle, seed, stream, first_group, n_groups):
+    """Groups first_group ... first_group + n_groups - 1 of the Philox sequence (seed, stream) from the CPU restatement, as [n_groups x 4] words."""
+    total = 4 * (first_group + n_groups)
+    out = np.zeros(total, np.uint32)
+    assert oracle.lib.rlt_oracle_rand_bits_u32(out.ctypes.data, total, seed, stream) == 0
+    return out.reshape(-1, 4)[first_group:]
 
 
 def collect_loop_draws(oracle, loop, batch, n_steps):
