@@ -1,0 +1,209 @@
+// The off-policy runner on devices::ROCM: malloc / free / init / truncate_all / step / gather_batch (the counterpart of
+// rl/components/off_policy_runner/operations_cuda.h:9-237).
+//
+// The CUDA backend compiles the environment's generic step into its prologue / epilogue kernels. This backend ships precompiled
+// kernels, so the runner steps the environments the C ABI has a kernel for: the Pendulum (rl/environments/pendulum). One step of all
+// environments -- reset where truncated, observe, the actor (an MLP with or without a sample_and_squash head, or given actions),
+// dynamics, reward, truncation and the replay add -- is ONE launch (rlt_rocm_pendulum_runner_step); the CUDA backend launches a
+// prologue kernel, the actor's layers and an epilogue kernel.
+//
+// Memory. runner.replay_buffers is, on every device, the block that holds the replay rings. Host code never looks inside it on a GPU
+// backend; here it holds the backend's own layout: the rings of all environments in one allocation (ring e = rows [e * capacity,
+// (e + 1) * capacity) of `data`, a row being [observation | action | reward | next observation | terminated | truncated] as in
+// rl/components/replay_buffer/replay_buffer.h:32-62), then episode_start, then the device-resident cursors position,
+// current_episode_start and full of every ring. runner.envs / env_parameters / episode_stats stay in host memory (host code reads them).
+#pragma once
+#include <rl_tools/devices/rocm.h>
+#include <rl_tools/rl/components/off_policy_runner/off_policy_runner.h>
+#include <rl_tools/rl/components/off_policy_runner/operations_generic.h>
+#include <rl_tools/rl/environments/pendulum/pendulum.h>
+#include <rl_tools/nn_models/mlp/network.h>
+#include <rl_tools/nn_models/sequential/model.h>
+#include <rl_tools/nn_models/random_uniform/model.h>
+#include <rl_tools/nn/layers/dense/operations_rocm.h>
+#include <rl_tools/nn/layers/sample_and_squash/operations_rocm.h>
+RL_TOOLS_NAMESPACE_WRAPPER_START
+namespace rl_tools{
+    namespace rl::components::off_policy_runner::rocm{
+        template <typename SPEC>
+        struct Layout{
+            using T = typename SPEC::TYPE_POLICY::DEFAULT;
+            using ENVIRONMENT = typename SPEC::ENVIRONMENT;
+            static_assert(utils::typing::is_same_v<T, float>, "the ROCM backend computes in fp32");
+            static_assert(!SPEC::PARAMETERS::ASYMMETRIC_OBSERVATIONS, "asymmetric observations are not available on devices::ROCM");
+            static constexpr size_t N = SPEC::PARAMETERS::N_ENVIRONMENTS, CAPACITY = SPEC::PARAMETERS::REPLAY_BUFFER_CAPACITY;
+            static constexpr size_t OBS = ENVIRONMENT::Observation::DIM, ACT = ENVIRONMENT::ACTION_DIM, ROW = 2 * OBS + ACT + 3;
+            static constexpr size_t align(size_t x){ return (x + 255) / 256 * 256; }
+            static constexpr size_t DATA = 0;
+            static constexpr size_t EPISODE_START = align(DATA + N * CAPACITY * ROW * sizeof(float));
+            static constexpr size_t POSITION = align(EPISODE_START + N * CAPACITY * sizeof(uint32_t));
+            static constexpr size_t CURRENT_EPISODE_START = POSITION + align(N * sizeof(uint32_t));
+            static constexpr size_t FULL = CURRENT_EPISODE_START + align(N * sizeof(uint32_t));
+            static constexpr size_t BYTES = FULL + align(N);
+        };
+        template <typename SPEC>
+        rlt_replay_buffer replay(rl::components::OffPolicyRunner<SPEC>& runner){
+            using L = Layout<SPEC>;
+            char* base = (char*)runner.replay_buffers._data;
+            rlt_replay_buffer rb = {};
+            rb.data = (float*)(base + L::DATA); rb.episode_start = (uint32_t*)(base + L::EPISODE_START); rb.position = (uint32_t*)(base + L::POSITION);
+            rb.current_episode_start = (uint32_t*)(base + L::CURRENT_EPISODE_START); rb.full = (uint8_t*)(base + L::FULL);
+            rb.n_envs = (int32_t)L::N; rb.capacity = (int32_t)L::CAPACITY; rb.observation_dim = (int32_t)L::OBS; rb.action_dim = (int32_t)L::ACT;
+            return rb;
+        }
+        template <typename SPEC>
+        rlt_pendulum_runner pendulum(rl::components::OffPolicyRunner<SPEC>& runner){
+            using ENVIRONMENT = typename SPEC::ENVIRONMENT;
+            using T = typename SPEC::TYPE_POLICY::DEFAULT;
+            using TI = typename SPEC::TI;
+            static_assert(utils::typing::is_same_v<ENVIRONMENT, rl::environments::Pendulum<typename ENVIRONMENT::SPEC>>, "the ROCM backend's runner steps the Pendulum; other environments have step kernels (rlt_rocm_acrobot_step, rlt_rocm_car_step) but no runner");
+            static_assert(sizeof(typename ENVIRONMENT::State) == 2 * sizeof(T) && sizeof(TI) == 4 && sizeof(bool) == 1);
+            using P = typename ENVIRONMENT::SPEC::PARAMETERS;
+            rlt_pendulum_runner r = {};
+            r.states = (float*)runner.states._data; r.episode_step = (uint32_t*)runner.episode_step._data; r.episode_return = (float*)runner.episode_return._data;
+            r.truncated = (uint8_t*)runner.truncated._data;
+            r.n_envs = SPEC::PARAMETERS::N_ENVIRONMENTS; r.episode_step_limit = SPEC::PARAMETERS::EPISODE_STEP_LIMIT;
+            r.env = rlt_pendulum_parameters{(float)P::g, (float)P::max_speed, (float)P::max_torque, (float)P::dt, (float)P::m, (float)P::l};
+            return r;
+        }
+        // the dense layers of a policy in evaluation order, and whether it ends in a sample_and_squash head
+        struct PolicyDescription{
+            static constexpr int MAX_LAYERS = 16;
+            rlt_dense_layer layers[MAX_LAYERS];
+            int n_layers = 0;
+            bool has_head = false;
+            rlt_sas_parameters head = {};
+        };
+        template <typename LAYER_SPEC>
+        void describe(const nn::layers::dense::LayerForward<LAYER_SPEC>& layer, PolicyDescription& d){
+            d.layers[d.n_layers++] = nn::layers::dense::rocm::describe_forward(layer);
+        }
+        template <typename LAYER_SPEC>
+        void describe(const nn::layers::sample_and_squash::LayerForward<LAYER_SPEC>& layer, PolicyDescription& d){
+            d.has_head = true;
+            d.head = nn::layers::sample_and_squash::rocm::parameters<LAYER_SPEC>();
+        }
+        template <typename MODEL_SPEC>
+        void describe(const nn_models::mlp::NeuralNetworkForward<MODEL_SPEC>& model, PolicyDescription& d){
+            static_assert(MODEL_SPEC::NUM_HIDDEN_LAYERS + 2 <= PolicyDescription::MAX_LAYERS);
+            describe(model.input_layer, d);
+            for(typename MODEL_SPEC::TI i = 0; i < MODEL_SPEC::NUM_HIDDEN_LAYERS; i++){ describe(model.hidden_layers[i], d); }
+            describe(model.output_layer, d);
+        }
+        template <typename MODULE_SPEC>
+        void describe(const nn_models::sequential::ModuleForward<MODULE_SPEC>& module, PolicyDescription& d){
+            describe(module.content, d);
+            if constexpr(!utils::typing::is_same_v<typename MODULE_SPEC::NEXT_MODULE, nn_models::sequential::OutputModule>){
+                describe(module.next_module, d);
+            }
+        }
+    }
+    // malloc / free           off_policy_runner/operations_cuda.h:100-133
+    template<typename DEV_SPEC, typename SPEC>
+    void malloc(devices::ROCM<DEV_SPEC>& device, rl::components::OffPolicyRunner<SPEC>& runner){
+        using RUNNER = rl::components::OffPolicyRunner<SPEC>;
+        using L = rl::components::off_policy_runner::rocm::Layout<SPEC>;
+        static_assert(SPEC::DYNAMIC_ALLOCATION, "runners on devices::ROCM are dynamically allocated");
+        malloc(device, runner.buffers);
+        malloc(device, runner.states);
+        malloc(device, runner.episode_return);
+        malloc(device, runner.episode_step);
+        malloc(device, runner.truncated);
+        void* block = nullptr;
+        devices::rocm::check(rlt_rocm_malloc(device.handle, &block, L::BYTES), "malloc(runner)");
+        runner.replay_buffers._data = (typename RUNNER::REPLAY_BUFFER_TYPE*)block;
+        count_malloc(device, L::BYTES);
+        runner.envs._data = new typename SPEC::ENVIRONMENT[SPEC::PARAMETERS::N_ENVIRONMENTS];
+        runner.env_parameters._data = new typename SPEC::ENVIRONMENT::Parameters[SPEC::PARAMETERS::N_ENVIRONMENTS];
+        runner.episode_stats._data = nullptr;       // episode statistics are not collected on the device
+        malloc(device, runner.policy_states);
+    }
+    template<typename DEV_SPEC, typename SPEC>
+    void free(devices::ROCM<DEV_SPEC>& device, rl::components::OffPolicyRunner<SPEC>& runner){
+        free(device, runner.buffers);
+        free(device, runner.states);
+        free(device, runner.episode_return);
+        free(device, runner.episode_step);
+        free(device, runner.truncated);
+        devices::rocm::check(rlt_rocm_free(device.handle, (void*)runner.replay_buffers._data), "free(runner)");
+        runner.replay_buffers._data = nullptr;
+        delete[] runner.envs._data; runner.envs._data = nullptr;
+        delete[] runner.env_parameters._data; runner.env_parameters._data = nullptr;
+        free(device, runner.policy_states);
+    }
+    // init                    off_policy_runner/operations_cuda.h:134-151: every environment starts a new episode at the next step, empty rings
+    template<typename DEV_SPEC, typename SPEC>
+    void init(devices::ROCM<DEV_SPEC>& device, rl::components::OffPolicyRunner<SPEC>& runner){
+        using L = rl::components::off_policy_runner::rocm::Layout<SPEC>;
+        truncate_all(device, runner);
+        set_all(device, runner.episode_step, 0);
+        set_all(device, runner.episode_return, 0);
+        devices::rocm::check(rlt_rocm_fill_u8(device.handle, (uint8_t*)runner.replay_buffers._data + L::POSITION, L::BYTES - L::POSITION, 0), "init(runner)");
+        for(typename SPEC::TI env_i = 0; env_i < SPEC::PARAMETERS::N_ENVIRONMENTS; env_i++){
+            auto& env = runner.envs._data[env_i];
+            init(device, env);
+            initial_parameters(device, env, runner.env_parameters._data[env_i]);
+        }
+        runner.previous_policy_set = false;
+        runner.previous_policy = 0;
+#ifdef RL_TOOLS_DEBUG_RL_COMPONENTS_OFF_POLICY_RUNNER_CHECK_INIT
+        runner.initialized = true;
+#endif
+    }
+    // step                    off_policy_runner/operations_cuda.h:164-185 (prologue + interlude + epilogue), one launch
+    template<auto POLICY_INDEX, typename DEV_SPEC, typename SPEC, typename POLICY, typename POLICY_BUFFERS, typename RNG>
+    void step(devices::ROCM<DEV_SPEC>& device, rl::components::OffPolicyRunner<SPEC>& runner, POLICY& policy, POLICY_BUFFERS& policy_eval_buffers, RNG& rng){
+        using TI = typename SPEC::TI;
+        constexpr TI N = SPEC::PARAMETERS::N_ENVIRONMENTS;
+        constexpr TI POLICY_INPUT_DIM = get_last(typename POLICY::INPUT_SHAPE{});
+        constexpr TI POLICY_OUTPUT_DIM = get_last(typename POLICY::OUTPUT_SHAPE{});
+        static_assert(POLICY_INPUT_DIM == SPEC::ENVIRONMENT::Observation::DIM, "The policy's input dimension must match the environment's observation dimension.");
+        static_assert(POLICY_OUTPUT_DIM == SPEC::ENVIRONMENT::ACTION_DIM, "The policy's output dimension must match the environment's action dimension.");
+        const bool policy_switch = runner.previous_policy_set && (POLICY_INDEX != runner.previous_policy);
+        if(policy_switch){
+            truncate_all(device, runner);
+        }
+        const rlt_pendulum_runner r = rl::components::off_policy_runner::rocm::pendulum(runner);
+        const rlt_replay_buffer rb = rl::components::off_policy_runner::rocm::replay(runner);
+        if constexpr(utils::typing::is_same_v<POLICY, nn_models::RandomUniform<typename POLICY::SPEC>>){
+            // the exploration policy of the warm-up phase: uniform actions (nn_models/random_uniform/operations_generic.h:28-44), drawn on the device
+            static_assert(POLICY::SPEC::RANGE == nn_models::random_uniform::Range::MINUS_ONE_TO_ONE);
+            auto actions = to_tensor(device, runner.buffers.actions);
+            rand(device, actions, rng, -1.0f, 1.0f);
+            devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 0, nullptr, 0, nullptr, runner.buffers.actions._data, nullptr, nullptr, rng.seed, random::next_stream(rng)), "step(runner, uniform policy)");
+        }
+        else{
+            rl::components::off_policy_runner::rocm::PolicyDescription d;
+            rl::components::off_policy_runner::rocm::describe(policy, d);
+            if(d.has_head){
+                auto& noise = get_last_buffer(policy_eval_buffers).noise;
+                static_assert(utils::typing::remove_reference_t<decltype(noise)>::ROWS == N);
+                randn(device, noise, rng);
+                devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 2, d.layers, d.n_layers, &d.head, nullptr, noise._data, nullptr, rng.seed, random::next_stream(rng)), "step(runner, stochastic actor)");
+            }
+            else{
+                devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 1, d.layers, d.n_layers, nullptr, nullptr, nullptr, nullptr, rng.seed, random::next_stream(rng)), "step(runner, deterministic actor)");
+            }
+        }
+        runner.previous_policy = POLICY_INDEX;
+        runner.previous_policy_set = true;
+    }
+    // gather_batch            off_policy_runner/operations_cuda.h:152-163: draws (environment, row) pairs on the device and copies the rows
+    template <typename DEV_SPEC, typename SPEC, typename BATCH_SPEC, typename RNG, bool DETERMINISTIC = false>
+    void gather_batch(devices::ROCM<DEV_SPEC>& device, rl::components::OffPolicyRunner<SPEC>& runner, rl::components::off_policy_runner::SequentialBatch<BATCH_SPEC>& batch, RNG& rng){
+        static_assert(utils::typing::is_same_v<SPEC, typename BATCH_SPEC::SPEC>);
+        static_assert(BATCH_SPEC::SEQUENCE_LENGTHH == 1, "sequence batches are gathered through rlt_rocm_gather_sequence_batch; this overload covers SEQUENCE_LENGTH = 1");
+        constexpr int BATCH_SIZE = BATCH_SPEC::BATCH_SIZE;
+        const rlt_replay_buffer rb = rl::components::off_policy_runner::rocm::replay(runner);
+        uint32_t* env_indices = nullptr; uint32_t* offsets = nullptr;
+        if constexpr(!DETERMINISTIC){
+            env_indices = (uint32_t*)devices::rocm::scratch(device, 2 * sizeof(uint32_t) * BATCH_SIZE);
+            offsets = env_indices + BATCH_SIZE;
+            devices::rocm::check(rlt_rocm_gather_draw(device.handle, &rb, BATCH_SIZE, rng.seed, random::next_stream(rng), env_indices, offsets), "gather_batch (draw)");
+        }
+        devices::rocm::check(rlt_rocm_gather_batch(device.handle, &rb, env_indices, offsets, DETERMINISTIC ? 1 : 0, SPEC::MAX_EPISODE_LENGTH, BATCH_SIZE,
+                                                   batch.observations_actions_base._data, batch.rewards._data, (uint8_t*)batch.terminated._data, (uint8_t*)batch.reset._data,
+                                                   (uint8_t*)batch.next_reset_base._data, (uint8_t*)batch.final_step_mask._data, (uint8_t*)batch.next_final_step_mask_base._data), "gather_batch");
+    }
+}
+RL_TOOLS_NAMESPACE_WRAPPER_END

@@ -80,6 +80,9 @@ int rlt_rocm_memcpy2d(rlt_rocm_device* device, void* dst, size_t dst_pitch, cons
 /* set_all                 containers/matrix/operations_cuda.h:62-74,201-207 */
 int rlt_rocm_fill_f32(rlt_rocm_device* device, float* dst, int rows, int cols, int ld, float value);
 int rlt_rocm_fill_u8(rlt_rocm_device* device, uint8_t* dst, size_t count, uint8_t value);
+/* set_all(t, value tensor) containers/tensor/operations_cuda.h:341-347: every element becomes the scalar `value` points to on the DEVICE
+ * (e.g. a loss weight computed by an earlier launch), no host round trip */
+int rlt_rocm_fill_from_f32(rlt_rocm_device* device, float* dst, int rows, int cols, int ld, const float* value);
 /* randn / rand            containers/tensor/operations_cuda.h:548-624
  * Counter-based (Philox4x32-10): element i of a call is word i % 4 of group i / 4 of the sequence that (seed, stream) selects --
  * key = seed, counter = (group index, stream). No state array exists. Calls with different `stream` values (or seeds) draw from

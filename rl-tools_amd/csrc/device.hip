@@ -38,6 +38,14 @@ __global__ __launch_bounds__(256) void fill_f32_kernel(float* __restrict__ dst, 
         dst[r * ld + c] = value;
     }
 }
+__global__ __launch_bounds__(256) void fill_from_f32_kernel(float* __restrict__ dst, int rows, int cols, int ld, const float* __restrict__ value) {
+    const size_t total = (size_t)rows * cols;
+    const float v = *value;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        size_t r = i / cols, c = i % cols;
+        dst[r * ld + c] = v;
+    }
+}
 __global__ __launch_bounds__(256) void fill_u8_kernel(uint8_t* __restrict__ dst, size_t count, uint8_t value) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) dst[i] = value;
 }
@@ -246,6 +254,12 @@ int rlt_rocm_fill_f32(rlt_rocm_device* device, float* dst, int rows, int cols, i
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(dst && rows > 0 && cols > 0 && ld >= cols);
     hipLaunchKernelGGL(fill_f32_kernel, dim3(grid_for((size_t)rows * cols)), dim3(256), 0, device->stream, dst, rows, cols, ld, value);
+    return rlt_launch_status(device);
+}
+int rlt_rocm_fill_from_f32(rlt_rocm_device* device, float* dst, int rows, int cols, int ld, const float* value) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(dst && value && rows > 0 && cols > 0 && ld >= cols);
+    hipLaunchKernelGGL(fill_from_f32_kernel, dim3(grid_for((size_t)rows * cols)), dim3(256), 0, device->stream, dst, rows, cols, ld, value);
     return rlt_launch_status(device);
 }
 int rlt_rocm_fill_u8(rlt_rocm_device* device, uint8_t* dst, size_t count, uint8_t value) {

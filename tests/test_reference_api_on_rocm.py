@@ -1,0 +1,67 @@
+"""The reference's own API on devices::ROCM (include/rl_tools/**/*_rocm.h + librlt_rocm.so).
+
+Without a GPU: where the reference's headers are mounted, the two programs of tests/integration compile against them (plain g++, no HIP
+compiler) and link against the library -- the SAC program is the reference's loop (rl::algorithms::sac::loop::core malloc / init / step)
+with nothing but the device type changed, the CUDA counterpart being src/rl/environments/pendulum/sac/cuda/sac.cu.
+On the GPU: the binaries built here run; the SAC loop has to learn the Pendulum to the reference's acceptance bar
+(tests/src/rl/algorithms/sac/cpu/test.cpp:9-43: mean evaluation return above -200)."""
+import os
+import re
+import subprocess
+
+import pytest
+
+import helpers
+
+HERE = os.path.join(helpers.ROOT, "tests", "integration")
+BUILD = os.path.join(HERE, "_build")
+REFERENCE = "/root/reference/include/rl_tools/version.h"
+
+
+@pytest.mark.skipif(not os.path.exists(REFERENCE), reason="the reference's headers are not mounted here")
+def test_programs_written_against_the_reference_api_compile_and_link():
+    helpers.package().load_library()
+    subprocess.run(["make", "-C", HERE, "syntax"], check=True, capture_output=True)
+    out = subprocess.run(["make", "-B", "-C", HERE, "all"], capture_output=True, text=True)
+    assert out.returncode == 0, out.stderr[-3000:]
+    for name in ("rocm_containers", "rocm_sac_pendulum"):
+        path = os.path.join(BUILD, name)
+        assert os.path.exists(path)
+        needed = subprocess.run(["readelf", "-d", path], capture_output=True, text=True).stdout
+        assert "librlt_rocm.so" in needed and "hip" not in needed.lower().replace("librlt_rocm", "")      # host code only: the HIP runtime comes in through the library
+
+
+def test_every_header_of_the_layer_cites_the_reference_and_names_no_cuda_runtime():
+    """Each *_rocm.h names the reference file it stands beside; none includes CUDA / HIP runtime headers (callers need no device compiler)."""
+    count = 0
+    for dirpath, _, files in os.walk(os.path.join(helpers.ROOT, "include", "rl_tools")):
+        for f in files:
+            text = open(os.path.join(dirpath, f)).read()
+            count += 1
+            assert re.search(r"(operations_cuda\.h|cuda\.h|cuda/group_\d\.h|operations_cpu\.h|cpu_mux\.h)", text), f
+            assert "hip_runtime" not in text and "<cuda" not in text and "__global__" not in text, f
+    assert count >= 15
+
+
+@pytest.mark.gpu
+def test_containers_program_runs():
+    path = os.path.join(BUILD, "rocm_containers")
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    assert subprocess.run([path], timeout=120).returncode == 0
+
+
+@pytest.mark.gpu
+def test_the_references_sac_loop_learns_the_pendulum_on_rocm():
+    path = os.path.join(BUILD, "rocm_sac_pendulum")
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    out = subprocess.run([path, "10000", "0"], capture_output=True, text=True, timeout=300)
+    print(out.stdout[-1500:], flush=True)
+    assert out.returncode == 0, out.stderr[-2000:]
+    returns = [float(m) for m in re.findall(r"step \d+ mean_return (-?[\d.]+)", out.stdout)]
+    final = float(re.search(r"final (-?[\d.]+)", out.stdout).group(1))
+    rate = float(re.search(r"loop_steps_per_second_including_evaluations ([\d.]+)", out.stdout).group(1))
+    assert returns[0] < -600                                  # the untrained actor
+    assert sorted(returns[1:])[int(len(returns[1:]) * 0.8)] > -200 and final > -250
+    assert rate > 300                                         # every operation runs on the device: the host-loop fallback manages 8 steps per second
