@@ -441,21 +441,37 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_opera
     else:                         # the persistent kernel: all `steps` loop steps in one launch
         ticks = rocm.zeros((16,), np.uint64)
         outputs = capi.SacLoopOutputs(None, None, None, None, None, ticks.ptr if phase_profile else None)
+        ev = HipEvents(lib.rlt_rocm_get_stream(h))
+        done = [0]
 
-        def run(n, offset):
-            rocm.check(lib.rlt_rocm_sac_pendulum_loop(h, C.byref(agent.c), C.byref(runner), C.byref(rb.c), n, seed, offset, None, C.byref(outputs)))
-        run(max(warmup, 1), 0)
+        def run(n):
+            rocm.check(lib.rlt_rocm_sac_pendulum_loop(h, C.byref(agent.c), C.byref(runner), C.byref(rb.c), n, seed, done[0], None, C.byref(outputs)))
+            done[0] += n
+        run(max(warmup, 1))
         rocm.sync()
-        t0 = time.perf_counter()
         ticks.upload(np.zeros(16, np.uint64))
-        run(steps, warmup)
-        rocm.sync()
-        dt = time.perf_counter() - t0
+        # HIP events on the library's stream around launches of `steps` loop steps each, repeated until at least 5 ms are timed (a single
+        # short launch would mostly measure the launch itself); everything the loop reads and writes is resident on the device
+        launches = 0
+        a = ev.record()
+        while True:
+            run(steps)
+            launches += 1
+            if launches * steps * 20e-6 >= 5e-3:       # about 20 us per loop step: enqueue enough work before the first look at the clock
+                b = ev.record()
+                dt = ev.elapsed_ms(a, b) * 1e-3
+                if dt >= 5e-3 or launches >= 4096:
+                    break
+        total_steps = launches * steps
+        long_run = None
+        if steps < 20000:         # the same measurement with one launch of 20,000 steps, for reference
+            a = ev.record(); run(20000); b = ev.record()
+            long_run = 20000 / (ev.elapsed_ms(a, b) * 1e-3)
         if phase_profile:
             names = ["env step", "critic phase: TD error + both backward passes", "announce critic gradients", "wait + critic Adam", "announce + wait for critic parameters", "critic weight refresh",
                      "actor phase", "announce + wait for actor gradients", "actor Adam", "announce + wait for actor parameters", "actor weight refresh"]
             names += ["critic phase: batch rows into LDS", "critic phase: actor on next obs | critic 1 forward", "critic phase: target critics", "critic phase: critic 0 forward", "unused"]
-            tk = ticks.numpy()[:16].astype(np.float64) / 100.0 / steps      # 100 MHz constant clock -> microseconds per step
+            tk = ticks.numpy()[:16].astype(np.float64) / 100.0 / (total_steps + (20000 if long_run else 0))      # 100 MHz constant clock -> microseconds per step
             shader_cycles = tk[15] * 100.0; tk = tk[:15]; names = names[:15]
             print("phase profile (us per loop step, workgroup 0):", {f"{i}:{n}": round(float(v), 2) for i, (n, v) in enumerate(zip(names, tk))}, "sum", round(float(tk.sum()), 2),
                   "shader clock MHz", round(shader_cycles / tk.sum(), 1), file=sys.stderr, flush=True)
@@ -467,7 +483,10 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_opera
     env = capi.pendulum_parameters()
     rocm.call("pendulum_evaluate", C.byref(env), 2, agent.actor.layers, agent.actor.n, ini.ptr, 100, 200, ret.ptr, length.ptr, summary.ptr)
     rocm.sync()
-    return {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3, "launches_per_step": (1.0 / steps) if not per_operation else None,
+    if per_operation:
+        total_steps, launches, long_run = steps, None, None
+    return {"steps_per_s": total_steps / dt, "ms_per_step": dt / total_steps * 1e3, "launches_per_step": (1.0 / steps) if not per_operation else None,
+            "timed_loop_steps": total_steps, "timed_launches": launches, "steps_per_s_one_launch_of_20000_steps": long_run,
             "evaluation_return_after_run": float(summary.numpy()[0])}
 
 
@@ -580,7 +599,7 @@ def main():
     ap.add_argument("--only", choices=["all", "mlp", "sac", "env", "ppo", "gru", "seq"], default="all")
     ap.add_argument("--sac-phase-profile", action="store_true", help="print the persistent kernel's per-phase time (stderr)")
     ap.add_argument("--pmc-probe", action="store_true", help="for counter runs under rocprofv3 --pmc: three 256 MiB device copies (a kernel of known traffic, to scale the counters by) "
-                    "and three MLP forward+backward calls, nothing timed")
+                    "three MLP forward+backward calls, then the environment-pipeline and PPO workloads (their figures discarded)")
     ap.add_argument("--sac-per-operation", action="store_true", help="time the one-launch-per-operation SAC path instead of the persistent kernel")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -593,6 +612,8 @@ def main():
     info = rocm.device.info()
     if args.pmc_probe:
         pmc_probe(helpers, rocm, args.mlp_batch)
+        bench_env(helpers, rocm)       # runner_fused_kernel, gather_kernel, acrobot_step_kernel
+        bench_ppo(helpers, rocm)       # gae_kernel, the minibatch update's kernels
         rocm.close()
         return
     mlp = bench_mlp(helpers, rocm, args.mlp_batch, args.mlp_iters, 3) if args.only in ("all", "mlp") else None
@@ -609,6 +630,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "SAC Pendulum loop step, batch 256, actor 3-64-64-2, critics 4-64-64-1, replay 10000; plus MLP 17-256-256-6 fwd+bwd at batch %d" % args.mlp_batch,
                    "device": info["name"], "compute_units": info["compute_units"]},
+        "timed": {"loop_steps": sac.get("timed_loop_steps"), "launches_of_steps_each": sac.get("timed_launches"), "clock": "HIP events on the library's stream"},
+        "steps_per_s_one_launch_of_20000_steps": sac.get("steps_per_s_one_launch_of_20000_steps"),
         "network_updates_per_s": 3 * sac["steps_per_s"], "mean_return_of_100_evaluation_episodes_after_the_run": sac.get("evaluation_return_after_run"), "sac_path": "per-operation launches" if args.sac_per_operation else "persistent kernel, one launch for all steps",
     }
     if mlp:

@@ -8,10 +8,68 @@
 #include "optim.h"
 
 namespace {
-// one lane per environment, reverse scan over the steps; at a fixed step adjacent lanes touch adjacent dataset rows
-__global__ __launch_bounds__(256) void gae_kernel(const float* __restrict__ rewards, const float* __restrict__ terminated, const float* __restrict__ truncated,
-                                                  const float* __restrict__ all_values, float* __restrict__ advantages, float* __restrict__ target_values,
-                                                  int ld, int n_envs, int steps, float gamma, float lambda, int ignore_termination) {
+// Generalized advantage estimation as a two-level reverse scan. The recurrence over the steps of one environment,
+//     A_t = c_t A_{t+1} + d_t,   c_t = lambda gamma (0 where step t is truncated),   d_t = r_t + gamma V_{t+1} [not terminated] - V_t (0 where truncated but not terminated),
+// is linear in A_{t+1}, so a run of steps composes into one pair (a, b) with A_first = a A_in + b. A thread takes GAE_CHUNK consecutive steps of one
+// environment: all its loads are independent of the recurrence and are in flight together (the dataset is step-major: row = step * n_envs + env, so at
+// a fixed step the lanes of neighbouring environments read neighbouring rows). It scans its chunk from zero, keeping per step the advantage so far and
+// the product of the coefficients up to the chunk's end; the chunks of an environment are then chained through LDS, and every step adds its product
+// times the advantage that enters its chunk. One round trip to memory instead of one per step.
+constexpr int GAE_THREADS = 256;
+template <int GAE_CHUNK>
+__global__ __launch_bounds__(GAE_THREADS) void gae_kernel(const float* __restrict__ rewards, const float* __restrict__ terminated, const float* __restrict__ truncated,
+                                                          const float* __restrict__ all_values, float* __restrict__ advantages, float* __restrict__ target_values,
+                                                          int ld, int n_envs, int steps, float gamma, float lambda, int ignore_termination, int n_chunks, int envs_per_block) {
+    __shared__ float chunk_b[GAE_THREADS], chunk_a[GAE_THREADS];      // per (chunk, environment): advantage at the chunk's first step for zero input, and its coefficient product
+    const int chunk = threadIdx.x / envs_per_block, env_local = threadIdx.x - chunk * envs_per_block;
+    const int env = blockIdx.x * envs_per_block + env_local;
+    const bool live = chunk < n_chunks && env < n_envs;
+    const int first = chunk * GAE_CHUNK;                             // steps [first, first + count) in forward numbering
+    const int count = live ? min(GAE_CHUNK, steps - first) : 0;
+    float value[GAE_CHUNK + 1], reward[GAE_CHUNK], term[GAE_CHUNK], trunc[GAE_CHUNK];
+#pragma unroll
+    for (int j = 0; j < GAE_CHUNK; j++) {
+        const bool in = j < count;
+        const size_t pos = ((size_t)(first + (in ? j : 0)) * n_envs + (live ? env : 0)) * ld;
+        value[j] = in ? all_values[pos] : 0.f; reward[j] = in ? rewards[pos] : 0.f; term[j] = in ? terminated[pos] : 0.f; trunc[j] = in ? truncated[pos] : 0.f;
+    }
+    // the value that follows the chunk's last step: the next chunk's first row, or the bootstrap row after the last step
+    float value_after = live ? all_values[((size_t)(first + count) * n_envs + env) * ld] : 0.f;
+    float adv[GAE_CHUNK], prod[GAE_CHUNK];
+    float previous_advantage = 0.f, previous_value = value_after, product = 1.f;
+#pragma unroll
+    for (int j = GAE_CHUNK - 1; j >= 0; j--) {
+        if (j < count) {
+            const bool tm = term[j] != 0.f, tr = trunc[j] != 0.f;
+            const float next_value = (tm && !ignore_termination) ? 0.f : previous_value;
+            float td_error = reward[j] + gamma * next_value - value[j];
+            float coefficient = lambda * gamma;
+            if (tr) { if (!tm) td_error = 0.f; previous_advantage = 0.f; coefficient = 0.f; }
+            const float advantage = lambda * gamma * previous_advantage + td_error;
+            product *= coefficient;
+            adv[j] = advantage; prod[j] = product;
+            previous_advantage = advantage; previous_value = value[j];
+        } else { adv[j] = 0.f; prod[j] = 0.f; }
+    }
+    chunk_b[threadIdx.x] = previous_advantage; chunk_a[threadIdx.x] = product;
+    __syncthreads();
+    // the advantage that enters this chunk: chain the later chunks of the same environment, last one first
+    float incoming = 0.f;
+    if (live) for (int k = n_chunks - 1; k > chunk; k--) incoming = chunk_b[k * envs_per_block + env_local] + chunk_a[k * envs_per_block + env_local] * incoming;
+#pragma unroll
+    for (int j = 0; j < GAE_CHUNK; j++) {
+        if (j < count) {
+            const size_t pos = ((size_t)(first + j) * n_envs + env) * ld;
+            const float advantage = adv[j] + prod[j] * incoming;
+            advantages[pos] = advantage;
+            target_values[pos] = advantage + value[j];
+        }
+    }
+}
+// one lane per environment, serial over the steps (any number of steps)
+__global__ __launch_bounds__(64) void gae_serial_kernel(const float* __restrict__ rewards, const float* __restrict__ terminated, const float* __restrict__ truncated,
+                                                       const float* __restrict__ all_values, float* __restrict__ advantages, float* __restrict__ target_values,
+                                                       int ld, int n_envs, int steps, float gamma, float lambda, int ignore_termination) {
     for (int env = blockIdx.x * blockDim.x + threadIdx.x; env < n_envs; env += gridDim.x * blockDim.x) {
         float previous_value = all_values[((size_t)steps * n_envs + env) * ld];
         float previous_advantage = 0.0f;
@@ -189,9 +247,26 @@ extern "C" int rlt_rocm_ppo_gae(rlt_rocm_device* device, const float* rewards, c
                                 float* advantages, float* target_values, int ld, int n_envs, int steps, float gamma, float lambda, int ignore_termination) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(rewards && terminated && truncated && all_values && advantages && target_values && ld >= 1 && n_envs > 0 && steps > 0);
-    int blocks = (n_envs + 63) / 64; if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(gae_kernel, dim3(blocks), dim3(64), 0, device->stream, rewards, terminated, truncated, all_values, advantages, target_values, ld, n_envs, steps,
-                       gamma, lambda, ignore_termination);
+    // short chunks put more threads (and more loads) in flight; 16 steps a thread reach 4,096 steps
+    const int chunk_steps = steps <= 8 * GAE_THREADS ? 8 : 16;
+    const int n_chunks = (steps + chunk_steps - 1) / chunk_steps;
+    const char* serial = std::getenv("RLT_GAE_SERIAL");
+    if (n_chunks <= GAE_THREADS && !(serial && serial[0] == '1')) {
+        int envs_per_block = GAE_THREADS / n_chunks;                  // threads of a block: n_chunks x envs_per_block, neighbouring lanes = neighbouring environments
+        if (envs_per_block > 64) envs_per_block = 64;
+        if (envs_per_block > n_envs) envs_per_block = n_envs;
+        const int blocks = (n_envs + envs_per_block - 1) / envs_per_block;
+        if (chunk_steps == 8)
+            hipLaunchKernelGGL(gae_kernel<8>, dim3(blocks), dim3(GAE_THREADS), 0, device->stream, rewards, terminated, truncated, all_values, advantages, target_values, ld, n_envs, steps,
+                               gamma, lambda, ignore_termination, n_chunks, envs_per_block);
+        else
+            hipLaunchKernelGGL(gae_kernel<16>, dim3(blocks), dim3(GAE_THREADS), 0, device->stream, rewards, terminated, truncated, all_values, advantages, target_values, ld, n_envs, steps,
+                               gamma, lambda, ignore_termination, n_chunks, envs_per_block);
+    } else {
+        int blocks = (n_envs + 63) / 64; if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(gae_serial_kernel, dim3(blocks), dim3(64), 0, device->stream, rewards, terminated, truncated, all_values, advantages, target_values, ld, n_envs, steps,
+                           gamma, lambda, ignore_termination);
+    }
     return rlt_launch_status(device);
 }
 

@@ -147,8 +147,11 @@ def test_pendulum_step_matches_oracle(oracle, rocm):
         assert rel_err(g, r) <= TOL
 
 
-@pytest.mark.parametrize("n_envs,steps,ld", [(64, 16, 1), (4096, 128, 9), (100, 7, 3)])
-def test_gae_matches_oracle(oracle, rocm, n_envs, steps, ld):
+# chunked scan: whole chunks (16, 128), ragged last chunk (7, 17, 33), more chunks than a wavefront (2000), one environment per workgroup (2000),
+# the serial kernel beyond 4,096 steps (5000), a single sample
+@pytest.mark.parametrize("n_envs,steps,ld,ignore_termination", [(64, 16, 1, 0), (4096, 128, 9, 0), (100, 7, 3, 0), (3, 2000, 2, 0), (2, 5000, 1, 0), (33, 17, 4, 1),
+                                                                  (1, 1, 1, 0), (700, 33, 2, 1), (129, 4096, 1, 0)])
+def test_gae_matches_oracle(oracle, rocm, n_envs, steps, ld, ignore_termination):
     rng = np.random.default_rng(n_envs)
     rows = (steps + 1) * n_envs
     data = rng.standard_normal((rows, 6 * ld)).astype(np.float32)
@@ -159,7 +162,7 @@ def test_gae_matches_oracle(oracle, rocm, n_envs, steps, ld):
         cols = [b.array(np.ascontiguousarray(np.repeat(v[:, None], ld, 1))) for v in
                 (data[:, 0], term.astype(np.float32), trunc.astype(np.float32), data[:, 1])]
         adv, tv = b.zeros((rows, ld)), b.zeros((rows, ld))
-        b.call("ppo_gae", cols[0].ptr, cols[1].ptr, cols[2].ptr, cols[3].ptr, adv.ptr, tv.ptr, ld, n_envs, steps, 0.99, 0.95, 0)
+        b.call("ppo_gae", cols[0].ptr, cols[1].ptr, cols[2].ptr, cols[3].ptr, adv.ptr, tv.ptr, ld, n_envs, steps, 0.99, 0.95, ignore_termination)
         b.sync()
         res.append((adv.numpy()[:steps * n_envs, 0], tv.numpy()[:steps * n_envs, 0]))
     for g, r in zip(res[1], res[0]):
