@@ -415,29 +415,20 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_opera
 
     rocm.check = rocm.device.check
 
-    def loop_step():
-        env_step(1)
-        c = counter[0]
-        rocm.check(lib.rlt_rocm_gather_draw(h, C.byref(rb.c), batch, seed, 8 * c + 2, env_idx.ptr, offs.ptr))
-        rocm.call("gather_batch", C.byref(rb.c), env_idx.ptr, offs.ptr, 0, 200, batch, agent.oab.ptr, agent.rewards.ptr, agent.terminated.ptr, None, None, None, None)
-        rocm.check(lib.rlt_rocm_randn_f32(h, noise_c.ptr, batch, seed, 8 * c + 3))
-        for k in range(2):
-            rocm.call("sac_train_critic", C.byref(agent.c), k, noise_c.ptr)
-        rocm.call("sac_update_critic_targets", C.byref(agent.c))
-        rocm.check(lib.rlt_rocm_randn_f32(h, noise_a.ptr, batch, seed, 8 * c + 4))
-        rocm.call("sac_train_actor", C.byref(agent.c), noise_a.ptr)
-
     for _ in range(batch):        # fill the replay buffer with the warm-up policy
         env_step(0)
-    if per_operation:             # one launch per reference operation (the API-compatible path)
-        for _ in range(warmup):
-            loop_step()
-        rocm.sync()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            loop_step()
-        rocm.sync()
-        dt = time.perf_counter() - t0
+    if per_operation:             # one launch per reference operation, driven by the library's host loop over its own entry points
+        scratch = capi.SacLoopScratch(rollout_noise.ptr, noise_c.ptr, noise_a.ptr, env_idx.ptr, offs.ptr)
+        rocm.call("sac_set_per_operation", 1)
+        try:
+            rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), warmup, seed, 1 << 20, C.byref(scratch))
+            rocm.sync()
+            t0 = time.perf_counter()
+            rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), steps, seed, (1 << 20) + warmup, C.byref(scratch))
+            rocm.sync()
+            dt = time.perf_counter() - t0
+        finally:
+            rocm.call("sac_set_per_operation", 0)
     else:                         # the persistent kernel: all `steps` loop steps in one launch
         ticks = rocm.zeros((16,), np.uint64)
         outputs = capi.SacLoopOutputs(None, None, None, None, None, ticks.ptr if phase_profile else None)
@@ -488,6 +479,60 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_opera
     return {"steps_per_s": total_steps / dt, "ms_per_step": dt / total_steps * 1e3, "launches_per_step": (1.0 / steps) if not per_operation else None,
             "timed_loop_steps": total_steps, "timed_launches": launches, "steps_per_s_one_launch_of_20000_steps": long_run,
             "evaluation_return_after_run": float(summary.numpy()[0])}
+
+
+def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=10000):
+    """The API path: the reference's loop step composed of the library's own entry points by its host loop (no Python between the calls),
+    with the fused three-launch updates; and the four update calls alone on synthetic batches for a wider agent (observation 27, action 8)."""
+    capi = helpers.capi
+    lib, h = rocm.device.lib, rocm.device.handle
+    rng = np.random.default_rng(1)
+    out = {}
+
+    def parameters(obs, act):
+        critics = [helpers.random_params(rng, [obs + act, 64, 64, 1]) for _ in range(2)]
+        return np.concatenate([helpers.random_params(rng, [obs, 64, 64, 2 * act])] + critics + critics + [np.array([np.log(0.5)], np.float32)])
+
+    agent = helpers.SacOnBackend(rocm, batch, 64, parameters(3, 1), masks=False)
+    rb = helpers.ReplayOnBackend(rocm, 1, capacity)
+    states, ep_step, ep_ret, trunc = rocm.zeros((1, 2)), rocm.zeros((1,), np.uint32), rocm.zeros((1,)), rocm.array(np.ones(1, np.uint8))
+    runner = capi.PendulumRunner(states.ptr, ep_step.ptr, ep_ret.ptr, trunc.ptr, 1, 200, capi.pendulum_parameters())
+    rollout_noise, warm_action = rocm.zeros((1, 1)), rocm.zeros((1, 1))
+    noise_c, noise_a = rocm.zeros((batch, 1)), rocm.zeros((batch, 1))
+    env_idx, offs = rocm.zeros((batch,), np.uint32), rocm.zeros((batch,), np.uint32)
+    seed = 99
+    for c in range(1, batch + 1):      # fill the replay buffer with the uniform warm-up policy
+        rocm.device.check(lib.rlt_rocm_rand_f32(h, warm_action.ptr, 1, -1.0, 1.0, seed, 8 * c))
+        rocm.device.check(lib.rlt_rocm_pendulum_runner_step(h, C.byref(runner), C.byref(rb.c), 0, agent.actor.layers, 3, C.byref(agent.c.sas), warm_action.ptr, None, None, seed, 8 * c + 1))
+    scratch = capi.SacLoopScratch(rollout_noise.ptr, noise_c.ptr, noise_a.ptr, env_idx.ptr, offs.ptr)
+    ev = HipEvents(lib.rlt_rocm_get_stream(h))
+    rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), warmup, seed, 1 << 20, C.byref(scratch))
+    rocm.sync()
+    t0 = time.perf_counter(); a = ev.record()
+    rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), steps, seed, (1 << 20) + warmup, C.byref(scratch))
+    b = ev.record()
+    device_s = ev.elapsed_ms(a, b) * 1e-3       # waits for the second event
+    wall_s = time.perf_counter() - t0
+    assert np.all(np.isfinite(agent.parameters())), "SAC parameters went non-finite"
+    out.update(steps_per_s=steps / wall_s, steps_per_s_by_device_clock=steps / device_s, steps=steps, launches_per_step=16)
+    # a wider agent: the update calls alone
+    obs, act = 27, 8
+    wide = helpers.SacOnBackend(rocm, batch, 64, parameters(obs, act), masks=False, obs=obs, act=act)
+    oab = rng.standard_normal((2, batch, obs + act)).astype(np.float32); oab[:, :, obs:] = np.tanh(oab[:, :, obs:])
+    wide.set_batch(oab, rng.standard_normal(batch).astype(np.float32), (rng.random(batch) < 0.05).astype(np.uint8))
+    noise = rocm.array(rng.standard_normal((batch, act)).astype(np.float32))
+
+    def updates(n):
+        for _ in range(n):
+            for k in range(2):
+                rocm.device.check(lib.rlt_rocm_sac_train_critic(h, C.byref(wide.c), k, noise.ptr))
+            rocm.device.check(lib.rlt_rocm_sac_update_critic_targets(h, C.byref(wide.c)))
+            rocm.device.check(lib.rlt_rocm_sac_train_actor(h, C.byref(wide.c), noise.ptr))
+    updates(20)
+    rocm.sync()
+    a = ev.record(); updates(300); b = ev.record()
+    out["wide_agent_obs27_act8_update_sets_per_s_by_device_clock"] = 300 / (ev.elapsed_ms(a, b) * 1e-3)
+    return out
 
 
 def cpu_baseline(batch=256, seconds=12.0):
@@ -596,7 +641,7 @@ def main():
     ap.add_argument("--mlp-batch", type=int, default=65536)
     ap.add_argument("--mlp-iters", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "mlp", "sac", "env", "ppo", "gru", "seq"], default="all")
+    ap.add_argument("--only", choices=["all", "mlp", "sac", "env", "ppo", "gru", "seq", "api"], default="all")
     ap.add_argument("--sac-phase-profile", action="store_true", help="print the persistent kernel's per-phase time (stderr)")
     ap.add_argument("--pmc-probe", action="store_true", help="for counter runs under rocprofv3 --pmc: three 256 MiB device copies (a kernel of known traffic, to scale the counters by) "
                     "three MLP forward+backward calls, then the environment-pipeline and PPO workloads (their figures discarded)")
@@ -618,11 +663,12 @@ def main():
         return
     mlp = bench_mlp(helpers, rocm, args.mlp_batch, args.mlp_iters, 3) if args.only in ("all", "mlp") else None
     sac = bench_sac(helpers, rocm, args.steps, args.warmup, per_operation=args.sac_per_operation, phase_profile=args.sac_phase_profile) if args.only in ("all", "sac") else {"steps_per_s": 0.0, "ms_per_step": 0.0}
+    api = bench_sac_api(helpers, rocm) if args.only in ("all", "sac", "api") else None
     env = bench_env(helpers, rocm) if args.only in ("all", "env") else None
     ppo = bench_ppo(helpers, rocm) if args.only in ("all", "ppo") else None
     gru = [bench_gru(helpers, rocm, b) for b in (64, 1024)] if args.only in ("all", "gru") else None
     seq = bench_sac_sequence(helpers, rocm) if args.only in ("all", "seq") else None
-    cpu = None if (args.no_cpu_baseline or args.only in ("mlp", "env", "ppo", "gru", "seq")) else cpu_baseline()
+    cpu = None if (args.no_cpu_baseline or args.only in ("mlp", "env", "ppo", "gru", "seq", "api")) else cpu_baseline()
     line = {
         "metric": "SAC updates/sec (critic+actor) at batch 256; fused MLP fwd+bwd TFLOP/s",
         "value": sac["steps_per_s"], "unit": "SAC loop steps/s (each = 2 critic + 1 actor update)",
@@ -634,6 +680,9 @@ def main():
         "steps_per_s_one_launch_of_20000_steps": sac.get("steps_per_s_one_launch_of_20000_steps"),
         "network_updates_per_s": 3 * sac["steps_per_s"], "mean_return_of_100_evaluation_episodes_after_the_run": sac.get("evaluation_return_after_run"), "sac_path": "per-operation launches" if args.sac_per_operation else "persistent kernel, one launch for all steps",
     }
+    if api:
+        line["sac_api_path_steps_per_s"] = api["steps_per_s"]
+        line["sac_api_path"] = api
     if mlp:
         line["mlp_fwd_bwd_tflops"] = mlp["tflops"]
         line["mlp"] = mlp

@@ -322,13 +322,22 @@ typedef struct rlt_sac_agent {
 } rlt_sac_agent;
 
 /* train_critic            rl/algorithms/sac/operations_generic.h:243-337 for critic `critic_index`;
- *   action_noise [batch x action_dim] is the externally drawn N(0,1) noise. */
+ *   action_noise [batch x action_dim] is the externally drawn N(0,1) noise.
+ *   Two implementations with the same results (to fp32 rounding). Where every network is in -> 64 -> 64 -> out with one hidden
+ *   activation (not GELU), obs + act <= 128, act <= 8 and all three masks are NULL, train_critic and train_actor each run as three
+ *   launches (all network passes of the update; sum of the workgroups' partial gradients; Adam) and update_critic_targets as one;
+ *   of the training buffers only next_log_probabilities and target_action_value (critic), actor_log_probabilities, actor_actions and
+ *   actor_pre_squashing (actor) are then written, and the gradients are overwritten without a prior zero_gradient. Every other
+ *   agent, or any agent after rlt_rocm_sac_set_per_operation(device, 1), takes one launch per reference operation and fills every
+ *   training buffer. */
 int rlt_rocm_sac_train_critic(rlt_rocm_device* device, const rlt_sac_agent* agent, int critic_index,
                               const float* action_noise);
 /* update_critic_targets   sac/operations_generic.h:488-527 */
 int rlt_rocm_sac_update_critic_targets(rlt_rocm_device* device, const rlt_sac_agent* agent);
 /* train_actor             sac/operations_generic.h:395-468 */
 int rlt_rocm_sac_train_actor(rlt_rocm_device* device, const rlt_sac_agent* agent, const float* action_noise);
+/* (no counterpart) enabled != 0: the three calls above always take the one-launch-per-operation path. */
+int rlt_rocm_sac_set_per_operation(rlt_rocm_device* device, int enabled);
 
 /* ------------------------------------------------- replay buffer / runner -- */
 
@@ -541,6 +550,25 @@ typedef struct rlt_sac_loop_outputs {  /* all optional */
 int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_pendulum_runner* runner,
                                const rlt_replay_buffer* rb, int n_steps, uint64_t seed, uint64_t step_offset,
                                const rlt_sac_loop_inputs* inputs, const rlt_sac_loop_outputs* outputs);
+
+/* Device buffers that rlt_rocm_sac_pendulum_loop_by_calls draws into. */
+typedef struct rlt_sac_loop_scratch {
+    float* rollout_noise;       /* [n_envs x action_dim] */
+    float* noise_critic;        /* [batch x action_dim]  */
+    float* noise_actor;         /* [batch x action_dim]  */
+    uint32_t* env_indices;      /* [batch] */
+    uint32_t* sample_offsets;   /* [batch] */
+} rlt_sac_loop_scratch;
+/* The same n_steps iterations of sac::loop::core::step (rl/algorithms/sac/loop/core/operations_generic.h:110-155 past the warm-up,
+ * SHARED_BATCH: runner step with the actor, one gather_batch and one critic noise draw for both train_critic calls,
+ * update_critic_targets, actor noise draw, train_actor on the same batch) as a host loop over this library's own entry points, for
+ * agents and runners of any size that rlt_rocm_sac_pendulum_loop does not cover: 16 launches per step where the fused updates fit
+ * (see rlt_rocm_sac_train_critic). Nothing synchronises with the host. Loop step g = step_offset + i draws from the Philox
+ * sequences (seed, 8 g + k): k = 1 rollout noise, 2 initial states of episodes that reset, 3 batch indices, 4 critic noise,
+ * 5 actor noise. */
+int rlt_rocm_sac_pendulum_loop_by_calls(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_pendulum_runner* runner,
+                                        const rlt_replay_buffer* rb, int n_steps, uint64_t seed, uint64_t step_offset,
+                                        const rlt_sac_loop_scratch* scratch);
 
 /* --------------------------------------------------------------------- PPO -- */
 

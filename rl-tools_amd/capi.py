@@ -128,6 +128,10 @@ class SacLoopOutputs(C.Structure):
                 ("drawn_noise_critic", C.c_void_p), ("drawn_noise_actor", C.c_void_p)]
 
 
+class SacLoopScratch(C.Structure):
+    _fields_ = [("rollout_noise", C.c_void_p), ("noise_critic", C.c_void_p), ("noise_actor", C.c_void_p), ("env_indices", C.c_void_p), ("sample_offsets", C.c_void_p)]
+
+
 class PpoParameters(C.Structure):
     _fields_ = [("epsilon_clip", C.c_float), ("action_entropy_coefficient", C.c_float), ("advantage_epsilon", C.c_float),
                 ("normalize_advantage", C.c_int32), ("learn_action_std", C.c_int32), ("reserved", C.c_int32 * 3)]
@@ -310,6 +314,7 @@ ROCM_ONLY = {
     "randn_f32": ([P, P, S, U64, U64], I), "rand_f32": ([P, P, S, F, F, U64, U64], I), "rand_bits_u32": ([P, P, S, U64, U64], I),
     "reduce_sum_f32": ([P, P, S, I, P], I),
     "dense_backward_static": ([P, LP, P, I, P, I, I], I),
+    "sac_set_per_operation": ([P, I], I),
     "mlp_workspace_bytes": ([LP, I, I], S),
     "ppo_workspace_bytes": ([C.POINTER(PpoAgent)], S),
     "gru_workspace_bytes": ([C.POINTER(GruLayer), I, I], S),
@@ -321,6 +326,7 @@ ROCM_ONLY = {
     "td3_sequence_workspace_bytes": ([C.POINTER(Td3SequenceAgent)], S),
     "on_policy_collect_workspace_bytes": ([C.POINTER(PendulumRunner), LP, I], S),
     "gather_draw": ([P, C.POINTER(ReplayBuffer), I, U64, U64, P, P], I),
+    "sac_pendulum_loop_by_calls": ([P, C.POINTER(SacAgent), C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, U64, U64, C.POINTER(SacLoopScratch)], I),
     "sac_pendulum_loop": ([P, C.POINTER(SacAgent), C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, U64, U64, C.POINTER(SacLoopInputs),
                            C.POINTER(SacLoopOutputs)], I),
     "pendulum_runner_step": ([P, C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, LP, I, C.POINTER(SasParameters), P, P, P, U64, U64], I),

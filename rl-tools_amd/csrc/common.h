@@ -19,6 +19,7 @@ struct rlt_rocm_device {
     int fault_armed;             // a kernel that can set it was launched since the last check
     int xcd_stride;              // workgroups b and b + xcd_stride run on the same XCD (0: not established; consecutive workgroups go round the XCDs)
     int sticky_error;
+    int sac_per_operation;       // rlt_rocm_sac_train_critic / _actor run one launch per reference operation even where the fused kernels fit
 };
 
 #define RLT_HIP(expr)                                                        \

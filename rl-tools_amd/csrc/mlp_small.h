@@ -30,3 +30,10 @@ int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* a
                                const float* stats, const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset,
                                const rlt_dense_layer* critic, int n_critic, const float* x_critic, float* values, int ld_values,
                                const float* target_values, float mse_scale, float* out_critic_loss, int ld, const uint32_t* rows, int batch);
+
+// For kernels that write blocks of partial sums in this file's layout (dW1 [64 x in], db1 [64], dW2 [64 x 64], db2 [64], dW3 [out x 64], db3 [out],
+// extra [16]): the floats per block, and the launch that adds `groups` blocks up in block order into the layers' gradients (overwrite != 0:
+// gradient = sum) and, if `extra` is given, extra[i] = sum_i * extra_scale + extra_offset for i < n_extra.
+int rlt_mlp3s_partial_count(int in_dim, int out_dim);
+int rlt_mlp3s_reduce(rlt_rocm_device* device, const rlt_dense_layer* layers, const float* partial, int groups, int overwrite, float* extra, int n_extra,
+                     float extra_scale, float extra_offset);

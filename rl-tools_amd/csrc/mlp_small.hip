@@ -506,6 +506,18 @@ SmallJob ppo_actor_job(const rlt_dense_layer* L, const float* x, int ldx, float*
 
 bool rlt_mlp3s_supported(const rlt_dense_layer* L, int n) { return shape_ok(L, n); }
 
+int rlt_mlp3s_partial_count(int in_dim, int out_dim) { return H * in_dim + H + H * H + H + out_dim * H + out_dim + N_EXTRA; }
+
+int rlt_mlp3s_reduce(rlt_rocm_device* device, const rlt_dense_layer* L, const float* partial, int groups, int overwrite, float* extra, int n_extra, float extra_scale,
+                     float extra_offset) {
+    for (int l = 0; l < 3; l++) RLT_REQUIRE(L[l].d_weights && L[l].d_biases);
+    const int in = L[0].in_dim, out = L[2].out_dim, count = rlt_mlp3s_partial_count(in, out);
+    SmallTargets T = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases, extra, in, out, n_extra, extra_scale, extra_offset, overwrite,
+                      partial, groups, count, ((extra ? count : count - N_EXTRA) + 63) / 64};
+    hipLaunchKernelGGL(mlp3s_reduce_kernel, dim3(T.blocks), dim3(256), 0, device->stream, T, T);
+    return rlt_launch_status(device);
+}
+
 int rlt_mlp3s_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n, const float* x, int ldx, float* y, int ldy, const float* d_output, int ldd,
                                const float* target, int ldt, float mse_scale, int batch) {
     if (!shape_ok(L, n)) return RLT_E_UNSUPPORTED;

@@ -4,6 +4,7 @@
 //            rl/algorithms/sac/operations_generic.h:133-527 (CUDA :12-128), nn/loss_functions/mse/operations_generic.h:9-97,
 //            random/operations_generic.h:72-105.
 #include "common.h"
+#include "sac_update.h"
 #include <algorithm>
 
 namespace {
@@ -247,10 +248,17 @@ static bool agent_ok(const rlt_sac_agent* A) {
            A->n_actor_layers >= 1 && A->n_critic_layers >= 1 && A->log_alpha.parameters;
 }
 
-// rl/algorithms/sac/operations_generic.h:243-337, one launch per reference operation (the op-by-op path)
+int rlt_rocm_sac_set_per_operation(rlt_rocm_device* device, int enabled) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    device->sac_per_operation = enabled != 0;
+    return 0;
+}
+
+// rl/algorithms/sac/operations_generic.h:243-337: the fused kernels where they fit, else one launch per reference operation
 int rlt_rocm_sac_train_critic(rlt_rocm_device* device, const rlt_sac_agent* A, int ci, const float* action_noise) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A) && (ci == 0 || ci == 1) && action_noise);
+    if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) return rlt_sac_update_critic(device, A, ci, action_noise);
     RLT_REQUIRE(A->next_state_action_value_input && A->next_q[0] && A->next_q[1] && A->next_log_probabilities && A->target_action_value && A->d_output_critic[ci]);
     const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
     const rlt_dense_layer* critic = A->critics[ci];
@@ -283,6 +291,17 @@ int rlt_rocm_sac_train_critic(rlt_rocm_device* device, const rlt_sac_agent* A, i
 int rlt_rocm_sac_update_critic_targets(rlt_rocm_device* device, const rlt_sac_agent* A) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A));
+    if (!device->sac_per_operation && 4 * A->n_critic_layers <= 64) {      // all tensors in one launch (per 16)
+        const float* sources[64]; float* targets[64]; uint32_t counts[64];
+        int n = 0;
+        for (int k = 0; k < 2; k++)
+            for (int l = 0; l < A->n_critic_layers; l++) {
+                const rlt_dense_layer& s = A->critics[k][l]; const rlt_dense_layer& t = A->critics_target[k][l];
+                sources[n] = s.weights; targets[n] = t.weights; counts[n++] = (uint32_t)s.in_dim * s.out_dim;
+                sources[n] = s.biases; targets[n] = t.biases; counts[n++] = (uint32_t)s.out_dim;
+            }
+        return rlt_sac_polyak_list(device, sources, targets, counts, n, A->polyak);
+    }
     for (int k = 0; k < 2; k++)
         for (int l = 0; l < A->n_critic_layers; l++) {
             const rlt_dense_layer& s = A->critics[k][l]; const rlt_dense_layer& t = A->critics_target[k][l];
@@ -297,6 +316,7 @@ int rlt_rocm_sac_update_critic_targets(rlt_rocm_device* device, const rlt_sac_ag
 int rlt_rocm_sac_train_actor(rlt_rocm_device* device, const rlt_sac_agent* A, const float* action_noise) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A) && action_noise);
+    if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) return rlt_sac_update_actor(device, A, action_noise);
     RLT_REQUIRE(A->state_action_value_input && A->d_output_actor_critics && A->d_critic_input[0] && A->d_critic_input[1] && A->d_actor_output_squashing &&
                 A->d_actor_output && A->actor_pre_squashing && A->actor_log_probabilities && A->actor_actions && A->log_alpha.gradient);
     const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
@@ -330,6 +350,32 @@ int rlt_rocm_sac_train_actor(rlt_rocm_device* device, const rlt_sac_agent* A, co
     if ((rc = rlt_rocm_mlp_backward(device, A->actor, A->n_actor_layers, obs, D, A->d_actor_output, 2 * ACT, nullptr, 0, B, 1, ws, ws_bytes))) return rc;
     if ((rc = rlt_rocm_adam_step(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, 0.0f, nullptr))) return rc;
     return rlt_rocm_adam_step(device, &A->log_alpha, 1, &A->alpha_adam, A->alpha_age, 0.0f, nullptr);
+}
+
+// rl/algorithms/sac/loop/core/operations_generic.h:110-155 past the warm-up, as a host loop over the entry points of this library
+int rlt_rocm_sac_pendulum_loop_by_calls(rlt_rocm_device* device, const rlt_sac_agent* A, const rlt_pendulum_runner* runner, const rlt_replay_buffer* rb, int n_steps,
+                                        uint64_t seed, uint64_t step_offset, const rlt_sac_loop_scratch* S) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(agent_ok(A) && runner && rb && S && n_steps >= 0);
+    RLT_REQUIRE(S->rollout_noise && S->noise_critic && S->noise_actor && S->env_indices && S->sample_offsets);
+    RLT_REQUIRE(rb->observation_dim == A->observation_dim && rb->action_dim == A->action_dim && rb->n_envs == runner->n_envs);
+    const int B = A->batch, ACT = A->action_dim;
+    int rc;
+    for (int i = 0; i < n_steps; i++) {
+        const uint64_t g = 8 * (step_offset + (uint64_t)i);
+        if ((rc = rlt_rocm_randn_f32(device, S->rollout_noise, (size_t)runner->n_envs * ACT, seed, g + 1))) return rc;
+        if ((rc = rlt_rocm_pendulum_runner_step(device, runner, rb, 2, A->actor, A->n_actor_layers, &A->sas, nullptr, S->rollout_noise, nullptr, seed, g + 2))) return rc;
+        if ((rc = rlt_rocm_gather_draw(device, rb, B, seed, g + 3, S->env_indices, S->sample_offsets))) return rc;
+        if ((rc = rlt_rocm_gather_batch(device, rb, S->env_indices, S->sample_offsets, 0, runner->episode_step_limit, B, A->observations_actions_base, A->rewards,
+                                        A->terminated, nullptr, nullptr, nullptr, nullptr))) return rc;
+        if ((rc = rlt_rocm_randn_f32(device, S->noise_critic, (size_t)B * ACT, seed, g + 4))) return rc;
+        for (int k = 0; k < 2; k++)
+            if ((rc = rlt_rocm_sac_train_critic(device, A, k, S->noise_critic))) return rc;
+        if ((rc = rlt_rocm_sac_update_critic_targets(device, A))) return rc;
+        if ((rc = rlt_rocm_randn_f32(device, S->noise_actor, (size_t)B * ACT, seed, g + 5))) return rc;
+        if ((rc = rlt_rocm_sac_train_actor(device, A, S->noise_actor))) return rc;
+    }
+    return 0;
 }
 
 // ---------------------------------------------------------------------------------------- sequence batches, sequential (recurrent) networks

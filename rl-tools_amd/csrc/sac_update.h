@@ -1,0 +1,14 @@
+// Internal entry points of sac_update.hip: the fused SAC updates for 3-layer networks of hidden width 64.
+#pragma once
+#include "common.h"
+
+// true if the agent fits the fused kernels: every network 3 layers in -> 64 -> 64 -> out with one hidden activation (not GELU), at most 128
+// critic inputs and 8 actions, no sequence masks
+bool rlt_sac_update_supported(const rlt_rocm_device* device, const rlt_sac_agent* agent);
+// train_critic / train_actor with the contracts of rlt_rocm_sac_train_critic / rlt_rocm_sac_train_actor; of the training buffers only
+// next_log_probabilities and target_action_value / actor_log_probabilities, actor_actions and actor_pre_squashing are written.
+// RLT_E_UNSUPPORTED unless rlt_sac_update_supported.
+int rlt_sac_update_critic(rlt_rocm_device* device, const rlt_sac_agent* agent, int critic_index, const float* action_noise);
+int rlt_sac_update_actor(rlt_rocm_device* device, const rlt_sac_agent* agent, const float* action_noise);
+// target[i] = polyak * target[i] + (1 - polyak) * source[i] for a list of tensors, one launch per 16 tensors
+int rlt_sac_polyak_list(rlt_rocm_device* device, const float* const* sources, float* const* targets, const uint32_t* counts, int n, float polyak);

@@ -323,20 +323,20 @@ class ReplayOnBackend:
 
 
 class SacOnBackend:
-    """All SAC state for the Pendulum shapes (observation 3, action 1) on one backend."""
+    """All SAC state on one backend (default: the Pendulum shapes, observation 3, action 1). params: actor, critic 0, critic 1, target 0, target 1, log_alpha."""
 
-    def __init__(self, backend, batch, hidden, params, adam_eps=1e-7, masks=True):
-        OBS, ACT, D = 3, 1, 4
+    def __init__(self, backend, batch, hidden, params, adam_eps=1e-7, masks=True, obs=3, act=1, hidden_act="relu"):
+        OBS, ACT, D = obs, act, obs + act
         self.backend, self.batch = backend, batch
         n_actor = mlp_param_count([OBS, hidden, hidden, 2 * ACT]); n_critic = mlp_param_count([D, hidden, hidden, 1])
         o = 0
-        self.actor = Mlp(backend, [OBS, hidden, hidden, 2 * ACT], params[o:o + n_actor], batch); o += n_actor
+        self.actor = Mlp(backend, [OBS, hidden, hidden, 2 * ACT], params[o:o + n_actor], batch, hidden_act); o += n_actor
         self.critics = []
         for _ in range(2):
-            self.critics.append(Mlp(backend, [D, hidden, hidden, 1], params[o:o + n_critic], batch)); o += n_critic
+            self.critics.append(Mlp(backend, [D, hidden, hidden, 1], params[o:o + n_critic], batch, hidden_act)); o += n_critic
         self.targets = []
         for _ in range(2):
-            self.targets.append(Mlp(backend, [D, hidden, hidden, 1], params[o:o + n_critic], batch, trainable=False)); o += n_critic
+            self.targets.append(Mlp(backend, [D, hidden, hidden, 1], params[o:o + n_critic], batch, hidden_act, trainable=False)); o += n_critic
         self.log_alpha = backend.array(np.array([params[o], 0, 0, 0], np.float32))
         self.alpha_age = backend.array(np.array([1], np.uint32))
         z = backend.zeros

@@ -1,0 +1,168 @@
+"""The fused SAC updates (three launches per train_critic / train_actor, one for update_critic_targets) for actors obs -> 64 -> 64 -> 2 act and
+critics obs + act -> 64 -> 64 -> 1 of any width: against the CPU checker's train_critic / train_actor / update_critic_targets
+(rl/algorithms/sac/operations_generic.h:243-337, 395-468, 488-527) and against the library's own one-launch-per-operation path, from
+identical parameters, batches and noise. Tolerance: 1e-5 relative to each tensor's largest magnitude (fp32, different summation orders)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import helpers
+from helpers import rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+
+
+def agent_parameters(rng, obs, act):
+    d = obs + act
+    critics = [helpers.random_params(rng, [d, 64, 64, 1]) for _ in range(2)]
+    targets = [c + rng.uniform(-0.01, 0.01, c.size).astype(np.float32) for c in critics]
+    return np.concatenate([helpers.random_params(rng, [obs, 64, 64, 2 * act])] + critics + targets + [np.array([np.log(0.5)], np.float32)])
+
+
+def batch_of(rng, batch, obs, act):
+    oab = rng.standard_normal((2, batch, obs + act)).astype(np.float32)
+    oab[:, :, obs:] = np.tanh(oab[:, :, obs:])
+    return oab, rng.standard_normal(batch).astype(np.float32), (rng.random(batch) < 0.1).astype(np.uint8)
+
+
+def snapshot(agent):
+    return dict(parameters=agent.parameters(), actor_gradient=agent.actor.grads.numpy(), critic0_gradient=agent.critics[0].grads.numpy(),
+                critic1_gradient=agent.critics[1].grads.numpy(), log_alpha_gradient=agent.log_alpha.numpy()[1:2],
+                actor_first_moment=agent.actor.m.numpy(), critic1_second_moment=agent.critics[1].v.numpy(),
+                target_action_value=agent.target_q.numpy(), next_log_probabilities=agent.next_lp.numpy(), actor_log_probabilities=agent.a_lp.numpy(),
+                actor_actions=agent.a_act.numpy(), actor_pre_squashing=agent.a_pre.numpy(),
+                next_state_action_value_input=agent.nsavi.numpy(),
+                ages=np.array([agent.actor.age.numpy()[0], agent.critics[0].age.numpy()[0], agent.critics[1].age.numpy()[0], agent.alpha_age.numpy()[0]], np.float64))
+
+
+def run_updates(agent, batches, noises):
+    """`len(batches)` loop steps' worth of updates: critic 0, critic 1, actor, targets, each critic and the actor on its own batch and noise"""
+    b = agent.backend
+    for (oab, rew, term), (n0, n1, na) in zip(batches, noises):
+        for k, noise in ((0, n0), (1, n1)):
+            agent.set_batch(oab[k], rew[k], term[k])
+            noise_on_backend = b.array(noise)
+            b.call("sac_train_critic", C.byref(agent.c), k, noise_on_backend.ptr)
+            b.sync()       # the batch buffers are rewritten for the next update
+        agent.set_batch(oab[2], rew[2], term[2])
+        noise_on_backend = b.array(na)
+        b.call("sac_train_actor", C.byref(agent.c), noise_on_backend.ptr)
+        b.call("sac_update_critic_targets", C.byref(agent.c))
+        b.sync()
+    return snapshot(agent)
+
+
+def make_inputs(seed, batch, obs, act, steps):
+    rng = np.random.default_rng(seed)
+    params = agent_parameters(rng, obs, act)
+    batches, noises = [], []
+    for _ in range(steps):
+        three = [batch_of(rng, batch, obs, act) for _ in range(3)]
+        batches.append(([t[0] for t in three], [t[1] for t in three], [t[2] for t in three]))
+        noises.append(tuple(rng.standard_normal((batch, act)).astype(np.float32) for _ in range(3)))
+    return params, batches, noises
+
+
+SHAPES = [  # batch, obs, act, hidden activation
+    (256, 3, 1, "relu"),        # Pendulum
+    (256, 27, 8, "relu"),       # Ant-sized: two input tiles, the widest head
+    (100, 17, 6, "tanh"),       # batch that is no multiple of 64 or 16
+    (64, 11, 3, "fast_tanh"),
+    (1, 5, 2, "relu"),
+    (300, 111, 8, "relu"),      # wide observations: the 128-input variant of the kernel
+    (130, 120, 8, "sigmoid"),   # the input limit exactly
+]
+
+
+@pytest.mark.parametrize("batch,obs,act,hidden_act", SHAPES)
+def test_fused_updates_match_the_checker_and_the_per_operation_path(oracle, rocm, batch, obs, act, hidden_act):
+    steps = 3
+    params, batches, noises = make_inputs(batch * 131 + obs, batch, obs, act, steps)
+    results = {}
+    for name, backend, per_operation in (("checker", oracle, None), ("fused", rocm, 0), ("per_operation", rocm, 1)):
+        agent = helpers.SacOnBackend(backend, batch, 64, params, masks=False, obs=obs, act=act, hidden_act=hidden_act)
+        if per_operation is not None:
+            rocm.call("sac_set_per_operation", per_operation)
+        try:
+            results[name] = run_updates(agent, batches, noises)
+        finally:
+            if per_operation is not None:
+                rocm.call("sac_set_per_operation", 0)
+    # which path ran: only the per-operation launches fill the critics' next-input buffer
+    assert not results["fused"].pop("next_state_action_value_input").any()
+    assert results["per_operation"].pop("next_state_action_value_input").any() and results["checker"].pop("next_state_action_value_input").any()
+    for other in ("checker", "per_operation"):
+        for key, ref in results[other].items():
+            err = rel_err(results["fused"][key], ref)
+            assert err <= TOL, (other, key, err)
+    # the update did something: three Adam steps moved every network
+    moved = np.abs(results["fused"]["parameters"] - params)
+    assert moved.max() > 1e-4 and results["fused"]["ages"].tolist() == [1 + steps] * 4
+
+
+def test_agents_outside_the_fused_shapes_take_the_per_operation_path(oracle, rocm):
+    """an agent with sequence masks: same entry points, same results as the checker"""
+    batch, obs, act = 64, 3, 1
+    out = []
+    for backend in (oracle, rocm):
+        loop, cfg = helpers.make_loop(oracle, batch)
+        params = helpers.loop_parameters(oracle, loop)
+        oracle.lib.rlt_oracle_sac_loop_destroy(loop)
+        agent = helpers.SacOnBackend(backend, batch, 64, params, masks=True)
+        oab, rew, term = batch_of(np.random.default_rng(1), batch, obs, act)
+        noise = np.random.default_rng(2).standard_normal((batch, act)).astype(np.float32)
+        agent.set_batch(oab, rew, term)
+        noise_on_backend = backend.array(noise)
+        backend.call("sac_train_critic", C.byref(agent.c), 0, noise_on_backend.ptr)
+        backend.call("sac_train_actor", C.byref(agent.c), noise_on_backend.ptr)
+        backend.call("sac_update_critic_targets", C.byref(agent.c))
+        backend.sync()
+        out.append((agent.parameters(), agent.nsavi.numpy(), agent.d_ci[0].numpy()))      # the per-operation path fills every training buffer
+    for got, ref in zip(out[1], out[0]):
+        assert rel_err(got, ref) <= TOL
+    assert np.abs(out[1][1]).max() > 0
+
+
+def test_loop_by_calls_equals_the_same_calls_issued_one_by_one(rocm):
+    """rlt_rocm_sac_pendulum_loop_by_calls is a host loop over public entry points with documented Philox sequences per step: issuing those
+    calls from here with the same sequence numbers leaves bit-identical parameters, replay rows and runner state."""
+    capi = helpers.capi
+    batch, capacity, steps, seed, first = 64, 500, 40, 11, 1000
+    rng = np.random.default_rng(0)
+    params = agent_parameters(rng, 3, 1)
+    final = []
+    for by_calls in (True, False):
+        agent = helpers.SacOnBackend(rocm, batch, 64, params, masks=False)
+        rb = helpers.ReplayOnBackend(rocm, 1, capacity)
+        states, ep_step, ep_ret, trunc = rocm.zeros((1, 2)), rocm.zeros((1,), np.uint32), rocm.zeros((1,)), rocm.array(np.ones(1, np.uint8))
+        runner = capi.PendulumRunner(states.ptr, ep_step.ptr, ep_ret.ptr, trunc.ptr, 1, 200, capi.pendulum_parameters())
+        rollout_noise, warm_action = rocm.zeros((1, 1)), rocm.zeros((1, 1))
+        noise_c, noise_a = rocm.zeros((batch, 1)), rocm.zeros((batch, 1))
+        env_idx, offs = rocm.zeros((batch,), np.uint32), rocm.zeros((batch,), np.uint32)
+        for c in range(batch + 10):      # uniform warm-up policy
+            rocm.call("rand_f32", warm_action.ptr, 1, -1.0, 1.0, seed, 8 * c + 1)
+            rocm.call("pendulum_runner_step", C.byref(runner), C.byref(rb.c), 0, agent.actor.layers, 3, C.byref(agent.c.sas), warm_action.ptr, None, None, seed, 8 * c + 2)
+        if by_calls:
+            scratch = capi.SacLoopScratch(rollout_noise.ptr, noise_c.ptr, noise_a.ptr, env_idx.ptr, offs.ptr)
+            rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), steps, seed, first, C.byref(scratch))
+        else:
+            for i in range(steps):
+                g = 8 * (first + i)
+                rocm.call("randn_f32", rollout_noise.ptr, 1, seed, g + 1)
+                rocm.call("pendulum_runner_step", C.byref(runner), C.byref(rb.c), 2, agent.actor.layers, 3, C.byref(agent.c.sas), None, rollout_noise.ptr, None, seed, g + 2)
+                rocm.call("gather_draw", C.byref(rb.c), batch, seed, g + 3, env_idx.ptr, offs.ptr)
+                rocm.call("gather_batch", C.byref(rb.c), env_idx.ptr, offs.ptr, 0, 200, batch, agent.oab.ptr, agent.rewards.ptr, agent.terminated.ptr, None, None, None, None)
+                rocm.call("randn_f32", noise_c.ptr, batch, seed, g + 4)
+                for k in range(2):
+                    rocm.call("sac_train_critic", C.byref(agent.c), k, noise_c.ptr)
+                rocm.call("sac_update_critic_targets", C.byref(agent.c))
+                rocm.call("randn_f32", noise_a.ptr, batch, seed, g + 5)
+                rocm.call("sac_train_actor", C.byref(agent.c), noise_a.ptr)
+        rocm.sync()
+        final.append((agent.parameters(), rb.data.numpy(), states.numpy(), ep_ret.numpy()))
+    for a, b in zip(*final):
+        assert np.array_equal(a, b)
+    assert np.abs(final[0][0] - params).max() > 1e-3 and np.all(np.isfinite(final[0][0]))
