@@ -23,7 +23,7 @@ namespace {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) float* lptr;
 constexpr int H = 64, HS = H + 1, WAVES = 4, ROWS = 16 * WAVES, THREADS = 64 * WAVES, MAX_D = 128, MAX_ACT = 8, MAX_OUT = 16, D3S = MAX_OUT + 1, N_EXTRA = 16,
-              N_SUMS = 2 * H + MAX_OUT + N_EXTRA, MISC = 16;
+              N_SUMS = 2 * H + MAX_OUT + N_EXTRA, MISC = 16, N_BIAS = 2 * H + MAX_OUT;
 enum { MODE_CRITIC = 0, MODE_ACTOR = 1 };
 
 struct Net { const float *W1, *b1, *W2, *b2, *W3, *b3; int in, out, act_h, act3; };
@@ -63,64 +63,77 @@ __device__ __forceinline__ float normal_log_prob(float mean, float log_std, floa
     return -0.9189385332046727f - log_std - 0.5f * z * z;
 }
 
+// hidden activation: a compile-time constant where the kernel is instantiated for it (ACT_H >= 0), else the network's run-time value
+template <int ACT_H> __device__ __forceinline__ float act_hidden(float x, int f) { return rlt_act(x, ACT_H >= 0 ? ACT_H : f); }
+template <int ACT_H> __device__ __forceinline__ float dact_hidden(float o, int f) { return rlt_dact_from_output(o, ACT_H >= 0 ? ACT_H : f); }
+
 constexpr size_t lds_floats(int nt1c) {
     const int sx = 16 * nt1c + 1;
-    return (size_t)H * sx + H * HS + MAX_OUT * HS + (size_t)ROWS * (sx + 4 * HS + D3S) + WAVES * MISC;
+    return (size_t)H * sx + H * HS + MAX_OUT * HS + N_BIAS + (size_t)ROWS * (sx + 4 * HS + D3S) + WAVES * MISC;
 }
 
-// the workgroup replaces the network in LDS: W1 rows padded to SX with zeros beyond the input width (so the padded reduction steps and
-// columns that hold something else add nothing), W3 rows beyond the output width zero
-template <int SX>
-__device__ __forceinline__ void stage_net(const Net& N, lptr w1s, lptr w2s, lptr w3s, int wave, int lane) {
-    const int IN = N.in, OUT = N.out;
-    float v1[H / WAVES][2], v2[H * H / THREADS], v3[MAX_OUT * H / THREADS];
+// The workgroup replaces the network in LDS in two halves, so that the loads travel while the previous network is still at work:
+// fetch_net requests this thread's share of the parameters into registers, commit_net waits for every wavefront to be done with the
+// previous network, stores them and meets again. W1 rows are padded to SX with zeros beyond the input width (so the padded reduction
+// steps and columns that hold something else add nothing), W3 rows and biases beyond the output width are zero.
+struct NetRegs { float v1[H / WAVES][2], v2[H * H / THREADS], v3[MAX_OUT * H / THREADS], bias; };
+__device__ __forceinline__ void fetch_net(const Net& N, NetRegs& R, int wave, int lane) {
+    const int IN = N.in, OUT = N.out, t = threadIdx.x;
 #pragma unroll
     for (int j = 0; j < H / WAVES; j++) {
         const float* src = N.W1 + (size_t)(wave * (H / WAVES) + j) * IN;
-        v1[j][0] = src[min(lane, IN - 1)];
-        v1[j][1] = IN > 64 ? src[min(64 + lane, IN - 1)] : 0.f;
+        R.v1[j][0] = src[min(lane, IN - 1)];
+        R.v1[j][1] = IN > 64 ? src[min(64 + lane, IN - 1)] : 0.f;
     }
 #pragma unroll
-    for (int u = 0; u < H * H / THREADS; u++) v2[u] = N.W2[u * THREADS + threadIdx.x];
+    for (int u = 0; u < H * H / THREADS; u++) R.v2[u] = N.W2[u * THREADS + t];
 #pragma unroll
-    for (int u = 0; u < MAX_OUT * H / THREADS; u++) v3[u] = N.W3[min(u * THREADS + (int)threadIdx.x, OUT * H - 1)];
+    for (int u = 0; u < MAX_OUT * H / THREADS; u++) R.v3[u] = N.W3[min(u * THREADS + t, OUT * H - 1)];
+    R.bias = t < H ? N.b1[t] : t < 2 * H ? N.b2[t - H] : N.b3[min(t - 2 * H, OUT - 1)];
+}
+template <int SX>
+__device__ __forceinline__ void commit_net(const NetRegs& R, int IN, int OUT, lptr w1s, lptr w2s, lptr w3s, lptr bs, int wave, int lane) {
     rlt_lds_barrier();      // nobody reads the previous network any more
 #pragma unroll
     for (int j = 0; j < H / WAVES; j++) {
         const lptr dst = w1s + (wave * (H / WAVES) + j) * SX;
-        if (lane < SX) dst[lane] = lane < IN ? v1[j][0] : 0.f;
-        if (64 + lane < SX) dst[64 + lane] = 64 + lane < IN ? v1[j][1] : 0.f;
+        if (lane < SX) dst[lane] = lane < IN ? R.v1[j][0] : 0.f;
+        if (64 + lane < SX) dst[64 + lane] = 64 + lane < IN ? R.v1[j][1] : 0.f;
         if (lane == 0 && SX > 128) dst[128] = 0.f;
     }
 #pragma unroll
-    for (int u = 0; u < H * H / THREADS; u++) { const int i = u * THREADS + threadIdx.x; w2s[(i >> 6) * HS + (i & 63)] = v2[u]; }
+    for (int u = 0; u < H * H / THREADS; u++) { const int i = u * THREADS + threadIdx.x; w2s[(i >> 6) * HS + (i & 63)] = R.v2[u]; }
 #pragma unroll
-    for (int u = 0; u < MAX_OUT * H / THREADS; u++) { const int i = u * THREADS + threadIdx.x; w3s[(i >> 6) * HS + (i & 63)] = (i >> 6) < OUT ? v3[u] : 0.f; }
+    for (int u = 0; u < MAX_OUT * H / THREADS; u++) { const int i = u * THREADS + threadIdx.x; w3s[(i >> 6) * HS + (i & 63)] = (i >> 6) < OUT ? R.v3[u] : 0.f; }
+    if (threadIdx.x < N_BIAS) bs[threadIdx.x] = (int)threadIdx.x < 2 * H + OUT ? R.bias : 0.f;
     rlt_lds_barrier();
 }
 
-// the wavefront's 16 rows of a [batch x ld] array into its input tile: columns [0, valid), zero beyond them and beyond the batch
-template <int SX, int NT1C>
-__device__ __forceinline__ void load_rows(lptr xs, const float* base, int ld, int row0, int batch, int valid, int lane) {
-    float va[16], vb[16];
+// the wavefront's 16 rows of a [batch x ld] array for its input tile: columns [0, valid), zero beyond them and beyond the batch; requested
+// into registers, stored later
+struct RowRegs { float va[16], vb[16]; };
+__device__ __forceinline__ void request_rows(RowRegs& X, const float* base, int ld, int row0, int batch, int valid, int lane) {
 #pragma unroll
     for (int row = 0; row < 16; row++) {
         const bool rok = row0 + row < batch;
         const float* src = base + (size_t)min(row0 + row, batch - 1) * ld;
-        va[row] = (rok && lane < valid) ? src[lane] : 0.f;
-        vb[row] = (rok && 64 + lane < valid) ? src[64 + lane] : 0.f;
+        X.va[row] = (rok && lane < valid) ? src[lane] : 0.f;
+        X.vb[row] = (rok && 64 + lane < valid) ? src[64 + lane] : 0.f;
     }
+}
+template <int SX, int NT1C>
+__device__ __forceinline__ void store_rows(const RowRegs& X, lptr xs, int lane) {
 #pragma unroll
     for (int row = 0; row < 16; row++) {
-        if (lane < 16 * NT1C) xs[row * SX + lane] = va[row];
-        if (64 + lane < 16 * NT1C) xs[row * SX + 64 + lane] = vb[row];
+        if (lane < 16 * NT1C) xs[row * SX + lane] = X.va[row];
+        if (64 + lane < 16 * NT1C) xs[row * SX + 64 + lane] = X.vb[row];
     }
 }
 
 // the three layers on the wavefront's rows; h1 and h2 (after the activation) stay in LDS; returns the last layer's sums before bias and
 // activation: element v of lane (r, kk) belongs to row 4 kk + v, output r
-template <int SX>
-__device__ __forceinline__ floatx4 forward16(const Net& N, lptr w1s, lptr w2s, lptr w3s, lptr xs, lptr h1s, lptr h2s, int r, int kk) {
+template <int SX, int ACT_H>
+__device__ __forceinline__ floatx4 forward16(const Net& N, lptr w1s, lptr w2s, lptr w3s, lptr bs, lptr xs, lptr h1s, lptr h2s, int r, int kk) {
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
     const int NT1 = (N.in + 15) >> 4;
     floatx4 acc[4] = {zero4, zero4, zero4, zero4};
@@ -134,9 +147,9 @@ __device__ __forceinline__ floatx4 forward16(const Net& N, lptr w1s, lptr w2s, l
     }
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) {
-        const float b = N.b1[16 * nt + r];
+        const float b = bs[16 * nt + r];
 #pragma unroll
-        for (int v = 0; v < 4; v++) h1s[(4 * kk + v) * HS + 16 * nt + r] = rlt_act(acc[nt][v] + b, N.act_h);
+        for (int v = 0; v < 4; v++) h1s[(4 * kk + v) * HS + 16 * nt + r] = act_hidden<ACT_H>(acc[nt][v] + b, N.act_h);
     }
     wave_sync();
 #pragma unroll
@@ -149,9 +162,9 @@ __device__ __forceinline__ floatx4 forward16(const Net& N, lptr w1s, lptr w2s, l
     }
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) {
-        const float b = N.b2[16 * nt + r];
+        const float b = bs[H + 16 * nt + r];
 #pragma unroll
-        for (int v = 0; v < 4; v++) h2s[(4 * kk + v) * HS + 16 * nt + r] = rlt_act(acc[nt][v] + b, N.act_h);
+        for (int v = 0; v < 4; v++) h2s[(4 * kk + v) * HS + 16 * nt + r] = act_hidden<ACT_H>(acc[nt][v] + b, N.act_h);
     }
     wave_sync();
     floatx4 y0 = zero4, y1 = zero4;
@@ -164,6 +177,7 @@ __device__ __forceinline__ floatx4 forward16(const Net& N, lptr w1s, lptr w2s, l
 }
 
 // d_pre2 = (d_pre3 W3) f'(h2) into g2s (may be h2s itself), accumulating its column sums
+template <int ACT_H>
 __device__ __forceinline__ void backward_layer3(const Net& N, lptr w3s, lptr d3s, lptr h2s, lptr g2s, float (&s2)[4], int r, int kk) {
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
     floatx4 acc[4] = {zero4, zero4, zero4, zero4};
@@ -178,11 +192,12 @@ __device__ __forceinline__ void backward_layer3(const Net& N, lptr w3s, lptr d3s
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const int idx = (4 * kk + v) * HS + 16 * nt + r;
-            const float dp = acc[nt][v] * rlt_dact_from_output(h2s[idx], N.act_h);
+            const float dp = acc[nt][v] * dact_hidden<ACT_H>(h2s[idx], N.act_h);
             g2s[idx] = dp; s2[nt] += dp;
         }
 }
 // d_pre1 = (d_pre2 W2) f'(h1) into p1s (may be h1s itself), accumulating its column sums
+template <int ACT_H>
 __device__ __forceinline__ void backward_layer2(const Net& N, lptr w2s, lptr g2s, lptr h1s, lptr p1s, float (&s1)[4], int r, int kk) {
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
     floatx4 acc[4] = {zero4, zero4, zero4, zero4};
@@ -197,14 +212,14 @@ __device__ __forceinline__ void backward_layer2(const Net& N, lptr w2s, lptr g2s
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const int idx = (4 * kk + v) * HS + 16 * nt + r;
-            const float dp = acc[nt][v] * rlt_dact_from_output(h1s[idx], N.act_h);
+            const float dp = acc[nt][v] * dact_hidden<ACT_H>(h1s[idx], N.act_h);
             p1s[idx] = dp; s1[nt] += dp;
         }
 }
 
 // sample_and_squash forward for the items of a lane: row r of the wavefront's tile, actions kk and kk + 4
 struct HeadItem { float mean, log_std_raw, noise, sample, action; };
-__device__ __forceinline__ float head_forward(const UpdateArgs& A, lptr d3s, lptr xs, int SX, int row0, int r, int kk, HeadItem (&item)[2]) {
+__device__ __forceinline__ float head_forward(const UpdateArgs& A, lptr d3s, lptr xs, int SX, const float (&noise)[2], int r, int kk, HeadItem (&item)[2]) {
     float log_prob = 0.f;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
@@ -216,7 +231,7 @@ __device__ __forceinline__ float head_forward(const UpdateArgs& A, lptr d3s, lpt
             I.log_std_raw = d3s[r * D3S + A.act + a];
             const float log_std = clampf(I.log_std_raw, A.sas.log_std_lower_bound, A.sas.log_std_upper_bound);
             const float sd = expf(log_std);
-            I.noise = row0 + r < A.batch ? A.noise[(size_t)(row0 + r) * A.act + a] : 0.f;
+            I.noise = noise[j];
             I.sample = I.mean + I.noise * sd;
             I.action = tanhf(I.sample);
             xs[r * SX + A.obs + a] = I.action;
@@ -226,37 +241,49 @@ __device__ __forceinline__ float head_forward(const UpdateArgs& A, lptr d3s, lpt
     return groups_sum(log_prob);
 }
 
-template <int NT1C, int MODE>
+template <int NT1C, int MODE, int ACT_H>
 __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
     extern __shared__ float lds_raw[];
     constexpr int SX = 16 * NT1C + 1;
     const int lane = threadIdx.x & 63, r = lane & 15, kk = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int OBS = A.obs, ACT = A.act, D = OBS + ACT, B = A.batch;
-    const lptr w1s = (lptr)lds_raw, w2s = w1s + H * SX, w3s = w2s + H * HS;
-    const lptr xs_all = w3s + MAX_OUT * HS, h1_all = xs_all + ROWS * SX, h2_all = h1_all + ROWS * HS, ta_all = h2_all + ROWS * HS, tb_all = ta_all + ROWS * HS,
+    const lptr w1s = (lptr)lds_raw, w2s = w1s + H * SX, w3s = w2s + H * HS, bs = w3s + MAX_OUT * HS;
+    const lptr xs_all = bs + N_BIAS, h1_all = xs_all + ROWS * SX, h2_all = h1_all + ROWS * HS, ta_all = h2_all + ROWS * HS, tb_all = ta_all + ROWS * HS,
                d3_all = tb_all + ROWS * HS, misc_all = d3_all + ROWS * D3S;
     const lptr xs = xs_all + 16 * wave * SX, h1s = h1_all + 16 * wave * HS, h2s = h2_all + 16 * wave * HS, tas = ta_all + 16 * wave * HS, tbs = tb_all + 16 * wave * HS,
                d3s = d3_all + 16 * wave * D3S, misc = misc_all + wave * MISC;
     const int row0 = blockIdx.x * ROWS + 16 * wave;
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
-    const float alpha = expf(*A.log_alpha);
     float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f}, s3 = 0.f, extra = 0.f, unused[4] = {0.f, 0.f, 0.f, 0.f};
     const Net& trained = MODE == MODE_CRITIC ? A.critic[0] : A.actor;
+    // every global load is requested one stage ahead of its use: the next network's parameters while the current one computes
+    NetRegs R;
+    RowRegs X;
+    fetch_net(A.actor, R, wave, lane);
+    request_rows(X, MODE == MODE_CRITIC ? A.batch_base + (size_t)B * D : A.batch_base, D, row0, B, MODE == MODE_CRITIC ? D : OBS, lane);
+    const float alpha = expf(*A.log_alpha);
+    float noise[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) noise[j] = (kk + 4 * j < ACT && row0 + r < B) ? A.noise[(size_t)(row0 + r) * ACT + kk + 4 * j] : 0.f;
+    HeadItem item[2];
 
     if (MODE == MODE_CRITIC) {
+        float reward[4]; bool terminated[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) { const int row = min(row0 + 4 * kk + v, B - 1); reward[v] = A.rewards[row]; terminated[v] = A.terminated[row] != 0; }
         // the actor on the next observations, its squashed sample into the action columns of the tile
-        load_rows<SX, NT1C>(xs, A.batch_base + (size_t)B * D, D, row0, B, D, lane);
-        stage_net<SX>(A.actor, w1s, w2s, w3s, wave, lane);
+        store_rows<SX, NT1C>(X, xs, lane);
+        commit_net<SX>(R, A.actor.in, A.actor.out, w1s, w2s, w3s, bs, wave, lane);
+        fetch_net(A.target[0], R, wave, lane);
         {
-            const floatx4 y = forward16<SX>(A.actor, w1s, w2s, w3s, xs, tas, tbs, r, kk);
-            const float b3 = A.actor.b3[min(r, A.actor.out - 1)];
+            const floatx4 y = forward16<SX, ACT_H>(A.actor, w1s, w2s, w3s, bs, xs, tas, tbs, r, kk);
+            const float b3 = bs[2 * H + r];
 #pragma unroll
             for (int v = 0; v < 4; v++) d3s[(4 * kk + v) * D3S + r] = r < A.actor.out ? rlt_act(y[v] + b3, A.actor.act3) : 0.f;
         }
         wave_sync();
-        HeadItem item[2];
-        const float next_log_prob = head_forward(A, d3s, xs, SX, row0, r, kk, item);
+        const float next_log_prob = head_forward(A, d3s, xs, SX, noise, r, kk, item);
         if (kk == 0) {
             misc[r] = next_log_prob;
             if (A.out_log_probabilities && row0 + r < B) A.out_log_probabilities[row0 + r] = next_log_prob;
@@ -266,9 +293,11 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
         float q_min[4];
 #pragma unroll
         for (int k = 0; k < 2; k++) {
-            stage_net<SX>(A.target[k], w1s, w2s, w3s, wave, lane);
-            const floatx4 y = forward16<SX>(A.target[k], w1s, w2s, w3s, xs, tas, tbs, r, kk);
-            const float b3 = A.target[k].b3[0];
+            commit_net<SX>(R, A.target[k].in, A.target[k].out, w1s, w2s, w3s, bs, wave, lane);
+            if (k == 0) fetch_net(A.target[1], R, wave, lane);
+            else { fetch_net(trained, R, wave, lane); request_rows(X, A.batch_base, D, row0, B, D, lane); }
+            const floatx4 y = forward16<SX, ACT_H>(A.target[k], w1s, w2s, w3s, bs, xs, tas, tbs, r, kk);
+            const float b3 = bs[2 * H];
 #pragma unroll
             for (int v = 0; v < 4; v++) { const float q = rlt_act(y[v] + b3, A.target[k].act3); q_min[v] = k ? fminf(q_min[v], q) : q; }
         }
@@ -276,18 +305,17 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
         float y_target[4];
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            const int row = min(row0 + 4 * kk + v, B - 1);
             const float min_q = q_min[v] - alpha * misc[4 * kk + v];
-            const float future = A.terminated[row] ? 0.0f : A.gamma * min_q;
-            y_target[v] = A.rewards[row] + future;
-            if (A.out_target_action_value && r == 0 && row0 + 4 * kk + v < B) A.out_target_action_value[row] = y_target[v];
+            const float future = terminated[v] ? 0.0f : A.gamma * min_q;
+            y_target[v] = reward[v] + future;
+            if (A.out_target_action_value && r == 0 && row0 + 4 * kk + v < B) A.out_target_action_value[row0 + 4 * kk + v] = y_target[v];
         }
         // the critic on the current rows, MSE gradient at its pre-activation
         wave_sync();
-        load_rows<SX, NT1C>(xs, A.batch_base, D, row0, B, D, lane);
-        stage_net<SX>(trained, w1s, w2s, w3s, wave, lane);
-        const floatx4 y = forward16<SX>(trained, w1s, w2s, w3s, xs, h1s, h2s, r, kk);
-        const float b3 = trained.b3[0];
+        store_rows<SX, NT1C>(X, xs, lane);
+        commit_net<SX>(R, trained.in, trained.out, w1s, w2s, w3s, bs, wave, lane);
+        const floatx4 y = forward16<SX, ACT_H>(trained, w1s, w2s, w3s, bs, xs, h1s, h2s, r, kk);
+        const float b3 = bs[2 * H];
         // loss weight batch * 0.5 / n with n = batch rows (no masks), times the MSE gradient's 2 / batch (rl/algorithms/sac/operations_generic.h:298-316)
         const float loss_weight = (1.0f / (float)B) * ((float)B * 0.5f);
         const float constant = 2.0f / (float)B * loss_weight;
@@ -303,17 +331,17 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
         }
     } else {
         // actor forward on the observations (its hidden activations are kept for the backward pass), squashed sample into the action columns
-        load_rows<SX, NT1C>(xs, A.batch_base, D, row0, B, OBS, lane);
-        stage_net<SX>(A.actor, w1s, w2s, w3s, wave, lane);
+        store_rows<SX, NT1C>(X, xs, lane);
+        commit_net<SX>(R, A.actor.in, A.actor.out, w1s, w2s, w3s, bs, wave, lane);
+        fetch_net(A.critic[0], R, wave, lane);
         {
-            const floatx4 y = forward16<SX>(A.actor, w1s, w2s, w3s, xs, h1s, h2s, r, kk);
-            const float b3 = A.actor.b3[min(r, A.actor.out - 1)];
+            const floatx4 y = forward16<SX, ACT_H>(A.actor, w1s, w2s, w3s, bs, xs, h1s, h2s, r, kk);
+            const float b3 = bs[2 * H + r];
 #pragma unroll
             for (int v = 0; v < 4; v++) d3s[(4 * kk + v) * D3S + r] = r < A.actor.out ? rlt_act(y[v] + b3, A.actor.act3) : 0.f;
         }
         wave_sync();
-        HeadItem item[2];
-        const float log_prob = head_forward(A, d3s, xs, SX, row0, r, kk, item);
+        const float log_prob = head_forward(A, d3s, xs, SX, noise, r, kk, item);
         const bool row_ok = row0 + r < B;
         if (row_ok) {
             if (kk == 0 && A.out_log_probabilities) A.out_log_probabilities[row0 + r] = log_prob;
@@ -331,9 +359,10 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
 #pragma unroll
         for (int k = 0; k < 2; k++) {
             const Net& C = A.critic[k];
-            stage_net<SX>(C, w1s, w2s, w3s, wave, lane);
-            const floatx4 y = forward16<SX>(C, w1s, w2s, w3s, xs, tas, tbs, r, kk);
-            const float b3 = C.b3[0];
+            commit_net<SX>(R, C.in, C.out, w1s, w2s, w3s, bs, wave, lane);
+            fetch_net(k == 0 ? A.critic[1] : A.actor, R, wave, lane);
+            const floatx4 y = forward16<SX, ACT_H>(C, w1s, w2s, w3s, bs, xs, tas, tbs, r, kk);
+            const float b3 = bs[2 * H];
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const float q = rlt_act(y[v] + b3, C.act3);
@@ -341,9 +370,9 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
                 d3s[(4 * kk + v) * D3S + r] = (r == 0 && row0 + 4 * kk + v < B) ? loss_weight * rlt_dact_from_output(q, C.act3) : 0.f;
             }
             wave_sync();
-            backward_layer3(C, w3s, d3s, tbs, tbs, unused, r, kk);
+            backward_layer3<ACT_H>(C, w3s, d3s, tbs, tbs, unused, r, kk);
             wave_sync();
-            backward_layer2(C, w2s, tbs, tas, tas, unused, r, kk);
+            backward_layer2<ACT_H>(C, w2s, tbs, tas, tas, unused, r, kk);
             wave_sync();
             q_row[k] = misc[r];
 #pragma unroll
@@ -390,7 +419,7 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
         wave_sync();
 #pragma unroll
         for (int v = 0; v < 4; v++) s3 += d3s[(4 * kk + v) * D3S + r];
-        stage_net<SX>(A.actor, w1s, w2s, w3s, wave, lane);
+        commit_net<SX>(R, A.actor.in, A.actor.out, w1s, w2s, w3s, bs, wave, lane);
     }
 
     // backward pass of the trained network with its weight gradients over the workgroup's 64 rows; h1, h2: its hidden activations,
@@ -406,7 +435,7 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
         const float a = d3_all[(4 * ks + kk) * D3S + r], b = h2_all[(4 * ks + kk) * HS + 16 * wave + r];
         if (ks & 1) aW3b = mfma16(a, b, aW3b); else aW3a = mfma16(a, b, aW3a);
     }
-    backward_layer3(trained, w3s, d3s, h2s, tas, s2, r, kk);
+    backward_layer3<ACT_H>(trained, w3s, d3s, h2s, tas, s2, r, kk);
     rlt_lds_barrier();      // every wavefront's d_pre2 is in place, and nobody reads h2 any more
 #pragma unroll
     for (int ks = 0; ks < ROWS / 4; ks++) {
@@ -414,7 +443,7 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
 #pragma unroll
         for (int nt = 0; nt < 4; nt++) aW2[nt] = mfma16(a, h1_all[(4 * ks + kk) * HS + 16 * nt + r], aW2[nt]);
     }
-    backward_layer2(trained, w2s, tas, h1s, h2s, s1, r, kk);
+    backward_layer2<ACT_H>(trained, w2s, tas, h1s, h2s, s1, r, kk);
     rlt_lds_barrier();      // every wavefront's d_pre1 is in place
 #pragma unroll 4
     for (int ks = 0; ks < ROWS / 4; ks++) {
@@ -490,13 +519,19 @@ int launch_update(rlt_rocm_device* device, UpdateArgs& a, int groups, const rlt_
     int rc = rlt_scratch(device, (size_t)groups * a.count * sizeof(float), &scratch);
     if (rc) return rc;
     a.partial = (float*)scratch;
+#define RLT_LAUNCH_UPDATE(NT, ACT)                                                                                                                              \
+    do {                                                                                                                                                        \
+        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sac_update_kernel<NT, MODE, ACT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
+        hipLaunchKernelGGL((sac_update_kernel<NT, MODE, ACT>), dim3(groups), dim3(THREADS), lds_bytes, device->stream, a);                                    \
+    } while (0)
+    // ReLU (the reference's default for SAC) and tanh are compiled in; any other hidden activation takes the variant that looks it up
+    const int act = a.actor.act_h == a.critic[0].act_h && a.actor.act_h == a.target[0].act_h ? a.actor.act_h : -1;
     if (bucket == 2) {
-        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sac_update_kernel<2, MODE>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-        hipLaunchKernelGGL((sac_update_kernel<2, MODE>), dim3(groups), dim3(THREADS), lds_bytes, device->stream, a);
+        if (act == RLT_ACT_RELU) RLT_LAUNCH_UPDATE(2, RLT_ACT_RELU); else if (act == RLT_ACT_TANH) RLT_LAUNCH_UPDATE(2, RLT_ACT_TANH); else RLT_LAUNCH_UPDATE(2, -1);
     } else {
-        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sac_update_kernel<MAX_D / 16, MODE>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-        hipLaunchKernelGGL((sac_update_kernel<MAX_D / 16, MODE>), dim3(groups), dim3(THREADS), lds_bytes, device->stream, a);
+        if (act == RLT_ACT_RELU) RLT_LAUNCH_UPDATE(MAX_D / 16, RLT_ACT_RELU); else if (act == RLT_ACT_TANH) RLT_LAUNCH_UPDATE(MAX_D / 16, RLT_ACT_TANH); else RLT_LAUNCH_UPDATE(MAX_D / 16, -1);
     }
+#undef RLT_LAUNCH_UPDATE
     if ((rc = rlt_launch_status(device))) return rc;
     return rlt_mlp3s_reduce(device, trained, a.partial, groups, 1, extra, extra ? 1 : 0, extra_scale, 0.0f);
 }
