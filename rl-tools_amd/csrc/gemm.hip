@@ -43,7 +43,7 @@ struct TileRegs { float4 v[(R * 4 + THREADS - 1) / THREADS]; };
 // source rows are contiguous along k: tile element (row r, k) = src[(row0+r)*ld + k0+k]
 template <int R>
 __device__ __forceinline__ void gload_kcontig(TileRegs<R>& t, const float* __restrict__ src, int ld, int row0, int nrows,
-                                              int k0, int kend, bool vec, int tid) {
+                                              int k0, int kend, int vec, int tid) {
     constexpr int NQ = (R * 4 + THREADS - 1) / THREADS;
 #pragma unroll
     for (int i = 0; i < NQ; i++) {
@@ -54,8 +54,11 @@ __device__ __forceinline__ void gload_kcontig(TileRegs<R>& t, const float* __res
             int gr = row0 + row, gk = k0 + kq;
             if (gr < nrows && gk < kend) {
                 const float* p = src + (size_t)gr * ld + gk;
-                if (vec && gk + 3 < kend) v = *reinterpret_cast<const float4*>(p);
-                else {
+                if (vec == 4 && gk + 3 < kend) v = *reinterpret_cast<const float4*>(p);
+                else if (vec == 2 && gk + 3 < kend) {       // rows that are only 8-byte aligned (an even leading dimension that is no multiple of 4)
+                    const float2 lo = *reinterpret_cast<const float2*>(p), hi = *reinterpret_cast<const float2*>(p + 2);
+                    v = make_float4(lo.x, lo.y, hi.x, hi.y);
+                } else {
                     v.x = p[0];
                     if (gk + 1 < kend) v.y = p[1];
                     if (gk + 2 < kend) v.z = p[2];
@@ -84,7 +87,7 @@ __device__ __forceinline__ void sstore_kcontig(const TileRegs<R>& t, float* s, i
 // source rows are k, contiguous along the tile's m/n: tile element (k, c) = src[(k0+k)*ld + col0+c]
 template <int R>
 __device__ __forceinline__ void gload_mncontig(TileRegs<R>& t, const float* __restrict__ src, int ld, int col0, int ncols,
-                                               int k0, int kend, bool vec, int tid) {
+                                               int k0, int kend, int vec, int tid) {
     constexpr int NQ = (R * 4 + THREADS - 1) / THREADS;
     constexpr int QPR = R / 4;  // quads per k-row
 #pragma unroll
@@ -96,8 +99,11 @@ __device__ __forceinline__ void gload_mncontig(TileRegs<R>& t, const float* __re
             int gk = k0 + k, gc = col0 + c4;
             if (gk < kend && gc < ncols) {
                 const float* p = src + (size_t)gk * ld + gc;
-                if (vec && gc + 3 < ncols) v = *reinterpret_cast<const float4*>(p);
-                else {
+                if (vec == 4 && gc + 3 < ncols) v = *reinterpret_cast<const float4*>(p);
+                else if (vec == 2 && gc + 3 < ncols) {
+                    const float2 lo = *reinterpret_cast<const float2*>(p), hi = *reinterpret_cast<const float2*>(p + 2);
+                    v = make_float4(lo.x, lo.y, hi.x, hi.y);
+                } else {
                     v.x = p[0];
                     if (gc + 1 < ncols) v.y = p[1];
                     if (gc + 2 < ncols) v.z = p[2];
@@ -234,7 +240,14 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(float* __restrict__ d
     const size_t stride = (size_t)mn + m;
     const int e = blockIdx.x * 64 + (threadIdx.x & 63), g = threadIdx.x >> 6;
     float s = 0.0f;
-    if (e < total) for (int k = g; k < splits; k += 4) s += ws[(size_t)k * stride + e];
+    if (e < total)
+        for (int k0 = g; k0 < splits; k0 += 32) {      // eight loads in flight, added in the order of the splits
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) { const int k = k0 + 4 * u; v[u] = k < splits ? ws[(size_t)k * stride + e] : 0.0f; }
+#pragma unroll
+            for (int u = 0; u < 8; u++) s += v[u];
+        }
     partial[g][threadIdx.x & 63] = s;
     __syncthreads();
     if (g == 0 && e < total) {
@@ -252,35 +265,56 @@ __global__ __launch_bounds__(256) void dpre_kernel(const float* src, int lds, fl
     }
 }
 
-inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+// widest vector a row-contiguous operand can be loaded with: 4 floats (16-byte aligned base, leading dimension a multiple of 4), 2, or 1
+inline int vector_width(const void* p, int ld) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    if ((a & 15u) == 0 && ld % 4 == 0) return 4;
+    if ((a & 7u) == 0 && ld % 2 == 0) return 2;
+    return 1;
+}
 
-// tile shape by problem shape: 128x128 for the wide contractions, 128x32 / 32x128 when one side is narrow, 64x64 when both are small
-enum TileShape { TILE_128x32, TILE_32x128, TILE_64x64, TILE_128x128 };
-TileShape pick_tile(int M, int N) {
+// Tile shape by problem shape. One side narrow: 128x32 / 32x128. Small problems: 64x64. Otherwise, measured on 65,536-row batches at widths 146-256:
+// the forward and input-gradient contractions (reduction over a layer width, i.e. a few k-steps per tile) run fastest on 128x64 tiles, which keep
+// more workgroups resident to hide the short reduction's prologue and epilogue; the weight-gradient contraction (reduction over the batch) on
+// 128x128 tiles unless those overhang the matrix by more than 15 % over 64x64 tiles (192 x 146 weights: 65,536 against 36,864 padded elements).
+enum TileShape { TILE_128x32, TILE_32x128, TILE_64x64, TILE_128x128, TILE_128x64 };
+void tile_dims(TileShape shape, int& bm, int& bn) {
+    switch (shape) {
+        case TILE_128x32: bm = 128; bn = 32; break;
+        case TILE_32x128: bm = 32; bn = 128; break;
+        case TILE_64x64: bm = 64; bn = 64; break;
+        case TILE_128x64: bm = 128; bn = 64; break;
+        default: bm = 128; bn = 128; break;
+    }
+}
+long long padded_area(int M, int N, TileShape shape) {
+    int bm, bn;
+    tile_dims(shape, bm, bn);
+    return (long long)rlt_div_up(M, bm) * bm * rlt_div_up(N, bn) * bn;
+}
+TileShape pick_tile(int M, int N, int mode) {
     if (N <= 32) return TILE_128x32;
     if (M <= 32) return TILE_32x128;
     if (M <= 64 || N <= 64 || (long long)M * N < 128ll * 128) return TILE_64x64;
-    return TILE_128x128;
+    if (mode != 2) return TILE_128x64;
+    return 100 * padded_area(M, N, TILE_128x128) <= 115 * padded_area(M, N, TILE_64x64) ? TILE_128x128 : TILE_64x64;
 }
 
 template <int MODE>
 int launch(rlt_rocm_device* device, const GemmParams& p, int splits) {
     dim3 block(THREADS);
-    TileShape shape = pick_tile(p.M, p.N);
-    // a grid of 128x128 tiles that leaves compute units idle runs faster as four times as many 64x64 tiles (no split over k to fill the chip here)
-    if (MODE != 2 && shape == TILE_128x128 && rlt_div_up(p.N, 128) * rlt_div_up(p.M, 128) < device->compute_units) shape = TILE_64x64;
-    if (shape == TILE_128x32) {
-        dim3 grid(rlt_div_up(p.N, 32), rlt_div_up(p.M, 128), splits);
-        hipLaunchKernelGGL((gemm_kernel<MODE, 4, 1, 1, 1>), grid, block, 0, device->stream, p);
-    } else if (shape == TILE_32x128) {
-        dim3 grid(rlt_div_up(p.N, 128), rlt_div_up(p.M, 32), splits);
-        hipLaunchKernelGGL((gemm_kernel<MODE, 1, 4, 1, 1>), grid, block, 0, device->stream, p);
-    } else if (shape == TILE_64x64) {
-        dim3 grid(rlt_div_up(p.N, 64), rlt_div_up(p.M, 64), splits);
-        hipLaunchKernelGGL((gemm_kernel<MODE, 2, 2, 1, 1>), grid, block, 0, device->stream, p);
-    } else {
-        dim3 grid(rlt_div_up(p.N, 128), rlt_div_up(p.M, 128), splits);
-        hipLaunchKernelGGL((gemm_kernel<MODE, 2, 2, 2, 2>), grid, block, 0, device->stream, p);
+    TileShape shape = pick_tile(p.M, p.N, MODE);
+    int bm, bn;
+    tile_dims(shape, bm, bn);
+    // a grid of large tiles that leaves compute units idle runs faster as 64x64 tiles (no split over k to fill the chip here)
+    if (MODE != 2 && bm >= 128 && bn >= 64 && rlt_div_up(p.N, bn) * rlt_div_up(p.M, bm) < device->compute_units) { shape = TILE_64x64; tile_dims(shape, bm, bn); }
+    const dim3 grid(rlt_div_up(p.N, bn), rlt_div_up(p.M, bm), splits);
+    switch (shape) {
+        case TILE_128x32: hipLaunchKernelGGL((gemm_kernel<MODE, 4, 1, 1, 1>), grid, block, 0, device->stream, p); break;
+        case TILE_32x128: hipLaunchKernelGGL((gemm_kernel<MODE, 1, 4, 1, 1>), grid, block, 0, device->stream, p); break;
+        case TILE_64x64: hipLaunchKernelGGL((gemm_kernel<MODE, 2, 2, 1, 1>), grid, block, 0, device->stream, p); break;
+        case TILE_128x64: hipLaunchKernelGGL((gemm_kernel<MODE, 2, 2, 2, 1>), grid, block, 0, device->stream, p); break;
+        default: hipLaunchKernelGGL((gemm_kernel<MODE, 2, 2, 2, 2>), grid, block, 0, device->stream, p); break;
     }
     return rlt_launch_status(device);
 }
@@ -292,7 +326,7 @@ int rlt_gemm_forward(rlt_rocm_device* device, const float* x, int ldx, const flo
     if (rlt_div_up(batch, 32) > 65535) return RLT_E_UNSUPPORTED;
     GemmParams p = {};
     p.A = x; p.lda = ldx; p.B = W; p.ldb = in_dim; p.M = batch; p.N = out_dim; p.K = in_dim; p.k_per_split = in_dim;
-    p.vecA = aligned16(x) && (ldx % 4 == 0); p.vecB = aligned16(W) && (in_dim % 4 == 0);
+    p.vecA = vector_width(x, ldx); p.vecB = vector_width(W, in_dim);
     p.bias = bias; p.act = act; p.pre = pre; p.out = out; p.y = y; p.ldy = ldy; p.splits = 1;
     return launch<0>(device, p, 1);
 }
@@ -302,7 +336,7 @@ int rlt_gemm_backward_input(rlt_rocm_device* device, const float* d_pre, int ldd
     if (rlt_div_up(batch, 32) > 65535) return RLT_E_UNSUPPORTED;
     GemmParams p = {};
     p.A = d_pre; p.lda = ldd; p.B = W; p.ldb = in_dim; p.M = batch; p.N = in_dim; p.K = out_dim; p.k_per_split = out_dim;
-    p.vecA = aligned16(d_pre) && (ldd % 4 == 0); p.vecB = aligned16(W) && (in_dim % 4 == 0);
+    p.vecA = vector_width(d_pre, ldd); p.vecB = vector_width(W, in_dim);
     p.C = d_in; p.ldc = ldi; p.dact_pre = dact_pre; p.dact_kind = dact_kind; p.dact_from_output = dact_from_output; p.splits = 1;
     return launch<1>(device, p, 1);
 }
@@ -310,9 +344,8 @@ int rlt_gemm_backward_input(rlt_rocm_device* device, const float* d_pre, int ldd
 // How the weight-gradient contraction splits the batch so that the grid fills the chip: about 2 workgroups per compute unit, at least
 // 256 rows per split. Each split writes one block of out_dim * in_dim + out_dim partial sums.
 static void wgrad_split(const rlt_rocm_device* device, int batch, int in_dim, int out_dim, int& splits, int& kps) {
-    const TileShape shape = pick_tile(out_dim, in_dim);
-    int bm = shape == TILE_128x32 ? 128 : (shape == TILE_32x128 ? 32 : (shape == TILE_64x64 ? 64 : 128));
-    int bn = shape == TILE_128x32 ? 32 : (shape == TILE_32x128 ? 128 : (shape == TILE_64x64 ? 64 : 128));
+    int bm, bn;
+    tile_dims(pick_tile(out_dim, in_dim, 2), bm, bn);
     int tiles = rlt_div_up(out_dim, bm) * rlt_div_up(in_dim, bn);
     splits = (2 * device->compute_units + tiles - 1) / tiles;
     int max_splits = rlt_div_up(batch, 256);
@@ -353,7 +386,7 @@ int rlt_gemm_wgrad(rlt_rocm_device* device, const float* d_pre, int ldd, const f
                    int batch, int in_dim, int out_dim, bool static_scratch) {
     GemmParams p = {};
     p.A = d_pre; p.lda = ldd; p.B = x; p.ldb = ldx; p.M = out_dim; p.N = in_dim; p.K = batch;
-    p.vecA = aligned16(d_pre) && (ldd % 4 == 0); p.vecB = aligned16(x) && (ldx % 4 == 0);
+    p.vecA = vector_width(d_pre, ldd); p.vecB = vector_width(x, ldx);
     p.dW = dW; p.dbias = dbias;
     int splits, kps;
     wgrad_split(device, batch, in_dim, out_dim, splits, kps);
