@@ -430,8 +430,10 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_opera
         finally:
             rocm.call("sac_set_per_operation", 0)
     else:                         # the persistent kernel: all `steps` loop steps in one launch
-        ticks = rocm.zeros((16,), np.uint64)
+        ticks, stage_ticks = rocm.zeros((16,), np.uint64), rocm.zeros((48,), np.uint64)
         outputs = capi.SacLoopOutputs(None, None, None, None, None, ticks.ptr if phase_profile else None)
+        if phase_profile == "stages":
+            outputs.stage_ticks = stage_ticks.ptr
         ev = HipEvents(lib.rlt_rocm_get_stream(h))
         done = [0]
 
@@ -440,7 +442,7 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_opera
             done[0] += n
         run(max(warmup, 1))
         rocm.sync()
-        ticks.upload(np.zeros(16, np.uint64))
+        ticks.upload(np.zeros(16, np.uint64)); stage_ticks.upload(np.zeros(48, np.uint64))
         # HIP events on the library's stream around launches of `steps` loop steps each, repeated until at least 5 ms are timed (a single
         # short launch would mostly measure the launch itself); everything the loop reads and writes is resident on the device
         launches = 0
@@ -466,6 +468,18 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_opera
             shader_cycles = tk[15] * 100.0; tk = tk[:15]; names = names[:15]
             print("phase profile (us per loop step, workgroup 0):", {f"{i}:{n}": round(float(v), 2) for i, (n, v) in enumerate(zip(names, tk))}, "sum", round(float(tk.sum()), 2),
                   "shader clock MHz", round(shader_cycles / tk.sum(), 1), file=sys.stderr, flush=True)
+            if phase_profile == "stages":
+                mhz = shader_cycles / tk.sum()
+                st = stage_ticks.numpy().astype(np.float64) / 100.0 / (total_steps + (20000 if long_run else 0)) * mhz      # shader cycles per loop step
+                stage_names = {0: "A layer 1 (actor on next obs | critic 1)", 2: "A layers 2+3", 4: "next action + log-probability (one wavefront)", 6: "B layer 1 (target critics)",
+                               8: "B layers 2+3", 10: "TD target + D layer 1 (critic 0 | actor on obs)", 12: "D layers 2+3", 14: "d_output, actor sample (one wavefront each)",
+                               16: "critics backward: layer 3, gate of layer 2", 18: "critics backward: dW2, layer 1",
+                               20: "critics on new action: layer 1", 22: "layers 2+3", 24: "backward layer 3, gate", 26: "backward layer 1 -> d action",
+                               28: "min-Q routing, sample_and_squash backward (one wavefront)", 30: "actor backward: layer 3, gate", 32: "actor backward: dW2 | layer 1, target polyak in LDS"}
+                print("stage profile (shader cycles per loop step, thread 0 of workgroup 0): stage's own instructions / wait at the barrier behind it", file=sys.stderr)
+                for i in sorted(stage_names):
+                    print("  %2d %-70s %7.0f  / %5.0f" % (i, stage_names[i], st[i], st[i + 1] if i + 1 < 48 and i not in (18, 32) else 0.0), file=sys.stderr)
+                print("  critic phase stages sum %.0f cycles, actor phase stages sum %.0f cycles" % (st[:19].sum(), st[20:33].sum()), file=sys.stderr, flush=True)
     p = agent.parameters()
     assert np.all(np.isfinite(p)), "SAC parameters went non-finite"
     # what the run has learned (untimed): 100 evaluation episodes of 200 steps with the actor as it stands after warmup + steps loop steps from random weights
@@ -642,7 +656,8 @@ def main():
     ap.add_argument("--mlp-iters", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", choices=["all", "mlp", "sac", "env", "ppo", "gru", "seq", "api"], default="all")
-    ap.add_argument("--sac-phase-profile", action="store_true", help="print the persistent kernel's per-phase time (stderr)")
+    ap.add_argument("--sac-phase-profile", nargs="?", const="phases", default=None, choices=["phases", "stages"],
+                    help="print the persistent kernel's per-phase time (stderr); 'stages' adds the clock between the barrier-separated stages of the critic and actor phases")
     ap.add_argument("--pmc-probe", action="store_true", help="for counter runs under rocprofv3 --pmc: three 256 MiB device copies (a kernel of known traffic, to scale the counters by) "
                     "three MLP forward+backward calls, then the environment-pipeline and PPO workloads (their figures discarded)")
     ap.add_argument("--sac-per-operation", action="store_true", help="time the one-launch-per-operation SAC path instead of the persistent kernel")

@@ -539,6 +539,11 @@ typedef struct rlt_sac_loop_outputs {  /* all optional */
     uint32_t* drawn_sample_offsets;    /* [n_steps x batch]                                                               */
     float* drawn_noise_critic;         /* [n_steps x batch]                                                               */
     float* drawn_noise_actor;          /* [n_steps x batch]                                                               */
+    uint64_t* stage_ticks;             /* [48] profiling aid, ADDED to what is there: the same clock as phase_ticks, read by thread 0 of
+                                          workgroup 0 after every stage and after every workgroup barrier of the critic phase (slots 0-18:
+                                          even = a stage's own instructions, odd = the wait at the barrier behind it) and of the actor
+                                          phase (slots 20-32). Reading the clock waits for the wavefront's outstanding LDS traffic, so a
+                                          run with this output set is a few percent slower than one without.                         */
 } rlt_sac_loop_outputs;
 
 /* n_steps iterations of sac::loop::core::step (rl/algorithms/sac/loop/core/operations_generic.h:110-155, past the warm-up:

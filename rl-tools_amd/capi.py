@@ -125,7 +125,7 @@ class SacLoopOutputs(C.Structure):
     _fields_ = [("critic_loss", C.c_void_p), ("observations_actions_base", C.c_void_p), ("rewards", C.c_void_p), ("terminated", C.c_void_p),
                 ("target_action_value", C.c_void_p), ("phase_ticks", C.c_void_p),
                 ("drawn_rollout_noise", C.c_void_p), ("drawn_initial_states", C.c_void_p), ("drawn_sample_offsets", C.c_void_p),
-                ("drawn_noise_critic", C.c_void_p), ("drawn_noise_actor", C.c_void_p)]
+                ("drawn_noise_critic", C.c_void_p), ("drawn_noise_actor", C.c_void_p), ("stage_ticks", C.c_void_p)]
 
 
 class SacLoopScratch(C.Structure):

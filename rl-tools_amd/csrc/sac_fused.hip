@@ -111,6 +111,7 @@ struct FusedArgs {
     // batch views for inspection (optional): last gathered batch / targets
     float* out_oab; float* out_rewards; uint8_t* out_terminated; float* out_target;
     unsigned long long* phase_ticks;   // [16] optional: constant-rate clock ticks workgroup 0 spent in each phase, summed over the steps
+    unsigned long long* stage_ticks;   // [48] optional: the same clock between the barrier-separated stages of the critic and actor phases (thread 0)
     // optional: the draws every step used (host-drawn or the kernel's own), so that a run can be replayed elsewhere
     float* drawn_rollout; float* drawn_initial; uint32_t* drawn_offsets; float* drawn_noise_c; float* drawn_noise_a;
 };
@@ -438,6 +439,7 @@ struct Shared {
     float dout_actor_critic[ROWS * 2];   // -1/batch: the gradient the actor loss puts on both critics' outputs
     float new_row[16];            // the transition added this step
     unsigned long long ticks[16]; // per-phase clock ticks of this workgroup (profiling aid), flushed at the end
+    unsigned long long sticks[48]; // per-stage clock ticks (profiling aid)
     int abort;                    // a wait for another workgroup failed: leave the step loop
     float alpha;                  // exp(log_alpha) of this step
     float rollout_eps[2];         // exploration noise of this step and the next (indexed by step parity)
@@ -497,6 +499,12 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
     const unsigned long long shader_clock_begin = A.phase_ticks ? clock64() : 0ull;
     auto tick = [&](int phase) {
         if (A.phase_ticks && g == 0 && threadIdx.x == 0) { const unsigned long long t = wall_clock64(); S->ticks[phase] += t - t_prev; t_prev = t; }
+    };
+    // finer clock for the stage profile: stage_begin() restarts it, stage(i) adds the time since the last call to slot i
+    unsigned long long s_prev = 0ull;
+    auto stage_begin = [&]() { if (A.stage_ticks && g == 0 && threadIdx.x == 0) s_prev = wall_clock64(); };
+    auto stage = [&](int i) {
+        if (A.stage_ticks && g == 0 && threadIdx.x == 0) { const unsigned long long t = wall_clock64(); S->sticks[i] += t - s_prev; s_prev = t; }
     };
     const int lane_invariant = lane, wave_base = wave << 6;
     for (int step = 0; step < A.n_steps; step++) {
@@ -627,17 +635,22 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         else if (tid < ROWS * 16 + 2 * ROWS) S->noise_a[tid & 15] = noise_reg;
         rlt_lds_barrier();
         tick(11);
+        stage_begin();
         // A: group 0 evaluates the actor on the next observations; group 1 meanwhile runs critic 1's training forward
         {
             Fwd1W f1; Fwd2W f2;
             if (grp == 0) { f1 = load_fwd1<NA>(w_actor, w, lane); f2 = load_fwd2<NA>(w_actor, w, lane); }
             else { f1 = load_fwd1<NC>(w_critic1, w, lane); f2 = load_fwd2<NC>(w_critic1, w, lane); }
             forward_stage1(grp == 0 ? Snx : Sx, grp == 0 ? Le1 : La1, f1, w, lane);
+            stage(0);
             rlt_lds_barrier();
+            stage(1);
             if (grp == 0) forward_stage2<2>(Le1, Le2, Lpart, f2, w, lane); else forward_stage2<1>(La1, La2, Lpart, f2, w, lane);
         }
         const Fwd1W t1 = load_fwd1<NC>(w_target, w, lane); const Fwd2W t2 = load_fwd2<NC>(w_target, w, lane);
+        stage(2);
         rlt_lds_barrier();
+        stage(3);
         if (wave == 0 && lane < ROWS) {   // sample_and_squash evaluate with the external noise -> next action, its log-probability
             const float mean = net_output<NA>(part0, w_actor, lane, 0);
             const float ls = clampf(net_output<NA>(part0, w_actor, lane, 1), A.sas.log_std_lower_bound, A.sas.log_std_upper_bound);
@@ -648,19 +661,25 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             Snx[lane * XS + OBS] = act;
         }
         if (wave == 4 && lane < ROWS) S->q[1][lane] = net_output<NC>(part1, w_critic1, lane, 0);
+        stage(4);
         rlt_lds_barrier();
         tick(12);
+        stage(5);
         // B: target critic k on [next_obs | next_action] by group k
         forward_stage1(Snx, Le1, t1, w, lane);
+        stage(6);
         rlt_lds_barrier();
+        stage(7);
         forward_stage2<1>(Le1, Le2, Lpart, t2, w, lane);
         // D (weights): group 0 runs critic 0's training forward (critic 1's is already there), group 1 the actor on the batch
         // observations, whose result the actor phase needs (x rows are [obs | action]; the actor's weights for the action column are zero)
         Fwd1W d1; Fwd2W d2;
         if (grp == 0) { d1 = load_fwd1<NC>(w_critic0, w, lane); d2 = load_fwd2<NC>(w_critic0, w, lane); }
         else { d1 = load_fwd1<NA>(w_actor, w, lane); d2 = load_fwd2<NA>(w_actor, w, lane); }
+        stage(8);
         rlt_lds_barrier();
         tick(13);
+        stage(9);
         // C: TD target (sac/operations_generic.h:133-179)
         if (wave == 0 && lane < ROWS) {
             const float alpha = S->alpha;
@@ -671,11 +690,15 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         }
         // D
         forward_stage1(Sx, grp == 0 ? La1 : Ah1, d1, w, lane);
+        stage(10);
         rlt_lds_barrier();
+        stage(11);
         if (grp == 0) forward_stage2<1>(La1, La2, Lpart, d2, w, lane); else forward_stage2<2>(Ah1, Ah2, Lpart, d2, w, lane);
         const Bwd1W cb1 = load_bwd1<NC>(w_critic, w, lane); const Bwd2W cb2 = load_bwd2<NC>(w_critic, w, lane);
+        stage(12);
         rlt_lds_barrier();
         tick(14);
+        stage(13);
         if (w == 0 && lane < ROWS) {
             // d_output = (Q - y) * 2/B * loss_weight, loss_weight = B*0.5 / num_final_steps = 0.5 (sac/operations_generic.h:298-312)
             float q;
@@ -691,9 +714,13 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             for (int j = 0; j < OBS; j++) Snx[lane * XS + j] = Sx[lane * XS + j];   // [obs | new action] rows for the critics of the actor phase
             Snx[lane * XS + OBS] = act;
         }
+        stage(14);
         rlt_lds_barrier();
+        stage(15);
         backward_stage1<NC, true, PACKED>(La2, Ldp2, Ldout, cb1, my_partial + grp * NC::total, w, lane);
+        stage(16);
         rlt_lds_barrier();
+        stage(17);
         backward_w2<NC, PACKED>(La1, Ldp2, my_partial + grp * NC::total, w, lane);
         backward_l1<NC, true, false, PACKED>(Sx, La1, Ldp2, Lpart, cb2, my_partial + grp * NC::total, w, lane);
         if (A.out_critic_loss && w == 0) {      // sum of squared TD errors of this workgroup's rows
@@ -701,6 +728,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             d = kk_sum(row16_sum(d * d));
             if (lane == 0) put_shared<PACKED>(my_partial + 2 * NC::total + NA::total + 1 + grp, d);
         }
+        stage(18);
         tick(1);
         announce<PACKED>(A.ready, READY_CRITIC_GRADIENTS, g, seq);
         tick(2);
@@ -752,25 +780,34 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         }
         rlt_lds_barrier();
         tick(5);
+        stage_begin();
         // ================= S3: actor phase =================
         // (the actor's forward on the batch observations and its sample_and_squash forward were done in the critic phase)
         // critic k forward + backward_input on [obs | new action] by group k
         {
             const Fwd1W f1 = load_fwd1<NC>(w_critic, w, lane); const Fwd2W f2 = load_fwd2<NC>(w_critic, w, lane);
             forward_stage1(Snx, Le1, f1, w, lane);
+            stage(20);
             rlt_lds_barrier();
+            stage(21);
             forward_stage2<1>(Le1, Le2, Lpart, f2, w, lane);
         }
         {
             const Bwd1W b1 = load_bwd1<NC>(w_critic, w, lane); const Bwd2W b2 = load_bwd2<NC>(w_critic, w, lane);
+            stage(22);
             rlt_lds_barrier();
+            stage(23);
             if (w == 0 && lane < ROWS) S->q[grp][lane] = net_output<NC>(Lpart, w_critic, lane, 0);
             backward_stage1<NC, false, PACKED>(Le2, Ldp2, &S->dout_actor_critic[0], b1, nullptr, w, lane);
+            stage(24);
             rlt_lds_barrier();
+            stage(25);
             backward_l1<NC, false, true, PACKED>(Snx, Le1, Ldp2, Lpart, b2, nullptr, w, lane);
         }
         const Bwd1W ab1 = load_bwd1<NA>(w_actor, w, lane); const Bwd2W ab2 = load_bwd2<NA>(w_actor, w, lane);
+        stage(26);
         rlt_lds_barrier();
+        stage(27);
         // min-Q routing (sac/operations_generic.h:358-393), sample_and_squash backward (nn/layers/sample_and_squash/operations_generic.h:289-398)
         if (wave == 0) {
             float alpha_term = 0.f;
@@ -795,17 +832,22 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             alpha_term = row16_sum(alpha_term);
             if (lane == 0) put_shared<PACKED>(my_partial + 2 * NC::total + NA::total, alpha_term);
         }
+        stage(28);
         rlt_lds_barrier();
+        stage(29);
         // actor backward: layer 3 and the layer-2 gate by group 0, then the layer-2 weight gradient by group 0 and layer 1 by group 1
         const lptr dp2a = &S->grp[0].dp2[0];
         if (grp == 0) backward_stage1<NA, true, PACKED>(Ah2, dp2a, &S->actor_dout[0], ab1, my_partial + 2 * NC::total, w, lane);
+        stage(30);
         rlt_lds_barrier();
+        stage(31);
         if (grp == 0) backward_w2<NA, PACKED>(Ah1, dp2a, my_partial + 2 * NC::total, w, lane);
         else backward_l1<NA, true, false, PACKED>(Sx, Ah1, dp2a, Lpart, ab2, my_partial + 2 * NC::total, w, lane);
         {
             const lptr dst_t[2] = {w_target0, w_target1};
             polyak_nets<NC, 2>(dst_t, fresh, A.polyak, tid);     // read next after several barriers
         }
+        stage(32);
         tick(6);
         announce<PACKED>(A.ready, READY_ACTOR_GRADIENTS, g, seq);
         await(A.ready, READY_ACTOR_GRADIENTS, G, seq, A.fault, &S->abort);
@@ -848,6 +890,8 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         S->ticks[15] = clock64() - shader_clock_begin;     // shader clock cycles of the whole run: with the sum of the others it gives the clock rate
         for (int i = 0; i < 16; i++) A.phase_ticks[i] += S->ticks[i];
     }
+    if (A.stage_ticks && g == 0 && tid == 0)
+        for (int i = 0; i < 48; i++) A.stage_ticks[i] += S->sticks[i];
     // the placement on one XCD is what makes plain stores visible to the other workgroups: a run that was placed otherwise is void
     if (PACKED && g == 0 && tid == 0) {
         const unsigned mask = __hip_atomic_load(A.xcd_mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -936,7 +980,7 @@ extern "C" int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac
                   a.noise_critic = inputs->noise_critic; a.noise_actor = inputs->noise_actor; }
     a.seed = seed; a.step_offset = step_offset;
     if (outputs) { a.out_critic_loss = outputs->critic_loss; a.out_oab = outputs->observations_actions_base; a.out_rewards = outputs->rewards;
-                   a.out_terminated = outputs->terminated; a.out_target = outputs->target_action_value; a.phase_ticks = (unsigned long long*)outputs->phase_ticks;
+                   a.out_terminated = outputs->terminated; a.out_target = outputs->target_action_value; a.phase_ticks = (unsigned long long*)outputs->phase_ticks; a.stage_ticks = (unsigned long long*)outputs->stage_ticks;
                    a.drawn_rollout = outputs->drawn_rollout_noise; a.drawn_initial = outputs->drawn_initial_states; a.drawn_offsets = outputs->drawn_sample_offsets;
                    a.drawn_noise_c = outputs->drawn_noise_critic; a.drawn_noise_a = outputs->drawn_noise_actor; }
     const size_t lds_floats = ((sizeof(Shared) / 4 + 3) & ~(size_t)3) + (size_t)(NA::ltotal + 4 * NC::ltotal);
