@@ -843,13 +843,13 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         stage(31);
         if (grp == 0) backward_w2<NA, PACKED>(Ah1, dp2a, my_partial + 2 * NC::total, w, lane);
         else backward_l1<NA, true, false, PACKED>(Sx, Ah1, dp2a, Lpart, ab2, my_partial + 2 * NC::total, w, lane);
-        {
-            const lptr dst_t[2] = {w_target0, w_target1};
-            polyak_nets<NC, 2>(dst_t, fresh, A.polyak, tid);     // read next after several barriers
-        }
         stage(32);
         tick(6);
         announce<PACKED>(A.ready, READY_ACTOR_GRADIENTS, g, seq);
+        {   // the target critics' soft update on the LDS copies, while the other workgroups' gradients arrive (read next after several barriers)
+            const lptr dst_t[2] = {w_target0, w_target1};
+            polyak_nets<NC, 2>(dst_t, fresh, A.polyak, tid);
+        }
         await(A.ready, READY_ACTOR_GRADIENTS, G, seq, A.fault, &S->abort);
         tick(7);
         // ================= S4: reduce + Adam for the actor and log_alpha =================
