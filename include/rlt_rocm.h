@@ -556,6 +556,42 @@ int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac_agent* age
                                const rlt_replay_buffer* rb, int n_steps, uint64_t seed, uint64_t step_offset,
                                const rlt_sac_loop_inputs* inputs, const rlt_sac_loop_outputs* outputs);
 
+/* The off-policy runner over any of the batched environments (rl/components/off_policy_runner/off_policy_runner.h:184-221 runner state,
+ * :158-183 Buffers). env_kind selects the environment and with it the widths:
+ *   RLT_ENV_PENDULUM          state 2, observation 3, action 1   (parameters: pendulum)
+ *   RLT_ENV_ACROBOT           state 4, observation 6, action 1   (parameters: acrobot)
+ *   RLT_ENV_ACROBOT_SWINGUP   state 4, observation 6, action 1   (parameters: acrobot)
+ *   RLT_ENV_CAR               state 6, observation 6, action 2   (parameters: car) */
+enum { RLT_ENV_PENDULUM = 0, RLT_ENV_ACROBOT = 1, RLT_ENV_ACROBOT_SWINGUP = 2, RLT_ENV_CAR = 3 };
+typedef struct rlt_env_runner {
+    int32_t env_kind, n_envs, episode_step_limit, reserved;
+    float* states;              /* [n_envs x state_dim] */
+    uint32_t* episode_step;     /* [n_envs] */
+    float* episode_return;      /* [n_envs] */
+    uint8_t* truncated;         /* [n_envs] initialised to 1 */
+    rlt_pendulum_parameters pendulum; rlt_acrobot_parameters acrobot; rlt_car_parameters car;    /* the one env_kind names is read */
+    /* the runner's per-step buffers, written by every step */
+    float* observations;        /* [n_envs x observation_dim] */
+    float* actions;             /* [n_envs x action_dim] */
+    float* next_observations;   /* [n_envs x observation_dim] */
+    float* rewards;             /* [n_envs] */
+    uint8_t* terminated;        /* [n_envs] */
+} rlt_env_runner;
+/* widths of an environment kind; each pointer may be NULL. RLT_E_INVALID_ARGUMENT for an unknown kind. */
+int rlt_rocm_env_dims(int env_kind, int* state_dim, int* observation_dim, int* action_dim);
+size_t rlt_rocm_env_runner_step_workspace_bytes(const rlt_env_runner* runner, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers);
+/* step<POLICY>(device, runner, policy, ...)   rl/components/off_policy_runner/operations_generic.h:183-238, operations_generic_per_env.h:8-108
+ *   prologue: environments whose `truncated` flag is set start again from initial_states [n_envs x state_dim] (what sample_initial_state
+ *   would draw; consumed only where a reset happens; the caller draws them, e.g. rlt_rocm_rand_f32 over (-0.1, 0.1) for the Acrobot), their
+ *   counters are cleared and the last row of their replay ring is marked truncated; observe.  interlude: the policy, as in
+ *   rlt_rocm_pendulum_runner_step (policy_kind 0 actions_in [n_envs x action_dim], 1 MLP -> action, 2 MLP -> [mean | log_std] + sample_and_squash
+ *   with action_noise [n_envs x action_dim]).  epilogue: environment step, reward, next observation, terminated; episode_step += 1,
+ *   episode_return += reward, truncated = terminated or episode_step == episode_step_limit; replay add. Five to seven launches. */
+int rlt_rocm_env_runner_step(rlt_rocm_device* device, const rlt_env_runner* runner, const rlt_replay_buffer* rb, int policy_kind,
+                             const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas,
+                             const float* actions_in, const float* action_noise, const float* initial_states,
+                             void* workspace, size_t workspace_bytes);
+
 /* Device buffers that rlt_rocm_sac_pendulum_loop_by_calls draws into. */
 typedef struct rlt_sac_loop_scratch {
     float* rollout_noise;       /* [n_envs x action_dim] */

@@ -1031,6 +1031,72 @@ int rlt_oracle_pendulum_runner_step(const rlt_pendulum_runner* rn, const rlt_rep
     return rlt_oracle_pendulum_runner_epilogue(rn, rb, obs.data(), actions.data());
 }
 
+// step<POLICY>(device, runner, policy, ...) for any of the environments restated here: rl/components/off_policy_runner/operations_generic.h:183-238 over
+// prologue_per_env / epilogue_per_env (operations_generic_per_env.h:8-108). The environment-independent part (reset bookkeeping, counters,
+// truncated = terminated or step limit, replay add) is the Pendulum runner's, which the seeded SAC loop pins against the reference; the
+// environments' own step / reward / observe / terminated are the functions above, pinned one by one.
+static int env_dims_of(int kind, int* state, int* obs, int* act) {
+    switch (kind) {
+        case RLT_ENV_PENDULUM: *state = 2; *obs = 3; *act = 1; return 0;
+        case RLT_ENV_ACROBOT: case RLT_ENV_ACROBOT_SWINGUP: *state = 4; *obs = 6; *act = 1; return 0;
+        case RLT_ENV_CAR: *state = 6; *obs = 6; *act = 2; return 0;
+        default: return RLT_E_INVALID_ARGUMENT;
+    }
+}
+static int env_step_of(const rlt_env_runner* rn, float* states, const float* actions, float* observations, float* next_observations, float* rewards, uint8_t* terminated) {
+    const int N = rn->n_envs;
+    switch (rn->env_kind) {
+        case RLT_ENV_PENDULUM: {
+            if (terminated) for (int e = 0; e < N; e++) terminated[e] = 0;
+            return rlt_oracle_pendulum_step(&rn->pendulum, states, actions, observations, next_observations, rewards, N);
+        }
+        case RLT_ENV_CAR: return rlt_oracle_car_step(&rn->car, states, actions, observations, next_observations, rewards, terminated, N);
+        default: return rlt_oracle_acrobot_step(&rn->acrobot, rn->env_kind == RLT_ENV_ACROBOT_SWINGUP, states, actions, observations, next_observations, rewards, terminated, N);
+    }
+}
+int rlt_oracle_env_runner_step(const rlt_env_runner* rn, const rlt_replay_buffer* rb, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers,
+                               const rlt_sas_parameters* sas, const float* actions_in, const float* action_noise, const float* initial_states) {
+    int SD, OBS, ACT;
+    if (!rn || !rb || !initial_states || env_dims_of(rn->env_kind, &SD, &OBS, &ACT) || rn->n_envs != rb->n_envs || rb->observation_dim != OBS || rb->action_dim != ACT)
+        return RLT_E_INVALID_ARGUMENT;
+    const int N = rn->n_envs, R = rb_row_dim(rb);
+    // prologue
+    for (int e = 0; e < N; e++)
+        if (rn->truncated[e]) {
+            for (int i = 0; i < SD; i++) rn->states[(size_t)e * SD + i] = initial_states[(size_t)e * SD + i];
+            rn->episode_step[e] = 0; rn->episode_return[e] = 0;
+            if (rb->full[e] || rb->position[e] > 0) {
+                const uint32_t prev = rb->position[e] == 0 ? (uint32_t)rb->capacity - 1 : rb->position[e] - 1;
+                rb->data[((size_t)e * rb->capacity + prev) * R + (R - 1)] = 1.0f;
+                rb->current_episode_start[e] = rb->position[e];
+            }
+        }
+    {   // observe: the environment's own step function on a copy of the states yields the observation of the state it was given
+        std::vector<float> scratch_states(rn->states, rn->states + (size_t)N * SD), zero_actions((size_t)N * ACT, 0.0f);
+        int rc = env_step_of(rn, scratch_states.data(), zero_actions.data(), rn->observations, nullptr, nullptr, nullptr);
+        if (rc) return rc;
+    }
+    // interlude
+    int rc = 0;
+    if (policy_kind == 0) { if (!actions_in) return RLT_E_INVALID_ARGUMENT; for (size_t i = 0; i < (size_t)N * ACT; i++) rn->actions[i] = actions_in[i]; }
+    else if (policy_kind == 1) rc = rlt_oracle_mlp_evaluate(actor, n_actor_layers, rn->observations, OBS, rn->actions, ACT, N);
+    else if (policy_kind == 2) {
+        std::vector<float> out((size_t)N * 2 * ACT), lp(N);
+        rc = rlt_oracle_mlp_evaluate(actor, n_actor_layers, rn->observations, OBS, out.data(), 2 * ACT, N);
+        if (!rc) rc = rlt_oracle_sas_forward(sas, out.data(), 2 * ACT, action_noise, ACT, rn->actions, ACT, nullptr, 0, lp.data(), N, ACT);
+    } else return RLT_E_INVALID_ARGUMENT;
+    if (rc) return rc;
+    // epilogue
+    if ((rc = env_step_of(rn, rn->states, rn->actions, nullptr, rn->next_observations, rn->rewards, rn->terminated))) return rc;
+    std::vector<uint8_t> trunc(N, 0);
+    for (int e = 0; e < N; e++) {
+        rn->episode_step[e] += 1; rn->episode_return[e] += rn->rewards[e];
+        trunc[e] = rn->terminated[e] || rn->episode_step[e] == (uint32_t)rn->episode_step_limit;
+        rn->truncated[e] = trunc[e];
+    }
+    return rlt_oracle_replay_add(rb, rn->observations, rn->actions, rn->rewards, rn->next_observations, rn->terminated, trunc.data());
+}
+
 // rl::utils::evaluation::evaluate (rl/utils/evaluation/operations_generic.h:106-233) with the Pendulum environment: n_episodes environments from the
 // given initial states (what sample_initial_state drew, :139-142), step_limit steps of observe -> policy in Evaluation mode -> step -> reward;
 // an episode stops counting once it has terminated (:188-197; Pendulum never terminates, pendulum/operations_generic.h:161-164). The statistics

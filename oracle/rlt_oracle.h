@@ -165,6 +165,8 @@ int rlt_oracle_gather_sequence_batch(const rlt_replay_buffer* rb, const rlt_sequ
 int rlt_oracle_gather_sequence_batch_with_rng(const rlt_replay_buffer* rb, const rlt_sequence_sampling* sampling, int max_episode_length, const rlt_sequence_batch* batch,
                                               char* rng_state, int rng_capacity, uint32_t* env_indices, uint32_t* sample_offsets, uint8_t* nominal, uint32_t* lengths);
 /* rl/environments/acrobot/operations_generic.h:56-193 */
+int rlt_oracle_env_runner_step(const rlt_env_runner* runner, const rlt_replay_buffer* rb, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers,
+                               const rlt_sas_parameters* sas, const float* actions_in, const float* action_noise, const float* initial_states);
 int rlt_oracle_acrobot_step(const rlt_acrobot_parameters* p, int swingup, float* states, const float* actions, float* observations, float* next_observations,
                             float* rewards, uint8_t* terminated, int n_envs);
 /* rl/environments/car/operations_generic.h:80-155 (the Car without a track) */

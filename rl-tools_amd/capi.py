@@ -116,6 +116,17 @@ class PendulumRunner(C.Structure):
                 ("n_envs", C.c_int32), ("episode_step_limit", C.c_int32), ("env", PendulumParameters)]
 
 
+ENV_PENDULUM, ENV_ACROBOT, ENV_ACROBOT_SWINGUP, ENV_CAR = 0, 1, 2, 3
+ENV_DIMS = {ENV_PENDULUM: (2, 3, 1), ENV_ACROBOT: (4, 6, 1), ENV_ACROBOT_SWINGUP: (4, 6, 1), ENV_CAR: (6, 6, 2)}      # state, observation, action widths
+
+
+class EnvRunner(C.Structure):
+    _fields_ = [("env_kind", C.c_int32), ("n_envs", C.c_int32), ("episode_step_limit", C.c_int32), ("reserved", C.c_int32),
+                ("states", C.c_void_p), ("episode_step", C.c_void_p), ("episode_return", C.c_void_p), ("truncated", C.c_void_p),
+                ("pendulum", PendulumParameters), ("acrobot", AcrobotParameters), ("car", CarParameters),
+                ("observations", C.c_void_p), ("actions", C.c_void_p), ("next_observations", C.c_void_p), ("rewards", C.c_void_p), ("terminated", C.c_void_p)]
+
+
 class SacLoopInputs(C.Structure):
     _fields_ = [("rollout_noise", C.c_void_p), ("initial_states", C.c_void_p), ("sample_offsets", C.c_void_p), ("noise_critic", C.c_void_p),
                 ("noise_actor", C.c_void_p)]
@@ -266,6 +277,7 @@ PROTOTYPES = {
     "gather_sequence_batch": [C.POINTER(ReplayBuffer), C.POINTER(SequenceSampling), C.POINTER(SequenceDraws), I, C.POINTER(SequenceBatch)],
     "acrobot_step": [C.POINTER(AcrobotParameters), I, P, P, P, P, P, P, I],
     "car_step": [C.POINTER(CarParameters), P, P, P, P, P, P, I],
+    "env_runner_step": [C.POINTER(EnvRunner), C.POINTER(ReplayBuffer), I, LP, I, C.POINTER(SasParameters), P, P, P, P, S],
     "car_track_step": [C.POINTER(CarParameters), P, I, I, F, P, P, P, P, P, P, I],
     "pendulum_evaluate": [C.POINTER(PendulumParameters), I, LP, I, P, I, I, P, P, P],
     "ppo_gae": [P, P, P, P, P, P, I, I, I, F, F, I],
@@ -315,6 +327,8 @@ ROCM_ONLY = {
     "reduce_sum_f32": ([P, P, S, I, P], I),
     "dense_backward_static": ([P, LP, P, I, P, I, I], I),
     "sac_set_per_operation": ([P, I], I),
+    "env_dims": ([I, C.POINTER(I), C.POINTER(I), C.POINTER(I)], I),
+    "env_runner_step_workspace_bytes": ([C.POINTER(EnvRunner), I, LP, I], S),
     "mlp_workspace_bytes": ([LP, I, I], S),
     "ppo_workspace_bytes": ([C.POINTER(PpoAgent)], S),
     "gru_workspace_bytes": ([C.POINTER(GruLayer), I, I], S),

@@ -180,3 +180,130 @@ extern "C" int rlt_rocm_acrobot_step(rlt_rocm_device* device, const rlt_acrobot_
     hipLaunchKernelGGL(acrobot_step_kernel, dim3(blocks), dim3(256), 0, device->stream, *p, swingup, states, actions, observations, next_observations, rewards, terminated, n_envs);
     return rlt_launch_status(device);
 }
+
+// ---- the off-policy runner over any of these environments (rl/components/off_policy_runner/operations_generic_per_env.h:8-108)
+namespace {
+struct EnvDims { int state, obs, act; };
+__host__ __device__ inline EnvDims env_dims(int kind) {
+    switch (kind) {
+        case RLT_ENV_PENDULUM: return {2, 3, 1};
+        case RLT_ENV_ACROBOT: case RLT_ENV_ACROBOT_SWINGUP: return {4, 6, 1};
+        case RLT_ENV_CAR: return {6, 6, 2};
+        default: return {0, 0, 0};
+    }
+}
+// prologue_per_env (:8-62): reset where the last step truncated (state from the caller's draw, counters, the ring's last row marked truncated,
+// a new episode start), then observe
+__global__ __launch_bounds__(256) void env_prologue_kernel(rlt_env_runner rn, rlt_replay_buffer rb, const float* __restrict__ initial_states) {
+    const EnvDims d = env_dims(rn.env_kind);
+    const int R = 2 * rb.observation_dim + rb.action_dim + 3;
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) {
+        float* state = rn.states + (size_t)e * d.state;
+        if (rn.truncated[e]) {
+            for (int i = 0; i < d.state; i++) state[i] = initial_states[(size_t)e * d.state + i];
+            rn.episode_step[e] = 0; rn.episode_return[e] = 0.0f;
+            if (rb.full[e] || rb.position[e] > 0) {
+                const uint32_t prev = rb.position[e] == 0 ? (uint32_t)rb.capacity - 1 : rb.position[e] - 1;
+                rb.data[((size_t)e * rb.capacity + prev) * R + (R - 1)] = 1.0f;
+                rb.current_episode_start[e] = rb.position[e];
+            }
+        }
+        float* o = rn.observations + (size_t)e * d.obs;
+        if (rn.env_kind == RLT_ENV_PENDULUM) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; o[2] = state[1]; }
+        else if (rn.env_kind == RLT_ENV_CAR) { for (int i = 0; i < 6; i++) o[i] = state[i]; }
+        else { const Acrobot4 s4 = {{state[0], state[1], state[2], state[3]}}; acrobot_observe(s4, o); }
+    }
+}
+// the rest of epilogue_per_env after the environment's own step (:88-104): counters, truncation, replay add (replay_buffer/operations_generic.h:54-78)
+__global__ __launch_bounds__(256) void env_epilogue_kernel(rlt_env_runner rn, rlt_replay_buffer rb) {
+    const EnvDims d = env_dims(rn.env_kind);
+    const int OBS = d.obs, ACT = d.act, R = 2 * OBS + ACT + 3;
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) {
+        const float reward = rn.rewards[e];
+        const bool terminated = rn.terminated[e] != 0;
+        const uint32_t step = rn.episode_step[e] + 1;
+        rn.episode_step[e] = step;
+        rn.episode_return[e] += reward;
+        const bool truncated = terminated || step == (uint32_t)rn.episode_step_limit;
+        rn.truncated[e] = truncated;
+        uint32_t pos = rb.position[e];
+        float* row = rb.data + ((size_t)e * rb.capacity + pos) * R;
+        for (int i = 0; i < OBS; i++) row[i] = rn.observations[(size_t)e * OBS + i];
+        for (int i = 0; i < ACT; i++) row[OBS + i] = rn.actions[(size_t)e * ACT + i];
+        row[OBS + ACT] = reward;
+        for (int i = 0; i < OBS; i++) row[OBS + ACT + 1 + i] = rn.next_observations[(size_t)e * OBS + i];
+        row[R - 2] = terminated ? 1.0f : 0.0f; row[R - 1] = truncated ? 1.0f : 0.0f;
+        rb.episode_start[(size_t)e * rb.capacity + pos] = rb.current_episode_start[e];
+        pos = (pos + 1) % (uint32_t)rb.capacity;
+        rb.position[e] = pos;
+        if (truncated) rb.current_episode_start[e] = pos;
+        if (pos == 0 && !rb.full[e]) rb.full[e] = 1;
+    }
+}
+__global__ __launch_bounds__(256) void env_copy_kernel(const float* __restrict__ src, float* __restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+}  // namespace
+
+extern "C" int rlt_rocm_env_dims(int env_kind, int* state_dim, int* observation_dim, int* action_dim) {
+    const EnvDims d = env_dims(env_kind);
+    if (!d.state) return RLT_E_INVALID_ARGUMENT;
+    if (state_dim) *state_dim = d.state;
+    if (observation_dim) *observation_dim = d.obs;
+    if (action_dim) *action_dim = d.act;
+    return 0;
+}
+
+extern "C" size_t rlt_rocm_env_runner_step_workspace_bytes(const rlt_env_runner* rn, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers) {
+    if (!rn || rn->n_envs < 1) return 0;
+    const EnvDims d = env_dims(rn->env_kind);
+    const size_t head = align256((size_t)rn->n_envs * (2 * d.act + 1) * sizeof(float));      // actor output [n x 2 act], log-probabilities [n]
+    return head + (policy_kind ? rlt_rocm_mlp_workspace_bytes(actor, n_actor_layers, rn->n_envs) : 0) + 256;
+}
+
+extern "C" int rlt_rocm_env_runner_step(rlt_rocm_device* device, const rlt_env_runner* rn, const rlt_replay_buffer* rb, int policy_kind, const rlt_dense_layer* actor,
+                                        int n_actor_layers, const rlt_sas_parameters* sas, const float* actions_in, const float* action_noise, const float* initial_states,
+                                        void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(rn && rb && rn->n_envs > 0 && rn->states && rn->episode_step && rn->episode_return && rn->truncated && initial_states);
+    RLT_REQUIRE(rn->observations && rn->actions && rn->next_observations && rn->rewards && rn->terminated);
+    RLT_REQUIRE(rb->data && rb->episode_start && rb->position && rb->current_episode_start && rb->full && rb->capacity > 0);
+    const EnvDims d = env_dims(rn->env_kind);
+    RLT_REQUIRE(d.state && rn->n_envs == rb->n_envs && rb->observation_dim == d.obs && rb->action_dim == d.act && policy_kind >= 0 && policy_kind <= 2);
+    RLT_REQUIRE(policy_kind != 0 || actions_in);
+    RLT_REQUIRE(policy_kind == 0 || (actor && n_actor_layers >= 1 && actor[0].in_dim == d.obs && actor[n_actor_layers - 1].out_dim == (policy_kind == 2 ? 2 : 1) * d.act));
+    RLT_REQUIRE(policy_kind != 2 || (sas && action_noise));
+    RLT_REQUIRE(policy_kind == 0 || (workspace && workspace_bytes >= rlt_rocm_env_runner_step_workspace_bytes(rn, policy_kind, actor, n_actor_layers)));
+    const int N = rn->n_envs;
+    const int blocks = rlt_div_up(N, 256) > 1024 ? 1024 : rlt_div_up(N, 256);
+    int rc;
+    hipLaunchKernelGGL(env_prologue_kernel, dim3(blocks), dim3(256), 0, device->stream, *rn, *rb, initial_states);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if (policy_kind == 0) {
+        hipLaunchKernelGGL(env_copy_kernel, dim3(blocks), dim3(256), 0, device->stream, actions_in, rn->actions, (size_t)N * d.act);
+        if ((rc = rlt_launch_status(device))) return rc;
+    } else {
+        char* w = reinterpret_cast<char*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+        float* actor_out = (float*)w; float* log_probabilities = actor_out + (size_t)N * 2 * d.act;
+        const size_t head = align256((size_t)N * (2 * d.act + 1) * sizeof(float));
+        void* mlp_ws = w + head; const size_t mlp_ws_bytes = rlt_rocm_mlp_workspace_bytes(actor, n_actor_layers, N);
+        if (policy_kind == 1) { if ((rc = rlt_rocm_mlp_evaluate(device, actor, n_actor_layers, rn->observations, d.obs, rn->actions, d.act, N, mlp_ws, mlp_ws_bytes))) return rc; }
+        else {
+            if ((rc = rlt_rocm_mlp_evaluate(device, actor, n_actor_layers, rn->observations, d.obs, actor_out, 2 * d.act, N, mlp_ws, mlp_ws_bytes))) return rc;
+            if ((rc = rlt_rocm_sas_forward(device, sas, actor_out, 2 * d.act, action_noise, d.act, rn->actions, d.act, nullptr, 0, log_probabilities, N, d.act))) return rc;
+        }
+    }
+    switch (rn->env_kind) {
+        case RLT_ENV_PENDULUM:
+            if ((rc = rlt_rocm_pendulum_step(device, &rn->pendulum, rn->states, rn->actions, nullptr, rn->next_observations, rn->rewards, N))) return rc;
+            if ((rc = rlt_rocm_fill_u8(device, rn->terminated, (size_t)N, 0))) return rc;      // the Pendulum has no terminal states
+            break;
+        case RLT_ENV_CAR: if ((rc = rlt_rocm_car_step(device, &rn->car, rn->states, rn->actions, nullptr, rn->next_observations, rn->rewards, rn->terminated, N))) return rc; break;
+        default:
+            if ((rc = rlt_rocm_acrobot_step(device, &rn->acrobot, rn->env_kind == RLT_ENV_ACROBOT_SWINGUP, rn->states, rn->actions, nullptr, rn->next_observations, rn->rewards,
+                                            rn->terminated, N))) return rc;
+    }
+    hipLaunchKernelGGL(env_epilogue_kernel, dim3(blocks), dim3(256), 0, device->stream, *rn, *rb);
+    return rlt_launch_status(device);
+}

@@ -44,7 +44,7 @@ class LoopConfig(C.Structure):
 
 
 WITH_WORKSPACE = ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward", "on_policy_collect", "seq_forward", "seq_backward", "seq_evaluate_step",
-                  "pendulum_runner_step_recurrent", "pendulum_evaluate_recurrent")
+                  "pendulum_runner_step_recurrent", "pendulum_evaluate_recurrent", "env_runner_step")
 
 
 def load_oracle():
@@ -320,6 +320,34 @@ class ReplayOnBackend:
         self.full = backend.zeros((n_envs,), np.uint8)
         self.c = capi.ReplayBuffer(self.data.ptr, self.episode_start.ptr, self.position.ptr, self.current_episode_start.ptr, self.full.ptr,
                                    n_envs, capacity, obs_dim, act_dim)
+
+
+class EnvRunnerOnBackend:
+    """The off-policy runner's state and per-step buffers for any environment kind on one backend (all environments truncated at the start,
+    as the reference initialises them)."""
+
+    def __init__(self, backend, env_kind, n_envs, episode_step_limit):
+        self.backend, self.kind, self.n = backend, env_kind, n_envs
+        sd, od, ad = capi.ENV_DIMS[env_kind]
+        z = backend.zeros
+        self.states, self.ep_step, self.ep_ret = z((n_envs, sd)), z((n_envs,), np.uint32), z((n_envs,))
+        self.trunc = backend.array(np.ones(n_envs, np.uint8))
+        self.obs, self.act, self.next_obs, self.rew, self.term = z((n_envs, od)), z((n_envs, ad)), z((n_envs, od)), z((n_envs,)), z((n_envs,), np.uint8)
+        c = capi.EnvRunner()
+        c.env_kind, c.n_envs, c.episode_step_limit = env_kind, n_envs, episode_step_limit
+        c.states, c.episode_step, c.episode_return, c.truncated = self.states.ptr, self.ep_step.ptr, self.ep_ret.ptr, self.trunc.ptr
+        c.pendulum, c.acrobot, c.car = capi.pendulum_parameters(), capi.acrobot_parameters(), capi.car_parameters()
+        c.observations, c.actions, c.next_observations, c.rewards, c.terminated = self.obs.ptr, self.act.ptr, self.next_obs.ptr, self.rew.ptr, self.term.ptr
+        self.c = c
+
+    def workspace(self, policy_kind, actor):
+        if self.backend.name == "oracle" or policy_kind == 0:
+            return None, 0
+        lib = self.backend.device.lib
+        return self.backend.workspace(lib.rlt_rocm_env_runner_step_workspace_bytes(C.byref(self.c), policy_kind, actor.layers if actor else None, actor.n if actor else 0))
+
+    def snapshot(self):
+        return [a.numpy() for a in (self.states, self.ep_step, self.ep_ret, self.trunc, self.obs, self.act, self.next_obs, self.rew, self.term)]
 
 
 class SacOnBackend:

@@ -1,0 +1,78 @@
+"""The off-policy runner step over every batched environment (rl/components/off_policy_runner/operations_generic.h:183-238,
+operations_generic_per_env.h:8-108): the HIP path against the CPU checker over several hundred steps with resets, terminations, ring wrap and
+all three policy kinds. Index work, flags and copies bit-exact; floats to 1e-5 of each tensor's largest magnitude (1e-4 for the Acrobot's
+states after many Runge-Kutta steps, whose double-precision sub-expressions the kernel computes in float)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import helpers
+from helpers import capi, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def initial_states(rng, kind, n):
+    if kind == capi.ENV_PENDULUM:
+        return np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n)], 1).astype(np.float32)
+    if kind == capi.ENV_CAR:
+        s = np.zeros((n, 6), np.float32)
+        s[::4, 0] = 0.97; s[::4, 3] = 3.0      # some cars start at the edge of the unit square, heading out
+        return s
+    s = rng.uniform(-0.1, 0.1, (n, 4)).astype(np.float32)
+    if kind == capi.ENV_ACROBOT:
+        s[::5, 0] += 2.2      # some episodes start with the first link raised: their tip crosses the line within a few steps
+    return s
+
+
+@pytest.mark.parametrize("kind,policy_kind,n_envs,capacity,limit,steps", [
+    (capi.ENV_PENDULUM, 2, 37, 50, 20, 120),
+    (capi.ENV_ACROBOT, 0, 64, 40, 30, 100),            # terminates when the tip swings above the bar
+    (capi.ENV_ACROBOT_SWINGUP, 2, 130, 25, 12, 60),
+    (capi.ENV_CAR, 1, 50, 30, 25, 80),                 # terminates when the car leaves the unit square
+    (capi.ENV_CAR, 2, 1, 7, 5, 30),
+])
+def test_env_runner_step_matches_the_checker(oracle, rocm, kind, policy_kind, n_envs, capacity, limit, steps):
+    sd, od, ad = capi.ENV_DIMS[kind]
+    rng = np.random.default_rng(kind * 10 + policy_kind)
+    out = ad * (2 if policy_kind == 2 else 1)
+    params = helpers.random_params(rng, [od, 32, 32, out])
+    draws = [(initial_states(rng, kind, n_envs), rng.uniform(-1, 1, (n_envs, ad)).astype(np.float32), rng.standard_normal((n_envs, ad)).astype(np.float32)) for _ in range(steps)]
+    results = []
+    for backend in (oracle, rocm):
+        runner = helpers.EnvRunnerOnBackend(backend, kind, n_envs, limit)
+        rb = helpers.ReplayOnBackend(backend, n_envs, capacity, od, ad)
+        actor = helpers.Mlp(backend, [od, 32, 32, out], params, n_envs, "relu", "tanh" if policy_kind == 1 else "identity", trainable=False) if policy_kind else None
+        sas = capi.SasParameters(-20.0, 2.0, 1e-6, -float(ad))
+        ws, wsn = runner.workspace(policy_kind, actor)
+        trace = []
+        for ini, given, noise in draws:
+            i_d, g_d, n_d = backend.array(ini), backend.array(given), backend.array(noise)
+            backend.call("env_runner_step", C.byref(runner.c), C.byref(rb.c), policy_kind, actor.layers if actor else None, actor.n if actor else 0, C.byref(sas),
+                         g_d.ptr, n_d.ptr, i_d.ptr, ws, wsn)
+            backend.sync()
+            trace.append(runner.snapshot())
+        results.append((trace, [a.numpy() for a in (rb.data, rb.episode_start, rb.position, rb.current_episode_start, rb.full)]))
+    (ref_trace, ref_rb), (got_trace, got_rb) = results
+    tol = 1e-4 if kind in (capi.ENV_ACROBOT, capi.ENV_ACROBOT_SWINGUP) else 1e-5
+    n_term = n_reset = 0
+    for step, (ref, got) in enumerate(zip(ref_trace, got_trace)):
+        for k in (1, 3, 8):      # episode_step, truncated, terminated: exact
+            assert np.array_equal(got[k], ref[k]), (step, k)
+        for k in (0, 2, 4, 5, 6, 7):
+            assert rel_err(got[k], ref[k]) <= tol, (step, k, rel_err(got[k], ref[k]))
+        n_term += int(ref[8].sum()); n_reset += int(ref[3].sum())
+    assert n_reset > 0 and (kind in (capi.ENV_PENDULUM, capi.ENV_ACROBOT_SWINGUP) or n_term > 0)      # the cases exercise what they are for
+    assert rel_err(got_rb[0], ref_rb[0]) <= tol
+    for k in range(1, 5):
+        assert np.array_equal(got_rb[k], ref_rb[k])
+    assert ref_rb[4].all() or steps < capacity      # the rings wrapped
+
+
+def test_env_dims(rocm):
+    lib = rocm.device.lib
+    for kind, dims in capi.ENV_DIMS.items():
+        s, o, a = C.c_int(), C.c_int(), C.c_int()
+        assert lib.rlt_rocm_env_dims(kind, C.byref(s), C.byref(o), C.byref(a)) == 0 and (s.value, o.value, a.value) == dims
+    assert lib.rlt_rocm_env_dims(9, None, None, None) == capi.RLT_E_INVALID_ARGUMENT
