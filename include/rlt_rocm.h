@@ -985,6 +985,21 @@ int rlt_rocm_on_policy_collect(rlt_rocm_device* device, const rlt_pendulum_runne
                                const float* action_noise, const float* initial_states, int truncate_on_each_iteration,
                                void* workspace, size_t workspace_bytes);
 
+/* collect for any of the batched environments and any sequential policy (dense and GRU layers): rl/components/on_policy_runner/
+ * operations_generic.h:105-146 over operations_generic_per_env.h:8-74. Per step: reset(policy, policy_state) where the runner's truncated flag
+ * is set (before the prologue clears it, :127-130; skipped when policy_state is NULL), the prologue (environments whose flag is set start
+ * again from initial_states [steps x n_envs x state_dim], consumed only where a reset happens; observe into the dataset), evaluate_step of the
+ * policy in Rollout mode (after the optional standardize layer) giving the action means, the epilogue (action = mean + exp(log_std) * noise
+ * with action_noise [steps x n_envs x action_dim], its log-probability, the environment's step, reward and terminated flag, counters,
+ * truncated = terminated or episode_step >= episode_step_limit > 0, the delayed reset flag); at the end the final observation. The runner's
+ * per-step buffers (actions, rewards, terminated) are used as staging. A policy of dense layers only is an MLP policy. */
+size_t rlt_rocm_env_on_policy_collect_workspace_bytes(const rlt_env_runner* runner, const rlt_seq_layer* policy, int n_policy_layers);
+int rlt_rocm_env_on_policy_collect(rlt_rocm_device* device, const rlt_env_runner* runner, const rlt_on_policy_dataset* dataset,
+                                   const rlt_seq_layer* policy, int n_policy_layers, const rlt_seq_state* policy_state, int auto_reset_period,
+                                   const float* log_std, const float* standardize_mean, const float* standardize_precision,
+                                   const float* action_noise, const float* initial_states, int truncate_on_each_iteration,
+                                   void* workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1104,6 +1104,69 @@ int rlt_oracle_env_runner_step(const rlt_env_runner* rn, const rlt_replay_buffer
 //   policy_kind 1: the actor's output is the action;  2: the actor's output is [mean | log_std] and the action is tanh(mean), which is what
 //   sample_and_squash yields in Evaluation mode (noise = 0, nn/layers/sample_and_squash/operations_generic.h:149-195)
 //   summary = {returns_mean, returns_std, episode_length_mean, episode_length_std, num_terminated, share_terminated}
+// collect for any of the environments restated here and any sequential policy: rl/components/on_policy_runner/operations_generic.h:105-146 over
+// operations_generic_per_env.h:8-74 (see on_policy_collect_impl further down for the Pendulum / MLP case, which the reference's PPO loop pins)
+int rlt_oracle_env_on_policy_collect(const rlt_env_runner* rn, const rlt_on_policy_dataset* D, const rlt_seq_layer* policy, int n_policy_layers,
+                                     const rlt_seq_state* policy_state, int auto_reset_period, const float* log_std, const float* st_mean, const float* st_precision,
+                                     const float* action_noise, const float* initial_states, int truncate_on_each_iteration) {
+    int SD, OBS, ACT;
+    if (!rn || !D || !policy || n_policy_layers < 1 || !log_std || !action_noise || !initial_states || env_dims_of(rn->env_kind, &SD, &OBS, &ACT)) return RLT_E_INVALID_ARGUMENT;
+    const int N = rn->n_envs, S = D->steps_per_env, ld = D->ld;
+    const rlt_seq_state no_state = {};
+    const rlt_seq_state* step_state = policy_state ? policy_state : &no_state;
+    if (truncate_on_each_iteration) for (int e = 0; e < N; e++) rn->truncated[e] = 1;                                           // :112-114
+    for (int e = 0; e < N; e++) D->all_reset[(size_t)e * ld] = rn->truncated[e];                                                  // :115-117
+    std::vector<float> standardized((size_t)N * OBS), packed_obs((size_t)N * OBS), scratch_states((size_t)N * SD), zero_actions((size_t)N * ACT, 0.0f);
+    auto observe_into = [&](float* rows) {      // the environment's own step function on a copy of the states yields the observation of the state it was given
+        std::copy(rn->states, rn->states + (size_t)N * SD, scratch_states.begin());
+        int rc = env_step_of(rn, scratch_states.data(), zero_actions.data(), packed_obs.data(), nullptr, nullptr, nullptr);
+        for (int e = 0; e < N && !rc; e++) for (int i = 0; i < OBS; i++) rows[(size_t)e * ld + i] = packed_obs[(size_t)e * OBS + i];
+        return rc;
+    };
+    int rc;
+    for (int step = 0; step < S; step++) {
+        float* obs = D->observations + (size_t)step * N * ld;
+        float* means = D->actions_mean + (size_t)step * N * ld;
+        float* actions = D->actions + (size_t)step * N * ld;
+        if (policy_state && (rc = rlt_oracle_seq_reset_state(policy, n_policy_layers, policy_state, rn->truncated, N))) return rc;     // :127-130, before the prologue clears the flags
+        for (int e = 0; e < N; e++)                                                                                            // prologue, per_env :8-35
+            if (rn->truncated[e]) {
+                rn->truncated[e] = 0; rn->episode_step[e] = 0; rn->episode_return[e] = 0;
+                for (int i = 0; i < SD; i++) rn->states[(size_t)e * SD + i] = initial_states[((size_t)step * N + e) * SD + i];
+            }
+        if ((rc = observe_into(obs))) return rc;
+        if (st_mean) {
+            if ((rc = rlt_oracle_standardize_forward(st_mean, st_precision, obs, ld, standardized.data(), OBS, N, OBS))) return rc;
+            if ((rc = rlt_oracle_seq_evaluate_step(policy, n_policy_layers, standardized.data(), OBS, step_state, auto_reset_period, means, ld, N))) return rc;
+        } else if ((rc = rlt_oracle_seq_evaluate_step(policy, n_policy_layers, obs, ld, step_state, auto_reset_period, means, ld, N))) return rc;
+        for (int e = 0; e < N; e++) {                                                                                          // epilogue, per_env :37-58
+            const size_t pos = (size_t)step * N + e;
+            float log_prob = 0;
+            for (int a = 0; a < ACT; a++) {
+                const float mean = means[(size_t)e * ld + a];
+                const float noisy = action_noise[pos * ACT + a] * std::exp(log_std[a]) + mean;
+                log_prob += normal_log_prob(mean, log_std[a], noisy);
+                actions[(size_t)e * ld + a] = noisy;
+                rn->actions[(size_t)e * ACT + a] = noisy;
+            }
+            D->action_log_probs[pos * ld] = log_prob;
+        }
+        if ((rc = env_step_of(rn, rn->states, rn->actions, nullptr, nullptr, rn->rewards, rn->terminated))) return rc;
+        for (int e = 0; e < N; e++) {                                                                                          // :59-74
+            const size_t pos = (size_t)step * N + e;
+            D->terminated[pos * ld] = rn->terminated[e] ? 1.0f : 0.0f;
+            rn->episode_return[e] += rn->rewards[e];
+            D->rewards[pos * ld] = rn->rewards[e];
+            rn->episode_step[e] += 1;
+            const bool truncated = rn->terminated[e] || (rn->episode_step_limit > 0 && rn->episode_step[e] >= (uint32_t)rn->episode_step_limit);
+            D->truncated[pos * ld] = truncated;
+            D->all_reset[(pos + N) * ld] = truncated;
+            rn->truncated[e] = truncated;
+        }
+    }
+    return observe_into(D->observations + (size_t)S * N * ld);                                                                   // :137-144
+}
+
 }  // extern "C"
 template <typename POLICY>
 static int pendulum_evaluate_impl(const rlt_pendulum_parameters* env, int policy_kind, POLICY&& policy, const float* initial_states,

@@ -307,3 +307,130 @@ extern "C" int rlt_rocm_env_runner_step(rlt_rocm_device* device, const rlt_env_r
     hipLaunchKernelGGL(env_epilogue_kernel, dim3(blocks), dim3(256), 0, device->stream, *rn, *rb);
     return rlt_launch_status(device);
 }
+
+// ---- on-policy collection over any of these environments (rl/components/on_policy_runner/operations_generic_per_env.h:8-74)
+namespace {
+__device__ __forceinline__ float mul_add_twice_rounded(float a, float b, float c) {
+#pragma clang fp contract(off)
+    const float product = a * b;
+    return product + c;
+}
+__device__ __forceinline__ void observe_any(int kind, const float* __restrict__ state, float* __restrict__ o) {
+    if (kind == RLT_ENV_PENDULUM) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; o[2] = state[1]; }
+    else if (kind == RLT_ENV_CAR) { for (int i = 0; i < 6; i++) o[i] = state[i]; }
+    else { const Acrobot4 s4 = {{state[0], state[1], state[2], state[3]}}; acrobot_observe(s4, o); }
+}
+// prologue of step `step` (:8-35): reset where truncated (the flag is cleared), observe into the dataset row of this step; final: only the observation
+__global__ __launch_bounds__(256) void env_collect_prologue_kernel(rlt_env_runner rn, rlt_on_policy_dataset D, const float* __restrict__ initial_states, int step, int final) {
+    const EnvDims d = env_dims(rn.env_kind);
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) {
+        const size_t row = (size_t)step * rn.n_envs + e;
+        float* state = rn.states + (size_t)e * d.state;
+        if (!final) {
+            const bool truncated = rn.truncated[e] != 0;
+            if (step == 0) D.all_reset[(size_t)e * D.ld] = truncated ? 1.0f : 0.0f;      // reset aliases the first rows of all_reset
+            if (truncated) {
+                rn.truncated[e] = 0; rn.episode_step[e] = 0; rn.episode_return[e] = 0.0f;
+                for (int i = 0; i < d.state; i++) state[i] = initial_states[row * d.state + i];
+            }
+        }
+        observe_any(rn.env_kind, state, D.observations + row * D.ld);
+    }
+}
+// first half of the epilogue (:37-58): the action around the mean, its log-probability (random/operations_generic.h:73-97); the action also packed for the step kernel
+__global__ __launch_bounds__(256) void env_collect_sample_kernel(rlt_env_runner rn, rlt_on_policy_dataset D, const float* __restrict__ log_std, const float* __restrict__ action_noise, int step) {
+    const int ACT = env_dims(rn.env_kind).act;
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) {
+        const size_t row = (size_t)step * rn.n_envs + e;
+        float log_prob = 0.0f;
+        for (int a = 0; a < ACT; a++) {
+            const float ls = log_std[a], sd = expf(ls);
+            const float mean = D.actions_mean[row * D.ld + a];
+            const float action = mul_add_twice_rounded(action_noise[row * ACT + a], sd, mean);      // z * std + mean, rounded twice as the reference's CPU build does
+            const float pre = (action - mean) / sd;
+            log_prob += (-0.9189385332046727f - ls) - 0.5f * pre * pre;
+            D.actions[row * D.ld + a] = action;
+            rn.actions[(size_t)e * ACT + a] = action;
+        }
+        D.action_log_probs[row * D.ld] = log_prob;
+    }
+}
+// second half of the epilogue (:59-74) after the environment's own step: flags, reward, counters, the delayed reset flag
+__global__ __launch_bounds__(256) void env_collect_epilogue_kernel(rlt_env_runner rn, rlt_on_policy_dataset D, int step) {
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) {
+        const size_t row = (size_t)step * rn.n_envs + e;
+        const bool terminated = rn.terminated[e] != 0;
+        const float reward = rn.rewards[e];
+        D.terminated[row * D.ld] = terminated ? 1.0f : 0.0f;
+        rn.episode_return[e] += reward;
+        D.rewards[row * D.ld] = reward;
+        const uint32_t n = rn.episode_step[e] + 1;
+        rn.episode_step[e] = n;
+        const bool truncated = terminated || (rn.episode_step_limit > 0 && n >= (uint32_t)rn.episode_step_limit);
+        D.truncated[row * D.ld] = truncated ? 1.0f : 0.0f;
+        D.all_reset[(row + rn.n_envs) * D.ld] = truncated ? 1.0f : 0.0f;
+        rn.truncated[e] = truncated;
+    }
+}
+int env_step_launch(rlt_rocm_device* device, const rlt_env_runner* rn, float* next_observations) {
+    const int N = rn->n_envs;
+    int rc;
+    switch (rn->env_kind) {
+        case RLT_ENV_PENDULUM:
+            if ((rc = rlt_rocm_pendulum_step(device, &rn->pendulum, rn->states, rn->actions, nullptr, next_observations, rn->rewards, N))) return rc;
+            return rlt_rocm_fill_u8(device, rn->terminated, (size_t)N, 0);      // the Pendulum has no terminal states
+        case RLT_ENV_CAR: return rlt_rocm_car_step(device, &rn->car, rn->states, rn->actions, nullptr, next_observations, rn->rewards, rn->terminated, N);
+        default: return rlt_rocm_acrobot_step(device, &rn->acrobot, rn->env_kind == RLT_ENV_ACROBOT_SWINGUP, rn->states, rn->actions, nullptr, next_observations, rn->rewards, rn->terminated, N);
+    }
+}
+}  // namespace
+
+extern "C" size_t rlt_rocm_env_on_policy_collect_workspace_bytes(const rlt_env_runner* rn, const rlt_seq_layer* policy, int n_policy_layers) {
+    if (!rn || rn->n_envs < 1 || !policy || n_policy_layers < 1) return 0;
+    const EnvDims d = env_dims(rn->env_kind);
+    return align256((size_t)rn->n_envs * d.obs * sizeof(float)) + rlt_rocm_seq_evaluate_step_workspace_bytes(policy, n_policy_layers, rn->n_envs) + 512;
+}
+
+extern "C" int rlt_rocm_env_on_policy_collect(rlt_rocm_device* device, const rlt_env_runner* rn, const rlt_on_policy_dataset* D, const rlt_seq_layer* policy, int n_policy_layers,
+                                              const rlt_seq_state* policy_state, int auto_reset_period, const float* log_std, const float* standardize_mean,
+                                              const float* standardize_precision, const float* action_noise, const float* initial_states, int truncate_on_each_iteration,
+                                              void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(rn && rn->n_envs > 0 && rn->states && rn->episode_step && rn->episode_return && rn->truncated && rn->actions && rn->rewards && rn->terminated);
+    const EnvDims d = env_dims(rn->env_kind);
+    RLT_REQUIRE(d.state && D && D->steps_per_env > 0 && D->ld >= d.obs && D->ld >= d.act);
+    RLT_REQUIRE(D->observations && D->actions_mean && D->actions && D->action_log_probs && D->rewards && D->terminated && D->truncated && D->all_reset);
+    RLT_REQUIRE(policy && n_policy_layers >= 1 && n_policy_layers <= RLT_SEQ_MAX_LAYERS && log_std && action_noise && initial_states);
+    RLT_REQUIRE((standardize_mean == nullptr) == (standardize_precision == nullptr));
+    bool recurrent = false;
+    for (int l = 0; l < n_policy_layers; l++) recurrent = recurrent || policy[l].kind != 0;
+    RLT_REQUIRE(!recurrent || policy_state);
+    RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_env_on_policy_collect_workspace_bytes(rn, policy, n_policy_layers));
+    const int N = rn->n_envs, blocks = rlt_div_up(N, 256) > 1024 ? 1024 : rlt_div_up(N, 256);
+    float* standardized = reinterpret_cast<float*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    char* step_ws = (char*)standardized + align256((size_t)N * d.obs * sizeof(float));
+    const size_t step_ws_bytes = workspace_bytes - (size_t)(step_ws - (char*)workspace);
+    int rc;
+    const rlt_seq_state no_state = {};      // a policy of dense layers keeps no state
+    const rlt_seq_state* step_state = policy_state ? policy_state : &no_state;
+    if (truncate_on_each_iteration && (rc = rlt_rocm_fill_u8(device, rn->truncated, (size_t)N, 1))) return rc;      // :112-114
+    for (int step = 0; step < D->steps_per_env; step++) {
+        if (policy_state && (rc = rlt_rocm_seq_reset_state(device, policy, n_policy_layers, policy_state, rn->truncated, N))) return rc;
+        hipLaunchKernelGGL(env_collect_prologue_kernel, dim3(blocks), dim3(256), 0, device->stream, *rn, *D, initial_states, step, 0);
+        if ((rc = rlt_launch_status(device))) return rc;
+        const float* obs = D->observations + (size_t)step * N * D->ld; int ldo = D->ld;
+        if (standardize_mean) {
+            if ((rc = rlt_rocm_standardize_forward(device, standardize_mean, standardize_precision, obs, D->ld, standardized, d.obs, N, d.obs))) return rc;
+            obs = standardized; ldo = d.obs;
+        }
+        if ((rc = rlt_rocm_seq_evaluate_step(device, policy, n_policy_layers, obs, ldo, step_state, auto_reset_period, D->actions_mean + (size_t)step * N * D->ld, D->ld, N,
+                                             step_ws, step_ws_bytes))) return rc;
+        hipLaunchKernelGGL(env_collect_sample_kernel, dim3(blocks), dim3(256), 0, device->stream, *rn, *D, log_std, action_noise, step);
+        if ((rc = rlt_launch_status(device))) return rc;
+        if ((rc = env_step_launch(device, rn, nullptr))) return rc;
+        hipLaunchKernelGGL(env_collect_epilogue_kernel, dim3(blocks), dim3(256), 0, device->stream, *rn, *D, step);
+        if ((rc = rlt_launch_status(device))) return rc;
+    }
+    hipLaunchKernelGGL(env_collect_prologue_kernel, dim3(blocks), dim3(256), 0, device->stream, *rn, *D, initial_states, D->steps_per_env, 1);
+    return rlt_launch_status(device);
+}

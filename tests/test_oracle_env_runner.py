@@ -80,3 +80,35 @@ def test_bookkeeping_around_the_environments_own_step(oracle, kind):
         assert np.array_equal(rows, np.concatenate([o, actions, r[:, None], no, t[:, None].astype(np.float32), truncated[:, None].astype(np.float32)], 1))
         position = (position + 1) % cap
     assert seen_termination
+
+
+@pytest.mark.parametrize("standardize,truncate", [(False, 0), (True, 1)])
+def test_generic_collect_on_the_pendulum_equals_the_pendulum_collect(oracle, standardize, truncate):
+    """rlt_oracle_env_on_policy_collect with a policy of dense layers on the Pendulum leaves the dataset and runner state that
+    rlt_oracle_on_policy_collect leaves, which the reference's PPO loop pins (tests/test_oracle_vs_reference.py)."""
+    n, steps, limit, ld = 19, 23, 7, 14
+    col = dict(observations=0, actions_mean=3, actions=4, action_log_probs=5, rewards=6, terminated=7, truncated=8, all_reset=9)
+    rng = np.random.default_rng(3)
+    dims = [3, 16, 16, 1]
+    params = helpers.random_params(rng, dims)
+    specs = [(0, 3, 16, "relu"), (0, 16, 16, "relu"), (0, 16, 1, "identity")]
+    log_std = np.array([-0.5], np.float32)
+    st = (rng.uniform(-0.2, 0.2, 3).astype(np.float32), rng.uniform(0.5, 2.0, 3).astype(np.float32)) if standardize else None
+    specific = helpers.OnPolicyOnBackend(oracle, n, steps, ld, col, limit)
+    actor = helpers.Mlp(oracle, dims, params, n, trainable=False)
+    runner = helpers.EnvRunnerOnBackend(oracle, capi.ENV_PENDULUM, n, limit)
+    policy = helpers.SeqNet(oracle, specs, params, 1, n, trainable=False)
+    for _ in range(3):
+        noise = rng.standard_normal((steps, n, 1)).astype(np.float32)
+        ini = np.stack([rng.uniform(-np.pi, np.pi, (steps, n)), rng.uniform(-1, 1, (steps, n))], 2).astype(np.float32)
+        specific.data.upload(np.zeros_like(specific.data.numpy()))
+        specific.collect(actor, log_std, noise, ini, st, truncate)
+        data = oracle.zeros(((steps + 1) * n, ld))
+        o = data.offset
+        d = capi.OnPolicyDataset(o(0), o(3), o(4), o(5), o(6), o(7), o(8), o(9), ld, steps)
+        oracle.call("env_on_policy_collect", C.byref(runner.c), C.byref(d), policy.layers, policy.n, None, 0, log_std.ctypes.data, st[0].ctypes.data if st else None,
+                    st[1].ctypes.data if st else None, noise.ctypes.data, ini.ctypes.data, truncate, None, 0)
+        assert np.array_equal(data.numpy(), specific.data.numpy())
+        for a, b in zip(runner.snapshot()[:4], (specific.states, specific.ep_step, specific.ep_ret, specific.trunc)):
+            assert np.array_equal(a, b.numpy())
+    assert data.numpy()[:, 9].sum() > n
