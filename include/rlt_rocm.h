@@ -985,6 +985,19 @@ int rlt_rocm_on_policy_collect(rlt_rocm_device* device, const rlt_pendulum_runne
                                const float* action_noise, const float* initial_states, int truncate_on_each_iteration,
                                void* workspace, size_t workspace_bytes);
 
+/* The runner step of rlt_rocm_env_runner_step with a sequential policy (dense and GRU layers) and its rollout state
+ * (rl/components/off_policy_runner/operations_generic.h:189-206): after the prologue the policy state of the environments that start a new
+ * episode is reset, then one evaluate_step in Rollout mode, then the policy's last layer:
+ *   head_kind 1  the output is the action
+ *             2  the output is [mean | log_std]: sample_and_squash with action_noise (SAC; `sas` required)
+ *             3  td3_sampling (nn/layers/td3_sampling/operations_generic.h:75-128): action = clamp(output + exploration_noise_std * action_noise, -1, 1) (TD3)
+ * action_noise [n_envs x action_dim] standard normal values (unused for head_kind 1). policy_state may be NULL for a policy of dense layers. */
+size_t rlt_rocm_env_runner_step_sequential_workspace_bytes(const rlt_env_runner* runner, const rlt_seq_layer* policy, int n_policy_layers);
+int rlt_rocm_env_runner_step_sequential(rlt_rocm_device* device, const rlt_env_runner* runner, const rlt_replay_buffer* rb,
+                                        const rlt_seq_layer* policy, int n_policy_layers, const rlt_seq_state* policy_state, int auto_reset_period,
+                                        int head_kind, const rlt_sas_parameters* sas, float exploration_noise_std, const float* action_noise,
+                                        const float* initial_states, void* workspace, size_t workspace_bytes);
+
 /* collect for any of the batched environments and any sequential policy (dense and GRU layers): rl/components/on_policy_runner/
  * operations_generic.h:105-146 over operations_generic_per_env.h:8-74. Per step: reset(policy, policy_state) where the runner's truncated flag
  * is set (before the prologue clears it, :127-130; skipped when policy_state is NULL), the prologue (environments whose flag is set start

@@ -1104,6 +1104,50 @@ int rlt_oracle_env_runner_step(const rlt_env_runner* rn, const rlt_replay_buffer
 //   policy_kind 1: the actor's output is the action;  2: the actor's output is [mean | log_std] and the action is tanh(mean), which is what
 //   sample_and_squash yields in Evaluation mode (noise = 0, nn/layers/sample_and_squash/operations_generic.h:149-195)
 //   summary = {returns_mean, returns_std, episode_length_mean, episode_length_std, num_terminated, share_terminated}
+// the same runner step with a sequential policy and its rollout state (rl/components/off_policy_runner/operations_generic.h:189-206: reset of the policy state
+// under the truncated mask after the prologue, evaluate_step in Rollout mode) and the policy's last layer: 1 none, 2 sample_and_squash, 3 td3_sampling
+int rlt_oracle_env_runner_step_sequential(const rlt_env_runner* rn, const rlt_replay_buffer* rb, const rlt_seq_layer* policy, int n_policy_layers,
+                                          const rlt_seq_state* policy_state, int auto_reset_period, int head_kind, const rlt_sas_parameters* sas, float exploration_noise_std,
+                                          const float* action_noise, const float* initial_states) {
+    int SD, OBS, ACT;
+    if (!rn || !rb || !policy || !initial_states || env_dims_of(rn->env_kind, &SD, &OBS, &ACT) || rn->n_envs != rb->n_envs || rb->observation_dim != OBS || rb->action_dim != ACT)
+        return RLT_E_INVALID_ARGUMENT;
+    if (head_kind < 1 || head_kind > 3 || (head_kind != 1 && !action_noise) || (head_kind == 2 && !sas)) return RLT_E_INVALID_ARGUMENT;
+    const int N = rn->n_envs, R = rb_row_dim(rb);
+    for (int e = 0; e < N; e++)
+        if (rn->truncated[e]) {
+            for (int i = 0; i < SD; i++) rn->states[(size_t)e * SD + i] = initial_states[(size_t)e * SD + i];
+            rn->episode_step[e] = 0; rn->episode_return[e] = 0;
+            if (rb->full[e] || rb->position[e] > 0) {
+                const uint32_t prev = rb->position[e] == 0 ? (uint32_t)rb->capacity - 1 : rb->position[e] - 1;
+                rb->data[((size_t)e * rb->capacity + prev) * R + (R - 1)] = 1.0f;
+                rb->current_episode_start[e] = rb->position[e];
+            }
+        }
+    int rc;
+    {
+        std::vector<float> scratch_states(rn->states, rn->states + (size_t)N * SD), zero_actions((size_t)N * ACT, 0.0f);
+        if ((rc = env_step_of(rn, scratch_states.data(), zero_actions.data(), rn->observations, nullptr, nullptr, nullptr))) return rc;
+    }
+    const rlt_seq_state no_state = {};
+    if (policy_state && (rc = rlt_oracle_seq_reset_state(policy, n_policy_layers, policy_state, rn->truncated, N))) return rc;
+    const int out_dim = (head_kind == 2 ? 2 : 1) * ACT;
+    std::vector<float> out((size_t)N * out_dim), lp(N);
+    if ((rc = rlt_oracle_seq_evaluate_step(policy, n_policy_layers, rn->observations, OBS, policy_state ? policy_state : &no_state, auto_reset_period, out.data(), out_dim, N))) return rc;
+    if (head_kind == 1) std::copy(out.begin(), out.end(), rn->actions);
+    else if (head_kind == 2) rc = rlt_oracle_sas_forward(sas, out.data(), 2 * ACT, action_noise, ACT, rn->actions, ACT, nullptr, 0, lp.data(), N, ACT);
+    else rc = rlt_oracle_td3_sampling_forward(out.data(), ACT, action_noise, ACT, exploration_noise_std, nullptr, 0, rn->actions, ACT, N, ACT);
+    if (rc) return rc;
+    if ((rc = env_step_of(rn, rn->states, rn->actions, nullptr, rn->next_observations, rn->rewards, rn->terminated))) return rc;
+    std::vector<uint8_t> trunc(N, 0);
+    for (int e = 0; e < N; e++) {
+        rn->episode_step[e] += 1; rn->episode_return[e] += rn->rewards[e];
+        trunc[e] = rn->terminated[e] || rn->episode_step[e] == (uint32_t)rn->episode_step_limit;
+        rn->truncated[e] = trunc[e];
+    }
+    return rlt_oracle_replay_add(rb, rn->observations, rn->actions, rn->rewards, rn->next_observations, rn->terminated, trunc.data());
+}
+
 // collect for any of the environments restated here and any sequential policy: rl/components/on_policy_runner/operations_generic.h:105-146 over
 // operations_generic_per_env.h:8-74 (see on_policy_collect_impl further down for the Pendulum / MLP case, which the reference's PPO loop pins)
 int rlt_oracle_env_on_policy_collect(const rlt_env_runner* rn, const rlt_on_policy_dataset* D, const rlt_seq_layer* policy, int n_policy_layers,

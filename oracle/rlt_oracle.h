@@ -170,6 +170,9 @@ int rlt_oracle_env_runner_step(const rlt_env_runner* runner, const rlt_replay_bu
 int rlt_oracle_env_on_policy_collect(const rlt_env_runner* runner, const rlt_on_policy_dataset* dataset, const rlt_seq_layer* policy, int n_policy_layers,
                                      const rlt_seq_state* policy_state, int auto_reset_period, const float* log_std, const float* standardize_mean,
                                      const float* standardize_precision, const float* action_noise, const float* initial_states, int truncate_on_each_iteration);
+int rlt_oracle_env_runner_step_sequential(const rlt_env_runner* runner, const rlt_replay_buffer* rb, const rlt_seq_layer* policy, int n_policy_layers,
+                                          const rlt_seq_state* policy_state, int auto_reset_period, int head_kind, const rlt_sas_parameters* sas, float exploration_noise_std,
+                                          const float* action_noise, const float* initial_states);
 int rlt_oracle_acrobot_step(const rlt_acrobot_parameters* p, int swingup, float* states, const float* actions, float* observations, float* next_observations,
                             float* rewards, uint8_t* terminated, int n_envs);
 /* rl/environments/car/operations_generic.h:80-155 (the Car without a track) */

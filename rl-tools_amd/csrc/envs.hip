@@ -434,3 +434,44 @@ extern "C" int rlt_rocm_env_on_policy_collect(rlt_rocm_device* device, const rlt
     hipLaunchKernelGGL(env_collect_prologue_kernel, dim3(blocks), dim3(256), 0, device->stream, *rn, *D, initial_states, D->steps_per_env, 1);
     return rlt_launch_status(device);
 }
+
+extern "C" size_t rlt_rocm_env_runner_step_sequential_workspace_bytes(const rlt_env_runner* rn, const rlt_seq_layer* policy, int n_policy_layers) {
+    if (!rn || rn->n_envs < 1 || !policy || n_policy_layers < 1) return 0;
+    const EnvDims d = env_dims(rn->env_kind);
+    return align256((size_t)rn->n_envs * (2 * d.act + 1) * sizeof(float)) + rlt_rocm_seq_evaluate_step_workspace_bytes(policy, n_policy_layers, rn->n_envs) + 512;
+}
+
+extern "C" int rlt_rocm_env_runner_step_sequential(rlt_rocm_device* device, const rlt_env_runner* rn, const rlt_replay_buffer* rb, const rlt_seq_layer* policy, int n_policy_layers,
+                                                   const rlt_seq_state* policy_state, int auto_reset_period, int head_kind, const rlt_sas_parameters* sas, float exploration_noise_std,
+                                                   const float* action_noise, const float* initial_states, void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(rn && rb && rn->n_envs > 0 && rn->states && rn->episode_step && rn->episode_return && rn->truncated && initial_states);
+    RLT_REQUIRE(rn->observations && rn->actions && rn->next_observations && rn->rewards && rn->terminated);
+    RLT_REQUIRE(rb->data && rb->episode_start && rb->position && rb->current_episode_start && rb->full && rb->capacity > 0);
+    const EnvDims d = env_dims(rn->env_kind);
+    RLT_REQUIRE(d.state && rn->n_envs == rb->n_envs && rb->observation_dim == d.obs && rb->action_dim == d.act && head_kind >= 1 && head_kind <= 3);
+    RLT_REQUIRE(policy && n_policy_layers >= 1 && n_policy_layers <= RLT_SEQ_MAX_LAYERS && (head_kind == 1 || action_noise) && (head_kind != 2 || sas));
+    bool recurrent = false;
+    for (int l = 0; l < n_policy_layers; l++) recurrent = recurrent || policy[l].kind != 0;
+    RLT_REQUIRE(!recurrent || policy_state);
+    RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_env_runner_step_sequential_workspace_bytes(rn, policy, n_policy_layers));
+    const int N = rn->n_envs, blocks = rlt_div_up(N, 256) > 1024 ? 1024 : rlt_div_up(N, 256);
+    float* policy_out = reinterpret_cast<float*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    float* log_probabilities = policy_out + (size_t)N * 2 * d.act;
+    char* step_ws = (char*)policy_out + align256((size_t)N * (2 * d.act + 1) * sizeof(float));
+    const size_t step_ws_bytes = workspace_bytes - (size_t)(step_ws - (char*)workspace);
+    const rlt_seq_state no_state = {};
+    int rc;
+    hipLaunchKernelGGL(env_prologue_kernel, dim3(blocks), dim3(256), 0, device->stream, *rn, *rb, initial_states);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if (policy_state && (rc = rlt_rocm_seq_reset_state(device, policy, n_policy_layers, policy_state, rn->truncated, N))) return rc;
+    const int out_dim = (head_kind == 2 ? 2 : 1) * d.act;
+    float* out = head_kind == 1 ? rn->actions : policy_out;
+    if ((rc = rlt_rocm_seq_evaluate_step(device, policy, n_policy_layers, rn->observations, d.obs, policy_state ? policy_state : &no_state, auto_reset_period, out, out_dim, N,
+                                         step_ws, step_ws_bytes))) return rc;
+    if (head_kind == 2) { if ((rc = rlt_rocm_sas_forward(device, sas, policy_out, 2 * d.act, action_noise, d.act, rn->actions, d.act, nullptr, 0, log_probabilities, N, d.act))) return rc; }
+    else if (head_kind == 3) { if ((rc = rlt_rocm_td3_sampling_forward(device, policy_out, d.act, action_noise, d.act, exploration_noise_std, nullptr, 0, rn->actions, d.act, N, d.act))) return rc; }
+    if ((rc = env_step_launch(device, rn, rn->next_observations))) return rc;
+    hipLaunchKernelGGL(env_epilogue_kernel, dim3(blocks), dim3(256), 0, device->stream, *rn, *rb);
+    return rlt_launch_status(device);
+}

@@ -44,7 +44,7 @@ class LoopConfig(C.Structure):
 
 
 WITH_WORKSPACE = ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward", "on_policy_collect", "seq_forward", "seq_backward", "seq_evaluate_step",
-                  "pendulum_runner_step_recurrent", "pendulum_evaluate_recurrent", "env_runner_step", "env_on_policy_collect")
+                  "pendulum_runner_step_recurrent", "pendulum_evaluate_recurrent", "env_runner_step", "env_on_policy_collect", "env_runner_step_sequential")
 
 
 def load_oracle():

@@ -112,3 +112,31 @@ def test_generic_collect_on_the_pendulum_equals_the_pendulum_collect(oracle, sta
         for a, b in zip(runner.snapshot()[:4], (specific.states, specific.ep_step, specific.ep_ret, specific.trunc)):
             assert np.array_equal(a, b.numpy())
     assert data.numpy()[:, 9].sum() > n
+
+
+def test_sequential_step_on_the_pendulum_equals_the_recurrent_pendulum_runner_step(oracle):
+    """head_kind 2 (sample_and_squash) with a dense-GRU-dense policy: the generic step leaves what rlt_oracle_pendulum_runner_step_recurrent leaves, which
+    the reference's recurrent SAC loop pins (tests/test_oracle_vs_reference.py, recurrent runner golden vectors)."""
+    n, cap, limit, period, steps = 11, 9, 6, 4, 40
+    specs = [(0, 3, 8, "relu"), (1, 8, 8, "identity"), (0, 8, 2, "identity")]
+    rng = np.random.default_rng(2)
+    params = helpers.random_seq_params(rng, specs)
+    specific = helpers.RecurrentRunnerOnBackend(oracle, specs, params, n, cap, limit, period)
+    runner = helpers.EnvRunnerOnBackend(oracle, capi.ENV_PENDULUM, n, limit)
+    rb = helpers.ReplayOnBackend(oracle, n, cap)
+    policy = helpers.SeqNet(oracle, specs, params, 1, n, trainable=False)
+    state = helpers.SeqStateOnBackend(oracle, specs, n)
+    sas = capi.SasParameters(-20.0, 2.0, 1e-6, -1.0)
+    for _ in range(steps):
+        noise = rng.standard_normal((n, 1)).astype(np.float32)
+        ini = np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n)], 1).astype(np.float32)
+        specific.step(noise, ini)
+        oracle.call("env_runner_step_sequential", C.byref(runner.c), C.byref(rb.c), policy.layers, policy.n, C.byref(state.c), period, 2, C.byref(sas), 0.0, noise.ctypes.data,
+                    ini.ctypes.data, None, 0)
+        want = specific.numpy()
+        for a, b in ((runner.states, want["states"]), (runner.ep_step, want["episode_step"]), (runner.ep_ret, want["episode_return"]), (runner.trunc, want["truncated"]),
+                     (rb.data, want["data"]), (rb.position, want["position"]), (rb.episode_start, want["episode_start"])):
+            assert np.array_equal(a.numpy(), b)
+        hidden, counters = state.numpy()
+        assert all(np.array_equal(a, b) for a, b in zip(hidden, want["hidden"])) and all(np.array_equal(a, b) for a, b in zip(counters, want["steps"]))
+    assert rb.full.numpy().all()

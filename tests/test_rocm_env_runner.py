@@ -76,3 +76,47 @@ def test_env_dims(rocm):
         s, o, a = C.c_int(), C.c_int(), C.c_int()
         assert lib.rlt_rocm_env_dims(kind, C.byref(s), C.byref(o), C.byref(a)) == 0 and (s.value, o.value, a.value) == dims
     assert lib.rlt_rocm_env_dims(9, None, None, None) == capi.RLT_E_INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("kind,specs,head_kind,n_envs,capacity,limit,period,steps", [
+    (capi.ENV_PENDULUM, [(0, 3, 16, "relu"), (1, 16, 16, "identity"), (0, 16, 1, "tanh")], 3, 40, 30, 12, 5, 70),        # TD3's exploration head on a recurrent policy
+    (capi.ENV_ACROBOT, [(0, 6, 16, "relu"), (1, 16, 16, "identity"), (1, 16, 16, "identity"), (0, 16, 2, "identity")], 2, 33, 20, 10, 0, 50),
+    (capi.ENV_CAR, [(0, 6, 32, "relu"), (0, 32, 2, "tanh")], 1, 50, 25, 9, 0, 40),                                   # a policy of dense layers, deterministic
+])
+def test_env_runner_step_with_a_sequential_policy(oracle, rocm, kind, specs, head_kind, n_envs, capacity, limit, period, steps):
+    sd, od, ad = capi.ENV_DIMS[kind]
+    rng = np.random.default_rng(kind + 40)
+    params = helpers.random_seq_params(rng, specs)
+    draws = [(initial_states(rng, kind, n_envs), rng.standard_normal((n_envs, ad)).astype(np.float32)) for _ in range(steps)]
+    recurrent = any(k for k, *_ in specs)
+    results = []
+    for backend in (oracle, rocm):
+        runner = helpers.EnvRunnerOnBackend(backend, kind, n_envs, limit)
+        rb = helpers.ReplayOnBackend(backend, n_envs, capacity, od, ad)
+        policy = helpers.SeqNet(backend, specs, params, 1, n_envs, trainable=False)
+        state = helpers.SeqStateOnBackend(backend, specs, n_envs)
+        sas = capi.SasParameters(-20.0, 2.0, 1e-6, -float(ad))
+        ws, wsn = (None, 0)
+        if backend.name == "rocm":
+            ws, wsn = backend.workspace(backend.device.lib.rlt_rocm_env_runner_step_sequential_workspace_bytes(C.byref(runner.c), policy.layers, policy.n))
+        trace = []
+        for ini, noise in draws:
+            i_d, n_d = backend.array(ini), backend.array(noise)
+            backend.call("env_runner_step_sequential", C.byref(runner.c), C.byref(rb.c), policy.layers, policy.n, C.byref(state.c) if recurrent else None, period, head_kind,
+                         C.byref(sas), 0.3, n_d.ptr, i_d.ptr, ws, wsn)
+            backend.sync()
+            trace.append(runner.snapshot() + list(state.numpy()[0]) + list(state.numpy()[1]))
+        results.append((trace, [a.numpy() for a in (rb.data, rb.episode_start, rb.position, rb.current_episode_start, rb.full)]))
+    (ref_trace, ref_rb), (got_trace, got_rb) = results
+    tol = 1e-4 if kind in (capi.ENV_ACROBOT, capi.ENV_ACROBOT_SWINGUP) else 1e-5
+    for step, (ref, got) in enumerate(zip(ref_trace, got_trace)):
+        for k, (a, b) in enumerate(zip(got, ref)):
+            if a.dtype in (np.uint8, np.uint32):
+                assert np.array_equal(a, b), (step, k)
+            else:
+                assert rel_err(a, b) <= tol, (step, k, rel_err(a, b))
+    assert rel_err(got_rb[0], ref_rb[0]) <= tol and all(np.array_equal(got_rb[k], ref_rb[k]) for k in range(1, 5))
+    assert ref_rb[4].all()
+    if head_kind == 3:      # the exploration head clipped some actions
+        acts = np.concatenate([t[5] for t in ref_trace])
+        assert np.abs(acts).max() <= 1.0 and (np.abs(acts) == 1.0).any()
