@@ -36,9 +36,11 @@ def test_library_has_no_oracle_dependency():
 
 def test_structure_sizes_match_the_header():
     capi = helpers.capi
-    names = {"rlt_dense_layer": capi.DenseLayer, "rlt_adam_parameters": capi.AdamParameters, "rlt_adam_tensor": capi.AdamTensor,
-             "rlt_sas_parameters": capi.SasParameters, "rlt_sac_agent": capi.SacAgent, "rlt_replay_buffer": capi.ReplayBuffer,
-             "rlt_pendulum_parameters": capi.PendulumParameters, "rlt_pendulum_runner": capi.PendulumRunner}
+    # every struct the header declares (the opaque device handle aside) against its ctypes mirror: rlt_foo_bar <-> capi.FooBar
+    text = open(os.path.join(helpers.ROOT, "include", "rlt_rocm.h")).read()
+    declared = [n for n in re.findall(r"^typedef struct (rlt_[a-z0-9_]+)", text, flags=re.M) if n != "rlt_rocm_device"]
+    assert len(declared) >= 26
+    names = {n: getattr(capi, "".join(part.capitalize() for part in n[4:].split("_"))) for n in declared}
     prog = '#include <stdio.h>\n#include "rlt_rocm.h"\nint main(){' + "".join(f'printf("{n} %zu\\n", sizeof({n}));' for n in names) + "return 0;}"
     with tempfile.TemporaryDirectory() as d:
         open(os.path.join(d, "s.c"), "w").write(prog)
