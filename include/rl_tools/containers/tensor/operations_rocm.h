@@ -144,6 +144,69 @@ namespace rl_tools{
         devices::rocm::check(rlt_rocm_free(device.handle, out), "squared_sum");
         return value;
     }
+    // unary_operation / binary_operation / ternary_operation   containers/tensor/operations_generic.h:573-760 (CUDA: operations_cuda.h:172-283, 359-544)
+    // on dense float tensors: the functor's type selects the library's operation, its members travel as the parameter
+    namespace tensor::rocm{
+        template<typename OPERATION> struct UnaryId{ static constexpr int ID = -1; static float parameter(const OPERATION&){ return 0; } };
+        template<> struct UnaryId<tensor::operations::unary::Negate>{ static constexpr int ID = RLT_UNARY_NEGATE; static float parameter(const tensor::operations::unary::Negate&){ return 0; } };
+        template<> struct UnaryId<tensor::operations::unary::Abs>{ static constexpr int ID = RLT_UNARY_ABS; static float parameter(const tensor::operations::unary::Abs&){ return 0; } };
+        template<> struct UnaryId<tensor::operations::unary::Constant<float>>{ static constexpr int ID = RLT_UNARY_CONSTANT; static float parameter(const tensor::operations::unary::Constant<float>& op){ return op.constant; } };
+        template<> struct UnaryId<tensor::operations::unary::Sigmoid>{ static constexpr int ID = RLT_UNARY_SIGMOID; static float parameter(const tensor::operations::unary::Sigmoid&){ return 0; } };
+        template<> struct UnaryId<tensor::operations::unary::FastSigmoid>{ static constexpr int ID = RLT_UNARY_FAST_SIGMOID; static float parameter(const tensor::operations::unary::FastSigmoid&){ return 0; } };
+        template<> struct UnaryId<tensor::operations::unary::Exp>{ static constexpr int ID = RLT_UNARY_EXP; static float parameter(const tensor::operations::unary::Exp&){ return 0; } };
+        template<> struct UnaryId<tensor::operations::unary::Tanh>{ static constexpr int ID = RLT_UNARY_TANH; static float parameter(const tensor::operations::unary::Tanh&){ return 0; } };
+        template<> struct UnaryId<tensor::operations::unary::FastTanh>{ static constexpr int ID = RLT_UNARY_FAST_TANH; static float parameter(const tensor::operations::unary::FastTanh&){ return 0; } };
+        template<> struct UnaryId<tensor::operations::unary::OneMinus>{ static constexpr int ID = RLT_UNARY_ONE_MINUS; static float parameter(const tensor::operations::unary::OneMinus&){ return 0; } };
+        template<typename OPERATION> struct BinaryId{ static constexpr int ID = -1; };
+        template<> struct BinaryId<tensor::operations::binary::Add>{ static constexpr int ID = RLT_BINARY_ADD; };
+        template<> struct BinaryId<tensor::operations::binary::Subtract>{ static constexpr int ID = RLT_BINARY_SUBTRACT; };
+        template<> struct BinaryId<tensor::operations::binary::Multiply>{ static constexpr int ID = RLT_BINARY_MULTIPLY; };
+        template<> struct BinaryId<tensor::operations::binary::Divide>{ static constexpr int ID = RLT_BINARY_DIVIDE; };
+        template<typename SPEC> constexpr bool dense_float(){ return utils::typing::is_same_v<utils::typing::remove_cv_t<typename SPEC::T>, float> && tensor::dense_row_major_layout<SPEC>(); }
+    }
+    template<typename DEV_SPEC, typename OPERATION, typename SPEC, typename SPEC_OUTPUT>
+    void unary_operation(devices::ROCM<DEV_SPEC>& device, const OPERATION& operation, Tensor<SPEC>& t, Tensor<SPEC_OUTPUT>& output){
+        static_assert(tensor::rocm::UnaryId<OPERATION>::ID >= 0 || utils::typing::is_same_v<OPERATION, tensor::operations::unary::Scale<float>>, "this functor has no counterpart in the ROCm library");
+        static_assert(tensor::rocm::dense_float<SPEC>() && tensor::rocm::dense_float<SPEC_OUTPUT>() && SPEC::SIZE == SPEC_OUTPUT::SIZE, "elementwise operations work on dense float tensors of one size");
+        if constexpr(utils::typing::is_same_v<OPERATION, tensor::operations::unary::Scale<float>>)
+            devices::rocm::check(rlt_rocm_unary_f32(device.handle, operation.reciprocal ? RLT_UNARY_SCALE_RECIPROCAL : RLT_UNARY_SCALE, operation.scale, t._data, (int)SPEC::SIZE, output._data, (int)SPEC::SIZE, 1, (int)SPEC::SIZE), "unary_operation");
+        else
+            devices::rocm::check(rlt_rocm_unary_f32(device.handle, tensor::rocm::UnaryId<OPERATION>::ID, tensor::rocm::UnaryId<OPERATION>::parameter(operation), t._data, (int)SPEC::SIZE, output._data, (int)SPEC::SIZE, 1, (int)SPEC::SIZE), "unary_operation");
+    }
+    template<typename DEV_SPEC, typename OPERATION, typename SPEC>
+    void unary_operation(devices::ROCM<DEV_SPEC>& device, const OPERATION& operation, Tensor<SPEC>& t){
+        unary_operation(device, operation, t, t);
+    }
+    template<typename DEV_SPEC, typename SPEC_1, typename SPEC_2, typename SPEC_OUT, typename OPERATION>
+    void binary_operation(devices::ROCM<DEV_SPEC>& device, const OPERATION& operation, Tensor<SPEC_1>& t1, Tensor<SPEC_2>& t2, Tensor<SPEC_OUT>& result){
+        static_assert(tensor::rocm::BinaryId<OPERATION>::ID >= 0, "this functor has no counterpart in the ROCm library");
+        static_assert(tensor::rocm::dense_float<SPEC_1>() && tensor::rocm::dense_float<SPEC_2>() && tensor::rocm::dense_float<SPEC_OUT>() && SPEC_1::SIZE == SPEC_2::SIZE && SPEC_1::SIZE == SPEC_OUT::SIZE);
+        devices::rocm::check(rlt_rocm_binary_f32(device.handle, tensor::rocm::BinaryId<OPERATION>::ID, t1._data, (int)SPEC_1::SIZE, t2._data, (int)SPEC_1::SIZE, result._data, (int)SPEC_1::SIZE, 1, (int)SPEC_1::SIZE), "binary_operation");
+    }
+    // the two-tensor form writes into the second operand (operations_generic.h:596-610)
+    template<typename DEV_SPEC, typename SPEC_1, typename SPEC_2, typename OPERATION>
+    void binary_operation(devices::ROCM<DEV_SPEC>& device, const OPERATION operation, const Tensor<SPEC_1>& t1, Tensor<SPEC_2>& t2){
+        static_assert(tensor::rocm::BinaryId<OPERATION>::ID >= 0, "this functor has no counterpart in the ROCm library");
+        static_assert(tensor::rocm::dense_float<SPEC_1>() && tensor::rocm::dense_float<SPEC_2>() && SPEC_1::SIZE == SPEC_2::SIZE);
+        devices::rocm::check(rlt_rocm_binary_f32(device.handle, tensor::rocm::BinaryId<OPERATION>::ID, t1._data, (int)SPEC_1::SIZE, t2._data, (int)SPEC_1::SIZE, t2._data, (int)SPEC_1::SIZE, 1, (int)SPEC_1::SIZE), "binary_operation");
+    }
+    // multiply_accumulate(t1, t2, t_output): t_output += t1 * t2   (operations_generic.h:475-481 and the ternary operation around it)
+    template<typename DEV_SPEC, typename SPEC_1, typename SPEC_2, typename SPEC_OUT>
+    void multiply_accumulate(devices::ROCM<DEV_SPEC>& device, const Tensor<SPEC_1>& t1, const Tensor<SPEC_2>& t2, Tensor<SPEC_OUT>& t_output){
+        static_assert(tensor::rocm::dense_float<SPEC_1>() && tensor::rocm::dense_float<SPEC_2>() && tensor::rocm::dense_float<SPEC_OUT>() && SPEC_1::SIZE == SPEC_2::SIZE && SPEC_1::SIZE == SPEC_OUT::SIZE);
+        devices::rocm::check(rlt_rocm_multiply_accumulate_f32(device.handle, t1._data, (int)SPEC_1::SIZE, t2._data, (int)SPEC_1::SIZE, t_output._data, (int)SPEC_1::SIZE, t_output._data, (int)SPEC_1::SIZE, 1, (int)SPEC_1::SIZE), "multiply_accumulate");
+    }
+    // abs_max   operations_generic.h:820-825 (the value is read back: the stream is waited for)
+    template<typename DEV_SPEC, typename SPEC>
+    typename SPEC::T abs_max(devices::ROCM<DEV_SPEC>& device, const Tensor<SPEC>& t){
+        static_assert(tensor::rocm::dense_float<SPEC>());
+        float* out = nullptr; float value = 0;
+        devices::rocm::check(rlt_rocm_malloc(device.handle, (void**)&out, sizeof(float)), "abs_max");
+        devices::rocm::check(rlt_rocm_reduce_abs_max_f32(device.handle, t._data, (size_t)SPEC::SIZE, out), "abs_max");
+        devices::rocm::check(rlt_rocm_memcpy_d2h(device.handle, &value, out, sizeof(float)), "abs_max");
+        devices::rocm::check(rlt_rocm_free(device.handle, out), "abs_max");
+        return value;
+    }
 #ifdef RL_TOOLS_ROCM_FORBID_HOST_ELEMENT_ACCESS
     // A tensor of this device is device memory: reading or writing one element from the host is never what a caller of this backend
     // means (on hosts that map device memory it works, slowly, and hides a missing overload: a generic host loop running over device

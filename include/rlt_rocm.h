@@ -101,6 +101,21 @@ int rlt_rocm_cast_reduce_sum_u8(rlt_rocm_device* device, const uint8_t* mask, si
 /* sum / squared-sum of a float tensor (gradient_norm, nn/parameters/operations_generic.h) */
 int rlt_rocm_reduce_sum_f32(rlt_rocm_device* device, const float* x, size_t count, int squared, float* out_sum);
 
+/* unary_operation(device, op, t[, output])   containers/tensor/operations_generic.h:573-640 with the functors of :365-446, on a 2-D view
+ * [rows x cols] (a contiguous tensor is one row); dst may be src. `parameter` is the functor's parameter (CONSTANT: the value; SCALE and
+ * SCALE_RECIPROCAL: the factor, the latter computing 1 / a * factor as Scale<..., RECIPROCAL> does). SIGMOID saturates beyond +-20 as :395-400. */
+enum { RLT_UNARY_NEGATE = 0, RLT_UNARY_ABS, RLT_UNARY_CONSTANT, RLT_UNARY_SIGMOID, RLT_UNARY_FAST_SIGMOID, RLT_UNARY_EXP, RLT_UNARY_TANH, RLT_UNARY_FAST_TANH,
+       RLT_UNARY_ONE_MINUS, RLT_UNARY_SCALE, RLT_UNARY_SCALE_RECIPROCAL };
+int rlt_rocm_unary_f32(rlt_rocm_device* device, int operation, float parameter, const float* src, int ld_src, float* dst, int ld_dst, int rows, int cols);
+/* binary_operation(device, op, a, b, output)   :641-700 with Add / Subtract / Multiply / Divide (:448-471); dst may be a or b */
+enum { RLT_BINARY_ADD = 0, RLT_BINARY_SUBTRACT, RLT_BINARY_MULTIPLY, RLT_BINARY_DIVIDE };
+int rlt_rocm_binary_f32(rlt_rocm_device* device, int operation, const float* a, int lda, const float* b, int ldb, float* dst, int ld_dst, int rows, int cols);
+/* ternary_operation with MultiplyAccumulate (:475-481, :701-760): dst = accumulator + a * b, the product rounded before the addition */
+int rlt_rocm_multiply_accumulate_f32(rlt_rocm_device* device, const float* a, int lda, const float* b, int ldb, const float* accumulator, int ldc,
+                                     float* dst, int ld_dst, int rows, int cols);
+/* unary_associative_reduce with the abs-max operation (:762-800; CUDA <<<1,1>>>, operations_cuda.h:287-307): max |x| into a device scalar (0 for count 0) */
+int rlt_rocm_reduce_abs_max_f32(rlt_rocm_device* device, const float* x, size_t count, float* out_max);
+
 /* ------------------------------------------------------------ dense / MLP -- */
 
 /* One dense layer as the reference stores it (nn/layers/dense/layer.h:82-135 plus the Adam

@@ -1031,6 +1031,57 @@ int rlt_oracle_pendulum_runner_step(const rlt_pendulum_runner* rn, const rlt_rep
     return rlt_oracle_pendulum_runner_epilogue(rn, rb, obs.data(), actions.data());
 }
 
+// The Tensor elementwise operations (containers/tensor/operations_generic.h:365-481 functors, :573-760 operations) on 2-D views
+static inline float fast_tanh_elementwise(float x) { x = std::min(std::max(x, -3.0f), 3.0f); const float x2 = x * x; return x * (27.0f + x2) / (27.0f + 9.0f * x2); }   // math/operations_generic.h:247-251
+int rlt_oracle_unary_f32(int operation, float parameter, const float* src, int ld_src, float* dst, int ld_dst, int rows, int cols) {
+    if (!src || !dst || rows <= 0 || cols <= 0 || operation < RLT_UNARY_NEGATE || operation > RLT_UNARY_SCALE_RECIPROCAL) return RLT_E_INVALID_ARGUMENT;
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) {
+            const float a = src[(size_t)r * ld_src + c];
+            float v = a;
+            switch (operation) {
+                case RLT_UNARY_NEGATE: v = -a; break;
+                case RLT_UNARY_ABS: v = std::fabs(a); break;
+                case RLT_UNARY_CONSTANT: v = parameter; break;
+                case RLT_UNARY_SIGMOID: v = a < -20 ? 0.0f : (a > 20 ? 1.0f : 1 / (1 + std::exp(-a))); break;       // :395-400
+                case RLT_UNARY_FAST_SIGMOID: v = 0.5f * fast_tanh_elementwise(0.5f * a) + 0.5f; break;                  // math/operations_generic.h:252-255
+                case RLT_UNARY_EXP: v = std::exp(a); break;
+                case RLT_UNARY_TANH: v = std::tanh(a); break;
+                case RLT_UNARY_FAST_TANH: v = fast_tanh_elementwise(a); break;
+                case RLT_UNARY_ONE_MINUS: v = 1 - a; break;
+                case RLT_UNARY_SCALE: v = a * parameter; break;
+                case RLT_UNARY_SCALE_RECIPROCAL: v = 1.0f / a * parameter; break;                                       // :436-441
+            }
+            dst[(size_t)r * ld_dst + c] = v;
+        }
+    return 0;
+}
+int rlt_oracle_binary_f32(int operation, const float* a, int lda, const float* b, int ldb, float* dst, int ld_dst, int rows, int cols) {
+    if (!a || !b || !dst || rows <= 0 || cols <= 0 || operation < RLT_BINARY_ADD || operation > RLT_BINARY_DIVIDE) return RLT_E_INVALID_ARGUMENT;
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) {
+            const float x = a[(size_t)r * lda + c], y = b[(size_t)r * ldb + c];
+            dst[(size_t)r * ld_dst + c] = operation == RLT_BINARY_ADD ? x + y : operation == RLT_BINARY_SUBTRACT ? x - y : operation == RLT_BINARY_MULTIPLY ? x * y : x / y;
+        }
+    return 0;
+}
+int rlt_oracle_multiply_accumulate_f32(const float* a, int lda, const float* b, int ldb, const float* accumulator, int ldc, float* dst, int ld_dst, int rows, int cols) {
+    if (!a || !b || !accumulator || !dst || rows <= 0 || cols <= 0) return RLT_E_INVALID_ARGUMENT;
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) {
+            volatile float product = a[(size_t)r * lda + c] * b[(size_t)r * ldb + c];      // rounded before the addition
+            dst[(size_t)r * ld_dst + c] = accumulator[(size_t)r * ldc + c] + product;
+        }
+    return 0;
+}
+int rlt_oracle_reduce_abs_max_f32(const float* x, size_t count, float* out_max) {
+    if (!x || !out_max) return RLT_E_INVALID_ARGUMENT;
+    float m = 0;
+    for (size_t i = 0; i < count; i++) m = std::max(m, std::fabs(x[i]));
+    *out_max = m;
+    return 0;
+}
+
 // step<POLICY>(device, runner, policy, ...) for any of the environments restated here: rl/components/off_policy_runner/operations_generic.h:183-238 over
 // prologue_per_env / epilogue_per_env (operations_generic_per_env.h:8-108). The environment-independent part (reset bookkeeping, counters,
 // truncated = terminated or step limit, replay add) is the Pendulum runner's, which the seeded SAC loop pins against the reference; the

@@ -116,6 +116,8 @@ class PendulumRunner(C.Structure):
                 ("n_envs", C.c_int32), ("episode_step_limit", C.c_int32), ("env", PendulumParameters)]
 
 
+UNARY = dict(negate=0, abs=1, constant=2, sigmoid=3, fast_sigmoid=4, exp=5, tanh=6, fast_tanh=7, one_minus=8, scale=9, scale_reciprocal=10)
+BINARY = dict(add=0, subtract=1, multiply=2, divide=3)
 ENV_PENDULUM, ENV_ACROBOT, ENV_ACROBOT_SWINGUP, ENV_CAR = 0, 1, 2, 3
 ENV_DIMS = {ENV_PENDULUM: (2, 3, 1), ENV_ACROBOT: (4, 6, 1), ENV_ACROBOT_SWINGUP: (4, 6, 1), ENV_CAR: (6, 6, 2)}      # state, observation, action widths
 
@@ -267,6 +269,10 @@ PROTOTYPES = {
     "mask_copy": [P, I, P, I, P, I, I, I],
     "mask_zero": [P, I, P, I, I, I],
     "scale_f32": [P, S, F, I],
+    "unary_f32": [I, F, P, I, P, I, I, I],
+    "binary_f32": [I, P, I, P, I, P, I, I, I],
+    "multiply_accumulate_f32": [P, I, P, I, P, I, P, I, I, I],
+    "reduce_abs_max_f32": [P, S, P],
     "cast_reduce_sum_u8": [P, S, P],
     "sac_train_critic": [C.POINTER(SacAgent), I, P],
     "sac_update_critic_targets": [C.POINTER(SacAgent)],

@@ -33,10 +33,33 @@ int main(){
     rlt::set_all(device, t_view, 0.0f);
     rlt::copy(device, cpu, t_dev, t_cpu);
     rlt::copy(cpu, device, t_cpu, t_dev);
+    // elementwise operations: the same calls on both devices, compared on the host
+    rlt::Tensor<rlt::tensor::Specification<T, TI, rlt::tensor::Shape<TI, 4, 8, 16>>> a_dev, b_dev, c_dev;
+    rlt::Tensor<rlt::tensor::Specification<T, DEVICE_CPU::index_t, rlt::tensor::Shape<DEVICE_CPU::index_t, 4, 8, 16>>> a_cpu, b_cpu, c_cpu, back;
+    rlt::malloc(device, a_dev); rlt::malloc(device, b_dev); rlt::malloc(device, c_dev);
+    rlt::malloc(cpu, a_cpu); rlt::malloc(cpu, b_cpu); rlt::malloc(cpu, c_cpu); rlt::malloc(cpu, back);
+    rlt::randn(device, a_dev, rng); rlt::rand(device, b_dev, rng, 0.5f, 2.0f); rlt::set_all(device, c_dev, 0.25f);
+    rlt::copy(device, cpu, a_dev, a_cpu); rlt::copy(device, cpu, b_dev, b_cpu); rlt::copy(device, cpu, c_dev, c_cpu);
+    T elementwise_diff = 0;
+    auto compare = [&](auto& on_device, auto& on_cpu){ rlt::copy(device, cpu, on_device, back); elementwise_diff += rlt::abs_diff(cpu, back, on_cpu); };
+    rlt::exp(device, a_dev, c_dev);                 rlt::exp(cpu, a_cpu, c_cpu);                 compare(c_dev, c_cpu);
+    rlt::sigmoid(device, a_dev, c_dev);             rlt::sigmoid(cpu, a_cpu, c_cpu);             compare(c_dev, c_cpu);
+    rlt::fast_sigmoid(device, a_dev, c_dev);        rlt::fast_sigmoid(cpu, a_cpu, c_cpu);        compare(c_dev, c_cpu);
+    rlt::tanh(device, a_dev, c_dev);                rlt::tanh(cpu, a_cpu, c_cpu);                compare(c_dev, c_cpu);
+    rlt::fast_tanh(device, a_dev, c_dev);           rlt::fast_tanh(cpu, a_cpu, c_cpu);           compare(c_dev, c_cpu);
+    rlt::one_minus(device, a_dev, c_dev);           rlt::one_minus(cpu, a_cpu, c_cpu);           compare(c_dev, c_cpu);
+    rlt::subtract(device, a_dev, b_dev, c_dev);     rlt::subtract(cpu, a_cpu, b_cpu, c_cpu);     compare(c_dev, c_cpu);
+    rlt::multiply(device, a_dev, b_dev, c_dev);     rlt::multiply(cpu, a_cpu, b_cpu, c_cpu);     compare(c_dev, c_cpu);
+    rlt::multiply_accumulate(device, a_dev, b_dev, c_dev); rlt::multiply_accumulate(cpu, a_cpu, b_cpu, c_cpu); compare(c_dev, c_cpu);
+    rlt::add(device, a_dev, b_dev);                 rlt::add(cpu, a_cpu, b_cpu);                 compare(b_dev, b_cpu);
+    rlt::abs(device, a_dev);                        rlt::abs(cpu, a_cpu);                        compare(a_dev, a_cpu);
+    const T max_dev = rlt::abs_max(device, b_dev), max_cpu = rlt::abs_max(cpu, b_cpu);
+    const bool elementwise_ok = elementwise_diff < 1e-3f && max_dev == max_cpu;      // 512 elements per comparison, a few ulp each
+    rlt::free(device, a_dev); rlt::free(device, b_dev); rlt::free(device, c_dev); rlt::free(cpu, a_cpu); rlt::free(cpu, b_cpu); rlt::free(cpu, c_cpu); rlt::free(cpu, back);
     rlt::check_status(device);
     T x = rlt::random::uniform_real_distribution(device.random, (T)0, (T)1, rng) + rlt::random::normal_distribution::sample(device.random, (T)0, (T)1, rng);
     TI k = rlt::random::uniform_int_distribution(device.random, (TI)0, (TI)9, rng);
     rlt::free(device, m_dev); rlt::free(device, m_dev2); rlt::free(cpu, m_cpu); rlt::free(cpu, m_cpu2); rlt::free(device, t_dev); rlt::free(cpu, t_cpu);
     rlt::free(device);
-    return (diff == 2500 * 5.5f && x > -10 && k < 10) ? 0 : 1;
+    return (diff == 2500 * 5.5f && x > -10 && k < 10 && elementwise_ok) ? 0 : 1;
 }
