@@ -247,29 +247,29 @@ def bench_gru(helpers, rocm, batch, S=64, I=146, H=64, iters=10):
     rows = S * batch
     head = helpers.Mlp(rocm, [H, 64, 4], helpers.xavier_params(rng, [H, 64, 4]), rows, "tanh", "identity")
     target = rocm.array(rng.standard_normal((rows, 4)).astype(np.float32))
-    d_out, d_h = rocm.zeros((rows, 4)), rocm.zeros((S, batch, H))
+    y_head, d_h = rocm.zeros((rows, 4)), rocm.zeros((S, batch, H))
     xd = rocm.array(x)
     moments = [rocm.zeros(a.shape) for a in (gru.W_i, gru.b_i, gru.W_h, gru.b_h) for _ in range(2)]
     tensors = []
     for k, (p, g, flag) in enumerate(((gru.W_i, gru.dW_i, 1), (gru.b_i, gru.db_i, 2), (gru.W_h, gru.dW_h, 1), (gru.b_h, gru.db_h, 2))):
         tensors.append(capi.AdamTensor(p.ptr, g.ptr, moments[2 * k].ptr, moments[2 * k + 1].ptr, None, int(np.prod(p.shape)), flag))
-    gru_adam = (capi.AdamTensor * 4)(*tensors)
+    # one optimiser for the whole model: the GRU's four tensors and the head's four in one Adam launch
+    tensors += [head.adam[i] for i in range(head.n_adam)]
+    model_adam = (capi.AdamTensor * len(tensors))(*tensors)
     age = rocm.array(np.array([1], np.uint32))
     adam = capi.adam_parameters(epsilon=1e-8)
     ws, wsn = head.workspace()
     ev = HipEvents(rocm.device.lib.rlt_rocm_get_stream(rocm.device.handle))
+    n_gru_gradients = int(np.prod(gru.grads.shape))
 
     def step():
-        for g in (gru.dW_i, gru.db_i, gru.dW_h, gru.db_h):
-            rocm.call("fill_f32", g.ptr, 1, int(np.prod(g.shape)), int(np.prod(g.shape)), 0.0)
+        rocm.call("fill_f32", gru.grads.ptr, 1, n_gru_gradients, n_gru_gradients, 0.0)      # the GRU's gradient tensors are one flat array
         rocm.call("mlp_zero_gradient", head.layers, head.n)
         rocm.call("gru_forward", C.byref(gru.c), xd.ptr, None, S, batch, gru.ws, gru.wsn)
-        rocm.call("mlp_forward", head.layers, head.n, gru.out.ptr, H, rows)
-        rocm.call("mse_gradient", head.out[-1].ptr, 4, target.ptr, 4, d_out.ptr, 4, rows, 4, 1.0, None)
-        rocm.call("mlp_backward", head.layers, head.n, gru.out.ptr, H, d_out.ptr, 4, d_h.ptr, H, rows, 1, ws, wsn)
+        # the head's forward, MSE gradient (2 / (rows * 4) * (y - target), loss weight 1) and backward_full with the gradient for the GRU's output
+        rocm.call("mlp_forward_backward_input", head.layers, head.n, gru.out.ptr, H, y_head.ptr, 4, None, 0, target.ptr, 4, 2.0 / (rows * 4), d_h.ptr, H, rows, ws, wsn)
         rocm.call("gru_backward", C.byref(gru.c), xd.ptr, d_h.ptr, None, None, S, batch, 1, gru.ws, gru.wsn)
-        rocm.call("adam_step", gru_adam, 4, C.byref(adam), age.ptr, 0.0, None)
-        rocm.call("adam_step", head.adam, head.n_adam, C.byref(adam), head.age.ptr, 0.0, None)
+        rocm.call("adam_step", model_adam, len(tensors), C.byref(adam), age.ptr, 0.0, None)
     for _ in range(3):
         step()
     rocm.sync()

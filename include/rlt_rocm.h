@@ -198,6 +198,16 @@ int rlt_rocm_mlp_forward_backward(rlt_rocm_device* device, const rlt_dense_layer
                                   const float* target, int ldt, float mse_scale,
                                   int batch, void* workspace, size_t workspace_bytes);
 
+/* The same with the gradient with respect to the input as a further output, d_input [batch x in] (overwritten): forward + loss gradient +
+ * backward_full of a network that sits on top of another model, e.g. a head in -> 64 -> out on a recurrent layer's output, in one pass over
+ * the batch where the network is in -> 64 -> out or in -> 64 -> 64 -> out (in <= 128, out <= 16). */
+int rlt_rocm_mlp_forward_backward_input(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers,
+                                        const float* x, int ldx, float* y, int ldy,
+                                        const float* d_output, int ldd,
+                                        const float* target, int ldt, float mse_scale,
+                                        float* d_input, int ldi,
+                                        int batch, void* workspace, size_t workspace_bytes);
+
 /* -------------------------------------------------------- optimiser/polyak -- */
 
 /* nn/optimizers/adam/adam.h:13-48 (Parameters<T>); the *_TENSORFLOW defaults are

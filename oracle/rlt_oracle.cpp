@@ -274,6 +274,11 @@ int rlt_oracle_mlp_zero_gradient(const rlt_dense_layer* layers, int n) {
 // with private activation storage so the caller's layers are left untouched.
 int rlt_oracle_mlp_forward_backward(const rlt_dense_layer* layers, int n, const float* x, int ldx, float* y, int ldy,
                                     const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch) {
+    return rlt_oracle_mlp_forward_backward_input(layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, nullptr, 0, batch);
+}
+// forward, loss gradient, backward_full (nn_models/mlp/operations_generic.h:128-260) with private activation storage
+int rlt_oracle_mlp_forward_backward_input(const rlt_dense_layer* layers, int n, const float* x, int ldx, float* y, int ldy,
+                                          const float* d_output, int ldd, const float* target, int ldt, float mse_scale, float* d_input, int ldi, int batch) {
     if (!layers || n < 1 || !x || batch <= 0 || (!d_output && !target)) return RLT_E_INVALID_ARGUMENT;
     std::vector<rlt_dense_layer> priv(layers, layers + n);
     std::vector<std::vector<float>> pre(n), out(n);
@@ -291,7 +296,7 @@ int rlt_oracle_mlp_forward_backward(const rlt_dense_layer* layers, int n, const 
             if (y) y[(size_t)b * ldy + o] = yv;
             d[(size_t)b * O + o] = target ? (yv - target[(size_t)b * ldt + o]) * mse_scale : d_output[(size_t)b * ldd + o];
         }
-    return rlt_oracle_mlp_backward(priv.data(), n, x, ldx, d.data(), O, nullptr, 0, batch, 1);
+    return rlt_oracle_mlp_backward(priv.data(), n, x, ldx, d.data(), O, d_input, ldi, batch, 1);
 }
 
 // nn/optimizers/adam/operations_generic.h:49-66 (_step: bias corrections from age, then age++) and

@@ -177,6 +177,8 @@ int rlt_oracle_unary_f32(int operation, float parameter, const float* src, int l
 int rlt_oracle_binary_f32(int operation, const float* a, int lda, const float* b, int ldb, float* dst, int ld_dst, int rows, int cols);
 int rlt_oracle_multiply_accumulate_f32(const float* a, int lda, const float* b, int ldb, const float* accumulator, int ldc, float* dst, int ld_dst, int rows, int cols);
 int rlt_oracle_reduce_abs_max_f32(const float* x, size_t count, float* out_max);
+int rlt_oracle_mlp_forward_backward_input(const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy, const float* d_output, int ldd,
+                                          const float* target, int ldt, float mse_scale, float* d_input, int ldi, int batch);
 int rlt_oracle_acrobot_step(const rlt_acrobot_parameters* p, int swingup, float* states, const float* actions, float* observations, float* next_observations,
                             float* rewards, uint8_t* terminated, int n_envs);
 /* rl/environments/car/operations_generic.h:80-155 (the Car without a track) */

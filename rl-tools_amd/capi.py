@@ -257,6 +257,7 @@ PROTOTYPES = {
     "mlp_backward": [LP, I, P, I, P, I, P, I, I, I, P, S],
     "mlp_zero_gradient": [LP, I],
     "mlp_forward_backward": [LP, I, P, I, P, I, P, I, P, I, F, I, P, S],
+    "mlp_forward_backward_input": [LP, I, P, I, P, I, P, I, P, I, F, P, I, I, P, S],
     "adam_step": [C.POINTER(AdamTensor), I, C.POINTER(AdamParameters), P, F, P],
     "adam_reset": [C.POINTER(AdamTensor), I, P],
     "polyak_update": [P, P, S, F, I],

@@ -180,33 +180,50 @@ int rlt_rocm_mlp_backward(rlt_rocm_device* device, const rlt_dense_layer* layers
 int rlt_rocm_mlp_zero_gradient(rlt_rocm_device* device, const rlt_dense_layer* layers, int n) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(layers && n >= 1);
-    for (int l = 0; l < n; l++) {
-        RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases && layers[l].in_dim > 0 && layers[l].out_dim > 0);
-        size_t nw = (size_t)layers[l].in_dim * layers[l].out_dim, nb = layers[l].out_dim;
-        int blocks = (int)((nw + nb + 255) / 256); if (blocks > 1024) blocks = 1024;
-        hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, device->stream, layers[l].d_weights, nw, layers[l].d_biases, nb);
-        int rc = rlt_launch_status(device);
+    for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases && layers[l].in_dim > 0 && layers[l].out_dim > 0);
+    // gradient tensors laid out back to back ([dW0 | db0 | dW1 | db1 | ...], the flat arena) are cleared by one launch, a run of layers at a time
+    for (int l = 0; l < n;) {
+        float* begin = layers[l].d_weights; float* end = begin;
+        int m = l;
+        for (; m < n; m++) {
+            const size_t nw = (size_t)layers[m].in_dim * layers[m].out_dim, nb = layers[m].out_dim;
+            if (layers[m].d_weights != end || layers[m].d_biases != end + nw) break;
+            end += nw + nb;
+        }
+        if (m == l) {       // this layer's two tensors lie apart
+            const size_t nw = (size_t)layers[l].in_dim * layers[l].out_dim, nb = layers[l].out_dim;
+            int blocks = (int)((nw + nb + 255) / 256); if (blocks > 1024) blocks = 1024;
+            hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, device->stream, layers[l].d_weights, nw, layers[l].d_biases, nb);
+            m = l + 1;
+        } else {
+            const size_t count = (size_t)(end - begin);
+            int blocks = (int)((count + 255) / 256); if (blocks > 1024) blocks = 1024;
+            hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, device->stream, begin, count, begin, (size_t)0);
+        }
+        const int rc = rlt_launch_status(device);
         if (rc) return rc;
+        l = m;
     }
     return 0;
 }
 
-int rlt_rocm_mlp_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n, const float* x, int ldx, float* y, int ldy,
+}  // extern "C"
+static int forward_backward_impl(rlt_rocm_device* device, const rlt_dense_layer* layers, int n, const float* x, int ldx, float* y, int ldy,
                                   const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch,
-                                  void* workspace, size_t workspace_bytes) {
+                                  void* workspace, size_t workspace_bytes, float* d_input, int ldi) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(chain_ok(layers, n) && x && batch > 0 && ldx >= layers[0].in_dim && (d_output || target));
     const int O = layers[n - 1].out_dim;
-    RLT_REQUIRE((!y || ldy >= O) && (!d_output || ldd >= O) && (!target || ldt >= O));
+    RLT_REQUIRE((!y || ldy >= O) && (!d_output || ldd >= O) && (!target || ldt >= O) && (!d_input || ldi >= layers[0].in_dim));
     for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases);
     RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_mlp_workspace_bytes(layers, n, batch));
-    {
+    if (!d_input) {
         // one pass over the batch with on-chip activations where the network has the shape that kernel is built for
         const int rc = rlt_mlp3_fused_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, workspace, workspace_bytes);
         if (rc != RLT_E_UNSUPPORTED) return rc;
     }
     if (single_pass_enabled()) {
-        const int rc = rlt_mlp3s_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch);
+        const int rc = rlt_mlp3s_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, d_input, ldi);
         if (rc != RLT_E_UNSUPPORTED) return rc;
     }
     // carve private activation storage out of the workspace
@@ -241,7 +258,20 @@ int rlt_rocm_mlp_forward_backward(rlt_rocm_device* device, const rlt_dense_layer
         const bool fo = last.pre_activations == nullptr;
         if ((rc = rlt_dpre(device, d_output, ldd, dlast, O, fo ? last.output : last.pre_activations, batch, O, last.activation, fo))) return rc;
     }
-    return mlp_backward_from_dpre(device, priv, n, x, ldx, dlast, O, nullptr, 0, batch, 1, tick, tock, true);
+    return mlp_backward_from_dpre(device, priv, n, x, ldx, dlast, O, d_input, ldi, batch, 1, tick, tock, true);
+}
+
+extern "C" {
+int rlt_rocm_mlp_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n, const float* x, int ldx, float* y, int ldy,
+                                  const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch, void* workspace, size_t workspace_bytes) {
+    return forward_backward_impl(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, workspace, workspace_bytes, nullptr, 0);
+}
+int rlt_rocm_mlp_forward_backward_input(rlt_rocm_device* device, const rlt_dense_layer* layers, int n, const float* x, int ldx, float* y, int ldy,
+                                        const float* d_output, int ldd, const float* target, int ldt, float mse_scale, float* d_input, int ldi, int batch,
+                                        void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(d_input);
+    return forward_backward_impl(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, workspace, workspace_bytes, d_input, ldi);
 }
 
 }  // extern "C"

@@ -2,13 +2,14 @@
 #pragma once
 #include "common.h"
 
-// true if the network has the shape the kernel is built for: 3 layers, in <= 128, both hidden widths 64 with the same activation
-// (relu, tanh or fast_tanh), out <= 16 with an activation whose derivative follows from the output
+// true if the network has a shape the kernel is built for: in -> 64 -> 64 -> out or in -> 64 -> out, in <= 128, hidden activation relu, tanh or
+// fast_tanh (the same in both hidden layers), out <= 16 with an activation whose derivative follows from the output
 bool rlt_mlp3s_supported(const rlt_dense_layer* layers, int n_layers);
 
-// same contract as rlt_rocm_mlp_forward_backward (partial sums live in the device handle's scratch); RLT_E_UNSUPPORTED if the shape does not fit
+// same contract as rlt_rocm_mlp_forward_backward (partial sums live in the device handle's scratch), plus the optional gradient with respect to x
+// into d_input [batch x in]; RLT_E_UNSUPPORTED if the shape does not fit
 int rlt_mlp3s_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy,
-                               const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch);
+                               const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch, float* d_input = nullptr, int ldi = 0);
 
 // PPO actor pass (rl/algorithms/ppo/operations_generic.h:203-285): forward, the clipped-surrogate gradient per sample, backward. `stats` =
 // {advantage mean, advantage std} on the device. Means go to `means` [batch x action_dim]; weight gradients are accumulated into the layers,

@@ -33,6 +33,7 @@ struct SmallArgs {
     const float* log_std; const float* actions; int ld_actions; const float* log_probs; int ld_lp; const float* advantages; int ld_adv; const float* stats;
     float epsilon_clip, advantage_epsilon; int normalize_advantage;
     float* partial; int count;      // per workgroup: dW1 [64 x in], db1 [64], dW2 [64 x 64], db2 [64], dW3 [out x 64], db3 [out], extra [16]
+    float* d_input; int ld_di;      // optional: gradient with respect to x, written at row b
 };
 
 __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
@@ -87,7 +88,9 @@ __device__ __forceinline__ void request_tile(const SmallArgs& A, uint32_t vrows,
 // tiles multiply zero columns and are never stored). Both are compile-time constants: a matrix instruction under a run-time
 // condition makes the compiler carry both versions of its accumulator.
 // One launch can carry two networks (PPO's actor and critic on the same minibatch): workgroups [0, groups0) work on A0, the rest on A1.
-template <int ACT_H, int NT1C>
+// LAYERS = 2: the network is in -> 64 -> out; layer 2, its weight gradient and its input gradient drop out, the output layer reads h1, and the
+// gradient at layer 1's pre-activations is formed directly from the output layer's.
+template <int ACT_H, int NT1C, int LAYERS>
 __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs A1, int groups0) {
     extern __shared__ float lds_raw[];
     const bool second = (int)blockIdx.x >= groups0;
@@ -108,7 +111,7 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
     request_tile(A, rows_next, lane, T);
     float b1r[4], b2r[4];
 #pragma unroll
-    for (int nt = 0; nt < 4; nt++) { b1r[nt] = A.b1[16 * nt + r]; b2r[nt] = A.b2[16 * nt + r]; }
+    for (int nt = 0; nt < 4; nt++) { b1r[nt] = A.b1[16 * nt + r]; b2r[nt] = LAYERS == 3 ? A.b2[16 * nt + r] : 0.f; }
     const float b3r = A.b3[min(r, OUT - 1)];
     float ls = 0.f, adv_mean = 0.f, adv_std = 0.f;
     if (A.loss == LOSS_PPO) {
@@ -126,7 +129,7 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
             v1[j][1] = IN > 64 ? src[min(64 + lane, IN - 1)] : 0.f;
         }
 #pragma unroll
-        for (int u = 0; u < H * H / THREADS; u++) v2[u] = A.W2[u * THREADS + threadIdx.x];
+        for (int u = 0; u < H * H / THREADS; u++) v2[u] = LAYERS == 3 ? A.W2[u * THREADS + threadIdx.x] : 0.f;
 #pragma unroll
         for (int u = 0; u < MAX_OUT * H / THREADS; u++) v3[u] = A.W3[min(u * THREADS + (int)threadIdx.x, OUT * H - 1)];
 #pragma unroll
@@ -209,26 +212,29 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
         wave_sync();
 
         // layer 2
+        if (LAYERS == 3) {
 #pragma unroll
-        for (int nt = 0; nt < 4; nt++) acc[nt] = zero4;
+            for (int nt = 0; nt < 4; nt++) acc[nt] = zero4;
 #pragma unroll
-        for (int s = 0; s < 16; s++) {
-            const float a = h1s[r * HS + 16 * kk + s];
+            for (int s = 0; s < 16; s++) {
+                const float a = h1s[r * HS + 16 * kk + s];
 #pragma unroll
-            for (int nt = 0; nt < 4; nt++) acc[nt] = mfma16(a, w2s[(16 * nt + r) * HS + 16 * kk + s], acc[nt]);
+                for (int nt = 0; nt < 4; nt++) acc[nt] = mfma16(a, w2s[(16 * nt + r) * HS + 16 * kk + s], acc[nt]);
+            }
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) h2s[(4 * kk + v) * HS + 16 * nt + r] = rlt_act(acc[nt][v] + b2r[nt], ACT_H);
+            wave_sync();
         }
-#pragma unroll
-        for (int nt = 0; nt < 4; nt++)
-#pragma unroll
-            for (int v = 0; v < 4; v++) h2s[(4 * kk + v) * HS + 16 * nt + r] = rlt_act(acc[nt][v] + b2r[nt], ACT_H);
-        wave_sync();
+        const lptr hls = LAYERS == 3 ? h2s : h1s, hls_all = LAYERS == 3 ? h2s_all : h1s_all;      // the last hidden layer's activations
 
         // layer 3 (two chains of matrix instructions) and the gradient at its pre-activations
         floatx4 y0 = zero4, y1 = zero4;
 #pragma unroll
         for (int s = 0; s < 16; s += 2) {
-            y0 = mfma16(h2s[r * HS + 16 * kk + s], w3s[r * HS + 16 * kk + s], y0);
-            y1 = mfma16(h2s[r * HS + 16 * kk + s + 1], w3s[r * HS + 16 * kk + s + 1], y1);
+            y0 = mfma16(hls[r * HS + 16 * kk + s], w3s[r * HS + 16 * kk + s], y0);
+            y1 = mfma16(hls[r * HS + 16 * kk + s + 1], w3s[r * HS + 16 * kk + s + 1], y1);
         }
 #pragma unroll
         for (int v = 0; v < 4; v++) {
@@ -259,15 +265,15 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
             s3 += dp;
             d3s[(4 * kk + v) * D3S + r] = dp;
         }
-        rlt_lds_barrier();      // every wavefront's h2 and d_pre3 are in place
+        rlt_lds_barrier();      // every wavefront's last hidden activations and d_pre3 are in place
 
-        // dW3 (columns 16 wave + r) += d_pre3^T h2 over the 64 rows, two chains
+        // dW3 (columns 16 wave + r) += d_pre3^T h over the 64 rows, two chains
         {
-            float a_c = d3s_all[kk * D3S + r], b_c = h2s_all[kk * HS + 16 * wave + r];
+            float a_c = d3s_all[kk * D3S + r], b_c = hls_all[kk * HS + 16 * wave + r];
 #pragma unroll
             for (int ks = 0; ks < ROWS / 4; ks++) {
                 const int kn = min(ks + 1, ROWS / 4 - 1);
-                const float a_n = d3s_all[(4 * kn + kk) * D3S + r], b_n = h2s_all[(4 * kn + kk) * HS + 16 * wave + r];
+                const float a_n = d3s_all[(4 * kn + kk) * D3S + r], b_n = hls_all[(4 * kn + kk) * HS + 16 * wave + r];
                 if (ks & 1) aW3b = mfma16(a_c, b_c, aW3b); else aW3a = mfma16(a_c, b_c, aW3a);
                 a_c = a_n; b_c = b_n;
             }
@@ -286,10 +292,12 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const int idx = (4 * kk + v) * HS + 16 * nt + r;
-                const float dp = acc[nt][v] * rlt_dact_from_output(h2s[idx], ACT_H);
-                g2s[idx] = dp; s2[nt] += dp;
+                const float dp = acc[nt][v] * rlt_dact_from_output(hls[idx], ACT_H);
+                if (LAYERS == 3) { g2s[idx] = dp; s2[nt] += dp; }
+                else { h2s[idx] = dp; s1[nt] += dp; }       // two layers: this is already the gradient at layer 1's pre-activations, kept where dW1 reads it
             }
         rlt_lds_barrier();      // every wavefront's d_pre2 is in place, and nobody reads h2 any more
+        if (LAYERS == 3) {
 
         // dW2 (rows 16 wave + ..) += d_pre2^T h1 over the 64 rows
         {
@@ -327,6 +335,19 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
                 h2s[idx] = dp; s1[nt] += dp;
             }
         rlt_lds_barrier();      // every wavefront's d_pre1 is in place
+        }
+
+        // gradient with respect to the input, for the wavefront's own rows: d_x = d_pre1 W1, one tile of 16 input columns at a time
+        if (A.d_input) {
+            for (int nt = 0; nt < NT1; nt++) {
+                floatx4 dx = zero4;
+#pragma unroll
+                for (int s = 0; s < 16; s++) dx = mfma16(h2s[r * HS + 16 * kk + s], w1s[(16 * kk + s) * SX + 16 * nt + r], dx);
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+                    if (row0 + 4 * kk + v < A.batch && 16 * nt + r < IN) A.d_input[(size_t)(row0 + 4 * kk + v) * A.ld_di + 16 * nt + r] = dx[v];
+            }
+        }
 
         // dW1 (rows 16 wave + ..) += d_pre1^T x over the 64 rows
         {
@@ -412,8 +433,8 @@ __global__ __launch_bounds__(256) void mlp3s_reduce_kernel(SmallTargets T0, Smal
     int i = e, n = H * T.in;
     if (i < n) slot = T.dW1 + i;
     else if ((i -= n) < H) slot = T.db1 + i;
-    else if ((i -= H) < H * H) slot = T.dW2 + i;
-    else if ((i -= H * H) < H) slot = T.db2 + i;
+    else if ((i -= H) < H * H) slot = T.dW2 ? T.dW2 + i : nullptr;      // a two-layer network has no middle layer: its block entries are skipped
+    else if ((i -= H * H) < H) slot = T.db2 ? T.db2 + i : nullptr;
     else if ((i -= H) < T.out * H) slot = T.dW3 + i;
     else if ((i -= T.out * H) < T.out) slot = T.db3 + i;
     else if ((i -= T.out) < T.n_extra && T.extra) { slot = T.extra + i; total = total * T.extra_scale + T.extra_offset; }
@@ -423,9 +444,12 @@ __global__ __launch_bounds__(256) void mlp3s_reduce_kernel(SmallTargets T0, Smal
 bool hidden_act_ok(int a) { return a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH; }
 bool out_act_ok(int a) { return a == RLT_ACT_IDENTITY || a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH || a == RLT_ACT_SIGMOID; }
 
-struct SmallJob { const rlt_dense_layer* L; SmallArgs a; float* extra; int n_extra; float extra_scale, extra_offset; int overwrite; };
+struct SmallJob { const rlt_dense_layer* L; int n_layers; SmallArgs a; float* extra; int n_extra; float extra_scale, extra_offset; int overwrite; };
 
 bool shape_ok(const rlt_dense_layer* L, int n) {
+    if (L && n == 2)
+        return L[0].in_dim >= 1 && L[0].in_dim <= MAX_IN && L[0].out_dim == H && L[1].in_dim == H && L[1].out_dim >= 1 && L[1].out_dim <= MAX_OUT &&
+               hidden_act_ok(L[0].activation) && out_act_ok(L[1].activation);
     return L && n == 3 && L[0].in_dim >= 1 && L[0].in_dim <= MAX_IN && L[0].out_dim == H && L[1].in_dim == H && L[1].out_dim == H && L[2].in_dim == H &&
            L[2].out_dim >= 1 && L[2].out_dim <= MAX_OUT && L[0].activation == L[1].activation && hidden_act_ok(L[0].activation) && out_act_ok(L[2].activation);
 }
@@ -437,9 +461,11 @@ int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
     size_t offset[2] = {0, 0}, total = 0;
     for (int j = 0; j < n_jobs; j++) {
         const rlt_dense_layer* L = jobs[j].L; SmallArgs& a = jobs[j].a;
-        for (int l = 0; l < 3; l++) RLT_REQUIRE(L[l].weights && L[l].biases && L[l].d_weights && L[l].d_biases);
-        a.in = L[0].in_dim; a.out = L[2].out_dim; a.act3 = L[2].activation;
-        a.W1 = L[0].weights; a.b1 = L[0].biases; a.W2 = L[1].weights; a.b2 = L[1].biases; a.W3 = L[2].weights; a.b3 = L[2].biases;
+        const int n = jobs[j].n_layers, last = n - 1;
+        RLT_REQUIRE((n == 2 || n == 3) && n == jobs[0].n_layers);
+        for (int l = 0; l < n; l++) RLT_REQUIRE(L[l].weights && L[l].biases && L[l].d_weights && L[l].d_biases);
+        a.in = L[0].in_dim; a.out = L[last].out_dim; a.act3 = L[last].activation;
+        a.W1 = L[0].weights; a.b1 = L[0].biases; a.W2 = n == 3 ? L[1].weights : nullptr; a.b2 = n == 3 ? L[1].biases : nullptr; a.W3 = L[last].weights; a.b3 = L[last].biases;
         a.count = H * a.in + H + H * H + H + a.out * H + a.out + N_EXTRA;
         const int rounds = (a.batch + ROWS - 1) / ROWS, share = device->compute_units / n_jobs;
         groups[j] = rounds < share ? rounds : share;
@@ -455,10 +481,16 @@ int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
     for (int j = 0; j < n_jobs; j++) jobs[j].a.partial = (float*)scratch + offset[j];
     const SmallArgs& a0 = jobs[0].a; const SmallArgs& a1 = jobs[n_jobs - 1].a;
     const int grid = groups[0] + (n_jobs == 2 ? groups[1] : 0);
-#define RLT_LAUNCH_SMALL(ACT, NT)                                                                                                                         \
-    do {                                                                                                                                                  \
-        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp3s_kernel<ACT, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
-        hipLaunchKernelGGL((mlp3s_kernel<ACT, NT>), dim3(grid), dim3(THREADS), lds_bytes, device->stream, a0, a1, groups[0]);                           \
+    const bool two_layers = jobs[0].n_layers == 2;
+#define RLT_LAUNCH_SMALL(ACT, NT)                                                                                                                               \
+    do {                                                                                                                                                        \
+        if (two_layers) {                                                                                                                                       \
+            RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp3s_kernel<ACT, NT, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
+            hipLaunchKernelGGL((mlp3s_kernel<ACT, NT, 2>), dim3(grid), dim3(THREADS), lds_bytes, device->stream, a0, a1, groups[0]);                           \
+        } else {                                                                                                                                                \
+            RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp3s_kernel<ACT, NT, 3>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
+            hipLaunchKernelGGL((mlp3s_kernel<ACT, NT, 3>), dim3(grid), dim3(THREADS), lds_bytes, device->stream, a0, a1, groups[0]);                           \
+        }                                                                                                                                                       \
     } while (0)
     switch (act) {
         case RLT_ACT_RELU: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_RELU, 2); else RLT_LAUNCH_SMALL(RLT_ACT_RELU, MAX_NT1); break;
@@ -472,7 +504,8 @@ int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
     for (int j = 0; j < n_jobs; j++) {
         const rlt_dense_layer* L = jobs[j].L; const SmallArgs& a = jobs[j].a;
         const int count = jobs[j].extra ? a.count : a.count - N_EXTRA;      // the extra slots sit at the end of a block
-        T[j] = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases, jobs[j].extra, a.in, a.out, jobs[j].n_extra,
+        const int last = jobs[j].n_layers - 1;
+        T[j] = {L[0].d_weights, L[0].d_biases, last == 2 ? L[1].d_weights : nullptr, last == 2 ? L[1].d_biases : nullptr, L[last].d_weights, L[last].d_biases, jobs[j].extra, a.in, a.out, jobs[j].n_extra,
                 jobs[j].extra_scale, jobs[j].extra_offset, jobs[j].overwrite, a.partial, groups[j], a.count, (count + 63) / 64};
         blocks += T[j].blocks;
     }
@@ -481,10 +514,10 @@ int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
     return rlt_launch_status(device);
 }
 
-SmallJob plain_job(const rlt_dense_layer* L, const float* x, int ldx, float* y, int ldy, const float* d_output, int ldd, const float* target, int ldt, float mse_scale,
-                   int batch, int overwrite, const uint32_t* rows) {
+SmallJob plain_job(const rlt_dense_layer* L, int n_layers, const float* x, int ldx, float* y, int ldy, const float* d_output, int ldd, const float* target, int ldt, float mse_scale,
+                   int batch, int overwrite, const uint32_t* rows, float* d_input = nullptr, int ld_di = 0) {
     SmallJob job = {};
-    job.L = L; job.overwrite = overwrite;
+    job.L = L; job.n_layers = n_layers; job.overwrite = overwrite; job.a.d_input = d_input; job.a.ld_di = ld_di;
     SmallArgs& a = job.a;
     a.rows = rows; a.x = x; a.ldx = ldx; a.batch = batch; a.y = y; a.ldy = ldy;
     a.loss = target ? LOSS_MSE : LOSS_GIVEN; a.d_output = d_output; a.ldd = ldd; a.target = target; a.ldt = ldt; a.mse_scale = mse_scale;
@@ -494,7 +527,7 @@ SmallJob ppo_actor_job(const rlt_dense_layer* L, const float* x, int ldx, float*
                        const float* log_probs, int ld_lp, const float* advantages, int ld_adv, const float* stats, const rlt_ppo_parameters* P, float* d_log_std,
                        float log_std_gradient_offset, int batch, int overwrite, const uint32_t* rows) {
     SmallJob job = {};
-    job.L = L; job.overwrite = overwrite; job.extra = d_log_std; job.n_extra = L[2].out_dim; job.extra_scale = 1.0f; job.extra_offset = log_std_gradient_offset;
+    job.L = L; job.n_layers = 3; job.overwrite = overwrite; job.extra = d_log_std; job.n_extra = L[2].out_dim; job.extra_scale = 1.0f; job.extra_offset = log_std_gradient_offset;
     SmallArgs& a = job.a;
     a.rows = rows; a.x = x; a.ldx = ldx; a.batch = batch; a.y = means; a.ldy = ld_means;
     a.loss = LOSS_PPO; a.log_std = log_std; a.actions = actions; a.ld_actions = ld_actions; a.log_probs = log_probs; a.ld_lp = ld_lp;
@@ -519,23 +552,23 @@ int rlt_mlp3s_reduce(rlt_rocm_device* device, const rlt_dense_layer* L, const fl
 }
 
 int rlt_mlp3s_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n, const float* x, int ldx, float* y, int ldy, const float* d_output, int ldd,
-                               const float* target, int ldt, float mse_scale, int batch) {
+                               const float* target, int ldt, float mse_scale, int batch, float* d_input, int ldi) {
     if (!shape_ok(L, n)) return RLT_E_UNSUPPORTED;
-    SmallJob job = plain_job(L, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, 0, nullptr);
+    SmallJob job = plain_job(L, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, 0, nullptr, d_input, ldi);
     return launch(device, &job, 1);
 }
 
 int rlt_mlp3s_ppo_actor(rlt_rocm_device* device, const rlt_dense_layer* L, int n, const float* x, int ldx, float* means, int ld_means, const float* log_std,
                         const float* actions, int ld_actions, const float* log_probs, int ld_lp, const float* advantages, int ld_adv, const float* stats,
                         const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset, int batch) {
-    if (!shape_ok(L, n)) return RLT_E_UNSUPPORTED;
+    if (!shape_ok(L, n) || n != 3) return RLT_E_UNSUPPORTED;
     SmallJob job = ppo_actor_job(L, x, ldx, means, ld_means, log_std, actions, ld_actions, log_probs, ld_lp, advantages, ld_adv, stats, P, d_log_std,
                                  log_std_gradient_offset, batch, 0, nullptr);
     return launch(device, &job, 1);
 }
 
 bool rlt_mlp3s_pair_supported(const rlt_dense_layer* a, int n_a, const rlt_dense_layer* b, int n_b) {
-    return shape_ok(a, n_a) && shape_ok(b, n_b) && a[0].activation == b[0].activation && tile_bucket(a[0].in_dim) == tile_bucket(b[0].in_dim);
+    return n_a == 3 && n_b == 3 && shape_ok(a, n_a) && shape_ok(b, n_b) && a[0].activation == b[0].activation && tile_bucket(a[0].in_dim) == tile_bucket(b[0].in_dim);
 }
 
 int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* actor, int n_actor, const float* x, float* means, int ld_means,
@@ -546,7 +579,7 @@ int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* a
     if (!rlt_mlp3s_pair_supported(actor, n_actor, critic, n_critic) || (out_critic_loss && critic[2].out_dim != 1)) return RLT_E_UNSUPPORTED;
     SmallJob jobs[2] = {ppo_actor_job(actor, x, ld, means, ld_means, log_std, actions, ld, log_probs, ld, advantages, ld, stats, P, d_log_std,
                                       log_std_gradient_offset, batch, 1, rows),
-                        plain_job(critic, x_critic, ld, values, ld_values, nullptr, 0, target_values, ld, mse_scale, batch, 1, rows)};
+                        plain_job(critic, 3, x_critic, ld, values, ld_values, nullptr, 0, target_values, ld, mse_scale, batch, 1, rows)};
     if (out_critic_loss) { jobs[1].extra = out_critic_loss; jobs[1].n_extra = 1; jobs[1].extra_scale = 1.0f / (float)batch; jobs[1].extra_offset = 0.0f; }
     return launch(device, jobs, 2);
 }

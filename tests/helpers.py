@@ -43,7 +43,7 @@ class LoopConfig(C.Structure):
                 ("n_warmup_steps", C.c_int32), ("episode_step_limit", C.c_int32), ("adam_epsilon", C.c_float)]
 
 
-WITH_WORKSPACE = ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "gru_forward", "gru_backward", "on_policy_collect", "seq_forward", "seq_backward", "seq_evaluate_step",
+WITH_WORKSPACE = ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "mlp_forward_backward_input", "gru_forward", "gru_backward", "on_policy_collect", "seq_forward", "seq_backward", "seq_evaluate_step",
                   "pendulum_runner_step_recurrent", "pendulum_evaluate_recurrent", "env_runner_step", "env_on_policy_collect", "env_runner_step_sequential")
 
 
@@ -237,14 +237,29 @@ REF_GRU_GENERIC = os.path.join(ORACLE_DIR, "_ref", "librlt_ref_gru_generic.so")
 REF_GRU_FAST_GENERIC = os.path.join(ORACLE_DIR, "_ref", "librlt_ref_gru_fast_generic.so")
 
 
+class ArenaView:
+    """A tensor inside a flat array of a backend: what the C ABI needs of it (`ptr`) and its contents."""
+
+    def __init__(self, arena, start, shape):
+        self.arena, self.start, self.shape = arena, start, tuple(shape)
+        self.ptr = arena.offset(start)
+
+    def numpy(self):
+        n = int(np.prod(self.shape))
+        return self.arena.numpy()[self.start:self.start + n].reshape(self.shape)
+
+
 class GruOnBackend:
-    """One GRU layer (parameters, gradients, kept intermediates) on a backend. params: dict W_i [3H x I], b_i, W_h [3H x H], b_h, h0."""
+    """One GRU layer (parameters, gradients, kept intermediates) on a backend. params: dict W_i [3H x I], b_i, W_h [3H x H], b_h, h0.
+    The four gradient tensors share one flat array (`grads`), so that one fill clears them."""
 
     def __init__(self, backend, S, B, I, H, params, fast_tanh=False):
         self.backend, self.S, self.B, self.I, self.H = backend, S, B, I, H
         f = lambda k: backend.array(np.asarray(params[k], np.float32))
         self.W_i, self.b_i, self.W_h, self.b_h, self.h0 = f("W_i"), f("b_i"), f("W_h"), f("b_h"), f("h0")
-        self.dW_i, self.db_i, self.dW_h, self.db_h = backend.zeros((3 * H, I)), backend.zeros((3 * H,)), backend.zeros((3 * H, H)), backend.zeros((3 * H,))
+        self.grads = backend.zeros((3 * H * I + 3 * H + 3 * H * H + 3 * H,))
+        self.dW_i, self.db_i = ArenaView(self.grads, 0, (3 * H, I)), ArenaView(self.grads, 3 * H * I, (3 * H,))
+        self.dW_h, self.db_h = ArenaView(self.grads, 3 * H * I + 3 * H, (3 * H, H)), ArenaView(self.grads, 3 * H * I + 3 * H + 3 * H * H, (3 * H,))
         self.post, self.npp, self.out = backend.zeros((S, B, 3 * H)), backend.zeros((S, B, H)), backend.zeros((S, B, H))
         self.c = capi.GruLayer(self.W_i.ptr, self.b_i.ptr, self.W_h.ptr, self.b_h.ptr, self.h0.ptr, self.dW_i.ptr, self.db_i.ptr, self.dW_h.ptr, self.db_h.ptr,
                                self.post.ptr, self.npp.ptr, self.out.ptr, I, H, int(fast_tanh), 0)

@@ -135,3 +135,46 @@ def test_ppo_update_narrow_networks_against_per_layer_kernels(rocm, monkeypatch,
     got, want = results
     for key in want:
         assert rel_err(got[key], want[key]) <= TOL, (key, rel_err(got[key], want[key]))
+
+
+# (batch, layer widths, hidden activation, output activation, MSE target instead of a given gradient)
+INPUT_GRADIENT_CASES = [(4096, [64, 64, 4], "tanh", "identity", True),        # the head of the sequence-model benchmark on a recurrent layer's output
+                        (300, [17, 64, 6], "relu", "identity", False), (70, [128, 64, 16], "fast_tanh", "tanh", False), (1, [3, 64, 1], "relu", "identity", True),
+                        (513, [33, 64, 64, 9], "relu", "identity", False), (256, [4, 64, 64, 1], "tanh", "identity", True),
+                        (200, [20, 48, 5], "relu", "identity", True)]          # hidden width 48: the per-layer kernels with the same contract
+
+
+@pytest.mark.parametrize("case", INPUT_GRADIENT_CASES)
+def test_forward_backward_with_input_gradient(oracle, rocm, case):
+    """rlt_rocm_mlp_forward_backward_input on two- and three-layer networks: output, weight gradients (accumulated twice) and the gradient with
+    respect to the input against the checker's forward / backward_full."""
+    B, dims, ha, oa, use_target = case
+    rng = np.random.default_rng(B + len(dims))
+    params = helpers.random_params(rng, dims)
+    x = rng.standard_normal((B, dims[0])).astype(np.float32); dy = rng.standard_normal((B, dims[-1])).astype(np.float32)
+    results = []
+    for backend in (oracle, rocm):
+        net = Mlp(backend, dims, params, B, ha, oa)
+        xd, yd, dyd = backend.array(x), backend.zeros((B, dims[-1])), backend.array(dy)
+        dx = backend.array(np.full((B, dims[0] + 3), 7.0, np.float32))      # a pitch: the three extra columns must stay untouched
+        ws, wsn = net.workspace()
+        backend.call("mlp_zero_gradient", net.layers, net.n)
+        for _ in range(2):
+            if use_target:
+                backend.call("mlp_forward_backward_input", net.layers, net.n, xd.ptr, dims[0], yd.ptr, dims[-1], None, 0, dyd.ptr, dims[-1], 2.0 / B, dx.ptr, dims[0] + 3, B, ws, wsn)
+            else:
+                backend.call("mlp_forward_backward_input", net.layers, net.n, xd.ptr, dims[0], yd.ptr, dims[-1], dyd.ptr, dims[-1], None, 0, 0.0, dx.ptr, dims[0] + 3, B, ws, wsn)
+        backend.sync()
+        results.append((yd.numpy(), net.grads.numpy(), dx.numpy()))
+    (wy, wg, wdx), (gy, gg, gdx) = results
+    assert rel_err(gy, wy) <= TOL
+    assert np.all(gdx[:, dims[0]:] == 7.0)
+    if ha == "relu" and max(rel_err(gg, wg), rel_err(gdx[:, :dims[0]], wdx[:, :dims[0]])) > TOL:
+        net = Mlp(oracle, dims, params, B, ha, oa)
+        xd = oracle.array(x)
+        oracle.call("mlp_forward", net.layers, net.n, xd.ptr, dims[0], B)
+        near = min(np.abs(p.numpy()).min() for p in net.pre[:-1])
+        assert near <= 1e-6, (near, rel_err(gg, wg))      # a pre-activation within rounding of zero switched sides
+        return
+    assert rel_err(gg, wg) <= TOL
+    assert rel_err(gdx[:, :dims[0]], wdx[:, :dims[0]]) <= TOL
