@@ -247,6 +247,9 @@ int rlt_rocm_adam_reset(rlt_rocm_device* device, const rlt_adam_tensor* tensors_
 /* utils::polyak::update / update_squared   utils/polyak/operations_generic.h:11-43, operations_cuda.h:13-48 */
 int rlt_rocm_polyak_update(rlt_rocm_device* device, const float* source, float* target, size_t count,
                            float polyak, int squared);
+/* The same soft update for a list of tensors (e.g. every tensor of both target critics) in one launch per 16 tensors. */
+int rlt_rocm_polyak_update_list(rlt_rocm_device* device, const float* const* sources, float* const* targets, const uint32_t* counts,
+                                int n_tensors, float polyak);
 
 /* ------------------------------------------------------------------- loss -- */
 

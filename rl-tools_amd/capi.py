@@ -336,6 +336,7 @@ ROCM_ONLY = {
     "reduce_sum_f32": ([P, P, S, I, P], I),
     "dense_backward_static": ([P, LP, P, I, P, I, I], I),
     "sac_set_per_operation": ([P, I], I),
+    "polyak_update_list": ([P, P, P, P, I, F], I),
     "env_dims": ([I, C.POINTER(I), C.POINTER(I), C.POINTER(I)], I),
     "env_runner_step_workspace_bytes": ([C.POINTER(EnvRunner), I, LP, I], S),
     "env_runner_step_sequential_workspace_bytes": ([C.POINTER(EnvRunner), C.POINTER(SeqLayer), I], S),

@@ -592,3 +592,10 @@ int rlt_sac_polyak_list(rlt_rocm_device* device, const float* const* sources, fl
     }
     return 0;
 }
+
+extern "C" int rlt_rocm_polyak_update_list(rlt_rocm_device* device, const float* const* sources, float* const* targets, const uint32_t* counts, int n_tensors, float polyak) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(sources && targets && counts && n_tensors >= 0);
+    for (int i = 0; i < n_tensors; i++) RLT_REQUIRE(sources[i] && targets[i]);
+    return rlt_sac_polyak_list(device, sources, targets, counts, n_tensors, polyak);
+}

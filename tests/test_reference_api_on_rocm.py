@@ -64,4 +64,6 @@ def test_the_references_sac_loop_learns_the_pendulum_on_rocm():
     rate = float(re.search(r"loop_steps_per_second_including_evaluations ([\d.]+)", out.stdout).group(1))
     assert returns[0] < -600                                  # the untrained actor
     assert sorted(returns[1:])[int(len(returns[1:]) * 0.8)] > -200 and final > -250
-    assert rate > 300                                         # every operation runs on the device: the host-loop fallback manages 8 steps per second
+    # every operation runs on the device (the host-loop fallback manages 8 steps per second), and the update calls resolve to the overloads
+    # that hand a whole update to the library (through the leaf overloads alone the loop runs at about 1,500 steps per second)
+    assert rate > 3000
