@@ -3,18 +3,26 @@
 // reference: rl/algorithms/sac/operations_generic.h:243-337 (train_critic), :395-468 (train_actor),
 //            nn/layers/sample_and_squash/operations_generic.h:148-398, nn_models/mlp/operations_generic.h:128-260.
 //
-// A workgroup of four wavefronts takes 64 rows of the batch, each wavefront its own 16 rows, through every pass of the update:
-//   critic update   actor on the next observations -> squashed sample and its log-probability -> both target critics -> TD target ->
-//                   critic forward, MSE gradient, backward
-//   actor update    actor forward -> squashed sample -> both critics forward and input gradient with d_output = -1 / batch -> gradient of
-//                   the smaller value per row -> sample_and_squash backward (entropy term, log_alpha gradient) -> actor backward
-// The networks take turns in one LDS region for the weights (staged by the whole workgroup between two barriers); activations stay in
-// LDS in the operand layouts of v_mfma_f32_16x16x4_f32 (lane l = r + 16 kk feeds A[r][kk] and B[kk][r], receives D[4 kk + v][r]). The
-// weight gradients of the trained network are reductions over the workgroup's 64 rows, split by output columns across the wavefronts
-// (wavefront w owns rows 16 w .. 16 w + 15 of dW1 and dW2 and 16 columns of dW3), so every accumulator tile lives in one wavefront's
-// registers; a workgroup writes one block of partial sums, which the reduction kernel of the small-MLP path adds up in workgroup order
-// (OVERWRITING the gradients: what zero_gradient followed by backward leaves). The Adam step is the library's usual launch.
-// Bound: latency (a batch of 256 is four workgroups); the point of this path is three launches per update instead of about twenty.
+// A workgroup of two teams of four wavefronts takes 16 rows of the batch through every pass of the update:
+//   critic update   stage A: actor on the next observations (team 0) | trained critic on the current rows (team 1)
+//                   -> squashed sample and its log-probability -> stage B: target critic 0 (team 0) | target critic 1 (team 1)
+//                   -> TD target, MSE gradient -> stage C: critic backward (team 1)
+//   actor update    stage A: actor forward (team 1) -> squashed sample -> stage B: critic 0 | critic 1 forward and input gradient with
+//                   d_output = -1 / batch -> gradient of the smaller value per row -> sample_and_squash backward (entropy term,
+//                   log_alpha gradient) -> stage C: actor backward (team 1)
+// The update is a chain of small dependent matrix products, so its duration is the length of that chain: independent networks run side
+// by side, and the four wavefronts of a team share every link of one network. Wavefront w of a team owns hidden units 16 w .. 16 w + 15:
+// in a hidden layer it computes that tile of the 16 x 64 activations from the whole previous layer (which the others read after a
+// workgroup barrier), in the output layer it contributes the quarter of the reduction that its units feed (the four partial tiles are
+// added in a fixed order), in the backward pass it owns the same units' pre-activation gradients and the rows of dW1, dW2 and columns of
+// dW3 that belong to them. The per-row arithmetic between the network passes (sample_and_squash, TD target, loss gradients) is one
+// wavefront's work.
+// Parameters go from global memory straight into the registers that feed v_mfma_f32_16x16x4_f32 as B operands (each wavefront needs
+// only its own units' rows and columns), all requested at the start of the kernel; activations stay in LDS in the instruction's
+// operand layouts (lane l = r + 16 kk feeds A[r][kk] and B[kk][r], receives D[4 kk + v][r]). A workgroup writes one block of partial
+// sums of the trained network's gradients, which the reduction kernel of the small-MLP path adds up in workgroup order (OVERWRITING the
+// gradients: what zero_gradient followed by backward leaves). The Adam step is the library's usual launch.
+// Bound: latency (a batch of 256 is sixteen workgroups); the point of this path is three launches per update instead of about twenty.
 #include "sac_update.h"
 #include "mlp_small.h"
 #include "optim.h"
@@ -22,11 +30,12 @@
 namespace {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) float* lptr;
-constexpr int H = 64, HS = H + 1, WAVES = 4, ROWS = 16 * WAVES, THREADS = 64 * WAVES, MAX_D = 128, MAX_ACT = 8, MAX_OUT = 16, D3S = MAX_OUT + 1, N_EXTRA = 16,
-              N_SUMS = 2 * H + MAX_OUT + N_EXTRA, MISC = 16, N_BIAS = 2 * H + MAX_OUT;
+constexpr int H = 64, HS = H + 1, TEAM_WAVES = 4, WAVES = 2 * TEAM_WAVES, ROWS = 16, THREADS = 64 * WAVES, MAX_D = 128, MAX_ACT = 8, MAX_OUT = 16, D3S = MAX_OUT + 1, N_EXTRA = 16,
+              MISC = 64;
+static_assert(H == 16 * TEAM_WAVES, "one 16-unit tile of the hidden layers per wavefront of a team");
 enum { MODE_CRITIC = 0, MODE_ACTOR = 1 };
 
-struct Net { const float *W1, *b1, *W2, *b2, *W3, *b3; int in, out, act_h, act3; };
+struct Net { const float *W1, *b1, *W2, *b2, *W3, *b3; int in, out, act_h; };      // the output layer has no activation
 struct UpdateArgs {
     Net actor, critic[2], target[2];       // critic update: critic[0] is the critic that is trained
     const float* batch_base;               // [2][batch][obs + act]: current rows, then next rows
@@ -67,157 +76,162 @@ __device__ __forceinline__ float normal_log_prob(float mean, float log_std, floa
 template <int ACT_H> __device__ __forceinline__ float act_hidden(float x, int f) { return rlt_act(x, ACT_H >= 0 ? ACT_H : f); }
 template <int ACT_H> __device__ __forceinline__ float dact_hidden(float o, int f) { return rlt_dact_from_output(o, ACT_H >= 0 ? ACT_H : f); }
 
+constexpr int YP = ROWS * D3S;      // one partial tile of an output layer
 constexpr size_t lds_floats(int nt1c) {
     const int sx = 16 * nt1c + 1;
-    return (size_t)H * sx + H * HS + MAX_OUT * HS + N_BIAS + (size_t)ROWS * (sx + 4 * HS + D3S) + WAVES * MISC;
+    // two input tiles, the trained network's h1 and h2, two scratch activations per team, d_pre3 of the trained network and of each
+    // team's critic, the output layers' partial tiles of two stages x two teams x four wavefronts, per-row scalars, a tile per
+    // wavefront to turn its parameters through
+    return (size_t)ROWS * (2 * sx + 6 * HS + 3 * D3S) + (size_t)4 * TEAM_WAVES * YP + MISC + (size_t)WAVES * 16 * (sx > HS ? sx : HS);
 }
 
-// The workgroup replaces the network in LDS in two halves, so that the loads travel while the previous network is still at work:
-// fetch_net requests this thread's share of the parameters into registers, commit_net waits for every wavefront to be done with the
-// previous network, stores them and meets again. W1 rows are padded to SX with zeros beyond the input width (so the padded reduction
-// steps and columns that hold something else add nothing), W3 rows and biases beyond the output width are zero.
-struct NetRegs { float v1[H / WAVES][2], v2[H * H / THREADS], v3[MAX_OUT * H / THREADS], bias; };
-__device__ __forceinline__ void fetch_net(const Net& N, NetRegs& R, int wave, int lane) {
-    const int IN = N.in, OUT = N.out, t = threadIdx.x;
+// A wavefront's share of a network in the registers that feed the matrix cores: the rows of W1 and W2 of its 16 hidden units, and the
+// columns of W3 that those units feed. Lane (r, kk) holds the B operand of every step of the reduction: k = 4 s + kk at step s.
+// The rows are stored [unit][input], so a lane's operands lie a row apart: they are requested as whole rows (one coalesced request per
+// row: 64 lanes, 64 consecutive floats -- requests with a lane per cache line each keep the address unit of the compute unit busy for
+// thousands of cycles) and turned through a tile of LDS that belongs to the wavefront.
+template <int NT1C> struct ForwardRegs { float w1[4 * NT1C], w2[16], w3[4], b1, b2; };
+template <int NT1C> struct RowRegs { float w2[16], w1[16][(NT1C + 3) / 4]; };
+template <int NT1C>
+__device__ __forceinline__ void request_forward(const Net& N, RowRegs<NT1C>& Q, ForwardRegs<NT1C>& F, int tile, int lane) {
+    const int IN = N.in, r = lane & 15, kk = lane >> 4, unit = 16 * tile + r;
 #pragma unroll
-    for (int j = 0; j < H / WAVES; j++) {
-        const float* src = N.W1 + (size_t)(wave * (H / WAVES) + j) * IN;
-        R.v1[j][0] = src[min(lane, IN - 1)];
-        R.v1[j][1] = IN > 64 ? src[min(64 + lane, IN - 1)] : 0.f;
+    for (int i = 0; i < 16; i++) {
+        Q.w2[i] = N.W2[(16 * tile + i) * H + lane];
+        const float* w1 = N.W1 + (size_t)(16 * tile + i) * IN;
+#pragma unroll
+        for (int c = 0; c < (NT1C + 3) / 4; c++) { const float v = w1[min(lane + 64 * c, IN - 1)]; Q.w1[i][c] = lane + 64 * c < IN ? v : 0.f; }
     }
+    const float* w3 = N.W3 + min(r, N.out - 1) * H + 16 * tile + kk;
 #pragma unroll
-    for (int u = 0; u < H * H / THREADS; u++) R.v2[u] = N.W2[u * THREADS + t];
-#pragma unroll
-    for (int u = 0; u < MAX_OUT * H / THREADS; u++) R.v3[u] = N.W3[min(u * THREADS + t, OUT * H - 1)];
-    R.bias = t < H ? N.b1[t] : t < 2 * H ? N.b2[t - H] : N.b3[min(t - 2 * H, OUT - 1)];
-}
-template <int SX>
-__device__ __forceinline__ void commit_net(const NetRegs& R, int IN, int OUT, lptr w1s, lptr w2s, lptr w3s, lptr bs, int wave, int lane) {
-    rlt_lds_barrier();      // nobody reads the previous network any more
-#pragma unroll
-    for (int j = 0; j < H / WAVES; j++) {
-        const lptr dst = w1s + (wave * (H / WAVES) + j) * SX;
-        if (lane < SX) dst[lane] = lane < IN ? R.v1[j][0] : 0.f;
-        if (64 + lane < SX) dst[64 + lane] = 64 + lane < IN ? R.v1[j][1] : 0.f;
-        if (lane == 0 && SX > 128) dst[128] = 0.f;
-    }
-#pragma unroll
-    for (int u = 0; u < H * H / THREADS; u++) { const int i = u * THREADS + threadIdx.x; w2s[(i >> 6) * HS + (i & 63)] = R.v2[u]; }
-#pragma unroll
-    for (int u = 0; u < MAX_OUT * H / THREADS; u++) { const int i = u * THREADS + threadIdx.x; w3s[(i >> 6) * HS + (i & 63)] = (i >> 6) < OUT ? R.v3[u] : 0.f; }
-    if (threadIdx.x < N_BIAS) bs[threadIdx.x] = (int)threadIdx.x < 2 * H + OUT ? R.bias : 0.f;
-    rlt_lds_barrier();
-}
-
-// the wavefront's 16 rows of a [batch x ld] array for its input tile: columns [0, valid), zero beyond them and beyond the batch; requested
-// into registers, stored later
-struct RowRegs { float va[16], vb[16]; };
-__device__ __forceinline__ void request_rows(RowRegs& X, const float* base, int ld, int row0, int batch, int valid, int lane) {
-#pragma unroll
-    for (int row = 0; row < 16; row++) {
-        const bool rok = row0 + row < batch;
-        const float* src = base + (size_t)min(row0 + row, batch - 1) * ld;
-        X.va[row] = (rok && lane < valid) ? src[lane] : 0.f;
-        X.vb[row] = (rok && 64 + lane < valid) ? src[64 + lane] : 0.f;
-    }
+    for (int q = 0; q < 4; q++) { const float v = w3[4 * q]; F.w3[q] = r < N.out ? v : 0.f; }
+    F.b1 = N.b1[unit]; F.b2 = N.b2[unit];
 }
 template <int SX, int NT1C>
-__device__ __forceinline__ void store_rows(const RowRegs& X, lptr xs, int lane) {
+__device__ __forceinline__ void turn_forward(const RowRegs<NT1C>& Q, ForwardRegs<NT1C>& F, lptr stage, int lane) {
+    const int r = lane & 15, kk = lane >> 4;
 #pragma unroll
-    for (int row = 0; row < 16; row++) {
-        if (lane < 16 * NT1C) xs[row * SX + lane] = X.va[row];
-        if (64 + lane < 16 * NT1C) xs[row * SX + 64 + lane] = X.vb[row];
-    }
+    for (int i = 0; i < 16; i++) stage[i * HS + lane] = Q.w2[i];
+    wave_sync();
+#pragma unroll
+    for (int s = 0; s < 16; s++) F.w2[s] = stage[r * HS + 4 * s + kk];
+    wave_sync();
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+#pragma unroll
+        for (int c = 0; c < (NT1C + 3) / 4; c++)
+            if (lane + 64 * c < 16 * NT1C) stage[i * SX + lane + 64 * c] = Q.w1[i][c];
+    wave_sync();
+#pragma unroll
+    for (int j = 0; j < 4 * NT1C; j++) F.w1[j] = stage[r * SX + 4 * j + kk];
+    wave_sync();
+}
+// the same units' columns of W2 and W3 (the transposed products of the backward pass)
+struct BackwardRegs { float w2t[16], w3t[4]; };
+__device__ __forceinline__ void fetch_backward(const Net& N, BackwardRegs& G, int tile, int r, int kk) {
+    const float* w2 = N.W2 + 16 * kk * H + 16 * tile + r;
+#pragma unroll
+    for (int s = 0; s < 16; s++) G.w2t[s] = w2[s * H];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) { const int o = 4 * ks + kk; const float v = N.W3[min(o, N.out - 1) * H + 16 * tile + r]; G.w3t[ks] = o < N.out ? v : 0.f; }
 }
 
-// the three layers on the wavefront's rows; h1 and h2 (after the activation) stay in LDS; returns the last layer's sums before bias and
-// activation: element v of lane (r, kk) belongs to row 4 kk + v, output r
-template <int SX, int ACT_H>
-__device__ __forceinline__ floatx4 forward16(const Net& N, lptr w1s, lptr w2s, lptr w3s, lptr bs, lptr xs, lptr h1s, lptr h2s, int r, int kk) {
+// The three layers on the workgroup's rows by the four wavefronts of a team: this wavefront's tile of h1 and of h2 (after the
+// activation) into LDS, then its quarter of the last layer's reduction into yp[tile]. Three workgroup barriers, which every wavefront
+// of the workgroup meets, working (on) or not; after the last one output_tile() returns the last layer's sums.
+template <int SX, int NT1C, int ACT_H>
+__device__ __forceinline__ void forward_wg(bool on, const ForwardRegs<NT1C>& F, int act_h, int NT1, lptr xs, lptr h1s, lptr h2s, lptr yp, int tile, int r, int kk) {
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
-    const int NT1 = (N.in + 15) >> 4;
-    floatx4 acc[4] = {zero4, zero4, zero4, zero4};
-    for (int g = 0; g < NT1; g++) {
+    const int col = 16 * tile + r;
+    if (on) {
+        floatx4 a0 = zero4, a1 = zero4;
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const float a = xs[r * SX + 16 * g + 4 * q + kk];
+        for (int g = 0; g < NT1C; g++)
+            if (g < NT1) {
 #pragma unroll
-            for (int nt = 0; nt < 4; nt++) acc[nt] = mfma16(a, w1s[(16 * nt + r) * SX + 16 * g + 4 * q + kk], acc[nt]);
+                for (int q = 0; q < 4; q += 2) {
+                    a0 = mfma16(xs[r * SX + 16 * g + 4 * q + kk], F.w1[4 * g + q], a0);
+                    a1 = mfma16(xs[r * SX + 16 * g + 4 * q + 4 + kk], F.w1[4 * g + q + 1], a1);
+                }
+            }
+        const floatx4 acc = a0 + a1;
+#pragma unroll
+        for (int v = 0; v < 4; v++) h1s[(4 * kk + v) * HS + col] = act_hidden<ACT_H>(acc[v] + F.b1, act_h);
+    }
+    rlt_lds_barrier();
+    if (on) {
+        floatx4 a0 = zero4, a1 = zero4;
+#pragma unroll
+        for (int s = 0; s < 16; s += 2) {
+            a0 = mfma16(h1s[r * HS + 4 * s + kk], F.w2[s], a0);
+            a1 = mfma16(h1s[r * HS + 4 * s + 4 + kk], F.w2[s + 1], a1);
         }
+        const floatx4 acc = a0 + a1;
+#pragma unroll
+        for (int v = 0; v < 4; v++) h2s[(4 * kk + v) * HS + col] = act_hidden<ACT_H>(acc[v] + F.b2, act_h);
     }
+    rlt_lds_barrier();
+    if (on) {
+        floatx4 a0 = zero4, a1 = zero4;
 #pragma unroll
-    for (int nt = 0; nt < 4; nt++) {
-        const float b = bs[16 * nt + r];
+        for (int q = 0; q < 4; q += 2) {
+            a0 = mfma16(h2s[r * HS + 16 * tile + 4 * q + kk], F.w3[q], a0);
+            a1 = mfma16(h2s[r * HS + 16 * tile + 4 * q + 4 + kk], F.w3[q + 1], a1);
+        }
+        const floatx4 y = a0 + a1;
 #pragma unroll
-        for (int v = 0; v < 4; v++) h1s[(4 * kk + v) * HS + 16 * nt + r] = act_hidden<ACT_H>(acc[nt][v] + b, N.act_h);
+        for (int v = 0; v < 4; v++) yp[(tile * ROWS + 4 * kk + v) * D3S + r] = y[v];
     }
-    wave_sync();
+    rlt_lds_barrier();
+}
+// the sums of four partial tiles, in a fixed order: element v of lane (r, kk) belongs to row 4 kk + v, column r
+__device__ __forceinline__ floatx4 output_tile(lptr yp, int r, int kk) {
+    floatx4 y;
 #pragma unroll
-    for (int nt = 0; nt < 4; nt++) acc[nt] = zero4;
-#pragma unroll
-    for (int s = 0; s < 16; s++) {
-        const float a = h1s[r * HS + 16 * kk + s];
-#pragma unroll
-        for (int nt = 0; nt < 4; nt++) acc[nt] = mfma16(a, w2s[(16 * nt + r) * HS + 16 * kk + s], acc[nt]);
+    for (int v = 0; v < 4; v++) {
+        const lptr p = yp + (4 * kk + v) * D3S + r;
+        y[v] = (p[0] + p[YP]) + (p[2 * YP] + p[3 * YP]);
     }
+    return y;
+}
+
+// this wavefront's tile of d_pre2 = (d_pre3 W3) f'(h2) into g2s (may be h2s itself); returns the lane's share of its column sum
+template <int ACT_H>
+__device__ __forceinline__ float backward_layer3(const BackwardRegs& G, int act_h, lptr d3s, lptr h2s, lptr g2s, int tile, int r, int kk) {
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int nt = 0; nt < 4; nt++) {
-        const float b = bs[H + 16 * nt + r];
+    for (int ks = 0; ks < MAX_OUT / 4; ks++) acc = mfma16(d3s[r * D3S + 4 * ks + kk], G.w3t[ks], acc);      // columns of d_pre3 beyond the output width are zero
+    float sum = 0.f;
 #pragma unroll
-        for (int v = 0; v < 4; v++) h2s[(4 * kk + v) * HS + 16 * nt + r] = act_hidden<ACT_H>(acc[nt][v] + b, N.act_h);
+    for (int v = 0; v < 4; v++) {
+        const int idx = (4 * kk + v) * HS + 16 * tile + r;
+        const float dp = acc[v] * dact_hidden<ACT_H>(h2s[idx], act_h);
+        g2s[idx] = dp; sum += dp;
     }
-    wave_sync();
-    floatx4 y0 = zero4, y1 = zero4;
+    return sum;
+}
+// this wavefront's tile of d_pre1 = (d_pre2 W2) f'(h1) into p1s (may be h1s itself); returns the lane's share of its column sum
+template <int ACT_H>
+__device__ __forceinline__ float backward_layer2(const BackwardRegs& G, int act_h, lptr g2s, lptr h1s, lptr p1s, int tile, int r, int kk) {
+    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    floatx4 a0 = zero4, a1 = zero4;
 #pragma unroll
     for (int s = 0; s < 16; s += 2) {
-        y0 = mfma16(h2s[r * HS + 16 * kk + s], w3s[r * HS + 16 * kk + s], y0);
-        y1 = mfma16(h2s[r * HS + 16 * kk + s + 1], w3s[r * HS + 16 * kk + s + 1], y1);
+        a0 = mfma16(g2s[r * HS + 16 * kk + s], G.w2t[s], a0);
+        a1 = mfma16(g2s[r * HS + 16 * kk + s + 1], G.w2t[s + 1], a1);
     }
-    return y0 + y1;
+    const floatx4 acc = a0 + a1;
+    float sum = 0.f;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int idx = (4 * kk + v) * HS + 16 * tile + r;
+        const float dp = acc[v] * dact_hidden<ACT_H>(h1s[idx], act_h);
+        p1s[idx] = dp; sum += dp;
+    }
+    return sum;
 }
 
-// d_pre2 = (d_pre3 W3) f'(h2) into g2s (may be h2s itself), accumulating its column sums
-template <int ACT_H>
-__device__ __forceinline__ void backward_layer3(const Net& N, lptr w3s, lptr d3s, lptr h2s, lptr g2s, float (&s2)[4], int r, int kk) {
-    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
-    floatx4 acc[4] = {zero4, zero4, zero4, zero4};
-#pragma unroll
-    for (int ks = 0; ks < MAX_OUT / 4; ks++) {      // columns of d_pre3 and rows of W3 beyond the output width are zero
-        const float a = d3s[r * D3S + 4 * ks + kk];
-#pragma unroll
-        for (int nt = 0; nt < 4; nt++) acc[nt] = mfma16(a, w3s[(4 * ks + kk) * HS + 16 * nt + r], acc[nt]);
-    }
-#pragma unroll
-    for (int nt = 0; nt < 4; nt++)
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const int idx = (4 * kk + v) * HS + 16 * nt + r;
-            const float dp = acc[nt][v] * dact_hidden<ACT_H>(h2s[idx], N.act_h);
-            g2s[idx] = dp; s2[nt] += dp;
-        }
-}
-// d_pre1 = (d_pre2 W2) f'(h1) into p1s (may be h1s itself), accumulating its column sums
-template <int ACT_H>
-__device__ __forceinline__ void backward_layer2(const Net& N, lptr w2s, lptr g2s, lptr h1s, lptr p1s, float (&s1)[4], int r, int kk) {
-    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
-    floatx4 acc[4] = {zero4, zero4, zero4, zero4};
-#pragma unroll
-    for (int s = 0; s < 16; s++) {
-        const float a = g2s[r * HS + 16 * kk + s];
-#pragma unroll
-        for (int nt = 0; nt < 4; nt++) acc[nt] = mfma16(a, w2s[(16 * kk + s) * HS + 16 * nt + r], acc[nt]);
-    }
-#pragma unroll
-    for (int nt = 0; nt < 4; nt++)
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const int idx = (4 * kk + v) * HS + 16 * nt + r;
-            const float dp = acc[nt][v] * dact_hidden<ACT_H>(h1s[idx], N.act_h);
-            p1s[idx] = dp; s1[nt] += dp;
-        }
-}
-
-// sample_and_squash forward for the items of a lane: row r of the wavefront's tile, actions kk and kk + 4
+// sample_and_squash forward for the items of a lane of the wavefront that does the per-row work: row r, actions kk and kk + 4
 struct HeadItem { float mean, log_std_raw, noise, sample, action; };
 __device__ __forceinline__ float head_forward(const UpdateArgs& A, lptr d3s, lptr xs, int SX, const float (&noise)[2], int r, int kk, HeadItem (&item)[2]) {
     float log_prob = 0.f;
@@ -246,104 +260,101 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
     extern __shared__ float lds_raw[];
     constexpr int SX = 16 * NT1C + 1;
     const int lane = threadIdx.x & 63, r = lane & 15, kk = lane >> 4;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), team = wave >> 2, tile = wave & 3;
+    const bool scalar_wave = wave == 0;        // the wavefront that does the per-row arithmetic between the network passes
+    const bool trainer = team == 1;            // the team that owns the trained network
     const int OBS = A.obs, ACT = A.act, D = OBS + ACT, B = A.batch;
-    const lptr w1s = (lptr)lds_raw, w2s = w1s + H * SX, w3s = w2s + H * HS, bs = w3s + MAX_OUT * HS;
-    const lptr xs_all = bs + N_BIAS, h1_all = xs_all + ROWS * SX, h2_all = h1_all + ROWS * HS, ta_all = h2_all + ROWS * HS, tb_all = ta_all + ROWS * HS,
-               d3_all = tb_all + ROWS * HS, misc_all = d3_all + ROWS * D3S;
-    const lptr xs = xs_all + 16 * wave * SX, h1s = h1_all + 16 * wave * HS, h2s = h2_all + 16 * wave * HS, tas = ta_all + 16 * wave * HS, tbs = tb_all + 16 * wave * HS,
-               d3s = d3_all + 16 * wave * D3S, misc = misc_all + wave * MISC;
-    const int row0 = blockIdx.x * ROWS + 16 * wave;
+    const lptr xsa = (lptr)lds_raw, xsb = xsa + ROWS * SX, h1s = xsb + ROWS * SX, h2s = h1s + ROWS * HS, tas = h2s + ROWS * HS + team * 2 * ROWS * HS, tbs = tas + ROWS * HS,
+               d3s = h2s + 5 * ROWS * HS, d3c = d3s + (1 + team) * ROWS * D3S, yps = d3s + 3 * ROWS * D3S, misc = yps + 4 * TEAM_WAVES * YP,
+               stage = misc + MISC + wave * 16 * (SX > HS ? SX : HS);
+    const lptr ypa = yps + team * TEAM_WAVES * YP, ypb = yps + (2 + team) * TEAM_WAVES * YP;      // stage A / stage B partial tiles of this team
+    const int row0 = blockIdx.x * ROWS;
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
-    float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f}, s3 = 0.f, extra = 0.f, unused[4] = {0.f, 0.f, 0.f, 0.f};
+    float s3 = 0.f, extra = 0.f;
     const Net& trained = MODE == MODE_CRITIC ? A.critic[0] : A.actor;
-    // every global load is requested one stage ahead of its use: the next network's parameters while the current one computes
-    NetRegs R;
-    RowRegs X;
-    fetch_net(A.actor, R, wave, lane);
-    request_rows(X, MODE == MODE_CRITIC ? A.batch_base + (size_t)B * D : A.batch_base, D, row0, B, MODE == MODE_CRITIC ? D : OBS, lane);
-    const float alpha = expf(*A.log_alpha);
-    float noise[2];
-#pragma unroll
-    for (int j = 0; j < 2; j++) noise[j] = (kk + 4 * j < ACT && row0 + r < B) ? A.noise[(size_t)(row0 + r) * ACT + kk + 4 * j] : 0.f;
-    HeadItem item[2];
+    const int NT1_D = (D + 15) >> 4, NT1_OBS = (OBS + 15) >> 4;
 
-    if (MODE == MODE_CRITIC) {
-        float reward[4]; bool terminated[4];
+    // the input tiles (32 threads share a row), then every parameter this wavefront multiplies with in the forward passes, are requested
+    // now; the backward pass's after the first forward pass has used its own
+    constexpr int XN = (NT1C + 1) / 2;
+    float xa[XN], xb[XN];
+    {
+        const int row = threadIdx.x >> 5, c0 = threadIdx.x & 31;
+        const bool rok = row0 + row < B;
+        const float* cur = A.batch_base + (size_t)min(row0 + row, B - 1) * D;
+        const float* nxt = cur + (size_t)B * D;
 #pragma unroll
-        for (int v = 0; v < 4; v++) { const int row = min(row0 + 4 * kk + v, B - 1); reward[v] = A.rewards[row]; terminated[v] = A.terminated[row] != 0; }
-        // the actor on the next observations, its squashed sample into the action columns of the tile
-        store_rows<SX, NT1C>(X, xs, lane);
-        commit_net<SX>(R, A.actor.in, A.actor.out, w1s, w2s, w3s, bs, wave, lane);
-        fetch_net(A.target[0], R, wave, lane);
-        {
-            const floatx4 y = forward16<SX, ACT_H>(A.actor, w1s, w2s, w3s, bs, xs, tas, tbs, r, kk);
-            const float b3 = bs[2 * H + r];
-#pragma unroll
-            for (int v = 0; v < 4; v++) d3s[(4 * kk + v) * D3S + r] = r < A.actor.out ? rlt_act(y[v] + b3, A.actor.act3) : 0.f;
+        for (int j = 0; j < XN; j++) {
+            const int c = c0 + 32 * j;
+            if (MODE == MODE_CRITIC) {
+                xa[j] = (rok && c < D) ? nxt[min(c, D - 1)] : 0.f;
+                xb[j] = (rok && c < D) ? cur[min(c, D - 1)] : 0.f;
+            } else {
+                xa[j] = (rok && c < OBS) ? cur[min(c, D - 1)] : 0.f;
+                xb[j] = 0.f;
+            }
         }
+    }
+    ForwardRegs<NT1C> FA, FB;
+    RowRegs<NT1C> QA, QB;
+    BackwardRegs GT, GC;
+    float wa[4] = {0.f, 0.f, 0.f, 0.f};
+    const bool stage_a_on = MODE == MODE_CRITIC || trainer;
+    if (stage_a_on) request_forward<NT1C>(MODE == MODE_CRITIC && !trainer ? A.actor : trained, QA, FA, tile, lane);
+    request_forward<NT1C>(MODE == MODE_CRITIC ? A.target[team] : A.critic[team], QB, FB, tile, lane);
+    {
+        const int row = threadIdx.x >> 5, c0 = threadIdx.x & 31;
+#pragma unroll
+        for (int j = 0; j < XN; j++) {
+            const int c = c0 + 32 * j;
+            if (c < 16 * NT1C) {
+                xsa[row * SX + c] = xa[j];
+                if (MODE == MODE_CRITIC) xsb[row * SX + c] = xb[j];
+            }
+        }
+    }
+    float noise[2] = {0.f, 0.f}, reward[4] = {0.f, 0.f, 0.f, 0.f}, alpha = 0.f, b3_actor = 0.f, b3_q[3] = {0.f, 0.f, 0.f};
+    bool terminated[4] = {false, false, false, false};
+    if (scalar_wave) {
+        alpha = expf(*A.log_alpha);
+        b3_actor = r < A.actor.out ? A.actor.b3[min(r, A.actor.out - 1)] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 2; j++) noise[j] = (kk + 4 * j < ACT && row0 + r < B) ? A.noise[(size_t)(row0 + r) * ACT + kk + 4 * j] : 0.f;
+        if (MODE == MODE_CRITIC) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) { const int row = min(row0 + 4 * kk + v, B - 1); reward[v] = A.rewards[row]; terminated[v] = A.terminated[row] != 0; }
+            b3_q[0] = A.target[0].b3[0]; b3_q[1] = A.target[1].b3[0]; b3_q[2] = trained.b3[0];
+        }
+    }
+    HeadItem item[2];
+    const bool row_ok = row0 + r < B;
+    if (stage_a_on) turn_forward<SX, NT1C>(QA, FA, stage, lane);
+    rlt_lds_barrier();      // the input tiles are in place
+
+    // stage A: the actor (critic update: on the next observations, by team 0, while team 1 takes the trained critic through the current
+    // rows; actor update: on the observations, by the team that will train it), then its squashed sample into the action columns
+    if (MODE == MODE_CRITIC) forward_wg<SX, NT1C, ACT_H>(true, FA, trainer ? trained.act_h : A.actor.act_h, trainer ? NT1_D : NT1_OBS, trainer ? xsb : xsa, trainer ? h1s : tas, trainer ? h2s : tbs, ypa, tile, r, kk);
+    else forward_wg<SX, NT1C, ACT_H>(trainer, FA, A.actor.act_h, NT1_OBS, xsa, h1s, h2s, ypa, tile, r, kk);
+    turn_forward<SX, NT1C>(QB, FB, stage, lane);
+    if (trainer) fetch_backward(trained, GT, tile, r, kk);
+    if (MODE == MODE_ACTOR) {
+        fetch_backward(A.critic[team], GC, tile, r, kk);
+        // the action columns of this wavefront's rows of W1: B operand of d_pre1 W1
+#pragma unroll
+        for (int q = 0; q < 4; q++) { const float v = A.critic[team].W1[(size_t)(16 * tile + 4 * q + kk) * D + OBS + min(r, ACT - 1)]; wa[q] = r < ACT ? v : 0.f; }
+    }
+    if (scalar_wave) {
+        const floatx4 y = output_tile(MODE == MODE_CRITIC ? yps : yps + TEAM_WAVES * YP, r, kk);
+#pragma unroll
+        for (int v = 0; v < 4; v++) d3s[(4 * kk + v) * D3S + r] = r < A.actor.out ? y[v] + b3_actor : 0.f;
         wave_sync();
-        const float next_log_prob = head_forward(A, d3s, xs, SX, noise, r, kk, item);
-        if (kk == 0) {
-            misc[r] = next_log_prob;
-            if (A.out_log_probabilities && row0 + r < B) A.out_log_probabilities[row0 + r] = next_log_prob;
-        }
-        wave_sync();
-        // both target critics on [next observation | sampled action]
-        float q_min[4];
-#pragma unroll
-        for (int k = 0; k < 2; k++) {
-            commit_net<SX>(R, A.target[k].in, A.target[k].out, w1s, w2s, w3s, bs, wave, lane);
-            if (k == 0) fetch_net(A.target[1], R, wave, lane);
-            else { fetch_net(trained, R, wave, lane); request_rows(X, A.batch_base, D, row0, B, D, lane); }
-            const floatx4 y = forward16<SX, ACT_H>(A.target[k], w1s, w2s, w3s, bs, xs, tas, tbs, r, kk);
-            const float b3 = bs[2 * H];
-#pragma unroll
-            for (int v = 0; v < 4; v++) { const float q = rlt_act(y[v] + b3, A.target[k].act3); q_min[v] = k ? fminf(q_min[v], q) : q; }
-        }
-        // TD target of rows 4 kk + v (meaningful in the lanes r == 0, which hold output 0)
-        float y_target[4];
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const float min_q = q_min[v] - alpha * misc[4 * kk + v];
-            const float future = terminated[v] ? 0.0f : A.gamma * min_q;
-            y_target[v] = reward[v] + future;
-            if (A.out_target_action_value && r == 0 && row0 + 4 * kk + v < B) A.out_target_action_value[row0 + 4 * kk + v] = y_target[v];
-        }
-        // the critic on the current rows, MSE gradient at its pre-activation
-        wave_sync();
-        store_rows<SX, NT1C>(X, xs, lane);
-        commit_net<SX>(R, trained.in, trained.out, w1s, w2s, w3s, bs, wave, lane);
-        const floatx4 y = forward16<SX, ACT_H>(trained, w1s, w2s, w3s, bs, xs, h1s, h2s, r, kk);
-        const float b3 = bs[2 * H];
-        // loss weight batch * 0.5 / n with n = batch rows (no masks), times the MSE gradient's 2 / batch (rl/algorithms/sac/operations_generic.h:298-316)
-        const float loss_weight = (1.0f / (float)B) * ((float)B * 0.5f);
-        const float constant = 2.0f / (float)B * loss_weight;
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const bool ok = r == 0 && row0 + 4 * kk + v < B;
-            const float q = rlt_act(y[v] + b3, trained.act3);
-            const float diff = q - y_target[v];
-            const float dp = ok ? diff * constant * rlt_dact_from_output(q, trained.act3) : 0.f;
-            if (ok) extra += diff * diff;
-            s3 += dp;
-            d3s[(4 * kk + v) * D3S + r] = dp;
-        }
-    } else {
-        // actor forward on the observations (its hidden activations are kept for the backward pass), squashed sample into the action columns
-        store_rows<SX, NT1C>(X, xs, lane);
-        commit_net<SX>(R, A.actor.in, A.actor.out, w1s, w2s, w3s, bs, wave, lane);
-        fetch_net(A.critic[0], R, wave, lane);
-        {
-            const floatx4 y = forward16<SX, ACT_H>(A.actor, w1s, w2s, w3s, bs, xs, h1s, h2s, r, kk);
-            const float b3 = bs[2 * H + r];
-#pragma unroll
-            for (int v = 0; v < 4; v++) d3s[(4 * kk + v) * D3S + r] = r < A.actor.out ? rlt_act(y[v] + b3, A.actor.act3) : 0.f;
-        }
-        wave_sync();
-        const float log_prob = head_forward(A, d3s, xs, SX, noise, r, kk, item);
-        const bool row_ok = row0 + r < B;
-        if (row_ok) {
+        const float log_prob = head_forward(A, d3s, xsa, SX, noise, r, kk, item);
+        if (MODE == MODE_CRITIC) {
+            if (kk == 0) {
+                misc[r] = log_prob;
+                if (A.out_log_probabilities && row_ok) A.out_log_probabilities[row0 + r] = log_prob;
+            }
+        } else if (row_ok) {
             if (kk == 0 && A.out_log_probabilities) A.out_log_probabilities[row0 + r] = log_prob;
 #pragma unroll
             for (int j = 0; j < 2; j++)
@@ -352,139 +363,158 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
                     if (A.out_pre_squashing) A.out_pre_squashing[(size_t)(row0 + r) * ACT + kk + 4 * j] = item[j].sample;
                 }
         }
-        wave_sync();
-        // both critics on [observation | sampled action]: value and the gradient of -value / batch with respect to the action
-        const float loss_weight = (1.0f / (float)B) * -1.0f;       // rl/algorithms/sac/operations_generic.h:437-453 with n = batch rows
-        float q_row[2], d_action[2][2];
-#pragma unroll
-        for (int k = 0; k < 2; k++) {
-            const Net& C = A.critic[k];
-            commit_net<SX>(R, C.in, C.out, w1s, w2s, w3s, bs, wave, lane);
-            fetch_net(k == 0 ? A.critic[1] : A.actor, R, wave, lane);
-            const floatx4 y = forward16<SX, ACT_H>(C, w1s, w2s, w3s, bs, xs, tas, tbs, r, kk);
-            const float b3 = bs[2 * H];
+    }
+    rlt_lds_barrier();      // the action columns are in place
+
+    // stage B: each team takes one of the two (target) critics through [observation | sampled action]
+    forward_wg<SX, NT1C, ACT_H>(true, FB, MODE == MODE_CRITIC ? A.target[team].act_h : A.critic[team].act_h, NT1_D, xsa, tas, tbs, ypb, tile, r, kk);
+    if (MODE == MODE_CRITIC) {
+        if (scalar_wave) {
+            // TD target of rows 4 kk + v (meaningful in the lanes r == 0, which hold output 0), MSE gradient at the critic's pre-activation
+            const floatx4 y0 = output_tile(yps + 2 * TEAM_WAVES * YP, r, kk), y1 = output_tile(yps + 3 * TEAM_WAVES * YP, r, kk), yc = output_tile(yps + TEAM_WAVES * YP, r, kk);
+            // loss weight batch * 0.5 / n with n = batch rows (no masks), times the MSE gradient's 2 / batch (rl/algorithms/sac/operations_generic.h:298-316)
+            const float loss_weight = (1.0f / (float)B) * ((float)B * 0.5f);
+            const float constant = 2.0f / (float)B * loss_weight;
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const float q = rlt_act(y[v] + b3, C.act3);
-                if (r == 0) misc[4 * kk + v] = q;
-                d3s[(4 * kk + v) * D3S + r] = (r == 0 && row0 + 4 * kk + v < B) ? loss_weight * rlt_dact_from_output(q, C.act3) : 0.f;
+                const float q_min = fminf(y0[v] + b3_q[0], y1[v] + b3_q[1]);
+                const float min_q = q_min - alpha * misc[4 * kk + v];
+                const float future = terminated[v] ? 0.0f : A.gamma * min_q;
+                const float y_target = reward[v] + future;
+                const bool ok = r == 0 && row0 + 4 * kk + v < B;
+                if (A.out_target_action_value && ok) A.out_target_action_value[row0 + 4 * kk + v] = y_target;
+                const float q = yc[v] + b3_q[2];
+                const float diff = q - y_target;
+                const float dp = ok ? diff * constant : 0.f;
+                if (ok) extra += diff * diff;
+                s3 += dp;
+                d3s[(4 * kk + v) * D3S + r] = dp;
             }
+        }
+        rlt_lds_barrier();      // d_pre3 is in place
+    } else {
+        // value and the gradient of -value / batch with respect to the action, each team for its critic
+        const float loss_weight = (1.0f / (float)B) * -1.0f;       // rl/algorithms/sac/operations_generic.h:437-453 with n = batch rows
+        const Net& C = A.critic[team];
+        if (tile == 0) {
+            const floatx4 y = output_tile(ypb, r, kk);
+            const float b3 = C.b3[0];
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float q = y[v] + b3;
+                if (r == 0) misc[16 * team + 4 * kk + v] = q;
+                d3c[(4 * kk + v) * D3S + r] = (r == 0 && row0 + 4 * kk + v < B) ? loss_weight : 0.f;
+            }
+        }
+        rlt_lds_barrier();
+        backward_layer3<ACT_H>(GC, C.act_h, d3c, tbs, tbs, tile, r, kk);
+        rlt_lds_barrier();
+        backward_layer2<ACT_H>(GC, C.act_h, tbs, tas, tas, tile, r, kk);
+        wave_sync();
+        {   // d value / d action = the action columns of d_pre1 W1: this wavefront's units' share of the reduction (stage A's partial tiles are free to hold it)
+            floatx4 acc = zero4;
+#pragma unroll
+            for (int q = 0; q < 4; q++) acc = mfma16(tas[r * HS + 16 * tile + 4 * q + kk], wa[q], acc);
+#pragma unroll
+            for (int v = 0; v < 4; v++) ypa[(tile * ROWS + 4 * kk + v) * D3S + r] = acc[v];
+        }
+        rlt_lds_barrier();
+        if (scalar_wave) {
+            // sample_and_squash backward (nn/layers/sample_and_squash/operations_generic.h:262-398) on the gradient of the smaller value
+            const bool first = misc[r] < misc[16 + r];
+            const lptr da = yps + (first ? 0 : 1) * TEAM_WAVES * YP + r * D3S;
+#pragma unroll
+            for (int v = 0; v < 4; v++) d3s[(4 * kk + v) * D3S + r] = 0.f;
             wave_sync();
-            backward_layer3<ACT_H>(C, w3s, d3s, tbs, tbs, unused, r, kk);
-            wave_sync();
-            backward_layer2<ACT_H>(C, w2s, tbs, tas, tas, unused, r, kk);
-            wave_sync();
-            q_row[k] = misc[r];
+            const float alpha_over_b = alpha / (float)B;
+            float entropy = 0.f;
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                float dot = 0.f;
-                if (kk + 4 * j < ACT)
-                    for (int n = 0; n < H; n++) dot += tas[r * HS + n] * w1s[n * SX + OBS + kk + 4 * j];
-                d_action[k][j] = dot;
-            }
-            wave_sync();
-        }
-        // sample_and_squash backward (nn/layers/sample_and_squash/operations_generic.h:262-398) on the gradient of the smaller value
-#pragma unroll
-        for (int v = 0; v < 4; v++) d3s[(4 * kk + v) * D3S + r] = 0.f;
-        wave_sync();
-        const float alpha_over_b = alpha / (float)B;
-        float entropy = 0.f;
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int a = kk + 4 * j;
-            if (a < ACT) {
-                const HeadItem& I = item[j];
-                const float d_out = q_row[0] < q_row[1] ? d_action[0][j] : d_action[1][j];
-                const float g = d_out * (1.0f - I.action * I.action);
-                const float log_std = clampf(I.log_std_raw, A.sas.log_std_lower_bound, A.sas.log_std_upper_bound);
-                const float sd = expf(log_std);
-                const float z = (I.sample - I.mean) / sd;
-                const float dlp_dmean = z / sd, dlp_dsample = -z / sd, dlp_dlogstd = z * z - 1.0f;
-                const float d_mu = g + alpha_over_b * (dlp_dmean + dlp_dsample + 2.0f * I.action);
-                float d_ls = sd * (g * I.noise) + alpha_over_b * (dlp_dlogstd + dlp_dsample * I.noise * sd + 2.0f * I.action * I.noise * sd);
-                if (I.log_std_raw < A.sas.log_std_lower_bound || I.log_std_raw > A.sas.log_std_upper_bound) d_ls = 0.0f;
-                if (row_ok) {
-                    d3s[r * D3S + a] = d_mu * rlt_dact_from_output(I.mean, A.actor.act3);
-                    d3s[r * D3S + ACT + a] = d_ls * rlt_dact_from_output(I.log_std_raw, A.actor.act3);
+                const int a = kk + 4 * j;
+                if (a < ACT) {
+                    const HeadItem& I = item[j];
+                    const float d_out = (da[a] + da[YP + a]) + (da[2 * YP + a] + da[3 * YP + a]);
+                    const float g = d_out * (1.0f - I.action * I.action);
+                    const float log_std = clampf(I.log_std_raw, A.sas.log_std_lower_bound, A.sas.log_std_upper_bound);
+                    const float sd = expf(log_std);
+                    const float z = (I.sample - I.mean) / sd;
+                    const float dlp_dmean = z / sd, dlp_dsample = -z / sd, dlp_dlogstd = z * z - 1.0f;
+                    const float d_mu = g + alpha_over_b * (dlp_dmean + dlp_dsample + 2.0f * I.action);
+                    float d_ls = sd * (g * I.noise) + alpha_over_b * (dlp_dlogstd + dlp_dsample * I.noise * sd + 2.0f * I.action * I.noise * sd);
+                    if (I.log_std_raw < A.sas.log_std_lower_bound || I.log_std_raw > A.sas.log_std_upper_bound) d_ls = 0.0f;
+                    if (row_ok) {
+                        d3s[r * D3S + a] = d_mu;
+                        d3s[r * D3S + ACT + a] = d_ls;
+                    }
+                    entropy -= normal_log_prob(I.mean, log_std, sd, I.sample) - logf(1.0f - I.action * I.action + A.sas.log_probability_epsilon);
                 }
-                entropy -= normal_log_prob(I.mean, log_std, sd, I.sample) - logf(1.0f - I.action * I.action + A.sas.log_probability_epsilon);
             }
-        }
-        entropy = groups_sum(entropy);
-        // d log_alpha: sum over the rows of alpha (entropy - target entropy), divided by the batch size by the reduction
-        const float per_row = (kk == 0 && row_ok) ? alpha * (entropy - A.sas.target_entropy) : 0.f;
-        const float tile_sum = row16_sum(per_row);
-        if (lane == 0) extra += tile_sum;
-        wave_sync();
+            entropy = groups_sum(entropy);
+            // d log_alpha: sum over the rows of alpha (entropy - target entropy), divided by the batch size by the reduction
+            const float per_row = (kk == 0 && row_ok) ? alpha * (entropy - A.sas.target_entropy) : 0.f;
+            const float tile_sum = row16_sum(per_row);
+            if (lane == 0) extra += tile_sum;
+            wave_sync();
 #pragma unroll
-        for (int v = 0; v < 4; v++) s3 += d3s[(4 * kk + v) * D3S + r];
-        commit_net<SX>(R, A.actor.in, A.actor.out, w1s, w2s, w3s, bs, wave, lane);
+            for (int v = 0; v < 4; v++) s3 += d3s[(4 * kk + v) * D3S + r];
+        }
+        rlt_lds_barrier();      // d_pre3 is in place
     }
 
-    // backward pass of the trained network with its weight gradients over the workgroup's 64 rows; h1, h2: its hidden activations,
-    // d3: the gradient at its last pre-activation; ta receives d_pre2, h2 is replaced by d_pre1
-    floatx4 aW1[NT1C], aW2[4], aW3a = zero4, aW3b = zero4;
+    // stage C: backward pass of the trained network with its weight gradients over the workgroup's 16 rows, by its team; h1, h2: its
+    // hidden activations, d3: the gradient at its last pre-activation; the team's ta receives d_pre2, tb receives d_pre1
+    float* dst = A.partial + (size_t)blockIdx.x * A.count;
+    const int IN = trained.in, OUT = trained.out, NT1 = (IN + 15) >> 4;
+    const int o_b1 = H * IN, o_w2 = o_b1 + H, o_b2 = o_w2 + H * H, o_w3 = o_b2 + H, o_b3 = o_w3 + OUT * H, o_ex = o_b3 + OUT;
+    const lptr xt = MODE == MODE_CRITIC ? xsb : xsa;
+    floatx4 aW1[NT1C], aW2[4], aW3 = zero4;
+    float s1 = 0.f, s2 = 0.f;
 #pragma unroll
     for (int nt = 0; nt < NT1C; nt++) aW1[nt] = zero4;
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) aW2[nt] = zero4;
-    rlt_lds_barrier();      // every wavefront's h2 and d_pre3 are in place
+    if (trainer) {
 #pragma unroll
-    for (int ks = 0; ks < ROWS / 4; ks++) {
-        const float a = d3_all[(4 * ks + kk) * D3S + r], b = h2_all[(4 * ks + kk) * HS + 16 * wave + r];
-        if (ks & 1) aW3b = mfma16(a, b, aW3b); else aW3a = mfma16(a, b, aW3a);
+        for (int ks = 0; ks < ROWS / 4; ks++) aW3 = mfma16(d3s[(4 * ks + kk) * D3S + r], h2s[(4 * ks + kk) * HS + 16 * tile + r], aW3);
+        s2 = backward_layer3<ACT_H>(GT, trained.act_h, d3s, h2s, tas, tile, r, kk);
     }
-    backward_layer3<ACT_H>(trained, w3s, d3s, h2s, tas, s2, r, kk);
-    rlt_lds_barrier();      // every wavefront's d_pre2 is in place, and nobody reads h2 any more
+    rlt_lds_barrier();      // every wavefront's tile of d_pre2 is in place
+    if (trainer) {
 #pragma unroll
-    for (int ks = 0; ks < ROWS / 4; ks++) {
-        const float a = ta_all[(4 * ks + kk) * HS + 16 * wave + r];
+        for (int ks = 0; ks < ROWS / 4; ks++) {
+            const float a = tas[(4 * ks + kk) * HS + 16 * tile + r];
 #pragma unroll
-        for (int nt = 0; nt < 4; nt++) aW2[nt] = mfma16(a, h1_all[(4 * ks + kk) * HS + 16 * nt + r], aW2[nt]);
+            for (int nt = 0; nt < 4; nt++) aW2[nt] = mfma16(a, h1s[(4 * ks + kk) * HS + 16 * nt + r], aW2[nt]);
+        }
+        s1 = backward_layer2<ACT_H>(GT, trained.act_h, tas, h1s, tbs, tile, r, kk);
+        wave_sync();            // dW1's rows are this wavefront's own tile of d_pre1
+#pragma unroll
+        for (int ks = 0; ks < ROWS / 4; ks++) {
+            const float a = tbs[(4 * ks + kk) * HS + 16 * tile + r];
+#pragma unroll
+            for (int nt = 0; nt < NT1C; nt++)
+                if (nt < NT1) aW1[nt] = mfma16(a, xt[(4 * ks + kk) * SX + 16 * nt + r], aW1[nt]);
+        }
+        // the workgroup's block of partial sums, straight from the registers that own them
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int m = 16 * tile + 4 * kk + v;
+#pragma unroll
+            for (int nt = 0; nt < NT1C; nt++)
+                if (nt < NT1 && 16 * nt + r < IN) dst[m * IN + 16 * nt + r] = aW1[nt][v];
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) dst[o_w2 + m * H + 16 * nt + r] = aW2[nt][v];
+            if (4 * kk + v < OUT) dst[o_w3 + (4 * kk + v) * H + 16 * tile + r] = aW3[v];
+        }
+        s1 = groups_sum(s1); s2 = groups_sum(s2);
+        if (kk == 0) { dst[o_b1 + 16 * tile + r] = s1; dst[o_b2 + 16 * tile + r] = s2; }
     }
-    backward_layer2<ACT_H>(trained, w2s, tas, h1s, h2s, s1, r, kk);
-    rlt_lds_barrier();      // every wavefront's d_pre1 is in place
-#pragma unroll 4
-    for (int ks = 0; ks < ROWS / 4; ks++) {
-        const float a = h2_all[(4 * ks + kk) * HS + 16 * wave + r];
-#pragma unroll
-        for (int nt = 0; nt < NT1C; nt++) aW1[nt] = mfma16(a, xs_all[(4 * ks + kk) * SX + 16 * nt + r], aW1[nt]);
-    }
-    rlt_lds_barrier();      // the weights may be overwritten
-
-    // the workgroup's block of partial sums: weight gradients straight from the registers that own them, ...
-    const int IN = trained.in, OUT = trained.out, NT1 = (IN + 15) >> 4;
-    float* dst = A.partial + (size_t)blockIdx.x * A.count;
-    const int o_b1 = H * IN, o_w2 = o_b1 + H, o_b2 = o_w2 + H * H, o_w3 = o_b2 + H, o_b3 = o_w3 + OUT * H, o_ex = o_b3 + OUT;
-#pragma unroll
-    for (int v = 0; v < 4; v++) {
-        const int m = 16 * wave + 4 * kk + v;
-#pragma unroll
-        for (int nt = 0; nt < NT1C; nt++)
-            if (nt < NT1 && 16 * nt + r < IN) dst[m * IN + 16 * nt + r] = aW1[nt][v];
-#pragma unroll
-        for (int nt = 0; nt < 4; nt++) dst[o_w2 + m * H + 16 * nt + r] = aW2[nt][v];
-        if (4 * kk + v < OUT) dst[o_w3 + (4 * kk + v) * H + 16 * wave + r] = aW3a[v] + aW3b[v];
-    }
-    // ... the bias gradients and the extra sum, which every wavefront holds for its own rows, summed in wavefront order through LDS
-    const lptr sums = (lptr)lds_raw;        // [WAVES][N_SUMS]
-#pragma unroll
-    for (int nt = 0; nt < 4; nt++) { s1[nt] = groups_sum(s1[nt]); s2[nt] = groups_sum(s2[nt]); }
-    s3 = groups_sum(s3); extra = groups_sum(extra);
-    if (kk == 0) {
-#pragma unroll
-        for (int nt = 0; nt < 4; nt++) { sums[wave * N_SUMS + 16 * nt + r] = s1[nt]; sums[wave * N_SUMS + H + 16 * nt + r] = s2[nt]; }
-        sums[wave * N_SUMS + 2 * H + r] = s3; sums[wave * N_SUMS + 2 * H + MAX_OUT + r] = extra;
-    }
-    rlt_lds_barrier();
-    if (threadIdx.x < N_SUMS) {
-        const int i = threadIdx.x;
-        const float total = (sums[i] + sums[N_SUMS + i]) + (sums[2 * N_SUMS + i] + sums[3 * N_SUMS + i]);
-        if (i < H) dst[o_b1 + i] = total;
-        else if (i < 2 * H) dst[o_b2 + i - H] = total;
-        else if (i < 2 * H + MAX_OUT) { if (i - 2 * H < OUT) dst[o_b3 + i - 2 * H] = total; }
-        else dst[o_ex + i - 2 * H - MAX_OUT] = total;
+    if (scalar_wave) {
+        s3 = groups_sum(s3); extra = groups_sum(extra);
+        if (kk == 0) {
+            if (r < OUT) dst[o_b3 + r] = s3;
+            dst[o_ex + r] = extra;
+        }
     }
 }
 
@@ -498,7 +528,7 @@ __global__ __launch_bounds__(256) void polyak_list_kernel(PolyakList P) {
 }
 
 bool hidden_ok(int a) { return a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH || a == RLT_ACT_SIGMOID; }
-bool out_ok(int a) { return a != RLT_ACT_GELU; }
+bool out_ok(int a) { return a == RLT_ACT_IDENTITY; }
 bool net_ok(const rlt_dense_layer* L, int n, int in, int out) {
     if (!L || n != 3) return false;
     for (int l = 0; l < 3; l++) if (!L[l].weights || !L[l].biases) return false;
@@ -506,7 +536,7 @@ bool net_ok(const rlt_dense_layer* L, int n, int in, int out) {
            L[0].activation == L[1].activation && hidden_ok(L[0].activation) && out_ok(L[2].activation);
 }
 Net net_of(const rlt_dense_layer* L) {
-    return {L[0].weights, L[0].biases, L[1].weights, L[1].biases, L[2].weights, L[2].biases, L[0].in_dim, L[2].out_dim, L[0].activation, L[2].activation};
+    return {L[0].weights, L[0].biases, L[1].weights, L[1].biases, L[2].weights, L[2].biases, L[0].in_dim, L[2].out_dim, L[0].activation};
 }
 int tile_bucket(int d) { return d <= 32 ? 2 : MAX_D / 16; }
 
