@@ -352,8 +352,9 @@ typedef struct rlt_sac_agent {
 /* train_critic            rl/algorithms/sac/operations_generic.h:243-337 for critic `critic_index`;
  *   action_noise [batch x action_dim] is the externally drawn N(0,1) noise.
  *   Two implementations with the same results (to fp32 rounding). Where every network is in -> 64 -> 64 -> out with one hidden
- *   activation (not GELU), obs + act <= 128, act <= 8 and all three masks are NULL, train_critic and train_actor each run as three
- *   launches (all network passes of the update; sum of the workgroups' partial gradients; Adam) and update_critic_targets as one;
+ *   activation (not GELU) and no output activation, obs + act <= 128, act <= 8 and all three masks are NULL, train_critic and
+ *   train_actor each run as two launches (all network passes of the update; sum of the workgroups' partial gradients + Adam, or three
+ *   where the Adam tensors are not the network's gradient buffers) and update_critic_targets as one;
  *   of the training buffers only next_log_probabilities and target_action_value (critic), actor_log_probabilities, actor_actions and
  *   actor_pre_squashing (actor) are then written, and the gradients are overwritten without a prior zero_gradient. Every other
  *   agent, or any agent after rlt_rocm_sac_set_per_operation(device, 1), takes one launch per reference operation and fills every

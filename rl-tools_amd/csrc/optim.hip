@@ -21,7 +21,34 @@ struct AdamLaunch {
     float* out_sq_norm;          // optional
     int increment_age;
     int accumulate_norm;         // add to *out_sq_norm instead of overwriting (later chunks of one step)
+    // optional: the gradients are still blocks of partial sums. Element j of tensor t is source_scale[t] times the sum over `groups`
+    // blocks of `block_stride` floats of source[g * block_stride + source_offset[t] + j], added up in the order of the small-MLP
+    // reduction kernel (four quarters of the blocks, each in block order, then (q0 + q1) + (q2 + q3)); it is stored in the tensor's
+    // gradient before it is used
+    const float* source;
+    int groups, block_stride;
+    uint32_t source_offset[MAX_T];
+    float source_scale[MAX_T];
 };
+
+__device__ __forceinline__ float sum_of_blocks(const float* __restrict__ p, int groups, int stride) {
+    const int per = (groups + 3) / 4;
+    float q[4];
+#pragma unroll
+    for (int qi = 0; qi < 4; qi++) {
+        const int g0 = qi * per, g1 = min(groups, g0 + per);
+        float s = 0.f;
+        for (int gb = g0; gb < g1; gb += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = p[(size_t)min(gb + u, g1 - 1) * stride];
+#pragma unroll
+            for (int u = 0; u < 8; u++) s += (gb + u < g1) ? v[u] : 0.f;
+        }
+        q[qi] = s;
+    }
+    return (q[0] + q[1]) + (q[2] + q[3]);
+}
 
 // the step for one optimiser by workgroups [0, n_blocks) numbered `block`
 __device__ __forceinline__ void adam_body(const AdamLaunch& a, uint32_t block, uint32_t n_blocks) {
@@ -37,7 +64,11 @@ __device__ __forceinline__ void adam_body(const AdamLaunch& a, uint32_t block, u
         for (int k = 1; k < MAX_T; k++) ti += (k < a.n && i >= a.prefix[k]) ? 1 : 0;
         const rlt_adam_tensor& T = a.t[ti];
         const uint32_t j = i - a.prefix[ti];
-        float g = T.gradient[j];
+        float g;
+        if (a.source) {
+            g = sum_of_blocks(a.source + a.source_offset[ti] + j, a.groups, a.block_stride) * a.source_scale[ti];
+            T.gradient[j] = g;
+        } else g = T.gradient[j];
         sq += g * g;
         if (a.p.enable_gradient_clipping) g = fminf(fmaxf(g, -a.p.gradient_clip_value), a.p.gradient_clip_value);
         float m = a.p.beta_1 * T.first_moment[j] + (1.0f - a.p.beta_1) * g;
@@ -134,10 +165,41 @@ static int adam_launch(rlt_rocm_device* device, const rlt_adam_tensor* tensors, 
     return 0;
 }
 
+static void set_source(AdamLaunch& a, const rlt_adam_source* source) {
+    if (!source) return;
+    a.source = source->partial; a.groups = source->groups; a.block_stride = source->block_stride;
+    for (int i = 0; i < a.n; i++) { a.source_offset[i] = source->offsets[i]; a.source_scale[i] = source->scales[i]; }
+}
+
+int rlt_adam_step_from_partials(rlt_rocm_device* device, const rlt_adam_tensor* tensors, int n, const rlt_adam_parameters* parameters, uint32_t* age, const rlt_adam_source* source) {
+    RLT_REQUIRE(tensors && n > 0 && n <= MAX_T && parameters && age && source && source->partial && source->groups > 0);
+    void* counters = nullptr;
+    int rc = rlt_counters(device, &counters);
+    if (rc) return rc;
+    AdamLaunch a = {};
+    a.n = n;
+    uint32_t total = 0;
+    for (int i = 0; i < n; i++) {
+        const rlt_adam_tensor& T = tensors[i];
+        if (!T.first_moment || !T.second_moment || !T.parameters || !T.gradient || T.count == 0) return RLT_E_INVALID_ARGUMENT;
+        a.t[i] = T; a.prefix[i] = total; total += T.count;
+    }
+    for (int i = n; i <= MAX_T; i++) a.prefix[i] = total;
+    a.p = *parameters; a.age = age;
+    a.done_counter = (uint32_t*)counters; a.block_partials = (float*)((char*)counters + 256);
+    a.increment_age = 1;
+    set_source(a, source);
+    int blocks = (int)((total + 255) / 256); if (blocks > 960) blocks = 960;
+    hipLaunchKernelGGL(adam_kernel, dim3(blocks), dim3(256), 0, device->stream, a);
+    return rlt_launch_status(device);
+}
+
 int rlt_adam_step_pair(rlt_rocm_device* device, const rlt_adam_tensor* tensors_a, int n_a, const rlt_adam_parameters* parameters_a, uint32_t* age_a,
-                       const rlt_adam_tensor* tensors_b, int n_b, const rlt_adam_parameters* parameters_b, uint32_t* age_b) {
+                       const rlt_adam_tensor* tensors_b, int n_b, const rlt_adam_parameters* parameters_b, uint32_t* age_b,
+                       const rlt_adam_source* source_a, const rlt_adam_source* source_b) {
     RLT_REQUIRE(tensors_a && tensors_b && n_a > 0 && n_b > 0 && parameters_a && parameters_b && age_a && age_b);
     if (n_a > MAX_T || n_b > MAX_T) {
+        RLT_REQUIRE(!source_a && !source_b);
         const int rc = adam_launch(device, tensors_a, n_a, parameters_a, age_a, 0.0f, nullptr, false);
         return rc ? rc : adam_launch(device, tensors_b, n_b, parameters_b, age_b, 0.0f, nullptr, false);
     }
@@ -162,6 +224,7 @@ int rlt_adam_step_pair(rlt_rocm_device* device, const rlt_adam_tensor* tensors_a
         // the second optimiser's ticket counter and partial sums sit in their own part of the counters block
         a.done_counter = (uint32_t*)((char*)counters + (k ? 64 : 0)); a.block_partials = (float*)((char*)counters + 256) + (k ? 480 : 0);
         a.increment_age = 1;
+        set_source(a, k ? source_b : source_a);
         blocks[k] = (total + 255) / 256; if (blocks[k] > 480) blocks[k] = 480; if (blocks[k] < 1) blocks[k] = 1;
     }
     hipLaunchKernelGGL(adam_pair_kernel, dim3(blocks[0] + blocks[1]), dim3(256), 0, device->stream, L[0], L[1], blocks[0]);

@@ -20,9 +20,10 @@
 // Parameters go from global memory straight into the registers that feed v_mfma_f32_16x16x4_f32 as B operands (each wavefront needs
 // only its own units' rows and columns), all requested at the start of the kernel; activations stay in LDS in the instruction's
 // operand layouts (lane l = r + 16 kk feeds A[r][kk] and B[kk][r], receives D[4 kk + v][r]). A workgroup writes one block of partial
-// sums of the trained network's gradients, which the reduction kernel of the small-MLP path adds up in workgroup order (OVERWRITING the
-// gradients: what zero_gradient followed by backward leaves). The Adam step is the library's usual launch.
-// Bound: latency (a batch of 256 is sixteen workgroups); the point of this path is three launches per update instead of about twenty.
+// sums of the trained network's gradients; the optimiser's launch adds the blocks up in workgroup order (in the order of the small-MLP
+// path's reduction kernel, which runs as a launch of its own where the Adam tensors are not the network's gradient buffers), stores the
+// sums as the gradients (OVERWRITING them: what zero_gradient followed by backward leaves) and steps.
+// Bound: latency (a batch of 256 is sixteen workgroups); the point of this path is two launches per update instead of about twenty.
 #include "sac_update.h"
 #include "mlp_small.h"
 #include "optim.h"
@@ -540,8 +541,54 @@ Net net_of(const rlt_dense_layer* L) {
 }
 int tile_bucket(int d) { return d <= 32 ? 2 : MAX_D / 16; }
 
+// Where each Adam tensor's gradient lies in a block of partial sums [dW1 | db1 | dW2 | db2 | dW3 | db3 | extra]: a tensor may span
+// several of the network's six gradient buffers where those follow each other in memory. False unless the tensors cover the six
+// buffers exactly, at most 12 of them: then the optimiser's launch can read the blocks itself.
+bool map_gradients(const rlt_dense_layer* L, const rlt_adam_tensor* T, int n, uint32_t* offsets) {
+    if (!T || n < 1 || n > 12) return false;
+    const float* seg[6] = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases};
+    const uint32_t size[6] = {(uint32_t)(H * L[0].in_dim), H, H * H, H, (uint32_t)(L[2].out_dim * H), (uint32_t)L[2].out_dim};
+    uint32_t off[6], covered = 0;
+    for (int k = 0, o = 0; k < 6; o += size[k], k++) off[k] = o;
+    for (int i = 0; i < n; i++) {
+        int s = 0;
+        while (s < 6 && seg[s] != T[i].gradient) s++;
+        if (s == 6 || T[i].polyak_target) return false;
+        uint32_t cnt = 0;
+        for (int k = s; k < 6 && cnt < T[i].count && seg[k] == seg[s] + cnt; k++) {
+            if (covered & (1u << k)) return false;
+            covered |= 1u << k; cnt += size[k];
+        }
+        if (cnt != T[i].count) return false;
+        offsets[i] = off[s];
+    }
+    return covered == 63u;
+}
+
+// the workgroups' blocks of partial sums -> gradients -> Adam step(s): one launch where the optimiser can read the blocks itself, else
+// the reduction kernel and then the optimiser. `second` (optional): an optimiser for one scalar whose gradient is extra[0] / batch.
+int reduce_and_step(rlt_rocm_device* device, const UpdateArgs& a, int groups, const rlt_dense_layer* trained, const rlt_adam_tensor* tensors, int n_tensors,
+                    const rlt_adam_parameters* parameters, uint32_t* age, const rlt_adam_tensor* second, const rlt_adam_parameters* second_parameters, uint32_t* second_age,
+                    float second_scale) {
+    uint32_t offsets[12];
+    if (map_gradients(trained, tensors, n_tensors, offsets) && (!second || !second->polyak_target)) {
+        float scales[12];
+        for (int i = 0; i < 12; i++) scales[i] = 1.0f;
+        const rlt_adam_source source = {a.partial, groups, a.count, offsets, scales};
+        if (!second) return rlt_adam_step_from_partials(device, tensors, n_tensors, parameters, age, &source);
+        const uint32_t second_offset = (uint32_t)(a.count - N_EXTRA);
+        const rlt_adam_source second_source = {a.partial, groups, a.count, &second_offset, &second_scale};
+        return rlt_adam_step_pair(device, tensors, n_tensors, parameters, age, second, 1, second_parameters, second_age, &source, &second_source);
+    }
+    int rc = rlt_mlp3s_reduce(device, trained, a.partial, groups, 1, second ? second->gradient : nullptr, second ? 1 : 0, second_scale, 0.0f);
+    if (rc) return rc;
+    if (second && n_tensors <= 12) return rlt_adam_step_pair(device, tensors, n_tensors, parameters, age, second, 1, second_parameters, second_age);
+    if ((rc = rlt_rocm_adam_step(device, tensors, n_tensors, parameters, age, 0.0f, nullptr))) return rc;
+    return second ? rlt_rocm_adam_step(device, second, 1, second_parameters, second_age, 0.0f, nullptr) : 0;
+}
+
 template <int MODE>
-int launch_update(rlt_rocm_device* device, UpdateArgs& a, int groups, const rlt_dense_layer* trained, float* extra, float extra_scale) {
+int launch_update(rlt_rocm_device* device, UpdateArgs& a, int groups, const rlt_dense_layer* trained) {
     const int bucket = tile_bucket(a.obs + a.act);
     const size_t lds_bytes = lds_floats(bucket) * sizeof(float);
     a.count = rlt_mlp3s_partial_count(trained[0].in_dim, trained[2].out_dim);
@@ -562,8 +609,7 @@ int launch_update(rlt_rocm_device* device, UpdateArgs& a, int groups, const rlt_
         if (act == RLT_ACT_RELU) RLT_LAUNCH_UPDATE(MAX_D / 16, RLT_ACT_RELU); else if (act == RLT_ACT_TANH) RLT_LAUNCH_UPDATE(MAX_D / 16, RLT_ACT_TANH); else RLT_LAUNCH_UPDATE(MAX_D / 16, -1);
     }
 #undef RLT_LAUNCH_UPDATE
-    if ((rc = rlt_launch_status(device))) return rc;
-    return rlt_mlp3s_reduce(device, trained, a.partial, groups, 1, extra, extra ? 1 : 0, extra_scale, 0.0f);
+    return rlt_launch_status(device);
 }
 }  // namespace
 
@@ -586,9 +632,10 @@ int rlt_sac_update_critic(rlt_rocm_device* device, const rlt_sac_agent* A, int c
     a.batch_base = A->observations_actions_base; a.rewards = A->rewards; a.terminated = A->terminated; a.noise = action_noise; a.log_alpha = A->log_alpha.parameters;
     a.sas = A->sas; a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
     a.out_log_probabilities = A->next_log_probabilities; a.out_target_action_value = A->target_action_value;
-    int rc = launch_update<MODE_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), A->critics[ci], nullptr, 0.0f);
+    const int groups = rlt_div_up(A->batch, ROWS);
+    int rc = launch_update<MODE_CRITIC>(device, a, groups, A->critics[ci]);
     if (rc) return rc;
-    return rlt_rocm_adam_step(device, A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], 0.0f, nullptr);
+    return reduce_and_step(device, a, groups, A->critics[ci], A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], nullptr, nullptr, nullptr, 0.0f);
 }
 
 int rlt_sac_update_actor(rlt_rocm_device* device, const rlt_sac_agent* A, const float* action_noise) {
@@ -601,12 +648,11 @@ int rlt_sac_update_actor(rlt_rocm_device* device, const rlt_sac_agent* A, const 
     a.batch_base = A->observations_actions_base; a.noise = action_noise; a.log_alpha = A->log_alpha.parameters;
     a.sas = A->sas; a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
     a.out_log_probabilities = A->actor_log_probabilities; a.out_actions = A->actor_actions; a.out_pre_squashing = A->actor_pre_squashing;
-    int rc = launch_update<MODE_ACTOR>(device, a, rlt_div_up(A->batch, ROWS), A->actor, A->log_alpha.gradient, 1.0f / (float)A->batch);
+    const int groups = rlt_div_up(A->batch, ROWS);
+    int rc = launch_update<MODE_ACTOR>(device, a, groups, A->actor);
     if (rc) return rc;
-    if (A->n_actor_adam_tensors <= 12)
-        return rlt_adam_step_pair(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, &A->log_alpha, 1, &A->alpha_adam, A->alpha_age);
-    if ((rc = rlt_rocm_adam_step(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, 0.0f, nullptr))) return rc;
-    return rlt_rocm_adam_step(device, &A->log_alpha, 1, &A->alpha_adam, A->alpha_age, 0.0f, nullptr);
+    return reduce_and_step(device, a, groups, A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, &A->log_alpha, &A->alpha_adam, A->alpha_age,
+                           1.0f / (float)A->batch);
 }
 
 int rlt_sac_polyak_list(rlt_rocm_device* device, const float* const* sources, float* const* targets, const uint32_t* counts, int n, float polyak) {

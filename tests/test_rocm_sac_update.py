@@ -1,4 +1,4 @@
-"""The fused SAC updates (three launches per train_critic / train_actor, one for update_critic_targets) for actors obs -> 64 -> 64 -> 2 act and
+"""The fused SAC updates (two launches per train_critic / train_actor, one for update_critic_targets) for actors obs -> 64 -> 64 -> 2 act and
 critics obs + act -> 64 -> 64 -> 1 of any width: against the CPU checker's train_critic / train_actor / update_critic_targets
 (rl/algorithms/sac/operations_generic.h:243-337, 395-468, 488-527) and against the library's own one-launch-per-operation path, from
 identical parameters, batches and noise. Tolerance: 1e-5 relative to each tensor's largest magnitude (fp32, different summation orders)."""
