@@ -4,19 +4,34 @@
 #include <rl_tools/devices/rocm.h>
 #include <rl_tools/containers/matrix/matrix.h>
 #include <rl_tools/random/operations_rocm.h>
+#include <new>
+#include <type_traits>
 RL_TOOLS_NAMESPACE_WRAPPER_START
 namespace rl_tools{
     // malloc / free           containers/matrix/operations_cuda.h:16-45
+    // Matrices of numbers and flags are device memory. Matrices of structs (environments, their parameters) are read and written by
+    // host code only -- the precompiled kernels know no struct layouts -- and are host memory; a component whose kernels do keep a struct
+    // array on the device (the runners' environment states) allocates it itself.
     template<typename DEV_SPEC, typename T, typename T_TI, T_TI SIZE_BYTES, bool T_CONST>
     void malloc(devices::ROCM<DEV_SPEC>& device, matrix::MatrixDynamic<T, T_TI, SIZE_BYTES, T_CONST>& matrix){
-        void* memory = nullptr;
-        devices::rocm::check(rlt_rocm_malloc(device.handle, &memory, SIZE_BYTES > 0 ? SIZE_BYTES : 1), "malloc(matrix)");
-        matrix._data = (T*)memory;
+        if constexpr(std::is_arithmetic_v<T>){
+            void* memory = nullptr;
+            devices::rocm::check(rlt_rocm_malloc(device.handle, &memory, SIZE_BYTES > 0 ? SIZE_BYTES : 1), "malloc(matrix)");
+            matrix._data = (T*)memory;
+        }
+        else{
+            matrix._data = (T*)::operator new(SIZE_BYTES > 0 ? SIZE_BYTES : 1, std::align_val_t(64));
+        }
         count_malloc(device, SIZE_BYTES);
     }
     template<typename DEV_SPEC, typename T, typename T_TI, T_TI SIZE_BYTES, bool T_CONST>
     void free(devices::ROCM<DEV_SPEC>& device, matrix::MatrixDynamic<T, T_TI, SIZE_BYTES, T_CONST>& matrix){
-        devices::rocm::check(rlt_rocm_free(device.handle, (void*)matrix._data), "free(matrix)");
+        if constexpr(std::is_arithmetic_v<T>){
+            devices::rocm::check(rlt_rocm_free(device.handle, (void*)matrix._data), "free(matrix)");
+        }
+        else{
+            ::operator delete((void*)matrix._data, std::align_val_t(64));
+        }
         matrix._data = nullptr;
     }
     template<typename DEV_SPEC, typename T, typename T_TI, T_TI SIZE>

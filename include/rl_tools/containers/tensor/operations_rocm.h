@@ -5,20 +5,34 @@
 #include <rl_tools/devices/rocm.h>
 #include <rl_tools/containers/tensor/tensor.h>
 #include <rl_tools/random/operations_rocm.h>
+#include <new>
+#include <type_traits>
 RL_TOOLS_NAMESPACE_WRAPPER_START
 namespace rl_tools{
     // malloc / free           containers/tensor/operations_cuda.h:15-39
+    // Tensors of numbers and flags are device memory. Tensors of structs (environments, their parameters, an optimiser's
+    // hyper-parameters) are read and written by host code only -- the precompiled kernels know no struct layouts -- and are host memory.
     template<typename DEV_SPEC, typename T, typename T_TI, T_TI SIZE, bool CONST>
     void malloc(devices::ROCM<DEV_SPEC>& device, tensor::TensorDynamic<T, T_TI, SIZE, CONST>& tensor){
-        void* memory = nullptr;
         constexpr size_t SIZE_BYTES = (size_t)SIZE * sizeof(T);
-        devices::rocm::check(rlt_rocm_malloc(device.handle, &memory, SIZE_BYTES > 0 ? SIZE_BYTES : 1), "malloc(tensor)");
-        tensor._data = (T*)memory;
+        if constexpr(std::is_arithmetic_v<T>){
+            void* memory = nullptr;
+            devices::rocm::check(rlt_rocm_malloc(device.handle, &memory, SIZE_BYTES > 0 ? SIZE_BYTES : 1), "malloc(tensor)");
+            tensor._data = (T*)memory;
+        }
+        else{
+            tensor._data = (T*)::operator new(SIZE_BYTES > 0 ? SIZE_BYTES : 1, std::align_val_t(64));
+        }
         count_malloc(device, SIZE_BYTES);
     }
     template <typename DEV_SPEC, typename T, typename T_TI, T_TI SIZE, bool CONST>
     void free(devices::ROCM<DEV_SPEC>& device, tensor::TensorDynamic<T, T_TI, SIZE, CONST>& tensor){
-        devices::rocm::check(rlt_rocm_free(device.handle, (void*)tensor._data), "free(tensor)");
+        if constexpr(std::is_arithmetic_v<T>){
+            devices::rocm::check(rlt_rocm_free(device.handle, (void*)tensor._data), "free(tensor)");
+        }
+        else{
+            ::operator delete((void*)tensor._data, std::align_val_t(64));
+        }
         tensor._data = nullptr;
     }
     template<typename DEV_SPEC, typename T, typename T_TI, T_TI SIZE>
@@ -207,19 +221,33 @@ namespace rl_tools{
         devices::rocm::check(rlt_rocm_free(device.handle, out), "abs_max");
         return value;
     }
+    // get                     containers/tensor/operations_generic.h: one element, copied to the host (waits for the stream): for the odd value that
+    // host code logs, never for loops
+    template<typename DEV_SPEC, typename SPEC>
+    typename SPEC::T get(devices::ROCM<DEV_SPEC>& device, const Tensor<SPEC>& tensor, typename devices::ROCM<DEV_SPEC>::index_t local_index){
+        static_assert(std::is_arithmetic_v<typename SPEC::T> && SPEC::SHAPE::LENGTH == 1);
+        utils::typing::remove_cv_t<typename SPEC::T> value;
+        devices::rocm::check(rlt_rocm_memcpy_d2h(device.handle, &value, tensor._data + index(device, tensor, local_index), sizeof(value)), "get(tensor)");
+        return value;
+    }
+    template<typename DEV_SPEC, typename SPEC, typename... INDICES>
+    typename SPEC::T get(devices::ROCM<DEV_SPEC>& device, const Tensor<SPEC>& tensor, typename devices::ROCM<DEV_SPEC>::index_t first_index, const INDICES... indices){
+        static_assert(std::is_arithmetic_v<typename SPEC::T> && SPEC::SHAPE::LENGTH == sizeof...(INDICES) + 1);
+        utils::typing::remove_cv_t<typename SPEC::T> value;
+        devices::rocm::check(rlt_rocm_memcpy_d2h(device.handle, &value, tensor._data + index(device, tensor, first_index, indices...), sizeof(value)), "get(tensor)");
+        return value;
+    }
 #ifdef RL_TOOLS_ROCM_FORBID_HOST_ELEMENT_ACCESS
-    // A tensor of this device is device memory: reading or writing one element from the host is never what a caller of this backend
-    // means (on hosts that map device memory it works, slowly, and hides a missing overload: a generic host loop running over device
-    // memory). With this macro such an access does not compile. The integration programs are checked with it.
-    template<typename DEV_SPEC, typename SPEC, typename... INDICES>
-    typename SPEC::T get(devices::ROCM<DEV_SPEC>& device, const Tensor<SPEC>& tensor, typename devices::ROCM<DEV_SPEC>::index_t index, const INDICES... indices) = delete;
-    template<typename DEV_SPEC, typename SPEC, typename... INDICES>
+    // A tensor of numbers on this device is device memory: a reference to one element, or writing one element from the host, is never
+    // what a caller of this backend means (on hosts that map device memory it works, slowly, and hides a missing overload: a generic
+    // host loop running over device memory). With this macro such an access does not compile. The integration programs are checked with it.
+    template<typename DEV_SPEC, typename SPEC, typename... INDICES, typename = utils::typing::enable_if_t<std::is_arithmetic_v<typename SPEC::T>>>
     typename SPEC::T& get_ref(devices::ROCM<DEV_SPEC>& device, Tensor<SPEC>& tensor, typename devices::ROCM<DEV_SPEC>::index_t index, const INDICES... indices) = delete;
-    template<typename DEV_SPEC, typename SPEC, typename... INDICES>
+    template<typename DEV_SPEC, typename SPEC, typename... INDICES, typename = utils::typing::enable_if_t<std::is_arithmetic_v<typename SPEC::T>>>
     const typename SPEC::T& get_ref(devices::ROCM<DEV_SPEC>& device, const Tensor<SPEC>& tensor, typename devices::ROCM<DEV_SPEC>::index_t index, const INDICES... indices) = delete;
-    template<typename DEV_SPEC, typename SPEC, typename TII, typename... INDICES>
+    template<typename DEV_SPEC, typename SPEC, typename TII, typename... INDICES, typename = utils::typing::enable_if_t<std::is_arithmetic_v<typename SPEC::T>>>
     void set(devices::ROCM<DEV_SPEC>& device, Tensor<SPEC>& tensor, typename SPEC::T value, const TII index, const INDICES... indices) = delete;
-    template<typename DEV_SPEC, typename SPEC, typename TII, typename... INDICES>
+    template<typename DEV_SPEC, typename SPEC, typename TII, typename... INDICES, typename = utils::typing::enable_if_t<std::is_arithmetic_v<typename SPEC::T>>>
     void increment(devices::ROCM<DEV_SPEC>& device, Tensor<SPEC>& tensor, typename SPEC::T value, const TII index, const INDICES... indices) = delete;
 #endif
     // randn / rand            containers/tensor/operations_cuda.h:545-624

@@ -14,7 +14,7 @@
 RL_TOOLS_NAMESPACE_WRAPPER_START
 namespace rl_tools{
     // train_critic / train_actor / update_critic_targets as calls of the library's own SAC entry points (rlt_rocm_sac_train_critic, ...), which run an
-    // update as three launches for 3-layer networks of hidden width 64 and as one launch per operation otherwise. These overloads take part only for
+    // update as two launches for 3-layer networks of hidden width 64 and as one launch per operation otherwise. These overloads take part only for
     // agents they can describe: single-step batches, actor = MLP followed by sample_and_squash, critics = MLPs, fp32, the reference's default
     // entropy handling. Any other agent goes through the reference's generic functions and the leaf overloads of this backend.
     namespace rl::algorithms::sac::rocm{

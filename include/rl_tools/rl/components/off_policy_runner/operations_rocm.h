@@ -105,7 +105,9 @@ namespace rl_tools{
         using L = rl::components::off_policy_runner::rocm::Layout<SPEC>;
         static_assert(SPEC::DYNAMIC_ALLOCATION, "runners on devices::ROCM are dynamically allocated");
         malloc(device, runner.buffers);
-        malloc(device, runner.states);
+        void* states = nullptr;     // the kernels' [N_ENVIRONMENTS x 2] float array
+        devices::rocm::check(rlt_rocm_malloc(device.handle, &states, sizeof(typename SPEC::ENVIRONMENT::State) * SPEC::PARAMETERS::N_ENVIRONMENTS), "malloc(runner)");
+        runner.states._data = (typename SPEC::ENVIRONMENT::State*)states;
         malloc(device, runner.episode_return);
         malloc(device, runner.episode_step);
         malloc(device, runner.truncated);
@@ -121,7 +123,8 @@ namespace rl_tools{
     template<typename DEV_SPEC, typename SPEC>
     void free(devices::ROCM<DEV_SPEC>& device, rl::components::OffPolicyRunner<SPEC>& runner){
         free(device, runner.buffers);
-        free(device, runner.states);
+        devices::rocm::check(rlt_rocm_free(device.handle, (void*)runner.states._data), "free(runner)");
+        runner.states._data = nullptr;
         free(device, runner.episode_return);
         free(device, runner.episode_step);
         free(device, runner.truncated);

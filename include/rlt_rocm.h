@@ -675,6 +675,11 @@ typedef struct rlt_ppo_agent {
     uint32_t* actor_age; uint32_t* critic_age;
     int observation_dim, observation_privileged_dim, action_dim, batch;
     void* workspace; size_t workspace_bytes;
+    /* optional standardize layers in front of the MLPs (nn/layers/standardize/operations_generic.h:68-86; the loop's approximators,
+     * rl/algorithms/ppo/loop/core/config.h:51-83): the networks then read (x - mean) * precision (the factor only where it is not 0).
+     * [observation_dim] / [observation_privileged_dim] floats; NULL = no such layer. The layer has no trainable parameters. */
+    const float* actor_standardize_mean; const float* actor_standardize_precision;
+    const float* critic_standardize_mean; const float* critic_standardize_precision;
 } rlt_ppo_agent;
 
 size_t rlt_rocm_ppo_workspace_bytes(const rlt_ppo_agent* agent);

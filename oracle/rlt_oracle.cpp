@@ -1432,6 +1432,22 @@ int rlt_oracle_ppo_train_minibatch(const rlt_ppo_agent* A, const rlt_ppo_paramet
         std::memcpy(&act[(size_t)b * AD], actions + row * ld, sizeof(float) * AD);
         lp[b] = action_log_probs[row * ld]; adv[b] = advantages[row * ld]; tgt[b] = target_values[row * ld];
     }
+    // the optional standardize layers in front of the networks (nn/layers/standardize/operations_generic.h:68-86; no trainable parameters,
+    // and the first layer's input gradient is not formed, so only the forward pass sees them)
+    if (A->actor_standardize_mean)
+        for (int b = 0; b < B; b++)
+            for (int c = 0; c < O; c++) {
+                float v = obs[(size_t)b * O + c] - A->actor_standardize_mean[c];
+                if (A->actor_standardize_precision[c] != 0) v *= A->actor_standardize_precision[c];
+                obs[(size_t)b * O + c] = v;
+            }
+    if (A->critic_standardize_mean)
+        for (int b = 0; b < B; b++)
+            for (int c = 0; c < OP; c++) {
+                float v = obsp[(size_t)b * OP + c] - A->critic_standardize_mean[c];
+                if (A->critic_standardize_precision[c] != 0) v *= A->critic_standardize_precision[c];
+                obsp[(size_t)b * OP + c] = v;
+            }
     int rc;
     if ((rc = rlt_oracle_mlp_zero_gradient(A->critic, A->n_critic_layers))) return rc;                   // :158
     if ((rc = rlt_oracle_mlp_zero_gradient(A->actor, A->n_actor_layers))) return rc;                     // :159 (clears the log_std gradient too)

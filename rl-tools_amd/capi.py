@@ -161,7 +161,9 @@ class PpoAgent(C.Structure):
                 ("critic_adam_tensors", C.POINTER(AdamTensor)), ("n_critic_adam_tensors", C.c_int32),
                 ("actor_adam", AdamParameters), ("critic_adam", AdamParameters), ("actor_age", C.c_void_p), ("critic_age", C.c_void_p),
                 ("observation_dim", C.c_int32), ("observation_privileged_dim", C.c_int32), ("action_dim", C.c_int32), ("batch", C.c_int32),
-                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+                ("actor_standardize_mean", C.c_void_p), ("actor_standardize_precision", C.c_void_p),
+                ("critic_standardize_mean", C.c_void_p), ("critic_standardize_precision", C.c_void_p)]
 
 
 class GruLayer(C.Structure):

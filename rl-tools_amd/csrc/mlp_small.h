@@ -25,12 +25,15 @@ bool rlt_mlp3s_pair_supported(const rlt_dense_layer* a, int n_a, const rlt_dense
 // straight from the dataset: every input column has the dataset's row stride `ld`, and minibatch row b is dataset row rows[b] (rows == NULL: b).
 // Means [batch x action_dim] and values [batch] are written packed; out_critic_loss (optional, critic output width 1) receives
 // mse::evaluate(values, targets) = sum((v - t)^2) / batch. The gradients are OVERWRITTEN (what zero_gradient followed by backward
-// leaves), so the caller skips zeroing them. RLT_E_UNSUPPORTED unless rlt_mlp3s_pair_supported.
+// leaves), so the caller skips zeroing them. RLT_E_UNSUPPORTED unless rlt_mlp3s_pair_supported. The optional standardize constants
+// ([in] floats each) put a standardize layer in front of the network: it reads (x - mean) * precision (the factor where it is not 0).
 int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* actor, int n_actor, const float* x, float* means, int ld_means,
                                const float* log_std, const float* actions, const float* log_probs, const float* advantages,
                                const float* stats, const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset,
                                const rlt_dense_layer* critic, int n_critic, const float* x_critic, float* values, int ld_values,
-                               const float* target_values, float mse_scale, float* out_critic_loss, int ld, const uint32_t* rows, int batch);
+                               const float* target_values, float mse_scale, float* out_critic_loss, int ld, const uint32_t* rows, int batch,
+                               const float* actor_std_mean = nullptr, const float* actor_std_precision = nullptr,
+                               const float* critic_std_mean = nullptr, const float* critic_std_precision = nullptr);
 
 // For kernels that write blocks of partial sums in this file's layout (dW1 [64 x in], db1 [64], dW2 [64 x 64], db2 [64], dW3 [out x 64], db3 [out],
 // extra [16]): the floats per block, and the launch that adds `groups` blocks up in block order into the layers' gradients (overwrite != 0:

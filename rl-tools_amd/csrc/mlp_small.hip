@@ -34,6 +34,7 @@ struct SmallArgs {
     float epsilon_clip, advantage_epsilon; int normalize_advantage;
     float* partial; int count;      // per workgroup: dW1 [64 x in], db1 [64], dW2 [64 x 64], db2 [64], dW3 [out x 64], db3 [out], extra [16]
     float* d_input; int ld_di;      // optional: gradient with respect to x, written at row b
+    const float* std_mean; const float* std_precision;      // optional standardize layer in front: the network reads (x - mean) * precision (the factor where it is not 0)
 };
 
 __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
@@ -156,14 +157,22 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
     for (int nt = 0; nt < 4; nt++) aW2[nt] = zero4;
     float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f}, s3 = 0.f, gls = 0.f;      // bias gradients and the extra sums (PPO: log_std gradient; MSE: squared error) over this wavefront's rows
 
+    // the standardize layer's constants for this lane's columns (nn/layers/standardize/operations_generic.h:68-86); without one: x - 0 times 1
+    float sm0 = 0.f, sp0 = 1.f, sm1 = 0.f, sp1 = 1.f;
+    if (A.std_mean) {
+        sm0 = A.std_mean[min(lane, IN - 1)]; sp0 = A.std_precision[min(lane, IN - 1)];
+        if (IN > 64) { sm1 = A.std_mean[min(64 + lane, IN - 1)]; sp1 = A.std_precision[min(64 + lane, IN - 1)]; }
+        sp0 = sp0 != 0.f ? sp0 : 1.f; sp1 = sp1 != 0.f ? sp1 : 1.f;
+    }
+
     for (int round = block; round < n_rounds; round += n_blocks) {
         const int tile = round * WAVES + wave, row0 = tile * 16;
         // inputs of the tile into LDS, zero beyond the batch and beyond the input width
 #pragma unroll
         for (int row = 0; row < 16; row++) {
             const bool rok = row0 + row < A.batch;
-            if (lane < 16 * NT1C) xs[row * SX + lane] = (rok && lane < IN) ? T.xa[row] : 0.f;
-            if (64 + lane < 16 * NT1C) xs[row * SX + 64 + lane] = (rok && 64 + lane < IN) ? T.xb[row] : 0.f;
+            if (lane < 16 * NT1C) xs[row * SX + lane] = (rok && lane < IN) ? (T.xa[row] - sm0) * sp0 : 0.f;
+            if (64 + lane < 16 * NT1C) xs[row * SX + 64 + lane] = (rok && 64 + lane < IN) ? (T.xb[row] - sm1) * sp1 : 0.f;
         }
         float in0[4], in1[4], in2[4];
 #pragma unroll
@@ -575,11 +584,14 @@ int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* a
                                const float* log_std, const float* actions, const float* log_probs, const float* advantages,
                                const float* stats, const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset,
                                const rlt_dense_layer* critic, int n_critic, const float* x_critic, float* values, int ld_values,
-                               const float* target_values, float mse_scale, float* out_critic_loss, int ld, const uint32_t* rows, int batch) {
+                               const float* target_values, float mse_scale, float* out_critic_loss, int ld, const uint32_t* rows, int batch,
+                               const float* actor_std_mean, const float* actor_std_precision, const float* critic_std_mean, const float* critic_std_precision) {
     if (!rlt_mlp3s_pair_supported(actor, n_actor, critic, n_critic) || (out_critic_loss && critic[2].out_dim != 1)) return RLT_E_UNSUPPORTED;
     SmallJob jobs[2] = {ppo_actor_job(actor, x, ld, means, ld_means, log_std, actions, ld, log_probs, ld, advantages, ld, stats, P, d_log_std,
                                       log_std_gradient_offset, batch, 1, rows),
                         plain_job(critic, 3, x_critic, ld, values, ld_values, nullptr, 0, target_values, ld, mse_scale, batch, 1, rows)};
     if (out_critic_loss) { jobs[1].extra = out_critic_loss; jobs[1].n_extra = 1; jobs[1].extra_scale = 1.0f / (float)batch; jobs[1].extra_offset = 0.0f; }
+    jobs[0].a.std_mean = actor_std_mean; jobs[0].a.std_precision = actor_std_mean ? actor_std_precision : nullptr;
+    jobs[1].a.std_mean = critic_std_mean; jobs[1].a.std_precision = critic_std_mean ? critic_std_precision : nullptr;
     return launch(device, jobs, 2);
 }

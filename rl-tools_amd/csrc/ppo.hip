@@ -96,12 +96,23 @@ __global__ __launch_bounds__(256) void ppo_gather_kernel(const float* __restrict
                                                          const float* __restrict__ actions, const float* __restrict__ log_probs, const float* __restrict__ advantages,
                                                          const float* __restrict__ targets, int ld, const uint32_t* __restrict__ row_indices, int batch, int O, int OP, int A,
                                                          float* __restrict__ obs, float* __restrict__ obsp, float* __restrict__ act, float* __restrict__ lp,
-                                                         float* __restrict__ adv, float* __restrict__ tgt) {
+                                                         float* __restrict__ adv, float* __restrict__ tgt,
+                                                         const float* __restrict__ actor_mean, const float* __restrict__ actor_precision,
+                                                         const float* __restrict__ critic_mean, const float* __restrict__ critic_precision) {
     const int sub = threadIdx.x & 15;
     for (int b = (blockIdx.x * blockDim.x + threadIdx.x) >> 4; b < batch; b += (gridDim.x * blockDim.x) >> 4) {
         const size_t row = row_indices ? row_indices[b] : (size_t)b;
-        for (int c = sub; c < O; c += 16) obs[(size_t)b * O + c] = observations[row * ld + c];
-        for (int c = sub; c < OP; c += 16) obsp[(size_t)b * OP + c] = observations_privileged[row * ld + c];
+        // the optional standardize layers in front of the networks (nn/layers/standardize/operations_generic.h:68-86) are applied here
+        for (int c = sub; c < O; c += 16) {
+            float v = observations[row * ld + c];
+            if (actor_mean) { v -= actor_mean[c]; const float p = actor_precision[c]; if (p != 0.f) v *= p; }
+            obs[(size_t)b * O + c] = v;
+        }
+        for (int c = sub; c < OP; c += 16) {
+            float v = observations_privileged[row * ld + c];
+            if (critic_mean) { v -= critic_mean[c]; const float p = critic_precision[c]; if (p != 0.f) v *= p; }
+            obsp[(size_t)b * OP + c] = v;
+        }
         for (int c = sub; c < A; c += 16) act[(size_t)b * A + c] = actions[row * ld + c];
         if (sub == 0) { lp[b] = log_probs[row * ld]; adv[b] = advantages[row * ld]; tgt[b] = targets[row * ld]; }
     }
@@ -236,7 +247,8 @@ bool ppo_agent_ok(const rlt_ppo_agent* A) {
     return A && A->actor && A->critic && A->n_actor_layers >= 1 && A->n_critic_layers >= 1 && A->log_std && A->actor_adam_tensors && A->critic_adam_tensors &&
            A->actor_age && A->critic_age && A->observation_dim >= 1 && A->observation_privileged_dim >= 1 && A->action_dim >= 1 && A->action_dim <= PPO_MAX_ACTION_DIM &&
            A->batch >= 1 && A->actor[0].in_dim == A->observation_dim && A->actor[A->n_actor_layers - 1].out_dim == A->action_dim &&
-           A->critic[0].in_dim == A->observation_privileged_dim && A->critic[A->n_critic_layers - 1].out_dim == 1 && A->actor[A->n_actor_layers - 1].output;
+           A->critic[0].in_dim == A->observation_privileged_dim && A->critic[A->n_critic_layers - 1].out_dim == 1 && A->actor[A->n_actor_layers - 1].output &&
+           !A->actor_standardize_mean == !A->actor_standardize_precision && !A->critic_standardize_mean == !A->critic_standardize_precision;
 }
 size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 // stats, surrogate partials, stats partials, then for an epoch's minibatches in chunks: their stats and stats partials
@@ -316,7 +328,8 @@ static int ppo_pair_update(rlt_rocm_device* device, const rlt_ppo_agent* A, cons
     int rc = rlt_mlp3s_ppo_actor_critic(device, A->actor, A->n_actor_layers, observations, A->actor[A->n_actor_layers - 1].output, AD, A->log_std, actions,
                                         action_log_probs, advantages, stats, P, P->learn_action_std ? A->d_log_std : nullptr, -P->action_entropy_coefficient,
                                         A->critic, A->n_critic_layers, observations_privileged, values, 1, target_values, 1.0f / (float)B, out_critic_loss,   // :303
-                                        ld, row_indices, B);
+                                        ld, row_indices, B, A->actor_standardize_mean, A->actor_standardize_precision, A->critic_standardize_mean,
+                                        A->critic_standardize_precision);
     if (rc) return rc;
     if (A->d_log_std && !P->learn_action_std) if ((rc = rlt_rocm_fill_f32(device, A->d_log_std, 1, AD, AD, 0.0f))) return rc;
     return rlt_adam_step_pair(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age,                                            // :305-306
@@ -350,7 +363,8 @@ extern "C" int rlt_rocm_ppo_train_minibatch(rlt_rocm_device* device, const rlt_p
     }
     int blocks = (B * 16 + 255) / 256; if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(ppo_gather_kernel, dim3(blocks), dim3(256), 0, device->stream, observations, observations_privileged, actions, action_log_probs, advantages, target_values,
-                       ld, row_indices, B, O, OP, AD, obs, obsp, act, lp, adv, tgt);
+                       ld, row_indices, B, O, OP, AD, obs, obsp, act, lp, adv, tgt, A->actor_standardize_mean, A->actor_standardize_precision,
+                       A->critic_standardize_mean, A->critic_standardize_precision);
     if ((rc = rlt_launch_status(device))) return rc;
     if ((rc = rlt_rocm_mlp_zero_gradient(device, A->critic, A->n_critic_layers))) return rc;                      // :158
     if ((rc = rlt_rocm_mlp_zero_gradient(device, A->actor, A->n_actor_layers))) return rc;                        // :159 (clears the log_std gradient too)

@@ -299,7 +299,7 @@ class PpoOnBackend:
     actor [W|b per layer], log_std, critic [W|b per layer] (what the reference harness exports)."""
 
     def __init__(self, backend, obs_dim, action_dim, actor_hidden, critic_hidden, batch, params, actor_act="relu", critic_act="relu",
-                 adam=None, obs_privileged_dim=None):
+                 adam=None, obs_privileged_dim=None, standardize=None):
         self.backend, self.batch, self.action_dim = backend, batch, action_dim
         opd = obs_dim if obs_privileged_dim is None else obs_privileged_dim
         adims, cdims = [obs_dim, actor_hidden, actor_hidden, action_dim], [opd, critic_hidden, critic_hidden, 1]
@@ -315,6 +315,10 @@ class PpoOnBackend:
         self.c = capi.PpoAgent(self.actor.layers, self.actor.n, self.critic.layers, self.critic.n, self.log_std.ptr, self.d_log_std.ptr,
                                self.actor_adam, len(tensors), self.critic.adam, self.critic.n_adam, adam, adam, self.actor.age.ptr, self.critic.age.ptr,
                                obs_dim, opd, action_dim, batch, None, 0)
+        if standardize is not None:     # (actor mean, actor precision, critic mean, critic precision): standardize layers in front of the networks
+            self.standardize = [backend.array(np.asarray(v, np.float32)) for v in standardize]
+            (self.c.actor_standardize_mean, self.c.actor_standardize_precision, self.c.critic_standardize_mean,
+             self.c.critic_standardize_precision) = [v.ptr for v in self.standardize]
         if backend.name == "rocm":
             n = backend.device.lib.rlt_rocm_ppo_workspace_bytes(C.byref(self.c))
             self.ws = backend.device.empty((int(n),), np.uint8)

@@ -91,6 +91,51 @@ def test_train_minibatch_matches_checker_on_synthetic_dataset(oracle, rocm):
     assert rel_err(p1, p0) <= 2e-4 and rel_err(l1, l0) <= 1e-4
 
 
+@pytest.mark.parametrize("O,A,H,B", [(105, 8, 64, 512), (3, 1, 64, 200), (17, 6, 256, 300)])
+def test_train_minibatch_with_standardize_layers_matches_checker(oracle, rocm, O, A, H, B):
+    """Standardize layers in front of actor and critic (the loop's approximators, rl/algorithms/ppo/loop/core/config.h:51-83): the networks
+    read (x - mean) * precision, the factor only where it is not 0 (nn/layers/standardize/operations_generic.h:68-86). Hidden width 64 takes
+    the kernel that reads the dataset rows itself, 256 the packed minibatch; four updates on shuffled rows, compared tensor by tensor after
+    the first and at the end. The third observation column has precision 0."""
+    capi = helpers.capi
+    N = 4 * B
+    rng = np.random.default_rng(O * 7 + A)
+    params = np.concatenate([helpers.random_params(rng, [O, H, H, A]), np.log(np.full(A, 0.5, np.float32)), helpers.random_params(rng, [O, H, H, 1])])
+    ld = O + 2 * A + 8
+    data = (rng.standard_normal((N, ld)) * 3 + 1.5).astype(np.float32)
+    col = dict(observations=0, actions=O + A, action_log_probs=O + 2 * A, advantages=O + 2 * A + 6, target_values=O + 2 * A + 7)
+    data[:, col["action_log_probs"]] = -A * 1.5 + 0.3 * rng.standard_normal(N).astype(np.float32)
+    data[:, col["actions"]:col["actions"] + A] = rng.standard_normal((N, A)).astype(np.float32)
+    standardize = [rng.standard_normal(O) * 0.5 + 1.5, 1.0 / (2.0 + rng.random(O)), rng.standard_normal(O) * 0.5 + 1.5, 1.0 / (2.0 + rng.random(O))]
+    standardize[1][2 % O] = 0.0
+    perm = rng.permutation(N).astype(np.uint32)
+    pp = capi.ppo_parameters()
+    results = []
+    for b in (oracle, rocm):
+        agent = helpers.PpoOnBackend(b, O, A, H, H, B, params, "tanh", "tanh", capi.adam_parameters(3e-4, epsilon=1e-8), standardize=standardize)
+        dd, idx, loss = b.array(data), b.array(perm), b.zeros((1,))
+        args = (dd.offset(col["observations"]), dd.offset(col["observations"]), dd.offset(col["actions"]), dd.offset(col["action_log_probs"]),
+                dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld)
+        b.call("ppo_train_minibatch", C.byref(agent.c), C.byref(pp), *args, None, loss.ptr)
+        b.sync()
+        first = dict(actor_grads=agent.actor.grads.numpy(), critic_grads=agent.critic.grads.numpy(), d_log_std=agent.d_log_std.numpy(), loss=loss.numpy())
+        for k in range(4):
+            b.call("ppo_train_minibatch", C.byref(agent.c), C.byref(pp), *args, idx.offset(k * B), loss.ptr)
+        b.sync()
+        results.append((first, agent.parameters(), loss.numpy()))
+    (f0, p0, l0), (f1, p1, l1) = results
+    for key in f0:
+        assert rel_err(f1[key], f0[key]) <= TOL, (key, rel_err(f1[key], f0[key]))
+    assert rel_err(p1, p0) <= 2e-4 and rel_err(l1, l0) <= 1e-4
+    # the layers matter: without them the first update's gradients differ
+    plain = helpers.PpoOnBackend(rocm, O, A, H, H, B, params, "tanh", "tanh", capi.adam_parameters(3e-4, epsilon=1e-8))
+    dd, loss = rocm.array(data), rocm.zeros((1,))
+    rocm.call("ppo_train_minibatch", C.byref(plain.c), C.byref(pp), dd.offset(0), dd.offset(0), dd.offset(col["actions"]), dd.offset(col["action_log_probs"]),
+              dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld, None, loss.ptr)
+    rocm.sync()
+    assert rel_err(plain.critic.grads.numpy(), f0["critic_grads"]) > 1e-2
+
+
 @pytest.mark.parametrize("normalize", [1, 0])
 def test_train_epoch_matches_checker_and_minibatch_calls(oracle, rocm, normalize):
     """One epoch call (advantage statistics of all minibatches formed up front, 40 minibatches = two chunks of that) against the checker's batch
