@@ -22,6 +22,7 @@
 #include <rl_tools/nn_models/random_uniform/model.h>
 #include <rl_tools/nn/layers/dense/operations_rocm.h>
 #include <rl_tools/nn/layers/sample_and_squash/operations_rocm.h>
+#include <rl_tools/nn/layers/td3_sampling/layer.h>
 RL_TOOLS_NAMESPACE_WRAPPER_START
 namespace rl_tools{
     namespace rl::components::off_policy_runner::rocm{
@@ -73,6 +74,8 @@ namespace rl_tools{
             int n_layers = 0;
             bool has_head = false;
             rlt_sas_parameters head = {};
+            bool has_td3_sampling = false;      // the policy ends in a td3_sampling layer: action = clamp(output + std * noise, -1, 1)
+            float td3_sampling_std = 0;
         };
         template <typename LAYER_SPEC>
         void describe(const nn::layers::dense::LayerForward<LAYER_SPEC>& layer, PolicyDescription& d){
@@ -82,6 +85,11 @@ namespace rl_tools{
         void describe(const nn::layers::sample_and_squash::LayerForward<LAYER_SPEC>& layer, PolicyDescription& d){
             d.has_head = true;
             d.head = nn::layers::sample_and_squash::rocm::parameters<LAYER_SPEC>();
+        }
+        template <typename LAYER_SPEC>
+        void describe(const nn::layers::td3_sampling::LayerForward<LAYER_SPEC>& layer, PolicyDescription& d){
+            d.has_td3_sampling = true;
+            d.td3_sampling_std = (float)LAYER_SPEC::PARAMETERS::STD;
         }
         template <typename MODEL_SPEC>
         void describe(const nn_models::mlp::NeuralNetworkForward<MODEL_SPEC>& model, PolicyDescription& d){
@@ -178,7 +186,36 @@ namespace rl_tools{
         else{
             rl::components::off_policy_runner::rocm::PolicyDescription d;
             rl::components::off_policy_runner::rocm::describe(policy, d);
-            if(d.has_head){
+            if(d.has_td3_sampling){
+                // TD3's exploring actor: the library's runner step for any environment and any sequential policy with a td3_sampling head (reset, observe,
+                // policy, clamp(output + std * noise), dynamics, reward, replay add: a handful of launches)
+                using ENVIRONMENT = typename SPEC::ENVIRONMENT;
+                using P = typename ENVIRONMENT::SPEC::PARAMETERS;
+                static_assert(P::initial_state_min_angle == -P::initial_state_max_angle && P::initial_state_min_speed == -P::initial_state_max_speed, "initial states are drawn from ranges that are symmetric about zero");
+                constexpr size_t ACT = ENVIRONMENT::ACTION_DIM;
+                rlt_env_runner e = {};
+                e.env_kind = RLT_ENV_PENDULUM; e.n_envs = r.n_envs; e.episode_step_limit = r.episode_step_limit;
+                e.states = r.states; e.episode_step = r.episode_step; e.episode_return = r.episode_return; e.truncated = r.truncated; e.pendulum = r.env;
+                e.observations = runner.buffers.observations._data; e.actions = runner.buffers.actions._data; e.next_observations = runner.buffers.next_observations._data;
+                rlt_seq_layer layers[rl::components::off_policy_runner::rocm::PolicyDescription::MAX_LAYERS] = {};
+                for(int l = 0; l < d.n_layers; l++){ layers[l].kind = 0; layers[l].dense = d.layers[l]; }
+                auto align = [](size_t bytes){ return (bytes + 255) / 256 * 256; };
+                const size_t rewards_bytes = align(N * sizeof(float)), terminated_bytes = align(N), noise_bytes = align(N * ACT * sizeof(float)), initial_bytes = align(N * 2 * sizeof(float));
+                // the workspace size depends on the runner's widths only, not on the pointers that are still to be carved out of the same block
+                const size_t workspace_bytes = rlt_rocm_env_runner_step_sequential_workspace_bytes(&e, layers, d.n_layers);
+                char* memory = (char*)devices::rocm::scratch(device, rewards_bytes + terminated_bytes + noise_bytes + initial_bytes + workspace_bytes);
+                e.rewards = (float*)memory; e.terminated = (uint8_t*)(memory + rewards_bytes);
+                float* noise = (float*)(memory + rewards_bytes + terminated_bytes); float* initial = (float*)(memory + rewards_bytes + terminated_bytes + noise_bytes);
+                void* workspace = memory + rewards_bytes + terminated_bytes + noise_bytes + initial_bytes;
+                devices::rocm::check(rlt_rocm_randn_f32(device.handle, noise, N * ACT, rng.seed, random::next_stream(rng)), "step(runner, noise)");
+                devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, N * 2, -1.0f, 1.0f, rng.seed, random::next_stream(rng)), "step(runner, initial states)");
+                devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_angle, initial, 2, initial, 2, (int)N, 1), "step(runner, initial states)");
+                if constexpr(P::initial_state_max_speed != 1){
+                    devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_speed, initial + 1, 2, initial + 1, 2, (int)N, 1), "step(runner, initial states)");
+                }
+                devices::rocm::check(rlt_rocm_env_runner_step_sequential(device.handle, &e, &rb, layers, d.n_layers, nullptr, 0, 3, nullptr, d.td3_sampling_std, noise, initial, workspace, workspace_bytes), "step(runner, td3 actor)");
+            }
+            else if(d.has_head){
                 auto& noise = get_last_buffer(policy_eval_buffers).noise;
                 static_assert(utils::typing::remove_reference_t<decltype(noise)>::ROWS == N);
                 randn(device, noise, rng);

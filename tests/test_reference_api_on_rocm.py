@@ -24,7 +24,7 @@ def test_programs_written_against_the_reference_api_compile_and_link():
     subprocess.run(["make", "-C", HERE, "syntax"], check=True, capture_output=True)
     out = subprocess.run(["make", "-B", "-C", HERE, "all"], capture_output=True, text=True)
     assert out.returncode == 0, out.stderr[-3000:]
-    for name in ("rocm_containers", "rocm_sac_pendulum", "rocm_ppo_pendulum"):
+    for name in ("rocm_containers", "rocm_sac_pendulum", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
         path = os.path.join(BUILD, name)
         assert os.path.exists(path)
         needed = subprocess.run(["readelf", "-d", path], capture_output=True, text=True).stdout
@@ -87,3 +87,21 @@ def test_the_references_ppo_loop_learns_the_pendulum_on_rocm():
     assert sorted(returns[-4:])[1] > -500 and final > -600    # seeds 0-3 end between -180 and -390
     # collection, advantage estimation and the update run on the device (the host loops manage about 14,000 environment steps per second)
     assert rate > 500000
+
+
+@pytest.mark.gpu
+def test_the_references_td3_loop_learns_the_pendulum_on_rocm():
+    """rl/algorithms/td3/loop/core instantiated on devices::ROCM: the runner step with the exploring actor (td3_sampling head), gather_batch,
+    target_action_noise, train_critic, train_actor and both target updates resolve to overloads of this backend."""
+    path = os.path.join(BUILD, "rocm_td3_pendulum")
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    out = subprocess.run([path, "10000", "0"], capture_output=True, text=True, timeout=300)
+    print(out.stdout[-1500:], flush=True)
+    assert out.returncode == 0, out.stderr[-2000:]
+    returns = [float(m) for m in re.findall(r"step \d+ mean_return (-?[\d.]+)", out.stdout)]
+    final = float(re.search(r"final (-?[\d.]+)", out.stdout).group(1))
+    rate = float(re.search(r"loop_steps_per_second_including_evaluations ([\d.]+)", out.stdout).group(1))
+    assert returns[0] < -600                                  # the untrained actor
+    assert max(returns[-3:]) > -250 and final > -300          # the reference's TD3 reaches about -150 on the Pendulum within 10,000 steps
+    assert rate > 1000                                        # every operation runs on the device (host loops over device memory: a few steps per second)
