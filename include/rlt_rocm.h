@@ -365,7 +365,7 @@ int rlt_rocm_sac_train_critic(rlt_rocm_device* device, const rlt_sac_agent* agen
 int rlt_rocm_sac_update_critic_targets(rlt_rocm_device* device, const rlt_sac_agent* agent);
 /* train_actor             sac/operations_generic.h:395-468 */
 int rlt_rocm_sac_train_actor(rlt_rocm_device* device, const rlt_sac_agent* agent, const float* action_noise);
-/* (no counterpart) enabled != 0: the three calls above always take the one-launch-per-operation path. */
+/* (no counterpart) enabled != 0: the three calls above, and rlt_rocm_td3_train_critic / _train_actor, always take the one-launch-per-operation path. */
 int rlt_rocm_sac_set_per_operation(rlt_rocm_device* device, int enabled);
 
 /* ------------------------------------------------- replay buffer / runner -- */
@@ -924,7 +924,13 @@ typedef struct rlt_td3_agent {
     void* workspace; size_t workspace_bytes;
 } rlt_td3_agent;
 
-/* train_critic            rl/algorithms/td3/operations_generic.h:170-235 for critic `critic_index`; sampling_noise [batch x act] are
+/* Two implementations with the same results (to fp32 rounding), as for SAC: where every network is in -> 64 -> 64 -> out with one hidden
+ * activation (not GELU), the actors end in tanh, obs + act <= 128, act <= 8 and both masks are NULL, train_critic and train_actor each run
+ * as two launches (all network passes of the update; sum of the workgroups' partial gradients + Adam); of the training buffers only
+ * target_action_value (critic) and actor_pre_clip (actor) are then written, and the gradients are overwritten without a prior
+ * zero_gradient. Every other agent, or any agent after rlt_rocm_sac_set_per_operation(device, 1), takes one launch per reference operation
+ * and fills every training buffer.
+ * train_critic            rl/algorithms/td3/operations_generic.h:170-235 for critic `critic_index`; sampling_noise [batch x act] are
  *   the N(0,1) draws of the target actor's sampling layer (its evaluate runs in the default mode, which samples). */
 int rlt_rocm_td3_train_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
 /* train_actor             td3/operations_generic.h:236-281; sampling_noise as above, for the actor's forward pass */

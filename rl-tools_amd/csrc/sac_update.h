@@ -12,3 +12,9 @@ int rlt_sac_update_critic(rlt_rocm_device* device, const rlt_sac_agent* agent, i
 int rlt_sac_update_actor(rlt_rocm_device* device, const rlt_sac_agent* agent, const float* action_noise);
 // target[i] = polyak * target[i] + (1 - polyak) * source[i] for a list of tensors, one launch per 16 tensors
 int rlt_sac_polyak_list(rlt_rocm_device* device, const float* const* sources, float* const* targets, const uint32_t* counts, int n, float polyak);
+
+// The same for TD3 (rl/algorithms/td3/operations_generic.h:170-281): actors obs -> 64 -> 64 -> act with a tanh output followed by the
+// td3_sampling layer, critics as above, no masks.
+bool rlt_td3_update_supported(const rlt_rocm_device* device, const rlt_td3_agent* agent);
+int rlt_td3_update_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
+int rlt_td3_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise);

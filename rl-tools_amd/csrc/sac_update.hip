@@ -1,5 +1,7 @@
 // One launch for the network passes of a SAC critic update, one for those of an actor update, for actors obs -> 64 -> 64 -> 2 act and
-// critics obs + act -> 64 -> 64 -> 1 of any observation / action width up to 128 inputs and 8 actions.
+// critics obs + act -> 64 -> 64 -> 1 of any observation / action width up to 128 inputs and 8 actions; and the same for TD3 (actors
+// obs -> 64 -> 64 -> act with a tanh output and the td3_sampling layer; rl/algorithms/td3/operations_generic.h:170-281), whose updates have
+// the same stages with another head, no entropy terms, and the policy gradient through critic 0 only.
 // reference: rl/algorithms/sac/operations_generic.h:243-337 (train_critic), :395-468 (train_actor),
 //            nn/layers/sample_and_squash/operations_generic.h:148-398, nn_models/mlp/operations_generic.h:128-260.
 //
@@ -34,7 +36,7 @@ typedef __attribute__((address_space(3))) float* lptr;
 constexpr int H = 64, HS = H + 1, TEAM_WAVES = 4, WAVES = 2 * TEAM_WAVES, ROWS = 16, THREADS = 64 * WAVES, MAX_D = 128, MAX_ACT = 8, MAX_OUT = 16, D3S = MAX_OUT + 1, N_EXTRA = 16,
               MISC = 64;
 static_assert(H == 16 * TEAM_WAVES, "one 16-unit tile of the hidden layers per wavefront of a team");
-enum { MODE_CRITIC = 0, MODE_ACTOR = 1 };
+enum { MODE_CRITIC = 0, MODE_ACTOR = 1, MODE_TD3_CRITIC = 2, MODE_TD3_ACTOR = 3 };     // SAC's two updates, TD3's two updates
 
 struct Net { const float *W1, *b1, *W2, *b2, *W3, *b3; int in, out, act_h; };      // the output layer has no activation
 struct UpdateArgs {
@@ -51,6 +53,11 @@ struct UpdateArgs {
     float* out_log_probabilities;          // critic update: next_log_probabilities; actor update: actor_log_probabilities
     float* out_target_action_value;        // critic update
     float* out_actions; float* out_pre_squashing;      // actor update, [batch][act]
+    // TD3 (rl/algorithms/td3/operations_generic.h:170-281): `actor` is the target actor in the critic update; its output passes tanh and the
+    // td3_sampling layer (action = clamp(tanh(output) + sampling_std * noise, -1, 1), nn/layers/td3_sampling/operations_generic.h:75-128)
+    float sampling_std; int ignore_termination;
+    const float* target_noise;             // critic update: [batch][act], already clamped (target_action_noise), added to the next action before a second clamp
+    float* out_pre_clip;                   // actor update: [batch][act], the sampling layer's value before the clamp
 };
 
 __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
@@ -256,8 +263,31 @@ __device__ __forceinline__ float head_forward(const UpdateArgs& A, lptr d3s, lpt
     return groups_sum(log_prob);
 }
 
+// TD3's actor head for the items of a lane: tanh of the MLP's output, the td3_sampling layer, and in the critic update the smoothing noise
+// of the target action (rl/algorithms/td3/operations_generic.h:129-145). mean = tanh(output), sample = value before the clamp.
+__device__ __forceinline__ void td3_head_forward(const UpdateArgs& A, lptr d3s, lptr xs, int SX, const float (&noise)[2], const float (&target_noise)[2], bool critic_update,
+                                                 int r, int kk, HeadItem (&item)[2]) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int a = kk + 4 * j;
+        HeadItem& I = item[j];
+        I = {0.f, 0.f, 0.f, 0.f, 0.f};
+        if (a < A.act) {
+            I.mean = tanhf(d3s[r * D3S + a]);
+            I.noise = noise[j];
+            float scaled = I.noise * A.sampling_std;
+            asm volatile("" : "+v"(scaled));        // the product is rounded before the addition, as the per-operation kernels and the reference's CPU build do
+            I.sample = scaled + I.mean;
+            I.action = clampf(I.sample, -1.0f, 1.0f);
+            if (critic_update) I.action = clampf(I.action + target_noise[j], -1.0f, 1.0f);
+            xs[r * SX + A.obs + a] = I.action;
+        }
+    }
+}
+
 template <int NT1C, int MODE, int ACT_H>
 __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
+    constexpr bool CRITIC = MODE == 0 || MODE == MODE_TD3_CRITIC, TD3 = MODE == MODE_TD3_CRITIC || MODE == MODE_TD3_ACTOR;
     extern __shared__ float lds_raw[];
     constexpr int SX = 16 * NT1C + 1;
     const int lane = threadIdx.x & 63, r = lane & 15, kk = lane >> 4;
@@ -272,7 +302,7 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
     const int row0 = blockIdx.x * ROWS;
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
     float s3 = 0.f, extra = 0.f;
-    const Net& trained = MODE == MODE_CRITIC ? A.critic[0] : A.actor;
+    const Net& trained = CRITIC ? A.critic[0] : A.actor;
     const int NT1_D = (D + 15) >> 4, NT1_OBS = (OBS + 15) >> 4;
 
     // the input tiles (32 threads share a row), then every parameter this wavefront multiplies with in the forward passes, are requested
@@ -287,7 +317,7 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
 #pragma unroll
         for (int j = 0; j < XN; j++) {
             const int c = c0 + 32 * j;
-            if (MODE == MODE_CRITIC) {
+            if (CRITIC) {
                 xa[j] = (rok && c < D) ? nxt[min(c, D - 1)] : 0.f;
                 xb[j] = (rok && c < D) ? cur[min(c, D - 1)] : 0.f;
             } else {
@@ -300,9 +330,9 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
     RowRegs<NT1C> QA, QB;
     BackwardRegs GT, GC;
     float wa[4] = {0.f, 0.f, 0.f, 0.f};
-    const bool stage_a_on = MODE == MODE_CRITIC || trainer;
-    if (stage_a_on) request_forward<NT1C>(MODE == MODE_CRITIC && !trainer ? A.actor : trained, QA, FA, tile, lane);
-    request_forward<NT1C>(MODE == MODE_CRITIC ? A.target[team] : A.critic[team], QB, FB, tile, lane);
+    const bool stage_a_on = CRITIC || trainer;
+    if (stage_a_on) request_forward<NT1C>(CRITIC && !trainer ? A.actor : trained, QA, FA, tile, lane);
+    request_forward<NT1C>(CRITIC ? A.target[team] : A.critic[team], QB, FB, tile, lane);
     {
         const int row = threadIdx.x >> 5, c0 = threadIdx.x & 31;
 #pragma unroll
@@ -310,18 +340,22 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
             const int c = c0 + 32 * j;
             if (c < 16 * NT1C) {
                 xsa[row * SX + c] = xa[j];
-                if (MODE == MODE_CRITIC) xsb[row * SX + c] = xb[j];
+                if (CRITIC) xsb[row * SX + c] = xb[j];
             }
         }
     }
-    float noise[2] = {0.f, 0.f}, reward[4] = {0.f, 0.f, 0.f, 0.f}, alpha = 0.f, b3_actor = 0.f, b3_q[3] = {0.f, 0.f, 0.f};
+    float noise[2] = {0.f, 0.f}, target_noise[2] = {0.f, 0.f}, reward[4] = {0.f, 0.f, 0.f, 0.f}, alpha = 0.f, b3_actor = 0.f, b3_q[3] = {0.f, 0.f, 0.f};
     bool terminated[4] = {false, false, false, false};
     if (scalar_wave) {
-        alpha = expf(*A.log_alpha);
+        if (!TD3) alpha = expf(*A.log_alpha);
+        if (MODE == MODE_TD3_CRITIC) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) target_noise[j] = (kk + 4 * j < ACT && row0 + r < B) ? A.target_noise[(size_t)(row0 + r) * ACT + kk + 4 * j] : 0.f;
+        }
         b3_actor = r < A.actor.out ? A.actor.b3[min(r, A.actor.out - 1)] : 0.f;
 #pragma unroll
         for (int j = 0; j < 2; j++) noise[j] = (kk + 4 * j < ACT && row0 + r < B) ? A.noise[(size_t)(row0 + r) * ACT + kk + 4 * j] : 0.f;
-        if (MODE == MODE_CRITIC) {
+        if (CRITIC) {
 #pragma unroll
             for (int v = 0; v < 4; v++) { const int row = min(row0 + 4 * kk + v, B - 1); reward[v] = A.rewards[row]; terminated[v] = A.terminated[row] != 0; }
             b3_q[0] = A.target[0].b3[0]; b3_q[1] = A.target[1].b3[0]; b3_q[2] = trained.b3[0];
@@ -334,23 +368,31 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
 
     // stage A: the actor (critic update: on the next observations, by team 0, while team 1 takes the trained critic through the current
     // rows; actor update: on the observations, by the team that will train it), then its squashed sample into the action columns
-    if (MODE == MODE_CRITIC) forward_wg<SX, NT1C, ACT_H>(true, FA, trainer ? trained.act_h : A.actor.act_h, trainer ? NT1_D : NT1_OBS, trainer ? xsb : xsa, trainer ? h1s : tas, trainer ? h2s : tbs, ypa, tile, r, kk);
+    if (CRITIC) forward_wg<SX, NT1C, ACT_H>(true, FA, trainer ? trained.act_h : A.actor.act_h, trainer ? NT1_D : NT1_OBS, trainer ? xsb : xsa, trainer ? h1s : tas, trainer ? h2s : tbs, ypa, tile, r, kk);
     else forward_wg<SX, NT1C, ACT_H>(trainer, FA, A.actor.act_h, NT1_OBS, xsa, h1s, h2s, ypa, tile, r, kk);
     turn_forward<SX, NT1C>(QB, FB, stage, lane);
     if (trainer) fetch_backward(trained, GT, tile, r, kk);
-    if (MODE == MODE_ACTOR) {
+    if (!CRITIC) {
         fetch_backward(A.critic[team], GC, tile, r, kk);
         // the action columns of this wavefront's rows of W1: B operand of d_pre1 W1
 #pragma unroll
         for (int q = 0; q < 4; q++) { const float v = A.critic[team].W1[(size_t)(16 * tile + 4 * q + kk) * D + OBS + min(r, ACT - 1)]; wa[q] = r < ACT ? v : 0.f; }
     }
     if (scalar_wave) {
-        const floatx4 y = output_tile(MODE == MODE_CRITIC ? yps : yps + TEAM_WAVES * YP, r, kk);
+        const floatx4 y = output_tile(CRITIC ? yps : yps + TEAM_WAVES * YP, r, kk);
 #pragma unroll
         for (int v = 0; v < 4; v++) d3s[(4 * kk + v) * D3S + r] = r < A.actor.out ? y[v] + b3_actor : 0.f;
         wave_sync();
-        const float log_prob = head_forward(A, d3s, xsa, SX, noise, r, kk, item);
-        if (MODE == MODE_CRITIC) {
+        float log_prob = 0.f;
+        if (TD3) td3_head_forward(A, d3s, xsa, SX, noise, target_noise, CRITIC, r, kk, item);
+        else log_prob = head_forward(A, d3s, xsa, SX, noise, r, kk, item);
+        if (TD3) {
+            if (!CRITIC && row_ok && A.out_pre_clip) {
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    if (kk + 4 * j < ACT) A.out_pre_clip[(size_t)(row0 + r) * ACT + kk + 4 * j] = item[j].sample;
+            }
+        } else if (CRITIC) {
             if (kk == 0) {
                 misc[r] = log_prob;
                 if (A.out_log_probabilities && row_ok) A.out_log_probabilities[row0 + r] = log_prob;
@@ -368,19 +410,20 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
     rlt_lds_barrier();      // the action columns are in place
 
     // stage B: each team takes one of the two (target) critics through [observation | sampled action]
-    forward_wg<SX, NT1C, ACT_H>(true, FB, MODE == MODE_CRITIC ? A.target[team].act_h : A.critic[team].act_h, NT1_D, xsa, tas, tbs, ypb, tile, r, kk);
-    if (MODE == MODE_CRITIC) {
+    forward_wg<SX, NT1C, ACT_H>(true, FB, CRITIC ? A.target[team].act_h : A.critic[team].act_h, NT1_D, xsa, tas, tbs, ypb, tile, r, kk);
+    if (CRITIC) {
         if (scalar_wave) {
             // TD target of rows 4 kk + v (meaningful in the lanes r == 0, which hold output 0), MSE gradient at the critic's pre-activation
             const floatx4 y0 = output_tile(yps + 2 * TEAM_WAVES * YP, r, kk), y1 = output_tile(yps + 3 * TEAM_WAVES * YP, r, kk), yc = output_tile(yps + TEAM_WAVES * YP, r, kk);
             // loss weight batch * 0.5 / n with n = batch rows (no masks), times the MSE gradient's 2 / batch (rl/algorithms/sac/operations_generic.h:298-316)
-            const float loss_weight = (1.0f / (float)B) * ((float)B * 0.5f);
+            // (TD3: loss weight batch / n, rl/algorithms/td3/operations_generic.h:200-212)
+            const float loss_weight = TD3 ? (float)B / (float)B : (1.0f / (float)B) * ((float)B * 0.5f);
             const float constant = 2.0f / (float)B * loss_weight;
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const float q_min = fminf(y0[v] + b3_q[0], y1[v] + b3_q[1]);
-                const float min_q = q_min - alpha * misc[4 * kk + v];
-                const float future = terminated[v] ? 0.0f : A.gamma * min_q;
+                const float min_q = TD3 ? q_min : q_min - alpha * misc[4 * kk + v];
+                const float future = (terminated[v] && !(TD3 && A.ignore_termination)) ? 0.0f : A.gamma * min_q;
                 const float y_target = reward[v] + future;
                 const bool ok = r == 0 && row0 + 4 * kk + v < B;
                 if (A.out_target_action_value && ok) A.out_target_action_value[row0 + 4 * kk + v] = y_target;
@@ -421,8 +464,10 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
         }
         rlt_lds_barrier();
         if (scalar_wave) {
-            // sample_and_squash backward (nn/layers/sample_and_squash/operations_generic.h:262-398) on the gradient of the smaller value
-            const bool first = misc[r] < misc[16 + r];
+            // sample_and_squash backward (nn/layers/sample_and_squash/operations_generic.h:262-398) on the gradient of the smaller value;
+            // TD3: the gradient through critic 0 (both teams ran it), the td3_sampling layer's backward (zero where the sample was clamped,
+            // nn/layers/td3_sampling/operations_generic.h:139-163) and the derivative of the actor's tanh output
+            const bool first = TD3 || misc[r] < misc[16 + r];
             const lptr da = yps + (first ? 0 : 1) * TEAM_WAVES * YP + r * D3S;
 #pragma unroll
             for (int v = 0; v < 4; v++) d3s[(4 * kk + v) * D3S + r] = 0.f;
@@ -435,6 +480,11 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
                 if (a < ACT) {
                     const HeadItem& I = item[j];
                     const float d_out = (da[a] + da[YP + a]) + (da[2 * YP + a] + da[3 * YP + a]);
+                    if (TD3) {
+                        const float d_mean = (I.sample < -1.0f || I.sample > 1.0f) ? 0.0f : d_out;
+                        if (row_ok) d3s[r * D3S + a] = d_mean * (1.0f - I.mean * I.mean);
+                        continue;
+                    }
                     const float g = d_out * (1.0f - I.action * I.action);
                     const float log_std = clampf(I.log_std_raw, A.sas.log_std_lower_bound, A.sas.log_std_upper_bound);
                     const float sd = expf(log_std);
@@ -467,7 +517,7 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
     float* dst = A.partial + (size_t)blockIdx.x * A.count;
     const int IN = trained.in, OUT = trained.out, NT1 = (IN + 15) >> 4;
     const int o_b1 = H * IN, o_w2 = o_b1 + H, o_b2 = o_w2 + H * H, o_w3 = o_b2 + H, o_b3 = o_w3 + OUT * H, o_ex = o_b3 + OUT;
-    const lptr xt = MODE == MODE_CRITIC ? xsb : xsa;
+    const lptr xt = CRITIC ? xsb : xsa;
     floatx4 aW1[NT1C], aW2[4], aW3 = zero4;
     float s1 = 0.f, s2 = 0.f;
 #pragma unroll
@@ -529,12 +579,11 @@ __global__ __launch_bounds__(256) void polyak_list_kernel(PolyakList P) {
 }
 
 bool hidden_ok(int a) { return a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH || a == RLT_ACT_SIGMOID; }
-bool out_ok(int a) { return a == RLT_ACT_IDENTITY; }
-bool net_ok(const rlt_dense_layer* L, int n, int in, int out) {
+bool net_ok(const rlt_dense_layer* L, int n, int in, int out, int out_activation = RLT_ACT_IDENTITY) {
     if (!L || n != 3) return false;
     for (int l = 0; l < 3; l++) if (!L[l].weights || !L[l].biases) return false;
     return L[0].in_dim == in && L[0].out_dim == H && L[1].in_dim == H && L[1].out_dim == H && L[2].in_dim == H && L[2].out_dim == out &&
-           L[0].activation == L[1].activation && hidden_ok(L[0].activation) && out_ok(L[2].activation);
+           L[0].activation == L[1].activation && hidden_ok(L[0].activation) && L[2].activation == out_activation;
 }
 Net net_of(const rlt_dense_layer* L) {
     return {L[0].weights, L[0].biases, L[1].weights, L[1].biases, L[2].weights, L[2].biases, L[0].in_dim, L[2].out_dim, L[0].activation};
@@ -653,6 +702,50 @@ int rlt_sac_update_actor(rlt_rocm_device* device, const rlt_sac_agent* A, const 
     if (rc) return rc;
     return reduce_and_step(device, a, groups, A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, &A->log_alpha, &A->alpha_adam, A->alpha_age,
                            1.0f / (float)A->batch);
+}
+
+// ---- TD3: the same kernel with the td3_sampling head (rl/algorithms/td3/operations_generic.h:170-281)
+
+bool rlt_td3_update_supported(const rlt_rocm_device* device, const rlt_td3_agent* A) {
+    const int OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    if (OBS < 1 || ACT < 1 || ACT > MAX_ACT || D > MAX_D || A->batch < 1) return false;
+    if (A->final_step_mask || A->next_final_step_mask) return false;       // the masked variants count rows over the whole batch first
+    if (!net_ok(A->actor, A->n_actor_layers, OBS, ACT, RLT_ACT_TANH) || !net_ok(A->actor_target, A->n_actor_layers, OBS, ACT, RLT_ACT_TANH)) return false;
+    for (int k = 0; k < 2; k++)
+        if (!net_ok(A->critics[k], A->n_critic_layers, D, 1) || !net_ok(A->critics_target[k], A->n_critic_layers, D, 1)) return false;
+    return lds_floats(tile_bucket(D)) * sizeof(float) <= (size_t)device->lds_bytes;
+}
+
+int rlt_td3_update_critic(rlt_rocm_device* device, const rlt_td3_agent* A, int ci, const float* sampling_noise) {
+    if (!rlt_td3_update_supported(device, A)) return RLT_E_UNSUPPORTED;
+    for (int l = 0; l < 3; l++) RLT_REQUIRE(A->critics[ci][l].d_weights && A->critics[ci][l].d_biases);
+    RLT_REQUIRE(A->target_next_action_noise);
+    UpdateArgs a = {};
+    a.actor = net_of(A->actor_target); a.critic[0] = net_of(A->critics[ci]); a.critic[1] = a.critic[0];
+    for (int k = 0; k < 2; k++) a.target[k] = net_of(A->critics_target[k]);
+    a.batch_base = A->observations_actions_base; a.rewards = A->rewards; a.terminated = A->terminated; a.noise = sampling_noise; a.target_noise = A->target_next_action_noise;
+    a.sampling_std = A->sampling_std; a.ignore_termination = A->ignore_termination;
+    a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
+    a.out_target_action_value = A->target_action_value;
+    const int groups = rlt_div_up(A->batch, ROWS);
+    int rc = launch_update<MODE_TD3_CRITIC>(device, a, groups, A->critics[ci]);
+    if (rc) return rc;
+    return reduce_and_step(device, a, groups, A->critics[ci], A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], nullptr, nullptr, nullptr, 0.0f);
+}
+
+int rlt_td3_update_actor(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise) {
+    if (!rlt_td3_update_supported(device, A)) return RLT_E_UNSUPPORTED;
+    for (int l = 0; l < 3; l++) RLT_REQUIRE(A->actor[l].d_weights && A->actor[l].d_biases);
+    UpdateArgs a = {};
+    a.actor = net_of(A->actor);
+    for (int k = 0; k < 2; k++) { a.critic[k] = net_of(A->critics[0]); a.target[k] = a.critic[k]; }       // the policy gradient goes through critic 0 (:260)
+    a.batch_base = A->observations_actions_base; a.noise = sampling_noise; a.sampling_std = A->sampling_std;
+    a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
+    a.out_pre_clip = A->actor_pre_clip;
+    const int groups = rlt_div_up(A->batch, ROWS);
+    int rc = launch_update<MODE_TD3_ACTOR>(device, a, groups, A->actor);
+    if (rc) return rc;
+    return reduce_and_step(device, a, groups, A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, nullptr, nullptr, nullptr, 0.0f);
 }
 
 int rlt_sac_polyak_list(rlt_rocm_device* device, const float* const* sources, float* const* targets, const uint32_t* counts, int n, float polyak) {

@@ -630,21 +630,21 @@ class Td3OnBackend:
     """All TD3 state for the Pendulum shapes (observation 3, action 1) on one backend. `params` is the flat vector
     [actor, actor_target, critic 0, critic 1, critic target 0, critic target 1], each [W|b] per layer."""
 
-    def __init__(self, backend, batch, hidden, params, hyper=None, masks=False, obs=3, act=1):
+    def __init__(self, backend, batch, hidden, params, hyper=None, masks=False, obs=3, act=1, hidden_act="relu"):
         OBS, ACT, D = obs, act, obs + act
         self.backend, self.batch, self.OBS, self.ACT = backend, batch, OBS, ACT
         adims, cdims = [OBS, hidden, hidden, ACT], [D, hidden, hidden, 1]
         na, nc = mlp_param_count(adims), mlp_param_count(cdims)
         assert params.size == 2 * na + 4 * nc
         o = 0
-        self.actor = Mlp(backend, adims, params[o:o + na], batch, out_act="tanh"); o += na
-        self.actor_target = Mlp(backend, adims, params[o:o + na], batch, out_act="tanh", trainable=False); o += na
+        self.actor = Mlp(backend, adims, params[o:o + na], batch, hidden_act, out_act="tanh"); o += na
+        self.actor_target = Mlp(backend, adims, params[o:o + na], batch, hidden_act, out_act="tanh", trainable=False); o += na
         self.critics = []
         for _ in range(2):
-            self.critics.append(Mlp(backend, cdims, params[o:o + nc], batch)); o += nc
+            self.critics.append(Mlp(backend, cdims, params[o:o + nc], batch, hidden_act)); o += nc
         self.targets = []
         for _ in range(2):
-            self.targets.append(Mlp(backend, cdims, params[o:o + nc], batch, trainable=False)); o += nc
+            self.targets.append(Mlp(backend, cdims, params[o:o + nc], batch, hidden_act, trainable=False)); o += nc
         z = backend.zeros
         self.oab = z((2, batch, D)); self.rewards = z((batch,)); self.terminated = z((batch,), np.uint8)
         self.m_final = backend.array(np.ones(batch, np.uint8)); self.m_next_final = backend.array(np.ones(batch, np.uint8))

@@ -104,4 +104,6 @@ def test_the_references_td3_loop_learns_the_pendulum_on_rocm():
     rate = float(re.search(r"loop_steps_per_second_including_evaluations ([\d.]+)", out.stdout).group(1))
     assert returns[0] < -600                                  # the untrained actor
     assert max(returns[-3:]) > -250 and final > -300          # the reference's TD3 reaches about -150 on the Pendulum within 10,000 steps
-    assert rate > 1000                                        # every operation runs on the device (host loops over device memory: a few steps per second)
+    # every operation runs on the device, and the update calls resolve to the overloads that hand a whole update to the library (its
+    # one-launch updates: 8,700 loop steps per second; one launch per reference operation: 2,000)
+    assert rate > 4000

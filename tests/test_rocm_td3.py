@@ -42,8 +42,11 @@ def test_elementwise_operations_bit_exact(oracle, rocm, B, A):
         assert np.array_equal(res["rocm"][k], want), k
 
 
-def test_lock_step_with_the_checker_on_the_references_run(oracle, rocm):
-    """The 36 loop steps of the committed reference run (72 critic updates, 18 delayed actor updates, 18 target updates of each kind).
+@pytest.mark.parametrize("per_operation", [1, 0])
+def test_lock_step_with_the_checker_on_the_references_run(oracle, rocm, per_operation):
+    """Both implementations of the updates: one launch per reference operation, and (the default for these shapes) the kernel that runs all
+    network passes of an update in one launch, which fills only target_action_value and the sampling layer's pre_clip of the training buffers.
+    The 36 loop steps of the committed reference run (72 critic updates, 18 delayed actor updates, 18 target updates of each kind).
     Before every step the HIP side gets the checker's exact state; both run the step on the reference's batch and draws; updated
     parameters of all six networks agree to 1e-5 of the largest parameter, gradients to 1e-5 of the largest gradient component times
     kappa = max|y| / max|Q - y| (rounding of Q is amplified by that factor in the TD error for any fp32 implementation)."""
@@ -51,20 +54,26 @@ def test_lock_step_with_the_checker_on_the_references_run(oracle, rocm):
     ref = helpers.Td3OnBackend(oracle, batch, hidden, g["parameters_before"], hyper=hyper)
     dev = helpers.Td3OnBackend(rocm, batch, hidden, g["parameters_before"], hyper=hyper)
     worst_p = worst_g = 0.0
+    rocm.call("sac_set_per_operation", per_operation)
     for i in range(steps):
         dev.push(ref.state())
         helpers.td3_golden_step(ref, g, i)
-        helpers.td3_golden_step(dev, g, i)
+        try:
+            helpers.td3_golden_step(dev, g, i)
+        finally:
+            rocm.call("sac_set_per_operation", 0)
+        rocm.call("sac_set_per_operation", per_operation)
         pe = rel_err(dev.parameters(), ref.parameters())
         y, td = ref.target_q.numpy(), ref.d_out_c.numpy() * batch / 2
         kappa = max(1.0, np.abs(y).max() / max(np.abs(td).max(), 1e-30))
         ge = rel_err(dev.gradients(), ref.gradients()) / kappa
         assert np.array_equal(dev.ages(), ref.ages())
-        assert rel_err(dev.target_q.numpy(), y) <= TOL and rel_err(dev.nsavi.numpy(), ref.nsavi.numpy()) <= TOL
+        assert rel_err(dev.target_q.numpy(), y) <= TOL and (not per_operation or rel_err(dev.nsavi.numpy(), ref.nsavi.numpy()) <= TOL)
         worst_p, worst_g = max(worst_p, pe), max(worst_g, ge)
         if i % 6 == 0:
             print(f"step {i}: parameters {pe:.2e} gradients/kappa {ge:.2e} kappa {kappa:.1f}", flush=True)
         assert pe <= TOL and ge <= TOL, (i, pe, ge)
+    rocm.call("sac_set_per_operation", 0)
     # the checker itself reproduced the reference's parameters bit for bit on the way (the CPU suite asserts the same)
     assert np.array_equal(ref.parameters(), g[f"s{steps - 1}_after"])
     print("worst: parameters %.2e gradients %.2e" % (worst_p, worst_g))
@@ -130,3 +139,51 @@ def test_one_update_at_other_shapes_with_masks(oracle, rocm, batch, hidden, obs,
         e = rel_err(got[k], want[k])
         print(k, "%.2e" % e, flush=True)
         assert e <= slack, (k, e)
+
+
+FUSED_SHAPES = [  # batch, obs, act, hidden activation
+    (256, 3, 1, "relu"),        # Pendulum
+    (256, 27, 8, "relu"),       # two input tiles, the widest action
+    (100, 17, 6, "tanh"),       # batch that is no multiple of 16
+    (1, 5, 2, "relu"),
+    (300, 111, 8, "fast_tanh"), # wide observations: the 128-input variant of the kernel
+]
+
+
+@pytest.mark.parametrize("batch,obs,act,hidden_act", FUSED_SHAPES)
+def test_fused_updates_match_the_checker_and_the_per_operation_path(oracle, rocm, batch, obs, act, hidden_act):
+    """The one-launch updates (rl/algorithms/td3/operations_generic.h:170-281 for actors obs -> 64 -> 64 -> act with tanh output and critics
+    obs + act -> 64 -> 64 -> 1): three loop steps (both critics, targets, actor, actor target each) from identical parameters, batches and noise
+    against the checker and against the one-launch-per-operation path; samples beyond [-1, 1] and terminated rows included. 1e-5 relative to
+    each tensor's largest magnitude."""
+    rng = np.random.default_rng(batch * 7 + obs)
+    D = obs + act
+    adims, cdims = [obs, 64, 64, act], [D, 64, 64, 1]
+    nets = [helpers.random_params(rng, adims)] * 2 + [helpers.random_params(rng, cdims) for _ in range(2)]
+    params = np.concatenate(nets + [nets[2] * 0.9, nets[3] * 1.1]).astype(np.float32)
+    hyper = dict(gamma=0.99, actor_polyak=0.995, critic_polyak=0.99, sampling_std=0.5, adam=helpers.capi.adam_parameters(epsilon=1e-7))
+    steps = []
+    for _ in range(3):
+        oab = rng.standard_normal((2, batch, D)).astype(np.float32); oab[:, :, obs:] = np.clip(oab[:, :, obs:], -1, 1)
+        steps.append((oab, rng.standard_normal(batch).astype(np.float32), (rng.random(batch) < 0.2).astype(np.uint8),
+                      np.clip(rng.standard_normal((batch, act)) * 0.2, -0.5, 0.5).astype(np.float32), [rng.standard_normal((batch, act)).astype(np.float32) for _ in range(3)]))
+    out = {}
+    for name, b, per_operation in (("checker", oracle, None), ("fused", rocm, 0), ("per_operation", rocm, 1)):
+        ag = helpers.Td3OnBackend(b, batch, 64, params, hyper=hyper, masks=False, obs=obs, act=act, hidden_act=hidden_act)
+        if per_operation is not None:
+            rocm.call("sac_set_per_operation", per_operation)
+        try:
+            for oab, rewards, term, tn, noises in steps:
+                ag.set_batch(oab, rewards, term, tn)
+                ag.loop_step([1, 1, 1, 1], *noises)
+        finally:
+            rocm.call("sac_set_per_operation", 0)
+        out[name] = dict(params=ag.parameters(), grads=ag.gradients(), y=ag.target_q.numpy(), pre_clip=ag.pre_clip.numpy(), ages=ag.ages(), nsavi=ag.nsavi.numpy())
+    # which path ran: only the per-operation launches fill the critics' next-input buffer
+    assert not out["fused"].pop("nsavi").any() and out["per_operation"].pop("nsavi").any() and out["checker"].pop("nsavi").any()
+    assert (np.abs(out["checker"]["pre_clip"]) > 1).sum() >= batch * act // 50
+    for other in ("checker", "per_operation"):
+        for key, ref in out[other].items():
+            err = rel_err(out["fused"][key], ref)
+            assert err <= TOL, (other, key, err)
+    assert np.abs(out["fused"]["params"] - params).max() > 1e-4
