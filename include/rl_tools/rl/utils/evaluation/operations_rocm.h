@@ -1,0 +1,59 @@
+// rl::utils::evaluation::evaluate on devices::ROCM (the generic version, rl/utils/evaluation/operations_generic.h:113-234, steps the
+// episodes one call at a time from the host; the reference's CUDA programs copy the actor to the CPU device and evaluate there,
+// src/rl/environments/pendulum/sac/cuda/sac.cu:6-27). With this overload the evaluation loop step
+// (rl/loop/steps/evaluation/operations_generic.h:56-92) runs on the device: all episodes of an evaluation are one call of the library
+// (rlt_rocm_pendulum_evaluate; actors 3 -> H -> H -> out with H <= 64 run every step of every episode in one launch).
+//
+// Covered: the Pendulum with an actor that is an MLP, alone or followed by sample_and_squash (SAC: action = tanh(mean) in evaluation
+// mode) or td3_sampling (TD3: the tanh output, no noise in evaluation mode); no per-step data collection.
+#pragma once
+#include <rl_tools/devices/rocm.h>
+#include <rl_tools/rl/utils/evaluation/evaluation.h>
+#include <rl_tools/rl/utils/evaluation/operations_generic.h>
+#include <rl_tools/rl/environments/pendulum/pendulum.h>
+#include <rl_tools/rl/components/off_policy_runner/operations_rocm.h>
+RL_TOOLS_NAMESPACE_WRAPPER_START
+namespace rl_tools{
+    template<typename DEV_SPEC, typename ENVIRONMENT, typename UI, typename POLICY, typename POLICY_STATE, typename POLICY_EVALUATION_BUFFERS, typename BUFFER_SPEC, typename DATA_SPEC, typename RNG, typename SPEC, typename MODE>
+    void evaluate(devices::ROCM<DEV_SPEC>& device, ENVIRONMENT& env_init, UI& ui, const POLICY& policy, POLICY_STATE& policy_state, POLICY_EVALUATION_BUFFERS& policy_evaluation_buffers, rl::utils::evaluation::Buffer<BUFFER_SPEC>& evaluation_buffers, rl::utils::evaluation::Result<SPEC>& results, rl::utils::evaluation::NoData<DATA_SPEC>& data, RNG& rng, const Mode<MODE>& mode){
+        using T = typename SPEC::T;
+        using TI = typename SPEC::TI;
+        using P = typename ENVIRONMENT::SPEC::PARAMETERS;
+        static_assert(utils::typing::is_same_v<ENVIRONMENT, rl::environments::Pendulum<typename ENVIRONMENT::SPEC>>, "the ROCM backend evaluates on the Pendulum; other environments are evaluated through rlt_rocm_env_evaluate");
+        static_assert(utils::typing::is_same_v<T, float> && sizeof(TI) == 4 && ENVIRONMENT::N_AGENTS == 1);
+        static_assert(mode::is<MODE, mode::Evaluation>, "the library's evaluation runs the actor in evaluation mode (no exploration noise)");
+        static_assert(P::initial_state_min_angle == -P::initial_state_max_angle && P::initial_state_min_speed == -P::initial_state_max_speed, "initial states are drawn from ranges that are symmetric about zero");
+        constexpr size_t N = SPEC::N_EPISODES;
+        rl::components::off_policy_runner::rocm::PolicyDescription d;
+        rl::components::off_policy_runner::rocm::describe(policy, d);
+        const rlt_pendulum_parameters parameters = {(float)P::g, (float)P::max_speed, (float)P::max_torque, (float)P::dt, (float)P::m, (float)P::l};
+        auto align = [](size_t bytes){ return (bytes + 255) / 256 * 256; };
+        const size_t initial_bytes = align(N * 2 * sizeof(float)), returns_bytes = align(N * sizeof(float)), length_bytes = align(N * sizeof(uint32_t));
+        char* memory = (char*)devices::rocm::scratch(device, initial_bytes + returns_bytes + length_bytes + 256);
+        float* initial = (float*)memory; float* returns = (float*)(memory + initial_bytes); uint32_t* episode_length = (uint32_t*)(memory + initial_bytes + returns_bytes);
+        float* summary = (float*)(memory + initial_bytes + returns_bytes + length_bytes);
+        if constexpr(SPEC::DETERMINISTIC_INITIAL_STATE){
+            // initial_state (rl/environments/pendulum/operations_generic.h:38-41): hanging down, at rest
+            float host[2 * N];
+            for(size_t e = 0; e < N; e++){ host[2 * e] = -math::PI<float>; host[2 * e + 1] = 0; }
+            devices::rocm::check(rlt_rocm_memcpy_h2d(device.handle, initial, host, sizeof(host)), "evaluate (initial states)");
+        }
+        else{
+            // sample_initial_state (:58-61): uniform in +- the largest angle and speed
+            devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, N * 2, -1.0f, 1.0f, rng.seed, random::next_stream(rng)), "evaluate (initial states)");
+            devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_angle, initial, 2, initial, 2, (int)N, 1), "evaluate (initial states)");
+            if constexpr(P::initial_state_max_speed != 1){
+                devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_speed, initial + 1, 2, initial + 1, 2, (int)N, 1), "evaluate (initial states)");
+            }
+        }
+        devices::rocm::check(rlt_rocm_pendulum_evaluate(device.handle, &parameters, d.has_head ? 2 : 1, d.layers, d.n_layers, initial, (int)N, (int)SPEC::STEP_LIMIT, returns, episode_length, summary), "evaluate");
+        float host_summary[6];
+        devices::rocm::check(rlt_rocm_memcpy_d2h(device.handle, results.returns, returns, N * sizeof(float)), "evaluate (results)");
+        devices::rocm::check(rlt_rocm_memcpy_d2h(device.handle, results.episode_length, episode_length, N * sizeof(uint32_t)), "evaluate (results)");
+        devices::rocm::check(rlt_rocm_memcpy_d2h(device.handle, host_summary, summary, sizeof(host_summary)), "evaluate (results)");
+        results.returns_mean = host_summary[0]; results.returns_std = host_summary[1];
+        results.episode_length_mean = host_summary[2]; results.episode_length_std = host_summary[3];
+        results.num_terminated = (TI)host_summary[4]; results.share_terminated = host_summary[5];
+    }
+}
+RL_TOOLS_NAMESPACE_WRAPPER_END

@@ -24,7 +24,7 @@ def test_programs_written_against_the_reference_api_compile_and_link():
     subprocess.run(["make", "-C", HERE, "syntax"], check=True, capture_output=True)
     out = subprocess.run(["make", "-B", "-C", HERE, "all"], capture_output=True, text=True)
     assert out.returncode == 0, out.stderr[-3000:]
-    for name in ("rocm_containers", "rocm_sac_pendulum", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
+    for name in ("rocm_containers", "rocm_sac_pendulum", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
         path = os.path.join(BUILD, name)
         assert os.path.exists(path)
         needed = subprocess.run(["readelf", "-d", path], capture_output=True, text=True).stdout
@@ -107,3 +107,21 @@ def test_the_references_td3_loop_learns_the_pendulum_on_rocm():
     # every operation runs on the device, and the update calls resolve to the overloads that hand a whole update to the library (its
     # one-launch updates: 8,700 loop steps per second; one launch per reference operation: 2,000)
     assert rate > 4000
+
+
+@pytest.mark.gpu
+def test_the_references_loop_steps_evaluate_on_the_device():
+    """The SAC loop inside the reference's evaluation and timing loop steps (rl/loop/steps/evaluation, rl/loop/steps/timing), the shape of its
+    training programs: `while(!step(device, ts))` and nothing else; the ten evaluations of 100 episodes run on the device through the evaluate
+    overload (rl/utils/evaluation/operations_rocm.h)."""
+    path = os.path.join(BUILD, "rocm_sac_pendulum_loop_steps")
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    out = subprocess.run([path, "0"], capture_output=True, text=True, timeout=300)
+    print(out.stdout[-1500:], flush=True)
+    assert out.returncode == 0, out.stderr[-2000:]
+    returns = [float(m) for m in re.findall(r"evaluation \d+ mean_return (-?[\d.]+)", out.stdout)]
+    rate = float(re.search(r"loop_steps_per_second_including_evaluations ([\d.]+)", out.stdout).group(1))
+    assert len(returns) == 10 and returns[0] < -600
+    assert sorted(returns[1:])[int(len(returns[1:]) * 0.8) - 1] > -200 and returns[-1] > -250
+    assert rate > 5000
