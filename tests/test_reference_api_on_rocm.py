@@ -24,7 +24,7 @@ def test_programs_written_against_the_reference_api_compile_and_link():
     subprocess.run(["make", "-C", HERE, "syntax"], check=True, capture_output=True)
     out = subprocess.run(["make", "-B", "-C", HERE, "all"], capture_output=True, text=True)
     assert out.returncode == 0, out.stderr[-3000:]
-    for name in ("rocm_containers", "rocm_sac_pendulum", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
+    for name in ("rocm_containers", "rocm_gru", "rocm_sac_pendulum", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
         path = os.path.join(BUILD, name)
         assert os.path.exists(path)
         needed = subprocess.run(["readelf", "-d", path], capture_output=True, text=True).stdout
@@ -125,3 +125,17 @@ def test_the_references_loop_steps_evaluate_on_the_device():
     assert len(returns) == 10 and returns[0] < -600
     assert sorted(returns[1:])[int(len(returns[1:]) * 0.8) - 1] > -200 and returns[-1] > -250
     assert rate > 5000
+
+
+@pytest.mark.gpu
+def test_gru_sequential_model_matches_the_references_cpu_device():
+    """A GRU -> dense sequential model of the reference on devices::ROCM next to the same model on the reference's CPU device, in one
+    program: forward, backward_full and an Adam step, with and without per-step resets; outputs, input gradients, parameter gradients and
+    updated parameters agree to 1e-4 of their largest magnitude (measured: 7e-8)."""
+    path = os.path.join(BUILD, "rocm_gru")
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    out = subprocess.run([path], capture_output=True, text=True, timeout=120)
+    print(out.stdout[-1500:], flush=True)
+    assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
+    assert float(re.search(r"worst ([\d.e+-]+)", out.stdout).group(1)) <= 1e-4

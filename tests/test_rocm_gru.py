@@ -26,7 +26,7 @@ def run_pair(oracle, rocm, S, B, I, H, seed, with_reset, **kw):
     return res
 
 
-@pytest.mark.parametrize("shape", [(7, 5, 6, 8), (1, 3, 4, 16), (12, 37, 20, 48), (9, 130, 3, 64), (5, 2, 7, 100)])
+@pytest.mark.parametrize("shape", [(7, 5, 6, 8), (1, 3, 4, 16), (24, 40, 11, 32), (12, 37, 20, 48), (9, 130, 3, 64), (5, 2, 7, 100)])
 @pytest.mark.parametrize("with_reset", [False, True])
 def test_gru_matches_checker(oracle, rocm, shape, with_reset):
     print("case", shape, with_reset, flush=True)
