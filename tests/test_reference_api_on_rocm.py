@@ -24,7 +24,7 @@ def test_programs_written_against_the_reference_api_compile_and_link():
     subprocess.run(["make", "-C", HERE, "syntax"], check=True, capture_output=True)
     out = subprocess.run(["make", "-B", "-C", HERE, "all"], capture_output=True, text=True)
     assert out.returncode == 0, out.stderr[-3000:]
-    for name in ("rocm_containers", "rocm_gru", "rocm_sac_pendulum", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
+    for name in ("rocm_containers", "rocm_gru", "rocm_sac_updates", "rocm_sac_pendulum", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
         path = os.path.join(BUILD, name)
         assert os.path.exists(path)
         needed = subprocess.run(["readelf", "-d", path], capture_output=True, text=True).stdout
@@ -139,3 +139,18 @@ def test_gru_sequential_model_matches_the_references_cpu_device():
     print(out.stdout[-1500:], flush=True)
     assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
     assert float(re.search(r"worst ([\d.e+-]+)", out.stdout).group(1)) <= 1e-4
+
+
+@pytest.mark.gpu
+def test_sac_updates_match_the_references_cpu_device():
+    """The reference itself as the checker: its train_critic / update_critic_targets / train_actor on its CPU device and the same calls on
+    devices::ROCM (which resolve to the library's one-launch updates), from one agent, on the batches the reference's runner gathered and
+    the noise its generator drew; 20 loop steps' worth of updates, every parameter tensor compared after each. Bound 1e-5 of the tensor's
+    largest magnitude (mean absolute difference); measured 2e-7."""
+    path = os.path.join(BUILD, "rocm_sac_updates")
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    out = subprocess.run([path], capture_output=True, text=True, timeout=120)
+    print(out.stdout[-2500:], flush=True)
+    assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
+    assert float(re.search(r"worst ([\d.e+-]+)", out.stdout).group(1)) <= 1e-5
