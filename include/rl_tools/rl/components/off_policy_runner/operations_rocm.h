@@ -23,6 +23,7 @@
 #include <rl_tools/nn/layers/dense/operations_rocm.h>
 #include <rl_tools/nn/layers/sample_and_squash/operations_rocm.h>
 #include <rl_tools/nn/layers/td3_sampling/layer.h>
+#include <rl_tools/nn/layers/standardize/layer.h>
 RL_TOOLS_NAMESPACE_WRAPPER_START
 namespace rl_tools{
     namespace rl::components::off_policy_runner::rocm{
@@ -76,7 +77,15 @@ namespace rl_tools{
             rlt_sas_parameters head = {};
             bool has_td3_sampling = false;      // the policy ends in a td3_sampling layer: action = clamp(output + std * noise, -1, 1)
             float td3_sampling_std = 0;
+            const float* standardize_mean = nullptr;        // the policy starts with a standardize layer: its statistics [input width], on the device
+            const float* standardize_precision = nullptr;
+            bool standardize_misplaced = false;             // ... anywhere else: no entry point of the library runs that
         };
+        template <typename LAYER_SPEC>
+        void describe(const nn::layers::standardize::LayerForward<LAYER_SPEC>& layer, PolicyDescription& d){
+            d.standardize_misplaced = d.standardize_misplaced || d.n_layers != 0 || d.standardize_mean != nullptr;
+            d.standardize_mean = layer.mean.parameters._data; d.standardize_precision = layer.precision.parameters._data;
+        }
         template <typename LAYER_SPEC>
         void describe(const nn::layers::dense::LayerForward<LAYER_SPEC>& layer, PolicyDescription& d){
             d.layers[d.n_layers++] = nn::layers::dense::rocm::describe_forward(layer);
@@ -186,6 +195,7 @@ namespace rl_tools{
         else{
             rl::components::off_policy_runner::rocm::PolicyDescription d;
             rl::components::off_policy_runner::rocm::describe(policy, d);
+            utils::assert_exit(device, d.standardize_mean == nullptr && !d.standardize_misplaced, "step(runner): the library's off-policy runner steps have no standardize layer");
             if(d.has_td3_sampling){
                 // TD3's exploring actor: the library's runner step for any environment and any sequential policy with a td3_sampling head (reset, observe,
                 // policy, clamp(output + std * noise), dynamics, reward, replay add: a handful of launches)

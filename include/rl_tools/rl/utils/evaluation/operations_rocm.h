@@ -5,7 +5,8 @@
 // (rlt_rocm_pendulum_evaluate; actors 3 -> H -> H -> out with H <= 64 run every step of every episode in one launch).
 //
 // Covered: the Pendulum with an actor that is an MLP, alone or followed by sample_and_squash (SAC: action = tanh(mean) in evaluation
-// mode) or td3_sampling (TD3: the tanh output, no noise in evaluation mode); no per-step data collection.
+// mode) or td3_sampling (TD3: the tanh output, no noise in evaluation mode), or preceded by a standardize layer (PPO: the action is the
+// mean of mlp_unconditional_stddev, nn_models/mlp_unconditional_stddev/operations_generic.h:23-49); no per-step data collection.
 #pragma once
 #include <rl_tools/devices/rocm.h>
 #include <rl_tools/rl/utils/evaluation/evaluation.h>
@@ -46,7 +47,8 @@ namespace rl_tools{
                 devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_speed, initial + 1, 2, initial + 1, 2, (int)N, 1), "evaluate (initial states)");
             }
         }
-        devices::rocm::check(rlt_rocm_pendulum_evaluate(device.handle, &parameters, d.has_head ? 2 : 1, d.layers, d.n_layers, initial, (int)N, (int)SPEC::STEP_LIMIT, returns, episode_length, summary), "evaluate");
+        utils::assert_exit(device, !d.standardize_misplaced, "evaluate: a standardize layer is supported in front of the first dense layer only");
+        devices::rocm::check(rlt_rocm_pendulum_evaluate_standardized(device.handle, &parameters, d.has_head ? 2 : 1, d.layers, d.n_layers, d.standardize_mean, d.standardize_precision, initial, (int)N, (int)SPEC::STEP_LIMIT, returns, episode_length, summary), "evaluate");
         float host_summary[6];
         devices::rocm::check(rlt_rocm_memcpy_d2h(device.handle, results.returns, returns, N * sizeof(float)), "evaluate (results)");
         devices::rocm::check(rlt_rocm_memcpy_d2h(device.handle, results.episode_length, episode_length, N * sizeof(uint32_t)), "evaluate (results)");

@@ -539,6 +539,13 @@ int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_ru
 int rlt_rocm_pendulum_evaluate(rlt_rocm_device* device, const rlt_pendulum_parameters* env, int policy_kind,
                                const rlt_dense_layer* actor, int n_actor_layers, const float* initial_states,
                                int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary);
+/* The same evaluation for an actor that starts with a standardize layer (nn/layers/standardize/operations_generic.h:69-135, the
+ * observation normalisation of PPO's actors, rl/algorithms/ppo/loop/core/approximators_sequential.h): every observation enters the
+ * first dense layer as (observation - observation_mean) * observation_precision, both [3] on the device; both NULL: no such layer. */
+int rlt_rocm_pendulum_evaluate_standardized(rlt_rocm_device* device, const rlt_pendulum_parameters* env, int policy_kind,
+                                            const rlt_dense_layer* actor, int n_actor_layers, const float* observation_mean,
+                                            const float* observation_precision, const float* initial_states, int n_episodes,
+                                            int step_limit, float* returns, uint32_t* episode_length, float* summary);
 
 /* Host-drawn randomness for rlt_rocm_sac_pendulum_loop (parity runs feed the draws the reference's CPU RNG made); any member
  * may be NULL, in which case the kernel draws it itself: Philox4x32-10 groups keyed by the launch's seed, one stream per kind of

@@ -1310,6 +1310,21 @@ int rlt_oracle_pendulum_evaluate(const rlt_pendulum_parameters* env, int policy_
                                   initial_states, n_episodes, step_limit, returns, episode_length, summary);
 }
 
+// with a standardize layer in front of the actor (nn/layers/standardize/operations_generic.h:69-135: output = (input - mean) * precision)
+int rlt_oracle_pendulum_evaluate_standardized(const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers, const float* observation_mean,
+                                              const float* observation_precision, const float* initial_states, int n_episodes, int step_limit, float* returns,
+                                              uint32_t* episode_length, float* summary) {
+    if (!env || !actor || n_actor_layers < 1 || !initial_states || n_episodes < 1 || step_limit < 1 || !returns || !episode_length || !summary) return RLT_E_INVALID_ARGUMENT;
+    if (policy_kind != 1 && policy_kind != 2) return RLT_E_INVALID_ARGUMENT;
+    if (actor[0].in_dim != 3 || actor[n_actor_layers - 1].out_dim != policy_kind || !observation_mean || !observation_precision) return RLT_E_INVALID_ARGUMENT;
+    std::vector<float> standardized((size_t)n_episodes * 3);
+    return pendulum_evaluate_impl(env, policy_kind, [&](const float* obs, float* out) {
+        for (int e = 0; e < n_episodes; e++)
+            for (int i = 0; i < 3; i++) standardized[(size_t)e * 3 + i] = (obs[(size_t)e * 3 + i] - observation_mean[i]) * observation_precision[i];
+        return rlt_oracle_mlp_evaluate(actor, n_actor_layers, standardized.data(), 3, out, policy_kind, n_episodes); },
+                                  initial_states, n_episodes, step_limit, returns, episode_length, summary);
+}
+
 // The same evaluation with a sequential (recurrent) policy: its kept state is reset for every episode before the first step (:135) and every step goes through
 // evaluate_step (:163), whose GRU layers restart their hidden state by themselves every auto_reset_period steps (nn/layers/gru/operations_generic.h:406-413;
 // 0: never). Terminated episodes keep being fed to the policy (:155-163), only their environment stops (:166-170).

@@ -47,6 +47,9 @@
  *   reduce_sum_f32, adam_reset: against numpy closed forms (tests/test_oracle_rng.py, tests/test_oracle_closed_forms.py).
  *   pendulum_evaluate_recurrent: returns, lengths and summary bit for bit against rl::utils::evaluation::evaluate on that loop's recurrent actor at two
  *   depths, untrained and trained; golden vectors; equality with pendulum_evaluate for a policy of dense layers only.
+ *   pendulum_evaluate_standardized: identity statistics give pendulum_evaluate's results exactly; other statistics give those of the network with the
+ *   statistics folded into its first layer (tests/test_oracle_closed_forms.py). The layer itself, (x - mean) * precision, is the one the PPO loop's
+ *   standardize pins cover (ppo_train_minibatch with standardize layers, on_policy_collect).
  */
 #ifndef RLT_ORACLE_H
 #define RLT_ORACLE_H
@@ -190,6 +193,9 @@ int rlt_oracle_car_track_step(const rlt_car_parameters* p, const uint8_t* track,
 int rlt_oracle_pendulum_evaluate(const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers, const float* initial_states,
                                  int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary);
 /* the same with a sequential (recurrent) policy: state reset before the first step, evaluate_step per step (:135,:163) */
+int rlt_oracle_pendulum_evaluate_standardized(const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers, const float* observation_mean,
+                                              const float* observation_precision, const float* initial_states, int n_episodes, int step_limit, float* returns,
+                                              uint32_t* episode_length, float* summary);
 int rlt_oracle_pendulum_evaluate_recurrent(const rlt_pendulum_parameters* env, int policy_kind, const rlt_seq_layer* policy, int n_layers, const rlt_seq_state* state,
                                            int auto_reset_period, const float* initial_states, int n_episodes, int step_limit, float* returns,
                                            uint32_t* episode_length, float* summary);

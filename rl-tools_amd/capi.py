@@ -291,6 +291,7 @@ PROTOTYPES = {
     "env_on_policy_collect": [C.POINTER(EnvRunner), C.POINTER(OnPolicyDataset), C.POINTER(SeqLayer), I, C.POINTER(SeqState), I, P, P, P, P, P, I, P, S],
     "car_track_step": [C.POINTER(CarParameters), P, I, I, F, P, P, P, P, P, P, I],
     "pendulum_evaluate": [C.POINTER(PendulumParameters), I, LP, I, P, I, I, P, P, P],
+    "pendulum_evaluate_standardized": [C.POINTER(PendulumParameters), I, LP, I, P, P, P, I, I, P, P, P],
     "ppo_gae": [P, P, P, P, P, P, I, I, I, F, F, I],
     "gru_forward": [C.POINTER(GruLayer), P, P, I, I, P, S],
     "gru_backward": [C.POINTER(GruLayer), P, P, P, P, I, I, I, P, S],

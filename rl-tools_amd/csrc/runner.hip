@@ -579,6 +579,7 @@ bool rb_ok(const rlt_replay_buffer* rb) {
 struct EvaluateArgs {
     rlt_pendulum_parameters env;
     const float *w1, *b1, *w2, *b2, *w3, *b3;
+    const float *std_mean, *std_precision;      // a standardize layer in front of the actor: (observation - mean) * precision; NULL: none
     int H, act1, act2, act_out, policy_kind, step_limit;
     const float* initial_states; float* returns; uint32_t* episode_length;
 };
@@ -590,11 +591,13 @@ __global__ __launch_bounds__(64) void pendulum_evaluate_kernel(EvaluateArgs A) {
     const bool live = j < H;
     const int jc = live ? j : 0;
     const float w10 = A.w1[jc * 3], w11 = A.w1[jc * 3 + 1], w12 = A.w1[jc * 3 + 2], b1 = A.b1[jc], b2 = A.b2[jc], w3 = live ? A.w3[jc] : 0.f, b3 = A.b3[0];
+    float m0 = 0.f, m1 = 0.f, m2 = 0.f, p0 = 1.f, p1 = 1.f, p2 = 1.f;
+    if (A.std_mean) { m0 = A.std_mean[0]; m1 = A.std_mean[1]; m2 = A.std_mean[2]; p0 = A.std_precision[0]; p1 = A.std_precision[1]; p2 = A.std_precision[2]; }
     float theta = A.initial_states[2 * e], theta_dot = A.initial_states[2 * e + 1], episode_return = 0.f;
     float sn, cs;
     sincosf(theta, &sn, &cs);
     for (int step = 0; step < A.step_limit; step++) {
-        const float h1 = live ? rlt_act(b1 + w10 * cs + w11 * sn + w12 * theta_dot, A.act1) : 0.f;
+        const float h1 = live ? rlt_act(b1 + w10 * ((cs - m0) * p0) + w11 * ((sn - m1) * p1) + w12 * ((theta_dot - m2) * p2), A.act1) : 0.f;
         float acc = b2;
         for (int k = 0; k < H; k++) acc += w2s[j * 65 + k] * __int_as_float(__builtin_amdgcn_readlane(__float_as_int(h1), k));
         const float h2 = live ? rlt_act(acc, A.act2) : 0.f;
@@ -613,11 +616,14 @@ __global__ __launch_bounds__(64) void pendulum_evaluate_kernel(EvaluateArgs A) {
     if (j == 0) { A.returns[e] = episode_return; A.episode_length[e] = (uint32_t)A.step_limit; }
 }
 // other actor shapes: one step of all episodes per launch around the per-layer network kernels
-__global__ __launch_bounds__(256) void evaluate_observe_kernel(const float* __restrict__ states, float* __restrict__ obs, int n) {
+__global__ __launch_bounds__(256) void evaluate_observe_kernel(const float* __restrict__ states, float* __restrict__ obs, int n, const float* __restrict__ std_mean,
+                                                               const float* __restrict__ std_precision) {
     const int e = blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= n) return;
     float sn, cs; sincosf(states[2 * e], &sn, &cs);
-    obs[3 * e] = cs; obs[3 * e + 1] = sn; obs[3 * e + 2] = states[2 * e + 1];
+    float o[3] = {cs, sn, states[2 * e + 1]};
+    if (std_mean) for (int i = 0; i < 3; i++) o[i] = (o[i] - std_mean[i]) * std_precision[i];
+    obs[3 * e] = o[0]; obs[3 * e + 1] = o[1]; obs[3 * e + 2] = o[2];
 }
 __global__ __launch_bounds__(256) void evaluate_step_kernel(rlt_pendulum_parameters env, float* __restrict__ states, const float* __restrict__ actor_out, int ld_out, int policy_kind,
                                                             float* __restrict__ returns, uint32_t* __restrict__ episode_length, int n) {
@@ -825,8 +831,16 @@ int rlt_rocm_on_policy_collect(rlt_rocm_device* device, const rlt_pendulum_runne
 // rl::utils::evaluation::evaluate with the Pendulum environment (rl/utils/evaluation/operations_generic.h:106-233)
 int rlt_rocm_pendulum_evaluate(rlt_rocm_device* device, const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers,
                                const float* initial_states, int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary) {
+    return rlt_rocm_pendulum_evaluate_standardized(device, env, policy_kind, actor, n_actor_layers, nullptr, nullptr, initial_states, n_episodes, step_limit, returns,
+                                                   episode_length, summary);
+}
+// the same with a standardize layer (nn/layers/standardize/operations_generic.h:69-135) in front of the actor, as PPO's actors have it
+int rlt_rocm_pendulum_evaluate_standardized(rlt_rocm_device* device, const rlt_pendulum_parameters* env, int policy_kind, const rlt_dense_layer* actor, int n_actor_layers,
+                                            const float* observation_mean, const float* observation_precision, const float* initial_states, int n_episodes,
+                                            int step_limit, float* returns, uint32_t* episode_length, float* summary) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(env && actor && n_actor_layers >= 1 && initial_states && n_episodes >= 1 && step_limit >= 1 && returns && episode_length && summary);
+    RLT_REQUIRE((observation_mean == nullptr) == (observation_precision == nullptr));
     RLT_REQUIRE((policy_kind == 1 || policy_kind == 2) && actor[0].in_dim == 3 && actor[n_actor_layers - 1].out_dim == policy_kind);
     for (int l = 0; l < n_actor_layers; l++) RLT_REQUIRE(actor[l].weights && actor[l].biases && (l == 0 || actor[l].in_dim == actor[l - 1].out_dim));
     const int N = n_episodes;
@@ -835,6 +849,7 @@ int rlt_rocm_pendulum_evaluate(rlt_rocm_device* device, const rlt_pendulum_param
         EvaluateArgs a = {};
         a.env = *env;
         a.w1 = actor[0].weights; a.b1 = actor[0].biases; a.w2 = actor[1].weights; a.b2 = actor[1].biases; a.w3 = actor[2].weights; a.b3 = actor[2].biases;
+        a.std_mean = observation_mean; a.std_precision = observation_precision;
         a.H = actor[0].out_dim; a.act1 = actor[0].activation; a.act2 = actor[1].activation; a.act_out = actor[2].activation; a.policy_kind = policy_kind; a.step_limit = step_limit;
         a.initial_states = initial_states; a.returns = returns; a.episode_length = episode_length;
         hipLaunchKernelGGL(pendulum_evaluate_kernel, dim3(N), dim3(64), 0, device->stream, a);
@@ -852,7 +867,7 @@ int rlt_rocm_pendulum_evaluate(rlt_rocm_device* device, const rlt_pendulum_param
         if ((rc = rlt_rocm_fill_f32(device, returns, 1, N, N, 0.0f))) return rc;
         if ((rc = rlt_rocm_fill_f32(device, (float*)episode_length, 1, N, N, 0.0f))) return rc;      // the bit pattern of 0.0f is the integer 0
         for (int step = 0; step < step_limit; step++) {
-            hipLaunchKernelGGL(evaluate_observe_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, states, obs, N);
+            hipLaunchKernelGGL(evaluate_observe_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, states, obs, N, observation_mean, observation_precision);
             if ((rc = rlt_launch_status(device))) return rc;
             if ((rc = rlt_rocm_mlp_evaluate(device, actor, n_actor_layers, obs, 3, out, out_dim, N, ws, mlp_ws))) return rc;
             hipLaunchKernelGGL(evaluate_step_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *env, states, out, out_dim, policy_kind, returns, episode_length, N);
@@ -890,7 +905,7 @@ int rlt_rocm_pendulum_evaluate_recurrent(rlt_rocm_device* device, const rlt_pend
     if ((rc = rlt_rocm_fill_f32(device, (float*)episode_length, 1, N, N, 0.0f))) return rc;      // the bit pattern of 0.0f is the integer 0
     if ((rc = rlt_rocm_seq_reset_state(device, policy, n_layers, state, nullptr, N))) return rc;
     for (int step = 0; step < step_limit; step++) {
-        hipLaunchKernelGGL(evaluate_observe_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, states, obs, N);
+        hipLaunchKernelGGL(evaluate_observe_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, states, obs, N, (const float*)nullptr, (const float*)nullptr);
         if ((rc = rlt_launch_status(device))) return rc;
         if ((rc = rlt_rocm_seq_evaluate_step(device, policy, n_layers, obs, 3, state, auto_reset_period, out, policy_kind, N, w + head, step_ws))) return rc;
         hipLaunchKernelGGL(evaluate_step_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *env, states, out, policy_kind, policy_kind, returns, episode_length, N);

@@ -191,6 +191,17 @@ def random_params(rng, dims, bias_scale=0.1):
     return np.concatenate(parts)
 
 
+def fold_standardize_into_first_layer(dims, params, mean, precision):
+    """The flat parameters of the network that computes W1 ((x - mean) * precision) + b1 as W1' x + b1' (in double, rounded once)."""
+    out = params.astype(np.float32).copy()
+    n_w = dims[1] * dims[0]
+    w = params[:n_w].reshape(dims[1], dims[0]).astype(np.float64) * np.asarray(precision, np.float64)[None, :]
+    b = params[n_w:n_w + dims[1]].astype(np.float64) - w @ np.asarray(mean, np.float64)
+    out[:n_w] = w.reshape(-1).astype(np.float32)
+    out[n_w:n_w + dims[1]] = b.astype(np.float32)
+    return out
+
+
 class Mlp:
     """A dense network laid out as flat arenas (parameters, gradients, Adam moments) on a backend, described to the C ABI
     by an array of rlt_dense_layer."""
@@ -856,13 +867,19 @@ def on_policy_golden_collect(backend, g, k, dims, col):
     return o
 
 
-def evaluate_on_backend(backend, dims, params, hidden_act, out_act, policy_kind, initial_states, step_limit):
-    """rl::utils::evaluation::evaluate on a backend: returns (returns, episode_length, summary) as numpy arrays."""
+def evaluate_on_backend(backend, dims, params, hidden_act, out_act, policy_kind, initial_states, step_limit, standardize=None):
+    """rl::utils::evaluation::evaluate on a backend: returns (returns, episode_length, summary) as numpy arrays. standardize = (mean [3], precision [3]): a
+    standardize layer in front of the actor."""
     n = initial_states.shape[0]
     actor = Mlp(backend, dims, params, n, hidden_act, out_act, trainable=False)
     ini, ret, length, summary = backend.array(initial_states.astype(np.float32)), backend.zeros((n,)), backend.zeros((n,), np.uint32), backend.zeros((6,))
     env = capi.pendulum_parameters()
-    backend.call("pendulum_evaluate", C.byref(env), policy_kind, actor.layers, actor.n, ini.ptr, n, step_limit, ret.ptr, length.ptr, summary.ptr)
+    if standardize is not None:
+        mean, precision = backend.array(np.asarray(standardize[0], np.float32)), backend.array(np.asarray(standardize[1], np.float32))
+        backend.call("pendulum_evaluate_standardized", C.byref(env), policy_kind, actor.layers, actor.n, mean.ptr, precision.ptr, ini.ptr, n, step_limit, ret.ptr, length.ptr,
+                     summary.ptr)
+    else:
+        backend.call("pendulum_evaluate", C.byref(env), policy_kind, actor.layers, actor.n, ini.ptr, n, step_limit, ret.ptr, length.ptr, summary.ptr)
     backend.sync()
     return ret.numpy(), length.numpy(), summary.numpy()
 

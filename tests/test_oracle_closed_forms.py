@@ -293,3 +293,21 @@ def test_gather_deterministic_mode_and_ring_index_brute_force(oracle):
         i = ring[(pos + max_ep + s) % cap]
         assert np.all(oab.numpy()[0, s, :3] == i) and oab.numpy()[0, s, 3] == -i and rew.numpy()[s] == i * 10
         assert np.all(oab.numpy()[1, s, :3] == i + 0.5) and oab.numpy()[1, s, 3] == 0 and term.numpy()[s] == (i % 5 == 0)
+
+
+def test_evaluation_with_a_standardize_layer_is_the_plain_one_with_folded_statistics(oracle):
+    """(x - m) * p in front of W x + b is W' x + b' with W' = W diag(p), b' = b - W' m: the checker's standardized evaluation against its plain
+    evaluation of the folded network (short horizon: the fold changes the rounding), and identity statistics against the plain one exactly."""
+    rng = np.random.default_rng(11)
+    dims = [3, 24, 24, 1]
+    params = helpers.random_params(rng, dims)
+    n = 12
+    ini = np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n)], 1).astype(np.float32)
+    mean, precision = rng.normal(0, 0.5, 3).astype(np.float32), rng.uniform(0.3, 3, 3).astype(np.float32)
+    plain = helpers.evaluate_on_backend(oracle, dims, params, "tanh", "identity", 1, ini, 10)
+    same = helpers.evaluate_on_backend(oracle, dims, params, "tanh", "identity", 1, ini, 10, (np.zeros(3), np.ones(3)))
+    assert np.array_equal(plain[0], same[0]) and np.array_equal(plain[2], same[2])
+    got = helpers.evaluate_on_backend(oracle, dims, params, "tanh", "identity", 1, ini, 10, (mean, precision))
+    folded = helpers.fold_standardize_into_first_layer(dims, params, mean, precision)
+    want = helpers.evaluate_on_backend(oracle, dims, folded, "tanh", "identity", 1, ini, 10)
+    assert helpers.rel_err(got[0], want[0]) <= 1e-4 and helpers.rel_err(got[0], plain[0]) > 1e-2

@@ -24,7 +24,7 @@ def test_programs_written_against_the_reference_api_compile_and_link():
     subprocess.run(["make", "-C", HERE, "syntax"], check=True, capture_output=True)
     out = subprocess.run(["make", "-B", "-C", HERE, "all"], capture_output=True, text=True)
     assert out.returncode == 0, out.stderr[-3000:]
-    for name in ("rocm_containers", "rocm_gru", "rocm_sac_updates", "rocm_sac_pendulum", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
+    for name in ("rocm_containers", "rocm_gru", "rocm_sac_updates", "rocm_zoo_pendulum_v1_sac", "rocm_zoo_pendulum_v1_td3", "rocm_zoo_pendulum_v1_ppo", "rocm_sac_pendulum", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
         path = os.path.join(BUILD, name)
         assert os.path.exists(path)
         needed = subprocess.run(["readelf", "-d", path], capture_output=True, text=True).stdout
@@ -154,3 +154,23 @@ def test_sac_updates_match_the_references_cpu_device():
     print(out.stdout[-2500:], flush=True)
     assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
     assert float(re.search(r"worst ([\d.e+-]+)", out.stdout).group(1)) <= 1e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("algorithm,best_at_least,seconds_at_most", [("sac", -300.0, 20.0), ("td3", -300.0, 20.0), ("ppo", -400.0, 60.0)])
+def test_zoo_configurations_of_the_pendulum_train_on_rocm(algorithm, best_at_least, seconds_at_most):
+    """The reference's zoo configurations (src/rl/zoo/pendulum-v1/{sac,td3,ppo}.h, included as they are: batch 100 and width 64 for SAC and TD3,
+    width 32 with fast_tanh, observation normalisation and an entropy bonus for PPO) inside its evaluation and timing loop steps on devices::ROCM,
+    to their own step limits (20,000 loop steps; 1,221 PPO iterations = 10 M environment steps) with 100 evaluations of 100 episodes on the device.
+    A random actor's mean return is about -1,300; measured best returns -125 (SAC, 1.6 s), -129 (TD3, 2.1 s), -158 (PPO, 6.5 s)."""
+    path = os.path.join(BUILD, "rocm_zoo_pendulum_v1_" + algorithm)
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    out = subprocess.run([path], capture_output=True, text=True, timeout=170)
+    print(out.stdout[-1200:], flush=True)
+    assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
+    final = re.search(r"final ([\d.e+-]+) best ([\d.e+-]+) loop_steps (\d+) seconds ([\d.e+-]+)", out.stdout)
+    first = float(re.search(r"evaluation 0 step 0 mean_return ([\d.e+-]+)", out.stdout).group(1))
+    assert first < -900.0
+    assert float(final.group(2)) >= best_at_least and float(final.group(4)) <= seconds_at_most
+    assert len(re.findall(r"^evaluation \d+ ", out.stdout, re.M)) == 100

@@ -45,6 +45,27 @@ def test_evaluation_matches_checker(oracle, rocm, case):
         assert rel_err(got[2][:2], want[2][:2]) <= tol and np.array_equal(got[2][2:], want[2][2:])
 
 
+@pytest.mark.parametrize("case", [(32, 3, 1, "fast_tanh", "identity", 100), (64, 3, 1, "tanh", "identity", 10), (128, 3, 1, "tanh", "identity", 16), (16, 3, 2, "relu", "identity", 5)])
+def test_evaluation_with_a_standardize_layer_matches_checker(oracle, rocm, case):
+    """PPO's actors: (observation - mean) * precision in front of the first layer (one launch for widths <= 64, step by step above)."""
+    print("case", case, flush=True)
+    H, layers, kind, ha, oa, n = case
+    dims = [3] + [H] * (layers - 1) + [kind]
+    rng = np.random.default_rng(3 * H + n)
+    params = helpers.random_params(rng, dims)
+    ini = np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n)], 1).astype(np.float32)
+    standardize = (rng.normal(0, 0.5, 3).astype(np.float32), rng.uniform(0.3, 3, 3).astype(np.float32))
+    plain = helpers.evaluate_on_backend(rocm, dims, params, ha, oa, kind, ini, 20)
+    for steps, tol in ((20, 1e-5), (200, 2e-3)):
+        want = helpers.evaluate_on_backend(oracle, dims, params, ha, oa, kind, ini, steps, standardize)
+        got = helpers.evaluate_on_backend(rocm, dims, params, ha, oa, kind, ini, steps, standardize)
+        assert np.array_equal(got[1], want[1]) and np.all(got[1] == steps)
+        assert rel_err(got[0], want[0]) <= tol, (steps, rel_err(got[0], want[0]))
+        assert rel_err(got[2][:2], want[2][:2]) <= tol and np.array_equal(got[2][2:], want[2][2:])
+        if steps == 20:
+            assert rel_err(got[0], plain[0]) > 1e-3      # the layer is not ignored
+
+
 def test_evaluation_rejects_bad_arguments(rocm):
     capi = helpers.capi
     import ctypes as C
