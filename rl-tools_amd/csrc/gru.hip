@@ -275,6 +275,174 @@ __global__ __launch_bounds__(GRU_THREADS) void gru_backward_reg_kernel(GruArgs A
     if (A.db_hn_partial) A.db_hn_partial[(size_t)b * H + u] = db_hn;
 }
 
+// ---- hidden width 64: the recurrence on the matrix cores -------------------------------------------------------------------------
+// A workgroup of four wavefronts carries FOUR batch rows through the sequence; W_h stays in registers as the B operand of
+// v_mfma_f32_4x4x1_16b_f32 (16 blocks of a 4 x 1 by 1 x 4 product: lane 4 blk + i supplies A[i], lane 4 blk + j supplies B[j], register i of
+// lane 4 blk + j receives D[i][j]; with the broadcast control set to 16 blocks every block takes its A from the block the instruction names,
+// so one register of previous hidden states feeds 16 reduction steps). The four rows are the A side (i = row), a block is one hidden unit and
+// its four columns are that unit's r, z and n gates (the fourth is idle): 64 instructions of 8 cycles replace the 192 multiply-adds and 64
+// lane reads per lane of the vector version, and a step takes about half its time at any batch size (the chain of dependent steps, not the
+// arithmetic, bounds both).
+// The gates at this width on the hardware's exponential and reciprocal (v_exp_f32, v_rcp_f32: 1 ulp each; absolute error of a gate below 3e-7, an order
+// below the tolerance the layer is held to): the library routines cost 500 cycles of every step's 1,900, these 300.
+__device__ __forceinline__ float hw_sigmoid(float x) { return __frcp_rn(1.0f + __expf(-x)); }
+__device__ __forceinline__ float hw_tanh(float x) { return 1.0f - 2.0f * __frcp_rn(__expf(2.0f * x) + 1.0f); }
+typedef float gru_floatx4 __attribute__((ext_vector_type(4)));
+constexpr int GM_ROWS = 4;
+template <int ABID> __device__ __forceinline__ gru_floatx4 mfma4(float a, float b, gru_floatx4 c) { return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, c, 4, ABID, 0); }
+// 16 reduction steps: A register `a` holds, in block blk, the four rows' values of reduction index base + blk
+__device__ __forceinline__ void mfma4_16(float a, const float* w, gru_floatx4& c0, gru_floatx4& c1, gru_floatx4& c2, gru_floatx4& c3) {
+    c0 = mfma4<0>(a, w[0], c0); c1 = mfma4<1>(a, w[1], c1); c2 = mfma4<2>(a, w[2], c2); c3 = mfma4<3>(a, w[3], c3);
+    c0 = mfma4<4>(a, w[4], c0); c1 = mfma4<5>(a, w[5], c1); c2 = mfma4<6>(a, w[6], c2); c3 = mfma4<7>(a, w[7], c3);
+    c0 = mfma4<8>(a, w[8], c0); c1 = mfma4<9>(a, w[9], c1); c2 = mfma4<10>(a, w[10], c2); c3 = mfma4<11>(a, w[11], c3);
+    c0 = mfma4<12>(a, w[12], c0); c1 = mfma4<13>(a, w[13], c1); c2 = mfma4<14>(a, w[14], c2); c3 = mfma4<15>(a, w[15], c3);
+}
+
+// Wavefront w owns hidden units 16 w ... 16 w + 15. hs (two copies, by the parity of the step) holds the previous hidden state of the four rows,
+// unit-major: hs[unit * 4 + row]. One workgroup barrier per step; the pre-activations pass from the matrix layout (lane = unit, gate; register =
+// row) to the lane that finishes (row, unit) through a slot of LDS private to the wavefront.
+template <bool FAST>
+__global__ __launch_bounds__(256) void gru_forward_mfma_kernel(GruArgs A) {
+    constexpr int H = 64;
+    __shared__ __align__(16) float hs[2][H * GM_ROWS];
+    __shared__ __align__(16) float xw[4][GM_ROWS * 64];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, blk = lane >> 2, j = lane & 3;
+    // B operand: column j of block blk = gate j of unit 16 w + blk, one register per reduction index
+    float wb[H];
+    {
+        const float4* src = reinterpret_cast<const float4*>(A.L.weights_hidden + ((size_t)(j < 3 ? j : 0) * H + 16 * w + blk) * H);
+#pragma unroll
+        for (int q = 0; q < H / 4; q++) {
+            const float4 v = src[q];
+            wb[4 * q] = j < 3 ? v.x : 0.f; wb[4 * q + 1] = j < 3 ? v.y : 0.f; wb[4 * q + 2] = j < 3 ? v.z : 0.f; wb[4 * q + 3] = j < 3 ? v.w : 0.f;
+        }
+    }
+    // the lane that finishes (row, unit)
+    const int row_local = lane >> 4, u = 16 * w + (lane & 15);
+    const int b_raw = blockIdx.x * GM_ROWS + row_local;
+    const bool live = b_raw < A.B;
+    const int b = live ? b_raw : A.B - 1;      // rows beyond the batch read the last row and store nothing
+    const float bhr = A.L.biases_hidden[u], bhz = A.L.biases_hidden[H + u], bhn = A.L.biases_hidden[2 * H + u];
+    const float h0 = A.L.initial_hidden_state[u];
+    const size_t stride = (size_t)A.B * 3 * H;
+    // The inputs W_i x + b_i (and the reset flag) of step t + D are requested during step t and wait in a queue: consecutive steps lie 12 H B bytes
+    // apart, and a load takes longer than a step.
+    constexpr int D = 4;
+    struct In { float r, z, n; int rs; };
+    auto request = [&](int t) {
+        const int tc = t < A.S ? t : A.S - 1;       // the last steps request the last one again: no branch around the loads
+        const float* p = A.L.post_activation + (size_t)tc * stride + (size_t)b * 3 * H;
+        In v; v.r = p[u]; v.z = p[H + u]; v.n = p[2 * H + u]; v.rs = A.reset ? A.reset[(size_t)tc * A.B + b] : 0;
+        return v;
+    };
+    In q[D];
+#pragma unroll
+    for (int d = 0; d < D; d++) q[d] = request(d);
+    float h = h0;
+    hs[0][u * GM_ROWS + row_local] = h;
+    for (int t = 0; t < A.S; t++) {
+        rlt_lds_barrier();
+        const float* hp = hs[t & 1];
+        const float a0 = hp[lane], a1 = hp[64 + lane], a2 = hp[128 + lane], a3 = hp[192 + lane];
+        const In far = request(t + D);
+        gru_floatx4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = c0, c2 = c0, c3 = c0;
+        mfma4_16(a0, wb, c0, c1, c2, c3); mfma4_16(a1, wb + 16, c0, c1, c2, c3); mfma4_16(a2, wb + 32, c0, c1, c2, c3); mfma4_16(a3, wb + 48, c0, c1, c2, c3);
+        const gru_floatx4 c = (c0 + c1) + (c2 + c3);
+        float* x = xw[w];
+        x[lane] = c[0]; x[64 + lane] = c[1]; x[128 + lane] = c[2]; x[192 + lane] = c[3];      // x[(row * 16 + unit) * 4 + gate]
+        wave_sync();
+        const float4 pre = *reinterpret_cast<const float4*>(x + 4 * lane);
+        wave_sync();
+        const float ar = bhr + pre.x, az = bhz + pre.y, an = bhn + pre.z;
+        const float r = FAST ? gate_sigmoid(q[0].r + ar, 1) : hw_sigmoid(q[0].r + ar), z = FAST ? gate_sigmoid(q[0].z + az, 1) : hw_sigmoid(q[0].z + az);
+        const float n = FAST ? gate_tanh(q[0].n + an * r, 1) : hw_tanh(q[0].n + an * r);
+        h = (1.0f - z) * n + z * h;
+        if (live) {
+            float* po = A.L.post_activation + (size_t)t * stride + (size_t)b * 3 * H;
+            po[u] = r; po[H + u] = z; po[2 * H + u] = n;
+            const size_t at = ((size_t)t * A.B + b) * H + u;
+            A.L.n_pre_pre_activation[at] = an;
+            A.L.output[at] = h;
+        }
+        if (t + 1 < A.S && q[1].rs) h = h0;       // the next step starts an episode
+        hs[(t + 1) & 1][u * GM_ROWS + row_local] = h;
+#pragma unroll
+        for (int d = 0; d + 1 < D; d++) q[d] = q[d + 1];
+        q[D - 1] = far;
+    }
+}
+
+// Reverse pass. The gate gradients of the four rows are the A side, the reduction runs over the 192 (gate, unit) pairs -- a quarter per
+// wavefront, whose B operands are rows 48 w ... 48 w + 47 of W_h (lane = column: coalesced) -- and the four partial sums of d h_prev meet in
+// LDS. Thread (w, lane) finishes (row w, unit lane): its loads and stores are whole rows. Two workgroup barriers per step.
+__global__ __launch_bounds__(256) void gru_backward_mfma_kernel(GruArgs A) {
+    constexpr int H = 64, GS = 3 * H + 16;      // row stride of the gate gradients in LDS: rows 16 banks apart
+    __shared__ float gs[GM_ROWS * GS];
+    __shared__ float part[4][GM_ROWS * 64];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, blk = lane >> 2, i = lane & 3;
+    float wb[48];
+#pragma unroll
+    for (int k = 0; k < 48; k++) wb[k] = A.L.weights_hidden[(size_t)(48 * w + k) * H + lane];
+    const int b_raw = blockIdx.x * GM_ROWS + w;
+    const bool live = b_raw < A.B;
+    const int b = live ? b_raw : A.B - 1;
+    const int u = lane;
+    const float h0 = A.L.initial_hidden_state[u];
+    float carry = 0.f, db_hn = 0.f;
+    struct Saved { float r, z, n, npp, dy, hp; int rs; };
+    auto request = [&](int t) {
+        const size_t a = (size_t)(t > 0 ? t : 0) * A.B + b;
+        Saved v;
+        v.r = A.L.post_activation[a * 3 * H + u]; v.z = A.L.post_activation[a * 3 * H + H + u]; v.n = A.L.post_activation[a * 3 * H + 2 * H + u];
+        v.npp = A.L.n_pre_pre_activation[a * H + u]; v.dy = A.d_output[a * H + u];
+        v.hp = A.L.output[((size_t)(t > 1 ? t - 1 : 0) * A.B + b) * H + u];
+        v.rs = A.reset ? A.reset[a] : 0;
+        return v;
+    };
+    // a step's saved values are requested D steps ahead (a load takes longer than a step); steps before the first read the first again
+    constexpr int D = 3;
+    Saved q[D];
+#pragma unroll
+    for (int d = 0; d < D; d++) q[d] = request(A.S - 1 - d);
+    for (int t = A.S - 1; t >= 0; t--) {
+        const size_t at = (size_t)t * A.B + b;
+        const Saved far = request(t - D);
+        const Saved cur = q[0];
+        const bool from_initial = t == 0 || cur.rs;
+        const float hp = from_initial ? h0 : cur.hp;
+        const float dh = cur.dy + carry;
+        const float gz = dh * (hp - cur.n) * cur.z * (1.0f - cur.z);
+        const float gn = dh * (1.0f - cur.z) * (1.0f - cur.n * cur.n);
+        const float gr = gn * cur.npp * cur.r * (1.0f - cur.r);
+        const float gnr = gn * cur.r;
+        if (live) {
+            A.d_output[at * H + u] = dh;
+            float* bi = A.buffer_input + at * 3 * H; float* bh = A.buffer_hidden + at * 3 * H;
+            bi[u] = gr; bi[H + u] = gz; bi[2 * H + u] = gn;
+            bh[u] = gr; bh[H + u] = gz; bh[2 * H + u] = gnr;
+            A.h_previous[at * H + u] = hp;
+        }
+        // the reference drops reset samples (t > 0) from the b_hn gradient (their buffer rows are zeroed before that sum, :716-749)
+        if (!(t > 0 && from_initial)) db_hn += gnr;
+        gs[w * GS + u] = gr; gs[w * GS + H + u] = gz; gs[w * GS + 2 * H + u] = gnr;
+        rlt_lds_barrier();
+        const float* ga = gs + i * GS + 48 * w + blk;
+        const float a0 = ga[0], a1 = ga[16], a2 = ga[32];
+        gru_floatx4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = c0, c2 = c0, c3 = c0;
+        mfma4_16(a0, wb, c0, c1, c2, c3); mfma4_16(a1, wb + 16, c0, c1, c2, c3); mfma4_16(a2, wb + 32, c0, c1, c2, c3);
+        const gru_floatx4 c = (c0 + c1) + (c2 + c3);
+        float* pw = part[w];
+        pw[lane] = c[0]; pw[64 + lane] = c[1]; pw[128 + lane] = c[2]; pw[192 + lane] = c[3];      // part[w][row * 64 + column]
+        rlt_lds_barrier();
+        const float sum = (part[0][w * 64 + u] + part[1][w * 64 + u]) + (part[2][w * 64 + u] + part[3][w * 64 + u]);
+        carry = from_initial ? 0.f : dh * cur.z + sum;
+#pragma unroll
+        for (int d = 0; d + 1 < D; d++) q[d] = q[d + 1];
+        q[D - 1] = far;
+    }
+    if (live && A.db_hn_partial) A.db_hn_partial[(size_t)b * H + u] = db_hn;
+}
+
 // db_h[n part] += sum over batch rows of the per-row sums, db_h[r, z parts] = db_i[r, z parts] (the reference copies, :679-681).
 // One workgroup per hidden unit.
 __global__ __launch_bounds__(256) void gru_bias_hidden_kernel(const float* __restrict__ partial, int B, int H, const float* __restrict__ db_i, float* __restrict__ db_h) {
@@ -319,7 +487,10 @@ int rlt_rocm_gru_forward(rlt_rocm_device* device, const rlt_gru_layer* L, const 
     if (H == 64 || H == 32 || H == 16) {
         const dim3 grid(rlt_div_up(B, GRU_THREADS / H)), block(GRU_THREADS);      // GRU_THREADS / 64 wavefronts of 64 / H rows
         const bool fast = L->fast_tanh != 0;      // a template parameter: as a run-time switch inside the step it cost 10% at width 64
-        if (H == 64) { if (fast) hipLaunchKernelGGL((gru_forward_reg_kernel<64, true>), grid, block, 0, device->stream, a); else hipLaunchKernelGGL((gru_forward_reg_kernel<64, false>), grid, block, 0, device->stream, a); }
+        if (H == 64) {
+            const dim3 grid4(rlt_div_up(B, GM_ROWS));
+            if (fast) hipLaunchKernelGGL(gru_forward_mfma_kernel<true>, grid4, block, 0, device->stream, a); else hipLaunchKernelGGL(gru_forward_mfma_kernel<false>, grid4, block, 0, device->stream, a);
+        }
         else if (H == 32) { if (fast) hipLaunchKernelGGL((gru_forward_reg_kernel<32, true>), grid, block, 0, device->stream, a); else hipLaunchKernelGGL((gru_forward_reg_kernel<32, false>), grid, block, 0, device->stream, a); }
         else { if (fast) hipLaunchKernelGGL((gru_forward_reg_kernel<16, true>), grid, block, 0, device->stream, a); else hipLaunchKernelGGL((gru_forward_reg_kernel<16, false>), grid, block, 0, device->stream, a); }
         return rlt_launch_status(device);
@@ -347,7 +518,7 @@ int rlt_rocm_gru_backward(rlt_rocm_device* device, const rlt_gru_layer* L, const
     a.h_previous = h_previous; a.db_hn_partial = want_weight_gradients ? db_hn_partial : nullptr; a.S = S; a.B = B; a.rows_per_group = rows_per_group(H);
     if (H == 64 || H == 32 || H == 16) {
         const dim3 grid(rlt_div_up(B, GRU_THREADS / H)), block(GRU_THREADS);
-        if (H == 64) hipLaunchKernelGGL(gru_backward_reg_kernel<64>, grid, block, 0, device->stream, a);
+        if (H == 64) hipLaunchKernelGGL(gru_backward_mfma_kernel, dim3(rlt_div_up(B, GM_ROWS)), block, 0, device->stream, a);
         else if (H == 32) hipLaunchKernelGGL(gru_backward_reg_kernel<32>, grid, block, 0, device->stream, a);
         else hipLaunchKernelGGL(gru_backward_reg_kernel<16>, grid, block, 0, device->stream, a);
     } else {
