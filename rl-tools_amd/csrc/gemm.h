@@ -11,8 +11,11 @@ int rlt_gemm_backward_input(rlt_rocm_device* device, const float* d_pre, int ldd
                             const float* dact_pre, int dact_kind, int dact_from_output, int batch, int in_dim, int out_dim);
 // dW += d_pre^T x ; dbias += column sums of d_pre (dbias may be NULL). The partial sums of a split batch go to the handle's grow-only
 // workspace, or, with static_scratch, to the library's fixed device array (RLT_E_WORKSPACE_TOO_SMALL beyond RLT_STATIC_SCRATCH_BYTES).
+// narrow_long: the caller's layers are narrow (at most 192 x 160) and its batches long; such shapes then take the kernel that keeps the whole
+// gradient in one workgroup's accumulators (another summation order than the tiled kernel's, so the dense-layer entry points, which promise
+// each other's bits, do not ask for it).
 int rlt_gemm_wgrad(rlt_rocm_device* device, const float* d_pre, int ldd, const float* x, int ldx, float* dW, float* dbias,
-                   int batch, int in_dim, int out_dim, bool static_scratch = false);
+                   int batch, int in_dim, int out_dim, bool static_scratch = false, bool narrow_long = false);
 // looks up, once per GPU, where that GPU keeps the fixed array (called by rlt_rocm_init with the handle's device)
 int rlt_gemm_static_scratch_setup(rlt_rocm_device* device);
 // dst <- act'(pre) * src (dst may alias src; then a no-op for the identity)

@@ -256,6 +256,127 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(float* __restrict__ d
     }
 }
 
+// ---- weight gradients of narrow layers over long batches ----------------------------------------------------------------------------
+// dW [M x N] with M <= 192, N <= 16 NT (a GRU's 3H x I and 3H x H at hidden width 64) over tens of thousands of rows: the tiled kernel above
+// cuts such a matrix into 64 x 64 tiles and every operand row is fetched by three workgroups, each with a short reduction of its own. Here a
+// workgroup keeps the WHOLE gradient in accumulators (wavefront w: rows 48 w ... 48 w + 47 of dW as 3 x NT tiles of v_mfma_f32_16x16x4_f32) and
+// walks its share of the batch 16 rows at a time: both operands are read from memory exactly once, staged through LDS (double buffered, the
+// next 16 rows requested before the current ones are multiplied, one barrier per 16 rows). The bias gradient is summed on the side from the
+// registers the d_pre rows pass through. A workgroup writes one block of partial sums in the layout wgrad_reduce_kernel adds up.
+typedef float wide_floatx4 __attribute__((ext_vector_type(4)));
+constexpr int WIDE_M = 192, WIDE_KT = 16, WIDE_GS = WIDE_M + 16;
+struct WideArgs { const float* G; int ldg; const float* X; int ldx; int M, N, K, rows_per_group; float* ws; int want_bias; };
+template <int NT, int PF>
+__global__ __launch_bounds__(THREADS) void wgrad_wide_kernel(WideArgs a) {
+    constexpr int XS = 16 * NT + 16;                        // both strides are 16 mod 32: the four k-rows a wavefront reads fall on two sets of banks
+    constexpr int GQ = WIDE_KT * WIDE_M / 4 / THREADS;      // float4 of d_pre per thread and 16 rows (3)
+    constexpr int XQ = (WIDE_KT * 8 * NT + THREADS - 1) / THREADS;      // float2 of x per thread and 16 rows
+    __shared__ __align__(16) float gs[2][WIDE_KT * WIDE_GS];
+    __shared__ __align__(16) float xs[2][WIDE_KT * XS];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r = lane & 15, kk = lane >> 4;
+    const int k_begin = blockIdx.x * a.rows_per_group, k_end = min(a.K, k_begin + a.rows_per_group);
+    // 16 rows of both operands as they travel from memory to LDS. A load under load takes longer than the matrix work on 16 rows, so PF such
+    // tiles are on their way at any time (with one, the kernel ran at the rate of one tile per memory latency: 2 TB/s over the whole device).
+    struct Tile { float4 g[GQ]; float2 x[XQ]; };
+    float4 bsum[GQ];
+#pragma unroll
+    for (int q = 0; q < GQ; q++) bsum[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto request = [&](int k0) {
+        Tile t;
+#pragma unroll
+        for (int q = 0; q < GQ; q++) {
+            const int idx = tid + THREADS * q, row = idx / (WIDE_M / 4), col = 4 * (idx % (WIDE_M / 4));
+            t.g[q] = (k0 + row < k_end && col < a.M) ? *reinterpret_cast<const float4*>(a.G + (size_t)(k0 + row) * a.ldg + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int q = 0; q < XQ; q++) {
+            const int idx = tid + THREADS * q, row = idx / (8 * NT), col = 2 * (idx % (8 * NT));
+            t.x[q] = (idx < WIDE_KT * 8 * NT && k0 + row < k_end && col < a.N) ? *reinterpret_cast<const float2*>(a.X + (size_t)(k0 + row) * a.ldx + col) : make_float2(0.f, 0.f);
+        }
+        return t;
+    };
+    auto stage = [&](const Tile& t, int buf) {
+#pragma unroll
+        for (int q = 0; q < GQ; q++) {
+            const int idx = tid + THREADS * q, row = idx / (WIDE_M / 4), col = 4 * (idx % (WIDE_M / 4));
+            *reinterpret_cast<float4*>(&gs[buf][row * WIDE_GS + col]) = t.g[q];
+            bsum[q].x += t.g[q].x; bsum[q].y += t.g[q].y; bsum[q].z += t.g[q].z; bsum[q].w += t.g[q].w;
+        }
+#pragma unroll
+        for (int q = 0; q < XQ; q++) {
+            const int idx = tid + THREADS * q, row = idx / (8 * NT), col = 2 * (idx % (8 * NT));
+            if (idx < WIDE_KT * 8 * NT) *reinterpret_cast<float2*>(&xs[buf][row * XS + col]) = t.x[q];
+        }
+    };
+    wide_floatx4 acc[3][NT];
+#pragma unroll
+    for (int i = 0; i < 3; i++)
+#pragma unroll
+        for (int j = 0; j < NT; j++) acc[i][j] = wide_floatx4{0.f, 0.f, 0.f, 0.f};
+    Tile queue[PF];
+    {
+        const Tile first = request(k_begin);
+#pragma unroll
+        for (int d = 0; d < PF; d++) queue[d] = request(k_begin + (d + 1) * WIDE_KT);
+        stage(first, 0);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = k_begin; k0 < k_end; k0 += WIDE_KT) {
+        const Tile far = request(k0 + (PF + 1) * WIDE_KT);
+        __builtin_amdgcn_sched_barrier(0);      // the requests go out first, and nothing that waits for them moves above the matrix work
+        const float* g = gs[buf] + kk * WIDE_GS + 48 * w + r;
+        const float* x = xs[buf] + kk * XS + r;
+#pragma unroll
+        for (int s4 = 0; s4 < WIDE_KT / 4; s4++) {
+            float av[3], bv[NT];
+#pragma unroll
+            for (int i = 0; i < 3; i++) av[i] = g[4 * s4 * WIDE_GS + 16 * i];
+#pragma unroll
+            for (int j = 0; j < NT; j++) bv[j] = x[4 * s4 * XS + 16 * j];
+#pragma unroll
+            for (int i = 0; i < 3; i++)
+#pragma unroll
+                for (int j = 0; j < NT; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (k0 + WIDE_KT < k_end) stage(queue[0], buf ^ 1);
+        rlt_lds_barrier();
+        buf ^= 1;
+#pragma unroll
+        for (int d = 0; d + 1 < PF; d++) queue[d] = queue[d + 1];
+        queue[PF - 1] = far;
+    }
+    // element v of lane (r, kk) of tile (i, j): dW[48 w + 16 i + 4 kk + v][16 j + r]
+    float* out = a.ws + (size_t)blockIdx.x * ((size_t)a.M * a.N + a.M);
+#pragma unroll
+    for (int i = 0; i < 3; i++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int m = 48 * w + 16 * i + 4 * kk + v;
+#pragma unroll
+            for (int j = 0; j < NT; j++) {
+                const int n = 16 * j + r;
+                if (m < a.M && n < a.N) out[(size_t)m * a.N + n] = acc[i][j][v];
+            }
+        }
+    if (a.want_bias) {      // 16 row slots of column sums meet in LDS and are added in the order of the slots
+        float* bs = gs[0];
+#pragma unroll
+        for (int q = 0; q < GQ; q++) {
+            const int idx = tid + THREADS * q, row = idx / (WIDE_M / 4), col = 4 * (idx % (WIDE_M / 4));
+            *reinterpret_cast<float4*>(&bs[row * WIDE_GS + col]) = bsum[q];
+        }
+        __syncthreads();
+        if (tid < a.M) {
+            float sum = 0.f;
+#pragma unroll
+            for (int row = 0; row < WIDE_KT; row++) sum += bs[row * WIDE_GS + tid];
+            out[(size_t)a.M * a.N + tid] = sum;
+        }
+    }
+}
+
 // d_pre = act'(pre) * d_output (nn/layers/dense/operations_cpu_blas.h:119-141); dst may alias src
 __global__ __launch_bounds__(256) void dpre_kernel(const float* src, int lds, float* dst, int ldd, const float* __restrict__ pre, int rows, int cols, int act, int from_output) {
     const size_t total = (size_t)rows * cols;
@@ -383,11 +504,26 @@ int rlt_gemm_static_scratch_setup(rlt_rocm_device* device) {
 }
 
 int rlt_gemm_wgrad(rlt_rocm_device* device, const float* d_pre, int ldd, const float* x, int ldx, float* dW, float* dbias,
-                   int batch, int in_dim, int out_dim, bool static_scratch) {
+                   int batch, int in_dim, int out_dim, bool static_scratch, bool narrow_long) {
     GemmParams p = {};
     p.A = d_pre; p.lda = ldd; p.B = x; p.ldb = ldx; p.M = out_dim; p.N = in_dim; p.K = batch;
     p.vecA = vector_width(d_pre, ldd); p.vecB = vector_width(x, ldx);
     p.dW = dW; p.dbias = dbias;
+    // narrow layer, long batch: one workgroup per share of the batch holds the whole gradient (wgrad_wide_kernel)
+    if (narrow_long && !static_scratch && out_dim <= WIDE_M && out_dim % 4 == 0 && in_dim > 64 && in_dim <= 160 && in_dim % 2 == 0 && batch >= 16384 && ldd % 4 == 0 && ldx % 2 == 0 &&
+        (reinterpret_cast<uintptr_t>(d_pre) & 15u) == 0 && (reinterpret_cast<uintptr_t>(x) & 7u) == 0) {
+        const int groups = device->compute_units < batch / 64 ? device->compute_units : batch / 64;
+        const int rows_per_group = rlt_div_up(rlt_div_up(batch, groups), WIDE_KT) * WIDE_KT, used = rlt_div_up(batch, rows_per_group);
+        void* ws = nullptr;
+        int rc = rlt_scratch(device, (size_t)used * ((size_t)out_dim * in_dim + out_dim) * sizeof(float), &ws);
+        if (rc) return rc;
+        WideArgs a = {d_pre, ldd, x, ldx, out_dim, in_dim, batch, rows_per_group, (float*)ws, 1};
+        hipLaunchKernelGGL((wgrad_wide_kernel<10, 2>), dim3(used), dim3(THREADS), 0, device->stream, a);
+        if ((rc = rlt_launch_status(device))) return rc;
+        const int mn = out_dim * in_dim;
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(rlt_div_up(mn + out_dim, 64)), dim3(256), 0, device->stream, dW, dbias, (const float*)ws, mn, out_dim, used);
+        return rlt_launch_status(device);
+    }
     int splits, kps;
     wgrad_split(device, batch, in_dim, out_dim, splits, kps);
     p.k_per_split = kps; p.splits = splits;

@@ -529,8 +529,8 @@ int rlt_rocm_gru_backward(rlt_rocm_device* device, const rlt_gru_layer* L, const
     int rc = rlt_launch_status(device);
     if (rc) return rc;
     if (want_weight_gradients) {
-        if ((rc = rlt_gemm_wgrad(device, buffer_input, 3 * H, input, I, L->d_weights_input, L->d_biases_input, rows, I, 3 * H))) return rc;       // :677-678
-        if ((rc = rlt_gemm_wgrad(device, buffer_hidden, 3 * H, h_previous, H, L->d_weights_hidden, nullptr, rows, H, 3 * H))) return rc;         // :693-742
+        if ((rc = rlt_gemm_wgrad(device, buffer_input, 3 * H, input, I, L->d_weights_input, L->d_biases_input, rows, I, 3 * H, false, true))) return rc;       // :677-678
+        if ((rc = rlt_gemm_wgrad(device, buffer_hidden, 3 * H, h_previous, H, L->d_weights_hidden, nullptr, rows, H, 3 * H, false, true))) return rc;         // :693-742
         hipLaunchKernelGGL(gru_bias_hidden_kernel, dim3(H), dim3(256), 0, device->stream, (const float*)db_hn_partial, B, H, (const float*)L->d_biases_input, L->d_biases_hidden);
         if ((rc = rlt_launch_status(device))) return rc;
     }

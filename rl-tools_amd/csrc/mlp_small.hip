@@ -462,7 +462,7 @@ bool shape_ok(const rlt_dense_layer* L, int n) {
     return L && n == 3 && L[0].in_dim >= 1 && L[0].in_dim <= MAX_IN && L[0].out_dim == H && L[1].in_dim == H && L[1].out_dim == H && L[2].in_dim == H &&
            L[2].out_dim >= 1 && L[2].out_dim <= MAX_OUT && L[0].activation == L[1].activation && hidden_act_ok(L[0].activation) && out_act_ok(L[2].activation);
 }
-int tile_bucket(int in) { return in <= 32 ? 2 : MAX_NT1; }
+int tile_bucket(int in) { return in <= 32 ? 2 : in <= 64 ? 4 : MAX_NT1; }
 
 // one or two networks in one launch; two only if they share the hidden activation and the input-width bucket
 int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
@@ -502,9 +502,9 @@ int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
         }                                                                                                                                                       \
     } while (0)
     switch (act) {
-        case RLT_ACT_RELU: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_RELU, 2); else RLT_LAUNCH_SMALL(RLT_ACT_RELU, MAX_NT1); break;
-        case RLT_ACT_TANH: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_TANH, 2); else RLT_LAUNCH_SMALL(RLT_ACT_TANH, MAX_NT1); break;
-        default: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_FAST_TANH, 2); else RLT_LAUNCH_SMALL(RLT_ACT_FAST_TANH, MAX_NT1); break;
+        case RLT_ACT_RELU: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_RELU, 2); else if (bucket == 4) RLT_LAUNCH_SMALL(RLT_ACT_RELU, 4); else RLT_LAUNCH_SMALL(RLT_ACT_RELU, MAX_NT1); break;
+        case RLT_ACT_TANH: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_TANH, 2); else if (bucket == 4) RLT_LAUNCH_SMALL(RLT_ACT_TANH, 4); else RLT_LAUNCH_SMALL(RLT_ACT_TANH, MAX_NT1); break;
+        default: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_FAST_TANH, 2); else if (bucket == 4) RLT_LAUNCH_SMALL(RLT_ACT_FAST_TANH, 4); else RLT_LAUNCH_SMALL(RLT_ACT_FAST_TANH, MAX_NT1); break;
     }
 #undef RLT_LAUNCH_SMALL
     if ((rc = rlt_launch_status(device))) return rc;

@@ -87,3 +87,29 @@ def test_gru_benchmark_shape(oracle, rocm):
     lin = g2.results()
     for k in ("dW_i", "db_i", "dW_h", "db_h", "dx"):
         assert rel_err(lin[k], -2.0 * big[k]) <= 2e-6, k
+
+
+def test_gru_weight_gradients_over_a_long_batch(oracle, rocm):
+    """16,384 (step, row) pairs and more take the weight-gradient kernel that keeps the whole 192 x 146 / 192 x 64 gradient in one workgroup's accumulators:
+    batch 256 against the checker; batch 1,024 as the sum of its four quarters run separately (the gradients add over batch rows)."""
+    S, I, H = 64, 146, 64
+    print("batch 256 against the checker", flush=True)
+    want, got = run_pair(oracle, rocm, S, 256, I, H, 33, True)
+    for k in KEYS:
+        assert rel_err(got[k], want[k]) <= 2e-5, (k, rel_err(got[k], want[k]))
+    print("batch 1,024 against its quarters", flush=True)
+    rng = np.random.default_rng(34)
+    params, x, dy, reset = helpers.gru_random_case(rng, S, 1024, I, H, True)
+    g = helpers.GruOnBackend(rocm, S, 1024, I, H, params)
+    g.forward(x, reset); g.backward(dy); rocm.sync()
+    whole = g.results()
+    parts = []
+    for q in range(4):
+        sl = slice(256 * q, 256 * (q + 1))
+        gq = helpers.GruOnBackend(rocm, S, 256, I, H, params)
+        gq.forward(np.ascontiguousarray(x[:, sl]), None if reset is None else np.ascontiguousarray(reset[:, sl])); gq.backward(np.ascontiguousarray(dy[:, sl])); rocm.sync()
+        parts.append(gq.results())
+    for k in ("dW_i", "db_i", "dW_h", "db_h"):
+        assert rel_err(whole[k], sum(p[k] for p in parts)) <= 1e-5, k
+    for k in ("output", "dx"):
+        assert rel_err(whole[k][:, 256:512], parts[1][k]) <= 2e-6, k
