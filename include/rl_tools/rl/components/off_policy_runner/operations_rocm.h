@@ -24,6 +24,7 @@
 #include <rl_tools/nn/layers/sample_and_squash/operations_rocm.h>
 #include <rl_tools/nn/layers/td3_sampling/layer.h>
 #include <rl_tools/nn/layers/standardize/layer.h>
+#include <rl_tools/nn/layers/gru/operations_rocm.h>
 RL_TOOLS_NAMESPACE_WRAPPER_START
 namespace rl_tools{
     namespace rl::components::off_policy_runner::rocm{
@@ -115,6 +116,58 @@ namespace rl_tools{
             }
         }
     }
+    namespace rl::components::off_policy_runner::rocm{
+        // a sequential policy with GRU layers and the state it carries between rollout steps, as the library's recurrent entry points take them
+        struct RecurrentPolicyDescription{
+            rlt_seq_layer layers[RLT_SEQ_MAX_LAYERS] = {};
+            rlt_seq_state state = {};
+            int n_layers = 0;
+            bool has_gru = false, has_head = false, unsupported = false;
+            rlt_sas_parameters head = {};
+        };
+        template <typename LAYER_SPEC, typename STATE>
+        void describe_recurrent(const nn::layers::dense::LayerForward<LAYER_SPEC>& layer, STATE&, RecurrentPolicyDescription& d){
+            if(d.n_layers >= RLT_SEQ_MAX_LAYERS){ d.unsupported = true; return; }
+            d.layers[d.n_layers].kind = 0; d.layers[d.n_layers].dense = nn::layers::dense::rocm::describe_forward(layer);
+            d.n_layers++;
+        }
+        template <typename LAYER_SPEC, typename STATE_SPEC>
+        void describe_recurrent(const nn::layers::gru::LayerForward<LAYER_SPEC>& layer, nn::layers::gru::State<STATE_SPEC>& state, RecurrentPolicyDescription& d){
+            static_assert(sizeof(typename LAYER_SPEC::TI) == 4, "the step counters of a GRU state are 32-bit on devices::ROCM");
+            if(d.n_layers >= RLT_SEQ_MAX_LAYERS){ d.unsupported = true; return; }
+            d.layers[d.n_layers].kind = 1; d.layers[d.n_layers].gru = nn::layers::gru::rocm::describe_forward(layer);
+            d.state.hidden[d.n_layers] = state.state._data; d.state.step[d.n_layers] = (uint32_t*)state.step._data;
+            d.has_gru = true;
+            d.n_layers++;
+        }
+        template <typename LAYER_SPEC, typename STATE>
+        void describe_recurrent(const nn::layers::sample_and_squash::LayerForward<LAYER_SPEC>& layer, STATE&, RecurrentPolicyDescription& d){
+            d.has_head = true;
+            d.head = nn::layers::sample_and_squash::rocm::parameters<LAYER_SPEC>();
+        }
+        template <typename MODULE_SPEC, typename CONTENT_STATE>
+        void describe_recurrent(const nn_models::sequential::ModuleForward<MODULE_SPEC>& module, CONTENT_STATE& state, RecurrentPolicyDescription& d){
+            describe_recurrent(module.content, state.state, d);
+            if constexpr(!utils::typing::is_same_v<typename MODULE_SPEC::NEXT_MODULE, nn_models::sequential::OutputModule>){
+                describe_recurrent(module.next_module, state.next_content_state, d);
+            }
+        }
+        // whether a policy type has a GRU layer (such policies take the recurrent runner step)
+        template <typename T> struct IsGru{ static constexpr bool value = false; };
+        template <typename SPEC> struct IsGru<nn::layers::gru::LayerForward<SPEC>>{ static constexpr bool value = true; };
+        template <typename SPEC> struct IsGru<nn::layers::gru::LayerBackward<SPEC>>{ static constexpr bool value = true; };
+        template <typename SPEC> struct IsGru<nn::layers::gru::LayerGradient<SPEC>>{ static constexpr bool value = true; };
+        template <typename MODULE_SPEC>
+        constexpr bool module_has_gru(){
+            if constexpr(IsGru<typename MODULE_SPEC::CONTENT>::value){ return true; }
+            else if constexpr(utils::typing::is_same_v<typename MODULE_SPEC::NEXT_MODULE, nn_models::sequential::OutputModule>){ return false; }
+            else{ return module_has_gru<typename MODULE_SPEC::NEXT_MODULE::SPEC>(); }
+        }
+        template <typename...> using void_t = void;
+        template <typename POLICY, typename = void> struct HasGru{ static constexpr bool value = false; };
+        // sequential models (nn_models::sequential::Build derives from its first module, so the module's SPEC is looked at, not the type)
+        template <typename POLICY> struct HasGru<POLICY, void_t<typename POLICY::SPEC::CONTENT, typename POLICY::SPEC::NEXT_MODULE>>{ static constexpr bool value = module_has_gru<typename POLICY::SPEC>(); };
+    }
     // malloc / free           off_policy_runner/operations_cuda.h:100-133
     template<typename DEV_SPEC, typename SPEC>
     void malloc(devices::ROCM<DEV_SPEC>& device, rl::components::OffPolicyRunner<SPEC>& runner){
@@ -192,6 +245,31 @@ namespace rl_tools{
             rand(device, actions, rng, -1.0f, 1.0f);
             devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 0, nullptr, 0, nullptr, runner.buffers.actions._data, nullptr, nullptr, rng.seed, random::next_stream(rng)), "step(runner, uniform policy)");
         }
+        else if constexpr(rl::components::off_policy_runner::rocm::HasGru<POLICY>::value){
+            // a recurrent actor (off_policy_runner/operations_generic.h:189-206): the policy state of the environments that start an episode is reset, then one
+            // evaluate_step in Rollout mode; GRU layers restart by themselves every SEQUENCE_LENGTH steps of their input shape (nn/layers/gru/operations_generic.h:406-413)
+            using ENVIRONMENT = typename SPEC::ENVIRONMENT;
+            using P = typename ENVIRONMENT::SPEC::PARAMETERS;
+            static_assert(P::initial_state_min_angle == -P::initial_state_max_angle && P::initial_state_min_speed == -P::initial_state_max_speed, "initial states are drawn from ranges that are symmetric about zero");
+            constexpr size_t ACT = ENVIRONMENT::ACTION_DIM;
+            rl::components::off_policy_runner::rocm::RecurrentPolicyDescription d;
+            rl::components::off_policy_runner::rocm::describe_recurrent(policy, get<POLICY_INDEX>(runner.policy_states).content_state, d);
+            utils::assert_exit(device, !d.unsupported && d.has_head, "step(runner): a recurrent policy is dense and GRU layers followed by sample_and_squash");
+            auto align = [](size_t bytes){ return (bytes + 255) / 256 * 256; };
+            const size_t noise_bytes = align(N * ACT * sizeof(float)), initial_bytes = align(N * 2 * sizeof(float));
+            const size_t workspace_bytes = rlt_rocm_pendulum_runner_step_recurrent_workspace_bytes(d.layers, d.n_layers, (int)N);
+            char* memory = (char*)devices::rocm::scratch(device, noise_bytes + initial_bytes + workspace_bytes);
+            float* noise = (float*)memory; float* initial = (float*)(memory + noise_bytes);
+            devices::rocm::check(rlt_rocm_randn_f32(device.handle, noise, N * ACT, rng.seed, random::next_stream(rng)), "step(runner, noise)");
+            devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, N * 2, -1.0f, 1.0f, rng.seed, random::next_stream(rng)), "step(runner, initial states)");
+            devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_angle, initial, 2, initial, 2, (int)N, 1), "step(runner, initial states)");
+            if constexpr(P::initial_state_max_speed != 1){
+                devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_speed, initial + 1, 2, initial + 1, 2, (int)N, 1), "step(runner, initial states)");
+            }
+            constexpr int AUTO_RESET_PERIOD = (int)get<0>(typename POLICY::INPUT_SHAPE{});
+            devices::rocm::check(rlt_rocm_pendulum_runner_step_recurrent(device.handle, &r, &rb, d.layers, d.n_layers, &d.state, AUTO_RESET_PERIOD, &d.head, noise, initial,
+                                                                         memory + noise_bytes + initial_bytes, workspace_bytes), "step(runner, recurrent actor)");
+        }
         else{
             rl::components::off_policy_runner::rocm::PolicyDescription d;
             rl::components::off_policy_runner::rocm::describe(policy, d);
@@ -242,9 +320,34 @@ namespace rl_tools{
     template <typename DEV_SPEC, typename SPEC, typename BATCH_SPEC, typename RNG, bool DETERMINISTIC = false>
     void gather_batch(devices::ROCM<DEV_SPEC>& device, rl::components::OffPolicyRunner<SPEC>& runner, rl::components::off_policy_runner::SequentialBatch<BATCH_SPEC>& batch, RNG& rng){
         static_assert(utils::typing::is_same_v<SPEC, typename BATCH_SPEC::SPEC>);
-        static_assert(BATCH_SPEC::SEQUENCE_LENGTHH == 1, "sequence batches are gathered through rlt_rocm_gather_sequence_batch; this overload covers SEQUENCE_LENGTH = 1");
         constexpr int BATCH_SIZE = BATCH_SPEC::BATCH_SIZE;
         const rlt_replay_buffer rb = rl::components::off_policy_runner::rocm::replay(runner);
+        if constexpr(BATCH_SPEC::SEQUENCE_LENGTHH > 1){
+            // gather_batch's multi-step branch (off_policy_runner/operations_generic.h:239-430): the per-sample draws are made on the device first
+            static_assert(!DETERMINISTIC, "deterministic sequence batches are not available on devices::ROCM");
+            using BP = typename BATCH_SPEC::PARAMETERS;
+            constexpr int S = BATCH_SPEC::SEQUENCE_LENGTHH, PADDED = S + 1;
+            rlt_sequence_sampling sampling = {};
+            sampling.always_sample_from_initial_state = BP::ALWAYS_SAMPLE_FROM_INITIAL_STATE; sampling.random_seq_length = BP::RANDOM_SEQ_LENGTH;
+            sampling.enable_nominal_sequence_length_probability = BP::ENABLE_NOMINAL_SEQUENCE_LENGTH_PROBABILITY;
+            sampling.nominal_sequence_length_probability = (float)BP::NOMINAL_SEQUENCE_LENGTH_PROBABILITY;
+            sampling.include_first_step_in_targets = BP::INCLUDE_FIRST_STEP_IN_TARGETS;
+            auto align = [](size_t bytes){ return (bytes + 255) / 256 * 256; };
+            const size_t env_bytes = align(sizeof(uint32_t) * BATCH_SIZE), offset_bytes = align(sizeof(uint32_t) * BATCH_SIZE * PADDED), nominal_bytes = align((size_t)BATCH_SIZE * (PADDED + 1));
+            const size_t length_bytes = align(sizeof(uint32_t) * BATCH_SIZE * (PADDED + 1));
+            char* memory = (char*)devices::rocm::scratch(device, env_bytes + offset_bytes + nominal_bytes + length_bytes);
+            uint32_t* env_indices = (uint32_t*)memory; uint32_t* offsets = (uint32_t*)(memory + env_bytes);
+            uint8_t* nominal = (uint8_t*)(memory + env_bytes + offset_bytes); uint32_t* lengths = (uint32_t*)(memory + env_bytes + offset_bytes + nominal_bytes);
+            devices::rocm::check(rlt_rocm_gather_sequence_draw(device.handle, &rb, &sampling, SPEC::MAX_EPISODE_LENGTH, BATCH_SIZE, S, rng.seed, random::next_stream(rng), env_indices, offsets,
+                                                               nominal, lengths), "gather_batch (draw)");
+            const rlt_sequence_draws draws = {env_indices, offsets, nominal, lengths};
+            rlt_sequence_batch b = {};
+            b.observations_actions_base = batch.observations_actions_base._data; b.rewards = batch.rewards._data; b.terminated = (uint8_t*)batch.terminated._data;
+            b.reset = (uint8_t*)batch.reset._data; b.next_reset_base = (uint8_t*)batch.next_reset_base._data; b.final_step_mask = (uint8_t*)batch.final_step_mask._data;
+            b.next_final_step_mask_base = (uint8_t*)batch.next_final_step_mask_base._data; b.batch = BATCH_SIZE; b.sequence_length = S;
+            devices::rocm::check(rlt_rocm_gather_sequence_batch(device.handle, &rb, &sampling, &draws, SPEC::MAX_EPISODE_LENGTH, &b), "gather_batch (sequences)");
+            return;
+        }
         uint32_t* env_indices = nullptr; uint32_t* offsets = nullptr;
         if constexpr(!DETERMINISTIC){
             env_indices = (uint32_t*)devices::rocm::scratch(device, 2 * sizeof(uint32_t) * BATCH_SIZE);

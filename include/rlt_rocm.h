@@ -444,6 +444,16 @@ int rlt_rocm_gather_sequence_batch(rlt_rocm_device* device, const rlt_replay_buf
 int rlt_rocm_gather_draw(rlt_rocm_device* device, const rlt_replay_buffer* rb, int batch,
                          uint64_t seed, uint64_t stream, uint32_t* env_indices, uint32_t* sample_offsets);
 
+/* Device-side draws for rlt_rocm_gather_sequence_batch: fills the four arrays of rlt_sequence_draws (sizes as documented there) with what
+ * gather_batch draws per sample (off_policy_runner/operations_generic.h:257-275,304,362-371,426): the environment; an offset uniform over the
+ * eligible rows of that environment's ring for each of the `padded` possible (re)starts (capacity - max_episode_length rows of a full ring when
+ * sequences start at episode starts); for each of the padded + 1 possible length decisions whether the nominal length is taken
+ * (uniform_real < nominal_sequence_length_probability) and a length uniform in [1, sequence_length - 1]. Sample b takes the words of Philox
+ * groups [b G, (b + 1) G), G = ceil((3 padded + 3) / 4), of the sequence that (seed, stream) selects, in that order. */
+int rlt_rocm_gather_sequence_draw(rlt_rocm_device* device, const rlt_replay_buffer* rb, const rlt_sequence_sampling* sampling,
+                                  int max_episode_length, int batch, int sequence_length, uint64_t seed, uint64_t stream,
+                                  uint32_t* env_indices, uint32_t* sample_offsets, uint8_t* nominal, uint32_t* lengths);
+
 /* rl/environments/pendulum/pendulum.h:12-25 */
 typedef struct rlt_pendulum_parameters {
     float g, max_speed, max_torque, dt, m, l;

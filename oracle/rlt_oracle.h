@@ -41,7 +41,7 @@
  *   equals the sequence forward pass.
  *   td3_sequence_*: every parameter and Adam age bit for bit against the reference's TD3 loop with its recurrent approximators over 300 loop steps at two
  *   depths (oracle/_ref/librlt_ref_td3_gru{4,5}_generic.so), target values and d_output too.
- *   philox4x32_10, rand_bits / rand / randn / gather_draw / pendulum_initial_states (rlt_oracle_rng.cpp): the block function against the three
+ *   philox4x32_10, rand_bits / rand / randn / gather_draw / gather_sequence_draw / pendulum_initial_states (rlt_oracle_rng.cpp): the block function against the three
  *   published known-answer vectors of Philox4x32-10; the conversions by range, moments and Kolmogorov-Smirnov distance; no reference counterpart
  *   fixes the sequence itself (the reference's CUDA and CPU generators differ from each other).
  *   reduce_sum_f32, adam_reset: against numpy closed forms (tests/test_oracle_rng.py, tests/test_oracle_closed_forms.py).
@@ -119,6 +119,8 @@ int rlt_oracle_rand_bits_u32(uint32_t* dst, size_t count, uint64_t seed, uint64_
 int rlt_oracle_rand_f32(float* dst, size_t count, float low, float high, uint64_t seed, uint64_t stream);
 int rlt_oracle_randn_f32(float* dst, size_t count, uint64_t seed, uint64_t stream);
 int rlt_oracle_gather_draw(const rlt_replay_buffer* rb, int batch, uint64_t seed, uint64_t stream, uint32_t* env_indices, uint32_t* sample_offsets);
+int rlt_oracle_gather_sequence_draw(const rlt_replay_buffer* rb, const rlt_sequence_sampling* sampling, int max_episode_length, int batch, int sequence_length, uint64_t seed,
+                                    uint64_t stream, uint32_t* env_indices, uint32_t* sample_offsets, uint8_t* nominal, uint32_t* lengths);
 int rlt_oracle_pendulum_initial_states(float* states, int n_envs, uint64_t seed, uint64_t stream);
 
 int rlt_oracle_sac_train_critic(const rlt_sac_agent* agent, int critic_index, const float* action_noise);

@@ -11,6 +11,7 @@
 // philox4x32-10 (tests/test_oracle_rng.py); the float conversions against closed forms (range, cell midpoints,
 // moments, Kolmogorov-Smirnov distance to the uniform and normal distributions); that streams and seeds select
 // different sequences by the absence of any repeated group among a million (seed, stream, index) triples.
+#include <vector>
 #include "rlt_oracle.h"
 #include <cmath>
 #include <cstdint>
@@ -92,6 +93,27 @@ int rlt_oracle_gather_draw(const rlt_replay_buffer* rb, int batch, uint64_t seed
         const uint32_t eligible = rb->full[env] ? (uint32_t)rb->capacity : rb->position[env];
         env_indices[i] = env;
         sample_offsets[i] = eligible ? (uint32_t)(((uint64_t)g[1] * eligible) >> 32) : 0u;
+    }
+    return 0;
+}
+
+// the draws of a sequence batch (off_policy_runner/operations_generic.h:257-275,304,362-371,426), in the word order documented at
+// rlt_rocm_gather_sequence_draw: environment, padded offsets, padded + 1 nominal decisions, padded + 1 lengths
+int rlt_oracle_gather_sequence_draw(const rlt_replay_buffer* rb, const rlt_sequence_sampling* sampling, int max_episode_length, int batch, int sequence_length, uint64_t seed,
+                                    uint64_t stream, uint32_t* env_indices, uint32_t* sample_offsets, uint8_t* nominal, uint32_t* lengths) {
+    if (!rb || !sampling || !env_indices || !sample_offsets || !nominal || !lengths || batch <= 0 || sequence_length < 1) return RLT_E_INVALID_ARGUMENT;
+    const int padded = sequence_length + 1, n_words = 3 * padded + 3, groups = (n_words + 3) / 4;
+    std::vector<uint32_t> words((size_t)groups * 4);
+    for (int b = 0; b < batch; b++) {
+        for (int g = 0; g < groups; g++) group(seed, stream, (uint64_t)b * groups + g, &words[4 * (size_t)g]);
+        const uint32_t env = (uint32_t)(((uint64_t)words[0] * (uint32_t)rb->n_envs) >> 32);
+        env_indices[b] = env;
+        const uint32_t eligible = rb->full[env] ? (uint32_t)(sampling->always_sample_from_initial_state ? rb->capacity - max_episode_length : rb->capacity) : rb->position[env];
+        for (int k = 0; k < padded; k++) sample_offsets[(size_t)b * padded + k] = eligible ? (uint32_t)(((uint64_t)words[1 + k] * eligible) >> 32) : 0u;
+        for (int k = 0; k <= padded; k++) {
+            nominal[(size_t)b * (padded + 1) + k] = unit(words[1 + padded + k]) < sampling->nominal_sequence_length_probability ? 1 : 0;
+            lengths[(size_t)b * (padded + 1) + k] = sequence_length > 1 ? 1u + (uint32_t)(((uint64_t)words[2 + 2 * padded + k] * (uint32_t)(sequence_length - 1)) >> 32) : 1u;
+        }
     }
     return 0;
 }

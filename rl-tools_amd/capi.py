@@ -284,6 +284,7 @@ PROTOTYPES = {
     "gather_batch": [C.POINTER(ReplayBuffer), P, P, I, I, I, P, P, P, P, P, P, P],
     "pendulum_step": [C.POINTER(PendulumParameters), P, P, P, P, P, I],
     "gather_sequence_batch": [C.POINTER(ReplayBuffer), C.POINTER(SequenceSampling), C.POINTER(SequenceDraws), I, C.POINTER(SequenceBatch)],
+    "gather_sequence_draw": [C.POINTER(ReplayBuffer), C.POINTER(SequenceSampling), I, I, I, U64, U64, P, P, P, P],
     "acrobot_step": [C.POINTER(AcrobotParameters), I, P, P, P, P, P, P, I],
     "car_step": [C.POINTER(CarParameters), P, P, P, P, P, P, I],
     "env_runner_step": [C.POINTER(EnvRunner), C.POINTER(ReplayBuffer), I, LP, I, C.POINTER(SasParameters), P, P, P, P, S],

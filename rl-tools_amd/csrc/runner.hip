@@ -183,6 +183,32 @@ __global__ __launch_bounds__(256) void gather_draw_kernel(rlt_replay_buffer rb, 
     }
 }
 
+// The draws of a sequence batch (the arrays of rlt_sequence_draws), on the device: sample b takes the words of groups [b G, (b + 1) G) of the call's
+// stream, G = ceil((3 padded + 3) / 4), in the order environment, padded offsets, padded + 1 nominal decisions, padded + 1 lengths.
+__global__ __launch_bounds__(256) void gather_sequence_draw_kernel(rlt_replay_buffer rb, rlt_sequence_sampling P, int max_episode_length, int batch, int sequence_length, uint64_t seed,
+                                                                   uint64_t stream, uint32_t* __restrict__ env_indices, uint32_t* __restrict__ sample_offsets,
+                                                                   uint8_t* __restrict__ nominal, uint32_t* __restrict__ lengths) {
+    const int PADDED = sequence_length + 1, WORDS = 3 * PADDED + 3, G = (WORDS + 3) / 4;
+    for (int b = blockIdx.x * blockDim.x + threadIdx.x; b < batch; b += gridDim.x * blockDim.x) {
+        uint32_t env = 0, eligible = 0;
+        for (int g = 0; g < G; g++) {
+            const rlt_u32x4 draw = rlt_philox(seed, stream, (uint64_t)b * G + g);
+            const uint32_t words[4] = {draw.x, draw.y, draw.z, draw.w};
+            for (int i = 0; i < 4; i++) {
+                const int w = 4 * g + i;
+                if (w >= WORDS) break;
+                if (w == 0) {
+                    env = rlt_uniform_below(words[i], (uint32_t)rb.n_envs);
+                    env_indices[b] = env;
+                    eligible = rb.full[env] ? (uint32_t)(P.always_sample_from_initial_state ? rb.capacity - max_episode_length : rb.capacity) : rb.position[env];
+                } else if (w <= PADDED) sample_offsets[(size_t)b * PADDED + (w - 1)] = eligible ? rlt_uniform_below(words[i], eligible) : 0u;
+                else if (w <= 2 * PADDED + 1) nominal[(size_t)b * (PADDED + 1) + (w - PADDED - 1)] = rlt_u01(words[i]) < P.nominal_sequence_length_probability ? 1 : 0;
+                else lengths[(size_t)b * (PADDED + 1) + (w - 2 * PADDED - 2)] = sequence_length > 1 ? 1u + rlt_uniform_below(words[i], (uint32_t)(sequence_length - 1)) : 1u;
+            }
+        }
+    }
+}
+
 // prologue of the runner step (operations_generic_per_env.h:8-66): reset where truncated, flag the previous replay row, observe
 __global__ __launch_bounds__(256) void runner_prologue_kernel(rlt_pendulum_runner rn, rlt_replay_buffer rb, const float* __restrict__ initial_states, uint64_t seed, uint64_t stream,
                                                               float* __restrict__ observations) {
@@ -686,6 +712,16 @@ int rlt_rocm_gather_draw(rlt_rocm_device* device, const rlt_replay_buffer* rb, i
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(rb_ok(rb) && batch > 0 && env_indices && sample_offsets);
     hipLaunchKernelGGL(gather_draw_kernel, dim3(grid1(batch)), dim3(256), 0, device->stream, *rb, batch, seed, stream, env_indices, sample_offsets);
+    return rlt_launch_status(device);
+}
+
+int rlt_rocm_gather_sequence_draw(rlt_rocm_device* device, const rlt_replay_buffer* rb, const rlt_sequence_sampling* sampling, int max_episode_length, int batch, int sequence_length,
+                                  uint64_t seed, uint64_t stream, uint32_t* env_indices, uint32_t* sample_offsets, uint8_t* nominal, uint32_t* lengths) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(rb_ok(rb) && sampling && batch > 0 && sequence_length >= 1 && max_episode_length >= 0 && env_indices && sample_offsets && nominal && lengths);
+    RLT_REQUIRE(!sampling->always_sample_from_initial_state || rb->capacity > max_episode_length);
+    hipLaunchKernelGGL(gather_sequence_draw_kernel, dim3(grid1(batch)), dim3(256), 0, device->stream, *rb, *sampling, max_episode_length, batch, sequence_length, seed, stream,
+                       env_indices, sample_offsets, nominal, lengths);
     return rlt_launch_status(device);
 }
 

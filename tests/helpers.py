@@ -64,6 +64,7 @@ def load_oracle():
     lib.rlt_oracle_rand_f32.argtypes = [P, S, F, F, U64, U64]
     lib.rlt_oracle_randn_f32.argtypes = [P, S, U64, U64]
     lib.rlt_oracle_gather_draw.argtypes = [C.POINTER(capi.ReplayBuffer), I, U64, U64, P, P]
+    lib.rlt_oracle_gather_sequence_draw.argtypes = [C.POINTER(capi.ReplayBuffer), C.POINTER(capi.SequenceSampling), I, I, I, U64, U64, P, P, P, P]
     lib.rlt_oracle_pendulum_initial_states.argtypes = [P, I, U64, U64]
     lib.rlt_oracle_reduce_sum_f32.argtypes = [P, S, I, P]
     lib.rlt_oracle_use_cblas.argtypes = [C.c_char_p]

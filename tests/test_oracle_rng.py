@@ -171,3 +171,35 @@ def test_reduce_sum_and_adam_reset(lib):
     gd = g.astype(np.float64)
     expected = p0 - 1e-3 * gd / (np.abs(gd) + 1e-7)
     assert np.allclose(p, expected, rtol=0, atol=2e-7)
+
+
+def test_gather_sequence_draw_follows_the_documented_words(lib):
+    """Every array against the raw words of the sample's groups (the documented order: environment, padded offsets, padded + 1 nominal
+    decisions, padded + 1 lengths), ranges, and uniformity of lengths and nominal share."""
+    capi = helpers.capi
+    n_envs, capacity, batch, S, limit = 4, 2000, 50_000, 7, 200
+    padded, words, groups = S + 1, 3 * (S + 1) + 3, (3 * (S + 1) + 3 + 3) // 4
+    position = np.array([10, 1999, 0, 700], np.uint32)
+    full = np.array([0, 0, 1, 1], np.uint8)
+    rb = capi.ReplayBuffer()
+    rb.position, rb.full, rb.n_envs, rb.capacity = position.ctypes.data, full.ctypes.data, n_envs, capacity
+    for from_initial in (0, 1):
+        P = capi.SequenceSampling()
+        P.always_sample_from_initial_state, P.random_seq_length, P.enable_nominal_sequence_length_probability, P.nominal_sequence_length_probability = from_initial, 1, 1, 0.3
+        env, off = np.zeros(batch, np.uint32), np.zeros((batch, padded), np.uint32)
+        nominal, lengths = np.zeros((batch, padded + 1), np.uint8), np.zeros((batch, padded + 1), np.uint32)
+        assert lib.rlt_oracle_gather_sequence_draw(C.byref(rb), C.byref(P), limit, batch, S, 9, 123, env.ctypes.data, off.ctypes.data, nominal.ctypes.data, lengths.ctypes.data) == 0
+        w = bits(lib, 4 * groups * batch, 9, 123).reshape(batch, 4 * groups).astype(np.uint64)
+        eligible = np.where(full != 0, capacity - limit if from_initial else capacity, position).astype(np.uint64)
+        assert np.array_equal(env, (w[:, 0] * n_envs) >> 32)
+        assert np.array_equal(off, (w[:, 1:1 + padded] * eligible[env][:, None]) >> 32) and np.all(off < eligible[env][:, None])
+        unit = ((w[:, 1 + padded:2 * padded + 2] >> 8).astype(np.float64) + 0.5) * 2.0 ** -24
+        assert np.array_equal(nominal, (unit.astype(np.float32) < np.float32(0.3)).astype(np.uint8))
+        assert np.array_equal(lengths, 1 + ((w[:, 2 * padded + 2:3 * padded + 3] * (S - 1)) >> 32))
+        assert lengths.min() == 1 and lengths.max() == S - 1
+        assert stats.chisquare(np.bincount(lengths.reshape(-1))[1:]).pvalue > 1e-3
+        assert abs(nominal.mean() - 0.3) < 4 * np.sqrt(0.21 / nominal.size)
+    one = np.zeros((4, 3), np.uint32)
+    assert lib.rlt_oracle_gather_sequence_draw(C.byref(rb), C.byref(P), limit, 4, 1, 9, 1, np.zeros(4, np.uint32).ctypes.data, np.zeros((4, 2), np.uint32).ctypes.data,
+                                               np.zeros((4, 3), np.uint8).ctypes.data, one.ctypes.data) == 0
+    assert np.all(one == 1)       # sequence length 1 leaves no choice

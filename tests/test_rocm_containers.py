@@ -320,3 +320,31 @@ def test_set_stream_routes_work_to_the_callers_stream(rocm):
     assert lib.rlt_rocm_set_stream(h, None) == 0 and lib.rlt_rocm_get_stream(h) == own
     assert np.all(d.numpy() == 3.0)
     assert hip.hipStreamDestroy(s) == 0
+
+
+@pytest.mark.parametrize("S,from_initial", [(1, 0), (7, 0), (16, 1)])
+def test_gather_sequence_draw_matches_the_checker(oracle, rocm, S, from_initial):
+    n_envs, capacity, batch, limit = 4, 2000, 20_000, 200
+    padded = S + 1
+    position = np.array([10, 1999, 0, 700], np.uint32)
+    full = np.array([0, 0, 1, 1], np.uint8)
+    res = []
+    for b in (oracle, rocm):
+        pos, fl = b.array(position), b.array(full)
+        rb = capi.ReplayBuffer()
+        rb.data = b.zeros((n_envs * capacity * 10,)).ptr
+        rb.episode_start = b.zeros((n_envs * capacity,), np.uint32).ptr
+        rb.position, rb.full, rb.current_episode_start = pos.ptr, fl.ptr, b.zeros((n_envs,), np.uint32).ptr
+        rb.n_envs, rb.capacity, rb.observation_dim, rb.action_dim = n_envs, capacity, 3, 1
+        P = capi.SequenceSampling()
+        P.always_sample_from_initial_state, P.random_seq_length, P.enable_nominal_sequence_length_probability, P.nominal_sequence_length_probability = from_initial, 1, 1, 0.3
+        env, off = b.zeros((batch,), np.uint32), b.zeros((batch, padded), np.uint32)
+        nominal, lengths = b.zeros((batch, padded + 1), np.uint8), b.zeros((batch, padded + 1), np.uint32)
+        if b is oracle:
+            assert oracle.lib.rlt_oracle_gather_sequence_draw(C.byref(rb), C.byref(P), limit, batch, S, 5, 11, env.ptr, off.ptr, nominal.ptr, lengths.ptr) == 0
+        else:
+            b.call("gather_sequence_draw", C.byref(rb), C.byref(P), limit, batch, S, 5, 11, env.ptr, off.ptr, nominal.ptr, lengths.ptr)
+        b.sync()
+        res.append([a.numpy() for a in (env, off, nominal, lengths)])
+    for want, got in zip(*res):
+        assert np.array_equal(got, want)
