@@ -6,7 +6,8 @@
 //
 // Covered: the Pendulum with an actor that is an MLP, alone or followed by sample_and_squash (SAC: action = tanh(mean) in evaluation
 // mode) or td3_sampling (TD3: the tanh output, no noise in evaluation mode), or preceded by a standardize layer (PPO: the action is the
-// mean of mlp_unconditional_stddev, nn_models/mlp_unconditional_stddev/operations_generic.h:23-49); no per-step data collection.
+// mean of mlp_unconditional_stddev, nn_models/mlp_unconditional_stddev/operations_generic.h:23-49), or a sequential model with GRU layers (the
+// recurrent approximators of SAC and TD3: rlt_rocm_pendulum_evaluate_recurrent, about ten launches per step); no per-step data collection.
 #pragma once
 #include <rl_tools/devices/rocm.h>
 #include <rl_tools/rl/utils/evaluation/evaluation.h>
@@ -25,12 +26,23 @@ namespace rl_tools{
         static_assert(mode::is<MODE, mode::Evaluation>, "the library's evaluation runs the actor in evaluation mode (no exploration noise)");
         static_assert(P::initial_state_min_angle == -P::initial_state_max_angle && P::initial_state_min_speed == -P::initial_state_max_speed, "initial states are drawn from ranges that are symmetric about zero");
         constexpr size_t N = SPEC::N_EPISODES;
+        constexpr bool RECURRENT = rl::components::off_policy_runner::rocm::HasGru<POLICY>::value;
         rl::components::off_policy_runner::rocm::PolicyDescription d;
-        rl::components::off_policy_runner::rocm::describe(policy, d);
+        rl::components::off_policy_runner::rocm::RecurrentPolicyDescription rd;
+        size_t workspace_bytes = 0;
+        if constexpr(RECURRENT){
+            // policy_state holds N_EPISODES rows; it is reset before the first step and left as the last step left it (rl/utils/evaluation/operations_generic.h:135,163)
+            rl::components::off_policy_runner::rocm::describe_recurrent(policy, policy_state.content_state, rd);
+            utils::assert_exit(device, !rd.unsupported, "evaluate: a recurrent policy is dense and GRU layers, with or without a sample_and_squash head");
+            workspace_bytes = rlt_rocm_pendulum_evaluate_recurrent_workspace_bytes(rd.layers, rd.n_layers, (int)N);
+        }
+        else{
+            rl::components::off_policy_runner::rocm::describe(policy, d);
+        }
         const rlt_pendulum_parameters parameters = {(float)P::g, (float)P::max_speed, (float)P::max_torque, (float)P::dt, (float)P::m, (float)P::l};
         auto align = [](size_t bytes){ return (bytes + 255) / 256 * 256; };
         const size_t initial_bytes = align(N * 2 * sizeof(float)), returns_bytes = align(N * sizeof(float)), length_bytes = align(N * sizeof(uint32_t));
-        char* memory = (char*)devices::rocm::scratch(device, initial_bytes + returns_bytes + length_bytes + 256);
+        char* memory = (char*)devices::rocm::scratch(device, initial_bytes + returns_bytes + length_bytes + 256 + workspace_bytes);
         float* initial = (float*)memory; float* returns = (float*)(memory + initial_bytes); uint32_t* episode_length = (uint32_t*)(memory + initial_bytes + returns_bytes);
         float* summary = (float*)(memory + initial_bytes + returns_bytes + length_bytes);
         if constexpr(SPEC::DETERMINISTIC_INITIAL_STATE){
@@ -47,8 +59,15 @@ namespace rl_tools{
                 devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_speed, initial + 1, 2, initial + 1, 2, (int)N, 1), "evaluate (initial states)");
             }
         }
+        if constexpr(RECURRENT){
+            constexpr int AUTO_RESET_PERIOD = (int)get<0>(typename POLICY::INPUT_SHAPE{});
+            devices::rocm::check(rlt_rocm_pendulum_evaluate_recurrent(device.handle, &parameters, rd.has_head ? 2 : 1, rd.layers, rd.n_layers, &rd.state, AUTO_RESET_PERIOD, initial, (int)N,
+                                                                      (int)SPEC::STEP_LIMIT, returns, episode_length, summary, memory + initial_bytes + returns_bytes + length_bytes + 256, workspace_bytes), "evaluate (recurrent)");
+        }
+        else{
         utils::assert_exit(device, !d.standardize_misplaced, "evaluate: a standardize layer is supported in front of the first dense layer only");
         devices::rocm::check(rlt_rocm_pendulum_evaluate_standardized(device.handle, &parameters, d.has_head ? 2 : 1, d.layers, d.n_layers, d.standardize_mean, d.standardize_precision, initial, (int)N, (int)SPEC::STEP_LIMIT, returns, episode_length, summary), "evaluate");
+        }
         float host_summary[6];
         devices::rocm::check(rlt_rocm_memcpy_d2h(device.handle, results.returns, returns, N * sizeof(float)), "evaluate (results)");
         devices::rocm::check(rlt_rocm_memcpy_d2h(device.handle, results.episode_length, episode_length, N * sizeof(uint32_t)), "evaluate (results)");

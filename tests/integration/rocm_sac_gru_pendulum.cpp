@@ -2,11 +2,14 @@
 // sample_and_squash head, dense -> GRU -> dense critics) and sequence batches (SEQUENCE_LENGTH > 1: gather_batch's multi-step branch,
 // rl/components/off_policy_runner/operations_generic.h:239-430) instantiated on devices::ROCM for the Pendulum; the CPU counterpart is the zoo's
 // src/rl/zoo/pendulum-position-v1/sac.h:8-52 (same approximators, same batch sampling parameters; that configuration hides the velocity from the
-// observation, this one does not, and is smaller so that it trains in seconds). Only the device type and the ROCM includes differ from a CPU program.
+// observation, this one does not, and is smaller so that it trains in seconds), inside the reference's evaluation and timing loop steps: the
+// evaluations (50 episodes every 1,000 loop steps, the recurrent actor stepped with its kept state) run on the device too. Only the device type and
+// the ROCM includes differ from a CPU program.
 //
 // With -DSAC_GRU_DEVICE_CPU the same program runs on the reference's CPU device (generic operations, one thread): the figure the device's is read against.
 //
-// Usage: rocm_sac_gru_pendulum [n_steps [seed]] ; prints "step <n> mean_return <r>" lines and a last line "final <r> loop_steps_per_second <x>".
+// Usage: rocm_sac_gru_pendulum [n_steps [seed]] ; prints "step <n> mean_return <r>" for the evaluation made at loop step n and a last line
+// "final <r> loop_steps_per_second_including_evaluations <x>" (r: the last evaluation made).
 #include <rl_tools/operations/cpu_mux.h>
 #ifndef SAC_GRU_DEVICE_CPU
 #include <rl_tools/operations/rocm.h>
@@ -25,11 +28,17 @@
 #include <rl_tools/nn/layers/gru/operations_rocm.h>
 #include <rl_tools/rl/components/off_policy_runner/operations_rocm.h>
 #include <rl_tools/rl/algorithms/sac/operations_rocm.h>
+#include <rl_tools/rl/utils/evaluation/operations_rocm.h>
+#else
+#include <rl_tools/rl/utils/evaluation/operations_cpu.h>
 #endif
 
 #include <rl_tools/rl/algorithms/sac/loop/core/config.h>
+#include <rl_tools/rl/loop/steps/evaluation/config.h>
+#include <rl_tools/rl/loop/steps/timing/config.h>
 #include <rl_tools/rl/algorithms/sac/loop/core/operations_generic.h>
-#include <rl_tools/rl/utils/evaluation/operations_generic.h>
+#include <rl_tools/rl/loop/steps/evaluation/operations_generic.h>
+#include <rl_tools/rl/loop/steps/timing/operations_cpu.h>
 
 #include <chrono>
 #include <cstdio>
@@ -42,7 +51,6 @@ using DEVICE = rlt::devices::DEVICE_FACTORY_ROCM<>;
 #else
 using DEVICE = rlt::devices::DEVICE_FACTORY<>;
 #endif
-using DEVICE_EVALUATION = rlt::devices::DEVICE_FACTORY<>;
 using TI = typename DEVICE::index_t;
 using T = float;
 using TYPE_POLICY = rlt::numeric_types::Policy<float>;
@@ -75,54 +83,38 @@ struct LOOP_CORE_PARAMETERS: rlt::rl::algorithms::sac::loop::core::DefaultParame
     };
 };
 using LOOP_CORE_CONFIG = rlt::rl::algorithms::sac::loop::core::Config<TYPE_POLICY, TI, RNG, ENVIRONMENT, LOOP_CORE_PARAMETERS, rlt::rl::algorithms::sac::loop::core::ConfigApproximatorsGRU>;
-using LOOP_STATE = typename LOOP_CORE_CONFIG::template State<LOOP_CORE_CONFIG>;
-
-constexpr TI NUM_EVALUATION_EPISODES = 50;
+struct LOOP_EVAL_PARAMETERS: rlt::rl::loop::steps::evaluation::Parameters<TYPE_POLICY, TI, LOOP_CORE_CONFIG>{
+    static constexpr TI EVALUATION_INTERVAL = 1000;
+    static constexpr TI NUM_EVALUATION_EPISODES = 50;
+    static constexpr TI N_EVALUATIONS = LOOP_CORE_PARAMETERS::STEP_LIMIT / EVALUATION_INTERVAL;
+};
+using LOOP_EVAL_CONFIG = rlt::rl::loop::steps::evaluation::Config<LOOP_CORE_CONFIG, LOOP_EVAL_PARAMETERS>;
+using LOOP_CONFIG = rlt::rl::loop::steps::timing::Config<LOOP_EVAL_CONFIG>;
+using LOOP_STATE = typename LOOP_CONFIG::template State<LOOP_CONFIG>;
 
 int main(int argc, char** argv){
     const TI n_steps = argc > 1 ? (TI)std::atoi(argv[1]) : LOOP_CORE_PARAMETERS::STEP_LIMIT;
     const TI seed = argc > 2 ? (TI)std::atoi(argv[2]) : 0;
     DEVICE device;
-    DEVICE_EVALUATION device_evaluation;
     LOOP_STATE ts;
-    DEVICE_EVALUATION::SPEC::RANDOM::ENGINE<> rng_evaluation;
-    rlt::init(device_evaluation, rng_evaluation, seed);
-    using ACTOR_TYPE_ORIG = rlt::utils::typing::remove_reference_t<decltype(rlt::get_actor(ts))>;
-    using ACTOR_TYPE_INFERENCE = ACTOR_TYPE_ORIG::template CHANGE_CAPABILITY<rlt::nn::capability::Forward<>>;
-    using ACTOR_TYPE_EVALUATION = ACTOR_TYPE_INFERENCE::template CHANGE_BATCH_SIZE<TI, NUM_EVALUATION_EPISODES>;
-    ACTOR_TYPE_EVALUATION actor_evaluation;
-    ENVIRONMENT env_evaluation;
-    rlt::rl::environments::DummyUI ui;
     rlt::init(device);
     rlt::malloc(device, ts);
-    rlt::malloc(device_evaluation, actor_evaluation);
     rlt::init(device, ts, seed);
-
-    auto evaluate = [&](){
-        rlt::copy(device, device_evaluation, rlt::get_actor(ts), actor_evaluation);
-        using RESULT_SPEC = rlt::rl::utils::evaluation::Specification<TYPE_POLICY, TI, ENVIRONMENT, NUM_EVALUATION_EPISODES, 200>;
-        rlt::rl::utils::evaluation::Result<RESULT_SPEC> result;
-        rlt::evaluate(device_evaluation, env_evaluation, ui, actor_evaluation, result, rng_evaluation, rlt::Mode<rlt::mode::Evaluation<>>{});
-        return result.returns_mean;
-    };
-    std::printf("step 0 mean_return %f\n", (double)evaluate());
     const auto start = std::chrono::steady_clock::now();
-    double seconds = 0;
-    for(TI step = 0; step < n_steps; step++){
-        const bool finished = rlt::step(device, ts);
-        if((step + 1) % 1000 == 0 || step + 1 == n_steps || finished){
-#ifndef SAC_GRU_DEVICE_CPU
-            rlt::check_status(device);
-#endif
-            seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - start).count();
-            std::printf("step %u mean_return %f\n", (unsigned)(step + 1), (double)evaluate());
-            std::fflush(stdout);
-        }
-        if(finished){ break; }
+    while(ts.step < n_steps && !rlt::step(device, ts)){
     }
-    std::printf("final %f loop_steps_per_second_including_evaluations %f\n", (double)evaluate(), (double)ts.step / seconds);
+#ifndef SAC_GRU_DEVICE_CPU
+    rlt::check_status(device);
+#endif
+    const double seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - start).count();
+    const TI made = (ts.step + LOOP_EVAL_PARAMETERS::EVALUATION_INTERVAL - 1) / LOOP_EVAL_PARAMETERS::EVALUATION_INTERVAL;
+    double last = 0;
+    for(TI i = 0; i < made && i < LOOP_EVAL_PARAMETERS::N_EVALUATIONS; i++){
+        last = (double)rlt::get(ts.evaluation_results, 0, i).returns_mean;
+        std::printf("step %u mean_return %f\n", (unsigned)(i * LOOP_EVAL_PARAMETERS::EVALUATION_INTERVAL), last);
+    }
+    std::printf("final %f loop_steps_per_second_including_evaluations %f\n", last, (double)ts.step / seconds);
     rlt::free(device, ts);
-    rlt::free(device_evaluation, actor_evaluation);
     rlt::free(device);
     return 0;
 }
