@@ -75,6 +75,10 @@ namespace rl_tools::devices{
         index_t malloc_counter = 0;
         void* scratch = nullptr;                // grow-only device memory for the draws of gather_batch (devices::rocm::scratch)
         size_t scratch_bytes = 0;
+        // Parity runs against another device: when set, TD3's train_critic / train_actor take the N(0, 1) draws of the td3_sampling layer (which the reference
+        // samples inside the layer's forward pass, nn/layers/td3_sampling/operations_generic.h:75-128) from this device array [BATCH_SIZE x ACTION_DIM]
+        // instead of drawing them, so that both devices can be given the draws one generator made. Null (the default): drawn on the device.
+        const float* td3_sampling_noise_override = nullptr;
     };
     struct DefaultROCMSpecification{
         using MATH = devices::math::CPU;

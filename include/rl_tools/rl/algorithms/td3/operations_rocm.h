@@ -111,7 +111,8 @@ namespace rl_tools{
         d.agent.d_output_critic = training_buffers.d_output._data;
         // the exploration noise of the target actor's td3_sampling layer (evaluate in the default mode samples it, nn/layers/td3_sampling/operations_generic.h:75-128)
         float* sampling_noise = d.extra();
-        devices::rocm::check(rlt_rocm_randn_f32(device.handle, sampling_noise, BATCH_SIZE * ACTION_DIM, rng.seed, random::next_stream(rng)), "train_critic (sampling noise)");
+        if(device.td3_sampling_noise_override){ devices::rocm::check(rlt_rocm_memcpy_d2d(device.handle, sampling_noise, device.td3_sampling_noise_override, BATCH_SIZE * ACTION_DIM * sizeof(float)), "train_critic (sampling noise)"); }
+        else{ devices::rocm::check(rlt_rocm_randn_f32(device.handle, sampling_noise, BATCH_SIZE * ACTION_DIM, rng.seed, random::next_stream(rng)), "train_critic (sampling noise)"); }
         devices::rocm::check(rlt_rocm_td3_train_critic(device.handle, &d.agent, critic_index, sampling_noise), "train_critic");
     }
     // train_actor             rl/algorithms/td3/operations_generic.h:236-281
@@ -129,7 +130,8 @@ namespace rl_tools{
         d.agent.d_critic_input = training_buffers.d_critic_input._data;
         d.agent.d_actor_output = training_buffers.d_actor_output._data;
         float* sampling_noise = d.extra();
-        devices::rocm::check(rlt_rocm_randn_f32(device.handle, sampling_noise, BATCH_SIZE * ACTION_DIM, rng.seed, random::next_stream(rng)), "train_actor (sampling noise)");
+        if(device.td3_sampling_noise_override){ devices::rocm::check(rlt_rocm_memcpy_d2d(device.handle, sampling_noise, device.td3_sampling_noise_override, BATCH_SIZE * ACTION_DIM * sizeof(float)), "train_actor (sampling noise)"); }
+        else{ devices::rocm::check(rlt_rocm_randn_f32(device.handle, sampling_noise, BATCH_SIZE * ACTION_DIM, rng.seed, random::next_stream(rng)), "train_actor (sampling noise)"); }
         devices::rocm::check(rlt_rocm_td3_train_actor(device.handle, &d.agent, sampling_noise), "train_actor");
     }
     // update_critic_targets / update_actor_target   rl/algorithms/td3/operations_generic.h:317-325
