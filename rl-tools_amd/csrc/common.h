@@ -14,6 +14,8 @@ struct rlt_rocm_device {
     char name[128];
     void* scratch;               // grow-only device workspace for split reductions and partial sums
     size_t scratch_bytes;
+    void* pad_scratch;           // a second grow-only buffer: zero-padded copies of narrow networks (pad.hip)
+    size_t pad_scratch_bytes;
     void* counters;              // 8 KiB, zero between launches: [0,256) ticket counters, [256,..) per-workgroup partial sums
     unsigned* fault;             // [0]: set by a persistent kernel that gave up waiting for another workgroup; read back by check_status
     int fault_armed;             // a kernel that can set it was launched since the last check

@@ -160,6 +160,7 @@ int rlt_rocm_destroy(rlt_rocm_device* device) {
     if (!device) return RLT_E_INVALID_ARGUMENT;
     (void)hipStreamSynchronize(device->own_stream);
     if (device->scratch) (void)hipFree(device->scratch);
+    if (device->pad_scratch) (void)hipFree(device->pad_scratch);
     if (device->counters) (void)hipFree(device->counters);
     (void)hipStreamDestroy(device->own_stream);
     delete device;

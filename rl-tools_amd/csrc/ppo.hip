@@ -5,6 +5,7 @@
 #include "common.h"
 #include <cstdlib>
 #include "mlp_small.h"
+#include "pad.h"
 #include "optim.h"
 
 namespace {
@@ -320,17 +321,45 @@ extern "C" int rlt_rocm_ppo_surrogate_gradient(rlt_rocm_device* device, const fl
                               d_log_std, batch, action_dim, (float*)scratch);
 }
 
+// Which way the pair of networks takes: 1 = both are in -> 64 -> 64 -> out and share the one-launch pass; 2 = they do once their hidden width (below 64) is padded
+// to 64 with zero rows and columns (pad.h); 0 = the per-layer kernels.
+static int pair_mode(const rlt_ppo_agent* A) {
+    if (!narrow_pass_enabled()) return 0;
+    if (rlt_mlp3s_pair_supported(A->actor, A->n_actor_layers, A->critic, A->n_critic_layers)) return 1;
+    const bool pad_a = rlt_pad_eligible(A->actor, A->n_actor_layers), pad_c = rlt_pad_eligible(A->critic, A->n_critic_layers);
+    if (!pad_a && !pad_c) return 0;
+    if (A->n_actor_layers != 3 || A->n_critic_layers != 3) return 0;
+    rlt_dense_layer a[3], c[3];
+    for (int l = 0; l < 3; l++) { a[l] = A->actor[l]; c[l] = A->critic[l]; }
+    if (pad_a) { a[0].out_dim = 64; a[1].in_dim = 64; a[1].out_dim = 64; a[2].in_dim = 64; }
+    if (pad_c) { c[0].out_dim = 64; c[1].in_dim = 64; c[1].out_dim = 64; c[2].in_dim = 64; }
+    return rlt_mlp3s_pair_supported(a, 3, c, 3) ? 2 : 0;
+}
+
 // actor and critic of the supported narrow shape in one launch (stats = {advantage mean, std} of the minibatch on the device), then both Adam steps in one
 static int ppo_pair_update(rlt_rocm_device* device, const rlt_ppo_agent* A, const rlt_ppo_parameters* P, const float* observations, const float* observations_privileged,
                            const float* actions, const float* action_log_probs, const float* advantages, const float* target_values, int ld, const uint32_t* row_indices,
                            const float* stats, float* values, float* out_critic_loss) {
     const int B = A->batch, AD = A->action_dim;
-    int rc = rlt_mlp3s_ppo_actor_critic(device, A->actor, A->n_actor_layers, observations, A->actor[A->n_actor_layers - 1].output, AD, A->log_std, actions,
-                                        action_log_probs, advantages, stats, P, P->learn_action_std ? A->d_log_std : nullptr, -P->action_entropy_coefficient,
-                                        A->critic, A->n_critic_layers, observations_privileged, values, 1, target_values, 1.0f / (float)B, out_critic_loss,   // :303
-                                        ld, row_indices, B, A->actor_standardize_mean, A->actor_standardize_precision, A->critic_standardize_mean,
-                                        A->critic_standardize_precision);
+    int rc;
+    const rlt_dense_layer* actor = A->actor; const rlt_dense_layer* critic = A->critic;
+    rlt_padded_net padded_actor, padded_critic;
+    const bool pad_a = rlt_pad_eligible(A->actor, A->n_actor_layers), pad_c = rlt_pad_eligible(A->critic, A->n_critic_layers);
+    if (pad_a || pad_c) {       // the parameters change with every minibatch's Adam step: the padded copies are made anew
+        const size_t floats_a = pad_a ? rlt_pad_floats(A->actor, true) : 0, floats_c = pad_c ? rlt_pad_floats(A->critic, true) : 0;
+        void* memory = nullptr;
+        if ((rc = rlt_pad_scratch(device, (floats_a + floats_c) * sizeof(float), &memory))) return rc;
+        if (pad_a) { if ((rc = rlt_pad_parameters(device, A->actor, (float*)memory, true, &padded_actor))) return rc; actor = padded_actor.L; }
+        if (pad_c) { if ((rc = rlt_pad_parameters(device, A->critic, (float*)memory + floats_a, true, &padded_critic))) return rc; critic = padded_critic.L; }
+    }
+    rc = rlt_mlp3s_ppo_actor_critic(device, actor, A->n_actor_layers, observations, A->actor[A->n_actor_layers - 1].output, AD, A->log_std, actions,
+                                    action_log_probs, advantages, stats, P, P->learn_action_std ? A->d_log_std : nullptr, -P->action_entropy_coefficient,
+                                    critic, A->n_critic_layers, observations_privileged, values, 1, target_values, 1.0f / (float)B, out_critic_loss,   // :303
+                                    ld, row_indices, B, A->actor_standardize_mean, A->actor_standardize_precision, A->critic_standardize_mean,
+                                    A->critic_standardize_precision);
     if (rc) return rc;
+    if (pad_a) if ((rc = rlt_unpad_gradients(device, A->actor, &padded_actor))) return rc;
+    if (pad_c) if ((rc = rlt_unpad_gradients(device, A->critic, &padded_critic))) return rc;
     if (A->d_log_std && !P->learn_action_std) if ((rc = rlt_rocm_fill_f32(device, A->d_log_std, 1, AD, AD, 0.0f))) return rc;
     return rlt_adam_step_pair(device, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age,                                            // :305-306
                               A->critic_adam_tensors, A->n_critic_adam_tensors, &A->critic_adam, A->critic_age);
@@ -352,8 +381,8 @@ extern "C" int rlt_rocm_ppo_train_minibatch(rlt_rocm_device* device, const rlt_p
     char* mlp_ws = (char*)A->workspace + align256((size_t)((char*)w - (char*)A->workspace) + 64 * sizeof(float));
     const size_t mlp_ws_bytes = A->workspace_bytes - (size_t)(mlp_ws - (char*)A->workspace);
     int rc;
-    if (narrow_pass_enabled() && rlt_mlp3s_pair_supported(A->actor, A->n_actor_layers, A->critic, A->n_critic_layers)) {
-        // both networks in -> 64 -> 64 -> out: one launch runs the actor (forward, surrogate gradient, backward, :203-285) on half of the compute units
+    if (pair_mode(A)) {
+        // both networks in -> 64 -> 64 -> out (or narrower and padded to that): one launch runs the actor (forward, surrogate gradient, backward, :203-285) on half of the compute units
         // and the critic (forward, MSE gradient with loss weight 0.5 = (v - target) / batch, backward, :289-300) on the other half, reading the
         // minibatch's rows straight out of the dataset; its gradients replace the old ones, which is what zero_gradient (:158-159) followed by
         // backward leaves. The means still land in the actor's last output buffer; the hidden layers' buffers are not written.
@@ -397,7 +426,7 @@ extern "C" int rlt_rocm_ppo_train_epoch(rlt_rocm_device* device, const rlt_ppo_a
     RLT_REQUIRE(row_indices && n_minibatches >= 1 && (!P->learn_action_std || A->d_log_std));
     RLT_REQUIRE(A->workspace && A->workspace_bytes >= rlt_rocm_ppo_workspace_bytes(A));
     const int B = A->batch, O = A->observation_dim, OP = A->observation_privileged_dim, AD = A->action_dim;
-    if (!(narrow_pass_enabled() && rlt_mlp3s_pair_supported(A->actor, A->n_actor_layers, A->critic, A->n_critic_layers))) {
+    if (!pair_mode(A)) {
         for (int mb = 0; mb < n_minibatches; mb++) {
             const int rc = rlt_rocm_ppo_train_minibatch(device, A, P, observations, observations_privileged, actions, action_log_probs, advantages, target_values, ld,
                                                         row_indices + (size_t)mb * B, out_critic_losses ? out_critic_losses + mb : nullptr);

@@ -2,6 +2,7 @@
 // reference: rl/components/replay_buffer/operations_generic.h:54-78, rl/components/off_policy_runner/operations_generic.h:183-430
 //            (CUDA :14-230), operations_generic_per_env.h:8-108, rl/environments/pendulum/operations_generic.h:14-160.
 #include "common.h"
+#include "pad.h"
 #include "rng.h"
 #include <cstdlib>
 
@@ -826,6 +827,15 @@ int rlt_rocm_on_policy_collect(rlt_rocm_device* device, const rlt_pendulum_runne
     RLT_REQUIRE((standardize_mean == nullptr) == (standardize_precision == nullptr));
     RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_on_policy_collect_workspace_bytes(rn, actor, n_actor_layers));
     const int N = rn->n_envs;
+    rlt_padded_net padded;
+    if (collect_one_launch_enabled() && !fused_collect_ok(actor, n_actor_layers) && rlt_pad_eligible(actor, n_actor_layers)) {
+        // hidden widths below 64 run the one-launch kernel on zero-padded copies of the parameters (pad.h)
+        void* memory = nullptr;
+        int rc = rlt_pad_scratch(device, rlt_pad_floats(actor, false) * sizeof(float), &memory);
+        if (rc) return rc;
+        if ((rc = rlt_pad_parameters(device, actor, (float*)memory, false, &padded))) return rc;
+        if (fused_collect_ok(padded.L, 3)) actor = padded.L;
+    }
     if (fused_collect_ok(actor, n_actor_layers) && collect_one_launch_enabled()) {
         CollectArgs a = {};
         a.rn = *rn; a.D = *D;

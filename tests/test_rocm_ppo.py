@@ -91,12 +91,14 @@ def test_train_minibatch_matches_checker_on_synthetic_dataset(oracle, rocm):
     assert rel_err(p1, p0) <= 2e-4 and rel_err(l1, l0) <= 1e-4
 
 
-@pytest.mark.parametrize("O,A,H,B", [(105, 8, 64, 512), (3, 1, 64, 200), (17, 6, 256, 300)])
-def test_train_minibatch_with_standardize_layers_matches_checker(oracle, rocm, O, A, H, B):
+@pytest.mark.parametrize("O,A,H,B,act", [(105, 8, 64, 512, "tanh"), (3, 1, 64, 200, "tanh"), (17, 6, 256, 300, "tanh"), (3, 1, 32, 256, "fast_tanh"), (11, 2, 16, 128, "tanh"),
+                                         (5, 3, 48, 96, "relu")])
+def test_train_minibatch_with_standardize_layers_matches_checker(oracle, rocm, O, A, H, B, act):
     """Standardize layers in front of actor and critic (the loop's approximators, rl/algorithms/ppo/loop/core/config.h:51-83): the networks
     read (x - mean) * precision, the factor only where it is not 0 (nn/layers/standardize/operations_generic.h:68-86). Hidden width 64 takes
-    the kernel that reads the dataset rows itself, 256 the packed minibatch; four updates on shuffled rows, compared tensor by tensor after
-    the first and at the end. The third observation column has precision 0."""
+    the kernel that reads the dataset rows itself, widths below 64 the same kernel on zero-padded copies of the parameters (the zoo's PPO configuration of
+    the Pendulum is width 32 with fast_tanh), 256 the packed minibatch; four updates on shuffled rows, compared tensor by tensor after the first and at
+    the end. The third observation column has precision 0."""
     capi = helpers.capi
     N = 4 * B
     rng = np.random.default_rng(O * 7 + A)
@@ -112,7 +114,7 @@ def test_train_minibatch_with_standardize_layers_matches_checker(oracle, rocm, O
     pp = capi.ppo_parameters()
     results = []
     for b in (oracle, rocm):
-        agent = helpers.PpoOnBackend(b, O, A, H, H, B, params, "tanh", "tanh", capi.adam_parameters(3e-4, epsilon=1e-8), standardize=standardize)
+        agent = helpers.PpoOnBackend(b, O, A, H, H, B, params, act, act, capi.adam_parameters(3e-4, epsilon=1e-8), standardize=standardize)
         dd, idx, loss = b.array(data), b.array(perm), b.zeros((1,))
         args = (dd.offset(col["observations"]), dd.offset(col["observations"]), dd.offset(col["actions"]), dd.offset(col["action_log_probs"]),
                 dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld)
@@ -128,7 +130,7 @@ def test_train_minibatch_with_standardize_layers_matches_checker(oracle, rocm, O
         assert rel_err(f1[key], f0[key]) <= TOL, (key, rel_err(f1[key], f0[key]))
     assert rel_err(p1, p0) <= 2e-4 and rel_err(l1, l0) <= 1e-4
     # the layers matter: without them the first update's gradients differ
-    plain = helpers.PpoOnBackend(rocm, O, A, H, H, B, params, "tanh", "tanh", capi.adam_parameters(3e-4, epsilon=1e-8))
+    plain = helpers.PpoOnBackend(rocm, O, A, H, H, B, params, act, act, capi.adam_parameters(3e-4, epsilon=1e-8))
     dd, loss = rocm.array(data), rocm.zeros((1,))
     rocm.call("ppo_train_minibatch", C.byref(plain.c), C.byref(pp), dd.offset(0), dd.offset(0), dd.offset(col["actions"]), dd.offset(col["action_log_probs"]),
               dd.offset(col["advantages"]), dd.offset(col["target_values"]), ld, None, loss.ptr)
