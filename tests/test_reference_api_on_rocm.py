@@ -24,7 +24,7 @@ def test_programs_written_against_the_reference_api_compile_and_link():
     subprocess.run(["make", "-C", HERE, "syntax"], check=True, capture_output=True)
     out = subprocess.run(["make", "-B", "-C", HERE, "all"], capture_output=True, text=True)
     assert out.returncode == 0, out.stderr[-3000:]
-    for name in ("rocm_containers", "rocm_gru", "rocm_sac_gru_pendulum", "rocm_sac_updates", "rocm_sac_gru_updates", "rocm_td3_updates", "rocm_ppo_updates", "rocm_zoo_pendulum_v1_sac", "rocm_zoo_pendulum_v1_td3", "rocm_zoo_pendulum_v1_ppo", "rocm_sac_pendulum", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
+    for name in ("rocm_containers", "rocm_gru", "rocm_td3_sampling", "rocm_sac_gru_pendulum", "rocm_sac_updates", "rocm_sac_gru_updates", "rocm_td3_updates", "rocm_ppo_updates", "rocm_zoo_pendulum_v1_sac", "rocm_zoo_pendulum_v1_td3", "rocm_zoo_pendulum_v1_ppo", "rocm_sac_pendulum", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
         path = os.path.join(BUILD, name)
         assert os.path.exists(path)
         needed = subprocess.run(["readelf", "-d", path], capture_output=True, text=True).stdout
@@ -212,5 +212,18 @@ def test_td3_and_ppo_updates_match_the_references_cpu_device(program):
         pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
     out = subprocess.run([path], capture_output=True, text=True, timeout=170)
     print(out.stdout[-2500:], flush=True)
+    assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
+    assert float(re.search(r"worst ([\d.e+-]+)", out.stdout).group(1)) <= 1e-5
+
+
+@pytest.mark.gpu
+def test_td3_sampling_layer_program_runs():
+    """A dense -> td3_sampling model of the reference on devices::ROCM next to its CPU device: forward and backward_full with the same external noise (a third of
+    the samples clipped), evaluate in Evaluation mode, and the Default mode against clamp(mean + std * noise) for the noise the device drew. Bound 1e-5; measured 7e-8."""
+    path = os.path.join(BUILD, "rocm_td3_sampling")
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    out = subprocess.run([path], capture_output=True, text=True, timeout=120)
+    print(out.stdout[-1500:], flush=True)
     assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
     assert float(re.search(r"worst ([\d.e+-]+)", out.stdout).group(1)) <= 1e-5
