@@ -463,13 +463,15 @@ int rlt_gemm_backward_input(rlt_rocm_device* device, const float* d_pre, int ldd
 }
 
 // How the weight-gradient contraction splits the batch so that the grid fills the chip: about 2 workgroups per compute unit, at least
-// 256 rows per split. Each split writes one block of out_dim * in_dim + out_dim partial sums.
+// 256 rows per split (64 for small gradients). Each split writes one block of out_dim * in_dim + out_dim partial sums.
 static void wgrad_split(const rlt_rocm_device* device, int batch, int in_dim, int out_dim, int& splits, int& kps) {
     int bm, bn;
     tile_dims(pick_tile(out_dim, in_dim, 2), bm, bn);
     int tiles = rlt_div_up(out_dim, bm) * rlt_div_up(in_dim, bn);
     splits = (2 * device->compute_units + tiles - 1) / tiles;
-    int max_splits = rlt_div_up(batch, 256);
+    // at least 256 rows per split; for small gradients (up to 96 x 64: the layers of width 16 and 32) 64 rows, i.e. 4 k-steps: a short batch is bound by the chain
+    // of k-steps in one workgroup, and such partial sums cost little
+    int max_splits = rlt_div_up(batch, (long long)in_dim * out_dim <= 96 * 64 ? 64 : 256);
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
     kps = rlt_div_up(rlt_div_up(batch, splits), BK) * BK;

@@ -182,7 +182,7 @@ def test_recurrent_sac_loop_trains_on_rocm():
     and sequence batches of 16 steps x 32 samples from four environments, on devices::ROCM: gather_batch's multi-step branch with its draws made on the
     device, the runner step with the policy state reset by the truncation mask and evaluate_step, train_critic / train_actor as the reference's generic
     code over the GRU, dense, sample_and_squash and tensor overloads, the evaluation loop step with the recurrent actor on the device. A random actor's mean
-    return is about -1,300; measured -280 after 3,000 loop steps and -150 after 9,000, at 900 loop steps/s including the evaluations (the same program on
+    return is about -1,300; measured -280 after 3,000 loop steps and -150 after 9,000, at 1,030 loop steps/s including the evaluations (the same program on
     the reference's CPU device: 190)."""
     path = os.path.join(BUILD, "rocm_sac_gru_pendulum")
     if not os.path.exists(path):
