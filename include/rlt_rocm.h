@@ -1070,6 +1070,20 @@ int rlt_rocm_env_on_policy_collect(rlt_rocm_device* device, const rlt_env_runner
                                    const float* action_noise, const float* initial_states, int truncate_on_each_iteration,
                                    void* workspace, size_t workspace_bytes);
 
+/* rl::utils::evaluation::evaluate  rl/utils/evaluation/operations_generic.h:113-233 for any of the batched environments and any sequential
+ * policy (dense and GRU layers): n_episodes episodes of at most step_limit steps from initial_states [n_episodes x state_dim]. Of `env` the
+ * env_kind and the parameters it names are read. reset(policy, policy_state) before the first step (:135; policy_state may be NULL for a
+ * policy of dense layers), then per step observe, the optional standardize layer (observation_mean / observation_precision [observation_dim],
+ * both NULL: none), evaluate_step in Evaluation mode, the head (policy_kind 1: the output [action_dim] is the action; 2: the output is
+ * [mean | log_std] and the action is tanh(mean)), the environment's step, reward and terminated. An episode counts rewards and steps up to and
+ * including the step that terminates it (:187-197). Outputs as rlt_rocm_pendulum_evaluate: returns [n_episodes], episode_length [n_episodes],
+ * summary [6] = {returns_mean, returns_std, episode_length_mean, episode_length_std, num_terminated, share_terminated}. */
+size_t rlt_rocm_env_evaluate_workspace_bytes(int env_kind, const rlt_seq_layer* policy, int n_policy_layers, int n_episodes);
+int rlt_rocm_env_evaluate(rlt_rocm_device* device, const rlt_env_runner* env, int policy_kind, const rlt_seq_layer* policy, int n_policy_layers,
+                          const rlt_seq_state* policy_state, int auto_reset_period, const float* observation_mean, const float* observation_precision,
+                          const float* initial_states, int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary,
+                          void* workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

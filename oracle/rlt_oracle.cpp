@@ -1340,6 +1340,53 @@ int rlt_oracle_pendulum_evaluate_recurrent(const rlt_pendulum_parameters* env, i
                                   initial_states, n_episodes, step_limit, returns, episode_length, summary);
 }
 
+// rl::utils::evaluation::evaluate over any of the environments restated here (rl/utils/evaluation/operations_generic.h:113-233): the loop of
+// pendulum_evaluate_impl with the environment's own step / reward / terminated (pinned one by one above) and the terminated bookkeeping that the Pendulum
+// never reaches: an episode that has terminated is skipped from then on, its state stays (:166-170), the step that terminates it still counts (:187-192).
+int rlt_oracle_env_evaluate(const rlt_env_runner* env, int policy_kind, const rlt_seq_layer* policy, int n_layers, const rlt_seq_state* state, int auto_reset_period,
+                            const float* observation_mean, const float* observation_precision, const float* initial_states, int n_episodes, int step_limit, float* returns,
+                            uint32_t* episode_length, float* summary) {
+    int SD, OBS, ACT;
+    if (!env || !policy || n_layers < 1 || !initial_states || n_episodes < 1 || step_limit < 1 || !returns || !episode_length || !summary) return RLT_E_INVALID_ARGUMENT;
+    if ((policy_kind != 1 && policy_kind != 2) || env_dims_of(env->env_kind, &SD, &OBS, &ACT) || (observation_mean == nullptr) != (observation_precision == nullptr))
+        return RLT_E_INVALID_ARGUMENT;
+    const int N = n_episodes, out_dim = policy_kind * ACT;
+    int rc;
+    const rlt_seq_state no_state = {};
+    if (state && (rc = rlt_oracle_seq_reset_state(policy, n_layers, state, nullptr, N))) return rc;
+    std::vector<float> states(initial_states, initial_states + (size_t)N * SD), obs((size_t)N * OBS), out((size_t)N * out_dim), action(ACT);
+    std::vector<uint8_t> terminated(N, 0);
+    uint32_t num_terminated = 0;
+    rlt_env_runner all = *env; all.n_envs = N;
+    rlt_env_runner one = *env; one.n_envs = 1;
+    for (int e = 0; e < N; e++) { returns[e] = 0; episode_length[e] = 0; }
+    for (int step = 0; step < step_limit; step++) {
+        {   // observe: the environment's own step function on a copy of the states yields the observation of the state it was given
+            std::vector<float> scratch_states(states), zero_actions((size_t)N * ACT, 0.0f);
+            if ((rc = env_step_of(&all, scratch_states.data(), zero_actions.data(), obs.data(), nullptr, nullptr, nullptr))) return rc;
+        }
+        if (observation_mean)
+            for (int e = 0; e < N; e++)
+                for (int i = 0; i < OBS; i++) obs[(size_t)e * OBS + i] = (obs[(size_t)e * OBS + i] - observation_mean[i]) * observation_precision[i];
+        if ((rc = rlt_oracle_seq_evaluate_step(policy, n_layers, obs.data(), OBS, state ? state : &no_state, auto_reset_period, out.data(), out_dim, N))) return rc;
+        for (int e = 0; e < N; e++) {
+            if (step > 0 && terminated[e]) continue;
+            for (int a = 0; a < ACT; a++) action[a] = policy_kind == 1 ? out[(size_t)e * out_dim + a] : std::tanh(out[(size_t)e * out_dim + a]);
+            float r; uint8_t t;
+            if ((rc = env_step_of(&one, &states[(size_t)e * SD], action.data(), nullptr, nullptr, &r, &t))) return rc;
+            if (!terminated[e]) { returns[e] += r; episode_length[e] += 1; num_terminated += t ? 1 : 0; }
+            terminated[e] = t || terminated[e];
+        }
+    }
+    float rm = 0, rs = 0, lm = 0, ls = 0;
+    for (int e = 0; e < N; e++) { rm += returns[e]; rs += returns[e] * returns[e]; lm += (float)episode_length[e]; ls += (float)(episode_length[e] * episode_length[e]); }
+    rm /= N; lm /= N;
+    summary[0] = rm; summary[1] = std::sqrt(std::max(0.0f, rs / N - rm * rm));
+    summary[2] = lm; summary[3] = std::sqrt(std::max(0.0f, ls / N - lm * lm));
+    summary[4] = (float)num_terminated; summary[5] = num_terminated / (float)N;
+    return 0;
+}
+
 // rl/algorithms/ppo/operations_generic.h:60-95
 int rlt_oracle_ppo_gae(const float* rewards, const float* terminated, const float* truncated, const float* all_values,
                        float* advantages, float* target_values, int ld, int n_envs, int steps, float gamma, float lambda,

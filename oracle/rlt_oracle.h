@@ -178,6 +178,9 @@ int rlt_oracle_env_on_policy_collect(const rlt_env_runner* runner, const rlt_on_
 int rlt_oracle_env_runner_step_sequential(const rlt_env_runner* runner, const rlt_replay_buffer* rb, const rlt_seq_layer* policy, int n_policy_layers,
                                           const rlt_seq_state* policy_state, int auto_reset_period, int head_kind, const rlt_sas_parameters* sas, float exploration_noise_std,
                                           const float* action_noise, const float* initial_states);
+int rlt_oracle_env_evaluate(const rlt_env_runner* env, int policy_kind, const rlt_seq_layer* policy, int n_policy_layers, const rlt_seq_state* policy_state, int auto_reset_period,
+                            const float* observation_mean, const float* observation_precision, const float* initial_states, int n_episodes, int step_limit, float* returns,
+                            uint32_t* episode_length, float* summary);
 int rlt_oracle_unary_f32(int operation, float parameter, const float* src, int ld_src, float* dst, int ld_dst, int rows, int cols);
 int rlt_oracle_binary_f32(int operation, const float* a, int lda, const float* b, int ldb, float* dst, int ld_dst, int rows, int cols);
 int rlt_oracle_multiply_accumulate_f32(const float* a, int lda, const float* b, int ldb, const float* accumulator, int ldc, float* dst, int ld_dst, int rows, int cols);

@@ -290,6 +290,7 @@ PROTOTYPES = {
     "env_runner_step": [C.POINTER(EnvRunner), C.POINTER(ReplayBuffer), I, LP, I, C.POINTER(SasParameters), P, P, P, P, S],
     "env_runner_step_sequential": [C.POINTER(EnvRunner), C.POINTER(ReplayBuffer), C.POINTER(SeqLayer), I, C.POINTER(SeqState), I, I, C.POINTER(SasParameters), F, P, P, P, S],
     "env_on_policy_collect": [C.POINTER(EnvRunner), C.POINTER(OnPolicyDataset), C.POINTER(SeqLayer), I, C.POINTER(SeqState), I, P, P, P, P, P, I, P, S],
+    "env_evaluate": [C.POINTER(EnvRunner), I, C.POINTER(SeqLayer), I, C.POINTER(SeqState), I, P, P, P, I, I, P, P, P, P, S],
     "car_track_step": [C.POINTER(CarParameters), P, I, I, F, P, P, P, P, P, P, I],
     "pendulum_evaluate": [C.POINTER(PendulumParameters), I, LP, I, P, I, I, P, P, P],
     "pendulum_evaluate_standardized": [C.POINTER(PendulumParameters), I, LP, I, P, P, P, I, I, P, P, P],
@@ -344,6 +345,7 @@ ROCM_ONLY = {
     "env_dims": ([I, C.POINTER(I), C.POINTER(I), C.POINTER(I)], I),
     "env_runner_step_workspace_bytes": ([C.POINTER(EnvRunner), I, LP, I], S),
     "env_runner_step_sequential_workspace_bytes": ([C.POINTER(EnvRunner), C.POINTER(SeqLayer), I], S),
+    "env_evaluate_workspace_bytes": ([I, C.POINTER(SeqLayer), I, I], S),
     "env_on_policy_collect_workspace_bytes": ([C.POINTER(EnvRunner), C.POINTER(SeqLayer), I], S),
     "mlp_workspace_bytes": ([LP, I, I], S),
     "ppo_workspace_bytes": ([C.POINTER(PpoAgent)], S),

@@ -475,3 +475,118 @@ extern "C" int rlt_rocm_env_runner_step_sequential(rlt_rocm_device* device, cons
     hipLaunchKernelGGL(env_epilogue_kernel, dim3(blocks), dim3(256), 0, device->stream, *rn, *rb);
     return rlt_launch_status(device);
 }
+
+// ---- rl::utils::evaluation::evaluate over any of these environments (rl/utils/evaluation/operations_generic.h:113-233)
+namespace {
+__global__ __launch_bounds__(256) void env_evaluate_observe_kernel(int kind, const float* __restrict__ states, float* __restrict__ obs, int n) {
+    const EnvDims d = env_dims(kind);
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) observe_any(kind, states + (size_t)e * d.state, obs + (size_t)e * d.obs);
+}
+// the standardize layer in front of a policy (nn/layers/standardize/operations_generic.h:69-135)
+__global__ __launch_bounds__(256) void env_evaluate_standardize_kernel(const float* __restrict__ raw, float* __restrict__ obs, const float* __restrict__ mean,
+                                                                       const float* __restrict__ precision, int n, int dim) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n * dim; i += gridDim.x * blockDim.x) obs[i] = (raw[i] - mean[i % dim]) * precision[i % dim];
+}
+// sample_and_squash in Evaluation mode (nn/layers/sample_and_squash/operations_generic.h:149-195 with zero noise): action = tanh(mean)
+__global__ __launch_bounds__(256) void env_evaluate_squash_kernel(const float* __restrict__ out, float* __restrict__ actions, int n, int act) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n * act; i += gridDim.x * blockDim.x) actions[i] = tanhf(out[(size_t)(i / act) * 2 * act + i % act]);
+}
+// :187-197: an episode counts its steps and rewards up to and including the step that terminates it
+__global__ __launch_bounds__(256) void env_evaluate_accumulate_kernel(const float* __restrict__ rewards, const uint8_t* __restrict__ terminated, uint8_t* __restrict__ done,
+                                                                      float* __restrict__ returns, uint32_t* __restrict__ episode_length, int n) {
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
+        if (done[e]) continue;
+        returns[e] += rewards[e]; episode_length[e] += 1;
+        if (terminated[e]) done[e] = 1;
+    }
+}
+// :213-228, sums in episode order as the reference makes them
+__global__ void env_evaluate_summary_kernel(const float* __restrict__ returns, const uint32_t* __restrict__ episode_length, const uint8_t* __restrict__ done, int n,
+                                            float* __restrict__ summary) {
+    if (blockIdx.x != 0 || threadIdx.x != 0) return;
+    float rm = 0.f, rs = 0.f, lm = 0.f, ls = 0.f;
+    uint32_t num_terminated = 0;
+    for (int e = 0; e < n; e++) {
+        rm += returns[e]; rs += returns[e] * returns[e]; lm += (float)episode_length[e]; ls += (float)(episode_length[e] * episode_length[e]);
+        num_terminated += done[e] ? 1 : 0;
+    }
+    rm /= (float)n; lm /= (float)n;
+    summary[0] = rm; summary[1] = sqrtf(fmaxf(0.f, rs / (float)n - rm * rm));
+    summary[2] = lm; summary[3] = sqrtf(fmaxf(0.f, ls / (float)n - lm * lm));
+    summary[4] = (float)num_terminated; summary[5] = (float)num_terminated / (float)n;
+}
+struct EvaluateLayout { size_t states, raw, obs, out, actions, rewards, terminated, done, step_ws, total; };
+EvaluateLayout evaluate_layout(const EnvDims& d, const rlt_seq_layer* policy, int n_layers, int N) {
+    EvaluateLayout L;
+    size_t at = 0;
+    auto take = [&](size_t bytes) { const size_t here = at; at += align256(bytes); return here; };
+    L.states = take((size_t)N * d.state * sizeof(float)); L.raw = take((size_t)N * d.obs * sizeof(float)); L.obs = take((size_t)N * d.obs * sizeof(float));
+    L.out = take((size_t)N * 2 * d.act * sizeof(float)); L.actions = take((size_t)N * d.act * sizeof(float)); L.rewards = take((size_t)N * sizeof(float));
+    L.terminated = take((size_t)N); L.done = take((size_t)N);
+    L.step_ws = at; L.total = at + rlt_rocm_seq_evaluate_step_workspace_bytes(policy, n_layers, N) + 512;
+    return L;
+}
+}  // namespace
+
+extern "C" size_t rlt_rocm_env_evaluate_workspace_bytes(int env_kind, const rlt_seq_layer* policy, int n_policy_layers, int n_episodes) {
+    const EnvDims d = env_dims(env_kind);
+    if (!d.state || !policy || n_policy_layers < 1 || n_episodes < 1) return 0;
+    return evaluate_layout(d, policy, n_policy_layers, n_episodes).total;
+}
+
+// Episodes that have terminated keep being stepped (their rows are never read again: every episode is a row of its own in the environment kernels and in the policy),
+// where the reference leaves their state as it was (:166-170); returns, lengths and the terminated count stop at the terminating step as there.
+extern "C" int rlt_rocm_env_evaluate(rlt_rocm_device* device, const rlt_env_runner* env, int policy_kind, const rlt_seq_layer* policy, int n_policy_layers,
+                                     const rlt_seq_state* policy_state, int auto_reset_period, const float* observation_mean, const float* observation_precision,
+                                     const float* initial_states, int n_episodes, int step_limit, float* returns, uint32_t* episode_length, float* summary,
+                                     void* workspace, size_t workspace_bytes) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(env && policy && n_policy_layers >= 1 && n_policy_layers <= RLT_SEQ_MAX_LAYERS && initial_states && n_episodes >= 1 && step_limit >= 1 && returns && episode_length && summary);
+    RLT_REQUIRE((policy_kind == 1 || policy_kind == 2) && (observation_mean == nullptr) == (observation_precision == nullptr) && auto_reset_period >= 0);
+    const EnvDims d = env_dims(env->env_kind);
+    RLT_REQUIRE(d.state != 0);
+    bool recurrent = false;
+    for (int l = 0; l < n_policy_layers; l++) recurrent = recurrent || policy[l].kind != 0;
+    RLT_REQUIRE(!recurrent || policy_state);
+    const rlt_seq_layer& first = policy[0]; const rlt_seq_layer& last = policy[n_policy_layers - 1];
+    RLT_REQUIRE((first.kind == 0 ? first.dense.in_dim : first.gru.input_dim) == d.obs && (last.kind == 0 ? last.dense.out_dim : last.gru.hidden_dim) == policy_kind * d.act);
+    const int N = n_episodes, blocks = rlt_div_up(N, 256) > 1024 ? 1024 : rlt_div_up(N, 256);
+    const EvaluateLayout L = evaluate_layout(d, policy, n_policy_layers, N);
+    RLT_REQUIRE(workspace && workspace_bytes >= L.total);
+    char* w = reinterpret_cast<char*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    float* states = (float*)(w + L.states); float* raw = (float*)(w + L.raw); float* obs = (float*)(w + L.obs); float* out = (float*)(w + L.out);
+    float* actions = (float*)(w + L.actions); uint8_t* done = (uint8_t*)(w + L.done);
+    const size_t step_ws_bytes = workspace_bytes - (size_t)((w + L.step_ws) - (char*)workspace);
+    rlt_env_runner rn = *env;
+    rn.n_envs = N; rn.states = states; rn.actions = actions; rn.rewards = (float*)(w + L.rewards); rn.terminated = (uint8_t*)(w + L.terminated);
+    float* next_obs = observation_mean ? raw : obs;      // the environment's step kernel leaves the observation of the state it arrives at
+    const rlt_seq_state no_state = {};
+    int rc;
+    hipLaunchKernelGGL(env_copy_kernel, dim3(blocks), dim3(256), 0, device->stream, initial_states, states, (size_t)N * d.state);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if ((rc = rlt_rocm_fill_f32(device, returns, 1, N, N, 0.0f))) return rc;
+    if ((rc = rlt_rocm_fill_f32(device, (float*)episode_length, 1, N, N, 0.0f))) return rc;      // the bit pattern of 0.0f is the integer 0
+    if ((rc = rlt_rocm_fill_u8(device, done, (size_t)N, 0))) return rc;
+    if (policy_state && (rc = rlt_rocm_seq_reset_state(device, policy, n_policy_layers, policy_state, nullptr, N))) return rc;      // :135
+    hipLaunchKernelGGL(env_evaluate_observe_kernel, dim3(blocks), dim3(256), 0, device->stream, (int)env->env_kind, (const float*)states, next_obs, N);
+    if ((rc = rlt_launch_status(device))) return rc;
+    for (int step = 0; step < step_limit; step++) {
+        if (observation_mean) {
+            hipLaunchKernelGGL(env_evaluate_standardize_kernel, dim3(blocks), dim3(256), 0, device->stream, (const float*)raw, obs, observation_mean, observation_precision, N, d.obs);
+            if ((rc = rlt_launch_status(device))) return rc;
+        }
+        float* y = policy_kind == 1 ? actions : out;
+        if ((rc = rlt_rocm_seq_evaluate_step(device, policy, n_policy_layers, obs, d.obs, policy_state ? policy_state : &no_state, auto_reset_period, y, policy_kind * d.act, N,
+                                             w + L.step_ws, step_ws_bytes))) return rc;
+        if (policy_kind == 2) {
+            hipLaunchKernelGGL(env_evaluate_squash_kernel, dim3(blocks), dim3(256), 0, device->stream, (const float*)out, actions, N, d.act);
+            if ((rc = rlt_launch_status(device))) return rc;
+        }
+        if ((rc = env_step_launch(device, &rn, next_obs))) return rc;
+        hipLaunchKernelGGL(env_evaluate_accumulate_kernel, dim3(blocks), dim3(256), 0, device->stream, (const float*)rn.rewards, (const uint8_t*)rn.terminated, done, returns,
+                           episode_length, N);
+        if ((rc = rlt_launch_status(device))) return rc;
+    }
+    hipLaunchKernelGGL(env_evaluate_summary_kernel, dim3(1), dim3(64), 0, device->stream, (const float*)returns, (const uint32_t*)episode_length, (const uint8_t*)done, N, summary);
+    return rlt_launch_status(device);
+}

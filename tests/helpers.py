@@ -44,7 +44,7 @@ class LoopConfig(C.Structure):
 
 
 WITH_WORKSPACE = ("mlp_evaluate", "mlp_backward", "mlp_forward_backward", "mlp_forward_backward_input", "gru_forward", "gru_backward", "on_policy_collect", "seq_forward", "seq_backward", "seq_evaluate_step",
-                  "pendulum_runner_step_recurrent", "pendulum_evaluate_recurrent", "env_runner_step", "env_on_policy_collect", "env_runner_step_sequential")
+                  "pendulum_runner_step_recurrent", "pendulum_evaluate_recurrent", "env_runner_step", "env_on_policy_collect", "env_runner_step_sequential", "env_evaluate")
 
 
 def load_oracle():
@@ -1616,3 +1616,29 @@ def ppo_pendulum_loop(be, iterations, seed=0, n_envs=64, steps=128, minibatch=10
             if log:
                 print(be.name, it + 1, round(returns[-1]), 'log_std', float(agent.log_std.numpy()[0]), flush=True)
     return returns
+
+
+def env_evaluate_on_backend(backend, env_kind, specs, params, policy_kind, initial_states, step_limit, period=0, standardize=None, acrobot_parameters=None):
+    """rl::utils::evaluation::evaluate for any batched environment and a sequential policy (specs as for SeqNet) on a backend: (returns, episode_length, summary)."""
+    N = len(initial_states)
+    policy = SeqNet(backend, specs, params, 1, N, trainable=False)
+    recurrent = any(kind == 1 for kind, *_ in specs)
+    state = SeqStateOnBackend(backend, specs, N)
+    for l in state.hidden:                                   # the call resets the state itself: start from values a missing reset would show
+        state.hidden[l].upload(np.full((N, specs[l][2]), 0.5, np.float32)); state.step[l].upload(np.full(N, 3, np.uint32))
+    env = capi.EnvRunner()
+    env.env_kind = env_kind
+    env.pendulum, env.acrobot, env.car = capi.pendulum_parameters(), acrobot_parameters or capi.acrobot_parameters(), capi.car_parameters()
+    ini = backend.array(np.ascontiguousarray(initial_states, np.float32))
+    ret, length, summary = backend.zeros((N,)), backend.zeros((N,), np.uint32), backend.zeros((6,))
+    mean = precision = None
+    if standardize is not None:
+        mean, precision = backend.array(np.asarray(standardize[0], np.float32)), backend.array(np.asarray(standardize[1], np.float32))
+    ws, wsn = None, 0
+    if backend.name == "rocm":
+        wsn = int(backend.device.lib.rlt_rocm_env_evaluate_workspace_bytes(env_kind, policy.layers, policy.n, N))
+        keep = backend.device.empty((wsn,), np.uint8); ws = keep.ptr
+    backend.call("env_evaluate", C.byref(env), policy_kind, policy.layers, policy.n, C.byref(state.c) if recurrent else None, period, mean.ptr if mean else None,
+                 precision.ptr if precision else None, ini.ptr, N, step_limit, ret.ptr, length.ptr, summary.ptr, ws, wsn)
+    backend.sync()
+    return ret.numpy(), length.numpy(), summary.numpy()

@@ -622,3 +622,36 @@ def test_evaluate_step_chain_equals_the_sequence_forward_pass(oracle, fast_tanh)
         oracle.call("seq_evaluate_step", net.layers, net.n, xt.ptr, I, C.byref(state.c), 3, y.ptr, O, B, None, 0)
         assert np.array_equal(y.numpy(), want3[t]), t
     assert not np.array_equal(want3[3:], want[3:])
+
+
+def test_env_evaluate_reproduces_reference_vectors_and_counts_terminations(oracle):
+    """The evaluation over any environment: with the Pendulum it gives the reference's own episodes bit for bit (the vectors above); with the Acrobot, whose
+    episodes terminate, every episode equals that episode run alone, one step at a time, until its first terminated flag -- the terminating step's
+    reward counted, nothing after it (rl/utils/evaluation/operations_generic.h:166-197)."""
+    g = np.load(os.path.join(helpers.GOLDEN, "evaluation_pendulum_seed0.npz"))
+    specs = [(0, 3, 64, "relu"), (0, 64, 64, "relu"), (0, 64, 2, "identity")]
+    for k in range(len(g["stops"])):
+        ret, length, summary = helpers.env_evaluate_on_backend(oracle, helpers.capi.ENV_PENDULUM, specs, g[f"e{k}_actor"], 2, g[f"e{k}_initial_states"], 200)
+        assert np.array_equal(ret, g[f"e{k}_returns"]) and np.array_equal(length, g[f"e{k}_episode_length"]) and np.array_equal(summary, g[f"e{k}_summary"])
+    rng = np.random.default_rng(11)
+    n, limit = 12, 60
+    specs = [(0, 6, 16, "tanh"), (0, 16, 1, "tanh")]
+    params = helpers.random_seq_params(rng, specs)
+    ini = rng.uniform(-0.1, 0.1, (n, 4)).astype(np.float32)
+    ini[::2, 0] += 2.0 + rng.uniform(0, 0.4, n // 2).astype(np.float32)      # every other episode starts with the first link raised
+    ret, length, summary = helpers.env_evaluate_on_backend(oracle, helpers.capi.ENV_ACROBOT, specs, params, 1, ini, limit)
+    W1, b1, W2, b2 = params[:96].reshape(16, 6), params[96:112], params[112:128].reshape(1, 16), params[128:129]
+    n_terminated = 0
+    for e in range(n):
+        state, total, steps = ini[e:e + 1].copy(), np.float32(0), 0
+        for _ in range(limit):
+            _, obs, _, _, _ = helpers.acrobot_on_backend(oracle, 0, state, np.zeros(1, np.float32))
+            action = np.tanh(np.tanh(obs.astype(np.float64) @ W1.T.astype(np.float64) + b1) @ W2.T.astype(np.float64) + b2).astype(np.float32).reshape(1)
+            state, _, _, r, t = helpers.acrobot_on_backend(oracle, 0, state, action)
+            total = np.float32(total + r[0]); steps += 1
+            if t[0]:
+                n_terminated += 1
+                break
+        assert length[e] == steps and abs(ret[e] - total) <= 1e-6 * steps, (e, length[e], steps, ret[e], total)
+    assert 0 < n_terminated < n and summary[4] == n_terminated and summary[5] == np.float32(n_terminated) / np.float32(n)
+    assert abs(summary[2] - length.mean()) <= 1e-4 and abs(summary[3] - length.std()) <= 1e-3
