@@ -2,10 +2,11 @@
 // rl/components/off_policy_runner/operations_cuda.h:9-237).
 //
 // The CUDA backend compiles the environment's generic step into its prologue / epilogue kernels. This backend ships precompiled
-// kernels, so the runner steps the environments the C ABI has a kernel for: the Pendulum (rl/environments/pendulum). One step of all
-// environments -- reset where truncated, observe, the actor (an MLP with or without a sample_and_squash head, or given actions),
-// dynamics, reward, truncation and the replay add -- is ONE launch (rlt_rocm_pendulum_runner_step); the CUDA backend launches a
-// prologue kernel, the actor's layers and an epilogue kernel.
+// kernels, so the runner steps the environments the C ABI has a kernel for (rl/environments/operations_rocm.h: the Pendulum, the Acrobot and
+// the AcrobotSwingup). On the Pendulum one step of all environments -- reset where truncated, observe, the actor (an MLP with or without a
+// sample_and_squash head, or given actions), dynamics, reward, truncation and the replay add -- is ONE launch
+// (rlt_rocm_pendulum_runner_step); on the others it is a prologue kernel, the actor's layers, its head, the environment's step kernel and an
+// epilogue kernel (rlt_rocm_env_runner_step_sequential), as the CUDA backend launches them.
 //
 // Memory. runner.replay_buffers is, on every device, the block that holds the replay rings. Host code never looks inside it on a GPU
 // backend; here it holds the backend's own layout: the rings of all environments in one allocation (ring e = rows [e * capacity,
@@ -16,7 +17,7 @@
 #include <rl_tools/devices/rocm.h>
 #include <rl_tools/rl/components/off_policy_runner/off_policy_runner.h>
 #include <rl_tools/rl/components/off_policy_runner/operations_generic.h>
-#include <rl_tools/rl/environments/pendulum/pendulum.h>
+#include <rl_tools/rl/environments/operations_rocm.h>
 #include <rl_tools/nn_models/mlp/network.h>
 #include <rl_tools/nn_models/sequential/model.h>
 #include <rl_tools/nn_models/random_uniform/model.h>
@@ -59,15 +60,53 @@ namespace rl_tools{
             using ENVIRONMENT = typename SPEC::ENVIRONMENT;
             using T = typename SPEC::TYPE_POLICY::DEFAULT;
             using TI = typename SPEC::TI;
-            static_assert(utils::typing::is_same_v<ENVIRONMENT, rl::environments::Pendulum<typename ENVIRONMENT::SPEC>>, "the ROCM backend's runner steps the Pendulum; other environments have step kernels (rlt_rocm_acrobot_step, rlt_rocm_car_step) but no runner");
+            static_assert(utils::typing::is_same_v<ENVIRONMENT, rl::environments::Pendulum<typename ENVIRONMENT::SPEC>>);
             static_assert(sizeof(typename ENVIRONMENT::State) == 2 * sizeof(T) && sizeof(TI) == 4 && sizeof(bool) == 1);
-            using P = typename ENVIRONMENT::SPEC::PARAMETERS;
             rlt_pendulum_runner r = {};
             r.states = (float*)runner.states._data; r.episode_step = (uint32_t*)runner.episode_step._data; r.episode_return = (float*)runner.episode_return._data;
             r.truncated = (uint8_t*)runner.truncated._data;
             r.n_envs = SPEC::PARAMETERS::N_ENVIRONMENTS; r.episode_step_limit = SPEC::PARAMETERS::EPISODE_STEP_LIMIT;
-            r.env = rlt_pendulum_parameters{(float)P::g, (float)P::max_speed, (float)P::max_torque, (float)P::dt, (float)P::m, (float)P::l};
+            r.env = rl::environments::rocm::Description<ENVIRONMENT>::parameters();
             return r;
+        }
+        // one step of the runner through the library's entry points for any environment: head_kind 0 uniform actions in [-1, 1] (the warm-up policy),
+        // 1 / 2 / 3 a sequential policy (its output is the action / sample_and_squash / td3_sampling with noise_std). Initial states, exploration noise and
+        // uniform actions are drawn on the device first.
+        template <typename DEV_SPEC, typename SPEC, typename RNG>
+        void env_step(devices::ROCM<DEV_SPEC>& device, rl::components::OffPolicyRunner<SPEC>& runner, int head_kind, const rlt_seq_layer* layers, int n_layers,
+                      const rlt_seq_state* policy_state, int auto_reset_period, const rlt_sas_parameters* sas, float noise_std, RNG& rng){
+            using ENVIRONMENT = typename SPEC::ENVIRONMENT;
+            using DESCRIPTION = rl::environments::rocm::Description<ENVIRONMENT>;
+            static_assert(DESCRIPTION::SUPPORTED, "the ROCM backend's runner steps the environments that rl/environments/operations_rocm.h describes");
+            static_assert(sizeof(typename ENVIRONMENT::State) == DESCRIPTION::STATE_DIM * sizeof(float) && sizeof(typename SPEC::TI) == 4 && sizeof(bool) == 1);
+            constexpr size_t N = SPEC::PARAMETERS::N_ENVIRONMENTS, ACT = ENVIRONMENT::ACTION_DIM, STATE = DESCRIPTION::STATE_DIM;
+            const rlt_replay_buffer rb = replay(runner);
+            rlt_env_runner e = {};
+            DESCRIPTION::set_parameters(e);
+            e.n_envs = (int32_t)N; e.episode_step_limit = (int32_t)SPEC::PARAMETERS::EPISODE_STEP_LIMIT;
+            e.states = (float*)runner.states._data; e.episode_step = (uint32_t*)runner.episode_step._data; e.episode_return = (float*)runner.episode_return._data;
+            e.truncated = (uint8_t*)runner.truncated._data;
+            e.observations = runner.buffers.observations._data; e.actions = runner.buffers.actions._data; e.next_observations = runner.buffers.next_observations._data;
+            auto align = [](size_t bytes){ return (bytes + 255) / 256 * 256; };
+            const size_t rewards_bytes = align(N * sizeof(float)), terminated_bytes = align(N), noise_bytes = align(N * ACT * sizeof(float)), initial_bytes = align(N * STATE * sizeof(float));
+            // the workspace size depends on the runner's widths only, not on the pointers that are still to be carved out of the same block
+            const size_t workspace_bytes = head_kind == 0 ? 0 : rlt_rocm_env_runner_step_sequential_workspace_bytes(&e, layers, n_layers);
+            char* memory = (char*)devices::rocm::scratch(device, rewards_bytes + terminated_bytes + noise_bytes + initial_bytes + workspace_bytes);
+            e.rewards = (float*)memory; e.terminated = (uint8_t*)(memory + rewards_bytes);
+            float* noise = (float*)(memory + rewards_bytes + terminated_bytes); float* initial = (float*)(memory + rewards_bytes + terminated_bytes + noise_bytes);
+            void* workspace = memory + rewards_bytes + terminated_bytes + noise_bytes + initial_bytes;
+            DESCRIPTION::sample_initial_states(device, initial, N, rng);
+            if(head_kind == 0){
+                devices::rocm::check(rlt_rocm_rand_f32(device.handle, noise, N * ACT, -1.0f, 1.0f, rng.seed, random::next_stream(rng)), "step(runner, uniform actions)");
+                devices::rocm::check(rlt_rocm_env_runner_step(device.handle, &e, &rb, 0, nullptr, 0, nullptr, noise, nullptr, initial, nullptr, 0), "step(runner, uniform policy)");
+            }
+            else{
+                if(head_kind != 1){
+                    devices::rocm::check(rlt_rocm_randn_f32(device.handle, noise, N * ACT, rng.seed, random::next_stream(rng)), "step(runner, noise)");
+                }
+                devices::rocm::check(rlt_rocm_env_runner_step_sequential(device.handle, &e, &rb, layers, n_layers, policy_state, auto_reset_period, head_kind, sas, noise_std, noise, initial,
+                                                                         workspace, workspace_bytes), "step(runner, policy)");
+            }
         }
         // the dense layers of a policy in evaluation order, and whether it ends in a sample_and_squash head
         struct PolicyDescription{
@@ -175,7 +214,7 @@ namespace rl_tools{
         using L = rl::components::off_policy_runner::rocm::Layout<SPEC>;
         static_assert(SPEC::DYNAMIC_ALLOCATION, "runners on devices::ROCM are dynamically allocated");
         malloc(device, runner.buffers);
-        void* states = nullptr;     // the kernels' [N_ENVIRONMENTS x 2] float array
+        void* states = nullptr;     // the kernels' [N_ENVIRONMENTS x state width] float array
         devices::rocm::check(rlt_rocm_malloc(device.handle, &states, sizeof(typename SPEC::ENVIRONMENT::State) * SPEC::PARAMETERS::N_ENVIRONMENTS), "malloc(runner)");
         runner.states._data = (typename SPEC::ENVIRONMENT::State*)states;
         malloc(device, runner.episode_return);
@@ -236,81 +275,72 @@ namespace rl_tools{
         if(policy_switch){
             truncate_all(device, runner);
         }
-        const rlt_pendulum_runner r = rl::components::off_policy_runner::rocm::pendulum(runner);
-        const rlt_replay_buffer rb = rl::components::off_policy_runner::rocm::replay(runner);
+        namespace rocm = rl::components::off_policy_runner::rocm;
+        using ENVIRONMENT = typename SPEC::ENVIRONMENT;
+        // the Pendulum has a runner step of its own (one launch); the other environments take the library's step for any environment
+        constexpr bool PENDULUM = utils::typing::is_same_v<ENVIRONMENT, rl::environments::Pendulum<typename ENVIRONMENT::SPEC>>;
         if constexpr(utils::typing::is_same_v<POLICY, nn_models::RandomUniform<typename POLICY::SPEC>>){
             // the exploration policy of the warm-up phase: uniform actions (nn_models/random_uniform/operations_generic.h:28-44), drawn on the device
             static_assert(POLICY::SPEC::RANGE == nn_models::random_uniform::Range::MINUS_ONE_TO_ONE);
-            auto actions = to_tensor(device, runner.buffers.actions);
-            rand(device, actions, rng, -1.0f, 1.0f);
-            devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 0, nullptr, 0, nullptr, runner.buffers.actions._data, nullptr, nullptr, rng.seed, random::next_stream(rng)), "step(runner, uniform policy)");
-        }
-        else if constexpr(rl::components::off_policy_runner::rocm::HasGru<POLICY>::value){
-            // a recurrent actor (off_policy_runner/operations_generic.h:189-206): the policy state of the environments that start an episode is reset, then one
-            // evaluate_step in Rollout mode; GRU layers restart by themselves every SEQUENCE_LENGTH steps of their input shape (nn/layers/gru/operations_generic.h:406-413)
-            using ENVIRONMENT = typename SPEC::ENVIRONMENT;
-            using P = typename ENVIRONMENT::SPEC::PARAMETERS;
-            static_assert(P::initial_state_min_angle == -P::initial_state_max_angle && P::initial_state_min_speed == -P::initial_state_max_speed, "initial states are drawn from ranges that are symmetric about zero");
-            constexpr size_t ACT = ENVIRONMENT::ACTION_DIM;
-            rl::components::off_policy_runner::rocm::RecurrentPolicyDescription d;
-            rl::components::off_policy_runner::rocm::describe_recurrent(policy, get<POLICY_INDEX>(runner.policy_states).content_state, d);
-            utils::assert_exit(device, !d.unsupported && d.has_head, "step(runner): a recurrent policy is dense and GRU layers followed by sample_and_squash");
-            auto align = [](size_t bytes){ return (bytes + 255) / 256 * 256; };
-            const size_t noise_bytes = align(N * ACT * sizeof(float)), initial_bytes = align(N * 2 * sizeof(float));
-            const size_t workspace_bytes = rlt_rocm_pendulum_runner_step_recurrent_workspace_bytes(d.layers, d.n_layers, (int)N);
-            char* memory = (char*)devices::rocm::scratch(device, noise_bytes + initial_bytes + workspace_bytes);
-            float* noise = (float*)memory; float* initial = (float*)(memory + noise_bytes);
-            devices::rocm::check(rlt_rocm_randn_f32(device.handle, noise, N * ACT, rng.seed, random::next_stream(rng)), "step(runner, noise)");
-            devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, N * 2, -1.0f, 1.0f, rng.seed, random::next_stream(rng)), "step(runner, initial states)");
-            devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_angle, initial, 2, initial, 2, (int)N, 1), "step(runner, initial states)");
-            if constexpr(P::initial_state_max_speed != 1){
-                devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_speed, initial + 1, 2, initial + 1, 2, (int)N, 1), "step(runner, initial states)");
-            }
-            constexpr int AUTO_RESET_PERIOD = (int)get<0>(typename POLICY::INPUT_SHAPE{});
-            devices::rocm::check(rlt_rocm_pendulum_runner_step_recurrent(device.handle, &r, &rb, d.layers, d.n_layers, &d.state, AUTO_RESET_PERIOD, &d.head, noise, initial,
-                                                                         memory + noise_bytes + initial_bytes, workspace_bytes), "step(runner, recurrent actor)");
-        }
-        else{
-            rl::components::off_policy_runner::rocm::PolicyDescription d;
-            rl::components::off_policy_runner::rocm::describe(policy, d);
-            utils::assert_exit(device, d.standardize_mean == nullptr && !d.standardize_misplaced, "step(runner): the library's off-policy runner steps have no standardize layer");
-            if(d.has_td3_sampling){
-                // TD3's exploring actor: the library's runner step for any environment and any sequential policy with a td3_sampling head (reset, observe,
-                // policy, clamp(output + std * noise), dynamics, reward, replay add: a handful of launches)
-                using ENVIRONMENT = typename SPEC::ENVIRONMENT;
-                using P = typename ENVIRONMENT::SPEC::PARAMETERS;
-                static_assert(P::initial_state_min_angle == -P::initial_state_max_angle && P::initial_state_min_speed == -P::initial_state_max_speed, "initial states are drawn from ranges that are symmetric about zero");
-                constexpr size_t ACT = ENVIRONMENT::ACTION_DIM;
-                rlt_env_runner e = {};
-                e.env_kind = RLT_ENV_PENDULUM; e.n_envs = r.n_envs; e.episode_step_limit = r.episode_step_limit;
-                e.states = r.states; e.episode_step = r.episode_step; e.episode_return = r.episode_return; e.truncated = r.truncated; e.pendulum = r.env;
-                e.observations = runner.buffers.observations._data; e.actions = runner.buffers.actions._data; e.next_observations = runner.buffers.next_observations._data;
-                rlt_seq_layer layers[rl::components::off_policy_runner::rocm::PolicyDescription::MAX_LAYERS] = {};
-                for(int l = 0; l < d.n_layers; l++){ layers[l].kind = 0; layers[l].dense = d.layers[l]; }
-                auto align = [](size_t bytes){ return (bytes + 255) / 256 * 256; };
-                const size_t rewards_bytes = align(N * sizeof(float)), terminated_bytes = align(N), noise_bytes = align(N * ACT * sizeof(float)), initial_bytes = align(N * 2 * sizeof(float));
-                // the workspace size depends on the runner's widths only, not on the pointers that are still to be carved out of the same block
-                const size_t workspace_bytes = rlt_rocm_env_runner_step_sequential_workspace_bytes(&e, layers, d.n_layers);
-                char* memory = (char*)devices::rocm::scratch(device, rewards_bytes + terminated_bytes + noise_bytes + initial_bytes + workspace_bytes);
-                e.rewards = (float*)memory; e.terminated = (uint8_t*)(memory + rewards_bytes);
-                float* noise = (float*)(memory + rewards_bytes + terminated_bytes); float* initial = (float*)(memory + rewards_bytes + terminated_bytes + noise_bytes);
-                void* workspace = memory + rewards_bytes + terminated_bytes + noise_bytes + initial_bytes;
-                devices::rocm::check(rlt_rocm_randn_f32(device.handle, noise, N * ACT, rng.seed, random::next_stream(rng)), "step(runner, noise)");
-                devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, N * 2, -1.0f, 1.0f, rng.seed, random::next_stream(rng)), "step(runner, initial states)");
-                devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_angle, initial, 2, initial, 2, (int)N, 1), "step(runner, initial states)");
-                if constexpr(P::initial_state_max_speed != 1){
-                    devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_speed, initial + 1, 2, initial + 1, 2, (int)N, 1), "step(runner, initial states)");
-                }
-                devices::rocm::check(rlt_rocm_env_runner_step_sequential(device.handle, &e, &rb, layers, d.n_layers, nullptr, 0, 3, nullptr, d.td3_sampling_std, noise, initial, workspace, workspace_bytes), "step(runner, td3 actor)");
-            }
-            else if(d.has_head){
-                auto& noise = get_last_buffer(policy_eval_buffers).noise;
-                static_assert(utils::typing::remove_reference_t<decltype(noise)>::ROWS == N);
-                randn(device, noise, rng);
-                devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 2, d.layers, d.n_layers, &d.head, nullptr, noise._data, nullptr, rng.seed, random::next_stream(rng)), "step(runner, stochastic actor)");
+            if constexpr(PENDULUM){
+                const rlt_pendulum_runner r = rocm::pendulum(runner);
+                const rlt_replay_buffer rb = rocm::replay(runner);
+                auto actions = to_tensor(device, runner.buffers.actions);
+                rand(device, actions, rng, -1.0f, 1.0f);
+                devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 0, nullptr, 0, nullptr, runner.buffers.actions._data, nullptr, nullptr, rng.seed, random::next_stream(rng)), "step(runner, uniform policy)");
             }
             else{
-                devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 1, d.layers, d.n_layers, nullptr, nullptr, nullptr, nullptr, rng.seed, random::next_stream(rng)), "step(runner, deterministic actor)");
+                rocm::env_step(device, runner, 0, nullptr, 0, nullptr, 0, nullptr, 0.0f, rng);
+            }
+        }
+        else if constexpr(rocm::HasGru<POLICY>::value){
+            // a recurrent actor (off_policy_runner/operations_generic.h:189-206): the policy state of the environments that start an episode is reset, then one
+            // evaluate_step in Rollout mode; GRU layers restart by themselves every SEQUENCE_LENGTH steps of their input shape (nn/layers/gru/operations_generic.h:406-413)
+            rocm::RecurrentPolicyDescription d;
+            rocm::describe_recurrent(policy, get<POLICY_INDEX>(runner.policy_states).content_state, d);
+            utils::assert_exit(device, !d.unsupported && d.has_head, "step(runner): a recurrent policy is dense and GRU layers followed by sample_and_squash");
+            constexpr int AUTO_RESET_PERIOD = (int)get<0>(typename POLICY::INPUT_SHAPE{});
+            if constexpr(PENDULUM){
+                const rlt_pendulum_runner r = rocm::pendulum(runner);
+                const rlt_replay_buffer rb = rocm::replay(runner);
+                constexpr size_t ACT = ENVIRONMENT::ACTION_DIM;
+                auto align = [](size_t bytes){ return (bytes + 255) / 256 * 256; };
+                const size_t noise_bytes = align(N * ACT * sizeof(float)), initial_bytes = align(N * 2 * sizeof(float));
+                const size_t workspace_bytes = rlt_rocm_pendulum_runner_step_recurrent_workspace_bytes(d.layers, d.n_layers, (int)N);
+                char* memory = (char*)devices::rocm::scratch(device, noise_bytes + initial_bytes + workspace_bytes);
+                float* noise = (float*)memory; float* initial = (float*)(memory + noise_bytes);
+                devices::rocm::check(rlt_rocm_randn_f32(device.handle, noise, N * ACT, rng.seed, random::next_stream(rng)), "step(runner, noise)");
+                rl::environments::rocm::Description<ENVIRONMENT>::sample_initial_states(device, initial, N, rng);
+                devices::rocm::check(rlt_rocm_pendulum_runner_step_recurrent(device.handle, &r, &rb, d.layers, d.n_layers, &d.state, AUTO_RESET_PERIOD, &d.head, noise, initial,
+                                                                             memory + noise_bytes + initial_bytes, workspace_bytes), "step(runner, recurrent actor)");
+            }
+            else{
+                rocm::env_step(device, runner, 2, d.layers, d.n_layers, &d.state, AUTO_RESET_PERIOD, &d.head, 0.0f, rng);
+            }
+        }
+        else{
+            rocm::PolicyDescription d;
+            rocm::describe(policy, d);
+            utils::assert_exit(device, d.standardize_mean == nullptr && !d.standardize_misplaced, "step(runner): the library's off-policy runner steps have no standardize layer");
+            if(d.has_td3_sampling || !PENDULUM){
+                // the library's runner step for any environment and any sequential policy: reset, observe, the policy's layers, its head (TD3's exploring actor:
+                // clamp(output + std * noise); SAC's: sample_and_squash; else the output is the action), dynamics, reward, replay add: a handful of launches
+                rlt_seq_layer layers[rocm::PolicyDescription::MAX_LAYERS] = {};
+                for(int l = 0; l < d.n_layers; l++){ layers[l].kind = 0; layers[l].dense = d.layers[l]; }
+                rocm::env_step(device, runner, d.has_td3_sampling ? 3 : (d.has_head ? 2 : 1), layers, d.n_layers, nullptr, 0, &d.head, d.td3_sampling_std, rng);
+            }
+            else if constexpr(PENDULUM){
+                const rlt_pendulum_runner r = rocm::pendulum(runner);
+                const rlt_replay_buffer rb = rocm::replay(runner);
+                if(d.has_head){
+                    auto& noise = get_last_buffer(policy_eval_buffers).noise;
+                    static_assert(utils::typing::remove_reference_t<decltype(noise)>::ROWS == N);
+                    randn(device, noise, rng);
+                    devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 2, d.layers, d.n_layers, &d.head, nullptr, noise._data, nullptr, rng.seed, random::next_stream(rng)), "step(runner, stochastic actor)");
+                }
+                else{
+                    devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 1, d.layers, d.n_layers, nullptr, nullptr, nullptr, nullptr, rng.seed, random::next_stream(rng)), "step(runner, deterministic actor)");
+                }
             }
         }
         runner.previous_policy = POLICY_INDEX;

@@ -1,0 +1,77 @@
+// The environments whose step, reward, observation and termination the library has kernels for, described to its entry points
+// (rlt_env_runner: a kind and that kind's parameters) from the reference's environment types, with their initial states drawn on the device:
+//   rl::environments::Pendulum        rl/environments/pendulum/pendulum.h,  sample_initial_state operations_generic.h:58-61
+//   rl::environments::Acrobot         rl/environments/acrobot/acrobot.h,    sample_initial_state operations_generic.h:39-44
+//   rl::environments::AcrobotSwingup  (the same dynamics, another reward),  sample_initial_state operations_generic.h:46-52
+// The parameters of these environments are static members of ENVIRONMENT::SPEC::PARAMETERS, so a description needs the type only. The Car keeps its
+// parameters in the environment object (rl/environments/car/car.h) and has kernels (rlt_rocm_car_step) but no description here yet.
+#pragma once
+#include <rl_tools/devices/rocm.h>
+#include <rl_tools/rl/environments/pendulum/pendulum.h>
+#include <rl_tools/rl/environments/acrobot/acrobot.h>
+RL_TOOLS_NAMESPACE_WRAPPER_START
+namespace rl_tools::rl::environments::rocm{
+    template <typename ENVIRONMENT>
+    struct Description{
+        static constexpr bool SUPPORTED = false;
+    };
+    template <typename SPEC>
+    struct Description<rl::environments::Pendulum<SPEC>>{
+        using P = typename SPEC::PARAMETERS;
+        static constexpr bool SUPPORTED = true;
+        static constexpr int KIND = RLT_ENV_PENDULUM;
+        static constexpr size_t STATE_DIM = 2;
+        static_assert(P::initial_state_min_angle == -P::initial_state_max_angle && P::initial_state_min_speed == -P::initial_state_max_speed, "initial states are drawn from ranges that are symmetric about zero");
+        static rlt_pendulum_parameters parameters(){
+            return rlt_pendulum_parameters{(float)P::g, (float)P::max_speed, (float)P::max_torque, (float)P::dt, (float)P::m, (float)P::l};
+        }
+        static void set_parameters(rlt_env_runner& runner){ runner.env_kind = KIND; runner.pendulum = parameters(); }
+        // uniform in +- the largest angle and speed
+        template <typename DEV_SPEC, typename RNG>
+        static void sample_initial_states(devices::ROCM<DEV_SPEC>& device, float* initial, size_t n, RNG& rng){
+            devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, n * 2, -1.0f, 1.0f, rng.seed, random::next_stream(rng)), "sample_initial_state (Pendulum)");
+            devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_angle, initial, 2, initial, 2, (int)n, 1), "sample_initial_state (Pendulum)");
+            if constexpr(P::initial_state_max_speed != 1){
+                devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_speed, initial + 1, 2, initial + 1, 2, (int)n, 1), "sample_initial_state (Pendulum)");
+            }
+        }
+        // initial_state (rl/environments/pendulum/operations_generic.h:38-41): hanging down, at rest
+        static void initial_state(float* host){ host[0] = -math::PI<float>; host[1] = 0; }
+    };
+    namespace acrobot{
+        template <typename P>
+        rlt_acrobot_parameters parameters(){
+            return rlt_acrobot_parameters{(float)P::DT, (float)P::LINK_LENGTH_1, (float)P::LINK_LENGTH_2, (float)P::LINK_MASS_1, (float)P::LINK_MASS_2, (float)P::LINK_COM_POS_1,
+                                          (float)P::LINK_COM_POS_2, (float)P::LINK_MOI, (float)P::MAX_VEL_1, (float)P::MAX_VEL_2, (float)P::MIN_TORQUE, (float)P::MAX_TORQUE};
+        }
+    }
+    template <typename SPEC>
+    struct Description<rl::environments::Acrobot<SPEC>>{
+        static constexpr bool SUPPORTED = true;
+        static constexpr int KIND = RLT_ENV_ACROBOT;
+        static constexpr size_t STATE_DIM = 4;
+        static void set_parameters(rlt_env_runner& runner){ runner.env_kind = KIND; runner.acrobot = acrobot::parameters<typename SPEC::PARAMETERS>(); }
+        // both angles and both velocities uniform in +- 0.1
+        template <typename DEV_SPEC, typename RNG>
+        static void sample_initial_states(devices::ROCM<DEV_SPEC>& device, float* initial, size_t n, RNG& rng){
+            devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, n * 4, -0.1f, 0.1f, rng.seed, random::next_stream(rng)), "sample_initial_state (Acrobot)");
+        }
+        // initial_state (rl/environments/acrobot/operations_generic.h:54-59): hanging down, at rest
+        static void initial_state(float* host){ host[0] = host[1] = host[2] = host[3] = 0; }
+    };
+    template <typename SPEC>
+    struct Description<rl::environments::AcrobotSwingup<SPEC>>{
+        static constexpr bool SUPPORTED = true;
+        static constexpr int KIND = RLT_ENV_ACROBOT_SWINGUP;
+        static constexpr size_t STATE_DIM = 4;
+        static void set_parameters(rlt_env_runner& runner){ runner.env_kind = KIND; runner.acrobot = acrobot::parameters<typename SPEC::PARAMETERS>(); }
+        // both angles uniform over the circle, at rest
+        template <typename DEV_SPEC, typename RNG>
+        static void sample_initial_states(devices::ROCM<DEV_SPEC>& device, float* initial, size_t n, RNG& rng){
+            devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, n * 4, -math::PI<float>, math::PI<float>, rng.seed, random::next_stream(rng)), "sample_initial_state (AcrobotSwingup)");
+            devices::rocm::check(rlt_rocm_fill_f32(device.handle, initial + 2, (int)n, 2, 4, 0.0f), "sample_initial_state (AcrobotSwingup)");
+        }
+        static void initial_state(float* host){ host[0] = host[1] = host[2] = host[3] = 0; }
+    };
+}
+RL_TOOLS_NAMESPACE_WRAPPER_END

@@ -37,20 +37,21 @@ struct GemmParams {
     float* dW; float* dbias; float* ws; int splits;
 };
 
-template <int R>
-struct TileRegs { float4 v[(R * 4 + THREADS - 1) / THREADS]; };
+// a KB-deep operand tile of R rows in registers: R * KB / 4 quads over the workgroup's lanes
+template <int R, int KB = BK>
+struct TileRegs { float4 v[(R * KB / 4 + THREADS - 1) / THREADS]; };
 
 // source rows are contiguous along k: tile element (row r, k) = src[(row0+r)*ld + k0+k]
-template <int R>
-__device__ __forceinline__ void gload_kcontig(TileRegs<R>& t, const float* __restrict__ src, int ld, int row0, int nrows,
+template <int R, int KB = BK>
+__device__ __forceinline__ void gload_kcontig(TileRegs<R, KB>& t, const float* __restrict__ src, int ld, int row0, int nrows,
                                               int k0, int kend, int vec, int tid) {
-    constexpr int NQ = (R * 4 + THREADS - 1) / THREADS;
+    constexpr int QUADS = R * KB / 4, NQ = (QUADS + THREADS - 1) / THREADS, QPK = KB / 4;
 #pragma unroll
     for (int i = 0; i < NQ; i++) {
         int q = tid + i * THREADS;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (q < R * 4) {
-            int row = q >> 2, kq = (q & 3) * 4;
+        if (q < QUADS) {
+            int row = q / QPK, kq = (q % QPK) * 4;
             int gr = row0 + row, gk = k0 + kq;
             if (gr < nrows && gk < kend) {
                 const float* p = src + (size_t)gr * ld + gk;
@@ -69,32 +70,32 @@ __device__ __forceinline__ void gload_kcontig(TileRegs<R>& t, const float* __res
         t.v[i] = v;
     }
 }
-template <int R>
-__device__ __forceinline__ void sstore_kcontig(const TileRegs<R>& t, float* s, int tid) {
-    constexpr int NQ = (R * 4 + THREADS - 1) / THREADS;
+template <int R, int KB = BK, int P = PAD>
+__device__ __forceinline__ void sstore_kcontig(const TileRegs<R, KB>& t, float* s, int tid) {
+    constexpr int QUADS = R * KB / 4, NQ = (QUADS + THREADS - 1) / THREADS, QPK = KB / 4;
 #pragma unroll
     for (int i = 0; i < NQ; i++) {
         int q = tid + i * THREADS;
-        if (q < R * 4) {
-            int row = q >> 2, kq = (q & 3) * 4;
-            s[(kq + 0) * (R + PAD) + row] = t.v[i].x;
-            s[(kq + 1) * (R + PAD) + row] = t.v[i].y;
-            s[(kq + 2) * (R + PAD) + row] = t.v[i].z;
-            s[(kq + 3) * (R + PAD) + row] = t.v[i].w;
+        if (q < QUADS) {
+            int row = q / QPK, kq = (q % QPK) * 4;
+            s[(kq + 0) * (R + P) + row] = t.v[i].x;
+            s[(kq + 1) * (R + P) + row] = t.v[i].y;
+            s[(kq + 2) * (R + P) + row] = t.v[i].z;
+            s[(kq + 3) * (R + P) + row] = t.v[i].w;
         }
     }
 }
 // source rows are k, contiguous along the tile's m/n: tile element (k, c) = src[(k0+k)*ld + col0+c]
-template <int R>
-__device__ __forceinline__ void gload_mncontig(TileRegs<R>& t, const float* __restrict__ src, int ld, int col0, int ncols,
+template <int R, int KB = BK>
+__device__ __forceinline__ void gload_mncontig(TileRegs<R, KB>& t, const float* __restrict__ src, int ld, int col0, int ncols,
                                                int k0, int kend, int vec, int tid) {
-    constexpr int NQ = (R * 4 + THREADS - 1) / THREADS;
+    constexpr int QUADS = R * KB / 4, NQ = (QUADS + THREADS - 1) / THREADS;
     constexpr int QPR = R / 4;  // quads per k-row
 #pragma unroll
     for (int i = 0; i < NQ; i++) {
         int q = tid + i * THREADS;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (q < R * 4) {
+        if (q < QUADS) {
             int k = q / QPR, c4 = (q % QPR) * 4;
             int gk = k0 + k, gc = col0 + c4;
             if (gk < kend && gc < ncols) {
@@ -114,27 +115,31 @@ __device__ __forceinline__ void gload_mncontig(TileRegs<R>& t, const float* __re
         t.v[i] = v;
     }
 }
-template <int R>
-__device__ __forceinline__ void sstore_mncontig(const TileRegs<R>& t, float* s, int tid) {
-    constexpr int NQ = (R * 4 + THREADS - 1) / THREADS;
+template <int R, int KB = BK, int P = PAD>
+__device__ __forceinline__ void sstore_mncontig(const TileRegs<R, KB>& t, float* s, int tid) {
+    constexpr int QUADS = R * KB / 4, NQ = (QUADS + THREADS - 1) / THREADS;
     constexpr int QPR = R / 4;
 #pragma unroll
     for (int i = 0; i < NQ; i++) {
         int q = tid + i * THREADS;
-        if (q < R * 4) {
+        if (q < QUADS) {
             int k = q / QPR, c4 = (q % QPR) * 4;
-            *reinterpret_cast<float4*>(&s[k * (R + PAD) + c4]) = t.v[i];
+            *reinterpret_cast<float4*>(&s[k * (R + P) + c4]) = t.v[i];
         }
     }
 }
 
-template <int MODE, int WAVES_M, int WAVES_N, int TM, int TN>
+// KB: rows of k per step. 16 with two LDS buffers (the next step's tile is stored while this one is multiplied) when many workgroups share a
+// compute unit and hide each other's memory latency; 64 with one buffer when the whole grid is a few workgroups, each alone on its compute unit
+// and waiting one memory latency per step: a quarter of the steps.
+template <int MODE, int WAVES_M, int WAVES_N, int TM, int TN, int KB = BK>
 __global__ __launch_bounds__(THREADS) void gemm_kernel(GemmParams p) {
     static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per workgroup");
     constexpr int BM = WAVES_M * TM * 32;
     constexpr int BN = WAVES_N * TN * 32;
-    __shared__ __attribute__((aligned(16))) float sA[2][BK * (BM + PAD)];
-    __shared__ __attribute__((aligned(16))) float sB[2][BK * (BN + PAD)];
+    constexpr int NBUF = KB > 32 ? 1 : 2;
+    __shared__ __attribute__((aligned(16))) float sA[NBUF][KB * (BM + PAD)];
+    __shared__ __attribute__((aligned(16))) float sB[NBUF][KB * (BN + PAD)];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -144,7 +149,7 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(GemmParams p) {
 
     int ks = 0, ke = p.K;
     if (MODE == 2) { ks = blockIdx.z * p.k_per_split; ke = min(p.K, ks + p.k_per_split); }
-    const int nk = (ke - ks + BK - 1) / BK;
+    const int nk = (ke - ks + KB - 1) / KB;
 
     floatx16 acc[TM][TN];
 #pragma unroll
@@ -154,17 +159,17 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(GemmParams p) {
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    TileRegs<BM> ra;
-    TileRegs<BN> rb;
+    TileRegs<BM, KB> ra;
+    TileRegs<BN, KB> rb;
     auto gload = [&](int k0) {
-        if (MODE == 2) gload_mncontig<BM>(ra, p.A, p.lda, m0, p.M, k0, ke, p.vecA, tid);
-        else gload_kcontig<BM>(ra, p.A, p.lda, m0, p.M, k0, ke, p.vecA, tid);
-        if (MODE == 0) gload_kcontig<BN>(rb, p.B, p.ldb, n0, p.N, k0, ke, p.vecB, tid);
-        else gload_mncontig<BN>(rb, p.B, p.ldb, n0, p.N, k0, ke, p.vecB, tid);
+        if (MODE == 2) gload_mncontig<BM, KB>(ra, p.A, p.lda, m0, p.M, k0, ke, p.vecA, tid);
+        else gload_kcontig<BM, KB>(ra, p.A, p.lda, m0, p.M, k0, ke, p.vecA, tid);
+        if (MODE == 0) gload_kcontig<BN, KB>(rb, p.B, p.ldb, n0, p.N, k0, ke, p.vecB, tid);
+        else gload_mncontig<BN, KB>(rb, p.B, p.ldb, n0, p.N, k0, ke, p.vecB, tid);
     };
     auto sstore = [&](int buf) {
-        if (MODE == 2) sstore_mncontig<BM>(ra, sA[buf], tid); else sstore_kcontig<BM>(ra, sA[buf], tid);
-        if (MODE == 0) sstore_kcontig<BN>(rb, sB[buf], tid); else sstore_mncontig<BN>(rb, sB[buf], tid);
+        if (MODE == 2) sstore_mncontig<BM, KB>(ra, sA[buf], tid); else sstore_kcontig<BM, KB>(ra, sA[buf], tid);
+        if (MODE == 0) sstore_kcontig<BN, KB>(rb, sB[buf], tid); else sstore_mncontig<BN, KB>(rb, sB[buf], tid);
     };
 
     const bool bias_block = (MODE == 2) && (blockIdx.x == 0) && (p.dbias != nullptr);
@@ -173,53 +178,93 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(GemmParams p) {
     if (nk > 0) { gload(ks); sstore(0); }
     __syncthreads();
     for (int t = 0; t < nk; t++) {
-        const int cur = t & 1;
-        if (t + 1 < nk) gload(ks + (t + 1) * BK);
+        const int cur = NBUF == 2 ? (t & 1) : 0;
+        if (t + 1 < nk) gload(ks + (t + 1) * KB);
         const float* a_base = sA[cur] + (lane >> 5) * (BM + PAD) + wm * (TM * 32) + (lane & 31);
         const float* b_base = sB[cur] + (lane >> 5) * (BN + PAD) + wn * (TN * 32) + (lane & 31);
+        // CH pairs of k at a time: their LDS reads are all in flight before the first multiply waits for its own (one read, one wait, one multiply in turn
+        // leaves a wavefront that is alone on its SIMD idle for an LDS latency per multiply). Small tiles, which run on few workgroups, take the longest runs.
+        constexpr int CH = TM * TN == 1 ? 8 : (TM * TN == 2 ? 4 : 1);
+        static_assert((KB / 2) % CH == 0);
 #pragma unroll
-        for (int kk = 0; kk < BK / 2; kk++) {
-            float a[TM], b[TN];
+        for (int kk0 = 0; kk0 < KB / 2; kk0 += CH) {
+            float a[CH][TM], b[CH][TN];
 #pragma unroll
-            for (int i = 0; i < TM; i++) a[i] = a_base[kk * 2 * (BM + PAD) + i * 32];
+            for (int c = 0; c < CH; c++) {
 #pragma unroll
-            for (int j = 0; j < TN; j++) b[j] = b_base[kk * 2 * (BN + PAD) + j * 32];
+                for (int i = 0; i < TM; i++) a[c][i] = a_base[(kk0 + c) * 2 * (BM + PAD) + i * 32];
 #pragma unroll
-            for (int i = 0; i < TM; i++)
+                for (int j = 0; j < TN; j++) b[c][j] = b_base[(kk0 + c) * 2 * (BN + PAD) + j * 32];
+            }
+            if constexpr (CH > 1) __builtin_amdgcn_sched_barrier(0);      // the instruction scheduler would otherwise move every read back next to its multiply
 #pragma unroll
-                for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+            for (int c = 0; c < CH; c++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[c][i], b[c][j], acc[i][j], 0, 0, 0);
         }
         if (bias_block && tid < BM) {
 #pragma unroll
-            for (int k = 0; k < BK; k++) bsum += sA[cur][k * (BM + PAD) + tid];
+            for (int k = 0; k < KB; k++) bsum += sA[cur][k * (BM + PAD) + tid];
         }
-        if (t + 1 < nk) sstore(cur ^ 1);
-        __syncthreads();
+        if constexpr (NBUF == 2) {
+            if (t + 1 < nk) sstore(cur ^ 1);
+            __syncthreads();
+        } else {
+            __syncthreads();      // every wavefront has read this step's tile
+            if (t + 1 < nk) sstore(0);
+            __syncthreads();
+        }
     }
 
-    // ---- epilogue. Accumulator element v of lane l in a 32x32 tile: row = 8*(v/4) + 4*(l/32) + v%4, col = l%32
+    // ---- epilogue. Accumulator element v of lane l in a 32x32 tile: row = 8*(v/4) + 4*(l/32) + v%4, col = l%32.
+    // What a tile reads from memory (the bias of its column, the activation-derivative operands or the gradient so far of its 16 elements) is
+    // requested before its first store: a read issued between the stores waits for every store before it, one memory round trip per element.
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+            const int row_base = m0 + wm * (TM * 32) + i * 32 + 4 * (lane >> 5);
+            const bool col_ok = col < p.N;
+            float bias_c = 0.0f;
+            if (MODE == 0 && p.bias && col_ok) bias_c = p.bias[col];
+            float operand[16];
+            const bool want_operand = MODE == 1 ? p.dact_pre != nullptr : (MODE == 2 && p.splits == 1);
+            if (MODE != 0 && want_operand) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int row = row_base + 8 * (v >> 2) + (v & 3);
+                    const float* src = MODE == 1 ? p.dact_pre : p.dW;
+                    operand[v] = (row < p.M && col_ok) ? src[(size_t)row * p.N + col] : 0.0f;
+                }
+            }
+            // everything that depends on those reads is computed before the first store too (a use of a loaded value further down, in a block of its own,
+            // would again wait for all memory operations before it)
+            float val[16];
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int row = m0 + wm * (TM * 32) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (row < p.M && col < p.N) {
-                    float val = acc[i][j][v];
+                val[v] = acc[i][j][v];
+                if (MODE == 0) val[v] += bias_c;
+                else if (MODE == 1) { if (p.dact_pre) val[v] *= p.dact_from_output ? rlt_dact_from_output(operand[v], p.dact_kind) : rlt_dact(operand[v], p.dact_kind); }
+                else if (p.splits == 1) val[v] = operand[v] + val[v];
+                asm volatile("" : "+v"(val[v]));      // the value is final here: the compiler would otherwise sink the arithmetic into the store's block
+            }
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = row_base + 8 * (v >> 2) + (v & 3);
+                if (row < p.M && col_ok) {
                     if (MODE == 0) {
-                        if (p.bias) val += p.bias[col];
-                        if (p.pre) p.pre[(size_t)row * p.N + col] = val;
-                        float o = rlt_act(val, p.act);
+                        if (p.pre) p.pre[(size_t)row * p.N + col] = val[v];
+                        float o = rlt_act(val[v], p.act);
                         if (p.out) p.out[(size_t)row * p.N + col] = o;
                         if (p.y) p.y[(size_t)row * p.ldy + col] = o;
                     } else if (MODE == 1) {
-                        if (p.dact_pre) { float a = p.dact_pre[(size_t)row * p.N + col]; val *= p.dact_from_output ? rlt_dact_from_output(a, p.dact_kind) : rlt_dact(a, p.dact_kind); }
-                        p.C[(size_t)row * p.ldc + col] = val;
+                        p.C[(size_t)row * p.ldc + col] = val[v];
                     } else {
-                        if (p.splits == 1) p.dW[(size_t)row * p.N + col] += val;
-                        else p.ws[(size_t)blockIdx.z * ((size_t)p.M * p.N + p.M) + (size_t)row * p.N + col] = val;
+                        if (p.splits == 1) p.dW[(size_t)row * p.N + col] = val[v];
+                        else p.ws[(size_t)blockIdx.z * ((size_t)p.M * p.N + p.M) + (size_t)row * p.N + col] = val[v];
                     }
                 }
             }
@@ -377,6 +422,108 @@ __global__ __launch_bounds__(THREADS) void wgrad_wide_kernel(WideArgs a) {
     }
 }
 
+// ---- the same contractions on tiles of 16x16 per wavefront -----------------------------------------------------------------------
+// A problem whose 64x64 tiles number fewer than the compute units (a batch of a few hundred rows through layers a few hundred wide) leaves most of the chip
+// idle while each of its workgroups works through hundreds of dependent 32x32x2 multiplies. Here a wavefront owns one 16x16 tile (v_mfma_f32_16x16x4_f32,
+// a quarter of the multiply time per unit of k) and a workgroup WAVES_M x WAVES_N of them (32x32, or 64x16 / 16x64 for one narrow side): four times the
+// workgroups, each with a quarter of the chain. 64 rows of k per step through one LDS buffer, LDS reads of eight multiplies in flight at a time.
+// Operand A/B lane layout of the instruction: lane l holds A[row l % 16][k l / 16] and B[k l / 16][col l % 16]; accumulator element v of lane l is
+// C[row 4 * (l / 16) + v][col l % 16].
+template <int MODE, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(THREADS) void gemm_small_kernel(GemmParams p) {
+    static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per workgroup");
+    constexpr int KB = 64, BM = WAVES_M * 16, BN = WAVES_N * 16;
+    constexpr int PA = (48 - BM % 32) % 32, PB = (48 - BN % 32) % 32;      // k-rows 16 banks apart: the four k of a multiply's operand read fall on disjoint halves in pairs
+    __shared__ __attribute__((aligned(16))) float sA[KB * (BM + PA)];
+    __shared__ __attribute__((aligned(16))) float sB[KB * (BN + PB)];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    int ks = 0, ke = p.K;
+    if (MODE == 2) { ks = blockIdx.z * p.k_per_split; ke = min(p.K, ks + p.k_per_split); }
+    const int nk = (ke - ks + KB - 1) / KB;
+    wide_floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    TileRegs<BM, KB> ra;
+    TileRegs<BN, KB> rb;
+    auto gload = [&](int k0) {
+        if (MODE == 2) gload_mncontig<BM, KB>(ra, p.A, p.lda, m0, p.M, k0, ke, p.vecA, tid);
+        else gload_kcontig<BM, KB>(ra, p.A, p.lda, m0, p.M, k0, ke, p.vecA, tid);
+        if (MODE == 0) gload_kcontig<BN, KB>(rb, p.B, p.ldb, n0, p.N, k0, ke, p.vecB, tid);
+        else gload_mncontig<BN, KB>(rb, p.B, p.ldb, n0, p.N, k0, ke, p.vecB, tid);
+    };
+    auto sstore = [&]() {
+        if (MODE == 2) sstore_mncontig<BM, KB, PA>(ra, sA, tid); else sstore_kcontig<BM, KB, PA>(ra, sA, tid);
+        if (MODE == 0) sstore_kcontig<BN, KB, PB>(rb, sB, tid); else sstore_mncontig<BN, KB, PB>(rb, sB, tid);
+    };
+    const bool bias_block = (MODE == 2) && (blockIdx.x == 0) && (p.dbias != nullptr);
+    float bsum = 0.0f;
+    if (nk > 0) { gload(ks); sstore(); }
+    __syncthreads();
+    for (int t = 0; t < nk; t++) {
+        if (t + 1 < nk) gload(ks + (t + 1) * KB);
+        const float* a_base = sA + (lane >> 4) * (BM + PA) + wm * 16 + (lane & 15);
+        const float* b_base = sB + (lane >> 4) * (BN + PB) + wn * 16 + (lane & 15);
+#pragma unroll
+        for (int kk0 = 0; kk0 < KB / 4; kk0 += 8) {
+            float a[8], b[8];
+#pragma unroll
+            for (int c = 0; c < 8; c++) { a[c] = a_base[(kk0 + c) * 4 * (BM + PA)]; b[c] = b_base[(kk0 + c) * 4 * (BN + PB)]; }
+            __builtin_amdgcn_sched_barrier(0);      // keeps the eight pairs of reads ahead of the multiplies
+#pragma unroll
+            for (int c = 0; c < 8; c++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[c], b[c], acc, 0, 0, 0);
+        }
+        if (bias_block && tid < BM) {
+#pragma unroll
+            for (int k = 0; k < KB; k++) bsum += sA[k * (BM + PA) + tid];
+        }
+        __syncthreads();      // every wavefront has read this step's tile
+        if (t + 1 < nk) sstore();
+        __syncthreads();
+    }
+    // epilogue: what the tile reads from memory is requested, and everything that depends on it computed, before the first store (see gemm_kernel)
+    const int col = n0 + wn * 16 + (lane & 15), row_base = m0 + wm * 16 + 4 * (lane >> 4);
+    const bool col_ok = col < p.N;
+    float bias_c = 0.0f;
+    if (MODE == 0 && p.bias && col_ok) bias_c = p.bias[col];
+    float operand[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bool want_operand = MODE == 1 ? p.dact_pre != nullptr : (MODE == 2 && p.splits == 1);
+    if (MODE != 0 && want_operand) {
+        const float* src = MODE == 1 ? p.dact_pre : p.dW;
+#pragma unroll
+        for (int v = 0; v < 4; v++) operand[v] = (row_base + v < p.M && col_ok) ? src[(size_t)(row_base + v) * p.N + col] : 0.0f;
+    }
+    float val[4];
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        val[v] = acc[v];
+        if (MODE == 0) val[v] += bias_c;
+        else if (MODE == 1) { if (p.dact_pre) val[v] *= p.dact_from_output ? rlt_dact_from_output(operand[v], p.dact_kind) : rlt_dact(operand[v], p.dact_kind); }
+        else if (p.splits == 1) val[v] = operand[v] + val[v];
+        asm volatile("" : "+v"(val[v]));
+    }
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int row = row_base + v;
+        if (row < p.M && col_ok) {
+            if (MODE == 0) {
+                if (p.pre) p.pre[(size_t)row * p.N + col] = val[v];
+                const float o = rlt_act(val[v], p.act);
+                if (p.out) p.out[(size_t)row * p.N + col] = o;
+                if (p.y) p.y[(size_t)row * p.ldy + col] = o;
+            } else if (MODE == 1) {
+                p.C[(size_t)row * p.ldc + col] = val[v];
+            } else {
+                if (p.splits == 1) p.dW[(size_t)row * p.N + col] = val[v];
+                else p.ws[(size_t)blockIdx.z * ((size_t)p.M * p.N + p.M) + (size_t)row * p.N + col] = val[v];
+            }
+        }
+    }
+    if (bias_block && tid < BM && m0 + tid < p.M) {
+        if (p.splits == 1) p.dbias[m0 + tid] += bsum;
+        else p.ws[(size_t)blockIdx.z * ((size_t)p.M * p.N + p.M) + (size_t)p.M * p.N + m0 + tid] = bsum;
+    }
+}
+
 // d_pre = act'(pre) * d_output (nn/layers/dense/operations_cpu_blas.h:119-141); dst may alias src
 __global__ __launch_bounds__(256) void dpre_kernel(const float* src, int lds, float* dst, int ldd, const float* __restrict__ pre, int rows, int cols, int act, int from_output) {
     const size_t total = (size_t)rows * cols;
@@ -421,15 +568,34 @@ TileShape pick_tile(int M, int N, int mode) {
     return 100 * padded_area(M, N, TILE_128x128) <= 115 * padded_area(M, N, TILE_64x64) ? TILE_128x128 : TILE_64x64;
 }
 
+// The tile shape a contraction runs with. A grid of large tiles that leaves compute units idle runs faster as 64x64 tiles (the forward and
+// input-gradient contractions do not split k to fill the chip); the weight gradient over a short batch (k_total rows) has few rows to split and
+// takes 64x64 tiles as well.
+constexpr int SHORT_BATCH = 2048;
+TileShape plan_tile(const rlt_rocm_device* device, int M, int N, int mode, int k_total) {
+    TileShape shape = pick_tile(M, N, mode);
+    int bm, bn;
+    tile_dims(shape, bm, bn);
+    if (mode != 2 && bm >= 128 && bn >= 64 && rlt_div_up(N, bn) * rlt_div_up(M, bm) < device->compute_units) shape = TILE_64x64;
+    if (mode == 2 && shape == TILE_128x128 && k_total <= SHORT_BATCH) shape = TILE_64x64;
+    return shape;
+}
+
 template <int MODE>
 int launch(rlt_rocm_device* device, const GemmParams& p, int splits) {
     dim3 block(THREADS);
-    TileShape shape = pick_tile(p.M, p.N, MODE);
+    const TileShape shape = plan_tile(device, p.M, p.N, MODE, p.K);
     int bm, bn;
     tile_dims(shape, bm, bn);
-    // a grid of large tiles that leaves compute units idle runs faster as 64x64 tiles (no split over k to fill the chip here)
-    if (MODE != 2 && bm >= 128 && bn >= 64 && rlt_div_up(p.N, bn) * rlt_div_up(p.M, bm) < device->compute_units) { shape = TILE_64x64; tile_dims(shape, bm, bn); }
     const dim3 grid(rlt_div_up(p.N, bn), rlt_div_up(p.M, bm), splits);
+    // at most one workgroup per compute unit and a reduction of some length: four times the workgroups on 16x16 tiles per wavefront (gemm_small_kernel)
+    const bool few = (long long)grid.x * grid.y * grid.z <= device->compute_units && p.k_per_split >= 64 && shape != TILE_128x64 && shape != TILE_128x128;
+    if (few) {
+        if (p.N <= 16) hipLaunchKernelGGL((gemm_small_kernel<MODE, 4, 1>), dim3(rlt_div_up(p.N, 16), rlt_div_up(p.M, 64), splits), block, 0, device->stream, p);
+        else if (p.M <= 16) hipLaunchKernelGGL((gemm_small_kernel<MODE, 1, 4>), dim3(rlt_div_up(p.N, 64), rlt_div_up(p.M, 16), splits), block, 0, device->stream, p);
+        else hipLaunchKernelGGL((gemm_small_kernel<MODE, 2, 2>), dim3(rlt_div_up(p.N, 32), rlt_div_up(p.M, 32), splits), block, 0, device->stream, p);
+        return rlt_launch_status(device);
+    }
     switch (shape) {
         case TILE_128x32: hipLaunchKernelGGL((gemm_kernel<MODE, 4, 1, 1, 1>), grid, block, 0, device->stream, p); break;
         case TILE_32x128: hipLaunchKernelGGL((gemm_kernel<MODE, 1, 4, 1, 1>), grid, block, 0, device->stream, p); break;
@@ -466,7 +632,7 @@ int rlt_gemm_backward_input(rlt_rocm_device* device, const float* d_pre, int ldd
 // 256 rows per split (64 for small gradients). Each split writes one block of out_dim * in_dim + out_dim partial sums.
 static void wgrad_split(const rlt_rocm_device* device, int batch, int in_dim, int out_dim, int& splits, int& kps) {
     int bm, bn;
-    tile_dims(pick_tile(out_dim, in_dim, 2), bm, bn);
+    tile_dims(plan_tile(device, out_dim, in_dim, 2, batch), bm, bn);
     int tiles = rlt_div_up(out_dim, bm) * rlt_div_up(in_dim, bn);
     splits = (2 * device->compute_units + tiles - 1) / tiles;
     // at least 256 rows per split; for small gradients (up to 96 x 64: the layers of width 16 and 32) 64 rows, i.e. 4 k-steps: a short batch is bound by the chain

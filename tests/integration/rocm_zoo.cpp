@@ -1,13 +1,14 @@
-// The reference's zoo configurations of the Pendulum (src/rl/zoo/pendulum-v1/{sac,td3,ppo}.h), included as they are and instantiated on
+// The reference's zoo configurations of the Pendulum (src/rl/zoo/pendulum-v1/{sac,td3,ppo}.h) and of the AcrobotSwingup
+// (src/rl/zoo/acrobot-swingup-v0/sac.h), included as they are and instantiated on
 // devices::ROCM the way src/rl/zoo/zoo.cpp:135-268 instantiates them on the CPU device: FACTORY<DEVICE, ...>::LOOP_CORE_CONFIG inside the
 // evaluation and timing loop steps (the experiment tracking, checkpoint and trajectory steps of zoo.cpp write files and are left out),
-// then `while(!step(device, ts))`. One source, three programs: -DZOO_SAC, -DZOO_TD3 or -DZOO_PPO selects the algorithm as
-// RL_TOOLS_RL_ZOO_ALGORITHM_* does there. Nothing of the configuration is restated here: batch sizes, widths, activation functions,
+// then `while(!step(device, ts))`. One source, four programs: -DZOO_SAC, -DZOO_TD3 or -DZOO_PPO selects the algorithm on the Pendulum as
+// RL_TOOLS_RL_ZOO_ALGORITHM_* does there, -DZOO_ACROBOT_SWINGUP_SAC the AcrobotSwingup with SAC (RL_TOOLS_RL_ZOO_ENVIRONMENT_ACROBOT_SWINGUP_V0). Nothing of the configuration is restated here: batch sizes, widths, activation functions,
 // step limits and optimizer parameters are the zoo's.
 //
 // With -DZOO_DEVICE_CPU the same program runs on the reference's CPU device (its generic operations, one thread): the figure the device's is read against.
 //
-// Usage: rocm_zoo_pendulum_v1_<algorithm> [seed [step_limit]] ; prints "evaluation <i> step <s> mean_return <r>" for every evaluation the
+// Usage: rocm_zoo_<environment>_<algorithm> [seed [step_limit]] ; prints "evaluation <i> step <s> mean_return <r>" for every evaluation the
 // loop made and a last line "final <r> best <r> loop_steps <n> seconds <s>".
 #include <rl_tools/operations/cpu_mux.h>
 #ifndef ZOO_DEVICE_CPU
@@ -24,6 +25,7 @@
 #include <rl_tools/nn_models/sequential/operations_generic.h>
 #include <rl_tools/nn/optimizers/adam/operations_generic.h>
 #include <rl_tools/rl/environments/pendulum/operations_cpu.h>
+#include <rl_tools/rl/environments/acrobot/operations_cpu.h>
 #ifndef ZOO_DEVICE_CPU
 #include <rl_tools/nn/operations_rocm.h>
 #include <rl_tools/nn/layers/standardize/operations_rocm.h>
@@ -48,8 +50,11 @@
 #elif defined(ZOO_PPO)
 #include <pendulum-v1/ppo.h>
 #include <rl_tools/rl/algorithms/ppo/loop/core/operations_generic.h>
+#elif defined(ZOO_ACROBOT_SWINGUP_SAC)
+#include <acrobot-swingup-v0/sac.h>
+#include <rl_tools/rl/algorithms/sac/loop/core/operations_generic.h>
 #else
-#error "define ZOO_SAC, ZOO_TD3 or ZOO_PPO"
+#error "define ZOO_SAC, ZOO_TD3, ZOO_PPO or ZOO_ACROBOT_SWINGUP_SAC"
 #endif
 #include <rl_tools/rl/loop/steps/evaluation/config.h>
 #include <rl_tools/rl/loop/steps/timing/config.h>
@@ -78,6 +83,9 @@ constexpr TI TIMING_INTERVAL = 10000;
 #elif defined(ZOO_TD3)
 using LOOP_CORE_CONFIG = rlt::rl::zoo::pendulum_v1::td3::FACTORY<DEVICE, TYPE_POLICY, TI, RNG, DYNAMIC_ALLOCATION>::LOOP_CORE_CONFIG;
 constexpr TI TIMING_INTERVAL = 10000;
+#elif defined(ZOO_ACROBOT_SWINGUP_SAC)
+using LOOP_CORE_CONFIG = rlt::rl::zoo::acrobot_swingup_v0::sac::FACTORY<DEVICE, TYPE_POLICY, TI, RNG, DYNAMIC_ALLOCATION>::LOOP_CORE_CONFIG;
+constexpr TI TIMING_INTERVAL = 100000;
 #else
 using LOOP_CORE_CONFIG = rlt::rl::zoo::pendulum_v1::ppo::FACTORY<DEVICE, TYPE_POLICY, TI, RNG, DYNAMIC_ALLOCATION>::LOOP_CORE_CONFIG;
 constexpr TI TIMING_INTERVAL = 100;

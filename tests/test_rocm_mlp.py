@@ -17,7 +17,8 @@ TOL = 1e-5
 # (batch, in, hidden, out) -- cuda_basics.cu:814-827 plus the benchmark shapes and ragged sizes
 SHAPES = [(1, 1, 1, 1), (1, 256, 10, 100), (2, 256, 10, 100), (32, 256, 10, 100), (1024, 256, 10, 100), (10, 256, 200, 100),
           (9, 256, 60, 100), (200, 256, 11, 100), (64, 256, 50, 101), (256, 256, 256, 256), (256, 4, 64, 1), (256, 3, 64, 2),
-          (300, 17, 256, 6), (4096, 17, 256, 6), (77, 5, 33, 3), (513, 130, 129, 37)]
+          (300, 17, 256, 6), (4096, 17, 256, 6), (77, 5, 33, 3), (513, 130, 129, 37),
+          (250, 70, 200, 5), (100, 6, 256, 1), (1024, 7, 256, 2), (2048, 65, 96, 3), (128, 64, 64, 64)]      # the last rows: grids of a few workgroups, reductions of 64 and more
 
 
 def build_pair(oracle, rocm, shape, seed, hidden_act="relu", out_act="identity"):
