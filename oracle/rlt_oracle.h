@@ -50,6 +50,11 @@
  *   pendulum_evaluate_standardized: identity statistics give pendulum_evaluate's results exactly; other statistics give those of the network with the
  *   statistics folded into its first layer (tests/test_oracle_closed_forms.py). The layer itself, (x - mean) * precision, is the one the PPO loop's
  *   standardize pins cover (ppo_train_minibatch with standardize layers, on_policy_collect).
+ *   env_evaluate: with the Pendulum it reproduces the reference's evaluation vectors bit for bit (the loop shared with pendulum_evaluate); with the Acrobot, whose
+ *   episodes terminate, every episode equals that episode run alone through acrobot_step (pinned against the reference's own step) until its first terminated
+ *   flag, the terminating step's reward counted and nothing after it, and the terminated count and share follow (tests/test_oracle_golden.py). The reference's
+ *   evaluate was not run on an environment that terminates: the bookkeeping after a termination (rl/utils/evaluation/operations_generic.h:166-197) is restated
+ *   from its text and pinned by that per-episode construction only.
  */
 #ifndef RLT_ORACLE_H
 #define RLT_ORACLE_H
