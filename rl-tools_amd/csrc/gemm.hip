@@ -129,17 +129,14 @@ __device__ __forceinline__ void sstore_mncontig(const TileRegs<R, KB>& t, float*
     }
 }
 
-// KB: rows of k per step. 16 with two LDS buffers (the next step's tile is stored while this one is multiplied) when many workgroups share a
-// compute unit and hide each other's memory latency; 64 with one buffer when the whole grid is a few workgroups, each alone on its compute unit
-// and waiting one memory latency per step: a quarter of the steps.
-template <int MODE, int WAVES_M, int WAVES_N, int TM, int TN, int KB = BK>
+template <int MODE, int WAVES_M, int WAVES_N, int TM, int TN>
 __global__ __launch_bounds__(THREADS) void gemm_kernel(GemmParams p) {
     static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per workgroup");
     constexpr int BM = WAVES_M * TM * 32;
     constexpr int BN = WAVES_N * TN * 32;
-    constexpr int NBUF = KB > 32 ? 1 : 2;
-    __shared__ __attribute__((aligned(16))) float sA[NBUF][KB * (BM + PAD)];
-    __shared__ __attribute__((aligned(16))) float sB[NBUF][KB * (BN + PAD)];
+    constexpr int KB = BK;
+    __shared__ __attribute__((aligned(16))) float sA[2][KB * (BM + PAD)];
+    __shared__ __attribute__((aligned(16))) float sB[2][KB * (BN + PAD)];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -178,44 +175,28 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(GemmParams p) {
     if (nk > 0) { gload(ks); sstore(0); }
     __syncthreads();
     for (int t = 0; t < nk; t++) {
-        const int cur = NBUF == 2 ? (t & 1) : 0;
+        const int cur = t & 1;
         if (t + 1 < nk) gload(ks + (t + 1) * KB);
         const float* a_base = sA[cur] + (lane >> 5) * (BM + PAD) + wm * (TM * 32) + (lane & 31);
         const float* b_base = sB[cur] + (lane >> 5) * (BN + PAD) + wn * (TN * 32) + (lane & 31);
-        // CH pairs of k at a time: their LDS reads are all in flight before the first multiply waits for its own (one read, one wait, one multiply in turn
-        // leaves a wavefront that is alone on its SIMD idle for an LDS latency per multiply). Small tiles, which run on few workgroups, take the longest runs.
-        constexpr int CH = TM * TN == 1 ? 8 : (TM * TN == 2 ? 4 : 1);
-        static_assert((KB / 2) % CH == 0);
 #pragma unroll
-        for (int kk0 = 0; kk0 < KB / 2; kk0 += CH) {
-            float a[CH][TM], b[CH][TN];
+        for (int kk = 0; kk < KB / 2; kk++) {
+            float a[TM], b[TN];
 #pragma unroll
-            for (int c = 0; c < CH; c++) {
+            for (int i = 0; i < TM; i++) a[i] = a_base[kk * 2 * (BM + PAD) + i * 32];
 #pragma unroll
-                for (int i = 0; i < TM; i++) a[c][i] = a_base[(kk0 + c) * 2 * (BM + PAD) + i * 32];
+            for (int j = 0; j < TN; j++) b[j] = b_base[kk * 2 * (BN + PAD) + j * 32];
 #pragma unroll
-                for (int j = 0; j < TN; j++) b[c][j] = b_base[(kk0 + c) * 2 * (BN + PAD) + j * 32];
-            }
-            if constexpr (CH > 1) __builtin_amdgcn_sched_barrier(0);      // the instruction scheduler would otherwise move every read back next to its multiply
+            for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int c = 0; c < CH; c++)
-#pragma unroll
-                for (int i = 0; i < TM; i++)
-#pragma unroll
-                    for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[c][i], b[c][j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
         }
         if (bias_block && tid < BM) {
 #pragma unroll
             for (int k = 0; k < KB; k++) bsum += sA[cur][k * (BM + PAD) + tid];
         }
-        if constexpr (NBUF == 2) {
-            if (t + 1 < nk) sstore(cur ^ 1);
-            __syncthreads();
-        } else {
-            __syncthreads();      // every wavefront has read this step's tile
-            if (t + 1 < nk) sstore(0);
-            __syncthreads();
-        }
+        if (t + 1 < nk) sstore(cur ^ 1);
+        __syncthreads();
     }
 
     // ---- epilogue. Accumulator element v of lane l in a 32x32 tile: row = 8*(v/4) + 4*(l/32) + v%4, col = l%32.
@@ -588,8 +569,9 @@ int launch(rlt_rocm_device* device, const GemmParams& p, int splits) {
     int bm, bn;
     tile_dims(shape, bm, bn);
     const dim3 grid(rlt_div_up(p.N, bn), rlt_div_up(p.M, bm), splits);
-    // at most one workgroup per compute unit and a reduction of some length: four times the workgroups on 16x16 tiles per wavefront (gemm_small_kernel)
-    const bool few = (long long)grid.x * grid.y * grid.z <= device->compute_units && p.k_per_split >= 64 && shape != TILE_128x64 && shape != TILE_128x128;
+    // workgroups for at most a quarter of the compute units and a reduction of some length: four times the workgroups on 16x16 tiles per wavefront (gemm_small_kernel);
+    // measured at 4,096 x 146 -> 192 (192 workgroups of 64x64): 13.7 us as it is, 15.5 us on 768 small ones
+    const bool few = 4ll * grid.x * grid.y * grid.z <= device->compute_units && p.k_per_split >= 64 && shape != TILE_128x64 && shape != TILE_128x128;
     if (few) {
         if (p.N <= 16) hipLaunchKernelGGL((gemm_small_kernel<MODE, 4, 1>), dim3(rlt_div_up(p.N, 16), rlt_div_up(p.M, 64), splits), block, 0, device->stream, p);
         else if (p.M <= 16) hipLaunchKernelGGL((gemm_small_kernel<MODE, 1, 4>), dim3(rlt_div_up(p.N, 64), rlt_div_up(p.M, 16), splits), block, 0, device->stream, p);
