@@ -5,6 +5,7 @@
 #include "gemm.h"
 #include "mlp_fused.h"
 #include "mlp_small.h"
+#include "mlp_rows.h"
 
 namespace {
 
@@ -19,6 +20,8 @@ int max_dim(const rlt_dense_layer* layers, int n) {
 size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 // below this batch the single-pass kernels (one 64-row tile per workgroup, plus the weight swizzle) do not pay against the per-layer kernels
 constexpr int FUSED_MIN_BATCH = 1024;
+// a few hundred rows through layers at most 256 wide: all layers in one launch (mlp_rows.hip)
+bool rows_enabled() { return rlt_mlp_rows_enabled(); }
 // RLT_MLP_SINGLE_PASS=0 keeps forward() / backward() on the per-layer kernels (tests compare the two paths with each other)
 bool single_pass_enabled() { const char* v = std::getenv("RLT_MLP_SINGLE_PASS"); return !(v && v[0] == '0'); }
 bool chain_ok(const rlt_dense_layer* layers, int n) {
@@ -94,6 +97,10 @@ int rlt_rocm_mlp_evaluate(rlt_rocm_device* device, const rlt_dense_layer* layers
     RLT_REQUIRE(chain_ok(layers, n) && x && y && batch > 0 && ldx >= layers[0].in_dim && ldy >= layers[n - 1].out_dim);
     const size_t buf = align_up((size_t)batch * max_dim(layers, n) * sizeof(float));
     RLT_REQUIRE(n == 1 || (workspace && workspace_bytes >= 2 * buf));
+    if (n > 1 && batch <= RLT_MLP_ROWS_MAX_BATCH && rows_enabled()) {
+        const int rc = rlt_mlp_rows_forward(device, layers, n, x, ldx, y, ldy, batch, false);
+        if (rc != RLT_E_UNSUPPORTED) return rc;
+    }
     float* tick = (float*)workspace; float* tock = (float*)((char*)workspace + buf);
     const float* in = x; int ldin = ldx;
     for (int l = 0; l < n; l++) {
@@ -110,6 +117,10 @@ int rlt_rocm_mlp_forward(rlt_rocm_device* device, const rlt_dense_layer* layers,
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(chain_ok(layers, n) && x && batch > 0 && ldx >= layers[0].in_dim);
     for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].pre_activations && layers[l].output);
+    if (n > 1 && batch <= RLT_MLP_ROWS_MAX_BATCH && batch < FUSED_MIN_BATCH && rows_enabled()) {
+        const int rc = rlt_mlp_rows_forward(device, layers, n, x, ldx, nullptr, 0, batch, true);
+        if (rc != RLT_E_UNSUPPORTED) return rc;
+    }
     if (batch >= FUSED_MIN_BATCH && single_pass_enabled()) {       // in -> 256 -> 256 -> out: one pass that keeps the hidden activations on chip on their way to the next layer
         const int rc = rlt_mlp3_fused_forward(device, layers, n, x, ldx, batch);
         if (rc != RLT_E_UNSUPPORTED) return rc;

@@ -3,6 +3,7 @@
 // reference: nn_models/sequential/operations_generic.h:277-428.
 #include "common.h"
 #include "gemm.h"
+#include "mlp_rows.h"
 #include <algorithm>
 
 namespace {
@@ -182,6 +183,14 @@ int rlt_rocm_seq_evaluate_step(rlt_rocm_device* device, const rlt_seq_layer* lay
     RLT_REQUIRE(ldx >= layer_in(layers[0]) && ldy >= layer_out(layers[n - 1]));
     for (int l = 1; l < n; l++) RLT_REQUIRE(layer_in(layers[l]) == layer_out(layers[l - 1]));
     RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_seq_evaluate_step_workspace_bytes(layers, n, batch));
+    bool dense_only = true;
+    for (int l = 0; l < n; l++) dense_only = dense_only && layers[l].kind == 0;
+    if (dense_only && n > 1 && batch <= RLT_MLP_ROWS_MAX_BATCH && rlt_mlp_rows_enabled()) {      // a policy without recurrent layers: all layers in one launch
+        rlt_dense_layer dense[RLT_SEQ_MAX_LAYERS];
+        for (int l = 0; l < n; l++) dense[l] = layers[l].dense;
+        const int fused = rlt_mlp_rows_forward(device, dense, n, x, ldx, y, ldy, batch, false);
+        if (fused != RLT_E_UNSUPPORTED) return fused;
+    }
     size_t width = 1;
     for (int l = 0; l < n; l++) width = std::max(width, (size_t)layer_out(layers[l]));
     char* w = reinterpret_cast<char*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);

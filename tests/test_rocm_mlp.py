@@ -4,6 +4,7 @@ Tolerance: 1e-5 relative to the largest magnitude of the reference tensor (fp32 
 states); the reference's own device-parity tests use an absolute 1e-6 on O(1) quantities
 (tests/src/nn/cuda/cuda_basics.cu:629-827), shapes below include theirs (:814-827)."""
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -189,3 +190,34 @@ def test_rejects_bad_arguments(rocm):
     assert lib.rlt_rocm_mlp_forward(h, net.layers, net.n, x.ptr, 4, 0) == -1
     assert lib.rlt_rocm_mlp_evaluate(h, net.layers, net.n, x.ptr, 4, x.ptr, 1, 16, None, 0) == -1   # missing workspace
     assert lib.rlt_rocm_check_status(h) == 0
+
+
+@pytest.mark.parametrize("dims,batch", [([33, 256, 40, 7, 256, 3], 300), ([7, 256, 256, 1], 256), ([6, 256], 17), ([256, 255, 254, 253, 252, 251, 250, 249, 2], 2048),
+                                        ([5, 16, 17, 15, 1], 1)])
+def test_all_layers_in_one_launch_match_the_checker_and_the_per_layer_kernels(oracle, rocm, dims, batch):
+    """Batches of up to 2,048 rows through layers at most 256 wide take one launch for all layers (evaluate, and forward with every layer's pre-activations and
+    outputs kept): networks of one to eight layers, widths that are no multiples of 4 or 16, batches that are no multiple of 16. Against the CPU checker to 1e-5 and
+    against the per-layer kernels (RLT_MLP_ROWS=0; another order of summation) to the same bound."""
+    print("case", dims, batch, flush=True)
+    rng = np.random.default_rng(sum(dims) + batch)
+    params = helpers.random_params(rng, dims)
+    x = rng.standard_normal((batch, dims[0])).astype(np.float32)
+    results = []
+    for backend, rows in ((oracle, None), (rocm, "1"), (rocm, "0")):
+        if rows is not None:
+            os.environ["RLT_MLP_ROWS"] = rows
+        try:
+            net = Mlp(backend, dims, params, batch, "tanh", "identity")
+            xd, yd = backend.array(x), backend.zeros((batch, dims[-1]))
+            ws, wsn = net.workspace()
+            backend.call("mlp_evaluate", net.layers, net.n, xd.ptr, dims[0], yd.ptr, dims[-1], batch, ws, wsn)
+            backend.call("mlp_forward", net.layers, net.n, xd.ptr, dims[0], batch)
+            backend.sync()
+            results.append([yd.numpy()] + [p.numpy() for p in net.pre] + [o.numpy() for o in net.out])
+        finally:
+            os.environ.pop("RLT_MLP_ROWS", None)
+    ref, one_launch, per_layer = results
+    for k in range(len(ref)):
+        assert rel_err(one_launch[k], ref[k]) <= TOL and rel_err(per_layer[k], ref[k]) <= TOL and rel_err(one_launch[k], per_layer[k]) <= TOL, k
+    if batch < 1024:      # from 1,024 rows forward() takes the per-layer or the single-pass kernels
+        assert np.array_equal(one_launch[0], one_launch[-1])      # evaluate and forward: the same kernel, the same bits
