@@ -503,9 +503,9 @@ def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=100
     rng = np.random.default_rng(1)
     out = {}
 
-    def parameters(obs, act):
-        critics = [helpers.random_params(rng, [obs + act, 64, 64, 1]) for _ in range(2)]
-        return np.concatenate([helpers.random_params(rng, [obs, 64, 64, 2 * act])] + critics + critics + [np.array([np.log(0.5)], np.float32)])
+    def parameters(obs, act, hidden=64):
+        critics = [helpers.random_params(rng, [obs + act, hidden, hidden, 1]) for _ in range(2)]
+        return np.concatenate([helpers.random_params(rng, [obs, hidden, hidden, 2 * act])] + critics + critics + [np.array([np.log(0.5)], np.float32)])
 
     agent = helpers.SacOnBackend(rocm, batch, 64, parameters(3, 1), masks=False)
     rb = helpers.ReplayOnBackend(rocm, 1, capacity)
@@ -546,6 +546,16 @@ def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=100
     rocm.sync()
     a = ev.record(); updates(300); b = ev.record()
     out["wide_agent_obs27_act8_update_sets_per_s_by_device_clock"] = 300 / (ev.elapsed_ms(a, b) * 1e-3)
+    # hidden width 256 (the zoo's AcrobotSwingup agent: observation 6, action 1): the per-operation path, about 60 launches per set of updates
+    obs, act = 6, 1
+    wide = helpers.SacOnBackend(rocm, batch, 256, parameters(obs, act, 256), masks=False, obs=obs, act=act)
+    oab = rng.standard_normal((2, batch, obs + act)).astype(np.float32); oab[:, :, obs:] = np.tanh(oab[:, :, obs:])
+    wide.set_batch(oab, rng.standard_normal(batch).astype(np.float32), (rng.random(batch) < 0.05).astype(np.uint8))
+    noise = rocm.array(rng.standard_normal((batch, act)).astype(np.float32))
+    updates(20)
+    rocm.sync()
+    a = ev.record(); updates(300); b = ev.record()
+    out["width256_agent_obs6_act1_update_sets_per_s_by_device_clock"] = 300 / (ev.elapsed_ms(a, b) * 1e-3)
     return out
 
 
