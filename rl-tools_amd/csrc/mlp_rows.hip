@@ -5,9 +5,11 @@
 // memory for the activations per layer (measured at batch 256, widths 256: 6.5 + 10.6 + 10.1 us for the three layers of a critic). Here a workgroup of
 // sixteen wavefronts takes 16 rows through all layers: the activations stay in LDS, wavefront w owns the output columns 16 w ... 16 w + 15 of every layer
 // and reads that tile's rows of W from memory straight into the B operands of v_mfma_f32_16x16x4_f32, all of them at once and a layer ahead: the next
-// layer's weights are requested before this layer's results are written, so their way from memory overlaps the epilogue and the barrier. Operand lane layout of the instruction: lane l = 16 g + c holds A[row c][k g] and B[k g][col c]; the four k of one instruction may be
-// any four as long as both operands agree, so lane group g takes k = 16 j + 4 g + i for the i-th of four consecutive instructions: one 16-byte read per
-// operand per four instructions. Accumulator element v of lane l is C[row 4 g + v][col c].
+// layer's weights are requested before this layer's results are written, so their way from memory overlaps the epilogue and the barrier.
+// Operand lane layout of the instruction: lane l = 16 g + c holds A[row c][k g] and B[k g][col c]; the four k of one instruction may be any four as long as
+// both operands agree, so lane group g takes k = 16 j + 4 g + i for the i-th of four consecutive instructions: one 16-byte read per operand per four
+// instructions. Accumulator element v of lane l is C[row 4 g + v][col c].
+// Two networks of one shape on the same rows (a pair of critics) share a launch: blockIdx.y selects the network.
 #include "mlp_rows.h"
 #include <cstdlib>
 
@@ -17,6 +19,7 @@ namespace {
 constexpr int ROWS = 16, MAX_WIDTH = 256, MAX_LAYERS = 8, STRIDE = MAX_WIDTH + 4, WAVES = MAX_WIDTH / 16;
 struct RowsLayer { const float* W; const float* b; float* pre; float* out; int in_dim, out_dim, act, vec; };
 struct RowsArgs { RowsLayer L[MAX_LAYERS]; int n; const float* x; int ldx; float* y; int ldy; int batch; };
+struct RowsPair { RowsArgs net[2]; };      // blockIdx.y selects the network: two networks of one shape on one batch (SAC's and TD3's pairs of critics) share a launch
 
 // what a lane needs of a layer: its column's row of W as B operands (lane group g: k = 16 j + 4 g ... + 3 of every 16), zero beyond the layer's shape, and its bias
 struct RowsWeights { float4 b[MAX_WIDTH / 16]; float bias; };
@@ -46,7 +49,8 @@ __device__ __forceinline__ void load_weights(const RowsLayer& L, int n, int g, R
     w.bias = n_ok ? L.b[n] : 0.0f;
 }
 
-__global__ __launch_bounds__(WAVES * 64) void mlp_rows_kernel(RowsArgs A) {
+__global__ __launch_bounds__(WAVES * 64) void mlp_rows_kernel(RowsPair P) {
+    const RowsArgs& A = P.net[blockIdx.y];
     __shared__ __attribute__((aligned(16))) float act[2][ROWS * STRIDE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, c = lane & 15;
     const int row0 = blockIdx.x * ROWS;
@@ -105,9 +109,9 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_rows_kernel(RowsArgs A) {
 
 bool rlt_mlp_rows_enabled() { const char* v = std::getenv("RLT_MLP_ROWS"); return !(v && v[0] == '0'); }
 
-int rlt_mlp_rows_forward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy, int batch, bool keep) {
+static int describe_rows(const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy, int batch, bool keep, RowsArgs& a) {
     if (n_layers < 1 || n_layers > MAX_LAYERS || batch < 1 || batch > RLT_MLP_ROWS_MAX_BATCH) return RLT_E_UNSUPPORTED;
-    RowsArgs a = {};
+    a = RowsArgs{};
     for (int l = 0; l < n_layers; l++) {
         const rlt_dense_layer& L = layers[l];
         if (L.in_dim > MAX_WIDTH || L.out_dim > MAX_WIDTH) return RLT_E_UNSUPPORTED;
@@ -115,6 +119,38 @@ int rlt_mlp_rows_forward(rlt_rocm_device* device, const rlt_dense_layer* layers,
         a.L[l] = RowsLayer{L.weights, L.biases, keep ? L.pre_activations : nullptr, keep ? L.output : nullptr, L.in_dim, L.out_dim, L.activation, vec ? 1 : 0};
     }
     a.n = n_layers; a.x = x; a.ldx = ldx; a.y = y; a.ldy = ldy; a.batch = batch;
-    hipLaunchKernelGGL(mlp_rows_kernel, dim3(rlt_div_up(batch, ROWS)), dim3(WAVES * 64), 0, device->stream, a);
+    return 0;
+}
+
+int rlt_mlp_rows_forward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy, int batch, bool keep) {
+    RowsPair p = {};
+    const int rc = describe_rows(layers, n_layers, x, ldx, y, ldy, batch, keep, p.net[0]);
+    if (rc) return rc;
+    hipLaunchKernelGGL(mlp_rows_kernel, dim3(rlt_div_up(batch, ROWS), 1), dim3(WAVES * 64), 0, device->stream, p);
     return rlt_launch_status(device);
+}
+
+int rlt_mlp_rows_forward_pair(rlt_rocm_device* device, const rlt_dense_layer* first, const rlt_dense_layer* second, int n_layers, const float* x, int ldx,
+                              float* y_first, float* y_second, int ldy, int batch, bool keep) {
+    RowsPair p = {};
+    int rc = describe_rows(first, n_layers, x, ldx, y_first, ldy, batch, keep, p.net[0]);
+    if (rc) return rc;
+    if ((rc = describe_rows(second, n_layers, x, ldx, y_second, ldy, batch, keep, p.net[1]))) return rc;
+    hipLaunchKernelGGL(mlp_rows_kernel, dim3(rlt_div_up(batch, ROWS), 2), dim3(WAVES * 64), 0, device->stream, p);
+    return rlt_launch_status(device);
+}
+
+int rlt_mlp_forward_pair(rlt_rocm_device* device, const rlt_dense_layer* first, const rlt_dense_layer* second, int n_layers, const float* x, int ldx, float* y_first,
+                         float* y_second, int ldy, int batch, bool keep, void* ws, size_t ws_bytes) {
+    if (n_layers > 1 && batch < 1024 && rlt_mlp_rows_enabled()) {      // from 1,024 rows forward() has a single-pass kernel of its own
+        const int rc = rlt_mlp_rows_forward_pair(device, first, second, n_layers, x, ldx, y_first, y_second, ldy, batch, keep);
+        if (rc != RLT_E_UNSUPPORTED) return rc;
+    }
+    const rlt_dense_layer* nets[2] = {first, second};
+    float* ys[2] = {y_first, y_second};
+    for (int k = 0; k < 2; k++) {
+        const int rc = keep ? rlt_rocm_mlp_forward(device, nets[k], n_layers, x, ldx, batch) : rlt_rocm_mlp_evaluate(device, nets[k], n_layers, x, ldx, ys[k], ldy, batch, ws, ws_bytes);
+        if (rc) return rc;
+    }
+    return 0;
 }

@@ -5,6 +5,7 @@
 //            random/operations_generic.h:72-105.
 #include "common.h"
 #include "sac_update.h"
+#include "mlp_rows.h"
 #include <algorithm>
 
 namespace {
@@ -254,6 +255,7 @@ int rlt_rocm_sac_set_per_operation(rlt_rocm_device* device, int enabled) {
     return 0;
 }
 
+
 // rl/algorithms/sac/operations_generic.h:243-337: the fused kernels where they fit, else one launch per reference operation
 int rlt_rocm_sac_train_critic(rlt_rocm_device* device, const rlt_sac_agent* A, int ci, const float* action_noise) {
     if (!device) return RLT_E_NOT_INITIALISED;
@@ -275,8 +277,7 @@ int rlt_rocm_sac_train_critic(rlt_rocm_device* device, const rlt_sac_agent* A, i
     if ((rc = rlt_rocm_sas_forward(device, &A->sas, actor_out, 2 * ACT, action_noise, ACT, next_actions, D, nullptr, 0, A->next_log_probabilities, B, ACT))) return rc;
     if (A->next_final_step_mask) if ((rc = rlt_rocm_mask_copy(device, obs_next + OBS, D, next_actions, D, A->next_final_step_mask, 1, B, ACT))) return rc;
     if ((rc = copy2d(device, obs_next, D, A->next_state_action_value_input, D, B, OBS))) return rc;
-    for (int k = 0; k < 2; k++)
-        if ((rc = rlt_rocm_mlp_evaluate(device, A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, A->next_q[k], 1, B, ws, ws_bytes))) return rc;
+    if ((rc = rlt_mlp_forward_pair(device, A->critics_target[0], A->critics_target[1], A->n_critic_layers, A->next_state_action_value_input, D, A->next_q[0], A->next_q[1], 1, B, false, ws, ws_bytes))) return rc;
     if ((rc = rlt_rocm_sac_target_action_values(device, A->next_q[0], A->next_q[1], A->rewards, A->terminated, A->next_log_probabilities, A->log_alpha.parameters,
                                                A->gamma, 0, A->target_action_value, B))) return rc;
     if ((rc = rlt_rocm_mlp_forward(device, critic, A->n_critic_layers, A->observations_actions_base, D, B))) return rc;
@@ -335,8 +336,7 @@ int rlt_rocm_sac_train_actor(rlt_rocm_device* device, const rlt_sac_agent* A, co
     if ((rc = copy2d(device, A->actor_actions, ACT, sav_actions, D, B, ACT))) return rc;
     if (A->final_step_mask) if ((rc = rlt_rocm_mask_copy(device, obs + OBS, D, sav_actions, D, A->final_step_mask, 1, B, ACT))) return rc;
     if ((rc = copy2d(device, obs, D, A->state_action_value_input, D, B, OBS))) return rc;
-    for (int k = 0; k < 2; k++)
-        if ((rc = rlt_rocm_mlp_forward(device, A->critics[k], A->n_critic_layers, A->state_action_value_input, D, B))) return rc;
+    if ((rc = rlt_mlp_forward_pair(device, A->critics[0], A->critics[1], A->n_critic_layers, A->state_action_value_input, D, nullptr, nullptr, 0, B, true, ws, ws_bytes))) return rc;
     hipLaunchKernelGGL(sac_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, (const float*)nullptr, (const float*)nullptr, A->final_step_mask,
                        A->d_output_actor_critics, B, 1);
     if ((rc = rlt_launch_status(device))) return rc;

@@ -4,6 +4,7 @@
 //            rl/algorithms/td3/operations_generic.h:116-325 (CUDA: operations_cuda.h:8-110).
 #include "common.h"
 #include "sac_update.h"
+#include "mlp_rows.h"
 
 namespace {
 
@@ -199,6 +200,7 @@ int rlt_rocm_td3_target_action_values(rlt_rocm_device* device, const float* q1_n
     return rlt_launch_status(device);
 }
 
+
 // rl/algorithms/td3/operations_generic.h:170-235. The elementwise steps between the network passes are folded into two launches.
 int rlt_rocm_td3_train_critic(rlt_rocm_device* device, const rlt_td3_agent* A, int ci, const float* sampling_noise) {
     if (!device) return RLT_E_NOT_INITIALISED;
@@ -221,8 +223,7 @@ int rlt_rocm_td3_train_critic(rlt_rocm_device* device, const rlt_td3_agent* A, i
     hipLaunchKernelGGL(td3_next_input_kernel, dim3(grid1((long)B * D)), dim3(256), 0, device->stream, (const float*)mean, sampling_noise, A->sampling_std,
                        (const float*)A->target_next_action_noise, A->next_final_step_mask, obs_next, A->next_state_action_value_input, B, OBS, ACT);
     if ((rc = rlt_launch_status(device))) return rc;
-    for (int k = 0; k < 2; k++)
-        if ((rc = rlt_rocm_mlp_evaluate(device, A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, A->next_q[k], 1, B, ws, ws_bytes))) return rc;
+    if ((rc = rlt_mlp_forward_pair(device, A->critics_target[0], A->critics_target[1], A->n_critic_layers, A->next_state_action_value_input, D, A->next_q[0], A->next_q[1], 1, B, false, ws, ws_bytes))) return rc;
     if ((rc = rlt_rocm_mlp_forward(device, critic, A->n_critic_layers, A->observations_actions_base, D, B))) return rc;
     float* q = critic[A->n_critic_layers - 1].output;
     hipLaunchKernelGGL(td3_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, q, (const float*)A->next_q[0], (const float*)A->next_q[1], (const float*)A->rewards,
