@@ -181,8 +181,8 @@ def test_zoo_configuration_of_the_acrobot_swingup_trains_on_rocm():
     """The reference's zoo configuration of the AcrobotSwingup (src/rl/zoo/acrobot-swingup-v0/sac.h, included as it is: SAC at batch 256 and width 256 with
     fast_tanh, episodes of 1,000 steps, 50,000 steps of uniform exploration, a replay ring of 1,000,000 rows) inside the evaluation and timing loop steps on
     devices::ROCM: the runner steps the environment through the library's step for any environment, the evaluations (100 episodes x 1,000 steps) run on
-    the device. Here the first 125,000 of its 1,000,000 loop steps; measured over the whole configuration: mean return -37 before training, -23 after 100,000
-    steps, -7 after 500,000, best -5.7, 408 s (2,450 loop steps/s including the 100 evaluations)."""
+    the device. Here the first 125,000 of its 1,000,000 loop steps; measured over the whole configuration: mean return -37 before training, -22 after 100,000
+    steps, -7 after 500,000, best -5.5, 359 s (2,780 loop steps/s including the 100 evaluations)."""
     path = os.path.join(BUILD, "rocm_zoo_acrobot_swingup_v0_sac")
     if not os.path.exists(path):
         pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
