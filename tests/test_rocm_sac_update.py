@@ -3,6 +3,7 @@ critics obs + act -> 64 -> 64 -> 1 of any width: against the CPU checker's train
 (rl/algorithms/sac/operations_generic.h:243-337, 395-468, 488-527) and against the library's own one-launch-per-operation path, from
 identical parameters, batches and noise. Tolerance: 1e-5 relative to each tensor's largest magnitude (fp32, different summation orders)."""
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -15,11 +16,11 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-5
 
 
-def agent_parameters(rng, obs, act):
+def agent_parameters(rng, obs, act, hidden=64):
     d = obs + act
-    critics = [helpers.random_params(rng, [d, 64, 64, 1]) for _ in range(2)]
+    critics = [helpers.random_params(rng, [d, hidden, hidden, 1]) for _ in range(2)]
     targets = [c + rng.uniform(-0.01, 0.01, c.size).astype(np.float32) for c in critics]
-    return np.concatenate([helpers.random_params(rng, [obs, 64, 64, 2 * act])] + critics + targets + [np.array([np.log(0.5)], np.float32)])
+    return np.concatenate([helpers.random_params(rng, [obs, hidden, hidden, 2 * act])] + critics + targets + [np.array([np.log(0.5)], np.float32)])
 
 
 def batch_of(rng, batch, obs, act):
@@ -55,9 +56,9 @@ def run_updates(agent, batches, noises):
     return snapshot(agent)
 
 
-def make_inputs(seed, batch, obs, act, steps):
+def make_inputs(seed, batch, obs, act, steps, hidden=64):
     rng = np.random.default_rng(seed)
-    params = agent_parameters(rng, obs, act)
+    params = agent_parameters(rng, obs, act, hidden)
     batches, noises = [], []
     for _ in range(steps):
         three = [batch_of(rng, batch, obs, act) for _ in range(3)]
@@ -101,6 +102,30 @@ def test_fused_updates_match_the_checker_and_the_per_operation_path(oracle, rocm
     # the update did something: three Adam steps moved every network
     moved = np.abs(results["fused"]["parameters"] - params)
     assert moved.max() > 1e-4 and results["fused"]["ages"].tolist() == [1 + steps] * 4
+
+
+@pytest.mark.parametrize("batch,obs,act,hidden,hidden_act", [(256, 6, 1, 256, "fast_tanh"), (100, 17, 6, 128, "relu"), (48, 3, 1, 200, "relu")])
+def test_wider_agents_on_the_per_operation_kernels_match_the_checker(oracle, rocm, batch, obs, act, hidden, hidden_act):
+    """Hidden widths other than 64 (the zoo's AcrobotSwingup agent: 6-256-256-2 and 7-256-256-1 at batch 256): every forward pass is one launch of the few-rows
+    kernel (pairs of critics share one), the backward contractions run a wavefront per 16x16 tile. Three loop steps' worth of updates against the CPU checker, and
+    against the same updates with one launch per layer (RLT_MLP_ROWS=0)."""
+    steps = 3
+    params, batches, noises = make_inputs(batch * 7 + hidden, batch, obs, act, steps, hidden)
+    results = {}
+    for name, backend, rows in (("checker", oracle, None), ("one_launch", rocm, "1"), ("per_layer", rocm, "0")):
+        if rows is not None:
+            os.environ["RLT_MLP_ROWS"] = rows
+        try:
+            agent = helpers.SacOnBackend(backend, batch, hidden, params, masks=False, obs=obs, act=act, hidden_act=hidden_act)
+            results[name] = run_updates(agent, batches, noises)
+        finally:
+            os.environ.pop("RLT_MLP_ROWS", None)
+    for other in ("checker", "per_layer"):
+        for key, ref in results[other].items():
+            err = rel_err(results["one_launch"][key], ref)
+            assert err <= TOL, (other, key, err)
+    moved = np.abs(results["one_launch"]["parameters"] - params)
+    assert moved.max() > 1e-4 and results["one_launch"]["ages"].tolist() == [1 + steps] * 4
 
 
 def test_agents_outside_the_fused_shapes_take_the_per_operation_path(oracle, rocm):
