@@ -35,6 +35,18 @@ __global__ __launch_bounds__(256) void zero_kernel(float* __restrict__ a, size_t
         if (i < na) a[i] = 0.0f; else b[i - na] = 0.0f;
     }
 }
+// up to 16 separate runs of floats cleared by one launch (a network whose gradient tensors are allocations of their own, as the reference's containers are)
+constexpr int ZERO_RUNS = 16;
+struct ZeroRuns { float* begin[ZERO_RUNS]; size_t prefix[ZERO_RUNS + 1]; int n; };
+__global__ __launch_bounds__(256) void zero_runs_kernel(ZeroRuns z) {
+    const size_t total = z.prefix[z.n];
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        int r = 0;
+#pragma unroll
+        for (int k = 1; k < ZERO_RUNS; k++) r += (k < z.n && i >= z.prefix[k]) ? 1 : 0;
+        z.begin[r][i - z.prefix[r]] = 0.0f;
+    }
+}
 // d = (y - target) * scale  (nn/loss_functions/mse/operations_generic.h:41-56 with scale = 2/(rows*cols)*w)
 __global__ __launch_bounds__(256) void mse_d_kernel(const float* __restrict__ y, int ldy, const float* __restrict__ t, int ldt, float* __restrict__ d, int ldd,
                                                     int rows, int cols, float scale) {
@@ -192,30 +204,30 @@ int rlt_rocm_mlp_zero_gradient(rlt_rocm_device* device, const rlt_dense_layer* l
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(layers && n >= 1);
     for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases && layers[l].in_dim > 0 && layers[l].out_dim > 0);
-    // gradient tensors laid out back to back ([dW0 | db0 | dW1 | db1 | ...], the flat arena) are cleared by one launch, a run of layers at a time
-    for (int l = 0; l < n;) {
-        float* begin = layers[l].d_weights; float* end = begin;
-        int m = l;
-        for (; m < n; m++) {
-            const size_t nw = (size_t)layers[m].in_dim * layers[m].out_dim, nb = layers[m].out_dim;
-            if (layers[m].d_weights != end || layers[m].d_biases != end + nw) break;
-            end += nw + nb;
-        }
-        if (m == l) {       // this layer's two tensors lie apart
-            const size_t nw = (size_t)layers[l].in_dim * layers[l].out_dim, nb = layers[l].out_dim;
-            int blocks = (int)((nw + nb + 255) / 256); if (blocks > 1024) blocks = 1024;
-            hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, device->stream, layers[l].d_weights, nw, layers[l].d_biases, nb);
-            m = l + 1;
-        } else {
-            const size_t count = (size_t)(end - begin);
-            int blocks = (int)((count + 255) / 256); if (blocks > 1024) blocks = 1024;
-            hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, device->stream, begin, count, begin, (size_t)0);
-        }
-        const int rc = rlt_launch_status(device);
+    // gradient tensors laid out back to back ([dW0 | db0 | dW1 | db1 | ...], the flat arena) form one run; tensors that are allocations of their own a run each;
+    // up to 16 runs per launch
+    ZeroRuns z = {};
+    auto flush = [&]() -> int {
+        if (z.n == 0) return 0;
+        const size_t total = z.prefix[z.n];
+        int blocks = (int)((total + 255) / 256); if (blocks > 1024) blocks = 1024;
+        if (z.n == 1) hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, device->stream, z.begin[0], total, z.begin[0], (size_t)0);
+        else hipLaunchKernelGGL(zero_runs_kernel, dim3(blocks), dim3(256), 0, device->stream, z);
+        z = ZeroRuns{};
+        return rlt_launch_status(device);
+    };
+    auto add = [&](float* begin, size_t count) -> int {
+        if (z.n > 0 && z.begin[z.n - 1] + (z.prefix[z.n] - z.prefix[z.n - 1]) == begin) { z.prefix[z.n] += count; return 0; }      // continues the last run
+        if (z.n == ZERO_RUNS) { const int rc = flush(); if (rc) return rc; }
+        z.begin[z.n] = begin; z.prefix[z.n + 1] = z.prefix[z.n] + count; z.n++;
+        return 0;
+    };
+    for (int l = 0; l < n; l++) {
+        int rc = add(layers[l].d_weights, (size_t)layers[l].in_dim * layers[l].out_dim);
         if (rc) return rc;
-        l = m;
+        if ((rc = add(layers[l].d_biases, (size_t)layers[l].out_dim))) return rc;
     }
-    return 0;
+    return flush();
 }
 
 }  // extern "C"

@@ -221,3 +221,33 @@ def test_all_layers_in_one_launch_match_the_checker_and_the_per_layer_kernels(or
         assert rel_err(one_launch[k], ref[k]) <= TOL and rel_err(per_layer[k], ref[k]) <= TOL and rel_err(one_launch[k], per_layer[k]) <= TOL, k
     if batch < 1024:      # from 1,024 rows forward() takes the per-layer or the single-pass kernels
         assert np.array_equal(one_launch[0], one_launch[-1])      # evaluate and forward: the same kernel, the same bits
+
+
+@pytest.mark.parametrize("n_layers", [1, 3, 10])
+def test_zero_gradient_of_tensors_that_lie_apart(rocm, n_layers):
+    """Gradient tensors that are allocations of their own (as the reference's containers are), here ranges of one buffer with gaps between them: cleared by
+    one launch per 16 runs, nothing outside them touched; two tensors that happen to lie back to back count as one run."""
+    rng = np.random.default_rng(n_layers)
+    dims = [int(d) for d in rng.integers(1, 40, n_layers + 1)]
+    sizes = []
+    for l in range(n_layers):
+        sizes += [dims[l] * dims[l + 1], dims[l + 1]]
+    gaps = [int(g) for g in rng.integers(0, 9, len(sizes) + 1)]      # a gap of zero makes two tensors adjacent
+    total = sum(sizes) + sum(gaps)
+    buffer = rocm.array(np.full(total, 7.0, np.float32))
+    params = rocm.array(np.ones(sum(sizes), np.float32))
+    layers = (capi.DenseLayer * n_layers)()
+    offsets, at, p_at = [], gaps[0], 0
+    for k, size in enumerate(sizes):
+        offsets.append((at, size)); at += size + gaps[k + 1]
+    for l in range(n_layers):
+        L = layers[l]
+        L.in_dim, L.out_dim, L.activation = dims[l], dims[l + 1], capi.ACT["relu"]
+        L.weights, L.biases = params.offset(p_at), params.offset(p_at + sizes[2 * l]); p_at += sizes[2 * l] + sizes[2 * l + 1]
+        L.d_weights, L.d_biases = buffer.offset(offsets[2 * l][0]), buffer.offset(offsets[2 * l + 1][0])
+    rocm.call("mlp_zero_gradient", layers, n_layers)
+    rocm.sync()
+    want = np.full(total, 7.0, np.float32)
+    for at, size in offsets:
+        want[at:at + size] = 0.0
+    assert np.array_equal(buffer.numpy(), want)
