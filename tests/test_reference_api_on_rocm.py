@@ -162,7 +162,7 @@ def test_zoo_configurations_of_the_pendulum_train_on_rocm(algorithm, best_at_lea
     """The reference's zoo configurations (src/rl/zoo/pendulum-v1/{sac,td3,ppo}.h, included as they are: batch 100 and width 64 for SAC and TD3,
     width 32 with fast_tanh, observation normalisation and an entropy bonus for PPO) inside its evaluation and timing loop steps on devices::ROCM,
     to their own step limits (20,000 loop steps; 1,221 PPO iterations = 10 M environment steps) with 100 evaluations of 100 episodes on the device.
-    A random actor's mean return is about -1,300; measured best returns -125 (SAC, 1.6 s), -129 (TD3, 2.1 s), -158 (PPO, 1.1 s)."""
+    A random actor's mean return is about -1,300; measured best returns -125 (SAC, 1.6 s), -129 (TD3, 1.8 s), -158 (PPO, 1.1 s)."""
     path = os.path.join(BUILD, "rocm_zoo_pendulum_v1_" + algorithm)
     if not os.path.exists(path):
         pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
@@ -220,7 +220,7 @@ def test_recurrent_sac_loop_trains_on_rocm():
     and sequence batches of 16 steps x 32 samples from four environments, on devices::ROCM: gather_batch's multi-step branch with its draws made on the
     device, the runner step with the policy state reset by the truncation mask and evaluate_step, train_critic / train_actor as the reference's generic
     code over the GRU, dense, sample_and_squash and tensor overloads, the evaluation loop step with the recurrent actor on the device. A random actor's mean
-    return is about -1,300; measured -280 after 3,000 loop steps and -150 after 9,000, at 1,030 loop steps/s including the evaluations (the same program on
+    return is about -1,300; measured -280 after 3,000 loop steps and -150 after 9,000, at 1,130 loop steps/s including the evaluations (the same program on
     the reference's CPU device: 190)."""
     path = os.path.join(BUILD, "rocm_sac_gru_pendulum")
     if not os.path.exists(path):
