@@ -520,15 +520,22 @@ def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=100
         rocm.device.check(lib.rlt_rocm_pendulum_runner_step(h, C.byref(runner), C.byref(rb.c), 0, agent.actor.layers, 3, C.byref(agent.c.sas), warm_action.ptr, None, None, seed, 8 * c + 1))
     scratch = capi.SacLoopScratch(rollout_noise.ptr, noise_c.ptr, noise_a.ptr, env_idx.ptr, offs.ptr)
     ev = HipEvents(lib.rlt_rocm_get_stream(h))
-    rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), warmup, seed, 1 << 20, C.byref(scratch))
-    rocm.sync()
-    t0 = time.perf_counter(); a = ev.record()
-    rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), steps, seed, (1 << 20) + warmup, C.byref(scratch))
-    b = ev.record()
-    device_s = ev.elapsed_ms(a, b) * 1e-3       # waits for the second event
-    wall_s = time.perf_counter() - t0
+    # how the update kernels finish and where their workgroups run (rlt_rocm_set_update_options); the library's default comes last and is the figure reported
+    variants = {}
+    offset = 1 << 20
+    for name, tail, one_xcd in (("optimiser_as_own_launch", 0, 1), ("optimiser_in_kernel_spread_over_xcds", 1, 0), ("optimiser_in_kernel_one_xcd", 1, 1)):
+        rocm.call("set_update_options", tail, one_xcd)
+        rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), warmup, seed, offset, C.byref(scratch))
+        rocm.sync()
+        t0 = time.perf_counter(); a = ev.record()
+        rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), steps, seed, offset + warmup, C.byref(scratch))
+        b = ev.record()
+        device_s = ev.elapsed_ms(a, b) * 1e-3       # waits for the second event
+        wall_s = time.perf_counter() - t0
+        offset += warmup + steps
+        variants[name] = {"steps_per_s": steps / wall_s, "steps_per_s_by_device_clock": steps / device_s, "launches_per_step": 4 if tail else 7}
     assert np.all(np.isfinite(agent.parameters())), "SAC parameters went non-finite"
-    out.update(steps_per_s=steps / wall_s, steps_per_s_by_device_clock=steps / device_s, steps=steps, launches_per_step=13)
+    out.update(steps_per_s=steps / wall_s, steps_per_s_by_device_clock=steps / device_s, steps=steps, launches_per_step=4, variants=variants)
     # a wider agent: the update calls alone
     obs, act = 27, 8
     wide = helpers.SacOnBackend(rocm, batch, 64, parameters(obs, act), masks=False, obs=obs, act=act)
@@ -538,9 +545,7 @@ def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=100
 
     def updates(n):
         for _ in range(n):
-            for k in range(2):
-                rocm.device.check(lib.rlt_rocm_sac_train_critic(h, C.byref(wide.c), k, noise.ptr))
-            rocm.device.check(lib.rlt_rocm_sac_update_critic_targets(h, C.byref(wide.c)))
+            rocm.device.check(lib.rlt_rocm_sac_train_critics(h, C.byref(wide.c), noise.ptr, 1))
             rocm.device.check(lib.rlt_rocm_sac_train_actor(h, C.byref(wide.c), noise.ptr))
     updates(20)
     rocm.sync()

@@ -646,13 +646,45 @@ typedef struct rlt_sac_loop_scratch {
     uint32_t* env_indices;      /* [batch] */
     uint32_t* sample_offsets;   /* [batch] */
 } rlt_sac_loop_scratch;
+/* The draws of a loop step made by the kernels that consume them instead of by launches before them. Each call leaves exactly what the
+ * named sequence of calls leaves, bit for bit, and echoes what it drew into the arrays those calls would have filled (the arrays may be
+ * NULL where the fused kernels serve the call; they are required where the call falls back to one launch per operation).
+ *   rlt_rocm_pendulum_runner_step_drawn  = rlt_rocm_randn_f32(drawn_noise, n_envs, seed, noise_stream), then rlt_rocm_pendulum_runner_step
+ *                                          with policy_kind 2, that noise, initial_states NULL and (seed, initial_state_stream)
+ *   rlt_rocm_gather_batch_drawn          = rlt_rocm_gather_draw(seed, stream) into the two index arrays, then rlt_rocm_gather_batch on them
+ *   rlt_rocm_sac_train_critics           = rlt_rocm_sac_train_critic for critic 0, then for critic 1, on the agent's batch with the same
+ *                                          noise (the loop's SHARED_BATCH case, rl/algorithms/sac/loop/core/operations_generic.h:127-138: the
+ *                                          two updates do not depend on each other), then, if update_targets, rlt_rocm_sac_update_critic_targets;
+ *                                          one launch where the fused update kernel fits the agent
+ *   rlt_rocm_sac_train_critics_drawn     = rlt_rocm_randn_f32(drawn_noise, batch x action_dim, seed, stream), then rlt_rocm_sac_train_critics
+ *   rlt_rocm_sac_train_actor_drawn       = the same draw, then rlt_rocm_sac_train_actor */
+int rlt_rocm_pendulum_runner_step_drawn(rlt_rocm_device* device, const rlt_pendulum_runner* runner, const rlt_replay_buffer* rb,
+                                        const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas, float* drawn_noise,
+                                        uint64_t seed, uint64_t noise_stream, uint64_t initial_state_stream);
+int rlt_rocm_gather_batch_drawn(rlt_rocm_device* device, const rlt_replay_buffer* rb, uint64_t seed, uint64_t stream,
+                                uint32_t* drawn_env_indices, uint32_t* drawn_sample_offsets, int max_episode_length, int batch,
+                                float* observations_actions_base, float* rewards, uint8_t* terminated,
+                                uint8_t* reset, uint8_t* next_reset_base, uint8_t* final_step_mask, uint8_t* next_final_step_mask_base);
+int rlt_rocm_sac_train_critics(rlt_rocm_device* device, const rlt_sac_agent* agent, const float* action_noise, int update_targets);
+int rlt_rocm_sac_train_critics_drawn(rlt_rocm_device* device, const rlt_sac_agent* agent, float* drawn_noise, uint64_t seed, uint64_t stream,
+                                     int update_targets);
+int rlt_rocm_sac_train_actor_drawn(rlt_rocm_device* device, const rlt_sac_agent* agent, float* drawn_noise, uint64_t seed, uint64_t stream);
+
+/* How the fused update kernels (SAC / TD3 / PPO minibatch, networks in -> 64 -> 64 -> out) finish. optimiser_in_kernel != 0 (default):
+ * the last workgroup of the launch to finish adds up the workgroups' partial gradients in a fixed order and applies the optimiser's
+ * step, so an update is one launch; 0: the optimiser runs as a launch of its own after the kernel (same bits). one_xcd != 0 (default):
+ * grids of at most 32 workgroups are placed on one XCD, whose L2 then serves the exchange; 0: spread over all XCDs. The environment
+ * variables RLT_UPDATE_TAIL=0 and RLT_UPDATE_PLACEMENT=spread set the defaults of a process. No counterpart in the reference. */
+int rlt_rocm_set_update_options(rlt_rocm_device* device, int optimiser_in_kernel, int one_xcd);
+
 /* The same n_steps iterations of sac::loop::core::step (rl/algorithms/sac/loop/core/operations_generic.h:110-155 past the warm-up,
  * SHARED_BATCH: runner step with the actor, one gather_batch and one critic noise draw for both train_critic calls,
  * update_critic_targets, actor noise draw, train_actor on the same batch) as a host loop over this library's own entry points, for
- * agents and runners of any size that rlt_rocm_sac_pendulum_loop does not cover: 16 launches per step where the fused updates fit
- * (see rlt_rocm_sac_train_critic). Nothing synchronises with the host. Loop step g = step_offset + i draws from the Philox
+ * agents and runners of any size that rlt_rocm_sac_pendulum_loop does not cover: four launches per step where the fused kernels fit
+ * (rlt_rocm_pendulum_runner_step_drawn, rlt_rocm_gather_batch_drawn, rlt_rocm_sac_train_critics_drawn with the target update,
+ * rlt_rocm_sac_train_actor_drawn). Nothing synchronises with the host. Loop step g = step_offset + i draws from the Philox
  * sequences (seed, 8 g + k): k = 1 rollout noise, 2 initial states of episodes that reset, 3 batch indices, 4 critic noise,
- * 5 actor noise. */
+ * 5 actor noise; the scratch arrays receive the draws of the last step. */
 int rlt_rocm_sac_pendulum_loop_by_calls(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_pendulum_runner* runner,
                                         const rlt_replay_buffer* rb, int n_steps, uint64_t seed, uint64_t step_offset,
                                         const rlt_sac_loop_scratch* scratch);

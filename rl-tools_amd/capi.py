@@ -362,6 +362,12 @@ ROCM_ONLY = {
     "sac_pendulum_loop": ([P, C.POINTER(SacAgent), C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, U64, U64, C.POINTER(SacLoopInputs),
                            C.POINTER(SacLoopOutputs)], I),
     "pendulum_runner_step": ([P, C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), I, LP, I, C.POINTER(SasParameters), P, P, P, U64, U64], I),
+    "pendulum_runner_step_drawn": ([P, C.POINTER(PendulumRunner), C.POINTER(ReplayBuffer), LP, I, C.POINTER(SasParameters), P, U64, U64, U64], I),
+    "gather_batch_drawn": ([P, C.POINTER(ReplayBuffer), U64, U64, P, P, I, I, P, P, P, P, P, P, P], I),
+    "sac_train_critics": ([P, C.POINTER(SacAgent), P, I], I),
+    "sac_train_critics_drawn": ([P, C.POINTER(SacAgent), P, U64, U64, I], I),
+    "sac_train_actor_drawn": ([P, C.POINTER(SacAgent), P, U64, U64], I),
+    "set_update_options": ([P, I, I], I),
 }
 
 

@@ -22,6 +22,8 @@ struct rlt_rocm_device {
     int xcd_stride;              // workgroups b and b + xcd_stride run on the same XCD (0: not established; consecutive workgroups go round the XCDs)
     int sticky_error;
     int sac_per_operation;       // rlt_rocm_sac_train_critic / _actor run one launch per reference operation even where the fused kernels fit
+    int update_tail;             // the fused update kernels step the optimiser themselves (their last workgroup), instead of in launches after them
+    int update_one_xcd;          // small grids of the fused update kernels are placed on one XCD
 };
 
 #define RLT_HIP(expr)                                                        \

@@ -2,6 +2,7 @@
 // (reference: devices/cuda.h:130-174, containers/matrix/operations_cuda.h:16-218, containers/tensor/operations_cuda.h:15-624).
 #include "common.h"
 #include "rng.h"
+#include <cstdlib>
 #include "gemm.h"
 #include <cstdio>
 #include <cstring>
@@ -153,7 +154,17 @@ int rlt_rocm_init(int hip_device_index, rlt_rocm_device** out_device) {
         const int rc = rlt_gemm_static_scratch_setup(device);
         if (rc) { (void)hipFree(device->counters); (void)hipStreamDestroy(device->own_stream); delete device; return rc; }
     }
+    {   // defaults of rlt_rocm_set_update_options; RLT_UPDATE_TAIL=0 / RLT_UPDATE_PLACEMENT=spread switch them off for a whole process
+        const char* t = std::getenv("RLT_UPDATE_TAIL"); const char* q = std::getenv("RLT_UPDATE_PLACEMENT");
+        device->update_tail = !(t && std::strcmp(t, "0") == 0);
+        device->update_one_xcd = !(q && std::strcmp(q, "spread") == 0);
+    }
     *out_device = device;
+    return 0;
+}
+int rlt_rocm_set_update_options(rlt_rocm_device* device, int optimiser_in_kernel, int one_xcd) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    device->update_tail = optimiser_in_kernel != 0; device->update_one_xcd = one_xcd != 0;
     return 0;
 }
 int rlt_rocm_destroy(rlt_rocm_device* device) {

@@ -54,8 +54,8 @@ __device__ __forceinline__ float sum_of_blocks(const float* __restrict__ p, int 
 __device__ __forceinline__ void adam_body(const AdamLaunch& a, uint32_t block, uint32_t n_blocks) {
     const uint32_t age = *a.age;
     // bias corrections from the un-incremented age (adam/operations_generic.h:49-58)
-    const float bc1 = 1.0f / (1.0f - powf(a.p.beta_1, (float)age));
-    const float bc2 = 1.0f / (1.0f - powf(a.p.beta_2, (float)age));
+    float bc1, bc2;
+    rlt_adam_bias_corrections(a.p, age, bc1, bc2);
     const uint32_t total = a.prefix[a.n];
     float sq = 0.0f;
     for (uint32_t i = block * blockDim.x + threadIdx.x; i < total; i += n_blocks * blockDim.x) {
@@ -70,18 +70,7 @@ __device__ __forceinline__ void adam_body(const AdamLaunch& a, uint32_t block, u
             T.gradient[j] = g;
         } else g = T.gradient[j];
         sq += g * g;
-        if (a.p.enable_gradient_clipping) g = fminf(fmaxf(g, -a.p.gradient_clip_value), a.p.gradient_clip_value);
-        float m = a.p.beta_1 * T.first_moment[j] + (1.0f - a.p.beta_1) * g;
-        float v = a.p.beta_2 * T.second_moment[j] + (1.0f - a.p.beta_2) * g * g;
-        T.first_moment[j] = m; T.second_moment[j] = v;
-        float pre_sqrt = fmaxf(v * bc2, a.p.epsilon_sqrt);
-        float update = a.p.alpha * bc1 * m / (sqrtf(pre_sqrt) + a.p.epsilon);
-        float param = T.parameters[j];
-        if ((T.flags & 2u) && a.p.enable_bias_lr_factor) update *= a.p.bias_lr_factor;
-        if ((T.flags & 1u) && a.p.enable_weight_decay) update += param * a.p.weight_decay / 2.0f;
-        param -= update;
-        T.parameters[j] = param;
-        if (T.polyak_target) T.polyak_target[j] = a.polyak * T.polyak_target[j] + (1.0f - a.polyak) * param;
+        rlt_adam_apply(a.p, T, j, g, bc1, bc2, a.polyak);
     }
     // gradient norm + age increment: the last workgroup to finish has seen every other one read `age`
     __shared__ float partial[4];
@@ -130,7 +119,7 @@ __global__ __launch_bounds__(256) void adam_reset_kernel(AdamLaunch a) {
 __global__ __launch_bounds__(256) void polyak_kernel(const float* __restrict__ source, float* __restrict__ target, size_t count, float polyak, int squared) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) {
         float s = source[i];
-        target[i] = squared ? polyak * target[i] + (1.0f - polyak) * s * s : polyak * target[i] + (1.0f - polyak) * s;
+        target[i] = squared ? polyak * target[i] + (1.0f - polyak) * s * s : rlt_polyak_value(polyak, target[i], s);
     }
 }
 

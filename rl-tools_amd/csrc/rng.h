@@ -44,3 +44,16 @@ RLT_RNG_FN float rlt_u01(uint32_t x) { return ((float)(x >> 8) + 0.5f) * (1.0f /
 
 // a uniform integer in [0, n) from 32 random bits (multiply-shift; bias below n / 2^32)
 RLT_RNG_FN uint32_t rlt_uniform_below(uint32_t x, uint32_t n) { return (uint32_t)(((uint64_t)x * (uint64_t)n) >> 32); }
+
+#ifndef RLT_RNG_HOST
+// Element i of a standard-normal stream as rlt_rocm_randn_f32 lays it out: word i % 4 of group i / 4, Box-Muller on the word pairs
+// (0, 1) and (2, 3) -- for kernels that take their noise from the stream directly instead of from an array filled beforehand.
+__device__ __forceinline__ float rlt_randn_element(uint64_t seed, uint64_t stream, uint64_t i) {
+    const rlt_u32x4 r = rlt_philox(seed, stream, i >> 2);
+    const bool second = (i & 2) != 0;
+    const float radius = sqrtf(-2.0f * logf(rlt_u01(second ? r.z : r.x)));
+    float s, c;
+    sincosf(6.283185307179586f * rlt_u01(second ? r.w : r.y), &s, &c);
+    return (i & 1) ? radius * s : radius * c;
+}
+#endif

@@ -69,12 +69,22 @@ __global__ __launch_bounds__(256) void replay_add_kernel(rlt_replay_buffer rb, c
 __global__ __launch_bounds__(256) void gather_kernel(rlt_replay_buffer rb, const uint32_t* __restrict__ env_indices, const uint32_t* __restrict__ sample_offsets,
                                                      int deterministic, int max_episode_length, int batch, float* __restrict__ oab, float* __restrict__ rewards,
                                                      uint8_t* __restrict__ terminated, uint8_t* __restrict__ reset, uint8_t* __restrict__ next_reset_base,
-                                                     uint8_t* __restrict__ final_step_mask, uint8_t* __restrict__ next_final_step_mask_base, int* __restrict__ error_flag) {
+                                                     uint8_t* __restrict__ final_step_mask, uint8_t* __restrict__ next_final_step_mask_base, int* __restrict__ error_flag,
+                                                     int draw, uint64_t seed, uint64_t stream, uint32_t* __restrict__ drawn_env_indices, uint32_t* __restrict__ drawn_sample_offsets) {
     const int OBS = rb.observation_dim, ACT = rb.action_dim, R = 2 * OBS + ACT + 3, D = OBS + ACT;
     const int sub = threadIdx.x & 15;
     for (int i = (blockIdx.x * blockDim.x + threadIdx.x) >> 4; i < batch; i += (gridDim.x * blockDim.x) >> 4) {
-        uint32_t e = deterministic ? 0u : env_indices[i];
-        uint32_t offset = deterministic ? (uint32_t)i : sample_offsets[i];
+        uint32_t e, offset;
+        if (draw) {      // what gather_draw_kernel would have put into the arrays: words 0 and 1 of group i of the call's stream (all 16 lanes compute it)
+            const rlt_u32x4 words = rlt_philox(seed, stream, (uint64_t)i);
+            e = rlt_uniform_below(words.x, (uint32_t)rb.n_envs);
+            const uint32_t eligible = rb.full[e] ? (uint32_t)rb.capacity : rb.position[e];
+            offset = eligible ? (uint32_t)(((uint64_t)words.y * eligible) >> 32) : 0u;
+            if (sub == 0) { if (drawn_env_indices) drawn_env_indices[i] = e; if (drawn_sample_offsets) drawn_sample_offsets[i] = offset; }
+        } else {
+            e = deterministic ? 0u : env_indices[i];
+            offset = deterministic ? (uint32_t)i : sample_offsets[i];
+        }
         if (e >= (uint32_t)rb.n_envs) { if (sub == 0) *error_flag = 1; continue; }
         uint32_t index = rb.full[e] ? (rb.position[e] + (uint32_t)max_episode_length + offset) % (uint32_t)rb.capacity : offset;
         if (index >= (uint32_t)rb.capacity) { if (sub == 0) *error_flag = 1; continue; }
@@ -289,6 +299,7 @@ struct FusedRunnerArgs {
     rlt_sas_parameters sas;
     const float* action_noise; const float* initial_states;
     uint64_t seed, stream;
+    uint64_t noise_stream; float* drawn_noise;      // action_noise == NULL: element e of the standard-normal stream (seed, noise_stream), also written to drawn_noise if given
 };
 
 template <int ACT_H>      // hidden activation, a compile-time constant: it sits inside the unrolled matrix-instruction loops
@@ -322,7 +333,10 @@ __global__ __launch_bounds__(64 * FWAVES) void runner_fused_kernel(FusedRunnerAr
             const float2 st = reinterpret_cast<const float2*>(A.rn.states)[e];
             th = st.x; thd = st.y; ep_step = A.rn.episode_step[e]; ep_ret = A.rn.episode_return[e];
             pos = A.rb.position[e]; ces = A.rb.current_episode_start[e]; full = A.rb.full[e];
-            if (A.policy_kind == 2) noise = A.action_noise[e];
+            if (A.policy_kind == 2) {
+                noise = A.action_noise ? A.action_noise[e] : rlt_randn_element(A.seed, A.noise_stream, (uint64_t)e);
+                if (A.drawn_noise) A.drawn_noise[e] = noise;
+            }
             if (A.rn.truncated[e]) {    // prologue (operations_generic_per_env.h:8-66): reset, flag the previous replay row
                 if (A.initial_states) { const float2 ini = reinterpret_cast<const float2*>(A.initial_states)[e]; th = ini.x; thd = ini.y; }
                 else {
@@ -693,7 +707,21 @@ int rlt_rocm_gather_batch(rlt_rocm_device* device, const rlt_replay_buffer* rb, 
     int* error_flag = (int*)(device->fault + 1);        // read back by rlt_rocm_check_status
     device->fault_armed = 1;
     hipLaunchKernelGGL(gather_kernel, dim3(grid1(batch * 16)), dim3(256), 0, device->stream, *rb, env_indices, sample_offsets, deterministic, max_episode_length, batch,
-                       observations_actions_base, rewards, terminated, reset, next_reset_base, final_step_mask, next_final_step_mask_base, error_flag);
+                       observations_actions_base, rewards, terminated, reset, next_reset_base, final_step_mask, next_final_step_mask_base, error_flag, 0, (uint64_t)0, (uint64_t)0,
+                       (uint32_t*)nullptr, (uint32_t*)nullptr);
+    return rlt_launch_status(device);
+}
+
+int rlt_rocm_gather_batch_drawn(rlt_rocm_device* device, const rlt_replay_buffer* rb, uint64_t seed, uint64_t stream, uint32_t* drawn_env_indices, uint32_t* drawn_sample_offsets,
+                                int max_episode_length, int batch, float* observations_actions_base, float* rewards, uint8_t* terminated,
+                                uint8_t* reset, uint8_t* next_reset_base, uint8_t* final_step_mask, uint8_t* next_final_step_mask_base) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(rb_ok(rb) && batch > 0 && observations_actions_base && rewards && terminated && max_episode_length >= 0);
+    int* error_flag = (int*)(device->fault + 1);
+    device->fault_armed = 1;
+    hipLaunchKernelGGL(gather_kernel, dim3(grid1(batch * 16)), dim3(256), 0, device->stream, *rb, (const uint32_t*)nullptr, (const uint32_t*)nullptr, 0, max_episode_length, batch,
+                       observations_actions_base, rewards, terminated, reset, next_reset_base, final_step_mask, next_final_step_mask_base, error_flag, 1, seed, stream,
+                       drawn_env_indices, drawn_sample_offsets);
     return rlt_launch_status(device);
 }
 
@@ -734,16 +762,38 @@ int rlt_rocm_pendulum_step(rlt_rocm_device* device, const rlt_pendulum_parameter
     return rlt_launch_status(device);
 }
 
+static int runner_step(rlt_rocm_device* device, const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, int policy_kind,
+                       const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas, const float* actions_in, const float* action_noise,
+                       const float* initial_states, uint64_t seed, uint64_t stream, bool draw_noise, uint64_t noise_stream, float* drawn_noise);
+
 int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, int policy_kind,
                                   const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas, const float* actions_in, const float* action_noise,
                                   const float* initial_states, uint64_t seed, uint64_t stream) {
+    return runner_step(device, rn, rb, policy_kind, actor, n_actor_layers, sas, actions_in, action_noise, initial_states, seed, stream, false, 0, nullptr);
+}
+
+int rlt_rocm_pendulum_runner_step_drawn(rlt_rocm_device* device, const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, const rlt_dense_layer* actor, int n_actor_layers,
+                                        const rlt_sas_parameters* sas, float* drawn_noise, uint64_t seed, uint64_t noise_stream, uint64_t initial_state_stream) {
+    return runner_step(device, rn, rb, 2, actor, n_actor_layers, sas, nullptr, nullptr, nullptr, seed, initial_state_stream, true, noise_stream, drawn_noise);
+}
+
+static int runner_step(rlt_rocm_device* device, const rlt_pendulum_runner* rn, const rlt_replay_buffer* rb, int policy_kind,
+                       const rlt_dense_layer* actor, int n_actor_layers, const rlt_sas_parameters* sas, const float* actions_in, const float* action_noise,
+                       const float* initial_states, uint64_t seed, uint64_t stream, bool draw_noise, uint64_t noise_stream, float* drawn_noise) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(rn && rn->states && rn->episode_step && rn->episode_return && rn->truncated && rn->n_envs > 0 && rb_ok(rb));
     RLT_REQUIRE(rn->n_envs == rb->n_envs && rb->observation_dim == 3 && rb->action_dim == 1 && policy_kind >= 0 && policy_kind <= 2);
     RLT_REQUIRE(policy_kind != 0 || actions_in);
     RLT_REQUIRE(policy_kind == 0 || (actor && n_actor_layers >= 1 && actor[0].in_dim == 3 && actor[n_actor_layers - 1].out_dim == (policy_kind == 2 ? 2 : 1)));
-    RLT_REQUIRE(policy_kind != 2 || (sas && action_noise));
+    RLT_REQUIRE(policy_kind != 2 || (sas && (action_noise || draw_noise)));
     const int N = rn->n_envs;
+    if (draw_noise && !fused_runner_ok(actor, n_actor_layers, policy_kind, rb, rn, initial_states)) {
+        // the per-operation launches read the noise from an array: fill it first
+        RLT_REQUIRE(drawn_noise);
+        const int rc = rlt_rocm_randn_f32(device, drawn_noise, (size_t)N, seed, noise_stream);
+        if (rc) return rc;
+        action_noise = drawn_noise;
+    }
     if (fused_runner_ok(actor, n_actor_layers, policy_kind, rb, rn, initial_states)) {
         FusedRunnerArgs a = {};
         a.rn = *rn; a.rb = *rb;
@@ -751,6 +801,7 @@ int rlt_rocm_pendulum_runner_step(rlt_rocm_device* device, const rlt_pendulum_ru
         a.act_hidden = actor[0].activation; a.act_out = actor[2].activation; a.out_dim = actor[2].out_dim; a.policy_kind = policy_kind;
         if (sas) a.sas = *sas;
         a.action_noise = action_noise; a.initial_states = initial_states; a.seed = seed; a.stream = stream;
+        a.noise_stream = noise_stream; a.drawn_noise = action_noise ? nullptr : drawn_noise;
         const int tiles = rlt_div_up(N, FTILE);
         int blocks = rlt_div_up(tiles, FWAVES); if (blocks > device->compute_units) blocks = device->compute_units;
         switch (a.act_hidden) {

@@ -260,7 +260,7 @@ int rlt_rocm_sac_set_per_operation(rlt_rocm_device* device, int enabled) {
 int rlt_rocm_sac_train_critic(rlt_rocm_device* device, const rlt_sac_agent* A, int ci, const float* action_noise) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A) && (ci == 0 || ci == 1) && action_noise);
-    if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) return rlt_sac_update_critic(device, A, ci, action_noise);
+    if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) { const rlt_update_noise noise = {action_noise, 0, 0, nullptr}; return rlt_sac_update_critic(device, A, ci, noise); }
     RLT_REQUIRE(A->next_state_action_value_input && A->next_q[0] && A->next_q[1] && A->next_log_probabilities && A->target_action_value && A->d_output_critic[ci]);
     const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
     const rlt_dense_layer* critic = A->critics[ci];
@@ -317,7 +317,7 @@ int rlt_rocm_sac_update_critic_targets(rlt_rocm_device* device, const rlt_sac_ag
 int rlt_rocm_sac_train_actor(rlt_rocm_device* device, const rlt_sac_agent* A, const float* action_noise) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A) && action_noise);
-    if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) return rlt_sac_update_actor(device, A, action_noise);
+    if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) { const rlt_update_noise noise = {action_noise, 0, 0, nullptr}; return rlt_sac_update_actor(device, A, noise); }
     RLT_REQUIRE(A->state_action_value_input && A->d_output_actor_critics && A->d_critic_input[0] && A->d_critic_input[1] && A->d_actor_output_squashing &&
                 A->d_actor_output && A->actor_pre_squashing && A->actor_log_probabilities && A->actor_actions && A->log_alpha.gradient);
     const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
@@ -352,6 +352,41 @@ int rlt_rocm_sac_train_actor(rlt_rocm_device* device, const rlt_sac_agent* A, co
     return rlt_rocm_adam_step(device, &A->log_alpha, 1, &A->alpha_adam, A->alpha_age, 0.0f, nullptr);
 }
 
+// both train_critic calls of a loop step with a shared batch (and update_critic_targets) as one launch where the fused kernel fits
+static int train_critics(rlt_rocm_device* device, const rlt_sac_agent* A, const rlt_update_noise& noise, int update_targets) {
+    if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) return rlt_sac_update_critics(device, A, noise, update_targets != 0);
+    int rc;
+    const float* values = noise.values;
+    if (!values) {
+        RLT_REQUIRE(noise.drawn);
+        if ((rc = rlt_rocm_randn_f32(device, noise.drawn, (size_t)A->batch * A->action_dim, noise.seed, noise.stream))) return rc;
+        values = noise.drawn;
+    }
+    for (int k = 0; k < 2; k++)
+        if ((rc = rlt_rocm_sac_train_critic(device, A, k, values))) return rc;
+    return update_targets ? rlt_rocm_sac_update_critic_targets(device, A) : 0;
+}
+int rlt_rocm_sac_train_critics(rlt_rocm_device* device, const rlt_sac_agent* A, const float* action_noise, int update_targets) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(agent_ok(A) && action_noise);
+    const rlt_update_noise noise = {action_noise, 0, 0, nullptr};
+    return train_critics(device, A, noise, update_targets);
+}
+int rlt_rocm_sac_train_critics_drawn(rlt_rocm_device* device, const rlt_sac_agent* A, float* drawn_noise, uint64_t seed, uint64_t stream, int update_targets) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(agent_ok(A));
+    const rlt_update_noise noise = {nullptr, seed, stream, drawn_noise};
+    return train_critics(device, A, noise, update_targets);
+}
+int rlt_rocm_sac_train_actor_drawn(rlt_rocm_device* device, const rlt_sac_agent* A, float* drawn_noise, uint64_t seed, uint64_t stream) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(agent_ok(A));
+    if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) { const rlt_update_noise noise = {nullptr, seed, stream, drawn_noise}; return rlt_sac_update_actor(device, A, noise); }
+    RLT_REQUIRE(drawn_noise);
+    const int rc = rlt_rocm_randn_f32(device, drawn_noise, (size_t)A->batch * A->action_dim, seed, stream);
+    return rc ? rc : rlt_rocm_sac_train_actor(device, A, drawn_noise);
+}
+
 // rl/algorithms/sac/loop/core/operations_generic.h:110-155 past the warm-up, as a host loop over the entry points of this library
 int rlt_rocm_sac_pendulum_loop_by_calls(rlt_rocm_device* device, const rlt_sac_agent* A, const rlt_pendulum_runner* runner, const rlt_replay_buffer* rb, int n_steps,
                                         uint64_t seed, uint64_t step_offset, const rlt_sac_loop_scratch* S) {
@@ -359,21 +394,16 @@ int rlt_rocm_sac_pendulum_loop_by_calls(rlt_rocm_device* device, const rlt_sac_a
     RLT_REQUIRE(agent_ok(A) && runner && rb && S && n_steps >= 0);
     RLT_REQUIRE(S->rollout_noise && S->noise_critic && S->noise_actor && S->env_indices && S->sample_offsets);
     RLT_REQUIRE(rb->observation_dim == A->observation_dim && rb->action_dim == A->action_dim && rb->n_envs == runner->n_envs);
-    const int B = A->batch, ACT = A->action_dim;
+    const int B = A->batch;
     int rc;
     for (int i = 0; i < n_steps; i++) {
         const uint64_t g = 8 * (step_offset + (uint64_t)i);
-        if ((rc = rlt_rocm_randn_f32(device, S->rollout_noise, (size_t)runner->n_envs * ACT, seed, g + 1))) return rc;
-        if ((rc = rlt_rocm_pendulum_runner_step(device, runner, rb, 2, A->actor, A->n_actor_layers, &A->sas, nullptr, S->rollout_noise, nullptr, seed, g + 2))) return rc;
-        if ((rc = rlt_rocm_gather_draw(device, rb, B, seed, g + 3, S->env_indices, S->sample_offsets))) return rc;
-        if ((rc = rlt_rocm_gather_batch(device, rb, S->env_indices, S->sample_offsets, 0, runner->episode_step_limit, B, A->observations_actions_base, A->rewards,
-                                        A->terminated, nullptr, nullptr, nullptr, nullptr))) return rc;
-        if ((rc = rlt_rocm_randn_f32(device, S->noise_critic, (size_t)B * ACT, seed, g + 4))) return rc;
-        for (int k = 0; k < 2; k++)
-            if ((rc = rlt_rocm_sac_train_critic(device, A, k, S->noise_critic))) return rc;
-        if ((rc = rlt_rocm_sac_update_critic_targets(device, A))) return rc;
-        if ((rc = rlt_rocm_randn_f32(device, S->noise_actor, (size_t)B * ACT, seed, g + 5))) return rc;
-        if ((rc = rlt_rocm_sac_train_actor(device, A, S->noise_actor))) return rc;
+        // every draw is made by the kernel that consumes it (and echoed into the scratch arrays): four launches per step where the fused kernels fit
+        if ((rc = rlt_rocm_pendulum_runner_step_drawn(device, runner, rb, A->actor, A->n_actor_layers, &A->sas, S->rollout_noise, seed, g + 1, g + 2))) return rc;
+        if ((rc = rlt_rocm_gather_batch_drawn(device, rb, seed, g + 3, S->env_indices, S->sample_offsets, runner->episode_step_limit, B, A->observations_actions_base, A->rewards,
+                                              A->terminated, nullptr, nullptr, nullptr, nullptr))) return rc;
+        if ((rc = rlt_rocm_sac_train_critics_drawn(device, A, S->noise_critic, seed, g + 4, 1))) return rc;
+        if ((rc = rlt_rocm_sac_train_actor_drawn(device, A, S->noise_actor, seed, g + 5))) return rc;
     }
     return 0;
 }

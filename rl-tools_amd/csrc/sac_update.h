@@ -5,11 +5,17 @@
 // true if the agent fits the fused kernels: every network 3 layers in -> 64 -> 64 -> out with one hidden activation (not GELU), at most 128
 // critic inputs and 8 actions, no sequence masks
 bool rlt_sac_update_supported(const rlt_rocm_device* device, const rlt_sac_agent* agent);
+// The N(0, 1) noise of an update: an array [batch x action_dim] filled beforehand (values), or, with values == NULL, the elements of
+// the stream (seed, stream) that rlt_rocm_randn_f32 would have put there, drawn by the kernel itself; `drawn` (optional) then receives them.
+struct rlt_update_noise { const float* values; uint64_t seed, stream; float* drawn; };
 // train_critic / train_actor with the contracts of rlt_rocm_sac_train_critic / rlt_rocm_sac_train_actor; of the training buffers only
 // next_log_probabilities and target_action_value / actor_log_probabilities, actor_actions and actor_pre_squashing are written.
-// RLT_E_UNSUPPORTED unless rlt_sac_update_supported.
-int rlt_sac_update_critic(rlt_rocm_device* device, const rlt_sac_agent* agent, int critic_index, const float* action_noise);
-int rlt_sac_update_actor(rlt_rocm_device* device, const rlt_sac_agent* agent, const float* action_noise);
+// One launch each where the Adam tensors are the networks' gradient buffers (the last workgroup to finish adds up the partial
+// gradients and steps), else the optimiser follows as launches of its own. RLT_E_UNSUPPORTED unless rlt_sac_update_supported.
+int rlt_sac_update_critic(rlt_rocm_device* device, const rlt_sac_agent* agent, int critic_index, const rlt_update_noise& noise);
+int rlt_sac_update_actor(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_update_noise& noise);
+// both train_critic calls on the agent's batch with the same noise in ONE launch and, if update_targets, update_critic_targets after them
+int rlt_sac_update_critics(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_update_noise& noise, bool update_targets);
 // target[i] = polyak * target[i] + (1 - polyak) * source[i] for a list of tensors, one launch per 16 tensors
 int rlt_sac_polyak_list(rlt_rocm_device* device, const float* const* sources, float* const* targets, const uint32_t* counts, int n, float polyak);
 

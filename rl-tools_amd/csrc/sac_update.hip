@@ -29,6 +29,7 @@
 #include "sac_update.h"
 #include "mlp_small.h"
 #include "optim.h"
+#include "rng.h"
 
 namespace {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -58,6 +59,24 @@ struct UpdateArgs {
     float sampling_std; int ignore_termination;
     const float* target_noise;             // critic update: [batch][act], already clamped (target_action_noise), added to the next action before a second clamp
     float* out_pre_clip;                   // actor update: [batch][act], the sampling layer's value before the clamp
+    // noise == NULL: element i of the noise is element i of the standard-normal stream (noise_seed, noise_stream), what
+    // rlt_rocm_randn_f32 would have put there; out_noise (optional) receives the values
+    uint64_t noise_seed, noise_stream; float* out_noise;
+    // every 8th workgroup of an 8 x larger grid works, so that all of them run on one XCD and share its L2 (the device hands out
+    // workgroups round robin over the XCDs)
+    int packed;
+    // The optimiser's step at the end of the launch: every workgroup announces its block of partial sums (tickets[0]), waits until all
+    // workgroups of the launch have, and steps a slice of its trained network's elements: sum over the blocks in the order of the
+    // small-MLP reduction kernel, Adam, and the soft update of a target where the tensor names one (opt[].t[].polyak_target; the targets
+    // are read by every workgroup of the launch, hence the wait for all of them). The grid must be resident as a whole: the host
+    // only asks for this with at most 64 workgroups. The wait is bounded; a workgroup that gives up sets *fault and leaves its slice
+    // undone. tickets[1] counts the workgroups that are through; the last one clears both words and advances the ages.
+    // Critic updates: blockIdx.y selects the trained critic (critic[y], opt[y]).
+    int tail;
+    uint32_t* tickets; unsigned* fault;
+    rlt_tail_optimizer opt[2];
+    float polyak;
+    int has_second; rlt_adam_tensor second; rlt_adam_parameters second_p; uint32_t* second_age; float second_scale;      // a scalar whose gradient is extra[0] * second_scale (log_alpha)
 };
 
 __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
@@ -285,6 +304,80 @@ __device__ __forceinline__ void td3_head_forward(const UpdateArgs& A, lptr d3s, 
     }
 }
 
+// The optimiser's step at the end of an update kernel (see UpdateArgs::tail). Every thread of every workgroup calls it after its last store.
+constexpr unsigned TAIL_MAX_POLL = 1u << 20;      // about a second
+template <bool SAME_XCD>
+__device__ __forceinline__ void tail_slice(const UpdateArgs& A, int y, int g, int G) {
+    const rlt_tail_optimizer& O = A.opt[y];
+    const float* blocks = A.partial + (size_t)y * G * A.count;
+    const uint32_t n = O.prefix[O.n], chunk = (n + G - 1) / G, begin = min(n, (uint32_t)g * chunk), end = min(n, begin + chunk);
+    const uint32_t age = *O.age;
+    float bc1, bc2;
+    rlt_adam_bias_corrections(O.p, age, bc1, bc2);
+    for (uint32_t base = begin; base < end; base += THREADS) {
+        const uint32_t i = base + threadIdx.x;
+        const bool ok = i < end;
+        const uint32_t ic = ok ? i : begin;
+        int t = 0;
+#pragma unroll
+        for (int k = 1; k < RLT_TAIL_TENSORS; k++) t += (k < O.n && ic >= O.prefix[k]) ? 1 : 0;
+        const uint32_t j = ic - O.prefix[t];
+        const float* const src[1] = {blocks + O.offset[t] + j};
+        float gs[1];
+        rlt_sum_of_blocks<1, SAME_XCD>(src, G, A.count, gs);
+        if (ok) {
+            const rlt_adam_tensor& T = O.t[t];
+            const float ge = gs[0] * O.scale[t];
+            T.gradient[j] = ge;
+            rlt_adam_apply(O.p, T, j, ge, bc1, bc2, A.polyak);
+        }
+    }
+    if (A.has_second && g == G - 1 && threadIdx.x == THREADS - 1) {
+        const float* const src[1] = {blocks + (A.count - N_EXTRA)};
+        float gs[1];
+        rlt_sum_of_blocks<1, SAME_XCD>(src, G, A.count, gs);
+        float b1, b2;
+        rlt_adam_bias_corrections(A.second_p, *A.second_age, b1, b2);
+        const float ge = gs[0] * A.second_scale;
+        A.second.gradient[0] = ge;
+        rlt_adam_apply(A.second_p, A.second, 0, ge, b1, b2, 0.0f);
+    }
+}
+__device__ __noinline__ void optimiser_tail(const UpdateArgs& A, int y, int g, int G, lptr flag_words) {
+    typedef __attribute__((address_space(3))) int* liptr;
+    const liptr flags = (liptr)flag_words;
+    const unsigned total = (unsigned)G * gridDim.y;
+    __builtin_amdgcn_s_waitcnt(0);            // this wavefront's stores have completed
+    if (!A.packed) __threadfence();           // and are visible beyond this XCD
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        __hip_atomic_fetch_add(A.tickets, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned tries = 0; int ok = 1;
+        while (__hip_atomic_load(A.tickets, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < total) {
+            __builtin_amdgcn_s_sleep(1);
+            if (++tries >= TAIL_MAX_POLL || ((tries & 63u) == 0u && __hip_atomic_load(A.fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+                __hip_atomic_store(A.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                ok = 0;
+                break;
+            }
+        }
+        flags[0] = ok;
+    }
+    __syncthreads();
+    if (flags[0]) {
+        if (A.packed) tail_slice<true>(A, y, g, G);
+        else { __threadfence(); tail_slice<false>(A, y, g, G); }
+    }
+    __syncthreads();        // every thread has read the ages it needs
+    if (threadIdx.x == 0 && __hip_atomic_fetch_add(A.tickets + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == total - 1) {
+        // the last workgroup through: nobody waits on the words any more, and every slice has been stepped with the old ages
+        __hip_atomic_store(A.tickets, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(A.tickets + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (unsigned k = 0; k < gridDim.y; k++) *A.opt[k].age += 1;
+        if (A.has_second) *A.second_age += 1;
+    }
+}
+
 template <int NT1C, int MODE, int ACT_H>
 __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
     constexpr bool CRITIC = MODE == 0 || MODE == MODE_TD3_CRITIC, TD3 = MODE == MODE_TD3_CRITIC || MODE == MODE_TD3_ACTOR;
@@ -299,10 +392,13 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
                d3s = h2s + 5 * ROWS * HS, d3c = d3s + (1 + team) * ROWS * D3S, yps = d3s + 3 * ROWS * D3S, misc = yps + 4 * TEAM_WAVES * YP,
                stage = misc + MISC + wave * 16 * (SX > HS ? SX : HS);
     const lptr ypa = yps + team * TEAM_WAVES * YP, ypb = yps + (2 + team) * TEAM_WAVES * YP;      // stage A / stage B partial tiles of this team
-    const int row0 = blockIdx.x * ROWS;
+    if (A.packed && (blockIdx.x & 7)) return;
+    const int g = A.packed ? blockIdx.x >> 3 : blockIdx.x, G = A.packed ? gridDim.x >> 3 : gridDim.x;
+    const int y = CRITIC ? blockIdx.y : 0;
+    const int row0 = g * ROWS;
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
     float s3 = 0.f, extra = 0.f;
-    const Net& trained = CRITIC ? A.critic[0] : A.actor;
+    const Net trained = CRITIC ? (y ? A.critic[1] : A.critic[0]) : A.actor;      // by value: an index into the kernel's argument would keep all of it in private memory
     const int NT1_D = (D + 15) >> 4, NT1_OBS = (OBS + 15) >> 4;
 
     // the input tiles (32 threads share a row), then every parameter this wavefront multiplies with in the forward passes, are requested
@@ -354,7 +450,13 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
         }
         b3_actor = r < A.actor.out ? A.actor.b3[min(r, A.actor.out - 1)] : 0.f;
 #pragma unroll
-        for (int j = 0; j < 2; j++) noise[j] = (kk + 4 * j < ACT && row0 + r < B) ? A.noise[(size_t)(row0 + r) * ACT + kk + 4 * j] : 0.f;
+        for (int j = 0; j < 2; j++) {
+            if (kk + 4 * j < ACT && row0 + r < B) {
+                const size_t i = (size_t)(row0 + r) * ACT + kk + 4 * j;
+                noise[j] = A.noise ? A.noise[i] : rlt_randn_element(A.noise_seed, A.noise_stream, i);
+                if (A.out_noise && y == 0) A.out_noise[i] = noise[j];
+            }
+        }
         if (CRITIC) {
 #pragma unroll
             for (int v = 0; v < 4; v++) { const int row = min(row0 + 4 * kk + v, B - 1); reward[v] = A.rewards[row]; terminated[v] = A.terminated[row] != 0; }
@@ -514,7 +616,7 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
 
     // stage C: backward pass of the trained network with its weight gradients over the workgroup's 16 rows, by its team; h1, h2: its
     // hidden activations, d3: the gradient at its last pre-activation; the team's ta receives d_pre2, tb receives d_pre1
-    float* dst = A.partial + (size_t)blockIdx.x * A.count;
+    float* dst = A.partial + ((size_t)y * G + g) * A.count;
     const int IN = trained.in, OUT = trained.out, NT1 = (IN + 15) >> 4;
     const int o_b1 = H * IN, o_w2 = o_b1 + H, o_b2 = o_w2 + H * H, o_w3 = o_b2 + H, o_b3 = o_w3 + OUT * H, o_ex = o_b3 + OUT;
     const lptr xt = CRITIC ? xsb : xsa;
@@ -567,6 +669,10 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
             dst[o_ex + r] = extra;
         }
     }
+    if (!A.tail) return;
+    // the kernel's arguments as they lie in its argument segment (the struct is the only explicit argument), so that the optimiser's
+    // part, a function of its own, indexes them there
+    optimiser_tail(*(const UpdateArgs*)__builtin_amdgcn_kernarg_segment_ptr(), y, g, G, (lptr)(misc + 48));
 }
 
 // soft update of up to 16 tensors in one launch (utils/polyak/operations_generic.h:11-27): workgroup b serves tensor b % n
@@ -575,7 +681,7 @@ struct PolyakList { const float* source[MAX_POLYAK]; float* target[MAX_POLYAK]; 
 __global__ __launch_bounds__(256) void polyak_list_kernel(PolyakList P) {
     const int t = blockIdx.x % P.n, part = blockIdx.x / P.n, parts = gridDim.x / P.n;
     const float* __restrict__ s = P.source[t]; float* __restrict__ d = P.target[t];
-    for (uint32_t i = part * 256 + threadIdx.x; i < P.count[t]; i += parts * 256) d[i] = P.polyak * d[i] + (1.0f - P.polyak) * s[i];
+    for (uint32_t i = part * 256 + threadIdx.x; i < P.count[t]; i += parts * 256) d[i] = rlt_polyak_value(P.polyak, d[i], s[i]);
 }
 
 bool hidden_ok(int a) { return a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH || a == RLT_ACT_SIGMOID; }
@@ -593,7 +699,7 @@ int tile_bucket(int d) { return d <= 32 ? 2 : MAX_D / 16; }
 // Where each Adam tensor's gradient lies in a block of partial sums [dW1 | db1 | dW2 | db2 | dW3 | db3 | extra]: a tensor may span
 // several of the network's six gradient buffers where those follow each other in memory. False unless the tensors cover the six
 // buffers exactly, at most 12 of them: then the optimiser's launch can read the blocks itself.
-bool map_gradients(const rlt_dense_layer* L, const rlt_adam_tensor* T, int n, uint32_t* offsets) {
+bool map_gradients(const rlt_dense_layer* L, const rlt_adam_tensor* T, int n, uint32_t* offsets, int* first_segment = nullptr, int* n_segments = nullptr) {
     if (!T || n < 1 || n > 12) return false;
     const float* seg[6] = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases};
     const uint32_t size[6] = {(uint32_t)(H * L[0].in_dim), H, H * H, H, (uint32_t)(L[2].out_dim * H), (uint32_t)L[2].out_dim};
@@ -603,63 +709,123 @@ bool map_gradients(const rlt_dense_layer* L, const rlt_adam_tensor* T, int n, ui
         int s = 0;
         while (s < 6 && seg[s] != T[i].gradient) s++;
         if (s == 6 || T[i].polyak_target) return false;
-        uint32_t cnt = 0;
-        for (int k = s; k < 6 && cnt < T[i].count && seg[k] == seg[s] + cnt; k++) {
+        uint32_t cnt = 0; int k = s;
+        for (; k < 6 && cnt < T[i].count && seg[k] == seg[s] + cnt; k++) {
             if (covered & (1u << k)) return false;
             covered |= 1u << k; cnt += size[k];
         }
         if (cnt != T[i].count) return false;
         offsets[i] = off[s];
+        if (first_segment) first_segment[i] = s;
+        if (n_segments) n_segments[i] = k - s;
     }
     return covered == 63u;
 }
-
-// the workgroups' blocks of partial sums -> gradients -> Adam step(s): one launch where the optimiser can read the blocks itself, else
-// the reduction kernel and then the optimiser. `second` (optional): an optimiser for one scalar whose gradient is extra[0] / batch.
-int reduce_and_step(rlt_rocm_device* device, const UpdateArgs& a, int groups, const rlt_dense_layer* trained, const rlt_adam_tensor* tensors, int n_tensors,
-                    const rlt_adam_parameters* parameters, uint32_t* age, const rlt_adam_tensor* second, const rlt_adam_parameters* second_parameters, uint32_t* second_age,
-                    float second_scale) {
-    uint32_t offsets[12];
-    if (map_gradients(trained, tensors, n_tensors, offsets) && (!second || !second->polyak_target)) {
-        float scales[12];
-        for (int i = 0; i < 12; i++) scales[i] = 1.0f;
-        const rlt_adam_source source = {a.partial, groups, a.count, offsets, scales};
-        if (!second) return rlt_adam_step_from_partials(device, tensors, n_tensors, parameters, age, &source);
-        const uint32_t second_offset = (uint32_t)(a.count - N_EXTRA);
-        const rlt_adam_source second_source = {a.partial, groups, a.count, &second_offset, &second_scale};
-        return rlt_adam_step_pair(device, tensors, n_tensors, parameters, age, second, 1, second_parameters, second_age, &source, &second_source);
-    }
-    int rc = rlt_mlp3s_reduce(device, trained, a.partial, groups, 1, second ? second->gradient : nullptr, second ? 1 : 0, second_scale, 0.0f);
-    if (rc) return rc;
-    if (second && n_tensors <= 12) return rlt_adam_step_pair(device, tensors, n_tensors, parameters, age, second, 1, second_parameters, second_age);
-    if ((rc = rlt_rocm_adam_step(device, tensors, n_tensors, parameters, age, 0.0f, nullptr))) return rc;
-    return second ? rlt_rocm_adam_step(device, second, 1, second_parameters, second_age, 0.0f, nullptr) : 0;
+// where the segments [first, first + count) of a network's parameters lie, if they follow each other in memory (NULL otherwise)
+float* parameter_segments(const rlt_dense_layer* L, int first, int count) {
+    float* seg[6] = {L[0].weights, L[0].biases, L[1].weights, L[1].biases, L[2].weights, L[2].biases};
+    const uint32_t size[6] = {(uint32_t)(H * L[0].in_dim), H, H * H, H, (uint32_t)(L[2].out_dim * H), (uint32_t)L[2].out_dim};
+    uint32_t cnt = 0;
+    for (int k = first; k < first + count; k++) { if (seg[k] != seg[first] + cnt) return nullptr; cnt += size[k]; }
+    return seg[first];
 }
 
+// The optimiser of one trained network of the launch; `soft_target` (optional): the network that follows the trained one by the soft update
+struct Optimiser {
+    const rlt_dense_layer* trained; const rlt_adam_tensor* tensors; int n_tensors; const rlt_adam_parameters* parameters; uint32_t* age;
+    const rlt_adam_tensor* second; const rlt_adam_parameters* second_parameters; uint32_t* second_age; float second_scale;
+    const rlt_dense_layer* soft_target;
+};
+constexpr int TAIL_MAX_WORKGROUPS = 64;      // a grid of this many workgroups of 512 threads is resident as a whole on any device this library runs on
+
+// The optimisers as the kernel's own last step: possible where the Adam tensors are the networks' gradient buffers (and the targets'
+// parameters are laid out as the trained networks' are) and the grid is small enough to wait for itself.
+bool configure_tail(rlt_rocm_device* device, UpdateArgs& a, const Optimiser* opts, int n_opts, int groups, float polyak) {
+    if (!device->update_tail || n_opts < 1 || n_opts > 2 || n_opts * groups > TAIL_MAX_WORKGROUPS) return false;
+    for (int k = 0; k < n_opts; k++) {
+        const Optimiser& O = opts[k];
+        uint32_t offsets[12]; int first[12], count[12];
+        if (!map_gradients(O.trained, O.tensors, O.n_tensors, offsets, first, count)) return false;
+        if (O.second && (O.second->polyak_target || n_opts != 1 || !O.second->parameters || !O.second->gradient || !O.second->first_moment || !O.second->second_moment)) return false;
+        if (!rlt_tail_optimizer_fill(a.opt[k], O.tensors, O.n_tensors, offsets, nullptr, O.parameters, O.age)) return false;
+        if (O.soft_target)
+            for (int i = 0; i < O.n_tensors; i++) {
+                // the tensor's parameters must be the trained network's own segments, so that the target's segments correspond element by element
+                if (parameter_segments(O.trained, first[i], count[i]) != O.tensors[i].parameters) return false;
+                if (!(a.opt[k].t[i].polyak_target = parameter_segments(O.soft_target, first[i], count[i]))) return false;
+            }
+        if (O.second) { a.has_second = 1; a.second = *O.second; a.second_p = *O.second_parameters; a.second_age = O.second_age; a.second_scale = O.second_scale; }
+    }
+    void* counters = nullptr;
+    if (rlt_counters(device, &counters)) return false;
+    a.tickets = (uint32_t*)counters + RLT_TICKET_TAIL;
+    a.fault = device->fault;
+    a.polyak = polyak;
+    a.tail = 1;
+    return true;
+}
+
+// the workgroups' blocks of partial sums -> gradients -> Adam step(s), as launches after the update kernel: one where the optimiser can
+// read the blocks itself, else the reduction kernel and then the optimiser. `second` (optional): an optimiser for one scalar whose
+// gradient is extra[0] * second_scale.
+int reduce_and_step(rlt_rocm_device* device, const UpdateArgs& a, const float* partial, int groups, const Optimiser& O) {
+    uint32_t offsets[12];
+    if (map_gradients(O.trained, O.tensors, O.n_tensors, offsets) && (!O.second || !O.second->polyak_target)) {
+        float scales[12];
+        for (int i = 0; i < 12; i++) scales[i] = 1.0f;
+        const rlt_adam_source source = {partial, groups, a.count, offsets, scales};
+        if (!O.second) return rlt_adam_step_from_partials(device, O.tensors, O.n_tensors, O.parameters, O.age, &source);
+        const uint32_t second_offset = (uint32_t)(a.count - N_EXTRA);
+        const rlt_adam_source second_source = {partial, groups, a.count, &second_offset, &O.second_scale};
+        return rlt_adam_step_pair(device, O.tensors, O.n_tensors, O.parameters, O.age, O.second, 1, O.second_parameters, O.second_age, &source, &second_source);
+    }
+    int rc = rlt_mlp3s_reduce(device, O.trained, partial, groups, 1, O.second ? O.second->gradient : nullptr, O.second ? 1 : 0, O.second_scale, 0.0f);
+    if (rc) return rc;
+    if (O.second && O.n_tensors <= 12) return rlt_adam_step_pair(device, O.tensors, O.n_tensors, O.parameters, O.age, O.second, 1, O.second_parameters, O.second_age);
+    if ((rc = rlt_rocm_adam_step(device, O.tensors, O.n_tensors, O.parameters, O.age, 0.0f, nullptr))) return rc;
+    return O.second ? rlt_rocm_adam_step(device, O.second, 1, O.second_parameters, O.second_age, 0.0f, nullptr) : 0;
+}
+
+// One launch for `n_opts` trained networks (2: both critics of a critic update, one per blockIdx.y) and their optimisers; where the
+// optimiser cannot be the kernel's last step it follows as launches of its own.
 template <int MODE>
-int launch_update(rlt_rocm_device* device, UpdateArgs& a, int groups, const rlt_dense_layer* trained) {
+int launch_update(rlt_rocm_device* device, UpdateArgs& a, int groups, const Optimiser* opts, int n_opts, float polyak = 0.0f) {
+    const rlt_dense_layer* trained = opts[0].trained;
     const int bucket = tile_bucket(a.obs + a.act);
     const size_t lds_bytes = lds_floats(bucket) * sizeof(float);
     a.count = rlt_mlp3s_partial_count(trained[0].in_dim, trained[2].out_dim);
     void* scratch = nullptr;
-    int rc = rlt_scratch(device, (size_t)groups * a.count * sizeof(float), &scratch);
+    int rc = rlt_scratch(device, (size_t)n_opts * groups * a.count * sizeof(float), &scratch);
     if (rc) return rc;
     a.partial = (float*)scratch;
+    const bool tail = configure_tail(device, a, opts, n_opts, groups, polyak);
+    if (tail) device->fault_armed = 1;
+    // up to 32 workgroups (one per compute unit of an XCD) are placed on one XCD where the device hands out workgroups round robin
+    a.packed = device->update_one_xcd && device->xcd_stride == 8 && n_opts * groups <= 32 ? 1 : 0;
+    const dim3 grid(a.packed ? 8 * groups : groups, n_opts);
 #define RLT_LAUNCH_UPDATE(NT, ACT)                                                                                                                              \
     do {                                                                                                                                                        \
         RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sac_update_kernel<NT, MODE, ACT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
-        hipLaunchKernelGGL((sac_update_kernel<NT, MODE, ACT>), dim3(groups), dim3(THREADS), lds_bytes, device->stream, a);                                    \
+        hipLaunchKernelGGL((sac_update_kernel<NT, MODE, ACT>), grid, dim3(THREADS), lds_bytes, device->stream, a);                                            \
     } while (0)
-    // ReLU (the reference's default for SAC) and tanh are compiled in; any other hidden activation takes the variant that looks it up
-    const int act = a.actor.act_h == a.critic[0].act_h && a.actor.act_h == a.target[0].act_h ? a.actor.act_h : -1;
+    // ReLU (the reference's default for SAC) and tanh are compiled in; any other hidden activation, or networks that differ in it, take
+    // the variant that looks it up per network
+    int act = a.actor.act_h;
+    for (int k = 0; k < 2; k++) if (a.critic[k].act_h != act || a.target[k].act_h != act) act = -1;
     if (bucket == 2) {
         if (act == RLT_ACT_RELU) RLT_LAUNCH_UPDATE(2, RLT_ACT_RELU); else if (act == RLT_ACT_TANH) RLT_LAUNCH_UPDATE(2, RLT_ACT_TANH); else RLT_LAUNCH_UPDATE(2, -1);
     } else {
         if (act == RLT_ACT_RELU) RLT_LAUNCH_UPDATE(MAX_D / 16, RLT_ACT_RELU); else if (act == RLT_ACT_TANH) RLT_LAUNCH_UPDATE(MAX_D / 16, RLT_ACT_TANH); else RLT_LAUNCH_UPDATE(MAX_D / 16, -1);
     }
 #undef RLT_LAUNCH_UPDATE
-    return rlt_launch_status(device);
+    if ((rc = rlt_launch_status(device))) return rc;
+    if (tail) return 0;
+    for (int k = 0; k < n_opts; k++)
+        if ((rc = reduce_and_step(device, a, a.partial + (size_t)k * groups * a.count, groups, opts[k]))) return rc;
+    return 0;
 }
+
+void set_noise(UpdateArgs& a, const rlt_update_noise& N) { a.noise = N.values; a.noise_seed = N.seed; a.noise_stream = N.stream; a.out_noise = N.values ? nullptr : N.drawn; }
 }  // namespace
 
 bool rlt_sac_update_supported(const rlt_rocm_device* device, const rlt_sac_agent* A) {
@@ -672,36 +838,54 @@ bool rlt_sac_update_supported(const rlt_rocm_device* device, const rlt_sac_agent
     return lds_floats(tile_bucket(D)) * sizeof(float) <= (size_t)device->lds_bytes;
 }
 
-int rlt_sac_update_critic(rlt_rocm_device* device, const rlt_sac_agent* A, int ci, const float* action_noise) {
+static void sac_critic_args(UpdateArgs& a, const rlt_sac_agent* A) {
+    a.actor = net_of(A->actor);
+    for (int k = 0; k < 2; k++) a.target[k] = net_of(A->critics_target[k]);
+    a.batch_base = A->observations_actions_base; a.rewards = A->rewards; a.terminated = A->terminated; a.log_alpha = A->log_alpha.parameters;
+    a.sas = A->sas; a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
+    a.out_log_probabilities = A->next_log_probabilities; a.out_target_action_value = A->target_action_value;
+}
+
+int rlt_sac_update_critic(rlt_rocm_device* device, const rlt_sac_agent* A, int ci, const rlt_update_noise& noise) {
     if (!rlt_sac_update_supported(device, A)) return RLT_E_UNSUPPORTED;
     for (int l = 0; l < 3; l++) RLT_REQUIRE(A->critics[ci][l].d_weights && A->critics[ci][l].d_biases);
     UpdateArgs a = {};
-    a.actor = net_of(A->actor); a.critic[0] = net_of(A->critics[ci]); a.critic[1] = a.critic[0];
-    for (int k = 0; k < 2; k++) a.target[k] = net_of(A->critics_target[k]);
-    a.batch_base = A->observations_actions_base; a.rewards = A->rewards; a.terminated = A->terminated; a.noise = action_noise; a.log_alpha = A->log_alpha.parameters;
-    a.sas = A->sas; a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
-    a.out_log_probabilities = A->next_log_probabilities; a.out_target_action_value = A->target_action_value;
-    const int groups = rlt_div_up(A->batch, ROWS);
-    int rc = launch_update<MODE_CRITIC>(device, a, groups, A->critics[ci]);
-    if (rc) return rc;
-    return reduce_and_step(device, a, groups, A->critics[ci], A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], nullptr, nullptr, nullptr, 0.0f);
+    sac_critic_args(a, A);
+    a.critic[0] = net_of(A->critics[ci]); a.critic[1] = a.critic[0];
+    set_noise(a, noise);
+    const Optimiser O = {A->critics[ci], A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], nullptr, nullptr, nullptr, 0.0f, nullptr};
+    return launch_update<MODE_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), &O, 1);
 }
 
-int rlt_sac_update_actor(rlt_rocm_device* device, const rlt_sac_agent* A, const float* action_noise) {
+// both critics' updates on the same batch and noise in one launch (they do not depend on each other: each reads the actor, both target
+// critics and itself), and after them, if asked for, the soft update of both targets by whichever workgroup finishes last
+int rlt_sac_update_critics(rlt_rocm_device* device, const rlt_sac_agent* A, const rlt_update_noise& noise, bool update_targets) {
+    if (!rlt_sac_update_supported(device, A)) return RLT_E_UNSUPPORTED;
+    for (int k = 0; k < 2; k++) for (int l = 0; l < 3; l++) RLT_REQUIRE(A->critics[k][l].d_weights && A->critics[k][l].d_biases);
+    UpdateArgs a = {};
+    sac_critic_args(a, A);
+    for (int k = 0; k < 2; k++) a.critic[k] = net_of(A->critics[k]);
+    set_noise(a, noise);
+    const Optimiser O[2] = {{A->critics[0], A->critic_adam_tensors[0], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[0], nullptr, nullptr, nullptr, 0.0f, update_targets ? A->critics_target[0] : nullptr},
+                            {A->critics[1], A->critic_adam_tensors[1], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[1], nullptr, nullptr, nullptr, 0.0f, update_targets ? A->critics_target[1] : nullptr}};
+    const int rc = launch_update<MODE_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), O, 2, A->polyak);
+    if (rc || !update_targets || a.tail) return rc;
+    return rlt_rocm_sac_update_critic_targets(device, A);      // the optimisers ran as launches of their own: so does the soft update
+}
+
+int rlt_sac_update_actor(rlt_rocm_device* device, const rlt_sac_agent* A, const rlt_update_noise& noise) {
     if (!rlt_sac_update_supported(device, A)) return RLT_E_UNSUPPORTED;
     for (int l = 0; l < 3; l++) RLT_REQUIRE(A->actor[l].d_weights && A->actor[l].d_biases);
     RLT_REQUIRE(A->log_alpha.gradient);
     UpdateArgs a = {};
     a.actor = net_of(A->actor);
     for (int k = 0; k < 2; k++) { a.critic[k] = net_of(A->critics[k]); a.target[k] = a.critic[k]; }
-    a.batch_base = A->observations_actions_base; a.noise = action_noise; a.log_alpha = A->log_alpha.parameters;
+    a.batch_base = A->observations_actions_base; a.log_alpha = A->log_alpha.parameters;
+    set_noise(a, noise);
     a.sas = A->sas; a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
     a.out_log_probabilities = A->actor_log_probabilities; a.out_actions = A->actor_actions; a.out_pre_squashing = A->actor_pre_squashing;
-    const int groups = rlt_div_up(A->batch, ROWS);
-    int rc = launch_update<MODE_ACTOR>(device, a, groups, A->actor);
-    if (rc) return rc;
-    return reduce_and_step(device, a, groups, A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, &A->log_alpha, &A->alpha_adam, A->alpha_age,
-                           1.0f / (float)A->batch);
+    const Optimiser O = {A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, &A->log_alpha, &A->alpha_adam, A->alpha_age, 1.0f / (float)A->batch, nullptr};
+    return launch_update<MODE_ACTOR>(device, a, rlt_div_up(A->batch, ROWS), &O, 1);
 }
 
 // ---- TD3: the same kernel with the td3_sampling head (rl/algorithms/td3/operations_generic.h:170-281)
@@ -719,7 +903,7 @@ bool rlt_td3_update_supported(const rlt_rocm_device* device, const rlt_td3_agent
 int rlt_td3_update_critic(rlt_rocm_device* device, const rlt_td3_agent* A, int ci, const float* sampling_noise) {
     if (!rlt_td3_update_supported(device, A)) return RLT_E_UNSUPPORTED;
     for (int l = 0; l < 3; l++) RLT_REQUIRE(A->critics[ci][l].d_weights && A->critics[ci][l].d_biases);
-    RLT_REQUIRE(A->target_next_action_noise);
+    RLT_REQUIRE(A->target_next_action_noise && sampling_noise);
     UpdateArgs a = {};
     a.actor = net_of(A->actor_target); a.critic[0] = net_of(A->critics[ci]); a.critic[1] = a.critic[0];
     for (int k = 0; k < 2; k++) a.target[k] = net_of(A->critics_target[k]);
@@ -727,25 +911,22 @@ int rlt_td3_update_critic(rlt_rocm_device* device, const rlt_td3_agent* A, int c
     a.sampling_std = A->sampling_std; a.ignore_termination = A->ignore_termination;
     a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
     a.out_target_action_value = A->target_action_value;
-    const int groups = rlt_div_up(A->batch, ROWS);
-    int rc = launch_update<MODE_TD3_CRITIC>(device, a, groups, A->critics[ci]);
-    if (rc) return rc;
-    return reduce_and_step(device, a, groups, A->critics[ci], A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], nullptr, nullptr, nullptr, 0.0f);
+    const Optimiser O = {A->critics[ci], A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], nullptr, nullptr, nullptr, 0.0f, nullptr};
+    return launch_update<MODE_TD3_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), &O, 1);
 }
 
 int rlt_td3_update_actor(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise) {
     if (!rlt_td3_update_supported(device, A)) return RLT_E_UNSUPPORTED;
     for (int l = 0; l < 3; l++) RLT_REQUIRE(A->actor[l].d_weights && A->actor[l].d_biases);
+    RLT_REQUIRE(sampling_noise);
     UpdateArgs a = {};
     a.actor = net_of(A->actor);
     for (int k = 0; k < 2; k++) { a.critic[k] = net_of(A->critics[0]); a.target[k] = a.critic[k]; }       // the policy gradient goes through critic 0 (:260)
     a.batch_base = A->observations_actions_base; a.noise = sampling_noise; a.sampling_std = A->sampling_std;
     a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
     a.out_pre_clip = A->actor_pre_clip;
-    const int groups = rlt_div_up(A->batch, ROWS);
-    int rc = launch_update<MODE_TD3_ACTOR>(device, a, groups, A->actor);
-    if (rc) return rc;
-    return reduce_and_step(device, a, groups, A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, nullptr, nullptr, nullptr, 0.0f);
+    const Optimiser O = {A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, nullptr, nullptr, nullptr, 0.0f, nullptr};
+    return launch_update<MODE_TD3_ACTOR>(device, a, rlt_div_up(A->batch, ROWS), &O, 1);
 }
 
 int rlt_sac_polyak_list(rlt_rocm_device* device, const float* const* sources, float* const* targets, const uint32_t* counts, int n, float polyak) {

@@ -191,3 +191,66 @@ def test_loop_by_calls_equals_the_same_calls_issued_one_by_one(rocm):
     for a, b in zip(*final):
         assert np.array_equal(a, b)
     assert np.abs(final[0][0] - params).max() > 1e-3 and np.all(np.isfinite(final[0][0]))
+
+
+@pytest.mark.parametrize("batch,obs,act,hidden_act", [(256, 3, 1, "relu"), (100, 17, 6, "tanh"), (300, 111, 8, "relu"), (1, 5, 2, "relu")])
+def test_optimiser_in_the_kernel_and_placement_leave_the_same_bits(rocm, batch, obs, act, hidden_act):
+    """The update kernel's own last step (its last workgroup adds up the partial gradients and applies Adam) against the optimiser as a launch
+    of its own, and the workgroups on one XCD against spread over all: the same sums in the same order, so every tensor is bit-identical."""
+    params, batches, noises = make_inputs(batch * 17 + act, batch, obs, act, 3)
+    results = []
+    try:
+        for tail, one_xcd in ((1, 1), (1, 0), (0, 1), (0, 0)):
+            rocm.call("set_update_options", tail, one_xcd)
+            agent = helpers.SacOnBackend(rocm, batch, 64, params, masks=False, obs=obs, act=act, hidden_act=hidden_act)
+            results.append(run_updates(agent, batches, noises))
+    finally:
+        rocm.call("set_update_options", 1, 1)
+    for other in results[1:]:
+        for key, ref in results[0].items():
+            assert np.array_equal(other[key], ref), key
+    assert results[0]["ages"].tolist() == [4] * 4
+
+
+@pytest.mark.parametrize("batch,obs,act", [(256, 3, 1), (64, 11, 3), (300, 27, 8)])
+def test_both_critics_in_one_launch_equal_the_separate_calls(oracle, rocm, batch, obs, act):
+    """rlt_rocm_sac_train_critics (both critics on the shared batch and the soft update of the targets in one launch; the noise an array or
+    drawn by the kernel from its Philox stream) against train_critic(0), train_critic(1), update_critic_targets: bit for bit, and against the
+    CPU checker's three calls to 1e-5; then train_actor with its noise drawn by the kernel against randn + train_actor."""
+    rng = np.random.default_rng(batch + obs)
+    params = agent_parameters(rng, obs, act)
+    oab, rew, term = batch_of(rng, batch, obs, act)
+    seed, stream = 77, 123
+    noise_dev = rocm.zeros((batch, act))
+    rocm.call("randn_f32", noise_dev.ptr, batch * act, seed, stream)
+    rocm.sync()
+    noise = noise_dev.numpy()
+    runs = {}
+    for name, backend in (("checker", oracle), ("separate", rocm), ("together", rocm), ("together_drawn", rocm)):
+        agent = helpers.SacOnBackend(backend, batch, 64, params, masks=False, obs=obs, act=act)
+        agent.set_batch(oab, rew, term)
+        n = backend.array(noise)
+        drawn = backend.zeros((batch, act))
+        for step in range(2):
+            if name in ("checker", "separate"):
+                for k in range(2):
+                    backend.call("sac_train_critic", C.byref(agent.c), k, n.ptr)
+                backend.call("sac_update_critic_targets", C.byref(agent.c))
+                backend.call("sac_train_actor", C.byref(agent.c), n.ptr)
+            elif name == "together":
+                backend.call("sac_train_critics", C.byref(agent.c), n.ptr, 1)
+                backend.call("sac_train_actor", C.byref(agent.c), n.ptr)
+            else:
+                backend.call("sac_train_critics_drawn", C.byref(agent.c), drawn.ptr, seed, stream, 1)
+                backend.call("sac_train_actor_drawn", C.byref(agent.c), drawn.ptr, seed, stream)
+        backend.sync()
+        runs[name] = snapshot(agent)
+        if name == "together_drawn":
+            assert np.array_equal(drawn.numpy(), noise)
+    for name in ("together", "together_drawn"):
+        for key, ref in runs["separate"].items():
+            assert np.array_equal(runs[name][key], ref), (name, key)
+    runs["checker"].pop("next_state_action_value_input"); runs["separate"].pop("next_state_action_value_input")
+    for key, ref in runs["checker"].items():
+        assert rel_err(runs["separate"][key], ref) <= TOL, key
+    assert runs["together"]["ages"].tolist() == [3] * 4
