@@ -335,8 +335,9 @@ namespace rl_tools{
                 if(d.has_head){
                     auto& noise = get_last_buffer(policy_eval_buffers).noise;
                     static_assert(utils::typing::remove_reference_t<decltype(noise)>::ROWS == N);
-                    randn(device, noise, rng);
-                    devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 2, d.layers, d.n_layers, &d.head, nullptr, noise._data, nullptr, rng.seed, random::next_stream(rng)), "step(runner, stochastic actor)");
+                    // the noise (what randn(device, noise, rng) leaves in the buffer) is drawn by the step's own launch
+                    const uint64_t noise_stream = random::next_stream(rng), initial_state_stream = random::next_stream(rng);
+                    devices::rocm::check(rlt_rocm_pendulum_runner_step_drawn(device.handle, &r, &rb, d.layers, d.n_layers, &d.head, noise._data, rng.seed, noise_stream, initial_state_stream), "step(runner, stochastic actor)");
                 }
                 else{
                     devices::rocm::check(rlt_rocm_pendulum_runner_step(device.handle, &r, &rb, 1, d.layers, d.n_layers, nullptr, nullptr, nullptr, nullptr, rng.seed, random::next_stream(rng)), "step(runner, deterministic actor)");
@@ -378,15 +379,17 @@ namespace rl_tools{
             devices::rocm::check(rlt_rocm_gather_sequence_batch(device.handle, &rb, &sampling, &draws, SPEC::MAX_EPISODE_LENGTH, &b), "gather_batch (sequences)");
             return;
         }
-        uint32_t* env_indices = nullptr; uint32_t* offsets = nullptr;
         if constexpr(!DETERMINISTIC){
-            env_indices = (uint32_t*)devices::rocm::scratch(device, 2 * sizeof(uint32_t) * BATCH_SIZE);
-            offsets = env_indices + BATCH_SIZE;
-            devices::rocm::check(rlt_rocm_gather_draw(device.handle, &rb, BATCH_SIZE, rng.seed, random::next_stream(rng), env_indices, offsets), "gather_batch (draw)");
+            // the (environment, row) pairs are drawn by the launch that copies the rows
+            devices::rocm::check(rlt_rocm_gather_batch_drawn(device.handle, &rb, rng.seed, random::next_stream(rng), nullptr, nullptr, SPEC::MAX_EPISODE_LENGTH, BATCH_SIZE,
+                                                             batch.observations_actions_base._data, batch.rewards._data, (uint8_t*)batch.terminated._data, (uint8_t*)batch.reset._data,
+                                                             (uint8_t*)batch.next_reset_base._data, (uint8_t*)batch.final_step_mask._data, (uint8_t*)batch.next_final_step_mask_base._data), "gather_batch");
         }
-        devices::rocm::check(rlt_rocm_gather_batch(device.handle, &rb, env_indices, offsets, DETERMINISTIC ? 1 : 0, SPEC::MAX_EPISODE_LENGTH, BATCH_SIZE,
-                                                   batch.observations_actions_base._data, batch.rewards._data, (uint8_t*)batch.terminated._data, (uint8_t*)batch.reset._data,
-                                                   (uint8_t*)batch.next_reset_base._data, (uint8_t*)batch.final_step_mask._data, (uint8_t*)batch.next_final_step_mask_base._data), "gather_batch");
+        else{
+            devices::rocm::check(rlt_rocm_gather_batch(device.handle, &rb, nullptr, nullptr, 1, SPEC::MAX_EPISODE_LENGTH, BATCH_SIZE,
+                                                       batch.observations_actions_base._data, batch.rewards._data, (uint8_t*)batch.terminated._data, (uint8_t*)batch.reset._data,
+                                                       (uint8_t*)batch.next_reset_base._data, (uint8_t*)batch.final_step_mask._data, (uint8_t*)batch.next_final_step_mask_base._data), "gather_batch");
+        }
     }
 }
 RL_TOOLS_NAMESPACE_WRAPPER_END

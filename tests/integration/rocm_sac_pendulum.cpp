@@ -20,6 +20,7 @@
 
 #include <rl_tools/rl/algorithms/sac/loop/core/config.h>
 #include <rl_tools/rl/algorithms/sac/loop/core/operations_generic.h>
+#include <rl_tools/rl/algorithms/sac/loop/core/operations_rocm.h>
 #include <rl_tools/rl/utils/evaluation/operations_generic.h>
 
 #include <chrono>

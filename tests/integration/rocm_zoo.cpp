@@ -44,6 +44,9 @@
 #if defined(ZOO_SAC)
 #include <pendulum-v1/sac.h>
 #include <rl_tools/rl/algorithms/sac/loop/core/operations_generic.h>
+#ifndef ZOO_DEVICE_CPU
+#include <rl_tools/rl/algorithms/sac/loop/core/operations_rocm.h>
+#endif
 #elif defined(ZOO_TD3)
 #include <pendulum-v1/td3.h>
 #include <rl_tools/rl/algorithms/td3/loop/core/operations_generic.h>
@@ -53,6 +56,9 @@
 #elif defined(ZOO_ACROBOT_SWINGUP_SAC)
 #include <acrobot-swingup-v0/sac.h>
 #include <rl_tools/rl/algorithms/sac/loop/core/operations_generic.h>
+#ifndef ZOO_DEVICE_CPU
+#include <rl_tools/rl/algorithms/sac/loop/core/operations_rocm.h>
+#endif
 #else
 #error "define ZOO_SAC, ZOO_TD3, ZOO_PPO or ZOO_ACROBOT_SWINGUP_SAC"
 #endif
