@@ -73,6 +73,7 @@ namespace rl_tools::devices{
         int hip_device_index = 0;
         bool initialized = false;
         index_t malloc_counter = 0;
+        bool graph_capture_active = false;      // the stream records a graph (devices/cuda.h:59): check_status does not wait, nothing allocates; set by devices::rocm::begin_capture
         void* scratch = nullptr;                // grow-only device memory for the draws of gather_batch (devices::rocm::scratch)
         size_t scratch_bytes = 0;
         // Parity runs against another device: when set, TD3's train_critic / train_actor take the N(0, 1) draws of the td3_sampling layer (which the reference
@@ -106,6 +107,7 @@ namespace rl_tools{
         template <typename DEVICE>
         void* scratch(DEVICE& device, size_t bytes){
             if(bytes > device.scratch_bytes){
+                if(device.graph_capture_active){ check(RLT_E_CAPTURING, "scratch (run the calls once before recording them, so that the buffer has its size)"); }
                 if(device.scratch){ check(rlt_rocm_check_status(device.handle), "scratch"); check(rlt_rocm_free(device.handle, device.scratch), "scratch"); }
                 const size_t want = bytes < 4096 ? 4096 : 2 * bytes;
                 check(rlt_rocm_malloc(device.handle, &device.scratch, want), "scratch");
@@ -113,6 +115,36 @@ namespace rl_tools{
             }
             return device.scratch;
         }
+    }
+    // Recording a stretch of calls into a graph and replaying it (the reference's CUDA programs call cudaStreamBeginCapture / cudaGraphLaunch
+    // themselves and set device.graph_capture_active around the recorded calls: src/rl/environments/pendulum/sac/cuda/sac.cu:122-164; programs
+    // on this backend are plain C++ without the HIP runtime's headers, so the calls come from the library):
+    //     devices::rocm::begin_capture(device);  step(device, ts);  auto* graph = devices::rocm::end_capture(device);
+    //     while(...){ devices::rocm::replay(device, graph); }
+    // Every operation between begin and end only records its launches. The recording ends with an advance of the device's stream offset by
+    // REPLAY_STREAM_STRIDE, so every replay of any graph draws from Philox streams no other replay or unrecorded call uses (stream numbers
+    // handed out by random::next_stream stay far below the stride).
+    namespace devices::rocm{
+        constexpr uint64_t REPLAY_STREAM_STRIDE = uint64_t(1) << 32;
+        template <typename SPEC>
+        void begin_capture(devices::ROCM<SPEC>& device){
+            check(rlt_rocm_graph_begin_capture(device.handle), "begin_capture");
+            device.graph_capture_active = true;
+        }
+        template <typename SPEC>
+        rlt_rocm_graph* end_capture(devices::ROCM<SPEC>& device){
+            rlt_rocm_graph* graph = nullptr;
+            const int advance = rlt_rocm_advance_streams(device.handle, REPLAY_STREAM_STRIDE);
+            const int end = rlt_rocm_graph_end_capture(device.handle, &graph);
+            device.graph_capture_active = false;
+            check(advance, "end_capture (stream advance)");
+            check(end, "end_capture");
+            return graph;
+        }
+        template <typename SPEC>
+        void replay(devices::ROCM<SPEC>& device, rlt_rocm_graph* graph){ check(rlt_rocm_graph_launch(device.handle, graph), "replay"); }
+        template <typename SPEC>
+        void free_graph(devices::ROCM<SPEC>& device, rlt_rocm_graph* graph){ check(rlt_rocm_graph_destroy(device.handle, graph), "free_graph"); }
     }
     // init(device)            devices/cuda.h:130-154
     template <typename SPEC>
@@ -136,6 +168,7 @@ namespace rl_tools{
     // check_status(device)    devices/cuda.h:156-174: waits for the stream and reports what went wrong since the last check
     template <typename SPEC>
     void check_status(devices::ROCM<SPEC>& device){
+        if(device.graph_capture_active){ return; }      // devices/cuda.h:163
         devices::rocm::check(device.handle ? rlt_rocm_check_status(device.handle) : RLT_E_NOT_INITIALISED, "check_status");
     }
     template <typename DEV_SPEC, typename TI>

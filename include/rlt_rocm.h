@@ -33,6 +33,7 @@ extern "C" {
 #define RLT_E_NOT_INITIALISED  (-3)
 #define RLT_E_DEVICE_TIMEOUT   (-4) /* a persistent kernel gave up waiting for another workgroup (reported by check_status) */
 #define RLT_E_WORKSPACE_TOO_SMALL (-5) /* the call needs more scratch memory than the fixed array of RLT_STATIC_SCRATCH_BYTES holds */
+#define RLT_E_CAPTURING (-6)           /* the call allocates, frees, copies to or from the host or waits while the stream records a graph */
 
 /* nn/activation_functions.h:11-18 -- same numbering as the reference enum */
 enum rlt_activation {
@@ -688,6 +689,30 @@ int rlt_rocm_set_update_options(rlt_rocm_device* device, int optimiser_in_kernel
 int rlt_rocm_sac_pendulum_loop_by_calls(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_pendulum_runner* runner,
                                         const rlt_replay_buffer* rb, int n_steps, uint64_t seed, uint64_t step_offset,
                                         const rlt_sac_loop_scratch* scratch);
+
+/* ------------------------------------------------------------ graph capture -- */
+
+/* Recording the launches of a stretch of calls into a graph and replaying it, for host loops whose speed the launches set
+ * (the reference's CUDA example captures its loop step into three graphs: src/rl/environments/pendulum/sac/cuda/sac.cu:122-164, with
+ * devices::CUDA::graph_capture_active making check_status skip its wait: devices/cuda.h:59,163).
+ *   rlt_rocm_graph_begin_capture  the handle's stream starts recording. Until rlt_rocm_graph_end_capture every entry point only records
+ *                                 its launches: none may allocate, free, copy to or from the host or wait -- those that would return
+ *                                 RLT_E_CAPTURING (rlt_rocm_malloc / _free / _memcpy_h2d / _d2h, a workspace of the library that would
+ *                                 have to grow: issue the same calls once before the capture), rlt_rocm_check_status returns 0 at once.
+ *   rlt_rocm_graph_end_capture    ends the recording (also after a failed call) and instantiates the graph.
+ *   rlt_rocm_graph_launch         enqueues one replay on the handle's stream; pointers, sizes, seeds and stream numbers are those of the
+ *                                 recording.
+ * Random numbers under replay: every draw made on the device takes its values from the Philox sequence (seed, stream + offset), where
+ * offset is a 64-bit word in device memory, zero after rlt_rocm_init. rlt_rocm_advance_streams enqueues offset += by, and can be
+ * recorded: a graph that ends with it draws fresh values on every replay, the same ones as the unrecorded calls with their stream
+ * numbers raised by `by` per repetition. rlt_rocm_set_stream_offset enqueues offset = value. */
+typedef struct rlt_rocm_graph rlt_rocm_graph;
+int rlt_rocm_graph_begin_capture(rlt_rocm_device* device);
+int rlt_rocm_graph_end_capture(rlt_rocm_device* device, rlt_rocm_graph** out_graph);
+int rlt_rocm_graph_launch(rlt_rocm_device* device, rlt_rocm_graph* graph);
+int rlt_rocm_graph_destroy(rlt_rocm_device* device, rlt_rocm_graph* graph);
+int rlt_rocm_advance_streams(rlt_rocm_device* device, uint64_t by);
+int rlt_rocm_set_stream_offset(rlt_rocm_device* device, uint64_t value);
 
 /* --------------------------------------------------------------------- PPO -- */
 

@@ -368,6 +368,8 @@ ROCM_ONLY = {
     "sac_train_critics_drawn": ([P, C.POINTER(SacAgent), P, U64, U64, I], I),
     "sac_train_actor_drawn": ([P, C.POINTER(SacAgent), P, U64, U64], I),
     "set_update_options": ([P, I, I], I),
+    "graph_begin_capture": ([P], I), "graph_end_capture": ([P, C.POINTER(P)], I), "graph_launch": ([P, P], I), "graph_destroy": ([P, P], I),
+    "advance_streams": ([P, U64], I), "set_stream_offset": ([P, U64], I),
 }
 
 

@@ -24,6 +24,8 @@ struct rlt_rocm_device {
     int sac_per_operation;       // rlt_rocm_sac_train_critic / _actor run one launch per reference operation even where the fused kernels fit
     int update_tail;             // the fused update kernels step the optimiser themselves (their last workgroup), instead of in launches after them
     int update_one_xcd;          // small grids of the fused update kernels are placed on one XCD
+    int capturing;               // the stream is recording a graph: nothing may allocate, free or wait (rlt_rocm_graph_begin_capture)
+    uint64_t* stream_offset;     // device word added to the stream number of every draw made on the device (rlt_rocm_advance_streams)
 };
 
 #define RLT_HIP(expr)                                                        \
@@ -33,6 +35,8 @@ struct rlt_rocm_device {
     } while (0)
 
 #define RLT_REQUIRE(cond) do { if (!(cond)) return RLT_E_INVALID_ARGUMENT; } while (0)
+// for entry points that allocate, free, copy to or from the host or wait: not while the stream records a graph
+#define RLT_NOT_WHILE_CAPTURING() do { if (device->capturing) return RLT_E_CAPTURING; } while (0)
 
 // Grow-only scratch owned by the device handle.
 int rlt_scratch(rlt_rocm_device* device, size_t bytes, void** out);

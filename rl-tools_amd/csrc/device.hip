@@ -15,6 +15,7 @@ int rlt_launch_status(rlt_rocm_device* device) {
 
 int rlt_scratch(rlt_rocm_device* device, size_t bytes, void** out) {
     if (bytes > device->scratch_bytes) {
+        if (device->capturing) return RLT_E_CAPTURING;      // the workspace grows on a warm-up call before the capture
         if (device->scratch) RLT_HIP(hipFree(device->scratch));   // hipFree waits for the work that still uses it
         device->scratch = nullptr; device->scratch_bytes = 0;
         size_t want = bytes < (size_t)(1u << 20) ? (size_t)(1u << 20) : bytes + bytes / 4;
@@ -57,8 +58,9 @@ __global__ __launch_bounds__(256) void scale_kernel(float* __restrict__ x, size_
 
 // randn / rand: element i is word i % 4 of Philox group i / 4 of the call's stream (rng.h). Two calls with different `stream` values
 // (or different seeds) share no group, whatever their lengths.
-__global__ __launch_bounds__(256) void rand_kernel(float* __restrict__ dst, size_t count, float low, float high, uint64_t seed, uint64_t stream, int normal) {
+__global__ __launch_bounds__(256) void rand_kernel(float* __restrict__ dst, size_t count, float low, float high, uint64_t seed, uint64_t stream, int normal, const uint64_t* __restrict__ stream_offset) {
     const size_t quads = (count + 3) / 4;
+    stream += *stream_offset;
     for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (size_t)gridDim.x * blockDim.x) {
         const rlt_u32x4 r = rlt_philox(seed, stream, q);
         float v[4];
@@ -76,8 +78,9 @@ __global__ __launch_bounds__(256) void rand_kernel(float* __restrict__ dst, size
     }
 }
 // the raw 32-bit words of a stream, for checking the generator against a host restatement
-__global__ __launch_bounds__(256) void rand_bits_kernel(uint32_t* __restrict__ dst, size_t count, uint64_t seed, uint64_t stream) {
+__global__ __launch_bounds__(256) void rand_bits_kernel(uint32_t* __restrict__ dst, size_t count, uint64_t seed, uint64_t stream, const uint64_t* __restrict__ stream_offset) {
     const size_t quads = (count + 3) / 4;
+    stream += *stream_offset;
     for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (size_t)gridDim.x * blockDim.x) {
         const rlt_u32x4 r = rlt_philox(seed, stream, q);
         const uint32_t v[4] = {r.x, r.y, r.z, r.w};
@@ -132,6 +135,7 @@ int rlt_rocm_init(int hip_device_index, rlt_rocm_device** out_device) {
     if (e == hipSuccess) e = hipMemset(device->counters, 0, 8192);
     if (e != hipSuccess) { (void)hipStreamDestroy(device->own_stream); delete device; return (int)e; }
     device->fault = (unsigned*)((char*)device->counters + 8192 - 64);   // the last 64 bytes of the block are never used as counters
+    device->stream_offset = (uint64_t*)((char*)device->counters + 8192 - 128);      // zero: stream numbers mean what the caller passes
     // Dispatch order over the XCDs: probe twice with 64 workgroups; if workgroup b always shares its XCD with b + 8 (and with no
     // workgroup in between), persistent kernels may place a small grid on one XCD by using every 8th workgroup of a larger one.
     {
@@ -179,6 +183,7 @@ int rlt_rocm_destroy(rlt_rocm_device* device) {
 }
 int rlt_rocm_check_status(rlt_rocm_device* device) {
     if (!device) return RLT_E_NOT_INITIALISED;
+    if (device->capturing) return 0;      // nothing runs while the stream records (devices/cuda.h:163: check_status does not wait under capture)
     hipError_t e = hipStreamSynchronize(device->stream);
     if (e != hipSuccess) device->sticky_error = (int)e;
     if (device->fault_armed && e == hipSuccess) {
@@ -205,6 +210,7 @@ const char* rlt_rocm_error_string(int code) {
     if (code == RLT_E_UNSUPPORTED) return "rlt_rocm: shape outside what the kernels support";
     if (code == RLT_E_DEVICE_TIMEOUT) return "rlt_rocm: a persistent kernel gave up waiting for another workgroup; its results are invalid";
     if (code == RLT_E_NOT_INITIALISED) return "rlt_rocm: device handle not initialised";
+    if (code == RLT_E_CAPTURING) return "rlt_rocm: the call allocates, frees, copies to or from the host or waits, which a stream that records a graph cannot do (size the workspaces with a call before the capture)";
     if (code == RLT_E_WORKSPACE_TOO_SMALL) return "rlt_rocm: the call needs more scratch memory than the library's fixed array (RLT_STATIC_SCRATCH_BYTES) holds; use the allocating entry point or a smaller batch";
     if (code > 0) return hipGetErrorString((hipError_t)code);
     return "rlt_rocm: unknown error";
@@ -219,18 +225,21 @@ int rlt_rocm_device_info(rlt_rocm_device* device, int* compute_units, int* lds_b
 
 int rlt_rocm_malloc(rlt_rocm_device* device, void** out_ptr, size_t bytes) {
     if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_NOT_WHILE_CAPTURING();
     RLT_REQUIRE(out_ptr && bytes > 0);
     RLT_HIP(hipMalloc(out_ptr, bytes));
     return 0;
 }
 int rlt_rocm_free(rlt_rocm_device* device, void* ptr) {
     if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_NOT_WHILE_CAPTURING();
     if (!ptr) return 0;
     RLT_HIP(hipFree(ptr));
     return 0;
 }
 int rlt_rocm_memcpy_h2d(rlt_rocm_device* device, void* dst, const void* src_host, size_t bytes) {
     if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_NOT_WHILE_CAPTURING();
     RLT_REQUIRE(dst && src_host);
     if (bytes == 0) return 0;
     RLT_HIP(hipMemcpyAsync(dst, src_host, bytes, hipMemcpyHostToDevice, device->stream));
@@ -239,6 +248,7 @@ int rlt_rocm_memcpy_h2d(rlt_rocm_device* device, void* dst, const void* src_host
 }
 int rlt_rocm_memcpy_d2h(rlt_rocm_device* device, void* dst_host, const void* src, size_t bytes) {
     if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_NOT_WHILE_CAPTURING();
     RLT_REQUIRE(dst_host && src);
     if (bytes == 0) return 0;
     RLT_HIP(hipMemcpyAsync(dst_host, src, bytes, hipMemcpyDeviceToHost, device->stream));
@@ -259,7 +269,7 @@ int rlt_rocm_memcpy2d(rlt_rocm_device* device, void* dst, size_t dst_pitch, cons
     if (width_bytes == 0 || rows == 0) return 0;
     hipMemcpyKind k = kind == 0 ? hipMemcpyDeviceToDevice : (kind == 1 ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost);
     RLT_HIP(hipMemcpy2DAsync(dst, dst_pitch, src, src_pitch, width_bytes, rows, k, device->stream));
-    if (kind != 0) RLT_HIP(hipStreamSynchronize(device->stream));
+    if (kind != 0) { RLT_NOT_WHILE_CAPTURING(); RLT_HIP(hipStreamSynchronize(device->stream)); }
     return 0;
 }
 int rlt_rocm_fill_f32(rlt_rocm_device* device, float* dst, int rows, int cols, int ld, float value) {
@@ -285,21 +295,21 @@ int rlt_rocm_rand_bits_u32(rlt_rocm_device* device, uint32_t* dst, size_t count,
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(dst);
     if (count == 0) return 0;
-    hipLaunchKernelGGL(rand_bits_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, seed, stream);
+    hipLaunchKernelGGL(rand_bits_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, seed, stream, (const uint64_t*)device->stream_offset);
     return rlt_launch_status(device);
 }
 int rlt_rocm_randn_f32(rlt_rocm_device* device, float* dst, size_t count, uint64_t seed, uint64_t stream) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(dst);
     if (count == 0) return 0;
-    hipLaunchKernelGGL(rand_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, 0.0f, 1.0f, seed, stream, 1);
+    hipLaunchKernelGGL(rand_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, 0.0f, 1.0f, seed, stream, 1, (const uint64_t*)device->stream_offset);
     return rlt_launch_status(device);
 }
 int rlt_rocm_rand_f32(rlt_rocm_device* device, float* dst, size_t count, float low, float high, uint64_t seed, uint64_t stream) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(dst);
     if (count == 0) return 0;
-    hipLaunchKernelGGL(rand_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, low, high, seed, stream, 0);
+    hipLaunchKernelGGL(rand_kernel, dim3(grid_for((count + 3) / 4)), dim3(256), 0, device->stream, dst, count, low, high, seed, stream, 0, (const uint64_t*)device->stream_offset);
     return rlt_launch_status(device);
 }
 int rlt_rocm_scale_f32(rlt_rocm_device* device, float* x, size_t count, float s, int reciprocal) {
@@ -323,4 +333,61 @@ int rlt_rocm_reduce_sum_f32(rlt_rocm_device* device, const float* x, size_t coun
     return rlt_launch_status(device);
 }
 
+}  // extern "C"
+
+namespace {
+__global__ void advance_streams_kernel(uint64_t* __restrict__ offset, uint64_t by, int absolute) { *offset = absolute ? by : *offset + by; }
+}
+struct rlt_rocm_graph { hipGraph_t graph; hipGraphExec_t executable; };
+
+extern "C" {
+int rlt_rocm_advance_streams(rlt_rocm_device* device, uint64_t by) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    hipLaunchKernelGGL(advance_streams_kernel, dim3(1), dim3(1), 0, device->stream, device->stream_offset, by, 0);
+    return rlt_launch_status(device);
+}
+int rlt_rocm_set_stream_offset(rlt_rocm_device* device, uint64_t value) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    hipLaunchKernelGGL(advance_streams_kernel, dim3(1), dim3(1), 0, device->stream, device->stream_offset, value, 1);
+    return rlt_launch_status(device);
+}
+int rlt_rocm_graph_begin_capture(rlt_rocm_device* device) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_NOT_WHILE_CAPTURING();
+    RLT_HIP(hipStreamBeginCapture(device->stream, hipStreamCaptureModeGlobal));
+    device->capturing = 1;
+    return 0;
+}
+int rlt_rocm_graph_end_capture(rlt_rocm_device* device, rlt_rocm_graph** out_graph) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(device->capturing);
+    hipGraph_t graph = nullptr;
+    const hipError_t e = hipStreamEndCapture(device->stream, &graph);      // ends the recording also where a recorded call failed
+    device->capturing = 0;
+    if (e != hipSuccess) { device->sticky_error = (int)e; if (out_graph) *out_graph = nullptr; return (int)e; }
+    if (!out_graph) { (void)hipGraphDestroy(graph); return RLT_E_INVALID_ARGUMENT; }
+    hipGraphExec_t executable = nullptr;
+    const hipError_t e2 = hipGraphInstantiate(&executable, graph, nullptr, nullptr, 0);
+    if (e2 != hipSuccess) { (void)hipGraphDestroy(graph); device->sticky_error = (int)e2; *out_graph = nullptr; return (int)e2; }
+    *out_graph = new rlt_rocm_graph{graph, executable};
+    return 0;
+}
+int rlt_rocm_graph_launch(rlt_rocm_device* device, rlt_rocm_graph* graph) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(graph && graph->executable);
+    RLT_NOT_WHILE_CAPTURING();
+    device->fault_armed = 1;      // a recorded kernel may be one that waits for other workgroups
+    RLT_HIP(hipGraphLaunch(graph->executable, device->stream));
+    return 0;
+}
+int rlt_rocm_graph_destroy(rlt_rocm_device* device, rlt_rocm_graph* graph) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    if (!graph) return 0;
+    RLT_NOT_WHILE_CAPTURING();
+    RLT_HIP(hipStreamSynchronize(device->stream));
+    (void)hipGraphExecDestroy(graph->executable);
+    (void)hipGraphDestroy(graph->graph);
+    delete graph;
+    return 0;
+}
 }  // extern "C"

@@ -85,6 +85,7 @@ int rlt_unpad_gradients(rlt_rocm_device* device, const rlt_dense_layer* L, const
 }
 int rlt_pad_scratch(rlt_rocm_device* device, size_t bytes, void** out) {
     if (bytes > device->pad_scratch_bytes) {
+        if (device->capturing) return RLT_E_CAPTURING;
         if (device->pad_scratch) RLT_HIP(hipFree(device->pad_scratch));      // hipFree waits for the work that still uses it
         device->pad_scratch = nullptr; device->pad_scratch_bytes = 0;
         const size_t want = bytes < (size_t)(1u << 18) ? (size_t)(1u << 18) : bytes + bytes / 4;

@@ -70,8 +70,9 @@ __global__ __launch_bounds__(256) void gather_kernel(rlt_replay_buffer rb, const
                                                      int deterministic, int max_episode_length, int batch, float* __restrict__ oab, float* __restrict__ rewards,
                                                      uint8_t* __restrict__ terminated, uint8_t* __restrict__ reset, uint8_t* __restrict__ next_reset_base,
                                                      uint8_t* __restrict__ final_step_mask, uint8_t* __restrict__ next_final_step_mask_base, int* __restrict__ error_flag,
-                                                     int draw, uint64_t seed, uint64_t stream, uint32_t* __restrict__ drawn_env_indices, uint32_t* __restrict__ drawn_sample_offsets) {
+                                                     int draw, uint64_t seed, uint64_t stream, uint32_t* __restrict__ drawn_env_indices, uint32_t* __restrict__ drawn_sample_offsets, const uint64_t* __restrict__ stream_offset) {
     const int OBS = rb.observation_dim, ACT = rb.action_dim, R = 2 * OBS + ACT + 3, D = OBS + ACT;
+    if (draw) stream += *stream_offset;
     const int sub = threadIdx.x & 15;
     for (int i = (blockIdx.x * blockDim.x + threadIdx.x) >> 4; i < batch; i += (gridDim.x * blockDim.x) >> 4) {
         uint32_t e, offset;
@@ -183,7 +184,8 @@ __global__ __launch_bounds__(256) void gather_sequence_kernel(rlt_replay_buffer 
     }
 }
 
-__global__ __launch_bounds__(256) void gather_draw_kernel(rlt_replay_buffer rb, int batch, uint64_t seed, uint64_t stream, uint32_t* __restrict__ env_indices, uint32_t* __restrict__ sample_offsets) {
+__global__ __launch_bounds__(256) void gather_draw_kernel(rlt_replay_buffer rb, int batch, uint64_t seed, uint64_t stream, uint32_t* __restrict__ env_indices, uint32_t* __restrict__ sample_offsets, const uint64_t* __restrict__ stream_offset) {
+    stream += *stream_offset;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < batch; i += gridDim.x * blockDim.x) {
         const rlt_u32x4 draw = rlt_philox(seed, stream, (uint64_t)i);   // sample i takes words 0 and 1 of group i of the call's stream
         const uint32_t r1 = draw.y;
@@ -198,7 +200,8 @@ __global__ __launch_bounds__(256) void gather_draw_kernel(rlt_replay_buffer rb, 
 // stream, G = ceil((3 padded + 3) / 4), in the order environment, padded offsets, padded + 1 nominal decisions, padded + 1 lengths.
 __global__ __launch_bounds__(256) void gather_sequence_draw_kernel(rlt_replay_buffer rb, rlt_sequence_sampling P, int max_episode_length, int batch, int sequence_length, uint64_t seed,
                                                                    uint64_t stream, uint32_t* __restrict__ env_indices, uint32_t* __restrict__ sample_offsets,
-                                                                   uint8_t* __restrict__ nominal, uint32_t* __restrict__ lengths) {
+                                                                   uint8_t* __restrict__ nominal, uint32_t* __restrict__ lengths, const uint64_t* __restrict__ stream_offset) {
+    stream += *stream_offset;
     const int PADDED = sequence_length + 1, WORDS = 3 * PADDED + 3, G = (WORDS + 3) / 4;
     for (int b = blockIdx.x * blockDim.x + threadIdx.x; b < batch; b += gridDim.x * blockDim.x) {
         uint32_t env = 0, eligible = 0;
@@ -222,7 +225,8 @@ __global__ __launch_bounds__(256) void gather_sequence_draw_kernel(rlt_replay_bu
 
 // prologue of the runner step (operations_generic_per_env.h:8-66): reset where truncated, flag the previous replay row, observe
 __global__ __launch_bounds__(256) void runner_prologue_kernel(rlt_pendulum_runner rn, rlt_replay_buffer rb, const float* __restrict__ initial_states, uint64_t seed, uint64_t stream,
-                                                              float* __restrict__ observations) {
+                                                              float* __restrict__ observations, const uint64_t* __restrict__ stream_offset) {
+    stream += *stream_offset;
     const int R = 2 * rb.observation_dim + rb.action_dim + 3;
     for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) {
         if (rn.truncated[e]) {
@@ -299,6 +303,7 @@ struct FusedRunnerArgs {
     rlt_sas_parameters sas;
     const float* action_noise; const float* initial_states;
     uint64_t seed, stream;
+    const uint64_t* stream_offset;                  // added to both stream numbers
     uint64_t noise_stream; float* drawn_noise;      // action_noise == NULL: element e of the standard-normal stream (seed, noise_stream), also written to drawn_noise if given
 };
 
@@ -334,14 +339,14 @@ __global__ __launch_bounds__(64 * FWAVES) void runner_fused_kernel(FusedRunnerAr
             th = st.x; thd = st.y; ep_step = A.rn.episode_step[e]; ep_ret = A.rn.episode_return[e];
             pos = A.rb.position[e]; ces = A.rb.current_episode_start[e]; full = A.rb.full[e];
             if (A.policy_kind == 2) {
-                noise = A.action_noise ? A.action_noise[e] : rlt_randn_element(A.seed, A.noise_stream, (uint64_t)e);
+                noise = A.action_noise ? A.action_noise[e] : rlt_randn_element(A.seed, A.noise_stream + *A.stream_offset, (uint64_t)e);
                 if (A.drawn_noise) A.drawn_noise[e] = noise;
             }
             if (A.rn.truncated[e]) {    // prologue (operations_generic_per_env.h:8-66): reset, flag the previous replay row
                 if (A.initial_states) { const float2 ini = reinterpret_cast<const float2*>(A.initial_states)[e]; th = ini.x; thd = ini.y; }
                 else {
                     const float PI = 3.14159265358979323846f;
-                    const rlt_u32x4 draw = rlt_philox(A.seed, A.stream, (uint64_t)e);
+                    const rlt_u32x4 draw = rlt_philox(A.seed, A.stream + *A.stream_offset, (uint64_t)e);
                     const float u0 = rlt_u01(draw.x), u1 = rlt_u01(draw.y);
                     th = -PI + 2.0f * PI * u0; thd = -1.0f + 2.0f * u1;
                 }
@@ -708,7 +713,7 @@ int rlt_rocm_gather_batch(rlt_rocm_device* device, const rlt_replay_buffer* rb, 
     device->fault_armed = 1;
     hipLaunchKernelGGL(gather_kernel, dim3(grid1(batch * 16)), dim3(256), 0, device->stream, *rb, env_indices, sample_offsets, deterministic, max_episode_length, batch,
                        observations_actions_base, rewards, terminated, reset, next_reset_base, final_step_mask, next_final_step_mask_base, error_flag, 0, (uint64_t)0, (uint64_t)0,
-                       (uint32_t*)nullptr, (uint32_t*)nullptr);
+                       (uint32_t*)nullptr, (uint32_t*)nullptr, (const uint64_t*)device->stream_offset);
     return rlt_launch_status(device);
 }
 
@@ -721,7 +726,7 @@ int rlt_rocm_gather_batch_drawn(rlt_rocm_device* device, const rlt_replay_buffer
     device->fault_armed = 1;
     hipLaunchKernelGGL(gather_kernel, dim3(grid1(batch * 16)), dim3(256), 0, device->stream, *rb, (const uint32_t*)nullptr, (const uint32_t*)nullptr, 0, max_episode_length, batch,
                        observations_actions_base, rewards, terminated, reset, next_reset_base, final_step_mask, next_final_step_mask_base, error_flag, 1, seed, stream,
-                       drawn_env_indices, drawn_sample_offsets);
+                       drawn_env_indices, drawn_sample_offsets, (const uint64_t*)device->stream_offset);
     return rlt_launch_status(device);
 }
 
@@ -740,7 +745,7 @@ int rlt_rocm_gather_sequence_batch(rlt_rocm_device* device, const rlt_replay_buf
 int rlt_rocm_gather_draw(rlt_rocm_device* device, const rlt_replay_buffer* rb, int batch, uint64_t seed, uint64_t stream, uint32_t* env_indices, uint32_t* sample_offsets) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(rb_ok(rb) && batch > 0 && env_indices && sample_offsets);
-    hipLaunchKernelGGL(gather_draw_kernel, dim3(grid1(batch)), dim3(256), 0, device->stream, *rb, batch, seed, stream, env_indices, sample_offsets);
+    hipLaunchKernelGGL(gather_draw_kernel, dim3(grid1(batch)), dim3(256), 0, device->stream, *rb, batch, seed, stream, env_indices, sample_offsets, (const uint64_t*)device->stream_offset);
     return rlt_launch_status(device);
 }
 
@@ -750,7 +755,7 @@ int rlt_rocm_gather_sequence_draw(rlt_rocm_device* device, const rlt_replay_buff
     RLT_REQUIRE(rb_ok(rb) && sampling && batch > 0 && sequence_length >= 1 && max_episode_length >= 0 && env_indices && sample_offsets && nominal && lengths);
     RLT_REQUIRE(!sampling->always_sample_from_initial_state || rb->capacity > max_episode_length);
     hipLaunchKernelGGL(gather_sequence_draw_kernel, dim3(grid1(batch)), dim3(256), 0, device->stream, *rb, *sampling, max_episode_length, batch, sequence_length, seed, stream,
-                       env_indices, sample_offsets, nominal, lengths);
+                       env_indices, sample_offsets, nominal, lengths, (const uint64_t*)device->stream_offset);
     return rlt_launch_status(device);
 }
 
@@ -801,7 +806,7 @@ static int runner_step(rlt_rocm_device* device, const rlt_pendulum_runner* rn, c
         a.act_hidden = actor[0].activation; a.act_out = actor[2].activation; a.out_dim = actor[2].out_dim; a.policy_kind = policy_kind;
         if (sas) a.sas = *sas;
         a.action_noise = action_noise; a.initial_states = initial_states; a.seed = seed; a.stream = stream;
-        a.noise_stream = noise_stream; a.drawn_noise = action_noise ? nullptr : drawn_noise;
+        a.noise_stream = noise_stream; a.drawn_noise = action_noise ? nullptr : drawn_noise; a.stream_offset = device->stream_offset;
         const int tiles = rlt_div_up(N, FTILE);
         int blocks = rlt_div_up(tiles, FWAVES); if (blocks > device->compute_units) blocks = device->compute_units;
         switch (a.act_hidden) {
@@ -820,7 +825,7 @@ static int runner_step(rlt_rocm_device* device, const rlt_pendulum_runner* rn, c
     void* scratch; int rc = rlt_scratch(device, head + mlp_ws, &scratch); if (rc) return rc;
     float* obs = (float*)scratch; float* actor_out = obs + (size_t)N * 3; float* actions = actor_out + (size_t)N * 2; float* lp = actions + N;
     void* ws = (char*)scratch + head;
-    hipLaunchKernelGGL(runner_prologue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *rb, initial_states, seed, stream, obs);
+    hipLaunchKernelGGL(runner_prologue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *rb, initial_states, seed, stream, obs, (const uint64_t*)device->stream_offset);
     if ((rc = rlt_launch_status(device))) return rc;
     const float* act_ptr = actions;
     if (policy_kind == 0) act_ptr = actions_in;
@@ -853,7 +858,7 @@ int rlt_rocm_pendulum_runner_step_recurrent(rlt_rocm_device* device, const rlt_p
     char* w = reinterpret_cast<char*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
     float* obs = (float*)w; float* policy_out = obs + (size_t)N * 3; float* actions = policy_out + (size_t)N * 2; float* lp = actions + N;
     int rc;
-    hipLaunchKernelGGL(runner_prologue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *rb, initial_states, (uint64_t)0, (uint64_t)0, obs);
+    hipLaunchKernelGGL(runner_prologue_kernel, dim3(grid1(N)), dim3(256), 0, device->stream, *rn, *rb, initial_states, (uint64_t)0, (uint64_t)0, obs, (const uint64_t*)device->stream_offset);
     if ((rc = rlt_launch_status(device))) return rc;
     if ((rc = rlt_rocm_seq_reset_state(device, policy, n_layers, state, rn->truncated, N))) return rc;
     if ((rc = rlt_rocm_seq_evaluate_step(device, policy, n_layers, obs, 3, state, auto_reset_period, policy_out, 2, N, w + head, step_ws))) return rc;

@@ -61,7 +61,7 @@ struct UpdateArgs {
     float* out_pre_clip;                   // actor update: [batch][act], the sampling layer's value before the clamp
     // noise == NULL: element i of the noise is element i of the standard-normal stream (noise_seed, noise_stream), what
     // rlt_rocm_randn_f32 would have put there; out_noise (optional) receives the values
-    uint64_t noise_seed, noise_stream; float* out_noise;
+    uint64_t noise_seed, noise_stream; float* out_noise; const uint64_t* stream_offset;      // *stream_offset is added to noise_stream
     // every 8th workgroup of an 8 x larger grid works, so that all of them run on one XCD and share its L2 (the device hands out
     // workgroups round robin over the XCDs)
     int packed;
@@ -453,7 +453,7 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
         for (int j = 0; j < 2; j++) {
             if (kk + 4 * j < ACT && row0 + r < B) {
                 const size_t i = (size_t)(row0 + r) * ACT + kk + 4 * j;
-                noise[j] = A.noise ? A.noise[i] : rlt_randn_element(A.noise_seed, A.noise_stream, i);
+                noise[j] = A.noise ? A.noise[i] : rlt_randn_element(A.noise_seed, A.noise_stream + *A.stream_offset, i);
                 if (A.out_noise && y == 0) A.out_noise[i] = noise[j];
             }
         }
@@ -798,6 +798,7 @@ int launch_update(rlt_rocm_device* device, UpdateArgs& a, int groups, const Opti
     int rc = rlt_scratch(device, (size_t)n_opts * groups * a.count * sizeof(float), &scratch);
     if (rc) return rc;
     a.partial = (float*)scratch;
+    a.stream_offset = device->stream_offset;
     const bool tail = configure_tail(device, a, opts, n_opts, groups, polyak);
     if (tail) device->fault_armed = 1;
     // up to 32 workgroups (one per compute unit of an XCD) are placed on one XCD where the device hands out workgroups round robin

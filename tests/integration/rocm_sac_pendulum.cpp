@@ -3,6 +3,9 @@
 // Only the device type and the two ROCM includes differ from a CPU program; every operation the loop calls resolves to an overload of this
 // backend. Evaluation runs on the CPU device on a copy of the actor, as in the CUDA program.
 //
+// Built with -DSAC_LOOP_GRAPH the loop step past the warm-up is recorded once into a graph and replayed (the counterpart of the CUDA program's three
+// graphs, sac.cu:122-164); -DSAC_LOOP_HIDDEN_WIDTH=<n> sets the width of all networks (64 unless given).
+//
 // Usage: rocm_sac_pendulum [n_steps [seed [batch-size tag ignored]]] ; prints "step <n> mean_return <r>" lines and a last line "final <r>".
 #include <rl_tools/operations/cpu_mux.h>
 #include <rl_tools/operations/rocm.h>
@@ -40,6 +43,9 @@ using ENVIRONMENT = rlt::rl::environments::Pendulum<PENDULUM_SPEC>;
 #ifndef BATCH_SIZE
 #define BATCH_SIZE 256
 #endif
+#ifndef SAC_LOOP_HIDDEN_WIDTH
+#define SAC_LOOP_HIDDEN_WIDTH 64
+#endif
 struct LOOP_CORE_PARAMETERS: rlt::rl::algorithms::sac::loop::core::DefaultParameters<TYPE_POLICY, TI, ENVIRONMENT>{
     struct SAC_PARAMETERS: rlt::rl::algorithms::sac::DefaultParameters<TYPE_POLICY, TI, ENVIRONMENT::ACTION_DIM>{
         static constexpr TI ACTOR_BATCH_SIZE = BATCH_SIZE;
@@ -51,9 +57,9 @@ struct LOOP_CORE_PARAMETERS: rlt::rl::algorithms::sac::loop::core::DefaultParame
     static constexpr TI STEP_LIMIT = 10000;
     static constexpr TI REPLAY_BUFFER_CAP = STEP_LIMIT;
     static constexpr TI ACTOR_NUM_LAYERS = 3;
-    static constexpr TI ACTOR_HIDDEN_DIM = 64;
+    static constexpr TI ACTOR_HIDDEN_DIM = SAC_LOOP_HIDDEN_WIDTH;
     static constexpr TI CRITIC_NUM_LAYERS = 3;
-    static constexpr TI CRITIC_HIDDEN_DIM = 64;
+    static constexpr TI CRITIC_HIDDEN_DIM = SAC_LOOP_HIDDEN_WIDTH;
     static constexpr bool COLLECT_EPISODE_STATS = false;
     static constexpr TI EPISODE_STATS_BUFFER_SIZE = 0;
 };
@@ -91,18 +97,51 @@ int main(int argc, char** argv){
     std::printf("step 0 mean_return %f\n", (double)evaluate());
     rlt::check_status(device);
     const auto start = std::chrono::steady_clock::now();
-    double training_seconds = 0;
+    auto stretch_start = start;
+    double training_seconds = 0, training_only_seconds = 0;
+#ifdef SAC_LOOP_GRAPH
+    rlt_rocm_graph* step_graph = nullptr;
+#endif
     for(TI step = 0; step < n_steps; step++){
+#ifdef SAC_LOOP_GRAPH
+        // past the warm-up every loop step issues the same launches: the first few run as they are (which also sizes every workspace), one is
+        // recorded, the rest are replays of it; the step counter, which the recorded calls do not read, advances on the host
+        bool finished = false;
+        if(ts.step < LOOP_CORE_PARAMETERS::N_WARMUP_STEPS + 3){
+            finished = rlt::step(device, ts);
+        }
+        else{
+            if(!step_graph){
+                const TI recorded_at = ts.step;
+                rlt::devices::rocm::begin_capture(device);
+                rlt::step(device, ts);
+                step_graph = rlt::devices::rocm::end_capture(device);
+                ts.step = recorded_at;      // recorded, not run
+            }
+            finished = ts.step >= LOOP_CORE_PARAMETERS::STEP_LIMIT;
+            if(!finished){
+                rlt::devices::rocm::replay(device, step_graph);
+                ts.step++;
+            }
+        }
+#else
         const bool finished = rlt::step(device, ts);
+#endif
         if((step + 1) % 1000 == 0 || step + 1 == n_steps || finished){
             rlt::check_status(device);
             training_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - start).count();
+            training_only_seconds += std::chrono::duration<double>(std::chrono::steady_clock::now() - stretch_start).count();
             std::printf("step %u mean_return %f\n", (unsigned)(step + 1), (double)evaluate());
             std::fflush(stdout);
+            stretch_start = std::chrono::steady_clock::now();
         }
         if(finished){ break; }
     }
-    std::printf("final %f loop_steps_per_second_including_evaluations %f\n", (double)evaluate(), (double)ts.step / training_seconds);
+    std::printf("final %f loop_steps_per_second_including_evaluations %f loop_steps_per_second_between_evaluations %f\n", (double)evaluate(), (double)ts.step / training_seconds,
+                (double)ts.step / training_only_seconds);
+#ifdef SAC_LOOP_GRAPH
+    rlt::devices::rocm::free_graph(device, step_graph);
+#endif
     rlt::free(device, ts);
     rlt::free(device_evaluation, actor_evaluation);
     rlt::free(device);

@@ -1,0 +1,102 @@
+"""Graph capture through the C ABI (rlt_rocm_graph_*; the reference's CUDA example records its loop step the same way,
+src/rl/environments/pendulum/sac/cuda/sac.cu:122-164, devices/cuda.h:59,163): one SAC loop step recorded once and replayed must leave, bit
+for bit, what the same number of unrecorded loop steps leaves -- parameters of all five networks, optimiser state, replay rows, runner state --
+with fresh random numbers on every replay (the recorded graph ends by advancing the device's stream offset)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import helpers
+from test_rocm_sac_update import agent_parameters
+
+pytestmark = pytest.mark.gpu
+
+RLT_E_CAPTURING = -6
+
+
+class Loop:
+    """agent, one Pendulum environment, its replay ring and the scratch arrays of rlt_rocm_sac_pendulum_loop_by_calls, warmed up with uniform actions"""
+
+    def __init__(self, rocm, batch, hidden, capacity, seed):
+        capi = helpers.capi
+        self.rocm, self.seed = rocm, seed
+        params = agent_parameters(np.random.default_rng(hidden), 3, 1, hidden)
+        self.agent = helpers.SacOnBackend(rocm, batch, hidden, params, masks=False)
+        self.rb = helpers.ReplayOnBackend(rocm, 1, capacity)
+        self.states, self.ep_step, self.ep_ret, self.trunc = rocm.zeros((1, 2)), rocm.zeros((1,), np.uint32), rocm.zeros((1,)), rocm.array(np.ones(1, np.uint8))
+        self.runner = capi.PendulumRunner(self.states.ptr, self.ep_step.ptr, self.ep_ret.ptr, self.trunc.ptr, 1, 200, capi.pendulum_parameters())
+        self.buffers = [rocm.zeros((1, 1)), rocm.zeros((batch, 1)), rocm.zeros((batch, 1)), rocm.zeros((batch,), np.uint32), rocm.zeros((batch,), np.uint32)]
+        self.scratch = capi.SacLoopScratch(*[b.ptr for b in self.buffers])
+        warm_action = rocm.zeros((1, 1))
+        for c in range(batch + 10):
+            rocm.call("rand_f32", warm_action.ptr, 1, -1.0, 1.0, seed, 8 * c + 1)
+            rocm.call("pendulum_runner_step", C.byref(self.runner), C.byref(self.rb.c), 0, self.agent.actor.layers, 3, C.byref(self.agent.c.sas), warm_action.ptr, None, None, seed, 8 * c + 2)
+
+    def steps(self, n, first):
+        self.rocm.call("sac_pendulum_loop_by_calls", C.byref(self.agent.c), C.byref(self.runner), C.byref(self.rb.c), n, self.seed, first, C.byref(self.scratch))
+
+    def state(self):
+        self.rocm.sync()
+        return [self.agent.parameters(), self.agent.actor.m.numpy(), self.agent.critics[1].v.numpy(), self.rb.data.numpy(), self.states.numpy(), self.ep_ret.numpy(),
+                self.agent.actor.age.numpy(), self.buffers[1].numpy(), self.buffers[3].numpy()]
+
+
+def record_one_step(rocm, loop, first):
+    graph = C.c_void_p()
+    rocm.call("graph_begin_capture")
+    try:
+        loop.steps(1, first)
+        rocm.call("advance_streams", 8)       # a loop step of the host loop uses the streams 8 g + 1 .. 8 g + 5
+    finally:
+        rocm.call("graph_end_capture", C.byref(graph))
+    return graph
+
+
+@pytest.mark.parametrize("hidden,batch,replays", [(64, 256, 1000), (256, 256, 1000)])
+def test_replays_of_a_recorded_loop_step_equal_the_unrecorded_steps(rocm, hidden, batch, replays):
+    """hidden 64: four launches per step (the fused kernels); hidden 256: the zoo's wider agents, one launch per operation (about sixty)"""
+    first, chunk = 5000, replays // 5
+    eager = Loop(rocm, batch, hidden, 1500, 21)
+    eager.steps(3, first - 3)          # sizes every workspace the recorded calls will need
+    checkpoints = []
+    for k in range(5):
+        eager.steps(chunk, first + k * chunk)
+        checkpoints.append(eager.state())
+    recorded = Loop(rocm, batch, hidden, 1500, 21)
+    recorded.steps(3, first - 3)
+    graph = record_one_step(rocm, recorded, first)
+    try:
+        for k in range(5):
+            for _ in range(chunk):
+                rocm.call("graph_launch", graph)
+            # between the chunks the program reads everything back (waits, eager copies): every chunk of replays is checked, not only the last
+            for got, ref in zip(recorded.state(), checkpoints[k]):
+                assert np.array_equal(got, ref), k
+    finally:
+        rocm.call("set_stream_offset", 0)
+        rocm.call("graph_destroy", graph)
+    assert np.abs(checkpoints[-1][0] - checkpoints[0][0]).max() > 1e-4      # the steps trained
+
+
+def test_what_a_recording_stream_cannot_do_is_refused(rocm):
+    """allocation, host copies and a growing workspace return RLT_E_CAPTURING instead of breaking the recording; check_status does not wait"""
+    lib, h = rocm.device.lib, rocm.device.handle
+    x = rocm.zeros((16,))
+    host = np.zeros(16, np.float32)
+    ptr = C.c_void_p()
+    graph = C.c_void_p()
+    rocm.call("graph_begin_capture")
+    try:
+        assert lib.rlt_rocm_malloc(h, C.byref(ptr), 1024) == RLT_E_CAPTURING
+        assert lib.rlt_rocm_memcpy_d2h(h, host.ctypes.data, x.ptr, 64) == RLT_E_CAPTURING
+        assert lib.rlt_rocm_graph_begin_capture(h) == RLT_E_CAPTURING
+        assert lib.rlt_rocm_check_status(h) == 0
+        rocm.call("fill_f32", x.ptr, 1, 16, 16, 3.0)
+    finally:
+        rocm.call("graph_end_capture", C.byref(graph))
+    assert not x.numpy().any()              # recorded, not run
+    rocm.call("graph_launch", graph)
+    assert np.all(x.numpy() == 3.0)
+    rocm.call("graph_destroy", graph)
+    assert lib.rlt_rocm_malloc(h, C.byref(ptr), 1024) == 0 and lib.rlt_rocm_free(h, ptr) == 0
