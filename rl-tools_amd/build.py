@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 OUT = os.path.join(HERE, "librlt_rocm.so")
-SOURCES = ["device.hip", "tensor_ops.hip", "gemm.hip", "mlp.hip", "mlp_fused.hip", "mlp_small.hip", "mlp_rows.hip", "optim.hip", "sac.hip", "sac_fused.hip", "sac_update.hip", "runner.hip",
+SOURCES = ["device.hip", "tensor_ops.hip", "gemm.hip", "mlp.hip", "mlp_fused.hip", "mlp_small.hip", "mlp_rows.hip", "optim.hip", "sac.hip", "sac_fused.hip", "sac_update.hip", "sac_wide.hip", "runner.hip",
            "ppo.hip", "pad.hip", "gru.hip", "td3.hip", "normalize.hip", "envs.hip", "seq.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

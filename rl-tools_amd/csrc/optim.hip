@@ -31,23 +31,12 @@ struct AdamLaunch {
     float source_scale[MAX_T];
 };
 
+// sum over the blocks of one element, every load in flight at once where there are at most 16 blocks
 __device__ __forceinline__ float sum_of_blocks(const float* __restrict__ p, int groups, int stride) {
-    const int per = (groups + 3) / 4;
-    float q[4];
-#pragma unroll
-    for (int qi = 0; qi < 4; qi++) {
-        const int g0 = qi * per, g1 = min(groups, g0 + per);
-        float s = 0.f;
-        for (int gb = g0; gb < g1; gb += 8) {
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; u++) v[u] = p[(size_t)min(gb + u, g1 - 1) * stride];
-#pragma unroll
-            for (int u = 0; u < 8; u++) s += (gb + u < g1) ? v[u] : 0.f;
-        }
-        q[qi] = s;
-    }
-    return (q[0] + q[1]) + (q[2] + q[3]);
+    const float* const src[1] = {p};
+    float out[1];
+    rlt_sum_of_blocks<1, 2>(src, groups, stride, out);
+    return out[0];
 }
 
 // the step for one optimiser by workgroups [0, n_blocks) numbered `block`
@@ -160,7 +149,7 @@ static void set_source(AdamLaunch& a, const rlt_adam_source* source) {
     for (int i = 0; i < a.n; i++) { a.source_offset[i] = source->offsets[i]; a.source_scale[i] = source->scales[i]; }
 }
 
-int rlt_adam_step_from_partials(rlt_rocm_device* device, const rlt_adam_tensor* tensors, int n, const rlt_adam_parameters* parameters, uint32_t* age, const rlt_adam_source* source) {
+int rlt_adam_step_from_partials(rlt_rocm_device* device, const rlt_adam_tensor* tensors, int n, const rlt_adam_parameters* parameters, uint32_t* age, const rlt_adam_source* source, float polyak) {
     RLT_REQUIRE(tensors && n > 0 && n <= MAX_T && parameters && age && source && source->partial && source->groups > 0);
     void* counters = nullptr;
     int rc = rlt_counters(device, &counters);
@@ -174,7 +163,7 @@ int rlt_adam_step_from_partials(rlt_rocm_device* device, const rlt_adam_tensor* 
         a.t[i] = T; a.prefix[i] = total; total += T.count;
     }
     for (int i = n; i <= MAX_T; i++) a.prefix[i] = total;
-    a.p = *parameters; a.age = age;
+    a.p = *parameters; a.age = age; a.polyak = polyak;
     a.done_counter = (uint32_t*)counters; a.block_partials = (float*)((char*)counters + 256);
     a.increment_age = 1;
     set_source(a, source);
@@ -185,7 +174,7 @@ int rlt_adam_step_from_partials(rlt_rocm_device* device, const rlt_adam_tensor* 
 
 int rlt_adam_step_pair(rlt_rocm_device* device, const rlt_adam_tensor* tensors_a, int n_a, const rlt_adam_parameters* parameters_a, uint32_t* age_a,
                        const rlt_adam_tensor* tensors_b, int n_b, const rlt_adam_parameters* parameters_b, uint32_t* age_b,
-                       const rlt_adam_source* source_a, const rlt_adam_source* source_b) {
+                       const rlt_adam_source* source_a, const rlt_adam_source* source_b, float polyak) {
     RLT_REQUIRE(tensors_a && tensors_b && n_a > 0 && n_b > 0 && parameters_a && parameters_b && age_a && age_b);
     if (n_a > MAX_T || n_b > MAX_T) {
         RLT_REQUIRE(!source_a && !source_b);
@@ -209,7 +198,7 @@ int rlt_adam_step_pair(rlt_rocm_device* device, const rlt_adam_tensor* tensors_a
         }
         for (int i = a.n; i <= MAX_T; i++) a.prefix[i] = total;
         a.p = k ? *parameters_b : *parameters_a;
-        a.age = k ? age_b : age_a;
+        a.age = k ? age_b : age_a; a.polyak = polyak;
         // the second optimiser's ticket counter and partial sums sit in their own part of the counters block
         a.done_counter = (uint32_t*)((char*)counters + (k ? 64 : 0)); a.block_partials = (float*)((char*)counters + 256) + (k ? 480 : 0);
         a.increment_age = 1;

@@ -261,6 +261,7 @@ int rlt_rocm_sac_train_critic(rlt_rocm_device* device, const rlt_sac_agent* A, i
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A) && (ci == 0 || ci == 1) && action_noise);
     if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) { const rlt_update_noise noise = {action_noise, 0, 0, nullptr}; return rlt_sac_update_critic(device, A, ci, noise); }
+    if (!device->sac_per_operation && rlt_sac_wide_supported(device, A)) { const rlt_update_noise noise = {action_noise, 0, 0, nullptr}; return rlt_sac_wide_update_critics(device, A, ci, 1, noise, false); }
     RLT_REQUIRE(A->next_state_action_value_input && A->next_q[0] && A->next_q[1] && A->next_log_probabilities && A->target_action_value && A->d_output_critic[ci]);
     const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
     const rlt_dense_layer* critic = A->critics[ci];
@@ -318,6 +319,7 @@ int rlt_rocm_sac_train_actor(rlt_rocm_device* device, const rlt_sac_agent* A, co
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A) && action_noise);
     if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) { const rlt_update_noise noise = {action_noise, 0, 0, nullptr}; return rlt_sac_update_actor(device, A, noise); }
+    if (!device->sac_per_operation && rlt_sac_wide_supported(device, A)) { const rlt_update_noise noise = {action_noise, 0, 0, nullptr}; return rlt_sac_wide_update_actor(device, A, noise); }
     RLT_REQUIRE(A->state_action_value_input && A->d_output_actor_critics && A->d_critic_input[0] && A->d_critic_input[1] && A->d_actor_output_squashing &&
                 A->d_actor_output && A->actor_pre_squashing && A->actor_log_probabilities && A->actor_actions && A->log_alpha.gradient);
     const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
@@ -355,6 +357,7 @@ int rlt_rocm_sac_train_actor(rlt_rocm_device* device, const rlt_sac_agent* A, co
 // both train_critic calls of a loop step with a shared batch (and update_critic_targets) as one launch where the fused kernel fits
 static int train_critics(rlt_rocm_device* device, const rlt_sac_agent* A, const rlt_update_noise& noise, int update_targets) {
     if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) return rlt_sac_update_critics(device, A, noise, update_targets != 0);
+    if (!device->sac_per_operation && rlt_sac_wide_supported(device, A)) return rlt_sac_wide_update_critics(device, A, 0, 2, noise, update_targets != 0);
     int rc;
     const float* values = noise.values;
     if (!values) {
@@ -382,6 +385,7 @@ int rlt_rocm_sac_train_actor_drawn(rlt_rocm_device* device, const rlt_sac_agent*
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A));
     if (!device->sac_per_operation && rlt_sac_update_supported(device, A)) { const rlt_update_noise noise = {nullptr, seed, stream, drawn_noise}; return rlt_sac_update_actor(device, A, noise); }
+    if (!device->sac_per_operation && rlt_sac_wide_supported(device, A)) { const rlt_update_noise noise = {nullptr, seed, stream, drawn_noise}; return rlt_sac_wide_update_actor(device, A, noise); }
     RLT_REQUIRE(drawn_noise);
     const int rc = rlt_rocm_randn_f32(device, drawn_noise, (size_t)A->batch * A->action_dim, seed, stream);
     return rc ? rc : rlt_rocm_sac_train_actor(device, A, drawn_noise);

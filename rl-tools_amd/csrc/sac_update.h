@@ -16,6 +16,12 @@ int rlt_sac_update_critic(rlt_rocm_device* device, const rlt_sac_agent* agent, i
 int rlt_sac_update_actor(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_update_noise& noise);
 // both train_critic calls on the agent's batch with the same noise in ONE launch and, if update_targets, update_critic_targets after them
 int rlt_sac_update_critics(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_update_noise& noise, bool update_targets);
+// The same updates for three-layer networks of any hidden width up to 256 (sac_wide.hip), always with the optimiser as the kernel's own last
+// step: supported only while that is switched on (rlt_rocm_set_update_options) and for batches of at most 512 rows. `first`, `count`: the
+// critics trained by the launch (one of them, or both on the same batch and noise; update_targets only with both).
+bool rlt_sac_wide_supported(const rlt_rocm_device* device, const rlt_sac_agent* agent);
+int rlt_sac_wide_update_critics(rlt_rocm_device* device, const rlt_sac_agent* agent, int first, int count, const rlt_update_noise& noise, bool update_targets);
+int rlt_sac_wide_update_actor(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_update_noise& noise);
 // target[i] = polyak * target[i] + (1 - polyak) * source[i] for a list of tensors, one launch per 16 tensors
 int rlt_sac_polyak_list(rlt_rocm_device* device, const float* const* sources, float* const* targets, const uint32_t* counts, int n, float polyak);
 

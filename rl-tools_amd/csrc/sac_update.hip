@@ -30,10 +30,10 @@
 #include "mlp_small.h"
 #include "optim.h"
 #include "rng.h"
+#include "sac_heads.h"
 
 namespace {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) float* lptr;
 constexpr int H = 64, HS = H + 1, TEAM_WAVES = 4, WAVES = 2 * TEAM_WAVES, ROWS = 16, THREADS = 64 * WAVES, MAX_D = 128, MAX_ACT = 8, MAX_OUT = 16, D3S = MAX_OUT + 1, N_EXTRA = 16,
               MISC = 64;
 static_assert(H == 16 * TEAM_WAVES, "one 16-unit tile of the hidden layers per wavefront of a team");
@@ -65,39 +65,12 @@ struct UpdateArgs {
     // every 8th workgroup of an 8 x larger grid works, so that all of them run on one XCD and share its L2 (the device hands out
     // workgroups round robin over the XCDs)
     int packed;
-    // The optimiser's step at the end of the launch: every workgroup announces its block of partial sums (tickets[0]), waits until all
-    // workgroups of the launch have, and steps a slice of its trained network's elements: sum over the blocks in the order of the
-    // small-MLP reduction kernel, Adam, and the soft update of a target where the tensor names one (opt[].t[].polyak_target; the targets
-    // are read by every workgroup of the launch, hence the wait for all of them). The grid must be resident as a whole: the host
-    // only asks for this with at most 64 workgroups. The wait is bounded; a workgroup that gives up sets *fault and leaves its slice
-    // undone. tickets[1] counts the workgroups that are through; the last one clears both words and advances the ages.
-    // Critic updates: blockIdx.y selects the trained critic (critic[y], opt[y]).
-    int tail;
-    uint32_t* tickets; unsigned* fault;
-    rlt_tail_optimizer opt[2];
-    float polyak;
-    int has_second; rlt_adam_tensor second; rlt_adam_parameters second_p; uint32_t* second_age; float second_scale;      // a scalar whose gradient is extra[0] * second_scale (log_alpha)
+    // the optimiser's step at the end of the launch (optim.h); critic updates: blockIdx.y selects the trained critic (critic[y], tail.opt[y])
+    rlt_tail_args tail;
 };
 
 __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
-template <int CTRL>
-__device__ __forceinline__ float dpp(float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true)); }
-// sum over the 16 lanes of a row (r = 0..15), every lane of the row receives it
-__device__ __forceinline__ float row16_sum(float x) { asm volatile("" : "+v"(x)); x += dpp<0xB1>(x); x += dpp<0x4E>(x); x += dpp<0x141>(x); x += dpp<0x140>(x); return x; }
-// sum over the four lane groups (lanes r, r + 16, r + 32, r + 48), in a fixed order
-__device__ __forceinline__ float groups_sum(float v) { asm volatile("" : "+v"(v)); v += __shfl_xor(v, 16, 64); v += __shfl_xor(v, 32, 64); return v; }
-// lanes of one wavefront exchange data through LDS: the hardware executes a wavefront's LDS instructions in order, the fences keep
-// the compiler from moving them across
-__device__ __forceinline__ void wave_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-__device__ __forceinline__ float clampf(float x, float lo, float hi) { return fminf(fmaxf(x, lo), hi); }
-__device__ __forceinline__ float normal_log_prob(float mean, float log_std, float sd, float value) {
-    const float z = (value - mean) / sd;
-    return -0.9189385332046727f - log_std - 0.5f * z * z;
-}
+using namespace rlt_sac;
 
 // hidden activation: a compile-time constant where the kernel is instantiated for it (ACT_H >= 0), else the network's run-time value
 template <int ACT_H> __device__ __forceinline__ float act_hidden(float x, int f) { return rlt_act(x, ACT_H >= 0 ? ACT_H : f); }
@@ -258,30 +231,6 @@ __device__ __forceinline__ float backward_layer2(const BackwardRegs& G, int act_
     return sum;
 }
 
-// sample_and_squash forward for the items of a lane of the wavefront that does the per-row work: row r, actions kk and kk + 4
-struct HeadItem { float mean, log_std_raw, noise, sample, action; };
-__device__ __forceinline__ float head_forward(const UpdateArgs& A, lptr d3s, lptr xs, int SX, const float (&noise)[2], int r, int kk, HeadItem (&item)[2]) {
-    float log_prob = 0.f;
-#pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int a = kk + 4 * j;
-        HeadItem& I = item[j];
-        I = {0.f, 0.f, 0.f, 0.f, 0.f};
-        if (a < A.act) {
-            I.mean = d3s[r * D3S + a];
-            I.log_std_raw = d3s[r * D3S + A.act + a];
-            const float log_std = clampf(I.log_std_raw, A.sas.log_std_lower_bound, A.sas.log_std_upper_bound);
-            const float sd = expf(log_std);
-            I.noise = noise[j];
-            I.sample = I.mean + I.noise * sd;
-            I.action = tanhf(I.sample);
-            xs[r * SX + A.obs + a] = I.action;
-            log_prob += normal_log_prob(I.mean, log_std, sd, I.sample) - logf(1.0f - I.action * I.action + A.sas.log_probability_epsilon);
-        }
-    }
-    return groups_sum(log_prob);
-}
-
 // TD3's actor head for the items of a lane: tanh of the MLP's output, the td3_sampling layer, and in the critic update the smoothing noise
 // of the target action (rl/algorithms/td3/operations_generic.h:129-145). mean = tanh(output), sample = value before the clamp.
 __device__ __forceinline__ void td3_head_forward(const UpdateArgs& A, lptr d3s, lptr xs, int SX, const float (&noise)[2], const float (&target_noise)[2], bool critic_update,
@@ -301,80 +250,6 @@ __device__ __forceinline__ void td3_head_forward(const UpdateArgs& A, lptr d3s, 
             if (critic_update) I.action = clampf(I.action + target_noise[j], -1.0f, 1.0f);
             xs[r * SX + A.obs + a] = I.action;
         }
-    }
-}
-
-// The optimiser's step at the end of an update kernel (see UpdateArgs::tail). Every thread of every workgroup calls it after its last store.
-constexpr unsigned TAIL_MAX_POLL = 1u << 20;      // about a second
-template <bool SAME_XCD>
-__device__ __forceinline__ void tail_slice(const UpdateArgs& A, int y, int g, int G) {
-    const rlt_tail_optimizer& O = A.opt[y];
-    const float* blocks = A.partial + (size_t)y * G * A.count;
-    const uint32_t n = O.prefix[O.n], chunk = (n + G - 1) / G, begin = min(n, (uint32_t)g * chunk), end = min(n, begin + chunk);
-    const uint32_t age = *O.age;
-    float bc1, bc2;
-    rlt_adam_bias_corrections(O.p, age, bc1, bc2);
-    for (uint32_t base = begin; base < end; base += THREADS) {
-        const uint32_t i = base + threadIdx.x;
-        const bool ok = i < end;
-        const uint32_t ic = ok ? i : begin;
-        int t = 0;
-#pragma unroll
-        for (int k = 1; k < RLT_TAIL_TENSORS; k++) t += (k < O.n && ic >= O.prefix[k]) ? 1 : 0;
-        const uint32_t j = ic - O.prefix[t];
-        const float* const src[1] = {blocks + O.offset[t] + j};
-        float gs[1];
-        rlt_sum_of_blocks<1, SAME_XCD>(src, G, A.count, gs);
-        if (ok) {
-            const rlt_adam_tensor& T = O.t[t];
-            const float ge = gs[0] * O.scale[t];
-            T.gradient[j] = ge;
-            rlt_adam_apply(O.p, T, j, ge, bc1, bc2, A.polyak);
-        }
-    }
-    if (A.has_second && g == G - 1 && threadIdx.x == THREADS - 1) {
-        const float* const src[1] = {blocks + (A.count - N_EXTRA)};
-        float gs[1];
-        rlt_sum_of_blocks<1, SAME_XCD>(src, G, A.count, gs);
-        float b1, b2;
-        rlt_adam_bias_corrections(A.second_p, *A.second_age, b1, b2);
-        const float ge = gs[0] * A.second_scale;
-        A.second.gradient[0] = ge;
-        rlt_adam_apply(A.second_p, A.second, 0, ge, b1, b2, 0.0f);
-    }
-}
-__device__ __noinline__ void optimiser_tail(const UpdateArgs& A, int y, int g, int G, lptr flag_words) {
-    typedef __attribute__((address_space(3))) int* liptr;
-    const liptr flags = (liptr)flag_words;
-    const unsigned total = (unsigned)G * gridDim.y;
-    __builtin_amdgcn_s_waitcnt(0);            // this wavefront's stores have completed
-    if (!A.packed) __threadfence();           // and are visible beyond this XCD
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        __hip_atomic_fetch_add(A.tickets, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        unsigned tries = 0; int ok = 1;
-        while (__hip_atomic_load(A.tickets, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < total) {
-            __builtin_amdgcn_s_sleep(1);
-            if (++tries >= TAIL_MAX_POLL || ((tries & 63u) == 0u && __hip_atomic_load(A.fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
-                __hip_atomic_store(A.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                ok = 0;
-                break;
-            }
-        }
-        flags[0] = ok;
-    }
-    __syncthreads();
-    if (flags[0]) {
-        if (A.packed) tail_slice<true>(A, y, g, G);
-        else { __threadfence(); tail_slice<false>(A, y, g, G); }
-    }
-    __syncthreads();        // every thread has read the ages it needs
-    if (threadIdx.x == 0 && __hip_atomic_fetch_add(A.tickets + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == total - 1) {
-        // the last workgroup through: nobody waits on the words any more, and every slice has been stepped with the old ages
-        __hip_atomic_store(A.tickets, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(A.tickets + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for (unsigned k = 0; k < gridDim.y; k++) *A.opt[k].age += 1;
-        if (A.has_second) *A.second_age += 1;
     }
 }
 
@@ -487,7 +362,7 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
         wave_sync();
         float log_prob = 0.f;
         if (TD3) td3_head_forward(A, d3s, xsa, SX, noise, target_noise, CRITIC, r, kk, item);
-        else log_prob = head_forward(A, d3s, xsa, SX, noise, r, kk, item);
+        else log_prob = head_forward(A.sas, A.obs, A.act, d3s, D3S, xsa, SX, noise, r, kk, item);
         if (TD3) {
             if (!CRITIC && row_ok && A.out_pre_clip) {
 #pragma unroll
@@ -669,10 +544,10 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
             dst[o_ex + r] = extra;
         }
     }
-    if (!A.tail) return;
+    if (!A.tail.enabled) return;
     // the kernel's arguments as they lie in its argument segment (the struct is the only explicit argument), so that the optimiser's
     // part, a function of its own, indexes them there
-    optimiser_tail(*(const UpdateArgs*)__builtin_amdgcn_kernarg_segment_ptr(), y, g, G, (lptr)(misc + 48));
+    rlt_optimiser_tail<THREADS>(&((const RLT_CONSTANT UpdateArgs*)__builtin_amdgcn_kernarg_segment_ptr())->tail, y, g, G, (__attribute__((address_space(3))) int*)(misc + 48));
 }
 
 // soft update of up to 16 tensors in one launch (utils/polyak/operations_generic.h:11-27): workgroup b serves tensor b % n
@@ -736,32 +611,33 @@ struct Optimiser {
     const rlt_adam_tensor* second; const rlt_adam_parameters* second_parameters; uint32_t* second_age; float second_scale;
     const rlt_dense_layer* soft_target;
 };
-constexpr int TAIL_MAX_WORKGROUPS = 64;      // a grid of this many workgroups of 512 threads is resident as a whole on any device this library runs on
 
 // The optimisers as the kernel's own last step: possible where the Adam tensors are the networks' gradient buffers (and the targets'
 // parameters are laid out as the trained networks' are) and the grid is small enough to wait for itself.
 bool configure_tail(rlt_rocm_device* device, UpdateArgs& a, const Optimiser* opts, int n_opts, int groups, float polyak) {
-    if (!device->update_tail || n_opts < 1 || n_opts > 2 || n_opts * groups > TAIL_MAX_WORKGROUPS) return false;
+    if (!device->update_tail || n_opts < 1 || n_opts > 2 || n_opts * groups > RLT_TAIL_MAX_WORKGROUPS) return false;
+    rlt_tail_args& T = a.tail;
     for (int k = 0; k < n_opts; k++) {
         const Optimiser& O = opts[k];
         uint32_t offsets[12]; int first[12], count[12];
         if (!map_gradients(O.trained, O.tensors, O.n_tensors, offsets, first, count)) return false;
         if (O.second && (O.second->polyak_target || n_opts != 1 || !O.second->parameters || !O.second->gradient || !O.second->first_moment || !O.second->second_moment)) return false;
-        if (!rlt_tail_optimizer_fill(a.opt[k], O.tensors, O.n_tensors, offsets, nullptr, O.parameters, O.age)) return false;
+        if (!rlt_tail_optimizer_fill(T.opt[k], O.tensors, O.n_tensors, offsets, nullptr, O.parameters, O.age)) return false;
         if (O.soft_target)
             for (int i = 0; i < O.n_tensors; i++) {
                 // the tensor's parameters must be the trained network's own segments, so that the target's segments correspond element by element
                 if (parameter_segments(O.trained, first[i], count[i]) != O.tensors[i].parameters) return false;
-                if (!(a.opt[k].t[i].polyak_target = parameter_segments(O.soft_target, first[i], count[i]))) return false;
+                if (!(T.opt[k].t[i].polyak_target = parameter_segments(O.soft_target, first[i], count[i]))) return false;
             }
-        if (O.second) { a.has_second = 1; a.second = *O.second; a.second_p = *O.second_parameters; a.second_age = O.second_age; a.second_scale = O.second_scale; }
+        if (O.second) { T.has_second = 1; T.second_offset = a.count - N_EXTRA; T.second = *O.second; T.second_p = *O.second_parameters; T.second_age = O.second_age; T.second_scale = O.second_scale; }
     }
     void* counters = nullptr;
     if (rlt_counters(device, &counters)) return false;
-    a.tickets = (uint32_t*)counters + RLT_TICKET_TAIL;
-    a.fault = device->fault;
-    a.polyak = polyak;
-    a.tail = 1;
+    T.tickets = (uint32_t*)counters + RLT_TICKET_TAIL;
+    T.fault = device->fault;
+    T.polyak = polyak;
+    T.partial = a.partial; T.count = a.count; T.same_xcd = a.packed;
+    T.enabled = 1;
     return true;
 }
 
@@ -799,10 +675,10 @@ int launch_update(rlt_rocm_device* device, UpdateArgs& a, int groups, const Opti
     if (rc) return rc;
     a.partial = (float*)scratch;
     a.stream_offset = device->stream_offset;
-    const bool tail = configure_tail(device, a, opts, n_opts, groups, polyak);
-    if (tail) device->fault_armed = 1;
     // up to 32 workgroups (one per compute unit of an XCD) are placed on one XCD where the device hands out workgroups round robin
     a.packed = device->update_one_xcd && device->xcd_stride == 8 && n_opts * groups <= 32 ? 1 : 0;
+    const bool tail = configure_tail(device, a, opts, n_opts, groups, polyak);
+    if (tail) device->fault_armed = 1;
     const dim3 grid(a.packed ? 8 * groups : groups, n_opts);
 #define RLT_LAUNCH_UPDATE(NT, ACT)                                                                                                                              \
     do {                                                                                                                                                        \
@@ -870,7 +746,7 @@ int rlt_sac_update_critics(rlt_rocm_device* device, const rlt_sac_agent* A, cons
     const Optimiser O[2] = {{A->critics[0], A->critic_adam_tensors[0], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[0], nullptr, nullptr, nullptr, 0.0f, update_targets ? A->critics_target[0] : nullptr},
                             {A->critics[1], A->critic_adam_tensors[1], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[1], nullptr, nullptr, nullptr, 0.0f, update_targets ? A->critics_target[1] : nullptr}};
     const int rc = launch_update<MODE_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), O, 2, A->polyak);
-    if (rc || !update_targets || a.tail) return rc;
+    if (rc || !update_targets || a.tail.enabled) return rc;
     return rlt_rocm_sac_update_critic_targets(device, A);      // the optimisers ran as launches of their own: so does the soft update
 }
 

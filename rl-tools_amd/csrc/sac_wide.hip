@@ -1,0 +1,644 @@
+// One launch for the network passes of a SAC critic update, one for those of an actor update, for three-layer networks of any hidden width
+// up to 256 (the zoo's agents are 256 wide: src/rl/zoo/acrobot-swingup-v0/sac.h, ant-v4): actors obs -> h -> h -> 2 act, critics
+// obs + act -> h -> h -> 1, at most 128 critic inputs and 8 actions.
+// reference: rl/algorithms/sac/operations_generic.h:243-337 (train_critic), :395-468 (train_actor),
+//            nn/layers/sample_and_squash/operations_generic.h:148-398, nn_models/mlp/operations_generic.h:128-260.
+//
+// A workgroup of sixteen wavefronts takes 16 rows of the batch through every pass of the update, one network after the other:
+//   critic update   actor on the next observations -> squashed sample and its log-probability -> target critic 0, target critic 1 on
+//                   [next observation | sample] -> TD target -> trained critic forward on the current rows -> MSE gradient -> backward
+//   actor update    actor forward -> squashed sample -> critic 0, then critic 1: forward and the gradient of -value / batch with respect
+//                   to the action -> gradient of the smaller value per row -> sample_and_squash backward (entropy term, log_alpha
+//                   gradient) -> actor backward
+// Wavefront w owns hidden units 16 w .. 16 w + 15 of every layer: it computes that tile of the 16 x h activations from the whole previous
+// layer (LDS, behind a workgroup barrier), contributes the units' share of the output layer's reduction (the partial tiles are added in
+// wavefront order), and in the backward pass owns the same units' pre-activation gradients and their rows of dW1, dW2 and columns of dW3.
+// Weights are read from memory (L2) straight into the B operands of v_mfma_f32_16x16x4_f32 when a layer needs them, the second
+// layer's first half a layer ahead; hidden widths that are no multiple of 16 are completed with zero operands. The reduction index of a
+// 16-deep chunk is dealt to the four lane groups as k = 16 j + 4 g + i for the i-th of four instructions, so that activations (LDS) and
+// weights (memory) are both read 16 bytes at a time.
+// A workgroup writes one block of partial sums of the trained network's gradients [dW1 | db1 | dW2 | db2 | dW3 | db3 | extra]; the
+// optimiser's launch adds the blocks up over the whole chip (one compute unit draws about 4 GB/s from memory and 20 GB/s from L2 with loads
+// of this kind: read by the update's own sixteen workgroups, the 4.4 MB of blocks at width 256 took 70 us; spread over all compute units, 10).
+// Bound: per workgroup, a 16 x 256 x 256 layer is 2.1 MFLOP = 3.4 us of one compute unit's matrix pipeline, and an update has six or seven
+// of them; a batch of 256 is sixteen workgroups (thirty-two where both critics share the launch).
+#include "sac_update.h"
+#include "optim.h"
+#include "rng.h"
+#include "sac_heads.h"
+
+namespace {
+using namespace rlt_sac;
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) floatx4* lptr4;
+constexpr int ROWS = 16, MAX_H = 256, WAVES = MAX_H / 16, THREADS = 64 * WAVES, S = MAX_H + 4, MAX_D = 128, SXS = MAX_D + 4, MAX_ACT = 8, MAX_OUT = 16, D3S = MAX_OUT + 1,
+              N_EXTRA = 16, MISC = 64, YP = ROWS * D3S;
+enum { MODE_CRITIC = 0, MODE_ACTOR = 1 };
+
+struct WNet { const float *W1, *b1, *W2, *b2, *W3, *b3; int in, hid, out, act_h, vec1, vec2, vec3; };      // vecN: the rows of WN can be read 16 bytes at a time
+struct WideArgs {
+    WNet actor, critic[2], target[2];
+    const float* batch_base;               // [2][batch][obs + act]: current rows, then next rows
+    const float* rewards; const uint8_t* terminated;
+    const float* noise;                    // [batch][act], or NULL: drawn from (noise_seed, noise_stream + *stream_offset)
+    uint64_t noise_seed, noise_stream; float* out_noise; const uint64_t* stream_offset;
+    const float* log_alpha;
+    rlt_sas_parameters sas;
+    float gamma;
+    int batch, obs, act;
+    float* partial; int count;             // per workgroup and trained network: count floats (the optimiser's launch adds the blocks up)
+    float* out_log_probabilities; float* out_target_action_value; float* out_actions; float* out_pre_squashing;
+    int packed;                            // every 8th workgroup of an 8 x larger grid works: all of them on one XCD
+};
+
+__device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+template <int ACT_H> __device__ __forceinline__ float act_hidden(float x, int f) { return rlt_act(x, ACT_H >= 0 ? ACT_H : f); }
+template <int ACT_H> __device__ __forceinline__ float dact_hidden(float o, int f) { return rlt_dact_from_output(o, ACT_H >= 0 ? ACT_H : f); }
+
+// B operands of one layer for this lane's output column n: W[n][16 j + 4 g ... + 3] for chunks j0 <= j < j0 + JN; zero beyond the layer's shape
+template <int JN>
+__device__ __forceinline__ void load_rows(const float* __restrict__ W, int K, int N, bool vec, int n, int g, int j0, floatx4 (&b)[JN]) {
+    const bool n_ok = n < N;
+    const float* row = W + (size_t)(n_ok ? n : 0) * K;
+#pragma unroll
+    for (int j = 0; j < JN; j++) {
+        const int k = 16 * (j0 + j) + 4 * g;
+        floatx4 v = {0.f, 0.f, 0.f, 0.f};
+        if (n_ok && k < K) {
+            if (vec) v = *reinterpret_cast<const floatx4*>(row + k);      // K is a multiple of 4 here
+            else { v[0] = row[k]; if (k + 1 < K) v[1] = row[k + 1]; if (k + 2 < K) v[2] = row[k + 2]; if (k + 3 < K) v[3] = row[k + 3]; }
+        }
+        b[j] = v;
+    }
+}
+// acc += in[rows][16 (j0 + j) + ...] * b[j], the workgroup's 16 rows against this lane's column
+template <int JN>
+__device__ __forceinline__ void chunks(floatx4& a0, floatx4& a1, lptr in, int stride, int c, int g, int j0, int steps, const floatx4 (&b)[JN]) {
+#pragma unroll
+    for (int j = 0; j < JN; j++) {
+        if (j0 + j < steps) {
+            const floatx4 a = *(lptr4)(in + c * stride + 16 * (j0 + j) + 4 * g);
+            a0 = mfma16(a[0], b[j][0], a0); a1 = mfma16(a[1], b[j][1], a1);
+            a0 = mfma16(a[2], b[j][2], a0); a1 = mfma16(a[3], b[j][3], a1);
+        }
+    }
+}
+
+// profiling builds (-DRLT_WIDE_PROFILE): thread 0 of workgroup 0 notes the constant-rate clock at the stage boundaries, rlt_sac_wide_ticks copies the notes out
+#ifdef RLT_WIDE_PROFILE
+__device__ unsigned long long rlt_wide_ticks[2][32];
+#define RLT_TICK(i) do { if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) rlt_wide_ticks[MODE][i] = wall_clock64(); } while (0)
+#else
+#define RLT_TICK(i) do {} while (0)
+#endif
+
+// The three layers of network N on the workgroup's rows x [16][xstride]: this wavefront's tile of h1 and h2 (after the activation) into
+// LDS, then its units' share of the output layer's reduction into yp[wave]. Three workgroup barriers, which every wavefront meets; after
+// the last one output_tile() returns the output layer's sums (without the bias).
+template <int ACT_H, int NT1C>
+__device__ __forceinline__ void forward3(const WNet& N, lptr x, int xstride, lptr h1, lptr h2, lptr yp, int wave, int c, int g) {
+    const int HID = N.hid, n = 16 * wave + c, tiles = (HID + 15) >> 4;
+    const bool on = wave < tiles, n_ok = n < HID;
+    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    floatx4 w2a[8], w2b[8], w3 = zero4;
+    float b1 = 0.f, b2 = 0.f;
+    if (on) {
+        floatx4 w1[NT1C];
+        load_rows<NT1C>(N.W1, N.in, HID, N.vec1, n, g, 0, w1);
+        load_rows<8>(N.W2, HID, HID, N.vec2, n, g, 0, w2a);      // on their way while the first layer runs
+        if (NT1C <= 2) load_rows<8>(N.W2, HID, HID, N.vec2, n, g, 8, w2b);      // few first-layer operands: room for the whole second layer at once
+        if (n_ok) { b1 = N.b1[n]; b2 = N.b2[n]; }
+        // the output layer's operands: row c of W3 (c < out), this wavefront's 16 units
+        if (c < N.out) {
+            const int k = 16 * wave + 4 * g;
+            const float* row = N.W3 + (size_t)c * HID;
+            if (N.vec3 && k + 3 < HID) w3 = *reinterpret_cast<const floatx4*>(row + k);
+            else { if (k < HID) w3[0] = row[k]; if (k + 1 < HID) w3[1] = row[k + 1]; if (k + 2 < HID) w3[2] = row[k + 2]; if (k + 3 < HID) w3[3] = row[k + 3]; }
+        }
+        floatx4 a0 = zero4, a1 = zero4;
+        chunks<NT1C>(a0, a1, x, xstride, c, g, 0, (N.in + 15) >> 4, w1);
+        const floatx4 acc = a0 + a1;
+#pragma unroll
+        for (int v = 0; v < 4; v++) h1[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + b1, N.act_h) : 0.f;
+        if (NT1C > 2) load_rows<8>(N.W2, HID, HID, N.vec2, n, g, 8, w2b);
+    }
+    rlt_lds_barrier();
+    if (on) {
+        floatx4 a0 = zero4, a1 = zero4;
+        chunks<8>(a0, a1, h1, S, c, g, 0, tiles, w2a);
+        chunks<8>(a0, a1, h1, S, c, g, 8, tiles, w2b);
+        const floatx4 acc = a0 + a1;
+#pragma unroll
+        for (int v = 0; v < 4; v++) h2[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + b2, N.act_h) : 0.f;
+    }
+    rlt_lds_barrier();
+    if (on) {
+        const floatx4 a = *(lptr4)(h2 + c * S + 16 * wave + 4 * g);
+        floatx4 y = zero4;
+        y = mfma16(a[0], w3[0], y); y = mfma16(a[1], w3[1], y); y = mfma16(a[2], w3[2], y); y = mfma16(a[3], w3[3], y);
+#pragma unroll
+        for (int v = 0; v < 4; v++) yp[(wave * ROWS + 4 * g + v) * D3S + c] = y[v];
+    }
+    rlt_lds_barrier();
+}
+// the sums of the partial tiles, in wavefront order: element v of lane (c, g) belongs to row 4 g + v, column c
+__device__ __forceinline__ floatx4 output_tile(lptr yp, int tiles, int c, int g) {
+    floatx4 y = {0.f, 0.f, 0.f, 0.f};
+    for (int w = 0; w < tiles; w++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) y[v] += yp[(w * ROWS + 4 * g + v) * D3S + c];
+    return y;
+}
+
+// this wavefront's tile of d_pre2 = (d_pre3 W3) f'(h2) into g2 (may be h2 itself); returns the lane's share of its unit's column sum
+template <int ACT_H>
+__device__ __forceinline__ float backward_layer3(const WNet& N, lptr d3, lptr h2, lptr g2, int wave, int c, int g) {
+    const int n = 16 * wave + c;
+    const bool n_ok = n < N.hid;
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < MAX_OUT / 4; ks++) {
+        const int o = 4 * ks + g;
+        const float w = (o < N.out && n_ok) ? N.W3[(size_t)o * N.hid + n] : 0.f;
+        acc = mfma16(d3[c * D3S + 4 * ks + g], w, acc);      // columns of d_pre3 beyond the output width are zero
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int idx = (4 * g + v) * S + n;
+        const float dp = n_ok ? acc[v] * dact_hidden<ACT_H>(h2[idx], N.act_h) : 0.f;
+        g2[idx] = dp; sum += dp;
+    }
+    return sum;
+}
+// this wavefront's tile of d_pre1 = (d_pre2 W2) f'(h1) into p1 (may be h1 itself); returns the lane's share of its unit's column sum
+template <int ACT_H>
+__device__ __forceinline__ float backward_layer2(const WNet& N, lptr g2, lptr h1, lptr p1, int wave, int c, int g) {
+    const int HID = N.hid, n = 16 * wave + c, tiles = (HID + 15) >> 4;
+    const bool n_ok = n < HID;
+    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    floatx4 a0 = zero4, a1 = zero4;
+    const float* col = N.W2 + (n_ok ? n : 0);
+#pragma unroll 1
+    for (int j0 = 0; j0 < tiles; j0 += 4) {
+        floatx4 b[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int k = 16 * (j0 + j) + 4 * g + i;
+                b[j][i] = (n_ok && k < HID) ? col[(size_t)k * HID] : 0.f;
+            }
+        chunks<4>(a0, a1, g2, S, c, g, j0, tiles, b);
+    }
+    const floatx4 acc = a0 + a1;
+    float sum = 0.f;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int idx = (4 * g + v) * S + n;
+        const float dp = n_ok ? acc[v] * dact_hidden<ACT_H>(h1[idx], N.act_h) : 0.f;
+        p1[idx] = dp; sum += dp;
+    }
+    return sum;
+}
+
+template <int MODE, int ACT_H, int NT1C>
+__global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
+    constexpr bool CRITIC = MODE == MODE_CRITIC;
+    extern __shared__ __attribute__((aligned(16))) float lds_wide[];
+    if (A.packed && (blockIdx.x & 7)) return;
+    const int gi = A.packed ? blockIdx.x >> 3 : blockIdx.x, G = A.packed ? gridDim.x >> 3 : gridDim.x;
+    const int y = CRITIC ? blockIdx.y : 0;
+    const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const bool scalar_wave = wave == 0;
+    const int OBS = A.obs, ACT = A.act, D = OBS + ACT, B = A.batch;
+    const lptr xa = (lptr)lds_wide, xb = xa + ROWS * SXS, h1 = xb + ROWS * SXS, h2 = h1 + ROWS * S, ta = h2 + ROWS * S, tb = ta + ROWS * S,
+               d3 = tb + ROWS * S, d3c = d3 + ROWS * D3S, da = d3c + ROWS * D3S, yp = da + 2 * ROWS * D3S, misc = yp + WAVES * YP;
+    const int row0 = gi * ROWS;
+    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    const WNet trained = CRITIC ? (y ? A.critic[1] : A.critic[0]) : A.actor;      // by value: an index into the kernel's argument would keep all of it in private memory
+    const int HID = trained.hid, tiles = (HID + 15) >> 4;
+    const bool on = wave < tiles;
+
+    // the input tiles: xa = next rows (critic update) or current rows (actor update; the actor reads its observation columns), xb = current rows
+    for (int e = threadIdx.x; e < ROWS * SXS; e += THREADS) {
+        const int r = e / SXS, k = e % SXS;
+        const bool ok = row0 + r < B && k < D;
+        const float* cur = A.batch_base + (size_t)min(row0 + r, B - 1) * D + min(k, D - 1);
+        if (CRITIC) { xa[e] = ok ? cur[(size_t)B * D] : 0.f; xb[e] = ok ? cur[0] : 0.f; }
+        else xa[e] = (ok && k < OBS) ? cur[0] : 0.f;
+    }
+    float noise[2] = {0.f, 0.f}, reward[4] = {0.f, 0.f, 0.f, 0.f}, alpha = 0.f, s3 = 0.f, extra = 0.f;
+    bool terminated[4] = {false, false, false, false};
+    if (scalar_wave) {
+        alpha = expf(*A.log_alpha);
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            if (g + 4 * j < ACT && row0 + c < B) {
+                const size_t i = (size_t)(row0 + c) * ACT + g + 4 * j;
+                noise[j] = A.noise ? A.noise[i] : rlt_randn_element(A.noise_seed, A.noise_stream + *A.stream_offset, i);
+                if (A.out_noise && y == 0) A.out_noise[i] = noise[j];
+            }
+        }
+        if (CRITIC) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) { const int row = min(row0 + 4 * g + v, B - 1); reward[v] = A.rewards[row]; terminated[v] = A.terminated[row] != 0; }
+        }
+    }
+    HeadItem item[2];
+    const bool row_ok = row0 + c < B;
+    RLT_TICK(0);
+    rlt_lds_barrier();      // the input tiles are in place
+    RLT_TICK(1);
+
+    // the actor (critic update: on the next observations; actor update: on the observations, activations kept for its backward pass)
+    forward3<ACT_H, NT1C>(A.actor, xa, SXS, CRITIC ? ta : h1, CRITIC ? tb : h2, yp, wave, c, g);
+    RLT_TICK(2);
+    if (scalar_wave) {
+        const floatx4 out = output_tile(yp, (A.actor.hid + 15) >> 4, c, g);
+        const float b3 = c < A.actor.out ? A.actor.b3[c] : 0.f;
+#pragma unroll
+        for (int v = 0; v < 4; v++) d3[(4 * g + v) * D3S + c] = c < A.actor.out ? out[v] + b3 : 0.f;
+        wave_sync();
+        const float log_prob = head_forward(A.sas, OBS, ACT, d3, D3S, xa, SXS, noise, c, g, item);
+        if (g == 0) {
+            if (CRITIC) misc[c] = log_prob;
+            if (A.out_log_probabilities && row_ok) A.out_log_probabilities[row0 + c] = log_prob;
+        }
+        if (!CRITIC && row_ok) {
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                if (g + 4 * j < ACT) {
+                    if (A.out_actions) A.out_actions[(size_t)(row0 + c) * ACT + g + 4 * j] = item[j].action;
+                    if (A.out_pre_squashing) A.out_pre_squashing[(size_t)(row0 + c) * ACT + g + 4 * j] = item[j].sample;
+                }
+        }
+    }
+    rlt_lds_barrier();      // the action columns of xa are in place
+    RLT_TICK(3);
+
+    if (CRITIC) {
+        // both target critics on [next observation | sampled action], then the trained critic on the current rows
+        floatx4 q_next[2];
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            const WNet T = k ? A.target[1] : A.target[0];
+            forward3<ACT_H, NT1C>(T, xa, SXS, ta, tb, yp, wave, c, g);
+            RLT_TICK(4 + k);
+            if (scalar_wave) { q_next[k] = output_tile(yp, (T.hid + 15) >> 4, c, g); const float b3 = T.b3[0]; for (int v = 0; v < 4; v++) q_next[k][v] += b3; }
+        }
+        forward3<ACT_H, NT1C>(trained, xb, SXS, h1, h2, yp, wave, c, g);
+        RLT_TICK(6);
+        if (scalar_wave) {
+            // TD target of rows 4 g + v (meaningful in the lanes c == 0, which hold output 0), MSE gradient at the critic's pre-activation:
+            // loss weight batch * 0.5 / n with n = batch rows (no masks), times the MSE gradient's 2 / batch (rl/algorithms/sac/operations_generic.h:298-316)
+            const floatx4 yc = output_tile(yp, tiles, c, g);
+            const float b3 = trained.b3[0];
+            const float loss_weight = (1.0f / (float)B) * ((float)B * 0.5f);
+            const float constant = 2.0f / (float)B * loss_weight;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float min_q = fminf(q_next[0][v], q_next[1][v]) - alpha * misc[4 * g + v];
+                const float future = terminated[v] ? 0.0f : A.gamma * min_q;
+                const float y_target = reward[v] + future;
+                const bool ok = c == 0 && row0 + 4 * g + v < B;
+                if (A.out_target_action_value && ok && y == 0) A.out_target_action_value[row0 + 4 * g + v] = y_target;
+                const float diff = (yc[v] + b3) - y_target;
+                const float dp = ok ? diff * constant : 0.f;
+                if (ok) extra += diff * diff;
+                s3 += dp;
+                d3[(4 * g + v) * D3S + c] = dp;
+            }
+        }
+        rlt_lds_barrier();      // d_pre3 is in place
+        RLT_TICK(7);
+    } else {
+        // each critic: value on [observation | sampled action], then the gradient of -value / batch with respect to the action
+        const float loss_weight = (1.0f / (float)B) * -1.0f;       // rl/algorithms/sac/operations_generic.h:437-453 with n = batch rows
+#pragma unroll 1
+        for (int k = 0; k < 2; k++) {
+            const WNet C = k ? A.critic[1] : A.critic[0];
+            const int ctiles = (C.hid + 15) >> 4;
+            forward3<ACT_H, NT1C>(C, xa, SXS, ta, tb, yp, wave, c, g);
+            RLT_TICK(4 + 4 * k);
+            if (scalar_wave) {
+                const floatx4 out = output_tile(yp, ctiles, c, g);
+                const float b3 = C.b3[0];
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    if (c == 0) misc[16 * k + 4 * g + v] = out[v] + b3;
+                    d3c[(4 * g + v) * D3S + c] = (c == 0 && row0 + 4 * g + v < B) ? loss_weight : 0.f;
+                }
+            }
+            rlt_lds_barrier();
+            if (wave < ctiles) backward_layer3<ACT_H>(C, d3c, tb, tb, wave, c, g);
+            rlt_lds_barrier();
+            RLT_TICK(5 + 4 * k);
+            if (wave < ctiles) {
+                backward_layer2<ACT_H>(C, tb, ta, ta, wave, c, g);
+                wave_sync();
+                // d value / d action = the action columns of d_pre1 W1: this wavefront's units' share of the reduction
+                floatx4 acc = zero4;
+                const floatx4 a = *(lptr4)(ta + c * S + 16 * wave + 4 * g);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int unit = 16 * wave + 4 * g + i;
+                    const float w = (c < ACT && unit < C.hid) ? C.W1[(size_t)unit * D + OBS + c] : 0.f;
+                    acc = mfma16(a[i], w, acc);
+                }
+#pragma unroll
+                for (int v = 0; v < 4; v++) yp[(wave * ROWS + 4 * g + v) * D3S + c] = acc[v];
+            }
+            rlt_lds_barrier();
+            RLT_TICK(6 + 4 * k);
+            if (scalar_wave) {
+                const floatx4 out = output_tile(yp, ctiles, c, g);
+#pragma unroll
+                for (int v = 0; v < 4; v++) da[(k * ROWS + 4 * g + v) * D3S + c] = out[v];
+            }
+        }
+        if (scalar_wave) {
+            // sample_and_squash backward on the gradient of the smaller value
+            wave_sync();
+            const lptr dak = da + (misc[c] < misc[16 + c] ? 0 : 1) * ROWS * D3S + c * D3S;
+#pragma unroll
+            for (int v = 0; v < 4; v++) d3[(4 * g + v) * D3S + c] = 0.f;
+            wave_sync();
+            const float alpha_over_b = alpha / (float)B;
+            float entropy = 0.f;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int a = g + 4 * j;
+                if (a < ACT) {
+                    float d_mu, d_ls;
+                    head_backward(A.sas, item[j], dak[a], alpha_over_b, d_mu, d_ls, entropy);
+                    if (row_ok) { d3[c * D3S + a] = d_mu; d3[c * D3S + ACT + a] = d_ls; }
+                }
+            }
+            entropy = groups_sum(entropy);
+            // d log_alpha: sum over the rows of alpha (entropy - target entropy), divided by the batch size by the reduction
+            const float per_row = (g == 0 && row_ok) ? alpha * (entropy - A.sas.target_entropy) : 0.f;
+            const float tile_sum = row16_sum(per_row);
+            if (lane == 0) extra += tile_sum;
+            wave_sync();
+#pragma unroll
+            for (int v = 0; v < 4; v++) s3 += d3[(4 * g + v) * D3S + c];
+        }
+        rlt_lds_barrier();      // d_pre3 is in place
+        RLT_TICK(12);
+    }
+
+    // backward pass of the trained network with its weight gradients over the workgroup's 16 rows; h1, h2: its hidden activations,
+    // d3: the gradient at its last pre-activation; ta receives d_pre2, tb receives d_pre1
+    float* dst = A.partial + ((size_t)y * G + gi) * A.count;
+    const int IN = trained.in, OUT = trained.out, NT1 = (IN + 15) >> 4;
+    const int o_b1 = HID * IN, o_w2 = o_b1 + HID, o_b2 = o_w2 + HID * HID, o_w3 = o_b2 + HID, o_b3 = o_w3 + OUT * HID, o_ex = o_b3 + OUT;
+    const lptr xt = CRITIC ? xb : xa;
+    const int n = 16 * wave + c;
+    const bool n_ok = n < HID;
+    float s2 = 0.f;
+    if (on) {
+        floatx4 aW3 = zero4;
+#pragma unroll
+        for (int ks = 0; ks < ROWS / 4; ks++) aW3 = mfma16(d3[(4 * ks + g) * D3S + c], h2[(4 * ks + g) * S + n], aW3);
+#pragma unroll
+        for (int v = 0; v < 4; v++)
+            if (4 * g + v < OUT && n_ok) dst[o_w3 + (4 * g + v) * HID + n] = aW3[v];
+        s2 = backward_layer3<ACT_H>(trained, d3, h2, ta, wave, c, g);
+    }
+    rlt_lds_barrier();      // every wavefront's tile of d_pre2 is in place
+    RLT_TICK(13);
+    if (on) {
+        {   // dW2: this wavefront's units' rows
+            float a[4];
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) a[ks] = ta[(4 * ks + g) * S + n];
+#pragma unroll 4
+            for (int nt = 0; nt < tiles; nt++) {
+                floatx4 acc = zero4;
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) acc = mfma16(a[ks], h1[(4 * ks + g) * S + 16 * nt + c], acc);
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int m = 16 * wave + 4 * g + v;
+                    if (m < HID && 16 * nt + c < HID) dst[o_w2 + (size_t)m * HID + 16 * nt + c] = acc[v];
+                }
+            }
+        }
+        RLT_TICK(14);
+        float s1 = backward_layer2<ACT_H>(trained, ta, h1, tb, wave, c, g);
+        RLT_TICK(15);
+        wave_sync();            // dW1's rows are this wavefront's own tile of d_pre1
+        {
+            float a[4];
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) a[ks] = tb[(4 * ks + g) * S + n];
+#pragma unroll 2
+            for (int nt = 0; nt < NT1; nt++) {
+                floatx4 acc = zero4;
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) acc = mfma16(a[ks], xt[(4 * ks + g) * SXS + 16 * nt + c], acc);
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int m = 16 * wave + 4 * g + v;
+                    if (m < HID && 16 * nt + c < IN) dst[(size_t)m * IN + 16 * nt + c] = acc[v];
+                }
+            }
+        }
+        s1 = groups_sum(s1); s2 = groups_sum(s2);
+        if (g == 0 && n_ok) { dst[o_b1 + n] = s1; dst[o_b2 + n] = s2; }
+    }
+    if (scalar_wave) {
+        s3 = groups_sum(s3); extra = groups_sum(extra);
+        if (g == 0) {
+            if (c < OUT) dst[o_b3 + c] = s3;
+            dst[o_ex + c] = extra;
+        }
+    }
+    RLT_TICK(16);
+}
+
+constexpr size_t LDS_FLOATS = (size_t)2 * ROWS * SXS + 4 * ROWS * S + 4 * ROWS * D3S + WAVES * YP + MISC;
+
+bool hidden_ok(int a) { return a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH || a == RLT_ACT_SIGMOID; }
+bool net_ok(const rlt_dense_layer* L, int n, int in, int out, int& hid) {
+    if (!L || n != 3) return false;
+    for (int l = 0; l < 3; l++) if (!L[l].weights || !L[l].biases) return false;
+    if (hid == 0) hid = L[0].out_dim;
+    return hid >= 1 && hid <= MAX_H && L[0].in_dim == in && L[0].out_dim == hid && L[1].in_dim == hid && L[1].out_dim == hid && L[2].in_dim == hid && L[2].out_dim == out &&
+           L[0].activation == L[1].activation && hidden_ok(L[0].activation) && L[2].activation == RLT_ACT_IDENTITY;
+}
+bool aligned16(const float* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+WNet net_of(const rlt_dense_layer* L) {
+    const int in = L[0].in_dim, hid = L[0].out_dim;
+    return {L[0].weights, L[0].biases, L[1].weights, L[1].biases, L[2].weights, L[2].biases, in, hid, L[2].out_dim, L[0].activation,
+            in % 4 == 0 && aligned16(L[0].weights), hid % 4 == 0 && aligned16(L[1].weights), hid % 4 == 0 && aligned16(L[2].weights)};
+}
+int partial_count(int in, int hid, int out) { return hid * in + hid + hid * hid + hid + out * hid + out + N_EXTRA; }
+
+// where each Adam tensor's gradient lies in a block of partial sums (a tensor may span several of the network's six gradient buffers
+// where those follow each other in memory); false unless the tensors cover the six buffers exactly
+bool map_gradients(const rlt_dense_layer* L, const rlt_adam_tensor* T, int n, uint32_t* offsets, int* first_segment, int* n_segments) {
+    if (!T || n < 1 || n > RLT_TAIL_TENSORS) return false;
+    const int hid = L[0].out_dim;
+    const float* seg[6] = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases};
+    const uint32_t size[6] = {(uint32_t)(hid * L[0].in_dim), (uint32_t)hid, (uint32_t)(hid * hid), (uint32_t)hid, (uint32_t)(L[2].out_dim * hid), (uint32_t)L[2].out_dim};
+    uint32_t off[6], covered = 0;
+    for (int k = 0, o = 0; k < 6; o += size[k], k++) off[k] = o;
+    for (int i = 0; i < n; i++) {
+        int s = 0;
+        while (s < 6 && seg[s] != T[i].gradient) s++;
+        if (s == 6 || T[i].polyak_target) return false;
+        uint32_t cnt = 0; int k = s;
+        for (; k < 6 && cnt < T[i].count && seg[k] == seg[s] + cnt; k++) {
+            if (covered & (1u << k)) return false;
+            covered |= 1u << k; cnt += size[k];
+        }
+        if (cnt != T[i].count) return false;
+        offsets[i] = off[s]; first_segment[i] = s; n_segments[i] = k - s;
+    }
+    return covered == 63u;
+}
+float* parameter_segments(const rlt_dense_layer* L, int first, int count) {
+    const int hid = L[0].out_dim;
+    float* seg[6] = {L[0].weights, L[0].biases, L[1].weights, L[1].biases, L[2].weights, L[2].biases};
+    const uint32_t size[6] = {(uint32_t)(hid * L[0].in_dim), (uint32_t)hid, (uint32_t)(hid * hid), (uint32_t)hid, (uint32_t)(L[2].out_dim * hid), (uint32_t)L[2].out_dim};
+    uint32_t cnt = 0;
+    for (int k = first; k < first + count; k++) { if (seg[k] != seg[first] + cnt) return nullptr; cnt += size[k]; }
+    return seg[first];
+}
+
+struct Optimiser {
+    const rlt_dense_layer* trained; const rlt_adam_tensor* tensors; int n_tensors; const rlt_adam_parameters* parameters; uint32_t* age;
+    const rlt_adam_tensor* second; const rlt_adam_parameters* second_parameters; uint32_t* second_age; float second_scale;
+    const rlt_dense_layer* soft_target;
+};
+
+// The optimisers' steps, as one launch after the update kernel that adds up the workgroups' blocks itself (16 blocks of 68 k floats at
+// width 256: read through one compute unit each, as the update kernel's own last step, that costs 70 us; spread over the chip 10): both
+// critics' optimisers share it, and a tensor's soft update of its target rides along where the layouts correspond.
+struct Step { rlt_adam_tensor tensors[RLT_TAIL_TENSORS]; uint32_t offsets[RLT_TAIL_TENSORS]; float scales[RLT_TAIL_TENSORS]; bool targets_fused; };
+bool describe_step(const Optimiser& O, Step& S) {
+    int first[RLT_TAIL_TENSORS], count[RLT_TAIL_TENSORS];
+    if (!map_gradients(O.trained, O.tensors, O.n_tensors, S.offsets, first, count)) return false;
+    S.targets_fused = O.soft_target != nullptr;
+    for (int i = 0; i < O.n_tensors; i++) {
+        S.tensors[i] = O.tensors[i]; S.scales[i] = 1.0f;
+        if (O.soft_target && (parameter_segments(O.trained, first[i], count[i]) != O.tensors[i].parameters || !(S.tensors[i].polyak_target = parameter_segments(O.soft_target, first[i], count[i])))) S.targets_fused = false;
+    }
+    if (!S.targets_fused) for (int i = 0; i < O.n_tensors; i++) S.tensors[i].polyak_target = nullptr;
+    return true;
+}
+
+// false: the agent's Adam tensors are not its networks' gradient buffers; the caller takes the per-operation path
+bool steps_describable(const Optimiser* opts, int n_opts) {
+    Step S;
+    for (int k = 0; k < n_opts; k++) {
+        if (!describe_step(opts[k], S)) return false;
+        if (opts[k].second && (opts[k].second->polyak_target || !opts[k].second->parameters || !opts[k].second->gradient || !opts[k].second->first_moment || !opts[k].second->second_moment)) return false;
+    }
+    return true;
+}
+
+template <int MODE>
+int launch_wide(rlt_rocm_device* device, WideArgs& a, int groups, const Optimiser* opts, int n_opts, float polyak, bool* targets_done) {
+    const rlt_dense_layer* trained = opts[0].trained;
+    if (!steps_describable(opts, n_opts)) return RLT_E_UNSUPPORTED;
+    a.count = partial_count(trained[0].in_dim, trained[0].out_dim, trained[2].out_dim);
+    void* scratch = nullptr;
+    int rc = rlt_scratch(device, (size_t)n_opts * groups * a.count * sizeof(float), &scratch);
+    if (rc) return rc;
+    a.partial = (float*)scratch;
+    a.stream_offset = device->stream_offset;
+    a.packed = device->update_one_xcd && device->xcd_stride == 8 && n_opts * groups <= 32 ? 1 : 0;
+    const size_t lds_bytes = LDS_FLOATS * sizeof(float);
+    const dim3 grid(a.packed ? 8 * groups : groups, n_opts);
+#define RLT_LAUNCH_WIDE(ACT, NT)                                                                                                                          \
+    do {                                                                                                                                                  \
+        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sac_wide_kernel<MODE, ACT, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
+        hipLaunchKernelGGL((sac_wide_kernel<MODE, ACT, NT>), grid, dim3(THREADS), lds_bytes, device->stream, a);                                          \
+    } while (0)
+    int act = a.actor.act_h;
+    for (int k = 0; k < 2; k++) if (a.critic[k].act_h != act || a.target[k].act_h != act) act = -1;
+    // first layers of at most 32 inputs (two 16-deep chunks) leave registers for all of a pass's weights at once
+    if (a.obs + a.act <= 32) {
+        if (act == RLT_ACT_RELU) RLT_LAUNCH_WIDE(RLT_ACT_RELU, 2); else if (act == RLT_ACT_FAST_TANH) RLT_LAUNCH_WIDE(RLT_ACT_FAST_TANH, 2); else RLT_LAUNCH_WIDE(-1, 2);
+    } else {
+        if (act == RLT_ACT_RELU) RLT_LAUNCH_WIDE(RLT_ACT_RELU, MAX_D / 16); else if (act == RLT_ACT_FAST_TANH) RLT_LAUNCH_WIDE(RLT_ACT_FAST_TANH, MAX_D / 16); else RLT_LAUNCH_WIDE(-1, MAX_D / 16);
+    }
+#undef RLT_LAUNCH_WIDE
+    if ((rc = rlt_launch_status(device))) return rc;
+    Step S[2];
+    rlt_adam_source source[2];
+    for (int k = 0; k < n_opts; k++) {
+        describe_step(opts[k], S[k]);
+        source[k] = {a.partial + (size_t)k * groups * a.count, groups, a.count, S[k].offsets, S[k].scales};
+    }
+    if (targets_done) *targets_done = n_opts == 2 && S[0].targets_fused && S[1].targets_fused;
+    if (targets_done && !*targets_done) for (int k = 0; k < n_opts; k++) for (int i = 0; i < opts[k].n_tensors; i++) S[k].tensors[i].polyak_target = nullptr;
+    if (n_opts == 2)
+        return rlt_adam_step_pair(device, S[0].tensors, opts[0].n_tensors, opts[0].parameters, opts[0].age, S[1].tensors, opts[1].n_tensors, opts[1].parameters, opts[1].age, &source[0], &source[1], polyak);
+    if (opts[0].second) {
+        const uint32_t second_offset = (uint32_t)(a.count - N_EXTRA);
+        const rlt_adam_source second_source = {a.partial, groups, a.count, &second_offset, &opts[0].second_scale};
+        return rlt_adam_step_pair(device, S[0].tensors, opts[0].n_tensors, opts[0].parameters, opts[0].age, opts[0].second, 1, opts[0].second_parameters, opts[0].second_age, &source[0], &second_source);
+    }
+    return rlt_adam_step_from_partials(device, S[0].tensors, opts[0].n_tensors, opts[0].parameters, opts[0].age, &source[0]);
+}
+
+void set_noise(WideArgs& a, const rlt_update_noise& N) { a.noise = N.values; a.noise_seed = N.seed; a.noise_stream = N.stream; a.out_noise = N.values ? nullptr : N.drawn; }
+void common_args(WideArgs& a, const rlt_sac_agent* A) {
+    a.actor = net_of(A->actor);
+    for (int k = 0; k < 2; k++) { a.critic[k] = net_of(A->critics[k]); a.target[k] = net_of(A->critics_target[k]); }
+    a.batch_base = A->observations_actions_base; a.rewards = A->rewards; a.terminated = A->terminated; a.log_alpha = A->log_alpha.parameters;
+    a.sas = A->sas; a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
+}
+}  // namespace
+
+bool rlt_sac_wide_supported(const rlt_rocm_device* device, const rlt_sac_agent* A) {
+    const int OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    if (OBS < 1 || ACT < 1 || ACT > MAX_ACT || D > MAX_D || A->batch < 1) return false;
+    if (A->final_step_mask || A->next_final_step_mask || A->reset) return false;
+    if (A->batch > 2048) return false;      // larger batches are the per-layer kernels' ground
+    int hid_a = 0, hid_c = 0;
+    if (!net_ok(A->actor, A->n_actor_layers, OBS, 2 * ACT, hid_a)) return false;
+    for (int k = 0; k < 2; k++)
+        if (!net_ok(A->critics[k], A->n_critic_layers, D, 1, hid_c) || !net_ok(A->critics_target[k], A->n_critic_layers, D, 1, hid_c)) return false;
+    return LDS_FLOATS * sizeof(float) <= (size_t)device->lds_bytes;
+}
+
+int rlt_sac_wide_update_critics(rlt_rocm_device* device, const rlt_sac_agent* A, int first, int count, const rlt_update_noise& noise, bool update_targets) {
+    if (!rlt_sac_wide_supported(device, A)) return RLT_E_UNSUPPORTED;
+    RLT_REQUIRE(first >= 0 && count >= 1 && first + count <= 2 && (!update_targets || count == 2));
+    for (int k = first; k < first + count; k++) for (int l = 0; l < 3; l++) RLT_REQUIRE(A->critics[k][l].d_weights && A->critics[k][l].d_biases);
+    WideArgs a = {};
+    common_args(a, A);
+    if (count == 1) { a.critic[0] = net_of(A->critics[first]); a.critic[1] = a.critic[0]; }
+    set_noise(a, noise);
+    a.out_log_probabilities = A->next_log_probabilities; a.out_target_action_value = A->target_action_value;
+    Optimiser O[2];
+    for (int k = 0; k < count; k++)
+        O[k] = {A->critics[first + k], A->critic_adam_tensors[first + k], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[first + k], nullptr, nullptr, nullptr, 0.0f,
+                update_targets ? A->critics_target[first + k] : nullptr};
+    bool targets_done = false;
+    const int rc = launch_wide<MODE_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), O, count, A->polyak, &targets_done);
+    if (rc || !update_targets || targets_done) return rc;
+    return rlt_rocm_sac_update_critic_targets(device, A);
+}
+
+int rlt_sac_wide_update_actor(rlt_rocm_device* device, const rlt_sac_agent* A, const rlt_update_noise& noise) {
+    if (!rlt_sac_wide_supported(device, A)) return RLT_E_UNSUPPORTED;
+    for (int l = 0; l < 3; l++) RLT_REQUIRE(A->actor[l].d_weights && A->actor[l].d_biases);
+    RLT_REQUIRE(A->log_alpha.gradient);
+    WideArgs a = {};
+    common_args(a, A);
+    set_noise(a, noise);
+    a.out_log_probabilities = A->actor_log_probabilities; a.out_actions = A->actor_actions; a.out_pre_squashing = A->actor_pre_squashing;
+    const Optimiser O = {A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, &A->log_alpha, &A->alpha_adam, A->alpha_age, 1.0f / (float)A->batch, nullptr};
+    return launch_wide<MODE_ACTOR>(device, a, rlt_div_up(A->batch, ROWS), &O, 1, 0.0f, nullptr);
+}
+
+#ifdef RLT_WIDE_PROFILE
+extern "C" int rlt_sac_wide_ticks(unsigned long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(rlt_wide_ticks), sizeof(unsigned long long) * 64); }
+#endif

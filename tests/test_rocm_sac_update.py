@@ -104,26 +104,36 @@ def test_fused_updates_match_the_checker_and_the_per_operation_path(oracle, rocm
     assert moved.max() > 1e-4 and results["fused"]["ages"].tolist() == [1 + steps] * 4
 
 
-@pytest.mark.parametrize("batch,obs,act,hidden,hidden_act", [(256, 6, 1, 256, "fast_tanh"), (100, 17, 6, 128, "relu"), (48, 3, 1, 200, "relu")])
-def test_wider_agents_on_the_per_operation_kernels_match_the_checker(oracle, rocm, batch, obs, act, hidden, hidden_act):
-    """Hidden widths other than 64 (the zoo's AcrobotSwingup agent: 6-256-256-2 and 7-256-256-1 at batch 256): every forward pass is one launch of the few-rows
-    kernel (pairs of critics share one), the backward contractions run a wavefront per 16x16 tile. Three loop steps' worth of updates against the CPU checker, and
-    against the same updates with one launch per layer (RLT_MLP_ROWS=0)."""
+@pytest.mark.parametrize("batch,obs,act,hidden,hidden_act", [(256, 6, 1, 256, "fast_tanh"), (100, 17, 6, 128, "relu"), (48, 3, 1, 200, "relu"), (256, 27, 8, 256, "relu"),
+                                                             (30, 111, 8, 72, "tanh"), (512, 5, 2, 16, "sigmoid")])
+def test_wider_agents_match_the_checker_on_both_paths(oracle, rocm, batch, obs, act, hidden, hidden_act):
+    """Hidden widths other than 64 (the zoo's AcrobotSwingup agent: 6-256-256-2 and 7-256-256-1 at batch 256; Ant-sized: 27 / 8): one launch per update on the
+    kernel for widths up to 256 (every network pass of the update by sixteen wavefronts per 16 rows, the optimiser as its last step), and one launch per
+    operation (the few-rows forward kernel, a wavefront per 16 x 16 tile in the backward contractions; also with one launch per layer, RLT_MLP_ROWS=0).
+    Three loop steps' worth of updates against the CPU checker."""
     steps = 3
     params, batches, noises = make_inputs(batch * 7 + hidden, batch, obs, act, steps, hidden)
     results = {}
-    for name, backend, rows in (("checker", oracle, None), ("one_launch", rocm, "1"), ("per_layer", rocm, "0")):
+    for name, backend, per_operation, rows in (("checker", oracle, None, None), ("one_launch", rocm, 0, None), ("per_operation", rocm, 1, "1"), ("per_layer", rocm, 1, "0")):
         if rows is not None:
             os.environ["RLT_MLP_ROWS"] = rows
+        if per_operation is not None:
+            rocm.call("sac_set_per_operation", per_operation)
         try:
             agent = helpers.SacOnBackend(backend, batch, hidden, params, masks=False, obs=obs, act=act, hidden_act=hidden_act)
             results[name] = run_updates(agent, batches, noises)
         finally:
             os.environ.pop("RLT_MLP_ROWS", None)
-    for other in ("checker", "per_layer"):
+            rocm.call("sac_set_per_operation", 0)
+    # which path ran: only the per-operation launches fill the critics' next-input buffer
+    assert not results["one_launch"].pop("next_state_action_value_input").any()
+    assert results["per_operation"].pop("next_state_action_value_input").any() and results["per_layer"].pop("next_state_action_value_input").any()
+    results["checker"].pop("next_state_action_value_input")
+    for other in ("checker", "per_operation", "per_layer"):
         for key, ref in results[other].items():
             err = rel_err(results["one_launch"][key], ref)
-            assert err <= TOL, (other, key, err)
+            # log(1 - a^2 + 1e-6) moves by 1e-4 per ulp of tanh for actions within 1e-3 of +-1: the log-probabilities get that much
+            assert err <= (1e-4 if "log_probabilities" in key else TOL), (other, key, err)
     moved = np.abs(results["one_launch"]["parameters"] - params)
     assert moved.max() > 1e-4 and results["one_launch"]["ages"].tolist() == [1 + steps] * 4
 
@@ -212,13 +222,13 @@ def test_optimiser_in_the_kernel_and_placement_leave_the_same_bits(rocm, batch, 
     assert results[0]["ages"].tolist() == [4] * 4
 
 
-@pytest.mark.parametrize("batch,obs,act", [(256, 3, 1), (64, 11, 3), (300, 27, 8)])
-def test_both_critics_in_one_launch_equal_the_separate_calls(oracle, rocm, batch, obs, act):
+@pytest.mark.parametrize("batch,obs,act,hidden", [(256, 3, 1, 64), (64, 11, 3, 64), (300, 27, 8, 64), (256, 6, 1, 256), (96, 17, 6, 200)])
+def test_both_critics_in_one_launch_equal_the_separate_calls(oracle, rocm, batch, obs, act, hidden):
     """rlt_rocm_sac_train_critics (both critics on the shared batch and the soft update of the targets in one launch; the noise an array or
     drawn by the kernel from its Philox stream) against train_critic(0), train_critic(1), update_critic_targets: bit for bit, and against the
     CPU checker's three calls to 1e-5; then train_actor with its noise drawn by the kernel against randn + train_actor."""
     rng = np.random.default_rng(batch + obs)
-    params = agent_parameters(rng, obs, act)
+    params = agent_parameters(rng, obs, act, hidden)
     oab, rew, term = batch_of(rng, batch, obs, act)
     seed, stream = 77, 123
     noise_dev = rocm.zeros((batch, act))
@@ -227,7 +237,7 @@ def test_both_critics_in_one_launch_equal_the_separate_calls(oracle, rocm, batch
     noise = noise_dev.numpy()
     runs = {}
     for name, backend in (("checker", oracle), ("separate", rocm), ("together", rocm), ("together_drawn", rocm)):
-        agent = helpers.SacOnBackend(backend, batch, 64, params, masks=False, obs=obs, act=act)
+        agent = helpers.SacOnBackend(backend, batch, hidden, params, masks=False, obs=obs, act=act)
         agent.set_batch(oab, rew, term)
         n = backend.array(noise)
         drawn = backend.zeros((batch, act))
