@@ -54,7 +54,13 @@ namespace rl_tools{
         template <typename DEVICE, typename SOURCE_SPEC, typename TARGET_SPEC>
         void strided_copy(DEVICE& device, const Matrix<SOURCE_SPEC>& source, Matrix<TARGET_SPEC>& target, int kind){
             using T = typename TARGET_SPEC::T;
-            if constexpr(dense<SOURCE_SPEC> && dense<TARGET_SPEC>){
+            if constexpr(!std::is_arithmetic_v<utils::typing::remove_cv_t<T>>){
+                // matrices of structs are host memory on every device (malloc above): copied element by element on the host, whatever the direction
+                for(size_t row = 0; row < (size_t)TARGET_SPEC::ROWS; row++){
+                    for(size_t col = 0; col < (size_t)TARGET_SPEC::COLS; col++){ target._data[row * leading_dimension<TARGET_SPEC> + col] = source._data[row * leading_dimension<SOURCE_SPEC> + col]; }
+                }
+            }
+            else if constexpr(dense<SOURCE_SPEC> && dense<TARGET_SPEC>){
                 const size_t bytes = (size_t)TARGET_SPEC::ROWS * TARGET_SPEC::COLS * sizeof(T);
                 const int rc = kind == 0 ? rlt_rocm_memcpy_d2d(device.handle, (void*)target._data, (const void*)source._data, bytes)
                              : kind == 1 ? rlt_rocm_memcpy_h2d(device.handle, (void*)target._data, (const void*)source._data, bytes)

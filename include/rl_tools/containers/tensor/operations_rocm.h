@@ -54,7 +54,12 @@ namespace rl_tools{
             static_assert(utils::typing::is_same_v<utils::typing::remove_cv_t<typename FROM_SPEC::T>, utils::typing::remove_cv_t<typename TO_SPEC::T>>, "copies across the host / device boundary keep the element type");
             using T = typename TO_SPEC::T;
             using TI = typename DEVICE::index_t;
-            if constexpr(tensor::dense_row_major_layout<FROM_SPEC>() && tensor::dense_row_major_layout<TO_SPEC>()){
+            if constexpr(!std::is_arithmetic_v<utils::typing::remove_cv_t<T>>){
+                // containers of structs (an optimiser's hyper-parameters) are host memory on every device (malloc above): copied element by element on the host, whatever the direction
+                static_assert(tensor::dense_row_major_layout<FROM_SPEC>() && tensor::dense_row_major_layout<TO_SPEC>(), "containers of structs are copied whole");
+                for(size_t i = 0; i < (size_t)FROM_SPEC::SIZE; i++){ to._data[i] = from._data[i]; }
+            }
+            else if constexpr(tensor::dense_row_major_layout<FROM_SPEC>() && tensor::dense_row_major_layout<TO_SPEC>()){
                 const size_t bytes = (size_t)FROM_SPEC::SIZE * sizeof(T);
                 const int rc = kind == 0 ? rlt_rocm_memcpy_d2d(device.handle, (void*)to._data, (const void*)from._data, bytes)
                              : kind == 1 ? rlt_rocm_memcpy_h2d(device.handle, (void*)to._data, (const void*)from._data, bytes)

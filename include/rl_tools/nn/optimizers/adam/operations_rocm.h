@@ -127,7 +127,8 @@ namespace rl_tools{
         p.enable_gradient_clipping = DEFAULTS::ENABLE_GRADIENT_CLIPPING; p.gradient_clip_value = DEFAULTS::GRADIENT_CLIP_VALUE;
         devices::rocm::check(rlt_rocm_adam_step(device.handle, tensors.data(), (int)tensors.size(), &p, (uint32_t*)optimizer.age._data, 0.0f, nullptr), "step(adam)");
     }
-    // copies of the optimiser between devices: age on the device, hyper-parameters on the host (operations_generic.h:67-71 copies both)
+    // copies of the optimiser between devices: age on the device, hyper-parameters on the host (operations_generic.h:67-71 copies both). X -> ROCM resolves to the
+    // reference's generic copy, whose two tensor copies land on the overloads of containers/tensor/operations_rocm.h (the hyper-parameters, a tensor of structs, stay on the host)
     template<typename SOURCE_DEV_SPEC, typename TARGET_DEVICE, typename SOURCE_SPEC, typename TARGET_SPEC>
     void copy(devices::ROCM<SOURCE_DEV_SPEC>& source_device, TARGET_DEVICE& target_device, const nn::optimizers::Adam<SOURCE_SPEC>& source, nn::optimizers::Adam<TARGET_SPEC>& target){
         copy(source_device, target_device, source.age, target.age);

@@ -131,6 +131,35 @@ int main(){
         if(print){ std::printf("\n"); }
     }
     rlt::check_status(device);
+    // the whole agent CPU -> ROCM -> CPU, optimisers included (their hyper-parameters are a container of structs, which stays in host memory on the device side)
+    bool optimisers_ok = true;
+    {
+        static typename CONFIG_DEV::ACTOR_CRITIC_TYPE there;
+        static typename CONFIG_CPU::ACTOR_CRITIC_TYPE and_back;
+        rlt::malloc(device, there); rlt::malloc(cpu, and_back);
+        ts_cpu.actor_critic.actor_optimizer.parameters._data[0].alpha = 0.0123f;
+        ts_cpu.actor_critic.critic_optimizers[1].parameters._data[0].beta_2 = 0.987f;
+        rlt::copy(cpu, device, ts_cpu.actor_critic, there);
+        rlt::copy(device, device, there, ts_dev.actor_critic);
+        rlt::copy(device, cpu, ts_dev.actor_critic, and_back);
+        rlt::check_status(device);
+        auto same = [&](auto& a, auto& b){
+            const auto& p = a.parameters._data[0]; const auto& q = b.parameters._data[0];
+            return p.alpha == q.alpha && p.beta_1 == q.beta_1 && p.beta_2 == q.beta_2 && p.epsilon == q.epsilon && p.epsilon_sqrt == q.epsilon_sqrt && p.bias_lr_factor == q.bias_lr_factor
+                && rlt::get(cpu, a.age, 0) == rlt::get(cpu, b.age, 0);
+        };
+        optimisers_ok = same(and_back.actor_optimizer, ts_cpu.actor_critic.actor_optimizer) && same(and_back.critic_optimizers[0], ts_cpu.actor_critic.critic_optimizers[0])
+                     && same(and_back.critic_optimizers[1], ts_cpu.actor_critic.critic_optimizers[1]) && same(and_back.alpha_optimizer, ts_cpu.actor_critic.alpha_optimizer)
+                     && and_back.actor_optimizer.parameters._data[0].alpha == 0.0123f && rlt::get(cpu, and_back.actor_optimizer.age, 0) == 21;
+        T worst_copy = 0;
+        auto compare_copy = [&](auto& a, auto& b){ const T d = rlt::abs_diff(cpu, a, b); worst_copy = d > worst_copy ? d : worst_copy; };
+        compare_copy(and_back.actor.content.hidden_layers[0].weights.parameters, ts_cpu.actor_critic.actor.content.hidden_layers[0].weights.parameters);
+        compare_copy(and_back.critics[1].content.input_layer.weights.gradient_first_order_moment, ts_cpu.actor_critic.critics[1].content.input_layer.weights.gradient_first_order_moment);
+        compare_copy(and_back.critics_target[0].content.output_layer.biases.parameters, ts_cpu.actor_critic.critics_target[0].content.output_layer.biases.parameters);
+        optimisers_ok = optimisers_ok && worst_copy == 0;
+        std::printf("whole-agent round trip: %s\n", optimisers_ok ? "identical" : "DIFFERENT");
+        rlt::free(device, there); rlt::free(cpu, and_back);
+    }
     std::printf("worst %.2e\n", worst);
-    return worst <= 1e-5f ? 0 : 1;
+    return (worst <= 1e-5f && optimisers_ok) ? 0 : 1;
 }

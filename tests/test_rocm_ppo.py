@@ -51,11 +51,12 @@ def test_surrogate_gradient_matches_checker(oracle, rocm, batch, action_dim, nor
         assert np.array_equal(res[1][1], np.full(action_dim, 0.25, np.float32))
 
 
-def test_train_minibatch_matches_checker_on_synthetic_dataset(oracle, rocm):
-    """The shape of the synthetic PPO benchmark (observation 105, action 8, hidden 64, tanh) at minibatch 512: one update compared
-    tensor by tensor, then eight updates on shuffled rows compared at the end."""
+@pytest.mark.parametrize("B,N,updates", [(512, 4096, 8), (8192, 32768, 3)])
+def test_train_minibatch_matches_checker_on_synthetic_dataset(oracle, rocm, B, N, updates):
+    """The shape of the synthetic PPO benchmark (observation 105, action 8, hidden 64, tanh) at minibatch 512 and at the benchmark's own 8,192:
+    one update compared tensor by tensor, then several updates on shuffled rows compared at the end."""
     capi = helpers.capi
-    O, A, H, B, N = 105, 8, 64, 512, 4096
+    O, A, H = 105, 8, 64
     rng = np.random.default_rng(2)
     na, nc = helpers.mlp_param_count([O, H, H, A]), helpers.mlp_param_count([O, H, H, 1])
     params = np.concatenate([helpers.random_params(rng, [O, H, H, A]), np.log(np.full(A, 0.5, np.float32)), helpers.random_params(rng, [O, H, H, 1])])
@@ -81,13 +82,16 @@ def test_train_minibatch_matches_checker_on_synthetic_dataset(oracle, rocm):
         b.sync()
         first = dict(actor_grads=agent.actor.grads.numpy(), critic_grads=agent.critic.grads.numpy(), d_log_std=agent.d_log_std.numpy(), loss=loss.numpy(),
                      params=agent.parameters())
-        for k in range(8):
+        for k in range(updates):
             b.call("ppo_train_minibatch", C.byref(agent.c), C.byref(pp), *args, idx.offset(k * B), loss.ptr)
         b.sync()
         results.append((first, agent.parameters(), loss.numpy()))
     (f0, p0, l0), (f1, p1, l1) = results
     for key in f0:
-        assert rel_err(f1[key], f0[key]) <= TOL, (key, rel_err(f1[key], f0[key]))
+        # d_log_std: the reference (and the checker, bit for bit) adds 2 * batch terms one by one into a single fp32 accumulator per action dimension,
+        # which carries a rounding error of up to batch * 2^-24 of the running magnitude; the kernel sums in a tree
+        bound = max(TOL, B * 2.0 ** -24) if key == "d_log_std" else TOL
+        assert rel_err(f1[key], f0[key]) <= bound, (key, rel_err(f1[key], f0[key]))
     assert rel_err(p1, p0) <= 2e-4 and rel_err(l1, l0) <= 1e-4
 
 
