@@ -672,11 +672,18 @@ int rlt_rocm_sac_train_critics_drawn(rlt_rocm_device* device, const rlt_sac_agen
 int rlt_rocm_sac_train_actor_drawn(rlt_rocm_device* device, const rlt_sac_agent* agent, float* drawn_noise, uint64_t seed, uint64_t stream);
 
 /* How the fused update kernels (SAC / TD3 / PPO minibatch, networks in -> 64 -> 64 -> out) finish. optimiser_in_kernel != 0 (default):
- * the last workgroup of the launch to finish adds up the workgroups' partial gradients in a fixed order and applies the optimiser's
- * step, so an update is one launch; 0: the optimiser runs as a launch of its own after the kernel (same bits). one_xcd != 0 (default):
+ * every workgroup waits (bounded, see rlt_rocm_set_wait_limit) until all have stored their partial gradients, then adds up a slice of them
+ * in a fixed order and applies the optimiser's step (and the targets' soft update) to that slice, so an update is one launch (grids of up to
+ * 64 workgroups); 0: the optimiser runs as a launch of its own after the kernel (same bits). one_xcd != 0 (default):
  * grids of at most 32 workgroups are placed on one XCD, whose L2 then serves the exchange; 0: spread over all XCDs. The environment
  * variables RLT_UPDATE_TAIL=0 and RLT_UPDATE_PLACEMENT=spread set the defaults of a process. No counterpart in the reference. */
 int rlt_rocm_set_update_options(rlt_rocm_device* device, int optimiser_in_kernel, int one_xcd);
+/* The kernels whose workgroups wait for each other (the persistent SAC loop; update kernels that end with the optimiser's step) poll a
+ * bounded number of times, then give up: the kernel still ends normally, its results are void, and the next rlt_rocm_check_status returns
+ * RLT_E_DEVICE_TIMEOUT. `polls` sets that bound (0: the default, about a second). With a bound of 1 every workgroup of an update kernel
+ * but the last to arrive gives up without looking at the counter, which makes the give-up path testable from the host. No counterpart in
+ * the reference. */
+int rlt_rocm_set_wait_limit(rlt_rocm_device* device, unsigned polls);
 
 /* The same n_steps iterations of sac::loop::core::step (rl/algorithms/sac/loop/core/operations_generic.h:110-155 past the warm-up,
  * SHARED_BATCH: runner step with the actor, one gather_batch and one critic noise draw for both train_critic calls,

@@ -367,7 +367,7 @@ ROCM_ONLY = {
     "sac_train_critics": ([P, C.POINTER(SacAgent), P, I], I),
     "sac_train_critics_drawn": ([P, C.POINTER(SacAgent), P, U64, U64, I], I),
     "sac_train_actor_drawn": ([P, C.POINTER(SacAgent), P, U64, U64], I),
-    "set_update_options": ([P, I, I], I),
+    "set_update_options": ([P, I, I], I), "set_wait_limit": ([P, C.c_uint32], I),
     "graph_begin_capture": ([P], I), "graph_end_capture": ([P, C.POINTER(P)], I), "graph_launch": ([P, P], I), "graph_destroy": ([P, P], I),
     "advance_streams": ([P, U64], I), "set_stream_offset": ([P, U64], I),
 }

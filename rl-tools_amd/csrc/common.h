@@ -24,6 +24,7 @@ struct rlt_rocm_device {
     int sac_per_operation;       // rlt_rocm_sac_train_critic / _actor run one launch per reference operation even where the fused kernels fit
     int update_tail;             // the fused update kernels step the optimiser themselves (their last workgroup), instead of in launches after them
     int update_one_xcd;          // small grids of the fused update kernels are placed on one XCD
+    unsigned wait_limit;         // polls after which a workgroup gives up waiting for another (rlt_rocm_set_wait_limit; about a second by default)
     int capturing;               // the stream is recording a graph: nothing may allocate, free or wait (rlt_rocm_graph_begin_capture)
     uint64_t* stream_offset;     // device word added to the stream number of every draw made on the device (rlt_rocm_advance_streams)
 };

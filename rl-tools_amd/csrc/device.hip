@@ -162,6 +162,7 @@ int rlt_rocm_init(int hip_device_index, rlt_rocm_device** out_device) {
         const char* t = std::getenv("RLT_UPDATE_TAIL"); const char* q = std::getenv("RLT_UPDATE_PLACEMENT");
         device->update_tail = !(t && std::strcmp(t, "0") == 0);
         device->update_one_xcd = !(q && std::strcmp(q, "spread") == 0);
+        device->wait_limit = 1u << 20;
     }
     *out_device = device;
     return 0;
@@ -169,6 +170,11 @@ int rlt_rocm_init(int hip_device_index, rlt_rocm_device** out_device) {
 int rlt_rocm_set_update_options(rlt_rocm_device* device, int optimiser_in_kernel, int one_xcd) {
     if (!device) return RLT_E_NOT_INITIALISED;
     device->update_tail = optimiser_in_kernel != 0; device->update_one_xcd = one_xcd != 0;
+    return 0;
+}
+int rlt_rocm_set_wait_limit(rlt_rocm_device* device, unsigned polls) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    device->wait_limit = polls ? polls : 1u << 20;
     return 0;
 }
 int rlt_rocm_destroy(rlt_rocm_device* device) {

@@ -154,9 +154,9 @@ inline bool rlt_tail_optimizer_fill(rlt_tail_optimizer& O, const rlt_adam_tensor
 // that are through; the last one clears both words (they are zero between launches) and advances the ages.
 // same_xcd: the working workgroups share one XCD (see rlt_load_shared).
 constexpr int RLT_TAIL_MAX_WORKGROUPS = 64;
-constexpr unsigned RLT_TAIL_MAX_POLL = 1u << 20;      // about a second
 struct rlt_tail_args {
     int enabled, same_xcd;
+    unsigned max_poll;                               // polls after which a waiting workgroup gives up (the device handle's wait limit)
     uint32_t* tickets; unsigned* fault;
     const float* partial; int count;                 // blocks of `count` floats
     rlt_tail_optimizer opt[2];                       // per trained network of the launch (blockIdx.y)
@@ -233,6 +233,7 @@ template <int THREADS>
 __device__ __noinline__ void rlt_optimiser_tail(rlt_tail_pointer A, int y, int g, int G, __attribute__((address_space(3))) int* flag_word) {
     const unsigned total = (unsigned)G * gridDim.y;
     const int same_xcd = A->same_xcd;
+    const unsigned max_poll = A->max_poll;
     uint32_t* const tickets = A->tickets;
     unsigned* const fault = A->fault;
     unsigned long long* const ticks = A->ticks;
@@ -240,15 +241,19 @@ __device__ __noinline__ void rlt_optimiser_tail(rlt_tail_pointer A, int y, int g
     if (!same_xcd) __threadfence();           // and are visible beyond this XCD
     __syncthreads();
     if (threadIdx.x == 0) {
-        __hip_atomic_fetch_add(tickets, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        unsigned tries = 0; int ok = 1;
-        while (__hip_atomic_load(tickets, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < total) {
-            __builtin_amdgcn_s_sleep(1);
-            if (++tries >= RLT_TAIL_MAX_POLL || ((tries & 63u) == 0u && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
-                __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                ok = 0;
-                break;
-            }
+        // the last workgroup to arrive learns so from its own ticket and goes on at once; every other one sleeps, then looks at the
+        // word, at most max_poll - 1 times (a bound of one poll makes all but the last give up without looking)
+        int ok = 1;
+        if (__hip_atomic_fetch_add(tickets, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u < total) {
+            unsigned tries = 0;
+            do {
+                if (++tries >= max_poll || ((tries & 63u) == 0u && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+                    __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ok = 0;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            } while (__hip_atomic_load(tickets, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < total);
         }
         *flag_word = ok;
     }

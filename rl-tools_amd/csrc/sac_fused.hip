@@ -58,7 +58,6 @@ constexpr int THREADS = 512;
 constexpr int MAX_G = 64;
 constexpr int R = 2 * OBS + ACT + 3;    // floats per replay row
 constexpr int MAX_PACKED_G = 32;        // workgroups that fit on one XCD (32 CUs) with one workgroup per CU
-constexpr unsigned MAX_POLL = 1u << 20; // bounded wait for another workgroup's data (about a second), then the run is abandoned
 
 // A 3-layer network IN -> H -> H -> OUT: offsets in its flat arena [W1|b1|W2|b2|W3|b3] and in the workgroup's LDS copy. The
 // LDS rows are padded to odd strides so that the 16 rows a tile reads side by side fall into different banks; W1 rows are
@@ -101,6 +100,7 @@ struct FusedArgs {
     rlt_replay_buffer rb;
     float* partial;            // [G + 1][N_PARTIAL], row G stays zero
     unsigned* fault;           // set when a workgroup gave up waiting
+    unsigned max_poll;         // polls after which a waiting workgroup gives up: bounded wait for another workgroup's data (about a second by default), then the run is abandoned
     unsigned* xcd_mask;        // bit x set: some workgroup of this launch ran on XCD x
     unsigned* ready;           // [4][64] per exchange kind and workgroup: the sequence number of the last completed exchange
     // optional host-drawn randomness (parity runs); NULL -> counter-based device RNG
@@ -149,10 +149,10 @@ __device__ __forceinline__ void give_up(unsigned* fault, __attribute__((address_
     *abort_flag = 1;
 }
 // true while waiting may go on: not too long yet, and no workgroup has given up
-__device__ __forceinline__ bool keep_waiting(unsigned& tries, const unsigned* fault) {
+__device__ __forceinline__ bool keep_waiting(unsigned& tries, const unsigned* fault, unsigned max_poll) {
     __builtin_amdgcn_s_sleep(1);      // a waiting wavefront should not keep the memory system busy
     ++tries;
-    if (tries >= MAX_POLL) return false;
+    if (tries >= max_poll) return false;
     if ((tries & 63u) == 0u && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) return false;
     return true;
 }
@@ -170,11 +170,11 @@ __device__ __forceinline__ void announce(unsigned* ready, int kind, int g, unsig
     }
 }
 // wavefront 0 waits for all G words, the others wait for it at the workgroup barrier
-__device__ __forceinline__ void await(const unsigned* ready, int kind, int G, unsigned tag, const unsigned* fault, __attribute__((address_space(3))) int* abort_flag) {
+__device__ __forceinline__ void await(const unsigned* ready, int kind, int G, unsigned tag, const unsigned* fault, __attribute__((address_space(3))) int* abort_flag, unsigned max_poll) {
     if (threadIdx.x < 64) {
         const unsigned* p = ready + kind * READY_STRIDE + min((int)threadIdx.x, G - 1);
         unsigned tries = 0;
-        while (__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < tag) if (!keep_waiting(tries, fault)) { give_up(const_cast<unsigned*>(fault), abort_flag); break; }
+        while (__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < tag) if (!keep_waiting(tries, fault, max_poll)) { give_up(const_cast<unsigned*>(fault), abort_flag); break; }
     }
     rlt_lds_barrier();
 }
@@ -733,7 +733,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         announce<PACKED>(A.ready, READY_CRITIC_GRADIENTS, g, seq);
         tick(2);
         // ================= S2: reduce + Adam + polyak for both critics =================
-        await(A.ready, READY_CRITIC_GRADIENTS, G, seq, A.fault, &S->abort);
+        await(A.ready, READY_CRITIC_GRADIENTS, G, seq, A.fault, &S->abort, A.max_poll);
         {
             constexpr int total = 2 * NC::total;
             const int chunk = (total + G - 1) / G;
@@ -768,7 +768,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         }
         tick(3);
         announce<PACKED>(A.ready, READY_CRITIC_PARAMETERS, g, seq);
-        await(A.ready, READY_CRITIC_PARAMETERS, G, seq, A.fault, &S->abort);
+        await(A.ready, READY_CRITIC_PARAMETERS, G, seq, A.fault, &S->abort, A.max_poll);
         tick(4);
         // both critics are needed now; the target critics, read next in the following step's critic phase, follow from them later in this step
         float fresh[2][NC::per_thread];
@@ -850,7 +850,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
             const lptr dst_t[2] = {w_target0, w_target1};
             polyak_nets<NC, 2>(dst_t, fresh, A.polyak, tid);
         }
-        await(A.ready, READY_ACTOR_GRADIENTS, G, seq, A.fault, &S->abort);
+        await(A.ready, READY_ACTOR_GRADIENTS, G, seq, A.fault, &S->abort, A.max_poll);
         tick(7);
         // ================= S4: reduce + Adam for the actor and log_alpha =================
         {
@@ -877,7 +877,7 @@ __global__ __launch_bounds__(THREADS) void sac_pendulum_loop_kernel(FusedArgs A)
         }
         tick(8);
         announce<PACKED>(A.ready, READY_ACTOR_PARAMETERS, g, seq);
-        await(A.ready, READY_ACTOR_PARAMETERS, G, seq, A.fault, &S->abort);
+        await(A.ready, READY_ACTOR_PARAMETERS, G, seq, A.fault, &S->abort, A.max_poll);
         tick(9);
         {
             const lptr dst_a[1] = {w_actor}; const float* const src_a[1] = {A.actor_p};
@@ -975,7 +975,7 @@ extern "C" int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac
     a.batch = B; a.n_steps = n_steps;
     a.runner = *runner; a.rb = *rb;
     a.xcd_mask = (unsigned*)scratch; a.ready = (unsigned*)((char*)scratch + 256); a.partial = (float*)((char*)scratch + 2048);
-    a.fault = device->fault;
+    a.fault = device->fault; a.max_poll = device->wait_limit;
     if (inputs) { a.rollout_noise = inputs->rollout_noise; a.initial_states = inputs->initial_states; a.sample_offsets = inputs->sample_offsets;
                   a.noise_critic = inputs->noise_critic; a.noise_actor = inputs->noise_actor; }
     a.seed = seed; a.step_offset = step_offset;

@@ -634,7 +634,7 @@ bool configure_tail(rlt_rocm_device* device, UpdateArgs& a, const Optimiser* opt
     void* counters = nullptr;
     if (rlt_counters(device, &counters)) return false;
     T.tickets = (uint32_t*)counters + RLT_TICKET_TAIL;
-    T.fault = device->fault;
+    T.fault = device->fault; T.max_poll = device->wait_limit;
     T.polyak = polyak;
     T.partial = a.partial; T.count = a.count; T.same_xcd = a.packed;
     T.enabled = 1;

@@ -74,5 +74,5 @@ def test_sizes_beyond_the_fixed_array_are_rejected(rocm):
     assert lib.rlt_rocm_dense_backward_static(h, None, x.ptr, i, d.ptr, o, batch) == capi.RLT_E_INVALID_ARGUMENT
     assert lib.rlt_rocm_dense_backward(h, C.byref(L), x.ptr, i, d.ptr, o, batch) == 0     # the allocating entry point takes the size
     rocm.sync()
-    for a in (x, d, pre):
+    for a in (x, d, pre, w, b, dw, db):
         a.free()
