@@ -21,6 +21,11 @@ int rlt_mlp3s_ppo_actor(rlt_rocm_device* device, const rlt_dense_layer* layers, 
 // true if the two networks can share a launch: both of the supported shape, the same hidden activation, input widths on the same side of 32
 bool rlt_mlp3s_pair_supported(const rlt_dense_layer* a, int n_a, const rlt_dense_layer* b, int n_b);
 
+// steps[0] (actor), steps[1] (critic), optional: the optimisers' steps (nn/optimizers/adam/operations_generic.h:43-66) follow in ONE launch that adds the
+// workgroups' blocks of partial gradient sums up itself, where each optimiser's tensors are exactly the network's gradient buffers (the actor's plus
+// d_log_std); *stepped then is true. Otherwise the gradients are formed as without `steps` and the caller steps the optimisers.
+struct rlt_mlp3s_step { const rlt_adam_tensor* tensors; int n; const rlt_adam_parameters* parameters; uint32_t* age; };
+
 // The same actor pass and the critic's forward + MSE gradient + backward (:289-300) in ONE launch, each network on half of the compute units,
 // straight from the dataset: every input column has the dataset's row stride `ld`, and minibatch row b is dataset row rows[b] (rows == NULL: b).
 // Means [batch x action_dim] and values [batch] are written packed; out_critic_loss (optional, critic output width 1) receives
@@ -33,7 +38,8 @@ int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* a
                                const rlt_dense_layer* critic, int n_critic, const float* x_critic, float* values, int ld_values,
                                const float* target_values, float mse_scale, float* out_critic_loss, int ld, const uint32_t* rows, int batch,
                                const float* actor_std_mean = nullptr, const float* actor_std_precision = nullptr,
-                               const float* critic_std_mean = nullptr, const float* critic_std_precision = nullptr);
+                               const float* critic_std_mean = nullptr, const float* critic_std_precision = nullptr,
+                               const rlt_mlp3s_step* steps = nullptr, bool* stepped = nullptr);
 
 // For kernels that write blocks of partial sums in this file's layout (dW1 [64 x in], db1 [64], dW2 [64 x 64], db2 [64], dW3 [out x 64], db3 [out],
 // extra [16]): the floats per block, and the launch that adds `groups` blocks up in block order into the layers' gradients (overwrite != 0:

@@ -14,6 +14,8 @@
 // once per workgroup in LDS (padded rows, read as both W and W^T). Four workgroup barriers per round order the two kinds of phase.
 // Bound: the fp32 matrix pipe, 2 (in + 64 + out) 64 flop per row forward and twice that backward less the input gradient of layer 1.
 #include "mlp_small.h"
+#include "optim.h"
+#include "xcd_reduce.h"
 
 namespace {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -57,14 +59,9 @@ constexpr size_t lds_floats(int nt1c) {
     return (size_t)H * sx + H * HS + MAX_OUT * HS + (size_t)ROWS * (sx + 3 * HS + D3S);
 }
 
-// lane l: the row of the input arrays that row (l & 15) of a tile reads; rows beyond the batch are clamped here and masked later
-__device__ __forceinline__ uint32_t tile_rows(const SmallArgs& A, int tile, int lane) {
-    const int b = min(tile * 16 + (lane & 15), A.batch - 1);
-    return A.rows ? A.rows[b] : (uint32_t)b;
-}
 // global loads of one tile of 16 rows, issued together: the inputs (lane = column, up to two columns per lane) and what the loss needs of the
 // rows this lane will hold after the forward pass (rows 4 kk + v, column r); columns beyond the extent are clamped here and masked later.
-// `vrows` comes from tile_rows(), requested a round earlier so that nothing waits for it here.
+// `vrows`: the rows' indices, requested a round earlier so that nothing waits for them here.
 struct TileRegs { float xa[16], xb[16], in0[4], in1[4], in2[4]; };
 __device__ __forceinline__ void request_tile(const SmallArgs& A, uint32_t vrows, int lane, TileRegs& T) {
     const int r = lane & 15, kk = lane >> 4;
@@ -85,17 +82,34 @@ __device__ __forceinline__ void request_tile(const SmallArgs& A, uint32_t vrows,
     }
 }
 
+
+// profiling builds (-DRLT_SMALL_PROFILE): thread 0 of workgroup 0 notes the constant-rate clock at the stage boundaries, rlt_mlp3s_ticks copies the notes out
+#ifdef RLT_SMALL_PROFILE
+__device__ unsigned long long rlt_small_ticks[32];
+__device__ unsigned long long rlt_small_spans[512][2];
+#define RLT_TICK(i) do { if (blockIdx.x == 0 && threadIdx.x == 0) rlt_small_ticks[i] = wall_clock64(); } while (0)
+#else
+#define RLT_TICK(i) do {} while (0)
+#endif
+
 // ACT_H: hidden activation; NT1C: number of 16-column tiles of dW1 the code is unrolled for (>= the NT1 the input width needs; the surplus
 // tiles multiply zero columns and are never stored). Both are compile-time constants: a matrix instruction under a run-time
 // condition makes the compiler carry both versions of its accumulator.
 // One launch can carry two networks (PPO's actor and critic on the same minibatch): workgroups [0, groups0) work on A0, the rest on A1.
 // LAYERS = 2: the network is in -> 64 -> out; layer 2, its weight gradient and its input gradient drop out, the output layer reads h1, and the
 // gradient at layer 1's pre-activations is formed directly from the output layer's.
+// xr (optional): the blocks of partial sums are added up per XCD inside the launch (xcd_reduce.h); network j's eight blocks of sums then lie at xsum[j]
+struct SmallLaunch { SmallArgs a0, a1; int groups0; rlt_xcd_reduce_args xr; float* xsum[2]; };
 template <int ACT_H, int NT1C, int LAYERS>
-__global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs A1, int groups0) {
+__global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallLaunch K) {
+    RLT_TICK(0);
+#ifdef RLT_SMALL_PROFILE
+    if (threadIdx.x == 0) rlt_small_spans[blockIdx.x][0] = wall_clock64();
+#endif
     extern __shared__ float lds_raw[];
+    const int groups0 = K.groups0;
     const bool second = (int)blockIdx.x >= groups0;
-    const SmallArgs& A = second ? A1 : A0;
+    const SmallArgs& A = second ? K.a1 : K.a0;
     const int block = second ? blockIdx.x - groups0 : blockIdx.x, n_blocks = second ? gridDim.x - groups0 : groups0;
     const int lane = threadIdx.x & 63, r = lane & 15, kk = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);      // wavefront-uniform: addresses derived from it are computed on the scalar unit
@@ -105,11 +119,32 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
     const lptr xs_all = w3s + MAX_OUT * HS, h1s_all = xs_all + ROWS * SX, h2s_all = h1s_all + ROWS * HS, g2s_all = h2s_all + ROWS * HS, d3s_all = g2s_all + ROWS * HS;
     const lptr xs = xs_all + 16 * wave * SX, h1s = h1s_all + 16 * wave * HS, h2s = h2s_all + 16 * wave * HS, g2s = g2s_all + 16 * wave * HS, d3s = d3s_all + 16 * wave * D3S;
     const int n_tiles = (A.batch + 15) >> 4, n_rounds = (n_tiles + WAVES - 1) / WAVES;
-    // row indices of this wavefront's first two tiles, then the first tile's loads, ahead of the weights'; a wavefront whose tile lies beyond the
-    // batch computes on clamped rows and masks them
-    uint32_t rows_next = tile_rows(A, min(block * WAVES + wave, n_tiles - 1), lane), rows_after = tile_rows(A, min((block + n_blocks) * WAVES + wave, n_tiles - 1), lane);
+    // lane l: the row of the input arrays that row (l & 15) of this wavefront's tile of round `round` reads; a tile beyond the batch is clamped here and masked later
+    auto rows_of = [&](int round) -> uint32_t {
+        const int b = min(min(round * WAVES + wave, n_tiles - 1) * 16 + (lane & 15), A.batch - 1);
+        return A.rows ? A.rows[b] : (uint32_t)b;
+    };
+    // The launch's critical path starts with two dependent trips to memory (the row indices, then the rows): the index loads go out first, the
+    // weights' and constants' loads follow while the indices travel, then the first tile's loads, and the weights are stored to LDS while those
+    // travel.
+    uint32_t rows_next = rows_of(block), rows_after = rows_next;
+    if (block + n_blocks < n_rounds) rows_after = rows_of(block + n_blocks);
     TileRegs T;
-    request_tile(A, rows_next, lane, T);
+    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    const int xgroup = (second ? RLT_XCD_GROUPS : 0) + (block & 7);      // with the XCD-level sums: this workgroup's group (network, XCD)
+    uint32_t xepoch = 0;
+    if (K.xr.enabled) xepoch = rlt_xcd_epoch(K.xr, xgroup);
+    float v1[H / WAVES][2], v2[H * H / THREADS], v3[MAX_OUT * H / THREADS];
+#pragma unroll
+    for (int j = 0; j < H / WAVES; j++) {
+        const float* src = A.W1 + (size_t)(wave * (H / WAVES) + j) * IN;
+        v1[j][0] = src[min(lane, IN - 1)];
+        v1[j][1] = IN > 64 ? src[min(64 + lane, IN - 1)] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < H * H / THREADS; u++) v2[u] = LAYERS == 3 ? A.W2[u * THREADS + threadIdx.x] : 0.f;
+#pragma unroll
+    for (int u = 0; u < MAX_OUT * H / THREADS; u++) v3[u] = A.W3[min(u * THREADS + (int)threadIdx.x, OUT * H - 1)];
     float b1r[4], b2r[4];
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) { b1r[nt] = A.b1[16 * nt + r]; b2r[nt] = LAYERS == 3 ? A.b2[16 * nt + r] : 0.f; }
@@ -119,20 +154,18 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
         ls = A.log_std[min(r, OUT - 1)];
         if (A.normalize_advantage) { adv_mean = A.stats[0]; adv_std = A.stats[1]; }
     }
-    // weights into LDS, rows padded to SX (zero beyond the input width, so the padded reduction steps add nothing); every load is in flight
-    // before the first is stored
+    // the standardize layer's constants for this lane's columns (nn/layers/standardize/operations_generic.h:68-86); without one: x - 0 times 1
+    float sm0 = 0.f, sp0 = 1.f, sm1 = 0.f, sp1 = 1.f;
+    if (A.std_mean) {
+        sm0 = A.std_mean[min(lane, IN - 1)]; sp0 = A.std_precision[min(lane, IN - 1)];
+        if (IN > 64) { sm1 = A.std_mean[min(64 + lane, IN - 1)]; sp1 = A.std_precision[min(64 + lane, IN - 1)]; }
+        sp0 = sp0 != 0.f ? sp0 : 1.f; sp1 = sp1 != 0.f ? sp1 : 1.f;
+    }
+    __builtin_amdgcn_sched_barrier(0);      // the loads above are issued before the first wait for the row indices
+    request_tile(A, rows_next, lane, T);
+    RLT_TICK(1);
+    // weights into LDS, rows padded to SX (zero beyond the input width, so the padded reduction steps add nothing)
     {
-        float v1[H / WAVES][2], v2[H * H / THREADS], v3[MAX_OUT * H / THREADS];
-#pragma unroll
-        for (int j = 0; j < H / WAVES; j++) {
-            const float* src = A.W1 + (size_t)(wave * (H / WAVES) + j) * IN;
-            v1[j][0] = src[min(lane, IN - 1)];
-            v1[j][1] = IN > 64 ? src[min(64 + lane, IN - 1)] : 0.f;
-        }
-#pragma unroll
-        for (int u = 0; u < H * H / THREADS; u++) v2[u] = LAYERS == 3 ? A.W2[u * THREADS + threadIdx.x] : 0.f;
-#pragma unroll
-        for (int u = 0; u < MAX_OUT * H / THREADS; u++) v3[u] = A.W3[min(u * THREADS + (int)threadIdx.x, OUT * H - 1)];
 #pragma unroll
         for (int j = 0; j < H / WAVES; j++) {
             const lptr dst = w1s + (wave * (H / WAVES) + j) * SX;
@@ -145,10 +178,11 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
 #pragma unroll
         for (int u = 0; u < MAX_OUT * H / THREADS; u++) { const int i = u * THREADS + threadIdx.x; w3s[(i >> 6) * HS + (i & 63)] = (i >> 6) < OUT ? v3[u] : 0.f; }
     }
+    RLT_TICK(2);
     const float sd = expf(ls);
     rlt_lds_barrier();
 
-    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    RLT_TICK(3);
     // this wavefront's share of the weight gradients: rows 16 wave + 4 kk + v of dW1 (columns 16 nt + r) and of dW2, columns 16 wave + r of dW3 (rows 4 kk + v)
     floatx4 aW1[NT1C], aW2[4], aW3a = zero4, aW3b = zero4;
 #pragma unroll
@@ -156,14 +190,6 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) aW2[nt] = zero4;
     float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f}, s3 = 0.f, gls = 0.f;      // bias gradients and the extra sums (PPO: log_std gradient; MSE: squared error) over this wavefront's rows
-
-    // the standardize layer's constants for this lane's columns (nn/layers/standardize/operations_generic.h:68-86); without one: x - 0 times 1
-    float sm0 = 0.f, sp0 = 1.f, sm1 = 0.f, sp1 = 1.f;
-    if (A.std_mean) {
-        sm0 = A.std_mean[min(lane, IN - 1)]; sp0 = A.std_precision[min(lane, IN - 1)];
-        if (IN > 64) { sm1 = A.std_mean[min(64 + lane, IN - 1)]; sp1 = A.std_precision[min(64 + lane, IN - 1)]; }
-        sp0 = sp0 != 0.f ? sp0 : 1.f; sp1 = sp1 != 0.f ? sp1 : 1.f;
-    }
 
     for (int round = block; round < n_rounds; round += n_blocks) {
         const int tile = round * WAVES + wave, row0 = tile * 16;
@@ -174,33 +200,40 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
             if (lane < 16 * NT1C) xs[row * SX + lane] = (rok && lane < IN) ? (T.xa[row] - sm0) * sp0 : 0.f;
             if (64 + lane < 16 * NT1C) xs[row * SX + 64 + lane] = (rok && 64 + lane < IN) ? (T.xb[row] - sm1) * sp1 : 0.f;
         }
+    RLT_TICK(4);
         float in0[4], in1[4], in2[4];
 #pragma unroll
         for (int v = 0; v < 4; v++) { in0[v] = T.in0[v]; in1[v] = T.in1[v]; in2[v] = T.in2[v]; }
         wave_sync();
-        // the next round's loads travel while this one is computed, with row indices requested a round earlier (the last rounds ask for the last tile again)
-        rows_next = rows_after;
-        rows_after = tile_rows(A, min((round + 2 * n_blocks) * WAVES + wave, n_tiles - 1), lane);
-        request_tile(A, rows_next, lane, T);
+        // the next round's loads travel while this one is computed, with row indices requested a round earlier
+        if (round + n_blocks < n_rounds) {
+            rows_next = rows_after;
+            if (round + 2 * n_blocks < n_rounds) rows_after = rows_of(round + 2 * n_blocks);
+            request_tile(A, rows_next, lane, T);
+        }
 
-        // layer 1: groups of four reduction steps, the operands of the next group requested before this group's matrix instructions
+    RLT_TICK(5);
+        // layer 1: groups of four reduction steps, the operands of the next group requested before this group's matrix instructions. Lane
+        // group kk supplies input column 32 (g / 2) + 4 (g % 2) + q + koff with koff = 0, 16, 8, 24: the two lane groups that the LDS serves
+        // together read columns 16 apart, that is different banks (rows are an odd number of floats apart)
         floatx4 acc[4] = {zero4, zero4, zero4, zero4};
         {
+            const int koff = 16 * (kk & 1) + 8 * (kk >> 1), n_groups = 2 * ((IN + 31) >> 5);
             float a_c[4], b_c[4][4];
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                a_c[q] = xs[r * SX + 4 * q + kk];
+                a_c[q] = xs[r * SX + koff + q];
 #pragma unroll
-                for (int nt = 0; nt < 4; nt++) b_c[q][nt] = w1s[(16 * nt + r) * SX + 4 * q + kk];
+                for (int nt = 0; nt < 4; nt++) b_c[q][nt] = w1s[(16 * nt + r) * SX + koff + q];
             }
-            for (int g = 0; g < NT1; g++) {
-                const int gn = min(g + 1, NT1 - 1);
+            for (int g = 0; g < n_groups; g++) {
+                const int gn = min(g + 1, n_groups - 1), kn = 32 * (gn >> 1) + 4 * (gn & 1) + koff;
                 float a_n[4], b_n[4][4];
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    a_n[q] = xs[r * SX + 16 * gn + 4 * q + kk];
+                    a_n[q] = xs[r * SX + kn + q];
 #pragma unroll
-                    for (int nt = 0; nt < 4; nt++) b_n[q][nt] = w1s[(16 * nt + r) * SX + 16 * gn + 4 * q + kk];
+                    for (int nt = 0; nt < 4; nt++) b_n[q][nt] = w1s[(16 * nt + r) * SX + kn + q];
                 }
 #pragma unroll
                 for (int q = 0; q < 4; q++)
@@ -220,6 +253,7 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
             for (int v = 0; v < 4; v++) h1s[(4 * kk + v) * HS + 16 * nt + r] = rlt_act(acc[nt][v] + b1r[nt], ACT_H);
         wave_sync();
 
+    RLT_TICK(6);
         // layer 2
         if (LAYERS == 3) {
 #pragma unroll
@@ -238,6 +272,7 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
         }
         const lptr hls = LAYERS == 3 ? h2s : h1s, hls_all = LAYERS == 3 ? h2s_all : h1s_all;      // the last hidden layer's activations
 
+    RLT_TICK(7);
         // layer 3 (two chains of matrix instructions) and the gradient at its pre-activations
         floatx4 y0 = zero4, y1 = zero4;
 #pragma unroll
@@ -274,19 +309,22 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
             s3 += dp;
             d3s[(4 * kk + v) * D3S + r] = dp;
         }
+    RLT_TICK(8);
         rlt_lds_barrier();      // every wavefront's last hidden activations and d_pre3 are in place
 
-        // dW3 (columns 16 wave + r) += d_pre3^T h over the 64 rows, two chains
+        // dW3 (columns 16 wave + r) += d_pre3^T h over the 64 rows, two chains; in the weight gradients' reductions lane group kk supplies rows
+        // 16 kk + ks (wavefront kk's tile), so that the lane groups served together read different LDS banks
         {
-            float a_c = d3s_all[kk * D3S + r], b_c = hls_all[kk * HS + 16 * wave + r];
+            float a_c = d3s_all[16 * kk * D3S + r], b_c = hls_all[16 * kk * HS + 16 * wave + r];
 #pragma unroll
             for (int ks = 0; ks < ROWS / 4; ks++) {
                 const int kn = min(ks + 1, ROWS / 4 - 1);
-                const float a_n = d3s_all[(4 * kn + kk) * D3S + r], b_n = hls_all[(4 * kn + kk) * HS + 16 * wave + r];
+                const float a_n = d3s_all[(16 * kk + kn) * D3S + r], b_n = hls_all[(16 * kk + kn) * HS + 16 * wave + r];
                 if (ks & 1) aW3b = mfma16(a_c, b_c, aW3b); else aW3a = mfma16(a_c, b_c, aW3a);
                 a_c = a_n; b_c = b_n;
             }
         }
+    RLT_TICK(9);
         // d_pre2 = (d_pre3 W3) f'(h2) for the wavefront's own rows, into g2
 #pragma unroll
         for (int nt = 0; nt < 4; nt++) acc[nt] = zero4;
@@ -305,20 +343,21 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
                 if (LAYERS == 3) { g2s[idx] = dp; s2[nt] += dp; }
                 else { h2s[idx] = dp; s1[nt] += dp; }       // two layers: this is already the gradient at layer 1's pre-activations, kept where dW1 reads it
             }
+    RLT_TICK(10);
         rlt_lds_barrier();      // every wavefront's d_pre2 is in place, and nobody reads h2 any more
         if (LAYERS == 3) {
 
         // dW2 (rows 16 wave + ..) += d_pre2^T h1 over the 64 rows
         {
-            float a_c = g2s_all[kk * HS + 16 * wave + r], b_c[4];
+            float a_c = g2s_all[16 * kk * HS + 16 * wave + r], b_c[4];
 #pragma unroll
-            for (int nt = 0; nt < 4; nt++) b_c[nt] = h1s_all[kk * HS + 16 * nt + r];
+            for (int nt = 0; nt < 4; nt++) b_c[nt] = h1s_all[16 * kk * HS + 16 * nt + r];
 #pragma unroll
             for (int ks = 0; ks < ROWS / 4; ks++) {
                 const int kn = min(ks + 1, ROWS / 4 - 1);
-                float a_n = g2s_all[(4 * kn + kk) * HS + 16 * wave + r], b_n[4];
+                float a_n = g2s_all[(16 * kk + kn) * HS + 16 * wave + r], b_n[4];
 #pragma unroll
-                for (int nt = 0; nt < 4; nt++) b_n[nt] = h1s_all[(4 * kn + kk) * HS + 16 * nt + r];
+                for (int nt = 0; nt < 4; nt++) b_n[nt] = h1s_all[(16 * kk + kn) * HS + 16 * nt + r];
 #pragma unroll
                 for (int nt = 0; nt < 4; nt++) aW2[nt] = mfma16(a_c, b_c[nt], aW2[nt]);
                 a_c = a_n;
@@ -326,6 +365,7 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
                 for (int nt = 0; nt < 4; nt++) b_c[nt] = b_n[nt];
             }
         }
+    RLT_TICK(11);
         // d_pre1 = (d_pre2 W2) f'(h1) for the wavefront's own rows, into the place of h2
 #pragma unroll
         for (int nt = 0; nt < 4; nt++) acc[nt] = zero4;
@@ -343,6 +383,7 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
                 const float dp = acc[nt][v] * rlt_dact_from_output(h1s[idx], ACT_H);
                 h2s[idx] = dp; s1[nt] += dp;
             }
+    RLT_TICK(12);
         rlt_lds_barrier();      // every wavefront's d_pre1 is in place
         }
 
@@ -358,17 +399,18 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
             }
         }
 
+    RLT_TICK(13);
         // dW1 (rows 16 wave + ..) += d_pre1^T x over the 64 rows
         {
-            float a_c = h2s_all[kk * HS + 16 * wave + r], b_c[NT1C];
+            float a_c = h2s_all[16 * kk * HS + 16 * wave + r], b_c[NT1C];
 #pragma unroll
-            for (int nt = 0; nt < NT1C; nt++) b_c[nt] = xs_all[kk * SX + 16 * nt + r];
+            for (int nt = 0; nt < NT1C; nt++) b_c[nt] = xs_all[16 * kk * SX + 16 * nt + r];
 #pragma unroll 4
             for (int ks = 0; ks < ROWS / 4; ks++) {
                 const int kn = min(ks + 1, ROWS / 4 - 1);
-                float a_n = h2s_all[(4 * kn + kk) * HS + 16 * wave + r], b_n[NT1C];
+                float a_n = h2s_all[(16 * kk + kn) * HS + 16 * wave + r], b_n[NT1C];
 #pragma unroll
-                for (int nt = 0; nt < NT1C; nt++) b_n[nt] = xs_all[(4 * kn + kk) * SX + 16 * nt + r];
+                for (int nt = 0; nt < NT1C; nt++) b_n[nt] = xs_all[(16 * kk + kn) * SX + 16 * nt + r];
 #pragma unroll
                 for (int nt = 0; nt < NT1C; nt++) aW1[nt] = mfma16(a_c, b_c[nt], aW1[nt]);
                 a_c = a_n;
@@ -376,9 +418,11 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
                 for (int nt = 0; nt < NT1C; nt++) b_c[nt] = b_n[nt];
             }
         }
+    RLT_TICK(14);
         rlt_lds_barrier();      // the round's tiles may be overwritten
     }
 
+    RLT_TICK(15);
     // the workgroup's block of partial sums: weight gradients straight from the registers that own them, ...
     float* dst = A.partial + (size_t)block * A.count;
     const int o_b1 = H * IN, o_w2 = o_b1 + H, o_b2 = o_w2 + H * H, o_w3 = o_b2 + H, o_b3 = o_w3 + OUT * H, o_ex = o_b3 + OUT;
@@ -392,6 +436,7 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
         for (int nt = 0; nt < 4; nt++) dst[o_w2 + m * H + 16 * nt + r] = aW2[nt][v];
         if (4 * kk + v < OUT) dst[o_w3 + (4 * kk + v) * H + 16 * wave + r] = aW3a[v] + aW3b[v];
     }
+    RLT_TICK(16);
     // ... the bias and log_std gradients, which every wavefront holds for its own rows, summed in wavefront order through LDS
     const lptr sums = (lptr)lds_raw;        // [WAVES][N_SUMS]; the weights are no longer needed
 #pragma unroll
@@ -411,6 +456,15 @@ __global__ __launch_bounds__(THREADS) void mlp3s_kernel(SmallArgs A0, SmallArgs 
         else if (i < 2 * H + MAX_OUT) { if (i - 2 * H < OUT) dst[o_b3 + i - 2 * H] = total; }
         else dst[o_ex + i - 2 * H - MAX_OUT] = total;
     }
+    RLT_TICK(17);
+    if (K.xr.enabled)       // the block joins those of the workgroups on this XCD: eight blocks of sums per network leave the launch
+        rlt_xcd_group_reduce<THREADS>(K.xr, xgroup, block >> 3, n_blocks >> 3, xepoch, A.partial + (size_t)(block & 7) * A.count, A.count,
+                                      (second ? K.xsum[1] : K.xsum[0]) + (size_t)(block & 7) * A.count, (__attribute__((address_space(3))) int*)((lptr)lds_raw + 4 * N_SUMS));
+    RLT_TICK(18);
+#ifdef RLT_SMALL_PROFILE
+    __builtin_amdgcn_s_waitcnt(0);
+    if (threadIdx.x == 0) rlt_small_spans[blockIdx.x][1] = wall_clock64();
+#endif
 }
 
 // where the elements of a block of partial sums go; overwrite: gradient = sum instead of gradient += sum (for a caller that would zero the gradient first)
@@ -464,8 +518,46 @@ bool shape_ok(const rlt_dense_layer* L, int n) {
 }
 int tile_bucket(int in) { return in <= 32 ? 2 : in <= 64 ? 4 : MAX_NT1; }
 
-// one or two networks in one launch; two only if they share the hidden activation and the input-width bucket
-int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
+// Where each tensor of an optimiser lies in the job's block of partial sums [dW1 | db1 | dW2 | db2 | dW3 | db3 | extra]: a tensor may span
+// several of the six gradient buffers where those follow each other in memory; the job's extra values (a gradient with its own scale
+// and offset) must be a tensor of their own. False unless the tensors cover all of these exactly once: then the optimiser's launch
+// can add the blocks up itself.
+bool map_step(const SmallJob& job, const rlt_mlp3s_step& S, bool extra_is_gradient, uint32_t* offsets, float* scales, float* adds) {
+    if (!S.tensors || S.n < 1 || S.n > 12 || job.n_layers != 3) return false;
+    const rlt_dense_layer* L = job.L;
+    const float* seg[6] = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases};
+    const uint32_t size[6] = {(uint32_t)(H * L[0].in_dim), H, H * H, H, (uint32_t)(L[2].out_dim * H), (uint32_t)L[2].out_dim};
+    uint32_t off[6], covered = 0;
+    for (int k = 0, o = 0; k < 6; o += size[k], k++) off[k] = o;
+    bool extra_covered = false;
+    for (int i = 0; i < S.n; i++) {
+        const rlt_adam_tensor& T = S.tensors[i];
+        if (T.polyak_target) return false;
+        if (extra_is_gradient && job.extra && T.gradient == job.extra) {
+            if (extra_covered || T.count != (uint32_t)job.n_extra) return false;
+            extra_covered = true;
+            offsets[i] = (uint32_t)(job.a.count - N_EXTRA); scales[i] = job.extra_scale; adds[i] = job.extra_offset;
+            continue;
+        }
+        int s = 0;
+        while (s < 6 && seg[s] != T.gradient) s++;
+        if (s == 6) return false;
+        uint32_t cnt = 0;
+        for (int k = s; k < 6 && cnt < T.count && seg[k] == seg[s] + cnt; k++) {
+            if (covered & (1u << k)) return false;
+            covered |= 1u << k; cnt += size[k];
+        }
+        if (cnt != T.count) return false;
+        offsets[i] = off[s]; scales[i] = 1.0f; adds[i] = 0.0f;
+    }
+    return covered == 63u && extra_covered == (extra_is_gradient && job.extra != nullptr);
+}
+
+// one or two networks in one launch; two only if they share the hidden activation and the input-width bucket. `steps` (optional, one per
+// job): the optimisers' steps follow in one launch that reads the blocks of partial sums itself (a gradient's extra values only for job 0;
+// job 1's single extra value is an output); *stepped tells whether they did, else the gradients were formed and the caller steps.
+int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs, const rlt_mlp3s_step* steps = nullptr, bool* stepped = nullptr) {
+    if (stepped) *stepped = false;
     int groups[2] = {0, 0};
     size_t offset[2] = {0, 0}, total = 0;
     for (int j = 0; j < n_jobs; j++) {
@@ -484,22 +576,41 @@ int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
     if (n_jobs == 2 && (tile_bucket(jobs[1].a.in) != bucket || jobs[1].L[0].activation != act)) return RLT_E_UNSUPPORTED;
     const size_t lds_bytes = lds_floats(bucket) * sizeof(float);
     if (lds_bytes > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
+    // the optimisers' steps follow in one launch that adds the blocks of partial sums up itself, where the tensors allow
+    uint32_t offsets[2][12]; float scales[2][12], adds[2][12];
+    const bool steps_mapped = steps && n_jobs == 2 && jobs[0].overwrite && jobs[1].overwrite && (!jobs[1].extra || jobs[1].n_extra == 1) &&
+                              map_step(jobs[0], steps[0], true, offsets[0], scales[0], adds[0]) && map_step(jobs[1], steps[1], false, offsets[1], scales[1], adds[1]);
+    SmallLaunch K = {};
+    // sums per XCD inside the launch: where workgroup i runs on XCD i % 8, every network's workgroups are a multiple of 8 (at most 32 per XCD)
+    // and the grid is resident as a whole
+    bool xcd_sums = device->update_tail && device->xcd_stride == 8 && groups[0] + groups[n_jobs - 1] * (n_jobs - 1) <= device->compute_units;
+    size_t xsum_offset[2] = {0, 0};
+    for (int j = 0; j < n_jobs; j++) {
+        xcd_sums = xcd_sums && groups[j] % RLT_XCD_GROUPS == 0 && groups[j] >= 2 * RLT_XCD_GROUPS && groups[j] <= RLT_XCD_GROUPS * RLT_XCD_MAX_MEMBERS;
+        xsum_offset[j] = total; total += ((size_t)RLT_XCD_GROUPS * jobs[j].a.count + 63) & ~(size_t)63;
+    }
     void* scratch = nullptr;
     int rc = rlt_scratch(device, total * sizeof(float), &scratch);
     if (rc) return rc;
     for (int j = 0; j < n_jobs; j++) jobs[j].a.partial = (float*)scratch + offset[j];
-    const SmallArgs& a0 = jobs[0].a; const SmallArgs& a1 = jobs[n_jobs - 1].a;
+    if (xcd_sums) {
+        void* counters = nullptr;
+        if ((rc = rlt_counters(device, &counters))) return rc;
+        K.xr.enabled = 1; K.xr.max_poll = device->wait_limit; K.xr.words = (uint32_t*)counters + RLT_XCD_WORDS_OFFSET; K.xr.fault = device->fault;
+        for (int j = 0; j < n_jobs; j++) K.xsum[j] = (float*)scratch + xsum_offset[j];
+        device->fault_armed = 1;
+    }
+    K.a0 = jobs[0].a; K.a1 = jobs[n_jobs - 1].a; K.groups0 = groups[0];
     const int grid = groups[0] + (n_jobs == 2 ? groups[1] : 0);
     const bool two_layers = jobs[0].n_layers == 2;
+#define RLT_LAUNCH_SMALL_AS(ACT, NT, LAYERS)                                                                                                                    \
+    do {                                                                                                                                                        \
+        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp3s_kernel<ACT, NT, LAYERS>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
+        hipLaunchKernelGGL((mlp3s_kernel<ACT, NT, LAYERS>), dim3(grid), dim3(THREADS), lds_bytes, device->stream, K);                                         \
+    } while (0)
 #define RLT_LAUNCH_SMALL(ACT, NT)                                                                                                                               \
     do {                                                                                                                                                        \
-        if (two_layers) {                                                                                                                                       \
-            RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp3s_kernel<ACT, NT, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
-            hipLaunchKernelGGL((mlp3s_kernel<ACT, NT, 2>), dim3(grid), dim3(THREADS), lds_bytes, device->stream, a0, a1, groups[0]);                           \
-        } else {                                                                                                                                                \
-            RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp3s_kernel<ACT, NT, 3>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
-            hipLaunchKernelGGL((mlp3s_kernel<ACT, NT, 3>), dim3(grid), dim3(THREADS), lds_bytes, device->stream, a0, a1, groups[0]);                           \
-        }                                                                                                                                                       \
+        if (two_layers) RLT_LAUNCH_SMALL_AS(ACT, NT, 2); else RLT_LAUNCH_SMALL_AS(ACT, NT, 3);                                                                  \
     } while (0)
     switch (act) {
         case RLT_ACT_RELU: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_RELU, 2); else if (bucket == 4) RLT_LAUNCH_SMALL(RLT_ACT_RELU, 4); else RLT_LAUNCH_SMALL(RLT_ACT_RELU, MAX_NT1); break;
@@ -507,7 +618,17 @@ int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
         default: if (bucket == 2) RLT_LAUNCH_SMALL(RLT_ACT_FAST_TANH, 2); else if (bucket == 4) RLT_LAUNCH_SMALL(RLT_ACT_FAST_TANH, 4); else RLT_LAUNCH_SMALL(RLT_ACT_FAST_TANH, MAX_NT1); break;
     }
 #undef RLT_LAUNCH_SMALL
+#undef RLT_LAUNCH_SMALL_AS
     if ((rc = rlt_launch_status(device))) return rc;
+    const float* sums[2]; int n_sums[2];      // what is left to add up: the workgroups' blocks, or one block per XCD
+    for (int j = 0; j < n_jobs; j++) { sums[j] = xcd_sums ? K.xsum[j] : jobs[j].a.partial; n_sums[j] = xcd_sums ? RLT_XCD_GROUPS : groups[j]; }
+    if (steps_mapped) {
+        rlt_adam_source src[2] = {};
+        for (int j = 0; j < 2; j++) { src[j].partial = sums[j]; src[j].groups = n_sums[j]; src[j].block_stride = jobs[j].a.count; src[j].offsets = offsets[j]; src[j].scales = scales[j]; src[j].adds = adds[j]; }
+        if (jobs[1].extra) { src[1].extra_out = jobs[1].extra; src[1].extra_offset = (uint32_t)(jobs[1].a.count - N_EXTRA); src[1].extra_scale = jobs[1].extra_scale; }
+        if (stepped) *stepped = true;
+        return rlt_adam_step_pair(device, steps[0].tensors, steps[0].n, steps[0].parameters, steps[0].age, steps[1].tensors, steps[1].n, steps[1].parameters, steps[1].age, &src[0], &src[1]);
+    }
     SmallTargets T[2] = {};
     int blocks = 0;
     for (int j = 0; j < n_jobs; j++) {
@@ -515,7 +636,7 @@ int launch(rlt_rocm_device* device, SmallJob* jobs, int n_jobs) {
         const int count = jobs[j].extra ? a.count : a.count - N_EXTRA;      // the extra slots sit at the end of a block
         const int last = jobs[j].n_layers - 1;
         T[j] = {L[0].d_weights, L[0].d_biases, last == 2 ? L[1].d_weights : nullptr, last == 2 ? L[1].d_biases : nullptr, L[last].d_weights, L[last].d_biases, jobs[j].extra, a.in, a.out, jobs[j].n_extra,
-                jobs[j].extra_scale, jobs[j].extra_offset, jobs[j].overwrite, a.partial, groups[j], a.count, (count + 63) / 64};
+                jobs[j].extra_scale, jobs[j].extra_offset, jobs[j].overwrite, sums[j], n_sums[j], a.count, (count + 63) / 64};
         blocks += T[j].blocks;
     }
     if (n_jobs == 1) T[1] = T[0];
@@ -585,7 +706,8 @@ int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* a
                                const float* stats, const rlt_ppo_parameters* P, float* d_log_std, float log_std_gradient_offset,
                                const rlt_dense_layer* critic, int n_critic, const float* x_critic, float* values, int ld_values,
                                const float* target_values, float mse_scale, float* out_critic_loss, int ld, const uint32_t* rows, int batch,
-                               const float* actor_std_mean, const float* actor_std_precision, const float* critic_std_mean, const float* critic_std_precision) {
+                               const float* actor_std_mean, const float* actor_std_precision, const float* critic_std_mean, const float* critic_std_precision,
+                               const rlt_mlp3s_step* steps, bool* stepped) {
     if (!rlt_mlp3s_pair_supported(actor, n_actor, critic, n_critic) || (out_critic_loss && critic[2].out_dim != 1)) return RLT_E_UNSUPPORTED;
     SmallJob jobs[2] = {ppo_actor_job(actor, x, ld, means, ld_means, log_std, actions, ld, log_probs, ld, advantages, ld, stats, P, d_log_std,
                                       log_std_gradient_offset, batch, 1, rows),
@@ -593,5 +715,10 @@ int rlt_mlp3s_ppo_actor_critic(rlt_rocm_device* device, const rlt_dense_layer* a
     if (out_critic_loss) { jobs[1].extra = out_critic_loss; jobs[1].n_extra = 1; jobs[1].extra_scale = 1.0f / (float)batch; jobs[1].extra_offset = 0.0f; }
     jobs[0].a.std_mean = actor_std_mean; jobs[0].a.std_precision = actor_std_mean ? actor_std_precision : nullptr;
     jobs[1].a.std_mean = critic_std_mean; jobs[1].a.std_precision = critic_std_mean ? critic_std_precision : nullptr;
-    return launch(device, jobs, 2);
+    return launch(device, jobs, 2, steps, stepped);
 }
+
+#ifdef RLT_SMALL_PROFILE
+extern "C" int rlt_mlp3s_spans(unsigned long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(rlt_small_spans), sizeof(unsigned long long) * 1024); }
+extern "C" int rlt_mlp3s_ticks(unsigned long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(rlt_small_ticks), sizeof(unsigned long long) * 32); }
+#endif

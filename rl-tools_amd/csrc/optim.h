@@ -5,8 +5,9 @@
 
 // Gradients that are still blocks of partial sums (one block of `block_stride` floats per workgroup of the kernel that made them): the
 // optimiser's launch adds them up, in the order of the small-MLP reduction kernel, stores the sums in the tensors' gradients and steps.
-// offsets[t]: where tensor t's gradient starts within a block; scales[t]: factor on its sums.
-struct rlt_adam_source { const float* partial; int groups, block_stride; const uint32_t* offsets; const float* scales; };
+// offsets[t]: where tensor t's gradient starts within a block; scales[t]: factor on its sums; adds[t] (optional array): added after scaling.
+// extra_out (optional): one more sum of the blocks, at extra_offset, times extra_scale, stored there (a loss that the kernel summed per block).
+struct rlt_adam_source { const float* partial; int groups, block_stride; const uint32_t* offsets; const float* scales; const float* adds; float* extra_out; uint32_t extra_offset; float extra_scale; };
 
 // rlt_rocm_adam_step for at most 12 tensors whose gradients are blocks of partial sums
 int rlt_adam_step_from_partials(rlt_rocm_device* device, const rlt_adam_tensor* tensors, int n, const rlt_adam_parameters* parameters, uint32_t* age, const rlt_adam_source* source,
@@ -29,6 +30,13 @@ __device__ __forceinline__ float rlt_polyak_value(float polyak, float target, fl
 #pragma clang fp contract(off)
     const float a = polyak * target, b = (1.0f - polyak) * source;
     return a + b;
+}
+
+// a gradient from its summed partial values: the product is rounded before the sum in every kernel, so that all of them leave the same bits
+__device__ __forceinline__ float rlt_scaled_sum(float sum, float scale, float add) {
+#pragma clang fp contract(off)
+    const float a = sum * scale;
+    return a + add;
 }
 
 // 1 / (1 - beta^age) for both moments (nn/optimizers/adam/operations_generic.h:49-58: from the age before the step)

@@ -28,7 +28,8 @@ struct AdamLaunch {
     const float* source;
     int groups, block_stride;
     uint32_t source_offset[MAX_T];
-    float source_scale[MAX_T];
+    float source_scale[MAX_T], source_add[MAX_T];
+    float* extra_out; uint32_t extra_offset; float extra_scale;      // optional: one more sum of the blocks, stored scaled (not a gradient)
 };
 
 // sum over the blocks of one element, every load in flight at once where there are at most 16 blocks
@@ -47,6 +48,52 @@ __device__ __forceinline__ void adam_body(const AdamLaunch& a, uint32_t block, u
     rlt_adam_bias_corrections(a.p, age, bc1, bc2);
     const uint32_t total = a.prefix[a.n];
     float sq = 0.0f;
+    if (a.source && a.groups > 16) {
+        // many blocks: 64 elements per pass of a workgroup, four threads per element each add up a quarter of the blocks (the order of
+        // rlt_sum_of_blocks) with all of a quarter's loads of up to 32 blocks in flight at once
+        __shared__ float quarter[4][64];
+        const uint32_t el = threadIdx.x & 63u, qtr = threadIdx.x >> 6;
+        const int per = (a.groups + 3) / 4, g0 = qtr * per, g1 = min(a.groups, g0 + per);
+        for (uint32_t base = block * 64u; base < total; base += n_blocks * 64u) {
+            const uint32_t i = min(base + el, total - 1u);
+            int ti = 0;
+#pragma unroll
+            for (int k = 1; k < MAX_T; k++) ti += (k < a.n && i >= a.prefix[k]) ? 1 : 0;
+            const uint32_t j = i - a.prefix[ti];
+            const float* __restrict__ p = a.source + a.source_offset[ti] + j;
+            // the element's moments and value travel while the blocks are added up
+            const rlt_adam_tensor& T = a.t[ti];
+            float m = 0.f, v2 = 0.f, param = 0.f, target = 0.f;
+            if (qtr == 0) { m = T.first_moment[j]; v2 = T.second_moment[j]; param = T.parameters[j]; if (T.polyak_target) target = T.polyak_target[j]; }
+            float s = 0.f;
+            int gb = g0;
+            for (; g1 - gb > 8; gb += 32) {
+                float v[32];
+#pragma unroll
+                for (int u = 0; u < 32; u++) v[u] = p[(size_t)min(gb + u, g1 - 1) * a.block_stride];
+#pragma unroll
+                for (int u = 0; u < 32; u++) s += (gb + u < g1) ? v[u] : 0.f;
+            }
+            for (; gb < g1; gb += 8) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = p[(size_t)min(gb + u, g1 - 1) * a.block_stride];
+#pragma unroll
+                for (int u = 0; u < 8; u++) s += (gb + u < g1) ? v[u] : 0.f;
+            }
+            quarter[qtr][el] = s;
+            __syncthreads();
+            if (qtr == 0 && base + el < total) {
+                const float g = rlt_scaled_sum((quarter[0][el] + quarter[1][el]) + (quarter[2][el] + quarter[3][el]), a.source_scale[ti], a.source_add[ti]);
+                T.gradient[j] = g;
+                sq += g * g;
+                rlt_adam_values(a.p, T.flags, g, bc1, bc2, m, v2, param);
+                T.first_moment[j] = m; T.second_moment[j] = v2; T.parameters[j] = param;
+                if (T.polyak_target) T.polyak_target[j] = rlt_polyak_value(a.polyak, target, param);
+            }
+            __syncthreads();
+        }
+    } else
     for (uint32_t i = block * blockDim.x + threadIdx.x; i < total; i += n_blocks * blockDim.x) {
         int ti = 0;
 #pragma unroll
@@ -55,12 +102,13 @@ __device__ __forceinline__ void adam_body(const AdamLaunch& a, uint32_t block, u
         const uint32_t j = i - a.prefix[ti];
         float g;
         if (a.source) {
-            g = sum_of_blocks(a.source + a.source_offset[ti] + j, a.groups, a.block_stride) * a.source_scale[ti];
+            g = rlt_scaled_sum(sum_of_blocks(a.source + a.source_offset[ti] + j, a.groups, a.block_stride), a.source_scale[ti], a.source_add[ti]);
             T.gradient[j] = g;
         } else g = T.gradient[j];
         sq += g * g;
         rlt_adam_apply(a.p, T, j, g, bc1, bc2, a.polyak);
     }
+    if (a.extra_out && block == n_blocks - 1 && threadIdx.x == blockDim.x - 1) *a.extra_out = sum_of_blocks(a.source + a.extra_offset, a.groups, a.block_stride) * a.extra_scale;
     // gradient norm + age increment: the last workgroup to finish has seen every other one read `age`
     __shared__ float partial[4];
     __shared__ bool last;
@@ -146,7 +194,8 @@ static int adam_launch(rlt_rocm_device* device, const rlt_adam_tensor* tensors, 
 static void set_source(AdamLaunch& a, const rlt_adam_source* source) {
     if (!source) return;
     a.source = source->partial; a.groups = source->groups; a.block_stride = source->block_stride;
-    for (int i = 0; i < a.n; i++) { a.source_offset[i] = source->offsets[i]; a.source_scale[i] = source->scales[i]; }
+    for (int i = 0; i < a.n; i++) { a.source_offset[i] = source->offsets[i]; a.source_scale[i] = source->scales[i]; a.source_add[i] = source->adds ? source->adds[i] : 0.0f; }
+    a.extra_out = source->extra_out; a.extra_offset = source->extra_offset; a.extra_scale = source->extra_scale;
 }
 
 int rlt_adam_step_from_partials(rlt_rocm_device* device, const rlt_adam_tensor* tensors, int n, const rlt_adam_parameters* parameters, uint32_t* age, const rlt_adam_source* source, float polyak) {
@@ -167,7 +216,8 @@ int rlt_adam_step_from_partials(rlt_rocm_device* device, const rlt_adam_tensor* 
     a.done_counter = (uint32_t*)counters; a.block_partials = (float*)((char*)counters + 256);
     a.increment_age = 1;
     set_source(a, source);
-    int blocks = (int)((total + 255) / 256); if (blocks > 960) blocks = 960;
+    const uint32_t per_block = source->groups > 16 ? 64 : 256;      // the many-block path takes 64 elements per workgroup pass
+    int blocks = (int)((total + per_block - 1) / per_block); if (blocks > 960) blocks = 960;
     hipLaunchKernelGGL(adam_kernel, dim3(blocks), dim3(256), 0, device->stream, a);
     return rlt_launch_status(device);
 }
@@ -202,8 +252,10 @@ int rlt_adam_step_pair(rlt_rocm_device* device, const rlt_adam_tensor* tensors_a
         // the second optimiser's ticket counter and partial sums sit in their own part of the counters block
         a.done_counter = (uint32_t*)((char*)counters + (k ? 64 : 0)); a.block_partials = (float*)((char*)counters + 256) + (k ? 480 : 0);
         a.increment_age = 1;
-        set_source(a, k ? source_b : source_a);
-        blocks[k] = (total + 255) / 256; if (blocks[k] > 480) blocks[k] = 480; if (blocks[k] < 1) blocks[k] = 1;
+        const rlt_adam_source* source = k ? source_b : source_a;
+        set_source(a, source);
+        const uint32_t per_block = source && source->groups > 16 ? 64 : 256;
+        blocks[k] = (total + per_block - 1) / per_block; if (blocks[k] > 480) blocks[k] = 480; if (blocks[k] < 1) blocks[k] = 1;
     }
     hipLaunchKernelGGL(adam_pair_kernel, dim3(blocks[0] + blocks[1]), dim3(256), 0, device->stream, L[0], L[1], blocks[0]);
     return rlt_launch_status(device);

@@ -352,12 +352,16 @@ static int ppo_pair_update(rlt_rocm_device* device, const rlt_ppo_agent* A, cons
         if (pad_a) { if ((rc = rlt_pad_parameters(device, A->actor, (float*)memory, true, &padded_actor))) return rc; actor = padded_actor.L; }
         if (pad_c) { if ((rc = rlt_pad_parameters(device, A->critic, (float*)memory + floats_a, true, &padded_critic))) return rc; critic = padded_critic.L; }
     }
+    // the optimisers' launch adds up the kernel's partial sums itself where it can (:305-306); not for padded copies, whose gradients are copied back first
+    const rlt_mlp3s_step steps[2] = {{A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age}, {A->critic_adam_tensors, A->n_critic_adam_tensors, &A->critic_adam, A->critic_age}};
+    const bool fuse_steps = !pad_a && !pad_c && (P->learn_action_std || !A->d_log_std);
+    bool stepped = false;
     rc = rlt_mlp3s_ppo_actor_critic(device, actor, A->n_actor_layers, observations, A->actor[A->n_actor_layers - 1].output, AD, A->log_std, actions,
                                     action_log_probs, advantages, stats, P, P->learn_action_std ? A->d_log_std : nullptr, -P->action_entropy_coefficient,
                                     critic, A->n_critic_layers, observations_privileged, values, 1, target_values, 1.0f / (float)B, out_critic_loss,   // :303
                                     ld, row_indices, B, A->actor_standardize_mean, A->actor_standardize_precision, A->critic_standardize_mean,
-                                    A->critic_standardize_precision);
-    if (rc) return rc;
+                                    A->critic_standardize_precision, fuse_steps ? steps : nullptr, &stepped);
+    if (rc || stepped) return rc;
     if (pad_a) if ((rc = rlt_unpad_gradients(device, A->actor, &padded_actor))) return rc;
     if (pad_c) if ((rc = rlt_unpad_gradients(device, A->critic, &padded_critic))) return rc;
     if (A->d_log_std && !P->learn_action_std) if ((rc = rlt_rocm_fill_f32(device, A->d_log_std, 1, AD, AD, 0.0f))) return rc;

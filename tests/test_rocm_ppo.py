@@ -95,6 +95,36 @@ def test_train_minibatch_matches_checker_on_synthetic_dataset(oracle, rocm, B, N
     assert rel_err(p1, p0) <= 2e-4 and rel_err(l1, l0) <= 1e-4
 
 
+def test_sums_per_xcd_and_sums_by_the_optimiser_agree(rocm):
+    """At 8,192 rows the minibatch kernel's 256 workgroups add their partial gradient sums up per XCD inside the launch (eight blocks per network
+    are left for the optimiser's launch); with that switched off (rlt_rocm_set_update_options) the optimiser's launch adds up all 128 blocks per
+    network. The two orders of summation differ in the last bits only."""
+    capi = helpers.capi
+    O, A, H, B = 105, 8, 64, 8192
+    rng = np.random.default_rng(6)
+    params = np.concatenate([helpers.random_params(rng, [O, H, H, A]), np.log(np.full(A, 0.5, np.float32)), helpers.random_params(rng, [O, H, H, 1])])
+    ld = O + A + 3
+    data = rng.standard_normal((B, ld)).astype(np.float32)
+    data[:, O + A] = -A * 1.5 + 0.3 * rng.standard_normal(B).astype(np.float32)
+    pp = capi.ppo_parameters()
+    results = []
+    for in_kernel in (1, 0):
+        rocm.call("set_update_options", in_kernel, 1)
+        try:
+            agent = helpers.PpoOnBackend(rocm, O, A, H, H, B, params, "tanh", "tanh", capi.adam_parameters(3e-4, epsilon=1e-8))
+            dd, loss = rocm.array(data), rocm.zeros((1,))
+            for _ in range(3):
+                rocm.call("ppo_train_minibatch", C.byref(agent.c), C.byref(pp), dd.offset(0), dd.offset(0), dd.offset(O), dd.offset(O + A), dd.offset(O + A + 1),
+                          dd.offset(O + A + 2), ld, None, loss.ptr)
+            rocm.sync()
+            results.append((agent.actor.grads.numpy(), agent.critic.grads.numpy(), agent.d_log_std.numpy(), agent.parameters(), loss.numpy()))
+        finally:
+            rocm.call("set_update_options", 1, 1)
+    for a, b in zip(*results):
+        assert rel_err(a, b) <= 2e-5, rel_err(a, b)
+    assert int(agent.actor.age.numpy()[0]) == 4 and int(agent.critic.age.numpy()[0]) == 4
+
+
 @pytest.mark.parametrize("O,A,H,B,act", [(105, 8, 64, 512, "tanh"), (3, 1, 64, 200, "tanh"), (17, 6, 256, 300, "tanh"), (3, 1, 32, 256, "fast_tanh"), (11, 2, 16, 128, "tanh"),
                                          (5, 3, 48, 96, "relu")])
 def test_train_minibatch_with_standardize_layers_matches_checker(oracle, rocm, O, A, H, B, act):

@@ -62,3 +62,37 @@ def test_persistent_loop_gives_up_and_reports(oracle):
     finally:
         impatient.close()
         oracle.lib.rlt_oracle_sac_loop_destroy(loop)
+
+
+def test_update_kernel_that_sums_per_xcd_gives_up_and_reports():
+    """PPO's minibatch kernel at 8,192 rows (rl/algorithms/ppo/operations_generic.h:163-309): its 256 workgroups add their blocks of partial gradient sums up
+    per XCD inside the launch, which makes the 16 workgroups of a network on one XCD wait for each other."""
+    O, A, H, B = 105, 8, 64, 8192
+    rng = np.random.default_rng(4)
+    params = np.concatenate([helpers.random_params(rng, [O, H, H, A]), np.log(np.full(A, 0.5, np.float32)), helpers.random_params(rng, [O, H, H, 1])])
+    ld = O + A + 3
+    data = rng.standard_normal((B, ld)).astype(np.float32)
+    pp = capi.ppo_parameters()
+
+    def one_update(backend):
+        agent = helpers.PpoOnBackend(backend, O, A, H, H, B, params, "tanh", "tanh", capi.adam_parameters(3e-4, epsilon=1e-8))
+        dd = backend.array(data)
+        rc = backend.device.lib.rlt_rocm_ppo_train_minibatch(backend.device.handle, C.byref(agent.c), C.byref(pp), dd.offset(0), dd.offset(0), dd.offset(O), dd.offset(O + A),
+                                                             dd.offset(O + A + 1), dd.offset(O + A + 2), ld, None, None)
+        return rc, agent
+
+    impatient = helpers.RocmBackend()
+    try:
+        impatient.call("set_wait_limit", 1)
+        rc, _ = one_update(impatient)
+        assert rc == 0
+        assert impatient.device.lib.rlt_rocm_check_status(impatient.device.handle) == capi.RLT_E_DEVICE_TIMEOUT
+    finally:
+        impatient.close()
+    patient = helpers.RocmBackend()
+    try:
+        rc, agent = one_update(patient)
+        assert rc == 0 and patient.device.lib.rlt_rocm_check_status(patient.device.handle) == 0
+        assert np.abs(agent.parameters() - params).max() > 1e-5 and int(agent.actor.age.numpy()[0]) == 2
+    finally:
+        patient.close()
