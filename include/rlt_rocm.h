@@ -608,8 +608,10 @@ int rlt_rocm_sac_pendulum_loop(rlt_rocm_device* device, const rlt_sac_agent* age
  *   RLT_ENV_PENDULUM          state 2, observation 3, action 1   (parameters: pendulum)
  *   RLT_ENV_ACROBOT           state 4, observation 6, action 1   (parameters: acrobot)
  *   RLT_ENV_ACROBOT_SWINGUP   state 4, observation 6, action 1   (parameters: acrobot)
- *   RLT_ENV_CAR               state 6, observation 6, action 2   (parameters: car) */
-enum { RLT_ENV_PENDULUM = 0, RLT_ENV_ACROBOT = 1, RLT_ENV_ACROBOT_SWINGUP = 2, RLT_ENV_CAR = 3 };
+ *   RLT_ENV_CAR               state 6, observation 6, action 2   (parameters: car)
+ *   RLT_ENV_PENDULUM_POSITION state 3 (theta, theta_dot, last action), observation 2 (cos, sin), action 1   (parameters: pendulum): the Pendulum that hides its velocity,
+ *                             rl/environments/pendulum/pendulum.h:117-124 (the environment of the reference's recurrent configurations) */
+enum { RLT_ENV_PENDULUM = 0, RLT_ENV_ACROBOT = 1, RLT_ENV_ACROBOT_SWINGUP = 2, RLT_ENV_CAR = 3, RLT_ENV_PENDULUM_POSITION = 4 };
 typedef struct rlt_env_runner {
     int32_t env_kind, n_envs, episode_step_limit, reserved;
     float* states;              /* [n_envs x state_dim] */

@@ -1096,6 +1096,7 @@ static int env_dims_of(int kind, int* state, int* obs, int* act) {
         case RLT_ENV_PENDULUM: *state = 2; *obs = 3; *act = 1; return 0;
         case RLT_ENV_ACROBOT: case RLT_ENV_ACROBOT_SWINGUP: *state = 4; *obs = 6; *act = 1; return 0;
         case RLT_ENV_CAR: *state = 6; *obs = 6; *act = 2; return 0;
+        case RLT_ENV_PENDULUM_POSITION: *state = 3; *obs = 2; *act = 1; return 0;
         default: return RLT_E_INVALID_ARGUMENT;
     }
 }
@@ -1105,6 +1106,21 @@ static int env_step_of(const rlt_env_runner* rn, float* states, const float* act
         case RLT_ENV_PENDULUM: {
             if (terminated) for (int e = 0; e < N; e++) terminated[e] = 0;
             return rlt_oracle_pendulum_step(&rn->pendulum, states, actions, observations, next_observations, rewards, N);
+        }
+        case RLT_ENV_PENDULUM_POSITION: {
+            // rl/environments/pendulum/pendulum.h:117-124: the Pendulum's dynamics and reward (the step above on the first two state entries), the observation's
+            // first two entries (operations_generic.h:168-181 with zero observation noise), and the action remembered in the state (:102-108)
+            std::vector<float> s2((size_t)N * 2), o3((size_t)N * 3), n3((size_t)N * 3);
+            for (int e = 0; e < N; e++) { s2[2 * e] = states[3 * e]; s2[2 * e + 1] = states[3 * e + 1]; }
+            const int rc = rlt_oracle_pendulum_step(&rn->pendulum, s2.data(), actions, o3.data(), n3.data(), rewards, N);
+            if (rc) return rc;
+            for (int e = 0; e < N; e++) {
+                states[3 * e] = s2[2 * e]; states[3 * e + 1] = s2[2 * e + 1]; states[3 * e + 2] = actions[e];
+                if (observations) { observations[2 * e] = o3[3 * e]; observations[2 * e + 1] = o3[3 * e + 1]; }
+                if (next_observations) { next_observations[2 * e] = n3[3 * e]; next_observations[2 * e + 1] = n3[3 * e + 1]; }
+                if (terminated) terminated[e] = 0;
+            }
+            return 0;
         }
         case RLT_ENV_CAR: return rlt_oracle_car_step(&rn->car, states, actions, observations, next_observations, rewards, terminated, N);
         default: return rlt_oracle_acrobot_step(&rn->acrobot, rn->env_kind == RLT_ENV_ACROBOT_SWINGUP, states, actions, observations, next_observations, rewards, terminated, N);

@@ -118,8 +118,8 @@ class PendulumRunner(C.Structure):
 
 UNARY = dict(negate=0, abs=1, constant=2, sigmoid=3, fast_sigmoid=4, exp=5, tanh=6, fast_tanh=7, one_minus=8, scale=9, scale_reciprocal=10)
 BINARY = dict(add=0, subtract=1, multiply=2, divide=3)
-ENV_PENDULUM, ENV_ACROBOT, ENV_ACROBOT_SWINGUP, ENV_CAR = 0, 1, 2, 3
-ENV_DIMS = {ENV_PENDULUM: (2, 3, 1), ENV_ACROBOT: (4, 6, 1), ENV_ACROBOT_SWINGUP: (4, 6, 1), ENV_CAR: (6, 6, 2)}      # state, observation, action widths
+ENV_PENDULUM, ENV_ACROBOT, ENV_ACROBOT_SWINGUP, ENV_CAR, ENV_PENDULUM_POSITION = 0, 1, 2, 3, 4
+ENV_DIMS = {ENV_PENDULUM: (2, 3, 1), ENV_ACROBOT: (4, 6, 1), ENV_ACROBOT_SWINGUP: (4, 6, 1), ENV_CAR: (6, 6, 2), ENV_PENDULUM_POSITION: (3, 2, 1)}      # state, observation, action widths
 
 
 class EnvRunner(C.Structure):

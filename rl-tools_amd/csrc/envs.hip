@@ -4,10 +4,10 @@
 // fp32 throughout, which stays within 1e-5 relative of it per step. 4 Runge-Kutta stages of ~60 flop: the kernel is bound by its 52 bytes per
 // environment (state in and out, observations, reward, flag) once there are enough environments to fill the device.
 #include "common.h"
+#include "pendulum.h"
 
 namespace {
 struct Acrobot4 { float v[4]; };
-__device__ __forceinline__ float clampf(float x, float lo, float hi) { return fminf(fmaxf(x, lo), hi); }
 __device__ __forceinline__ float angle_normalize(float x) {
     const float PI = 3.14159265358979323846f;
     const float a = x + PI, b = 2.0f * PI;
@@ -189,8 +189,28 @@ __host__ __device__ inline EnvDims env_dims(int kind) {
         case RLT_ENV_PENDULUM: return {2, 3, 1};
         case RLT_ENV_ACROBOT: case RLT_ENV_ACROBOT_SWINGUP: return {4, 6, 1};
         case RLT_ENV_CAR: return {6, 6, 2};
+        case RLT_ENV_PENDULUM_POSITION: return {3, 2, 1};
         default: return {0, 0, 0};
     }
+}
+// The Pendulum whose observation is the position only and whose state also remembers the last action (rl/environments/pendulum/pendulum.h:117-124,
+// step operations_generic.h:102-108, observe :168-181): states [n x 3] = (theta, theta_dot, last_action), observations [n x 2] = (cos, sin)
+__global__ __launch_bounds__(256) void pendulum_position_step_kernel(rlt_pendulum_parameters p, float* __restrict__ states, const float* __restrict__ actions,
+                                                                     float* __restrict__ next_observations, float* __restrict__ rewards, uint8_t* __restrict__ terminated, int n) {
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
+        Transition t;
+        pendulum_transition(p, states[3 * (size_t)e], states[3 * (size_t)e + 1], actions[e], t);
+        if (next_observations) { next_observations[2 * (size_t)e] = t.next_obs[0]; next_observations[2 * (size_t)e + 1] = t.next_obs[1]; }
+        if (rewards) rewards[e] = t.reward;
+        if (terminated) terminated[e] = 0;      // the Pendulum has no terminal states
+        states[3 * (size_t)e] = t.theta; states[3 * (size_t)e + 1] = t.theta_dot; states[3 * (size_t)e + 2] = actions[e];
+    }
+}
+int pendulum_position_step(rlt_rocm_device* device, const rlt_env_runner* rn, float* next_observations) {
+    int blocks = (rn->n_envs + 255) / 256; if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(pendulum_position_step_kernel, dim3(blocks), dim3(256), 0, device->stream, rn->pendulum, rn->states, (const float*)rn->actions, next_observations, rn->rewards,
+                       rn->terminated, rn->n_envs);
+    return rlt_launch_status(device);
 }
 // prologue_per_env (:8-62): reset where the last step truncated (state from the caller's draw, counters, the ring's last row marked truncated,
 // a new episode start), then observe
@@ -210,6 +230,7 @@ __global__ __launch_bounds__(256) void env_prologue_kernel(rlt_env_runner rn, rl
         }
         float* o = rn.observations + (size_t)e * d.obs;
         if (rn.env_kind == RLT_ENV_PENDULUM) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; o[2] = state[1]; }
+        else if (rn.env_kind == RLT_ENV_PENDULUM_POSITION) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; }
         else if (rn.env_kind == RLT_ENV_CAR) { for (int i = 0; i < 6; i++) o[i] = state[i]; }
         else { const Acrobot4 s4 = {{state[0], state[1], state[2], state[3]}}; acrobot_observe(s4, o); }
     }
@@ -299,6 +320,7 @@ extern "C" int rlt_rocm_env_runner_step(rlt_rocm_device* device, const rlt_env_r
             if ((rc = rlt_rocm_pendulum_step(device, &rn->pendulum, rn->states, rn->actions, nullptr, rn->next_observations, rn->rewards, N))) return rc;
             if ((rc = rlt_rocm_fill_u8(device, rn->terminated, (size_t)N, 0))) return rc;      // the Pendulum has no terminal states
             break;
+        case RLT_ENV_PENDULUM_POSITION: if ((rc = pendulum_position_step(device, rn, rn->next_observations))) return rc; break;
         case RLT_ENV_CAR: if ((rc = rlt_rocm_car_step(device, &rn->car, rn->states, rn->actions, nullptr, rn->next_observations, rn->rewards, rn->terminated, N))) return rc; break;
         default:
             if ((rc = rlt_rocm_acrobot_step(device, &rn->acrobot, rn->env_kind == RLT_ENV_ACROBOT_SWINGUP, rn->states, rn->actions, nullptr, rn->next_observations, rn->rewards,
@@ -317,6 +339,7 @@ __device__ __forceinline__ float mul_add_twice_rounded(float a, float b, float c
 }
 __device__ __forceinline__ void observe_any(int kind, const float* __restrict__ state, float* __restrict__ o) {
     if (kind == RLT_ENV_PENDULUM) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; o[2] = state[1]; }
+    else if (kind == RLT_ENV_PENDULUM_POSITION) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; }
     else if (kind == RLT_ENV_CAR) { for (int i = 0; i < 6; i++) o[i] = state[i]; }
     else { const Acrobot4 s4 = {{state[0], state[1], state[2], state[3]}}; acrobot_observe(s4, o); }
 }
@@ -379,6 +402,7 @@ int env_step_launch(rlt_rocm_device* device, const rlt_env_runner* rn, float* ne
         case RLT_ENV_PENDULUM:
             if ((rc = rlt_rocm_pendulum_step(device, &rn->pendulum, rn->states, rn->actions, nullptr, next_observations, rn->rewards, N))) return rc;
             return rlt_rocm_fill_u8(device, rn->terminated, (size_t)N, 0);      // the Pendulum has no terminal states
+        case RLT_ENV_PENDULUM_POSITION: return pendulum_position_step(device, rn, next_observations);
         case RLT_ENV_CAR: return rlt_rocm_car_step(device, &rn->car, rn->states, rn->actions, nullptr, next_observations, rn->rewards, rn->terminated, N);
         default: return rlt_rocm_acrobot_step(device, &rn->acrobot, rn->env_kind == RLT_ENV_ACROBOT_SWINGUP, rn->states, rn->actions, nullptr, next_observations, rn->rewards, rn->terminated, N);
     }

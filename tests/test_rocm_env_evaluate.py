@@ -16,6 +16,8 @@ pytestmark = pytest.mark.gpu
 def initial_states(rng, kind, n):
     if kind == capi.ENV_PENDULUM:
         return np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n)], 1).astype(np.float32)
+    if kind == capi.ENV_PENDULUM_POSITION:
+        return np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n), np.zeros(n)], 1).astype(np.float32)
     if kind == capi.ENV_CAR:
         s = np.zeros((n, 6), np.float32)
         s[:, :2] = rng.uniform(-0.5, 0.5, (n, 2))
@@ -44,6 +46,7 @@ CASES = [
     (capi.ENV_PENDULUM, 2, 17, None, 0, False),
     (capi.ENV_ACROBOT_SWINGUP, 2, 12, "gru", 8, False),
     (capi.ENV_ACROBOT, 1, 20, "gru", 0, False),
+    (capi.ENV_PENDULUM_POSITION, 2, 50, "gru", 100, False),      # the reference's recurrent configuration of the Pendulum: position only, restart of the hidden state every 100 steps
 ]
 
 

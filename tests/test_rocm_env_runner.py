@@ -16,6 +16,8 @@ pytestmark = pytest.mark.gpu
 def initial_states(rng, kind, n):
     if kind == capi.ENV_PENDULUM:
         return np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n)], 1).astype(np.float32)
+    if kind == capi.ENV_PENDULUM_POSITION:      # (theta, theta_dot, last action = 0)
+        return np.stack([rng.uniform(-np.pi, np.pi, n), rng.uniform(-1, 1, n), np.zeros(n)], 1).astype(np.float32)
     if kind == capi.ENV_CAR:
         s = np.zeros((n, 6), np.float32)
         s[::4, 0] = 0.97; s[::4, 3] = 3.0      # some cars start at the edge of the unit square, heading out
@@ -28,6 +30,8 @@ def initial_states(rng, kind, n):
 
 @pytest.mark.parametrize("kind,policy_kind,n_envs,capacity,limit,steps", [
     (capi.ENV_PENDULUM, 2, 37, 50, 20, 120),
+    (capi.ENV_PENDULUM_POSITION, 2, 41, 30, 15, 90),   # the velocity is hidden from the observation, the state remembers the last action
+    (capi.ENV_PENDULUM_POSITION, 0, 300, 8, 6, 40),
     (capi.ENV_ACROBOT, 0, 64, 40, 30, 100),            # terminates when the tip swings above the bar
     (capi.ENV_ACROBOT_SWINGUP, 2, 130, 25, 12, 60),
     (capi.ENV_CAR, 1, 50, 30, 25, 80),                 # terminates when the car leaves the unit square
@@ -63,7 +67,7 @@ def test_env_runner_step_matches_the_checker(oracle, rocm, kind, policy_kind, n_
         for k in (0, 2, 4, 5, 6, 7):
             assert rel_err(got[k], ref[k]) <= tol, (step, k, rel_err(got[k], ref[k]))
         n_term += int(ref[8].sum()); n_reset += int(ref[3].sum())
-    assert n_reset > 0 and (kind in (capi.ENV_PENDULUM, capi.ENV_ACROBOT_SWINGUP) or n_term > 0)      # the cases exercise what they are for
+    assert n_reset > 0 and (kind in (capi.ENV_PENDULUM, capi.ENV_PENDULUM_POSITION, capi.ENV_ACROBOT_SWINGUP) or n_term > 0)      # the cases exercise what they are for
     assert rel_err(got_rb[0], ref_rb[0]) <= tol
     for k in range(1, 5):
         assert np.array_equal(got_rb[k], ref_rb[k])
@@ -81,6 +85,7 @@ def test_env_dims(rocm):
 @pytest.mark.parametrize("kind,specs,head_kind,n_envs,capacity,limit,period,steps", [
     (capi.ENV_PENDULUM, [(0, 3, 16, "relu"), (1, 16, 16, "identity"), (0, 16, 1, "tanh")], 3, 40, 30, 12, 5, 70),        # TD3's exploration head on a recurrent policy
     (capi.ENV_ACROBOT, [(0, 6, 16, "relu"), (1, 16, 16, "identity"), (1, 16, 16, "identity"), (0, 16, 2, "identity")], 2, 33, 20, 10, 0, 50),
+    (capi.ENV_PENDULUM_POSITION, [(0, 2, 16, "relu"), (1, 16, 16, "identity"), (1, 16, 16, "identity"), (0, 16, 2, "identity")], 2, 32, 40, 20, 8, 60),     # the reference's recurrent SAC actor on the Pendulum without velocity
     (capi.ENV_CAR, [(0, 6, 32, "relu"), (0, 32, 2, "tanh")], 1, 50, 25, 9, 0, 40),                                   # a policy of dense layers, deterministic
 ])
 def test_env_runner_step_with_a_sequential_policy(oracle, rocm, kind, specs, head_kind, n_envs, capacity, limit, period, steps):
