@@ -1,6 +1,7 @@
 // The environments whose step, reward, observation and termination the library has kernels for, described to its entry points
 // (rlt_env_runner: a kind and that kind's parameters) from the reference's environment types, with their initial states drawn on the device:
 //   rl::environments::Pendulum        rl/environments/pendulum/pendulum.h,  sample_initial_state operations_generic.h:58-61
+//   rl::environments::PendulumPosition (pendulum.h:117-124: the velocity is hidden from the observation, the state remembers the last action), :62-66
 //   rl::environments::Acrobot         rl/environments/acrobot/acrobot.h,    sample_initial_state operations_generic.h:39-44
 //   rl::environments::AcrobotSwingup  (the same dynamics, another reward),  sample_initial_state operations_generic.h:46-52
 // The parameters of these environments are static members of ENVIRONMENT::SPEC::PARAMETERS, so a description needs the type only. The Car keeps its
@@ -37,6 +38,28 @@ namespace rl_tools::rl::environments::rocm{
         }
         // initial_state (rl/environments/pendulum/operations_generic.h:38-41): hanging down, at rest
         static void initial_state(float* host){ host[0] = -math::PI<float>; host[1] = 0; }
+    };
+    template <typename SPEC>
+    struct Description<rl::environments::PendulumPosition<SPEC>>{
+        using P = typename SPEC::PARAMETERS;
+        static constexpr bool SUPPORTED = true;
+        static constexpr int KIND = RLT_ENV_PENDULUM_POSITION;
+        static constexpr size_t STATE_DIM = 3;      // theta, theta_dot, last_action
+        static_assert(P::initial_state_min_angle == -P::initial_state_max_angle && P::initial_state_min_speed == -P::initial_state_max_speed, "initial states are drawn from ranges that are symmetric about zero");
+        static_assert(P::OBSERVATION_NOISE_POSITION == 0, "the library's kernels observe without noise");
+        static void set_parameters(rlt_env_runner& runner){ runner.env_kind = KIND; runner.pendulum = Description<rl::environments::Pendulum<SPEC>>::parameters(); }
+        // angle and speed uniform in +- their largest values, last_action = 0 (operations_generic.h:62-66)
+        template <typename DEV_SPEC, typename RNG>
+        static void sample_initial_states(devices::ROCM<DEV_SPEC>& device, float* initial, size_t n, RNG& rng){
+            devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, n * 3, -1.0f, 1.0f, rng.seed, random::next_stream(rng)), "sample_initial_state (PendulumPosition)");
+            devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_angle, initial, 3, initial, 3, (int)n, 1), "sample_initial_state (PendulumPosition)");
+            if constexpr(P::initial_state_max_speed != 1){
+                devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_speed, initial + 1, 3, initial + 1, 3, (int)n, 1), "sample_initial_state (PendulumPosition)");
+            }
+            devices::rocm::check(rlt_rocm_fill_f32(device.handle, initial + 2, (int)n, 1, 3, 0.0f), "sample_initial_state (PendulumPosition)");
+        }
+        // initial_state (operations_generic.h:42-46): hanging down, at rest, no action yet
+        static void initial_state(float* host){ host[0] = -math::PI<float>; host[1] = 0; host[2] = 0; }
     };
     namespace acrobot{
         template <typename P>

@@ -3,7 +3,8 @@
 // devices::ROCM the way src/rl/zoo/zoo.cpp:135-268 instantiates them on the CPU device: FACTORY<DEVICE, ...>::LOOP_CORE_CONFIG inside the
 // evaluation and timing loop steps (the experiment tracking, checkpoint and trajectory steps of zoo.cpp write files and are left out),
 // then `while(!step(device, ts))`. One source, four programs: -DZOO_SAC, -DZOO_TD3 or -DZOO_PPO selects the algorithm on the Pendulum as
-// RL_TOOLS_RL_ZOO_ALGORITHM_* does there, -DZOO_ACROBOT_SWINGUP_SAC the AcrobotSwingup with SAC (RL_TOOLS_RL_ZOO_ENVIRONMENT_ACROBOT_SWINGUP_V0). Nothing of the configuration is restated here: batch sizes, widths, activation functions,
+// RL_TOOLS_RL_ZOO_ALGORITHM_* does there, -DZOO_ACROBOT_SWINGUP_SAC the AcrobotSwingup with SAC (RL_TOOLS_RL_ZOO_ENVIRONMENT_ACROBOT_SWINGUP_V0),
+// -DZOO_PENDULUM_POSITION_SAC the Pendulum without velocity observations with SAC's recurrent approximators on sequences of 100 steps (src/rl/zoo/pendulum-position-v1/sac.h). Nothing of the configuration is restated here: batch sizes, widths, activation functions,
 // step limits and optimizer parameters are the zoo's.
 //
 // With -DZOO_DEVICE_CPU the same program runs on the reference's CPU device (its generic operations, one thread): the figure the device's is read against.
@@ -23,12 +24,14 @@
 #include <rl_tools/nn_models/mlp_unconditional_stddev/operations_generic.h>
 #include <rl_tools/nn_models/random_uniform/operations_generic.h>
 #include <rl_tools/nn_models/sequential/operations_generic.h>
+#include <rl_tools/nn/layers/gru/operations_generic.h>
 #include <rl_tools/nn/optimizers/adam/operations_generic.h>
 #include <rl_tools/rl/environments/pendulum/operations_cpu.h>
 #include <rl_tools/rl/environments/acrobot/operations_cpu.h>
 #ifndef ZOO_DEVICE_CPU
 #include <rl_tools/nn/operations_rocm.h>
 #include <rl_tools/nn/layers/standardize/operations_rocm.h>
+#include <rl_tools/nn/layers/gru/operations_rocm.h>
 #include <rl_tools/rl/components/running_normalizer/operations_rocm.h>
 #include <rl_tools/rl/components/off_policy_runner/operations_rocm.h>
 #include <rl_tools/rl/components/on_policy_runner/operations_rocm.h>
@@ -59,8 +62,14 @@
 #ifndef ZOO_DEVICE_CPU
 #include <rl_tools/rl/algorithms/sac/loop/core/operations_rocm.h>
 #endif
+#elif defined(ZOO_PENDULUM_POSITION_SAC)
+#include <pendulum-position-v1/sac.h>
+#include <rl_tools/rl/algorithms/sac/loop/core/operations_generic.h>
+#ifndef ZOO_DEVICE_CPU
+#include <rl_tools/rl/algorithms/sac/loop/core/operations_rocm.h>
+#endif
 #else
-#error "define ZOO_SAC, ZOO_TD3, ZOO_PPO or ZOO_ACROBOT_SWINGUP_SAC"
+#error "define ZOO_SAC, ZOO_TD3, ZOO_PPO, ZOO_ACROBOT_SWINGUP_SAC or ZOO_PENDULUM_POSITION_SAC"
 #endif
 #include <rl_tools/rl/loop/steps/evaluation/config.h>
 #include <rl_tools/rl/loop/steps/timing/config.h>
@@ -91,6 +100,9 @@ using LOOP_CORE_CONFIG = rlt::rl::zoo::pendulum_v1::td3::FACTORY<DEVICE, TYPE_PO
 constexpr TI TIMING_INTERVAL = 10000;
 #elif defined(ZOO_ACROBOT_SWINGUP_SAC)
 using LOOP_CORE_CONFIG = rlt::rl::zoo::acrobot_swingup_v0::sac::FACTORY<DEVICE, TYPE_POLICY, TI, RNG, DYNAMIC_ALLOCATION>::LOOP_CORE_CONFIG;
+constexpr TI TIMING_INTERVAL = 100000;
+#elif defined(ZOO_PENDULUM_POSITION_SAC)
+using LOOP_CORE_CONFIG = rlt::rl::zoo::pendulum_position_v1::sac::FACTORY<DEVICE, TYPE_POLICY, TI, RNG, DYNAMIC_ALLOCATION>::LOOP_CORE_CONFIG;
 constexpr TI TIMING_INTERVAL = 100000;
 #else
 using LOOP_CORE_CONFIG = rlt::rl::zoo::pendulum_v1::ppo::FACTORY<DEVICE, TYPE_POLICY, TI, RNG, DYNAMIC_ALLOCATION>::LOOP_CORE_CONFIG;
