@@ -200,3 +200,4 @@ namespace rl_tools{
     }
 }
 RL_TOOLS_NAMESPACE_WRAPPER_END
+#include <rl_tools/rl/algorithms/sac/operations_rocm_sequence.h>      // the same three functions for sequence batches and recurrent networks
