@@ -18,6 +18,10 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 FP32_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBPS = 8000.0
+# one SAC loop step at batch 256 with 3-64-64-2 / 4-64-64-1 networks: per sample 52,480 flop per critic update (actor and both target critics forward on the next
+# observations, critic forward + backward) and 61,440 per actor update (actor forward, both critics forward + backward_input, actor backward)
+SAC_STEP_FLOP = 256 * (2 * 52480 + 61440)
 MLP_FLOP_PER_SAMPLE_FWD = 2 * (17 * 256 + 256 * 256 + 256 * 6)                       # 142,848
 MLP_FLOP_PER_SAMPLE_BWD = 2 * (17 * 256 + 256 * 256 + 256 * 6) + 2 * (256 * 256 + 256 * 6)   # weight grads + d_input of layers 2,3: 276,992
 
@@ -54,6 +58,15 @@ class HipEvents:
 # HBM bytes of one mlp_forward_backward call at batch 65,536, from two counter runs (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch,
 # the factors being what the same counters read for a 256 MiB copy): fused kernel 15.4 + 77.7, reduce kernel 106.0 + 0.3, prepare 1.2 + 0.5 MiB
 MLP_CALL_HBM_BYTES = int((15422 + 77676 + 106016 + 281 + 1228 + 544) * 1024)
+
+
+def checker():
+    """tests/helpers.py: the loader of the CPU checker (oracle/), used by the CPU legs only."""
+    tests = os.path.join(ROOT, "tests")
+    if tests not in sys.path:
+        sys.path.insert(0, tests)
+    import helpers as tests_helpers
+    return tests_helpers
 
 
 def bench_mlp(helpers, rocm, batch, iters, warmup):
@@ -299,7 +312,7 @@ def bench_sac_sequence(helpers, rocm, S=100, B=100, iters=10, cpu_seconds=1.5):
                 terminated=np.zeros((S, B), np.uint8), reset=reset, next_reset_base=next_reset, final_step_mask=final, next_final_step_mask_base=next_final)
     nc, na = rng.standard_normal((S + 1, B, ACT)).astype(np.float32), rng.standard_normal((S, B, ACT)).astype(np.float32)
     out = {"sequence_length": S, "batch": B, "actor": "3-16-GRU16-GRU16-2", "critic": "4-32-GRU32-GRU32-1"}
-    for be in (rocm, helpers.HostBackend()):
+    for be in (rocm, checker().HostBackend()):      # the CPU leg: the same calls on the checker
         agent = helpers.SacSequenceOnBackend(be, actor_specs, critic_specs, params, S, B, OBS, ACT, True)
         agent.set_batch(data)
         ncd, nad = be.array(nc), be.array(na)
@@ -534,6 +547,27 @@ def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=100
         wall_s = time.perf_counter() - t0
         offset += warmup + steps
         variants[name] = {"steps_per_s": steps / wall_s, "steps_per_s_by_device_clock": steps / device_s, "launches_per_step": 4 if tail else 7}
+    # the same loop step recorded into a HIP graph (rlt_rocm_graph_*; what rl/environments/pendulum/sac/cuda/sac.cu:122-164 does with its step) and replayed
+    graph = C.c_void_p()
+    rocm.call("graph_begin_capture")
+    try:
+        rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), 1, seed, offset, C.byref(scratch))
+        rocm.call("advance_streams", 8)
+    finally:
+        rocm.call("graph_end_capture", C.byref(graph))
+    try:
+        for _ in range(warmup):
+            rocm.call("graph_launch", graph)
+        rocm.sync()
+        t0 = time.perf_counter(); a = ev.record()
+        for _ in range(steps):
+            rocm.call("graph_launch", graph)
+        b = ev.record()
+        graph_device_s = ev.elapsed_ms(a, b) * 1e-3
+        variants["recorded_graph_replayed"] = {"steps_per_s": steps / (time.perf_counter() - t0), "steps_per_s_by_device_clock": steps / graph_device_s, "launches_per_step": 4}
+    finally:
+        rocm.call("set_stream_offset", 0)
+        rocm.call("graph_destroy", graph)
     assert np.all(np.isfinite(agent.parameters())), "SAC parameters went non-finite"
     out.update(steps_per_s=steps / wall_s, steps_per_s_by_device_clock=steps / device_s, steps=steps, launches_per_step=4, variants=variants)
     # a wider agent: the update calls alone
@@ -587,10 +621,8 @@ def cpu_baseline(batch=256, seconds=12.0):
             lib.rlt_ref_sac_destroy(hdl)
         return {"value": n / total, "unit": "loop steps/s", "cores": cores, "kind": "reference", "cblas_path": lib.rlt_ref_cblas_name(),
                 "sample": f"{n} post-warm-up loop steps of the reference's Pendulum SAC loop at batch {batch}, CBLAS = {os.path.basename(lib.rlt_ref_cblas_name().decode())}, 1 thread"}
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import helpers
-    o = helpers.HostBackend()
-    cfg = helpers.LoopConfig(0, batch, 64, 10000, batch, 200, 1e-7)
+    o = checker().HostBackend()
+    cfg = checker().LoopConfig(0, batch, 64, 10000, batch, 200, 1e-7)
     loop = C.c_void_p(o.lib.rlt_oracle_sac_loop_create(C.byref(cfg)))
     for _ in range(batch + 10):
         o.lib.rlt_oracle_sac_loop_step(loop)
@@ -606,7 +638,7 @@ def cpu_baseline(batch=256, seconds=12.0):
 def cpu_other_configurations(helpers, cblas_path):
     """The other configurations on this host's CPU, one thread, bounded samples (a few seconds in all): the CPU restatement with its three GEMMs per dense
     layer routed through the same CBLAS the reference's CPU build uses (what its CPU_BLAS device does), or plain loops where no CBLAS was found."""
-    o = helpers.HostBackend()
+    o = checker().HostBackend()
     capi = helpers.capi
     blas = bool(cblas_path) and o.lib.rlt_oracle_use_cblas(cblas_path) == 0
     out = {"kind": "port", "cores": 1, "gemm": os.path.basename(cblas_path.decode()) if blas else "plain loops"}
@@ -680,9 +712,7 @@ def main():
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the hot path has no cross-GPU part); use --gpus 1", file=sys.stderr)
         sys.exit(2)
-    package()
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import helpers
+    helpers = package().builders      # networks, agents, runners on a backend (rl-tools_amd/builders.py)
     rocm = helpers.RocmBackend()
     info = rocm.device.info()
     if args.pmc_probe:
@@ -693,6 +723,7 @@ def main():
         return
     mlp = bench_mlp(helpers, rocm, args.mlp_batch, args.mlp_iters, 3) if args.only in ("all", "mlp") else None
     sac = bench_sac(helpers, rocm, args.steps, args.warmup, per_operation=args.sac_per_operation, phase_profile=args.sac_phase_profile) if args.only in ("all", "sac") else {"steps_per_s": 0.0, "ms_per_step": 0.0}
+    mlp_other = {str(b): bench_mlp(helpers, rocm, b, 100, 10) for b in (256, 4096)} if args.only in ("all", "mlp") else None      # configuration 1's other two batch sizes
     api = bench_sac_api(helpers, rocm) if args.only in ("all", "sac", "api") else None
     env = bench_env(helpers, rocm) if args.only in ("all", "env") else None
     ppo = bench_ppo(helpers, rocm) if args.only in ("all", "ppo") else None
@@ -720,6 +751,33 @@ def main():
         line["roofline"] = {"bound": "mfma", "achieved": mlp["tflops"], "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": mlp["tflops"] / FP32_PEAK_TFLOPS,
                             "traffic": MLP_CALL_HBM_BYTES if mlp["batch"] == 65536 else None, "traffic_unit": "bytes per call, from rocprofv3 FETCH_SIZE / WRITE_SIZE",
                             "kernel": "mlp_forward_backward call = mlp3_prepare_kernel + mlp3_fused_kernel + mlp3_reduce_kernel", "flop_per_launch": flop}
+    if mlp_other:
+        line["mlp_by_batch"] = mlp_other
+    # one roofline object per configuration (the dominant kernel of each; `roofline` above stays the benchmark's own): algorithmic bytes or flop over the measured
+    # time against MI355X's published peaks; traffic = HBM bytes per launch from the counter runs summarised under profiles/ (null where none was made)
+    def hbm(kernel, gbps, traffic, note):
+        return {"kernel": kernel, "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic, "algorithmic": note}
+
+    def mfma(kernel, tflops, traffic, note):
+        return {"kernel": kernel, "bound": "mfma", "achieved": tflops, "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / FP32_PEAK_TFLOPS, "traffic": traffic, "algorithmic": note}
+    rooflines = {}
+    if sac.get("steps_per_s"):
+        rooflines["sac_loop_step_b256"] = mfma("sac_pendulum_loop_kernel", SAC_STEP_FLOP * sac["steps_per_s"] / 1e12, None, "%.1f MFLOP per loop step (2 critic + 1 actor update at batch 256, widths 64)" % (SAC_STEP_FLOP / 1e6))
+    if mlp_other:
+        for b, m in mlp_other.items():
+            rooflines["mlp_forward_backward_b" + b] = mfma("mlp_forward_backward call", m["tflops"], None, "%d flop per sample" % (MLP_FLOP_PER_SAMPLE_FWD + MLP_FLOP_PER_SAMPLE_BWD))
+    if env:
+        rooflines["env_step_65536"] = hbm("runner_fused_kernel", env["algorithmic_GBps"], 9.98e6, "68 B per environment step")
+        rooflines["gather_batch_4096"] = hbm("gather_kernel", env["gather_algorithmic_GBps"], 1.72e6, "85 B per row")
+        rooflines["acrobot_step_1048576"] = hbm("acrobot_step_kernel", env["acrobot"]["algorithmic_GBps"], 93.6e6, "89 B per environment step")
+    if ppo:
+        rooflines["ppo_gae_4096x128"] = hbm("gae_kernel", ppo["gae_algorithmic_GBps"], 91.9e6, "24 B per dataset row")
+        rooflines["ppo_minibatch_update_8192"] = mfma("mlp3s_kernel + adam_pair_kernel", ppo["tflops"], None, "106,368 flop per row and epoch (actor 105-64-64-8 and critic 105-64-64-1, forward + backward)")
+    if gru:
+        for g in gru:
+            rooflines["gru_training_step_b%d" % g["batch"]] = mfma("gru_forward_mfma_kernel + gru_backward_mfma_kernel + projections", g["tflops"], None, "forward + backward through time, 64 steps, input 146, hidden 64")
+    if rooflines:
+        line["rooflines"] = rooflines
     if env:
         line["env_pipeline"] = env
     if ppo:

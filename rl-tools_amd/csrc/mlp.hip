@@ -240,8 +240,9 @@ static int forward_backward_impl(rlt_rocm_device* device, const rlt_dense_layer*
     RLT_REQUIRE((!y || ldy >= O) && (!d_output || ldd >= O) && (!target || ldt >= O) && (!d_input || ldi >= layers[0].in_dim));
     for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases);
     RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_mlp_workspace_bytes(layers, n, batch));
-    if (!d_input) {
-        // one pass over the batch with on-chip activations where the network has the shape that kernel is built for
+    if (!d_input && batch >= FUSED_MIN_BATCH) {
+        // one pass over the batch with on-chip activations where the network has the shape that kernel is built for (below that batch size its three launches
+        // and the per-call copy of the weights cost more than the per-layer path)
         const int rc = rlt_mlp3_fused_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, workspace, workspace_bytes);
         if (rc != RLT_E_UNSUPPORTED) return rc;
     }
@@ -255,15 +256,22 @@ static int forward_backward_impl(rlt_rocm_device* device, const rlt_dense_layer*
     char* w = (char*)workspace;
     const size_t buf = align_up((size_t)batch * max_dim(layers, n) * sizeof(float));
     float* tick = (float*)w; w += buf; float* tock = (float*)w; w += buf; float* dlast = (float*)w; w += buf;
+    const bool few_rows = n > 1 && batch <= RLT_MLP_ROWS_MAX_BATCH && rows_enabled();      // all layers' forward passes in one launch, which writes both buffers of a layer
     for (int l = 0; l < n; l++) {
         priv[l] = layers[l];
         // the activation derivative is recovered from the output wherever the activation allows it, so only GELU layers keep both
         priv[l].pre_activations = nullptr;
-        if (layers[l].activation == RLT_ACT_GELU) { priv[l].pre_activations = (float*)w; w += (size_t)batch * layers[l].out_dim * sizeof(float); }
+        if (few_rows || layers[l].activation == RLT_ACT_GELU) { priv[l].pre_activations = (float*)w; w += (size_t)batch * layers[l].out_dim * sizeof(float); }
         priv[l].output = (float*)w; w += (size_t)batch * layers[l].out_dim * sizeof(float);
     }
+    bool forwarded = false;
+    if (few_rows) {
+        const int rc = rlt_mlp_rows_forward(device, priv, n, x, ldx, y, ldy, batch, true);
+        if (rc && rc != RLT_E_UNSUPPORTED) return rc;
+        forwarded = rc == 0;
+    }
     const float* in = x; int ldin = ldx;
-    for (int l = 0; l < n; l++) {
+    for (int l = 0; l < n && !forwarded; l++) {
         int rc = rlt_gemm_forward(device, in, ldin, priv[l].weights, priv[l].biases, priv[l].activation, priv[l].pre_activations, priv[l].output,
                                   (l == n - 1) ? y : nullptr, ldy, batch, priv[l].in_dim, priv[l].out_dim);
         if (rc) return rc;
