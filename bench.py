@@ -508,7 +508,7 @@ def bench_sac(helpers, rocm, steps, warmup, batch=256, capacity=10000, per_opera
             "evaluation_return_after_run": float(summary.numpy()[0])}
 
 
-def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=10000):
+def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=10000, graph_replay=True):
     """The API path: the reference's loop step composed of the library's own entry points by its host loop (no Python between the calls),
     with the fused three-launch updates; and the four update calls alone on synthetic batches for a wider agent (observation 27, action 8)."""
     capi = helpers.capi
@@ -549,25 +549,28 @@ def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=100
         variants[name] = {"steps_per_s": steps / wall_s, "steps_per_s_by_device_clock": steps / device_s, "launches_per_step": 4 if tail else 7}
     # the same loop step recorded into a HIP graph (rlt_rocm_graph_*; what rl/environments/pendulum/sac/cuda/sac.cu:122-164 does with its step) and replayed
     graph = C.c_void_p()
-    rocm.call("graph_begin_capture")
+    if graph_replay:
+        rocm.call("graph_begin_capture")
+        try:
+            rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), 1, seed, offset, C.byref(scratch))
+            rocm.call("advance_streams", 8)
+        finally:
+            rocm.call("graph_end_capture", C.byref(graph))
     try:
-        rocm.call("sac_pendulum_loop_by_calls", C.byref(agent.c), C.byref(runner), C.byref(rb.c), 1, seed, offset, C.byref(scratch))
-        rocm.call("advance_streams", 8)
-    finally:
-        rocm.call("graph_end_capture", C.byref(graph))
-    try:
-        for _ in range(warmup):
+        for _ in range(warmup if graph_replay else 0):
             rocm.call("graph_launch", graph)
         rocm.sync()
         t0 = time.perf_counter(); a = ev.record()
-        for _ in range(steps):
+        for _ in range(steps if graph_replay else 0):
             rocm.call("graph_launch", graph)
         b = ev.record()
         graph_device_s = ev.elapsed_ms(a, b) * 1e-3
-        variants["recorded_graph_replayed"] = {"steps_per_s": steps / (time.perf_counter() - t0), "steps_per_s_by_device_clock": steps / graph_device_s, "launches_per_step": 4}
+        if graph_replay:
+            variants["recorded_graph_replayed"] = {"steps_per_s": steps / (time.perf_counter() - t0), "steps_per_s_by_device_clock": steps / graph_device_s, "launches_per_step": 4}
     finally:
         rocm.call("set_stream_offset", 0)
-        rocm.call("graph_destroy", graph)
+        if graph_replay:
+            rocm.call("graph_destroy", graph)
     assert np.all(np.isfinite(agent.parameters())), "SAC parameters went non-finite"
     out.update(steps_per_s=steps / wall_s, steps_per_s_by_device_clock=steps / device_s, steps=steps, launches_per_step=4, variants=variants)
     # a wider agent: the update calls alone
@@ -707,6 +710,7 @@ def main():
                     help="print the persistent kernel's per-phase time (stderr); 'stages' adds the clock between the barrier-separated stages of the critic and actor phases")
     ap.add_argument("--pmc-probe", action="store_true", help="for counter runs under rocprofv3 --pmc: three 256 MiB device copies (a kernel of known traffic, to scale the counters by) "
                     "three MLP forward+backward calls, then the environment-pipeline and PPO workloads (their figures discarded)")
+    ap.add_argument("--no-graph-replay", action="store_true", help="leave out the replay of a recorded loop step (for runs under rocprofv3, whose kernel tracing does not survive hipGraphLaunch here)")
     ap.add_argument("--sac-per-operation", action="store_true", help="time the one-launch-per-operation SAC path instead of the persistent kernel")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -724,7 +728,7 @@ def main():
     mlp = bench_mlp(helpers, rocm, args.mlp_batch, args.mlp_iters, 3) if args.only in ("all", "mlp") else None
     sac = bench_sac(helpers, rocm, args.steps, args.warmup, per_operation=args.sac_per_operation, phase_profile=args.sac_phase_profile) if args.only in ("all", "sac") else {"steps_per_s": 0.0, "ms_per_step": 0.0}
     mlp_other = {str(b): bench_mlp(helpers, rocm, b, 100, 10) for b in (256, 4096)} if args.only in ("all", "mlp") else None      # configuration 1's other two batch sizes
-    api = bench_sac_api(helpers, rocm) if args.only in ("all", "sac", "api") else None
+    api = bench_sac_api(helpers, rocm, graph_replay=not args.no_graph_replay) if args.only in ("all", "sac", "api") else None
     env = bench_env(helpers, rocm) if args.only in ("all", "env") else None
     ppo = bench_ppo(helpers, rocm) if args.only in ("all", "ppo") else None
     gru = [bench_gru(helpers, rocm, b) for b in (64, 1024)] if args.only in ("all", "gru") else None

@@ -1120,6 +1120,17 @@ int rlt_rocm_env_runner_step_sequential(rlt_rocm_device* device, const rlt_env_r
                                         const rlt_seq_layer* policy, int n_policy_layers, const rlt_seq_state* policy_state, int auto_reset_period,
                                         int head_kind, const rlt_sas_parameters* sas, float exploration_noise_std, const float* action_noise,
                                         const float* initial_states, void* workspace, size_t workspace_bytes);
+/* The same step with every draw made by the launch itself, for at most 16 environments and a policy of at most 8 dense layers no wider than 256 (the loops that
+ * step one or a few environments per training step): ONE launch for reset, observation, policy, head, dynamics, counters and the replay add.
+ *   head_kind 0 (n_policy_layers = 0): uniform actions in (-1, 1), the exploration policy of the warm-up phase (nn_models/random_uniform/operations_generic.h:28-44);
+ *   1, 2, 3 as above. Draws: element e * action_dim + c of stream noise_stream under `seed` (what rlt_rocm_randn_f32 would write there; for head_kind 0 what
+ *   rlt_rocm_rand_f32(-1, 1) would), and for an environment that starts an episode state component i = initial_low[i] + (initial_high[i] - initial_low[i]) * u
+ *   with u element e * state_dim + i of rlt_rocm_rand_f32(0, 1) on stream initial_state_stream (the environments' sample_initial_state, e.g.
+ *   rl/environments/acrobot/operations_generic.h:39-52); initial_low and initial_high are HOST arrays of state_dim floats. drawn_noise (optional, device) [n_envs x action_dim] receives the noise or the uniform actions.
+ * RLT_E_UNSUPPORTED for more environments, a recurrent or wider policy: draw into arrays and call rlt_rocm_env_runner_step_sequential then. */
+int rlt_rocm_env_runner_step_drawn(rlt_rocm_device* device, const rlt_env_runner* runner, const rlt_replay_buffer* rb, const rlt_seq_layer* policy, int n_policy_layers,
+                                   int head_kind, const rlt_sas_parameters* sas, float exploration_noise_std, const float* initial_low, const float* initial_high,
+                                   float* drawn_noise, uint64_t seed, uint64_t noise_stream, uint64_t initial_state_stream);
 
 /* collect for any of the batched environments and any sequential policy (dense and GRU layers): rl/components/on_policy_runner/
  * operations_generic.h:105-146 over operations_generic_per_env.h:8-74. Per step: reset(policy, policy_state) where the runner's truncated flag

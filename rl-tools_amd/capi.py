@@ -337,6 +337,7 @@ ROCM_ONLY = {
     "memcpy_h2d": ([P, P, P, S], I), "memcpy_d2h": ([P, P, P, S], I), "memcpy_d2d": ([P, P, P, S], I),
     "memcpy2d": ([P, P, S, P, S, S, S, I], I),
     "fill_f32": ([P, P, I, I, I, F], I), "fill_from_f32": ([P, P, I, I, I, P], I), "fill_u8": ([P, P, S, C.c_uint8], I),
+    "env_runner_step_drawn": ([P, C.POINTER(EnvRunner), C.POINTER(ReplayBuffer), C.POINTER(SeqLayer), I, I, C.POINTER(SasParameters), F, P, P, P, U64, U64, U64], I),
     "randn_f32": ([P, P, S, U64, U64], I), "rand_f32": ([P, P, S, F, F, U64, U64], I), "rand_bits_u32": ([P, P, S, U64, U64], I),
     "reduce_sum_f32": ([P, P, S, I, P], I),
     "dense_backward_static": ([P, LP, P, I, P, I, I], I),

@@ -5,6 +5,7 @@
 // environment (state in and out, observations, reward, flag) once there are enough environments to fill the device.
 #include "common.h"
 #include "pendulum.h"
+#include "rng.h"
 
 namespace {
 struct Acrobot4 { float v[4]; };
@@ -35,30 +36,34 @@ __device__ __forceinline__ void acrobot_observe(const Acrobot4& s, float* __rest
     o[4] = s.v[2]; o[5] = s.v[3];
 }
 
+// one environment's step: Runge-Kutta over one time step (:98-117), reward, flag, observations
+__device__ __forceinline__ void acrobot_step_one(const rlt_acrobot_parameters& P, int swingup, float* __restrict__ states, const float* __restrict__ actions,
+                                                 float* __restrict__ observations, float* __restrict__ next_observations, float* __restrict__ rewards,
+                                                 uint8_t* __restrict__ terminated, int e) {
+    const float PI = 3.14159265358979323846f;
+    const float4 raw = reinterpret_cast<const float4*>(states)[e];
+    const Acrobot4 s = {{raw.x, raw.y, raw.z, raw.w}};
+    if (observations) acrobot_observe(s, observations + 6 * (size_t)e);
+    const float action = (clampf(actions[e], -1.0f, 1.0f) + 1.0f) / 2.0f * (P.max_torque - P.min_torque) + P.min_torque;
+    const Acrobot4 k1 = acrobot_dsdt(P, s, action);
+    const Acrobot4 k2 = acrobot_dsdt(P, axpy(s, P.dt / 2.0f, k1), action);
+    const Acrobot4 k3 = acrobot_dsdt(P, axpy(s, P.dt / 2.0f, k2), action);
+    const Acrobot4 k4 = acrobot_dsdt(P, axpy(s, P.dt, k3), action);
+    Acrobot4 next;
+#pragma unroll
+    for (int i = 0; i < 4; i++) next.v[i] = s.v[i] + P.dt / 6.0f * (k1.v[i] + 2.0f * k2.v[i] + 2.0f * k3.v[i] + k4.v[i]);
+    next.v[0] = angle_normalize(next.v[0]); next.v[1] = angle_normalize(next.v[1]);
+    next.v[2] = clampf(next.v[2], -P.max_vel_1, P.max_vel_1); next.v[3] = clampf(next.v[3], -P.max_vel_2, P.max_vel_2);
+    if (rewards) rewards[e] = swingup ? (-fabsf(angle_normalize(next.v[0] - PI)) - fabsf(angle_normalize(next.v[1]))) / 100.0f * P.dt / 0.02f : -1.0f;
+    if (terminated) terminated[e] = swingup ? 0 : ((-cosf(next.v[0]) - cosf(next.v[1] + next.v[0])) > 1.0f);
+    if (next_observations) acrobot_observe(next, next_observations + 6 * (size_t)e);
+    reinterpret_cast<float4*>(states)[e] = make_float4(next.v[0], next.v[1], next.v[2], next.v[3]);
+}
 __global__ __launch_bounds__(256) void acrobot_step_kernel(rlt_acrobot_parameters P, int swingup, float* __restrict__ states, const float* __restrict__ actions,
                                                            float* __restrict__ observations, float* __restrict__ next_observations, float* __restrict__ rewards,
                                                            uint8_t* __restrict__ terminated, int n) {
-    const float PI = 3.14159265358979323846f;
-    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
-        const float4 raw = reinterpret_cast<const float4*>(states)[e];
-        const Acrobot4 s = {{raw.x, raw.y, raw.z, raw.w}};
-        if (observations) acrobot_observe(s, observations + 6 * (size_t)e);
-        const float action = (clampf(actions[e], -1.0f, 1.0f) + 1.0f) / 2.0f * (P.max_torque - P.min_torque) + P.min_torque;
-        // classic Runge-Kutta over one time step (:98-117)
-        const Acrobot4 k1 = acrobot_dsdt(P, s, action);
-        const Acrobot4 k2 = acrobot_dsdt(P, axpy(s, P.dt / 2.0f, k1), action);
-        const Acrobot4 k3 = acrobot_dsdt(P, axpy(s, P.dt / 2.0f, k2), action);
-        const Acrobot4 k4 = acrobot_dsdt(P, axpy(s, P.dt, k3), action);
-        Acrobot4 next;
-#pragma unroll
-        for (int i = 0; i < 4; i++) next.v[i] = s.v[i] + P.dt / 6.0f * (k1.v[i] + 2.0f * k2.v[i] + 2.0f * k3.v[i] + k4.v[i]);
-        next.v[0] = angle_normalize(next.v[0]); next.v[1] = angle_normalize(next.v[1]);
-        next.v[2] = clampf(next.v[2], -P.max_vel_1, P.max_vel_1); next.v[3] = clampf(next.v[3], -P.max_vel_2, P.max_vel_2);
-        if (rewards) rewards[e] = swingup ? (-fabsf(angle_normalize(next.v[0] - PI)) - fabsf(angle_normalize(next.v[1]))) / 100.0f * P.dt / 0.02f : -1.0f;
-        if (terminated) terminated[e] = swingup ? 0 : ((-cosf(next.v[0]) - cosf(next.v[1] + next.v[0])) > 1.0f);
-        if (next_observations) acrobot_observe(next, next_observations + 6 * (size_t)e);
-        reinterpret_cast<float4*>(states)[e] = make_float4(next.v[0], next.v[1], next.v[2], next.v[3]);
-    }
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x)
+        acrobot_step_one(P, swingup, states, actions, observations, next_observations, rewards, terminated, e);
 }
 
 // Car: single-track model with Pacejka tire forces, explicit Euler over dt (rl/environments/car/operations_generic.h:99-127)
@@ -95,17 +100,19 @@ __device__ __forceinline__ void car_store(float* __restrict__ rows, size_t row_f
 }
 
 // without a track: the reward comes from the pre-step state (:128-135), terminated from the next one (:80-84), the observation is the state (:143-155)
+__device__ __forceinline__ void car_step_one(const rlt_car_parameters& p, float* __restrict__ states, const float* __restrict__ actions, float* __restrict__ observations,
+                                             float* __restrict__ next_observations, float* __restrict__ rewards, uint8_t* __restrict__ terminated, int e) {
+    const Car6 s = car_load(states, e);
+    if (observations) car_store(observations, 6, e, s);
+    const Car6 nx = car_dynamics(p, s, reinterpret_cast<const float2*>(actions)[e]);
+    if (rewards) { const float an = angle_normalize(s.mu); rewards[e] = expf(-5.0f * (0.1f * an * an + s.x * s.x + s.y * s.y)); }
+    if (terminated) terminated[e] = nx.x > 1.0f || nx.x < -1.0f || nx.y > 1.0f || nx.y < -1.0f;
+    if (next_observations) car_store(next_observations, 6, e, nx);
+    car_store(states, 6, e, nx);
+}
 __global__ __launch_bounds__(256) void car_step_kernel(rlt_car_parameters p, float* __restrict__ states, const float* __restrict__ actions, float* __restrict__ observations,
                                                        float* __restrict__ next_observations, float* __restrict__ rewards, uint8_t* __restrict__ terminated, int n) {
-    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
-        const Car6 s = car_load(states, e);
-        if (observations) car_store(observations, 6, e, s);
-        const Car6 nx = car_dynamics(p, s, reinterpret_cast<const float2*>(actions)[e]);
-        if (rewards) { const float an = angle_normalize(s.mu); rewards[e] = expf(-5.0f * (0.1f * an * an + s.x * s.x + s.y * s.y)); }
-        if (terminated) terminated[e] = nx.x > 1.0f || nx.x < -1.0f || nx.y > 1.0f || nx.y < -1.0f;
-        if (next_observations) car_store(next_observations, 6, e, nx);
-        car_store(states, 6, e, nx);
-    }
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) car_step_one(p, states, actions, observations, next_observations, rewards, terminated, e);
 }
 
 // on a track (:85-98 terminated, :136-141 reward, :156-190 observe): cell coordinates in double, as the reference's double literal makes them
@@ -195,16 +202,18 @@ __host__ __device__ inline EnvDims env_dims(int kind) {
 }
 // The Pendulum whose observation is the position only and whose state also remembers the last action (rl/environments/pendulum/pendulum.h:117-124,
 // step operations_generic.h:102-108, observe :168-181): states [n x 3] = (theta, theta_dot, last_action), observations [n x 2] = (cos, sin)
+__device__ __forceinline__ void pendulum_position_step_one(const rlt_pendulum_parameters& p, float* __restrict__ states, const float* __restrict__ actions,
+                                                           float* __restrict__ next_observations, float* __restrict__ rewards, uint8_t* __restrict__ terminated, int e) {
+    Transition t;
+    pendulum_transition(p, states[3 * (size_t)e], states[3 * (size_t)e + 1], actions[e], t);
+    if (next_observations) { next_observations[2 * (size_t)e] = t.next_obs[0]; next_observations[2 * (size_t)e + 1] = t.next_obs[1]; }
+    if (rewards) rewards[e] = t.reward;
+    if (terminated) terminated[e] = 0;      // the Pendulum has no terminal states
+    states[3 * (size_t)e] = t.theta; states[3 * (size_t)e + 1] = t.theta_dot; states[3 * (size_t)e + 2] = actions[e];
+}
 __global__ __launch_bounds__(256) void pendulum_position_step_kernel(rlt_pendulum_parameters p, float* __restrict__ states, const float* __restrict__ actions,
                                                                      float* __restrict__ next_observations, float* __restrict__ rewards, uint8_t* __restrict__ terminated, int n) {
-    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
-        Transition t;
-        pendulum_transition(p, states[3 * (size_t)e], states[3 * (size_t)e + 1], actions[e], t);
-        if (next_observations) { next_observations[2 * (size_t)e] = t.next_obs[0]; next_observations[2 * (size_t)e + 1] = t.next_obs[1]; }
-        if (rewards) rewards[e] = t.reward;
-        if (terminated) terminated[e] = 0;      // the Pendulum has no terminal states
-        states[3 * (size_t)e] = t.theta; states[3 * (size_t)e + 1] = t.theta_dot; states[3 * (size_t)e + 2] = actions[e];
-    }
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) pendulum_position_step_one(p, states, actions, next_observations, rewards, terminated, e);
 }
 int pendulum_position_step(rlt_rocm_device* device, const rlt_env_runner* rn, float* next_observations) {
     int blocks = (rn->n_envs + 255) / 256; if (blocks > 4096) blocks = 4096;
@@ -214,57 +223,199 @@ int pendulum_position_step(rlt_rocm_device* device, const rlt_env_runner* rn, fl
 }
 // prologue_per_env (:8-62): reset where the last step truncated (state from the caller's draw, counters, the ring's last row marked truncated,
 // a new episode start), then observe
-__global__ __launch_bounds__(256) void env_prologue_kernel(rlt_env_runner rn, rlt_replay_buffer rb, const float* __restrict__ initial_states) {
+__device__ __forceinline__ void env_observe_one(int kind, const float* __restrict__ state, float* __restrict__ o) {
+    if (kind == RLT_ENV_PENDULUM) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; o[2] = state[1]; }
+    else if (kind == RLT_ENV_PENDULUM_POSITION) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; }
+    else if (kind == RLT_ENV_CAR) { for (int i = 0; i < 6; i++) o[i] = state[i]; }
+    else { const Acrobot4 s4 = {{state[0], state[1], state[2], state[3]}}; acrobot_observe(s4, o); }
+}
+// `initial`: the state this environment starts its next episode from
+__device__ __forceinline__ void env_prologue_one(const rlt_env_runner& rn, const rlt_replay_buffer& rb, const float* initial, int e) {
     const EnvDims d = env_dims(rn.env_kind);
     const int R = 2 * rb.observation_dim + rb.action_dim + 3;
-    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) {
-        float* state = rn.states + (size_t)e * d.state;
-        if (rn.truncated[e]) {
-            for (int i = 0; i < d.state; i++) state[i] = initial_states[(size_t)e * d.state + i];
-            rn.episode_step[e] = 0; rn.episode_return[e] = 0.0f;
-            if (rb.full[e] || rb.position[e] > 0) {
-                const uint32_t prev = rb.position[e] == 0 ? (uint32_t)rb.capacity - 1 : rb.position[e] - 1;
-                rb.data[((size_t)e * rb.capacity + prev) * R + (R - 1)] = 1.0f;
-                rb.current_episode_start[e] = rb.position[e];
-            }
+    float* state = rn.states + (size_t)e * d.state;
+    if (rn.truncated[e]) {
+        for (int i = 0; i < d.state; i++) state[i] = initial[i];
+        rn.episode_step[e] = 0; rn.episode_return[e] = 0.0f;
+        if (rb.full[e] || rb.position[e] > 0) {
+            const uint32_t prev = rb.position[e] == 0 ? (uint32_t)rb.capacity - 1 : rb.position[e] - 1;
+            rb.data[((size_t)e * rb.capacity + prev) * R + (R - 1)] = 1.0f;
+            rb.current_episode_start[e] = rb.position[e];
         }
-        float* o = rn.observations + (size_t)e * d.obs;
-        if (rn.env_kind == RLT_ENV_PENDULUM) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; o[2] = state[1]; }
-        else if (rn.env_kind == RLT_ENV_PENDULUM_POSITION) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; }
-        else if (rn.env_kind == RLT_ENV_CAR) { for (int i = 0; i < 6; i++) o[i] = state[i]; }
-        else { const Acrobot4 s4 = {{state[0], state[1], state[2], state[3]}}; acrobot_observe(s4, o); }
     }
+    env_observe_one(rn.env_kind, state, rn.observations + (size_t)e * d.obs);
+}
+__global__ __launch_bounds__(256) void env_prologue_kernel(rlt_env_runner rn, rlt_replay_buffer rb, const float* __restrict__ initial_states) {
+    const int state_dim = env_dims(rn.env_kind).state;
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) env_prologue_one(rn, rb, initial_states + (size_t)e * state_dim, e);
 }
 // the rest of epilogue_per_env after the environment's own step (:88-104): counters, truncation, replay add (replay_buffer/operations_generic.h:54-78)
-__global__ __launch_bounds__(256) void env_epilogue_kernel(rlt_env_runner rn, rlt_replay_buffer rb) {
+__device__ __forceinline__ void env_epilogue_one(const rlt_env_runner& rn, const rlt_replay_buffer& rb, int e) {
     const EnvDims d = env_dims(rn.env_kind);
     const int OBS = d.obs, ACT = d.act, R = 2 * OBS + ACT + 3;
-    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) {
-        const float reward = rn.rewards[e];
-        const bool terminated = rn.terminated[e] != 0;
-        const uint32_t step = rn.episode_step[e] + 1;
-        rn.episode_step[e] = step;
-        rn.episode_return[e] += reward;
-        const bool truncated = terminated || step == (uint32_t)rn.episode_step_limit;
-        rn.truncated[e] = truncated;
-        uint32_t pos = rb.position[e];
-        float* row = rb.data + ((size_t)e * rb.capacity + pos) * R;
-        for (int i = 0; i < OBS; i++) row[i] = rn.observations[(size_t)e * OBS + i];
-        for (int i = 0; i < ACT; i++) row[OBS + i] = rn.actions[(size_t)e * ACT + i];
-        row[OBS + ACT] = reward;
-        for (int i = 0; i < OBS; i++) row[OBS + ACT + 1 + i] = rn.next_observations[(size_t)e * OBS + i];
-        row[R - 2] = terminated ? 1.0f : 0.0f; row[R - 1] = truncated ? 1.0f : 0.0f;
-        rb.episode_start[(size_t)e * rb.capacity + pos] = rb.current_episode_start[e];
-        pos = (pos + 1) % (uint32_t)rb.capacity;
-        rb.position[e] = pos;
-        if (truncated) rb.current_episode_start[e] = pos;
-        if (pos == 0 && !rb.full[e]) rb.full[e] = 1;
+    const float reward = rn.rewards[e];
+    const bool terminated = rn.terminated[e] != 0;
+    const uint32_t step = rn.episode_step[e] + 1;
+    rn.episode_step[e] = step;
+    rn.episode_return[e] += reward;
+    const bool truncated = terminated || step == (uint32_t)rn.episode_step_limit;
+    rn.truncated[e] = truncated;
+    uint32_t pos = rb.position[e];
+    float* row = rb.data + ((size_t)e * rb.capacity + pos) * R;
+    for (int i = 0; i < OBS; i++) row[i] = rn.observations[(size_t)e * OBS + i];
+    for (int i = 0; i < ACT; i++) row[OBS + i] = rn.actions[(size_t)e * ACT + i];
+    row[OBS + ACT] = reward;
+    for (int i = 0; i < OBS; i++) row[OBS + ACT + 1 + i] = rn.next_observations[(size_t)e * OBS + i];
+    row[R - 2] = terminated ? 1.0f : 0.0f; row[R - 1] = truncated ? 1.0f : 0.0f;
+    rb.episode_start[(size_t)e * rb.capacity + pos] = rb.current_episode_start[e];
+    pos = (pos + 1) % (uint32_t)rb.capacity;
+    rb.position[e] = pos;
+    if (truncated) rb.current_episode_start[e] = pos;
+    if (pos == 0 && !rb.full[e]) rb.full[e] = 1;
+}
+__global__ __launch_bounds__(256) void env_epilogue_kernel(rlt_env_runner rn, rlt_replay_buffer rb) {
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < rn.n_envs; e += gridDim.x * blockDim.x) env_epilogue_one(rn, rb, e);
+}
+// one environment's own step, whatever its kind
+__device__ __forceinline__ void env_step_one(const rlt_env_runner& rn, float* __restrict__ next_observations, int e) {
+    switch (rn.env_kind) {
+        case RLT_ENV_PENDULUM: {
+            Transition t;
+            pendulum_transition(rn.pendulum, rn.states[2 * (size_t)e], rn.states[2 * (size_t)e + 1], rn.actions[e], t);
+            if (next_observations) for (int i = 0; i < 3; i++) next_observations[3 * (size_t)e + i] = t.next_obs[i];
+            rn.rewards[e] = t.reward; rn.terminated[e] = 0;
+            rn.states[2 * (size_t)e] = t.theta; rn.states[2 * (size_t)e + 1] = t.theta_dot;
+            break;
+        }
+        case RLT_ENV_PENDULUM_POSITION: pendulum_position_step_one(rn.pendulum, rn.states, rn.actions, next_observations, rn.rewards, rn.terminated, e); break;
+        case RLT_ENV_CAR: car_step_one(rn.car, rn.states, rn.actions, nullptr, next_observations, rn.rewards, rn.terminated, e); break;
+        default: acrobot_step_one(rn.acrobot, rn.env_kind == RLT_ENV_ACROBOT_SWINGUP, rn.states, rn.actions, nullptr, next_observations, rn.rewards, rn.terminated, e);
+    }
+}
+
+// ---- The runner's whole step in ONE launch for a handful of environments and a policy of dense layers (rl/components/off_policy_runner/operations_generic.h:183-238 over
+// operations_generic_per_env.h:8-108): reset and observe, the policy's layers, its head, the environment's step, counters and the replay add. One workgroup of sixteen
+// wavefronts: a wavefront forms an output unit's dot products for all environments at once (lanes across the input width, the weights' row read coalesced, the sums
+// folded across the lanes), the activations of a layer wait in LDS for the next. For the loops that step one or a few environments per training step, where the
+// launches of the separate kernels (nine of them) are the whole cost.
+__device__ __forceinline__ float mul_add_twice_rounded(float a, float b, float c) {
+#pragma clang fp contract(off)
+    const float product = a * b;
+    return product + c;
+}
+constexpr int FUSED_MAX_ENVS = 16, FUSED_MAX_WIDTH = 256, FUSED_MAX_LAYERS = 8, FUSED_THREADS = 1024;
+struct FusedLayer { const float* weights; const float* biases; int in_dim, out_dim, activation; };
+struct EnvFusedArgs {
+    rlt_env_runner rn; rlt_replay_buffer rb;
+    FusedLayer L[FUSED_MAX_LAYERS]; int n_layers;
+    int head_kind;              // 0: the actions are given (no policy); 1: the policy's output is the action; 2: sample_and_squash; 3: clamp(output + std * noise, -1, 1)
+    rlt_sas_parameters sas; float noise_std;
+    const float* noise;         // [n_envs x action_dim] standard normal draws (head kinds 2 and 3) or the caller's actions (head kind 0)
+    const float* initial_states;
+    // the kernel's own draws where both arrays are NULL: element e * action_dim + c of the noise stream (standard normal for head kinds 2 and 3; for head kind 0 the
+    // action itself, uniform in (-1, 1)), and for an environment that starts an episode state component i = low[i] + (high[i] - low[i]) * element e * state_dim + i
+    // of the initial-state stream (rng.h: the elements rlt_rocm_randn_f32 / rlt_rocm_rand_f32 would write)
+    int draw; uint64_t seed, noise_stream, initial_stream; const uint64_t* stream_offset;
+    float initial_low[8], initial_high[8];
+    float* drawn_noise;         // optional: the noise (or uniform actions) drawn
+};
+__global__ __launch_bounds__(FUSED_THREADS) void env_runner_fused_kernel(EnvFusedArgs A) {
+    __shared__ float act[2][FUSED_MAX_ENVS][FUSED_MAX_WIDTH + 1];
+    const int N = A.rn.n_envs, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const EnvDims d = env_dims(A.rn.env_kind);
+    __shared__ float drawn[FUSED_MAX_ENVS][8];      // this step's initial states, then its noise, where the kernel draws them
+    if (tid < N) {
+        const float* initial = A.initial_states ? A.initial_states + (size_t)tid * d.state : nullptr;
+        if (A.draw) {
+            const uint64_t stream = A.initial_stream + *A.stream_offset;
+            if (A.rn.truncated[tid])
+                for (int i = 0; i < d.state; i++) drawn[tid][i] = A.initial_low[i] + (A.initial_high[i] - A.initial_low[i]) * rlt_rand_element(A.seed, stream, (uint64_t)tid * d.state + i);
+            initial = &drawn[tid][0];
+        }
+        env_prologue_one(A.rn, A.rb, initial, tid);
+        for (int i = 0; i < d.obs; i++) act[0][tid][i] = A.rn.observations[(size_t)tid * d.obs + i];
+        if (A.draw) {
+            const uint64_t stream = A.noise_stream + *A.stream_offset;
+            for (int c = 0; c < d.act; c++) {
+                const uint64_t i = (uint64_t)tid * d.act + c;
+                const float v = A.head_kind == 0 ? -1.0f + 2.0f * rlt_rand_element(A.seed, stream, i) : rlt_randn_element(A.seed, stream, i);
+                drawn[tid][c] = v;
+                if (A.drawn_noise) A.drawn_noise[i] = v;
+            }
+        }
+    }
+    __syncthreads();
+    int cur = 0;
+    for (int l = 0; l < A.n_layers; l++) {
+        const FusedLayer& L = A.L[l];
+        for (int o = wave; o < L.out_dim; o += FUSED_THREADS / 64) {
+            float w[FUSED_MAX_WIDTH / 64];
+#pragma unroll
+            for (int j = 0; j < FUSED_MAX_WIDTH / 64; j++) w[j] = lane + 64 * j < L.in_dim ? L.weights[(size_t)o * L.in_dim + lane + 64 * j] : 0.f;
+            const float bias = L.biases[o];
+            for (int r = 0; r < N; r++) {
+                float s = 0.f;
+#pragma unroll
+                for (int j = 0; j < FUSED_MAX_WIDTH / 64; j++) s += lane + 64 * j < L.in_dim ? w[j] * act[cur][r][lane + 64 * j] : 0.f;
+                s = rlt_wave_sum(s);
+                if (lane == 0) act[cur ^ 1][r][o] = rlt_act(s + bias, L.activation);
+            }
+        }
+        __syncthreads();
+        cur ^= 1;
+    }
+    if (tid < N) {
+        const int e = tid;
+        const float* noise_row = A.draw ? &drawn[e][0] : (A.noise ? A.noise + (size_t)e * d.act : nullptr);
+        if (A.head_kind == 0) { for (int c = 0; c < d.act; c++) A.rn.actions[(size_t)e * d.act + c] = noise_row[c]; }      // the caller's actions, or uniform draws
+        else if (A.head_kind == 1) { for (int c = 0; c < d.act; c++) A.rn.actions[(size_t)e * d.act + c] = act[cur][e][c]; }
+        else if (A.head_kind == 2) {       // nn/layers/sample_and_squash/operations_generic.h:149-195 in rollout mode
+            for (int c = 0; c < d.act; c++) {
+                const float mean = act[cur][e][c];
+                const float log_std = fminf(fmaxf(act[cur][e][d.act + c], A.sas.log_std_lower_bound), A.sas.log_std_upper_bound);
+                A.rn.actions[(size_t)e * d.act + c] = tanhf(mean + noise_row[c] * expf(log_std));
+            }
+        } else if (A.head_kind == 3) {     // nn/layers/td3_sampling/operations_generic.h:75-128
+            for (int c = 0; c < d.act; c++) {
+                const float sample = mul_add_twice_rounded(noise_row[c], A.noise_std, act[cur][e][c]);
+                A.rn.actions[(size_t)e * d.act + c] = sample < -1.0f ? -1.0f : (sample > 1.0f ? 1.0f : sample);
+            }
+        }
+        env_step_one(A.rn, A.rn.next_observations, e);
+        env_epilogue_one(A.rn, A.rb, e);
     }
 }
 __global__ __launch_bounds__(256) void env_copy_kernel(const float* __restrict__ src, float* __restrict__ dst, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
 }
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+}  // namespace
+
+namespace {
+// the one-launch step where it applies: a few environments, dense layers of moderate width (or no policy at all); false: the caller takes the separate kernels
+struct EnvDraws { uint64_t seed, noise_stream, initial_stream; const float* low; const float* high; float* drawn_noise; };
+bool env_runner_fused(rlt_rocm_device* device, const rlt_env_runner* rn, const rlt_replay_buffer* rb, const rlt_dense_layer* const* layers, int n_layers, int head_kind,
+                      const rlt_sas_parameters* sas, float noise_std, const float* noise, const float* initial_states, int* rc, const EnvDraws* draws = nullptr) {
+    if (rn->n_envs > FUSED_MAX_ENVS || n_layers > FUSED_MAX_LAYERS) return false;
+    const EnvDims d = env_dims(rn->env_kind);
+    if (n_layers > 0 && (layers[0]->in_dim != d.obs || layers[n_layers - 1]->out_dim != (head_kind == 2 ? 2 : 1) * d.act)) return false;      // the separate kernels report it
+    EnvFusedArgs A = {};
+    for (int l = 0; l < n_layers; l++) {
+        const rlt_dense_layer& L = *layers[l];
+        if (L.in_dim < 1 || L.out_dim < 1 || L.in_dim > FUSED_MAX_WIDTH || L.out_dim > FUSED_MAX_WIDTH || !L.weights || !L.biases || (l > 0 && L.in_dim != layers[l - 1]->out_dim)) return false;
+        A.L[l] = FusedLayer{L.weights, L.biases, L.in_dim, L.out_dim, L.activation};
+    }
+    A.rn = *rn; A.rb = *rb; A.n_layers = n_layers; A.head_kind = head_kind; A.noise_std = noise_std; A.noise = noise; A.initial_states = initial_states;
+    if (sas) A.sas = *sas;
+    if (draws) {
+        A.draw = 1; A.seed = draws->seed; A.noise_stream = draws->noise_stream; A.initial_stream = draws->initial_stream; A.stream_offset = (const uint64_t*)device->stream_offset;
+        for (int i = 0; i < d.state && i < 8; i++) { A.initial_low[i] = draws->low[i]; A.initial_high[i] = draws->high[i]; }
+        A.drawn_noise = draws->drawn_noise;
+    }
+    hipLaunchKernelGGL(env_runner_fused_kernel, dim3(1), dim3(FUSED_THREADS), 0, device->stream, A);
+    *rc = rlt_launch_status(device);
+    return true;
+}
 }  // namespace
 
 extern "C" int rlt_rocm_env_dims(int env_kind, int* state_dim, int* observation_dim, int* action_dim) {
@@ -296,6 +447,13 @@ extern "C" int rlt_rocm_env_runner_step(rlt_rocm_device* device, const rlt_env_r
     RLT_REQUIRE(policy_kind == 0 || (actor && n_actor_layers >= 1 && actor[0].in_dim == d.obs && actor[n_actor_layers - 1].out_dim == (policy_kind == 2 ? 2 : 1) * d.act));
     RLT_REQUIRE(policy_kind != 2 || (sas && action_noise));
     RLT_REQUIRE(policy_kind == 0 || (workspace && workspace_bytes >= rlt_rocm_env_runner_step_workspace_bytes(rn, policy_kind, actor, n_actor_layers)));
+    {
+        const rlt_dense_layer* list[FUSED_MAX_LAYERS];
+        const int n_list = policy_kind == 0 ? 0 : n_actor_layers;
+        for (int l = 0; l < n_list && l < FUSED_MAX_LAYERS; l++) list[l] = actor + l;
+        int frc = 0;
+        if (env_runner_fused(device, rn, rb, list, n_list, policy_kind, sas, 0.0f, policy_kind == 0 ? actions_in : action_noise, initial_states, &frc)) return frc;
+    }
     const int N = rn->n_envs;
     const int blocks = rlt_div_up(N, 256) > 1024 ? 1024 : rlt_div_up(N, 256);
     int rc;
@@ -330,13 +488,30 @@ extern "C" int rlt_rocm_env_runner_step(rlt_rocm_device* device, const rlt_env_r
     return rlt_launch_status(device);
 }
 
+extern "C" int rlt_rocm_env_runner_step_drawn(rlt_rocm_device* device, const rlt_env_runner* rn, const rlt_replay_buffer* rb, const rlt_seq_layer* policy, int n_policy_layers,
+                                              int head_kind, const rlt_sas_parameters* sas, float exploration_noise_std, const float* initial_low, const float* initial_high,
+                                              float* drawn_noise, uint64_t seed, uint64_t noise_stream, uint64_t initial_state_stream) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(rn && rb && rn->n_envs > 0 && rn->states && rn->episode_step && rn->episode_return && rn->truncated && initial_low && initial_high);
+    RLT_REQUIRE(rn->observations && rn->actions && rn->next_observations && rn->rewards && rn->terminated);
+    RLT_REQUIRE(rb->data && rb->episode_start && rb->position && rb->current_episode_start && rb->full && rb->capacity > 0);
+    const EnvDims d = env_dims(rn->env_kind);
+    RLT_REQUIRE(d.state && d.state <= 8 && rn->n_envs == rb->n_envs && rb->observation_dim == d.obs && rb->action_dim == d.act && head_kind >= 0 && head_kind <= 3);
+    RLT_REQUIRE((head_kind == 0) == (n_policy_layers == 0) && n_policy_layers >= 0 && n_policy_layers <= RLT_SEQ_MAX_LAYERS && (n_policy_layers == 0 || policy) && (head_kind != 2 || sas));
+    const rlt_dense_layer* list[RLT_SEQ_MAX_LAYERS];
+    for (int l = 0; l < n_policy_layers; l++) {
+        if (policy[l].kind != 0) return RLT_E_UNSUPPORTED;
+        list[l] = &policy[l].dense;
+    }
+    if (n_policy_layers > 0) RLT_REQUIRE(list[0]->in_dim == d.obs && list[n_policy_layers - 1]->out_dim == (head_kind == 2 ? 2 : 1) * d.act);
+    const EnvDraws draws = {seed, noise_stream, initial_state_stream, initial_low, initial_high, drawn_noise};
+    int rc = 0;
+    if (!env_runner_fused(device, rn, rb, list, n_policy_layers, head_kind, sas, exploration_noise_std, nullptr, nullptr, &rc, &draws)) return RLT_E_UNSUPPORTED;
+    return rc;
+}
+
 // ---- on-policy collection over any of these environments (rl/components/on_policy_runner/operations_generic_per_env.h:8-74)
 namespace {
-__device__ __forceinline__ float mul_add_twice_rounded(float a, float b, float c) {
-#pragma clang fp contract(off)
-    const float product = a * b;
-    return product + c;
-}
 __device__ __forceinline__ void observe_any(int kind, const float* __restrict__ state, float* __restrict__ o) {
     if (kind == RLT_ENV_PENDULUM) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; o[2] = state[1]; }
     else if (kind == RLT_ENV_PENDULUM_POSITION) { float sn, cs; sincosf(state[0], &sn, &cs); o[0] = cs; o[1] = sn; }
@@ -479,6 +654,12 @@ extern "C" int rlt_rocm_env_runner_step_sequential(rlt_rocm_device* device, cons
     for (int l = 0; l < n_policy_layers; l++) recurrent = recurrent || policy[l].kind != 0;
     RLT_REQUIRE(!recurrent || policy_state);
     RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_env_runner_step_sequential_workspace_bytes(rn, policy, n_policy_layers));
+    if (!recurrent) {
+        const rlt_dense_layer* list[RLT_SEQ_MAX_LAYERS];
+        for (int l = 0; l < n_policy_layers; l++) list[l] = &policy[l].dense;
+        int frc = 0;
+        if (env_runner_fused(device, rn, rb, list, n_policy_layers, head_kind, sas, exploration_noise_std, action_noise, initial_states, &frc)) return frc;
+    }
     const int N = rn->n_envs, blocks = rlt_div_up(N, 256) > 1024 ? 1024 : rlt_div_up(N, 256);
     float* policy_out = reinterpret_cast<float*>(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
     float* log_probabilities = policy_out + (size_t)N * 2 * d.act;

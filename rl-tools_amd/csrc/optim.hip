@@ -100,13 +100,18 @@ __device__ __forceinline__ void adam_body(const AdamLaunch& a, uint32_t block, u
         for (int k = 1; k < MAX_T; k++) ti += (k < a.n && i >= a.prefix[k]) ? 1 : 0;
         const rlt_adam_tensor& T = a.t[ti];
         const uint32_t j = i - a.prefix[ti];
+        // the element's moments, value and target travel together with its gradient (or the blocks that add up to it)
+        float m = T.first_moment[j], v = T.second_moment[j], param = T.parameters[j];
+        const float target = T.polyak_target ? T.polyak_target[j] : 0.f;
         float g;
         if (a.source) {
             g = rlt_scaled_sum(sum_of_blocks(a.source + a.source_offset[ti] + j, a.groups, a.block_stride), a.source_scale[ti], a.source_add[ti]);
             T.gradient[j] = g;
         } else g = T.gradient[j];
         sq += g * g;
-        rlt_adam_apply(a.p, T, j, g, bc1, bc2, a.polyak);
+        rlt_adam_values(a.p, T.flags, g, bc1, bc2, m, v, param);
+        T.first_moment[j] = m; T.second_moment[j] = v; T.parameters[j] = param;
+        if (T.polyak_target) T.polyak_target[j] = rlt_polyak_value(a.polyak, target, param);
     }
     if (a.extra_out && block == n_blocks - 1 && threadIdx.x == blockDim.x - 1) *a.extra_out = sum_of_blocks(a.source + a.extra_offset, a.groups, a.block_stride) * a.extra_scale;
     // gradient norm + age increment: the last workgroup to finish has seen every other one read `age`

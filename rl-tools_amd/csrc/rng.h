@@ -46,6 +46,12 @@ RLT_RNG_FN float rlt_u01(uint32_t x) { return ((float)(x >> 8) + 0.5f) * (1.0f /
 RLT_RNG_FN uint32_t rlt_uniform_below(uint32_t x, uint32_t n) { return (uint32_t)(((uint64_t)x * (uint64_t)n) >> 32); }
 
 #ifndef RLT_RNG_HOST
+// Element i of a uniform stream as rlt_rocm_rand_f32 lays it out (word i % 4 of group i / 4), in (0, 1)
+__device__ __forceinline__ float rlt_rand_element(uint64_t seed, uint64_t stream, uint64_t i) {
+    const rlt_u32x4 r = rlt_philox(seed, stream, i >> 2);
+    const uint32_t k = (uint32_t)(i & 3);
+    return rlt_u01(k == 0 ? r.x : k == 1 ? r.y : k == 2 ? r.z : r.w);
+}
 // Element i of a standard-normal stream as rlt_rocm_randn_f32 lays it out: word i % 4 of group i / 4, Box-Muller on the word pairs
 // (0, 1) and (2, 3) -- for kernels that take their noise from the stream directly instead of from an array filled beforehand.
 __device__ __forceinline__ float rlt_randn_element(uint64_t seed, uint64_t stream, uint64_t i) {
