@@ -95,6 +95,21 @@ namespace rl_tools{
             e.rewards = (float*)memory; e.terminated = (uint8_t*)(memory + rewards_bytes);
             float* noise = (float*)(memory + rewards_bytes + terminated_bytes); float* initial = (float*)(memory + rewards_bytes + terminated_bytes + noise_bytes);
             void* workspace = memory + rewards_bytes + terminated_bytes + noise_bytes + initial_bytes;
+            if(N <= 16 && policy_state == nullptr){
+                // few environments and a policy of dense layers: ONE launch that draws its own initial states and noise (the same stream numbers, taken in the
+                // same order, as the draws into arrays below); the library declines (RLT_E_UNSUPPORTED) a policy it cannot hold in one workgroup
+                float low[8], high[8];
+                DESCRIPTION::initial_ranges(low, high);
+                const uint64_t counter = rng.counter;
+                const uint64_t initial_stream = random::next_stream(rng);
+                const uint64_t noise_stream = head_kind == 1 ? 0 : random::next_stream(rng);
+                const int rc = rlt_rocm_env_runner_step_drawn(device.handle, &e, &rb, layers, n_layers, head_kind, sas, noise_std, low, high, noise, rng.seed, noise_stream, initial_stream);
+                if(rc != RLT_E_UNSUPPORTED){
+                    devices::rocm::check(rc, "step(runner, one launch)");
+                    return;
+                }
+                rng.counter = counter;
+            }
             DESCRIPTION::sample_initial_states(device, initial, N, rng);
             if(head_kind == 0){
                 devices::rocm::check(rlt_rocm_rand_f32(device.handle, noise, N * ACT, -1.0f, 1.0f, rng.seed, random::next_stream(rng)), "step(runner, uniform actions)");

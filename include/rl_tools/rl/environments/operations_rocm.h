@@ -36,6 +36,10 @@ namespace rl_tools::rl::environments::rocm{
                 devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_speed, initial + 1, 2, initial + 1, 2, (int)n, 1), "sample_initial_state (Pendulum)");
             }
         }
+        // the same ranges per state component, for the runner step that draws inside its launch
+        static void initial_ranges(float* low, float* high){
+            high[0] = (float)P::initial_state_max_angle; high[1] = (float)P::initial_state_max_speed; low[0] = -high[0]; low[1] = -high[1];
+        }
         // initial_state (rl/environments/pendulum/operations_generic.h:38-41): hanging down, at rest
         static void initial_state(float* host){ host[0] = -math::PI<float>; host[1] = 0; }
     };
@@ -58,6 +62,9 @@ namespace rl_tools::rl::environments::rocm{
             }
             devices::rocm::check(rlt_rocm_fill_f32(device.handle, initial + 2, (int)n, 1, 3, 0.0f), "sample_initial_state (PendulumPosition)");
         }
+        static void initial_ranges(float* low, float* high){
+            high[0] = (float)P::initial_state_max_angle; high[1] = (float)P::initial_state_max_speed; low[0] = -high[0]; low[1] = -high[1]; low[2] = high[2] = 0;
+        }
         // initial_state (operations_generic.h:42-46): hanging down, at rest, no action yet
         static void initial_state(float* host){ host[0] = -math::PI<float>; host[1] = 0; host[2] = 0; }
     };
@@ -79,6 +86,7 @@ namespace rl_tools::rl::environments::rocm{
         static void sample_initial_states(devices::ROCM<DEV_SPEC>& device, float* initial, size_t n, RNG& rng){
             devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, n * 4, -0.1f, 0.1f, rng.seed, random::next_stream(rng)), "sample_initial_state (Acrobot)");
         }
+        static void initial_ranges(float* low, float* high){ for(int i = 0; i < 4; i++){ low[i] = -0.1f; high[i] = 0.1f; } }
         // initial_state (rl/environments/acrobot/operations_generic.h:54-59): hanging down, at rest
         static void initial_state(float* host){ host[0] = host[1] = host[2] = host[3] = 0; }
     };
@@ -94,6 +102,7 @@ namespace rl_tools::rl::environments::rocm{
             devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, n * 4, -math::PI<float>, math::PI<float>, rng.seed, random::next_stream(rng)), "sample_initial_state (AcrobotSwingup)");
             devices::rocm::check(rlt_rocm_fill_f32(device.handle, initial + 2, (int)n, 2, 4, 0.0f), "sample_initial_state (AcrobotSwingup)");
         }
+        static void initial_ranges(float* low, float* high){ low[0] = low[1] = -math::PI<float>; high[0] = high[1] = math::PI<float>; low[2] = low[3] = high[2] = high[3] = 0; }
         static void initial_state(float* host){ host[0] = host[1] = host[2] = host[3] = 0; }
     };
 }

@@ -225,7 +225,7 @@ def test_zoo_configuration_of_the_acrobot_swingup_trains_on_rocm():
     first = float(re.search(r"evaluation 0 step 0 mean_return ([\d.e+-]+)", out.stdout).group(1))
     assert first < -30.0 and float(final.group(2)) >= -25.0
     assert int(final.group(3)) == 125000
-    assert imports(path, "rlt_rocm_env_runner_step_sequential", "rlt_rocm_sac_train_critics_drawn", "rlt_rocm_env_evaluate")      # the calls resolved to the device overloads
+    assert imports(path, "rlt_rocm_env_runner_step_drawn", "rlt_rocm_env_runner_step_sequential", "rlt_rocm_sac_train_critics_drawn", "rlt_rocm_env_evaluate")      # the calls resolved to the device overloads
     assert len(re.findall(r"^evaluation \d+ ", out.stdout, re.M)) == 13
 
 
@@ -245,7 +245,7 @@ def test_td3_on_the_acrobot_swingup_trains_on_rocm():
     first = float(re.search(r"evaluation 0 step 0 mean_return ([\d.e+-]+)", out.stdout).group(1))
     assert first < -100.0 and float(final.group(2)) >= -85.0
     assert int(final.group(3)) == 60000
-    assert imports(path, "rlt_rocm_env_runner_step_sequential", "rlt_rocm_td3_train_critic", "rlt_rocm_env_evaluate")
+    assert imports(path, "rlt_rocm_env_runner_step_drawn", "rlt_rocm_env_runner_step_sequential", "rlt_rocm_td3_train_critic", "rlt_rocm_env_evaluate")
 
 
 @pytest.mark.gpu
