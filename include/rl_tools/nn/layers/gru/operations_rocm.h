@@ -4,6 +4,9 @@
 // sequence is one call of the library (rlt_rocm_gru_forward / rlt_rocm_gru_backward: the input projection of all steps as one matrix
 // product, the recurrence in one launch, the weight gradients as matrix products over all steps).
 //
+// A rollout step (evaluate_step with the State a policy carries from one environment step to the next, and reset of that State) is one call of the library too
+// (rlt_rocm_seq_evaluate_step / rlt_rocm_seq_reset_state on a one-layer description); the generic versions (:87-120, :348-416) loop over the batch rows on the host.
+//
 // malloc / free / init_weights / zero_gradient / update / copy are the generic functions over this backend's container and optimiser
 // overloads. LEARN_INITIAL_HIDDEN_STATE = false (the reference's configuration, nn/layers/gru/layer.h:14-24).
 #pragma once
@@ -93,6 +96,40 @@ namespace rl_tools{
     void backward_input(devices::ROCM<DEV_SPEC>& device, nn::layers::gru::LayerGradient<LAYER_SPEC>& layer, Tensor<D_OUTPUT_SPEC>& d_output, Tensor<D_INPUT_SPEC>& d_input, nn::layers::gru::buffers::Backward<BUFFER_SPEC>& buffers, const Mode<MODE>& mode = Mode<mode::Default<>>{}){
         static_assert(nn::layers::gru::rocm::dense<D_OUTPUT_SPEC>() && nn::layers::gru::rocm::dense<D_INPUT_SPEC>(), "sequences are dense [steps x batch x features] tensors");
         nn::layers::gru::rocm::backward(device, layer, nullptr, d_output._data, d_input._data, get<0>(typename D_INPUT_SPEC::SHAPE{}), get<1>(typename D_INPUT_SPEC::SHAPE{}), false, mode, "backward_input(gru)");
+    }
+    // reset(layer, state)     nn/layers/gru/operations_generic.h:87-120: all rows (Default mode) or the rows of a ResetMask start again from the initial hidden state, step 0
+    template<typename DEV_SPEC, typename SPEC, typename STATE_SPEC, typename RNG, typename MODE = mode::Default<>>
+    void reset(devices::ROCM<DEV_SPEC>& device, const nn::layers::gru::LayerForward<SPEC>& layer, nn::layers::gru::State<STATE_SPEC>& state, RNG&, Mode<MODE> mode = Mode<mode::Default<>>{}){
+        constexpr size_t B = get<0>(typename decltype(state.state)::SPEC::SHAPE{});
+        static_assert(sizeof(typename decltype(state.step)::T) == 4, "the step counters of a GRU state are 32-bit on devices::ROCM");
+        rlt_seq_layer l = {}; l.kind = 1; l.gru = nn::layers::gru::rocm::describe_forward(layer);
+        rlt_seq_state s = {}; s.hidden[0] = state.state._data; s.step[0] = (uint32_t*)state.step._data;
+        const uint8_t* mask = nullptr;
+        if constexpr(mode::is<MODE, mode::sequential::ResetMask>){
+            static_assert(sizeof(typename decltype(mode.mask)::T) == 1 && decltype(mode.mask)::ROWS == 1 && decltype(mode.mask)::COLS == B && decltype(mode.mask)::SPEC::COL_PITCH == 1, "the reset mask is one byte per batch row");
+            mask = (const uint8_t*)mode.mask._data;
+        }
+        else{
+            static_assert(mode::is<MODE, mode::Default>, "reset(gru state): Default mode or a ResetMask");
+        }
+        devices::rocm::check(rlt_rocm_seq_reset_state(device.handle, &l, 1, &s, mask, (int)B), "reset(gru state)");
+    }
+    // evaluate_step           nn/layers/gru/operations_generic.h:348-416: one step of the recurrence on the state's rows; rows that have run SEQUENCE_LENGTH steps start
+    //                         again from the initial hidden state (before the step and after it), unless the mode is NoAutoResetMode
+    template<typename DEV_SPEC, typename LAYER_SPEC, typename INPUT_SPEC, typename STATE_SPEC, typename OUTPUT_SPEC, typename BUFFER_SPEC, typename RNG, typename MODE = mode::Default<>>
+    void evaluate_step(devices::ROCM<DEV_SPEC>& device, const nn::layers::gru::LayerForward<LAYER_SPEC>& layer, const Tensor<INPUT_SPEC>& input, nn::layers::gru::State<STATE_SPEC>& state, Tensor<OUTPUT_SPEC>& output, nn::layers::gru::buffers::Evaluation<BUFFER_SPEC>&, RNG&, const Mode<MODE>& mode = Mode<mode::Default<>>{}){
+        static_assert(length(typename INPUT_SPEC::SHAPE{}) == 2 && length(typename OUTPUT_SPEC::SHAPE{}) == 2, "evaluate_step has no sequence dimension (batch x features)");
+        static_assert(nn::layers::gru::rocm::dense<INPUT_SPEC>() && nn::layers::gru::rocm::dense<OUTPUT_SPEC>());
+        static_assert(sizeof(typename decltype(state.step)::T) == 4, "the step counters of a GRU state are 32-bit on devices::ROCM");
+        constexpr size_t B = get<0>(typename INPUT_SPEC::SHAPE{});
+        static_assert(get<1>(typename INPUT_SPEC::SHAPE{}) == LAYER_SPEC::INPUT_DIM && get<0>(typename OUTPUT_SPEC::SHAPE{}) == B && get<1>(typename OUTPUT_SPEC::SHAPE{}) == LAYER_SPEC::HIDDEN_DIM);
+        rlt_seq_layer l = {}; l.kind = 1; l.gru = nn::layers::gru::rocm::describe_forward(layer);
+        rlt_seq_state s = {}; s.hidden[0] = state.state._data; s.step[0] = (uint32_t*)state.step._data;
+        const int auto_reset_period = mode::is<MODE, nn::layers::gru::NoAutoResetMode> ? 0 : (int)LAYER_SPEC::SEQUENCE_LENGTH;
+        const size_t workspace_bytes = rlt_rocm_seq_evaluate_step_workspace_bytes(&l, 1, (int)B);
+        void* workspace = devices::rocm::scratch(device, workspace_bytes);
+        devices::rocm::check(rlt_rocm_seq_evaluate_step(device.handle, &l, 1, input._data, (int)LAYER_SPEC::INPUT_DIM, &s, auto_reset_period, output._data, (int)LAYER_SPEC::HIDDEN_DIM, (int)B,
+                                                        workspace, workspace_bytes), "evaluate_step(gru)");
     }
 }
 RL_TOOLS_NAMESPACE_WRAPPER_END

@@ -2,11 +2,12 @@
 // operations_generic.h:50-146 with operations_generic_per_env.h:8-74, are host loops over environments and steps; the CPU backend's
 // operations_cpu.h:17-64 spreads the environments over threads; the reference has no CUDA version of this component).
 //
-// This backend ships precompiled kernels, so the runner steps the environment the C ABI's collect has a kernel for: the Pendulum
-// (rl/environments/pendulum), with an actor that is a sequential model of a standardize layer followed by an MLP with a
-// state-independent action standard deviation (the loop's ConfigApproximatorsSequential, rl/algorithms/ppo/loop/core/config.h:51-66).
+// This backend ships precompiled kernels, so the runner steps the environments the C ABI has kernels for (rl/environments/operations_rocm.h describes them:
+// the Pendulum, the PendulumPosition, the Acrobot, the AcrobotSwingup, the Car), with an actor that is a sequential model of a standardize layer followed by an
+// MLP with a state-independent action standard deviation (the loop's ConfigApproximatorsSequential, rl/algorithms/ppo/loop/core/config.h:51-66).
 // One call of collect is STEPS_PER_ENV + 1 launches per stage (reset and observe, the actor, sample and step) on the device; the noise
-// of all steps and the initial states of all possible resets are drawn beforehand, by two launches.
+// of all steps and the initial states of all possible resets are drawn beforehand, by a few launches. The Pendulum takes rlt_rocm_on_policy_collect (its step and
+// the sampling share a launch), the other environments rlt_rocm_env_on_policy_collect.
 //
 // Memory. runner.environments and runner.env_parameters hold structs that only host code reads: host memory (containers of structs
 // are host memory on this backend). runner.states is the kernels' [N_ENVIRONMENTS x 2] float array (angle, angular velocity): device
@@ -16,6 +17,7 @@
 #include <rl_tools/rl/components/on_policy_runner/on_policy_runner.h>
 #include <rl_tools/rl/components/on_policy_runner/operations_generic.h>
 #include <rl_tools/rl/environments/pendulum/pendulum.h>
+#include <rl_tools/rl/environments/operations_rocm.h>
 #include <rl_tools/nn_models/mlp/network.h>
 #include <rl_tools/nn_models/mlp_unconditional_stddev/network.h>
 #include <rl_tools/nn_models/sequential/model.h>
@@ -106,35 +108,61 @@ namespace rl_tools{
 #endif
         using SPEC = typename DATASET_SPEC::SPEC;
         using ENVIRONMENT = typename SPEC::ENVIRONMENT;
-        using P = typename ENVIRONMENT::SPEC::PARAMETERS;
         using DATASET = rl::components::on_policy_runner::Dataset<DATASET_SPEC>;
-        constexpr size_t N = SPEC::N_ENVIRONMENTS, S = DATASET_SPEC::STEPS_PER_ENV, A = ENVIRONMENT::ACTION_DIM;
-        static_assert(P::initial_state_min_angle == -P::initial_state_max_angle && P::initial_state_min_speed == -P::initial_state_max_speed, "initial states are drawn from ranges that are symmetric about zero");
-        static_assert(P::OBSERVATION_NOISE_POSITION == 0 && P::OBSERVATION_NOISE_VELOCITY == 0);
+        using DESCRIPTION = rl::environments::rocm::Description<ENVIRONMENT>;
+        static_assert(DESCRIPTION::SUPPORTED, "the ROCM backend's on-policy runner steps the environments that rl/environments/operations_rocm.h describes");
+        constexpr size_t N = SPEC::N_ENVIRONMENTS, S = DATASET_SPEC::STEPS_PER_ENV, A = ENVIRONMENT::ACTION_DIM, STATE = DESCRIPTION::STATE_DIM;
+        constexpr bool PENDULUM = utils::typing::is_same_v<ENVIRONMENT, rl::environments::Pendulum<typename ENVIRONMENT::SPEC>>;
         static_assert(decltype(dataset.data)::SPEC::COL_PITCH == 1 && decltype(dataset.data)::SPEC::ROW_PITCH == DATASET::DATA_DIM);
-        const rlt_pendulum_runner r = rl::components::on_policy_runner::rocm::pendulum(runner);
+        static_assert(sizeof(typename ENVIRONMENT::State) == STATE * sizeof(float) && sizeof(typename SPEC::TI) == 4 && sizeof(bool) == 1);
+        static_assert(!SPEC::ASYMMETRIC_OBSERVATIONS && SPEC::N_AGENTS_PER_ENV == 1);
         rl::components::on_policy_runner::rocm::ActorDescription d;
         rl::components::on_policy_runner::rocm::describe(actor, d);
         utils::assert_exit(device, d.n_layers > 0 && d.log_std, "collect: the actor is not a [standardize ->] mlp_unconditional_stddev model");
-        // device memory for this call: the noise of every step, the initial state of every possible reset, the library's workspace
-        const size_t workspace_bytes = rlt_rocm_on_policy_collect_workspace_bytes(&r, d.layers, d.n_layers);
-        const size_t noise_bytes = (S * N * A * sizeof(float) + 255) / 256 * 256, initial_bytes = (S * N * 2 * sizeof(float) + 255) / 256 * 256;
-        char* memory = (char*)devices::rocm::scratch(device, noise_bytes + initial_bytes + workspace_bytes);
-        float* noise = (float*)memory; float* initial = (float*)(memory + noise_bytes); void* workspace = memory + noise_bytes + initial_bytes;
-        devices::rocm::check(rlt_rocm_randn_f32(device.handle, noise, S * N * A, rng.seed, random::next_stream(rng)), "collect (noise)");
-        // sample_initial_state (rl/environments/pendulum/operations_generic.h:58-61): uniform in +- the largest angle and speed
-        devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, S * N * 2, -1.0f, 1.0f, rng.seed, random::next_stream(rng)), "collect (initial states)");
-        devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_angle, initial, 2, initial, 2, (int)(S * N), 1), "collect (initial states)");
-        if constexpr(P::initial_state_max_speed != 1){
-            devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, (float)P::initial_state_max_speed, initial + 1, 2, initial + 1, 2, (int)(S * N), 1), "collect (initial states)");
-        }
         rlt_on_policy_dataset columns = {};
         columns.observations = dataset.observations._data; columns.actions_mean = dataset.actions_mean._data; columns.actions = dataset.actions._data;
         columns.action_log_probs = dataset.action_log_probs._data; columns.rewards = dataset.rewards._data; columns.terminated = dataset.terminated._data;
         columns.truncated = dataset.truncated._data; columns.all_reset = dataset.all_reset._data;
         columns.ld = (int32_t)DATASET::DATA_DIM; columns.steps_per_env = (int32_t)S;
-        devices::rocm::check(rlt_rocm_on_policy_collect(device.handle, &r, &columns, d.layers, d.n_layers, d.log_std, d.standardize_mean, d.standardize_precision, noise, initial,
-                                                        SPEC::TRUNCATE_ON_EACH_ITERATION ? 1 : 0, workspace, workspace_bytes), "collect");
+        auto align = [](size_t bytes){ return (bytes + 255) / 256 * 256; };
+        // device memory for this call: the noise of every step, the initial state of every possible reset (sample_initial_state of the environment), the library's workspace
+        const size_t noise_bytes = align(S * N * A * sizeof(float)), initial_bytes = align(S * N * STATE * sizeof(float));
+        if constexpr(PENDULUM){
+            const rlt_pendulum_runner r = rl::components::on_policy_runner::rocm::pendulum(runner);
+            const size_t workspace_bytes = rlt_rocm_on_policy_collect_workspace_bytes(&r, d.layers, d.n_layers);
+            char* memory = (char*)devices::rocm::scratch(device, noise_bytes + initial_bytes + workspace_bytes);
+            float* noise = (float*)memory; float* initial = (float*)(memory + noise_bytes); void* workspace = memory + noise_bytes + initial_bytes;
+            devices::rocm::check(rlt_rocm_randn_f32(device.handle, noise, S * N * A, rng.seed, random::next_stream(rng)), "collect (noise)");
+            DESCRIPTION::sample_initial_states(device, initial, S * N, rng);
+            devices::rocm::check(rlt_rocm_on_policy_collect(device.handle, &r, &columns, d.layers, d.n_layers, d.log_std, d.standardize_mean, d.standardize_precision, noise, initial,
+                                                            SPEC::TRUNCATE_ON_EACH_ITERATION ? 1 : 0, workspace, workspace_bytes), "collect");
+        }
+        else{
+            rlt_env_runner e = {};
+            DESCRIPTION::set_parameters(e);
+            e.n_envs = (int32_t)N; e.episode_step_limit = (int32_t)SPEC::STEP_LIMIT;
+            e.states = (float*)runner.states._data; e.episode_step = (uint32_t*)runner.episode_step._data; e.episode_return = (float*)runner.episode_return._data;
+            e.truncated = (uint8_t*)runner.truncated._data;
+            rlt_seq_layer layers[rl::components::on_policy_runner::rocm::MAX_LAYERS] = {};
+            for(int l = 0; l < d.n_layers; l++){ layers[l].kind = 0; layers[l].dense = d.layers[l]; }
+            // the per-step staging buffers of the library's runner description (observations and next observations are written into the dataset)
+            constexpr size_t OBS = ENVIRONMENT::Observation::DIM;
+            const size_t staging_bytes = align(N * A * sizeof(float)) + align(N * sizeof(float)) + align(N) + 2 * align(N * OBS * sizeof(float));
+            const size_t workspace_bytes = rlt_rocm_env_on_policy_collect_workspace_bytes(&e, layers, d.n_layers);
+            char* memory = (char*)devices::rocm::scratch(device, noise_bytes + initial_bytes + staging_bytes + workspace_bytes);
+            float* noise = (float*)memory; float* initial = (float*)(memory + noise_bytes);
+            char* staging = memory + noise_bytes + initial_bytes;
+            e.actions = (float*)staging; staging += align(N * A * sizeof(float));
+            e.rewards = (float*)staging; staging += align(N * sizeof(float));
+            e.terminated = (uint8_t*)staging; staging += align(N);
+            e.observations = (float*)staging; staging += align(N * OBS * sizeof(float));
+            e.next_observations = (float*)staging; staging += align(N * OBS * sizeof(float));
+            void* workspace = staging;
+            devices::rocm::check(rlt_rocm_randn_f32(device.handle, noise, S * N * A, rng.seed, random::next_stream(rng)), "collect (noise)");
+            DESCRIPTION::sample_initial_states(device, initial, S * N, rng);
+            devices::rocm::check(rlt_rocm_env_on_policy_collect(device.handle, &e, &columns, layers, d.n_layers, nullptr, 0, d.log_std, d.standardize_mean, d.standardize_precision, noise, initial,
+                                                                SPEC::TRUNCATE_ON_EACH_ITERATION ? 1 : 0, workspace, workspace_bytes), "collect");
+        }
         runner.step += SPEC::N_ENVIRONMENTS * DATASET_SPEC::STEPS_PER_ENV;
     }
 }

@@ -4,12 +4,15 @@
 //   rl::environments::PendulumPosition (pendulum.h:117-124: the velocity is hidden from the observation, the state remembers the last action), :62-66
 //   rl::environments::Acrobot         rl/environments/acrobot/acrobot.h,    sample_initial_state operations_generic.h:39-44
 //   rl::environments::AcrobotSwingup  (the same dynamics, another reward),  sample_initial_state operations_generic.h:46-52
-// The parameters of these environments are static members of ENVIRONMENT::SPEC::PARAMETERS, so a description needs the type only. The Car keeps its
-// parameters in the environment object (rl/environments/car/car.h) and has kernels (rlt_rocm_car_step) but no description here yet.
+//   rl::environments::Car             rl/environments/car/car.h (the variant without a track), sample_initial_state operations_generic.h:70-78
+// The parameters of the first four are static members of ENVIRONMENT::SPEC::PARAMETERS. The Car's are the member initialisers of its Parameters struct
+// (car.h:19-33; initial_parameters leaves them as they are, operations_generic.h:52-54), so a value-initialised Parameters object holds them: a description needs
+// the type only here too. CarTrack (a track bitmap in the environment object) has a kernel (rlt_rocm_car_track_step) and no description.
 #pragma once
 #include <rl_tools/devices/rocm.h>
 #include <rl_tools/rl/environments/pendulum/pendulum.h>
 #include <rl_tools/rl/environments/acrobot/acrobot.h>
+#include <rl_tools/rl/environments/car/car.h>
 RL_TOOLS_NAMESPACE_WRAPPER_START
 namespace rl_tools::rl::environments::rocm{
     template <typename ENVIRONMENT>
@@ -104,6 +107,30 @@ namespace rl_tools::rl::environments::rocm{
         }
         static void initial_ranges(float* low, float* high){ low[0] = low[1] = -math::PI<float>; high[0] = high[1] = math::PI<float>; low[2] = low[3] = high[2] = high[3] = 0; }
         static void initial_state(float* host){ host[0] = host[1] = host[2] = host[3] = 0; }
+    };
+    template <typename SPEC>
+    struct Description<rl::environments::Car<SPEC>>{
+        static constexpr bool SUPPORTED = true;
+        static constexpr int KIND = RLT_ENV_CAR;
+        static constexpr size_t STATE_DIM = 6;      // x, y, mu, vx, vy, omega
+        static rlt_car_parameters parameters(){
+            const typename SPEC::PARAMETERS p{};
+            return rlt_car_parameters{(float)p.g, (float)p.m, (float)p.I, (float)p.lf, (float)p.lr, (float)p.tf.B, (float)p.tf.C, (float)p.tf.D, (float)p.tr.B, (float)p.tr.C, (float)p.tr.D,
+                                      (float)p.cm, (float)p.cr0, (float)p.cr2, (float)p.vt, (float)p.dt};
+        }
+        static void set_parameters(rlt_env_runner& runner){ runner.env_kind = KIND; runner.car = parameters(); }
+        // position uniform in +- 0.2, heading uniform over the circle, at rest
+        static void initial_ranges(float* low, float* high){
+            low[0] = low[1] = -0.2f; high[0] = high[1] = 0.2f; low[2] = -math::PI<float>; high[2] = math::PI<float>; low[3] = low[4] = low[5] = high[3] = high[4] = high[5] = 0;
+        }
+        template <typename DEV_SPEC, typename RNG>
+        static void sample_initial_states(devices::ROCM<DEV_SPEC>& device, float* initial, size_t n, RNG& rng){
+            devices::rocm::check(rlt_rocm_rand_f32(device.handle, initial, n * 6, -0.2f, 0.2f, rng.seed, random::next_stream(rng)), "sample_initial_state (Car)");
+            devices::rocm::check(rlt_rocm_unary_f32(device.handle, RLT_UNARY_SCALE, math::PI<float> / 0.2f, initial + 2, 6, initial + 2, 6, (int)n, 1), "sample_initial_state (Car)");
+            devices::rocm::check(rlt_rocm_fill_f32(device.handle, initial + 3, (int)n, 3, 6, 0.0f), "sample_initial_state (Car)");
+        }
+        // initial_state (rl/environments/car/operations_generic.h:61-69): at the origin, at rest
+        static void initial_state(float* host){ for(int i = 0; i < 6; i++){ host[i] = 0; } }
     };
 }
 RL_TOOLS_NAMESPACE_WRAPPER_END

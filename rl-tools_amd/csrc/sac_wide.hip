@@ -96,7 +96,12 @@ __device__ unsigned long long rlt_wide_ticks[2][32];
 // LDS, then its units' share of the output layer's reduction into yp[wave]. Three workgroup barriers, which every wavefront meets; after
 // the last one output_tile() returns the output layer's sums (without the bias).
 template <int ACT_H, int NT1C>
-__device__ __forceinline__ void forward3(const WNet& N, lptr x, int xstride, lptr h1, lptr h2, lptr yp, int wave, int c, int g) {
+__device__ __forceinline__ void forward3(const WNet& N, lptr x, int xstride, lptr h1, lptr h2, lptr yp, int wave, int c, int g, int tick = -1) {
+#ifdef RLT_WIDE_PROFILE
+#define FT(i) do { if (tick >= 0 && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) rlt_wide_ticks[0][tick + i] = wall_clock64(); } while (0)
+#else
+#define FT(i) do {} while (0)
+#endif
     const int HID = N.hid, n = 16 * wave + c, tiles = (HID + 15) >> 4;
     const bool on = wave < tiles, n_ok = n < HID;
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -116,22 +121,30 @@ __device__ __forceinline__ void forward3(const WNet& N, lptr x, int xstride, lpt
             else { if (k < HID) w3[0] = row[k]; if (k + 1 < HID) w3[1] = row[k + 1]; if (k + 2 < HID) w3[2] = row[k + 2]; if (k + 3 < HID) w3[3] = row[k + 3]; }
         }
         floatx4 a0 = zero4, a1 = zero4;
+        FT(0);
         chunks<NT1C>(a0, a1, x, xstride, c, g, 0, (N.in + 15) >> 4, w1);
+        FT(1);
         const floatx4 acc = a0 + a1;
 #pragma unroll
         for (int v = 0; v < 4; v++) h1[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + b1, N.act_h) : 0.f;
         if (NT1C > 2) load_rows<8>(N.W2, HID, HID, N.vec2, n, g, 8, w2b);
     }
+    FT(2);
     rlt_lds_barrier();
+    FT(3);
     if (on) {
         floatx4 a0 = zero4, a1 = zero4;
         chunks<8>(a0, a1, h1, S, c, g, 0, tiles, w2a);
+        FT(4);
         chunks<8>(a0, a1, h1, S, c, g, 8, tiles, w2b);
+        FT(5);
         const floatx4 acc = a0 + a1;
 #pragma unroll
         for (int v = 0; v < 4; v++) h2[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + b2, N.act_h) : 0.f;
     }
+    FT(6);
     rlt_lds_barrier();
+    FT(7);
     if (on) {
         const floatx4 a = *(lptr4)(h2 + c * S + 16 * wave + 4 * g);
         floatx4 y = zero4;
@@ -284,7 +297,7 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
 #pragma unroll
         for (int k = 0; k < 2; k++) {
             const WNet T = k ? A.target[1] : A.target[0];
-            forward3<ACT_H, NT1C>(T, xa, SXS, ta, tb, yp, wave, c, g);
+            forward3<ACT_H, NT1C>(T, xa, SXS, ta, tb, yp, wave, c, g, k == 0 && CRITIC ? 20 : -1);
             RLT_TICK(4 + k);
             if (scalar_wave) { q_next[k] = output_tile(yp, (T.hid + 15) >> 4, c, g); const float b3 = T.b3[0]; for (int v = 0; v < 4; v++) q_next[k][v] += b3; }
         }

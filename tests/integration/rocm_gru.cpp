@@ -2,7 +2,9 @@
 // rl/algorithms/sac/loop/core/approximators_gru.h:9-75) on devices::ROCM next to the same model on the CPU device: identical weights
 // (initialised on the CPU, copied over), identical inputs and output gradients, with and without per-step resets; forward, backward_full
 // and an Adam step on both, compared on the host. Exit code 0 if outputs, input gradients, parameter gradients and updated parameters
-// agree to 1e-4 relative to their largest magnitude.
+// agree to 1e-4 relative to their largest magnitude. Then a rollout: evaluate_step of the model with the state a policy carries between environment steps
+// (nn_models/sequential/operations_generic.h:303-327), for more steps than the sequence length so that rows restart by themselves, with a reset of some rows through
+// a ResetMask on the way; every step's output next to the CPU device's.
 #include <rl_tools/operations/cpu_mux.h>
 #include <rl_tools/operations/rocm.h>
 #include <rl_tools/nn/optimizers/adam/instance/operations_generic.h>
@@ -113,6 +115,39 @@ int main(){
         rlt::Mode<rlt::nn::layers::gru::ResetMode<rlt::mode::Default<>, rlt::nn::layers::gru::ResetModeSpecification<TI, decltype(reset_dev)>>> mode_dev;
         mode_cpu.reset_container = reset_cpu; mode_dev.reset_container = reset_dev;
         run(mode_cpu, mode_dev, "with per-step resets");
+    }
+    {
+        MODEL::State<> state_cpu, state_dev;
+        rlt::malloc(cpu, state_cpu); rlt::malloc(device, state_dev);
+        rlt::Mode<rlt::mode::Evaluation<>> mode;
+        rlt::reset(cpu, model_cpu, state_cpu, rng_cpu);
+        rlt::reset(device, model_dev, state_dev, rng);
+        rlt::Tensor<rlt::tensor::Specification<T, TI, rlt::tensor::Shape<TI, BATCH_SIZE, INPUT_DIM>>> step_input_cpu, step_input_dev;
+        rlt::Tensor<rlt::tensor::Specification<T, TI, rlt::tensor::Shape<TI, BATCH_SIZE, OUTPUT_DIM>>> step_output_cpu, step_output_dev, step_output_back;
+        rlt::Matrix<rlt::matrix::Specification<bool, TI, 1, BATCH_SIZE>> mask_cpu, mask_dev;
+        rlt::malloc(cpu, step_input_cpu); rlt::malloc(device, step_input_dev); rlt::malloc(cpu, step_output_cpu); rlt::malloc(device, step_output_dev); rlt::malloc(cpu, step_output_back);
+        rlt::malloc(cpu, mask_cpu); rlt::malloc(device, mask_dev);
+        T e_rollout = 0;
+        for(TI step = 0; step < 2 * SEQUENCE_LENGTH + 5; step++){
+            if(step == 9){      // some environments start a new episode: their rows of the state start again
+                for(TI sample = 0; sample < BATCH_SIZE; sample++){ rlt::set(mask_cpu, 0, sample, sample % 3 == 1); }
+                rlt::copy(cpu, device, mask_cpu, mask_dev);
+                rlt::Mode<rlt::mode::sequential::ResetMask<rlt::mode::Default<>, rlt::mode::sequential::ResetMaskSpecification<decltype(mask_cpu)>>> reset_cpu_mode;
+                rlt::Mode<rlt::mode::sequential::ResetMask<rlt::mode::Default<>, rlt::mode::sequential::ResetMaskSpecification<decltype(mask_dev)>>> reset_dev_mode;
+                reset_cpu_mode.mask = mask_cpu; reset_dev_mode.mask = mask_dev;
+                rlt::reset(cpu, model_cpu, state_cpu, rng_cpu, reset_cpu_mode);
+                rlt::reset(device, model_dev, state_dev, rng, reset_dev_mode);
+            }
+            rlt::randn(cpu, step_input_cpu, rng_cpu);
+            rlt::copy(cpu, device, step_input_cpu, step_input_dev);
+            rlt::evaluate_step(cpu, model_cpu, step_input_cpu, state_cpu, step_output_cpu, buffer_cpu, rng_cpu, mode);
+            rlt::evaluate_step(device, model_dev, step_input_dev, state_dev, step_output_dev, buffer_dev, rng, mode);
+            rlt::copy(device, cpu, step_output_dev, step_output_back);
+            const T e = relative(rlt::abs_diff(cpu, step_output_back, step_output_cpu), (T)(BATCH_SIZE * OUTPUT_DIM), rlt::abs_max(cpu, step_output_cpu));
+            e_rollout = (std::isnan(e) || e > e_rollout) ? (std::isnan(e) ? 1 : e) : e_rollout;
+        }
+        std::printf("rollout of %u steps (evaluate_step): worst mean |difference| / largest magnitude of a step's output %.2e\n", (unsigned)(2 * SEQUENCE_LENGTH + 5), e_rollout);
+        worst = e_rollout > worst ? e_rollout : worst;
     }
     rlt::check_status(device);
     std::printf("worst %.2e\n", worst);

@@ -4,12 +4,18 @@
 // ROCM includes differ from a CPU program; every operation the loop calls resolves to an overload of this backend. Evaluation runs on
 // the CPU device on a copy of the actor.
 //
+// With -DPPO_ACROBOT_SWINGUP the environment is the AcrobotSwingup (rl/environments/acrobot, EasyParameters): collect then goes through the library's collection for
+// any environment, the rest of the program is the same.
+//
 // Usage: rocm_ppo_pendulum [n_steps [seed]] ; prints "step <n> mean_return <r>" lines and a last line "final <r> ...".
 #include <rl_tools/operations/cpu_mux.h>
 #include <rl_tools/operations/rocm.h>
 #include <rl_tools/nn/optimizers/adam/instance/operations_generic.h>
 #include <rl_tools/nn/operations_cpu_mux.h>
 #include <rl_tools/rl/environments/pendulum/operations_cpu.h>
+#ifdef PPO_ACROBOT_SWINGUP
+#include <rl_tools/rl/environments/acrobot/operations_generic.h>
+#endif
 #include <rl_tools/nn/layers/standardize/operations_generic.h>
 #include <rl_tools/nn_models/mlp/operations_generic.h>
 #include <rl_tools/nn_models/mlp_unconditional_stddev/operations_generic.h>
@@ -39,7 +45,12 @@ using TYPE_POLICY = rlt::numeric_types::Policy<float>;
 using RNG = DEVICE::SPEC::RANDOM::ENGINE<>;
 
 using PENDULUM_SPEC = rlt::rl::environments::pendulum::Specification<float, TI, rlt::rl::environments::pendulum::DefaultParameters<float>>;
+#ifdef PPO_ACROBOT_SWINGUP
+using ACROBOT_SPEC = rlt::rl::environments::acrobot::Specification<float, TI, rlt::rl::environments::acrobot::EasyParameters<float>>;
+using ENVIRONMENT = rlt::rl::environments::AcrobotSwingup<ACROBOT_SPEC>;
+#else
 using ENVIRONMENT = rlt::rl::environments::Pendulum<PENDULUM_SPEC>;
+#endif
 #ifndef NORMALIZE
 #define NORMALIZE true
 #endif

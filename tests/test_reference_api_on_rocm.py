@@ -30,7 +30,7 @@ def test_programs_written_against_the_reference_api_compile_and_link():
     subprocess.run(["make", "-C", HERE, "syntax"], check=True, capture_output=True)
     out = subprocess.run(["make", "-B", "-C", HERE, "all"], capture_output=True, text=True)
     assert out.returncode == 0, out.stderr[-3000:]
-    for name in ("rocm_containers", "rocm_gru", "rocm_td3_sampling", "rocm_sac_gru_pendulum", "rocm_sac_updates", "rocm_sac_gru_updates", "rocm_td3_updates", "rocm_ppo_updates", "rocm_zoo_pendulum_v1_sac", "rocm_zoo_pendulum_v1_td3", "rocm_zoo_pendulum_v1_ppo", "rocm_zoo_acrobot_swingup_v0_sac", "rocm_zoo_pendulum_position_v1_sac", "rocm_td3_acrobot", "rocm_sac_pendulum", "rocm_sac_pendulum_graph", "rocm_sac_pendulum_w256_graph", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
+    for name in ("rocm_containers", "rocm_gru", "rocm_td3_sampling", "rocm_sac_gru_pendulum", "rocm_sac_updates", "rocm_sac_gru_updates", "rocm_td3_updates", "rocm_ppo_updates", "rocm_zoo_pendulum_v1_sac", "rocm_zoo_pendulum_v1_td3", "rocm_zoo_pendulum_v1_ppo", "rocm_zoo_acrobot_swingup_v0_sac", "rocm_zoo_pendulum_position_v1_sac", "rocm_td3_acrobot", "rocm_sac_car", "rocm_ppo_acrobot_swingup", "rocm_sac_pendulum", "rocm_sac_pendulum_graph", "rocm_sac_pendulum_w256_graph", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
         path = os.path.join(BUILD, name)
         assert os.path.exists(path)
         needed = subprocess.run(["readelf", "-d", path], capture_output=True, text=True).stdout
@@ -120,6 +120,40 @@ def test_the_references_ppo_loop_learns_the_pendulum_on_rocm():
 
 
 @pytest.mark.gpu
+def test_the_references_ppo_loop_collects_from_the_acrobot_swingup_on_rocm():
+    """The same PPO program on the AcrobotSwingup (rl/environments/acrobot, EasyParameters): collect (rl/components/on_policy_runner/operations_generic.h:105-146)
+    resolves to the library's collection for any environment. 200 loop steps of 64 environments x 128 steps; measured: mean return of 100 evaluation episodes of 200
+    steps -67 before training, -42 after."""
+    path = os.path.join(BUILD, "rocm_ppo_acrobot_swingup")
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    out = subprocess.run([path, "200", "0"], capture_output=True, text=True, timeout=300)
+    print(out.stdout[-1500:], flush=True)
+    assert out.returncode == 0, out.stderr[-2000:]
+    returns = [float(m) for m in re.findall(r"step \d+ mean_return (-?[\d.]+)", out.stdout)]
+    final = float(re.search(r"final (-?[\d.]+)", out.stdout).group(1))
+    assert returns[0] < -60 and final > -50
+    assert imports(path, "rlt_rocm_env_on_policy_collect", "rlt_rocm_ppo_gae", "rlt_rocm_ppo_train_epoch")
+
+
+@pytest.mark.gpu
+def test_the_references_sac_loop_learns_the_car_on_rocm():
+    """rl/algorithms/sac/loop/core inside the evaluation loop step on the Car without a track (rl/environments/car/operations_generic.h:80-155; a car that stays at the
+    origin collects one unit of reward per step, episodes of 200 steps end early when it leaves the unit square): the runner's step and the evaluations take the Car's
+    description. Measured: mean return of 100 evaluation episodes 49 before training, 146 after 18,000 loop steps."""
+    path = os.path.join(BUILD, "rocm_sac_car")
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    out = subprocess.run([path, "0", "20000"], capture_output=True, text=True, timeout=170)
+    print(out.stdout[-1200:], flush=True)
+    assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
+    final = re.search(r"final ([\d.e+-]+) best ([\d.e+-]+) loop_steps (\d+) seconds ([\d.e+-]+)", out.stdout)
+    first = float(re.search(r"evaluation 0 step 0 mean_return ([\d.e+-]+)", out.stdout).group(1))
+    assert first < 70.0 and float(final.group(2)) >= 110.0 and int(final.group(3)) == 20000
+    assert imports(path, "rlt_rocm_env_runner_step_drawn", "rlt_rocm_sac_train_critics_drawn", "rlt_rocm_env_evaluate")
+
+
+@pytest.mark.gpu
 def test_the_references_td3_loop_learns_the_pendulum_on_rocm():
     """rl/algorithms/td3/loop/core instantiated on devices::ROCM: the runner step with the exploring actor (td3_sampling head), gather_batch,
     target_action_noise, train_critic, train_actor and both target updates resolve to overloads of this backend."""
@@ -162,7 +196,9 @@ def test_the_references_loop_steps_evaluate_on_the_device():
 def test_gru_sequential_model_matches_the_references_cpu_device():
     """A GRU -> dense sequential model of the reference on devices::ROCM next to the same model on the reference's CPU device, in one
     program: forward, backward_full and an Adam step, with and without per-step resets; outputs, input gradients, parameter gradients and
-    updated parameters agree to 1e-4 of their largest magnitude (measured: 7e-8)."""
+    updated parameters agree to 1e-4 of their largest magnitude (measured: 7e-8). Then a rollout of 53 evaluate_step calls on the state a policy carries between
+    environment steps (nn_models/sequential/operations_generic.h:303-327), longer than two sequence lengths so that rows restart by themselves, with a ResetMask reset of
+    some rows on the way: reset and evaluate_step of the GRU layer resolve to the library's calls."""
     path = os.path.join(BUILD, "rocm_gru")
     if not os.path.exists(path):
         pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
@@ -170,6 +206,7 @@ def test_gru_sequential_model_matches_the_references_cpu_device():
     print(out.stdout[-1500:], flush=True)
     assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
     assert float(re.search(r"worst ([\d.e+-]+)", out.stdout).group(1)) <= 1e-4
+    assert "rollout of 53 steps" in out.stdout and imports(path, "rlt_rocm_seq_evaluate_step", "rlt_rocm_seq_reset_state")
 
 
 @pytest.mark.gpu
