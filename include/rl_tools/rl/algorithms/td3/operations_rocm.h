@@ -166,3 +166,4 @@ namespace rl_tools{
     }
 }
 RL_TOOLS_NAMESPACE_WRAPPER_END
+#include <rl_tools/rl/algorithms/td3/operations_rocm_sequence.h>      // the same functions for sequence batches and recurrent networks

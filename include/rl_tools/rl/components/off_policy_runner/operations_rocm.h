@@ -313,9 +313,13 @@ namespace rl_tools{
             // evaluate_step in Rollout mode; GRU layers restart by themselves every SEQUENCE_LENGTH steps of their input shape (nn/layers/gru/operations_generic.h:406-413)
             rocm::RecurrentPolicyDescription d;
             rocm::describe_recurrent(policy, get<POLICY_INDEX>(runner.policy_states).content_state, d);
-            utils::assert_exit(device, !d.unsupported && d.has_head, "step(runner): a recurrent policy is dense and GRU layers followed by sample_and_squash");
+            utils::assert_exit(device, !d.unsupported, "step(runner): a recurrent policy is dense and GRU layers, optionally followed by sample_and_squash");
             constexpr int AUTO_RESET_PERIOD = (int)get<0>(typename POLICY::INPUT_SHAPE{});
-            if constexpr(PENDULUM){
+            if(!d.has_head){
+                // TD3's recurrent actor (rl/algorithms/td3/loop/core/approximators_gru.h:13-40) has no sampling layer: its output is the action
+                rocm::env_step(device, runner, 1, d.layers, d.n_layers, &d.state, AUTO_RESET_PERIOD, nullptr, 0.0f, rng);
+            }
+            else if constexpr(PENDULUM){
                 const rlt_pendulum_runner r = rocm::pendulum(runner);
                 const rlt_replay_buffer rb = rocm::replay(runner);
                 constexpr size_t ACT = ENVIRONMENT::ACTION_DIM;

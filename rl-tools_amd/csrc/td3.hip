@@ -323,7 +323,7 @@ bool td3_sequence_agent_ok(const rlt_td3_sequence_agent* A) {
         !K.next_final_step_mask_base) return false;
     if (seq_last_dim(A->actor, A->n_actor_layers) != A->action_dim || seq_last_dim(A->actor_target, A->n_actor_layers) != A->action_dim) return false;
     for (int k = 0; k < 2; k++) if (seq_last_dim(A->critics[k], A->n_critic_layers) != 1 || seq_last_dim(A->critics_target[k], A->n_critic_layers) != 1) return false;
-    if (!A->actor_input || !A->d_output || !A->target_action_value) return false;
+    if (!A->actor_input || !A->d_output) return false;
     return A->workspace && A->workspace_bytes >= rlt_rocm_td3_sequence_workspace_bytes(A);
 }
 }  // namespace
@@ -343,7 +343,7 @@ size_t rlt_rocm_td3_sequence_workspace_bytes(const rlt_td3_sequence_agent* A) {
 int rlt_rocm_td3_sequence_train_critic(rlt_rocm_device* device, const rlt_td3_sequence_agent* A, int ci) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(td3_sequence_agent_ok(A) && (ci == 0 || ci == 1));
-    RLT_REQUIRE(A->target_next_action_noise && A->next_state_action_value_input && A->next_q[0] && A->next_q[1]);
+    RLT_REQUIRE(A->target_next_action_noise && A->next_state_action_value_input && A->next_q[0] && A->next_q[1] && A->target_action_value);
     const rlt_sequence_batch& K = A->batch;
     const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
     const int first = A->include_first_step_in_targets ? 1 : 0, T = S + first, next_offset = first ? 0 : 1;   // off_policy_runner/operations_generic.h:85-92

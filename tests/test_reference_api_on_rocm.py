@@ -30,7 +30,7 @@ def test_programs_written_against_the_reference_api_compile_and_link():
     subprocess.run(["make", "-C", HERE, "syntax"], check=True, capture_output=True)
     out = subprocess.run(["make", "-B", "-C", HERE, "all"], capture_output=True, text=True)
     assert out.returncode == 0, out.stderr[-3000:]
-    for name in ("rocm_containers", "rocm_gru", "rocm_td3_sampling", "rocm_sac_gru_pendulum", "rocm_sac_updates", "rocm_sac_gru_updates", "rocm_td3_updates", "rocm_ppo_updates", "rocm_zoo_pendulum_v1_sac", "rocm_zoo_pendulum_v1_td3", "rocm_zoo_pendulum_v1_ppo", "rocm_zoo_acrobot_swingup_v0_sac", "rocm_zoo_pendulum_position_v1_sac", "rocm_td3_acrobot", "rocm_sac_car", "rocm_ppo_acrobot_swingup", "rocm_sac_pendulum", "rocm_sac_pendulum_graph", "rocm_sac_pendulum_w256_graph", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
+    for name in ("rocm_containers", "rocm_gru", "rocm_td3_sampling", "rocm_sac_gru_pendulum", "rocm_sac_updates", "rocm_sac_gru_updates", "rocm_td3_updates", "rocm_ppo_updates", "rocm_zoo_pendulum_v1_sac", "rocm_zoo_pendulum_v1_td3", "rocm_zoo_pendulum_v1_ppo", "rocm_zoo_acrobot_swingup_v0_sac", "rocm_zoo_pendulum_position_v1_sac", "rocm_td3_acrobot", "rocm_td3_gru_pendulum", "rocm_td3_gru_updates", "rocm_sac_car", "rocm_ppo_acrobot_swingup", "rocm_sac_pendulum", "rocm_sac_pendulum_graph", "rocm_sac_pendulum_w256_graph", "rocm_sac_pendulum_loop_steps", "rocm_td3_pendulum", "rocm_ppo_pendulum"):
         path = os.path.join(BUILD, name)
         assert os.path.exists(path)
         needed = subprocess.run(["readelf", "-d", path], capture_output=True, text=True).stdout
@@ -134,6 +134,40 @@ def test_the_references_ppo_loop_collects_from_the_acrobot_swingup_on_rocm():
     final = float(re.search(r"final (-?[\d.]+)", out.stdout).group(1))
     assert returns[0] < -60 and final > -50
     assert imports(path, "rlt_rocm_env_on_policy_collect", "rlt_rocm_ppo_gae", "rlt_rocm_ppo_train_epoch")
+
+
+@pytest.mark.gpu
+def test_td3_updates_on_sequence_batches_match_the_references_cpu_device():
+    """The reference itself as the checker for TD3 with the recurrent approximators (rl/algorithms/td3/loop/core/approximators_gru.h: GRU -> GRU -> dense) on sequence
+    batches of 16 steps x 32: its train_critic / update_critic_targets / train_actor / update_actor_target on its CPU device and the same calls on devices::ROCM (which
+    resolve to the library's entry points for sequence batches), from one agent, on the batches the reference's runner gathered and the noise it drew. Ten loop steps'
+    worth of updates; measured: parameters agree to 6e-9 of their largest magnitude, gradients to 5e-7."""
+    path = os.path.join(BUILD, "rocm_td3_gru_updates")
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    out = subprocess.run([path], capture_output=True, text=True, timeout=170)
+    print(out.stdout[-1500:], flush=True)
+    assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
+    worst = re.search(r"worst ([\d.e+-]+) worst_gradient ([\d.e+-]+)", out.stdout)
+    assert float(worst.group(1)) <= 1e-5 and float(worst.group(2)) <= 5e-5
+    assert imports(path, "rlt_rocm_td3_sequence_train_critic", "rlt_rocm_td3_sequence_train_actor", "rlt_rocm_polyak_update_list")
+
+
+@pytest.mark.gpu
+def test_the_references_recurrent_td3_loop_runs_on_rocm():
+    """rl/algorithms/td3/loop/core with ConfigApproximatorsGRU (sequences of 16 steps x 32, four environments) inside the evaluation and timing loop steps on
+    devices::ROCM: the runner steps the recurrent actor whose output is the action (no sampling layer), the updates are the sequence entry points, evaluations run on the
+    device. Measured (seed 0): mean return of 50 evaluation episodes -1,248 before training, -555 at its best within 10,000 loop steps (this actor explores through
+    nothing but its own changes, so the curve is uneven), 2,090 loop steps/s including the evaluations; the reference's CPU device (generic operations, one thread): 413."""
+    path = os.path.join(BUILD, "rocm_td3_gru_pendulum")
+    if not os.path.exists(path):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    out = subprocess.run([path, "8000", "0"], capture_output=True, text=True, timeout=170)
+    print(out.stdout[-1200:], flush=True)
+    assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
+    returns = [float(m) for m in re.findall(r"^step \d+ mean_return (-?[\d.]+)", out.stdout, re.M)]
+    assert len(returns) == 8 and returns[0] < -1100 and max(returns) > -900
+    assert imports(path, "rlt_rocm_env_runner_step_sequential", "rlt_rocm_gather_sequence_batch", "rlt_rocm_td3_sequence_train_critic", "rlt_rocm_td3_sequence_train_actor", "rlt_rocm_pendulum_evaluate_recurrent")
 
 
 @pytest.mark.gpu
