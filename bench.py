@@ -711,6 +711,7 @@ def main():
     ap.add_argument("--pmc-probe", action="store_true", help="for counter runs under rocprofv3 --pmc: three 256 MiB device copies (a kernel of known traffic, to scale the counters by) "
                     "three MLP forward+backward calls, then the environment-pipeline and PPO workloads (their figures discarded)")
     ap.add_argument("--no-graph-replay", action="store_true", help="leave out the replay of a recorded loop step (for runs under rocprofv3, whose kernel tracing does not survive hipGraphLaunch here)")
+    ap.add_argument("--no-mlp-by-batch", action="store_true", help="leave out configuration 1's other two batch sizes (for a kernel trace of the batch named by --mlp-batch alone)")
     ap.add_argument("--sac-per-operation", action="store_true", help="time the one-launch-per-operation SAC path instead of the persistent kernel")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -727,7 +728,7 @@ def main():
         return
     mlp = bench_mlp(helpers, rocm, args.mlp_batch, args.mlp_iters, 3) if args.only in ("all", "mlp") else None
     sac = bench_sac(helpers, rocm, args.steps, args.warmup, per_operation=args.sac_per_operation, phase_profile=args.sac_phase_profile) if args.only in ("all", "sac") else {"steps_per_s": 0.0, "ms_per_step": 0.0}
-    mlp_other = {str(b): bench_mlp(helpers, rocm, b, 100, 10) for b in (256, 4096)} if args.only in ("all", "mlp") else None      # configuration 1's other two batch sizes
+    mlp_other = {str(b): bench_mlp(helpers, rocm, b, 100, 10) for b in (256, 4096)} if args.only in ("all", "mlp") and not args.no_mlp_by_batch else None      # configuration 1's other two batch sizes
     api = bench_sac_api(helpers, rocm, graph_replay=not args.no_graph_replay) if args.only in ("all", "sac", "api") else None
     env = bench_env(helpers, rocm) if args.only in ("all", "env") else None
     ppo = bench_ppo(helpers, rocm) if args.only in ("all", "ppo") else None

@@ -55,7 +55,7 @@ struct Mlp3Args {
     int batch, in, out, act1, act2, act3, n_tiles;
     const float* b1; const float* b2; const float* b3;
     const float* w2f; const float* w2b; const float* w1s; const float* W3;
-    float* partial;      // [workgroups][count]
+    float* partial;      // [workgroups][count rounded up to a multiple of 64]
 };
 
 __device__ __forceinline__ floatx16 mfma32(float a, float b, floatx16 c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
@@ -455,7 +455,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
     // ---- this workgroup's partial gradients: [dW1 | db1 | dW2 | db2 | dW3 | db3]
     const int tid = threadIdx.x, c32 = lane & 31, hi = lane >> 5, r16 = lane & 15, q = lane >> 4;
     const int count = HID * A.in + HID + HID * HID + HID + A.out * HID + A.out;
-    float* P = A.partial + (size_t)blockIdx.x * count;
+    float* P = A.partial + (size_t)blockIdx.x * ((count + 63) & ~63);      // blocks start on 256-byte boundaries: a wavefront's 256-byte load or store touches two 128-byte lines, not three
     float* pW1 = P; float* pb1 = pW1 + HID * A.in; float* pW2 = pb1 + HID; float* pb2 = pW2 + HID * HID; float* pW3 = pb2 + HID; float* pb3 = pW3 + A.out * HID;
 #pragma unroll
     for (int a = 0; a < 2; a++)
@@ -494,6 +494,7 @@ __device__ __forceinline__ float* grad_slot(const GradTargets& T, int e) {
 // gradient[e] += sum over the workgroups' partial values, in workgroup order. A block of 256 threads handles 64 elements; four
 // threads per element each sum a quarter of the workgroups, 16 loads in flight at a time, and are combined in a fixed order.
 __global__ __launch_bounds__(256) void mlp3_reduce_kernel(const float* __restrict__ partial, int groups, int count, GradTargets T) {
+    const size_t stride = (size_t)((count + 63) & ~63);
     __shared__ float part[4][64];
     const int el = threadIdx.x & 63, qtr = threadIdx.x >> 6, e = blockIdx.x * 64 + el;
     const int ec = e < count ? e : count - 1;
@@ -502,7 +503,7 @@ __global__ __launch_bounds__(256) void mlp3_reduce_kernel(const float* __restric
     for (int gb = g0; gb < g1; gb += 16) {
         float v[16];
 #pragma unroll
-        for (int u = 0; u < 16; u++) v[u] = partial[(size_t)min(gb + u, g1 - 1) * count + ec];
+        for (int u = 0; u < 16; u++) v[u] = partial[(size_t)min(gb + u, g1 - 1) * stride + ec];
 #pragma unroll
         for (int u = 0; u < 16; u++) s += (gb + u < g1) ? v[u] : 0.f;
     }
@@ -523,7 +524,7 @@ size_t gradient_count(const rlt_dense_layer* L) { return (size_t)HID * L[0].in_d
 
 size_t rlt_mlp3_fused_workspace_bytes(const rlt_dense_layer* layers, int n_layers, int batch) {
     if (!shape_ok(layers, n_layers) || batch < 1) return 0;
-    return (PREP_FLOATS + (size_t)workgroups_for(batch) * gradient_count(layers)) * sizeof(float) + 256;
+    return (PREP_FLOATS + (size_t)workgroups_for(batch) * ((gradient_count(layers) + 63) & ~(size_t)63)) * sizeof(float) + 256;
 }
 
 namespace {

@@ -92,16 +92,103 @@ __device__ unsigned long long rlt_wide_ticks[2][32];
 #define RLT_TICK(i) do {} while (0)
 #endif
 
+// A wavefront's weight operands of one network: its 16 units' rows of W1 and W2 (the B operands of layers 1 and 2), row c of W3 for its 16 units, its lane's biases
+template <int NT1C>
+struct Operands { floatx4 w1[NT1C], w2a[8], w2b[8], w3; float b1, b2; };
+__device__ __forceinline__ floatx4 load_w3(const WNet& N, int wave, int c, int g) {
+    floatx4 w3 = {0.f, 0.f, 0.f, 0.f};
+    if (c < N.out) {      // row c of W3 (c < out), this wavefront's 16 units
+        const int k = 16 * wave + 4 * g;
+        const float* row = N.W3 + (size_t)c * N.hid;
+        if (N.vec3 && k + 3 < N.hid) w3 = *reinterpret_cast<const floatx4*>(row + k);
+        else { if (k < N.hid) w3[0] = row[k]; if (k + 1 < N.hid) w3[1] = row[k + 1]; if (k + 2 < N.hid) w3[2] = row[k + 2]; if (k + 3 < N.hid) w3[3] = row[k + 3]; }
+    }
+    return w3;
+}
+// everything of network N that forward3 reads from memory, requested at once (few first-layer operands leave room for the whole second layer; otherwise its second
+// half is requested after the first layer has run)
+template <int NT1C>
+__device__ __forceinline__ void load_operands(const WNet& N, int wave, int c, int g, Operands<NT1C>& W) {
+    const int n = 16 * wave + c;
+    if (wave < ((N.hid + 15) >> 4)) {
+        load_rows<NT1C>(N.W1, N.in, N.hid, N.vec1, n, g, 0, W.w1);
+        load_rows<8>(N.W2, N.hid, N.hid, N.vec2, n, g, 0, W.w2a);
+        if (NT1C <= 2) load_rows<8>(N.W2, N.hid, N.hid, N.vec2, n, g, 8, W.w2b);
+        W.b1 = n < N.hid ? N.b1[n] : 0.f; W.b2 = n < N.hid ? N.b2[n] : 0.f;
+        W.w3 = load_w3(N, wave, c, g);
+    }
+}
+
 // The three layers of network N on the workgroup's rows x [16][xstride]: this wavefront's tile of h1 and h2 (after the activation) into
 // LDS, then its units' share of the output layer's reduction into yp[wave]. Three workgroup barriers, which every wavefront meets; after
 // the last one output_tile() returns the output layer's sums (without the bias).
-template <int ACT_H, int NT1C>
-__device__ __forceinline__ void forward3(const WNet& N, lptr x, int xstride, lptr h1, lptr h2, lptr yp, int wave, int c, int g, int tick = -1) {
+// The operands W are in registers (or on their way) when the call starts. With PREFETCH each group of them is requested again for network `next` as soon as this
+// network has used it, so that the next forward3 finds its operands loaded: a wavefront's weights are 16 KB per layer from L2, a compute unit's 256 KB, which
+// took as long as the layers' arithmetic when they were requested at the start of each pass.
+// First layers of more than two chunks fill too many registers for that: then only the second layer's first half (and the small operands) are requested ahead, the
+// first layer's own operands at the start of the pass (W1_READY = false) and the second half after the first layer, as before.
+template <int ACT_H, int NT1C, bool PREFETCH, bool W1_READY>
+__device__ __forceinline__ void forward3(const WNet& N, Operands<NT1C>& W, const WNet& next, lptr x, int xstride, lptr h1, lptr h2, lptr yp, int wave, int c, int g, int tick = -1) {
 #ifdef RLT_WIDE_PROFILE
 #define FT(i) do { if (tick >= 0 && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) rlt_wide_ticks[0][tick + i] = wall_clock64(); } while (0)
 #else
 #define FT(i) do {} while (0)
 #endif
+    const int HID = N.hid, n = 16 * wave + c, tiles = (HID + 15) >> 4;
+    const bool on = wave < tiles, n_ok = n < HID;
+    const int n_next = 16 * wave + c;
+    const bool next_on = PREFETCH && wave < ((next.hid + 15) >> 4);
+    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    if (on) {
+        if (!W1_READY) load_rows<NT1C>(N.W1, N.in, HID, N.vec1, n, g, 0, W.w1);
+        floatx4 a0 = zero4, a1 = zero4;
+        FT(0);
+        chunks<NT1C>(a0, a1, x, xstride, c, g, 0, (N.in + 15) >> 4, W.w1);
+        FT(1);
+        const floatx4 acc = a0 + a1;
+#pragma unroll
+        for (int v = 0; v < 4; v++) h1[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + W.b1, N.act_h) : 0.f;
+        if (NT1C > 2) load_rows<8>(N.W2, HID, HID, N.vec2, n, g, 8, W.w2b);
+    }
+    if (next_on) {
+        if (NT1C <= 2) load_rows<NT1C>(next.W1, next.in, next.hid, next.vec1, n_next, g, 0, W.w1);
+        W.b1 = n_next < next.hid ? next.b1[n_next] : 0.f;
+    }
+    FT(2);
+    rlt_lds_barrier();
+    FT(3);
+    {
+        floatx4 a0 = zero4, a1 = zero4;
+        if (on) chunks<8>(a0, a1, h1, S, c, g, 0, tiles, W.w2a);
+        if (next_on) load_rows<8>(next.W2, next.hid, next.hid, next.vec2, n_next, g, 0, W.w2a);
+        FT(4);
+        if (on) chunks<8>(a0, a1, h1, S, c, g, 8, tiles, W.w2b);
+        if (next_on && NT1C <= 2) load_rows<8>(next.W2, next.hid, next.hid, next.vec2, n_next, g, 8, W.w2b);
+        FT(5);
+        if (on) {
+            const floatx4 acc = a0 + a1;
+#pragma unroll
+            for (int v = 0; v < 4; v++) h2[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + W.b2, N.act_h) : 0.f;
+        }
+        if (next_on) W.b2 = n_next < next.hid ? next.b2[n_next] : 0.f;
+    }
+    FT(6);
+    rlt_lds_barrier();
+    FT(7);
+    if (on) {
+        const floatx4 a = *(lptr4)(h2 + c * S + 16 * wave + 4 * g);
+        floatx4 y = zero4;
+        y = mfma16(a[0], W.w3[0], y); y = mfma16(a[1], W.w3[1], y); y = mfma16(a[2], W.w3[2], y); y = mfma16(a[3], W.w3[3], y);
+#pragma unroll
+        for (int v = 0; v < 4; v++) yp[(wave * ROWS + 4 * g + v) * D3S + c] = y[v];
+    }
+    if (next_on) W.w3 = load_w3(next, wave, c, g);
+    rlt_lds_barrier();
+}
+// The same three layers for a pass that requests its own operands when it starts (the actor update: its passes are separated by the head and the critics' backward
+// passes, which need the registers)
+template <int ACT_H, int NT1C>
+__device__ __forceinline__ void forward3_own_loads(const WNet& N, lptr x, int xstride, lptr h1, lptr h2, lptr yp, int wave, int c, int g) {
     const int HID = N.hid, n = 16 * wave + c, tiles = (HID + 15) >> 4;
     const bool on = wave < tiles, n_ok = n < HID;
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -121,30 +208,22 @@ __device__ __forceinline__ void forward3(const WNet& N, lptr x, int xstride, lpt
             else { if (k < HID) w3[0] = row[k]; if (k + 1 < HID) w3[1] = row[k + 1]; if (k + 2 < HID) w3[2] = row[k + 2]; if (k + 3 < HID) w3[3] = row[k + 3]; }
         }
         floatx4 a0 = zero4, a1 = zero4;
-        FT(0);
         chunks<NT1C>(a0, a1, x, xstride, c, g, 0, (N.in + 15) >> 4, w1);
-        FT(1);
         const floatx4 acc = a0 + a1;
 #pragma unroll
         for (int v = 0; v < 4; v++) h1[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + b1, N.act_h) : 0.f;
         if (NT1C > 2) load_rows<8>(N.W2, HID, HID, N.vec2, n, g, 8, w2b);
     }
-    FT(2);
     rlt_lds_barrier();
-    FT(3);
     if (on) {
         floatx4 a0 = zero4, a1 = zero4;
         chunks<8>(a0, a1, h1, S, c, g, 0, tiles, w2a);
-        FT(4);
         chunks<8>(a0, a1, h1, S, c, g, 8, tiles, w2b);
-        FT(5);
         const floatx4 acc = a0 + a1;
 #pragma unroll
         for (int v = 0; v < 4; v++) h2[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + b2, N.act_h) : 0.f;
     }
-    FT(6);
     rlt_lds_barrier();
-    FT(7);
     if (on) {
         const floatx4 a = *(lptr4)(h2 + c * S + 16 * wave + 4 * g);
         floatx4 y = zero4;
@@ -261,12 +340,15 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
     }
     HeadItem item[2];
     const bool row_ok = row0 + c < B;
+    Operands<NT1C> W;
+    if (CRITIC) load_operands<NT1C>(A.actor, wave, c, g, W);      // on their way while the input tiles are written
     RLT_TICK(0);
     rlt_lds_barrier();      // the input tiles are in place
     RLT_TICK(1);
 
     // the actor (critic update: on the next observations; actor update: on the observations, activations kept for its backward pass)
-    forward3<ACT_H, NT1C>(A.actor, xa, SXS, CRITIC ? ta : h1, CRITIC ? tb : h2, yp, wave, c, g);
+    if (CRITIC) forward3<ACT_H, NT1C, true, true>(A.actor, W, A.target[0], xa, SXS, ta, tb, yp, wave, c, g);
+    else forward3_own_loads<ACT_H, NT1C>(A.actor, xa, SXS, h1, h2, yp, wave, c, g);
     RLT_TICK(2);
     if (scalar_wave) {
         const floatx4 out = output_tile(yp, (A.actor.hid + 15) >> 4, c, g);
@@ -297,11 +379,12 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
 #pragma unroll
         for (int k = 0; k < 2; k++) {
             const WNet T = k ? A.target[1] : A.target[0];
-            forward3<ACT_H, NT1C>(T, xa, SXS, ta, tb, yp, wave, c, g, k == 0 && CRITIC ? 20 : -1);
+            const WNet after = k ? trained : A.target[1];
+            forward3<ACT_H, NT1C, true, NT1C <= 2>(T, W, after, xa, SXS, ta, tb, yp, wave, c, g, k == 0 && CRITIC ? 20 : -1);
             RLT_TICK(4 + k);
             if (scalar_wave) { q_next[k] = output_tile(yp, (T.hid + 15) >> 4, c, g); const float b3 = T.b3[0]; for (int v = 0; v < 4; v++) q_next[k][v] += b3; }
         }
-        forward3<ACT_H, NT1C>(trained, xb, SXS, h1, h2, yp, wave, c, g);
+        forward3<ACT_H, NT1C, false, NT1C <= 2>(trained, W, trained, xb, SXS, h1, h2, yp, wave, c, g);
         RLT_TICK(6);
         if (scalar_wave) {
             // TD target of rows 4 g + v (meaningful in the lanes c == 0, which hold output 0), MSE gradient at the critic's pre-activation:
@@ -333,7 +416,7 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
         for (int k = 0; k < 2; k++) {
             const WNet C = k ? A.critic[1] : A.critic[0];
             const int ctiles = (C.hid + 15) >> 4;
-            forward3<ACT_H, NT1C>(C, xa, SXS, ta, tb, yp, wave, c, g);
+            forward3_own_loads<ACT_H, NT1C>(C, xa, SXS, ta, tb, yp, wave, c, g);
             RLT_TICK(4 + 4 * k);
             if (scalar_wave) {
                 const floatx4 out = output_tile(yp, ctiles, c, g);
