@@ -56,8 +56,10 @@ class HipEvents:
 
 
 # HBM bytes of one mlp_forward_backward call at batch 65,536, from two counter runs (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch,
-# the factors being what the same counters read for a 256 MiB copy): fused kernel 15.4 + 77.7, reduce kernel 106.0 + 0.3, prepare 1.2 + 0.5 MiB
-MLP_CALL_HBM_BYTES = int((15422 + 77676 + 106016 + 281 + 1228 + 544) * 1024)
+# the factors being what the same counters read for a 256 MiB copy): fused kernel 15.0 + 75.8, reduce kernel 70.6 + 0.3, prepare 1.2 + 0.5 MiB
+MLP_CALL_HBM_BYTES = int((15392 + 77617 + 72292 + 281 + 1228 + 544) * 1024)
+# the same for one PPO minibatch update of 8,192 rows: mlp3s_kernel 16.9 + 12.0, adam_pair_kernel 1.3 + 0.3 MiB
+PPO_UPDATE_HBM_BYTES = int((17308 + 12270 + 1355 + 357) * 1024)
 
 
 def checker():
@@ -777,7 +779,7 @@ def main():
         rooflines["acrobot_step_1048576"] = hbm("acrobot_step_kernel", env["acrobot"]["algorithmic_GBps"], 93.6e6, "89 B per environment step")
     if ppo:
         rooflines["ppo_gae_4096x128"] = hbm("gae_kernel", ppo["gae_algorithmic_GBps"], 91.9e6, "24 B per dataset row")
-        rooflines["ppo_minibatch_update_8192"] = mfma("mlp3s_kernel + adam_pair_kernel", ppo["tflops"], None, "106,368 flop per row and epoch (actor 105-64-64-8 and critic 105-64-64-1, forward + backward)")
+        rooflines["ppo_minibatch_update_8192"] = mfma("mlp3s_kernel + adam_pair_kernel", ppo["tflops"], PPO_UPDATE_HBM_BYTES, "106,368 flop per row and epoch (actor 105-64-64-8 and critic 105-64-64-1, forward + backward)")
     if gru:
         for g in gru:
             rooflines["gru_training_step_b%d" % g["batch"]] = mfma("gru_forward_mfma_kernel + gru_backward_mfma_kernel + projections", g["tflops"], None, "forward + backward through time, 64 steps, input 146, hidden 64")
