@@ -35,7 +35,8 @@ constexpr int ROWS = 16, MAX_H = 256, WAVES = MAX_H / 16, THREADS = 64 * WAVES, 
               N_EXTRA = 16, MISC = 64, YP = ROWS * D3S;
 enum { MODE_CRITIC = 0, MODE_ACTOR = 1 };
 
-struct WNet { const float *W1, *b1, *W2, *b2, *W3, *b3; int in, hid, out, act_h, vec1, vec2, vec3; };      // vecN: the rows of WN can be read 16 bytes at a time
+// W2f / W2b: copies of the second layer's weights in the order the wavefronts consume them (wide_prepare_kernel): 16 bytes per lane, a wavefront's load 1 KB in a row
+struct WNet { const float *W1, *b1, *W2, *b2, *W3, *b3; int in, hid, out, act_h, vec1, vec2, vec3; const float *W2f, *W2b; };      // vecN: the rows of WN can be read 16 bytes at a time
 struct WideArgs {
     WNet actor, critic[2], target[2];
     const float* batch_base;               // [2][batch][obs + act]: current rows, then next rows
@@ -68,6 +69,18 @@ __device__ __forceinline__ void load_rows(const float* __restrict__ W, int K, in
             if (vec) v = *reinterpret_cast<const floatx4*>(row + k);      // K is a multiple of 4 here
             else { v[0] = row[k]; if (k + 1 < K) v[1] = row[k + 1]; if (k + 2 < K) v[2] = row[k + 2]; if (k + 3 < K) v[3] = row[k + 3]; }
         }
+        b[j] = v;
+    }
+}
+// The same operands from a copy laid out in consumption order: [wavefront's 16 units][16-deep chunk j][lane][4] -- lane (c, g) finds W[16 w + c][16 j + 4 g ... + 3]
+// (forward copy) or W[16 j + 4 g ... + 3][16 w + c] (backward copy), zero beyond the layer's shape, and a wavefront's load is 1 KB of consecutive addresses. Straight from
+// W a lane's 16 bytes lie a row (1 KB) apart from its neighbour's: 64 lines per load, which the compute unit's address pipeline takes 64 cycles for.
+template <int JN>
+__device__ __forceinline__ void load_swizzled(const float* __restrict__ copy, int tiles, int wave, int lane, int j0, floatx4 (&b)[JN]) {
+#pragma unroll
+    for (int j = 0; j < JN; j++) {
+        floatx4 v = {0.f, 0.f, 0.f, 0.f};
+        if (j0 + j < tiles) v = *reinterpret_cast<const floatx4*>(copy + ((size_t)(wave * tiles + j0 + j) * 64 + lane) * 4);
         b[j] = v;
     }
 }
@@ -112,8 +125,9 @@ __device__ __forceinline__ void load_operands(const WNet& N, int wave, int c, in
     const int n = 16 * wave + c;
     if (wave < ((N.hid + 15) >> 4)) {
         load_rows<NT1C>(N.W1, N.in, N.hid, N.vec1, n, g, 0, W.w1);
-        load_rows<8>(N.W2, N.hid, N.hid, N.vec2, n, g, 0, W.w2a);
-        if (NT1C <= 2) load_rows<8>(N.W2, N.hid, N.hid, N.vec2, n, g, 8, W.w2b);
+        const int tiles = (N.hid + 15) >> 4, lane = c + 16 * g;
+        load_swizzled<8>(N.W2f, tiles, wave, lane, 0, W.w2a);
+        if (NT1C <= 2) load_swizzled<8>(N.W2f, tiles, wave, lane, 8, W.w2b);
         W.b1 = n < N.hid ? N.b1[n] : 0.f; W.b2 = n < N.hid ? N.b2[n] : 0.f;
         W.w3 = load_w3(N, wave, c, g);
     }
@@ -148,7 +162,7 @@ __device__ __forceinline__ void forward3(const WNet& N, Operands<NT1C>& W, const
         const floatx4 acc = a0 + a1;
 #pragma unroll
         for (int v = 0; v < 4; v++) h1[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + W.b1, N.act_h) : 0.f;
-        if (NT1C > 2) load_rows<8>(N.W2, HID, HID, N.vec2, n, g, 8, W.w2b);
+        if (NT1C > 2) load_swizzled<8>(N.W2f, tiles, wave, c + 16 * g, 8, W.w2b);
     }
     if (next_on) {
         if (NT1C <= 2) load_rows<NT1C>(next.W1, next.in, next.hid, next.vec1, n_next, g, 0, W.w1);
@@ -160,10 +174,10 @@ __device__ __forceinline__ void forward3(const WNet& N, Operands<NT1C>& W, const
     {
         floatx4 a0 = zero4, a1 = zero4;
         if (on) chunks<8>(a0, a1, h1, S, c, g, 0, tiles, W.w2a);
-        if (next_on) load_rows<8>(next.W2, next.hid, next.hid, next.vec2, n_next, g, 0, W.w2a);
+        if (next_on) load_swizzled<8>(next.W2f, (next.hid + 15) >> 4, wave, c + 16 * g, 0, W.w2a);
         FT(4);
         if (on) chunks<8>(a0, a1, h1, S, c, g, 8, tiles, W.w2b);
-        if (next_on && NT1C <= 2) load_rows<8>(next.W2, next.hid, next.hid, next.vec2, n_next, g, 8, W.w2b);
+        if (next_on && NT1C <= 2) load_swizzled<8>(next.W2f, (next.hid + 15) >> 4, wave, c + 16 * g, 8, W.w2b);
         FT(5);
         if (on) {
             const floatx4 acc = a0 + a1;
@@ -197,8 +211,8 @@ __device__ __forceinline__ void forward3_own_loads(const WNet& N, lptr x, int xs
     if (on) {
         floatx4 w1[NT1C];
         load_rows<NT1C>(N.W1, N.in, HID, N.vec1, n, g, 0, w1);
-        load_rows<8>(N.W2, HID, HID, N.vec2, n, g, 0, w2a);      // on their way while the first layer runs
-        if (NT1C <= 2) load_rows<8>(N.W2, HID, HID, N.vec2, n, g, 8, w2b);      // few first-layer operands: room for the whole second layer at once
+        load_swizzled<8>(N.W2f, tiles, wave, c + 16 * g, 0, w2a);      // on their way while the first layer runs
+        if (NT1C <= 2) load_swizzled<8>(N.W2f, tiles, wave, c + 16 * g, 8, w2b);      // few first-layer operands: room for the whole second layer at once
         if (n_ok) { b1 = N.b1[n]; b2 = N.b2[n]; }
         // the output layer's operands: row c of W3 (c < out), this wavefront's 16 units
         if (c < N.out) {
@@ -212,7 +226,7 @@ __device__ __forceinline__ void forward3_own_loads(const WNet& N, lptr x, int xs
         const floatx4 acc = a0 + a1;
 #pragma unroll
         for (int v = 0; v < 4; v++) h1[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + b1, N.act_h) : 0.f;
-        if (NT1C > 2) load_rows<8>(N.W2, HID, HID, N.vec2, n, g, 8, w2b);
+        if (NT1C > 2) load_swizzled<8>(N.W2f, tiles, wave, c + 16 * g, 8, w2b);
     }
     rlt_lds_barrier();
     if (on) {
@@ -270,17 +284,10 @@ __device__ __forceinline__ float backward_layer2(const WNet& N, lptr g2, lptr h1
     const bool n_ok = n < HID;
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
     floatx4 a0 = zero4, a1 = zero4;
-    const float* col = N.W2 + (n_ok ? n : 0);
 #pragma unroll 1
     for (int j0 = 0; j0 < tiles; j0 += 4) {
         floatx4 b[4];
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int k = 16 * (j0 + j) + 4 * g + i;
-                b[j][i] = (n_ok && k < HID) ? col[(size_t)k * HID] : 0.f;
-            }
+        load_swizzled<4>(N.W2b, tiles, wave, c + 16 * g, j0, b);      // W2[16 j + 4 g + i][n]
         chunks<4>(a0, a1, g2, S, c, g, j0, tiles, b);
     }
     const floatx4 acc = a0 + a1;
@@ -292,6 +299,27 @@ __device__ __forceinline__ float backward_layer2(const WNet& N, lptr g2, lptr h1
         p1[idx] = dp; sum += dp;
     }
     return sum;
+}
+
+// The copies of the second layers' weights that load_swizzled reads, made anew before every update (the optimisers change the weights between them): thread t of
+// block (x, job) writes the 16 bytes of lane t % 64 of one (wavefront, chunk) pair. Forward copies read 16 consecutive bytes of a row of W2, backward copies four
+// values a row apart (the 16 lanes of a group read 64 consecutive bytes each time).
+constexpr int PREP_JOBS = 8;
+struct PrepArgs { const float* W2[PREP_JOBS]; float* dst[PREP_JOBS]; int hid[PREP_JOBS]; int backward[PREP_JOBS]; };
+__global__ __launch_bounds__(256) void wide_prepare_kernel(PrepArgs P) {
+    const int job = blockIdx.y, HID = P.hid[job], tiles = (HID + 15) >> 4;
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= tiles * tiles * 64) return;
+    const int lane = t & 63, pair = t >> 6, w = pair / tiles, j = pair - w * tiles, c = lane & 15, g = lane >> 4;
+    const int n = 16 * w + c, k = 16 * j + 4 * g;
+    const float* W = P.W2[job];
+    floatx4 v = {0.f, 0.f, 0.f, 0.f};
+    if (n < HID) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (k + i < HID) v[i] = P.backward[job] ? W[(size_t)(k + i) * HID + n] : W[(size_t)n * HID + k + i];
+    }
+    *reinterpret_cast<floatx4*>(P.dst[job] + (size_t)t * 4) = v;
 }
 
 template <int MODE, int ACT_H, int NT1C>
@@ -642,10 +670,38 @@ int launch_wide(rlt_rocm_device* device, WideArgs& a, int groups, const Optimise
     const rlt_dense_layer* trained = opts[0].trained;
     if (!steps_describable(opts, n_opts)) return RLT_E_UNSUPPORTED;
     a.count = partial_count(trained[0].in_dim, trained[0].out_dim, trained[2].out_dim);
+    // the copies of the second layers' weights: forward copies of every network that runs forward, backward copies of those whose second layer is also walked backwards
+    WNet* forward_nets[5]; WNet* backward_nets[3];
+    int n_forward = 0, n_backward = 0;
+    forward_nets[n_forward++] = &a.actor;
+    for (int k = 0; k < 2; k++) forward_nets[n_forward++] = &a.critic[k];
+    if (MODE == MODE_CRITIC) for (int k = 0; k < 2; k++) forward_nets[n_forward++] = &a.target[k];
+    for (int k = 0; k < 2; k++) backward_nets[n_backward++] = &a.critic[k];
+    if (MODE == MODE_ACTOR) backward_nets[n_backward++] = &a.actor;
+    const size_t copy_floats = (size_t)256 * WAVES * WAVES;      // [16 wavefronts][16 chunks][64 lanes][4] at width 256
+    const size_t partial_bytes = ((size_t)n_opts * groups * a.count * sizeof(float) + 255) & ~(size_t)255;
     void* scratch = nullptr;
-    int rc = rlt_scratch(device, (size_t)n_opts * groups * a.count * sizeof(float), &scratch);
+    int rc = rlt_scratch(device, partial_bytes + (size_t)PREP_JOBS * copy_floats * sizeof(float), &scratch);
     if (rc) return rc;
     a.partial = (float*)scratch;
+    {
+        PrepArgs P = {};
+        float* copies = (float*)((char*)scratch + partial_bytes);
+        int jobs = 0, max_tiles = 1;
+        auto job = [&](WNet* net, bool backward) {
+            for (int q = 0; q < jobs; q++)      // networks given twice (one critic trained alone) share a copy
+                if (P.W2[q] == net->W2 && P.backward[q] == (backward ? 1 : 0)) { (backward ? net->W2b : net->W2f) = P.dst[q]; return; }
+            P.W2[jobs] = net->W2; P.dst[jobs] = copies + (size_t)jobs * copy_floats; P.hid[jobs] = net->hid; P.backward[jobs] = backward ? 1 : 0;
+            (backward ? net->W2b : net->W2f) = P.dst[jobs];
+            const int tiles = (net->hid + 15) >> 4;
+            if (tiles > max_tiles) max_tiles = tiles;
+            jobs++;
+        };
+        for (int q = 0; q < n_forward; q++) job(forward_nets[q], false);
+        for (int q = 0; q < n_backward; q++) job(backward_nets[q], true);
+        hipLaunchKernelGGL(wide_prepare_kernel, dim3(rlt_div_up(max_tiles * max_tiles * 64, 256), jobs), dim3(256), 0, device->stream, P);
+        if ((rc = rlt_launch_status(device))) return rc;
+    }
     a.stream_offset = device->stream_offset;
     a.packed = device->update_one_xcd && device->xcd_stride == 8 && n_opts * groups <= 32 ? 1 : 0;
     const size_t lds_bytes = LDS_FLOATS * sizeof(float);
