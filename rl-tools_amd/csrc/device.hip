@@ -13,6 +13,22 @@ int rlt_launch_status(rlt_rocm_device* device) {
     return 0;
 }
 
+bool rlt_side_begin(rlt_rocm_device* device) {
+    if (!device->side_stream || device->capturing || device->side_return) return false;
+    if (hipEventRecord(device->fork_event, device->stream) != hipSuccess || hipStreamWaitEvent(device->side_stream, device->fork_event, 0) != hipSuccess) { (void)hipGetLastError(); return false; }
+    device->side_return = device->stream;
+    device->stream = device->side_stream;
+    return true;
+}
+void rlt_side_end(rlt_rocm_device* device) {
+    if (device->side_return) { device->stream = device->side_return; device->side_return = nullptr; }
+}
+int rlt_side_join(rlt_rocm_device* device) {
+    if (!device->side_stream) return 0;
+    RLT_HIP(hipEventRecord(device->join_event, device->side_stream));
+    RLT_HIP(hipStreamWaitEvent(device->stream, device->join_event, 0));
+    return 0;
+}
 int rlt_scratch(rlt_rocm_device* device, size_t bytes, void** out) {
     if (bytes > device->scratch_bytes) {
         if (device->capturing) return RLT_E_CAPTURING;      // the workspace grows on a warm-up call before the capture
@@ -164,6 +180,12 @@ int rlt_rocm_init(int hip_device_index, rlt_rocm_device** out_device) {
         device->update_one_xcd = !(q && std::strcmp(q, "spread") == 0);
         device->wait_limit = 1u << 20;
     }
+    // a second stream for independent passes; without it (or its events) everything stays on the one stream
+    if (hipStreamCreate(&device->side_stream) != hipSuccess) device->side_stream = nullptr;
+    if (device->side_stream && (hipEventCreateWithFlags(&device->fork_event, hipEventDisableTiming) != hipSuccess || hipEventCreateWithFlags(&device->join_event, hipEventDisableTiming) != hipSuccess)) {
+        (void)hipStreamDestroy(device->side_stream); device->side_stream = nullptr;
+    }
+    (void)hipGetLastError();
     *out_device = device;
     return 0;
 }
@@ -180,6 +202,11 @@ int rlt_rocm_set_wait_limit(rlt_rocm_device* device, unsigned polls) {
 int rlt_rocm_destroy(rlt_rocm_device* device) {
     if (!device) return RLT_E_INVALID_ARGUMENT;
     (void)hipStreamSynchronize(device->own_stream);
+    if (device->side_stream) {
+        (void)hipStreamSynchronize(device->side_stream);
+        (void)hipEventDestroy(device->fork_event); (void)hipEventDestroy(device->join_event);
+        (void)hipStreamDestroy(device->side_stream);
+    }
     if (device->scratch) (void)hipFree(device->scratch);
     if (device->pad_scratch) (void)hipFree(device->pad_scratch);
     if (device->counters) (void)hipFree(device->counters);

@@ -426,12 +426,17 @@ static bool sequence_agent_ok(const rlt_sac_sequence_agent* A) {
     return A->workspace && A->workspace_bytes >= rlt_rocm_sac_sequence_workspace_bytes(A);
 }
 
+// what one pass of any of the agent's networks needs, rounded up so that the second half of a doubled workspace is aligned like the first
+static size_t sequence_pass_workspace_bytes(const rlt_sac_sequence_agent* A, int T, int B) {
+    size_t n = rlt_rocm_seq_workspace_bytes(A->actor, A->n_actor_layers, T, B);
+    n = std::max(n, rlt_rocm_seq_workspace_bytes(A->critics[0], A->n_critic_layers, T, B));
+    n = std::max(n, rlt_rocm_seq_workspace_bytes(A->critics_target[0], A->n_critic_layers, T, B));
+    return (n + 255) & ~(size_t)255;
+}
 size_t rlt_rocm_sac_sequence_workspace_bytes(const rlt_sac_sequence_agent* A) {
     if (!A || !A->actor || !A->critics[0] || !A->critics_target[0]) return 0;
     const int T = A->batch.sequence_length + 1, B = A->batch.batch;
-    size_t n = rlt_rocm_seq_workspace_bytes(A->actor, A->n_actor_layers, T, B);
-    n = std::max(n, rlt_rocm_seq_workspace_bytes(A->critics[0], A->n_critic_layers, T, B));
-    return std::max(n, rlt_rocm_seq_workspace_bytes(A->critics_target[0], A->n_critic_layers, T, B));
+    return 2 * sequence_pass_workspace_bytes(A, T, B);      // two passes may run at the same time (rlt_side_begin), each in its own half
 }
 
 // rl/algorithms/sac/operations_generic.h:243-337 on a sequence batch, one launch per reference operation
@@ -443,9 +448,19 @@ int rlt_rocm_sac_sequence_train_critic(rlt_rocm_device* device, const rlt_sac_se
     const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
     const int first = A->include_first_step_in_targets ? 1 : 0, T = S + first, next_offset = first ? 0 : 1;   // off_policy_runner/operations_generic.h:85-92
     const rlt_seq_layer* critic = A->critics[ci];
-    void* ws = A->workspace; const size_t ws_bytes = A->workspace_bytes;
+    // two halves of the workspace: passes that do not depend on each other run at the same time, one on the handle's side stream -- the trained critic's forward
+    // pass next to the actor's on the next rows, then the second target critic next to the first (each recurrence fills a twentieth of the chip)
+    const size_t ws_bytes = sequence_pass_workspace_bytes(A, S + 1, B);
+    void* ws = A->workspace; void* ws_side = (char*)A->workspace + ws_bytes;
+    const bool overlap = S >= 48;      // short sequences: a pass is shorter than the two events that fork and join a stream cost on the host
     int rc;
     if ((rc = rlt_rocm_seq_zero_gradient(device, critic, A->n_critic_layers))) return rc;                                                  // :263
+    {
+        const bool side = overlap && rlt_side_begin(device);
+        rc = rlt_rocm_seq_forward(device, critic, A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, side ? ws_side : ws, ws_bytes);   // :294
+        rlt_side_end(device);
+        if (rc) return rc;
+    }
     const float* base_next = K.observations_actions_base + (size_t)next_offset * B * D;
     const uint8_t* next_reset = K.next_reset_base + (size_t)next_offset * B;
     const uint8_t* next_final = K.next_final_step_mask_base + (size_t)next_offset * B;
@@ -455,14 +470,17 @@ int rlt_rocm_sac_sequence_train_critic(rlt_rocm_device* device, const rlt_sac_se
                                    A->next_log_probabilities, T * B, ACT))) return rc;
     if ((rc = rlt_rocm_mask_copy(device, base_next + OBS, D, next_actions, D, next_final, 1, T * B, ACT))) return rc;                      // :274-277
     if ((rc = copy2d(device, base_next, D, A->next_state_action_value_input, D, T * B, OBS))) return rc;                                   // :278
-    for (int k = 0; k < 2; k++) {                                                                                                          // :283-284
-        if ((rc = rlt_rocm_seq_forward(device, A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, next_reset, T, B, ws, ws_bytes))) return rc;
-        if ((rc = rlt_rocm_memcpy_d2d(device, A->next_q[k], seq_output(A->critics_target[k], A->n_critic_layers), sizeof(float) * T * B))) return rc;
+    for (int k = 1; k >= 0; k--) {                                                                                                         // :283-284 (target critic 1 on the side stream)
+        const bool side = k == 1 && overlap && rlt_side_begin(device);
+        rc = rlt_rocm_seq_forward(device, A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, next_reset, T, B, side ? ws_side : ws, ws_bytes);
+        if (!rc) rc = rlt_rocm_memcpy_d2d(device, A->next_q[k], seq_output(A->critics_target[k], A->n_critic_layers), sizeof(float) * T * B);
+        rlt_side_end(device);
+        if (rc) return rc;
     }
+    if (overlap && (rc = rlt_side_join(device))) return rc;
     // the value of the step after (offset B where the first step is included), the log-probability at the same index (:144-154)
     if ((rc = rlt_rocm_sac_target_action_values(device, A->next_q[0] + first * B, A->next_q[1] + first * B, K.rewards, K.terminated, A->next_log_probabilities,
                                                A->log_alpha.parameters, A->gamma, 0, A->target_action_value, S * B))) return rc;             // :289
-    if ((rc = rlt_rocm_seq_forward(device, critic, A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, ws, ws_bytes))) return rc;   // :294
     hipLaunchKernelGGL(sac_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, seq_output(critic, A->n_critic_layers), (const float*)A->target_action_value,
                        (const uint8_t*)K.final_step_mask, A->d_output, S * B, 0);                                                          // :298-316
     if ((rc = rlt_launch_status(device))) return rc;
@@ -502,7 +520,9 @@ int rlt_rocm_sac_sequence_train_actor(rlt_rocm_device* device, const rlt_sac_seq
                 A->actor_pre_squashing && A->actor_log_probabilities && A->actor_actions && A->log_alpha.gradient);
     const rlt_sequence_batch& K = A->batch;
     const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT, R = S * B;
-    void* ws = A->workspace; const size_t ws_bytes = A->workspace_bytes;
+    const size_t ws_bytes = sequence_pass_workspace_bytes(A, S + 1, B);
+    void* ws = A->workspace; void* ws_side = (char*)A->workspace + ws_bytes;
+    const bool overlap = S >= 48;      // short sequences: a pass is shorter than the two events that fork and join a stream cost on the host
     int rc;
     if ((rc = rlt_rocm_seq_zero_gradient(device, A->actor, A->n_actor_layers))) return rc;                                                  // :414
     if ((rc = rlt_rocm_fill_f32(device, A->log_alpha.gradient, 1, 1, 1, 0.0f))) return rc;
@@ -515,15 +535,22 @@ int rlt_rocm_sac_sequence_train_actor(rlt_rocm_device* device, const rlt_sac_seq
     if ((rc = copy2d(device, A->actor_actions, ACT, sav_actions, D, R, ACT))) return rc;
     if ((rc = rlt_rocm_mask_copy(device, obs + OBS, D, sav_actions, D, K.final_step_mask, 1, R, ACT))) return rc;                           // :428-430
     if ((rc = copy2d(device, obs, D, A->state_action_value_input, D, R, OBS))) return rc;                                                   // :431
-    for (int k = 0; k < 2; k++)                                                                                                            // :432-433
-        if ((rc = rlt_rocm_seq_forward(device, A->critics[k], A->n_critic_layers, A->state_action_value_input, D, K.reset, S, B, ws, ws_bytes))) return rc;
+    // the gradient at the critics' outputs is a constant per row (:437-453): formed first, so that each critic's forward pass and its gradient towards the input
+    // (:432-433, :458-459) can follow each other on a stream of their own -- critic 1 on the side stream, critic 0 on the main stream
     hipLaunchKernelGGL(sac_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, (const float*)nullptr, (const float*)nullptr, (const uint8_t*)K.final_step_mask,
-                       A->d_output, R, 1);                                                                                                 // :437-453
+                       A->d_output, R, 1);
     if ((rc = rlt_launch_status(device))) return rc;
-    // :458-459: the inner layers of backward_input run without the reset mode (nn_models/sequential/operations_generic.h:399-407); the critics'
-    // output layer has no activation function, so d_output survives the first call unchanged
-    for (int k = 0; k < 2; k++)
-        if ((rc = rlt_rocm_seq_backward(device, A->critics[k], A->n_critic_layers, nullptr, 0, A->d_output, A->d_critic_input[k], K.reset, S, B, 0, 0, ws, ws_bytes))) return rc;
+    // the inner layers of backward_input run without the reset mode (nn_models/sequential/operations_generic.h:399-407); the critics'
+    // output layer has no activation function, so d_output survives the calls unchanged (both read it)
+    for (int k = 1; k >= 0; k--) {
+        const bool side = k == 1 && overlap && rlt_side_begin(device);
+        void* w = side ? ws_side : ws;
+        rc = rlt_rocm_seq_forward(device, A->critics[k], A->n_critic_layers, A->state_action_value_input, D, K.reset, S, B, w, ws_bytes);
+        if (!rc) rc = rlt_rocm_seq_backward(device, A->critics[k], A->n_critic_layers, nullptr, 0, A->d_output, A->d_critic_input[k], K.reset, S, B, 0, 0, w, ws_bytes);
+        rlt_side_end(device);
+        if (rc) return rc;
+    }
+    if (overlap && (rc = rlt_side_join(device))) return rc;
     if ((rc = rlt_rocm_sac_min_value_d_output(device, seq_output(A->critics[0], A->n_critic_layers), seq_output(A->critics[1], A->n_critic_layers), A->d_critic_input[0],
                                              A->d_critic_input[1], D, D, ACT, A->d_actor_output_squashing, ACT, R))) return rc;             // :460
     if ((rc = rlt_rocm_mask_zero(device, A->d_actor_output_squashing, ACT, K.final_step_mask, 1, R, ACT))) return rc;                       // :461-463

@@ -330,13 +330,18 @@ bool td3_sequence_agent_ok(const rlt_td3_sequence_agent* A) {
 
 extern "C" {
 
-size_t rlt_rocm_td3_sequence_workspace_bytes(const rlt_td3_sequence_agent* A) {
-    if (!A || !A->actor || !A->actor_target || !A->critics[0] || !A->critics_target[0]) return 0;
+// what one pass of any of the agent's networks needs, rounded up so that the second half of a doubled workspace is aligned like the first
+static size_t td3_sequence_pass_workspace_bytes(const rlt_td3_sequence_agent* A) {
     const int T = A->batch.sequence_length + 1, B = A->batch.batch;
     size_t n = rlt_rocm_seq_workspace_bytes(A->actor, A->n_actor_layers, T, B);
     n = std::max(n, rlt_rocm_seq_workspace_bytes(A->actor_target, A->n_actor_layers, T, B));
     n = std::max(n, rlt_rocm_seq_workspace_bytes(A->critics[0], A->n_critic_layers, T, B));
-    return std::max(n, rlt_rocm_seq_workspace_bytes(A->critics_target[0], A->n_critic_layers, T, B));
+    n = std::max(n, rlt_rocm_seq_workspace_bytes(A->critics_target[0], A->n_critic_layers, T, B));
+    return (n + 255) & ~(size_t)255;
+}
+size_t rlt_rocm_td3_sequence_workspace_bytes(const rlt_td3_sequence_agent* A) {
+    if (!A || !A->actor || !A->actor_target || !A->critics[0] || !A->critics_target[0]) return 0;
+    return 2 * td3_sequence_pass_workspace_bytes(A);      // two passes may run at the same time (rlt_side_begin), each in its own half
 }
 
 // rl/algorithms/td3/operations_generic.h:170-235 on a sequence batch, one launch per reference operation
@@ -348,9 +353,19 @@ int rlt_rocm_td3_sequence_train_critic(rlt_rocm_device* device, const rlt_td3_se
     const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
     const int first = A->include_first_step_in_targets ? 1 : 0, T = S + first, next_offset = first ? 0 : 1;   // off_policy_runner/operations_generic.h:85-92
     const rlt_seq_layer* critic = A->critics[ci];
-    void* ws = A->workspace; const size_t ws_bytes = A->workspace_bytes;
+    // passes that do not depend on each other run at the same time, one on the handle's side stream, each in its own half of the workspace: the trained critic's
+    // forward pass next to the target actor's, then the second target critic next to the first
+    const size_t ws_bytes = td3_sequence_pass_workspace_bytes(A);
+    void* ws = A->workspace; void* ws_side = (char*)A->workspace + ws_bytes;
+    const bool overlap = S >= 48;      // short sequences: a pass is shorter than the two events that fork and join a stream cost on the host
     int rc;
     if ((rc = rlt_rocm_seq_zero_gradient(device, critic, A->n_critic_layers))) return rc;                                                  // :185
+    {
+        const bool side = overlap && rlt_side_begin(device);
+        rc = rlt_rocm_seq_forward(device, critic, A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, side ? ws_side : ws, ws_bytes);   // :205
+        rlt_side_end(device);
+        if (rc) return rc;
+    }
     const float* base_next = K.observations_actions_base + (size_t)next_offset * B * D;
     const uint8_t* next_reset = K.next_reset_base + (size_t)next_offset * B;
     const uint8_t* next_final = K.next_final_step_mask_base + (size_t)next_offset * B;
@@ -361,11 +376,14 @@ int rlt_rocm_td3_sequence_train_critic(rlt_rocm_device* device, const rlt_td3_se
     if ((rc = rlt_rocm_td3_noisy_next_actions(device, next_actions, D, A->target_next_action_noise, ACT, T * B, ACT))) return rc;          // :192
     if ((rc = rlt_rocm_mask_copy(device, base_next + OBS, D, next_actions, D, next_final, 1, T * B, ACT))) return rc;                      // :193-195
     if ((rc = copy_columns(device, base_next, D, A->next_state_action_value_input, D, T * B, OBS))) return rc;                             // :196
-    for (int k = 0; k < 2; k++) {                                                                                                          // :197-198
-        if ((rc = rlt_rocm_seq_forward(device, A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, next_reset, T, B, ws, ws_bytes))) return rc;
-        if ((rc = rlt_rocm_memcpy_d2d(device, A->next_q[k], seq_last_output(A->critics_target[k], A->n_critic_layers), sizeof(float) * T * B))) return rc;
+    for (int k = 1; k >= 0; k--) {                                                                                                         // :197-198 (target critic 1 on the side stream)
+        const bool side = k == 1 && overlap && rlt_side_begin(device);
+        rc = rlt_rocm_seq_forward(device, A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, next_reset, T, B, side ? ws_side : ws, ws_bytes);
+        if (!rc) rc = rlt_rocm_memcpy_d2d(device, A->next_q[k], seq_last_output(A->critics_target[k], A->n_critic_layers), sizeof(float) * T * B);
+        rlt_side_end(device);
+        if (rc) return rc;
     }
-    if ((rc = rlt_rocm_seq_forward(device, critic, A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, ws, ws_bytes))) return rc;   // :205
+    if (overlap && (rc = rlt_side_join(device))) return rc;
     // :200-227: targets from the value of the step after (offset B where the first step is included), reweighted and masked gradient
     hipLaunchKernelGGL(td3_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, const_cast<float*>(seq_last_output(critic, A->n_critic_layers)),
                        (const float*)(A->next_q[0] + (size_t)first * B), (const float*)(A->next_q[1] + (size_t)first * B), (const float*)K.rewards, (const uint8_t*)K.terminated,
