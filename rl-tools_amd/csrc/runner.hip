@@ -85,15 +85,23 @@ __global__ __launch_bounds__(256) void gather_kernel(rlt_replay_buffer rb, const
     }
 }
 
-// gather_batch_step for sequences (rl/components/off_policy_runner/operations_generic.h:239-418): a lane per sample walks its padded steps through one
+// gather_batch_step for sequences (rl/components/off_policy_runner/operations_generic.h:239-418): a wavefront per sample walks its padded steps through one
 // ring; the draws come from arrays, the k-th use of a kind by sample b being entry [b][k]. Copies and index arithmetic only.
+// The reference's loop is one step after the other because whether a step ends a sequence is read from its own row. Between two ends the rows are consecutive,
+// so the wavefront takes a run of up to 64 steps at once: lane l reads the row of step s + l, the first lane whose step ends the sequence (its row's truncated
+// flag, the ring's cursor, the last padded step, the drawn length) is found by a vote, the lanes up to it write their steps, and the walk goes on behind it -- one
+// trip to memory per run instead of one per step. The bookkeeping between runs is the same on every lane. The four masks are collected in LDS and written once.
+constexpr int GATHER_SEQ_MAX_PADDED = 1024;
 __global__ __launch_bounds__(256) void gather_sequence_kernel(rlt_replay_buffer rb, rlt_sequence_sampling P, rlt_sequence_draws draws, int max_episode_length, rlt_sequence_batch B,
                                                               int* __restrict__ error_flag) {
+    __shared__ uint8_t masks[4][4][GATHER_SEQ_MAX_PADDED];      // per wavefront: final_step, reset, next_final_step, next_reset
     const int OBS = rb.observation_dim, ACT = rb.action_dim, R = 2 * OBS + ACT + 3, D = OBS + ACT, N = B.batch, SEQ = B.sequence_length, PADDED = SEQ + 1;
     const uint32_t CAP = (uint32_t)rb.capacity;
-    for (int b = blockIdx.x * blockDim.x + threadIdx.x; b < N; b += gridDim.x * blockDim.x) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    volatile uint8_t* final_mask = masks[wave][0]; volatile uint8_t* reset_mask = masks[wave][1]; volatile uint8_t* next_final_mask = masks[wave][2]; volatile uint8_t* next_reset_mask = masks[wave][3];
+    for (int b = blockIdx.x * 4 + wave; b < N; b += gridDim.x * 4) {
         const uint32_t e = draws.env_indices[b];
-        if (e >= (uint32_t)rb.n_envs) { *error_flag = 1; continue; }
+        if (e >= (uint32_t)rb.n_envs) { if (lane == 0) *error_flag = 1; continue; }
         const uint32_t position = rb.position[e];
         const bool full = rb.full[e] != 0;
         const uint32_t* offsets = draws.sample_offsets + (size_t)b * PADDED;
@@ -113,51 +121,76 @@ __global__ __launch_bounds__(256) void gather_sequence_kernel(rlt_replay_buffer 
         if (P.random_seq_length) current_seq_length = draw_length();
         int current_seq_step = 0;
         bool previous_step_truncated = false, previous_padding_step = true;
-        for (int s = 0; s < SEQ; s++) { B.final_step_mask[(size_t)s * N + b] = 0; B.reset[(size_t)s * N + b] = 0; }
-        for (int s = 0; s < PADDED; s++) { B.next_final_step_mask_base[(size_t)s * N + b] = 0; B.next_reset_base[(size_t)s * N + b] = 0; }
-        B.reset[b] = 1; B.next_reset_base[b] = 1;
-        B.next_reset_base[(size_t)(P.include_first_step_in_targets ? 0 : 1) * N + b] = 1;
-        for (int s = 0; s < PADDED; s++) {
+        for (int s = lane; s < PADDED; s += 64) { final_mask[s] = 0; reset_mask[s] = 0; next_final_mask[s] = 0; next_reset_mask[s] = 0; }
+        __builtin_amdgcn_wave_barrier();
+        if (lane == 0) { reset_mask[0] = 1; next_reset_mask[0] = 1; next_reset_mask[P.include_first_step_in_targets ? 0 : 1] = 1; }
+        bool failed = false;
+        int s = 0;
+        while (s < PADDED) {
             if (previous_step_truncated) {
                 previous_step_truncated = false; previous_padding_step = true;
-                B.next_final_step_mask_base[(size_t)s * N + b] = 1;
-                if (s < PADDED - 1) B.reset[(size_t)s * N + b] = 1;
+                if (lane == 0) { next_final_mask[s] = 1; if (s < PADDED - 1) reset_mask[s] = 1; }
+                s++;
                 continue;
             }
             if (previous_padding_step) {
-                if (s < PADDED - 1) B.reset[(size_t)s * N + b] = 1;
-                B.next_reset_base[(size_t)s * N + b] = 1;
+                if (lane == 0) { if (s < PADDED - 1) reset_mask[s] = 1; next_reset_mask[s] = 1; }
                 const uint32_t sample_offset = offsets[n_offset++];
                 sample_index = full ? (position + (uint32_t)max_episode_length + sample_offset) % CAP : sample_offset;
                 if (P.always_sample_from_initial_state && sample_index < CAP) sample_index = rb.episode_start[(size_t)e * CAP + sample_index];
             }
-            if (sample_index >= CAP) { *error_flag = 1; break; }
-            const float* row = rb.data + ((size_t)e * CAP + sample_index) * R;
-            float* step = B.observations_actions_base + ((size_t)s * N + b) * D;
-            for (int k = 0; k < D; k++) step[k] = row[k];
-            if (s < PADDED - 1) { B.rewards[(size_t)s * N + b] = row[D]; B.terminated[(size_t)s * N + b] = row[2 * OBS + ACT + 1] != 0.0f; }
+            if (sample_index >= CAP) { failed = true; break; }
+            // the run that starts at step s and row sample_index: lane l takes step s + l and the l-th row behind sample_index
+            const int step = s + lane;
+            const bool in_range = step < PADDED;
+            uint32_t index = sample_index + (uint32_t)lane;
+            if (full) index %= CAP;
+            const bool readable = in_range && index < CAP;
+            const float* row = rb.data + ((size_t)e * CAP + (readable ? index : sample_index)) * R;
             bool truncated = row[2 * OBS + ACT + 2] != 0.0f;
-            uint32_t next_sample_index = sample_index + 1;
-            if (full) next_sample_index %= CAP;
-            if (next_sample_index == position) truncated = true;
-            if (s == PADDED - 2) truncated = true;
-            if (P.random_seq_length) {
-                if (current_seq_step == current_seq_length - 1) {
-                    truncated = true;
-                    current_seq_length = SEQ > 1 ? draw_length() : SEQ;
+            uint32_t next_index = index + 1;
+            if (full) next_index %= CAP;
+            if (next_index == position) truncated = true;
+            if (step == PADDED - 2) truncated = true;
+            const bool length_ends = P.random_seq_length && current_seq_step + lane == current_seq_length - 1;
+            if (length_ends) truncated = true;
+            // a lane past the ring's last written row (not full: index >= CAP) would be an error if the walk reached it; the cursor ends the run before
+            const unsigned long long ends = __ballot(in_range && (truncated || !readable));
+            const int last = ends ? __ffsll((long long)ends) - 1 : min(63, PADDED - 1 - s);      // the run's last lane
+            const bool run_truncated = ends != 0ull;
+            if (lane == last && run_truncated && !readable) failed = true;
+            if (__ballot(failed)) { failed = true; break; }
+            if (lane <= last && in_range) {
+                float* out = B.observations_actions_base + ((size_t)step * N + b) * D;
+                for (int k = 0; k < D; k++) out[k] = row[k];
+                if (step < PADDED - 1) { B.rewards[(size_t)step * N + b] = row[D]; B.terminated[(size_t)step * N + b] = row[2 * OBS + ACT + 1] != 0.0f; }
+                if (lane == last && run_truncated && step < PADDED - 1) {
+                    final_mask[step] = 1;
+                    float* next = B.observations_actions_base + ((size_t)(step + 1) * N + b) * D;
+                    for (int k = 0; k < OBS; k++) next[k] = row[D + 1 + k];
+                    for (int k = 0; k < ACT; k++) next[OBS + k] = 0.0f;
                 }
-                current_seq_step = truncated ? 0 : current_seq_step + 1;
             }
-            if (truncated && s < PADDED - 1) {
-                B.final_step_mask[(size_t)s * N + b] = 1;
-                float* next = B.observations_actions_base + ((size_t)(s + 1) * N + b) * D;
-                for (int k = 0; k < OBS; k++) next[k] = row[D + 1 + k];
-                for (int k = 0; k < ACT; k++) next[OBS + k] = 0.0f;
+            // the bookkeeping behind the run's last step, the same on every lane
+            const bool last_length_ends = P.random_seq_length && current_seq_step + last == current_seq_length - 1;
+            if (P.random_seq_length) {
+                if (last_length_ends) current_seq_length = SEQ > 1 ? draw_length() : SEQ;
+                current_seq_step = run_truncated ? 0 : current_seq_step + last + 1;
             }
-            sample_index = next_sample_index;
+            uint32_t after = sample_index + (uint32_t)last + 1;
+            if (full) after %= CAP;
+            sample_index = after;
             previous_padding_step = false;
-            previous_step_truncated = truncated;
+            previous_step_truncated = run_truncated;
+            s += last + 1;
         }
+        if (failed && lane == 0) *error_flag = 1;
+        __builtin_amdgcn_wave_barrier();
+        for (int t = lane; t < PADDED; t += 64) {
+            if (t < SEQ) { B.final_step_mask[(size_t)t * N + b] = final_mask[t]; B.reset[(size_t)t * N + b] = reset_mask[t]; }
+            B.next_final_step_mask_base[(size_t)t * N + b] = next_final_mask[t]; B.next_reset_base[(size_t)t * N + b] = next_reset_mask[t];
+        }
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
@@ -180,22 +213,21 @@ __global__ __launch_bounds__(256) void gather_sequence_draw_kernel(rlt_replay_bu
                                                                    uint8_t* __restrict__ nominal, uint32_t* __restrict__ lengths, const uint64_t* __restrict__ stream_offset) {
     stream += *stream_offset;
     const int PADDED = sequence_length + 1, WORDS = 3 * PADDED + 3, G = (WORDS + 3) / 4;
-    for (int b = blockIdx.x * blockDim.x + threadIdx.x; b < batch; b += gridDim.x * blockDim.x) {
-        uint32_t env = 0, eligible = 0;
-        for (int g = 0; g < G; g++) {
-            const rlt_u32x4 draw = rlt_philox(seed, stream, (uint64_t)b * G + g);
-            const uint32_t words[4] = {draw.x, draw.y, draw.z, draw.w};
-            for (int i = 0; i < 4; i++) {
-                const int w = 4 * g + i;
-                if (w >= WORDS) break;
-                if (w == 0) {
-                    env = rlt_uniform_below(words[i], (uint32_t)rb.n_envs);
-                    env_indices[b] = env;
-                    eligible = rb.full[env] ? (uint32_t)(P.always_sample_from_initial_state ? rb.capacity - max_episode_length : rb.capacity) : rb.position[env];
-                } else if (w <= PADDED) sample_offsets[(size_t)b * PADDED + (w - 1)] = eligible ? rlt_uniform_below(words[i], eligible) : 0u;
-                else if (w <= 2 * PADDED + 1) nominal[(size_t)b * (PADDED + 1) + (w - PADDED - 1)] = rlt_u01(words[i]) < P.nominal_sequence_length_probability ? 1 : 0;
-                else lengths[(size_t)b * (PADDED + 1) + (w - 2 * PADDED - 2)] = sequence_length > 1 ? 1u + rlt_uniform_below(words[i], (uint32_t)(sequence_length - 1)) : 1u;
-            }
+    // a thread per (sample, group of four words); the offsets need the sample's environment, which is word 0 of its first group
+    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < (size_t)batch * G; t += (size_t)gridDim.x * blockDim.x) {
+        const int b = (int)(t / G), g = (int)(t - (size_t)b * G);
+        const rlt_u32x4 draw = rlt_philox(seed, stream, (uint64_t)b * G + g);
+        const uint32_t first_word = g == 0 ? draw.x : rlt_philox(seed, stream, (uint64_t)b * G).x;
+        const uint32_t env = rlt_uniform_below(first_word, (uint32_t)rb.n_envs);
+        const uint32_t eligible = rb.full[env] ? (uint32_t)(P.always_sample_from_initial_state ? rb.capacity - max_episode_length : rb.capacity) : rb.position[env];
+        const uint32_t words[4] = {draw.x, draw.y, draw.z, draw.w};
+        for (int i = 0; i < 4; i++) {
+            const int w = 4 * g + i;
+            if (w >= WORDS) break;
+            if (w == 0) env_indices[b] = env;
+            else if (w <= PADDED) sample_offsets[(size_t)b * PADDED + (w - 1)] = eligible ? rlt_uniform_below(words[i], eligible) : 0u;
+            else if (w <= 2 * PADDED + 1) nominal[(size_t)b * (PADDED + 1) + (w - PADDED - 1)] = rlt_u01(words[i]) < P.nominal_sequence_length_probability ? 1 : 0;
+            else lengths[(size_t)b * (PADDED + 1) + (w - 2 * PADDED - 2)] = sequence_length > 1 ? 1u + rlt_uniform_below(words[i], (uint32_t)(sequence_length - 1)) : 1u;
         }
     }
 }
@@ -714,8 +746,9 @@ int rlt_rocm_gather_sequence_batch(rlt_rocm_device* device, const rlt_replay_buf
     RLT_REQUIRE(B->observations_actions_base && B->rewards && B->terminated && B->reset && B->next_reset_base && B->final_step_mask && B->next_final_step_mask_base);
     RLT_REQUIRE(draws->env_indices && draws->sample_offsets && (!sampling->random_seq_length || (draws->nominal && draws->lengths)));
     RLT_REQUIRE(!sampling->always_sample_from_initial_state || rb->capacity > max_episode_length);      // otherwise no row is eligible once a ring is full (:259)
+    if (B->sequence_length + 1 > GATHER_SEQ_MAX_PADDED) return RLT_E_UNSUPPORTED;      // the kernel keeps a sample's four masks in LDS
     device->fault_armed = 1;
-    hipLaunchKernelGGL(gather_sequence_kernel, dim3(grid1(B->batch)), dim3(256), 0, device->stream, *rb, *sampling, *draws, max_episode_length, *B, (int*)(device->fault + 1));
+    hipLaunchKernelGGL(gather_sequence_kernel, dim3(grid1((size_t)B->batch * 64)), dim3(256), 0, device->stream, *rb, *sampling, *draws, max_episode_length, *B, (int*)(device->fault + 1));
     return rlt_launch_status(device);
 }
 
@@ -731,7 +764,7 @@ int rlt_rocm_gather_sequence_draw(rlt_rocm_device* device, const rlt_replay_buff
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(rb_ok(rb) && sampling && batch > 0 && sequence_length >= 1 && max_episode_length >= 0 && env_indices && sample_offsets && nominal && lengths);
     RLT_REQUIRE(!sampling->always_sample_from_initial_state || rb->capacity > max_episode_length);
-    hipLaunchKernelGGL(gather_sequence_draw_kernel, dim3(grid1(batch)), dim3(256), 0, device->stream, *rb, *sampling, max_episode_length, batch, sequence_length, seed, stream,
+    hipLaunchKernelGGL(gather_sequence_draw_kernel, dim3(grid1((size_t)batch * ((3 * (sequence_length + 1) + 3 + 3) / 4))), dim3(256), 0, device->stream, *rb, *sampling, max_episode_length, batch, sequence_length, seed, stream,
                        env_indices, sample_offsets, nominal, lengths, (const uint64_t*)device->stream_offset);
     return rlt_launch_status(device);
 }
