@@ -30,6 +30,7 @@ struct AdamLaunch {
     uint32_t source_offset[MAX_T];
     float source_scale[MAX_T], source_add[MAX_T];
     float* extra_out; uint32_t extra_offset; float extra_scale;      // optional: one more sum of the blocks, stored scaled (not a gradient)
+    uint32_t vec_end;            // elements [0, vec_end) can be stepped four at a time (16-byte loads of the blocks, moments and values): see vector_end()
 };
 
 // sum over the blocks of one element, every load in flight at once where there are at most 16 blocks
@@ -93,8 +94,51 @@ __device__ __forceinline__ void adam_body(const AdamLaunch& a, uint32_t block, u
             }
             __syncthreads();
         }
-    } else
-    for (uint32_t i = block * blockDim.x + threadIdx.x; i < total; i += n_blocks * blockDim.x) {
+    } else {
+    // at most 16 blocks, four neighbouring elements per thread: every load is 16 bytes per lane (the same sums in the same order per element)
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    for (uint32_t i = (block * blockDim.x + threadIdx.x) * 4u; i < a.vec_end; i += n_blocks * blockDim.x * 4u) {
+        int ti = 0;
+#pragma unroll
+        for (int k = 1; k < MAX_T; k++) ti += (k < a.n && i >= a.prefix[k]) ? 1 : 0;
+        const rlt_adam_tensor& T = a.t[ti];
+        const uint32_t j = i - a.prefix[ti];
+        f4 m = *reinterpret_cast<const f4*>(T.first_moment + j), v = *reinterpret_cast<const f4*>(T.second_moment + j), param = *reinterpret_cast<const f4*>(T.parameters + j);
+        f4 target = {0.f, 0.f, 0.f, 0.f};
+        if (T.polyak_target) target = *reinterpret_cast<const f4*>(T.polyak_target + j);
+        const float* __restrict__ p = a.source + a.source_offset[ti] + j;
+        const int per = (a.groups + 3) / 4;
+        f4 blk[16];
+#pragma unroll
+        for (int qi = 0; qi < 4; qi++)
+#pragma unroll
+            for (int u = 0; u < 4; u++) blk[4 * qi + u] = *reinterpret_cast<const f4*>(p + (size_t)min(qi * per + u, a.groups - 1) * a.block_stride);
+        __builtin_amdgcn_sched_barrier(0);
+        f4 q[4];
+#pragma unroll
+        for (int qi = 0; qi < 4; qi++) {
+            const int g0 = qi * per, g1 = min(a.groups, g0 + per);
+            f4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < 4; u++) if (u < per && g0 + u < g1) sum += blk[4 * qi + u];
+            q[qi] = sum;
+        }
+        const f4 total4 = (q[0] + q[1]) + (q[2] + q[3]);
+        f4 g;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            g[c] = rlt_scaled_sum(total4[c], a.source_scale[ti], a.source_add[ti]);
+            sq += g[c] * g[c];
+            float mc = m[c], vc = v[c], pc = param[c];
+            rlt_adam_values(a.p, T.flags, g[c], bc1, bc2, mc, vc, pc);
+            m[c] = mc; v[c] = vc; param[c] = pc;
+            if (T.polyak_target) target[c] = rlt_polyak_value(a.polyak, target[c], pc);
+        }
+        *reinterpret_cast<f4*>(T.gradient + j) = g;
+        *reinterpret_cast<f4*>(T.first_moment + j) = m; *reinterpret_cast<f4*>(T.second_moment + j) = v; *reinterpret_cast<f4*>(T.parameters + j) = param;
+        if (T.polyak_target) *reinterpret_cast<f4*>(T.polyak_target + j) = target;
+    }
+    for (uint32_t i = a.vec_end + block * blockDim.x + threadIdx.x; i < total; i += n_blocks * blockDim.x) {
         int ti = 0;
 #pragma unroll
         for (int k = 1; k < MAX_T; k++) ti += (k < a.n && i >= a.prefix[k]) ? 1 : 0;
@@ -112,6 +156,7 @@ __device__ __forceinline__ void adam_body(const AdamLaunch& a, uint32_t block, u
         rlt_adam_values(a.p, T.flags, g, bc1, bc2, m, v, param);
         T.first_moment[j] = m; T.second_moment[j] = v; T.parameters[j] = param;
         if (T.polyak_target) T.polyak_target[j] = rlt_polyak_value(a.polyak, target, param);
+    }
     }
     if (a.extra_out && block == n_blocks - 1 && threadIdx.x == blockDim.x - 1) *a.extra_out = sum_of_blocks(a.source + a.extra_offset, a.groups, a.block_stride) * a.extra_scale;
     // gradient norm + age increment: the last workgroup to finish has seen every other one read `age`
@@ -196,11 +241,33 @@ static int adam_launch(rlt_rocm_device* device, const rlt_adam_tensor* tensors, 
     return 0;
 }
 
+// how far the elements can be stepped four at a time: up to the first tensor whose start, pointers or place in the blocks is not a multiple of 16 bytes, or that
+// ends off one (then its last one to three elements and everything behind them are stepped one by one)
+static uint32_t vector_end(const AdamLaunch& a) {
+    auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    if (!a.source || a.groups > 16 || a.block_stride % 4 != 0 || !aligned(a.source)) return 0;
+    uint32_t end = 0;
+    for (int i = 0; i < a.n; i++) {
+        const rlt_adam_tensor& T = a.t[i];
+        if (a.prefix[i] % 4 != 0 || a.source_offset[i] % 4 != 0 || !aligned(T.parameters) || !aligned(T.gradient) || !aligned(T.first_moment) || !aligned(T.second_moment) ||
+            (T.polyak_target && !aligned(T.polyak_target))) break;
+        end = a.prefix[i] + (T.count & ~3u);
+        if (T.count % 4 != 0) break;
+    }
+    return end;
+}
 static void set_source(AdamLaunch& a, const rlt_adam_source* source) {
     if (!source) return;
     a.source = source->partial; a.groups = source->groups; a.block_stride = source->block_stride;
     for (int i = 0; i < a.n; i++) { a.source_offset[i] = source->offsets[i]; a.source_scale[i] = source->scales[i]; a.source_add[i] = source->adds ? source->adds[i] : 0.0f; }
     a.extra_out = source->extra_out; a.extra_offset = source->extra_offset; a.extra_scale = source->extra_scale;
+    a.vec_end = vector_end(a);
+}
+// workgroups for an optimiser of `total` elements: 64 elements per workgroup pass on the many-block path, 256 threads of four elements each where those apply
+static uint32_t blocks_for(const AdamLaunch& a, uint32_t total, const rlt_adam_source* source) {
+    if (source && source->groups > 16) return (total + 63) / 64;
+    const uint32_t threads = a.vec_end / 4 > total - a.vec_end ? a.vec_end / 4 : total - a.vec_end;
+    return (threads + 255) / 256;
 }
 
 int rlt_adam_step_from_partials(rlt_rocm_device* device, const rlt_adam_tensor* tensors, int n, const rlt_adam_parameters* parameters, uint32_t* age, const rlt_adam_source* source, float polyak) {
@@ -221,8 +288,7 @@ int rlt_adam_step_from_partials(rlt_rocm_device* device, const rlt_adam_tensor* 
     a.done_counter = (uint32_t*)counters; a.block_partials = (float*)((char*)counters + 256);
     a.increment_age = 1;
     set_source(a, source);
-    const uint32_t per_block = source->groups > 16 ? 64 : 256;      // the many-block path takes 64 elements per workgroup pass
-    int blocks = (int)((total + per_block - 1) / per_block); if (blocks > 960) blocks = 960;
+    int blocks = (int)blocks_for(a, total, source); if (blocks > 960) blocks = 960; if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL(adam_kernel, dim3(blocks), dim3(256), 0, device->stream, a);
     return rlt_launch_status(device);
 }
@@ -259,8 +325,7 @@ int rlt_adam_step_pair(rlt_rocm_device* device, const rlt_adam_tensor* tensors_a
         a.increment_age = 1;
         const rlt_adam_source* source = k ? source_b : source_a;
         set_source(a, source);
-        const uint32_t per_block = source && source->groups > 16 ? 64 : 256;
-        blocks[k] = (total + per_block - 1) / per_block; if (blocks[k] > 480) blocks[k] = 480; if (blocks[k] < 1) blocks[k] = 1;
+        blocks[k] = blocks_for(a, total, source); if (blocks[k] > 480) blocks[k] = 480; if (blocks[k] < 1) blocks[k] = 1;
     }
     hipLaunchKernelGGL(adam_pair_kernel, dim3(blocks[0] + blocks[1]), dim3(256), 0, device->stream, L[0], L[1], blocks[0]);
     return rlt_launch_status(device);

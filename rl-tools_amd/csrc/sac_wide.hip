@@ -669,7 +669,8 @@ template <int MODE>
 int launch_wide(rlt_rocm_device* device, WideArgs& a, int groups, const Optimiser* opts, int n_opts, float polyak, bool* targets_done) {
     const rlt_dense_layer* trained = opts[0].trained;
     if (!steps_describable(opts, n_opts)) return RLT_E_UNSUPPORTED;
-    a.count = partial_count(trained[0].in_dim, trained[0].out_dim, trained[2].out_dim);
+    const int exact_count = partial_count(trained[0].in_dim, trained[0].out_dim, trained[2].out_dim);
+    a.count = (exact_count + 63) & ~63;      // blocks start on 256-byte boundaries: the optimisers' launch reads them 16 bytes per lane
     // the copies of the second layers' weights: forward copies of every network that runs forward, backward copies of those whose second layer is also walked backwards
     WNet* forward_nets[5]; WNet* backward_nets[3];
     int n_forward = 0, n_backward = 0;
@@ -732,7 +733,7 @@ int launch_wide(rlt_rocm_device* device, WideArgs& a, int groups, const Optimise
     if (n_opts == 2)
         return rlt_adam_step_pair(device, S[0].tensors, opts[0].n_tensors, opts[0].parameters, opts[0].age, S[1].tensors, opts[1].n_tensors, opts[1].parameters, opts[1].age, &source[0], &source[1], polyak);
     if (opts[0].second) {
-        const uint32_t second_offset = (uint32_t)(a.count - N_EXTRA);
+        const uint32_t second_offset = (uint32_t)(exact_count - N_EXTRA);
         const rlt_adam_source second_source = {a.partial, groups, a.count, &second_offset, &opts[0].second_scale};
         return rlt_adam_step_pair(device, S[0].tensors, opts[0].n_tensors, opts[0].parameters, opts[0].age, opts[0].second, 1, opts[0].second_parameters, opts[0].second_age, &source[0], &second_source);
     }
