@@ -65,4 +65,27 @@ __device__ __forceinline__ void head_backward(const rlt_sas_parameters& sas, con
     if (I.log_std_raw < sas.log_std_lower_bound || I.log_std_raw > sas.log_std_upper_bound) d_ls = 0.0f;
     entropy -= normal_log_prob(I.mean, log_std, sd, I.sample) - logf(1.0f - I.action * I.action + sas.log_probability_epsilon);
 }
+
+// TD3's actor head for the items of a lane: tanh of the MLP's output, the td3_sampling layer (action = clamp(tanh(output) + sampling_std * noise, -1, 1),
+// nn/layers/td3_sampling/operations_generic.h:75-128), and in the critic update the smoothing noise of the target action
+// (rl/algorithms/td3/operations_generic.h:129-145). mean = tanh(output), sample = value before the clamp.
+__device__ __forceinline__ void td3_head_forward(int OBS, int ACT, float sampling_std, lptr d3s, int D3S, lptr xs, int SX, const float (&noise)[2], const float (&target_noise)[2],
+                                                 bool critic_update, int r, int kk, HeadItem (&item)[2]) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int a = kk + 4 * j;
+        HeadItem& I = item[j];
+        I = {0.f, 0.f, 0.f, 0.f, 0.f};
+        if (a < ACT) {
+            I.mean = tanhf(d3s[r * D3S + a]);
+            I.noise = noise[j];
+            float scaled = I.noise * sampling_std;
+            asm volatile("" : "+v"(scaled));        // the product is rounded before the addition, as the per-operation kernels and the reference's CPU build do
+            I.sample = scaled + I.mean;
+            I.action = clampf(I.sample, -1.0f, 1.0f);
+            if (critic_update) I.action = clampf(I.action + target_noise[j], -1.0f, 1.0f);
+            xs[r * SX + OBS + a] = I.action;
+        }
+    }
+}
 }  // namespace rlt_sac

@@ -16,9 +16,9 @@ int rlt_sac_update_critic(rlt_rocm_device* device, const rlt_sac_agent* agent, i
 int rlt_sac_update_actor(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_update_noise& noise);
 // both train_critic calls on the agent's batch with the same noise in ONE launch and, if update_targets, update_critic_targets after them
 int rlt_sac_update_critics(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_update_noise& noise, bool update_targets);
-// The same updates for three-layer networks of any hidden width up to 256 (sac_wide.hip), always with the optimiser as the kernel's own last
-// step: supported only while that is switched on (rlt_rocm_set_update_options) and for batches of at most 512 rows. `first`, `count`: the
-// critics trained by the launch (one of them, or both on the same batch and noise; update_targets only with both).
+// The same updates for three-layer networks of any hidden width up to 256 (sac_wide.hip): a launch that lays the second layers' weights out for the
+// wavefronts, the update kernel, and the optimisers' launch, which adds up the workgroups' blocks of partial sums; batches of at most 2,048 rows, no masks.
+// `first`, `count`: the critics trained by the launch (one of them, or both on the same batch and noise; update_targets only with both).
 bool rlt_sac_wide_supported(const rlt_rocm_device* device, const rlt_sac_agent* agent);
 int rlt_sac_wide_update_critics(rlt_rocm_device* device, const rlt_sac_agent* agent, int first, int count, const rlt_update_noise& noise, bool update_targets);
 int rlt_sac_wide_update_actor(rlt_rocm_device* device, const rlt_sac_agent* agent, const rlt_update_noise& noise);
@@ -30,3 +30,7 @@ int rlt_sac_polyak_list(rlt_rocm_device* device, const float* const* sources, fl
 bool rlt_td3_update_supported(const rlt_rocm_device* device, const rlt_td3_agent* agent);
 int rlt_td3_update_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
 int rlt_td3_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise);
+// and at hidden widths up to 256 (sac_wide.hip)
+bool rlt_td3_wide_supported(const rlt_rocm_device* device, const rlt_td3_agent* agent);
+int rlt_td3_wide_update_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
+int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise);

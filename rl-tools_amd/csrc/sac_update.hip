@@ -231,28 +231,6 @@ __device__ __forceinline__ float backward_layer2(const BackwardRegs& G, int act_
     return sum;
 }
 
-// TD3's actor head for the items of a lane: tanh of the MLP's output, the td3_sampling layer, and in the critic update the smoothing noise
-// of the target action (rl/algorithms/td3/operations_generic.h:129-145). mean = tanh(output), sample = value before the clamp.
-__device__ __forceinline__ void td3_head_forward(const UpdateArgs& A, lptr d3s, lptr xs, int SX, const float (&noise)[2], const float (&target_noise)[2], bool critic_update,
-                                                 int r, int kk, HeadItem (&item)[2]) {
-#pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int a = kk + 4 * j;
-        HeadItem& I = item[j];
-        I = {0.f, 0.f, 0.f, 0.f, 0.f};
-        if (a < A.act) {
-            I.mean = tanhf(d3s[r * D3S + a]);
-            I.noise = noise[j];
-            float scaled = I.noise * A.sampling_std;
-            asm volatile("" : "+v"(scaled));        // the product is rounded before the addition, as the per-operation kernels and the reference's CPU build do
-            I.sample = scaled + I.mean;
-            I.action = clampf(I.sample, -1.0f, 1.0f);
-            if (critic_update) I.action = clampf(I.action + target_noise[j], -1.0f, 1.0f);
-            xs[r * SX + A.obs + a] = I.action;
-        }
-    }
-}
-
 template <int NT1C, int MODE, int ACT_H>
 __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
     constexpr bool CRITIC = MODE == 0 || MODE == MODE_TD3_CRITIC, TD3 = MODE == MODE_TD3_CRITIC || MODE == MODE_TD3_ACTOR;
@@ -361,7 +339,7 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
         for (int v = 0; v < 4; v++) d3s[(4 * kk + v) * D3S + r] = r < A.actor.out ? y[v] + b3_actor : 0.f;
         wave_sync();
         float log_prob = 0.f;
-        if (TD3) td3_head_forward(A, d3s, xsa, SX, noise, target_noise, CRITIC, r, kk, item);
+        if (TD3) td3_head_forward(A.obs, A.act, A.sampling_std, d3s, D3S, xsa, SX, noise, target_noise, CRITIC, r, kk, item);
         else log_prob = head_forward(A.sas, A.obs, A.act, d3s, D3S, xsa, SX, noise, r, kk, item);
         if (TD3) {
             if (!CRITIC && row_ok && A.out_pre_clip) {

@@ -10,6 +10,8 @@
 //   actor update    actor forward -> squashed sample -> critic 0, then critic 1: forward and the gradient of -value / batch with respect
 //                   to the action -> gradient of the smaller value per row -> sample_and_squash backward (entropy term, log_alpha
 //                   gradient) -> actor backward
+// The same kernel runs TD3's two updates (rl/algorithms/td3/operations_generic.h:170-281; actors obs -> h -> h -> act with a tanh output followed by the
+// td3_sampling layer): the critic update with the target actor, the smoothing noise on the next action and no entropy term, the actor update through critic 0 only.
 // Wavefront w owns hidden units 16 w .. 16 w + 15 of every layer: it computes that tile of the 16 x h activations from the whole previous
 // layer (LDS, behind a workgroup barrier), contributes the units' share of the output layer's reduction (the partial tiles are added in
 // wavefront order), and in the backward pass owns the same units' pre-activation gradients and their rows of dW1, dW2 and columns of dW3.
@@ -33,7 +35,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) floatx4* lptr4;
 constexpr int ROWS = 16, MAX_H = 256, WAVES = MAX_H / 16, THREADS = 64 * WAVES, S = MAX_H + 4, MAX_D = 128, SXS = MAX_D + 4, MAX_ACT = 8, MAX_OUT = 16, D3S = MAX_OUT + 1,
               N_EXTRA = 16, MISC = 64, YP = ROWS * D3S;
-enum { MODE_CRITIC = 0, MODE_ACTOR = 1 };
+enum { MODE_CRITIC = 0, MODE_ACTOR = 1, MODE_TD3_CRITIC = 2, MODE_TD3_ACTOR = 3 };      // SAC's two updates, TD3's two updates
 
 // W2f / W2b: copies of the second layer's weights in the order the wavefronts consume them (wide_prepare_kernel): 16 bytes per lane, a wavefront's load 1 KB in a row
 struct WNet { const float *W1, *b1, *W2, *b2, *W3, *b3; int in, hid, out, act_h, vec1, vec2, vec3; const float *W2f, *W2b; };      // vecN: the rows of WN can be read 16 bytes at a time
@@ -49,6 +51,9 @@ struct WideArgs {
     int batch, obs, act;
     float* partial; int count;             // per workgroup and trained network: count floats (the optimiser's launch adds the blocks up)
     float* out_log_probabilities; float* out_target_action_value; float* out_actions; float* out_pre_squashing;
+    // TD3 (rl/algorithms/td3/operations_generic.h:170-281): `actor` is the target actor in the critic update and has `act` outputs; they pass tanh and the
+    // td3_sampling layer (sac_heads.h); the critic update adds target_noise [batch][act] (already clamped) to the next action; the actor update goes through critic[0] only
+    float sampling_std; int ignore_termination; const float* target_noise; float* out_pre_clip;
     int packed;                            // every 8th workgroup of an 8 x larger grid works: all of them on one XCD
 };
 
@@ -100,7 +105,7 @@ __device__ __forceinline__ void chunks(floatx4& a0, floatx4& a1, lptr in, int st
 // profiling builds (-DRLT_WIDE_PROFILE): thread 0 of workgroup 0 notes the constant-rate clock at the stage boundaries, rlt_sac_wide_ticks copies the notes out
 #ifdef RLT_WIDE_PROFILE
 __device__ unsigned long long rlt_wide_ticks[2][32];
-#define RLT_TICK(i) do { if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) rlt_wide_ticks[MODE][i] = wall_clock64(); } while (0)
+#define RLT_TICK(i) do { if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) rlt_wide_ticks[MODE & 1][i] = wall_clock64(); } while (0)
 #else
 #define RLT_TICK(i) do {} while (0)
 #endif
@@ -324,7 +329,7 @@ __global__ __launch_bounds__(256) void wide_prepare_kernel(PrepArgs P) {
 
 template <int MODE, int ACT_H, int NT1C>
 __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
-    constexpr bool CRITIC = MODE == MODE_CRITIC;
+    constexpr bool CRITIC = MODE == MODE_CRITIC || MODE == MODE_TD3_CRITIC, TD3 = MODE == MODE_TD3_CRITIC || MODE == MODE_TD3_ACTOR;
     extern __shared__ __attribute__((aligned(16))) float lds_wide[];
     if (A.packed && (blockIdx.x & 7)) return;
     const int gi = A.packed ? blockIdx.x >> 3 : blockIdx.x, G = A.packed ? gridDim.x >> 3 : gridDim.x;
@@ -349,10 +354,14 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
         if (CRITIC) { xa[e] = ok ? cur[(size_t)B * D] : 0.f; xb[e] = ok ? cur[0] : 0.f; }
         else xa[e] = (ok && k < OBS) ? cur[0] : 0.f;
     }
-    float noise[2] = {0.f, 0.f}, reward[4] = {0.f, 0.f, 0.f, 0.f}, alpha = 0.f, s3 = 0.f, extra = 0.f;
+    float noise[2] = {0.f, 0.f}, target_noise[2] = {0.f, 0.f}, reward[4] = {0.f, 0.f, 0.f, 0.f}, alpha = 0.f, s3 = 0.f, extra = 0.f;
     bool terminated[4] = {false, false, false, false};
     if (scalar_wave) {
-        alpha = expf(*A.log_alpha);
+        if (!TD3) alpha = expf(*A.log_alpha);
+        if (MODE == MODE_TD3_CRITIC) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) target_noise[j] = (g + 4 * j < ACT && row0 + c < B) ? A.target_noise[(size_t)(row0 + c) * ACT + g + 4 * j] : 0.f;
+        }
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             if (g + 4 * j < ACT && row0 + c < B) {
@@ -384,12 +393,20 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
 #pragma unroll
         for (int v = 0; v < 4; v++) d3[(4 * g + v) * D3S + c] = c < A.actor.out ? out[v] + b3 : 0.f;
         wave_sync();
-        const float log_prob = head_forward(A.sas, OBS, ACT, d3, D3S, xa, SXS, noise, c, g, item);
-        if (g == 0) {
+        float log_prob = 0.f;
+        if (TD3) td3_head_forward(OBS, ACT, A.sampling_std, d3, D3S, xa, SXS, noise, target_noise, CRITIC, c, g, item);
+        else log_prob = head_forward(A.sas, OBS, ACT, d3, D3S, xa, SXS, noise, c, g, item);
+        if (TD3) {
+            if (!CRITIC && row_ok && A.out_pre_clip) {
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    if (g + 4 * j < ACT) A.out_pre_clip[(size_t)(row0 + c) * ACT + g + 4 * j] = item[j].sample;
+            }
+        } else if (g == 0) {
             if (CRITIC) misc[c] = log_prob;
             if (A.out_log_probabilities && row_ok) A.out_log_probabilities[row0 + c] = log_prob;
         }
-        if (!CRITIC && row_ok) {
+        if (!TD3 && !CRITIC && row_ok) {
 #pragma unroll
             for (int j = 0; j < 2; j++)
                 if (g + 4 * j < ACT) {
@@ -419,12 +436,14 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
             // loss weight batch * 0.5 / n with n = batch rows (no masks), times the MSE gradient's 2 / batch (rl/algorithms/sac/operations_generic.h:298-316)
             const floatx4 yc = output_tile(yp, tiles, c, g);
             const float b3 = trained.b3[0];
-            const float loss_weight = (1.0f / (float)B) * ((float)B * 0.5f);
+            // (TD3: loss weight batch / n, rl/algorithms/td3/operations_generic.h:200-212)
+            const float loss_weight = TD3 ? (float)B / (float)B : (1.0f / (float)B) * ((float)B * 0.5f);
             const float constant = 2.0f / (float)B * loss_weight;
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const float min_q = fminf(q_next[0][v], q_next[1][v]) - alpha * misc[4 * g + v];
-                const float future = terminated[v] ? 0.0f : A.gamma * min_q;
+                const float q_min = fminf(q_next[0][v], q_next[1][v]);
+                const float min_q = TD3 ? q_min : q_min - alpha * misc[4 * g + v];
+                const float future = (terminated[v] && !(TD3 && A.ignore_termination)) ? 0.0f : A.gamma * min_q;
                 const float y_target = reward[v] + future;
                 const bool ok = c == 0 && row0 + 4 * g + v < B;
                 if (A.out_target_action_value && ok && y == 0) A.out_target_action_value[row0 + 4 * g + v] = y_target;
@@ -438,10 +457,11 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
         rlt_lds_barrier();      // d_pre3 is in place
         RLT_TICK(7);
     } else {
-        // each critic: value on [observation | sampled action], then the gradient of -value / batch with respect to the action
+        // each critic (TD3: critic 0 only, rl/algorithms/td3/operations_generic.h:260): value on [observation | sampled action], then the gradient of -value / batch
+        // with respect to the action
         const float loss_weight = (1.0f / (float)B) * -1.0f;       // rl/algorithms/sac/operations_generic.h:437-453 with n = batch rows
 #pragma unroll 1
-        for (int k = 0; k < 2; k++) {
+        for (int k = 0; k < (TD3 ? 1 : 2); k++) {
             const WNet C = k ? A.critic[1] : A.critic[0];
             const int ctiles = (C.hid + 15) >> 4;
             forward3_own_loads<ACT_H, NT1C>(C, xa, SXS, ta, tb, yp, wave, c, g);
@@ -483,9 +503,10 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
             }
         }
         if (scalar_wave) {
-            // sample_and_squash backward on the gradient of the smaller value
+            // sample_and_squash backward on the gradient of the smaller value; TD3: the td3_sampling layer's backward (zero where the sample was clamped,
+            // nn/layers/td3_sampling/operations_generic.h:139-163) and the derivative of the actor's tanh output
             wave_sync();
-            const lptr dak = da + (misc[c] < misc[16 + c] ? 0 : 1) * ROWS * D3S + c * D3S;
+            const lptr dak = da + ((TD3 || misc[c] < misc[16 + c]) ? 0 : 1) * ROWS * D3S + c * D3S;
 #pragma unroll
             for (int v = 0; v < 4; v++) d3[(4 * g + v) * D3S + c] = 0.f;
             wave_sync();
@@ -495,6 +516,11 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
             for (int j = 0; j < 2; j++) {
                 const int a = g + 4 * j;
                 if (a < ACT) {
+                    if (TD3) {
+                        const float d_mean = (item[j].sample < -1.0f || item[j].sample > 1.0f) ? 0.0f : dak[a];
+                        if (row_ok) d3[c * D3S + a] = d_mean * (1.0f - item[j].mean * item[j].mean);
+                        continue;
+                    }
                     float d_mu, d_ls;
                     head_backward(A.sas, item[j], dak[a], alpha_over_b, d_mu, d_ls, entropy);
                     if (row_ok) { d3[c * D3S + a] = d_mu; d3[c * D3S + ACT + a] = d_ls; }
@@ -586,12 +612,12 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
 constexpr size_t LDS_FLOATS = (size_t)2 * ROWS * SXS + 4 * ROWS * S + 4 * ROWS * D3S + WAVES * YP + MISC;
 
 bool hidden_ok(int a) { return a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH || a == RLT_ACT_SIGMOID; }
-bool net_ok(const rlt_dense_layer* L, int n, int in, int out, int& hid) {
+bool net_ok(const rlt_dense_layer* L, int n, int in, int out, int& hid, int last_activation = RLT_ACT_IDENTITY) {
     if (!L || n != 3) return false;
     for (int l = 0; l < 3; l++) if (!L[l].weights || !L[l].biases) return false;
     if (hid == 0) hid = L[0].out_dim;
     return hid >= 1 && hid <= MAX_H && L[0].in_dim == in && L[0].out_dim == hid && L[1].in_dim == hid && L[1].out_dim == hid && L[2].in_dim == hid && L[2].out_dim == out &&
-           L[0].activation == L[1].activation && hidden_ok(L[0].activation) && L[2].activation == RLT_ACT_IDENTITY;
+           L[0].activation == L[1].activation && hidden_ok(L[0].activation) && L[2].activation == last_activation;
 }
 bool aligned16(const float* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 WNet net_of(const rlt_dense_layer* L) {
@@ -676,9 +702,10 @@ int launch_wide(rlt_rocm_device* device, WideArgs& a, int groups, const Optimise
     int n_forward = 0, n_backward = 0;
     forward_nets[n_forward++] = &a.actor;
     for (int k = 0; k < 2; k++) forward_nets[n_forward++] = &a.critic[k];
-    if (MODE == MODE_CRITIC) for (int k = 0; k < 2; k++) forward_nets[n_forward++] = &a.target[k];
+    constexpr bool CRITIC_UPDATE = MODE == MODE_CRITIC || MODE == MODE_TD3_CRITIC;
+    if (CRITIC_UPDATE) for (int k = 0; k < 2; k++) forward_nets[n_forward++] = &a.target[k];
     for (int k = 0; k < 2; k++) backward_nets[n_backward++] = &a.critic[k];
-    if (MODE == MODE_ACTOR) backward_nets[n_backward++] = &a.actor;
+    if (!CRITIC_UPDATE) backward_nets[n_backward++] = &a.actor;
     const size_t copy_floats = (size_t)256 * WAVES * WAVES;      // [16 wavefronts][16 chunks][64 lanes][4] at width 256
     const size_t partial_bytes = ((size_t)n_opts * groups * a.count * sizeof(float) + 255) & ~(size_t)255;
     void* scratch = nullptr;
@@ -790,6 +817,48 @@ int rlt_sac_wide_update_actor(rlt_rocm_device* device, const rlt_sac_agent* A, c
     a.out_log_probabilities = A->actor_log_probabilities; a.out_actions = A->actor_actions; a.out_pre_squashing = A->actor_pre_squashing;
     const Optimiser O = {A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, &A->log_alpha, &A->alpha_adam, A->alpha_age, 1.0f / (float)A->batch, nullptr};
     return launch_wide<MODE_ACTOR>(device, a, rlt_div_up(A->batch, ROWS), &O, 1, 0.0f, nullptr);
+}
+
+// ---- TD3: the same kernel with the td3_sampling head (rl/algorithms/td3/operations_generic.h:170-281)
+
+bool rlt_td3_wide_supported(const rlt_rocm_device* device, const rlt_td3_agent* A) {
+    const int OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    if (OBS < 1 || ACT < 1 || ACT > MAX_ACT || D > MAX_D || A->batch < 1 || A->batch > 2048) return false;
+    if (A->final_step_mask || A->next_final_step_mask) return false;
+    int hid_a = 0, hid_c = 0;
+    if (!net_ok(A->actor, A->n_actor_layers, OBS, ACT, hid_a, RLT_ACT_TANH) || !net_ok(A->actor_target, A->n_actor_layers, OBS, ACT, hid_a, RLT_ACT_TANH)) return false;
+    for (int k = 0; k < 2; k++)
+        if (!net_ok(A->critics[k], A->n_critic_layers, D, 1, hid_c) || !net_ok(A->critics_target[k], A->n_critic_layers, D, 1, hid_c)) return false;
+    return LDS_FLOATS * sizeof(float) <= (size_t)device->lds_bytes;
+}
+
+int rlt_td3_wide_update_critic(rlt_rocm_device* device, const rlt_td3_agent* A, int ci, const float* sampling_noise) {
+    if (!rlt_td3_wide_supported(device, A)) return RLT_E_UNSUPPORTED;
+    for (int l = 0; l < 3; l++) RLT_REQUIRE(A->critics[ci][l].d_weights && A->critics[ci][l].d_biases);
+    RLT_REQUIRE(A->target_next_action_noise && sampling_noise);
+    WideArgs a = {};
+    a.actor = net_of(A->actor_target); a.critic[0] = net_of(A->critics[ci]); a.critic[1] = a.critic[0];
+    for (int k = 0; k < 2; k++) a.target[k] = net_of(A->critics_target[k]);
+    a.batch_base = A->observations_actions_base; a.rewards = A->rewards; a.terminated = A->terminated; a.noise = sampling_noise; a.target_noise = A->target_next_action_noise;
+    a.sampling_std = A->sampling_std; a.ignore_termination = A->ignore_termination;
+    a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
+    a.out_target_action_value = A->target_action_value;
+    const Optimiser O = {A->critics[ci], A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], nullptr, nullptr, nullptr, 0.0f, nullptr};
+    return launch_wide<MODE_TD3_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), &O, 1, 0.0f, nullptr);
+}
+
+int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise) {
+    if (!rlt_td3_wide_supported(device, A)) return RLT_E_UNSUPPORTED;
+    for (int l = 0; l < 3; l++) RLT_REQUIRE(A->actor[l].d_weights && A->actor[l].d_biases);
+    RLT_REQUIRE(sampling_noise);
+    WideArgs a = {};
+    a.actor = net_of(A->actor);
+    for (int k = 0; k < 2; k++) { a.critic[k] = net_of(A->critics[0]); a.target[k] = a.critic[k]; }       // the policy gradient goes through critic 0 (:260)
+    a.batch_base = A->observations_actions_base; a.noise = sampling_noise; a.sampling_std = A->sampling_std;
+    a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
+    a.out_pre_clip = A->actor_pre_clip;
+    const Optimiser O = {A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, nullptr, nullptr, nullptr, 0.0f, nullptr};
+    return launch_wide<MODE_TD3_ACTOR>(device, a, rlt_div_up(A->batch, ROWS), &O, 1, 0.0f, nullptr);
 }
 
 #ifdef RLT_WIDE_PROFILE

@@ -208,6 +208,7 @@ int rlt_rocm_td3_train_critic(rlt_rocm_device* device, const rlt_td3_agent* A, i
     RLT_REQUIRE(A->target_next_action_noise && A->next_state_action_value_input && A->next_q[0] && A->next_q[1] && A->target_action_value && A->d_output_critic);
     RLT_REQUIRE(A->critic_adam_tensors[ci] && A->critic_age[ci]);
     if (!device->sac_per_operation && rlt_td3_update_supported(device, A)) return rlt_td3_update_critic(device, A, ci, sampling_noise);
+    if (!device->sac_per_operation && rlt_td3_wide_supported(device, A)) return rlt_td3_wide_update_critic(device, A, ci, sampling_noise);
     const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
     const rlt_dense_layer* critic = A->critics[ci];
     const size_t mean_bytes = ((size_t)B * ACT * sizeof(float) + 255) & ~(size_t)255;
@@ -239,6 +240,7 @@ int rlt_rocm_td3_train_actor(rlt_rocm_device* device, const rlt_td3_agent* A, co
     RLT_REQUIRE(agent_ok(A) && sampling_noise);
     RLT_REQUIRE(A->state_action_value_input && A->actor_pre_clip && A->d_output_actor && A->d_critic_input && A->d_actor_output && A->actor_adam_tensors && A->actor_age);
     if (!device->sac_per_operation && rlt_td3_update_supported(device, A)) return rlt_td3_update_actor(device, A, sampling_noise);
+    if (!device->sac_per_operation && rlt_td3_wide_supported(device, A)) return rlt_td3_wide_update_actor(device, A, sampling_noise);
     const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
     RLT_REQUIRE(A->workspace_bytes >= rlt_rocm_mlp_workspace_bytes(A->critics[0], A->n_critic_layers, B));
     RLT_REQUIRE(A->workspace_bytes >= rlt_rocm_mlp_workspace_bytes(A->actor, A->n_actor_layers, B));

@@ -305,7 +305,7 @@ def test_td3_on_the_acrobot_swingup_trains_on_rocm():
     """The configuration of the reference's TD3 program for the AcrobotSwingup (src/rl/environments/acrobot/td3/acrobot.cpp: EasyParameters, actor and critics
     3 x 256, the loop's default TD3 parameters) inside the evaluation loop step on devices::ROCM: the exploring actor's td3_sampling head in the library's runner
     step for any environment, evaluations of 10 episodes x 500 steps on the device. Here the first 60,000 of its 100,000 loop steps; measured over all of them:
-    mean return -129 before training, -58 after 50,000 steps, best -10, 37 s (2,700 loop steps/s including the 100 evaluations)."""
+    mean return -129 before training, best -6, 22.5 s (4,440 loop steps/s including the 100 evaluations; the updates on the one-launch kernel for widths up to 256)."""
     path = os.path.join(BUILD, "rocm_td3_acrobot")
     if not os.path.exists(path):
         pytest.skip("tests/integration/_build is built where the reference's headers are mounted")

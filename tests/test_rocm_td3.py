@@ -156,9 +156,21 @@ def test_fused_updates_match_the_checker_and_the_per_operation_path(oracle, rocm
     obs + act -> 64 -> 64 -> 1): three loop steps (both critics, targets, actor, actor target each) from identical parameters, batches and noise
     against the checker and against the one-launch-per-operation path; samples beyond [-1, 1] and terminated rows included. 1e-5 relative to
     each tensor's largest magnitude."""
+    fused_against_checker_and_per_operation(oracle, rocm, batch, obs, act, hidden_act, 64)
+
+
+@pytest.mark.parametrize("batch,obs,act,hidden,hidden_act", [(256, 6, 1, 256, "fast_tanh"), (100, 17, 6, 128, "relu"), (48, 3, 1, 200, "relu"), (256, 27, 8, 256, "relu"),
+                                                             (30, 111, 8, 72, "tanh"), (512, 5, 2, 16, "sigmoid")])
+def test_wider_agents_match_the_checker_on_both_paths(oracle, rocm, batch, obs, act, hidden, hidden_act):
+    """The same at hidden widths other than 64 (up to 256; the kernel that takes 16 rows per workgroup of sixteen wavefronts through every pass, with the
+    optimiser's launch adding up the workgroups' partial sums): the shapes that the SAC updates are tested at."""
+    fused_against_checker_and_per_operation(oracle, rocm, batch, obs, act, hidden_act, hidden)
+
+
+def fused_against_checker_and_per_operation(oracle, rocm, batch, obs, act, hidden_act, hidden):
     rng = np.random.default_rng(batch * 7 + obs)
     D = obs + act
-    adims, cdims = [obs, 64, 64, act], [D, 64, 64, 1]
+    adims, cdims = [obs, hidden, hidden, act], [D, hidden, hidden, 1]
     nets = [helpers.random_params(rng, adims)] * 2 + [helpers.random_params(rng, cdims) for _ in range(2)]
     params = np.concatenate(nets + [nets[2] * 0.9, nets[3] * 1.1]).astype(np.float32)
     hyper = dict(gamma=0.99, actor_polyak=0.995, critic_polyak=0.99, sampling_std=0.5, adam=helpers.capi.adam_parameters(epsilon=1e-7))
@@ -169,7 +181,7 @@ def test_fused_updates_match_the_checker_and_the_per_operation_path(oracle, rocm
                       np.clip(rng.standard_normal((batch, act)) * 0.2, -0.5, 0.5).astype(np.float32), [rng.standard_normal((batch, act)).astype(np.float32) for _ in range(3)]))
     out = {}
     for name, b, per_operation in (("checker", oracle, None), ("fused", rocm, 0), ("per_operation", rocm, 1)):
-        ag = helpers.Td3OnBackend(b, batch, 64, params, hyper=hyper, masks=False, obs=obs, act=act, hidden_act=hidden_act)
+        ag = helpers.Td3OnBackend(b, batch, hidden, params, hyper=hyper, masks=False, obs=obs, act=act, hidden_act=hidden_act)
         if per_operation is not None:
             rocm.call("sac_set_per_operation", per_operation)
         try:
