@@ -6,6 +6,7 @@
 #include "common.h"
 #include "pendulum.h"
 #include "rng.h"
+#include "sac_heads.h"
 
 namespace {
 struct Acrobot4 { float v[4]; };
@@ -295,8 +296,8 @@ __device__ __forceinline__ void env_step_one(const rlt_env_runner& rn, float* __
 
 // ---- The runner's whole step in ONE launch for a handful of environments and a policy of dense layers (rl/components/off_policy_runner/operations_generic.h:183-238 over
 // operations_generic_per_env.h:8-108): reset and observe, the policy's layers, its head, the environment's step, counters and the replay add. One workgroup of sixteen
-// wavefronts: a wavefront forms an output unit's dot products for all environments at once (lanes across the input width, the weights' row read coalesced, the sums
-// folded across the lanes), the activations of a layer wait in LDS for the next. For the loops that step one or a few environments per training step, where the
+// wavefronts: a wavefront forms the dot products of its sixteen output units (lanes across the input width, the weights' rows read coalesced and all at once, the
+// sums folded across the lanes), the activations of a layer wait in LDS for the next. For the loops that step one or a few environments per training step, where the
 // launches of the separate kernels (nine of them) are the whole cost.
 __device__ __forceinline__ float mul_add_twice_rounded(float a, float b, float c) {
 #pragma clang fp contract(off)
@@ -346,19 +347,39 @@ __global__ __launch_bounds__(FUSED_THREADS) void env_runner_fused_kernel(EnvFuse
     }
     __syncthreads();
     int cur = 0;
+    // A layer: wavefront w owns output units 16 w .. 16 w + 15. All of their rows of W are requested at once, with addresses clamped into the matrix instead of
+    // branches (a launch of one workgroup finds nothing of the weights in its caches: one trip to memory per layer, not one per unit; and straight-line code,
+    // because the instructions come from memory as well). Lanes hold the input positions lane + 64 j; positions beyond the layer's width meet zero activations,
+    // units beyond it are not stored. After the sums over the lanes, lane q of the first sixteen keeps unit q, adds the bias and applies the activation.
+    constexpr int UNITS = 16, CHUNKS = FUSED_MAX_WIDTH / 64;
+    static_assert(UNITS * (FUSED_THREADS / 64) == FUSED_MAX_WIDTH, "a wavefront's units times the wavefronts cover the widest layer");
     for (int l = 0; l < A.n_layers; l++) {
         const FusedLayer& L = A.L[l];
-        for (int o = wave; o < L.out_dim; o += FUSED_THREADS / 64) {
-            float w[FUSED_MAX_WIDTH / 64];
+        const int in = L.in_dim, out = L.out_dim;
+        if (UNITS * wave < out) {
+            float w[UNITS][CHUNKS];
 #pragma unroll
-            for (int j = 0; j < FUSED_MAX_WIDTH / 64; j++) w[j] = lane + 64 * j < L.in_dim ? L.weights[(size_t)o * L.in_dim + lane + 64 * j] : 0.f;
-            const float bias = L.biases[o];
+            for (int q = 0; q < UNITS; q++) {
+                const float* row = L.weights + (size_t)min(UNITS * wave + q, out - 1) * in;
+#pragma unroll
+                for (int j = 0; j < CHUNKS; j++) w[q][j] = row[min(lane + 64 * j, in - 1)];
+            }
+            const int mine = UNITS * wave + (lane & 15);
+            const float bias = L.biases[min(mine, out - 1)];
             for (int r = 0; r < N; r++) {
-                float s = 0.f;
+                float a[CHUNKS];
 #pragma unroll
-                for (int j = 0; j < FUSED_MAX_WIDTH / 64; j++) s += lane + 64 * j < L.in_dim ? w[j] * act[cur][r][lane + 64 * j] : 0.f;
-                s = rlt_wave_sum(s);
-                if (lane == 0) act[cur ^ 1][r][o] = rlt_act(s + bias, L.activation);
+                for (int j = 0; j < CHUNKS; j++) a[j] = lane + 64 * j < in ? act[cur][r][lane + 64 * j] : 0.f;
+                float kept = 0.f;
+#pragma unroll
+                for (int q = 0; q < UNITS; q++) {
+                    float sum = w[q][0] * a[0];
+#pragma unroll
+                    for (int j = 1; j < CHUNKS; j++) sum += w[q][j] * a[j];
+                    sum = rlt_sac::groups_sum(rlt_sac::row16_sum(sum));
+                    kept = (lane & 15) == q ? sum : kept;
+                }
+                if (lane < 16 && mine < out) act[cur ^ 1][r][mine] = rlt_act(kept + bias, L.activation);
             }
         }
         __syncthreads();
