@@ -600,6 +600,27 @@ def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=100
     rocm.sync()
     a = ev.record(); updates(300); b = ev.record()
     out["width256_agent_obs6_act1_update_sets_per_s_by_device_clock"] = 300 / (ev.elapsed_ms(a, b) * 1e-3)
+    # TD3 at the shapes of the zoo's Ant agent (src/rl/zoo/ant-v4/td3.h: observation 27, action 8, hidden width 256, ReLU, batch 256): both critics, the actor, the three
+    # target updates per set
+    obs, act = 27, 8
+    adims, cdims = [obs, 256, 256, act], [obs + act, 256, 256, 1]
+    nets = [helpers.random_params(rng, adims)] * 2 + [helpers.random_params(rng, cdims) for _ in range(2)]
+    td3 = helpers.Td3OnBackend(rocm, batch, 256, np.concatenate(nets + [nets[2], nets[3]]).astype(np.float32), masks=False, obs=obs, act=act)
+    oab = rng.standard_normal((2, batch, obs + act)).astype(np.float32); oab[:, :, obs:] = np.tanh(oab[:, :, obs:])
+    td3.set_batch(oab, rng.standard_normal(batch).astype(np.float32), (rng.random(batch) < 0.05).astype(np.uint8), np.clip(rng.standard_normal((batch, act)) * 0.2, -0.5, 0.5).astype(np.float32))
+    noise = rocm.array(rng.standard_normal((batch, act)).astype(np.float32))
+
+    def td3_updates(n):
+        for _ in range(n):
+            for k in (0, 1):
+                rocm.device.check(lib.rlt_rocm_td3_train_critic(h, C.byref(td3.c), k, noise.ptr))
+            rocm.device.check(lib.rlt_rocm_td3_update_critic_targets(h, C.byref(td3.c)))
+            rocm.device.check(lib.rlt_rocm_td3_train_actor(h, C.byref(td3.c), noise.ptr))
+            rocm.device.check(lib.rlt_rocm_td3_update_actor_target(h, C.byref(td3.c)))
+    td3_updates(20)
+    rocm.sync()
+    a = ev.record(); td3_updates(300); b = ev.record()
+    out["td3_width256_agent_obs27_act8_update_sets_per_s_by_device_clock"] = 300 / (ev.elapsed_ms(a, b) * 1e-3)
     return out
 
 
