@@ -319,22 +319,35 @@ def bench_sac_sequence(helpers, rocm, S=100, B=100, iters=10, cpu_seconds=1.5):
         agent.set_batch(data)
         ncd, nad = be.array(nc), be.array(na)
 
-        def step():
-            for k in range(2):
+        def step(together=False):
+            if together:      # both critics in one call: the loop's shared batch (what the devices::ROCM loop step issues)
+                be.call("sac_sequence_train_critics", C.byref(agent.c), ncd.ptr)
+            for k in range(0 if together else 2):
                 be.call("sac_sequence_train_critic", C.byref(agent.c), k, ncd.ptr)
             be.call("sac_sequence_update_critic_targets", C.byref(agent.c))
             be.call("sac_sequence_train_actor", C.byref(agent.c), nad.ptr)
         if be.name == "rocm":
             ev = HipEvents(rocm.device.lib.rlt_rocm_get_stream(rocm.device.handle))
             for _ in range(3):
-                step()
+                step(True)
             rocm.sync()
             a = ev.record()
             for _ in range(iters):
+                step(True)
+            e = ev.record()
+            out["ms_per_training_step_both_critics_in_one_call"] = ev.elapsed_ms(a, e) / iters
+            for _ in range(3):
                 step()
+            rocm.sync()
+            a = ev.record()
+            t0 = time.perf_counter()
+            for _ in range(iters):
+                step()
+            host_ms = (time.perf_counter() - t0) * 1e3 / iters      # what the host needs to issue a step's launches (it does not wait for them)
             e = ev.record()
             ms = ev.elapsed_ms(a, e) / iters
             out["ms_per_training_step"] = ms
+            out["host_ms_to_issue_a_training_step"] = host_ms
             out["sequences_per_s"] = 3 * B / (ms * 1e-3)
         else:
             step()

@@ -83,5 +83,54 @@ namespace rl_tools{
         ts.step++;
         return false;
     }
+    // The same loop step for recurrent agents on sequence batches (rl/algorithms/sac/operations_rocm_sequence.h) where the loop shares one batch among the updates: the
+    // generic step's operations in its order on its random streams, with the two train_critic calls as one call of the library (what the second would recompute on
+    // unchanged inputs is computed once, the two critics' passes run side by side). Same bits as the generic step.
+    namespace rl::algorithms::sac::loop::core::rocm{
+        template <typename CONFIG>
+        constexpr bool shared_sequence_updates(){
+            return CONFIG::CORE_PARAMETERS::SHARED_BATCH && rl::algorithms::sac::rocm::sequence_describable<typename CONFIG::ACTOR_CRITIC_SPEC, typename CONFIG::CRITIC_BATCH_SPEC>();
+        }
+    }
+    template <typename DEV_SPEC, typename T_CONFIG, utils::typing::enable_if_t<rl::algorithms::sac::loop::core::rocm::shared_sequence_updates<T_CONFIG>(), int> = 0>
+    bool step(devices::ROCM<DEV_SPEC>& device, rl::algorithms::sac::loop::core::State<T_CONFIG>& ts){
+        using CORE = typename T_CONFIG::CORE_PARAMETERS;
+        using SAC = typename CORE::SAC_PARAMETERS;
+        if(ts.step >= CORE::STEP_LIMIT){
+            return true;
+        }
+        set_step(device, device.logger, ts.step);
+        if(ts.step >= CORE::N_WARMUP_STEPS){
+            step<1>(device, ts.off_policy_runner, get_actor(ts), ts.actor_buffers_eval, ts.rng);
+        }
+        else{
+            typename T_CONFIG::EXPLORATION_POLICY exploration_policy;
+            typename T_CONFIG::EXPLORATION_POLICY::template Buffer<> exploration_policy_buffer;
+            step<0>(device, ts.off_policy_runner, exploration_policy, exploration_policy_buffer, ts.rng);
+        }
+        const bool critics_due = ts.step >= CORE::N_WARMUP_STEPS_CRITIC && ts.step % SAC::CRITIC_TRAINING_INTERVAL == 0;
+        const bool targets_due = ts.step >= CORE::N_WARMUP_STEPS_CRITIC && ts.step % SAC::CRITIC_TARGET_UPDATE_INTERVAL == 0;
+        const bool actor_due = ts.step >= CORE::N_WARMUP_STEPS_ACTOR && ts.step % SAC::ACTOR_TRAINING_INTERVAL == 0;
+        if(critics_due || actor_due){
+            gather_batch(device, ts.off_policy_runner, ts.critic_batch, ts.rng);
+            randn(device, ts.action_noise_critic, ts.rng);
+        }
+        if(critics_due){
+            if(!rl::algorithms::sac::rocm::train_critics(device, ts.actor_critic, ts.critic_batch, ts.actor_critic.critic_optimizers, ts.critic_training_buffers[0], ts.action_noise_critic)){
+                for(int critic_i = 0; critic_i < 2; critic_i++){
+                    train_critic(device, ts.actor_critic, ts.actor_critic.critics[critic_i], ts.critic_batch, ts.actor_critic.critic_optimizers[critic_i], ts.actor_target_buffers[critic_i], ts.critic_buffers[critic_i], ts.critic_target_buffers[critic_i], ts.critic_training_buffers[critic_i], ts.action_noise_critic, ts.rng);
+                }
+            }
+        }
+        if(targets_due){
+            update_critic_targets(device, ts.actor_critic);
+        }
+        if(actor_due){
+            randn(device, ts.action_noise_actor, ts.rng);
+            train_actor(device, ts.actor_critic, ts.critic_batch, ts.actor_critic.actor_optimizer, ts.actor_buffers[0], ts.critic_buffers[0], ts.actor_training_buffers, ts.action_noise_actor, ts.rng);
+        }
+        ts.step++;
+        return false;
+    }
 }
 RL_TOOLS_NAMESPACE_WRAPPER_END

@@ -12,6 +12,7 @@
 #include <rl_tools/nn/layers/gru/operations_rocm.h>
 #include <rl_tools/nn/layers/sample_and_squash/operations_rocm.h>
 #include <type_traits>
+#include <cstring>
 RL_TOOLS_NAMESPACE_WRAPPER_START
 namespace rl_tools{
     namespace rl::algorithms::sac::rocm{
@@ -166,6 +167,41 @@ namespace rl_tools{
         a.workspace = memory; a.workspace_bytes = workspace_bytes;
         const int critic_index = &critic == &actor_critic.critics[1] ? 1 : 0;
         devices::rocm::check(rlt_rocm_sac_sequence_train_critic(device.handle, &a, critic_index, action_noise._data), "train_critic (sequences)");
+    }
+    namespace rl::algorithms::sac::rocm{
+        // train_critic for critic 0 and then for critic 1 on one batch and one set of noise, the loop's SHARED_BATCH case (rl/algorithms/sac/loop/core/operations_generic.h:127-138),
+        // as one call of the library: the second train_critic would repeat the actor's pass over the next steps, its sample, both target critics and the target values on
+        // unchanged inputs; the library computes them once and runs the two critics' passes side by side. Same bits as the two calls. The training buffers of critic 0
+        // receive what both calls would write there except d_output, which holds critic 1's loss gradient (critic 0's stays in the library's workspace).
+        // false: the two optimisers differ in their parameters; the caller makes the two calls.
+        template <typename DEV_SPEC, typename SPEC, typename BATCH_SPEC, typename OPTIMIZER, typename TRAINING_BUFFER_SPEC, typename ACTION_NOISE_SPEC>
+        bool train_critics(devices::ROCM<DEV_SPEC>& device, rl::algorithms::sac::ActorCritic<SPEC>& actor_critic, rl::components::off_policy_runner::SequentialBatch<BATCH_SPEC>& batch, OPTIMIZER (&optimizers)[2],
+                           rl::algorithms::sac::CriticTrainingBuffers<TRAINING_BUFFER_SPEC>& training_buffers, Matrix<ACTION_NOISE_SPEC>& action_noise){
+            using DEVICE = devices::ROCM<DEV_SPEC>;
+            constexpr size_t S = BATCH_SPEC::SEQUENCE_LENGTHH, B = BATCH_SPEC::BATCH_SIZE, ACTION_DIM = SPEC::ENVIRONMENT::ACTION_DIM;
+            constexpr size_t T = S + (BATCH_SPEC::PARAMETERS::INCLUDE_FIRST_STEP_IN_TARGETS ? 1 : 0);
+            static_assert(ACTION_NOISE_SPEC::ROWS == T * B && ACTION_NOISE_SPEC::COLS == ACTION_DIM && ACTION_NOISE_SPEC::COL_PITCH == 1 && ACTION_NOISE_SPEC::ROW_PITCH == ACTION_DIM, "one row of noise per evaluated `next` step, back to back");
+            const rlt_adam_parameters first = adam_parameters(optimizers[0]), second = adam_parameters(optimizers[1]);
+            if(std::memcmp(&first, &second, sizeof(first)) != 0){ return false; }
+            SequenceDescription<DEVICE, SPEC> d(device, actor_critic);
+            d.set_batch(batch);
+            rlt_sac_sequence_agent& a = d.agent;
+            a.critic_adam = first;
+            a.next_state_action_value_input = training_buffers.next_state_action_value_input._data;
+            a.next_q[0] = training_buffers.next_state_action_value_critic_1._data; a.next_q[1] = training_buffers.next_state_action_value_critic_2._data;
+            a.next_log_probabilities = training_buffers.next_action_log_probs._data;
+            a.target_action_value = training_buffers.target_action_value._data;
+            a.d_output = training_buffers.d_output._data;
+            const size_t intermediates = intermediates_bytes(d.actor, T * B) + intermediates_bytes(d.targets[0], T * B) + intermediates_bytes(d.targets[1], T * B);
+            const size_t workspace_bytes = rlt_rocm_sac_sequence_workspace_bytes(&a);
+            char* memory = (char*)devices::rocm::scratch(device, intermediates + workspace_bytes + 256);
+            memory = attach_intermediates(d.actor, T * B, memory);
+            memory = attach_intermediates(d.targets[0], T * B, memory);
+            memory = attach_intermediates(d.targets[1], T * B, memory);
+            a.workspace = memory; a.workspace_bytes = workspace_bytes;
+            devices::rocm::check(rlt_rocm_sac_sequence_train_critics(device.handle, &a, action_noise._data), "train_critic x 2 (sequences)");
+            return true;
+        }
     }
     // train_actor             rl/algorithms/sac/operations_generic.h:395-468 on a sequence batch
     template <typename DEV_SPEC, typename SPEC, typename BATCH_SPEC, typename OPTIMIZER, typename ACTOR_BUFFERS, typename CRITIC_BUFFERS, typename TRAINING_BUFFERS_SPEC, typename ACTION_NOISE_SPEC, typename RNG,

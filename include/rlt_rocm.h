@@ -950,6 +950,11 @@ size_t rlt_rocm_sac_sequence_workspace_bytes(const rlt_sac_sequence_agent* agent
  *   As in the reference, the target of step t takes the target critics' value of step t + 1 but the entropy bonus from the
  *   log-probability at index t of the evaluated `next` steps (operations_generic.h:144-154). */
 int rlt_rocm_sac_sequence_train_critic(rlt_rocm_device* device, const rlt_sac_sequence_agent* agent, int critic_index, const float* action_noise);
+/* train_critic for critic 0, then for critic 1, on the agent's batch with the same noise: the loop's SHARED_BATCH case (rl/algorithms/sac/loop/core/operations_generic.h:127-138,
+ * where the second call repeats the actor's pass over the next rows, its sample, both target critics and the target values on unchanged inputs). Those are computed
+ * once here, the two critics' own passes run next to each other on the handle's two streams, and the results are those of the two calls bit for bit (critic 1's loss
+ * gradient is left in agent->d_output, as they leave it; critic 0's goes to the end of the workspace). */
+int rlt_rocm_sac_sequence_train_critics(rlt_rocm_device* device, const rlt_sac_sequence_agent* agent, const float* action_noise);
 /* update_critic_targets   sac/operations_generic.h:486-527 (dense and GRU layers, incl. the initial hidden state) */
 int rlt_rocm_sac_sequence_update_critic_targets(rlt_rocm_device* device, const rlt_sac_sequence_agent* agent);
 /* train_actor on a sequence batch   sac/operations_generic.h:395-468; action_noise [S x B x action_dim] */

@@ -647,11 +647,13 @@ class SacSequenceOnBackend:
         for k in SEQUENCE_BATCH_FIELDS:
             self.batch.arrays[k].upload(data[k])
 
-    def train(self, noise_critic, noise_actor):
+    def train(self, noise_critic, noise_actor, both_critics_in_one_call=False):
         """The training part of one loop step with a shared batch (rl/algorithms/sac/loop/core/operations_generic.h:127-154)."""
         be = self.backend
         nc, na = be.array(np.ascontiguousarray(noise_critic, np.float32)), be.array(np.ascontiguousarray(noise_actor, np.float32))
-        for k in range(2):
+        if both_critics_in_one_call:
+            be.call("sac_sequence_train_critics", C.byref(self.c), nc.ptr)
+        for k in range(0 if both_critics_in_one_call else 2):
             be.call("sac_sequence_train_critic", C.byref(self.c), k, nc.ptr)
         be.call("sac_sequence_update_critic_targets", C.byref(self.c))
         be.call("sac_sequence_train_actor", C.byref(self.c), na.ptr)

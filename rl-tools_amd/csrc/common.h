@@ -30,13 +30,15 @@ struct rlt_rocm_device {
     hipStream_t side_stream;     // a second stream (default priority) for passes that do not depend on what the main stream does next (rlt_side_begin)
     hipEvent_t fork_event, join_event;
     hipStream_t side_return;     // the stream to switch back to while work goes to the side stream (null otherwise)
+    void* side_scratch; size_t side_scratch_bytes;      // what rlt_scratch hands out while work goes to the side stream: passes that run at the same time do not share split sums
 };
 
 // Network passes that are independent of each other (the two target critics of a sequence update, a critic's forward pass and the actor's) overlap on two
 // streams: between rlt_side_begin and rlt_side_end every launch of the library goes to the handle's side stream, which first waits for everything enqueued
 // on the main stream so far; rlt_side_join makes the main stream wait for the side stream. While the main stream records a graph (or if the side stream could
-// not be made) rlt_side_begin returns false and the work simply stays on the main stream, in order. Passes that run at the same time must not share a workspace,
-// and only one of them may form weight gradients (their split sums use the handle's one scratch buffer).
+// not be made) rlt_side_begin returns false and the work simply stays on the main stream, in order. Passes that run at the same time must not share a workspace;
+// the handle's scratch buffer (rlt_scratch: split sums of weight gradients) has a second instance for the side stream. The ticket counters (rlt_counters) have not:
+// optimiser steps stay on the main stream.
 bool rlt_side_begin(rlt_rocm_device* device);
 void rlt_side_end(rlt_rocm_device* device);
 int rlt_side_join(rlt_rocm_device* device);

@@ -30,15 +30,17 @@ int rlt_side_join(rlt_rocm_device* device) {
     return 0;
 }
 int rlt_scratch(rlt_rocm_device* device, size_t bytes, void** out) {
-    if (bytes > device->scratch_bytes) {
+    void*& buffer = device->side_return ? device->side_scratch : device->scratch;       // work that goes to the side stream has a scratch buffer of its own
+    size_t& have = device->side_return ? device->side_scratch_bytes : device->scratch_bytes;
+    if (bytes > have) {
         if (device->capturing) return RLT_E_CAPTURING;      // the workspace grows on a warm-up call before the capture
-        if (device->scratch) RLT_HIP(hipFree(device->scratch));   // hipFree waits for the work that still uses it
-        device->scratch = nullptr; device->scratch_bytes = 0;
+        if (buffer) RLT_HIP(hipFree(buffer));   // hipFree waits for the work that still uses it
+        buffer = nullptr; have = 0;
         size_t want = bytes < (size_t)(1u << 20) ? (size_t)(1u << 20) : bytes + bytes / 4;
-        RLT_HIP(hipMalloc(&device->scratch, want));
-        device->scratch_bytes = want;
+        RLT_HIP(hipMalloc(&buffer, want));
+        have = want;
     }
-    *out = device->scratch;
+    *out = buffer;
     return 0;
 }
 
@@ -209,6 +211,7 @@ int rlt_rocm_destroy(rlt_rocm_device* device) {
     }
     if (device->scratch) (void)hipFree(device->scratch);
     if (device->pad_scratch) (void)hipFree(device->pad_scratch);
+    if (device->side_scratch) (void)hipFree(device->side_scratch);
     if (device->counters) (void)hipFree(device->counters);
     (void)hipStreamDestroy(device->own_stream);
     delete device;

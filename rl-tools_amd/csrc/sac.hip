@@ -436,7 +436,8 @@ static size_t sequence_pass_workspace_bytes(const rlt_sac_sequence_agent* A, int
 size_t rlt_rocm_sac_sequence_workspace_bytes(const rlt_sac_sequence_agent* A) {
     if (!A || !A->actor || !A->critics[0] || !A->critics_target[0]) return 0;
     const int T = A->batch.sequence_length + 1, B = A->batch.batch;
-    return 2 * sequence_pass_workspace_bytes(A, T, B);      // two passes may run at the same time (rlt_side_begin), each in its own half
+    // two passes may run at the same time (rlt_side_begin), each in its own half; then the loss gradient of the first critic where both critics train in one call
+    return 2 * sequence_pass_workspace_bytes(A, T, B) + ((sizeof(float) * (size_t)A->batch.sequence_length * B + 255) & ~(size_t)255);
 }
 
 // rl/algorithms/sac/operations_generic.h:243-337 on a sequence batch, one launch per reference operation
@@ -486,6 +487,68 @@ int rlt_rocm_sac_sequence_train_critic(rlt_rocm_device* device, const rlt_sac_se
     if ((rc = rlt_launch_status(device))) return rc;
     if ((rc = rlt_rocm_seq_backward(device, critic, A->n_critic_layers, K.observations_actions_base, D, A->d_output, nullptr, K.reset, S, B, 1, 0, ws, ws_bytes))) return rc;   // :329
     return rlt_rocm_adam_step(device, A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], 0.0f, nullptr);   // :336
+}
+
+// Both critics on one batch and one set of noise (the loop's SHARED_BATCH case, rl/algorithms/sac/loop/core/operations_generic.h:127-138): what the two calls of
+// train_critic would compute twice -- the actor on the next rows, its sample, both target critics, the target values -- is computed once, and the two critics'
+// passes run next to each other on the handle's two streams: side stream critic 0 forward, then target critic 1; main stream actor, sample, target critic 0, critic 1
+// forward; after the join the target values and both loss gradients, then critic 0's backward pass on the main stream next to critic 1's on the side stream, then
+// both optimisers. Every pass is the launch sequence that the single calls make, on the same inputs: the results are theirs bit for bit.
+int rlt_rocm_sac_sequence_train_critics(rlt_rocm_device* device, const rlt_sac_sequence_agent* A, const float* action_noise) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(sequence_agent_ok(A) && action_noise);
+    RLT_REQUIRE(A->next_state_action_value_input && A->next_q[0] && A->next_q[1] && A->next_log_probabilities && A->target_action_value && A->d_output);
+    const rlt_sequence_batch& K = A->batch;
+    const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    const int first = A->include_first_step_in_targets ? 1 : 0, T = S + first, next_offset = first ? 0 : 1;
+    const size_t ws_bytes = sequence_pass_workspace_bytes(A, S + 1, B);
+    void* ws = A->workspace; void* ws_side = (char*)A->workspace + ws_bytes;
+    float* d_output_first = (float*)((char*)A->workspace + 2 * ws_bytes);      // critic 0's loss gradient; critic 1's goes to the agent's buffer, where two single calls leave it
+    const bool overlap = S >= 48;      // short sequences: a pass is shorter than the two events that fork and join a stream cost on the host
+    int rc;
+    for (int k = 0; k < 2; k++) if ((rc = rlt_rocm_seq_zero_gradient(device, A->critics[k], A->n_critic_layers))) return rc;
+    {
+        if (overlap) rlt_side_begin(device);      // (without a second stream everything below simply runs in order on the one stream)
+        rc = rlt_rocm_seq_forward(device, A->critics[0], A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, device->side_return ? ws_side : ws, ws_bytes);
+        rlt_side_end(device);
+        if (rc) return rc;
+    }
+    const float* base_next = K.observations_actions_base + (size_t)next_offset * B * D;
+    const uint8_t* next_reset = K.next_reset_base + (size_t)next_offset * B;
+    const uint8_t* next_final = K.next_final_step_mask_base + (size_t)next_offset * B;
+    if ((rc = rlt_rocm_seq_forward(device, A->actor, A->n_actor_layers, base_next, D, next_reset, T, B, ws, ws_bytes))) return rc;
+    float* next_actions = A->next_state_action_value_input + OBS;
+    if ((rc = rlt_rocm_sas_forward(device, &A->sas, seq_output(A->actor, A->n_actor_layers), 2 * ACT, action_noise, ACT, next_actions, D, nullptr, 0,
+                                   A->next_log_probabilities, T * B, ACT))) return rc;
+    if ((rc = rlt_rocm_mask_copy(device, base_next + OBS, D, next_actions, D, next_final, 1, T * B, ACT))) return rc;
+    if ((rc = copy2d(device, base_next, D, A->next_state_action_value_input, D, T * B, OBS))) return rc;
+    for (int k = 1; k >= 0; k--) {      // target critic 1 behind critic 0's forward pass on the side stream (it waits for the copies above), target critic 0 on the main stream
+        if (k == 1 && overlap) rlt_side_begin(device);
+        rc = rlt_rocm_seq_forward(device, A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, next_reset, T, B, device->side_return ? ws_side : ws, ws_bytes);
+        if (!rc) rc = rlt_rocm_memcpy_d2d(device, A->next_q[k], seq_output(A->critics_target[k], A->n_critic_layers), sizeof(float) * T * B);
+        rlt_side_end(device);
+        if (rc) return rc;
+    }
+    if ((rc = rlt_rocm_seq_forward(device, A->critics[1], A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, ws, ws_bytes))) return rc;
+    if (overlap && (rc = rlt_side_join(device))) return rc;
+    if ((rc = rlt_rocm_sac_target_action_values(device, A->next_q[0] + first * B, A->next_q[1] + first * B, K.rewards, K.terminated, A->next_log_probabilities,
+                                               A->log_alpha.parameters, A->gamma, 0, A->target_action_value, S * B))) return rc;
+    for (int k = 0; k < 2; k++) {
+        hipLaunchKernelGGL(sac_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, seq_output(A->critics[k], A->n_critic_layers), (const float*)A->target_action_value,
+                           (const uint8_t*)K.final_step_mask, k ? A->d_output : d_output_first, S * B, 0);
+        if ((rc = rlt_launch_status(device))) return rc;
+    }
+    {
+        if (overlap) rlt_side_begin(device);
+        rc = rlt_rocm_seq_backward(device, A->critics[1], A->n_critic_layers, K.observations_actions_base, D, A->d_output, nullptr, K.reset, S, B, 1, 0, device->side_return ? ws_side : ws, ws_bytes);
+        rlt_side_end(device);
+        if (rc) return rc;
+    }
+    if ((rc = rlt_rocm_seq_backward(device, A->critics[0], A->n_critic_layers, K.observations_actions_base, D, d_output_first, nullptr, K.reset, S, B, 1, 0, ws, ws_bytes))) return rc;
+    if (overlap && (rc = rlt_side_join(device))) return rc;
+    for (int k = 0; k < 2; k++)
+        if ((rc = rlt_rocm_adam_step(device, A->critic_adam_tensors[k], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[k], 0.0f, nullptr))) return rc;
+    return 0;
 }
 
 // sac/operations_generic.h:486-527

@@ -135,6 +135,34 @@ def test_sac_sequence_updates_at_larger_shapes(oracle, rocm, case):
         compare_agents(agents[1], agents[0], (case, i), tol=2e-5)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", [(100, 100, 3, 1, 32, True), (10, 100, 5, 2, 32, False), (48, 64, 11, 3, 64, True)])
+def test_both_critics_in_one_call_leave_the_bits_of_the_two_calls(rocm, case):
+    """rlt_rocm_sac_sequence_train_critics (the target part once, the two critics' passes side by side on the handle's two streams from 48 steps up) against
+    rlt_rocm_sac_sequence_train_critic for critic 0 and then for critic 1: three loop steps each from the same parameters, batches and noise; every parameter and the
+    training buffers that both leave behind, bit for bit."""
+    S, B, OBS, ACT, H, first = case
+    rng = np.random.default_rng(S * 3 + B)
+    actor_specs = [(0, OBS, H, "relu"), (1, H, H, "identity"), (0, H, 2 * ACT, "identity")]
+    critic_specs = [(0, OBS + ACT, H, "relu"), (1, H, H, "identity"), (1, H, H, "identity"), (0, H, 1, "identity")]
+    critics = [helpers.random_seq_params(rng, critic_specs) for _ in range(2)]
+    params = np.concatenate([helpers.random_seq_params(rng, actor_specs)] + critics + [c.copy() * 0.9 for c in critics] + [np.array([np.log(0.5)], np.float32)])
+    hyper = dict(sas=helpers.capi.SasParameters(-20.0, 2.0, 1e-6, -float(ACT)))
+    agents = [helpers.SacSequenceOnBackend(rocm, actor_specs, critic_specs, params, S, B, OBS, ACT, first, hyper) for _ in range(2)]
+    T = S + 1 if first else S
+    for i in range(3):
+        data = synthetic_sequence_batch(rng, S, B, OBS + ACT)
+        nc, na = rng.standard_normal((T, B, ACT)).astype(np.float32), rng.standard_normal((S, B, ACT)).astype(np.float32)
+        for a, together in zip(agents, (False, True)):
+            a.set_batch(data); a.train(nc, na, both_critics_in_one_call=together)
+        assert np.array_equal(agents[0].parameters(), agents[1].parameters()), (case, i)
+        for key in ("target", "d_output", "next_q0", "next_q1", "next_lp", "nsavi"):
+            if key in agents[0].buf:
+                assert np.array_equal(agents[0].buf[key].numpy(), agents[1].buf[key].numpy()), (case, i, key)
+        assert agents[0].ages() == agents[1].ages()
+    assert np.abs(agents[1].parameters() - params).max() > 1e-4
+
+
 def test_sac_sequence_of_length_one_equals_single_step_update_on_device(rocm):
     """Sequence length 1, dense layers only, every step final: the sequence entry points and the single-step entry points of the same library."""
     rng = np.random.default_rng(5)
