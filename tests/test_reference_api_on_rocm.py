@@ -332,7 +332,7 @@ def test_recurrent_sac_loop_trains_on_rocm():
     and sequence batches of 16 steps x 32 samples from four environments, on devices::ROCM: gather_batch's multi-step branch with its draws made on the
     device, the runner step with the policy state reset by the truncation mask and evaluate_step, train_critic / train_actor as one call each of the library's
     entry points for sequence batches, the evaluation loop step with the recurrent actor on the device. A random actor's mean
-    return is about -1,300; measured -290 after 3,000 loop steps, at 1,380 loop steps/s including the evaluations (the same program on
+    return is about -1,300; measured -293 after 3,000 loop steps, at 1,660 loop steps/s including the evaluations (the same program on
     the reference's CPU device: 190)."""
     path = os.path.join(BUILD, "rocm_sac_gru_pendulum")
     if not os.path.exists(path):
@@ -343,7 +343,7 @@ def test_recurrent_sac_loop_trains_on_rocm():
     returns = [float(x) for x in re.findall(r"mean_return ([\d.e+-]+)", out.stdout)]
     final = re.search(r"final ([\d.e+-]+) loop_steps_per_second_including_evaluations ([\d.e+-]+)", out.stdout)
     assert returns[0] < -900.0 and max(returns + [float(final.group(1))]) >= -600.0
-    assert imports(path, "rlt_rocm_sac_sequence_train_critic", "rlt_rocm_sac_sequence_train_actor", "rlt_rocm_gather_sequence_batch", "rlt_rocm_pendulum_runner_step_recurrent", "rlt_rocm_pendulum_evaluate_recurrent")
+    assert imports(path, "rlt_rocm_sac_sequence_train_critics", "rlt_rocm_sac_sequence_train_actor", "rlt_rocm_gather_sequence_batch", "rlt_rocm_pendulum_runner_step_recurrent", "rlt_rocm_pendulum_evaluate_recurrent")
 
 
 @pytest.mark.gpu
