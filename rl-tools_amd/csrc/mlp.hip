@@ -6,6 +6,7 @@
 #include "mlp_fused.h"
 #include "mlp_small.h"
 #include "mlp_rows.h"
+#include "sac_update.h"
 
 namespace {
 
@@ -24,6 +25,8 @@ constexpr int FUSED_MIN_BATCH = 1024;
 bool rows_enabled() { return rlt_mlp_rows_enabled(); }
 // RLT_MLP_SINGLE_PASS=0 keeps forward() / backward() on the per-layer kernels (tests compare the two paths with each other)
 bool single_pass_enabled() { const char* v = std::getenv("RLT_MLP_SINGLE_PASS"); return !(v && v[0] == '0'); }
+// RLT_MLP_WIDE=0 keeps forward + backward calls of a few thousand rows off the sixteen-row-tile kernel (tests and measurements compare the paths)
+bool wide_enabled() { const char* v = std::getenv("RLT_MLP_WIDE"); return !(v && v[0] == '0'); }
 bool chain_ok(const rlt_dense_layer* layers, int n) {
     if (!layers || n < 1) return false;
     for (int i = 0; i < n; i++) { if (!layer_ok(&layers[i])) return false; if (i > 0 && layers[i].in_dim != layers[i - 1].out_dim) return false; }
@@ -240,14 +243,22 @@ static int forward_backward_impl(rlt_rocm_device* device, const rlt_dense_layer*
     RLT_REQUIRE((!y || ldy >= O) && (!d_output || ldd >= O) && (!target || ldt >= O) && (!d_input || ldi >= layers[0].in_dim));
     for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases);
     RLT_REQUIRE(workspace && workspace_bytes >= rlt_rocm_mlp_workspace_bytes(layers, n, batch));
-    if (!d_input && batch >= FUSED_MIN_BATCH) {
-        // one pass over the batch with on-chip activations where the network has the shape that kernel is built for (below that batch size its three launches
-        // and the per-call copy of the weights cost more than the per-layer path)
+    if (!d_input && batch > RLT_MLP_WIDE_MAX_BATCH) {
+        // one pass over the batch with on-chip activations where the network has the shape that kernel is built for
         const int rc = rlt_mlp3_fused_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, workspace, workspace_bytes);
         if (rc != RLT_E_UNSUPPORTED) return rc;
     }
     if (single_pass_enabled()) {
-        const int rc = rlt_mlp3s_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, d_input, ldi);
+        int rc = rlt_mlp3s_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, d_input, ldi);
+        if (rc != RLT_E_UNSUPPORTED) return rc;
+        // a few thousand rows at most, hidden widths up to 256: sixteen-row tiles, one workgroup each (the 64-row tiles of the kernel above leave most of the chip idle there)
+        if (!d_input && wide_enabled()) {
+            rc = rlt_mlp_wide_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch);
+            if (rc != RLT_E_UNSUPPORTED) return rc;
+        }
+    }
+    if (!d_input && batch >= FUSED_MIN_BATCH) {
+        const int rc = rlt_mlp3_fused_forward_backward(device, layers, n, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, workspace, workspace_bytes);
         if (rc != RLT_E_UNSUPPORTED) return rc;
     }
     // carve private activation storage out of the workspace

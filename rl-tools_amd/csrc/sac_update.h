@@ -34,3 +34,10 @@ int rlt_td3_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, co
 bool rlt_td3_wide_supported(const rlt_rocm_device* device, const rlt_td3_agent* agent);
 int rlt_td3_wide_update_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
 int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise);
+
+// forward + backward (with weight gradients, added onto the layers' gradients) of one three-layer network of hidden width up to 256 over at most RLT_MLP_WIDE_MAX_BATCH
+// rows on the wide update kernels' machinery (sac_wide.hip): input width up to 128, output width up to 16, no output activation. d_output or target (the MSE's
+// gradient (y - target) * mse_scale) as in rlt_rocm_mlp_forward_backward. RLT_E_UNSUPPORTED for any other network.
+constexpr int RLT_MLP_WIDE_MAX_BATCH = 4096;
+int rlt_mlp_wide_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy,
+                                  const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch);

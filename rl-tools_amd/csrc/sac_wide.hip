@@ -611,6 +611,133 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
 
 constexpr size_t LDS_FLOATS = (size_t)2 * ROWS * SXS + 4 * ROWS * S + 4 * ROWS * D3S + WAVES * YP + MISC;
 
+// ---- Forward and backward pass of one three-layer network over a few thousand rows at most, on the same machinery (nn_models/mlp/operations_generic.h:103-204: forward, the
+// loss gradient given or formed from a target as the MSE's, backward with weight gradients): a workgroup takes 16 rows through the three layers and back, the activations
+// never leave LDS, and writes one block of partial sums [dW1 | db1 | dW2 | db2 | dW3 | db3]; mlp_wide_reduce_kernel adds the blocks up in workgroup order onto the layers'
+// gradients. Where a batch is too small to fill the chip with the 64-row tiles of the one-pass kernel for large batches (mlp_fused.hip: 4,096 rows are 64 tiles for 256
+// compute units, and a tile takes its 74 us whatever the batch), sixteen-row tiles are a launch of 256 workgroups.
+struct MlpWideArgs {
+    WNet net;
+    const float* x; int ldx; float* y; int ldy;
+    const float* d_output; int ldd; const float* target; int ldt; float mse_scale;
+    int batch;
+    float* partial; int count;
+};
+template <int ACT_H, int NT1C>
+__global__ __launch_bounds__(THREADS) void mlp_wide_kernel(MlpWideArgs A) {
+    extern __shared__ __attribute__((aligned(16))) float lds_wide[];
+    const int gi = blockIdx.x;
+    const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const lptr xa = (lptr)lds_wide, h1 = xa + 2 * ROWS * SXS, h2 = h1 + ROWS * S, ta = h2 + ROWS * S, tb = ta + ROWS * S, d3 = tb + ROWS * S, yp = d3 + 4 * ROWS * D3S;
+    const WNet N = A.net;
+    const int B = A.batch, IN = N.in, HID = N.hid, OUT = N.out, tiles = (HID + 15) >> 4, row0 = gi * ROWS;
+    const bool on = wave < tiles;
+    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    for (int e = threadIdx.x; e < ROWS * SXS; e += THREADS) {
+        const int r = e / SXS, k = e % SXS;
+        xa[e] = (row0 + r < B && k < IN) ? A.x[(size_t)(row0 + r) * A.ldx + k] : 0.f;
+    }
+    rlt_lds_barrier();
+    forward3_own_loads<ACT_H, NT1C>(N, xa, SXS, h1, h2, yp, wave, c, g);
+    float s3 = 0.f;
+    if (wave == 0) {
+        // lane (c, g): output column c of rows 4 g + v; the gradient at the output (the last layer has no activation): given, or the MSE's against the target
+        const floatx4 out = output_tile(yp, tiles, c, g);
+        const float b3 = c < OUT ? N.b3[c] : 0.f;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int row = row0 + 4 * g + v;
+            const bool ok = c < OUT && row < B;
+            const float yv = out[v] + b3;
+            if (ok && A.y) A.y[(size_t)row * A.ldy + c] = yv;
+            float d = 0.f;
+            if (ok) d = A.target ? (yv - A.target[(size_t)row * A.ldt + c]) * A.mse_scale : A.d_output[(size_t)row * A.ldd + c];
+            d3[(4 * g + v) * D3S + c] = d;
+            s3 += d;
+        }
+    }
+    rlt_lds_barrier();      // d_pre3 is in place
+    // backward pass with the weight gradients over the workgroup's 16 rows: ta receives d_pre2, tb receives d_pre1
+    float* dst = A.partial + (size_t)gi * A.count;
+    const int NT1 = (IN + 15) >> 4;
+    const int o_b1 = HID * IN, o_w2 = o_b1 + HID, o_b2 = o_w2 + HID * HID, o_w3 = o_b2 + HID, o_b3 = o_w3 + OUT * HID;
+    const int n = 16 * wave + c;
+    const bool n_ok = n < HID;
+    float s2 = 0.f;
+    if (on) {
+        floatx4 aW3 = zero4;
+#pragma unroll
+        for (int ks = 0; ks < ROWS / 4; ks++) aW3 = mfma16(d3[(4 * ks + g) * D3S + c], h2[(4 * ks + g) * S + n], aW3);
+#pragma unroll
+        for (int v = 0; v < 4; v++)
+            if (4 * g + v < OUT && n_ok) dst[o_w3 + (4 * g + v) * HID + n] = aW3[v];
+        s2 = backward_layer3<ACT_H>(N, d3, h2, ta, wave, c, g);
+    }
+    rlt_lds_barrier();      // every wavefront's tile of d_pre2 is in place
+    if (on) {
+        {   // dW2: this wavefront's units' rows
+            float a[4];
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) a[ks] = ta[(4 * ks + g) * S + n];
+#pragma unroll 4
+            for (int nt = 0; nt < tiles; nt++) {
+                floatx4 acc = zero4;
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) acc = mfma16(a[ks], h1[(4 * ks + g) * S + 16 * nt + c], acc);
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int m = 16 * wave + 4 * g + v;
+                    if (m < HID && 16 * nt + c < HID) dst[o_w2 + (size_t)m * HID + 16 * nt + c] = acc[v];
+                }
+            }
+        }
+        float s1 = backward_layer2<ACT_H>(N, ta, h1, tb, wave, c, g);
+        wave_sync();            // dW1's rows are this wavefront's own tile of d_pre1
+        {
+            float a[4];
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) a[ks] = tb[(4 * ks + g) * S + n];
+#pragma unroll 2
+            for (int nt = 0; nt < NT1; nt++) {
+                floatx4 acc = zero4;
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) acc = mfma16(a[ks], xa[(4 * ks + g) * SXS + 16 * nt + c], acc);
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int m = 16 * wave + 4 * g + v;
+                    if (m < HID && 16 * nt + c < IN) dst[(size_t)m * IN + 16 * nt + c] = acc[v];
+                }
+            }
+        }
+        s1 = groups_sum(s1); s2 = groups_sum(s2);
+        if (g == 0 && n_ok) { dst[o_b1 + n] = s1; dst[o_b2 + n] = s2; }
+    }
+    if (wave == 0) {
+        s3 = groups_sum(s3);
+        if (g == 0 && c < OUT) dst[o_b3 + c] = s3;
+    }
+}
+// gradient[e] += the sum over the workgroups' blocks of element e, in workgroup order; thread = one element, sixteen blocks' loads in flight
+struct WideReduceArgs { const float* partial; int blocks, count, total; float* dst[6]; int end[6]; };
+__global__ __launch_bounds__(256) void mlp_wide_reduce_kernel(WideReduceArgs R) {
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= R.total) return;
+    float sum = 0.f;
+    for (int b0 = 0; b0 < R.blocks; b0 += 16) {
+        float v[16];
+#pragma unroll
+        for (int u = 0; u < 16; u++) v[u] = b0 + u < R.blocks ? R.partial[(size_t)(b0 + u) * R.count + e] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 16; u++) sum += v[u];
+    }
+    int k = 0, begin = 0;
+#pragma unroll
+    for (int q = 0; q < 5; q++) if (e >= R.end[q]) { k = q + 1; begin = R.end[q]; }
+    float* const dst = k == 0 ? R.dst[0] : k == 1 ? R.dst[1] : k == 2 ? R.dst[2] : k == 3 ? R.dst[3] : k == 4 ? R.dst[4] : R.dst[5];
+    dst[e - begin] += sum;
+}
+
 bool hidden_ok(int a) { return a == RLT_ACT_RELU || a == RLT_ACT_TANH || a == RLT_ACT_FAST_TANH || a == RLT_ACT_SIGMOID; }
 bool net_ok(const rlt_dense_layer* L, int n, int in, int out, int& hid, int last_activation = RLT_ACT_IDENTITY) {
     if (!L || n != 3) return false;
@@ -859,6 +986,56 @@ int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* A, c
     a.out_pre_clip = A->actor_pre_clip;
     const Optimiser O = {A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, nullptr, nullptr, nullptr, 0.0f, nullptr};
     return launch_wide<MODE_TD3_ACTOR>(device, a, rlt_div_up(A->batch, ROWS), &O, 1, 0.0f, nullptr);
+}
+
+
+// ---- forward + backward of a three-layer network on sixteen-row tiles (see mlp_wide_kernel); RLT_E_UNSUPPORTED: the caller takes another path
+int rlt_mlp_wide_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n_layers, const float* x, int ldx, float* y, int ldy,
+                                  const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch) {
+    if (n_layers != 3 || batch < 1 || batch > RLT_MLP_WIDE_MAX_BATCH || L[0].in_dim < 1 || L[0].in_dim > MAX_D || L[2].out_dim < 1 || L[2].out_dim > MAX_OUT) return RLT_E_UNSUPPORTED;
+    int hid = 0;
+    if (!net_ok(L, 3, L[0].in_dim, L[2].out_dim, hid)) return RLT_E_UNSUPPORTED;
+    for (int l = 0; l < 3; l++) if (!L[l].d_weights || !L[l].d_biases) return RLT_E_UNSUPPORTED;
+    if (LDS_FLOATS * sizeof(float) > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
+    MlpWideArgs a = {};
+    a.net = net_of(L);
+    a.x = x; a.ldx = ldx; a.y = y; a.ldy = ldy; a.d_output = d_output; a.ldd = ldd; a.target = target; a.ldt = ldt; a.mse_scale = mse_scale; a.batch = batch;
+    const int IN = L[0].in_dim, OUT = L[2].out_dim, groups = rlt_div_up(batch, ROWS);
+    const int exact = hid * IN + hid + hid * hid + hid + OUT * hid + OUT;
+    a.count = (exact + 63) & ~63;
+    const size_t copy_floats = (size_t)256 * WAVES * WAVES;
+    const size_t partial_bytes = ((size_t)groups * a.count * sizeof(float) + 255) & ~(size_t)255;
+    void* scratch = nullptr;
+    int rc = rlt_scratch(device, partial_bytes + 2 * copy_floats * sizeof(float), &scratch);
+    if (rc) return rc;
+    a.partial = (float*)scratch;
+    {
+        PrepArgs P = {};
+        float* copies = (float*)((char*)scratch + partial_bytes);
+        for (int q = 0; q < 2; q++) { P.W2[q] = a.net.W2; P.dst[q] = copies + (size_t)q * copy_floats; P.hid[q] = hid; P.backward[q] = q; }
+        a.net.W2f = P.dst[0]; a.net.W2b = P.dst[1];
+        const int tiles = (hid + 15) >> 4;
+        hipLaunchKernelGGL(wide_prepare_kernel, dim3(rlt_div_up(tiles * tiles * 64, 256), 2), dim3(256), 0, device->stream, P);
+        if ((rc = rlt_launch_status(device))) return rc;
+    }
+    const size_t lds_bytes = LDS_FLOATS * sizeof(float);
+#define RLT_LAUNCH_MLP_WIDE(ACT, NT)                                                                                                                   \
+    do {                                                                                                                                               \
+        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp_wide_kernel<ACT, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
+        hipLaunchKernelGGL((mlp_wide_kernel<ACT, NT>), dim3(groups), dim3(THREADS), lds_bytes, device->stream, a);                                    \
+    } while (0)
+    const int act = a.net.act_h;
+    if (IN <= 32) { if (act == RLT_ACT_RELU) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, 2); else RLT_LAUNCH_MLP_WIDE(-1, 2); }
+    else { if (act == RLT_ACT_RELU) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, MAX_D / 16); else RLT_LAUNCH_MLP_WIDE(-1, MAX_D / 16); }
+#undef RLT_LAUNCH_MLP_WIDE
+    if ((rc = rlt_launch_status(device))) return rc;
+    WideReduceArgs R = {};
+    R.partial = a.partial; R.blocks = groups; R.count = a.count; R.total = exact;
+    float* const dst[6] = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases};
+    const int size[6] = {hid * IN, hid, hid * hid, hid, OUT * hid, OUT};
+    for (int k = 0, end = 0; k < 6; k++) { end += size[k]; R.dst[k] = dst[k]; R.end[k] = end; }
+    hipLaunchKernelGGL(mlp_wide_reduce_kernel, dim3(rlt_div_up(exact, 256)), dim3(256), 0, device->stream, R);
+    return rlt_launch_status(device);
 }
 
 #ifdef RLT_WIDE_PROFILE

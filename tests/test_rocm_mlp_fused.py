@@ -39,8 +39,9 @@ CASES = [
 
 
 @pytest.mark.parametrize("case", CASES)
-def test_fused_matches_checker(oracle, rocm, case):
+def test_fused_matches_checker(oracle, rocm, case, monkeypatch):
     print("case", case, flush=True)
+    monkeypatch.setenv("RLT_MLP_WIDE", "0")      # batches of at most 4,096 rows would take the sixteen-row tiles (tests/test_rocm_mlp_wide.py); this file is about the 64-row tiles
     B, I, O, ha, oa, use_target = case
     dims = [I, 256, 256, O]
     rng = np.random.default_rng(B * 31 + I)
@@ -56,7 +57,8 @@ def test_fused_matches_checker(oracle, rocm, case):
         assert ew <= TOL and eb <= TOL, (off, ew, eb)
 
 
-def test_fused_accumulates_and_tolerates_null_output(oracle, rocm):
+def test_fused_accumulates_and_tolerates_null_output(oracle, rocm, monkeypatch):
+    monkeypatch.setenv("RLT_MLP_WIDE", "0")
     dims = [17, 256, 256, 6]
     rng = np.random.default_rng(5)
     params = helpers.random_params(rng, dims)
