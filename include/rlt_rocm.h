@@ -942,8 +942,8 @@ typedef struct rlt_sac_sequence_agent {
 
 /* The sequence updates below run network passes that do not depend on each other at the same time -- the trained critic's forward pass next to the (target) actor's,
  * the second target critic next to the first, in train_actor the second critic's forward pass and input gradient next to the first's -- the second of each pair on a
- * stream of the handle's own that waits for, and is waited for by, the stream the calls are enqueued on (each recurrence fills about a twentieth of the chip). The
- * workspace is two halves for that reason. Results are those of the passes in sequence, bit for bit. While the stream records a graph the passes stay in sequence. */
+ * stream of the handle's own that waits for, and is waited for by, the stream the calls are enqueued on (each recurrence fills about a twentieth of the chip);
+ * rlt_rocm_sac_sequence_train_critics uses two such streams. The workspace is three parts for that reason. Results are those of the passes in sequence, bit for bit. While the stream records a graph the passes stay in sequence. */
 size_t rlt_rocm_sac_sequence_workspace_bytes(const rlt_sac_sequence_agent* agent);
 /* train_critic on a sequence batch   rl/algorithms/sac/operations_generic.h:243-337
  *   action_noise [T x B x action_dim]: the N(0,1) noise of the actor's sample_and_squash layer on the `next` views.

@@ -5,6 +5,7 @@
 #include <stddef.h>
 #include "../../include/rlt_rocm.h"
 
+constexpr int RLT_SIDE_STREAMS = 2;
 struct rlt_rocm_device {
     int hip_device;
     hipStream_t own_stream;
@@ -27,19 +28,22 @@ struct rlt_rocm_device {
     unsigned wait_limit;         // polls after which a workgroup gives up waiting for another (rlt_rocm_set_wait_limit; about a second by default)
     int capturing;               // the stream is recording a graph: nothing may allocate, free or wait (rlt_rocm_graph_begin_capture)
     uint64_t* stream_offset;     // device word added to the stream number of every draw made on the device (rlt_rocm_advance_streams)
-    hipStream_t side_stream;     // a second stream (default priority) for passes that do not depend on what the main stream does next (rlt_side_begin)
-    hipEvent_t fork_event, join_event;
-    hipStream_t side_return;     // the stream to switch back to while work goes to the side stream (null otherwise)
-    void* side_scratch; size_t side_scratch_bytes;      // what rlt_scratch hands out while work goes to the side stream: passes that run at the same time do not share split sums
+    // two more streams (default priority) for passes that do not depend on what the main stream does next (rlt_side_begin); side_stream[0] null: none could be made
+    hipStream_t side_stream[RLT_SIDE_STREAMS];
+    hipEvent_t fork_event[RLT_SIDE_STREAMS], join_event[RLT_SIDE_STREAMS];
+    int side_pending[RLT_SIDE_STREAMS];      // work has gone to the stream since the main stream last waited for it
+    hipStream_t side_return;     // the stream to switch back to while work goes to a side stream (null otherwise)
+    int side_active;             // which side stream that is
+    void* side_scratch[RLT_SIDE_STREAMS]; size_t side_scratch_bytes[RLT_SIDE_STREAMS];      // what rlt_scratch hands out while work goes to a side stream: passes that run at the same time do not share split sums
 };
 
-// Network passes that are independent of each other (the two target critics of a sequence update, a critic's forward pass and the actor's) overlap on two
-// streams: between rlt_side_begin and rlt_side_end every launch of the library goes to the handle's side stream, which first waits for everything enqueued
-// on the main stream so far; rlt_side_join makes the main stream wait for the side stream. While the main stream records a graph (or if the side stream could
-// not be made) rlt_side_begin returns false and the work simply stays on the main stream, in order. Passes that run at the same time must not share a workspace;
+// Network passes that are independent of each other (the two target critics of a sequence update, a critic's forward pass and the actor's) overlap on up to
+// three streams: between rlt_side_begin(device, which) and rlt_side_end every launch of the library goes to the handle's side stream `which`, which first waits
+// for everything enqueued on the main stream so far; rlt_side_join makes the main stream wait for every side stream that has received work. While the main stream
+// records a graph (or if the side streams could not be made) rlt_side_begin returns false and the work simply stays on the main stream, in order. Passes that run at the same time must not share a workspace;
 // the handle's scratch buffer (rlt_scratch: split sums of weight gradients) has a second instance for the side stream. The ticket counters (rlt_counters) have not:
 // optimiser steps stay on the main stream.
-bool rlt_side_begin(rlt_rocm_device* device);
+bool rlt_side_begin(rlt_rocm_device* device, int which = 0);
 void rlt_side_end(rlt_rocm_device* device);
 int rlt_side_join(rlt_rocm_device* device);
 

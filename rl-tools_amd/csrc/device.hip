@@ -13,25 +13,30 @@ int rlt_launch_status(rlt_rocm_device* device) {
     return 0;
 }
 
-bool rlt_side_begin(rlt_rocm_device* device) {
-    if (!device->side_stream || device->capturing || device->side_return) return false;
-    if (hipEventRecord(device->fork_event, device->stream) != hipSuccess || hipStreamWaitEvent(device->side_stream, device->fork_event, 0) != hipSuccess) { (void)hipGetLastError(); return false; }
+bool rlt_side_begin(rlt_rocm_device* device, int which) {
+    if (which < 0 || which >= RLT_SIDE_STREAMS || !device->side_stream[which] || device->capturing || device->side_return) return false;
+    if (hipEventRecord(device->fork_event[which], device->stream) != hipSuccess || hipStreamWaitEvent(device->side_stream[which], device->fork_event[which], 0) != hipSuccess) { (void)hipGetLastError(); return false; }
     device->side_return = device->stream;
-    device->stream = device->side_stream;
+    device->side_active = which;
+    device->side_pending[which] = 1;
+    device->stream = device->side_stream[which];
     return true;
 }
 void rlt_side_end(rlt_rocm_device* device) {
     if (device->side_return) { device->stream = device->side_return; device->side_return = nullptr; }
 }
 int rlt_side_join(rlt_rocm_device* device) {
-    if (!device->side_stream) return 0;
-    RLT_HIP(hipEventRecord(device->join_event, device->side_stream));
-    RLT_HIP(hipStreamWaitEvent(device->stream, device->join_event, 0));
+    for (int k = 0; k < RLT_SIDE_STREAMS; k++) {
+        if (!device->side_stream[k] || !device->side_pending[k]) continue;
+        RLT_HIP(hipEventRecord(device->join_event[k], device->side_stream[k]));
+        RLT_HIP(hipStreamWaitEvent(device->stream, device->join_event[k], 0));
+        device->side_pending[k] = 0;
+    }
     return 0;
 }
 int rlt_scratch(rlt_rocm_device* device, size_t bytes, void** out) {
-    void*& buffer = device->side_return ? device->side_scratch : device->scratch;       // work that goes to the side stream has a scratch buffer of its own
-    size_t& have = device->side_return ? device->side_scratch_bytes : device->scratch_bytes;
+    void*& buffer = device->side_return ? device->side_scratch[device->side_active] : device->scratch;       // work that goes to a side stream has a scratch buffer of its own
+    size_t& have = device->side_return ? device->side_scratch_bytes[device->side_active] : device->scratch_bytes;
     if (bytes > have) {
         if (device->capturing) return RLT_E_CAPTURING;      // the workspace grows on a warm-up call before the capture
         if (buffer) RLT_HIP(hipFree(buffer));   // hipFree waits for the work that still uses it
@@ -182,10 +187,13 @@ int rlt_rocm_init(int hip_device_index, rlt_rocm_device** out_device) {
         device->update_one_xcd = !(q && std::strcmp(q, "spread") == 0);
         device->wait_limit = 1u << 20;
     }
-    // a second stream for independent passes; without it (or its events) everything stays on the one stream
-    if (hipStreamCreate(&device->side_stream) != hipSuccess) device->side_stream = nullptr;
-    if (device->side_stream && (hipEventCreateWithFlags(&device->fork_event, hipEventDisableTiming) != hipSuccess || hipEventCreateWithFlags(&device->join_event, hipEventDisableTiming) != hipSuccess)) {
-        (void)hipStreamDestroy(device->side_stream); device->side_stream = nullptr;
+    // streams for independent passes; without one (or its events) its work stays on the main stream
+    for (int k = 0; k < RLT_SIDE_STREAMS; k++) {
+        if (hipStreamCreate(&device->side_stream[k]) != hipSuccess) { device->side_stream[k] = nullptr; continue; }
+        if (hipEventCreateWithFlags(&device->fork_event[k], hipEventDisableTiming) != hipSuccess) { (void)hipStreamDestroy(device->side_stream[k]); device->side_stream[k] = nullptr; continue; }
+        if (hipEventCreateWithFlags(&device->join_event[k], hipEventDisableTiming) != hipSuccess) {
+            (void)hipEventDestroy(device->fork_event[k]); (void)hipStreamDestroy(device->side_stream[k]); device->side_stream[k] = nullptr;
+        }
     }
     (void)hipGetLastError();
     *out_device = device;
@@ -204,14 +212,15 @@ int rlt_rocm_set_wait_limit(rlt_rocm_device* device, unsigned polls) {
 int rlt_rocm_destroy(rlt_rocm_device* device) {
     if (!device) return RLT_E_INVALID_ARGUMENT;
     (void)hipStreamSynchronize(device->own_stream);
-    if (device->side_stream) {
-        (void)hipStreamSynchronize(device->side_stream);
-        (void)hipEventDestroy(device->fork_event); (void)hipEventDestroy(device->join_event);
-        (void)hipStreamDestroy(device->side_stream);
+    for (int k = 0; k < RLT_SIDE_STREAMS; k++) {
+        if (!device->side_stream[k]) continue;
+        (void)hipStreamSynchronize(device->side_stream[k]);
+        (void)hipEventDestroy(device->fork_event[k]); (void)hipEventDestroy(device->join_event[k]);
+        (void)hipStreamDestroy(device->side_stream[k]);
+        if (device->side_scratch[k]) (void)hipFree(device->side_scratch[k]);
     }
     if (device->scratch) (void)hipFree(device->scratch);
     if (device->pad_scratch) (void)hipFree(device->pad_scratch);
-    if (device->side_scratch) (void)hipFree(device->side_scratch);
     if (device->counters) (void)hipFree(device->counters);
     (void)hipStreamDestroy(device->own_stream);
     delete device;

@@ -20,3 +20,5 @@ int rlt_gemm_wgrad(rlt_rocm_device* device, const float* d_pre, int ldd, const f
 int rlt_gemm_static_scratch_setup(rlt_rocm_device* device);
 // dst <- act'(pre) * src (dst may alias src; then a no-op for the identity)
 int rlt_dpre(rlt_rocm_device* device, const float* src, int lds, float* dst, int ldd, const float* pre, int rows, int cols, int act, int from_output);
+// zeroes n tensors (mlp.hip): one launch per 16 runs of tensors that lie back to back
+int rlt_zero_tensors(rlt_rocm_device* device, float* const* begins, const size_t* counts, int n);

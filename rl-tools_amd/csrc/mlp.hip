@@ -62,6 +62,29 @@ __global__ __launch_bounds__(256) void mse_d_kernel(const float* __restrict__ y,
 
 }  // namespace
 
+// zeroes a list of tensors: tensors laid out back to back (the flat arena [dW0 | db0 | dW1 | db1 | ...]) form one run, tensors that are allocations of their own a run
+// each; up to 16 runs per launch
+int rlt_zero_tensors(rlt_rocm_device* device, float* const* begins, const size_t* counts, int n) {
+    ZeroRuns z = {};
+    auto flush = [&]() -> int {
+        if (z.n == 0) return 0;
+        const size_t total = z.prefix[z.n];
+        int blocks = (int)((total + 255) / 256); if (blocks > 1024) blocks = 1024;
+        if (z.n == 1) hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, device->stream, z.begin[0], total, z.begin[0], (size_t)0);
+        else hipLaunchKernelGGL(zero_runs_kernel, dim3(blocks), dim3(256), 0, device->stream, z);
+        z = ZeroRuns{};
+        return rlt_launch_status(device);
+    };
+    for (int i = 0; i < n; i++) {
+        if (!begins[i]) return RLT_E_INVALID_ARGUMENT;
+        if (counts[i] == 0) continue;
+        if (z.n > 0 && z.begin[z.n - 1] + (z.prefix[z.n] - z.prefix[z.n - 1]) == begins[i]) { z.prefix[z.n] += counts[i]; continue; }      // continues the last run
+        if (z.n == ZERO_RUNS) { const int rc = flush(); if (rc) return rc; }
+        z.begin[z.n] = begins[i]; z.prefix[z.n + 1] = z.prefix[z.n] + counts[i]; z.n++;
+    }
+    return flush();
+}
+
 extern "C" {
 
 int rlt_rocm_dense_evaluate(rlt_rocm_device* device, const rlt_dense_layer* L, const float* x, int ldx, float* y, int ldy, int batch) {
@@ -205,32 +228,14 @@ int rlt_rocm_mlp_backward(rlt_rocm_device* device, const rlt_dense_layer* layers
 
 int rlt_rocm_mlp_zero_gradient(rlt_rocm_device* device, const rlt_dense_layer* layers, int n) {
     if (!device) return RLT_E_NOT_INITIALISED;
-    RLT_REQUIRE(layers && n >= 1);
-    for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases && layers[l].in_dim > 0 && layers[l].out_dim > 0);
-    // gradient tensors laid out back to back ([dW0 | db0 | dW1 | db1 | ...], the flat arena) form one run; tensors that are allocations of their own a run each;
-    // up to 16 runs per launch
-    ZeroRuns z = {};
-    auto flush = [&]() -> int {
-        if (z.n == 0) return 0;
-        const size_t total = z.prefix[z.n];
-        int blocks = (int)((total + 255) / 256); if (blocks > 1024) blocks = 1024;
-        if (z.n == 1) hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, device->stream, z.begin[0], total, z.begin[0], (size_t)0);
-        else hipLaunchKernelGGL(zero_runs_kernel, dim3(blocks), dim3(256), 0, device->stream, z);
-        z = ZeroRuns{};
-        return rlt_launch_status(device);
-    };
-    auto add = [&](float* begin, size_t count) -> int {
-        if (z.n > 0 && z.begin[z.n - 1] + (z.prefix[z.n] - z.prefix[z.n - 1]) == begin) { z.prefix[z.n] += count; return 0; }      // continues the last run
-        if (z.n == ZERO_RUNS) { const int rc = flush(); if (rc) return rc; }
-        z.begin[z.n] = begin; z.prefix[z.n + 1] = z.prefix[z.n] + count; z.n++;
-        return 0;
-    };
+    RLT_REQUIRE(layers && n >= 1 && n <= 64);
+    float* begins[128]; size_t counts[128];
     for (int l = 0; l < n; l++) {
-        int rc = add(layers[l].d_weights, (size_t)layers[l].in_dim * layers[l].out_dim);
-        if (rc) return rc;
-        if ((rc = add(layers[l].d_biases, (size_t)layers[l].out_dim))) return rc;
+        RLT_REQUIRE(layers[l].d_weights && layers[l].d_biases && layers[l].in_dim > 0 && layers[l].out_dim > 0);
+        begins[2 * l] = layers[l].d_weights; counts[2 * l] = (size_t)layers[l].in_dim * layers[l].out_dim;
+        begins[2 * l + 1] = layers[l].d_biases; counts[2 * l + 1] = (size_t)layers[l].out_dim;
     }
-    return flush();
+    return rlt_zero_tensors(device, begins, counts, 2 * n);
 }
 
 }  // extern "C"

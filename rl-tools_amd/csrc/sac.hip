@@ -436,8 +436,8 @@ static size_t sequence_pass_workspace_bytes(const rlt_sac_sequence_agent* A, int
 size_t rlt_rocm_sac_sequence_workspace_bytes(const rlt_sac_sequence_agent* A) {
     if (!A || !A->actor || !A->critics[0] || !A->critics_target[0]) return 0;
     const int T = A->batch.sequence_length + 1, B = A->batch.batch;
-    // two passes may run at the same time (rlt_side_begin), each in its own half; then the loss gradient of the first critic where both critics train in one call
-    return 2 * sequence_pass_workspace_bytes(A, T, B) + ((sizeof(float) * (size_t)A->batch.sequence_length * B + 255) & ~(size_t)255);
+    // up to three passes run at the same time (rlt_side_begin), each in its own third; then the loss gradient of the first critic where both critics train in one call
+    return 3 * sequence_pass_workspace_bytes(A, T, B) + ((sizeof(float) * (size_t)A->batch.sequence_length * B + 255) & ~(size_t)255);
 }
 
 // rl/algorithms/sac/operations_generic.h:243-337 on a sequence batch, one launch per reference operation
@@ -491,9 +491,9 @@ int rlt_rocm_sac_sequence_train_critic(rlt_rocm_device* device, const rlt_sac_se
 
 // Both critics on one batch and one set of noise (the loop's SHARED_BATCH case, rl/algorithms/sac/loop/core/operations_generic.h:127-138): what the two calls of
 // train_critic would compute twice -- the actor on the next rows, its sample, both target critics, the target values -- is computed once, and the two critics'
-// passes run next to each other on the handle's two streams: side stream critic 0 forward, then target critic 1; main stream actor, sample, target critic 0, critic 1
-// forward; after the join the target values and both loss gradients, then critic 0's backward pass on the main stream next to critic 1's on the side stream, then
-// both optimisers. Every pass is the launch sequence that the single calls make, on the same inputs: the results are theirs bit for bit.
+// passes run next to each other on the handle's three streams: first side stream critic 0 forward, then target critic 1; second side stream critic 1 forward; main
+// stream actor, sample, target critic 0; after the join the target values and both loss gradients, then critic 0's backward pass on the main stream next to critic 1's
+// on a side stream, then both optimisers. Every pass is the launch sequence that the single calls make, on the same inputs: the results are theirs bit for bit.
 int rlt_rocm_sac_sequence_train_critics(rlt_rocm_device* device, const rlt_sac_sequence_agent* A, const float* action_noise) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(sequence_agent_ok(A) && action_noise);
@@ -502,14 +502,18 @@ int rlt_rocm_sac_sequence_train_critics(rlt_rocm_device* device, const rlt_sac_s
     const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
     const int first = A->include_first_step_in_targets ? 1 : 0, T = S + first, next_offset = first ? 0 : 1;
     const size_t ws_bytes = sequence_pass_workspace_bytes(A, S + 1, B);
-    void* ws = A->workspace; void* ws_side = (char*)A->workspace + ws_bytes;
-    float* d_output_first = (float*)((char*)A->workspace + 2 * ws_bytes);      // critic 0's loss gradient; critic 1's goes to the agent's buffer, where two single calls leave it
+    void* ws = A->workspace; void* ws_side = (char*)A->workspace + ws_bytes; void* ws_second = (char*)A->workspace + 2 * ws_bytes;
+    float* d_output_first = (float*)((char*)A->workspace + 3 * ws_bytes);      // critic 0's loss gradient; critic 1's goes to the agent's buffer, where two single calls leave it
     const bool overlap = S >= 48;      // short sequences: a pass is shorter than the two events that fork and join a stream cost on the host
     int rc;
     for (int k = 0; k < 2; k++) if ((rc = rlt_rocm_seq_zero_gradient(device, A->critics[k], A->n_critic_layers))) return rc;
     {
         if (overlap) rlt_side_begin(device);      // (without a second stream everything below simply runs in order on the one stream)
         rc = rlt_rocm_seq_forward(device, A->critics[0], A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, device->side_return ? ws_side : ws, ws_bytes);
+        rlt_side_end(device);
+        if (rc) return rc;
+        if (overlap) rlt_side_begin(device, 1);
+        rc = rlt_rocm_seq_forward(device, A->critics[1], A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, device->side_return ? ws_second : ws, ws_bytes);
         rlt_side_end(device);
         if (rc) return rc;
     }
@@ -529,7 +533,6 @@ int rlt_rocm_sac_sequence_train_critics(rlt_rocm_device* device, const rlt_sac_s
         rlt_side_end(device);
         if (rc) return rc;
     }
-    if ((rc = rlt_rocm_seq_forward(device, A->critics[1], A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, ws, ws_bytes))) return rc;
     if (overlap && (rc = rlt_side_join(device))) return rc;
     if ((rc = rlt_rocm_sac_target_action_values(device, A->next_q[0] + first * B, A->next_q[1] + first * B, K.rewards, K.terminated, A->next_log_probabilities,
                                                A->log_alpha.parameters, A->gamma, 0, A->target_action_value, S * B))) return rc;
@@ -554,25 +557,26 @@ int rlt_rocm_sac_sequence_train_critics(rlt_rocm_device* device, const rlt_sac_s
 // sac/operations_generic.h:486-527
 int rlt_rocm_sac_sequence_update_critic_targets(rlt_rocm_device* device, const rlt_sac_sequence_agent* A) {
     if (!device) return RLT_E_NOT_INITIALISED;
-    RLT_REQUIRE(sequence_agent_ok(A));
-    int rc;
+    RLT_REQUIRE(sequence_agent_ok(A) && A->n_critic_layers <= RLT_SEQ_MAX_LAYERS);
+    // every tensor of both target critics in one launch per sixteen tensors
+    const float* sources[2 * 5 * RLT_SEQ_MAX_LAYERS]; float* targets[2 * 5 * RLT_SEQ_MAX_LAYERS]; uint32_t counts[2 * 5 * RLT_SEQ_MAX_LAYERS];
+    int n = 0;
+    auto pair = [&](const float* source, float* target, size_t count) { sources[n] = source; targets[n] = target; counts[n++] = (uint32_t)count; };
     for (int k = 0; k < 2; k++)
         for (int l = 0; l < A->n_critic_layers; l++) {
             const rlt_seq_layer& s = A->critics[k][l]; const rlt_seq_layer& t = A->critics_target[k][l];
             RLT_REQUIRE(s.kind == t.kind);
             if (s.kind == 0) {
-                if ((rc = rlt_rocm_polyak_update(device, s.dense.weights, t.dense.weights, (size_t)s.dense.in_dim * s.dense.out_dim, A->polyak, 0))) return rc;
-                if ((rc = rlt_rocm_polyak_update(device, s.dense.biases, t.dense.biases, (size_t)s.dense.out_dim, A->polyak, 0))) return rc;
+                pair(s.dense.weights, t.dense.weights, (size_t)s.dense.in_dim * s.dense.out_dim); pair(s.dense.biases, t.dense.biases, (size_t)s.dense.out_dim);
             } else {
                 const size_t H = s.gru.hidden_dim, I = s.gru.input_dim;
-                if ((rc = rlt_rocm_polyak_update(device, s.gru.weights_input, t.gru.weights_input, 3 * H * I, A->polyak, 0))) return rc;
-                if ((rc = rlt_rocm_polyak_update(device, s.gru.biases_input, t.gru.biases_input, 3 * H, A->polyak, 0))) return rc;
-                if ((rc = rlt_rocm_polyak_update(device, s.gru.weights_hidden, t.gru.weights_hidden, 3 * H * H, A->polyak, 0))) return rc;
-                if ((rc = rlt_rocm_polyak_update(device, s.gru.biases_hidden, t.gru.biases_hidden, 3 * H, A->polyak, 0))) return rc;
-                if ((rc = rlt_rocm_polyak_update(device, s.gru.initial_hidden_state, t.gru.initial_hidden_state, H, A->polyak, 0))) return rc;
+                pair(s.gru.weights_input, t.gru.weights_input, 3 * H * I); pair(s.gru.biases_input, t.gru.biases_input, 3 * H);
+                pair(s.gru.weights_hidden, t.gru.weights_hidden, 3 * H * H); pair(s.gru.biases_hidden, t.gru.biases_hidden, 3 * H);
+                pair(s.gru.initial_hidden_state, t.gru.initial_hidden_state, H);
             }
         }
-    return 0;
+    for (int i = 0; i < n; i++) RLT_REQUIRE(sources[i] && targets[i]);
+    return rlt_sac_polyak_list(device, sources, targets, counts, n, A->polyak);
 }
 
 // sac/operations_generic.h:395-468 on a sequence batch

@@ -227,20 +227,21 @@ int rlt_rocm_seq_evaluate_step(rlt_rocm_device* device, const rlt_seq_layer* lay
 
 int rlt_rocm_seq_zero_gradient(rlt_rocm_device* device, const rlt_seq_layer* layers, int n) {
     if (!device) return RLT_E_NOT_INITIALISED;
-    RLT_REQUIRE(layers && n > 0);
-    int rc;
-    auto zero = [&](float* p, size_t count) { return p ? rlt_rocm_fill_f32(device, p, 1, (int)count, (int)count, 0.0f) : RLT_E_INVALID_ARGUMENT; };
+    RLT_REQUIRE(layers && n > 0 && n <= RLT_SEQ_MAX_LAYERS);
+    float* begins[4 * RLT_SEQ_MAX_LAYERS]; size_t counts[4 * RLT_SEQ_MAX_LAYERS];
+    int m = 0;
+    auto add = [&](float* p, size_t count) { begins[m] = p; counts[m++] = count; };
     for (int l = 0; l < n; l++) {
         if (layers[l].kind == 0) {
             const rlt_dense_layer& D = layers[l].dense;
-            if ((rc = zero(D.d_weights, (size_t)D.in_dim * D.out_dim)) || (rc = zero(D.d_biases, D.out_dim))) return rc;
+            add(D.d_weights, (size_t)D.in_dim * D.out_dim); add(D.d_biases, D.out_dim);
         } else {
             const rlt_gru_layer& G = layers[l].gru;
             const size_t H = G.hidden_dim, I = G.input_dim;
-            if ((rc = zero(G.d_weights_input, 3 * H * I)) || (rc = zero(G.d_biases_input, 3 * H)) || (rc = zero(G.d_weights_hidden, 3 * H * H)) || (rc = zero(G.d_biases_hidden, 3 * H))) return rc;
+            add(G.d_weights_input, 3 * H * I); add(G.d_biases_input, 3 * H); add(G.d_weights_hidden, 3 * H * H); add(G.d_biases_hidden, 3 * H);
         }
     }
-    return 0;
+    return rlt_zero_tensors(device, begins, counts, m);      // all of the network's gradient tensors in one launch (two beyond sixteen separate allocations)
 }
 
 }  // extern "C"

@@ -298,24 +298,26 @@ int copy_columns(rlt_rocm_device* device, const float* src, int lds, float* dst,
 }
 inline const float* seq_last_output(const rlt_seq_layer* layers, int n) { const rlt_seq_layer& L = layers[n - 1]; return L.kind ? L.gru.output : L.dense.output; }
 inline int seq_last_dim(const rlt_seq_layer* layers, int n) { const rlt_seq_layer& L = layers[n - 1]; return L.kind ? L.gru.hidden_dim : L.dense.out_dim; }
+// every tensor of a target network in one launch per sixteen tensors
 int polyak_seq(rlt_rocm_device* device, const rlt_seq_layer* source, const rlt_seq_layer* target, int n, float polyak) {
-    int rc;
+    RLT_REQUIRE(n <= RLT_SEQ_MAX_LAYERS);
+    const float* sources[5 * RLT_SEQ_MAX_LAYERS]; float* targets[5 * RLT_SEQ_MAX_LAYERS]; uint32_t counts[5 * RLT_SEQ_MAX_LAYERS];
+    int m = 0;
+    auto pair = [&](const float* from, float* to, size_t count) { sources[m] = from; targets[m] = to; counts[m++] = (uint32_t)count; };
     for (int l = 0; l < n; l++) {
         const rlt_seq_layer& s = source[l]; const rlt_seq_layer& t = target[l];
         RLT_REQUIRE(s.kind == t.kind);
         if (s.kind == 0) {
-            if ((rc = rlt_rocm_polyak_update(device, s.dense.weights, t.dense.weights, (size_t)s.dense.in_dim * s.dense.out_dim, polyak, 0))) return rc;
-            if ((rc = rlt_rocm_polyak_update(device, s.dense.biases, t.dense.biases, (size_t)s.dense.out_dim, polyak, 0))) return rc;
+            pair(s.dense.weights, t.dense.weights, (size_t)s.dense.in_dim * s.dense.out_dim); pair(s.dense.biases, t.dense.biases, (size_t)s.dense.out_dim);
         } else {
             const size_t H = s.gru.hidden_dim, I = s.gru.input_dim;
-            if ((rc = rlt_rocm_polyak_update(device, s.gru.weights_input, t.gru.weights_input, 3 * H * I, polyak, 0))) return rc;
-            if ((rc = rlt_rocm_polyak_update(device, s.gru.biases_input, t.gru.biases_input, 3 * H, polyak, 0))) return rc;
-            if ((rc = rlt_rocm_polyak_update(device, s.gru.weights_hidden, t.gru.weights_hidden, 3 * H * H, polyak, 0))) return rc;
-            if ((rc = rlt_rocm_polyak_update(device, s.gru.biases_hidden, t.gru.biases_hidden, 3 * H, polyak, 0))) return rc;
-            if ((rc = rlt_rocm_polyak_update(device, s.gru.initial_hidden_state, t.gru.initial_hidden_state, H, polyak, 0))) return rc;
+            pair(s.gru.weights_input, t.gru.weights_input, 3 * H * I); pair(s.gru.biases_input, t.gru.biases_input, 3 * H);
+            pair(s.gru.weights_hidden, t.gru.weights_hidden, 3 * H * H); pair(s.gru.biases_hidden, t.gru.biases_hidden, 3 * H);
+            pair(s.gru.initial_hidden_state, t.gru.initial_hidden_state, H);
         }
     }
-    return 0;
+    for (int i = 0; i < m; i++) RLT_REQUIRE(sources[i] && targets[i]);
+    return rlt_sac_polyak_list(device, sources, targets, counts, m, polyak);
 }
 bool td3_sequence_agent_ok(const rlt_td3_sequence_agent* A) {
     if (!A || A->observation_dim <= 0 || A->action_dim <= 0 || A->n_actor_layers < 1 || A->n_critic_layers < 1) return false;

@@ -158,7 +158,7 @@ def test_the_references_recurrent_td3_loop_runs_on_rocm():
     """rl/algorithms/td3/loop/core with ConfigApproximatorsGRU (sequences of 16 steps x 32, four environments) inside the evaluation and timing loop steps on
     devices::ROCM: the runner steps the recurrent actor whose output is the action (no sampling layer), the updates are the sequence entry points, evaluations run on the
     device. Measured (seed 0): mean return of 50 evaluation episodes -1,248 before training, -555 at its best within 10,000 loop steps (this actor explores through
-    nothing but its own changes, so the curve is uneven), 2,090 loop steps/s including the evaluations; the reference's CPU device (generic operations, one thread): 413."""
+    nothing but its own changes, so the curve is uneven), 2,290 loop steps/s including the evaluations; the reference's CPU device (generic operations, one thread): 413."""
     path = os.path.join(BUILD, "rocm_td3_gru_pendulum")
     if not os.path.exists(path):
         pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
@@ -332,7 +332,7 @@ def test_recurrent_sac_loop_trains_on_rocm():
     and sequence batches of 16 steps x 32 samples from four environments, on devices::ROCM: gather_batch's multi-step branch with its draws made on the
     device, the runner step with the policy state reset by the truncation mask and evaluate_step, train_critic / train_actor as one call each of the library's
     entry points for sequence batches, the evaluation loop step with the recurrent actor on the device. A random actor's mean
-    return is about -1,300; measured -293 after 3,000 loop steps, at 1,660 loop steps/s including the evaluations (the same program on
+    return is about -1,300; measured -293 after 3,000 loop steps, at 1,750 loop steps/s including the evaluations (the same program on
     the reference's CPU device: 190)."""
     path = os.path.join(BUILD, "rocm_sac_gru_pendulum")
     if not os.path.exists(path):
@@ -351,7 +351,7 @@ def test_zoo_configuration_of_the_pendulum_without_velocity_trains_on_rocm():
     """The reference's zoo configuration with memory (src/rl/zoo/pendulum-position-v1/sac.h, included as it is: the Pendulum whose observation hides the velocity, SAC with
     the recurrent approximators dense -> GRU -> GRU -> dense at widths 16 and 32, 100 sequences of 100 steps per update, 32 environments, a replay ring of 500,000 rows)
     inside the evaluation and timing loop steps on devices::ROCM. Here the first 12,000 of its 500,000 loop steps: measured mean return -1,219 before training, -778 after
-    5,000 steps, -365 after 10,000, at 591 loop steps/s including the evaluations (the reference's CPU device with its CBLAS backend, one thread: 33 loop steps/s). The loop
+    5,000 steps, -365 after 10,000, at 646 loop steps/s including the evaluations (the reference's CPU device with its CBLAS backend, one thread: 33 loop steps/s). The loop
     step is the overload for shared batches: both critics are trained by one call of the library."""
     path = os.path.join(BUILD, "rocm_zoo_pendulum_position_v1_sac")
     if not os.path.exists(path):
