@@ -219,6 +219,10 @@ int rlt_rocm_mlp_backward(rlt_rocm_device* device, const rlt_dense_layer* layers
     const rlt_dense_layer& last = layers[n - 1];
     int rc = rlt_dpre(device, d_output, ldd, d_output, ldd, last.pre_activations, batch, last.out_dim, last.activation, 0);
     if (rc) return rc;
+    if (want_w && !d_input && batch <= RLT_MLP_WIDE_MAX_BATCH && single_pass_enabled() && wide_enabled()) {      // a few thousand rows at most: sixteen-row tiles
+        rc = rlt_mlp_wide_backward(device, layers, n, x, ldx, d_output, ldd, batch);
+        if (rc != RLT_E_UNSUPPORTED) return rc;
+    }
     if (want_w && !d_input && batch >= FUSED_MIN_BATCH && single_pass_enabled()) {
         rc = rlt_mlp3_fused_backward(device, layers, n, x, ldx, d_output, ldd, batch, workspace, workspace_bytes);
         if (rc != RLT_E_UNSUPPORTED) return rc;

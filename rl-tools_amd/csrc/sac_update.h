@@ -41,3 +41,6 @@ int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agen
 constexpr int RLT_MLP_WIDE_MAX_BATCH = 4096;
 int rlt_mlp_wide_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy,
                                   const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch);
+// the backward pass alone (weight gradients, no input gradient) from the outputs that a forward() left in layers 1 and 2; d_pre_last [batch x out] is the gradient at the last
+// layer's pre-activations, whatever that layer's activation
+int rlt_mlp_wide_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, const float* d_pre_last, int ldd, int batch);

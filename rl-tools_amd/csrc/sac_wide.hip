@@ -622,8 +622,9 @@ struct MlpWideArgs {
     const float* d_output; int ldd; const float* target; int ldt; float mse_scale;
     int batch;
     float* partial; int count;
+    const float* out1; const float* out2;      // BACKWARD_ONLY: the outputs of layers 1 and 2 that a forward() left in memory, [batch x hid] each; d_output is then the gradient at the last pre-activations
 };
-template <int ACT_H, int NT1C>
+template <int ACT_H, int NT1C, bool BACKWARD_ONLY>
 __global__ __launch_bounds__(THREADS) void mlp_wide_kernel(MlpWideArgs A) {
     extern __shared__ __attribute__((aligned(16))) float lds_wide[];
     const int gi = blockIdx.x;
@@ -638,10 +639,30 @@ __global__ __launch_bounds__(THREADS) void mlp_wide_kernel(MlpWideArgs A) {
         const int r = e / SXS, k = e % SXS;
         xa[e] = (row0 + r < B && k < IN) ? A.x[(size_t)(row0 + r) * A.ldx + k] : 0.f;
     }
+    if (BACKWARD_ONLY) {
+        // the hidden activations come back from memory (zero beyond the batch and beyond the width, up to the multiple of 16 that the tiles run to)
+        const int HP = 16 * tiles;
+        for (int e = threadIdx.x; e < ROWS * HP; e += THREADS) {
+            const int r = e / HP, k = e - r * HP;
+            const bool ok = row0 + r < B && k < HID;
+            h1[r * S + k] = ok ? A.out1[(size_t)(row0 + r) * HID + k] : 0.f;
+            h2[r * S + k] = ok ? A.out2[(size_t)(row0 + r) * HID + k] : 0.f;
+        }
+    }
     rlt_lds_barrier();
-    forward3_own_loads<ACT_H, NT1C>(N, xa, SXS, h1, h2, yp, wave, c, g);
+    if (!BACKWARD_ONLY) forward3_own_loads<ACT_H, NT1C>(N, xa, SXS, h1, h2, yp, wave, c, g);
     float s3 = 0.f;
-    if (wave == 0) {
+    if (BACKWARD_ONLY) {
+        if (wave == 0) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = row0 + 4 * g + v;
+                const float d = (c < OUT && row < B) ? A.d_output[(size_t)row * A.ldd + c] : 0.f;
+                d3[(4 * g + v) * D3S + c] = d;
+                s3 += d;
+            }
+        }
+    } else if (wave == 0) {
         // lane (c, g): output column c of rows 4 g + v; the gradient at the output (the last layer has no activation): given, or the MSE's against the target
         const floatx4 out = output_tile(yp, tiles, c, g);
         const float b3 = c < OUT ? N.b3[c] : 0.f;
@@ -989,17 +1010,21 @@ int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* A, c
 }
 
 
-// ---- forward + backward of a three-layer network on sixteen-row tiles (see mlp_wide_kernel); RLT_E_UNSUPPORTED: the caller takes another path
-int rlt_mlp_wide_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n_layers, const float* x, int ldx, float* y, int ldy,
-                                  const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch) {
+// ---- forward + backward of a three-layer network on sixteen-row tiles (see mlp_wide_kernel), or the backward pass alone from the outputs that a forward() left in
+// the layers; RLT_E_UNSUPPORTED: the caller takes another path
+static int mlp_wide_launch(rlt_rocm_device* device, const rlt_dense_layer* L, int n_layers, const float* x, int ldx, float* y, int ldy,
+                           const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch, bool backward_only) {
     if (n_layers != 3 || batch < 1 || batch > RLT_MLP_WIDE_MAX_BATCH || L[0].in_dim < 1 || L[0].in_dim > MAX_D || L[2].out_dim < 1 || L[2].out_dim > MAX_OUT) return RLT_E_UNSUPPORTED;
     int hid = 0;
-    if (!net_ok(L, 3, L[0].in_dim, L[2].out_dim, hid)) return RLT_E_UNSUPPORTED;
+    // the backward pass alone is handed the gradient at the last pre-activations: the last layer's activation plays no part in it
+    if (!net_ok(L, 3, L[0].in_dim, L[2].out_dim, hid, backward_only ? L[2].activation : RLT_ACT_IDENTITY)) return RLT_E_UNSUPPORTED;
     for (int l = 0; l < 3; l++) if (!L[l].d_weights || !L[l].d_biases) return RLT_E_UNSUPPORTED;
+    if (backward_only && (!L[0].output || !L[1].output)) return RLT_E_UNSUPPORTED;
     if (LDS_FLOATS * sizeof(float) > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
     MlpWideArgs a = {};
     a.net = net_of(L);
     a.x = x; a.ldx = ldx; a.y = y; a.ldy = ldy; a.d_output = d_output; a.ldd = ldd; a.target = target; a.ldt = ldt; a.mse_scale = mse_scale; a.batch = batch;
+    a.out1 = L[0].output; a.out2 = L[1].output;
     const int IN = L[0].in_dim, OUT = L[2].out_dim, groups = rlt_div_up(batch, ROWS);
     const int exact = hid * IN + hid + hid * hid + hid + OUT * hid + OUT;
     a.count = (exact + 63) & ~63;
@@ -1010,23 +1035,30 @@ int rlt_mlp_wide_forward_backward(rlt_rocm_device* device, const rlt_dense_layer
     if (rc) return rc;
     a.partial = (float*)scratch;
     {
+        // the second layer's weights in the order the wavefronts consume them: the copy for d_pre2 W2, and for the forward pass the one for h1 W2^T
         PrepArgs P = {};
         float* copies = (float*)((char*)scratch + partial_bytes);
-        for (int q = 0; q < 2; q++) { P.W2[q] = a.net.W2; P.dst[q] = copies + (size_t)q * copy_floats; P.hid[q] = hid; P.backward[q] = q; }
-        a.net.W2f = P.dst[0]; a.net.W2b = P.dst[1];
+        const int jobs = backward_only ? 1 : 2;
+        for (int q = 0; q < jobs; q++) { P.W2[q] = a.net.W2; P.dst[q] = copies + (size_t)q * copy_floats; P.hid[q] = hid; P.backward[q] = q == 0 ? 1 : 0; }
+        a.net.W2b = P.dst[0]; a.net.W2f = backward_only ? nullptr : P.dst[1];
         const int tiles = (hid + 15) >> 4;
-        hipLaunchKernelGGL(wide_prepare_kernel, dim3(rlt_div_up(tiles * tiles * 64, 256), 2), dim3(256), 0, device->stream, P);
+        hipLaunchKernelGGL(wide_prepare_kernel, dim3(rlt_div_up(tiles * tiles * 64, 256), jobs), dim3(256), 0, device->stream, P);
         if ((rc = rlt_launch_status(device))) return rc;
     }
     const size_t lds_bytes = LDS_FLOATS * sizeof(float);
-#define RLT_LAUNCH_MLP_WIDE(ACT, NT)                                                                                                                   \
-    do {                                                                                                                                               \
-        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp_wide_kernel<ACT, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
-        hipLaunchKernelGGL((mlp_wide_kernel<ACT, NT>), dim3(groups), dim3(THREADS), lds_bytes, device->stream, a);                                    \
+#define RLT_LAUNCH_MLP_WIDE(ACT, NT, BWD)                                                                                                                   \
+    do {                                                                                                                                                    \
+        RLT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(mlp_wide_kernel<ACT, NT, BWD>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)); \
+        hipLaunchKernelGGL((mlp_wide_kernel<ACT, NT, BWD>), dim3(groups), dim3(THREADS), lds_bytes, device->stream, a);                                    \
     } while (0)
-    const int act = a.net.act_h;
-    if (IN <= 32) { if (act == RLT_ACT_RELU) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, 2); else RLT_LAUNCH_MLP_WIDE(-1, 2); }
-    else { if (act == RLT_ACT_RELU) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, MAX_D / 16); else RLT_LAUNCH_MLP_WIDE(-1, MAX_D / 16); }
+    const bool relu = a.net.act_h == RLT_ACT_RELU;
+    if (backward_only) {
+        if (IN <= 32) { if (relu) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, 2, true); else RLT_LAUNCH_MLP_WIDE(-1, 2, true); }
+        else { if (relu) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, MAX_D / 16, true); else RLT_LAUNCH_MLP_WIDE(-1, MAX_D / 16, true); }
+    } else {
+        if (IN <= 32) { if (relu) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, 2, false); else RLT_LAUNCH_MLP_WIDE(-1, 2, false); }
+        else { if (relu) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, MAX_D / 16, false); else RLT_LAUNCH_MLP_WIDE(-1, MAX_D / 16, false); }
+    }
 #undef RLT_LAUNCH_MLP_WIDE
     if ((rc = rlt_launch_status(device))) return rc;
     WideReduceArgs R = {};
@@ -1036,6 +1068,13 @@ int rlt_mlp_wide_forward_backward(rlt_rocm_device* device, const rlt_dense_layer
     for (int k = 0, end = 0; k < 6; k++) { end += size[k]; R.dst[k] = dst[k]; R.end[k] = end; }
     hipLaunchKernelGGL(mlp_wide_reduce_kernel, dim3(rlt_div_up(exact, 256)), dim3(256), 0, device->stream, R);
     return rlt_launch_status(device);
+}
+int rlt_mlp_wide_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n_layers, const float* x, int ldx, float* y, int ldy,
+                                  const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch) {
+    return mlp_wide_launch(device, L, n_layers, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, false);
+}
+int rlt_mlp_wide_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n_layers, const float* x, int ldx, const float* d_pre_last, int ldd, int batch) {
+    return mlp_wide_launch(device, L, n_layers, x, ldx, nullptr, 0, d_pre_last, ldd, nullptr, 0, 0.0f, batch, true);
 }
 
 #ifdef RLT_WIDE_PROFILE

@@ -85,3 +85,41 @@ def test_the_call_takes_the_sixteen_row_tiles_where_this_file_says_so(rocm, monk
     monkeypatch.setenv("RLT_MLP_WIDE", "0")
     other = run(rocm, dims, params, x, dy, "relu", False, 0.0)
     assert rel_err(wide[1], other[1]) <= TOL and not np.array_equal(wide[1], other[1])
+
+
+def forward_then_backward(backend, dims, params, x, dy, ha, oa):
+    """The reference's call pattern: forward() (keeps every layer's pre-activations and outputs), then backward() of a given gradient."""
+    B = x.shape[0]
+    net = Mlp(backend, dims, params, B, ha, oa)
+    xd, dyd = backend.array(x), backend.array(dy)
+    ws, wsn = net.workspace()
+    backend.call("mlp_zero_gradient", net.layers, net.n)
+    backend.call("mlp_forward", net.layers, net.n, xd.ptr, dims[0], B)
+    backend.call("mlp_backward", net.layers, net.n, xd.ptr, dims[0], dyd.ptr, dims[-1], None, 0, B, 1, ws, wsn)
+    backend.sync()
+    return dict(grads=net.grads.numpy(), d_output=dyd.numpy(), offsets=net.offsets)
+
+
+@pytest.mark.parametrize("case", [(256, 17, 256, 6, "relu", "identity"), (4096, 17, 256, 6, "relu", "tanh"), (37, 35, 200, 1, "tanh", "identity"), (100, 128, 72, 16, "fast_tanh", "sigmoid"),
+                                  (1000, 3, 64, 2, "sigmoid", "identity")])
+def test_backward_alone_on_sixteen_row_tiles_matches_the_checker_and_the_other_paths(oracle, rocm, case, monkeypatch):
+    """backward() after forward(): the tiles read the hidden layers' outputs back from memory; the last layer may have any activation (its derivative is applied to the
+    given gradient before the kernel runs, in place as in the reference)."""
+    print("case", case, flush=True)
+    B, I, H, O, ha, oa = case
+    dims = [I, H, H, O]
+    rng = np.random.default_rng(B + 7 * I + H)
+    params = helpers.random_params(rng, dims)
+    x, dy = rng.standard_normal((B, I)).astype(np.float32), rng.standard_normal((B, O)).astype(np.float32)
+    ref = forward_then_backward(oracle, dims, params, x, dy, ha, oa)
+    got = forward_then_backward(rocm, dims, params, x, dy, ha, oa)
+    monkeypatch.setenv("RLT_MLP_WIDE", "0")
+    other = forward_then_backward(rocm, dims, params, x, dy, ha, oa)
+    monkeypatch.delenv("RLT_MLP_WIDE")
+    for name, want in (("checker", ref), ("other path", other)):
+        assert rel_err(got["d_output"], want["d_output"]) <= TOL, name
+        for (off, nw, nb) in ref["offsets"]:
+            ew = rel_err(got["grads"][off:off + nw], want["grads"][off:off + nw]); eb = rel_err(got["grads"][off + nw:off + nw + nb], want["grads"][off + nw:off + nw + nb])
+            assert ew <= TOL and eb <= TOL, (name, off, ew, eb)
+    assert not np.array_equal(got["grads"], other["grads"])      # two different kernels ran
+
