@@ -17,6 +17,7 @@ struct rlt_rocm_device {
     size_t scratch_bytes;
     void* pad_scratch;           // a second grow-only buffer: zero-padded copies of narrow networks (pad.hip)
     size_t pad_scratch_bytes;
+    void* copy_scratch; size_t copy_scratch_bytes;      // weight copies in consumption order of the MLP calls on sixteen-row tiles: not the handle's scratch buffer, which callers of forward() / evaluate() may hold across the call
     void* counters;              // 8 KiB, zero between launches: [0,256) ticket counters, [256,..) per-workgroup partial sums
     unsigned* fault;             // [0]: set by a persistent kernel that gave up waiting for another workgroup; read back by check_status
     int fault_armed;             // a kernel that can set it was launched since the last check

@@ -221,6 +221,7 @@ int rlt_rocm_destroy(rlt_rocm_device* device) {
     }
     if (device->scratch) (void)hipFree(device->scratch);
     if (device->pad_scratch) (void)hipFree(device->pad_scratch);
+    if (device->copy_scratch) (void)hipFree(device->copy_scratch);
     if (device->counters) (void)hipFree(device->counters);
     (void)hipStreamDestroy(device->own_stream);
     delete device;

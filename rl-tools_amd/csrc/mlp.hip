@@ -135,6 +135,10 @@ int rlt_rocm_mlp_evaluate(rlt_rocm_device* device, const rlt_dense_layer* layers
     RLT_REQUIRE(chain_ok(layers, n) && x && y && batch > 0 && ldx >= layers[0].in_dim && ldy >= layers[n - 1].out_dim);
     const size_t buf = align_up((size_t)batch * max_dim(layers, n) * sizeof(float));
     RLT_REQUIRE(n == 1 || (workspace && workspace_bytes >= 2 * buf));
+    if (n == 3 && batch <= RLT_MLP_WIDE_MAX_BATCH && layers[0].out_dim > 64 && single_pass_enabled() && wide_enabled()) {      // as forward(): the same kernel, the same bits
+        const int rc = rlt_mlp_wide_forward(device, layers, n, x, ldx, y, ldy, batch, false);
+        if (rc != RLT_E_UNSUPPORTED) return rc;
+    }
     if (n > 1 && batch <= RLT_MLP_ROWS_MAX_BATCH && rows_enabled()) {
         const int rc = rlt_mlp_rows_forward(device, layers, n, x, ldx, y, ldy, batch, false);
         if (rc != RLT_E_UNSUPPORTED) return rc;
@@ -155,6 +159,12 @@ int rlt_rocm_mlp_forward(rlt_rocm_device* device, const rlt_dense_layer* layers,
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(chain_ok(layers, n) && x && batch > 0 && ldx >= layers[0].in_dim);
     for (int l = 0; l < n; l++) RLT_REQUIRE(layers[l].pre_activations && layers[l].output);
+    if (n == 3 && batch <= RLT_MLP_WIDE_MAX_BATCH && layers[0].out_dim > 64 && single_pass_enabled() && wide_enabled()) {
+        // hidden widths beyond 64 over a few thousand rows at most: sixteen-row tiles with the second layer's weights read from a copy in consumption order
+        // (narrower networks' weights are few enough for the few-rows kernel below to read them as they lie)
+        const int rc = rlt_mlp_wide_forward(device, layers, n, x, ldx, nullptr, 0, batch, true);
+        if (rc != RLT_E_UNSUPPORTED) return rc;
+    }
     if (n > 1 && batch <= RLT_MLP_ROWS_MAX_BATCH && batch < FUSED_MIN_BATCH && rows_enabled()) {
         const int rc = rlt_mlp_rows_forward(device, layers, n, x, ldx, nullptr, 0, batch, true);
         if (rc != RLT_E_UNSUPPORTED) return rc;

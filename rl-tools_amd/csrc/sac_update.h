@@ -44,3 +44,6 @@ int rlt_mlp_wide_forward_backward(rlt_rocm_device* device, const rlt_dense_layer
 // the backward pass alone (weight gradients, no input gradient) from the outputs that a forward() left in layers 1 and 2; d_pre_last [batch x out] is the gradient at the last
 // layer's pre-activations, whatever that layer's activation
 int rlt_mlp_wide_backward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, const float* d_pre_last, int ldd, int batch);
+// forward() alone, storing every layer's pre-activations and outputs (those of the layers that have the buffers) where `keep` is set, and the network's output into y
+// (optional, leading dimension ldy); any output activation
+int rlt_mlp_wide_forward(rlt_rocm_device* device, const rlt_dense_layer* layers, int n_layers, const float* x, int ldx, float* y, int ldy, int batch, bool keep);

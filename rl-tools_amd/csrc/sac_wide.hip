@@ -206,8 +206,10 @@ __device__ __forceinline__ void forward3(const WNet& N, Operands<NT1C>& W, const
 }
 // The same three layers for a pass that requests its own operands when it starts (the actor update: its passes are separated by the head and the critics' backward
 // passes, which need the registers)
-template <int ACT_H, int NT1C>
-__device__ __forceinline__ void forward3_own_loads(const WNet& N, lptr x, int xstride, lptr h1, lptr h2, lptr yp, int wave, int c, int g) {
+// KEEP: the hidden layers' pre-activations and outputs are also stored to memory, rows [row0, row0 + 16) of [batch x hid] arrays (forward() of a network keeps them)
+struct KeepArgs { float* pre[2]; float* out[2]; int row0, batch; };
+template <int ACT_H, int NT1C, bool KEEP = false>
+__device__ __forceinline__ void forward3_own_loads(const WNet& N, lptr x, int xstride, lptr h1, lptr h2, lptr yp, int wave, int c, int g, const KeepArgs* keep = nullptr) {
     const int HID = N.hid, n = 16 * wave + c, tiles = (HID + 15) >> 4;
     const bool on = wave < tiles, n_ok = n < HID;
     const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -230,7 +232,15 @@ __device__ __forceinline__ void forward3_own_loads(const WNet& N, lptr x, int xs
         chunks<NT1C>(a0, a1, x, xstride, c, g, 0, (N.in + 15) >> 4, w1);
         const floatx4 acc = a0 + a1;
 #pragma unroll
-        for (int v = 0; v < 4; v++) h1[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + b1, N.act_h) : 0.f;
+        for (int v = 0; v < 4; v++) {
+            const float pre = acc[v] + b1, o = act_hidden<ACT_H>(pre, N.act_h);
+            h1[(4 * g + v) * S + n] = n_ok ? o : 0.f;
+            if (KEEP && n_ok && keep->row0 + 4 * g + v < keep->batch) {
+                const size_t at = (size_t)(keep->row0 + 4 * g + v) * HID + n;
+                if (keep->pre[0]) keep->pre[0][at] = pre;
+                if (keep->out[0]) keep->out[0][at] = o;
+            }
+        }
         if (NT1C > 2) load_swizzled<8>(N.W2f, tiles, wave, c + 16 * g, 8, w2b);
     }
     rlt_lds_barrier();
@@ -240,7 +250,15 @@ __device__ __forceinline__ void forward3_own_loads(const WNet& N, lptr x, int xs
         chunks<8>(a0, a1, h1, S, c, g, 8, tiles, w2b);
         const floatx4 acc = a0 + a1;
 #pragma unroll
-        for (int v = 0; v < 4; v++) h2[(4 * g + v) * S + n] = n_ok ? act_hidden<ACT_H>(acc[v] + b2, N.act_h) : 0.f;
+        for (int v = 0; v < 4; v++) {
+            const float pre = acc[v] + b2, o = act_hidden<ACT_H>(pre, N.act_h);
+            h2[(4 * g + v) * S + n] = n_ok ? o : 0.f;
+            if (KEEP && n_ok && keep->row0 + 4 * g + v < keep->batch) {
+                const size_t at = (size_t)(keep->row0 + 4 * g + v) * HID + n;
+                if (keep->pre[1]) keep->pre[1][at] = pre;
+                if (keep->out[1]) keep->out[1][at] = o;
+            }
+        }
     }
     rlt_lds_barrier();
     if (on) {
@@ -622,10 +640,13 @@ struct MlpWideArgs {
     const float* d_output; int ldd; const float* target; int ldt; float mse_scale;
     int batch;
     float* partial; int count;
-    const float* out1; const float* out2;      // BACKWARD_ONLY: the outputs of layers 1 and 2 that a forward() left in memory, [batch x hid] each; d_output is then the gradient at the last pre-activations
+    const float* out1; const float* out2;      // MLP_BACKWARD: the outputs of layers 1 and 2 that a forward() left in memory, [batch x hid] each; d_output is then the gradient at the last pre-activations
+    float* keep_pre[3]; float* keep_out[3]; int act3;      // MLP_FORWARD: every layer's pre-activations and outputs as forward() keeps them (each may be NULL); the last layer's activation
 };
-template <int ACT_H, int NT1C, bool BACKWARD_ONLY>
+enum { MLP_FORWARD_BACKWARD = 0, MLP_BACKWARD = 1, MLP_FORWARD = 2 };
+template <int ACT_H, int NT1C, int PASS>
 __global__ __launch_bounds__(THREADS) void mlp_wide_kernel(MlpWideArgs A) {
+    constexpr bool BACKWARD_ONLY = PASS == MLP_BACKWARD;
     extern __shared__ __attribute__((aligned(16))) float lds_wide[];
     const int gi = blockIdx.x;
     const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
@@ -650,7 +671,27 @@ __global__ __launch_bounds__(THREADS) void mlp_wide_kernel(MlpWideArgs A) {
         }
     }
     rlt_lds_barrier();
-    if (!BACKWARD_ONLY) forward3_own_loads<ACT_H, NT1C>(N, xa, SXS, h1, h2, yp, wave, c, g);
+    if (PASS == MLP_FORWARD) {
+        const KeepArgs keep = {{A.keep_pre[0], A.keep_pre[1]}, {A.keep_out[0], A.keep_out[1]}, row0, B};
+        forward3_own_loads<ACT_H, NT1C, true>(N, xa, SXS, h1, h2, yp, wave, c, g, &keep);
+        if (wave == 0) {
+            const floatx4 out = output_tile(yp, tiles, c, g);
+            const float b3 = c < OUT ? N.b3[c] : 0.f;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = row0 + 4 * g + v;
+                if (c < OUT && row < B) {
+                    const float pre = out[v] + b3;
+                    if (A.keep_pre[2]) A.keep_pre[2][(size_t)row * OUT + c] = pre;
+                    const float o = rlt_act(pre, A.act3);
+                    if (A.keep_out[2]) A.keep_out[2][(size_t)row * OUT + c] = o;
+                    if (A.y) A.y[(size_t)row * A.ldy + c] = o;
+                }
+            }
+        }
+        return;
+    }
+    if (PASS == MLP_FORWARD_BACKWARD) forward3_own_loads<ACT_H, NT1C>(N, xa, SXS, h1, h2, yp, wave, c, g);
     float s3 = 0.f;
     if (BACKWARD_ONLY) {
         if (wave == 0) {
@@ -1013,34 +1054,48 @@ int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* A, c
 // ---- forward + backward of a three-layer network on sixteen-row tiles (see mlp_wide_kernel), or the backward pass alone from the outputs that a forward() left in
 // the layers; RLT_E_UNSUPPORTED: the caller takes another path
 static int mlp_wide_launch(rlt_rocm_device* device, const rlt_dense_layer* L, int n_layers, const float* x, int ldx, float* y, int ldy,
-                           const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch, bool backward_only) {
+                           const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch, int pass) {
+    const bool backward_only = pass == MLP_BACKWARD, forward_only = pass == MLP_FORWARD;
     if (n_layers != 3 || batch < 1 || batch > RLT_MLP_WIDE_MAX_BATCH || L[0].in_dim < 1 || L[0].in_dim > MAX_D || L[2].out_dim < 1 || L[2].out_dim > MAX_OUT) return RLT_E_UNSUPPORTED;
     int hid = 0;
     // the backward pass alone is handed the gradient at the last pre-activations: the last layer's activation plays no part in it
-    if (!net_ok(L, 3, L[0].in_dim, L[2].out_dim, hid, backward_only ? L[2].activation : RLT_ACT_IDENTITY)) return RLT_E_UNSUPPORTED;
-    for (int l = 0; l < 3; l++) if (!L[l].d_weights || !L[l].d_biases) return RLT_E_UNSUPPORTED;
+    // (forward() applies the last layer's activation per element when it stores the outputs)
+    if (!net_ok(L, 3, L[0].in_dim, L[2].out_dim, hid, pass == MLP_FORWARD_BACKWARD ? RLT_ACT_IDENTITY : L[2].activation)) return RLT_E_UNSUPPORTED;
+    for (int l = 0; l < 3; l++) if (!forward_only && (!L[l].d_weights || !L[l].d_biases)) return RLT_E_UNSUPPORTED;
     if (backward_only && (!L[0].output || !L[1].output)) return RLT_E_UNSUPPORTED;
     if (LDS_FLOATS * sizeof(float) > (size_t)device->lds_bytes) return RLT_E_UNSUPPORTED;
     MlpWideArgs a = {};
     a.net = net_of(L);
     a.x = x; a.ldx = ldx; a.y = y; a.ldy = ldy; a.d_output = d_output; a.ldd = ldd; a.target = target; a.ldt = ldt; a.mse_scale = mse_scale; a.batch = batch;
     a.out1 = L[0].output; a.out2 = L[1].output;
+    if (forward_only) for (int l = 0; l < 3; l++) { a.keep_pre[l] = L[l].pre_activations; a.keep_out[l] = L[l].output; }
+    a.act3 = L[2].activation;
     const int IN = L[0].in_dim, OUT = L[2].out_dim, groups = rlt_div_up(batch, ROWS);
     const int exact = hid * IN + hid + hid * hid + hid + OUT * hid + OUT;
     a.count = (exact + 63) & ~63;
     const size_t copy_floats = (size_t)256 * WAVES * WAVES;
-    const size_t partial_bytes = ((size_t)groups * a.count * sizeof(float) + 255) & ~(size_t)255;
+    const size_t partial_bytes = forward_only ? 0 : ((size_t)groups * a.count * sizeof(float) + 255) & ~(size_t)255;
     void* scratch = nullptr;
-    int rc = rlt_scratch(device, partial_bytes + 2 * copy_floats * sizeof(float), &scratch);
-    if (rc) return rc;
-    a.partial = (float*)scratch;
+    int rc = 0;
+    if (!forward_only) {
+        if ((rc = rlt_scratch(device, partial_bytes, &scratch))) return rc;
+        a.partial = (float*)scratch;
+    }
+    // the weight copies have a buffer of their own: forward() and evaluate() have never touched the handle's scratch buffer at these batch sizes, and callers hold data there across them
+    if (device->copy_scratch_bytes < 2 * copy_floats * sizeof(float)) {
+        if (device->capturing) return RLT_E_CAPTURING;
+        if (device->copy_scratch) RLT_HIP(hipFree(device->copy_scratch));
+        device->copy_scratch = nullptr; device->copy_scratch_bytes = 0;
+        RLT_HIP(hipMalloc(&device->copy_scratch, 2 * copy_floats * sizeof(float)));
+        device->copy_scratch_bytes = 2 * copy_floats * sizeof(float);
+    }
     {
         // the second layer's weights in the order the wavefronts consume them: the copy for d_pre2 W2, and for the forward pass the one for h1 W2^T
         PrepArgs P = {};
-        float* copies = (float*)((char*)scratch + partial_bytes);
-        const int jobs = backward_only ? 1 : 2;
-        for (int q = 0; q < jobs; q++) { P.W2[q] = a.net.W2; P.dst[q] = copies + (size_t)q * copy_floats; P.hid[q] = hid; P.backward[q] = q == 0 ? 1 : 0; }
-        a.net.W2b = P.dst[0]; a.net.W2f = backward_only ? nullptr : P.dst[1];
+        float* copies = (float*)device->copy_scratch;
+        const int jobs = pass == MLP_FORWARD_BACKWARD ? 2 : 1;
+        for (int q = 0; q < jobs; q++) { P.W2[q] = a.net.W2; P.dst[q] = copies + (size_t)q * copy_floats; P.hid[q] = hid; P.backward[q] = (q == 0 && !forward_only) ? 1 : 0; }
+        a.net.W2b = forward_only ? nullptr : P.dst[0]; a.net.W2f = forward_only ? P.dst[0] : (backward_only ? nullptr : P.dst[1]);
         const int tiles = (hid + 15) >> 4;
         hipLaunchKernelGGL(wide_prepare_kernel, dim3(rlt_div_up(tiles * tiles * 64, 256), jobs), dim3(256), 0, device->stream, P);
         if ((rc = rlt_launch_status(device))) return rc;
@@ -1052,15 +1107,16 @@ static int mlp_wide_launch(rlt_rocm_device* device, const rlt_dense_layer* L, in
         hipLaunchKernelGGL((mlp_wide_kernel<ACT, NT, BWD>), dim3(groups), dim3(THREADS), lds_bytes, device->stream, a);                                    \
     } while (0)
     const bool relu = a.net.act_h == RLT_ACT_RELU;
-    if (backward_only) {
-        if (IN <= 32) { if (relu) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, 2, true); else RLT_LAUNCH_MLP_WIDE(-1, 2, true); }
-        else { if (relu) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, MAX_D / 16, true); else RLT_LAUNCH_MLP_WIDE(-1, MAX_D / 16, true); }
-    } else {
-        if (IN <= 32) { if (relu) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, 2, false); else RLT_LAUNCH_MLP_WIDE(-1, 2, false); }
-        else { if (relu) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, MAX_D / 16, false); else RLT_LAUNCH_MLP_WIDE(-1, MAX_D / 16, false); }
-    }
+#define RLT_LAUNCH_MLP_WIDE_PASS(P)                                                                                                       \
+    do {                                                                                                                                  \
+        if (IN <= 32) { if (relu) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, 2, P); else RLT_LAUNCH_MLP_WIDE(-1, 2, P); }                          \
+        else { if (relu) RLT_LAUNCH_MLP_WIDE(RLT_ACT_RELU, MAX_D / 16, P); else RLT_LAUNCH_MLP_WIDE(-1, MAX_D / 16, P); }                  \
+    } while (0)
+    if (backward_only) RLT_LAUNCH_MLP_WIDE_PASS(MLP_BACKWARD); else if (forward_only) RLT_LAUNCH_MLP_WIDE_PASS(MLP_FORWARD); else RLT_LAUNCH_MLP_WIDE_PASS(MLP_FORWARD_BACKWARD);
+#undef RLT_LAUNCH_MLP_WIDE_PASS
 #undef RLT_LAUNCH_MLP_WIDE
     if ((rc = rlt_launch_status(device))) return rc;
+    if (forward_only) return 0;
     WideReduceArgs R = {};
     R.partial = a.partial; R.blocks = groups; R.count = a.count; R.total = exact;
     float* const dst[6] = {L[0].d_weights, L[0].d_biases, L[1].d_weights, L[1].d_biases, L[2].d_weights, L[2].d_biases};
@@ -1071,10 +1127,17 @@ static int mlp_wide_launch(rlt_rocm_device* device, const rlt_dense_layer* L, in
 }
 int rlt_mlp_wide_forward_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n_layers, const float* x, int ldx, float* y, int ldy,
                                   const float* d_output, int ldd, const float* target, int ldt, float mse_scale, int batch) {
-    return mlp_wide_launch(device, L, n_layers, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, false);
+    return mlp_wide_launch(device, L, n_layers, x, ldx, y, ldy, d_output, ldd, target, ldt, mse_scale, batch, MLP_FORWARD_BACKWARD);
 }
 int rlt_mlp_wide_backward(rlt_rocm_device* device, const rlt_dense_layer* L, int n_layers, const float* x, int ldx, const float* d_pre_last, int ldd, int batch) {
-    return mlp_wide_launch(device, L, n_layers, x, ldx, nullptr, 0, d_pre_last, ldd, nullptr, 0, 0.0f, batch, true);
+    return mlp_wide_launch(device, L, n_layers, x, ldx, nullptr, 0, d_pre_last, ldd, nullptr, 0, 0.0f, batch, MLP_BACKWARD);
+}
+int rlt_mlp_wide_forward(rlt_rocm_device* device, const rlt_dense_layer* L, int n_layers, const float* x, int ldx, float* y, int ldy, int batch, bool keep) {
+    if (keep) return mlp_wide_launch(device, L, n_layers, x, ldx, y, ldy, nullptr, 0, nullptr, 0, 0.0f, batch, MLP_FORWARD);
+    rlt_dense_layer plain[3];      // evaluate(): nothing is kept
+    if (n_layers != 3) return RLT_E_UNSUPPORTED;
+    for (int l = 0; l < 3; l++) { plain[l] = L[l]; plain[l].pre_activations = nullptr; plain[l].output = nullptr; }
+    return mlp_wide_launch(device, plain, n_layers, x, ldx, y, ldy, nullptr, 0, nullptr, 0, 0.0f, batch, MLP_FORWARD);
 }
 
 #ifdef RLT_WIDE_PROFILE

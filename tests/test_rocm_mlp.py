@@ -206,6 +206,7 @@ def test_all_layers_in_one_launch_match_the_checker_and_the_per_layer_kernels(or
     for backend, rows in ((oracle, None), (rocm, "1"), (rocm, "0")):
         if rows is not None:
             os.environ["RLT_MLP_ROWS"] = rows
+            os.environ["RLT_MLP_WIDE"] = rows      # three layers wider than 64 take the sixteen-row tiles (tests/test_rocm_mlp_wide.py): off with the few-rows kernel
         try:
             net = Mlp(backend, dims, params, batch, "tanh", "identity")
             xd, yd = backend.array(x), backend.zeros((batch, dims[-1]))
@@ -215,7 +216,7 @@ def test_all_layers_in_one_launch_match_the_checker_and_the_per_layer_kernels(or
             backend.sync()
             results.append([yd.numpy()] + [p.numpy() for p in net.pre] + [o.numpy() for o in net.out])
         finally:
-            os.environ.pop("RLT_MLP_ROWS", None)
+            os.environ.pop("RLT_MLP_ROWS", None); os.environ.pop("RLT_MLP_WIDE", None)
     ref, one_launch, per_layer = results
     for k in range(len(ref)):
         assert rel_err(one_launch[k], ref[k]) <= TOL and rel_err(per_layer[k], ref[k]) <= TOL and rel_err(one_launch[k], per_layer[k]) <= TOL, k

@@ -97,7 +97,7 @@ def forward_then_backward(backend, dims, params, x, dy, ha, oa):
     backend.call("mlp_forward", net.layers, net.n, xd.ptr, dims[0], B)
     backend.call("mlp_backward", net.layers, net.n, xd.ptr, dims[0], dyd.ptr, dims[-1], None, 0, B, 1, ws, wsn)
     backend.sync()
-    return dict(grads=net.grads.numpy(), d_output=dyd.numpy(), offsets=net.offsets)
+    return dict(grads=net.grads.numpy(), d_output=dyd.numpy(), offsets=net.offsets, pre=[p.numpy() for p in net.pre], out=[o.numpy() for o in net.out])
 
 
 @pytest.mark.parametrize("case", [(256, 17, 256, 6, "relu", "identity"), (4096, 17, 256, 6, "relu", "tanh"), (37, 35, 200, 1, "tanh", "identity"), (100, 128, 72, 16, "fast_tanh", "sigmoid"),
@@ -118,6 +118,8 @@ def test_backward_alone_on_sixteen_row_tiles_matches_the_checker_and_the_other_p
     monkeypatch.delenv("RLT_MLP_WIDE")
     for name, want in (("checker", ref), ("other path", other)):
         assert rel_err(got["d_output"], want["d_output"]) <= TOL, name
+        for l in range(3):      # what forward() keeps: every layer's pre-activations and outputs (hidden widths beyond 64 take the tiles in forward() as well)
+            assert rel_err(got["pre"][l], want["pre"][l]) <= TOL and rel_err(got["out"][l], want["out"][l]) <= TOL, (name, l)
         for (off, nw, nb) in ref["offsets"]:
             ew = rel_err(got["grads"][off:off + nw], want["grads"][off:off + nw]); eb = rel_err(got["grads"][off + nw:off + nw + nb], want["grads"][off + nw:off + nw + nb])
             assert ew <= TOL and eb <= TOL, (name, off, ew, eb)
