@@ -623,9 +623,11 @@ def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=100
     td3.set_batch(oab, rng.standard_normal(batch).astype(np.float32), (rng.random(batch) < 0.05).astype(np.uint8), np.clip(rng.standard_normal((batch, act)) * 0.2, -0.5, 0.5).astype(np.float32))
     noise = rocm.array(rng.standard_normal((batch, act)).astype(np.float32))
 
-    def td3_updates(n):
+    def td3_updates(n, one_call=True):
         for _ in range(n):
-            for k in (0, 1):
+            if one_call:        # the loop's shared-batch case: both critics by one launch
+                rocm.device.check(lib.rlt_rocm_td3_train_critics(h, C.byref(td3.c), noise.ptr, noise.ptr))
+            for k in (() if one_call else (0, 1)):
                 rocm.device.check(lib.rlt_rocm_td3_train_critic(h, C.byref(td3.c), k, noise.ptr))
             rocm.device.check(lib.rlt_rocm_td3_update_critic_targets(h, C.byref(td3.c)))
             rocm.device.check(lib.rlt_rocm_td3_train_actor(h, C.byref(td3.c), noise.ptr))
@@ -634,6 +636,10 @@ def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=100
     rocm.sync()
     a = ev.record(); td3_updates(300); b = ev.record()
     out["td3_width256_agent_obs27_act8_update_sets_per_s_by_device_clock"] = 300 / (ev.elapsed_ms(a, b) * 1e-3)
+    td3_updates(20, False)
+    rocm.sync()
+    a = ev.record(); td3_updates(300, False); b = ev.record()
+    out["td3_width256_agent_obs27_act8_update_sets_per_s_a_call_per_critic"] = 300 / (ev.elapsed_ms(a, b) * 1e-3)
     return out
 
 

@@ -6,6 +6,7 @@
 // they can describe: single-step batches, actor = MLP followed by td3_sampling, critics = MLPs, fp32, symmetric observations. The noise
 // that the reference draws inside evaluate / forward of the td3_sampling layer is drawn on the device into a buffer first.
 #pragma once
+#include <cstring>
 #include <rl_tools/devices/rocm.h>
 #include <rl_tools/rl/algorithms/td3/td3.h>
 #include <rl_tools/rl/components/off_policy_runner/off_policy_runner.h>
@@ -114,6 +115,34 @@ namespace rl_tools{
         if(device.td3_sampling_noise_override){ devices::rocm::check(rlt_rocm_memcpy_d2d(device.handle, sampling_noise, device.td3_sampling_noise_override, BATCH_SIZE * ACTION_DIM * sizeof(float)), "train_critic (sampling noise)"); }
         else{ devices::rocm::check(rlt_rocm_randn_f32(device.handle, sampling_noise, BATCH_SIZE * ACTION_DIM, rng.seed, random::next_stream(rng)), "train_critic (sampling noise)"); }
         devices::rocm::check(rlt_rocm_td3_train_critic(device.handle, &d.agent, critic_index, sampling_noise), "train_critic");
+    }
+    namespace rl::algorithms::td3::rocm{
+        // train_critic for critic 0 and then for critic 1 on one batch and one target noise, the loop's SHARED_BATCH case (rl/algorithms/td3/loop/core/operations_generic.h:98-112),
+        // as one call of the library (one launch for hidden widths beyond 64 and up to 256: the two updates side by side). The sampling noise of the target actor's
+        // td3_sampling layer is drawn for critic 0 and then for critic 1 from the streams the two calls would take. Same bits as the two calls.
+        // false: the two optimisers differ in their parameters; the caller makes the two calls.
+        template <typename DEV_SPEC, typename SPEC, typename BATCH_SPEC, typename OPTIMIZER, typename TRAINING_BUFFERS_SPEC, typename RNG>
+        bool train_critics(devices::ROCM<DEV_SPEC>& device, rl::algorithms::td3::ActorCritic<SPEC>& actor_critic, rl::components::off_policy_runner::SequentialBatch<BATCH_SPEC>& batch, OPTIMIZER (&optimizers)[2],
+                           rl::algorithms::td3::CriticTrainingBuffers<TRAINING_BUFFERS_SPEC>& training_buffers, RNG& rng){
+            using DEVICE = devices::ROCM<DEV_SPEC>;
+            constexpr size_t BATCH_SIZE = BATCH_SPEC::BATCH_SIZE, ACTION_DIM = SPEC::ENVIRONMENT::ACTION_DIM, NOISE = BATCH_SIZE * ACTION_DIM;
+            const rlt_adam_parameters first = rl::algorithms::sac::rocm::adam_parameters(optimizers[0]), second = rl::algorithms::sac::rocm::adam_parameters(optimizers[1]);
+            if(std::memcmp(&first, &second, sizeof(first)) != 0 || device.td3_sampling_noise_override){ return false; }
+            Description<DEVICE, SPEC> d(device, actor_critic);
+            d.set_batch(device, batch, 2 * NOISE * sizeof(float));
+            d.agent.critic_adam = first;
+            d.agent.target_next_action_noise = training_buffers.target_next_action_noise._data;
+            d.agent.next_state_action_value_input = training_buffers.next_state_action_value_input._data;
+            d.agent.next_q[0] = training_buffers.next_state_action_value_critic_1._data; d.agent.next_q[1] = training_buffers.next_state_action_value_critic_2._data;
+            d.agent.target_action_value = training_buffers.target_action_value._data;
+            d.agent.d_output_critic = training_buffers.d_output._data;
+            float* sampling_noise = d.extra();
+            for(int k = 0; k < 2; k++){
+                devices::rocm::check(rlt_rocm_randn_f32(device.handle, sampling_noise + k * NOISE, NOISE, rng.seed, random::next_stream(rng)), "train_critic x 2 (sampling noise)");
+            }
+            devices::rocm::check(rlt_rocm_td3_train_critics(device.handle, &d.agent, sampling_noise, sampling_noise + NOISE), "train_critic x 2");
+            return true;
+        }
     }
     // train_actor             rl/algorithms/td3/operations_generic.h:236-281
     template <typename DEV_SPEC, typename SPEC, typename BATCH_SPEC, typename OPTIMIZER, typename ACTOR_BUFFERS, typename CRITIC_BUFFERS, typename TRAINING_BUFFER_SPEC, typename RNG,

@@ -1025,6 +1025,9 @@ typedef struct rlt_td3_agent {
  * train_critic            rl/algorithms/td3/operations_generic.h:170-235 for critic `critic_index`; sampling_noise [batch x act] are
  *   the N(0,1) draws of the target actor's sampling layer (its evaluate runs in the default mode, which samples). */
 int rlt_rocm_td3_train_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
+/* rlt_rocm_td3_train_critic for critic 0 with sampling_noise_first and then for critic 1 with sampling_noise_second on the agent's batch and target noise (the loop's shared
+ * batch, rl/algorithms/td3/loop/core/operations_generic.h:98-112): same results bit for bit; for hidden widths beyond 64 and up to 256 the two updates are one launch. */
+int rlt_rocm_td3_train_critics(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise_first, const float* sampling_noise_second);
 /* train_actor             td3/operations_generic.h:236-281; sampling_noise as above, for the actor's forward pass */
 int rlt_rocm_td3_train_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise);
 /* update_critic_targets   td3/operations_generic.h:317-321 */

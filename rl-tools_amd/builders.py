@@ -402,10 +402,14 @@ class Td3OnBackend:
     def set_batch(self, oab, rewards, terminated, target_noise):
         self.oab.upload(oab); self.rewards.upload(rewards); self.terminated.upload(terminated); self.target_noise.upload(target_noise)
 
-    def loop_step(self, flags, noise_c0, noise_c1, noise_a):
+    def loop_step(self, flags, noise_c0, noise_c1, noise_a, both_critics_in_one_call=False):
         """The training half of td3::loop::core::step (rl/algorithms/td3/loop/core/operations_generic.h:98-133) on the batch set before."""
         b = self.backend
-        if flags[0]:
+        if flags[0] and both_critics_in_one_call:
+            n0, n1 = b.array(noise_c0.astype(np.float32)), b.array(noise_c1.astype(np.float32))
+            b.call("td3_train_critics", C.byref(self.c), n0.ptr, n1.ptr)
+            b.sync()
+        elif flags[0]:
             for k, nz in enumerate((noise_c0, noise_c1)):
                 n = b.array(nz.astype(np.float32))
                 b.call("td3_train_critic", C.byref(self.c), k, n.ptr)

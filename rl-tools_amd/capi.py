@@ -342,6 +342,7 @@ ROCM_ONLY = {
     "reduce_sum_f32": ([P, P, S, I, P], I),
     "dense_backward_static": ([P, LP, P, I, P, I, I], I),
     "sac_sequence_train_critics": ([P, C.POINTER(SacSequenceAgent), P], I),
+    "td3_train_critics": ([P, C.POINTER(Td3Agent), P, P], I),
     "sac_set_per_operation": ([P, I], I),
     "polyak_update_list": ([P, P, P, P, I, F], I),
     "env_dims": ([I, C.POINTER(I), C.POINTER(I), C.POINTER(I)], I),

@@ -33,6 +33,7 @@ int rlt_td3_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, co
 // and at hidden widths up to 256 (sac_wide.hip)
 bool rlt_td3_wide_supported(const rlt_rocm_device* device, const rlt_td3_agent* agent);
 int rlt_td3_wide_update_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
+int rlt_td3_wide_update_critics(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise_first, const float* sampling_noise_second);
 int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise);
 
 // forward + backward (with weight gradients, added onto the layers' gradients) of one three-layer network of hidden width up to 256 over at most RLT_MLP_WIDE_MAX_BATCH

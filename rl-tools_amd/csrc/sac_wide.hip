@@ -54,6 +54,7 @@ struct WideArgs {
     // TD3 (rl/algorithms/td3/operations_generic.h:170-281): `actor` is the target actor in the critic update and has `act` outputs; they pass tanh and the
     // td3_sampling layer (sac_heads.h); the critic update adds target_noise [batch][act] (already clamped) to the next action; the actor update goes through critic[0] only
     float sampling_std; int ignore_termination; const float* target_noise; float* out_pre_clip;
+    const float* noise_second;             // TD3 critic update of both critics in one launch: the sampling noise of the second (blockIdx.y = 1), each critic's targets being formed with its own
     int packed;                            // every 8th workgroup of an 8 x larger grid works: all of them on one XCD
 };
 
@@ -384,7 +385,8 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
         for (int j = 0; j < 2; j++) {
             if (g + 4 * j < ACT && row0 + c < B) {
                 const size_t i = (size_t)(row0 + c) * ACT + g + 4 * j;
-                noise[j] = A.noise ? A.noise[i] : rlt_randn_element(A.noise_seed, A.noise_stream + *A.stream_offset, i);
+                const float* const given = (MODE == MODE_TD3_CRITIC && y) ? A.noise_second : A.noise;
+                noise[j] = given ? given[i] : rlt_randn_element(A.noise_seed, A.noise_stream + *A.stream_offset, i);
                 if (A.out_noise && y == 0) A.out_noise[i] = noise[j];
             }
         }
@@ -464,7 +466,8 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
                 const float future = (terminated[v] && !(TD3 && A.ignore_termination)) ? 0.0f : A.gamma * min_q;
                 const float y_target = reward[v] + future;
                 const bool ok = c == 0 && row0 + 4 * g + v < B;
-                if (A.out_target_action_value && ok && y == 0) A.out_target_action_value[row0 + 4 * g + v] = y_target;
+                // (SAC's critics share their targets; TD3's are formed with each critic's own sampling noise: the last critic's stay, as after two calls)
+                if (A.out_target_action_value && ok && y == (TD3 ? (int)gridDim.y - 1 : 0)) A.out_target_action_value[row0 + 4 * g + v] = y_target;
                 const float diff = (yc[v] + b3) - y_target;
                 const float dp = ok ? diff * constant : 0.f;
                 if (ok) extra += diff * diff;
@@ -1034,6 +1037,25 @@ int rlt_td3_wide_update_critic(rlt_rocm_device* device, const rlt_td3_agent* A, 
     a.out_target_action_value = A->target_action_value;
     const Optimiser O = {A->critics[ci], A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], nullptr, nullptr, nullptr, 0.0f, nullptr};
     return launch_wide<MODE_TD3_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), &O, 1, 0.0f, nullptr);
+}
+
+// both critics on the agent's batch in one launch (blockIdx.y selects the critic), each with its own sampling noise for the target actor's td3_sampling layer:
+// what rlt_td3_wide_update_critic for critic 0 and then for critic 1 leave, bit for bit
+int rlt_td3_wide_update_critics(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise_first, const float* sampling_noise_second) {
+    if (!rlt_td3_wide_supported(device, A)) return RLT_E_UNSUPPORTED;
+    for (int k = 0; k < 2; k++) for (int l = 0; l < 3; l++) RLT_REQUIRE(A->critics[k][l].d_weights && A->critics[k][l].d_biases);
+    RLT_REQUIRE(A->target_next_action_noise && sampling_noise_first && sampling_noise_second);
+    WideArgs a = {};
+    a.actor = net_of(A->actor_target);
+    for (int k = 0; k < 2; k++) { a.critic[k] = net_of(A->critics[k]); a.target[k] = net_of(A->critics_target[k]); }
+    a.batch_base = A->observations_actions_base; a.rewards = A->rewards; a.terminated = A->terminated; a.noise = sampling_noise_first; a.noise_second = sampling_noise_second;
+    a.target_noise = A->target_next_action_noise;
+    a.sampling_std = A->sampling_std; a.ignore_termination = A->ignore_termination;
+    a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
+    a.out_target_action_value = A->target_action_value;
+    Optimiser O[2];
+    for (int k = 0; k < 2; k++) O[k] = {A->critics[k], A->critic_adam_tensors[k], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[k], nullptr, nullptr, nullptr, 0.0f, nullptr};
+    return launch_wide<MODE_TD3_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), O, 2, 0.0f, nullptr);
 }
 
 int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise) {

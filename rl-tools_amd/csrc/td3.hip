@@ -234,6 +234,20 @@ int rlt_rocm_td3_train_critic(rlt_rocm_device* device, const rlt_td3_agent* A, i
     return rlt_rocm_adam_step(device, A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], 0.0f, nullptr);
 }
 
+// train_critic for critic 0 with sampling_noise_first, then for critic 1 with sampling_noise_second, on the agent's batch and target noise (the loop's shared batch,
+// rl/algorithms/td3/loop/core/operations_generic.h:98-112): for hidden widths beyond 64 and up to 256 both run in one launch, side by side; otherwise the two calls
+int rlt_rocm_td3_train_critics(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise_first, const float* sampling_noise_second) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(agent_ok(A) && sampling_noise_first && sampling_noise_second);
+    if (!device->sac_per_operation && !rlt_td3_update_supported(device, A) && rlt_td3_wide_supported(device, A)) {
+        RLT_REQUIRE(A->target_next_action_noise && A->target_action_value);
+        for (int k = 0; k < 2; k++) RLT_REQUIRE(A->critic_adam_tensors[k] && A->critic_age[k]);
+        return rlt_td3_wide_update_critics(device, A, sampling_noise_first, sampling_noise_second);
+    }
+    const int rc = rlt_rocm_td3_train_critic(device, A, 0, sampling_noise_first);
+    return rc ? rc : rlt_rocm_td3_train_critic(device, A, 1, sampling_noise_second);
+}
+
 // rl/algorithms/td3/operations_generic.h:236-281
 int rlt_rocm_td3_train_actor(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise) {
     if (!device) return RLT_E_NOT_INITIALISED;

@@ -28,6 +28,9 @@
 #include <rl_tools/rl/algorithms/td3/loop/core/config.h>
 #include <rl_tools/rl/loop/steps/evaluation/config.h>
 #include <rl_tools/rl/algorithms/td3/loop/core/operations_generic.h>
+#ifndef TD3_ACROBOT_DEVICE_CPU
+#include <rl_tools/rl/algorithms/td3/loop/core/operations_rocm.h>
+#endif
 #include <rl_tools/rl/loop/steps/evaluation/operations_generic.h>
 
 #include <chrono>

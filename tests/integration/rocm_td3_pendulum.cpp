@@ -21,6 +21,7 @@
 
 #include <rl_tools/rl/algorithms/td3/loop/core/config.h>
 #include <rl_tools/rl/algorithms/td3/loop/core/operations_generic.h>
+#include <rl_tools/rl/algorithms/td3/loop/core/operations_rocm.h>
 #include <rl_tools/rl/utils/evaluation/operations_generic.h>
 
 #include <chrono>

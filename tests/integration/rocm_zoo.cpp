@@ -53,6 +53,9 @@
 #elif defined(ZOO_TD3)
 #include <pendulum-v1/td3.h>
 #include <rl_tools/rl/algorithms/td3/loop/core/operations_generic.h>
+#ifndef ZOO_DEVICE_CPU
+#include <rl_tools/rl/algorithms/td3/loop/core/operations_rocm.h>
+#endif
 #elif defined(ZOO_PPO)
 #include <pendulum-v1/ppo.h>
 #include <rl_tools/rl/algorithms/ppo/loop/core/operations_generic.h>

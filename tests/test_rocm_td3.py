@@ -199,3 +199,31 @@ def fused_against_checker_and_per_operation(oracle, rocm, batch, obs, act, hidde
             err = rel_err(out["fused"][key], ref)
             assert err <= TOL, (other, key, err)
     assert np.abs(out["fused"]["params"] - params).max() > 1e-4
+
+
+@pytest.mark.parametrize("batch,obs,act,hidden,hidden_act", [(256, 27, 8, 256, "relu"), (100, 6, 1, 256, "relu"), (48, 3, 1, 200, "tanh"), (256, 3, 1, 64, "relu")])
+def test_both_critics_in_one_call_leave_the_bits_of_the_two_calls(rocm, batch, obs, act, hidden, hidden_act):
+    """rlt_rocm_td3_train_critics against rlt_rocm_td3_train_critic for critic 0 and then critic 1 on the same batch and target noise, each critic with its own sampling
+    noise: three loop steps from the same parameters; every parameter, the gradients, the optimisers' ages and the target values (the second critic's), bit for bit.
+    Hidden widths beyond 64 run both updates as one launch; at 64 the call makes the two calls."""
+    rng = np.random.default_rng(batch + hidden)
+    D = obs + act
+    adims, cdims = [obs, hidden, hidden, act], [D, hidden, hidden, 1]
+    nets = [helpers.random_params(rng, adims)] * 2 + [helpers.random_params(rng, cdims) for _ in range(2)]
+    params = np.concatenate(nets + [nets[2] * 0.9, nets[3] * 1.1]).astype(np.float32)
+    hyper = dict(gamma=0.99, actor_polyak=0.995, critic_polyak=0.99, sampling_std=0.5, adam=helpers.capi.adam_parameters(epsilon=1e-7))
+    agents = [helpers.Td3OnBackend(rocm, batch, hidden, params, hyper=hyper, masks=False, obs=obs, act=act, hidden_act=hidden_act) for _ in range(2)]
+    for step in range(3):
+        oab = rng.standard_normal((2, batch, D)).astype(np.float32); oab[:, :, obs:] = np.clip(oab[:, :, obs:], -1, 1)
+        rewards, term = rng.standard_normal(batch).astype(np.float32), (rng.random(batch) < 0.2).astype(np.uint8)
+        tn = np.clip(rng.standard_normal((batch, act)) * 0.2, -0.5, 0.5).astype(np.float32)
+        noises = [rng.standard_normal((batch, act)).astype(np.float32) for _ in range(3)]
+        for ag, together in zip(agents, (False, True)):
+            ag.set_batch(oab, rewards, term, tn)
+            ag.loop_step([1, 1, 1, 1], *noises, both_critics_in_one_call=together)
+        for what in ("parameters", "gradients", "ages"):
+            a, b = (getattr(ag, what)() for ag in agents)
+            assert np.array_equal(a, b), (step, what)
+        assert np.array_equal(agents[0].target_q.numpy(), agents[1].target_q.numpy()), step
+    assert np.abs(agents[1].parameters() - params).max() > 1e-4
+
