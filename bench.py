@@ -623,14 +623,18 @@ def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=100
     td3.set_batch(oab, rng.standard_normal(batch).astype(np.float32), (rng.random(batch) < 0.05).astype(np.uint8), np.clip(rng.standard_normal((batch, act)) * 0.2, -0.5, 0.5).astype(np.float32))
     noise = rocm.array(rng.standard_normal((batch, act)).astype(np.float32))
 
+    draws = helpers.capi.Td3CriticDraws(1, 4, (C.c_uint64 * 2)(5, 6), 0.2, 0.5)
+
     def td3_updates(n, one_call=True):
         for _ in range(n):
-            if one_call:        # the loop's shared-batch case: both critics by one launch
-                rocm.device.check(lib.rlt_rocm_td3_train_critics(h, C.byref(td3.c), noise.ptr, noise.ptr))
-            for k in (() if one_call else (0, 1)):
-                rocm.device.check(lib.rlt_rocm_td3_train_critic(h, C.byref(td3.c), k, noise.ptr))
-            rocm.device.check(lib.rlt_rocm_td3_update_critic_targets(h, C.byref(td3.c)))
-            rocm.device.check(lib.rlt_rocm_td3_train_actor(h, C.byref(td3.c), noise.ptr))
+            if one_call:        # the loop's shared-batch case: the smoothing noise, both critics and their targets by one call with the draws made inside
+                rocm.device.check(lib.rlt_rocm_td3_train_critics_drawn(h, C.byref(td3.c), C.byref(draws), None, 1))
+                rocm.device.check(lib.rlt_rocm_td3_train_actor_drawn(h, C.byref(td3.c), 1, 7, None))
+            else:               # a call per operation on noise tensors that are given
+                for k in (0, 1):
+                    rocm.device.check(lib.rlt_rocm_td3_train_critic(h, C.byref(td3.c), k, noise.ptr))
+                rocm.device.check(lib.rlt_rocm_td3_update_critic_targets(h, C.byref(td3.c)))
+                rocm.device.check(lib.rlt_rocm_td3_train_actor(h, C.byref(td3.c), noise.ptr))
             rocm.device.check(lib.rlt_rocm_td3_update_actor_target(h, C.byref(td3.c)))
     td3_updates(20)
     rocm.sync()

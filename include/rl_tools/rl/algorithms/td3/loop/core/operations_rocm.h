@@ -1,7 +1,7 @@
 // One step of the TD3 training loop on devices::ROCM (the reference's is rl/algorithms/td3/loop/core/operations_generic.h:78-133; it has no counterpart in the CUDA
 // backend). For loops that share one batch among the updates: the generic step's operations in its order on its random streams, with the two train_critic calls as
-// one call of the library (rlt_rocm_td3_train_critics: one launch for both critics at hidden widths beyond 64 and up to 256, each critic with the sampling noise the
-// separate calls would have drawn for it). Same bits as the generic step. Every other configuration resolves to the reference's generic step.
+// one call of the library that also makes target_action_noise (rlt_rocm_td3_train_critics_drawn: one launch for both critics at hidden widths beyond 64 and up to 256,
+// the smoothing noise and each critic's sampling noise drawn inside it on the streams the separate calls would have taken). Same bits as the generic step. Every other configuration resolves to the reference's generic step.
 // Include after rl/algorithms/td3/loop/core/operations_generic.h.
 #pragma once
 #include <rl_tools/rl/algorithms/td3/operations_rocm.h>
@@ -33,19 +33,24 @@ namespace rl_tools{
         const bool critic_targets_due = ts.step >= CORE::N_WARMUP_STEPS_CRITIC && ts.step % TD3::CRITIC_TARGET_UPDATE_INTERVAL == 0;
         const bool actor_due = ts.step >= CORE::N_WARMUP_STEPS_ACTOR && ts.step % TD3::ACTOR_TRAINING_INTERVAL == 0;
         const bool actor_target_due = ts.step >= CORE::N_WARMUP_STEPS_ACTOR && ts.step % TD3::ACTOR_TARGET_UPDATE_INTERVAL == 0;
+        bool critics_done = false;
         if(critics_due || actor_due){
             gather_batch(device, ts.off_policy_runner, ts.critic_batch, ts.rng);
-            auto action_noise_matrix_view = matrix_view(device, ts.critic_training_buffers.target_next_action_noise);
-            target_action_noise(device, ts.actor_critic, action_noise_matrix_view, ts.rng);
+            // the smoothing noise, both critic updates and (when due) the targets' soft update as one call with its three draws, on the streams the separate calls take in this order
+            critics_done = critics_due && rl::algorithms::td3::rocm::train_critics<true>(device, ts.actor_critic, ts.critic_batch, ts.actor_critic.critic_optimizers, ts.critic_training_buffers, ts.rng, critic_targets_due);
+            if(!critics_done){
+                auto action_noise_matrix_view = matrix_view(device, ts.critic_training_buffers.target_next_action_noise);
+                target_action_noise(device, ts.actor_critic, action_noise_matrix_view, ts.rng);
+            }
         }
-        if(critics_due){
+        if(critics_due && !critics_done){
             if(!rl::algorithms::td3::rocm::train_critics(device, ts.actor_critic, ts.critic_batch, ts.actor_critic.critic_optimizers, ts.critic_training_buffers, ts.rng)){
                 for(int critic_i = 0; critic_i < 2; critic_i++){
                     train_critic(device, ts.actor_critic, ts.actor_critic.critics[critic_i], ts.critic_batch, ts.actor_critic.critic_optimizers[critic_i], ts.actor_buffers[critic_i], ts.actor_target_buffers[critic_i], ts.critic_buffers[critic_i], ts.critic_target_buffers[critic_i], ts.critic_training_buffers, ts.rng);
                 }
             }
         }
-        if(critic_targets_due){
+        if(critic_targets_due && !critics_done){
             update_critic_targets(device, ts.actor_critic);
         }
         if(actor_due){

@@ -120,10 +120,12 @@ namespace rl_tools{
         // train_critic for critic 0 and then for critic 1 on one batch and one target noise, the loop's SHARED_BATCH case (rl/algorithms/td3/loop/core/operations_generic.h:98-112),
         // as one call of the library (one launch for hidden widths beyond 64 and up to 256: the two updates side by side). The sampling noise of the target actor's
         // td3_sampling layer is drawn for critic 0 and then for critic 1 from the streams the two calls would take. Same bits as the two calls.
-        // false: the two optimisers differ in their parameters; the caller makes the two calls.
-        template <typename DEV_SPEC, typename SPEC, typename BATCH_SPEC, typename OPTIMIZER, typename TRAINING_BUFFERS_SPEC, typename RNG>
+        // DRAW_TARGET_NOISE: target_action_noise into the training buffers first (the stream before the two sampling noises', as the loop step calls it), all three draws
+        // made by the library inside the launch where it is one; update_targets (with DRAW_TARGET_NOISE only): update_critic_targets afterwards, in the same call.
+        // false, before any stream is taken: the two optimisers differ in their parameters, or the sampling noise is given; the caller makes the separate calls.
+        template <bool DRAW_TARGET_NOISE = false, typename DEV_SPEC, typename SPEC, typename BATCH_SPEC, typename OPTIMIZER, typename TRAINING_BUFFERS_SPEC, typename RNG>
         bool train_critics(devices::ROCM<DEV_SPEC>& device, rl::algorithms::td3::ActorCritic<SPEC>& actor_critic, rl::components::off_policy_runner::SequentialBatch<BATCH_SPEC>& batch, OPTIMIZER (&optimizers)[2],
-                           rl::algorithms::td3::CriticTrainingBuffers<TRAINING_BUFFERS_SPEC>& training_buffers, RNG& rng){
+                           rl::algorithms::td3::CriticTrainingBuffers<TRAINING_BUFFERS_SPEC>& training_buffers, RNG& rng, bool update_targets = false){
             using DEVICE = devices::ROCM<DEV_SPEC>;
             constexpr size_t BATCH_SIZE = BATCH_SPEC::BATCH_SIZE, ACTION_DIM = SPEC::ENVIRONMENT::ACTION_DIM, NOISE = BATCH_SIZE * ACTION_DIM;
             const rlt_adam_parameters first = rl::algorithms::sac::rocm::adam_parameters(optimizers[0]), second = rl::algorithms::sac::rocm::adam_parameters(optimizers[1]);
@@ -137,6 +139,15 @@ namespace rl_tools{
             d.agent.target_action_value = training_buffers.target_action_value._data;
             d.agent.d_output_critic = training_buffers.d_output._data;
             float* sampling_noise = d.extra();
+            if(DRAW_TARGET_NOISE){
+                rlt_td3_critic_draws draws;
+                draws.seed = rng.seed;
+                draws.target_noise_stream = random::next_stream(rng);
+                for(int k = 0; k < 2; k++){ draws.sampling_stream[k] = random::next_stream(rng); }
+                draws.target_noise_std = (float)actor_critic.target_next_action_noise_std; draws.target_noise_clip = (float)actor_critic.target_next_action_noise_clip;
+                devices::rocm::check(rlt_rocm_td3_train_critics_drawn(device.handle, &d.agent, &draws, sampling_noise, update_targets ? 1 : 0), "target_action_noise, train_critic x 2");
+                return true;
+            }
             for(int k = 0; k < 2; k++){
                 devices::rocm::check(rlt_rocm_randn_f32(device.handle, sampling_noise + k * NOISE, NOISE, rng.seed, random::next_stream(rng)), "train_critic x 2 (sampling noise)");
             }
@@ -160,7 +171,10 @@ namespace rl_tools{
         d.agent.d_actor_output = training_buffers.d_actor_output._data;
         float* sampling_noise = d.extra();
         if(device.td3_sampling_noise_override){ devices::rocm::check(rlt_rocm_memcpy_d2d(device.handle, sampling_noise, device.td3_sampling_noise_override, BATCH_SIZE * ACTION_DIM * sizeof(float)), "train_actor (sampling noise)"); }
-        else{ devices::rocm::check(rlt_rocm_randn_f32(device.handle, sampling_noise, BATCH_SIZE * ACTION_DIM, rng.seed, random::next_stream(rng)), "train_actor (sampling noise)"); }
+        else{       // the draw inside the update's launch where the library has one
+            devices::rocm::check(rlt_rocm_td3_train_actor_drawn(device.handle, &d.agent, rng.seed, random::next_stream(rng), sampling_noise), "train_actor");
+            return;
+        }
         devices::rocm::check(rlt_rocm_td3_train_actor(device.handle, &d.agent, sampling_noise), "train_actor");
     }
     // update_critic_targets / update_actor_target   rl/algorithms/td3/operations_generic.h:317-325

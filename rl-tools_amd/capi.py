@@ -217,6 +217,10 @@ class Td3SequenceAgent(C.Structure):
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
 
 
+class Td3CriticDraws(C.Structure):
+    _fields_ = [("seed", C.c_uint64), ("target_noise_stream", C.c_uint64), ("sampling_stream", C.c_uint64 * 2), ("target_noise_std", C.c_float), ("target_noise_clip", C.c_float)]
+
+
 class Td3Agent(C.Structure):
     _fields_ = [("batch", C.c_int32), ("observation_dim", C.c_int32), ("action_dim", C.c_int32), ("n_actor_layers", C.c_int32),
                 ("n_critic_layers", C.c_int32), ("ignore_termination", C.c_int32),
@@ -343,6 +347,8 @@ ROCM_ONLY = {
     "dense_backward_static": ([P, LP, P, I, P, I, I], I),
     "sac_sequence_train_critics": ([P, C.POINTER(SacSequenceAgent), P], I),
     "td3_train_critics": ([P, C.POINTER(Td3Agent), P, P], I),
+    "td3_train_critics_drawn": ([P, C.POINTER(Td3Agent), C.POINTER(Td3CriticDraws), P, I], I),
+    "td3_train_actor_drawn": ([P, C.POINTER(Td3Agent), C.c_uint64, C.c_uint64, P], I),
     "sac_set_per_operation": ([P, I], I),
     "polyak_update_list": ([P, P, P, P, I, F], I),
     "env_dims": ([I, C.POINTER(I), C.POINTER(I), C.POINTER(I)], I),

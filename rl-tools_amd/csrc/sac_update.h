@@ -33,8 +33,11 @@ int rlt_td3_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, co
 // and at hidden widths up to 256 (sac_wide.hip)
 bool rlt_td3_wide_supported(const rlt_rocm_device* device, const rlt_td3_agent* agent);
 int rlt_td3_wide_update_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
-int rlt_td3_wide_update_critics(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise_first, const float* sampling_noise_second);
-int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise);
+// draws != NULL: the two sampling noises and the smoothing noise are drawn inside the launch
+int rlt_td3_wide_update_critics(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise_first, const float* sampling_noise_second, const rlt_td3_critic_draws* draws, bool update_targets);
+// (update_targets: update_critic_targets after the two updates, in the optimisers' launch where the tensors correspond)
+// sampling_noise NULL: drawn inside the launch from (seed, stream)
+int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise, uint64_t seed, uint64_t stream);
 
 // forward + backward (with weight gradients, added onto the layers' gradients) of one three-layer network of hidden width up to 256 over at most RLT_MLP_WIDE_MAX_BATCH
 // rows on the wide update kernels' machinery (sac_wide.hip): input width up to 128, output width up to 16, no output activation. d_output or target (the MSE's

@@ -45,6 +45,9 @@ struct WideArgs {
     const float* rewards; const uint8_t* terminated;
     const float* noise;                    // [batch][act], or NULL: drawn from (noise_seed, noise_stream + *stream_offset)
     uint64_t noise_seed, noise_stream; float* out_noise; const uint64_t* stream_offset;
+    // TD3's critic update with its draws made here (noise, noise_second and target_noise NULL): the second critic's sampling noise and the smoothing noise
+    // clamp(N(0, 1) * target_noise_std, -clip, clip) on streams of their own, the latter stored to out_target_noise
+    uint64_t noise_stream_second, target_noise_stream; float target_noise_std, target_noise_clip; float* out_target_noise;
     const float* log_alpha;
     rlt_sas_parameters sas;
     float gamma;
@@ -379,14 +382,24 @@ __global__ __launch_bounds__(THREADS) void sac_wide_kernel(WideArgs A) {
         if (!TD3) alpha = expf(*A.log_alpha);
         if (MODE == MODE_TD3_CRITIC) {
 #pragma unroll
-            for (int j = 0; j < 2; j++) target_noise[j] = (g + 4 * j < ACT && row0 + c < B) ? A.target_noise[(size_t)(row0 + c) * ACT + g + 4 * j] : 0.f;
+            for (int j = 0; j < 2; j++) {
+                if (g + 4 * j < ACT && row0 + c < B) {
+                    const size_t i = (size_t)(row0 + c) * ACT + g + 4 * j;
+                    if (A.target_noise) target_noise[j] = A.target_noise[i];
+                    else {
+                        const float scaled = rlt_randn_element(A.noise_seed, A.target_noise_stream + *A.stream_offset, i) * A.target_noise_std + 0.0f;
+                        target_noise[j] = clampf(scaled, -A.target_noise_clip, A.target_noise_clip);
+                        if (y == 0) A.out_target_noise[i] = target_noise[j];
+                    }
+                }
+            }
         }
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             if (g + 4 * j < ACT && row0 + c < B) {
                 const size_t i = (size_t)(row0 + c) * ACT + g + 4 * j;
                 const float* const given = (MODE == MODE_TD3_CRITIC && y) ? A.noise_second : A.noise;
-                noise[j] = given ? given[i] : rlt_randn_element(A.noise_seed, A.noise_stream + *A.stream_offset, i);
+                noise[j] = given ? given[i] : rlt_randn_element(A.noise_seed, ((MODE == MODE_TD3_CRITIC && y) ? A.noise_stream_second : A.noise_stream) + *A.stream_offset, i);
                 if (A.out_noise && y == 0) A.out_noise[i] = noise[j];
             }
         }
@@ -1041,31 +1054,38 @@ int rlt_td3_wide_update_critic(rlt_rocm_device* device, const rlt_td3_agent* A, 
 
 // both critics on the agent's batch in one launch (blockIdx.y selects the critic), each with its own sampling noise for the target actor's td3_sampling layer:
 // what rlt_td3_wide_update_critic for critic 0 and then for critic 1 leave, bit for bit
-int rlt_td3_wide_update_critics(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise_first, const float* sampling_noise_second) {
+int rlt_td3_wide_update_critics(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise_first, const float* sampling_noise_second, const rlt_td3_critic_draws* draws, bool update_targets) {
     if (!rlt_td3_wide_supported(device, A)) return RLT_E_UNSUPPORTED;
     for (int k = 0; k < 2; k++) for (int l = 0; l < 3; l++) RLT_REQUIRE(A->critics[k][l].d_weights && A->critics[k][l].d_biases);
-    RLT_REQUIRE(A->target_next_action_noise && sampling_noise_first && sampling_noise_second);
+    RLT_REQUIRE(A->target_next_action_noise && (draws || (sampling_noise_first && sampling_noise_second)));
     WideArgs a = {};
     a.actor = net_of(A->actor_target);
     for (int k = 0; k < 2; k++) { a.critic[k] = net_of(A->critics[k]); a.target[k] = net_of(A->critics_target[k]); }
-    a.batch_base = A->observations_actions_base; a.rewards = A->rewards; a.terminated = A->terminated; a.noise = sampling_noise_first; a.noise_second = sampling_noise_second;
-    a.target_noise = A->target_next_action_noise;
+    a.batch_base = A->observations_actions_base; a.rewards = A->rewards; a.terminated = A->terminated;
+    if (draws) {        // the three noise tensors are drawn by the kernel; the smoothing noise is left in the agent's buffer as target_action_noise leaves it
+        a.noise_seed = draws->seed; a.noise_stream = draws->sampling_stream[0]; a.noise_stream_second = draws->sampling_stream[1]; a.target_noise_stream = draws->target_noise_stream;
+        a.target_noise_std = draws->target_noise_std; a.target_noise_clip = draws->target_noise_clip; a.out_target_noise = A->target_next_action_noise;
+    } else { a.noise = sampling_noise_first; a.noise_second = sampling_noise_second; a.target_noise = A->target_next_action_noise; }
     a.sampling_std = A->sampling_std; a.ignore_termination = A->ignore_termination;
     a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
     a.out_target_action_value = A->target_action_value;
     Optimiser O[2];
-    for (int k = 0; k < 2; k++) O[k] = {A->critics[k], A->critic_adam_tensors[k], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[k], nullptr, nullptr, nullptr, 0.0f, nullptr};
-    return launch_wide<MODE_TD3_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), O, 2, 0.0f, nullptr);
+    for (int k = 0; k < 2; k++)
+        O[k] = {A->critics[k], A->critic_adam_tensors[k], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[k], nullptr, nullptr, nullptr, 0.0f, update_targets ? A->critics_target[k] : nullptr};
+    bool targets_done = false;      // the targets' soft update rides along in the optimisers' launch where the tensors correspond
+    const int rc = launch_wide<MODE_TD3_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), O, 2, A->critic_polyak, &targets_done);
+    if (rc || !update_targets || targets_done) return rc;
+    return rlt_rocm_td3_update_critic_targets(device, A);
 }
 
-int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise) {
+int rlt_td3_wide_update_actor(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise, uint64_t seed, uint64_t stream) {
     if (!rlt_td3_wide_supported(device, A)) return RLT_E_UNSUPPORTED;
     for (int l = 0; l < 3; l++) RLT_REQUIRE(A->actor[l].d_weights && A->actor[l].d_biases);
-    RLT_REQUIRE(sampling_noise);
     WideArgs a = {};
     a.actor = net_of(A->actor);
     for (int k = 0; k < 2; k++) { a.critic[k] = net_of(A->critics[0]); a.target[k] = a.critic[k]; }       // the policy gradient goes through critic 0 (:260)
-    a.batch_base = A->observations_actions_base; a.noise = sampling_noise; a.sampling_std = A->sampling_std;
+    a.batch_base = A->observations_actions_base; a.noise = sampling_noise; a.noise_seed = seed; a.noise_stream = stream;      // sampling_noise NULL: drawn from (seed, stream)
+    a.sampling_std = A->sampling_std;
     a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
     a.out_pre_clip = A->actor_pre_clip;
     const Optimiser O = {A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, nullptr, nullptr, nullptr, 0.0f, nullptr};

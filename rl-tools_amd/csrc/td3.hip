@@ -242,10 +242,40 @@ int rlt_rocm_td3_train_critics(rlt_rocm_device* device, const rlt_td3_agent* A, 
     if (!device->sac_per_operation && !rlt_td3_update_supported(device, A) && rlt_td3_wide_supported(device, A)) {
         RLT_REQUIRE(A->target_next_action_noise && A->target_action_value);
         for (int k = 0; k < 2; k++) RLT_REQUIRE(A->critic_adam_tensors[k] && A->critic_age[k]);
-        return rlt_td3_wide_update_critics(device, A, sampling_noise_first, sampling_noise_second);
+        return rlt_td3_wide_update_critics(device, A, sampling_noise_first, sampling_noise_second, nullptr, false);
     }
     const int rc = rlt_rocm_td3_train_critic(device, A, 0, sampling_noise_first);
     return rc ? rc : rlt_rocm_td3_train_critic(device, A, 1, sampling_noise_second);
+}
+
+// the critic update of a shared batch with its draws: inside the one launch where that path applies, by three rlt_rocm_randn_f32 calls otherwise
+int rlt_rocm_td3_train_critics_drawn(rlt_rocm_device* device, const rlt_td3_agent* A, const rlt_td3_critic_draws* draws, float* sampling_noise, int update_targets) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(agent_ok(A) && draws && A->target_next_action_noise && draws->target_noise_std >= 0.0f && draws->target_noise_clip >= 0.0f);
+    if (!device->sac_per_operation && !rlt_td3_update_supported(device, A) && rlt_td3_wide_supported(device, A)) {
+        RLT_REQUIRE(A->target_action_value);
+        for (int k = 0; k < 2; k++) RLT_REQUIRE(A->critic_adam_tensors[k] && A->critic_age[k]);
+        return rlt_td3_wide_update_critics(device, A, nullptr, nullptr, draws, update_targets != 0);
+    }
+    RLT_REQUIRE(sampling_noise);
+    const size_t count = (size_t)A->batch * A->action_dim;
+    int rc = rlt_rocm_randn_f32(device, A->target_next_action_noise, count, draws->seed, draws->target_noise_stream);
+    if (!rc) rc = rlt_rocm_td3_target_action_noise(device, A->target_next_action_noise, draws->target_noise_std, draws->target_noise_clip, A->target_next_action_noise, count);
+    for (int k = 0; k < 2 && !rc; k++) rc = rlt_rocm_randn_f32(device, sampling_noise + k * count, count, draws->seed, draws->sampling_stream[k]);
+    if (!rc) rc = rlt_rocm_td3_train_critics(device, A, sampling_noise, sampling_noise + count);
+    return (rc || !update_targets) ? rc : rlt_rocm_td3_update_critic_targets(device, A);
+}
+
+int rlt_rocm_td3_train_actor_drawn(rlt_rocm_device* device, const rlt_td3_agent* A, uint64_t seed, uint64_t stream, float* sampling_noise) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(agent_ok(A));
+    if (!device->sac_per_operation && !rlt_td3_update_supported(device, A) && rlt_td3_wide_supported(device, A)) {
+        RLT_REQUIRE(A->state_action_value_input && A->actor_pre_clip && A->d_output_actor && A->d_critic_input && A->d_actor_output && A->actor_adam_tensors && A->actor_age);
+        return rlt_td3_wide_update_actor(device, A, nullptr, seed, stream);
+    }
+    RLT_REQUIRE(sampling_noise);
+    const int rc = rlt_rocm_randn_f32(device, sampling_noise, (size_t)A->batch * A->action_dim, seed, stream);
+    return rc ? rc : rlt_rocm_td3_train_actor(device, A, sampling_noise);
 }
 
 // rl/algorithms/td3/operations_generic.h:236-281
@@ -254,7 +284,7 @@ int rlt_rocm_td3_train_actor(rlt_rocm_device* device, const rlt_td3_agent* A, co
     RLT_REQUIRE(agent_ok(A) && sampling_noise);
     RLT_REQUIRE(A->state_action_value_input && A->actor_pre_clip && A->d_output_actor && A->d_critic_input && A->d_actor_output && A->actor_adam_tensors && A->actor_age);
     if (!device->sac_per_operation && rlt_td3_update_supported(device, A)) return rlt_td3_update_actor(device, A, sampling_noise);
-    if (!device->sac_per_operation && rlt_td3_wide_supported(device, A)) return rlt_td3_wide_update_actor(device, A, sampling_noise);
+    if (!device->sac_per_operation && rlt_td3_wide_supported(device, A)) return rlt_td3_wide_update_actor(device, A, sampling_noise, 0, 0);
     const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
     RLT_REQUIRE(A->workspace_bytes >= rlt_rocm_mlp_workspace_bytes(A->critics[0], A->n_critic_layers, B));
     RLT_REQUIRE(A->workspace_bytes >= rlt_rocm_mlp_workspace_bytes(A->actor, A->n_actor_layers, B));

@@ -28,8 +28,8 @@
 #include <rl_tools/rl/algorithms/td3/loop/core/config.h>
 #include <rl_tools/rl/loop/steps/evaluation/config.h>
 #include <rl_tools/rl/algorithms/td3/loop/core/operations_generic.h>
-#ifndef TD3_ACROBOT_DEVICE_CPU
-#include <rl_tools/rl/algorithms/td3/loop/core/operations_rocm.h>
+#if !defined(TD3_ACROBOT_DEVICE_CPU) && !defined(TD3_ACROBOT_GENERIC_STEP)
+#include <rl_tools/rl/algorithms/td3/loop/core/operations_rocm.h>       // the loop step with the smoothing noise and both critic updates as one call
 #endif
 #include <rl_tools/rl/loop/steps/evaluation/operations_generic.h>
 

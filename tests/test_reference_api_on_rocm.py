@@ -305,8 +305,8 @@ def test_td3_on_the_acrobot_swingup_trains_on_rocm():
     """The configuration of the reference's TD3 program for the AcrobotSwingup (src/rl/environments/acrobot/td3/acrobot.cpp: EasyParameters, actor and critics
     3 x 256, the loop's default TD3 parameters) inside the evaluation loop step on devices::ROCM: the exploring actor's td3_sampling head in the library's runner
     step for any environment, evaluations of 10 episodes x 500 steps on the device. Here the first 60,000 of its 100,000 loop steps; measured over all of them:
-    mean return -129 before training, best -7, 14.9 s (6,690 loop steps/s including the 100 evaluations; the updates on the one-launch kernel for widths up to 256,
-    both critics by one launch through the loop step of rl/algorithms/td3/loop/core/operations_rocm.h).
+    mean return -129 before training, best -7, 13.7 s (7,310 loop steps/s including the 100 evaluations; the updates on the one-launch kernel for widths up to 256,
+    the smoothing noise, both critics and the targets' soft update by one call through the loop step of rl/algorithms/td3/loop/core/operations_rocm.h).
     TD3 with one environment does not take off from every seed on this task (of seeds 0, 1, 2 two reach -7 within the 100,000 steps and one stays near -110, and
     which one changes with the last bit of a kernel's sums): the test asks that the first or the second seed learns."""
     path = os.path.join(BUILD, "rocm_td3_acrobot")
@@ -324,7 +324,25 @@ def test_td3_on_the_acrobot_swingup_trains_on_rocm():
         if best[-1] >= -85.0:
             break
     assert max(best) >= -85.0, best
-    assert imports(path, "rlt_rocm_env_runner_step_drawn", "rlt_rocm_env_runner_step_sequential", "rlt_rocm_td3_train_critics", "rlt_rocm_env_evaluate")
+    assert imports(path, "rlt_rocm_env_runner_step_drawn", "rlt_rocm_env_runner_step_sequential", "rlt_rocm_td3_train_critics_drawn", "rlt_rocm_env_evaluate")
+
+
+@pytest.mark.gpu
+def test_td3_loop_step_for_rocm_leaves_the_returns_of_the_generic_step():
+    """rl/algorithms/td3/loop/core/operations_rocm.h (the smoothing noise and both critic updates as one call with their draws inside) against the reference's generic
+    loop step on devices::ROCM (a call per operation, the critic updates' noise tensors drawn by rlt_rocm_randn_f32): the same program built both ways prints the same evaluation
+    returns, digit for digit, over 12,000 loop steps (11,000 of them with updates; this task's returns change with the last bit of any sum)."""
+    paths = [os.path.join(BUILD, name) for name in ("rocm_td3_acrobot", "rocm_td3_acrobot_generic_step")]
+    if not all(os.path.exists(p) for p in paths):
+        pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
+    curves = []
+    for path in paths:
+        out = subprocess.run([path, "1", "12000"], capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
+        curves.append(re.findall(r"^evaluation \d+ step \d+ mean_return [\d.e+-]+", out.stdout, re.M))
+    print(curves[0][-3:], flush=True)
+    assert len(curves[0]) == 12 and curves[0] == curves[1]
+    assert imports(paths[0], "rlt_rocm_td3_train_critics_drawn", "rlt_rocm_td3_train_actor_drawn") and not imports(paths[1], "rlt_rocm_td3_train_critics_drawn")
 
 
 @pytest.mark.gpu

@@ -227,3 +227,49 @@ def test_both_critics_in_one_call_leave_the_bits_of_the_two_calls(rocm, batch, o
         assert np.array_equal(agents[0].target_q.numpy(), agents[1].target_q.numpy()), step
     assert np.abs(agents[1].parameters() - params).max() > 1e-4
 
+
+
+@pytest.mark.parametrize("batch,obs,act,hidden,hidden_act", [(256, 27, 8, 256, "relu"), (100, 6, 1, 256, "relu"), (48, 3, 2, 200, "tanh"), (256, 3, 1, 64, "relu")])
+def test_updates_with_their_draws_leave_the_bits_of_the_separate_calls(rocm, batch, obs, act, hidden, hidden_act):
+    """rlt_rocm_td3_train_critics_drawn and rlt_rocm_td3_train_actor_drawn (the smoothing noise and the sampling noises drawn by the library, inside the update's launch
+    at hidden widths beyond 64) against rlt_rocm_randn_f32 on the same streams, rlt_rocm_td3_target_action_noise, rlt_rocm_td3_train_critics and _train_actor: three
+    loop steps from the same parameters (in the second the drawn call also makes update_critic_targets); the smoothing noise left in the agent's buffer, every parameter, the gradients, the optimisers' ages and the target values,
+    bit for bit."""
+    rng = np.random.default_rng(7 * batch + hidden)
+    D, count = obs + act, batch * act
+    adims, cdims = [obs, hidden, hidden, act], [D, hidden, hidden, 1]
+    nets = [helpers.random_params(rng, adims)] * 2 + [helpers.random_params(rng, cdims) for _ in range(2)]
+    params = np.concatenate(nets + [nets[2] * 0.9, nets[3] * 1.1]).astype(np.float32)
+    hyper = dict(gamma=0.99, actor_polyak=0.995, critic_polyak=0.99, sampling_std=0.5, adam=helpers.capi.adam_parameters(epsilon=1e-7))
+    agents = [helpers.Td3OnBackend(rocm, batch, hidden, params, hyper=hyper, masks=False, obs=obs, act=act, hidden_act=hidden_act) for _ in range(2)]
+    seed, std, clip = 1234, 0.2, 0.25         # the clamp reaches one draw in five
+    for step in range(3):
+        oab = rng.standard_normal((2, batch, D)).astype(np.float32); oab[:, :, obs:] = np.clip(oab[:, :, obs:], -1, 1)
+        rewards, term = rng.standard_normal(batch).astype(np.float32), (rng.random(batch) < 0.2).astype(np.uint8)
+        streams = [10 * step + k for k in range(4)]
+        for ag, drawn in zip(agents, (False, True)):
+            ag.set_batch(oab, rewards, term, np.zeros((batch, act), np.float32))
+            noise = rocm.zeros((3, batch, act))
+            if drawn:
+                draws = helpers.capi.Td3CriticDraws(seed, streams[0], (C.c_uint64 * 2)(streams[1], streams[2]), std, clip)
+                rocm.call("td3_train_critics_drawn", C.byref(ag.c), C.byref(draws), noise.ptr, step % 2)
+                if step % 2 == 0:
+                    rocm.call("td3_update_critic_targets", C.byref(ag.c))
+                rocm.call("td3_train_actor_drawn", C.byref(ag.c), seed, streams[3], noise.ptr)
+            else:
+                rocm.call("randn_f32", ag.target_noise.ptr, count, seed, streams[0])
+                rocm.call("td3_target_action_noise", ag.target_noise.ptr, std, clip, ag.target_noise.ptr, count)
+                for k in range(3):
+                    rocm.call("randn_f32", noise.ptr + 4 * count * k, count, seed, streams[1 + k])
+                rocm.call("td3_train_critics", C.byref(ag.c), noise.ptr, noise.ptr + 4 * count)
+                rocm.call("td3_update_critic_targets", C.byref(ag.c))
+                rocm.call("td3_train_actor", C.byref(ag.c), noise.ptr + 8 * count)
+            rocm.call("td3_update_actor_target", C.byref(ag.c))
+            rocm.sync()
+        assert np.array_equal(agents[0].target_noise.numpy(), agents[1].target_noise.numpy()), step
+        assert np.abs(agents[1].target_noise.numpy()).max() == np.float32(clip)
+        for what in ("parameters", "gradients", "ages"):
+            a, b = (getattr(ag, what)() for ag in agents)
+            assert np.array_equal(a, b), (step, what)
+        assert np.array_equal(agents[0].target_q.numpy(), agents[1].target_q.numpy()), step
+    assert np.abs(agents[1].parameters() - params).max() > 1e-4
