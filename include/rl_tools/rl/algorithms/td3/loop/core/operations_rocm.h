@@ -66,4 +66,59 @@ namespace rl_tools{
         return finished;
     }
 }
+// The same for recurrent agents on sequence batches (rl/algorithms/td3/operations_rocm_sequence.h): the generic step with the two train_critic calls of a shared batch as one
+// rlt_rocm_td3_sequence_train_critics. Same bits as the generic step.
+#include <rl_tools/rl/algorithms/td3/operations_rocm_sequence.h>
+RL_TOOLS_NAMESPACE_WRAPPER_START
+namespace rl_tools{
+    namespace rl::algorithms::td3::loop::core::rocm{
+        template <typename CONFIG>
+        constexpr bool shared_sequence_updates(){
+            return CONFIG::CORE_PARAMETERS::SHARED_BATCH && rl::algorithms::td3::rocm::sequence_describable<typename CONFIG::ACTOR_CRITIC_SPEC, typename CONFIG::CRITIC_BATCH_SPEC>();
+        }
+    }
+    template <typename DEV_SPEC, typename T_CONFIG, utils::typing::enable_if_t<rl::algorithms::td3::loop::core::rocm::shared_sequence_updates<T_CONFIG>(), char> = 0>
+    bool step(devices::ROCM<DEV_SPEC>& device, rl::algorithms::td3::loop::core::State<T_CONFIG>& ts){
+        using CORE = typename T_CONFIG::CORE_PARAMETERS;
+        using TD3 = typename CORE::TD3_PARAMETERS;
+        set_step(device, device.logger, ts.step);
+        bool finished = false;
+        if(ts.step >= CORE::N_WARMUP_STEPS){
+            step<1>(device, ts.off_policy_runner, get_actor(ts), ts.actor_buffers_eval, ts.rng);
+        }
+        else{
+            typename T_CONFIG::EXPLORATION_POLICY exploration_policy;
+            typename T_CONFIG::EXPLORATION_POLICY::template Buffer<> exploration_policy_buffer;
+            step<0>(device, ts.off_policy_runner, exploration_policy, exploration_policy_buffer, ts.rng);
+        }
+        const bool critics_due = ts.step >= CORE::N_WARMUP_STEPS_CRITIC && ts.step % TD3::CRITIC_TRAINING_INTERVAL == 0;
+        const bool actor_due = ts.step >= CORE::N_WARMUP_STEPS_ACTOR && ts.step % TD3::ACTOR_TRAINING_INTERVAL == 0;
+        if(critics_due || actor_due){
+            gather_batch(device, ts.off_policy_runner, ts.critic_batch, ts.rng);
+            auto action_noise_matrix_view = matrix_view(device, ts.critic_training_buffers.target_next_action_noise);
+            target_action_noise(device, ts.actor_critic, action_noise_matrix_view, ts.rng);
+        }
+        if(critics_due){
+            if(!rl::algorithms::td3::rocm::train_critics_on_sequences(device, ts.actor_critic, ts.critic_batch, ts.actor_critic.critic_optimizers, ts.critic_training_buffers)){
+                for(int critic_i = 0; critic_i < 2; critic_i++){
+                    train_critic(device, ts.actor_critic, ts.actor_critic.critics[critic_i], ts.critic_batch, ts.actor_critic.critic_optimizers[critic_i], ts.actor_buffers[critic_i], ts.actor_target_buffers[critic_i], ts.critic_buffers[critic_i], ts.critic_target_buffers[critic_i], ts.critic_training_buffers, ts.rng);
+                }
+            }
+        }
+        if(ts.step >= CORE::N_WARMUP_STEPS_CRITIC && ts.step % TD3::CRITIC_TARGET_UPDATE_INTERVAL == 0){
+            update_critic_targets(device, ts.actor_critic);
+        }
+        if(actor_due){
+            train_actor(device, ts.actor_critic, ts.critic_batch, ts.actor_critic.actor_optimizer, ts.actor_buffers[0], ts.critic_buffers[0], ts.actor_training_buffers, ts.rng);
+        }
+        if(ts.step >= CORE::N_WARMUP_STEPS_ACTOR && ts.step % TD3::ACTOR_TARGET_UPDATE_INTERVAL == 0){
+            update_actor_target(device, ts.actor_critic);
+        }
+        ts.step++;
+        if(ts.step > CORE::STEP_LIMIT){
+            return true;
+        }
+        return finished;
+    }
+}
 RL_TOOLS_NAMESPACE_WRAPPER_END

@@ -7,6 +7,7 @@
 // memory for the duration of a call: the kept intermediates of the target actor and the target critics on the `next` views, the observation columns of the
 // batch laid out back to back for an actor whose first layer is a GRU, and the library's workspace.
 #pragma once
+#include <cstring>
 #include <rl_tools/rl/algorithms/td3/operations_rocm.h>
 #include <rl_tools/rl/algorithms/sac/operations_rocm_sequence.h>
 RL_TOOLS_NAMESPACE_WRAPPER_START
@@ -127,6 +128,38 @@ namespace rl_tools{
         memory = sac_rocm::attach_intermediates(d.targets[1], T * B, memory);
         const int critic_index = &critic == &actor_critic.critics[1] ? 1 : 0;
         devices::rocm::check(rlt_rocm_td3_sequence_train_critic(device.handle, &a, critic_index), "train_critic (sequences)");
+    }
+    namespace rl::algorithms::td3::rocm{
+        // train_critic for critic 0 and then for critic 1 on one sequence batch and one target noise, the loop's SHARED_BATCH case (rl/algorithms/td3/loop/core/operations_generic.h:98-112),
+        // as one call of the library: the second train_critic would repeat the target actor's pass, the noisy next actions, both target critics and the target values on
+        // unchanged inputs; the library computes them once and runs the two critics' passes side by side. Same bits as the two calls; d_output holds critic 1's loss
+        // gradient (critic 0's stays in the library's workspace). false: the two optimisers differ in their parameters; the caller makes the two calls.
+        template <typename DEV_SPEC, typename SPEC, typename BATCH_SPEC, typename OPTIMIZER, typename TRAINING_BUFFERS_SPEC>
+        bool train_critics_on_sequences(devices::ROCM<DEV_SPEC>& device, rl::algorithms::td3::ActorCritic<SPEC>& actor_critic, rl::components::off_policy_runner::SequentialBatch<BATCH_SPEC>& batch, OPTIMIZER (&optimizers)[2],
+                                        rl::algorithms::td3::CriticTrainingBuffers<TRAINING_BUFFERS_SPEC>& training_buffers){
+            using DEVICE = devices::ROCM<DEV_SPEC>;
+            namespace sac_rocm = rl::algorithms::sac::rocm;
+            constexpr size_t S = BATCH_SPEC::SEQUENCE_LENGTHH, B = BATCH_SPEC::BATCH_SIZE;
+            constexpr size_t T = S + (BATCH_SPEC::PARAMETERS::INCLUDE_FIRST_STEP_IN_TARGETS ? 1 : 0);
+            const rlt_adam_parameters first = sac_rocm::adam_parameters(optimizers[0]), second = sac_rocm::adam_parameters(optimizers[1]);
+            if(std::memcmp(&first, &second, sizeof(first)) != 0){ return false; }
+            SequenceDescription<DEVICE, SPEC> d(device, actor_critic);
+            d.set_batch(batch);
+            rlt_td3_sequence_agent& a = d.agent;
+            a.critic_adam = first;
+            a.target_next_action_noise = training_buffers.target_next_action_noise._data;
+            a.next_state_action_value_input = training_buffers.next_state_action_value_input._data;
+            a.next_q[0] = training_buffers.next_state_action_value_critic_1._data; a.next_q[1] = training_buffers.next_state_action_value_critic_2._data;
+            a.target_action_value = training_buffers.target_action_value._data;
+            a.d_output = training_buffers.d_output._data;
+            const size_t intermediates = sac_rocm::intermediates_bytes(d.actor_target, T * B) + sac_rocm::intermediates_bytes(d.targets[0], T * B) + sac_rocm::intermediates_bytes(d.targets[1], T * B);
+            char* memory = d.attach_workspace(device, intermediates, T * B);
+            memory = sac_rocm::attach_intermediates(d.actor_target, T * B, memory);
+            memory = sac_rocm::attach_intermediates(d.targets[0], T * B, memory);
+            memory = sac_rocm::attach_intermediates(d.targets[1], T * B, memory);
+            devices::rocm::check(rlt_rocm_td3_sequence_train_critics(device.handle, &a), "train_critic x 2 (sequences)");
+            return true;
+        }
     }
     // train_actor             rl/algorithms/td3/operations_generic.h:236-281 on a sequence batch (through critic 0)
     template <typename DEV_SPEC, typename SPEC, typename BATCH_SPEC, typename OPTIMIZER, typename ACTOR_BUFFERS, typename CRITIC_BUFFERS, typename TRAINING_BUFFER_SPEC, typename RNG,

@@ -1082,6 +1082,10 @@ size_t rlt_rocm_td3_sequence_workspace_bytes(const rlt_td3_sequence_agent* agent
  * `next` views with next_reset, noisy clamped next actions, actions of non-final steps taken from the batch, targets from the
  * step after, loss reweighted by S*B / (number of final steps), gradient masked to the final steps */
 int rlt_rocm_td3_sequence_train_critic(rlt_rocm_device* device, const rlt_td3_sequence_agent* agent, int critic_index);
+/* rlt_rocm_td3_sequence_train_critic for critic 0 and then for critic 1 on the agent's batch and target noise (the loop's shared batch,
+ * rl/algorithms/td3/loop/core/operations_generic.h:98-112): same results bit for bit; what the second call would repeat is computed once and independent passes run
+ * side by side on the handle's side streams. */
+int rlt_rocm_td3_sequence_train_critics(rlt_rocm_device* device, const rlt_td3_sequence_agent* agent);
 /* train_actor on a sequence batch    td3/operations_generic.h:236-281 (through critic 0) */
 int rlt_rocm_td3_sequence_train_actor(rlt_rocm_device* device, const rlt_td3_sequence_agent* agent);
 /* update_critic_targets / update_actor_target   td3/operations_generic.h:283-325 (dense and GRU layers incl. the initial hidden state) */

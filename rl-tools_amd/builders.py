@@ -716,12 +716,14 @@ class Td3SequenceOnBackend:
         for k in SEQUENCE_BATCH_FIELDS:
             self.batch.arrays[k].upload(data[k])
 
-    def train(self, noise, flags=(1, 1, 1, 1)):
+    def train(self, noise, flags=(1, 1, 1, 1), both_critics_in_one_call=False):
         """The training part of one loop step with a shared batch (rl/algorithms/td3/loop/core/operations_generic.h:91-127); noise: the clamped target-action
         noise [T x B x act]; flags: (train critics, update critic targets, train actor, update actor target)."""
         be = self.backend
         self.buf["noise"].upload(np.ascontiguousarray(noise, np.float32).reshape(self.buf["noise"].shape))
-        if flags[0]:
+        if flags[0] and both_critics_in_one_call:
+            be.call("td3_sequence_train_critics", C.byref(self.c))
+        elif flags[0]:
             for k in range(2):
                 be.call("td3_sequence_train_critic", C.byref(self.c), k)
         if flags[1]:

@@ -346,6 +346,7 @@ ROCM_ONLY = {
     "reduce_sum_f32": ([P, P, S, I, P], I),
     "dense_backward_static": ([P, LP, P, I, P, I, I], I),
     "sac_sequence_train_critics": ([P, C.POINTER(SacSequenceAgent), P], I),
+    "td3_sequence_train_critics": ([P, C.POINTER(Td3SequenceAgent)], I),
     "td3_train_critics": ([P, C.POINTER(Td3Agent), P, P], I),
     "td3_train_critics_drawn": ([P, C.POINTER(Td3Agent), C.POINTER(Td3CriticDraws), P, I], I),
     "td3_train_actor_drawn": ([P, C.POINTER(Td3Agent), C.c_uint64, C.c_uint64, P], I),

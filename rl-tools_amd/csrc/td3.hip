@@ -389,7 +389,8 @@ static size_t td3_sequence_pass_workspace_bytes(const rlt_td3_sequence_agent* A)
 }
 size_t rlt_rocm_td3_sequence_workspace_bytes(const rlt_td3_sequence_agent* A) {
     if (!A || !A->actor || !A->actor_target || !A->critics[0] || !A->critics_target[0]) return 0;
-    return 2 * td3_sequence_pass_workspace_bytes(A);      // two passes may run at the same time (rlt_side_begin), each in its own half
+    // three passes may run at the same time (rlt_side_begin), each in its own part; behind them the first critic's loss gradient of rlt_rocm_td3_sequence_train_critics
+    return 3 * td3_sequence_pass_workspace_bytes(A) + (((size_t)A->batch.sequence_length * A->batch.batch * sizeof(float) + 255) & ~(size_t)255);
 }
 
 // rl/algorithms/td3/operations_generic.h:170-235 on a sequence batch, one launch per reference operation
@@ -439,6 +440,70 @@ int rlt_rocm_td3_sequence_train_critic(rlt_rocm_device* device, const rlt_td3_se
     if ((rc = rlt_launch_status(device))) return rc;
     if ((rc = rlt_rocm_seq_backward(device, critic, A->n_critic_layers, K.observations_actions_base, D, A->d_output, nullptr, K.reset, S, B, 1, 0, ws, ws_bytes))) return rc;   // :233
     return rlt_rocm_adam_step(device, A->critic_adam_tensors[ci], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[ci], 0.0f, nullptr);   // :234
+}
+
+// rlt_rocm_td3_sequence_train_critic for critic 0 and then for critic 1 on one batch and one target noise (the loop's shared batch, td3/loop/core/operations_generic.h:98-112):
+// what the second call would repeat (the target actor's pass, the noisy next actions, both target critics' passes, the targets) is computed once, and the passes that do
+// not depend on each other run side by side: critic 0's forward pass and then target critic 1 on one side stream, critic 1's forward pass on the other, the target actor
+// and target critic 0 on the main stream; then the two backward passes side by side. Same results bit for bit (every pass is the same launches on the same inputs).
+int rlt_rocm_td3_sequence_train_critics(rlt_rocm_device* device, const rlt_td3_sequence_agent* A) {
+    if (!device) return RLT_E_NOT_INITIALISED;
+    RLT_REQUIRE(td3_sequence_agent_ok(A));
+    RLT_REQUIRE(A->target_next_action_noise && A->next_state_action_value_input && A->next_q[0] && A->next_q[1] && A->target_action_value);
+    const rlt_sequence_batch& K = A->batch;
+    const int S = K.sequence_length, B = K.batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
+    const int first = A->include_first_step_in_targets ? 1 : 0, T = S + first, next_offset = first ? 0 : 1;
+    const size_t ws_bytes = td3_sequence_pass_workspace_bytes(A);
+    void* ws = A->workspace; void* ws_side = (char*)A->workspace + ws_bytes; void* ws_second = (char*)A->workspace + 2 * ws_bytes;
+    float* d_output_first = (float*)((char*)A->workspace + 3 * ws_bytes);      // critic 0's loss gradient; critic 1's goes to the agent's buffer, where two single calls leave it
+    const bool overlap = S >= 48;
+    int rc;
+    for (int k = 0; k < 2; k++) if ((rc = rlt_rocm_seq_zero_gradient(device, A->critics[k], A->n_critic_layers))) return rc;
+    {
+        if (overlap) rlt_side_begin(device);      // (without a second stream everything below simply runs in order on the one stream)
+        rc = rlt_rocm_seq_forward(device, A->critics[0], A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, device->side_return ? ws_side : ws, ws_bytes);
+        rlt_side_end(device);
+        if (rc) return rc;
+        if (overlap) rlt_side_begin(device, 1);
+        rc = rlt_rocm_seq_forward(device, A->critics[1], A->n_critic_layers, K.observations_actions_base, D, K.reset, S, B, device->side_return ? ws_second : ws, ws_bytes);
+        rlt_side_end(device);
+        if (rc) return rc;
+    }
+    const float* base_next = K.observations_actions_base + (size_t)next_offset * B * D;
+    const uint8_t* next_reset = K.next_reset_base + (size_t)next_offset * B;
+    const uint8_t* next_final = K.next_final_step_mask_base + (size_t)next_offset * B;
+    if ((rc = copy_columns(device, base_next, D, A->actor_input, OBS, T * B, OBS))) return rc;
+    if ((rc = rlt_rocm_seq_forward(device, A->actor_target, A->n_actor_layers, A->actor_input, OBS, next_reset, T, B, ws, ws_bytes))) return rc;
+    float* next_actions = A->next_state_action_value_input + OBS;
+    if ((rc = copy_columns(device, seq_last_output(A->actor_target, A->n_actor_layers), ACT, next_actions, D, T * B, ACT))) return rc;
+    if ((rc = rlt_rocm_td3_noisy_next_actions(device, next_actions, D, A->target_next_action_noise, ACT, T * B, ACT))) return rc;
+    if ((rc = rlt_rocm_mask_copy(device, base_next + OBS, D, next_actions, D, next_final, 1, T * B, ACT))) return rc;
+    if ((rc = copy_columns(device, base_next, D, A->next_state_action_value_input, D, T * B, OBS))) return rc;
+    for (int k = 1; k >= 0; k--) {      // target critic 1 behind critic 0's forward pass on the side stream (it waits for the copies above), target critic 0 on the main stream
+        if (k == 1 && overlap) rlt_side_begin(device);
+        rc = rlt_rocm_seq_forward(device, A->critics_target[k], A->n_critic_layers, A->next_state_action_value_input, D, next_reset, T, B, device->side_return ? ws_side : ws, ws_bytes);
+        if (!rc) rc = rlt_rocm_memcpy_d2d(device, A->next_q[k], seq_last_output(A->critics_target[k], A->n_critic_layers), sizeof(float) * T * B);
+        rlt_side_end(device);
+        if (rc) return rc;
+    }
+    if (overlap && (rc = rlt_side_join(device))) return rc;
+    for (int k = 0; k < 2; k++) {
+        hipLaunchKernelGGL(td3_d_output_kernel, dim3(1), dim3(1024), 0, device->stream, const_cast<float*>(seq_last_output(A->critics[k], A->n_critic_layers)),
+                           (const float*)(A->next_q[0] + (size_t)first * B), (const float*)(A->next_q[1] + (size_t)first * B), (const float*)K.rewards, (const uint8_t*)K.terminated,
+                           A->gamma, A->ignore_termination, A->target_action_value, (const uint8_t*)K.final_step_mask, k ? A->d_output : d_output_first, S * B, 0);
+        if ((rc = rlt_launch_status(device))) return rc;
+    }
+    {
+        if (overlap) rlt_side_begin(device);
+        rc = rlt_rocm_seq_backward(device, A->critics[1], A->n_critic_layers, K.observations_actions_base, D, A->d_output, nullptr, K.reset, S, B, 1, 0, device->side_return ? ws_side : ws, ws_bytes);
+        rlt_side_end(device);
+        if (rc) return rc;
+    }
+    if ((rc = rlt_rocm_seq_backward(device, A->critics[0], A->n_critic_layers, K.observations_actions_base, D, d_output_first, nullptr, K.reset, S, B, 1, 0, ws, ws_bytes))) return rc;
+    if (overlap && (rc = rlt_side_join(device))) return rc;
+    for (int k = 0; k < 2; k++)
+        if ((rc = rlt_rocm_adam_step(device, A->critic_adam_tensors[k], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[k], 0.0f, nullptr))) return rc;
+    return 0;
 }
 
 // td3/operations_generic.h:236-281 on a sequence batch

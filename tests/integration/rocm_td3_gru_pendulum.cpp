@@ -34,6 +34,9 @@
 #include <rl_tools/rl/loop/steps/evaluation/config.h>
 #include <rl_tools/rl/loop/steps/timing/config.h>
 #include <rl_tools/rl/algorithms/td3/loop/core/operations_generic.h>
+#ifndef TD3_GRU_DEVICE_CPU
+#include <rl_tools/rl/algorithms/td3/loop/core/operations_rocm.h>       // the loop step with both critic updates of the shared sequence batch as one call
+#endif
 #include <rl_tools/rl/loop/steps/evaluation/operations_generic.h>
 #include <rl_tools/rl/loop/steps/timing/operations_cpu.h>
 

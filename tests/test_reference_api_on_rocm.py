@@ -158,7 +158,7 @@ def test_the_references_recurrent_td3_loop_runs_on_rocm():
     """rl/algorithms/td3/loop/core with ConfigApproximatorsGRU (sequences of 16 steps x 32, four environments) inside the evaluation and timing loop steps on
     devices::ROCM: the runner steps the recurrent actor whose output is the action (no sampling layer), the updates are the sequence entry points, evaluations run on the
     device. Measured (seed 0): mean return of 50 evaluation episodes -1,248 before training, -555 at its best within 10,000 loop steps (this actor explores through
-    nothing but its own changes, so the curve is uneven), 2,290 loop steps/s including the evaluations; the reference's CPU device (generic operations, one thread): 413."""
+    nothing but its own changes, so the curve is uneven), 2,820 loop steps/s including the evaluations (both critics of the shared batch by one call of the library; 2,290 with two); the reference's CPU device (generic operations, one thread): 413."""
     path = os.path.join(BUILD, "rocm_td3_gru_pendulum")
     if not os.path.exists(path):
         pytest.skip("tests/integration/_build is built where the reference's headers are mounted")
@@ -167,7 +167,7 @@ def test_the_references_recurrent_td3_loop_runs_on_rocm():
     assert out.returncode == 0, out.stdout[-1500:] + out.stderr[-1500:]
     returns = [float(m) for m in re.findall(r"^step \d+ mean_return (-?[\d.]+)", out.stdout, re.M)]
     assert len(returns) == 8 and returns[0] < -1100 and max(returns) > -900
-    assert imports(path, "rlt_rocm_env_runner_step_sequential", "rlt_rocm_gather_sequence_batch", "rlt_rocm_td3_sequence_train_critic", "rlt_rocm_td3_sequence_train_actor", "rlt_rocm_pendulum_evaluate_recurrent")
+    assert imports(path, "rlt_rocm_env_runner_step_sequential", "rlt_rocm_gather_sequence_batch", "rlt_rocm_td3_sequence_train_critics", "rlt_rocm_td3_sequence_train_actor", "rlt_rocm_pendulum_evaluate_recurrent")
 
 
 @pytest.mark.gpu

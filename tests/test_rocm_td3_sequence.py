@@ -70,3 +70,31 @@ def test_td3_sequence_rejects_inconsistent_arguments(rocm):
     agent.c.workspace_bytes = int(lib.rlt_rocm_td3_sequence_workspace_bytes(C.byref(agent.c)))
     assert lib.rlt_rocm_td3_sequence_train_critic(h, C.byref(agent.c), 0) == 0 and lib.rlt_rocm_td3_sequence_train_actor(h, C.byref(agent.c)) == 0
     rocm.sync()
+
+
+@pytest.mark.parametrize("case", [(100, 100, 3, 1, 16, 2, True), (10, 100, 3, 1, 64, 1, False), (48, 64, 5, 2, 32, 2, True)])
+def test_both_critics_in_one_call_leave_the_bits_of_the_two_calls(rocm, case):
+    """rlt_rocm_td3_sequence_train_critics (the target part once, the two critics' passes side by side on the handle's streams from 48 steps up) against
+    rlt_rocm_td3_sequence_train_critic for critic 0 and then for critic 1: three training steps each from the same parameters, batches and noise; every parameter,
+    gradient and optimiser age and the training buffers that both leave behind, bit for bit."""
+    S, B, OBS, ACT, H, variant, include_first = case
+    rng = np.random.default_rng(S * B + 7 * H)
+    body = [(1, None, H, "identity"), (1, H, H, "identity")] + ([(0, H, H, "relu")] if variant == 2 else [])
+    actor_specs, critic_specs = ([(k, in_dim if i is None else i, o, a) for k, i, o, a in body] + [(0, H, out_dim, "identity")] for in_dim, out_dim in ((OBS, ACT), (OBS + ACT, 1)))
+    pa, pc = helpers.random_seq_params(rng, actor_specs), [helpers.random_seq_params(rng, critic_specs) for _ in range(2)]
+    params = np.concatenate([pa, pc[0], pc[1], pa, pc[0] * 0.9, pc[1] * 1.1])
+    agents = [helpers.Td3SequenceOnBackend(rocm, actor_specs, critic_specs, params, S, B, OBS, ACT, include_first) for _ in range(2)]
+    T = S + (1 if include_first else 0)
+    for step in range(3):
+        data = synthetic_sequence_batch(rng, S, B, OBS + ACT)
+        noise = np.clip(rng.standard_normal((T, B, ACT)) * 0.2, -0.5, 0.5).astype(np.float32)
+        for ag, together in zip(agents, (False, True)):
+            ag.set_batch(data)
+            ag.train(noise, both_critics_in_one_call=together)
+        assert np.array_equal(agents[0].parameters(), agents[1].parameters()), (case, step)
+        assert agents[0].ages() == agents[1].ages()
+        for a, b in zip([agents[0].actor, *agents[0].critics], [agents[1].actor, *agents[1].critics]):
+            assert np.array_equal(a.grads.numpy(), b.grads.numpy()), (case, step)
+        for k in ("nsavi", "next_q0", "next_q1", "target", "savi", "d_ci", "d_ao", "d_output"):
+            assert np.array_equal(agents[0].buf[k].numpy(), agents[1].buf[k].numpy()), (case, step, k)
+    assert np.abs(agents[1].parameters() - params).max() > 1e-4
