@@ -100,3 +100,58 @@ def test_what_a_recording_stream_cannot_do_is_refused(rocm):
     assert np.all(x.numpy() == 3.0)
     rocm.call("graph_destroy", graph)
     assert lib.rlt_rocm_malloc(h, C.byref(ptr), 1024) == 0 and lib.rlt_rocm_free(h, ptr) == 0
+
+
+def test_replays_of_recorded_td3_updates_with_their_draws_equal_the_unrecorded_calls(rocm):
+    """TD3 at width 256 (batch 100, observation 6, action 1: the update kernel for hidden widths beyond 64): one update set -- the smoothing noise,
+    both critics and their targets by rlt_rocm_td3_train_critics_drawn, the actor by rlt_rocm_td3_train_actor_drawn, the actor's target -- recorded once with the stream
+    offset advanced at its end, replayed 200 times on one batch, against the same calls unrecorded with the stream numbers written out: every parameter, gradient and
+    optimiser age and the smoothing noise of the last set, bit for bit, at four points on the way."""
+    batch, obs, act, hidden, sets = 100, 6, 1, 256, 200
+    rng = np.random.default_rng(11)
+    D = obs + act
+    nets = [helpers.random_params(rng, [obs, hidden, hidden, act])] * 2 + [helpers.random_params(rng, [D, hidden, hidden, 1]) for _ in range(2)]
+    params = np.concatenate(nets + [nets[2], nets[3]]).astype(np.float32)
+    hyper = dict(gamma=0.99, actor_polyak=0.995, critic_polyak=0.995, sampling_std=0.1, adam=helpers.capi.adam_parameters(epsilon=1e-7))
+    oab = rng.standard_normal((2, batch, D)).astype(np.float32); oab[:, :, obs:] = np.clip(oab[:, :, obs:], -1, 1)
+    rewards, term = rng.standard_normal(batch).astype(np.float32), (rng.random(batch) < 0.1).astype(np.uint8)
+    agents = [helpers.Td3OnBackend(rocm, batch, hidden, params, hyper=hyper, masks=False, obs=obs, act=act) for _ in range(2)]
+    for ag in agents:
+        ag.set_batch(oab, rewards, term, np.zeros((batch, act), np.float32))
+    seed, base = 77, 1000
+
+    def update_set(ag, first_stream):
+        draws = helpers.capi.Td3CriticDraws(seed, first_stream, (C.c_uint64 * 2)(first_stream + 1, first_stream + 2), 0.2, 0.5)
+        rocm.call("td3_train_critics_drawn", C.byref(ag.c), C.byref(draws), None, 1)
+        rocm.call("td3_train_actor_drawn", C.byref(ag.c), seed, first_stream + 3, None)
+        rocm.call("td3_update_actor_target", C.byref(ag.c))
+
+    def state(ag):
+        rocm.sync()
+        return [ag.parameters(), ag.gradients(), ag.ages(), ag.target_noise.numpy(), ag.target_q.numpy()]
+
+    eager, recorded = agents
+    for ag in agents:
+        update_set(ag, base - 4)         # sizes every workspace the recorded calls will need
+    checkpoints = []
+    for g in range(sets):
+        update_set(eager, base + 4 * g)
+        if g % 50 == 49:
+            checkpoints.append(state(eager))
+    graph = C.c_void_p()
+    rocm.call("graph_begin_capture")
+    try:
+        update_set(recorded, base)
+        rocm.call("advance_streams", 4)
+    finally:
+        rocm.call("graph_end_capture", C.byref(graph))
+    try:
+        for k in range(4):
+            for _ in range(50):
+                rocm.call("graph_launch", graph)
+            for got, ref in zip(state(recorded), checkpoints[k]):
+                assert np.array_equal(got, ref), k
+    finally:
+        rocm.call("set_stream_offset", 0)
+        rocm.call("graph_destroy", graph)
+    assert np.abs(checkpoints[-1][0] - params).max() > 1e-4
