@@ -1,6 +1,6 @@
 // One step of the TD3 training loop on devices::ROCM (the reference's is rl/algorithms/td3/loop/core/operations_generic.h:78-133; it has no counterpart in the CUDA
 // backend). For loops that share one batch among the updates: the generic step's operations in its order on its random streams, with the two train_critic calls as
-// one call of the library that also makes target_action_noise (rlt_rocm_td3_train_critics_drawn: one launch for both critics at hidden widths beyond 64 and up to 256,
+// one call of the library that also makes target_action_noise (rlt_rocm_td3_train_critics_drawn: one launch for both critics at hidden widths up to 256,
 // the smoothing noise and each critic's sampling noise drawn inside it on the streams the separate calls would have taken). Same bits as the generic step. Every other configuration resolves to the reference's generic step.
 // Include after rl/algorithms/td3/loop/core/operations_generic.h.
 #pragma once

@@ -118,7 +118,7 @@ namespace rl_tools{
     }
     namespace rl::algorithms::td3::rocm{
         // train_critic for critic 0 and then for critic 1 on one batch and one target noise, the loop's SHARED_BATCH case (rl/algorithms/td3/loop/core/operations_generic.h:98-112),
-        // as one call of the library (one launch for hidden widths beyond 64 and up to 256: the two updates side by side). The sampling noise of the target actor's
+        // as one call of the library (one launch for hidden widths up to 256: the two updates side by side). The sampling noise of the target actor's
         // td3_sampling layer is drawn for critic 0 and then for critic 1 from the streams the two calls would take. Same bits as the two calls.
         // DRAW_TARGET_NOISE: target_action_noise into the training buffers first (the stream before the two sampling noises', as the loop step calls it), all three draws
         // made by the library inside the launch where it is one; update_targets (with DRAW_TARGET_NOISE only): update_critic_targets afterwards, in the same call.

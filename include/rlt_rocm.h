@@ -1026,7 +1026,7 @@ typedef struct rlt_td3_agent {
  *   the N(0,1) draws of the target actor's sampling layer (its evaluate runs in the default mode, which samples). */
 int rlt_rocm_td3_train_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
 /* rlt_rocm_td3_train_critic for critic 0 with sampling_noise_first and then for critic 1 with sampling_noise_second on the agent's batch and target noise (the loop's shared
- * batch, rl/algorithms/td3/loop/core/operations_generic.h:98-112): same results bit for bit; for hidden widths beyond 64 and up to 256 the two updates are one launch. */
+ * batch, rl/algorithms/td3/loop/core/operations_generic.h:98-112): same results bit for bit; for hidden widths up to 256 the two updates are one launch. */
 int rlt_rocm_td3_train_critics(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise_first, const float* sampling_noise_second);
 /* The draws of a critic update on a shared batch: target_action_noise (td3/operations_generic.h:116-128: clamp(N(0, 1) * std, -clip, clip)) from
  * (seed, target_noise_stream), critic k's sampling noise from (seed, sampling_stream[k]); element i of a tensor is element i of rlt_rocm_randn_f32 on that stream. */
@@ -1035,13 +1035,13 @@ typedef struct rlt_td3_critic_draws {
     float target_noise_std, target_noise_clip;
 } rlt_td3_critic_draws;
 /* target_action_noise into agent->target_next_action_noise and rlt_rocm_td3_train_critics with all three noise tensors drawn as `draws` says: same results bit for bit as
- * rlt_rocm_randn_f32 x 3, rlt_rocm_td3_target_action_noise and rlt_rocm_td3_train_critics. For hidden widths beyond 64 and up to 256 the draws are made inside the one
+ * rlt_rocm_randn_f32 x 3, rlt_rocm_td3_target_action_noise and rlt_rocm_td3_train_critics. For hidden widths up to 256 the draws are made inside the one
  * launch; otherwise sampling_noise [2 x batch x act] receives the two sampling noises (it may be NULL where the draws are made inside). update_targets != 0:
  * rlt_rocm_td3_update_critic_targets afterwards as well (same bits; with the one launch, inside the optimisers' launch). */
 int rlt_rocm_td3_train_critics_drawn(rlt_rocm_device* device, const rlt_td3_agent* agent, const rlt_td3_critic_draws* draws, float* sampling_noise, int update_targets);
 /* train_actor             td3/operations_generic.h:236-281; sampling_noise as above, for the actor's forward pass */
 int rlt_rocm_td3_train_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise);
-/* rlt_rocm_td3_train_actor with the sampling noise drawn from (seed, stream) as rlt_rocm_randn_f32 draws it: inside the launch for hidden widths beyond 64 and up to 256,
+/* rlt_rocm_td3_train_actor with the sampling noise drawn from (seed, stream) as rlt_rocm_randn_f32 draws it: inside the launch for hidden widths up to 256,
  * otherwise into sampling_noise [batch x act] first. */
 int rlt_rocm_td3_train_actor_drawn(rlt_rocm_device* device, const rlt_td3_agent* agent, uint64_t seed, uint64_t stream, float* sampling_noise);
 /* update_critic_targets   td3/operations_generic.h:317-321 */

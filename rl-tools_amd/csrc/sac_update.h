@@ -29,7 +29,10 @@ int rlt_sac_polyak_list(rlt_rocm_device* device, const float* const* sources, fl
 // td3_sampling layer, critics as above, no masks.
 bool rlt_td3_update_supported(const rlt_rocm_device* device, const rlt_td3_agent* agent);
 int rlt_td3_update_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);
-int rlt_td3_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise);
+// both critics in one launch; draws != NULL: the noise tensors are drawn inside it; update_targets: update_critic_targets afterwards
+int rlt_td3_update_critics(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise_first, const float* sampling_noise_second, const rlt_td3_critic_draws* draws, bool update_targets);
+// sampling_noise NULL: drawn inside the launch from (seed, stream)
+int rlt_td3_update_actor(rlt_rocm_device* device, const rlt_td3_agent* agent, const float* sampling_noise, uint64_t seed, uint64_t stream);
 // and at hidden widths up to 256 (sac_wide.hip)
 bool rlt_td3_wide_supported(const rlt_rocm_device* device, const rlt_td3_agent* agent);
 int rlt_td3_wide_update_critic(rlt_rocm_device* device, const rlt_td3_agent* agent, int critic_index, const float* sampling_noise);

@@ -62,6 +62,9 @@ struct UpdateArgs {
     // noise == NULL: element i of the noise is element i of the standard-normal stream (noise_seed, noise_stream), what
     // rlt_rocm_randn_f32 would have put there; out_noise (optional) receives the values
     uint64_t noise_seed, noise_stream; float* out_noise; const uint64_t* stream_offset;      // *stream_offset is added to noise_stream
+    // TD3's critic update for both critics (blockIdx.y): the second critic's sampling noise (noise_second, or its stream where the draws are made here), and the
+    // smoothing noise clamp(N(0, 1) * target_noise_std, -clip, clip) drawn here where target_noise is NULL and stored to out_target_noise
+    const float* noise_second; uint64_t noise_stream_second, target_noise_stream; float target_noise_std, target_noise_clip; float* out_target_noise;
     // every 8th workgroup of an 8 x larger grid works, so that all of them run on one XCD and share its L2 (the device hands out
     // workgroups round robin over the XCDs)
     int packed;
@@ -299,14 +302,26 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
         if (!TD3) alpha = expf(*A.log_alpha);
         if (MODE == MODE_TD3_CRITIC) {
 #pragma unroll
-            for (int j = 0; j < 2; j++) target_noise[j] = (kk + 4 * j < ACT && row0 + r < B) ? A.target_noise[(size_t)(row0 + r) * ACT + kk + 4 * j] : 0.f;
+            for (int j = 0; j < 2; j++) {
+                if (kk + 4 * j < ACT && row0 + r < B) {
+                    const size_t i = (size_t)(row0 + r) * ACT + kk + 4 * j;
+                    if (A.target_noise) target_noise[j] = A.target_noise[i];
+                    else {
+                        const float scaled = rlt_randn_element(A.noise_seed, A.target_noise_stream + *A.stream_offset, i) * A.target_noise_std + 0.0f;
+                        target_noise[j] = clampf(scaled, -A.target_noise_clip, A.target_noise_clip);
+                        if (y == 0) A.out_target_noise[i] = target_noise[j];
+                    }
+                }
+            }
         }
         b3_actor = r < A.actor.out ? A.actor.b3[min(r, A.actor.out - 1)] : 0.f;
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             if (kk + 4 * j < ACT && row0 + r < B) {
                 const size_t i = (size_t)(row0 + r) * ACT + kk + 4 * j;
-                noise[j] = A.noise ? A.noise[i] : rlt_randn_element(A.noise_seed, A.noise_stream + *A.stream_offset, i);
+                const bool second = MODE == MODE_TD3_CRITIC && y;      // TD3's critics each take their own sampling noise
+                const float* const given = second ? A.noise_second : A.noise;
+                noise[j] = given ? given[i] : rlt_randn_element(A.noise_seed, (second ? A.noise_stream_second : A.noise_stream) + *A.stream_offset, i);
                 if (A.out_noise && y == 0) A.out_noise[i] = noise[j];
             }
         }
@@ -381,7 +396,8 @@ __global__ __launch_bounds__(THREADS) void sac_update_kernel(UpdateArgs A) {
                 const float future = (terminated[v] && !(TD3 && A.ignore_termination)) ? 0.0f : A.gamma * min_q;
                 const float y_target = reward[v] + future;
                 const bool ok = r == 0 && row0 + 4 * kk + v < B;
-                if (A.out_target_action_value && ok) A.out_target_action_value[row0 + 4 * kk + v] = y_target;
+                // (SAC's critics share their targets; TD3's are formed with each critic's own sampling noise: the last critic's stay, as after two calls)
+                if (A.out_target_action_value && ok && (!TD3 || y == (int)gridDim.y - 1)) A.out_target_action_value[row0 + 4 * kk + v] = y_target;
                 const float q = yc[v] + b3_q[2];
                 const float diff = q - y_target;
                 const float dp = ok ? diff * constant : 0.f;
@@ -770,14 +786,39 @@ int rlt_td3_update_critic(rlt_rocm_device* device, const rlt_td3_agent* A, int c
     return launch_update<MODE_TD3_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), &O, 1);
 }
 
-int rlt_td3_update_actor(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise) {
+// both critics on the agent's batch in one launch (blockIdx.y selects the critic), each with its own sampling noise; draws != NULL: the two sampling noises and the
+// smoothing noise are drawn inside the launch; update_targets: the targets' soft update afterwards (by the launch's last workgroup where the optimisers run there)
+int rlt_td3_update_critics(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise_first, const float* sampling_noise_second, const rlt_td3_critic_draws* draws, bool update_targets) {
+    if (!rlt_td3_update_supported(device, A)) return RLT_E_UNSUPPORTED;
+    for (int k = 0; k < 2; k++) for (int l = 0; l < 3; l++) RLT_REQUIRE(A->critics[k][l].d_weights && A->critics[k][l].d_biases);
+    RLT_REQUIRE(A->target_next_action_noise && (draws || (sampling_noise_first && sampling_noise_second)));
+    UpdateArgs a = {};
+    a.actor = net_of(A->actor_target);
+    for (int k = 0; k < 2; k++) { a.critic[k] = net_of(A->critics[k]); a.target[k] = net_of(A->critics_target[k]); }
+    a.batch_base = A->observations_actions_base; a.rewards = A->rewards; a.terminated = A->terminated;
+    if (draws) {
+        a.noise_seed = draws->seed; a.noise_stream = draws->sampling_stream[0]; a.noise_stream_second = draws->sampling_stream[1]; a.target_noise_stream = draws->target_noise_stream;
+        a.target_noise_std = draws->target_noise_std; a.target_noise_clip = draws->target_noise_clip; a.out_target_noise = A->target_next_action_noise;
+    } else { a.noise = sampling_noise_first; a.noise_second = sampling_noise_second; a.target_noise = A->target_next_action_noise; }
+    a.sampling_std = A->sampling_std; a.ignore_termination = A->ignore_termination;
+    a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
+    a.out_target_action_value = A->target_action_value;
+    Optimiser O[2];
+    for (int k = 0; k < 2; k++)
+        O[k] = {A->critics[k], A->critic_adam_tensors[k], A->n_critic_adam_tensors, &A->critic_adam, A->critic_age[k], nullptr, nullptr, nullptr, 0.0f, update_targets ? A->critics_target[k] : nullptr};
+    const int rc = launch_update<MODE_TD3_CRITIC>(device, a, rlt_div_up(A->batch, ROWS), O, 2, A->critic_polyak);
+    if (rc || !update_targets || a.tail.enabled) return rc;
+    return rlt_rocm_td3_update_critic_targets(device, A);      // the optimisers ran as launches of their own: so does the soft update
+}
+
+int rlt_td3_update_actor(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise, uint64_t seed, uint64_t stream) {
     if (!rlt_td3_update_supported(device, A)) return RLT_E_UNSUPPORTED;
     for (int l = 0; l < 3; l++) RLT_REQUIRE(A->actor[l].d_weights && A->actor[l].d_biases);
-    RLT_REQUIRE(sampling_noise);
     UpdateArgs a = {};
     a.actor = net_of(A->actor);
     for (int k = 0; k < 2; k++) { a.critic[k] = net_of(A->critics[0]); a.target[k] = a.critic[k]; }       // the policy gradient goes through critic 0 (:260)
-    a.batch_base = A->observations_actions_base; a.noise = sampling_noise; a.sampling_std = A->sampling_std;
+    a.batch_base = A->observations_actions_base; a.noise = sampling_noise; a.noise_seed = seed; a.noise_stream = stream;      // sampling_noise NULL: drawn from (seed, stream)
+    a.sampling_std = A->sampling_std;
     a.gamma = A->gamma; a.batch = A->batch; a.obs = A->observation_dim; a.act = A->action_dim;
     a.out_pre_clip = A->actor_pre_clip;
     const Optimiser O = {A->actor, A->actor_adam_tensors, A->n_actor_adam_tensors, &A->actor_adam, A->actor_age, nullptr, nullptr, nullptr, 0.0f, nullptr};

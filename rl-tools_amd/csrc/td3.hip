@@ -235,11 +235,16 @@ int rlt_rocm_td3_train_critic(rlt_rocm_device* device, const rlt_td3_agent* A, i
 }
 
 // train_critic for critic 0 with sampling_noise_first, then for critic 1 with sampling_noise_second, on the agent's batch and target noise (the loop's shared batch,
-// rl/algorithms/td3/loop/core/operations_generic.h:98-112): for hidden widths beyond 64 and up to 256 both run in one launch, side by side; otherwise the two calls
+// rl/algorithms/td3/loop/core/operations_generic.h:98-112): for hidden widths up to 256 both run in one launch, side by side; otherwise the two calls
 int rlt_rocm_td3_train_critics(rlt_rocm_device* device, const rlt_td3_agent* A, const float* sampling_noise_first, const float* sampling_noise_second) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A) && sampling_noise_first && sampling_noise_second);
-    if (!device->sac_per_operation && !rlt_td3_update_supported(device, A) && rlt_td3_wide_supported(device, A)) {
+    if (!device->sac_per_operation && rlt_td3_update_supported(device, A)) {
+        RLT_REQUIRE(A->target_next_action_noise && A->target_action_value);
+        for (int k = 0; k < 2; k++) RLT_REQUIRE(A->critic_adam_tensors[k] && A->critic_age[k]);
+        return rlt_td3_update_critics(device, A, sampling_noise_first, sampling_noise_second, nullptr, false);
+    }
+    if (!device->sac_per_operation && rlt_td3_wide_supported(device, A)) {
         RLT_REQUIRE(A->target_next_action_noise && A->target_action_value);
         for (int k = 0; k < 2; k++) RLT_REQUIRE(A->critic_adam_tensors[k] && A->critic_age[k]);
         return rlt_td3_wide_update_critics(device, A, sampling_noise_first, sampling_noise_second, nullptr, false);
@@ -252,7 +257,12 @@ int rlt_rocm_td3_train_critics(rlt_rocm_device* device, const rlt_td3_agent* A, 
 int rlt_rocm_td3_train_critics_drawn(rlt_rocm_device* device, const rlt_td3_agent* A, const rlt_td3_critic_draws* draws, float* sampling_noise, int update_targets) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A) && draws && A->target_next_action_noise && draws->target_noise_std >= 0.0f && draws->target_noise_clip >= 0.0f);
-    if (!device->sac_per_operation && !rlt_td3_update_supported(device, A) && rlt_td3_wide_supported(device, A)) {
+    if (!device->sac_per_operation && rlt_td3_update_supported(device, A)) {
+        RLT_REQUIRE(A->target_action_value);
+        for (int k = 0; k < 2; k++) RLT_REQUIRE(A->critic_adam_tensors[k] && A->critic_age[k]);
+        return rlt_td3_update_critics(device, A, nullptr, nullptr, draws, update_targets != 0);
+    }
+    if (!device->sac_per_operation && rlt_td3_wide_supported(device, A)) {
         RLT_REQUIRE(A->target_action_value);
         for (int k = 0; k < 2; k++) RLT_REQUIRE(A->critic_adam_tensors[k] && A->critic_age[k]);
         return rlt_td3_wide_update_critics(device, A, nullptr, nullptr, draws, update_targets != 0);
@@ -269,9 +279,9 @@ int rlt_rocm_td3_train_critics_drawn(rlt_rocm_device* device, const rlt_td3_agen
 int rlt_rocm_td3_train_actor_drawn(rlt_rocm_device* device, const rlt_td3_agent* A, uint64_t seed, uint64_t stream, float* sampling_noise) {
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A));
-    if (!device->sac_per_operation && !rlt_td3_update_supported(device, A) && rlt_td3_wide_supported(device, A)) {
+    if (!device->sac_per_operation && (rlt_td3_update_supported(device, A) || rlt_td3_wide_supported(device, A))) {
         RLT_REQUIRE(A->state_action_value_input && A->actor_pre_clip && A->d_output_actor && A->d_critic_input && A->d_actor_output && A->actor_adam_tensors && A->actor_age);
-        return rlt_td3_wide_update_actor(device, A, nullptr, seed, stream);
+        return rlt_td3_update_supported(device, A) ? rlt_td3_update_actor(device, A, nullptr, seed, stream) : rlt_td3_wide_update_actor(device, A, nullptr, seed, stream);
     }
     RLT_REQUIRE(sampling_noise);
     const int rc = rlt_rocm_randn_f32(device, sampling_noise, (size_t)A->batch * A->action_dim, seed, stream);
@@ -283,7 +293,7 @@ int rlt_rocm_td3_train_actor(rlt_rocm_device* device, const rlt_td3_agent* A, co
     if (!device) return RLT_E_NOT_INITIALISED;
     RLT_REQUIRE(agent_ok(A) && sampling_noise);
     RLT_REQUIRE(A->state_action_value_input && A->actor_pre_clip && A->d_output_actor && A->d_critic_input && A->d_actor_output && A->actor_adam_tensors && A->actor_age);
-    if (!device->sac_per_operation && rlt_td3_update_supported(device, A)) return rlt_td3_update_actor(device, A, sampling_noise);
+    if (!device->sac_per_operation && rlt_td3_update_supported(device, A)) return rlt_td3_update_actor(device, A, sampling_noise, 0, 0);
     if (!device->sac_per_operation && rlt_td3_wide_supported(device, A)) return rlt_td3_wide_update_actor(device, A, sampling_noise, 0, 0);
     const int B = A->batch, OBS = A->observation_dim, ACT = A->action_dim, D = OBS + ACT;
     RLT_REQUIRE(A->workspace_bytes >= rlt_rocm_mlp_workspace_bytes(A->critics[0], A->n_critic_layers, B));

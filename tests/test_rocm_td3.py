@@ -205,7 +205,7 @@ def fused_against_checker_and_per_operation(oracle, rocm, batch, obs, act, hidde
 def test_both_critics_in_one_call_leave_the_bits_of_the_two_calls(rocm, batch, obs, act, hidden, hidden_act):
     """rlt_rocm_td3_train_critics against rlt_rocm_td3_train_critic for critic 0 and then critic 1 on the same batch and target noise, each critic with its own sampling
     noise: three loop steps from the same parameters; every parameter, the gradients, the optimisers' ages and the target values (the second critic's), bit for bit.
-    Hidden widths beyond 64 run both updates as one launch; at 64 the call makes the two calls."""
+    Both updates run as one launch (at width 64 in the update kernel for that width, beyond it in the one for widths up to 256)."""
     rng = np.random.default_rng(batch + hidden)
     D = obs + act
     adims, cdims = [obs, hidden, hidden, act], [D, hidden, hidden, 1]
