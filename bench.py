@@ -644,6 +644,19 @@ def bench_sac_api(helpers, rocm, steps=2000, warmup=200, batch=256, capacity=100
     rocm.sync()
     a = ev.record(); td3_updates(300, False); b = ev.record()
     out["td3_width256_agent_obs27_act8_update_sets_per_s_a_call_per_critic"] = 300 / (ev.elapsed_ms(a, b) * 1e-3)
+    # TD3 at the shapes of the zoo's Pendulum agent (src/rl/zoo/pendulum-v1/td3.h: observation 3, action 1, hidden width 64, batch 100): the same two ways
+    obs, act, td3_batch = 3, 1, 100
+    nets = [helpers.random_params(rng, [obs, 64, 64, act])] * 2 + [helpers.random_params(rng, [obs + act, 64, 64, 1]) for _ in range(2)]
+    td3 = helpers.Td3OnBackend(rocm, td3_batch, 64, np.concatenate(nets + [nets[2], nets[3]]).astype(np.float32), masks=False, obs=obs, act=act)
+    oab = rng.standard_normal((2, td3_batch, obs + act)).astype(np.float32); oab[:, :, obs:] = np.tanh(oab[:, :, obs:])
+    td3.set_batch(oab, rng.standard_normal(td3_batch).astype(np.float32), (rng.random(td3_batch) < 0.05).astype(np.uint8),
+                  np.clip(rng.standard_normal((td3_batch, act)) * 0.2, -0.5, 0.5).astype(np.float32))
+    noise = rocm.array(rng.standard_normal((td3_batch, act)).astype(np.float32))
+    for one_call, key in ((True, "td3_width64_agent_obs3_act1_b100_update_sets_per_s_by_device_clock"), (False, "td3_width64_agent_obs3_act1_b100_update_sets_per_s_a_call_per_critic")):
+        td3_updates(20, one_call)
+        rocm.sync()
+        a = ev.record(); td3_updates(300, one_call); b = ev.record()
+        out[key] = 300 / (ev.elapsed_ms(a, b) * 1e-3)
     return out
 
 
